@@ -1,0 +1,275 @@
+"""Write golden input/output vectors by running the reference's own CPU code.
+
+Run in the build container only (the reference checkout does not travel):
+
+    python tests/golden/make_golden.py [/root/reference]
+
+The reference's tests hold no golden bytes for this path, so the functions whose
+exact output only its implementation can pin are executed here on small seeded
+inputs (CPU tensors, no kernel launches) and the inputs + outputs are stored as
+plain ``.npz`` arrays next to this script.  Nothing from the reference's source
+text is stored.
+"""
+from __future__ import annotations
+
+import dataclasses
+import os
+import sys
+
+import numpy as np
+import torch
+
+REF = sys.argv[1] if len(sys.argv) > 1 else "/root/reference"
+sys.path.insert(0, REF)
+
+from obkv_accel import bitpack as rb            # noqa: E402
+from obkv_accel import packing as rp            # noqa: E402
+from obkv_accel import trizone_decompress as rt  # noqa: E402
+from obkv_accel.triton_k_kernel import k_mixed_qk_dot_ref  # noqa: E402
+from obkv_accel.triton_v_kernel import v_dequant_weighted_sum_ref  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def npy(x):
+    if torch.is_tensor(x):
+        return x.detach().cpu().numpy()
+    return np.asarray(x)
+
+
+def put_layer(out: dict, prefix: str, pl) -> None:
+    none_fields = []
+    for f in dataclasses.fields(pl):
+        v = getattr(pl, f.name)
+        if v is None:
+            none_fields.append(f.name)
+        else:
+            out[f"{prefix}.{f.name}"] = npy(v)
+    out[f"{prefix}.__none__"] = np.array(",".join(none_fields))
+
+
+def save(name: str, d: dict) -> None:
+    path = os.path.join(HERE, name + ".npz")
+    np.savez_compressed(path, **d)
+    print(f"{name}: {len(d)} arrays, {os.path.getsize(path)} bytes")
+
+
+# ---------------------------------------------------------------- bitpack
+def case_bitpack():
+    g = torch.Generator().manual_seed(101)
+    d = {}
+    x2 = torch.randint(0, 4, (2, 3, 5, 32), generator=g, dtype=torch.uint8)
+    d["in2"] = npy(x2.clone())
+    xin = x2.clone()
+    d["packed2"] = npy(rb.transfer_8bit_to_2bit_batchwise(xin))
+    d["in2_after"] = npy(xin)
+    x4 = torch.randint(0, 16, (2, 3, 5, 32), generator=g, dtype=torch.uint8)
+    d["in4"] = npy(x4.clone())
+    xin = x4.clone()
+    d["packed4"] = npy(rb.transfer_8bit_to_4bit_batchwise(xin))
+    d["in4_after"] = npy(xin)
+    b = torch.randint(0, 256, (3, 7, 16), generator=g, dtype=torch.uint8)
+    d["bytes"] = npy(b)
+    d["unpacked2"] = npy(rb.transfer_2bit_to_8bit_batchwise(b))
+    d["unpacked4"] = npy(rb.transfer_4bit_to_8bit_batchwise(b))
+    save("bitpack", d)
+
+
+# ---------------------------------------------------------------- quantizer
+def case_quantizer():
+    g = torch.Generator().manual_seed(202)
+    d = {}
+    x = torch.randn(1, 2, 37, 16, generator=g).half()
+    x[0, 0, 3, :] = 0.75          # constant token row
+    x[0, 1, :, 5] = -1.25         # constant channel column
+    x[0, 0, 5, :] = 0.0
+    x[0, 1, 7, :4] = torch.tensor([-3.0, 3.0, 0.0, 1.0]).half()
+    x[0, 0, :, 9] *= 8.0          # outlier channel
+    d["x"] = npy(x)
+    for bits in (2, 4, 8):
+        for dim in (2, 3):
+            q, s, z = rp.quantize_and_pack(x, bits, dim)
+            d[f"q_b{bits}_d{dim}"] = npy(q)
+            d[f"s_b{bits}_d{dim}"] = npy(s)
+            d[f"z_b{bits}_d{dim}"] = npy(z)
+    # D=128 rows like the V path, larger dynamic range
+    y = (torch.randn(1, 1, 64, 128, generator=g) * torch.rand(1, 1, 64, 1, generator=g) * 4).half()
+    d["y"] = npy(y)
+    for bits in (2, 4, 8):
+        q, s, z = rp.quantize_and_pack(y, bits, 3)
+        d[f"yq_b{bits}"] = npy(q); d[f"ys_b{bits}"] = npy(s); d[f"yz_b{bits}"] = npy(z)
+    save("quantizer", d)
+
+
+# ---------------------------------------------------------------- reference test inputs
+def case_ref_test_segment_counts():
+    """Inputs of the reference's own packing test (seed 1, tests/test_blockwise_rdkv.py:120-140)."""
+    torch.manual_seed(1)
+    keys = torch.randn(1, 1, 7, 8, dtype=torch.float16)
+    k_bits = torch.tensor([0, 2, 4, 8, 16, 2, 4, 8])
+    d = {"keys": npy(keys), "k_bits": npy(k_bits)}
+    ek = rp.pack_k_mixed(keys.clone(), k_bits)
+    names = ["K_2bit", "K_4bit", "K_8bit", "K_ch_scale", "K_ch_zp", "ch_sort_idx",
+             "ch_perm_padded_idx", "seg_bounds"]
+    for n, v in zip(names, ek):
+        d["k." + n] = npy(v)
+    values = torch.randn(1, 1, 6, 8, dtype=torch.float16)
+    v_bits = torch.tensor([2, 4, 8, 2, 8, 4])
+    d["values"] = npy(values); d["v_bits"] = npy(v_bits)
+    ev = rp.pack_v_segments(values.clone(), v_bits)
+    names = ["V_2bit", "V_4bit", "V_8bit", "V_scale", "V_zp", "sort_idx", "seg_bounds"]
+    for n, v in zip(names, ev):
+        d["v." + n] = npy(v)
+    save("ref_test_segment_counts", d)
+
+
+def perhead_pack(keys, values, v_bits_ph, k_bits, groups, head_dim):
+    h_kv = keys.shape[1]
+    layers, v16s = [], []
+    for head in range(h_kv):
+        vb = v_bits_ph[head]
+        kept = (vb > 0).nonzero(as_tuple=True)[0]
+        kept_bits = vb.index_select(0, kept)
+        counts = tuple(int((kept_bits == bit).sum()) for bit in (2, 4, 8))
+        layer, _, v16 = rp.build_packed_layer(
+            keys[:, head:head + 1].index_select(2, kept),
+            values[:, head:head + 1].index_select(2, kept),
+            kept_bits, k_bits[head],
+            v_segment_counts=counts if sum(counts) > 0 else None,
+            defer_k_for_per_head_stack=True)
+        layers.append(layer); v16s.append(v16)
+    packed, new_v_only = rp._pad_and_stack_per_head_layers(
+        layers, v16s, H_q=h_kv * groups, gqa_factor=groups, head_dim=head_dim,
+        device=keys.device, dtype=keys.dtype, k_bits_per_head=k_bits)
+    return packed, new_v_only
+
+
+def attend(d, packed, new_v_only, q, groups, head_dim):
+    """Composition the reference uses to validate packed layers
+    (blockwise_decode.py:681-753) with its own ref functions."""
+    t_k = packed.T_eff_k if packed.T_eff_k > 0 else packed.T_eff
+    scores = k_mixed_qk_dot_ref(q, packed, t_k) if head_dim == 128 else (
+        torch.einsum("hd,htd->ht", q.float(),
+                     rp.unpack_k_mixed(packed, D=head_dim)[0].float()
+                     .repeat_interleave(groups, dim=0)) / (head_dim ** 0.5))
+    d["scores"] = npy(scores)
+    s = scores.clone()
+    if packed.softmax_mask is not None:
+        s.add_(packed.softmax_mask)
+    w = torch.nn.functional.softmax(s, dim=-1)
+    d["weights"] = npy(w)
+    if packed.seg_bounds_per_head is not None:
+        v_a = rt._unpack_v_perhead(packed, head_dim=head_dim)[0].float()
+    else:
+        va = rt._unpack_v_zone_a(packed)
+        v_a = va[0].float() if va.shape[2] > 0 else torch.zeros(q.shape[0] // groups, 0, head_dim)
+    d["V_zone_a"] = npy(v_a.half())
+    v_full = torch.cat([v_a, new_v_only[0].float()], dim=1) if new_v_only is not None else v_a
+    out = (w.view(v_full.shape[0], groups, t_k) @ v_full).reshape(q.shape[0], head_dim)
+    d["out"] = npy(out)
+    d["K_hat"] = npy(rp.unpack_k_mixed(packed, D=head_dim))
+
+
+def case_ref_test_deferred_stack():
+    """Inputs of tests/test_blockwise_rdkv.py:142-228 (seed 11) + stacked outputs."""
+    torch.manual_seed(11)
+    h_kv, t_len, head_dim, groups = 2, 7, 8, 2
+    keys = torch.randn(1, h_kv, t_len, head_dim, dtype=torch.float16)
+    values = torch.randn_like(keys)
+    v_bits = torch.stack([torch.tensor([2, 4, 8, 16, 0, 2, 4]),
+                          torch.tensor([4, 16, 2, 8, 0, 4, 2])])
+    k_bits = torch.tensor([[2, 4, 8, 0, 16, 2, 4, 8], [4, 2, 0, 8, 16, 4, 2, 8]])
+    d = {"keys": npy(keys), "values": npy(values), "v_bits": npy(v_bits), "k_bits": npy(k_bits),
+         "groups": np.array(groups)}
+    packed, nvo = perhead_pack(keys, values, v_bits, k_bits, groups, head_dim)
+    put_layer(d, "pl", packed)
+    if nvo is not None:
+        d["new_v_only"] = npy(nvo)
+    q = torch.randn(h_kv * groups, head_dim).half()
+    d["q"] = npy(q)
+    attend(d, packed, nvo, q, groups, head_dim)
+    save("ref_test_deferred_stack", d)
+
+
+def case_perhead_d128(name, seed, h_kv, groups, t_len, fr, k_keep, outliers=True):
+    g = torch.Generator().manual_seed(seed)
+    D = 128
+    keys = torch.randn(1, h_kv, t_len, D, generator=g)
+    values = torch.randn(1, h_kv, t_len, D, generator=g)
+    k_bits = torch.zeros(h_kv, D, dtype=torch.long)
+    v_bits = torch.zeros(h_kv, t_len, dtype=torch.long)
+    for h in range(h_kv):
+        if outliers:
+            oc = torch.randperm(D, generator=g)[:4]
+            keys[0, h, :, oc] *= 8.0
+        perm = torch.randperm(D, generator=g)[:k_keep[h][0] + k_keep[h][1] + k_keep[h][2]]
+        c2, c4, c8 = k_keep[h]
+        k_bits[h, perm[:c2]] = 2
+        k_bits[h, perm[c2:c2 + c4]] = 4
+        k_bits[h, perm[c2 + c4:c2 + c4 + c8 // 2]] = 8
+        k_bits[h, perm[c2 + c4 + c8 // 2:]] = 16
+        tp = torch.randperm(t_len, generator=g)
+        n = [int(f * t_len) for f in fr[h]]   # counts for 2,4,8,16 ; rest evicted
+        o = 0
+        for b, c in zip((2, 4, 8, 16), n):
+            v_bits[h, tp[o:o + c]] = b
+            o += c
+    keys, values = keys.half(), values.half()
+    d = {"keys": npy(keys), "values": npy(values), "v_bits": npy(v_bits), "k_bits": npy(k_bits),
+         "groups": np.array(groups)}
+    packed, nvo = perhead_pack(keys, values, v_bits, k_bits, groups, D)
+    put_layer(d, "pl", packed)
+    if nvo is not None:
+        d["new_v_only"] = npy(nvo)
+    q = torch.randn(h_kv * groups, D, generator=g).half()
+    d["q"] = npy(q)
+    attend(d, packed, nvo, q, groups, D)
+    save(name, d)
+
+
+def case_shared_layout():
+    """Legacy shared layout: one v_bits for all heads, 1-D k_bits (build_packed_cache path)."""
+    g = torch.Generator().manual_seed(404)
+    h_kv, groups, t_len, D = 2, 4, 96, 128
+    keys = torch.randn(1, h_kv, t_len, D, generator=g).half()
+    values = torch.randn(1, h_kv, t_len, D, generator=g).half()
+    v_bits = torch.tensor([0, 2, 4, 8, 16, 4, 4, 2])[torch.randint(0, 8, (t_len,), generator=g)]
+    k_bits = torch.tensor([0, 2, 4, 8, 16, 4, 0, 2])[torch.randint(0, 8, (D,), generator=g)]
+    d = {"keys": npy(keys), "values": npy(values), "v_bits": npy(v_bits), "k_bits": npy(k_bits),
+         "groups": np.array(groups)}
+    cache = rp.build_packed_cache(((keys, values),), v_bits, k_bits, original_seq_len=t_len)
+    packed, nvo = cache.packed[0], cache.new_v_only[0]
+    put_layer(d, "pl", packed)
+    if nvo is not None:
+        d["new_v_only"] = npy(nvo)
+    q = torch.randn(h_kv * groups, D, generator=g).half()
+    d["q"] = npy(q)
+    attend(d, packed, nvo, q, groups, D)
+    # the reference's shared-layout V reference on zone-A weights
+    w = torch.from_numpy(d["weights"])
+    sq = lambda t: None if t is None else t.squeeze(0)
+    d["v_ref_zone_a"] = npy(v_dequant_weighted_sum_ref(
+        w[:, :packed.T_eff].contiguous(), sq(packed.V_2bit), sq(packed.V_4bit), sq(packed.V_8bit),
+        packed.V_scale.squeeze(0), packed.V_zp.squeeze(0), packed.seg_bounds))
+    # 2-D per-head k_bits through build_packed_layer directly (non-deferred)
+    k_bits2 = torch.stack([k_bits, k_bits.flip(0)])
+    pl2, tk2, v16 = rp.build_packed_layer(keys, values, v_bits, k_bits2, gqa_factor=groups)
+    d["k_bits2"] = npy(k_bits2)
+    put_layer(d, "pl2", pl2)
+    d["pl2.K_hat"] = npy(rp.unpack_k_mixed(pl2, D=D))
+    save("shared_layout", d)
+
+
+if __name__ == "__main__":
+    torch.set_num_threads(1)
+    case_bitpack()
+    case_quantizer()
+    case_ref_test_segment_counts()
+    case_ref_test_deferred_stack()
+    case_perhead_d128("perhead_d128_a", 303, 2, 4, 80,
+                      fr=[(0.2, 0.3, 0.2, 0.1), (0.1, 0.25, 0.35, 0.2)],
+                      k_keep=[(16, 32, 16), (10, 33, 21)])
+    case_perhead_d128("perhead_d128_b", 305, 3, 2, 50,
+                      fr=[(0.0, 0.0, 0.0, 0.6), (0.5, 0.0, 0.3, 0.0), (0.0, 0.9, 0.0, 0.1)],
+                      k_keep=[(0, 64, 0), (7, 0, 30), (3, 5, 2)], outliers=False)
+    case_shared_layout()
