@@ -1,0 +1,127 @@
+/*
+ * rdkv.h - C ABI of librdkv_hip.so: packed mixed-precision KV decode attention for gfx950.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the name ends in _host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream);
+ *   - strides are in ELEMENTS of the pointed-to type;
+ *   - functions return 0 on success and a negative RDKV_E* code on failure;
+ *     rdkv_last_error() returns a thread-local message for the last failure;
+ *   - no function allocates device memory or synchronizes the device: work is
+ *     only enqueued on `stream`, so every call can be captured in a HIP graph.
+ *     Scratch memory is passed in by the caller (see the *_workspace_bytes calls).
+ *
+ * File:line citations name the reference (package obkv_accel) interface each
+ * entry point replaces.
+ */
+#ifndef RDKV_H
+#define RDKV_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RDKV_OK            0
+#define RDKV_EINVAL       -1   /* bad argument (shape, alignment, range)      */
+#define RDKV_EUNSUPPORTED -2   /* valid request this build does not implement */
+#define RDKV_ELAUNCH      -3   /* HIP reported a launch/runtime error         */
+#define RDKV_EWORKSPACE   -4   /* workspace missing or too small              */
+
+#define RDKV_DTYPE_F32  0
+#define RDKV_DTYPE_F16  1
+#define RDKV_DTYPE_BF16 2
+
+int         rdkv_version(void);
+const char *rdkv_last_error(void);
+
+/* ---- bitpack.py ---------------------------------------------------------- */
+/* transfer_8bit_to_2bit_batchwise (bitpack.py:13-23): rows x n_codes codes (0..3),
+ * n_codes % 4 == 0 -> rows x n_codes/4 bytes, byte[i] = c[i] | c[i+n]<<2 | c[i+2n]<<4 | c[i+3n]<<6. */
+int rdkv_bitpack2(const uint8_t *codes, uint8_t *packed, int64_t rows, int64_t n_codes, void *stream);
+/* transfer_2bit_to_8bit_batchwise (bitpack.py:26-32). */
+int rdkv_bitunpack2(const uint8_t *packed, uint8_t *codes, int64_t rows, int64_t n_packed, void *stream);
+/* transfer_8bit_to_4bit_batchwise (bitpack.py:35-40): byte[i] = c[i] | c[i+n]<<4. */
+int rdkv_bitpack4(const uint8_t *codes, uint8_t *packed, int64_t rows, int64_t n_codes, void *stream);
+/* transfer_4bit_to_8bit_batchwise (bitpack.py:43-47): the reference returns float32. */
+int rdkv_bitunpack4_f32(const uint8_t *packed, float *codes, int64_t rows, int64_t n_packed, void *stream);
+
+/* ---- packing.py : quantizer ---------------------------------------------- */
+/* quantize_and_pack(x, n_bits, dim=last) (packing.py:141-165) fused with the bit-pack of
+ * pack_v_segments (packing.py:751-773).  x: fp16 rows of D channels, row r read at
+ * x + row_idx[r]*x_row_stride (row_idx NULL = identity; this fuses V[:, :, sort_idx]).
+ * pack != 0 writes D*n_bits/8 packed bytes per row, pack == 0 writes D raw codes. */
+int rdkv_quantize_rows(const void *x_f16, int64_t x_row_stride, const int64_t *row_idx,
+                       int64_t rows, int D, int n_bits, int pack,
+                       uint8_t *out, void *scale_f16, void *zp_f16, void *stream);
+
+/* Column (per-channel over T) min/max of K[T, D] fp16 (first half of quantize_and_pack(dim=2)
+ * inside pack_k_mixed, packing.py:315,331,347).  minmax: float[2*D] = {min[D], max[D]}. */
+int rdkv_col_minmax(const void *x_f16, int64_t x_row_stride, int64_t T, int D,
+                    float *minmax, void *stream);
+
+/* Second half of pack_k_mixed (packing.py:296-351): gather sorted channels, zero-pad,
+ * quantize per channel with the min/max from rdkv_col_minmax, bit-pack per segment.
+ * slot_channel[D_padded] maps padded sorted slot -> source channel, -1 = zero pad channel.
+ * Slots [0,n2p) 2-bit (n2p%4==0), [n2p,n2p+n4p) 4-bit (n4p%2==0), then n8 8-bit slots.
+ * Outputs K2[T,n2p/4], K4[T,n4p/2], K8[T,n8] (contiguous; may be NULL when the segment is
+ * empty) and scale/zp fp16 [D_padded]. */
+int rdkv_k_quantize_pack(const void *k_f16, int64_t k_row_stride, int64_t T, int D,
+                         const float *minmax, const int32_t *slot_channel,
+                         int n2p, int n4p, int n8,
+                         uint8_t *K2, uint8_t *K4, uint8_t *K8,
+                         void *scale_f16, void *zp_f16, void *stream);
+
+/* Dequantize (codes - zp) * scale -> fp16 (unpack_v_segment packing.py:1427-1444 and the
+ * per-segment step of unpack_k_mixed packing.py:629-651).  per_row != 0: scale/zp indexed by
+ * row (V); per_row == 0: indexed by unpacked column (K).  out row stride in elements. */
+int rdkv_dequant_f16(const uint8_t *packed, int64_t rows, int n_cols_unpacked, int n_bits,
+                     const void *scale_f16, const void *zp_f16, int per_row,
+                     void *out_f16, int64_t out_row_stride, void *stream);
+
+/* ---- triton_k_kernel.py : k_mixed_qk_dot_into (:1211-1411) ---------------- */
+/* out[hq, t] = (sum_c code[hkv,t,c] * q[hq, perm[c]] * s[hkv,c] - sum_c z*q*s) / sqrt(128),
+ * t < T_eff, reading the reference's padded layout.  q: [H_q,128] of q_dtype.
+ * perm: int64 [H_q or 1, D_padded] (perm_stride_h == 0 for the shared permutation).
+ * K2/K4/K8 may be NULL when their segment is empty. */
+int rdkv_k_qk_dot(const void *q, int q_dtype, int64_t q_stride_h, int H_q, int H_kv,
+                  const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
+                  const uint8_t *K4, int64_t k4_stride_h, int64_t k4_stride_t,
+                  const uint8_t *K8, int64_t k8_stride_h, int64_t k8_stride_t,
+                  const void *scale_f16, const void *zp_f16, int64_t ks_stride_h,
+                  const int64_t *perm, int64_t perm_stride_h,
+                  int n2p, int n4p, int n8, int64_t T_eff,
+                  float *out, int64_t out_stride_h, void *stream);
+
+/* Row softmax over [scores_old + mask | scores_new] written as weights into the same
+ * layout (fast_decode.py:1743-1755).  In place: w_old may alias scores_old.  mask may be
+ * NULL; scores_new may be NULL (n_new = 0). */
+int rdkv_softmax_rows(const float *scores_old, int64_t so_stride_h, const float *mask,
+                      int64_t mask_stride_h, int64_t T_old,
+                      const float *scores_new, int64_t sn_stride_h, int64_t n_new,
+                      float *w_old, int64_t wo_stride_h, float *w_new, int64_t wn_stride_h,
+                      int H_q, void *stream);
+
+/* ---- triton_v_kernel.py : v_dequant_weighted_sum_dispatch_into (:1729-1760) */
+/* out[hq,d] = sum over 2/4/8-bit segments of w*(code-zp)*scale + fp16 zone B
+ * (kernel math triton_v_kernel.py:638-750).  seg_bounds_dev: int32 [H_kv,3] per-head
+ * counts read on the device, or NULL to use the host counts N2,N4,N8 for every head.
+ * V16/n_v16_dev may be NULL (no zone B).  Zone-B weights are read at column max_T_v + t.
+ * workspace: rdkv_v_weighted_sum_workspace_bytes(H_q) bytes. */
+int64_t rdkv_v_weighted_sum_workspace_bytes(int H_q);
+int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, int H_kv,
+                        const uint8_t *V2, int64_t v2_stride_h,
+                        const uint8_t *V4, int64_t v4_stride_h,
+                        const uint8_t *V8, int64_t v8_stride_h,
+                        const void *scale_f16, const void *zp_f16, int64_t vs_stride_h,
+                        const int32_t *seg_bounds_dev, int N2, int N4, int N8,
+                        const void *V16_f16, int64_t v16_stride_h, const int32_t *n_v16_dev,
+                        int64_t max_T_v,
+                        float *out, int64_t out_stride_h,
+                        void *workspace, int64_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RDKV_H */

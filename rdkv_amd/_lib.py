@@ -1,0 +1,127 @@
+"""ctypes binding of librdkv_hip.so (the C ABI declared in include/rdkv.h).
+
+The library is the only compute backend: there is no CPU or PyTorch fallback.  When it
+has not been built, or a tensor does not live on a HIP device, calls raise RuntimeError
+(the reference raises RuntimeError("Triton is not available.") in the same situation,
+obkv_accel/triton_k_kernel.py:1230-1231).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_int, c_int64, c_void_p
+from typing import Optional
+
+import torch
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "librdkv_hip.so")
+
+RDKV_OK = 0
+RDKV_EINVAL = -1
+RDKV_EUNSUPPORTED = -2
+RDKV_ELAUNCH = -3
+RDKV_EWORKSPACE = -4
+
+DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+P = c_void_p
+I = c_int
+L = c_int64
+
+# name -> (restype, argtypes); must list every symbol include/rdkv.h declares.
+SIGNATURES = {
+    "rdkv_version": (I, []),
+    "rdkv_last_error": (c_char_p, []),
+    "rdkv_bitpack2": (I, [P, P, L, L, P]),
+    "rdkv_bitunpack2": (I, [P, P, L, L, P]),
+    "rdkv_bitpack4": (I, [P, P, L, L, P]),
+    "rdkv_bitunpack4_f32": (I, [P, P, L, L, P]),
+    "rdkv_quantize_rows": (I, [P, L, P, L, I, I, I, P, P, P, P]),
+    "rdkv_col_minmax": (I, [P, L, L, I, P, P]),
+    "rdkv_k_quantize_pack": (I, [P, L, L, I, P, P, I, I, I, P, P, P, P, P, P]),
+    "rdkv_dequant_f16": (I, [P, L, I, I, P, P, I, P, L, P]),
+    "rdkv_k_qk_dot": (I, [P, I, L, I, I, P, L, L, P, L, L, P, L, L, P, P, L, P, L, I, I, I, L, P, L, P]),
+    "rdkv_softmax_rows": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P]),
+    "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
+    "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def available() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library (once) and declare every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"rdkv HIP backend is not available: {LIB_PATH} has not been built "
+            "(run `python -m rdkv_amd.build_ext`)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int) -> None:
+    """Map a C status code onto the exception types the reference uses."""
+    if rc == RDKV_OK:
+        return
+    msg = load().rdkv_last_error().decode("utf-8", "replace")
+    if rc == RDKV_EINVAL:
+        raise AssertionError(msg)
+    if rc == RDKV_EUNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(f"rdkv HIP backend error {rc}: {msg}")
+
+
+def require_device(*tensors: Optional[torch.Tensor]) -> torch.device:
+    """All tensors must live on one HIP device; returns it."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "rdkv HIP backend needs tensors on a HIP device (got a "
+                f"{t.device.type} tensor); there is no CPU fallback")
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} vs {t.device}")
+    if dev is None:
+        raise RuntimeError("rdkv HIP backend: no device tensor given")
+    return dev
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None or t.numel() == 0:
+        return None
+    return t.data_ptr()
+
+
+def stream_of(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+_workspaces = {}
+
+
+def workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Per (device, stream) scratch buffer, grown on demand and then reused so that
+    steady-state calls (and HIP-graph capture after a warm-up call) never allocate."""
+    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=dev)
+        _workspaces[key] = buf
+    return buf

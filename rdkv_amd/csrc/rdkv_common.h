@@ -1,0 +1,87 @@
+// Shared host/device helpers for librdkv_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "rdkv.h"
+
+#define RDKV_API extern "C" __attribute__((visibility("default")))
+
+void rdkv_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
+
+#define RDKV_REQUIRE(cond, ...)                 \
+  do {                                          \
+    if (!(cond)) {                              \
+      rdkv_set_error(__VA_ARGS__);              \
+      return RDKV_EINVAL;                       \
+    }                                           \
+  } while (0)
+
+// Checks the launch of the kernel enqueued just before it (no device synchronization).
+#define RDKV_CHECK_LAUNCH(name)                                                     \
+  do {                                                                              \
+    hipError_t e_ = hipGetLastError();                                              \
+    if (e_ != hipSuccess) {                                                         \
+      rdkv_set_error("%s: %s", name, hipGetErrorString(e_));                        \
+      return RDKV_ELAUNCH;                                                          \
+    }                                                                               \
+  } while (0)
+
+static inline int64_t rdkv_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+#define RDKV_WAVE 64
+
+__device__ __forceinline__ float rdkv_h2f(uint16_t bits) {
+  return __half2float(__ushort_as_half(bits));
+}
+__device__ __forceinline__ uint16_t rdkv_f2h(float v) {
+  return __half_as_ushort(__float2half_rn(v));
+}
+
+// Order-preserving float <-> uint mapping so min/max can use integer atomics
+// (min/max are exact and order-independent, so the result is deterministic).
+__device__ __forceinline__ uint32_t rdkv_float_to_ordered(float f) {
+  uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float rdkv_ordered_to_float(uint32_t u) {
+  return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
+__device__ __forceinline__ float rdkv_wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float rdkv_wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float rdkv_wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// The reference's quantizer (packing.py:153-163) for one value, IEEE fp32 with its
+// operation order: scale = max((mx-mn)/qmax, 1e-8); zp = rint(clamp(0 - mn/scale));
+// q = rint(clamp(x/scale + zp)).  Division must be the correctly rounded one.
+struct RdkvQParams {
+  float scale;
+  float zp;
+};
+__device__ __forceinline__ RdkvQParams rdkv_qparams(float mn, float mx, float qmax) {
+  RdkvQParams p;
+  p.scale = fmaxf(__fdiv_rn(__fsub_rn(mx, mn), qmax), 1e-8f);
+  float z = __fsub_rn(0.0f, __fdiv_rn(mn, p.scale));
+  p.zp = rintf(fminf(fmaxf(z, 0.0f), qmax));
+  return p;
+}
+__device__ __forceinline__ uint32_t rdkv_qcode(float x, RdkvQParams p, float qmax) {
+  float v = __fadd_rn(__fdiv_rn(x, p.scale), p.zp);
+  return (uint32_t)rintf(fminf(fmaxf(v, 0.0f), qmax));
+}

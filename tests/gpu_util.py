@@ -1,0 +1,71 @@
+"""Helpers shared by the GPU parity tests (which call the HIP path through the C ABI)."""
+import numpy as np
+import torch
+
+from oracle import rdkv_oracle as O
+
+DEV = "cuda:0"
+
+
+def require_gpu():
+    assert torch.cuda.is_available(), "GPU tests need a HIP device"
+    from rdkv_amd import _lib
+    _lib.load()
+
+
+def t2n(t):
+    return None if t is None else t.detach().cpu().numpy()
+
+
+def to_dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if dtype is not None:
+        t = t.to(dtype)
+    return t.to(DEV)
+
+
+def assert_bits_equal(got, exp, name=""):
+    got, exp = np.asarray(got), np.asarray(exp)
+    assert got.shape == exp.shape, f"{name}: shape {got.shape} != {exp.shape}"
+    assert got.dtype == exp.dtype, f"{name}: dtype {got.dtype} != {exp.dtype}"
+    assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), f"{name}: bits differ"
+
+
+def assert_layers_equal(dev_layer, ora_layer, skip=()):
+    """Field-by-field bit-exact comparison of a device PackedKVLayer with an oracle one."""
+    import dataclasses
+    for f in dataclasses.fields(O.PackedKVLayer):
+        if f.name in skip:
+            continue
+        a, b = getattr(dev_layer, f.name), getattr(ora_layer, f.name)
+        if b is None:
+            assert a is None, f.name
+        elif isinstance(b, tuple):
+            assert tuple(int(v) for v in a) == b, f.name
+        elif isinstance(b, (int, np.integer)):
+            assert int(a) == int(b), f.name
+        else:
+            assert a is not None, f.name
+            assert_bits_equal(t2n(a), b, f.name)
+
+
+def layer_to_device(pl):
+    """Oracle (NumPy) PackedKVLayer -> rdkv_amd PackedKVLayer with device tensors."""
+    import dataclasses
+    from rdkv_amd.packing import PackedKVLayer
+    kw = {}
+    for f in dataclasses.fields(O.PackedKVLayer):
+        v = getattr(pl, f.name)
+        kw[f.name] = to_dev(v) if isinstance(v, np.ndarray) else v
+    return PackedKVLayer(**kw)
+
+
+def attn_close(got, exp, what=""):
+    """Tolerance of the attention outputs: max-abs <= 2e-3 and relative error <= 1e-2
+    (relative = max-abs error / max-abs reference value)."""
+    got, exp = np.asarray(got, np.float64), np.asarray(exp, np.float64)
+    err = np.abs(got - exp).max() if exp.size else 0.0
+    ref = np.abs(exp).max() if exp.size else 1.0
+    assert err <= 2e-3, f"{what}: max-abs error {err:.3e} > 2e-3"
+    assert err <= 1e-2 * max(ref, 1e-30), f"{what}: relative error {err / ref:.3e} > 1e-2"
+    return err

@@ -1,0 +1,122 @@
+"""GPU parity of the reference-layout attention entry points (K scores, softmax, V sum)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import rdkv_oracle as O
+from rdkv_amd import packing, synth
+from rdkv_amd import triton_k_kernel as kk
+from rdkv_amd import triton_v_kernel as vk
+from tests.gpu_util import (DEV, attn_close, layer_to_device, require_gpu, t2n, to_dev)
+from tests.helpers import golden_to_oracle_layer, load_golden
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    require_gpu()
+
+
+def _attend_padded(pl, nvo, q):
+    """fast_decode.py:1707-1768 with the three entry points: K scores -> +mask -> softmax -> V."""
+    T_old = pl.T_eff_k if pl.T_eff_k > 0 else pl.T_eff
+    scores = kk.k_mixed_qk_dot(q.float(), pl, T_old)
+    raw = scores.clone()
+    if pl.softmax_mask is not None:
+        scores.add_(pl.softmax_mask)
+    w = torch.softmax(scores, dim=-1)
+    V16 = nvo[0].contiguous() if nvo is not None else None
+    out = vk.v_dequant_weighted_sum_dispatch(w, pl, V16=V16, n_v16_per_head=pl.n_v16_per_head,
+                                             max_T_v=pl.T_eff)
+    return raw, w, out
+
+
+@pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b"])
+def test_padded_attention_golden(name):
+    g = load_golden(name)
+    pl = layer_to_device(golden_to_oracle_layer(g, "pl"))
+    nvo = to_dev(g["new_v_only"]) if "new_v_only" in g else None
+    q = to_dev(g["q"])
+    raw, w, out = _attend_padded(pl, nvo, q)
+    valid = np.isfinite(g["scores"] + (g["pl.softmax_mask"]))
+    attn_close(t2n(raw)[valid], g["scores"][valid], "scores")
+    attn_close(t2n(w), g["weights"], "weights")
+    attn_close(t2n(out), g["out"], "out")
+    # V kernel alone on the reference's weights, strided views for weights and out
+    wbuf = torch.zeros(w.shape[0], w.shape[1] + 13, device=DEV)
+    wbuf[:, :w.shape[1]] = to_dev(g["weights"])
+    obuf = torch.zeros(w.shape[0], 128 * 2, device=DEV)
+    vk.v_dequant_weighted_sum_dispatch_into(
+        wbuf[:, :w.shape[1]], pl, obuf[:, :128], V16=nvo[0].contiguous() if nvo is not None else None,
+        n_v16_per_head=pl.n_v16_per_head, max_T_v=pl.T_eff)
+    attn_close(t2n(obuf[:, :128]), g["out"], "out(strided)")
+    assert float(obuf[:, 128:].abs().max()) == 0.0
+    # K kernel into a strided buffer; fp16 query accepted as is
+    sbuf = torch.full((q.shape[0], raw.shape[1] + 7), 123.0, device=DEV)
+    kk.k_mixed_qk_dot_into(q, pl, raw.shape[1], sbuf)
+    assert torch.equal(sbuf[:, :raw.shape[1]], raw)
+    assert float((sbuf[:, raw.shape[1]:] - 123.0).abs().max()) == 0.0
+    # the on-device dequantize-then-matmul form agrees too
+    attn_close(t2n(kk.k_mixed_qk_dot_ref(q, pl, raw.shape[1]))[valid], g["scores"][valid], "k ref")
+
+
+def test_shared_layout_golden_attention():
+    g = load_golden("shared_layout")
+    pl = layer_to_device(golden_to_oracle_layer(g, "pl"))
+    q = to_dev(g["q"])
+    T_old = pl.T_eff_k
+    scores = kk.k_mixed_qk_dot(q, pl, T_old)
+    attn_close(t2n(scores), g["scores"], "scores")
+    # pre-squeezed 3-D tensors are accepted (fast_decode.py:637-681)
+    import dataclasses
+    sq = dataclasses.replace(pl, **{k: getattr(pl, k).squeeze(0) for k in
+                                    ("K_2bit", "K_4bit", "K_8bit", "K_ch_scale", "K_ch_zp", "V_2bit", "V_4bit",
+                                     "V_8bit", "V_scale", "V_zp") if getattr(pl, k) is not None})
+    assert torch.equal(kk.k_mixed_qk_dot(q, sq, T_old), scores)
+    w = to_dev(g["weights"])
+    za = vk.v_dequant_weighted_sum_dispatch(w[:, :pl.T_eff].contiguous(), sq)
+    attn_close(t2n(za), g["v_ref_zone_a"], "zone A")
+    za_ref = vk.v_dequant_weighted_sum_ref(w[:, :pl.T_eff].contiguous(), sq.V_2bit, sq.V_4bit, sq.V_8bit,
+                                           sq.V_scale, sq.V_zp, sq.seg_bounds)
+    attn_close(t2n(za_ref), g["v_ref_zone_a"], "zone A torch form")
+    # single-width entry points
+    n2, n4, n8 = pl.seg_bounds
+    parts = (vk.v_weighted_sum_2bit(w[:, :n2].contiguous(), sq.V_2bit, sq.V_scale[:, :n2], sq.V_zp[:, :n2], n2)
+             + vk.v_weighted_sum_4bit(w[:, n2:n2 + n4].contiguous(), sq.V_4bit, sq.V_scale[:, n2:n2 + n4],
+                                      sq.V_zp[:, n2:n2 + n4], n4)
+             + vk.v_weighted_sum_8bit(w[:, n2 + n4:n2 + n4 + n8].contiguous(), sq.V_8bit,
+                                      sq.V_scale[:, n2 + n4:], sq.V_zp[:, n2 + n4:], n8))
+    attn_close(t2n(parts), g["v_ref_zone_a"], "zone A by width")
+
+
+def test_degenerate_layers():
+    q = torch.randn(8, 128, device=DEV).half()
+    K = torch.randn(1, 2, 16, 128, device=DEV).half()
+    V = torch.randn(1, 2, 16, 128, device=DEV).half()
+    # zero kept channels -> zero scores (triton_k_kernel.py:1265-1268)
+    pl, tk, _ = packing.build_packed_layer(K, V, torch.full((16,), 4), torch.zeros(128, dtype=torch.long))
+    s = torch.full((8, 16), 5.0, device=DEV)
+    kk.k_mixed_qk_dot_into(q, pl, 16, s)
+    assert float(s.abs().max()) == 0.0
+    # no tokens -> zero output (triton_v_kernel.py:1345,1507)
+    empty = packing._empty_packed_layer(2, 128, DEV, torch.float16)
+    out = torch.full((8, 128), 3.0, device=DEV)
+    vk.v_dequant_weighted_sum_dispatch_into(torch.zeros(8, 0, device=DEV), empty, out)
+    assert float(out.abs().max()) == 0.0
+    with pytest.raises(AssertionError):
+        kk.k_mixed_qk_dot_into(torch.zeros(8, 64, device=DEV), pl, 16, s)
+
+
+@pytest.mark.parametrize("cfg_idx,ctx", [(0, 4096), (1, 3000), (3, 1500)])
+def test_config_shaped_attention_vs_oracle(cfg_idx, ctx):
+    """C0 at full size (its CPU-runnable case), C1/C3 shapes at reduced context."""
+    cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, q = synth.layer_data(cfg, 0, "cpu", outliers=oc)
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), cfg.G)
+    exp_out, exp_lse, exp_w = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, cfg.G)
+    raw, w, out = _attend_padded(pl, nvo, q.to(DEV))
+    attn_close(t2n(w), exp_w, "weights")
+    attn_close(t2n(out), exp_out, "out")

@@ -1,0 +1,168 @@
+"""GPU parity: bitpack, quantizer and segment packing are bit-exact against the golden
+vectors of the reference and against the oracle on seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import rdkv_oracle as O
+from rdkv_amd import bitpack, packing, synth
+from tests.gpu_util import (DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev)
+from tests.helpers import assert_layer_equal, load_golden
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    require_gpu()
+
+
+def test_bitpack_golden_and_roundtrip():
+    g = load_golden("bitpack")
+    x = to_dev(g["in2"])
+    assert_bits_equal(t2n(bitpack.transfer_8bit_to_2bit_batchwise(x)), g["packed2"])
+    assert_bits_equal(t2n(x), g["in2_after"])
+    x = to_dev(g["in4"])
+    assert_bits_equal(t2n(bitpack.transfer_8bit_to_4bit_batchwise(x)), g["packed4"])
+    assert_bits_equal(t2n(x), g["in4_after"])
+    b = to_dev(g["bytes"])
+    assert_bits_equal(t2n(bitpack.transfer_2bit_to_8bit_batchwise(b)), g["unpacked2"])
+    u4 = bitpack.transfer_4bit_to_8bit_batchwise(b)
+    assert u4.dtype == torch.float32
+    assert_bits_equal(t2n(u4), g["unpacked4"])
+    # exhaustive: every byte value survives unpack -> pack for both widths
+    allb = torch.arange(256, dtype=torch.uint8, device=DEV).reshape(4, 64)
+    assert torch.equal(bitpack.transfer_8bit_to_2bit_batchwise(
+        bitpack.transfer_2bit_to_8bit_batchwise(allb)), allb)
+    assert torch.equal(bitpack.transfer_8bit_to_4bit_batchwise(
+        bitpack.transfer_4bit_to_8bit_batchwise(allb).to(torch.uint8)), allb)
+    # empty and ragged leading shapes
+    e = torch.empty(0, 8, dtype=torch.uint8, device=DEV)
+    assert bitpack.transfer_8bit_to_2bit_batchwise(e).shape == (0, 2)
+    with pytest.raises(AssertionError):
+        bitpack.transfer_8bit_to_2bit_batchwise(torch.zeros(3, 6, dtype=torch.uint8, device=DEV))
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+@pytest.mark.parametrize("dim", [2, 3])
+def test_quantizer_golden(bits, dim):
+    g = load_golden("quantizer")
+    q, s, z = packing.quantize_and_pack(to_dev(g["x"]), bits, dim)
+    assert_bits_equal(t2n(q), g[f"q_b{bits}_d{dim}"])
+    assert_bits_equal(t2n(s), g[f"s_b{bits}_d{dim}"])
+    assert_bits_equal(t2n(z), g[f"z_b{bits}_d{dim}"])
+    if dim == 3:
+        q, s, z = packing.quantize_and_pack(to_dev(g["y"]), bits, 3)
+        assert_bits_equal(t2n(q), g[f"yq_b{bits}"])
+        assert_bits_equal(t2n(s), g[f"ys_b{bits}"])
+        assert_bits_equal(t2n(z), g[f"yz_b{bits}"])
+
+
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_quantizer_random_vs_oracle(bits):
+    rng = np.random.default_rng(bits)
+    x = (rng.standard_normal((1, 3, 257, 128)) * rng.uniform(0.01, 30, (1, 3, 257, 1))).astype(np.float16)
+    x[0, 0, 0] = 0
+    x[0, 1, 5] = 65504.0
+    x[0, 2, 7] = -1.5
+    for dim in (2, 3):
+        q, s, z = packing.quantize_and_pack(to_dev(x), bits, dim)
+        eq, es, ez = O.quantize_and_pack(x, bits, dim)
+        assert_bits_equal(t2n(q), eq)
+        assert_bits_equal(t2n(s), es)
+        assert_bits_equal(t2n(z), ez)
+
+
+def test_reference_test_inputs_segment_counts():
+    """tests/test_blockwise_rdkv.py:120-140 with the stored reference outputs as expectation."""
+    g = load_golden("ref_test_segment_counts")
+    names = ["K_2bit", "K_4bit", "K_8bit", "K_ch_scale", "K_ch_zp", "ch_sort_idx",
+             "ch_perm_padded_idx", "seg_bounds"]
+    for kw in ({}, {"segment_counts": (2, 2, 3)}):
+        got = packing.pack_k_mixed(to_dev(g["keys"]), torch.from_numpy(g["k_bits"]), **kw)
+        for n, v in zip(names, got):
+            v = np.asarray(v) if isinstance(v, tuple) else t2n(v)
+            assert np.array_equal(v, g["k." + n]), n
+    names = ["V_2bit", "V_4bit", "V_8bit", "V_scale", "V_zp", "sort_idx", "seg_bounds"]
+    for kw in ({}, {"segment_counts": (2, 2, 2)}):
+        got = packing.pack_v_segments(to_dev(g["values"]), torch.from_numpy(g["v_bits"]), **kw)
+        for n, v in zip(names, got):
+            v = np.asarray(v) if isinstance(v, tuple) else t2n(v)
+            assert np.array_equal(v, g["v." + n]), n
+    with pytest.raises(AssertionError):
+        packing.pack_v_segments(to_dev(g["values"]), torch.from_numpy(g["v_bits"]), segment_counts=(2, 2, 1))
+
+
+@pytest.mark.parametrize("name", ["ref_test_deferred_stack", "perhead_d128_a", "perhead_d128_b"])
+def test_perhead_stack_golden(name):
+    g = load_golden(name)
+    G = int(g["groups"])
+    pl, nvo = packing.pack_layer_per_head(to_dev(g["keys"]), to_dev(g["values"]),
+                                          torch.from_numpy(g["v_bits"]), torch.from_numpy(g["k_bits"]), G)
+    assert_layer_equal(pl, g, "pl")
+    if "new_v_only" in g:
+        assert_bits_equal(t2n(nvo), g["new_v_only"])
+    else:
+        assert nvo is None
+    D = g["keys"].shape[-1]
+    assert_bits_equal(t2n(packing.unpack_k_mixed(pl, D=D)), g["K_hat"])
+    assert pl.deferred_k_for_stack is None
+
+
+def test_shared_layout_golden():
+    g = load_golden("shared_layout")
+    G = int(g["groups"])
+    K, V = to_dev(g["keys"]), to_dev(g["values"])
+    cache = packing.build_packed_cache(((K, V),), torch.from_numpy(g["v_bits"]),
+                                       torch.from_numpy(g["k_bits"]), original_seq_len=K.shape[2])
+    assert_layer_equal(cache.packed[0], g, "pl")
+    assert_bits_equal(t2n(cache.new_v_only[0]), g["new_v_only"])
+    assert_bits_equal(t2n(packing.unpack_k_mixed(cache.packed[0], D=128)), g["K_hat"])
+    pl2, _, _ = packing.build_packed_layer(K, V, torch.from_numpy(g["v_bits"]),
+                                           torch.from_numpy(g["k_bits2"]), gqa_factor=G)
+    assert_layer_equal(pl2, g, "pl2")
+    assert_bits_equal(t2n(packing.unpack_k_mixed(pl2, D=128)), g["pl2.K_hat"])
+    # V zone A dequantization per segment
+    pl = cache.packed[0]
+    off = 0
+    parts = []
+    for n, seg, bits in zip(pl.seg_bounds, (pl.V_2bit, pl.V_4bit, pl.V_8bit), (2, 4, 8)):
+        if n:
+            parts.append(packing.unpack_v_segment(seg, pl.V_scale[:, :, off:off + n], pl.V_zp[:, :, off:off + n], bits))
+            off += n
+    assert_bits_equal(t2n(torch.cat(parts, dim=2))[0], g["V_zone_a"])
+
+
+def test_contract_violations_and_degenerate_inputs():
+    K = torch.randn(1, 2, 6, 8, device=DEV).half()
+    V = torch.randn(1, 2, 6, 8, device=DEV).half()
+    # no kept token -> empty layer (packing.py:860-861)
+    pl, tk, v16 = packing.build_packed_layer(K, V, torch.zeros(6, dtype=torch.long), torch.full((8,), 4))
+    assert tk == 0 and v16 is None and pl.T_eff == 0 and pl.K_4bit is None
+    # all kept tokens are v=16
+    pl, tk, v16 = packing.build_packed_layer(K, V, torch.full((6,), 16), torch.full((8,), 4))
+    assert tk == 6 and pl.T_eff == 0 and pl.V_2bit is None and torch.equal(v16, V)
+    with pytest.raises(ValueError):
+        packing.build_packed_layer(K, V, torch.full((6,), 4), torch.full((8,), 4),
+                                   defer_k_for_per_head_stack=True)          # packing.py:914-917
+    with pytest.raises(AssertionError):
+        packing.build_packed_layer(K, V, torch.full((6,), 4), torch.full((2, 8), 4))  # gqa_factor missing
+    with pytest.raises(ValueError):
+        packing.build_packed_cache(((K, V),), torch.full((6,), 4), torch.full((3, 8), 4), original_seq_len=6)
+    with pytest.raises(AssertionError):
+        packing.pack_k_mixed(K[0], torch.full((8,), 4))
+    # zero kept channels
+    out = packing.pack_k_mixed(K, torch.zeros(8, dtype=torch.long))
+    assert out[0] is None and out[1] is None and out[2] is None and out[3].shape == (1, 2, 1, 0)
+
+
+@pytest.mark.parametrize("cfg_idx,ctx", [(0, 512), (1, 700), (2, 384)])
+def test_config_shaped_layer_vs_oracle(cfg_idx, ctx):
+    """Per-head packing of a configuration-shaped layer (reduced context) is bit-identical to the oracle."""
+    cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, q = synth.layer_data(cfg, 0, "cpu", outliers=oc)
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), cfg.G)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, cfg.G)
+    assert_layers_equal(pl, ora)
+    assert_bits_equal(t2n(nvo), ora_nvo)

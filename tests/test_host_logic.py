@@ -1,0 +1,101 @@
+"""CPU-side checks: host planning logic, C-ABI symbol export, loud failure without a device."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from rdkv_amd import _lib, packing, synth
+from oracle import rdkv_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_k_plan_known_answer():
+    # hand-derived from the reference's test input (tests/test_blockwise_rdkv.py:122-127)
+    plan = packing._plan_k_channels([0, 2, 4, 8, 16, 2, 4, 8])
+    assert plan.ch_sort_idx == [1, 5, 2, 6, 3, 4, 7]
+    assert plan.counts == (2, 2, 3)
+    assert plan.padded == (4, 2, 3)
+    assert plan.perm_padded == [1, 5, 0, 0, 2, 6, 3, 4, 7]
+    assert plan.slot_channel == [1, 5, -1, -1, 2, 6, 3, 4, 7]
+    same = packing._plan_k_channels([0, 2, 4, 8, 16, 2, 4, 8], segment_counts=(2, 2, 3))
+    assert same == plan
+
+
+def test_k_plan_targets_and_contract_violations():
+    plan = packing._plan_k_channels([2, 0, 8, 4], sub_2_target=2, sub_4_target=2, n_ch_8_target=3)
+    assert plan.padded == (8, 4, 3)
+    assert plan.slot_channel == [0] + [-1] * 7 + [3] + [-1] * 3 + [2, -1, -1]
+    with pytest.raises(AssertionError):
+        packing._plan_k_channels([2, 2, 2, 2, 2], sub_2_target=1)        # needs 2 bytes
+    with pytest.raises(AssertionError):
+        packing._plan_k_channels([8, 8], n_ch_8_target=1)
+    with pytest.raises(AssertionError):
+        packing._plan_k_channels([2, 4, 8], segment_counts=(1, 1, 2))    # packing.py:260
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_k_plan_matches_oracle(seed):
+    rng = np.random.default_rng(seed)
+    kb = rng.choice([0, 2, 4, 8, 16], size=32)
+    K = rng.standard_normal((1, 1, 5, 32)).astype(np.float16)
+    ref = O.pack_k_mixed(K, kb)
+    plan = packing._plan_k_channels(kb.tolist())
+    assert plan.ch_sort_idx == ref[5].tolist()
+    assert plan.perm_padded == ref[6].tolist()
+    assert plan.counts == ref[7]
+
+
+def test_header_symbols_exported():
+    hdr = open(os.path.join(ROOT, "include", "rdkv.h")).read()
+    hdr = re.sub(r"/\*.*?\*/", "", hdr, flags=re.S)
+    declared = set(re.findall(r"\b(rdkv_[a-z0-9_]+)\s*\(", hdr))
+    assert declared, "no declarations parsed"
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.rdkv_version() >= 100
+
+
+def test_no_cpu_fallback():
+    x = torch.zeros(2, 8, dtype=torch.uint8)
+    from rdkv_amd import bitpack
+    with pytest.raises(RuntimeError):
+        bitpack.transfer_8bit_to_2bit_batchwise(x)
+    with pytest.raises(RuntimeError):
+        packing.quantize_and_pack(torch.zeros(1, 1, 4, 8, dtype=torch.float16), 4, 3)
+
+
+def test_argument_errors_without_device_work():
+    lib = _lib.load()
+    assert lib.rdkv_bitpack2(None, None, 1, 6, None) == _lib.RDKV_EINVAL
+    assert b"multiple of 4" in lib.rdkv_last_error()
+    with pytest.raises(AssertionError):
+        _lib.check(lib.rdkv_quantize_rows(None, 0, None, 1, 128, 3, 1, None, None, None, None))
+
+
+def test_product_does_not_import_oracle():
+    pkg = os.path.join(ROOT, "rdkv_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith(".py"):
+                for line in open(os.path.join(dirpath, f)):
+                    if re.match(r"\s*(from|import)\s", line):
+                        assert "oracle" not in line, (f, line)
+
+
+def test_synth_allocations():
+    cfg = synth.CONFIGS[0]
+    vb, kb, oc = synth.head_allocation(cfg, 0, 3)
+    T = cfg.context
+    assert [(vb == b).sum() for b in (0, 2, 4, 8, 16)] == [821, 819, 1228, 819, 409]
+    assert [(kb == b).sum() for b in (2, 4, 8)] == [16, 32, 16] and (kb > 0).sum() == 64
+    assert all(kb[c] > 0 for c in oc)
+    cfg1 = synth.scaled(synth.CONFIGS[1], context=512, layers=2)
+    vb, kb, _ = synth.head_allocation(cfg1, 1, 2)
+    assert vb.shape == (512,) and (kb > 0).sum() == 64
+    vb2, kb2, _ = synth.head_allocation(cfg1, 1, 2)
+    assert np.array_equal(vb, vb2) and np.array_equal(kb, kb2)
