@@ -121,6 +121,66 @@ int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, int H_kv,
                         float *out, int64_t out_stride_h,
                         void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- streaming format + fused flash-decoding kernel ------------------------------------
+ * No counterpart in the reference as an interface: it replaces the sequence
+ * k_mixed_qk_dot -> +softmax_mask -> softmax -> v_dequant_weighted_sum_dispatch of
+ * fast_decode.py:1707-1768 by one pass over a re-laid-out copy of the packed layer.
+ *
+ * A "unit" is one (sequence, layer, KV head).  Its tokens are ordered by V class
+ * (2-bit, 4-bit, 8-bit, fp16 zone B), each class padded to whole 64-token tiles.  Per unit
+ * the blob holds K tiles (64 tokens x R dwords, R = d8+d4+d2), V tiles per class
+ * (2/4/8/16 KiB), per-token (scale,zp) fp16 pairs and a per-slot table for the query side.
+ * See rdkv_amd/csrc/stream_format.h for the exact bit placement. */
+typedef struct RdkvUnit {
+  uint64_t k_off;        /* byte offset of the unit's K tiles in the blob (256 B aligned)     */
+  uint64_t v_off[4];     /* byte offsets of the V tiles of class 2-bit, 4-bit, 8-bit, fp16    */
+  uint64_t sz_off;       /* byte offset of per-token {scale,zp} fp16 pairs (quantized tiles)  */
+  uint64_t qtab_off;     /* byte offset of the slot table: 4*(d8+2*d4+4*d2) x RdkvSlot        */
+  int32_t  n_tok[4];     /* tokens per class                                                   */
+  int32_t  d8, d4, d2;   /* K row dwords holding 8-, 4- and 2-bit channel fields              */
+  int32_t  q_row;        /* first query/output row of this unit (G consecutive rows)          */
+  int32_t  work_begin;   /* first work item / partial slot of this unit                       */
+  int32_t  work_count;   /* number of work items of this unit                                  */
+} RdkvUnit;
+
+typedef struct RdkvSlot {   /* one K channel slot in MFMA consumption order */
+  uint16_t channel;         /* original channel index of q to multiply with                */
+  uint16_t scale_f16;       /* per-channel scale (0 for pad slots)                          */
+  uint16_t zp_f16;          /* per-channel zero-point                                        */
+  uint16_t reserved;
+} RdkvSlot;
+
+typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgroup */
+  int32_t unit, tile_begin, tile_end, reserved;
+} RdkvWork;
+
+/* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.
+ * src_slot: int16 [H_kv][n_slots_max] = for each stream slot the index of the source channel
+ * in the padded sorted order of K_ch_scale (-1 = pad slot).  units: the layer's H_kv
+ * descriptors (device).  n2p/n4p: padded 2-/4-bit channel counts of the source layout. */
+int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
+                               const uint8_t *K4, int64_t k4_stride_h, int64_t k4_stride_t,
+                               const uint8_t *K8, int64_t k8_stride_h, int64_t k8_stride_t,
+                               int n2p, int n4p,
+                               const uint8_t *V2, int64_t v2_stride_h,
+                               const uint8_t *V4, int64_t v4_stride_h,
+                               const uint8_t *V8, int64_t v8_stride_h,
+                               const void *vscale_f16, const void *vzp_f16, int64_t vs_stride_h,
+                               const void *V16_f16, int64_t v16_stride_h, int64_t max_T_v,
+                               const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
+                               int H_kv, uint8_t *blob, void *stream);
+
+/* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
+ * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit
+ * without tokens), so callers can merge further zones exactly.  G = query heads per KV head
+ * (1..8).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes. */
+int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G);
+int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                      const RdkvWork *work, int n_work,
+                      const void *q, int q_dtype, int64_t q_stride_row, int G,
+                      float *out, int64_t out_stride_row, float *lse,
+                      void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,240 @@
+"""Streaming KV format + fused flash-decoding entry point.
+
+``build_stream_cache`` re-lays packed layers (the reference's padded ``PackedKVLayer`` +
+``new_v_only``) into contiguous per-(layer, KV head) blobs that the fused HIP kernel streams
+with 16-byte loads: ragged per head (no max-over-heads padding, so no softmax mask is
+needed), K rows as whole dwords per bit-width, V tiles in matrix-core operand order, and a
+per-unit slot table that carries the query-side channel permutation and the per-channel
+scale / zero-point.  ``decode_attn_fused`` then replaces the K-scores -> mask -> softmax ->
+V-sum sequence of the reference's decode step (obkv_accel/fast_decode.py:1707-1768) with one
+launch for any number of layers / sequences and returns the output together with the
+log-sum-exp, so the small fp32 zone of decode-appended tokens can be merged exactly.
+
+The format is immutable: it is built once for a frozen prompt cache.  Callers that overwrite
+packed tensors in place keep using the padded-layout entry points.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+from .packing import PackedKVLayer, _seg_padded_len
+
+TILE = 64
+V_TILE_BYTES = (2048, 4096, 8192, 16384)       # 2-bit, 4-bit, 8-bit, fp16 tiles of 64 tokens
+MAX_STEPS = 36
+
+UNIT_DTYPE = np.dtype([
+    ("k_off", "<u8"), ("v_off", "<u8", (4,)), ("sz_off", "<u8"), ("qtab_off", "<u8"),
+    ("n_tok", "<i4", (4,)), ("d8", "<i4"), ("d4", "<i4"), ("d2", "<i4"),
+    ("q_row", "<i4"), ("work_begin", "<i4"), ("work_count", "<i4")], align=True)
+SLOT_DTYPE = np.dtype([("channel", "<u2"), ("scale", "<u2"), ("zp", "<u2"), ("reserved", "<u2")])
+WORK_DTYPE = np.dtype([("unit", "<i4"), ("tile_begin", "<i4"), ("tile_end", "<i4"), ("reserved", "<i4")])
+assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.itemsize == 16
+
+
+
+def _align(x: int, a: int = 256) -> int:
+    return -(-x // a) * a
+
+
+def slot_plan(c2: int, c4: int, c8: int, n2p: int, n4p: int):
+    """Stream slot order of one head: 8-bit channels first, then 4-bit, then 2-bit, each padded
+    to whole dwords (4 / 8 / 16 channels).  Returns (d8, d4, d2, src) where src[slot] is the
+    channel's index in the source layer's padded sorted order ([2-bit | 4-bit | 8-bit],
+    obkv_accel/packing.py:364-388) or -1 for a pad slot."""
+    d8, d4, d2 = -(-c8 // 4), -(-c4 // 8), -(-c2 // 16)
+    src = []
+    src += [n2p + n4p + i for i in range(c8)] + [-1] * (4 * d8 - c8)
+    src += [n2p + i for i in range(c4)] + [-1] * (8 * d4 - c4)
+    src += list(range(c2)) + [-1] * (16 * d2 - c2)
+    return d8, d4, d2, src
+
+
+@dataclass
+class StreamCache:
+    blobs: List[torch.Tensor]            # device byte buffers (offsets in ``units`` are absolute addresses)
+    units: torch.Tensor                  # device bytes of RdkvUnit[n_units]
+    work: torch.Tensor                   # device bytes of RdkvWork[n_work]
+    units_host: np.ndarray
+    work_host: np.ndarray
+    n_units: int
+    n_work: int
+    G: int
+    rows: int                            # query / output rows = groups * H_q
+    stream_bytes: int                    # bytes the fused kernel reads from the blobs per step
+    algorithmic_bytes: int               # unpadded bytes (reference accounting) incl. q and out
+
+    @property
+    def device(self):
+        return self.units.device
+
+
+def _layer_counts(pl: PackedKVLayer, H_kv: int):
+    """Per-head (n2,n4,n8,n16) tokens and (c2,c4,c8) channels of a packed layer."""
+    if pl.seg_bounds_per_head is not None:
+        vb = pl.seg_bounds_per_head.detach().cpu().tolist()
+        n16 = pl.n_v16_per_head.detach().cpu().tolist() if pl.n_v16_per_head is not None else [0] * H_kv
+    else:
+        vb = [list(pl.seg_bounds)] * H_kv
+        n16 = [int(pl.n_v16)] * H_kv
+    if pl.K_ch_seg_bounds_per_head is not None:
+        kb = pl.K_ch_seg_bounds_per_head.detach().cpu().tolist()
+    else:
+        kb = [list(pl.K_ch_seg_bounds)] * H_kv
+    return [tuple(int(x) for x in v) + (int(n),) for v, n in zip(vb, n16)], [tuple(int(x) for x in k) for k in kb]
+
+
+def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
+                       work_bytes: int = 256 * 1024) -> StreamCache:
+    """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
+    layer)) into the streaming format.  Query/output row of entry g, query head hq is
+    ``g * H_q + hq``.  ``work_bytes`` is the target number of streamed bytes per workgroup."""
+    lib = _lib.load()
+    dev = _lib.require_device(layers[0][0].K_ch_scale)
+    stream = _lib.stream_of(dev)
+    units_all, work_all, blobs = [], [], []
+    stream_bytes = algo_bytes = 0
+    n_groups = len(layers)
+    H_q = None
+    for gi, (pl, nvo) in enumerate(layers):
+        H_kv = pl.K_ch_scale.shape[1]
+        H_q = H_kv * G
+        tok, ch = _layer_counts(pl, H_kv)
+        m2, m4, m8 = (int(v) for v in pl.K_ch_seg_bounds)
+        n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
+        Dp = n2p + n4p + m8
+        scale_h = pl.K_ch_scale.reshape(H_kv, Dp).detach().cpu().numpy().view(np.uint16)
+        zp_h = pl.K_ch_zp.reshape(H_kv, Dp).detach().cpu().numpy().view(np.uint16)
+        if pl.K_ch_perm_padded_idx_per_head is not None:
+            perm_h = pl.K_ch_perm_padded_idx_per_head.detach().cpu().numpy()
+        else:
+            perm_h = np.broadcast_to(pl.K_ch_perm_padded_idx.detach().cpu().numpy(), (H_kv, Dp))
+        units = np.zeros(H_kv, dtype=UNIT_DTYPE)
+        src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
+        qtabs = []
+        off = 0
+        for h in range(H_kv):
+            n_tok = tok[h]
+            c2, c4, c8 = ch[h]
+            d8, d4, d2, src = slot_plan(c2, c4, c8, n2p, n4p)
+            steps = d8 + 2 * d4 + 4 * d2
+            assert steps <= MAX_STEPS, f"{steps} channel steps exceed {MAX_STEPS}"
+            src_tab[h, :len(src)] = src
+            qt = np.zeros(len(src), dtype=SLOT_DTYPE)
+            for s, r in enumerate(src):
+                if r >= 0:
+                    qt[s] = (int(perm_h[h, r]), int(scale_h[h, r]), int(zp_h[h, r]), 0)
+            qtabs.append(qt)
+            tiles = [-(-n // TILE) for n in n_tok]
+            R = d8 + d4 + d2
+            u = units[h]
+            u["n_tok"] = n_tok
+            u["d8"], u["d4"], u["d2"] = d8, d4, d2
+            u["q_row"] = gi * H_q + h * G
+            u["k_off"] = off
+            off = _align(off + sum(tiles) * TILE * 4 * R)
+            for c in range(4):
+                u["v_off"][c] = off
+                off = _align(off + tiles[c] * V_TILE_BYTES[c])
+            u["sz_off"] = off
+            off = _align(off + sum(tiles[:3]) * TILE * 4)
+            u["qtab_off"] = off
+            off = _align(off + qt.nbytes)
+            # accounting
+            stream_bytes += (sum(tiles) * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
+                             + sum(tiles[:3]) * TILE * 4 + qt.nbytes)
+            row = -(-c2 // 4) + -(-c4 // 2) + c8
+            algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
+                           + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
+                           + 256 * n_tok[3])
+            # work items: runs of tiles of about work_bytes streamed bytes
+            costs = []
+            for c in range(4):
+                costs += [TILE * 4 * R + V_TILE_BYTES[c] + (TILE * 4 if c < 3 else 0)] * tiles[c]
+            u["work_begin"] = len(work_all)
+            t0, acc = 0, 0
+            for t, cst in enumerate(costs):
+                acc += cst
+                if acc >= work_bytes or t == len(costs) - 1:
+                    work_all.append((len(units_all) + h, t0, t + 1, 0))
+                    t0, acc = t + 1, 0
+            u["work_count"] = len(work_all) - int(u["work_begin"])
+        blob = torch.zeros(max(off, 256), dtype=torch.uint8, device=dev)
+        base = blob.data_ptr()
+        assert base % 256 == 0
+        for h in range(H_kv):
+            qoff = int(units[h]["qtab_off"])
+            if qtabs[h].nbytes:
+                blob[qoff:qoff + qtabs[h].nbytes] = torch.from_numpy(qtabs[h].view(np.uint8).copy()).to(dev)
+        rel_units = torch.from_numpy(units.view(np.uint8).copy()).to(dev)
+        src_dev = torch.from_numpy(src_tab).to(dev)
+
+        def seg3(t):
+            if t is None or t.numel() == 0:
+                return None, 0, 0
+            t = t.squeeze(0) if t.dim() == 4 else t
+            t = t if t.is_contiguous() else t.contiguous()
+            return t, t.stride(0), t.stride(1)
+
+        K2, k2h, k2t = seg3(pl.K_2bit)
+        K4, k4h, k4t = seg3(pl.K_4bit)
+        K8, k8h, k8t = seg3(pl.K_8bit)
+        V2, v2h, _ = seg3(pl.V_2bit)
+        V4, v4h, _ = seg3(pl.V_4bit)
+        V8, v8h, _ = seg3(pl.V_8bit)
+        vs = pl.V_scale.reshape(H_kv, -1).contiguous()
+        vz = pl.V_zp.reshape(H_kv, -1).contiguous()
+        V16, v16h, _ = seg3(nvo)
+        _lib.check(lib.rdkv_stream_relayout_layer(
+            _lib.ptr(K2), k2h, k2t, _lib.ptr(K4), k4h, k4t, _lib.ptr(K8), k8h, k8t, n2p, n4p,
+            _lib.ptr(V2), v2h, _lib.ptr(V4), v4h, _lib.ptr(V8), v8h,
+            _lib.ptr(vs), _lib.ptr(vz), vs.stride(0) if vs.numel() else 0,
+            _lib.ptr(V16), v16h, int(pl.T_eff),
+            rel_units.data_ptr(), src_dev.data_ptr(), src_tab.shape[1], H_kv, blob.data_ptr(), stream))
+        # kernel-side descriptors carry absolute addresses
+        for name in ("k_off", "sz_off", "qtab_off"):
+            units[name] += base
+        units["v_off"] += base
+        units_all.extend(units)
+        blobs.append(blob)
+        # keep the temporaries alive until the relayout kernel has run
+        torch.cuda.current_stream(dev).synchronize()
+    units_np = np.array(units_all, dtype=UNIT_DTYPE)
+    work_np = np.array(work_all, dtype=WORK_DTYPE) if work_all else np.zeros(0, dtype=WORK_DTYPE)
+    rows = n_groups * H_q
+    algo_bytes += rows * 128 * 2 + rows * 128 * 4
+    units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
+    work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
+        16, dtype=torch.uint8, device=dev)
+    return StreamCache(blobs=blobs, units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
+                       n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
+                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(algo_bytes))
+
+
+def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
+                      lse: Optional[torch.Tensor] = None):
+    """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
+    rotated); returns (out fp32 [rows,128], lse fp32 [rows]).  Graph-capturable once the
+    workspace exists (first call)."""
+    lib = _lib.load()
+    dev = _lib.require_device(q)
+    assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
+    if q.dtype not in _lib.DTYPE_CODE:
+        q = q.float()
+    if out is None:
+        out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
+    if lse is None:
+        lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
+    assert out.dtype == torch.float32 and out.stride(1) == 1 and lse.dtype == torch.float32 and lse.is_contiguous()
+    need = lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G)
+    ws = _lib.workspace(dev, need)
+    _lib.check(lib.rdkv_decode_fused(
+        None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
+        out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
+    return out, lse
