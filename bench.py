@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Benchmark of the packed decode-attention hot path on one MI355X.
+
+A "step" is one decode step of the attention hot path over every layer of the workload:
+the fused flash-decoding kernel reads the whole packed cache (all layers, all KV heads) once
+for one query per layer and writes out [L*H_q,128] + lse.  Inputs are synthetic, seeded, and
+resident in HBM before the timed region.  Default workload: configuration 1 (Llama-3.1-8B
+shapes, 32 layers, 32k context, per-head Dirichlet bit allocation).
+
+Prints ONE JSON line (see README / DESIGN for the fields).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--config", type=int, default=1, help="workload configuration 0..4 (default 1)")
+    ap.add_argument("--layers", type=int, default=None, help="override the layer count (debug)")
+    ap.add_argument("--context", type=int, default=None, help="override the context length (debug)")
+    ap.add_argument("--batch", type=int, default=None, help="override the batch (config 4)")
+    ap.add_argument("--work-kib", type=int, default=256, help="streamed KiB per workgroup")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--no-check", action="store_true")
+    return ap.parse_args()
+
+
+def time_region(fn, steps, torch):
+    """HIP-event time of `steps` back-to-back calls on the current stream (ms per call)."""
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the hot path shards by KV head / sequence "
+              "without any exchange; no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    from rdkv_amd import _lib, packing, stream_cache, synth
+
+    if not _lib.available():
+        import __graft_entry__
+        __graft_entry__.build()
+    assert torch.cuda.is_available(), "bench.py needs a HIP device"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    lib = _lib.load()
+
+    cfg = synth.CONFIGS[args.config]
+    cfg = synth.scaled(cfg, context=args.context, layers=args.layers, batch=args.batch)
+    t_build = time.time()
+    groups = []          # (packed layer, new_v_only) per (sequence, layer)
+    keep_first = None    # layer 0 of sequence 0: inputs kept for the CPU baseline / checks / dense run
+    for seq in range(cfg.batch):
+        for layer in range(cfg.layers):
+            vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
+            K, V, q = synth.layer_data(cfg, layer, dev, seq, outliers=oc)
+            pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+            groups.append((pl, nvo, q))
+            if keep_first is None:
+                keep_first = (K, V, q, pl, nvo)
+            del K, V
+    qs = torch.cat([g[2] for g in groups]).contiguous()
+    cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
+                                            work_bytes=args.work_kib * 1024)
+    padded_bytes = 0
+    first_pl, first_nvo = groups[0][0], groups[0][1]
+    del groups
+    torch.cuda.empty_cache()
+    torch.cuda.synchronize()
+    t_build = time.time() - t_build
+    n_groups = cfg.batch * cfg.layers
+
+    out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
+    lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
+
+    def step():
+        stream_cache.decode_attn_fused(cache, qs, out, lse)
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    ms_step = time_region(step, args.steps, torch)
+
+    # dominant kernel alone (streaming kernel without the merge launch)
+    ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
+    stream = _lib.stream_of(dev)
+
+    def partials_only():
+        _lib.check(lib.rdkv_decode_fused_partials(
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, ws.data_ptr(), ws.numel(), stream))
+
+    partials_only()
+    ms_kernel = time_region(partials_only, args.steps, torch)
+
+    algo = cache.algorithmic_bytes
+    gbps = algo / (ms_step * 1e-3) / 1e9
+    kernel_gbps = algo / (ms_kernel * 1e-3) / 1e9
+
+    # ---- correctness of what was timed (layer 0 against the CPU oracle) -------------------
+    check = None
+    cpu_base = None
+    if not (args.no_check and args.no_cpu_baseline):
+        from oracle import rdkv_oracle as O
+        import dataclasses
+        kw = {}
+        for f in dataclasses.fields(O.PackedKVLayer):
+            v = getattr(first_pl, f.name)
+            kw[f.name] = v.detach().cpu().numpy() if torch.is_tensor(v) else v
+        ora = O.PackedKVLayer(**kw)
+        ora_nvo = first_nvo.cpu().numpy() if first_nvo is not None else None
+        q0 = qs[:cfg.H_q].cpu().numpy()
+        reps = []
+        for i in range(1 if args.no_cpu_baseline else 4):
+            t0 = time.perf_counter()
+            exp_out, exp_lse, _ = O.decode_attn_ref(q0, ora, ora_nvo)
+            reps.append(time.perf_counter() - t0)
+        got = out[:cfg.H_q].cpu().numpy()
+        err = float(np.abs(got - exp_out).max())
+        check = {"layer0_max_abs_err": err, "layer0_ref_max_abs": float(np.abs(exp_out).max()),
+                 "within_tolerance": bool(err <= 2e-3 and err <= 1e-2 * np.abs(exp_out).max())}
+        if not args.no_cpu_baseline:
+            t_cpu = float(np.median(reps[1:]))
+            layer_bytes = O.algorithmic_bytes(ora, cfg.H_q)
+            cpu_base = {"value": layer_bytes / t_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                        "sample": f"NumPy dequantize-then-attend oracle on layer 0 of the workload "
+                                  f"({layer_bytes} algorithmic bytes), 1 warm-up + 3 repeats, median",
+                        "ms_per_layer": t_cpu * 1e3, "host_cpus": os.cpu_count()}
+
+    result = {
+        "metric": "packed decode-attn achieved HBM GB/s (algorithmic bytes / step time)",
+        "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8/fp16 codes, fp32 accumulate", "data": "synthetic",
+        "us_per_step_per_layer": ms_step * 1e3 / n_groups,
+        "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
+        "config": {"workload": cfg.name, "config_index": cfg.index, "layers": cfg.layers, "batch": cfg.batch,
+                   "H_q": cfg.H_q, "H_kv": cfg.H_kv, "head_dim": cfg.D, "context": cfg.context,
+                   "token_budget_metadata": cfg.token_budget,
+                   "launch": "one fused launch + one merge launch per step over all layers",
+                   "class_fractions_apply_to": "context tokens",
+                   "algorithmic_bytes_per_step": algo, "algorithmic_bytes_per_layer": algo / n_groups,
+                   "streamed_bytes_per_step": cache.stream_bytes, "work_items": cache.n_work,
+                   "dense_fp16_bytes_per_layer": synth.dense_fp16_bytes(cfg),
+                   "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo,
+                   "build_seconds": t_build},
+        "roofline": {"bound": "hbm", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": kernel_gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "decode_fused_kernel", "ms_per_launch": ms_kernel,
+                     "algorithmic_bytes_per_launch": algo},
+        "cpu_baseline": cpu_base,
+        "check": check,
+    }
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -180,6 +180,16 @@ int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
                       const void *q, int q_dtype, int64_t q_stride_row, int G,
                       float *out, int64_t out_stride_row, float *lse,
                       void *workspace, int64_t workspace_bytes, void *stream);
+/* The two launches of rdkv_decode_fused as separate calls (same arguments): the streaming
+ * kernel that writes one partial (max, sum, 128 accumulators per head) per work item, and
+ * the fixed-order merge of a unit's partials into out / lse. */
+int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                               const RdkvWork *work, int n_work,
+                               const void *q, int q_dtype, int64_t q_stride_row, int G,
+                               void *workspace, int64_t workspace_bytes, void *stream);
+int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G,
+                            float *out, int64_t out_stride_row, float *lse,
+                            void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

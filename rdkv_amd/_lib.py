@@ -49,6 +49,8 @@ SIGNATURES = {
                                        P, P, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),
     "rdkv_decode_fused": (I, [P, P, I, P, I, P, I, L, I, P, L, P, P, L, P]),
+    "rdkv_decode_fused_partials": (I, [P, P, I, P, I, P, I, L, I, P, L, P]),
+    "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -417,33 +417,63 @@ RDKV_API int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G) {
   return (int64_t)n_work * G * kPartialStride * (int64_t)sizeof(float);
 }
 
+static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, const RdkvWork *work,
+                            int n_work, int G, void *workspace, int64_t workspace_bytes) {
+  RDKV_REQUIRE(n_units >= 0 && n_work >= 0, "%s: negative counts", fn);
+  RDKV_REQUIRE(G >= 1 && G <= 8, "%s: G=%d outside 1..8", fn, G);
+  RDKV_REQUIRE(n_units == 0 || units, "%s: null unit table", fn);
+  RDKV_REQUIRE(n_work == 0 || work, "%s: null work list", fn);
+  if (n_work > 0 && (!workspace || workspace_bytes < rdkv_decode_fused_workspace_bytes(n_work, G))) {
+    rdkv_set_error("%s: workspace of %lld bytes required", fn,
+                   (long long)rdkv_decode_fused_workspace_bytes(n_work, G));
+    return RDKV_EWORKSPACE;
+  }
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                                        const RdkvWork *work, int n_work, const void *q, int q_dtype,
+                                        int64_t q_stride_row, int G, void *workspace,
+                                        int64_t workspace_bytes, void *stream) {
+  int rc = check_fused_args("rdkv_decode_fused_partials", units, n_units, work, n_work, G, workspace,
+                            workspace_bytes);
+  if (rc != RDKV_OK) return rc;
+  RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "rdkv_decode_fused_partials: unknown q dtype %d", q_dtype);
+  if (n_work == 0) return RDKV_OK;
+  RDKV_REQUIRE(q, "rdkv_decode_fused_partials: null q");
+  hipStream_t s = (hipStream_t)stream;
+  float *partials = (float *)workspace;
+  if (G <= 4)
+    hipLaunchKernelGGL(decode_fused_kernel<1>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
+                       q_stride_row, G, partials);
+  else
+    hipLaunchKernelGGL(decode_fused_kernel<2>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
+                       q_stride_row, G, partials);
+  RDKV_CHECK_LAUNCH("rdkv_decode_fused_partials");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G, float *out,
+                                     int64_t out_stride_row, float *lse, void *workspace,
+                                     int64_t workspace_bytes, void *stream) {
+  int rc = check_fused_args("rdkv_decode_fused_merge", units, n_units, (const RdkvWork *)units, n_work, G,
+                            workspace, workspace_bytes);
+  if (rc != RDKV_OK) return rc;
+  if (n_units == 0) return RDKV_OK;
+  RDKV_REQUIRE(out, "rdkv_decode_fused_merge: null out");
+  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(128), 0, (hipStream_t)stream, units,
+                     (const float *)workspace, G, out, out_stride_row, lse);
+  RDKV_CHECK_LAUNCH("rdkv_decode_fused_merge");
+  return RDKV_OK;
+}
+
 RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units, const RdkvWork *work,
                                int n_work, const void *q, int q_dtype, int64_t q_stride_row, int G,
                                float *out, int64_t out_stride_row, float *lse, void *workspace,
                                int64_t workspace_bytes, void *stream) {
-  RDKV_REQUIRE(n_units >= 0 && n_work >= 0, "rdkv_decode_fused: negative counts");
-  RDKV_REQUIRE(G >= 1 && G <= 8, "rdkv_decode_fused: G=%d outside 1..8", G);
-  RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "rdkv_decode_fused: unknown q dtype %d", q_dtype);
-  if (n_units == 0) return RDKV_OK;
-  RDKV_REQUIRE(units && q && out, "rdkv_decode_fused: null pointer");
-  RDKV_REQUIRE(n_work == 0 || work, "rdkv_decode_fused: null work list");
-  if (n_work > 0 && (!workspace || workspace_bytes < rdkv_decode_fused_workspace_bytes(n_work, G))) {
-    rdkv_set_error("rdkv_decode_fused: workspace of %lld bytes required",
-                   (long long)rdkv_decode_fused_workspace_bytes(n_work, G));
-    return RDKV_EWORKSPACE;
-  }
-  hipStream_t s = (hipStream_t)stream;
-  float *partials = (float *)workspace;
-  if (n_work > 0) {
-    if (G <= 4)
-      hipLaunchKernelGGL(decode_fused_kernel<1>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
-                         q_stride_row, G, partials);
-    else
-      hipLaunchKernelGGL(decode_fused_kernel<2>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
-                         q_stride_row, G, partials);
-    RDKV_CHECK_LAUNCH("rdkv_decode_fused");
-  }
-  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(128), 0, s, units, partials, G, out, out_stride_row, lse);
-  RDKV_CHECK_LAUNCH("rdkv_decode_fused(merge)");
-  return RDKV_OK;
+  int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, q, q_dtype, q_stride_row, G,
+                                      workspace, workspace_bytes, stream);
+  if (rc != RDKV_OK) return rc;
+  return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
+                                 workspace_bytes, stream);
 }
