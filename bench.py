@@ -114,7 +114,7 @@ def main():
 
     def partials_only():
         _lib.check(lib.rdkv_decode_fused_partials(
-            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work, cache.max_row_dwords,
             qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, ws.data_ptr(), ws.numel(), stream))
 
     partials_only()

@@ -173,10 +173,11 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit
  * without tokens), so callers can merge further zones exactly.  G = query heads per KV head
- * (1..8).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes. */
+ * (1..8).  max_row_dwords = max over units of d8+d4+d2 (<= 32; selects the register budget of
+ * the kernel).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes. */
 int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G);
 int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                      const RdkvWork *work, int n_work,
+                      const RdkvWork *work, int n_work, int max_row_dwords,
                       const void *q, int q_dtype, int64_t q_stride_row, int G,
                       float *out, int64_t out_stride_row, float *lse,
                       void *workspace, int64_t workspace_bytes, void *stream);
@@ -184,12 +185,19 @@ int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
  * kernel that writes one partial (max, sum, 128 accumulators per head) per work item, and
  * the fixed-order merge of a unit's partials into out / lse. */
 int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                               const RdkvWork *work, int n_work,
+                               const RdkvWork *work, int n_work, int max_row_dwords,
                                const void *q, int q_dtype, int64_t q_stride_row, int G,
                                void *workspace, int64_t workspace_bytes, void *stream);
 int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G,
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);
+
+/* ---- measurement helpers (no counterpart in the reference) --------------------------------
+ * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
+ * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)
+ * and a read-only sweep in contiguous spans of span_bytes per workgroup (sink: >= 1 KiB). */
+int rdkv_probe_copy(const void *src, void *dst, int64_t bytes, void *stream);
+int rdkv_probe_read(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -79,23 +79,103 @@ struct Smem {
   float wo[kWaves][NH * 4][kD];
 };
 
-template <int NH>
+// Register image of the loads of one pipeline stage: the K row of the lane's token and the
+// {scale,zp} pairs of the lane's quad (needed by the first piece of a tile only) and one V
+// piece of up to 16 dwords per lane.
+template <int RMAX>
+struct StageRegs {
+  uint32_t k[RMAX];
+  uint4 sz;
+  uint4 v[4];
+};
+
+struct Cursor {  // wave-uniform position in the tile/piece sequence of this wavefront
+  int ti, cls, pc, npc, n_valid;
+  const uint8_t *vtile;  // the tile's V data (pointer derived from the kernel argument: global loads)
+  bool valid;
+};
+
+// Select by class without indexing an array (keeps everything in scalar registers).
+template <typename T>
+__device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
+  return c == 0 ? a0 : (c == 1 ? a1 : (c == 2 ? a2 : a3));
+}
+
+template <int NH, int RMAX>
 __global__ void __launch_bounds__(256)
 decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
                     const RdkvWork *__restrict__ work, const void *__restrict__ q, int q_dtype,
                     int64_t q_stride, int G, float *__restrict__ partials) {
   __shared__ Smem<NH> sm;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // the wavefront index is uniform; say so, or every tile-level decision becomes per-lane
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 3, lb = lane >> 2;
-  const RdkvWork wk = work[blockIdx.x];
-  const RdkvUnit u = units[wk.unit];
-  const int d8 = u.d8, d4 = u.d4, d2 = u.d2;
+  const RdkvWork *wkp = work + blockIdx.x;
+  const int tile_begin = wkp->tile_begin, tile_end = wkp->tile_end;
+  const RdkvUnit *up = units + wkp->unit;
+  const int d8 = up->d8, d4 = up->d4, d2 = up->d2;
   const int R = d8 + d4 + d2;
   const int NS = d8 + 2 * d4 + 4 * d2;
+  const int n0 = up->n_tok[0], n1 = up->n_tok[1], n2 = up->n_tok[2], n3 = up->n_tok[3];
+  const int ts1 = (n0 + RDKV_TILE - 1) / RDKV_TILE;
+  const int ts2 = ts1 + (n1 + RDKV_TILE - 1) / RDKV_TILE;
+  const int ts3 = ts2 + (n2 + RDKV_TILE - 1) / RDKV_TILE;
+  // keep every address as `blob + offset` so the loads stay in the global address space
+  const uint8_t *k_base = blob + up->k_off, *sz_base = blob + up->sz_off;
+  const uint8_t *v_base0 = blob + up->v_off[0], *v_base1 = blob + up->v_off[1];
+  const uint8_t *v_base2 = blob + up->v_off[2], *v_base3 = blob + up->v_off[3];
+  const uint8_t *qtab_base = blob + up->qtab_off;
+  const int q_row = up->q_row;
+  const int nchunk_full = R >> 2, wc_last = R & 3;
+
+  auto set_tile = [&](Cursor &c, int ti) {
+    c.ti = ti;
+    c.pc = 0;
+    c.valid = ti < tile_end;
+    const int cls = (ti >= ts1) + (ti >= ts2) + (ti >= ts3);
+    c.cls = cls;
+    const int tl = ti - sel4(cls, 0, ts1, ts2, ts3);
+    c.n_valid = sel4(cls, n0, n1, n2, n3) - tl * RDKV_TILE;  // tokens >= n_valid are padding
+    c.vtile = sel4(cls, v_base0, v_base1, v_base2, v_base3) + (uint64_t)tl * (uint64_t)(2048 << cls);
+    c.npc = cls < 2 ? 1 : (cls == 2 ? 2 : 4);  // V pieces of 16 dwords per lane (8 for 2-bit)
+  };
+  auto advance = [&](const Cursor &c) {
+    Cursor n = c;
+    if (c.pc + 1 < c.npc) n.pc = c.pc + 1;
+    else set_tile(n, c.ti + kWaves);
+    return n;
+  };
+  // Issue the global loads of one stage.  All addresses are wave-uniform base + lane offset.
+  // The number of load instructions per stage is fixed (unused K chunks / V slots re-read an
+  // address already being fetched, which the vector cache absorbs) so that the hardware load
+  // counter can be waited on precisely while the next stage's loads are still in flight.
+  const int nchunks = nchunk_full + (wc_last ? 1 : 0);
+  auto issue = [&](const Cursor &c, StageRegs<RMAX> &r) {
+    if (c.pc == 0) {
+      const uint8_t *ktile = k_base + (uint64_t)c.ti * (RDKV_TILE * 4) * R;
+#pragma unroll
+      for (int ch = 0; ch < RMAX / 4; ++ch) {
+        const int che = ch < nchunks ? ch : 0;
+        const int wce = che == nchunk_full ? wc_last : 4;
+        // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
+        // the next token (or the region that follows) and are never used
+        const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
+        r.k[4 * ch] = v.x; r.k[4 * ch + 1] = v.y; r.k[4 * ch + 2] = v.z; r.k[4 * ch + 3] = v.w;
+      }
+      r.sz = *reinterpret_cast<const uint4 *>(sz_base + (c.cls < 3 ? (uint64_t)c.ti * (RDKV_TILE * 4) + lb * 16 : 0));
+    }
+    const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
+    const int hi = c.cls != 0 ? 128 : 0;
+    r.v[0] = vt[0];
+    r.v[1] = vt[64];
+    r.v[2] = vt[hi];
+    r.v[3] = vt[hi + 64];
+  };
 
   // ---------------- prologue: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias ----------
   {
-    const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(blob + u.qtab_off);
+    const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(qtab_base);
     const int nslot = 4 * NS;
     for (int i = tid; i < nslot * NH * 4; i += 256) {
       const int slot = i % nslot, head = i / nslot;
@@ -103,7 +183,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       if (head < G) {
         const RdkvSlot s = tab[slot];
         const float sc = (float)__builtin_bit_cast(_Float16, s.scale_f16);
-        const float qv = load_qv(q, q_dtype, (int64_t)(u.q_row + head) * q_stride + s.channel);
+        const float qv = load_qv(q, q_dtype, (int64_t)(q_row + head) * q_stride + s.channel);
         v = (_Float16)(qv * sc * (kLog2eOverSqrtD * kQScale));
       }
       sm.qs[slot >> 2][head >> 2][head & 3][slot & 3] = v;
@@ -139,56 +219,21 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     }
   }
 
-  int tstart[4];
-  {
-    int nt = 0;
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      tstart[c] = nt;
-      nt += (u.n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
-    }
-  }
-  const int nchunk_full = R >> 2, wc_last = R & 3;
+  auto p_op = [&](int quad, int hg) -> half4_t {
+    return *reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]);
+  };
 
-  for (int ti = wk.tile_begin + wave; ti < wk.tile_end; ti += kWaves) {
-    int cls = 0;
-    if (ti >= tstart[1]) cls = 1;
-    if (ti >= tstart[2]) cls = 2;
-    if (ti >= tstart[3]) cls = 3;
-    const int tl = ti - tstart[cls];
-    const int n_valid = u.n_tok[cls] - tl * RDKV_TILE;  // > 0 ; tokens >= n_valid are padding
-
-    // ---- issue loads: K row (lane = token), scale/zp of the lane's quad, V tile ----------
-    const uint8_t *ktile = blob + u.k_off + (int64_t)ti * (RDKV_TILE * 4) * R;
-    uint32_t kr[32];
+  auto compute = [&](const Cursor &c, const StageRegs<RMAX> &r) {
+    if (c.pc == 0) {
+      // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
+      floatx4 sacc[NH];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-      if (c < nchunk_full) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(ktile + c * 1024 + lane * 16);
-        kr[4 * c] = v.x; kr[4 * c + 1] = v.y; kr[4 * c + 2] = v.z; kr[4 * c + 3] = v.w;
-      } else if (c == nchunk_full && wc_last) {
-        const uint32_t *p = reinterpret_cast<const uint32_t *>(ktile + c * 1024 + lane * 4 * wc_last);
-        kr[4 * c] = p[0];
-        kr[4 * c + 1] = wc_last > 1 ? p[1] : 0u;
-        kr[4 * c + 2] = wc_last > 2 ? p[2] : 0u;
-        kr[4 * c + 3] = 0u;
-      }
-    }
-    uint4 sz = make_uint4(0, 0, 0, 0);
-    if (cls < 3)
-      sz = *reinterpret_cast<const uint4 *>(blob + u.sz_off + (int64_t)ti * (RDKV_TILE * 4) + lb * 16);
-    const uint4 *vt = reinterpret_cast<const uint4 *>(blob + u.v_off[cls] + (int64_t)tl * rdkv_v_tile_bytes(cls)) + lane;
-
-    // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln ---------------------------
-    floatx4 sacc[NH];
-#pragma unroll
-    for (int hg = 0; hg < NH; ++hg) sacc[hg] = floatx4{0.f, 0.f, 0.f, 0.f};
-    {
+      for (int hg = 0; hg < NH; ++hg) sacc[hg] = floatx4{0.f, 0.f, 0.f, 0.f};
       int step = 0;
 #pragma unroll
-      for (int j = 0; j < 32; ++j) {
+      for (int j = 0; j < RMAX; ++j) {
         if (j < R) {
-          const uint32_t w = kr[j];
+          const uint32_t w = r.k[j];
           if (j < d8) {
             const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
@@ -216,76 +261,75 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
           }
         }
       }
-    }
-
-    // ---- online softmax (base-2 domain) ----------------------------------------------------
-    const float pscale = cls < 3 ? kPScaleQ : kPScaleH;
-    float sc4[4], zp4[4];
-    {
-      const uint32_t szw[4] = {sz.x, sz.y, sz.z, sz.w};
+      // ---- online softmax (base-2 domain) --------------------------------------------------
+      const int n_valid = c.n_valid;
+      const float pscale = c.cls < 3 ? kPScaleQ : kPScaleH;
+      float sc4[4], zp4[4];
+      {
+        const uint32_t szw[4] = {r.sz.x, r.sz.y, r.sz.z, r.sz.w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        sc4[j] = cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] & 0xffffu)) : 1.0f;
-        zp4[j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] >> 16));
+        for (int j = 0; j < 4; ++j) {
+          sc4[j] = c.cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] & 0xffffu)) : 1.0f;
+          zp4[j] = c.cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] >> 16)) : 0.0f;
+        }
       }
-    }
-    bool grew = false;
-    float s2[NH][4], m_new[NH];
-#pragma unroll
-    for (int hg = 0; hg < NH; ++hg) {
-      float mx = -INFINITY;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float s = sacc[hg][j] * kSBack - bias_own[hg];
-        s = (4 * lb + j < n_valid) ? s : -INFINITY;
-        s2[hg][j] = s;
-        mx = fmaxf(mx, s);
-      }
-      mx = quadcol_max(mx);
-      m_new[hg] = fmaxf(m_run[hg], mx);
-      grew = grew || (m_new[hg] > m_run[hg]);
-    }
-    if (__any(grew)) {  // wave-uniform: rescale the running state
+      bool grew = false;
+      float s2[NH][4], m_new[NH];
 #pragma unroll
       for (int hg = 0; hg < NH; ++hg) {
-        const float f_own = exp2f(m_run[hg] - m_new[hg]);  // 0 on the first tile (m_run = -inf)
-        l_run[hg] *= f_own;
-        zb_run[hg] *= f_own;
-        m_run[hg] = m_new[hg];
+        float mx = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float f = __shfl(f_own, r, 64);  // lane r holds head r's factor
+        for (int j = 0; j < 4; ++j) {
+          float sv = sacc[hg][j] * kSBack - bias_own[hg];
+          sv = (4 * lb + j < n_valid) ? sv : -INFINITY;
+          s2[hg][j] = sv;
+          mx = fmaxf(mx, sv);
+        }
+        mx = quadcol_max(mx);
+        m_new[hg] = fmaxf(m_run[hg], mx);
+        grew = grew || (m_new[hg] > m_run[hg]);
+      }
+      if (__any(grew)) {  // wave-uniform: rescale the running state
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
-            accq[hg][j][r] *= f;
-            acch[hg][j][r] *= f;
+        for (int hg = 0; hg < NH; ++hg) {
+          const float f_own = exp2f(m_run[hg] - m_new[hg]);  // 0 on the first tile (m_run = -inf)
+          l_run[hg] *= f_own;
+          zb_run[hg] *= f_own;
+          m_run[hg] = m_new[hg];
+#pragma unroll
+          for (int rr = 0; rr < 4; ++rr) {
+            const float f = __shfl(f_own, rr, 64);  // lane rr holds head rr's factor
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+              accq[hg][j][rr] *= f;
+              acch[hg][j][rr] *= f;
+            }
           }
         }
       }
-    }
 #pragma unroll
-    for (int hg = 0; hg < NH; ++hg) {
-      _Float16 ph[4];
-      float lsum = 0.0f, zsum = 0.0f;
+      for (int hg = 0; hg < NH; ++hg) {
+        _Float16 ph[4];
+        float lsum = 0.0f, zsum = 0.0f;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float p = exp2f(s2[hg][j] - m_run[hg]);  // masked tokens: exp2(-inf) = 0
-        lsum += p;
-        ph[j] = (_Float16)(p * sc4[j] * pscale);
-        zsum += (float)ph[j] * zp4[j];
+        for (int j = 0; j < 4; ++j) {
+          const float p = exp2f(s2[hg][j] - m_run[hg]);  // masked tokens: exp2(-inf) = 0
+          lsum += p;
+          ph[j] = (_Float16)(p * sc4[j] * pscale);
+          zsum += (float)ph[j] * zp4[j];
+        }
+        l_run[hg] += lsum;
+        zb_run[hg] += zsum;
+        *reinterpret_cast<half4_t *>(&sm.p[wave][lb][hg][ln][0]) = half4_t{ph[0], ph[1], ph[2], ph[3]};
       }
-      l_run[hg] += lsum;
-      zb_run[hg] += zsum;
-      *reinterpret_cast<half4_t *>(&sm.p[wave][lb][hg][ln][0]) = half4_t{ph[0], ph[1], ph[2], ph[3]};
+      __builtin_amdgcn_wave_barrier();
     }
-    __builtin_amdgcn_wave_barrier();
 
-    // ---- V side -----------------------------------------------------------------------------
-    if (cls == 0) {  // 2-bit: 8 dwords per lane, dword i = quads 2i, 2i+1
+    // ---- V side: one piece -------------------------------------------------------------------
+    if (c.cls == 0) {  // 2-bit: 8 dwords, dword i = quads 2i, 2i+1
 #pragma unroll
       for (int x = 0; x < 2; ++x) {
-        const uint4 v = vt[x * 64];
-        const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t vw[4] = {r.v[x].x, r.v[x].y, r.v[x].z, r.v[x].w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t w = vw[e];
@@ -293,59 +337,71 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 #pragma unroll
           for (int s = 0; s < 4; ++s) {
             const half4_t b = mk_op((w >> (4 * s)) & 0x00030003u, (w >> (4 * s + 2)) & 0x00030003u);
-            const int quad = 2 * i + (s >> 1), j = s & 1;
 #pragma unroll
             for (int hg = 0; hg < NH; ++hg)
-              accq[hg][j] = mfma(*reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]), b, accq[hg][j]);
+              accq[hg][s & 1] = mfma(p_op(2 * i + (s >> 1), hg), b, accq[hg][s & 1]);
           }
         }
       }
-    } else if (cls == 1) {  // 4-bit: 16 dwords per lane, dword i = quad i
+    } else if (c.cls == 1) {  // 4-bit: 16 dwords, dword i = quad i
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
-        const uint4 v = vt[x * 64];
-        const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+        const uint32_t vw[4] = {r.v[x].x, r.v[x].y, r.v[x].z, r.v[x].w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t w = vw[e];
-          const int quad = 4 * x + e;
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
             const half4_t b = mk_op((w >> (8 * s)) & 0x000F000Fu, (w >> (8 * s + 4)) & 0x000F000Fu);
 #pragma unroll
-            for (int hg = 0; hg < NH; ++hg)
-              accq[hg][s] = mfma(*reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]), b, accq[hg][s]);
+            for (int hg = 0; hg < NH; ++hg) accq[hg][s] = mfma(p_op(4 * x + e, hg), b, accq[hg][s]);
           }
         }
       }
-    } else if (cls == 2) {  // 8-bit: 32 dwords per lane, dword i = (quad i>>1, j = i&1)
+    } else if (c.cls == 2) {  // 8-bit: piece pc holds dwords 16*pc.., dword i = (quad i>>1, j = i&1)
+      const int q0 = 8 * c.pc;
 #pragma unroll
-      for (int x = 0; x < 8; ++x) {
-        const uint4 v = vt[x * 64];
-        const uint32_t vw[4] = {v.x, v.y, v.z, v.w};
+      for (int x = 0; x < 4; ++x) {
+        const uint32_t vw[4] = {r.v[x].x, r.v[x].y, r.v[x].z, r.v[x].w};
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t w = vw[e];
-          const int quad = 2 * x + (e >> 1), j = e & 1;
           const half4_t b = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
           for (int hg = 0; hg < NH; ++hg)
-            accq[hg][j] = mfma(*reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]), b, accq[hg][j]);
+            accq[hg][e & 1] = mfma(p_op(q0 + 2 * x + (e >> 1), hg), b, accq[hg][e & 1]);
         }
       }
-    } else {  // fp16: 64 dwords per lane, one 16-byte load per quad
+    } else {  // fp16: piece pc holds quads 4*pc .. 4*pc+3, one 16-byte load per quad
+      const int q0 = 4 * c.pc;
 #pragma unroll
-      for (int x = 0; x < 16; ++x) {
-        const uint4 v = vt[x * 64];
+      for (int x = 0; x < 4; ++x) {
 #pragma unroll
         for (int hg = 0; hg < NH; ++hg) {
-          const half4_t a = *reinterpret_cast<const half4_t *>(&sm.p[wave][x][hg][ln][0]);
-          acch[hg][0] = mfma(a, mk_op(v.x, v.y), acch[hg][0]);
-          acch[hg][1] = mfma(a, mk_op(v.z, v.w), acch[hg][1]);
+          const half4_t a = p_op(q0 + x, hg);
+          acch[hg][0] = mfma(a, mk_op(r.v[x].x, r.v[x].y), acch[hg][0]);
+          acch[hg][1] = mfma(a, mk_op(r.v[x].z, r.v[x].w), acch[hg][1]);
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();
+  };
+
+  // ---------------- software-pipelined main loop: loads of stage n+1 fly during stage n ----
+  {
+    StageRegs<RMAX> ra, rb;
+    Cursor c0;
+    set_tile(c0, tile_begin + wave);
+    if (c0.valid) issue(c0, ra);
+    while (c0.valid) {
+      const Cursor c1 = advance(c0);
+      if (c1.valid) issue(c1, rb);
+      compute(c0, ra);
+      if (!c1.valid) break;
+      const Cursor c2 = advance(c1);
+      if (c2.valid) issue(c2, ra);
+      compute(c1, rb);
+      c0 = c2;
+    }
   }
 
   // ---------------- merge the four wavefront states and write the partial -----------------
@@ -387,27 +443,28 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   }
 }
 
-// One workgroup (128 threads = channels) per unit; partials combined in index order.
+// One workgroup (128 threads = channels) per (unit, head); partials combined in index order.
 __global__ void __launch_bounds__(128)
 merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
   const RdkvUnit u = units[blockIdx.x];
-  const int d = threadIdx.x;
-  for (int h = 0; h < G; ++h) {
-    float M = -INFINITY;
-    for (int i = 0; i < u.work_count; ++i)
-      M = fmaxf(M, partials[((int64_t)(u.work_begin + i) * G + h) * kPartialStride + 128]);
-    float o = 0.0f, l = 0.0f;
-    for (int i = 0; i < u.work_count; ++i) {
-      const float *p = partials + ((int64_t)(u.work_begin + i) * G + h) * kPartialStride;
-      const float f = exp2f(p[128] - M);
-      o += f * p[d];
-      l += f * p[129];
-    }
-    const int64_t row = u.q_row + h;
-    out[row * out_stride + d] = u.work_count > 0 ? o / l : 0.0f;
-    if (lse && d == 0) lse[row] = u.work_count > 0 ? (M + log2f(l)) * kLn2 : -INFINITY;
+  const int h = blockIdx.y, d = threadIdx.x;
+  const int n = u.work_count;
+  const float *base = partials + ((int64_t)u.work_begin * G + h) * kPartialStride;
+  const int64_t pstride = (int64_t)G * kPartialStride;
+  float M = -INFINITY;
+  for (int i = 0; i < n; ++i) M = fmaxf(M, base[i * pstride + 128]);
+  float o = 0.0f, l = 0.0f;
+#pragma unroll 4
+  for (int i = 0; i < n; ++i) {
+    const float *p = base + i * pstride;
+    const float f = exp2f(p[128] - M);
+    o += f * p[d];
+    l += f * p[129];
   }
+  const int64_t row = u.q_row + h;
+  out[row * out_stride + d] = n > 0 ? o / l : 0.0f;
+  if (lse && d == 0) lse[row] = n > 0 ? (M + log2f(l)) * kLn2 : -INFINITY;
 }
 
 }  // namespace
@@ -432,23 +489,34 @@ static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, 
 }
 
 RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                                        const RdkvWork *work, int n_work, const void *q, int q_dtype,
-                                        int64_t q_stride_row, int G, void *workspace,
-                                        int64_t workspace_bytes, void *stream) {
+                                        const RdkvWork *work, int n_work, int max_row_dwords,
+                                        const void *q, int q_dtype, int64_t q_stride_row, int G,
+                                        void *workspace, int64_t workspace_bytes, void *stream) {
   int rc = check_fused_args("rdkv_decode_fused_partials", units, n_units, work, n_work, G, workspace,
                             workspace_bytes);
   if (rc != RDKV_OK) return rc;
   RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "rdkv_decode_fused_partials: unknown q dtype %d", q_dtype);
+  RDKV_REQUIRE(max_row_dwords >= 0 && max_row_dwords <= 32,
+               "rdkv_decode_fused_partials: max_row_dwords=%d outside 0..32", max_row_dwords);
   if (n_work == 0) return RDKV_OK;
   RDKV_REQUIRE(q, "rdkv_decode_fused_partials: null q");
   hipStream_t s = (hipStream_t)stream;
   float *partials = (float *)workspace;
-  if (G <= 4)
-    hipLaunchKernelGGL(decode_fused_kernel<1>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
-                       q_stride_row, G, partials);
-  else
-    hipLaunchKernelGGL(decode_fused_kernel<2>, dim3(n_work), dim3(256), 0, s, blob, units, work, q, q_dtype,
-                       q_stride_row, G, partials);
+#define RDKV_LAUNCH_FUSED(NH, RMAX)                                                                   \
+  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX>), dim3(n_work), dim3(256), 0, s, blob, units, work, q, \
+                     q_dtype, q_stride_row, G, partials)
+  if (G <= 4) {
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(1, 16);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(1, 20);
+    else RDKV_LAUNCH_FUSED(1, 32);
+  } else {
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(2, 12);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(2, 16);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(2, 20);
+    else RDKV_LAUNCH_FUSED(2, 32);
+  }
+#undef RDKV_LAUNCH_FUSED
   RDKV_CHECK_LAUNCH("rdkv_decode_fused_partials");
   return RDKV_OK;
 }
@@ -461,18 +529,18 @@ RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_w
   if (rc != RDKV_OK) return rc;
   if (n_units == 0) return RDKV_OK;
   RDKV_REQUIRE(out, "rdkv_decode_fused_merge: null out");
-  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(128), 0, (hipStream_t)stream, units,
+  hipLaunchKernelGGL(merge_kernel, dim3(n_units, G), dim3(128), 0, (hipStream_t)stream, units,
                      (const float *)workspace, G, out, out_stride_row, lse);
   RDKV_CHECK_LAUNCH("rdkv_decode_fused_merge");
   return RDKV_OK;
 }
 
 RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units, const RdkvWork *work,
-                               int n_work, const void *q, int q_dtype, int64_t q_stride_row, int G,
-                               float *out, int64_t out_stride_row, float *lse, void *workspace,
-                               int64_t workspace_bytes, void *stream) {
-  int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, q, q_dtype, q_stride_row, G,
-                                      workspace, workspace_bytes, stream);
+                               int n_work, int max_row_dwords, const void *q, int q_dtype,
+                               int64_t q_stride_row, int G, float *out, int64_t out_stride_row, float *lse,
+                               void *workspace, int64_t workspace_bytes, void *stream) {
+  int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, max_row_dwords, q, q_dtype,
+                                      q_stride_row, G, workspace, workspace_bytes, stream);
   if (rc != RDKV_OK) return rc;
   return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
                                  workspace_bytes, stream);

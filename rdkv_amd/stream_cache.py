@@ -68,6 +68,7 @@ class StreamCache:
     rows: int                            # query / output rows = groups * H_q
     stream_bytes: int                    # bytes the fused kernel reads from the blobs per step
     algorithmic_bytes: int               # unpadded bytes (reference accounting) incl. q and out
+    max_row_dwords: int = 32             # max over units of the K row length in dwords
 
     @property
     def device(self):
@@ -164,7 +165,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
                     work_all.append((len(units_all) + h, t0, t + 1, 0))
                     t0, acc = t + 1, 0
             u["work_count"] = len(work_all) - int(u["work_begin"])
-        blob = torch.zeros(max(off, 256), dtype=torch.uint8, device=dev)
+        blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
         assert base % 256 == 0
         for h in range(H_kv):
@@ -213,7 +214,9 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         16, dtype=torch.uint8, device=dev)
     return StreamCache(blobs=blobs, units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
                        n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
-                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(algo_bytes))
+                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(algo_bytes),
+                       max_row_dwords=int(max((int(u["d8"]) + int(u["d4"]) + int(u["d2"]) for u in units_np),
+                                              default=0)))
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
@@ -235,6 +238,6 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     ws = _lib.workspace(dev, need)
     _lib.check(lib.rdkv_decode_fused(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
+        cache.max_row_dwords, q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
         out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
     return out, lse
