@@ -120,6 +120,19 @@ def main():
     partials_only()
     ms_kernel = time_region(partials_only, args.steps, torch)
 
+    # plain copy kernel of known size (1 GiB in, 1 GiB out): reference launch for scaling the
+    # hardware traffic counters of a profiler run of this same command
+    probe_bytes = 1 << 30
+    probe_src = torch.empty(probe_bytes, dtype=torch.uint8, device=dev).random_(0, 255)
+    probe_dst = torch.empty_like(probe_src)
+    _lib.check(lib.rdkv_probe_copy(probe_src.data_ptr(), probe_dst.data_ptr(), probe_bytes, stream))
+    ms_copy = time_region(lambda: _lib.check(lib.rdkv_probe_copy(
+        probe_src.data_ptr(), probe_dst.data_ptr(), probe_bytes, stream)), 5, torch)
+    sink = torch.zeros(1024, dtype=torch.uint8, device=dev)
+    ms_read = time_region(lambda: _lib.check(lib.rdkv_probe_read(
+        probe_src.data_ptr(), probe_bytes, 256 * 1024, sink.data_ptr(), stream)), 5, torch)
+    del probe_src, probe_dst
+
     algo = cache.algorithmic_bytes
     gbps = algo / (ms_step * 1e-3) / 1e9
     kernel_gbps = algo / (ms_kernel * 1e-3) / 1e9
@@ -174,7 +187,10 @@ def main():
         "roofline": {"bound": "hbm", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": kernel_gbps / HBM_PEAK_GBPS, "traffic": None,
                      "kernel": "decode_fused_kernel", "ms_per_launch": ms_kernel,
-                     "algorithmic_bytes_per_launch": algo},
+                     "algorithmic_bytes_per_launch": algo,
+                     "streamed_bytes_per_launch": cache.stream_bytes,
+                     "device_read_ceiling_GBps": probe_bytes / (ms_read * 1e-3) / 1e9,
+                     "device_copy_GBps_read_plus_write": 2 * probe_bytes / (ms_copy * 1e-3) / 1e9},
         "cpu_baseline": cpu_base,
         "check": check,
     }

@@ -174,7 +174,9 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit
  * without tokens), so callers can merge further zones exactly.  G = query heads per KV head
  * (1..8).  max_row_dwords = max over units of d8+d4+d2 (<= 32; selects the register budget of
- * the kernel).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes. */
+ * the kernel).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes.
+ * Two launches: the streaming kernel writes one partial per work item, a small kernel merges
+ * the partials of each unit in index order.  Calls that share a workspace must not overlap. */
 int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G);
 int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
                       const RdkvWork *work, int n_work, int max_row_dwords,

@@ -19,6 +19,8 @@
 #include "rdkv_common.h"
 #include "stream_format.h"
 
+#include <stdlib.h>
+
 namespace {
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -69,6 +71,71 @@ __device__ __forceinline__ float quadcol_max(float v) {
   return v;
 }
 
+// Combine the partials [work_begin, work_begin + n) of one unit in index order.
+// Combine the partials [work_begin, work_begin + n) of one unit in index order with a whole
+// workgroup.  The max / sum columns are staged in LDS first (scratch: 2 * kMergeMaxK * 8
+// floats) so that the accumulator loads of a thread are independent and overlap: the merge
+// costs about one memory latency instead of one per partial.
+constexpr int kMergeMaxK = 128;
+
+__device__ __forceinline__ void merge_unit(const float *partials, int work_begin, int n, int G, int q_row,
+                                           float *out, int64_t out_stride, float *lse, int tid, int nthreads,
+                                           float *scratch) {
+  const int64_t pstride = (int64_t)G * kPartialStride;
+  const float *base0 = partials + (int64_t)work_begin * pstride;
+  if (n <= kMergeMaxK) {
+    float *s_m = scratch, *s_l = scratch + kMergeMaxK * 8;
+    for (int i = tid; i < n * G; i += nthreads) {
+      const int k = i / G, h = i - k * G;
+      s_m[k * 8 + h] = *(base0 + k * pstride + h * kPartialStride + 128);
+      s_l[k * 8 + h] = *(base0 + k * pstride + h * kPartialStride + 129);
+    }
+    __syncthreads();
+    for (int i = tid; i < G * kD; i += nthreads) {
+      const int h = i >> 7, d = i & 127;
+      float M = -INFINITY;
+      for (int k = 0; k < n; ++k) M = fmaxf(M, s_m[k * 8 + h]);
+      float o = 0.0f, l = 0.0f;
+      const float *base = base0 + h * kPartialStride + d;
+      for (int k0 = 0; k0 < n; k0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = k0 + e < n ? *(base + (k0 + e) * pstride) : 0.0f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          if (k0 + e < n) {
+            const float mk = s_m[(k0 + e) * 8 + h];
+            const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
+            o += f * v[e];
+            l += f * s_l[(k0 + e) * 8 + h];
+          }
+        }
+      }
+      const int64_t row = q_row + h;
+      out[row * out_stride + d] = l > 0.0f ? o / l : 0.0f;  // a unit without tokens gives 0 / -inf
+      if (lse && d == 0) lse[row] = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+    }
+    return;
+  }
+  for (int i = tid; i < G * kD; i += nthreads) {  // very long units: plain two-pass loop
+    const int h = i >> 7, d = i & 127;
+    const float *base = base0 + h * kPartialStride;
+    float M = -INFINITY;
+    for (int k = 0; k < n; ++k) M = fmaxf(M, *(base + k * pstride + 128));
+    float o = 0.0f, l = 0.0f;
+    for (int k = 0; k < n; ++k) {
+      const float *p = base + k * pstride;
+      const float mk = *(p + 128);
+      const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
+      o += f * *(p + d);
+      l += f * *(p + 129);
+    }
+    const int64_t row = q_row + h;
+    out[row * out_stride + d] = l > 0.0f ? o / l : 0.0f;
+    if (lse && d == 0) lse[row] = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+  }
+}
+
 template <int NH>
 struct Smem {
   alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][4][4];   // [step][head group][head][k]
@@ -101,8 +168,8 @@ __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
   return c == 0 ? a0 : (c == 1 ? a1 : (c == 2 ? a2 : a3));
 }
 
-template <int NH, int RMAX>
-__global__ void __launch_bounds__(256)
+template <int NH, int RMAX, int WPE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
                     const RdkvWork *__restrict__ work, const void *__restrict__ q, int q_dtype,
                     int64_t q_stride, int G, float *__restrict__ partials) {
@@ -431,7 +498,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     float o = 0.0f, l = 0.0f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) {
-      const float f = exp2f(sm.wm[w][h] - M);  // idle wavefront: exp2(-inf - M) = 0
+      const float mw = sm.wm[w][h];
+      const float f = mw == -INFINITY ? 0.0f : exp2f(mw - M);  // idle wavefront contributes nothing
       o += f * sm.wo[w][h][d];
       l += f * sm.wl[w][h];
     }
@@ -443,28 +511,15 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   }
 }
 
-// One workgroup (128 threads = channels) per (unit, head); partials combined in index order.
-__global__ void __launch_bounds__(128)
+// One workgroup per unit combines its partials (second launch of a step).  Merging inside the
+// streaming kernel (last-arriver ticket with device-scope stores) was measured 7% slower.
+__global__ void __launch_bounds__(256)
 merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
-  const RdkvUnit u = units[blockIdx.x];
-  const int h = blockIdx.y, d = threadIdx.x;
-  const int n = u.work_count;
-  const float *base = partials + ((int64_t)u.work_begin * G + h) * kPartialStride;
-  const int64_t pstride = (int64_t)G * kPartialStride;
-  float M = -INFINITY;
-  for (int i = 0; i < n; ++i) M = fmaxf(M, base[i * pstride + 128]);
-  float o = 0.0f, l = 0.0f;
-#pragma unroll 4
-  for (int i = 0; i < n; ++i) {
-    const float *p = base + i * pstride;
-    const float f = exp2f(p[128] - M);
-    o += f * p[d];
-    l += f * p[129];
-  }
-  const int64_t row = u.q_row + h;
-  out[row * out_stride + d] = n > 0 ? o / l : 0.0f;
-  if (lse && d == 0) lse[row] = n > 0 ? (M + log2f(l)) * kLn2 : -INFINITY;
+  __shared__ float scratch[2 * kMergeMaxK * 8];
+  const RdkvUnit *u = units + blockIdx.x;
+  merge_unit(partials, u->work_begin, u->work_count, G, u->q_row, out, out_stride, lse, threadIdx.x, 256,
+                    scratch);
 }
 
 }  // namespace
@@ -488,23 +543,33 @@ static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, 
   return RDKV_OK;
 }
 
-RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                                        const RdkvWork *work, int n_work, int max_row_dwords,
-                                        const void *q, int q_dtype, int64_t q_stride_row, int G,
-                                        void *workspace, int64_t workspace_bytes, void *stream) {
-  int rc = check_fused_args("rdkv_decode_fused_partials", units, n_units, work, n_work, G, workspace,
-                            workspace_bytes);
+// Launch of the streaming kernel (writes one partial per work item).
+static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *units, int n_units,
+                        const RdkvWork *work, int n_work, int max_row_dwords, const void *q, int q_dtype,
+                        int64_t q_stride_row, int G, void *workspace, int64_t workspace_bytes, void *stream) {
+  int rc = check_fused_args(fn, units, n_units, work, n_work, G, workspace, workspace_bytes);
   if (rc != RDKV_OK) return rc;
-  RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "rdkv_decode_fused_partials: unknown q dtype %d", q_dtype);
-  RDKV_REQUIRE(max_row_dwords >= 0 && max_row_dwords <= 32,
-               "rdkv_decode_fused_partials: max_row_dwords=%d outside 0..32", max_row_dwords);
+  RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "%s: unknown q dtype %d", fn, q_dtype);
+  RDKV_REQUIRE(max_row_dwords >= 0 && max_row_dwords <= 32, "%s: max_row_dwords=%d outside 0..32", fn,
+               max_row_dwords);
   if (n_work == 0) return RDKV_OK;
-  RDKV_REQUIRE(q, "rdkv_decode_fused_partials: null q");
+  RDKV_REQUIRE(q, "%s: null q", fn);
   hipStream_t s = (hipStream_t)stream;
   float *partials = (float *)workspace;
-#define RDKV_LAUNCH_FUSED(NH, RMAX)                                                                   \
-  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX>), dim3(n_work), dim3(256), 0, s, blob, units, work, q, \
-                     q_dtype, q_stride_row, G, partials)
+  // occupancy target of the kernel variant (registers per lane); 3 wavefronts per SIMD measured best
+  static const int wpe = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 3;
+#define RDKV_LAUNCH_FUSED(NH, RMAX)                                                                        \
+  do {                                                                                                     \
+    if (wpe >= 4)                                                                                          \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 4>), dim3(n_work), dim3(256), 0, s, blob, units,   \
+                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+    else if (wpe == 3)                                                                                     \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 3>), dim3(n_work), dim3(256), 0, s, blob, units,   \
+                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+    else                                                                                                   \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 2>), dim3(n_work), dim3(256), 0, s, blob, units,   \
+                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+  } while (0)
   if (G <= 4) {
     if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12);
     else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(1, 16);
@@ -517,8 +582,16 @@ RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *uni
     else RDKV_LAUNCH_FUSED(2, 32);
   }
 #undef RDKV_LAUNCH_FUSED
-  RDKV_CHECK_LAUNCH("rdkv_decode_fused_partials");
+  RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
+}
+
+RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                                        const RdkvWork *work, int n_work, int max_row_dwords,
+                                        const void *q, int q_dtype, int64_t q_stride_row, int G,
+                                        void *workspace, int64_t workspace_bytes, void *stream) {
+  return launch_fused("rdkv_decode_fused_partials", blob, units, n_units, work, n_work, max_row_dwords, q,
+                      q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
 }
 
 RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G, float *out,
@@ -529,7 +602,7 @@ RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_w
   if (rc != RDKV_OK) return rc;
   if (n_units == 0) return RDKV_OK;
   RDKV_REQUIRE(out, "rdkv_decode_fused_merge: null out");
-  hipLaunchKernelGGL(merge_kernel, dim3(n_units, G), dim3(128), 0, (hipStream_t)stream, units,
+  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(256), 0, (hipStream_t)stream, units,
                      (const float *)workspace, G, out, out_stride_row, lse);
   RDKV_CHECK_LAUNCH("rdkv_decode_fused_merge");
   return RDKV_OK;

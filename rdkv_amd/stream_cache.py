@@ -164,6 +164,8 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
                 if acc >= work_bytes or t == len(costs) - 1:
                     work_all.append((len(units_all) + h, t0, t + 1, 0))
                     t0, acc = t + 1, 0
+            if not costs:                      # a unit without tokens still gets one (empty) work item
+                work_all.append((len(units_all) + h, 0, 0, 0))
             u["work_count"] = len(work_all) - int(u["work_begin"])
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
@@ -223,7 +225,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                       lse: Optional[torch.Tensor] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated); returns (out fp32 [rows,128], lse fp32 [rows]).  Graph-capturable once the
-    workspace exists (first call)."""
+    workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
     assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
