@@ -138,7 +138,7 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
 
 template <int NH>
 struct Smem {
-  alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][4][4];   // [step][head group][head][k]
+  alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][2][4][4];  // [step][head group][hi|lo][head][k]
   alignas(16) _Float16 p[kWaves][16][NH][4][4];        // [wave][quad][head group][head][k]
   float bias[NH * 4];
   float wm[kWaves][NH * 4];
@@ -246,14 +246,19 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     const int nslot = 4 * NS;
     for (int i = tid; i < nslot * NH * 4; i += 256) {
       const int slot = i % nslot, head = i / nslot;
-      _Float16 v = (_Float16)0.0f;
+      _Float16 hi = (_Float16)0.0f, lo = (_Float16)0.0f;
       if (head < G) {
         const RdkvSlot s = tab[slot];
         const float sc = (float)__builtin_bit_cast(_Float16, s.scale_f16);
         const float qv = load_qv(q, q_dtype, (int64_t)(q_row + head) * q_stride + s.channel);
-        v = (_Float16)(qv * sc * (kLog2eOverSqrtD * kQScale));
+        // two fp16 terms carry ~22 bits of q*scale: one fp16 alone loses the outlier channels'
+        // low bits and costs ~1e-3 in the scores
+        const float x = qv * sc * (kLog2eOverSqrtD * kQScale);
+        hi = (_Float16)x;
+        lo = (_Float16)(x - (float)hi);
       }
-      sm.qs[slot >> 2][head >> 2][head & 3][slot & 3] = v;
+      sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] = hi;
+      sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3] = lo;
     }
     __syncthreads();
     // bias[h] = sum_slot qs[h][slot] * zp[slot] / 2^8, one wavefront per head, fixed tree
@@ -261,7 +266,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       float b = 0.0f;
       for (int slot = lane; slot < nslot; slot += 64) {
         const float zp = (float)__builtin_bit_cast(_Float16, tab[slot].zp_f16);
-        b += (float)sm.qs[slot >> 2][head >> 2][head & 3][slot & 3] * zp;
+        b += ((float)sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] +
+              (float)sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3]) * zp;
       }
       b = rdkv_wave_sum(b);
       if (lane == 0) sm.bias[head] = b * (1.0f / kQScale);
@@ -304,16 +310,20 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
           if (j < d8) {
             const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
-            for (int hg = 0; hg < NH; ++hg)
-              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][ln][0]), sacc[hg]);
+            for (int hg = 0; hg < NH; ++hg) {
+              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][0][ln][0]), sacc[hg]);
+              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][1][ln][0]), sacc[hg]);
+            }
             step += 1;
           } else if (j < d8 + d4) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
               const half4_t a = mk_op((w >> (8 * s)) & 0x000F000Fu, (w >> (8 * s + 4)) & 0x000F000Fu);
 #pragma unroll
-              for (int hg = 0; hg < NH; ++hg)
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][ln][0]), sacc[hg]);
+              for (int hg = 0; hg < NH; ++hg) {
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][0][ln][0]), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][1][ln][0]), sacc[hg]);
+              }
             }
             step += 2;
           } else {
@@ -321,8 +331,10 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
             for (int s = 0; s < 4; ++s) {
               const half4_t a = mk_op((w >> (4 * s)) & 0x00030003u, (w >> (4 * s + 2)) & 0x00030003u);
 #pragma unroll
-              for (int hg = 0; hg < NH; ++hg)
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][ln][0]), sacc[hg]);
+              for (int hg = 0; hg < NH; ++hg) {
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][0][ln][0]), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][1][ln][0]), sacc[hg]);
+              }
             }
             step += 4;
           }

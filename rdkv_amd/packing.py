@@ -229,9 +229,9 @@ def pack_k_mixed(K: Tensor, k_bits: Tensor, *, sub_2_target: Optional[int] = Non
     def stack(i, width):
         if width == 0:
             return None
-        return torch.stack([hd[i] for hd in heads], 0).reshape(1, H, T, -1)
+        return torch.stack([hd[i] for hd in heads], 0).reshape(1, H, T, width)
 
-    K2, K4, K8 = stack(0, n2p), stack(1, n4p), stack(2, n8o)
+    K2, K4, K8 = stack(0, n2p // 4), stack(1, n4p // 2), stack(2, n8o)
     Dp = n2p + n4p + n8o
     if Dp:
         scale = torch.stack([hd[3] for hd in heads], 0).reshape(1, H, 1, Dp)
@@ -279,7 +279,7 @@ def pack_k_mixed_per_head(K: Tensor, k_bits_ph: Tensor):
     def stack(i, width):
         if width == 0:
             return None
-        return torch.stack([hd[i] for hd in heads], 0).reshape(1, H, T, -1)
+        return torch.stack([hd[i] for hd in heads], 0).reshape(1, H, T, width)
 
     K2, K4, K8 = stack(0, sub2), stack(1, sub4), stack(2, m8)
     if Dp:
