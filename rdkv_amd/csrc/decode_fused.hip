@@ -71,7 +71,6 @@ __device__ __forceinline__ float quadcol_max(float v) {
   return v;
 }
 
-// Combine the partials [work_begin, work_begin + n) of one unit in index order.
 // Combine the partials [work_begin, work_begin + n) of one unit in index order with a whole
 // workgroup.  The max / sum columns are staged in LDS first (scratch: 2 * kMergeMaxK * 8
 // floats) so that the accumulator loads of a thread are independent and overlap: the merge
@@ -146,13 +145,16 @@ struct Smem {
   float wo[kWaves][NH * 4][kD];
 };
 
-// Register image of the loads of one pipeline stage: the K row of the lane's token and the
-// {scale,zp} pairs of the lane's quad (needed by the first piece of a tile only) and one V
-// piece of up to 16 dwords per lane.
+// Register images of the loads in flight.  KRegs: the K row of the lane's token and the
+// {scale,zp} pairs of the lane's quad for one tile (single buffer: the next tile's row is
+// requested as soon as the current one has been consumed, a whole V phase ahead of its use).
+// VRegs: one V piece of up to 16 dwords per lane (two buffers, one stage ahead).
 template <int RMAX>
-struct StageRegs {
+struct KRegs {
   uint32_t k[RMAX];
   uint4 sz;
+};
+struct VRegs {
   uint4 v[4];
 };
 
@@ -218,20 +220,20 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // address already being fetched, which the vector cache absorbs) so that the hardware load
   // counter can be waited on precisely while the next stage's loads are still in flight.
   const int nchunks = nchunk_full + (wc_last ? 1 : 0);
-  auto issue = [&](const Cursor &c, StageRegs<RMAX> &r) {
-    if (c.pc == 0) {
-      const uint8_t *ktile = k_base + (uint64_t)c.ti * (RDKV_TILE * 4) * R;
+  auto issue_k = [&](int ti, KRegs<RMAX> &r) {
+    const uint8_t *ktile = k_base + (uint64_t)ti * (RDKV_TILE * 4) * R;
 #pragma unroll
-      for (int ch = 0; ch < RMAX / 4; ++ch) {
-        const int che = ch < nchunks ? ch : 0;
-        const int wce = che == nchunk_full ? wc_last : 4;
-        // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
-        // the next token (or the region that follows) and are never used
-        const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
-        r.k[4 * ch] = v.x; r.k[4 * ch + 1] = v.y; r.k[4 * ch + 2] = v.z; r.k[4 * ch + 3] = v.w;
-      }
-      r.sz = *reinterpret_cast<const uint4 *>(sz_base + (c.cls < 3 ? (uint64_t)c.ti * (RDKV_TILE * 4) + lb * 16 : 0));
+    for (int ch = 0; ch < RMAX / 4; ++ch) {
+      const int che = ch < nchunks ? ch : 0;
+      const int wce = che == nchunk_full ? wc_last : 4;
+      // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
+      // the next token (or the region that follows) and are never used
+      const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
+      r.k[4 * ch] = v.x; r.k[4 * ch + 1] = v.y; r.k[4 * ch + 2] = v.z; r.k[4 * ch + 3] = v.w;
     }
+    r.sz = *reinterpret_cast<const uint4 *>(sz_base + (ti < ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0));
+  };
+  auto issue_v = [&](const Cursor &c, VRegs &r) {
     const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
     const int hi = c.cls != 0 ? 128 : 0;
     r.v[0] = vt[0];
@@ -296,7 +298,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     return *reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]);
   };
 
-  auto compute = [&](const Cursor &c, const StageRegs<RMAX> &r) {
+  KRegs<RMAX> kr;
+  auto compute = [&](const Cursor &c, const VRegs &r) {
     if (c.pc == 0) {
       // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
       floatx4 sacc[NH];
@@ -306,7 +309,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 #pragma unroll
       for (int j = 0; j < RMAX; ++j) {
         if (j < R) {
-          const uint32_t w = r.k[j];
+          const uint32_t w = kr.k[j];
           if (j < d8) {
             const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
@@ -345,13 +348,16 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       const float pscale = c.cls < 3 ? kPScaleQ : kPScaleH;
       float sc4[4], zp4[4];
       {
-        const uint32_t szw[4] = {r.sz.x, r.sz.y, r.sz.z, r.sz.w};
+        const uint32_t szw[4] = {kr.sz.x, kr.sz.y, kr.sz.z, kr.sz.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           sc4[j] = c.cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] & 0xffffu)) : 1.0f;
           zp4[j] = c.cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] >> 16)) : 0.0f;
         }
       }
+      // the K registers are free now: request this wavefront's next tile (at the end of the
+      // work item the same tile again, so the number of loads in flight stays fixed)
+      issue_k(c.ti + kWaves < tile_end ? c.ti + kWaves : c.ti, kr);
       bool grew = false;
       float s2[NH][4], m_new[NH];
 #pragma unroll
@@ -465,20 +471,26 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     }
   };
 
-  // ---------------- software-pipelined main loop: loads of stage n+1 fly during stage n ----
+  // ---------------- software-pipelined main loop ------------------------------------------
+  // V pieces are requested one stage ahead into alternating buffers, K rows one tile ahead.
+  // Past the last stage the same piece is requested again instead of branching, so every
+  // stage issues the same number of loads and the waits on the load counter stay exact.
   {
-    StageRegs<RMAX> ra, rb;
+    VRegs va, vb;
     Cursor c0;
     set_tile(c0, tile_begin + wave);
-    if (c0.valid) issue(c0, ra);
+    if (c0.valid) {
+      issue_k(c0.ti, kr);
+      issue_v(c0, va);
+    }
     while (c0.valid) {
       const Cursor c1 = advance(c0);
-      if (c1.valid) issue(c1, rb);
-      compute(c0, ra);
+      issue_v(c1.valid ? c1 : c0, vb);
+      compute(c0, va);
       if (!c1.valid) break;
       const Cursor c2 = advance(c1);
-      if (c2.valid) issue(c2, ra);
-      compute(c1, rb);
+      issue_v(c2.valid ? c2 : c1, va);
+      compute(c1, vb);
       c0 = c2;
     }
   }
@@ -568,8 +580,8 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   RDKV_REQUIRE(q, "%s: null q", fn);
   hipStream_t s = (hipStream_t)stream;
   float *partials = (float *)workspace;
-  // occupancy target of the kernel variant (registers per lane); 3 wavefronts per SIMD measured best
-  static const int wpe = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 3;
+  // occupancy target of the kernel variant (registers per lane); 4 wavefronts per SIMD measured best
+  static const int wpe = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 4;
 #define RDKV_LAUNCH_FUSED(NH, RMAX)                                                                        \
   do {                                                                                                     \
     if (wpe >= 4)                                                                                          \
