@@ -33,7 +33,10 @@ def parse():
     ap.add_argument("--layers", type=int, default=None, help="override the layer count (debug)")
     ap.add_argument("--context", type=int, default=None, help="override the context length (debug)")
     ap.add_argument("--batch", type=int, default=None, help="override the batch (config 4)")
-    ap.add_argument("--work-kib", type=int, default=256, help="streamed KiB per workgroup")
+    ap.add_argument("--work-kib", type=int, default=None,
+                    help="streamed KiB per work item, one workgroup each (default: balanced resident groups)")
+    ap.add_argument("--groups-per-cu", type=int, default=1, help="workgroups per compute unit")
+    ap.add_argument("--tile-overhead", type=int, default=8192, help="per-tile cost term of the work partition (bytes)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-check", action="store_true")
@@ -88,7 +91,8 @@ def main():
             del K, V
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
-                                            work_bytes=args.work_kib * 1024)
+                                            work_bytes=args.work_kib * 1024 if args.work_kib else None,
+                                            groups_per_cu=args.groups_per_cu, tile_overhead=args.tile_overhead)
     padded_bytes = 0
     first_pl, first_nvo = groups[0][0], groups[0][1]
     del groups
@@ -121,7 +125,8 @@ def main():
 
     def partials_only():
         _lib.check(lib.rdkv_decode_fused_partials(
-            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work, cache.max_row_dwords,
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
             qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, ws.data_ptr(), ws.numel(), stream))
 
     partials_only()
@@ -212,7 +217,7 @@ def main():
                    "launch": "one fused launch + one merge launch per step over all layers",
                    "class_fractions_apply_to": "context tokens",
                    "algorithmic_bytes_per_step": algo, "algorithmic_bytes_per_layer": algo / n_groups,
-                   "streamed_bytes_per_step": cache.stream_bytes, "work_items": cache.n_work,
+                   "streamed_bytes_per_step": cache.stream_bytes, "work_items": cache.n_work, "workgroups": cache.n_groups or cache.n_work,
                    "dense_fp16_bytes_per_layer": synth.dense_fp16_bytes(cfg),
                    "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo,
                    "build_seconds": t_build},

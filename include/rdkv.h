@@ -175,21 +175,26 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
  * without tokens), so callers can merge further zones exactly.  G = query heads per KV head
  * (1..8).  max_row_dwords = max over units of d8+d4+d2 (<= 32; selects the register budget of
  * the kernel).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes.
+ * groups: int32 [n_groups + 1] ascending offsets into the work list; workgroup g of the
+ * streaming launch processes work items groups[g] .. groups[g+1]-1 one after the other (items
+ * of one unit should be adjacent: the staged query operands are reused).  Size the table so
+ * that all workgroups are resident at once (4 per compute unit) and carry equal bytes.
+ * groups == NULL (n_groups = 0): one workgroup per work item.
  * Two launches: the streaming kernel writes one partial per work item, a small kernel merges
  * the partials of each unit in index order.  Calls that share a workspace must not overlap. */
 int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G);
 int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                      const RdkvWork *work, int n_work, int max_row_dwords,
-                      const void *q, int q_dtype, int64_t q_stride_row, int G,
+                      const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                      int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
                       float *out, int64_t out_stride_row, float *lse,
                       void *workspace, int64_t workspace_bytes, void *stream);
 /* The two launches of rdkv_decode_fused as separate calls (same arguments): the streaming
  * kernel that writes one partial (max, sum, 128 accumulators per head) per work item, and
  * the fixed-order merge of a unit's partials into out / lse. */
 int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                               const RdkvWork *work, int n_work, int max_row_dwords,
-                               const void *q, int q_dtype, int64_t q_stride_row, int G,
-                               void *workspace, int64_t workspace_bytes, void *stream);
+                               const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                               int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row,
+                               int G, void *workspace, int64_t workspace_bytes, void *stream);
 int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G,
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);

@@ -1,11 +1,15 @@
 // Fused flash-decoding over the streaming KV format (stream_format.h): one pass reads every
 // packed byte once and produces softmax(q.K/sqrt(D)).V for all G query heads of a KV head.
 //
-// Work decomposition: a work item is a run of 64-token tiles of one unit, handled by one
-// workgroup of 4 wavefronts; wavefront w takes tiles tile_begin + w, +4, ...  Each wavefront
-// keeps an online-softmax state (running max, sum, 128-channel accumulators) in registers,
-// the four states are merged through LDS and written as one partial; merge_kernel combines
-// the partials of a unit in index order (deterministic, no float atomics).
+// Work decomposition: a work item is a run of 64-token tiles of one unit.  A workgroup fills
+// one compute unit (16 wavefronts at the default register budget) and walks the items of its
+// group; the host cuts the tile stream into one group of equal cost per compute unit, so all
+// workgroups are resident from start to end and the per-item set-up (a chain of dependent
+// loads, several microseconds under load) is paid about twice per compute unit.
+// Wavefront w takes tiles tile_begin + w, + n_waves, ...  Each wavefront keeps an
+// online-softmax state (running max, sum, 128-channel accumulators) in registers, the states
+// are merged through LDS and written as one partial per item; merge_kernel combines the
+// partials of a unit in index order (deterministic, no float atomics).
 //
 // Matrix cores: v_mfma_f32_4x4x4_16b_f16 (16 independent 4x4x4 blocks per wavefront).
 //   K side: block = token quad; A = 4 tokens x 4 channel codes, B = 4 channels x 4 heads of
@@ -26,7 +30,6 @@ namespace {
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kWaves = 4;
 constexpr int kD = 128;
 constexpr int kPartialStride = 132;  // 128 acc + max + sum + 2 pad (floats, per head)
 // fixed-point style power-of-two scalings (all exact)
@@ -135,14 +138,14 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
   }
 }
 
-template <int NH>
+template <int NH, int NW>
 struct Smem {
   alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][2][4][4];  // [step][head group][hi|lo][head][k]
-  alignas(16) _Float16 p[kWaves][16][NH][4][4];        // [wave][quad][head group][head][k]
+  alignas(16) _Float16 p[NW][16][NH][4][4];              // [wave][quad][head group][head][k]
   float bias[NH * 4];
-  float wm[kWaves][NH * 4];
-  float wl[kWaves][NH * 4];
-  float wo[kWaves][NH * 4][kD];
+  float wm[NW][NH * 4];
+  float wl[NW][NH * 4];
+  float wo[NW][4][kD];                                   // one head group at a time
 };
 
 // Register images of the loads in flight.  KRegs: the K row of the lane's token and the
@@ -170,19 +173,36 @@ __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
   return c == 0 ? a0 : (c == 1 ? a1 : (c == 2 ? a2 : a3));
 }
 
+// A workgroup fills a whole compute unit: 4 * WPE wavefronts (WPE per SIMD), all of the same
+// age, so the hardware's oldest-first issue order cannot favour one part of the work.
 template <int NH, int RMAX, int WPE>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
+__global__ void __launch_bounds__(256 * WPE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
-                    const RdkvWork *__restrict__ work, const void *__restrict__ q, int q_dtype,
-                    int64_t q_stride, int G, float *__restrict__ partials) {
-  __shared__ Smem<NH> sm;
+                    const RdkvWork *__restrict__ work, const int32_t *__restrict__ groups,
+                    const void *__restrict__ q, int q_dtype, int64_t q_stride, int G,
+                    float *__restrict__ partials) {
+  constexpr int kWaves = 4 * WPE, kThreads = 64 * kWaves;
+  __shared__ Smem<NH, kWaves> sm;
   const int tid = threadIdx.x, lane = tid & 63;
   // the wavefront index is uniform; say so, or every tile-level decision becomes per-lane
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 3, lb = lane >> 2;
-  const RdkvWork *wkp = work + blockIdx.x;
+  // a workgroup walks the work items of its group; consecutive items of one unit reuse the
+  // query operands already staged in LDS
+  const int item_begin = groups ? groups[blockIdx.x] : (int)blockIdx.x;
+  const int item_end = groups ? groups[blockIdx.x + 1] : (int)blockIdx.x + 1;
+  int staged_unit = -1;
+  for (int item = item_begin; item < item_end; ++item) {
+  // Index values used only before and after the tile loop are re-derived per item from an
+  // opaque copy of the thread id: hoisted out of the item loop they would stay live across
+  // the tile loop and push the kernel over its register budget.
+  int tid_o = tid;
+  asm volatile("" : "+v"(tid_o));
+  const int lane_o = tid_o & 63;
+  const RdkvWork *wkp = work + item;
   const int tile_begin = wkp->tile_begin, tile_end = wkp->tile_end;
-  const RdkvUnit *up = units + wkp->unit;
+  const int unit_index = wkp->unit;
+  const RdkvUnit *up = units + unit_index;
   const int d8 = up->d8, d4 = up->d4, d2 = up->d2;
   const int R = d8 + d4 + d2;
   const int NS = d8 + 2 * d4 + 4 * d2;
@@ -242,11 +262,22 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     r.v[3] = vt[hi + 64];
   };
 
+  // The first tile's loads go out before anything else so that they overlap the prologue.
+  KRegs<RMAX> kr;
+  VRegs va, vb;
+  Cursor c0;
+  set_tile(c0, tile_begin + wave);
+  if (c0.valid) {
+    issue_k(c0.ti, kr);
+    issue_v(c0, va);
+  }
+
   // ---------------- prologue: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias ----------
-  {
+  if (unit_index != staged_unit) {
+    staged_unit = unit_index;
     const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(qtab_base);
     const int nslot = 4 * NS;
-    for (int i = tid; i < nslot * NH * 4; i += 256) {
+    for (int i = tid_o; i < nslot * NH * 4; i += kThreads) {
       const int slot = i % nslot, head = i / nslot;
       _Float16 hi = (_Float16)0.0f, lo = (_Float16)0.0f;
       if (head < G) {
@@ -266,20 +297,25 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     // bias[h] = sum_slot qs[h][slot] * zp[slot] / 2^8, one wavefront per head, fixed tree
     for (int head = wave; head < NH * 4; head += kWaves) {
       float b = 0.0f;
-      for (int slot = lane; slot < nslot; slot += 64) {
+      for (int slot = lane_o; slot < nslot; slot += 64) {
         const float zp = (float)__builtin_bit_cast(_Float16, tab[slot].zp_f16);
         b += ((float)sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] +
               (float)sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3]) * zp;
       }
       b = rdkv_wave_sum(b);
-      if (lane == 0) sm.bias[head] = b * (1.0f / kQScale);
+      if (lane_o == 0) sm.bias[head] = b * (1.0f / kQScale);
     }
     __syncthreads();
   }
 
   // ---------------- per-wavefront online-softmax state -----------------------------------
   float m_run[NH], l_run[NH], zb_run[NH];  // for head 4*hg + ln (own column)
-  floatx4 accq[NH][2], acch[NH][2];        // rows = heads of group, column = channel lane+64*j
+  // One accumulator set: rows = heads of group, column = channel lane+64*j.  It is in the
+  // quantized classes' scaling (2^-18) until the wavefront reaches its first fp16 tile, then
+  // it is multiplied by 2^32 once (exact) and continues in the fp16 class' scaling (2^14);
+  // classes only ascend along a work item.
+  floatx4 accq[NH][2];
+  bool acc_fp16 = false;
   float bias_own[NH];
 #pragma unroll
   for (int hg = 0; hg < NH; ++hg) {
@@ -290,7 +326,6 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       accq[hg][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-      acch[hg][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
   }
 
@@ -298,7 +333,6 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     return *reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]);
   };
 
-  KRegs<RMAX> kr;
   auto compute = [&](const Cursor &c, const VRegs &r) {
     if (c.pc == 0) {
       // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
@@ -387,7 +421,6 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               accq[hg][j][rr] *= f;
-              acch[hg][j][rr] *= f;
             }
           }
         }
@@ -459,13 +492,20 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       }
     } else {  // fp16: piece pc holds quads 4*pc .. 4*pc+3, one 16-byte load per quad
       const int q0 = 4 * c.pc;
+      if (!acc_fp16) {
+        acc_fp16 = true;
+#pragma unroll
+        for (int hg = 0; hg < NH; ++hg)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) accq[hg][j] *= kOBackQ / kOBackH;
+      }
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
 #pragma unroll
         for (int hg = 0; hg < NH; ++hg) {
           const half4_t a = p_op(q0 + x, hg);
-          acch[hg][0] = mfma(a, mk_op(r.v[x].x, r.v[x].y), acch[hg][0]);
-          acch[hg][1] = mfma(a, mk_op(r.v[x].z, r.v[x].w), acch[hg][1]);
+          accq[hg][0] = mfma(a, mk_op(r.v[x].x, r.v[x].y), accq[hg][0]);
+          accq[hg][1] = mfma(a, mk_op(r.v[x].z, r.v[x].w), accq[hg][1]);
         }
       }
     }
@@ -476,13 +516,6 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // Past the last stage the same piece is requested again instead of branching, so every
   // stage issues the same number of loads and the waits on the load counter stay exact.
   {
-    VRegs va, vb;
-    Cursor c0;
-    set_tile(c0, tile_begin + wave);
-    if (c0.valid) {
-      issue_k(c0.ti, kr);
-      issue_v(c0, va);
-    }
     while (c0.valid) {
       const Cursor c1 = advance(c0);
       issue_v(c1.valid ? c1 : c0, vb);
@@ -495,44 +528,49 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     }
   }
 
-  // ---------------- merge the four wavefront states and write the partial -----------------
+  // ---------------- merge the wavefront states and write the partial ---------------------
+  float *part = partials + (int64_t)item * G * kPartialStride;
 #pragma unroll
   for (int hg = 0; hg < NH; ++hg) {
     const float l_tot = quadcol_sum(l_run[hg]);
     const float zb_tot = quadcol_sum(zb_run[hg]) * (1.0f / kPScaleQ);
-    if (lane < 4) {
-      sm.wm[wave][hg * 4 + lane] = m_run[hg];
-      sm.wl[wave][hg * 4 + lane] = l_tot;
+    if (hg > 0) __syncthreads();  // the previous head group's rows have been read
+    if (lane_o < 4) {
+      sm.wm[wave][hg * 4 + lane_o] = m_run[hg];
+      sm.wl[wave][hg * 4 + lane_o] = l_tot;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float zb = __shfl(zb_tot, r, 64);
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        sm.wo[wave][hg * 4 + r][lane + 64 * j] = accq[hg][j][r] * kOBackQ + acch[hg][j][r] * kOBackH - zb;
+        sm.wo[wave][r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : kOBackQ) - zb;
+    }
+    __syncthreads();
+    for (int i = tid_o; i < 4 * kD; i += kThreads) {
+      const int r = i >> 7, d = i & 127, h = hg * 4 + r;
+      if (h < G) {
+        float M = sm.wm[0][h];
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) M = fmaxf(M, sm.wm[w][h]);
+        float o = 0.0f, l = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; ++w) {
+          const float mw = sm.wm[w][h];
+          const float f = mw == -INFINITY ? 0.0f : exp2f(mw - M);  // idle wavefront contributes nothing
+          o += f * sm.wo[w][r][d];
+          l += f * sm.wl[w][h];
+        }
+        part[h * kPartialStride + d] = o;
+        if (d == 0) {
+          part[h * kPartialStride + 128] = M;
+          part[h * kPartialStride + 129] = l;
+        }
+      }
     }
   }
-  __syncthreads();
-  float *part = partials + (int64_t)blockIdx.x * G * kPartialStride;
-  for (int i = tid; i < G * kD; i += 256) {
-    const int h = i >> 7, d = i & 127;
-    float M = sm.wm[0][h];
-#pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, sm.wm[w][h]);
-    float o = 0.0f, l = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float mw = sm.wm[w][h];
-      const float f = mw == -INFINITY ? 0.0f : exp2f(mw - M);  // idle wavefront contributes nothing
-      o += f * sm.wo[w][h][d];
-      l += f * sm.wl[w][h];
-    }
-    part[h * kPartialStride + d] = o;
-    if (d == 0) {
-      part[h * kPartialStride + 128] = M;
-      part[h * kPartialStride + 129] = l;
-    }
-  }
+  __syncthreads();  // the next item overwrites the LDS state read above
+  }  // items of this group
 }
 
 // One workgroup per unit combines its partials (second launch of a step).  Merging inside the
@@ -569,10 +607,14 @@ static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, 
 
 // Launch of the streaming kernel (writes one partial per work item).
 static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *units, int n_units,
-                        const RdkvWork *work, int n_work, int max_row_dwords, const void *q, int q_dtype,
-                        int64_t q_stride_row, int G, void *workspace, int64_t workspace_bytes, void *stream) {
+                        const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                        int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
+                        void *workspace, int64_t workspace_bytes, void *stream) {
   int rc = check_fused_args(fn, units, n_units, work, n_work, G, workspace, workspace_bytes);
   if (rc != RDKV_OK) return rc;
+  RDKV_REQUIRE(groups ? n_groups >= 1 : n_groups == 0, "%s: n_groups=%d does not match the group table", fn,
+               n_groups);
+  const int n_wg = groups ? n_groups : n_work;
   RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "%s: unknown q dtype %d", fn, q_dtype);
   RDKV_REQUIRE(max_row_dwords >= 0 && max_row_dwords <= 32, "%s: max_row_dwords=%d outside 0..32", fn,
                max_row_dwords);
@@ -580,30 +622,33 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   RDKV_REQUIRE(q, "%s: null q", fn);
   hipStream_t s = (hipStream_t)stream;
   float *partials = (float *)workspace;
-  // occupancy target of the kernel variant (registers per lane); 4 wavefronts per SIMD measured best
-  static const int wpe = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 4;
-#define RDKV_LAUNCH_FUSED(NH, RMAX)                                                                        \
+  // Occupancy target (wavefronts per SIMD) of each variant: the highest at which the variant
+  // keeps everything in registers; spilling costs far more than the lost occupancy.
+  // RDKV_FUSED_WPE overrides it (2, 3 or 4) for experiments.
+  static const int wpe_env = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 0;
+#define RDKV_LAUNCH_FUSED(NH, RMAX, WPE_DEFAULT)                                                           \
   do {                                                                                                     \
+    const int wpe = wpe_env ? wpe_env : WPE_DEFAULT;                                                       \
     if (wpe >= 4)                                                                                          \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 4>), dim3(n_work), dim3(256), 0, s, blob, units,   \
-                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 4>), dim3(n_wg), dim3(1024), 0, s, blob, units,    \
+                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
     else if (wpe == 3)                                                                                     \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 3>), dim3(n_work), dim3(256), 0, s, blob, units,   \
-                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 3>), dim3(n_wg), dim3(768), 0, s, blob, units,     \
+                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
     else                                                                                                   \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 2>), dim3(n_work), dim3(256), 0, s, blob, units,   \
-                         work, q, q_dtype, q_stride_row, G, partials);                                     \
+      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 2>), dim3(n_wg), dim3(512), 0, s, blob, units,     \
+                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
   } while (0)
   if (G <= 4) {
-    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12);
-    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(1, 16);
-    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(1, 20);
-    else RDKV_LAUNCH_FUSED(1, 32);
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12, 4);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(1, 16, 4);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(1, 20, 4);
+    else RDKV_LAUNCH_FUSED(1, 32, 3);
   } else {
-    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(2, 12);
-    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(2, 16);
-    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(2, 20);
-    else RDKV_LAUNCH_FUSED(2, 32);
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(2, 12, 3);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(2, 16, 3);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(2, 20, 3);
+    else RDKV_LAUNCH_FUSED(2, 32, 2);
   }
 #undef RDKV_LAUNCH_FUSED
   RDKV_CHECK_LAUNCH(fn);
@@ -611,11 +656,12 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
 }
 
 RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
-                                        const RdkvWork *work, int n_work, int max_row_dwords,
-                                        const void *q, int q_dtype, int64_t q_stride_row, int G,
-                                        void *workspace, int64_t workspace_bytes, void *stream) {
-  return launch_fused("rdkv_decode_fused_partials", blob, units, n_units, work, n_work, max_row_dwords, q,
-                      q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
+                                        const RdkvWork *work, int n_work, const int32_t *groups,
+                                        int n_groups, int max_row_dwords, const void *q, int q_dtype,
+                                        int64_t q_stride_row, int G, void *workspace,
+                                        int64_t workspace_bytes, void *stream) {
+  return launch_fused("rdkv_decode_fused_partials", blob, units, n_units, work, n_work, groups, n_groups,
+                      max_row_dwords, q, q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
 }
 
 RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G, float *out,
@@ -633,11 +679,12 @@ RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_w
 }
 
 RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units, const RdkvWork *work,
-                               int n_work, int max_row_dwords, const void *q, int q_dtype,
-                               int64_t q_stride_row, int G, float *out, int64_t out_stride_row, float *lse,
-                               void *workspace, int64_t workspace_bytes, void *stream) {
-  int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, max_row_dwords, q, q_dtype,
-                                      q_stride_row, G, workspace, workspace_bytes, stream);
+                               int n_work, const int32_t *groups, int n_groups, int max_row_dwords,
+                               const void *q, int q_dtype, int64_t q_stride_row, int G, float *out,
+                               int64_t out_stride_row, float *lse, void *workspace, int64_t workspace_bytes,
+                               void *stream) {
+  int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, groups, n_groups, max_row_dwords, q,
+                                      q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
   if (rc != RDKV_OK) return rc;
   return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
                                  workspace_bytes, stream);

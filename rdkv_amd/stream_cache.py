@@ -69,6 +69,9 @@ class StreamCache:
     stream_bytes: int                    # bytes the fused kernel reads from the blobs per step
     algorithmic_bytes: int               # unpadded bytes (reference accounting) incl. q and out
     max_row_dwords: int = 32             # max over units of the K row length in dwords
+    groups: Optional[torch.Tensor] = None  # device int32 [n_groups + 1] offsets into ``work`` (or None)
+    groups_host: Optional[np.ndarray] = None
+    n_groups: int = 0
 
     @property
     def device(self):
@@ -90,17 +93,88 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
     return [tuple(int(x) for x in v) + (int(n),) for v, n in zip(vb, n16)], [tuple(int(x) for x in k) for k in kb]
 
 
+def _tile_costs(unit_tiles: np.ndarray, unit_R: np.ndarray, tile_overhead: int) -> np.ndarray:
+    """Cost (streamed bytes + a fixed per-tile term) of every tile, unit-major, class-minor."""
+    seg_cost = (256 * unit_R[:, None] + np.asarray(V_TILE_BYTES)[None, :]
+                + np.asarray([256, 256, 256, 0])[None, :] + tile_overhead)
+    return np.repeat(seg_cost.reshape(-1), unit_tiles.reshape(-1))
+
+
+def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Optional[int] = None,
+                   work_bytes: Optional[int] = None, tile_overhead: int = 0):
+    """Cut the unit-major tile sequence into work items.
+
+    ``n_groups``: that many contiguous runs of equal cost, one per workgroup; a run that
+    crosses a unit boundary becomes several items.  ``work_bytes``: items of about that many
+    streamed bytes, one workgroup each (no group table).  A unit without tiles gets one empty
+    item.  Returns (work [n_work] of WORK_DTYPE, groups int32 [n_groups+1] or None,
+    work_begin [U], work_count [U])."""
+    U = len(unit_tiles)
+    per_unit = unit_tiles.sum(axis=1)
+    unit_start = np.concatenate([[0], np.cumsum(per_unit)]).astype(np.int64)
+    total = int(unit_start[-1])
+    cost = _tile_costs(unit_tiles, unit_R, tile_overhead)
+    cum = np.cumsum(cost)
+    if work_bytes is not None:
+        # greedy runs inside each unit, closed when the running cost reaches work_bytes
+        cuts = [0]
+        for u in range(U):
+            a, b = int(unit_start[u]), int(unit_start[u + 1])
+            acc = 0
+            for t in range(a, b):
+                acc += int(cost[t])
+                if acc >= work_bytes or t == b - 1:
+                    cuts.append(t + 1)
+                    acc = 0
+        group_cuts = None
+        cut_pts = np.unique(np.asarray(cuts, dtype=np.int64))
+    else:
+        n_groups = max(1, int(n_groups))
+        target = (float(cum[-1]) if total else 0.0) / n_groups
+        group_cuts = np.searchsorted(cum, target * np.arange(1, n_groups), side="left") + 1 if total else \
+            np.zeros(n_groups - 1, dtype=np.int64)
+        group_cuts = np.minimum(np.concatenate([[0], group_cuts, [total]]).astype(np.int64), total)
+        group_cuts = np.maximum.accumulate(group_cuts)
+        cut_pts = np.unique(np.concatenate([group_cuts, unit_start]))
+    starts, ends = cut_pts[:-1], cut_pts[1:]
+    item_unit = np.searchsorted(unit_start, starts, side="right") - 1
+    empty_units = np.nonzero(per_unit == 0)[0]
+    pos = np.concatenate([starts, unit_start[empty_units]])
+    unit = np.concatenate([item_unit, empty_units]).astype(np.int64)
+    tb = np.concatenate([starts - unit_start[item_unit], np.zeros(len(empty_units), dtype=np.int64)])
+    te = np.concatenate([ends - unit_start[item_unit], np.zeros(len(empty_units), dtype=np.int64)])
+    order = np.lexsort((unit, pos))
+    pos, unit, tb, te = pos[order], unit[order], tb[order], te[order]
+    work = np.zeros(len(unit), dtype=WORK_DTYPE)
+    work["unit"], work["tile_begin"], work["tile_end"] = unit, tb, te
+    work_begin = np.searchsorted(unit, np.arange(U), side="left").astype(np.int32)
+    work_count = (np.searchsorted(unit, np.arange(U), side="right") - work_begin).astype(np.int32)
+    groups = None
+    if group_cuts is not None:
+        item_group = np.minimum(np.searchsorted(group_cuts[1:], pos, side="right"), n_groups - 1)
+        groups = np.searchsorted(item_group, np.arange(n_groups + 1), side="left").astype(np.int32)
+    return work, groups, work_begin, work_count
+
+
 def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
-                       work_bytes: int = 256 * 1024) -> StreamCache:
+                       work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
+                       groups_per_cu: int = 1, tile_overhead: int = 8192) -> StreamCache:
     """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
     layer)) into the streaming format.  Query/output row of entry g, query head hq is
-    ``g * H_q + hq``.  ``work_bytes`` is the target number of streamed bytes per workgroup."""
+    ``g * H_q + hq``.
+
+    Work decomposition: by default the tile stream is cut into one run of equal cost per
+    compute unit (the fused kernel's workgroups fill a compute unit each); cost = streamed
+    bytes + ``tile_overhead`` per tile.  ``n_groups`` overrides the count; small caches get
+    fewer runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
+    many streamed bytes with one workgroup per item."""
     lib = _lib.load()
     dev = _lib.require_device(layers[0][0].K_ch_scale)
     stream = _lib.stream_of(dev)
-    units_all, work_all, blobs = [], [], []
+    units_all, blobs = [], []
+    unit_tiles, unit_R = [], []
     stream_bytes = algo_bytes = 0
-    n_groups = len(layers)
+    n_entries = len(layers)
     H_q = None
     for gi, (pl, nvo) in enumerate(layers):
         H_kv = pl.K_ch_scale.shape[1]
@@ -153,20 +227,8 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
                            + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
                            + 256 * n_tok[3])
-            # work items: runs of tiles of about work_bytes streamed bytes
-            costs = []
-            for c in range(4):
-                costs += [TILE * 4 * R + V_TILE_BYTES[c] + (TILE * 4 if c < 3 else 0)] * tiles[c]
-            u["work_begin"] = len(work_all)
-            t0, acc = 0, 0
-            for t, cst in enumerate(costs):
-                acc += cst
-                if acc >= work_bytes or t == len(costs) - 1:
-                    work_all.append((len(units_all) + h, t0, t + 1, 0))
-                    t0, acc = t + 1, 0
-            if not costs:                      # a unit without tokens still gets one (empty) work item
-                work_all.append((len(units_all) + h, 0, 0, 0))
-            u["work_count"] = len(work_all) - int(u["work_begin"])
+            unit_tiles.append(tiles)
+            unit_R.append(R)
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
         assert base % 256 == 0
@@ -208,17 +270,27 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         # keep the temporaries alive until the relayout kernel has run
         torch.cuda.current_stream(dev).synchronize()
     units_np = np.array(units_all, dtype=UNIT_DTYPE)
-    work_np = np.array(work_all, dtype=WORK_DTYPE) if work_all else np.zeros(0, dtype=WORK_DTYPE)
-    rows = n_groups * H_q
+    tiles_np = np.asarray(unit_tiles, dtype=np.int64).reshape(-1, 4)
+    if work_bytes is None and n_groups is None:
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
+    work_np, groups_np, wb, wc = partition_work(tiles_np, np.asarray(unit_R, dtype=np.int64),
+                                                n_groups=n_groups, work_bytes=work_bytes,
+                                                tile_overhead=tile_overhead)
+    units_np["work_begin"], units_np["work_count"] = wb, wc
+    rows = n_entries * H_q
     algo_bytes += rows * 128 * 2 + rows * 128 * 4
     units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
     work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
         16, dtype=torch.uint8, device=dev)
+    groups_dev = torch.from_numpy(groups_np).to(dev) if groups_np is not None else None
     return StreamCache(blobs=blobs, units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
                        n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
                        stream_bytes=int(stream_bytes), algorithmic_bytes=int(algo_bytes),
                        max_row_dwords=int(max((int(u["d8"]) + int(u["d4"]) + int(u["d2"]) for u in units_np),
-                                              default=0)))
+                                              default=0)),
+                       groups=groups_dev, groups_host=groups_np,
+                       n_groups=0 if groups_np is None else len(groups_np) - 1)
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
@@ -240,6 +312,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     ws = _lib.workspace(dev, need)
     _lib.check(lib.rdkv_decode_fused(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-        cache.max_row_dwords, q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
+        _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
         out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
     return out, lse

@@ -104,6 +104,13 @@ def test_fused_attention_golden(name):
         [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G, work_bytes=1)
     out1, lse1 = stream_cache.decode_attn_fused(cache1, to_dev(g["q"]))
     attn_close(t2n(out1), g["out"], "out(work_bytes=1)")
+    # ... and with three workgroups that each walk several items across unit boundaries
+    cache3 = stream_cache.build_stream_cache(
+        [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G, n_groups=3)
+    assert cache3.n_groups == 3 and cache3.n_work >= cache3.n_units
+    out3, lse3 = stream_cache.decode_attn_fused(cache3, to_dev(g["q"]))
+    attn_close(t2n(out3), g["out"], "out(n_groups=3)")
+    attn_close(t2n(lse3), exp_lse, "lse(n_groups=3)")
     # run-to-run determinism
     out2, _ = stream_cache.decode_attn_fused(cache, to_dev(g["q"]))
     assert torch.equal(out, out2)
@@ -123,13 +130,19 @@ def _config_case(cfg, layers):
     return packed, torch.cat(qs).to(DEV), oracle_out
 
 
+@pytest.mark.parametrize("partition", ["groups", "few_groups", "items"])
 @pytest.mark.parametrize("cfg_idx,ctx,layers", [(0, 4096, 1), (1, 3000, 2), (2, 2500, 1), (3, 1500, 2)])
-def test_fused_attention_config_shaped(cfg_idx, ctx, layers):
+def test_fused_attention_config_shaped(cfg_idx, ctx, layers, partition):
     """C0 at its full size; C1/C2/C3 shapes (incl. GQA 8) at reduced context, several layers in
-    one launch."""
+    one launch; with the default balanced workgroups and with one workgroup per 64 KiB item, and with
+    three workgroups that each walk many items across unit boundaries."""
     cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=layers)
     packed, q, exp = _config_case(cfg, layers)
-    cache = stream_cache.build_stream_cache(packed, cfg.G, work_bytes=64 * 1024)
+    kw = {"groups": {}, "few_groups": {"n_groups": 3}, "items": {"work_bytes": 64 * 1024}}[partition]
+    cache = stream_cache.build_stream_cache(packed, cfg.G, **kw)
+    assert (cache.groups is not None) == (partition != "items")
+    if partition == "few_groups":      # workgroups walk several units each
+        assert cache.n_groups == 3 and np.diff(cache.groups_host).min() >= 3
     out, lse = stream_cache.decode_attn_fused(cache, q)
     out, lse = t2n(out), t2n(lse)
     for layer, (eo, el, _) in enumerate(exp):

@@ -99,3 +99,66 @@ def test_synth_allocations():
     assert vb.shape == (512,) and (kb > 0).sum() == 64
     vb2, kb2, _ = synth.head_allocation(cfg1, 1, 2)
     assert np.array_equal(vb, vb2) and np.array_equal(kb, kb2)
+
+
+def _check_partition(tiles, R, work, groups, wb, wc):
+    from rdkv_amd.stream_cache import _tile_costs
+    U = len(tiles)
+    per_unit = tiles.sum(axis=1)
+    # every tile of every unit is covered exactly once, in order; empty units get one empty item
+    for u in range(U):
+        items = work[wb[u]:wb[u] + wc[u]]
+        assert wc[u] >= 1 and (items["unit"] == u).all()
+        if per_unit[u] == 0:
+            assert wc[u] == 1 and items[0]["tile_begin"] == 0 and items[0]["tile_end"] == 0
+            continue
+        assert items[0]["tile_begin"] == 0 and items[-1]["tile_end"] == per_unit[u]
+        assert (items["tile_begin"][1:] == items["tile_end"][:-1]).all()
+        assert (items["tile_end"] > items["tile_begin"]).all()
+    assert wc.sum() == len(work)
+    assert (np.diff(work["unit"]) >= 0).all()
+    if groups is not None:
+        assert groups[0] == 0 and groups[-1] == len(work) and (np.diff(groups) >= 0).all()
+        cost = _tile_costs(tiles, R, 0)
+        start = np.concatenate([[0], np.cumsum(per_unit)])
+        cum = np.concatenate([[0], np.cumsum(cost)])
+        gcost = []
+        for g in range(len(groups) - 1):
+            c = 0
+            for it in work[groups[g]:groups[g + 1]]:
+                a = start[it["unit"]]
+                c += cum[a + it["tile_end"]] - cum[a + it["tile_begin"]]
+            gcost.append(c)
+        gcost = np.asarray(gcost, dtype=np.float64)
+        if cost.size:
+            assert gcost.sum() == cum[-1]
+            assert gcost.max() - gcost.min() <= 2 * cost.max()   # equal up to one tile either side
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_partition_work_groups_and_items(seed):
+    from rdkv_amd.stream_cache import partition_work
+    rng = np.random.default_rng(seed)
+    U = int(rng.integers(1, 40))
+    tiles = rng.integers(0, 30, size=(U, 4)).astype(np.int64)
+    tiles[rng.random(U) < 0.2] = 0                       # units whose tokens were all evicted
+    R = rng.integers(0, 33, size=U).astype(np.int64)
+    for n_groups in (1, 3, 16, 64):
+        work, groups, wb, wc = partition_work(tiles, R, n_groups=n_groups)
+        assert len(groups) == n_groups + 1
+        _check_partition(tiles, R, work, groups, wb, wc)
+    for wbytes in (1, 50_000, 10**9):
+        work, groups, wb, wc = partition_work(tiles, R, work_bytes=wbytes)
+        assert groups is None
+        _check_partition(tiles, R, work, groups, wb, wc)
+        if wbytes == 1:
+            assert len(work) == tiles.sum() + (tiles.sum(axis=1) == 0).sum()
+        if wbytes == 10**9:
+            assert len(work) == U
+
+
+def test_partition_work_all_empty():
+    from rdkv_amd.stream_cache import partition_work
+    tiles = np.zeros((3, 4), dtype=np.int64)
+    work, groups, wb, wc = partition_work(tiles, np.asarray([4, 0, 7]), n_groups=1)
+    assert len(work) == 3 and list(groups) == [0, 3] and list(wc) == [1, 1, 1]
