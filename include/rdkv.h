@@ -202,9 +202,11 @@ int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int 
 /* ---- measurement helpers (no counterpart in the reference) --------------------------------
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)
- * and a read-only sweep in contiguous spans of span_bytes per workgroup (sink: >= 1 KiB). */
+ * and a read-only sweep in contiguous spans of span_bytes per workgroup (sink: >= 1 KiB),
+ * with plain loads or with the streaming (nontemporal) hint the decode kernel uses for V. */
 int rdkv_probe_copy(const void *src, void *dst, int64_t bytes, void *stream);
 int rdkv_probe_read(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream);
+int rdkv_probe_read_stream(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

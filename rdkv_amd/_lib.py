@@ -53,6 +53,7 @@ SIGNATURES = {
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
     "rdkv_probe_copy": (I, [P, P, L, P]),
     "rdkv_probe_read": (I, [P, L, L, P, P]),
+    "rdkv_probe_read_stream": (I, [P, L, L, P, P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None

@@ -42,6 +42,17 @@ constexpr float kOBackH = 1.0f / 16384.0f;
 constexpr float kLog2eOverSqrtD = 0.12751743074602468f;  // log2(e)/sqrt(128)
 constexpr float kLn2 = 0.6931471805599453f;
 
+
+// 16-byte load with the streaming (nontemporal) hint.  V tiles are read once per step and
+// make up three quarters of the stream: keeping them from displacing other lines in the
+// cache hierarchy (K rows, tables, partials) was measured 10% faster end to end; the same
+// hint on the K rows was measured slower.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld16_stream(const void *p) {
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+  return make_uint4(t.x, t.y, t.z, t.w);
+}
+
 __device__ __forceinline__ half4_t mk_op(uint32_t a, uint32_t b) {
   union { uint32_t u[2]; half4_t h; } x;
   x.u[0] = a;
@@ -256,10 +267,10 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   auto issue_v = [&](const Cursor &c, VRegs &r) {
     const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
     const int hi = c.cls != 0 ? 128 : 0;
-    r.v[0] = vt[0];
-    r.v[1] = vt[64];
-    r.v[2] = vt[hi];
-    r.v[3] = vt[hi + 64];
+    r.v[0] = ld16_stream(vt);
+    r.v[1] = ld16_stream(vt + 64);
+    r.v[2] = ld16_stream(vt + hi);
+    r.v[3] = ld16_stream(vt + hi + 64);
   };
 
   // The first tile's loads go out before anything else so that they overlap the prologue.

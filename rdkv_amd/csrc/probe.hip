@@ -12,6 +12,9 @@ probe_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_
 
 // Each workgroup reads a contiguous span (like a work item of the decode kernel) and folds
 // it into one dword so the loads cannot be removed.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <bool STREAM>
 __global__ void __launch_bounds__(256)
 probe_read_kernel(const uint4 *__restrict__ src, int64_t n16, int64_t span16, uint32_t *__restrict__ sink) {
   const int64_t b0 = (int64_t)blockIdx.x * span16;
@@ -22,7 +25,14 @@ probe_read_kernel(const uint4 *__restrict__ src, int64_t n16, int64_t span16, ui
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
       const int64_t j = i + k * 256;
-      v[k] = j < b1 ? src[j] : make_uint4(0, 0, 0, 0);
+      if (j >= b1) {
+        v[k] = make_uint4(0, 0, 0, 0);
+      } else if (STREAM) {  // nontemporal hint, as the decode kernel uses for V tiles
+        const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + j));
+        v[k] = make_uint4(t.x, t.y, t.z, t.w);
+      } else {
+        v[k] = src[j];
+      }
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k) acc ^= v[k].x ^ v[k].y ^ v[k].z ^ v[k].w;
@@ -40,13 +50,27 @@ RDKV_API int rdkv_probe_copy(const void *src, void *dst, int64_t bytes, void *st
   return RDKV_OK;
 }
 
-RDKV_API int rdkv_probe_read(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream) {
+static int probe_read(const char *fn, bool stream_hint, const void *src, int64_t bytes, int64_t span_bytes,
+                      void *sink, void *stream) {
   RDKV_REQUIRE(src && sink && bytes > 0 && bytes % 16 == 0 && span_bytes >= 4096 && span_bytes % 16 == 0,
-               "rdkv_probe_read: bad sizes");
+               "%s: bad sizes", fn);
   const int64_t blocks = rdkv_cdiv(bytes, span_bytes);
-  RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_probe_read: too many spans");
-  hipLaunchKernelGGL(probe_read_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                     (const uint4 *)src, bytes / 16, span_bytes / 16, (uint32_t *)sink);
-  RDKV_CHECK_LAUNCH("rdkv_probe_read");
+  RDKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many spans", fn);
+  if (stream_hint)
+    hipLaunchKernelGGL(probe_read_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, bytes / 16, span_bytes / 16, (uint32_t *)sink);
+  else
+    hipLaunchKernelGGL(probe_read_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4 *)src, bytes / 16, span_bytes / 16, (uint32_t *)sink);
+  RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
+}
+
+RDKV_API int rdkv_probe_read(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream) {
+  return probe_read("rdkv_probe_read", false, src, bytes, span_bytes, sink, stream);
+}
+
+RDKV_API int rdkv_probe_read_stream(const void *src, int64_t bytes, int64_t span_bytes, void *sink,
+                                    void *stream) {
+  return probe_read("rdkv_probe_read_stream", true, src, bytes, span_bytes, sink, stream);
 }

@@ -93,15 +93,26 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
     return [tuple(int(x) for x in v) + (int(n),) for v, n in zip(vb, n16)], [tuple(int(x) for x in k) for k in kb]
 
 
-def _tile_costs(unit_tiles: np.ndarray, unit_R: np.ndarray, tile_overhead: int) -> np.ndarray:
-    """Cost (streamed bytes + a fixed per-tile term) of every tile, unit-major, class-minor."""
-    seg_cost = (256 * unit_R[:, None] + np.asarray(V_TILE_BYTES)[None, :]
-                + np.asarray([256, 256, 256, 0])[None, :] + tile_overhead)
-    return np.repeat(seg_cost.reshape(-1), unit_tiles.reshape(-1))
+# Cost model of the fused kernel for the work partition, in nanoseconds of one compute unit:
+# per tile of each V class, per dword of K row per tile, per work item (its set-up is a chain
+# of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X with G <= 4.
+DEFAULT_COST = {"tile": (199.0, 209.0, 347.0, 603.0), "k_dword": 7.0, "item": 5600.0}
+BYTES_COST = {"tile": (2048.0 + 256, 4096.0 + 256, 8192.0 + 256, 16384.0), "k_dword": 256.0, "item": 0.0}
+
+
+def _tile_costs(unit_tiles: np.ndarray, unit_R: np.ndarray, cost: dict) -> np.ndarray:
+    """Cost of every tile, unit-major, class-minor; the first tile of a unit also carries the
+    item cost (a run that crosses into a unit starts a new item there)."""
+    seg_cost = cost["k_dword"] * unit_R[:, None].astype(np.float64) + np.asarray(cost["tile"])[None, :]
+    out = np.repeat(seg_cost.reshape(-1), unit_tiles.reshape(-1))
+    per_unit = unit_tiles.sum(axis=1)
+    first = np.concatenate([[0], np.cumsum(per_unit)])[:-1][per_unit > 0]
+    out[first] += cost["item"]
+    return out
 
 
 def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Optional[int] = None,
-                   work_bytes: Optional[int] = None, tile_overhead: int = 0):
+                   work_bytes: Optional[int] = None, cost: Optional[dict] = None):
     """Cut the unit-major tile sequence into work items.
 
     ``n_groups``: that many contiguous runs of equal cost, one per workgroup; a run that
@@ -113,7 +124,7 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     per_unit = unit_tiles.sum(axis=1)
     unit_start = np.concatenate([[0], np.cumsum(per_unit)]).astype(np.int64)
     total = int(unit_start[-1])
-    cost = _tile_costs(unit_tiles, unit_R, tile_overhead)
+    cost = _tile_costs(unit_tiles, unit_R, BYTES_COST if work_bytes is not None else (cost or DEFAULT_COST))
     cum = np.cumsum(cost)
     if work_bytes is not None:
         # greedy runs inside each unit, closed when the running cost reaches work_bytes
@@ -158,14 +169,14 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
 
 def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
                        work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
-                       groups_per_cu: int = 1, tile_overhead: int = 8192) -> StreamCache:
+                       groups_per_cu: int = 1, cost: Optional[dict] = None) -> StreamCache:
     """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
     layer)) into the streaming format.  Query/output row of entry g, query head hq is
     ``g * H_q + hq``.
 
     Work decomposition: by default the tile stream is cut into one run of equal cost per
-    compute unit (the fused kernel's workgroups fill a compute unit each); cost = streamed
-    bytes + ``tile_overhead`` per tile.  ``n_groups`` overrides the count; small caches get
+    compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
+    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; small caches get
     fewer runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
     many streamed bytes with one workgroup per item."""
     lib = _lib.load()
@@ -276,7 +287,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
     work_np, groups_np, wb, wc = partition_work(tiles_np, np.asarray(unit_R, dtype=np.int64),
                                                 n_groups=n_groups, work_bytes=work_bytes,
-                                                tile_overhead=tile_overhead)
+                                                cost=cost)
     units_np["work_begin"], units_np["work_count"] = wb, wc
     rows = n_entries * H_q
     algo_bytes += rows * 128 * 2 + rows * 128 * 4

@@ -102,7 +102,7 @@ def test_synth_allocations():
 
 
 def _check_partition(tiles, R, work, groups, wb, wc):
-    from rdkv_amd.stream_cache import _tile_costs
+    from rdkv_amd.stream_cache import BYTES_COST, DEFAULT_COST, _tile_costs
     U = len(tiles)
     per_unit = tiles.sum(axis=1)
     # every tile of every unit is covered exactly once, in order; empty units get one empty item
@@ -119,7 +119,7 @@ def _check_partition(tiles, R, work, groups, wb, wc):
     assert (np.diff(work["unit"]) >= 0).all()
     if groups is not None:
         assert groups[0] == 0 and groups[-1] == len(work) and (np.diff(groups) >= 0).all()
-        cost = _tile_costs(tiles, R, 0)
+        cost = _tile_costs(tiles, R, DEFAULT_COST)
         start = np.concatenate([[0], np.cumsum(per_unit)])
         cum = np.concatenate([[0], np.cumsum(cost)])
         gcost = []
@@ -131,7 +131,7 @@ def _check_partition(tiles, R, work, groups, wb, wc):
             gcost.append(c)
         gcost = np.asarray(gcost, dtype=np.float64)
         if cost.size:
-            assert gcost.sum() == cum[-1]
+            assert np.isclose(gcost.sum(), cum[-1])
             assert gcost.max() - gcost.min() <= 2 * cost.max()   # equal up to one tile either side
 
 
