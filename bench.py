@@ -22,6 +22,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the fused kernel on the default workload, from two rocprofv3 --pmc
+# runs of this command (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors a plain copy
+# kernel of known size gives): (553 874 x 2 + 1 052) KiB.  Other workloads: not measured.
+MEASURED_TRAFFIC_BYTES = {1: 1135411200}
 
 
 def parse():
@@ -57,6 +61,8 @@ def time_region(fn, steps, torch):
 
 def main():
     args = parse()
+    default_workload = (args.layers is None and args.context is None and args.batch is None
+                        and args.work_kib is None and args.groups_per_cu == 1)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the hot path shards by KV head / sequence "
               "without any exchange; no multi-GPU figure is produced). Run with --gpus 1.", file=sys.stderr)
@@ -240,7 +246,8 @@ def main():
                    "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo,
                    "build_seconds": t_build},
         "roofline": {"bound": "hbm", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": kernel_gbps / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": kernel_gbps / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if default_workload else None,
                      "kernel": "decode_fused_kernel", "ms_per_launch": ms_kernel,
                      "algorithmic_bytes_per_launch": algo,
                      "streamed_bytes_per_launch": cache.stream_bytes,

@@ -96,7 +96,7 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
 # Cost model of the fused kernel for the work partition, in nanoseconds of one compute unit:
 # per tile of each V class, per dword of K row per tile, per work item (its set-up is a chain
 # of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X with G <= 4.
-DEFAULT_COST = {"tile": (199.0, 209.0, 347.0, 603.0), "k_dword": 7.0, "item": 5600.0}
+DEFAULT_COST = {"tile": (198.0, 195.0, 280.0, 499.0), "k_dword": 5.9, "item": 7400.0}
 BYTES_COST = {"tile": (2048.0 + 256, 4096.0 + 256, 8192.0 + 256, 16384.0), "k_dword": 256.0, "item": 0.0}
 
 
