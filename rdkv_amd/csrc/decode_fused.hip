@@ -353,9 +353,13 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       int step = 0;
 #pragma unroll
       for (int j = 0; j < RMAX; ++j) {
-        if (j < R) {
+        // compare right here, every tile: hoisted, the 3 * RMAX loop-invariant comparisons no
+        // longer fit the scalar registers and come back through lane reads
+        int R_o = R, d8_o = d8, d84_o = d8 + d4;
+        asm volatile("" : "+s"(R_o), "+s"(d8_o), "+s"(d84_o));
+        if (j < R_o) {
           const uint32_t w = kr.k[j];
-          if (j < d8) {
+          if (j < d8_o) {
             const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
             for (int hg = 0; hg < NH; ++hg) {
@@ -363,7 +367,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
               sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][1][ln][0]), sacc[hg]);
             }
             step += 1;
-          } else if (j < d8 + d4) {
+          } else if (j < d84_o) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
               const half4_t a = mk_op((w >> (8 * s)) & 0x000F000Fu, (w >> (8 * s + 4)) & 0x000F000Fu);

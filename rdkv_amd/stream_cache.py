@@ -95,8 +95,10 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
 
 # Cost model of the fused kernel for the work partition, in nanoseconds of one compute unit:
 # per tile of each V class, per dword of K row per tile, per work item (its set-up is a chain
-# of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X with G <= 4.
+# of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X, for G <= 4 (one
+# head group, 16 wavefronts) and for G = 5..8 (two head groups, 12 wavefronts).
 DEFAULT_COST = {"tile": (198.0, 195.0, 280.0, 499.0), "k_dword": 5.9, "item": 7400.0}
+DEFAULT_COST_TWO_HEAD_GROUPS = {"tile": (301.0, 307.0, 337.0, 419.0), "k_dword": 8.0, "item": 13600.0}
 BYTES_COST = {"tile": (2048.0 + 256, 4096.0 + 256, 8192.0 + 256, 16384.0), "k_dword": 256.0, "item": 0.0}
 
 
@@ -287,7 +289,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
     work_np, groups_np, wb, wc = partition_work(tiles_np, np.asarray(unit_R, dtype=np.int64),
                                                 n_groups=n_groups, work_bytes=work_bytes,
-                                                cost=cost)
+                                                cost=cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS))
     units_np["work_begin"], units_np["work_count"] = wb, wc
     rows = n_entries * H_q
     algo_bytes += rows * 128 * 2 + rows * 128 * 4
