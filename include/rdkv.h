@@ -73,6 +73,29 @@ int rdkv_k_quantize_pack(const void *k_f16, int64_t k_row_stride, int64_t T, int
                          uint8_t *K2, uint8_t *K4, uint8_t *K8,
                          void *scale_f16, void *zp_f16, void *stream);
 
+/* Whole-layer prefill packer: the composition the reference runs per layer
+ * (obkv_fast.py:1141-1155: per head build_packed_layer with deferred K, packing.py:801-1013,
+ * then _pad_and_stack_per_head_layers, packing.py:1019-1317) without its per-head loop and
+ * without materializing the zero-padded K canvas.  K, V: fp16 [H_kv, T, D] (strides in
+ * elements).  order[h]: token ids of head h, first its compressed tokens in V's sorted order
+ * (2-bit, 4-bit, 8-bit; ascending position inside a class = stable argsort, packing.py:734),
+ * then its fp16-zone tokens ascending (packing.py:904).  counts: int32 [H_kv,4] = n2,n4,n8,n16
+ * (device).  mN2/mN4/mN8/max_tv/max_n16: maxima over heads (host).  slot_channel: int32
+ * [H_kv, n2p+n4p+n8] padded sorted slot -> source channel, -1 = pad (shared-max widths).
+ * Outputs, all head-stacked and zero-padded as the reference lays them out:
+ * V2 [H_kv,mN2,D/4], V4 [H_kv,mN4,D/2], V8 [H_kv,mN8,D], V_scale/V_zp fp16 [H_kv,max_tv]
+ * (rows beyond a head's count are NOT written: pass zeroed buffers), V16 fp16
+ * [H_kv,max_n16,D], K2/K4/K8 [H_kv,max_tv+max_n16,sub], K_scale/K_zp fp16 [H_kv,Dp].
+ * A head with fewer rows than the maxima has zero rows in the K canvas, so 0 joins its
+ * per-channel min/max.  minmax_ws: H_kv*2*D floats of scratch. */
+int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
+                             int H_kv, int D, const int32_t *order, int64_t order_stride_h,
+                             const int32_t *counts, int mN2, int mN4, int mN8, int64_t max_tv,
+                             int max_n16, const int32_t *slot_channel, int n2p, int n4p, int n8,
+                             uint8_t *V2, uint8_t *V4, uint8_t *V8, void *V_scale_f16, void *V_zp_f16,
+                             void *V16_f16, uint8_t *K2, uint8_t *K4, uint8_t *K8,
+                             void *K_scale_f16, void *K_zp_f16, float *minmax_ws, void *stream);
+
 /* Dequantize (codes - zp) * scale -> fp16 (unpack_v_segment packing.py:1427-1444 and the
  * per-segment step of unpack_k_mixed packing.py:629-651).  per_row != 0: scale/zp indexed by
  * row (V); per_row == 0: indexed by unpacked column (K).  out row stride in elements. */

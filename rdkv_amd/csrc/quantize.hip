@@ -9,19 +9,12 @@ namespace {
 // ---------------------------------------------------------------------------
 // Per-row (per-token) quantizer, one wavefront per row.
 // ---------------------------------------------------------------------------
+// One wavefront quantizes one row of D channels: min/max -> scale/zp -> codes -> packed bytes.
 template <int BITS>
-__global__ void __launch_bounds__(256)
-quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
-                     const int64_t *__restrict__ row_idx, int64_t rows, int D, int pack,
-                     uint8_t *__restrict__ out, __half *__restrict__ scale_out,
-                     __half *__restrict__ zp_out) {
-  const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-  if (r >= rows) return;
-  const int64_t src = row_idx ? row_idx[r] : r;
-  const __half *xr = x + src * x_row_stride;
+__device__ __forceinline__ void quantize_one_row(const __half *__restrict__ xr, int D, int pack, int lane,
+                                                 uint8_t *__restrict__ o, __half *__restrict__ scale_out,
+                                                 __half *__restrict__ zp_out) {
   const float qmax = (float)((1 << BITS) - 1);
-
   float mn = INFINITY, mx = -INFINITY;
   for (int c = lane; c < D; c += 64) {
     float v = __half2float(xr[c]);
@@ -32,15 +25,13 @@ quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
   mx = rdkv_wave_max(mx);
   const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
   if (lane == 0) {
-    scale_out[r] = __float2half_rn(p.scale);
-    zp_out[r] = __float2half_rn(p.zp);
+    *scale_out = __float2half_rn(p.scale);
+    *zp_out = __float2half_rn(p.zp);
   }
   if (!pack || BITS == 8) {
-    uint8_t *o = out + r * (int64_t)D;
     for (int c = lane; c < D; c += 64) o[c] = (uint8_t)rdkv_qcode(__half2float(xr[c]), p, qmax);
   } else if (BITS == 4) {
     const int n = D >> 1;
-    uint8_t *o = out + r * (int64_t)n;
     for (int i = lane; i < n; i += 64) {
       uint32_t lo = rdkv_qcode(__half2float(xr[i]), p, qmax);
       uint32_t hi = rdkv_qcode(__half2float(xr[i + n]), p, qmax);
@@ -48,13 +39,144 @@ quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
     }
   } else {
     const int n = D >> 2;
-    uint8_t *o = out + r * (int64_t)n;
     for (int i = lane; i < n; i += 64) {
       uint32_t b = rdkv_qcode(__half2float(xr[i]), p, qmax);
       b |= rdkv_qcode(__half2float(xr[i + n]), p, qmax) << 2;
       b |= rdkv_qcode(__half2float(xr[i + 2 * n]), p, qmax) << 4;
       b |= rdkv_qcode(__half2float(xr[i + 3 * n]), p, qmax) << 6;
       o[i] = (uint8_t)b;
+    }
+  }
+}
+
+template <int BITS>
+__global__ void __launch_bounds__(256)
+quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
+                     const int64_t *__restrict__ row_idx, int64_t rows, int D, int pack,
+                     uint8_t *__restrict__ out, __half *__restrict__ scale_out,
+                     __half *__restrict__ zp_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const int64_t src = row_idx ? row_idx[r] : r;
+  const int width = (!pack || BITS == 8) ? D : (BITS == 4 ? D >> 1 : D >> 2);
+  quantize_one_row<BITS>(x + src * x_row_stride, D, pack, lane, out + r * (int64_t)width, scale_out + r,
+                         zp_out + r);
+}
+
+// ---------------------------------------------------------------------------
+// Whole-layer V side: every row of the head-stacked, per-class zero-padded V tensors and of
+// the fp16 zone-B tensor in one launch.  Row i of head h: [0,mN2) 2-bit rows, then mN4 4-bit,
+// mN8 8-bit, max_n16 fp16 rows; rows beyond the head's own count are zero.
+// ---------------------------------------------------------------------------
+// D == 128: lane l owns channels l and l+64, so a 4-bit byte (channels i, i+64) is lane-local
+// and a 2-bit byte (channels i, i+32, i+64, i+96) needs one exchange with lane i+32.
+template <int BITS>
+__device__ __forceinline__ void quantize_values_d128(float x0, float x1, int lane, uint8_t *__restrict__ o,
+                                                     __half *__restrict__ scale_out,
+                                                     __half *__restrict__ zp_out) {
+  const float qmax = (float)((1 << BITS) - 1);
+  const float mn = rdkv_wave_min(fminf(x0, x1));
+  const float mx = rdkv_wave_max(fmaxf(x0, x1));
+  const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
+  if (lane == 0) {
+    *scale_out = __float2half_rn(p.scale);
+    *zp_out = __float2half_rn(p.zp);
+  }
+  const uint32_t q0 = rdkv_qcode(x0, p, qmax), q1 = rdkv_qcode(x1, p, qmax);
+  if (BITS == 8) {
+    o[lane] = (uint8_t)q0;
+    o[lane + 64] = (uint8_t)q1;
+  } else if (BITS == 4) {
+    o[lane] = (uint8_t)(q0 | (q1 << 4));
+  } else {
+    const uint32_t p0 = __shfl_down(q0, 32, 64), p1 = __shfl_down(q1, 32, 64);
+    if (lane < 32) o[lane] = (uint8_t)(q0 | (p0 << 2) | (q1 << 4) | (p1 << 6));
+  }
+}
+
+#define RDKV_PACK_V_ROWS_PER_WAVE 8
+__global__ void __launch_bounds__(256)
+pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stride_t, int D,
+                    const int32_t *__restrict__ order, int64_t order_stride_h,
+                    const int32_t *__restrict__ counts, int mN2, int mN4, int mN8, int max_n16,
+                    int64_t max_tv, uint8_t *__restrict__ V2, uint8_t *__restrict__ V4,
+                    uint8_t *__restrict__ V8, __half *__restrict__ vs, __half *__restrict__ vz,
+                    __half *__restrict__ V16) {
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.y;
+  const int n2 = counts[4 * h], n4 = counts[4 * h + 1], n8 = counts[4 * h + 2], n16 = counts[4 * h + 3];
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Vh = V + (int64_t)h * stride_h;
+  __half *vsh = vs + (int64_t)h * max_tv, *vzh = vz + (int64_t)h * max_tv;
+  const bool d128 = D == 128;
+  auto zero_bytes = [&](uint8_t *o, int n) {
+    for (int c = lane; c < n; c += 64) o[c] = 0;
+  };
+  const int64_t total = (int64_t)mN2 + mN4 + mN8 + max_n16;
+  const int64_t i0 = ((int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * RDKV_PACK_V_ROWS_PER_WAVE;
+  // row i -> (class, row in class j, row in the head's sorted order r, valid)
+  auto locate = [&](int64_t i, int &cls, int64_t &j, int64_t &r, bool &valid) {
+    if (i < mN2) { cls = 0; j = i; r = j; valid = j < n2; }
+    else if (i < (int64_t)mN2 + mN4) { cls = 1; j = i - mN2; r = n2 + j; valid = j < n4; }
+    else if (i < (int64_t)mN2 + mN4 + mN8) { cls = 2; j = i - mN2 - mN4; r = n2 + n4 + j; valid = j < n8; }
+    else { cls = 3; j = i - mN2 - mN4 - mN8; r = n2 + n4 + n8 + j; valid = j < n16; }
+  };
+  if (d128) {
+    // all row loads of the wavefront go out before the first is used
+    __half xa[RDKV_PACK_V_ROWS_PER_WAVE], xb[RDKV_PACK_V_ROWS_PER_WAVE];
+#pragma unroll
+    for (int k = 0; k < RDKV_PACK_V_ROWS_PER_WAVE; ++k) {
+      int cls; int64_t j, r; bool valid;
+      xa[k] = xb[k] = __float2half_rn(0.0f);
+      if (i0 + k < total) {
+        locate(i0 + k, cls, j, r, valid);
+        if (valid) {
+          const __half *xr = Vh + (int64_t)ord[r] * stride_t;
+          xa[k] = xr[lane];
+          xb[k] = xr[lane + 64];
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < RDKV_PACK_V_ROWS_PER_WAVE; ++k) {
+      if (i0 + k >= total) break;
+      int cls; int64_t j, r; bool valid;
+      locate(i0 + k, cls, j, r, valid);
+      const float x0 = __half2float(xa[k]), x1 = __half2float(xb[k]);
+      if (cls == 0) {
+        uint8_t *o = V2 + ((int64_t)h * mN2 + j) * 32;
+        if (valid) quantize_values_d128<2>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 32);
+      } else if (cls == 1) {
+        uint8_t *o = V4 + ((int64_t)h * mN4 + j) * 64;
+        if (valid) quantize_values_d128<4>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 64);
+      } else if (cls == 2) {
+        uint8_t *o = V8 + ((int64_t)h * mN8 + j) * 128;
+        if (valid) quantize_values_d128<8>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 128);
+      } else {
+        __half *o = V16 + ((int64_t)h * max_n16 + j) * 128;
+        o[lane] = xa[k];          // zero when the row is padding
+        o[lane + 64] = xb[k];
+      }
+    }
+    return;
+  }
+  for (int64_t i = i0; i < i0 + RDKV_PACK_V_ROWS_PER_WAVE && i < total; ++i) {
+    int cls; int64_t j, r; bool valid;
+    locate(i, cls, j, r, valid);
+    const __half *xr = Vh + (valid ? (int64_t)ord[r] * stride_t : 0);
+    if (cls == 0) {
+      uint8_t *o = V2 + ((int64_t)h * mN2 + j) * (D >> 2);
+      if (valid) quantize_one_row<2>(xr, D, 1, lane, o, vsh + r, vzh + r); else zero_bytes(o, D >> 2);
+    } else if (cls == 1) {
+      uint8_t *o = V4 + ((int64_t)h * mN4 + j) * (D >> 1);
+      if (valid) quantize_one_row<4>(xr, D, 1, lane, o, vsh + r, vzh + r); else zero_bytes(o, D >> 1);
+    } else if (cls == 2) {
+      uint8_t *o = V8 + ((int64_t)h * mN8 + j) * D;
+      if (valid) quantize_one_row<8>(xr, D, 1, lane, o, vsh + r, vzh + r); else zero_bytes(o, D);
+    } else {
+      __half *o = V16 + ((int64_t)h * max_n16 + j) * D;
+      for (int c = lane; c < D; c += 64) o[c] = valid ? xr[c] : __float2half_rn(0.0f);
     }
   }
 }
@@ -189,6 +311,164 @@ k_quantize_pack_kernel(const __half *__restrict__ k, int64_t k_row_stride, int64
 }
 
 // ---------------------------------------------------------------------------
+// Whole-layer K side.  The reference re-quantizes K from a zero-padded canvas
+// [H_kv, max_tv + max_n16, D]: head h's compressed rows at [0,tv_h) in V's sorted order, its
+// fp16-zone rows at [max_tv, max_tv+n16_h), zeros elsewhere (packing.py:1186-1221).  Here the
+// canvas is never built: rows are gathered through `order`, and a head that has pad rows
+// folds 0 into its per-channel min/max.
+// ---------------------------------------------------------------------------
+#define RDKV_LAYER_MINMAX_ROWS 128
+__global__ void minmax_init_layer_kernel(uint32_t *mm, int D, int H) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < (int64_t)H * 2 * D)
+    mm[i] = rdkv_float_to_ordered(((i / D) & 1) ? -INFINITY : INFINITY);
+}
+
+__global__ void __launch_bounds__(256)
+k_minmax_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t, int D,
+                      const int32_t *__restrict__ order, int64_t order_stride_h,
+                      const int32_t *__restrict__ counts, uint32_t *__restrict__ mm) {
+  // blockDim = (64, 4): threadIdx.x walks column pairs, threadIdx.y walks rows.
+  const int h = blockIdx.y;
+  const int tk = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2] + counts[4 * h + 3];
+  const int64_t t0 = (int64_t)blockIdx.x * RDKV_LAYER_MINMAX_ROWS;
+  if (t0 >= tk) return;
+  const int64_t t1 = (t0 + RDKV_LAYER_MINMAX_ROWS < tk) ? t0 + RDKV_LAYER_MINMAX_ROWS : tk;
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Kh = K + (int64_t)h * stride_h;
+  uint32_t *mmh = mm + (int64_t)h * 2 * D;
+  __shared__ float s_mn[4][64 * 2 + 2];
+  __shared__ float s_mx[4][64 * 2 + 2];
+  for (int c0 = 0; c0 < D; c0 += 128) {
+    const int c = c0 + 2 * threadIdx.x;
+    float mn0 = INFINITY, mn1 = INFINITY, mx0 = -INFINITY, mx1 = -INFINITY;
+    if (c + 1 < D) {
+      for (int64_t t = t0 + threadIdx.y; t < t1; t += 4) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(Kh + (int64_t)ord[t] * stride_t + c);
+        const float a = __low2float(v), b = __high2float(v);
+        mn0 = fminf(mn0, a); mx0 = fmaxf(mx0, a);
+        mn1 = fminf(mn1, b); mx1 = fmaxf(mx1, b);
+      }
+    } else if (c < D) {
+      for (int64_t t = t0 + threadIdx.y; t < t1; t += 4) {
+        const float a = __half2float(Kh[(int64_t)ord[t] * stride_t + c]);
+        mn0 = fminf(mn0, a); mx0 = fmaxf(mx0, a);
+      }
+    }
+    s_mn[threadIdx.y][2 * threadIdx.x] = mn0; s_mn[threadIdx.y][2 * threadIdx.x + 1] = mn1;
+    s_mx[threadIdx.y][2 * threadIdx.x] = mx0; s_mx[threadIdx.y][2 * threadIdx.x + 1] = mx1;
+    __syncthreads();
+    if (threadIdx.y == 0) {
+      for (int k = 0; k < 2; ++k) {
+        const int cc = c + k;
+        if (cc < D) {
+          float a = s_mn[0][2 * threadIdx.x + k], b = s_mx[0][2 * threadIdx.x + k];
+          for (int y = 1; y < 4; ++y) {
+            a = fminf(a, s_mn[y][2 * threadIdx.x + k]);
+            b = fmaxf(b, s_mx[y][2 * threadIdx.x + k]);
+          }
+          atomicMin(&mmh[cc], rdkv_float_to_ordered(a));
+          atomicMax(&mmh[D + cc], rdkv_float_to_ordered(b));
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// One wavefront per canvas row: lanes read the row coalesced (channels l, l+64, ...), quantize
+// with their channel's parameters, scatter the codes to their sorted slots in an LDS row
+// buffer, then lanes assemble and store the packed bytes.
+__global__ void __launch_bounds__(256)
+k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t, int D,
+                    const int32_t *__restrict__ order, int64_t order_stride_h,
+                    const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
+                    const uint32_t *__restrict__ mm, const int32_t *__restrict__ slot_channel,
+                    int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
+                    uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
+                    __half *__restrict__ zp_out, int rows_per_block) {
+  // dynamic LDS: per channel {scale, zp, qmax} floats and slot (int), then one code row of
+  // Dp bytes (padded to 4) per wavefront
+  extern __shared__ float smem[];
+  const int h = blockIdx.y;
+  const int Dp = n2p + n4p + n8;
+  const int Dp4 = (Dp + 3) & ~3;
+  const int tv = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2], n16 = counts[4 * h + 3];
+  const bool has_pad = tv < max_tv || n16 < max_n16;   // zero rows of the canvas join the min/max
+  const int64_t max_tk = max_tv + max_n16;
+  float *c_scale = smem, *c_zp = smem + D, *c_qmax = smem + 2 * D;
+  int *c_slot = reinterpret_cast<int *>(smem + 3 * D);
+  uint8_t *rowbufs = reinterpret_cast<uint8_t *>(smem + 4 * D);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const uint32_t *mmh = mm + (int64_t)h * 2 * D;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) c_slot[c] = -1;
+  for (int i = threadIdx.x; i < nwaves * Dp4; i += blockDim.x) rowbufs[i] = 0;  // pad slots stay 0
+  __syncthreads();
+  for (int s = threadIdx.x; s < Dp; s += blockDim.x) {
+    const int ch = slot_channel[(int64_t)h * Dp + s];
+    const float qmax = s < n2p ? 3.0f : (s < n2p + n4p ? 15.0f : 255.0f);
+    float mn = 0.0f, mx = 0.0f;
+    if (ch >= 0) {
+      mn = rdkv_ordered_to_float(mmh[ch]);
+      mx = rdkv_ordered_to_float(mmh[D + ch]);
+      if (has_pad) {
+        mn = fminf(mn, 0.0f);
+        mx = fmaxf(mx, 0.0f);
+      }
+    }
+    const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
+    if (ch >= 0) {
+      c_scale[ch] = p.scale;
+      c_zp[ch] = p.zp;
+      c_qmax[ch] = qmax;
+      c_slot[ch] = s;
+    }
+    if (blockIdx.x == 0) {
+      scale_out[(int64_t)h * Dp + s] = __float2half_rn(p.scale);
+      zp_out[(int64_t)h * Dp + s] = __float2half_rn(p.zp);
+    }
+  }
+  __syncthreads();
+  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
+  const int rowbytes = sub2 + sub4 + n8;
+  if (rowbytes == 0) return;
+  const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t t1 = (t0 + rows_per_block < max_tk) ? t0 + rows_per_block : max_tk;
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Kh = K + (int64_t)h * stride_h;
+  uint8_t *rb = rowbufs + wave * Dp4;
+  for (int64_t t = t0 + wave; t < t1; t += nwaves) {
+    // canvas row -> source token (or a zero row)
+    const __half *kr = nullptr;
+    if (t < tv) kr = Kh + (int64_t)ord[t] * stride_t;
+    else if (t >= max_tv && t - max_tv < n16) kr = Kh + (int64_t)ord[tv + (t - max_tv)] * stride_t;
+    for (int c = lane; c < D; c += 64) {
+      const int slot = c_slot[c];
+      if (slot >= 0) {
+        RdkvQParams p;
+        p.scale = c_scale[c];
+        p.zp = c_zp[c];
+        rb[slot] = (uint8_t)rdkv_qcode(kr ? __half2float(kr[c]) : 0.0f, p, c_qmax[c]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    const int64_t row = (int64_t)h * max_tk + t;
+    for (int j = lane; j < rowbytes; j += 64) {
+      if (j < sub2) {
+        K2[row * sub2 + j] = (uint8_t)(rb[j] | (rb[j + sub2] << 2) | (rb[j + 2 * sub2] << 4) | (rb[j + 3 * sub2] << 6));
+      } else if (j < sub2 + sub4) {
+        const int i = j - sub2;
+        K4[row * sub4 + i] = (uint8_t)(rb[n2p + i] | (rb[n2p + i + sub4] << 4));
+      } else {
+        const int i = j - sub2 - sub4;
+        K8[row * (int64_t)n8 + i] = rb[n2p + n4p + i];
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Dequantize to fp16: out = half((code - zp) * scale), one thread per output element.
 // ---------------------------------------------------------------------------
 template <int BITS>
@@ -312,5 +592,65 @@ RDKV_API int rdkv_dequant_f16(const uint8_t *packed, int64_t rows, int n_cols_un
   else
     hipLaunchKernelGGL(dequant_f16_kernel<8>, g, b, 0, s, packed, rows, n_cols_unpacked, sc, zp, per_row, o, out_row_stride);
   RDKV_CHECK_LAUNCH("rdkv_dequant_f16");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
+                                      int H_kv, int D, const int32_t *order, int64_t order_stride_h,
+                                      const int32_t *counts, int mN2, int mN4, int mN8, int64_t max_tv,
+                                      int max_n16, const int32_t *slot_channel, int n2p, int n4p, int n8,
+                                      uint8_t *V2, uint8_t *V4, uint8_t *V8, void *V_scale_f16,
+                                      void *V_zp_f16, void *V16_f16, uint8_t *K2, uint8_t *K4, uint8_t *K8,
+                                      void *K_scale_f16, void *K_zp_f16, float *minmax_ws, void *stream) {
+  const char *fn = "rdkv_pack_layer_per_head";
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D > 0 && D % 4 == 0, "%s: bad H_kv=%d / D=%d", fn, H_kv, D);
+  RDKV_REQUIRE(mN2 >= 0 && mN4 >= 0 && mN8 >= 0 && max_n16 >= 0 && max_tv >= 0, "%s: negative counts", fn);
+  RDKV_REQUIRE(max_tv <= (int64_t)mN2 + mN4 + mN8, "%s: max_tv exceeds the class maxima", fn);
+  RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
+               "%s: bad segment sizes (%d,%d,%d)", fn, n2p, n4p, n8);
+  const int Dp = n2p + n4p + n8;
+  RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "%s: %d padded channels > %d", fn, Dp, RDKV_MAX_SLOTS);
+  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0,
+               "%s: rows must be 4-byte aligned", fn);
+  const int64_t v_rows = (int64_t)mN2 + mN4 + mN8 + max_n16;
+  const int64_t max_tk = max_tv + max_n16;
+  if (v_rows == 0 && max_tk == 0) return RDKV_OK;
+  RDKV_REQUIRE(K_f16 && V_f16 && order && counts, "%s: null input", fn);
+  RDKV_REQUIRE((mN2 == 0 || V2) && (mN4 == 0 || V4) && (mN8 == 0 || V8) && (max_n16 == 0 || V16_f16) &&
+                   (max_tv == 0 || (V_scale_f16 && V_zp_f16)),
+               "%s: null V output", fn);
+  hipStream_t s = (hipStream_t)stream;
+  if (v_rows > 0) {
+    const int waves = 4;
+    const int64_t blocks = rdkv_cdiv(v_rows, waves * RDKV_PACK_V_ROWS_PER_WAVE);
+    RDKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many rows", fn);
+    hipLaunchKernelGGL(pack_v_layer_kernel, dim3((unsigned)blocks, H_kv), dim3(64 * waves), 0, s,
+                       (const __half *)V_f16, stride_h, stride_t, D, order, order_stride_h, counts, mN2, mN4,
+                       mN8, max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16,
+                       (__half *)V16_f16);
+  }
+  if (Dp > 0 && max_tk > 0) {
+    RDKV_REQUIRE(slot_channel && minmax_ws && K_scale_f16 && K_zp_f16 && (n2p == 0 || K2) &&
+                     (n4p == 0 || K4) && (n8 == 0 || K8),
+                 "%s: null K output", fn);
+    uint32_t *mm = reinterpret_cast<uint32_t *>(minmax_ws);
+    // (+inf, -inf) in the ordered-int encoding, per head D mins then D maxes
+    hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256),
+                       0, s, mm, D, H_kv);
+    const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
+    RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
+    hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
+                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+    const int rows_per_block = 64;
+    const int64_t eblocks = rdkv_cdiv(max_tk, rows_per_block);
+    RDKV_REQUIRE(eblocks <= 0x7fffffffLL, "%s: too many rows", fn);
+    const size_t emit_lds = (size_t)D * 16 + 4 * (size_t)((Dp + 3) & ~3);
+    RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
+    hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
+                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv,
+                       max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
+                       (__half *)K_zp_f16, rows_per_block);
+  }
+  RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

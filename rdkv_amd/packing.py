@@ -614,11 +614,128 @@ def _pad_and_stack_per_head_layers(
     return packed, new_v_only
 
 
+_CLASS_TABLES = {}
+
+
+def _class_tables(dev):
+    """(v_bits -> class rank lookup, class rank list) on ``dev``, built once per device."""
+    t = _CLASS_TABLES.get(dev)
+    if t is None:
+        lut = torch.full((17,), 255, dtype=torch.uint8)
+        lut[torch.tensor([2, 4, 8, 16, 0])] = torch.arange(5, dtype=torch.uint8)
+        t = (lut.to(dev), torch.tensor([0, 1, 2, 3, 4, 255], dtype=torch.uint8).to(dev))
+        _CLASS_TABLES[dev] = t
+    return t
+
+
 def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,
                         gqa_factor: int) -> Tuple[PackedKVLayer, Optional[Tensor]]:
-    """The reference's per-layer prefill packing composition (obkv_fast.py:1141-1155): for every
-    KV head ``build_packed_layer`` on the kept tokens with deferred K, then
-    ``_pad_and_stack_per_head_layers``.  K, V [1,H_kv,T,D]; v_bits [H_kv,T]; k_bits [H_kv,D]."""
+    """Prefill packing of one layer with per-head allocations: the result of the reference's
+    composition (obkv_fast.py:1141-1155: per head ``build_packed_layer`` with deferred K,
+    packing.py:801-1013, then ``_pad_and_stack_per_head_layers``, packing.py:1019-1317),
+    bit for bit, without the per-head loop: one stable sort of the token classes, then
+    ``rdkv_pack_layer_per_head`` (V rows, K min/max, K emit).  K, V [1,H_kv,T,D] fp16;
+    v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
+    dev = _lib.require_device(K, V)
+    assert K.dim() == 4 and K.shape[0] == 1 and K.shape == V.shape, (
+        f"Expected K, V [1,H_kv,T,D], got {tuple(K.shape)} / {tuple(V.shape)}")
+    H_kv, T, D = int(K.shape[1]), int(K.shape[2]), int(K.shape[3])
+    assert tuple(v_bits_per_head.shape) == (H_kv, T) and tuple(k_bits_per_head.shape) == (H_kv, D)
+    if T == 0:
+        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
+    Kf, Vf = _as_f16_heads(K)[0], _as_f16_heads(V)[0]
+    if Vf.stride() != Kf.stride():
+        Kf, Vf = Kf.contiguous(), Vf.contiguous()
+    # class rank of every token: 2-bit 0, 4-bit 1, 8-bit 2, fp16 3, evicted 4 (255 = invalid)
+    lut, classes = _class_tables(dev)
+    vb = v_bits_per_head.to(dev)
+    key = lut[torch.where((vb >= 0) & (vb <= 16), vb, 1).long()]
+    order = torch.sort(key, dim=1, stable=True).indices.to(torch.int32)
+    counts = (key.unsqueeze(-1) == classes).sum(1)              # [H_kv, 6] on the device
+    counts_h = counts.cpu().tolist()                            # the one synchronization
+    assert all(row[5] == 0 for row in counts_h), "v_bits must be in {0,2,4,8,16}"
+    seg = [tuple(int(v) for v in row[:3]) for row in counts_h]
+    n16 = [int(row[3]) for row in counts_h]
+    tv = [sum(s3) for s3 in seg]
+    tk = [a + b for a, b in zip(tv, n16)]
+    max_tv, max_n16 = max(tv), max(n16)
+    max_tk = max_tv + max_n16
+    mN = [max(s3[i] for s3 in seg) for i in range(3)]
+    rows = k_bits_per_head.detach().cpu().tolist()
+    n_h, (m2, m4, m8) = _per_head_counts(rows)
+    sub2 = _seg_padded_len(m2, 4) // 4
+    sub4 = _seg_padded_len(m4, 2) // 2
+    Dp = 4 * sub2 + 2 * sub4 + m8
+    if max_tk == 0 or Dp == 0:
+        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
+    plans = [_plan_k_channels(rows[h], sub2 or None, sub4 or None, m8 or None, tuple(n_h[h]))
+             for h in range(H_kv)]
+    # all host-built index tables travel in one copy: [slot_channel | perm | sort | seg] per head
+    kept_max = max((len(p.ch_sort_idx) for p in plans), default=0)
+    table = torch.tensor([p.slot_channel + p.perm_padded + p.ch_sort_idx + [0] * (kept_max - len(p.ch_sort_idx))
+                          + list(n_h[h]) for h, p in enumerate(plans)], dtype=torch.long).to(dev)
+    slot_ch = table[:, :Dp].to(torch.int32).contiguous()
+    perm_ph = table[:, Dp:2 * Dp].contiguous()
+    sort_ph = table[:, 2 * Dp:2 * Dp + kept_max].contiguous()
+    seg_ph = table[:, 2 * Dp + kept_max:].to(torch.int32).contiguous()
+    counts_dev = counts[:, :4].to(torch.int32).contiguous()
+
+    def u8(n, w):
+        return torch.empty(1, H_kv, n, w, dtype=torch.uint8, device=dev) if n > 0 and w > 0 else None
+
+    V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
+    V_scale = torch.zeros(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)
+    V_zp = torch.zeros_like(V_scale)
+    new_v_only = (torch.empty(1, H_kv, max_n16, D, dtype=torch.float16, device=dev) if max_n16 > 0 else None)
+    K2, K4, K8 = u8(max_tk, sub2), u8(max_tk, sub4), u8(max_tk, m8)
+    ks = torch.empty(1, H_kv, 1, Dp, dtype=torch.float16, device=dev)
+    kz = torch.empty_like(ks)
+    mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().rdkv_pack_layer_per_head(
+        Kf.data_ptr(), Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D,
+        order.data_ptr(), order.stride(0), counts_dev.data_ptr(), mN[0], mN[1], mN[2], max_tv, max_n16,
+        slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8,
+        _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only),
+        _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(),
+        _lib.stream_of(dev)))
+
+    # metadata exactly as _pad_and_stack_per_head_layers / pack_k_mixed_per_head produce it
+    ref = next((h for h in range(H_kv) if tk[h] > 0), 0)
+    if tv[ref] > 0:      # pack_v_segments' argsort indexes the head's compressed tokens
+        rank = torch.cumsum((key[ref] < 3).to(torch.long), 0) - 1
+        sort_idx = rank[order[ref, :tv[ref]].long()]
+    else:
+        sort_idx = torch.empty(0, dtype=torch.long, device=dev)
+    tv_t = counts_dev[:, :3].sum(1, keepdim=True)
+    n16_t = counts_dev[:, 3:4]
+    col = torch.arange(max_tk, device=dev).unsqueeze(0)
+    valid = (col < tv_t) | ((col >= max_tv) & (col < max_tv + n16_t))
+    mask_kv = torch.zeros(H_kv, max_tk, dtype=torch.float32, device=dev)
+    mask_kv.masked_fill_(~valid, float("-inf"))
+    packed = PackedKVLayer(
+        K_2bit=K2, K_4bit=K4, K_8bit=K8, K_ch_scale=ks, K_ch_zp=kz, K_ch_sort_idx=sort_ph[0],
+        K_ch_seg_bounds=(m2, m4, m8), K_ch_perm_padded_idx=perm_ph[0],
+        V_2bit=V2, V_4bit=V4, V_8bit=V8, V_scale=V_scale, V_zp=V_zp,
+        sort_idx=sort_idx, seg_bounds=(mN[0], mN[1], mN[2]), T_eff=max_tv,
+        seg_bounds_per_head=counts_dev[:, :3].contiguous(),
+        T_eff_per_head=tv_t.reshape(H_kv).to(torch.int32),
+        softmax_mask=mask_kv.repeat_interleave(gqa_factor, dim=0).contiguous(),
+        n_fp16_per_head=None, fp16_gap_mask=None,
+        K_ch_sort_idx_per_head=sort_ph, K_ch_perm_padded_idx_per_head=perm_ph,
+        K_ch_seg_bounds_per_head=seg_ph,
+        K_ch_perm_padded_idx_for_Q=perm_ph.repeat_interleave(gqa_factor, dim=0),
+        T_eff_k=max_tk, n_v16=max_n16, T_eff_k_per_head=counts_dev.sum(1).to(torch.int32),
+        n_v16_per_head=counts_dev[:, 3].contiguous(), allocation_v_bits=None, allocation_k_bits=None)
+    return packed, new_v_only
+
+
+def _pack_layer_per_head_composed(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,
+                        gqa_factor: int) -> Tuple[PackedKVLayer, Optional[Tensor]]:
+    """The reference's per-layer prefill packing composition, call for call
+    (obkv_fast.py:1141-1155): for every KV head ``build_packed_layer`` on the kept tokens with
+    deferred K, then ``_pad_and_stack_per_head_layers``.  ``pack_layer_per_head`` produces the
+    same tensors in a handful of launches; this form is kept for degenerate layers and as its
+    cross-check."""
     dev = _lib.require_device(K, V)
     H_kv, D = K.shape[1], K.shape[3]
     vb_all = v_bits_per_head.detach().cpu()

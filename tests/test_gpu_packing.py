@@ -166,3 +166,51 @@ def test_config_shaped_layer_vs_oracle(cfg_idx, ctx):
     pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, cfg.G)
     assert_layers_equal(pl, ora)
     assert_bits_equal(t2n(nvo), ora_nvo)
+
+
+def _layers_identical(a, b):
+    import dataclasses
+    for f in dataclasses.fields(a):
+        x, y = getattr(a, f.name), getattr(b, f.name)
+        if torch.is_tensor(x) or torch.is_tensor(y):
+            assert torch.is_tensor(x) and torch.is_tensor(y), f.name
+            assert x.dtype == y.dtype and x.shape == y.shape, (f.name, x.dtype, y.dtype, x.shape, y.shape)
+            assert torch.equal(x.view(torch.uint8) if x.dtype == torch.float16 else x,
+                               y.view(torch.uint8) if y.dtype == torch.float16 else y), f.name
+        else:
+            assert x == y, (f.name, x, y)
+
+
+@pytest.mark.parametrize("case", ["ragged", "equal_counts", "empty_head", "fp16_only_head", "no_fp16",
+                                  "one_class", "strided_input"])
+def test_whole_layer_packer_matches_composition(case):
+    """The few-launch layer packer against the call-for-call composition it replaces (which is
+    itself pinned to the oracle and the golden vectors), on layouts that stress the padding."""
+    rng = np.random.default_rng(sum(map(ord, case)))
+    H, T, D, G = 3, 157, 128, 2
+    K = torch.randn(1, H, T, D, device=DEV).half()
+    V = torch.randn(1, H, T, D, device=DEV).half()
+    choices = np.array([0, 2, 4, 8, 16])
+    vb = torch.from_numpy(rng.choice(choices, size=(H, T)))
+    if case == "equal_counts":       # no head has pad rows: 0 must not join any min/max
+        row = rng.choice(choices, size=T)
+        vb = torch.from_numpy(np.stack([rng.permutation(row) for _ in range(H)]))
+        K = K.abs() + 1.0            # strictly positive, so a spurious 0 would change the codes
+    elif case == "empty_head":
+        vb[1] = 0
+    elif case == "fp16_only_head":
+        vb[0] = torch.from_numpy(rng.choice(np.array([0, 16]), size=T))
+    elif case == "no_fp16":
+        vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8]), size=(H, T)))
+    elif case == "one_class":
+        vb = torch.full((H, T), 4)
+    elif case == "strided_input":
+        big = torch.randn(1, H, T, 2 * D, device=DEV).half()
+        K, V = big[..., :D], big[..., D:]
+    kb = torch.from_numpy(rng.choice(np.array([0, 0, 2, 4, 8, 16]), size=(H, D)))
+    got, got_nvo = packing.pack_layer_per_head(K, V, vb, kb, G)
+    exp, exp_nvo = packing._pack_layer_per_head_composed(K, V, vb, kb, G)
+    _layers_identical(got, exp)
+    assert (got_nvo is None) == (exp_nvo is None)
+    if exp_nvo is not None:
+        assert torch.equal(got_nvo.view(torch.uint8), exp_nvo.view(torch.uint8))
