@@ -115,7 +115,7 @@ def main():
                              "relayout_ms_per_layer": float(np.median(relayout_ms[1:])),
                              "note": "wall time of packing.pack_layer_per_head (+ stream_cache.build_stream_cache) "
                                      "on layer 0, median of 5 after 1 warm-up; K is read twice (min/max pass, "
-                                     "then emit; the second read is served by the last-level cache at these sizes)"}
+                                     "then emit)"}
             del K, V
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
