@@ -1,6 +1,6 @@
 // Quarter-split 2-bit and half-split 4-bit pack/unpack on the last dimension
-// (reference: obkv_accel/bitpack.py:13-47).  Pure byte work, HBM bound: every thread
-// produces 4 output bytes from 4-byte loads where alignment allows.
+// (reference: obkv_accel/bitpack.py:13-47).  Pure byte work, HBM bound: one thread per
+// packed byte, consecutive threads on consecutive bytes of a row.
 #include "rdkv_common.h"
 
 namespace {

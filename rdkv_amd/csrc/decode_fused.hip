@@ -154,6 +154,9 @@ struct Smem {
   alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][2][4][4];  // [step][head group][hi|lo][head][k]
   alignas(16) _Float16 p[NW][16][NH][4][4];              // [wave][quad][head group][head][k]
   float bias[NH * 4];
+  float qraw[NH * 4][kD];                                // the unit's query rows as loaded
+  float slot_scale[4 * RDKV_MAX_STEPS], slot_zp[4 * RDKV_MAX_STEPS];
+  uint16_t slot_channel[4 * RDKV_MAX_STEPS];
   float wm[NW][NH * 4];
   float wl[NW][NH * 4];
   float wo[NW][4][kD];                                   // one head group at a time
@@ -286,18 +289,26 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // ---------------- prologue: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias ----------
   if (unit_index != staged_unit) {
     staged_unit = unit_index;
+    // The slot table and the query rows are fetched side by side (one memory latency, not a
+    // table -> gather chain) and combined from LDS.
     const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(qtab_base);
     const int nslot = 4 * NS;
+    for (int i = tid_o; i < nslot; i += kThreads) {
+      const RdkvSlot s = tab[i];
+      sm.slot_channel[i] = s.channel;
+      sm.slot_scale[i] = (float)__builtin_bit_cast(_Float16, s.scale_f16);
+      sm.slot_zp[i] = (float)__builtin_bit_cast(_Float16, s.zp_f16);
+    }
+    for (int i = tid_o; i < G * kD; i += kThreads)
+      sm.qraw[i >> 7][i & 127] = load_qv(q, q_dtype, (int64_t)(q_row + (i >> 7)) * q_stride + (i & 127));
+    __syncthreads();
     for (int i = tid_o; i < nslot * NH * 4; i += kThreads) {
       const int slot = i % nslot, head = i / nslot;
       _Float16 hi = (_Float16)0.0f, lo = (_Float16)0.0f;
       if (head < G) {
-        const RdkvSlot s = tab[slot];
-        const float sc = (float)__builtin_bit_cast(_Float16, s.scale_f16);
-        const float qv = load_qv(q, q_dtype, (int64_t)(q_row + head) * q_stride + s.channel);
         // two fp16 terms carry ~22 bits of q*scale: one fp16 alone loses the outlier channels'
         // low bits and costs ~1e-3 in the scores
-        const float x = qv * sc * (kLog2eOverSqrtD * kQScale);
+        const float x = sm.qraw[head][sm.slot_channel[slot]] * sm.slot_scale[slot] * (kLog2eOverSqrtD * kQScale);
         hi = (_Float16)x;
         lo = (_Float16)(x - (float)hi);
       }
@@ -308,11 +319,9 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     // bias[h] = sum_slot qs[h][slot] * zp[slot] / 2^8, one wavefront per head, fixed tree
     for (int head = wave; head < NH * 4; head += kWaves) {
       float b = 0.0f;
-      for (int slot = lane_o; slot < nslot; slot += 64) {
-        const float zp = (float)__builtin_bit_cast(_Float16, tab[slot].zp_f16);
+      for (int slot = lane_o; slot < nslot; slot += 64)
         b += ((float)sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] +
-              (float)sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3]) * zp;
-      }
+              (float)sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3]) * sm.slot_zp[slot];
       b = rdkv_wave_sum(b);
       if (lane_o == 0) sm.bias[head] = b * (1.0f / kQScale);
     }

@@ -69,7 +69,6 @@ def assert_layer_equal(actual, g, prefix, skip=()):
         assert tuple(got.shape) == tuple(exp.shape), f"{name}: shape {got.shape} != {exp.shape}"
         if exp.dtype.kind == "f":
             assert got.dtype == exp.dtype, f"{name}: dtype {got.dtype} != {exp.dtype}"
-            assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)) or np.array_equal(
-                got, exp, equal_nan=True), f"{name}: values differ"
+            assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), f"{name}: bits differ"
         else:
             assert np.array_equal(got.astype(np.int64), exp.astype(np.int64)), f"{name}: values differ"
