@@ -149,17 +149,20 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
   }
 }
 
+constexpr int kBatch = 2;  // work items a workgroup handles between two barriers
+
 template <int NH, int NW>
 struct Smem {
-  alignas(16) _Float16 qs[RDKV_MAX_STEPS][NH][2][4][4];  // [step][head group][hi|lo][head][k]
-  alignas(16) _Float16 p[NW][16][NH][4][4];              // [wave][quad][head group][head][k]
-  float bias[NH * 4];
-  float qraw[NH * 4][kD];                                // the unit's query rows as loaded
-  float slot_scale[4 * RDKV_MAX_STEPS], slot_zp[4 * RDKV_MAX_STEPS];
-  uint16_t slot_channel[4 * RDKV_MAX_STEPS];
-  float wm[NW][NH * 4];
-  float wl[NW][NH * 4];
-  float wo[NW][4][kD];                                   // one head group at a time
+  alignas(16) _Float16 qs[kBatch][RDKV_MAX_STEPS][NH][2][4][4];  // [item][step][head group][hi|lo][head][k]
+  alignas(16) _Float16 p[NW][16][NH][4][4];                      // [wave][quad][head group][head][k]
+  float bias[kBatch][NH * 4];
+  float qraw[kBatch][NH * 4][kD];                                // the unit's query rows as loaded
+  float slot_scale[kBatch][4 * RDKV_MAX_STEPS], slot_zp[kBatch][4 * RDKV_MAX_STEPS];
+  uint16_t slot_channel[kBatch][4 * RDKV_MAX_STEPS];
+  int progress[16];                                              // tiles done per wavefront
+  float wm[kBatch][NW][NH * 4];                                  // per-wavefront results of an item
+  float wl[kBatch][NW][NH * 4];
+  float wo[kBatch][NW][NH * 4][kD];
 };
 
 // Register images of the loads in flight.  KRegs: the K row of the lane's token and the
@@ -181,6 +184,13 @@ struct Cursor {  // wave-uniform position in the tile/piece sequence of this wav
   bool valid;
 };
 
+// Scalar description of one work item (all wave-uniform, read with scalar loads).
+struct Item {
+  int tile_begin, tile_end, d8, d4, d2, R, NS, n0, n1, n2, n3, ts1, ts2, ts3, q_row;
+  int nchunk_full, wc_last, nchunks;
+  const uint8_t *k_base, *sz_base, *v_base0, *v_base1, *v_base2, *v_base3, *qtab_base;
+};
+
 // Select by class without indexing an array (keeps everything in scalar registers).
 template <typename T>
 __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
@@ -189,6 +199,11 @@ __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
 
 // A workgroup fills a whole compute unit: 4 * WPE wavefronts (WPE per SIMD), all of the same
 // age, so the hardware's oldest-first issue order cannot favour one part of the work.
+// It walks the work items of its group kBatch at a time: the query operands of the batch are
+// staged first, then every wavefront runs through its tiles of all items of the batch without
+// waiting for the others (wavefronts drift apart by several tiles over an item; a barrier per
+// item cost 12-15 us of idle time each), parks its result per item in LDS, and one barrier
+// later the workgroup combines and writes the partials of the batch.
 template <int NH, int RMAX, int WPE>
 __global__ void __launch_bounds__(256 * WPE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
@@ -201,46 +216,43 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // the wavefront index is uniform; say so, or every tile-level decision becomes per-lane
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ln = lane & 3, lb = lane >> 2;
-  // a workgroup walks the work items of its group; consecutive items of one unit reuse the
-  // query operands already staged in LDS
   const int item_begin = groups ? groups[blockIdx.x] : (int)blockIdx.x;
   const int item_end = groups ? groups[blockIdx.x + 1] : (int)blockIdx.x + 1;
-  int staged_unit = -1;
-  for (int item = item_begin; item < item_end; ++item) {
-  // Index values used only before and after the tile loop are re-derived per item from an
-  // opaque copy of the thread id: hoisted out of the item loop they would stay live across
-  // the tile loop and push the kernel over its register budget.
-  int tid_o = tid;
-  asm volatile("" : "+v"(tid_o));
-  const int lane_o = tid_o & 63;
-  const RdkvWork *wkp = work + item;
-  const int tile_begin = wkp->tile_begin, tile_end = wkp->tile_end;
-  const int unit_index = wkp->unit;
-  const RdkvUnit *up = units + unit_index;
-  const int d8 = up->d8, d4 = up->d4, d2 = up->d2;
-  const int R = d8 + d4 + d2;
-  const int NS = d8 + 2 * d4 + 4 * d2;
-  const int n0 = up->n_tok[0], n1 = up->n_tok[1], n2 = up->n_tok[2], n3 = up->n_tok[3];
-  const int ts1 = (n0 + RDKV_TILE - 1) / RDKV_TILE;
-  const int ts2 = ts1 + (n1 + RDKV_TILE - 1) / RDKV_TILE;
-  const int ts3 = ts2 + (n2 + RDKV_TILE - 1) / RDKV_TILE;
-  // keep every address as `blob + offset` so the loads stay in the global address space
-  const uint8_t *k_base = blob + up->k_off, *sz_base = blob + up->sz_off;
-  const uint8_t *v_base0 = blob + up->v_off[0], *v_base1 = blob + up->v_off[1];
-  const uint8_t *v_base2 = blob + up->v_off[2], *v_base3 = blob + up->v_off[3];
-  const uint8_t *qtab_base = blob + up->qtab_off;
-  const int q_row = up->q_row;
-  const int nchunk_full = R >> 2, wc_last = R & 3;
 
+  auto load_item = [&](int item) -> Item {
+    const RdkvWork *wkp = work + item;
+    const RdkvUnit *up = units + wkp->unit;
+    Item it;
+    it.tile_begin = wkp->tile_begin;
+    it.tile_end = wkp->tile_end;
+    it.d8 = up->d8; it.d4 = up->d4; it.d2 = up->d2;
+    it.R = it.d8 + it.d4 + it.d2;
+    it.NS = it.d8 + 2 * it.d4 + 4 * it.d2;
+    it.n0 = up->n_tok[0]; it.n1 = up->n_tok[1]; it.n2 = up->n_tok[2]; it.n3 = up->n_tok[3];
+    it.ts1 = (it.n0 + RDKV_TILE - 1) / RDKV_TILE;
+    it.ts2 = it.ts1 + (it.n1 + RDKV_TILE - 1) / RDKV_TILE;
+    it.ts3 = it.ts2 + (it.n2 + RDKV_TILE - 1) / RDKV_TILE;
+    // keep every address as `blob + offset` so the loads stay in the global address space
+    it.k_base = blob + up->k_off; it.sz_base = blob + up->sz_off;
+    it.v_base0 = blob + up->v_off[0]; it.v_base1 = blob + up->v_off[1];
+    it.v_base2 = blob + up->v_off[2]; it.v_base3 = blob + up->v_off[3];
+    it.qtab_base = blob + up->qtab_off;
+    it.q_row = up->q_row;
+    it.nchunk_full = it.R >> 2; it.wc_last = it.R & 3;
+    it.nchunks = it.nchunk_full + (it.wc_last ? 1 : 0);
+    return it;
+  };
+
+  Item it;  // the item the tile loop is working on
   auto set_tile = [&](Cursor &c, int ti) {
     c.ti = ti;
     c.pc = 0;
-    c.valid = ti < tile_end;
-    const int cls = (ti >= ts1) + (ti >= ts2) + (ti >= ts3);
+    c.valid = ti < it.tile_end;
+    const int cls = (ti >= it.ts1) + (ti >= it.ts2) + (ti >= it.ts3);
     c.cls = cls;
-    const int tl = ti - sel4(cls, 0, ts1, ts2, ts3);
-    c.n_valid = sel4(cls, n0, n1, n2, n3) - tl * RDKV_TILE;  // tokens >= n_valid are padding
-    c.vtile = sel4(cls, v_base0, v_base1, v_base2, v_base3) + (uint64_t)tl * (uint64_t)(2048 << cls);
+    const int tl = ti - sel4(cls, 0, it.ts1, it.ts2, it.ts3);
+    c.n_valid = sel4(cls, it.n0, it.n1, it.n2, it.n3) - tl * RDKV_TILE;  // tokens >= n_valid are padding
+    c.vtile = sel4(cls, it.v_base0, it.v_base1, it.v_base2, it.v_base3) + (uint64_t)tl * (uint64_t)(2048 << cls);
     c.npc = cls < 2 ? 1 : (cls == 2 ? 2 : 4);  // V pieces of 16 dwords per lane (8 for 2-bit)
   };
   auto advance = [&](const Cursor &c) {
@@ -253,19 +265,19 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // The number of load instructions per stage is fixed (unused K chunks / V slots re-read an
   // address already being fetched, which the vector cache absorbs) so that the hardware load
   // counter can be waited on precisely while the next stage's loads are still in flight.
-  const int nchunks = nchunk_full + (wc_last ? 1 : 0);
   auto issue_k = [&](int ti, KRegs<RMAX> &r) {
-    const uint8_t *ktile = k_base + (uint64_t)ti * (RDKV_TILE * 4) * R;
+    const uint8_t *ktile = it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R;
 #pragma unroll
     for (int ch = 0; ch < RMAX / 4; ++ch) {
-      const int che = ch < nchunks ? ch : 0;
-      const int wce = che == nchunk_full ? wc_last : 4;
+      const int che = ch < it.nchunks ? ch : 0;
+      const int wce = che == it.nchunk_full ? it.wc_last : 4;
       // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
       // the next token (or the region that follows) and are never used
       const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
       r.k[4 * ch] = v.x; r.k[4 * ch + 1] = v.y; r.k[4 * ch + 2] = v.z; r.k[4 * ch + 3] = v.w;
     }
-    r.sz = *reinterpret_cast<const uint4 *>(sz_base + (ti < ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0));
+    r.sz = *reinterpret_cast<const uint4 *>(
+        it.sz_base + (ti < it.ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0));
   };
   auto issue_v = [&](const Cursor &c, VRegs &r) {
     const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
@@ -276,59 +288,86 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     r.v[3] = ld16_stream(vt + hi + 64);
   };
 
-  // The first tile's loads go out before anything else so that they overlap the prologue.
   KRegs<RMAX> kr;
   VRegs va, vb;
   Cursor c0;
-  set_tile(c0, tile_begin + wave);
-  if (c0.valid) {
-    issue_k(c0.ti, kr);
-    issue_v(c0, va);
-  }
+  // Load an item's description and put its first tile's loads in flight.
+  auto start_item = [&](int item) {
+    it = load_item(item);
+    set_tile(c0, it.tile_begin + wave);
+    if (c0.valid) {
+      issue_k(c0.ti, kr);
+      issue_v(c0, va);
+    }
+  };
 
-  // ---------------- prologue: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias ----------
-  if (unit_index != staged_unit) {
-    staged_unit = unit_index;
-    // The slot table and the query rows are fetched side by side (one memory latency, not a
-    // table -> gather chain) and combined from LDS.
-    const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(qtab_base);
-    const int nslot = 4 * NS;
+  for (int batch = item_begin; batch < item_end; batch += kBatch) {
+  const int nb = item_end - batch < kBatch ? item_end - batch : kBatch;
+  // Index values used only before and after the tile loops are re-derived per batch from a
+  // fresh read of the lane id: hoisted out of the loop (or derived from the thread id the
+  // kernel was entered with) they would stay live across the tile loops and push the kernel
+  // over its register budget.
+  int lane_o;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_o));
+  const int tid_o = wave * 64 + lane_o;
+
+  // The first item's first loads go out before anything else so that they overlap the staging.
+  start_item(batch);
+
+  // ---------------- staging: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias, per item ---
+  // The slot tables and the query rows of all items are fetched side by side (one memory
+  // latency, not a table -> gather chain) and combined from LDS.
+  for (int b = 0; b < nb; ++b) {
+    const Item sb = load_item(batch + b);
+    const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(sb.qtab_base);
+    const int nslot = 4 * sb.NS;
     for (int i = tid_o; i < nslot; i += kThreads) {
-      const RdkvSlot s = tab[i];
-      sm.slot_channel[i] = s.channel;
-      sm.slot_scale[i] = (float)__builtin_bit_cast(_Float16, s.scale_f16);
-      sm.slot_zp[i] = (float)__builtin_bit_cast(_Float16, s.zp_f16);
+      const RdkvSlot sl = tab[i];
+      sm.slot_channel[b][i] = sl.channel;
+      sm.slot_scale[b][i] = (float)__builtin_bit_cast(_Float16, sl.scale_f16);
+      sm.slot_zp[b][i] = (float)__builtin_bit_cast(_Float16, sl.zp_f16);
     }
     for (int i = tid_o; i < G * kD; i += kThreads)
-      sm.qraw[i >> 7][i & 127] = load_qv(q, q_dtype, (int64_t)(q_row + (i >> 7)) * q_stride + (i & 127));
-    __syncthreads();
+      sm.qraw[b][i >> 7][i & 127] =
+          load_qv(q, q_dtype, (int64_t)(sb.q_row + (i >> 7)) * q_stride + (i & 127));
+  }
+  __syncthreads();
+  for (int b = 0; b < nb; ++b) {
+    const int nslot = 4 * load_item(batch + b).NS;
     for (int i = tid_o; i < nslot * NH * 4; i += kThreads) {
       const int slot = i % nslot, head = i / nslot;
       _Float16 hi = (_Float16)0.0f, lo = (_Float16)0.0f;
       if (head < G) {
         // two fp16 terms carry ~22 bits of q*scale: one fp16 alone loses the outlier channels'
         // low bits and costs ~1e-3 in the scores
-        const float x = sm.qraw[head][sm.slot_channel[slot]] * sm.slot_scale[slot] * (kLog2eOverSqrtD * kQScale);
+        const float x = sm.qraw[b][head][sm.slot_channel[b][slot]] * sm.slot_scale[b][slot] *
+                        (kLog2eOverSqrtD * kQScale);
         hi = (_Float16)x;
         lo = (_Float16)(x - (float)hi);
       }
-      sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] = hi;
-      sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3] = lo;
+      sm.qs[b][slot >> 2][head >> 2][0][head & 3][slot & 3] = hi;
+      sm.qs[b][slot >> 2][head >> 2][1][head & 3][slot & 3] = lo;
     }
-    __syncthreads();
-    // bias[h] = sum_slot qs[h][slot] * zp[slot] / 2^8, one wavefront per head, fixed tree
-    for (int head = wave; head < NH * 4; head += kWaves) {
-      float b = 0.0f;
-      for (int slot = lane_o; slot < nslot; slot += 64)
-        b += ((float)sm.qs[slot >> 2][head >> 2][0][head & 3][slot & 3] +
-              (float)sm.qs[slot >> 2][head >> 2][1][head & 3][slot & 3]) * sm.slot_zp[slot];
-      b = rdkv_wave_sum(b);
-      if (lane_o == 0) sm.bias[head] = b * (1.0f / kQScale);
-    }
-    __syncthreads();
   }
+  __syncthreads();
+  // bias[h] = sum_slot qs[h][slot] * zp[slot] / 2^8, one wavefront per (item, head), fixed tree
+  for (int bh = wave; bh < nb * NH * 4; bh += kWaves) {
+    const int b = bh / (NH * 4), head = bh - b * (NH * 4);
+    const int nslot = 4 * load_item(batch + b).NS;
+    float bsum = 0.0f;
+    for (int slot = lane_o; slot < nslot; slot += 64)
+      bsum += ((float)sm.qs[b][slot >> 2][head >> 2][0][head & 3][slot & 3] +
+               (float)sm.qs[b][slot >> 2][head >> 2][1][head & 3][slot & 3]) * sm.slot_zp[b][slot];
+    bsum = rdkv_wave_sum(bsum);
+    if (lane_o == 0) sm.bias[b][head] = bsum * (1.0f / kQScale);
+  }
+  __syncthreads();
 
-  // ---------------- per-wavefront online-softmax state -----------------------------------
+  // ---------------- tiles: every item of the batch, no barrier in between ------------------
+  int tiles_done = 0;
+  if (lane == 0) sm.progress[wave] = 0;
+  for (int b = 0; b < nb; ++b) {
+  // per-wavefront online-softmax state
   float m_run[NH], l_run[NH], zb_run[NH];  // for head 4*hg + ln (own column)
   // One accumulator set: rows = heads of group, column = channel lane+64*j.  It is in the
   // quantized classes' scaling (2^-18) until the wavefront reaches its first fp16 tile, then
@@ -342,12 +381,16 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     m_run[hg] = -INFINITY;
     l_run[hg] = 0.0f;
     zb_run[hg] = 0.0f;
-    bias_own[hg] = sm.bias[hg * 4 + ln];
+    bias_own[hg] = sm.bias[b][hg * 4 + ln];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       accq[hg][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
   }
+  const _Float16 *qs_item = &sm.qs[b][0][0][0][0][0];
+  auto qs_op = [&](int step, int hg, int part) -> const _Float16 * {
+    return qs_item + (((step * NH + hg) * 2 + part) * 4 + ln) * 4;
+  };
 
   auto p_op = [&](int quad, int hg) -> half4_t {
     return *reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]);
@@ -355,6 +398,22 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 
   auto compute = [&](const Cursor &c, const VRegs &r) {
     if (c.pc == 0) {
+      // Progress feedback: the hardware issues oldest-wavefront-first, which lets the
+      // wavefronts of a workgroup drift 20% apart over an item.  Every wavefront publishes
+      // its tile count and takes a priority that grows with the number of wavefronts ahead
+      // of it (stale reads are harmless).
+      {
+        if (lane == 0) sm.progress[wave] = tiles_done;
+        const int other = sm.progress[lane & 15];
+        const unsigned long long ahead = __ballot(lane < kWaves && other > tiles_done);
+        switch ((__popcll(ahead) * 4) / kWaves) {
+          case 0: __builtin_amdgcn_s_setprio(0); break;
+          case 1: __builtin_amdgcn_s_setprio(1); break;
+          case 2: __builtin_amdgcn_s_setprio(2); break;
+          default: __builtin_amdgcn_s_setprio(3); break;
+        }
+        ++tiles_done;
+      }
       // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
       floatx4 sacc[NH];
 #pragma unroll
@@ -364,7 +423,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       for (int j = 0; j < RMAX; ++j) {
         // compare right here, every tile: hoisted, the 3 * RMAX loop-invariant comparisons no
         // longer fit the scalar registers and come back through lane reads
-        int R_o = R, d8_o = d8, d84_o = d8 + d4;
+        int R_o = it.R, d8_o = it.d8, d84_o = it.d8 + it.d4;
         asm volatile("" : "+s"(R_o), "+s"(d8_o), "+s"(d84_o));
         if (j < R_o) {
           const uint32_t w = kr.k[j];
@@ -372,8 +431,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
             const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
 #pragma unroll
             for (int hg = 0; hg < NH; ++hg) {
-              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][0][ln][0]), sacc[hg]);
-              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step][hg][1][ln][0]), sacc[hg]);
+              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step, hg, 0)), sacc[hg]);
+              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step, hg, 1)), sacc[hg]);
             }
             step += 1;
           } else if (j < d84_o) {
@@ -382,8 +441,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
               const half4_t a = mk_op((w >> (8 * s)) & 0x000F000Fu, (w >> (8 * s + 4)) & 0x000F000Fu);
 #pragma unroll
               for (int hg = 0; hg < NH; ++hg) {
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][0][ln][0]), sacc[hg]);
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][1][ln][0]), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 0)), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 1)), sacc[hg]);
               }
             }
             step += 2;
@@ -393,8 +452,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
               const half4_t a = mk_op((w >> (4 * s)) & 0x00030003u, (w >> (4 * s + 2)) & 0x00030003u);
 #pragma unroll
               for (int hg = 0; hg < NH; ++hg) {
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][0][ln][0]), sacc[hg]);
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(&sm.qs[step + s][hg][1][ln][0]), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 0)), sacc[hg]);
+                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 1)), sacc[hg]);
               }
             }
             step += 4;
@@ -415,7 +474,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       }
       // the K registers are free now: request this wavefront's next tile (at the end of the
       // work item the same tile again, so the number of loads in flight stays fixed)
-      issue_k(c.ti + kWaves < tile_end ? c.ti + kWaves : c.ti, kr);
+      issue_k(c.ti + kWaves < it.tile_end ? c.ti + kWaves : c.ti, kr);
       bool grew = false;
       float s2[NH][4], m_new[NH];
 #pragma unroll
@@ -539,62 +598,64 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // V pieces are requested one stage ahead into alternating buffers, K rows one tile ahead.
   // Past the last stage the same piece is requested again instead of branching, so every
   // stage issues the same number of loads and the waits on the load counter stay exact.
-  {
-    while (c0.valid) {
-      const Cursor c1 = advance(c0);
-      issue_v(c1.valid ? c1 : c0, vb);
-      compute(c0, va);
-      if (!c1.valid) break;
-      const Cursor c2 = advance(c1);
-      issue_v(c2.valid ? c2 : c1, va);
-      compute(c1, vb);
-      c0 = c2;
-    }
+  while (c0.valid) {
+    const Cursor c1 = advance(c0);
+    issue_v(c1.valid ? c1 : c0, vb);
+    compute(c0, va);
+    if (!c1.valid) break;
+    const Cursor c2 = advance(c1);
+    issue_v(c2.valid ? c2 : c1, va);
+    compute(c1, vb);
+    c0 = c2;
   }
 
-  // ---------------- merge the wavefront states and write the partial ---------------------
-  float *part = partials + (int64_t)item * G * kPartialStride;
+  // ---------------- park this wavefront's result of the item ------------------------------
 #pragma unroll
   for (int hg = 0; hg < NH; ++hg) {
     const float l_tot = quadcol_sum(l_run[hg]);
     const float zb_tot = quadcol_sum(zb_run[hg]) * (1.0f / kPScaleQ);
-    if (hg > 0) __syncthreads();  // the previous head group's rows have been read
     if (lane_o < 4) {
-      sm.wm[wave][hg * 4 + lane_o] = m_run[hg];
-      sm.wl[wave][hg * 4 + lane_o] = l_tot;
+      sm.wm[b][wave][hg * 4 + lane_o] = m_run[hg];
+      sm.wl[b][wave][hg * 4 + lane_o] = l_tot;
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const float zb = __shfl(zb_tot, r, 64);
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        sm.wo[wave][r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : kOBackQ) - zb;
+        sm.wo[b][wave][hg * 4 + r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : kOBackQ) - zb;
     }
-    __syncthreads();
-    for (int i = tid_o; i < 4 * kD; i += kThreads) {
-      const int r = i >> 7, d = i & 127, h = hg * 4 + r;
-      if (h < G) {
-        float M = sm.wm[0][h];
+  }
+  // straight on to the next item of the batch: its first loads go out now
+  if (b + 1 < nb) start_item(batch + b + 1);
+  }  // items of the batch
+  __syncthreads();
+
+  // ---------------- combine the wavefront results and write the partials ------------------
+  for (int b = 0; b < nb; ++b) {
+    float *part = partials + (int64_t)(batch + b) * G * kPartialStride;
+    for (int i = tid_o; i < G * kD; i += kThreads) {
+      const int h = i >> 7, d = i & 127;
+      float M = sm.wm[b][0][h];
 #pragma unroll
-        for (int w = 1; w < kWaves; ++w) M = fmaxf(M, sm.wm[w][h]);
-        float o = 0.0f, l = 0.0f;
+      for (int w = 1; w < kWaves; ++w) M = fmaxf(M, sm.wm[b][w][h]);
+      float o = 0.0f, l = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) {
-          const float mw = sm.wm[w][h];
-          const float f = mw == -INFINITY ? 0.0f : exp2f(mw - M);  // idle wavefront contributes nothing
-          o += f * sm.wo[w][r][d];
-          l += f * sm.wl[w][h];
-        }
-        part[h * kPartialStride + d] = o;
-        if (d == 0) {
-          part[h * kPartialStride + 128] = M;
-          part[h * kPartialStride + 129] = l;
-        }
+      for (int w = 0; w < kWaves; ++w) {
+        const float mw = sm.wm[b][w][h];
+        const float f = mw == -INFINITY ? 0.0f : exp2f(mw - M);  // idle wavefront contributes nothing
+        o += f * sm.wo[b][w][h][d];
+        l += f * sm.wl[b][w][h];
+      }
+      part[h * kPartialStride + d] = o;
+      if (d == 0) {
+        part[h * kPartialStride + 128] = M;
+        part[h * kPartialStride + 129] = l;
       }
     }
   }
-  __syncthreads();  // the next item overwrites the LDS state read above
-  }  // items of this group
+  __syncthreads();  // the next batch overwrites the LDS state read above
+  }  // batches of this group
 }
 
 // One workgroup per unit combines its partials (second launch of a step).  Merging inside the
@@ -650,18 +711,23 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   // keeps everything in registers; spilling costs far more than the lost occupancy.
   // RDKV_FUSED_WPE overrides it (2, 3 or 4) for experiments.
   static const int wpe_env = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 0;
+#define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE)                                                               \
+  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE>), dim3(n_wg), dim3(256 * WPE), 0, s, blob, units, \
+                     work, groups, q, q_dtype, q_stride_row, G, partials)
+  // one head group: 2..4 wavefronts per SIMD
 #define RDKV_LAUNCH_FUSED(NH, RMAX, WPE_DEFAULT)                                                           \
   do {                                                                                                     \
     const int wpe = wpe_env ? wpe_env : WPE_DEFAULT;                                                       \
-    if (wpe >= 4)                                                                                          \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 4>), dim3(n_wg), dim3(1024), 0, s, blob, units,    \
-                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
-    else if (wpe == 3)                                                                                     \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 3>), dim3(n_wg), dim3(768), 0, s, blob, units,     \
-                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
-    else                                                                                                   \
-      hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, 2>), dim3(n_wg), dim3(512), 0, s, blob, units,     \
-                         work, groups, q, q_dtype, q_stride_row, G, partials);                             \
+    if (wpe >= 4) RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 4);                                                      \
+    else if (wpe == 3) RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 3);                                                 \
+    else RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 2);                                                               \
+  } while (0)
+  // two head groups: the per-wavefront result buffers of 16 wavefronts would not fit in LDS
+#define RDKV_LAUNCH_FUSED2(RMAX, WPE_DEFAULT)                                                              \
+  do {                                                                                                     \
+    const int wpe = wpe_env ? wpe_env : WPE_DEFAULT;                                                       \
+    if (wpe >= 3) RDKV_LAUNCH_FUSED_WPE(2, RMAX, 3);                                                       \
+    else RDKV_LAUNCH_FUSED_WPE(2, RMAX, 2);                                                                \
   } while (0)
   if (G <= 4) {
     if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12, 4);
@@ -669,11 +735,13 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
     else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(1, 20, 4);
     else RDKV_LAUNCH_FUSED(1, 32, 3);
   } else {
-    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(2, 12, 3);
-    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(2, 16, 3);
-    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(2, 20, 3);
-    else RDKV_LAUNCH_FUSED(2, 32, 2);
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED2(12, 3);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED2(16, 3);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED2(20, 3);
+    else RDKV_LAUNCH_FUSED2(32, 2);
   }
+#undef RDKV_LAUNCH_FUSED2
+#undef RDKV_LAUNCH_FUSED_WPE
 #undef RDKV_LAUNCH_FUSED
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
