@@ -210,3 +210,33 @@ def test_fused_empty_unit_and_lse_merge():
     # K is re-quantized per source (per-channel ranges differ), so compare loosely to the
     # single-source result and tightly to the two-source oracle
     assert float((merged - out[:2]).abs().max()) < 5e-2
+
+
+def test_fused_attention_under_graph_replay():
+    """The fused step captured into a HIP graph: every replay, with eager work and
+    synchronizations in between and a changed query, matches the eager result bit for bit."""
+    cfg = synth.scaled(synth.CONFIGS[1], context=2000, layers=2)
+    packed, q, _ = _config_case(cfg, 2)
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    q_static = q.clone()
+    out_g = torch.empty(cache.rows, 128, device=DEV)
+    lse_g = torch.empty(cache.rows, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        stream_cache.decode_attn_fused(cache, q_static, out_g, lse_g)     # workspace exists before capture
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            stream_cache.decode_attn_fused(cache, q_static, out_g, lse_g)
+    torch.cuda.current_stream().wait_stream(side)
+    gen = torch.Generator().manual_seed(5)
+    for rep in range(4):
+        q_new = torch.randn(q.shape, generator=gen).half().to(DEV)
+        q_static.copy_(q_new)
+        out_g.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        exp_out, exp_lse = stream_cache.decode_attn_fused(cache, q_new)   # eager, default stream
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, exp_out) and torch.equal(lse_g, exp_lse), f"replay {rep}"
