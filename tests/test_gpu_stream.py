@@ -240,3 +240,23 @@ def test_fused_attention_under_graph_replay():
         exp_out, exp_lse = stream_cache.decode_attn_fused(cache, q_new)   # eager, default stream
         torch.cuda.synchronize()
         assert torch.equal(out_g, exp_out) and torch.equal(lse_g, exp_lse), f"replay {rep}"
+
+
+@pytest.mark.parametrize("cfg_idx", [1, 3])
+def test_fused_attention_full_size_layer(cfg_idx):
+    """One layer at the configuration's full context (32k for C1, 128k with 8 query heads per
+    KV head for C3), packed on the GPU, against the CPU oracle of the same packed layer."""
+    import dataclasses
+    cfg = synth.scaled(synth.CONFIGS[cfg_idx], layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, q = synth.layer_data(cfg, 0, DEV, outliers=oc)
+    pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+    del K, V
+    cache = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
+    out, lse = stream_cache.decode_attn_fused(cache, q)
+    kw = {f.name: (t2n(getattr(pl, f.name)) if torch.is_tensor(getattr(pl, f.name)) else getattr(pl, f.name))
+          for f in dataclasses.fields(O.PackedKVLayer)}
+    exp_out, exp_lse, _ = O.decode_attn_ref(t2n(q), O.PackedKVLayer(**kw), t2n(nvo) if nvo is not None else None)
+    attn_close(t2n(out), exp_out, "out")
+    attn_close(t2n(lse), exp_lse, "lse")
+    assert cache.n_groups >= 128      # the layer alone already spreads over the compute units
