@@ -174,7 +174,8 @@ def main():
         _lib.check(lib.rdkv_decode_fused_partials(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
             _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
-            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, ws.data_ptr(), ws.numel(), stream))
+            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, None, None, 0,
+            ws.data_ptr(), ws.numel(), stream))
 
     partials_only()
     ms_kernel = time_region(partials_only, args.steps, torch)

@@ -144,6 +144,15 @@ int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, int H_kv,
                         float *out, int64_t out_stride_h,
                         void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- triton_rope.py : fused_rope (:86-108) -------------------------------- */
+/* Half-split rotary embedding of one decode step, in place: for every head of q [H_q, D] and
+ * k [H_kv, D] (dtype code `dtype`, head strides in elements) and i < D/2:
+ * x[i], x[i+D/2] <- x[i]*cos[i] - x[i+D/2]*sin[i], x[i+D/2]*cos[i] + x[i]*sin[i], computed in
+ * fp32 without fused multiply-add and rounded to `dtype`.  cos_half / sin_half: D/2 values of
+ * cs_dtype. */
+int rdkv_rope(void *q, int64_t q_stride_h, int H_q, void *k, int64_t k_stride_h, int H_kv, int D,
+              int dtype, const void *cos_half, const void *sin_half, int cs_dtype, void *stream);
+
 /* ---- streaming format + fused flash-decoding kernel ------------------------------------
  * No counterpart in the reference as an interface: it replaces the sequence
  * k_mixed_qk_dot -> +softmax_mask -> softmax -> v_dequant_weighted_sum_dispatch of
@@ -198,6 +207,9 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
  * without tokens), so callers can merge further zones exactly.  G = query heads per KV head
  * (1..8).  max_row_dwords = max over units of d8+d4+d2 (<= 32; selects the register budget of
  * the kernel).  workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes.
+ * rope_cos / rope_sin: NULL, or D/2 = 64 values of rope_dtype each: the query rows are then
+ * rotated on the fly exactly as rdkv_rope would have rewritten them (rounded to q_dtype), so
+ * the caller passes the un-rotated projection output and skips that launch.
  * groups: int32 [n_groups + 1] ascending offsets into the work list; workgroup g of the
  * streaming launch processes work items groups[g] .. groups[g+1]-1 one after the other (items
  * of one unit should be adjacent: the staged query operands are reused).  Size the table so
@@ -209,6 +221,7 @@ int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G);
 int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
                       const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
                       int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
+                      const void *rope_cos, const void *rope_sin, int rope_dtype,
                       float *out, int64_t out_stride_row, float *lse,
                       void *workspace, int64_t workspace_bytes, void *stream);
 /* The two launches of rdkv_decode_fused as separate calls (same arguments): the streaming
@@ -217,7 +230,8 @@ int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units,
 int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
                                const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
                                int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row,
-                               int G, void *workspace, int64_t workspace_bytes, void *stream);
+                               int G, const void *rope_cos, const void *rope_sin, int rope_dtype,
+                               void *workspace, int64_t workspace_bytes, void *stream);
 int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G,
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);

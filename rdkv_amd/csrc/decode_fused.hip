@@ -21,6 +21,7 @@
 // sum_t p'_t*zp_t per head next to the MFMA accumulators.
 // HBM-bound by design: the MFMA and VALU work per byte is far below the machine balance.
 #include "rdkv_common.h"
+#include "rope_device.h"
 #include "stream_format.h"
 
 #include <stdlib.h>
@@ -209,6 +210,7 @@ __global__ void __launch_bounds__(256 * WPE) __attribute__((amdgpu_waves_per_eu(
 decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
                     const RdkvWork *__restrict__ work, const int32_t *__restrict__ groups,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride, int G,
+                    const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
                     float *__restrict__ partials) {
   constexpr int kWaves = 4 * WPE, kThreads = 64 * kWaves;
   __shared__ Smem<NH, kWaves> sm;
@@ -327,9 +329,23 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       sm.slot_scale[b][i] = (float)__builtin_bit_cast(_Float16, sl.scale_f16);
       sm.slot_zp[b][i] = (float)__builtin_bit_cast(_Float16, sl.zp_f16);
     }
-    for (int i = tid_o; i < G * kD; i += kThreads)
-      sm.qraw[b][i >> 7][i & 127] =
-          load_qv(q, q_dtype, (int64_t)(sb.q_row + (i >> 7)) * q_stride + (i & 127));
+    for (int i = tid_o; i < G * kD; i += kThreads) {
+      const int c = i & 127;
+      const int64_t row = (int64_t)(sb.q_row + (i >> 7)) * q_stride;
+      float v = load_qv(q, q_dtype, row + c);
+      if (rope_cos) {
+        // rotary embedding of the query on the fly (triton_rope.py:36-77): what the reference
+        // writes back to q in its storage type before the K kernel reads it
+        const float other = load_qv(q, q_dtype, row + (c ^ 64));
+        const float cs = rdkv_load_as_float(rope_cos, rope_dtype, c & 63);
+        const float sn = rdkv_load_as_float(rope_sin, rope_dtype, c & 63);
+        float out_lo, out_hi;
+        if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
+        else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
+        v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+      }
+      sm.qraw[b][i >> 7][c] = v;
+    }
   }
   __syncthreads();
   for (int b = 0; b < nb; ++b) {
@@ -694,8 +710,11 @@ static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, 
 static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *units, int n_units,
                         const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
                         int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
-                        void *workspace, int64_t workspace_bytes, void *stream) {
+                        const void *rope_cos, const void *rope_sin, int rope_dtype, void *workspace,
+                        int64_t workspace_bytes, void *stream) {
   int rc = check_fused_args(fn, units, n_units, work, n_work, G, workspace, workspace_bytes);
+  RDKV_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), "%s: rope_cos and rope_sin go together", fn);
+  RDKV_REQUIRE(!rope_cos || (rope_dtype >= 0 && rope_dtype <= 2), "%s: unknown rope dtype %d", fn, rope_dtype);
   if (rc != RDKV_OK) return rc;
   RDKV_REQUIRE(groups ? n_groups >= 1 : n_groups == 0, "%s: n_groups=%d does not match the group table", fn,
                n_groups);
@@ -713,7 +732,7 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   static const int wpe_env = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 0;
 #define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE)                                                               \
   hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE>), dim3(n_wg), dim3(256 * WPE), 0, s, blob, units, \
-                     work, groups, q, q_dtype, q_stride_row, G, partials)
+                     work, groups, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, partials)
   // one head group: 2..4 wavefronts per SIMD
 #define RDKV_LAUNCH_FUSED(NH, RMAX, WPE_DEFAULT)                                                           \
   do {                                                                                                     \
@@ -750,10 +769,12 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
 RDKV_API int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n_units,
                                         const RdkvWork *work, int n_work, const int32_t *groups,
                                         int n_groups, int max_row_dwords, const void *q, int q_dtype,
-                                        int64_t q_stride_row, int G, void *workspace,
+                                        int64_t q_stride_row, int G, const void *rope_cos,
+                                        const void *rope_sin, int rope_dtype, void *workspace,
                                         int64_t workspace_bytes, void *stream) {
   return launch_fused("rdkv_decode_fused_partials", blob, units, n_units, work, n_work, groups, n_groups,
-                      max_row_dwords, q, q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
+                      max_row_dwords, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, workspace,
+                      workspace_bytes, stream);
 }
 
 RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G, float *out,
@@ -772,11 +793,13 @@ RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_w
 
 RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n_units, const RdkvWork *work,
                                int n_work, const int32_t *groups, int n_groups, int max_row_dwords,
-                               const void *q, int q_dtype, int64_t q_stride_row, int G, float *out,
+                               const void *q, int q_dtype, int64_t q_stride_row, int G,
+                               const void *rope_cos, const void *rope_sin, int rope_dtype, float *out,
                                int64_t out_stride_row, float *lse, void *workspace, int64_t workspace_bytes,
                                void *stream) {
   int rc = rdkv_decode_fused_partials(blob, units, n_units, work, n_work, groups, n_groups, max_row_dwords, q,
-                                      q_dtype, q_stride_row, G, workspace, workspace_bytes, stream);
+                                      q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, workspace,
+                                      workspace_bytes, stream);
   if (rc != RDKV_OK) return rc;
   return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
                                  workspace_bytes, stream);

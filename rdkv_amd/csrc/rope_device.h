@@ -1,0 +1,39 @@
+// Device helpers shared by the rotary-embedding kernel and the fused decode kernel's query
+// staging: typed element access by dtype code and the rotation of one channel pair.
+#pragma once
+#include "rdkv_common.h"
+
+__device__ __forceinline__ float rdkv_load_as_float(const void *p, int dtype, int64_t idx) {
+  if (dtype == RDKV_DTYPE_F32) return reinterpret_cast<const float *>(p)[idx];
+  if (dtype == RDKV_DTYPE_F16) return (float)reinterpret_cast<const _Float16 *>(p)[idx];
+  return __uint_as_float((uint32_t)reinterpret_cast<const uint16_t *>(p)[idx] << 16);
+}
+
+// fp32 -> bf16 bits, round to nearest even (NaN stays NaN)
+__device__ __forceinline__ uint16_t rdkv_float_to_bf16_bits(float v) {
+  uint32_t u = __float_as_uint(v);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// the value a store in `dtype` would keep, as fp32
+__device__ __forceinline__ float rdkv_round_to_dtype(float v, int dtype) {
+  if (dtype == RDKV_DTYPE_F32) return v;
+  if (dtype == RDKV_DTYPE_F16) return (float)(_Float16)v;
+  return __uint_as_float((uint32_t)rdkv_float_to_bf16_bits(v) << 16);
+}
+
+__device__ __forceinline__ void rdkv_store_from_float(void *p, int dtype, int64_t idx, float v) {
+  if (dtype == RDKV_DTYPE_F32) reinterpret_cast<float *>(p)[idx] = v;
+  else if (dtype == RDKV_DTYPE_F16) reinterpret_cast<_Float16 *>(p)[idx] = (_Float16)v;
+  else reinterpret_cast<uint16_t *>(p)[idx] = rdkv_float_to_bf16_bits(v);
+}
+
+// out_lo = lo*c - hi*s, out_hi = hi*c + lo*s with every operation rounded on its own
+// (triton_rope.py:68-70; its PyTorch statement :127-131)
+__device__ __forceinline__ void rdkv_rope_pair(float lo, float hi, float c, float s, float &out_lo,
+                                               float &out_hi) {
+  out_lo = __fsub_rn(__fmul_rn(lo, c), __fmul_rn(hi, s));
+  out_hi = __fadd_rn(__fmul_rn(hi, c), __fmul_rn(lo, s));
+}

@@ -307,9 +307,12 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
-                      lse: Optional[torch.Tensor] = None):
+                      lse: Optional[torch.Tensor] = None, *,
+                      rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
-    rotated); returns (out fp32 [rows,128], lse fp32 [rows]).  Graph-capturable once the
+    rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
+    kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
+    query); returns (out fp32 [rows,128], lse fp32 [rows]).  Graph-capturable once the
     workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
@@ -321,11 +324,19 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     if lse is None:
         lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
     assert out.dtype == torch.float32 and out.stride(1) == 1 and lse.dtype == torch.float32 and lse.is_contiguous()
+    rc = rs = None
+    rope_dt = 0
+    if rope is not None:
+        rc, rs = rope
+        _lib.require_device(rc, rs)
+        assert rc.numel() == 64 and rs.numel() == 64 and rc.dtype == rs.dtype and rc.dtype in _lib.DTYPE_CODE
+        rc, rs = rc.contiguous(), rs.contiguous()
+        rope_dt = _lib.DTYPE_CODE[rc.dtype]
     need = lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G)
     ws = _lib.workspace(dev, need)
     _lib.check(lib.rdkv_decode_fused(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
         _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
-        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G,
+        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
     return out, lse

@@ -27,6 +27,7 @@ from obkv_accel import packing as rp            # noqa: E402
 from obkv_accel import trizone_decompress as rt  # noqa: E402
 from obkv_accel.triton_k_kernel import k_mixed_qk_dot_ref  # noqa: E402
 from obkv_accel.triton_v_kernel import v_dequant_weighted_sum_ref  # noqa: E402
+from obkv_accel.triton_rope import fused_rope_ref  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
@@ -260,8 +261,30 @@ def case_shared_layout():
     save("shared_layout", d)
 
 
+# ---------------------------------------------------------------- rotary embedding
+def case_rope():
+    """fused_rope_ref (triton_rope.py:110-136) on fp16 and bf16 heads, cos/sin of a few positions."""
+    g = torch.Generator().manual_seed(707)
+    d = {}
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, 128, 2).float() / 128))
+    for tag, dt in (("f16", torch.float16), ("bf16", torch.bfloat16)):
+        for pos in (0, 1, 4097, 131071):
+            ang = pos * inv_freq
+            cos, sin = ang.cos().to(dt), ang.sin().to(dt)
+            q = torch.randn(8, 128, generator=g).to(dt)
+            k = torch.randn(2, 128, generator=g).to(dt)
+            qo, ko = fused_rope_ref(q, k, cos, sin)
+            key = f"{tag}.{pos}"
+            for n, t in (("q", q), ("k", k), ("cos", cos), ("sin", sin), ("q_out", qo), ("k_out", ko)):
+                d[f"{key}.{n}"] = npy(t.view(torch.int16))       # raw 16-bit patterns
+    save("rope", d)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
+    if len(sys.argv) > 2:                      # python make_golden.py <ref> <case> : one case only
+        globals()["case_" + sys.argv[2]]()
+        sys.exit(0)
     case_bitpack()
     case_quantizer()
     case_ref_test_segment_counts()

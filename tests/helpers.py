@@ -72,3 +72,14 @@ def assert_layer_equal(actual, g, prefix, skip=()):
             assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), f"{name}: bits differ"
         else:
             assert np.array_equal(got.astype(np.int64), exp.astype(np.int64)), f"{name}: values differ"
+
+
+def decode_16bit(raw, kind):
+    """int16 bit patterns of an fp16 / bf16 array -> fp32 values."""
+    u = np.asarray(raw).astype(np.int16).view(np.uint16)
+    if kind == "f16":
+        return u.view(np.float16).astype(np.float32)
+    return (u.astype(np.uint32) << 16).view(np.float32)
+
+
+ROPE_CASES = [(kind, pos) for kind in ("f16", "bf16") for pos in (0, 1, 4097, 131071)]

@@ -134,3 +134,50 @@ def test_retired_hook_names_raise():
     cache = packing.TriZoneCache((pl,), [None], [None], [None], 80)
     w = decode_hook.PackedCacheWrapper(cache)
     assert len(w) == 1 and w.get_seq_length(0) == pl.T_eff_k
+
+
+def _t16(raw, kind):
+    t = torch.from_numpy(np.asarray(raw).astype(np.int16))
+    return t.view(torch.float16 if kind == "f16" else torch.bfloat16)
+
+
+def test_fused_rope_golden():
+    """triton_rope.fused_rope (in place) bit-exact against the reference's output vectors."""
+    from rdkv_amd import triton_rope
+    from tests.helpers import ROPE_CASES
+    g = load_golden("rope")
+    for kind, pos in ROPE_CASES:
+        key = f"{kind}.{pos}"
+        q, k = _t16(g[f"{key}.q"], kind).to(DEV), _t16(g[f"{key}.k"], kind).to(DEV)
+        cos, sin = _t16(g[f"{key}.cos"], kind).to(DEV), _t16(g[f"{key}.sin"], kind).to(DEV)
+        rq, rk = triton_rope.fused_rope(q, k, cos, sin)
+        assert rq is q and rk is k
+        assert torch.equal(q.view(torch.int16).cpu(), torch.from_numpy(g[f"{key}.q_out"].astype(np.int16))), key
+        assert torch.equal(k.view(torch.int16).cpu(), torch.from_numpy(g[f"{key}.k_out"].astype(np.int16))), key
+    with pytest.raises(AssertionError):
+        triton_rope.fused_rope(q[:, :64], k, cos, sin)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_rope_inside_the_fused_kernel(dtype):
+    """Rotating the query while it is staged gives the bits of rotate-then-attend."""
+    from rdkv_amd import triton_rope
+    cfg = synth.scaled(synth.CONFIGS[1], context=1500, layers=2)
+    packed, qs = [], []
+    for layer in range(2):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, q = synth.layer_data(cfg, layer, DEV, outliers=oc)
+        packed.append(packing.pack_layer_per_head(K, V, vb, kb, cfg.G))
+        qs.append(q)
+    q_all = torch.cat(qs).to(dtype).contiguous()
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, 128, 2).float() / 128))
+    ang = 4097 * inv_freq
+    cos, sin = ang.cos().to(dtype).to(DEV), ang.sin().to(dtype).to(DEV)
+    got, got_lse = stream_cache.decode_attn_fused(cache, q_all, rope=(cos, sin))
+    q_rot = q_all.clone()
+    dummy_k = torch.zeros(1, 128, dtype=dtype, device=DEV)
+    triton_rope.fused_rope(q_rot, dummy_k, cos, sin)
+    assert not torch.equal(q_rot, q_all)
+    exp, exp_lse = stream_cache.decode_attn_fused(cache, q_rot)
+    assert torch.equal(got, exp) and torch.equal(got_lse, exp_lse)

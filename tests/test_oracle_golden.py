@@ -107,3 +107,32 @@ def test_shared_layout_golden():
     assert_layer_equal(pl2, g, "pl2")
     assert np.array_equal(O.unpack_k_mixed(pl2, D=128).view(np.uint16),
                           g["pl2.K_hat"].view(np.uint16))
+
+
+def test_rope_golden():
+    """oracle.fused_rope_ref against the reference's fused_rope_ref output (fp16 and bf16)."""
+    from tests.helpers import ROPE_CASES, decode_16bit
+    g = load_golden("rope")
+    for kind, pos in ROPE_CASES:
+        key = f"{kind}.{pos}"
+        q, k, c, s = (decode_16bit(g[f"{key}.{n}"], kind) for n in ("q", "k", "cos", "sin"))
+        qo, ko = O.fused_rope_ref(q, k, c, s, kind)
+        assert np.array_equal(qo.view(np.uint32), decode_16bit(g[f"{key}.q_out"], kind).view(np.uint32)), key
+        assert np.array_equal(ko.view(np.uint32), decode_16bit(g[f"{key}.k_out"], kind).view(np.uint32)), key
+
+
+def test_rope_closed_forms():
+    """Identity at angle 0, exact quarter turn (lo, hi) -> (-hi, lo), and norm preservation."""
+    rng = np.random.default_rng(3)
+    q = rng.standard_normal((4, 128)).astype(np.float16).astype(np.float32)
+    k = rng.standard_normal((2, 128)).astype(np.float16).astype(np.float32)
+    one, zero = np.ones(64, np.float32), np.zeros(64, np.float32)
+    qo, ko = O.fused_rope_ref(q, k, one, zero)
+    assert np.array_equal(qo, q) and np.array_equal(ko, k)
+    qo, _ = O.fused_rope_ref(q, k, zero, one)
+    assert np.array_equal(qo[:, :64], -q[:, 64:]) and np.array_equal(qo[:, 64:], q[:, :64])
+    ang = rng.uniform(0, 6.28, 64).astype(np.float32)
+    qo, _ = O.fused_rope_ref(q, k, np.cos(ang), np.sin(ang), "f16")
+    n0 = q[:, :64] ** 2 + q[:, 64:] ** 2
+    n1 = qo[:, :64] ** 2 + qo[:, 64:] ** 2
+    assert np.allclose(n0, n1, rtol=4e-3, atol=1e-4)
