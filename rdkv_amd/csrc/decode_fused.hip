@@ -78,12 +78,21 @@ __device__ __forceinline__ float quadcol_sum(float v) {
   v += __shfl_xor(v, 32, 64);
   return v;
 }
+// Maximum over the 16 lanes that share (lane & 3), without LDS traffic: rotations by 8 and 4
+// inside each row of 16 lanes (DPP), then an exchange of rows 0<->1, 2<->3 and of the two
+// halves of the wavefront (lane-permute swaps).  Four dependent ds_bpermute round trips took
+// about 500 cycles per tile on the critical path of every wavefront.
 __device__ __forceinline__ float quadcol_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 4, 64));
-  v = fmaxf(v, __shfl_xor(v, 8, 64));
-  v = fmaxf(v, __shfl_xor(v, 16, 64));
-  v = fmaxf(v, __shfl_xor(v, 32, 64));
-  return v;
+  float a = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true));
+  v = fmaxf(v, a);
+  a = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, true));
+  v = fmaxf(v, a);
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = fmaxf(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+  u = __builtin_bit_cast(unsigned, v);
+  auto t = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, (unsigned)t[0]), __builtin_bit_cast(float, (unsigned)t[1]));
 }
 
 // Combine the partials [work_begin, work_begin + n) of one unit in index order with a whole
@@ -516,7 +525,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
           m_run[hg] = m_new[hg];
 #pragma unroll
           for (int rr = 0; rr < 4; ++rr) {
-            const float f = __shfl(f_own, rr, 64);  // lane rr holds head rr's factor
+            // lane rr holds head rr's factor: a scalar broadcast, no LDS round trip
+            const float f = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, f_own), rr));
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
               accq[hg][j][rr] *= f;
@@ -636,7 +646,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float zb = __shfl(zb_tot, r, 64);
+      const float zb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zb_tot), r));
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         sm.wo[b][wave][hg * 4 + r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : kOBackQ) - zb;
