@@ -64,6 +64,10 @@ __device__ __forceinline__ floatx4 mfma(half4_t a, half4_t b, floatx4 c) {
   return __builtin_amdgcn_mfma_f32_4x4x4f16(a, b, c, 0, 0, 0);
 }
 
+// 2^x for x <= 0 as the bare hardware instruction (1 ulp; results below 2^-126 flush to 0,
+// which is what a softmax weight that small is worth).
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 __device__ __forceinline__ float load_qv(const void *q, int dtype, int64_t idx) {
   if (dtype == RDKV_DTYPE_F32) return reinterpret_cast<const float *>(q)[idx];
   if (dtype == RDKV_DTYPE_F16) return (float)reinterpret_cast<const _Float16 *>(q)[idx];
@@ -519,7 +523,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       if (__any(grew)) {  // wave-uniform: rescale the running state
 #pragma unroll
         for (int hg = 0; hg < NH; ++hg) {
-          const float f_own = exp2f(m_run[hg] - m_new[hg]);  // 0 on the first tile (m_run = -inf)
+          const float f_own = fast_exp2(m_run[hg] - m_new[hg]);  // 0 on the first tile (m_run = -inf)
           l_run[hg] *= f_own;
           zb_run[hg] *= f_own;
           m_run[hg] = m_new[hg];
@@ -540,7 +544,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
         float lsum = 0.0f, zsum = 0.0f;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const float p = exp2f(s2[hg][j] - m_run[hg]);  // masked tokens: exp2(-inf) = 0
+          const float p = fast_exp2(s2[hg][j] - m_run[hg]);  // masked tokens: exp2(-inf) = 0
           lsum += p;
           ph[j] = (_Float16)(p * sc4[j] * pscale);
           zsum += (float)ph[j] * zp4[j];
