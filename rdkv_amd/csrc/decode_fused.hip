@@ -179,15 +179,11 @@ struct Smem {
   float wo[kBatch][NW][NH * 4][kD];
 };
 
-// Register images of the loads in flight.  KRegs: the K row of the lane's token and the
-// {scale,zp} pairs of the lane's quad for one tile (single buffer: the next tile's row is
-// requested as soon as the current one has been consumed, a whole V phase ahead of its use).
-// VRegs: one V piece of up to 16 dwords per lane (two buffers, one stage ahead).
-template <int RMAX>
-struct KRegs {
-  uint32_t k[RMAX];
-  uint4 sz;
-};
+// Register images of the loads in flight.  The K row of the lane's token and the {scale,zp}
+// pairs of the lane's quad for one tile are plain locals of the kernel (single buffer: the
+// next tile's row is requested as soon as the current one has been consumed, a whole V phase
+// ahead of its use).  VRegs: one V piece of up to 16 dwords per lane (two buffers, one stage
+// ahead).
 struct VRegs {
   uint4 v[4];
 };
@@ -234,7 +230,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   const int item_begin = groups ? groups[blockIdx.x] : (int)blockIdx.x;
   const int item_end = groups ? groups[blockIdx.x + 1] : (int)blockIdx.x + 1;
 
-  auto load_item = [&](int item) -> Item {
+  auto load_item = [&](int item) __attribute__((always_inline)) -> Item {
     const RdkvWork *wkp = work + item;
     const RdkvUnit *up = units + wkp->unit;
     Item it;
@@ -259,7 +255,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   };
 
   Item it;  // the item the tile loop is working on
-  auto set_tile = [&](Cursor &c, int ti) {
+  auto set_tile = [&](Cursor &c, int ti) __attribute__((always_inline)) {
     c.ti = ti;
     c.pc = 0;
     c.valid = ti < it.tile_end;
@@ -270,7 +266,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     c.vtile = sel4(cls, it.v_base0, it.v_base1, it.v_base2, it.v_base3) + (uint64_t)tl * (uint64_t)(2048 << cls);
     c.npc = cls < 2 ? 1 : (cls == 2 ? 2 : 4);  // V pieces of 16 dwords per lane (8 for 2-bit)
   };
-  auto advance = [&](const Cursor &c) {
+  auto advance = [&](const Cursor &c) __attribute__((always_inline)) {
     Cursor n = c;
     if (c.pc + 1 < c.npc) n.pc = c.pc + 1;
     else set_tile(n, c.ti + kWaves);
@@ -280,7 +276,14 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   // The number of load instructions per stage is fixed (unused K chunks / V slots re-read an
   // address already being fetched, which the vector cache absorbs) so that the hardware load
   // counter can be waited on precisely while the next stage's loads are still in flight.
-  auto issue_k = [&](int ti, KRegs<RMAX> &r) {
+  // (the K row is a plain local array, not a struct member: it is indexed dynamically and
+  // has to stay promotable to a register vector)
+  // Register tuples come in sizes 12, 16 and 32: a row of 20 dwords is held as 16 + 4.
+  constexpr int kRowA = RMAX == 20 ? 16 : RMAX, kRowB = RMAX - kRowA;
+  uint32_t krow[kRowA];
+  uint32_t ktail[kRowB > 0 ? kRowB : 1];
+  uint4 ksz;
+  auto issue_k = [&](int ti) __attribute__((always_inline)) {
     const uint8_t *ktile = it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R;
 #pragma unroll
     for (int ch = 0; ch < RMAX / 4; ++ch) {
@@ -289,12 +292,17 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
       // the next token (or the region that follows) and are never used
       const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
-      r.k[4 * ch] = v.x; r.k[4 * ch + 1] = v.y; r.k[4 * ch + 2] = v.z; r.k[4 * ch + 3] = v.w;
+      if (4 * ch < kRowA) {
+        krow[4 * ch] = v.x; krow[4 * ch + 1] = v.y; krow[4 * ch + 2] = v.z; krow[4 * ch + 3] = v.w;
+      } else {
+        ktail[4 * ch - kRowA] = v.x; ktail[4 * ch - kRowA + 1] = v.y;
+        ktail[4 * ch - kRowA + 2] = v.z; ktail[4 * ch - kRowA + 3] = v.w;
+      }
     }
-    r.sz = *reinterpret_cast<const uint4 *>(
+    ksz = *reinterpret_cast<const uint4 *>(
         it.sz_base + (ti < it.ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0));
   };
-  auto issue_v = [&](const Cursor &c, VRegs &r) {
+  auto issue_v = [&](const Cursor &c, VRegs &r) __attribute__((always_inline)) {
     const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
     const int hi = c.cls != 0 ? 128 : 0;
     r.v[0] = ld16_stream(vt);
@@ -303,15 +311,14 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     r.v[3] = ld16_stream(vt + hi + 64);
   };
 
-  KRegs<RMAX> kr;
   VRegs va, vb;
   Cursor c0;
   // Load an item's description and put its first tile's loads in flight.
-  auto start_item = [&](int item) {
+  auto start_item = [&](int item) __attribute__((always_inline)) {
     it = load_item(item);
     set_tile(c0, it.tile_begin + wave);
     if (c0.valid) {
-      issue_k(c0.ti, kr);
+      issue_k(c0.ti);
       issue_v(c0, va);
     }
   };
@@ -425,7 +432,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     return *reinterpret_cast<const half4_t *>(&sm.p[wave][quad][hg][ln][0]);
   };
 
-  auto compute = [&](const Cursor &c, const VRegs &r) {
+  auto compute = [&](const Cursor &c, const VRegs &r) __attribute__((always_inline)) {
     if (c.pc == 0) {
       // Progress feedback: the hardware issues oldest-wavefront-first, which lets the
       // wavefronts of a workgroup drift 20% apart over an item.  Every wavefront publishes
@@ -444,57 +451,89 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
         ++tiles_done;
       }
       // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
-      floatx4 sacc[NH];
+      // Three loops, one per field width, over the dwords of that width; the K row is indexed
+      // dynamically (register-relative addressing), so each loop body is straight-line code for
+      // its width and the accumulators never leave their registers.  The hi and lo terms of
+      // q*scale feed separate accumulators: two independent matrix-core chains.
+      floatx4 sacc[NH], sacc_lo[NH];
 #pragma unroll
-      for (int hg = 0; hg < NH; ++hg) sacc[hg] = floatx4{0.f, 0.f, 0.f, 0.f};
-      int step = 0;
+      for (int hg = 0; hg < NH; ++hg) {
+        sacc[hg] = floatx4{0.f, 0.f, 0.f, 0.f};
+        sacc_lo[hg] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+      auto k_dword = [&](int idx) __attribute__((always_inline)) -> uint32_t {
+        // one opaque index per array: a base + counter address chain (or a choice between two
+        // addresses) would keep the row from being held in registers
+        int ia = (kRowB > 0 && idx >= kRowA) ? kRowA - 1 : idx;
+        asm volatile("" : "+s"(ia));
+        const uint32_t a = krow[ia];
+        if (kRowB == 0) return a;
+        int ib = (idx - kRowA) & (kRowB > 0 ? kRowB - 1 : 0);
+        asm volatile("" : "+s"(ib));
+        const uint32_t b = ktail[ib];
+        return idx >= kRowA ? b : a;
+      };
+      // q*scale operands of one step: [hg][hi|lo]
+      struct QOp { half4_t v[NH][2]; };
+      auto q_load = [&](int step) __attribute__((always_inline)) -> QOp {
+        QOp o;
 #pragma unroll
-      for (int j = 0; j < RMAX; ++j) {
-        // compare right here, every tile: hoisted, the 3 * RMAX loop-invariant comparisons no
-        // longer fit the scalar registers and come back through lane reads
-        int R_o = it.R, d8_o = it.d8, d84_o = it.d8 + it.d4;
-        asm volatile("" : "+s"(R_o), "+s"(d8_o), "+s"(d84_o));
-        if (j < R_o) {
-          const uint32_t w = kr.k[j];
-          if (j < d8_o) {
-            const half4_t a = mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
+        for (int hg = 0; hg < NH; ++hg) {
+          o.v[hg][0] = *reinterpret_cast<const half4_t *>(qs_op(step, hg, 0));
+          o.v[hg][1] = *reinterpret_cast<const half4_t *>(qs_op(step, hg, 1));
+        }
+        return o;
+      };
+      auto k_step = [&](const half4_t a, const QOp &o) __attribute__((always_inline)) {
 #pragma unroll
-            for (int hg = 0; hg < NH; ++hg) {
-              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step, hg, 0)), sacc[hg]);
-              sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step, hg, 1)), sacc[hg]);
-            }
-            step += 1;
-          } else if (j < d84_o) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-              const half4_t a = mk_op((w >> (8 * s)) & 0x000F000Fu, (w >> (8 * s + 4)) & 0x000F000Fu);
-#pragma unroll
-              for (int hg = 0; hg < NH; ++hg) {
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 0)), sacc[hg]);
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 1)), sacc[hg]);
-              }
-            }
-            step += 2;
-          } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-              const half4_t a = mk_op((w >> (4 * s)) & 0x00030003u, (w >> (4 * s + 2)) & 0x00030003u);
-#pragma unroll
-              for (int hg = 0; hg < NH; ++hg) {
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 0)), sacc[hg]);
-                sacc[hg] = mfma(a, *reinterpret_cast<const half4_t *>(qs_op(step + s, hg, 1)), sacc[hg]);
-              }
-            }
-            step += 4;
-          }
+        for (int hg = 0; hg < NH; ++hg) {
+          sacc[hg] = mfma(a, o.v[hg][0], sacc[hg]);
+          sacc_lo[hg] = mfma(a, o.v[hg][1], sacc_lo[hg]);
+        }
+      };
+      {
+        // Software-pipelined: the operands of the next step(s) are read from LDS while the
+        // current ones are multiplied (reads one step past the end stay inside the LDS block).
+        const int d8 = it.d8, d4 = it.d4, d2 = it.d2;
+        int step = 0;
+        QOp cur = q_load(0);
+#pragma unroll 2
+        for (int i = 0; i < d8; ++i) {
+          const QOp nxt = q_load(step + 1);
+          const uint32_t w = k_dword(i);
+          k_step(mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu), cur);
+          cur = nxt;
+          step += 1;
+        }
+        for (int i = 0; i < d4; ++i) {
+          const QOp n1 = q_load(step + 1), n2 = q_load(step + 2);
+          const uint32_t w = k_dword(d8 + i);
+          k_step(mk_op(w & 0x000F000Fu, (w >> 4) & 0x000F000Fu), cur);
+          k_step(mk_op((w >> 8) & 0x000F000Fu, (w >> 12) & 0x000F000Fu), n1);
+          cur = n2;
+          step += 2;
+        }
+        for (int i = 0; i < d2; ++i) {  // few dwords of this width: operands fetched per dword
+          const QOp n1 = q_load(step + 1);
+          const uint32_t w = k_dword(d8 + d4 + i);
+          k_step(mk_op(w & 0x00030003u, (w >> 2) & 0x00030003u), cur);
+          const QOp n2 = q_load(step + 2);
+          k_step(mk_op((w >> 4) & 0x00030003u, (w >> 6) & 0x00030003u), n1);
+          const QOp n3 = q_load(step + 3);
+          k_step(mk_op((w >> 8) & 0x00030003u, (w >> 10) & 0x00030003u), n2);
+          cur = q_load(step + 4);
+          k_step(mk_op((w >> 12) & 0x00030003u, (w >> 14) & 0x00030003u), n3);
+          step += 4;
         }
       }
+#pragma unroll
+      for (int hg = 0; hg < NH; ++hg) sacc[hg] += sacc_lo[hg];
       // ---- online softmax (base-2 domain) --------------------------------------------------
       const int n_valid = c.n_valid;
       const float pscale = c.cls < 3 ? kPScaleQ : kPScaleH;
       float sc4[4], zp4[4];
       {
-        const uint32_t szw[4] = {kr.sz.x, kr.sz.y, kr.sz.z, kr.sz.w};
+        const uint32_t szw[4] = {ksz.x, ksz.y, ksz.z, ksz.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           sc4[j] = c.cls < 3 ? (float)__builtin_bit_cast(_Float16, (uint16_t)(szw[j] & 0xffffu)) : 1.0f;
@@ -503,7 +542,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       }
       // the K registers are free now: request this wavefront's next tile (at the end of the
       // work item the same tile again, so the number of loads in flight stays fixed)
-      issue_k(c.ti + kWaves < it.tile_end ? c.ti + kWaves : c.ti, kr);
+      issue_k(c.ti + kWaves < it.tile_end ? c.ti + kWaves : c.ti);
       bool grew = false;
       float s2[NH][4], m_new[NH];
 #pragma unroll
