@@ -97,8 +97,8 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
 # per tile of each V class, per dword of K row per tile, per work item (its set-up is a chain
 # of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X, for G <= 4 (one
 # head group, 16 wavefronts) and for G = 5..8 (two head groups, 12 wavefronts).
-DEFAULT_COST = {"tile": (198.0, 195.0, 280.0, 499.0), "k_dword": 5.9, "item": 7400.0}
-DEFAULT_COST_TWO_HEAD_GROUPS = {"tile": (340.0, 346.0, 363.0, 433.0), "k_dword": 7.2, "item": 9700.0}
+DEFAULT_COST = {"tile": (173.0, 172.0, 264.0, 492.0), "k_dword": 6.5, "item": 9900.0}
+DEFAULT_COST_TWO_HEAD_GROUPS = {"tile": (304.0, 310.0, 325.0, 413.0), "k_dword": 7.0, "item": 8800.0}
 BYTES_COST = {"tile": (2048.0 + 256, 4096.0 + 256, 8192.0 + 256, 16384.0), "k_dword": 256.0, "item": 0.0}
 
 
