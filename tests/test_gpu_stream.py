@@ -260,3 +260,33 @@ def test_fused_attention_full_size_layer(cfg_idx):
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
     assert cache.n_groups >= 128      # the layer alone already spreads over the compute units
+
+
+@pytest.mark.parametrize("counts", [(1, 1, 120), (128, 0, 0), (0, 128, 0), (0, 0, 128), (60, 60, 8), (17, 9, 5),
+                                    (0, 0, 1), (3, 0, 0)])
+def test_fused_attention_k_row_shapes(counts):
+    """K rows of every shape the kernel variants cover: the widest (36 channel steps, 32
+    dwords), a single field width only, a single channel; against the oracle."""
+    c2, c4, c8 = counts
+    H_kv, G, T, D = 2, 4, 333, 128
+    rng = np.random.default_rng(c2 * 10007 + c4 * 101 + c8)
+    g = torch.Generator().manual_seed(c2 + 3 * c4 + 7 * c8)
+    K = torch.randn(1, H_kv, T, D, generator=g).half()
+    V = torch.randn(1, H_kv, T, D, generator=g).half()
+    q = torch.randn(H_kv * G, D, generator=g).half()
+    vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T)))
+    kb = np.zeros((H_kv, D), dtype=np.int64)
+    for h in range(H_kv):
+        ch = rng.permutation(D)
+        kb[h, ch[:c2]] = 2
+        kb[h, ch[c2:c2 + c4]] = 4
+        kb[h, ch[c2 + c4:c2 + c4 + c8]] = 8
+    kb = torch.from_numpy(kb)
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+    exp_out, exp_lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
+    cache = stream_cache.build_stream_cache([(pl, nvo)], G)
+    assert cache.max_row_dwords == -(-c8 // 4) + -(-c4 // 8) + -(-c2 // 16)
+    out, lse = stream_cache.decode_attn_fused(cache, q.to(DEV))
+    attn_close(t2n(out), exp_out, "out")
+    attn_close(t2n(lse), exp_lse, "lse")
