@@ -128,6 +128,15 @@ def trizone_attention_fused(cache: StreamCache, q_all: torch.Tensor, K_new: List
     return res
 
 
+def pre_extract_weights(model):
+    """Name of the reference's weight collector for the decode loop (fast_decode.py:418).  It
+    gathers projection / MLP / LM-head weights of a loaded model, which this package does not
+    drive: keep the reference's function next to its loop."""
+    raise NotImplementedError(
+        "pre_extract_weights belongs to the model loop (weights, projections, LM head), which is "
+        "outside this package; only the loop's attention section is provided here")
+
+
 def greedy_decode_fast(model, dual_cache, next_token_logits, max_new_tokens, eos_token_ids, primary_device,
                        decode_position_start, use_cuda_graph=False, return_logits=False,
                        next_token_hidden=None, logits_observer=None, hidden_observer=None):

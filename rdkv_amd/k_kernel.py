@@ -49,6 +49,15 @@ def _as_3d(t):
     return t
 
 
+def _ensure_tensor(t, H_kv: int, last_dim: int, device, dtype=torch.uint8):
+    """None / empty -> a [H_kv,1,max(1,last_dim)] zero placeholder, else the 3-D view
+    (triton_k_kernel.py:1203-1208)."""
+    t3 = _as_3d(t)
+    if t3 is not None and t3.numel() > 0:
+        return t3
+    return torch.zeros((H_kv, 1, max(1, last_dim)), dtype=dtype, device=device)
+
+
 def _runtime_gqa(Q, K_scale):
     H_kv = K_scale.shape[1] if K_scale.dim() == 4 else K_scale.shape[0]
     return Q.shape[0] // H_kv

@@ -129,6 +129,13 @@ def test_retired_hook_names_raise():
         decode_hook.greedy_decode_packed(None, None, None, 1, [], None, 0)
     with pytest.raises(NotImplementedError):
         fast_decode.greedy_decode_fast(None, None, None, 1, [], None, 0)
+    with pytest.raises(NotImplementedError):
+        fast_decode.pre_extract_weights(None)
+    from rdkv_amd import triton_k_kernel as tk
+    ph = tk._ensure_tensor(None, 3, 0, DEV)
+    assert ph.shape == (3, 1, 1) and ph.dtype == torch.uint8 and int(ph.sum()) == 0
+    real = torch.ones(1, 3, 5, 2, dtype=torch.uint8, device=DEV)
+    assert tk._ensure_tensor(real, 3, 2, DEV).shape == (3, 5, 2)
     g = load_golden("perhead_d128_a")
     pl = layer_to_device(golden_to_oracle_layer(g, "pl"))
     cache = packing.TriZoneCache((pl,), [None], [None], [None], 80)
