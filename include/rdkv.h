@@ -236,6 +236,20 @@ int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int 
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);
 
+/* rdkv_decode_fused_merge plus the attention over the decode-appended tokens of every unit
+ * (zone C; fast_decode.py:1719-1735 scores of the new tokens, :1743-1755 softmax over
+ * [old | new], :1777-1784 their V sum): the exact softmax over zones A+B+C, out and lse of the
+ * union.  k_new / v_new: fp32 [n_units, >= n_new, 128] (unit u at + u*new_stride_unit, token t
+ * at + t*new_stride_tok, elements); n_new tokens per unit, or n_new_per_unit[u] (device int32)
+ * when not NULL (n_new is then ignored).  q / rope_*: as passed to rdkv_decode_fused_partials. */
+int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G,
+                                   const void *q, int q_dtype, int64_t q_stride_row,
+                                   const void *rope_cos, const void *rope_sin, int rope_dtype,
+                                   const float *k_new, const float *v_new, int64_t new_stride_unit,
+                                   int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit,
+                                   float *out, int64_t out_stride_row, float *lse,
+                                   void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- measurement helpers (no counterpart in the reference) --------------------------------
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)

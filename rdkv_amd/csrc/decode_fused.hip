@@ -105,9 +105,11 @@ __device__ __forceinline__ float quadcol_max(float v) {
 // costs about one memory latency instead of one per partial.
 constexpr int kMergeMaxK = 128;
 
+// keep_o / keep_lse (LDS, [8][128] and [8], or null): when given, the normalized result and the
+// natural-log sum-exp stay there for a following zone-C pass instead of being written out.
 __device__ __forceinline__ void merge_unit(const float *partials, int work_begin, int n, int G, int q_row,
                                            float *out, int64_t out_stride, float *lse, int tid, int nthreads,
-                                           float *scratch) {
+                                           float *scratch, float *keep_o = nullptr, float *keep_lse = nullptr) {
   const int64_t pstride = (int64_t)G * kPartialStride;
   const float *base0 = partials + (int64_t)work_begin * pstride;
   if (n <= kMergeMaxK) {
@@ -139,8 +141,15 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
         }
       }
       const int64_t row = q_row + h;
-      out[row * out_stride + d] = l > 0.0f ? o / l : 0.0f;  // a unit without tokens gives 0 / -inf
-      if (lse && d == 0) lse[row] = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+      const float o_n = l > 0.0f ? o / l : 0.0f;  // a unit without tokens gives 0 / -inf
+      const float lse_n = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+      if (keep_o) {
+        keep_o[i] = o_n;
+        if (d == 0) keep_lse[h] = lse_n;
+      } else {
+        out[row * out_stride + d] = o_n;
+        if (lse && d == 0) lse[row] = lse_n;
+      }
     }
     return;
   }
@@ -158,8 +167,15 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
       l += f * *(p + 129);
     }
     const int64_t row = q_row + h;
-    out[row * out_stride + d] = l > 0.0f ? o / l : 0.0f;
-    if (lse && d == 0) lse[row] = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+    const float o_n = l > 0.0f ? o / l : 0.0f;
+    const float lse_n = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+    if (keep_o) {
+      keep_o[i] = o_n;
+      if (d == 0) keep_lse[h] = lse_n;
+    } else {
+      out[row * out_stride + d] = o_n;
+      if (lse && d == 0) lse[row] = lse_n;
+    }
   }
 }
 
@@ -738,6 +754,109 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
                     scratch);
 }
 
+// Merge of a unit's partials followed by the attention over its decode-appended tokens
+// (zone C: fp32 K/V rows that are not part of the packed cache), the exact softmax over the
+// union (fast_decode.py:1719-1735, 1777-1784): the zones A+B result enters as one pseudo-token
+// of weight exp(lse_ab) and value out_ab; the new tokens are folded in 64 at a time with a
+// running maximum.  Natural-log domain, fp32 throughout, q scaled by 1/sqrt(D) first as the
+// reference does.
+constexpr int kZcChunk = 64;
+__global__ void __launch_bounds__(256)
+merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
+                    const void *__restrict__ q, int q_dtype, int64_t q_stride,
+                    const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
+                    const float *__restrict__ k_new, const float *__restrict__ v_new, int64_t new_stride_unit,
+                    int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
+                    float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
+  __shared__ float scratch[2 * kMergeMaxK * 8];
+  __shared__ float acc_ab[8 * kD];      // normalized zones A+B output, later unused
+  __shared__ float qz[8][kD];           // q / sqrt(D)
+  __shared__ float sc[8][kZcChunk];     // scores, then weights, of the current chunk
+  __shared__ float m_run[8], l_run[8], f_old[8], lse_ab[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const RdkvUnit *u = units + blockIdx.x;
+  const int q_row = u->q_row;
+  merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, 256, scratch, acc_ab,
+             lse_ab);
+  const int n_new = n_new_per_unit ? n_new_per_unit[blockIdx.x] : n_new_all;
+  for (int i = tid; i < G * kD; i += 256) {
+    const int c = i & 127;
+    const int64_t row = (int64_t)(q_row + (i >> 7)) * q_stride;
+    float v = load_qv(q, q_dtype, row + c);
+    if (rope_cos) {
+      const float other = load_qv(q, q_dtype, row + (c ^ 64));
+      const float cs = rdkv_load_as_float(rope_cos, rope_dtype, c & 63);
+      const float sn = rdkv_load_as_float(rope_sin, rope_dtype, c & 63);
+      float out_lo, out_hi;
+      if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
+      else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
+      v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+    }
+    qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
+  }
+  __syncthreads();
+  if (tid < G) {
+    m_run[tid] = lse_ab[tid];
+    l_run[tid] = lse_ab[tid] == -INFINITY ? 0.0f : 1.0f;
+  }
+  // each thread owns the outputs i = tid + 256*k (head i>>7, channel i&127)
+  float acc[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) acc[k] = tid + 256 * k < G * kD ? acc_ab[tid + 256 * k] : 0.0f;
+  const float *kn = k_new + (int64_t)blockIdx.x * new_stride_unit;
+  const float *vn = v_new + (int64_t)blockIdx.x * new_stride_unit;
+  for (int t0 = 0; t0 < n_new; t0 += kZcChunk) {
+    const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
+    __syncthreads();
+    // scores: one wavefront per token, lanes over the channels
+    for (int t = wave; t < nt; t += 4) {
+      const float *kr = kn + (int64_t)(t0 + t) * new_stride_tok;
+      const float k0 = kr[lane], k1 = kr[lane + 64];
+      for (int h = 0; h < G; ++h) {
+        const float s = rdkv_wave_sum(qz[h][lane] * k0 + qz[h][lane + 64] * k1);
+        if (lane == 0) sc[h][t] = s;
+      }
+    }
+    __syncthreads();
+    if (tid < G) {
+      float cm = -INFINITY;
+      for (int t = 0; t < nt; ++t) cm = fmaxf(cm, sc[tid][t]);
+      const float m_new = fmaxf(m_run[tid], cm);
+      f_old[tid] = m_run[tid] == -INFINITY ? 0.0f : expf(m_run[tid] - m_new);
+      float ls = 0.0f;
+      for (int t = 0; t < nt; ++t) {
+        const float w = expf(sc[tid][t] - m_new);
+        sc[tid][t] = w;
+        ls += w;
+      }
+      l_run[tid] = l_run[tid] * f_old[tid] + ls;
+      m_run[tid] = m_new;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = tid + 256 * k;
+      if (i < G * kD) {
+        const int h = i >> 7, d = i & 127;
+        float a = acc[k] * f_old[h];
+        for (int t = 0; t < nt; ++t) a += sc[h][t] * vn[(int64_t)(t0 + t) * new_stride_tok + d];
+        acc[k] = a;
+      }
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int i = tid + 256 * k;
+    if (i < G * kD) {
+      const int h = i >> 7, d = i & 127;
+      const float l = l_run[h];
+      out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? acc[k] / l : 0.0f;
+      if (lse && d == 0) lse[q_row + h] = l > 0.0f ? m_run[h] + logf(l) : -INFINITY;
+    }
+  }
+}
+
 }  // namespace
 
 RDKV_API int64_t rdkv_decode_fused_workspace_bytes(int n_work, int G) {
@@ -856,4 +975,28 @@ RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n
   if (rc != RDKV_OK) return rc;
   return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
                                  workspace_bytes, stream);
+}
+
+RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
+                                            int q_dtype, int64_t q_stride_row, const void *rope_cos,
+                                            const void *rope_sin, int rope_dtype, const float *k_new,
+                                            const float *v_new, int64_t new_stride_unit, int64_t new_stride_tok,
+                                            int n_new, const int32_t *n_new_per_unit, float *out,
+                                            int64_t out_stride_row, float *lse, void *workspace,
+                                            int64_t workspace_bytes, void *stream) {
+  const char *fn = "rdkv_decode_fused_merge_zone_c";
+  int rc = check_fused_args(fn, units, n_units, (const RdkvWork *)units, n_work, G, workspace, workspace_bytes);
+  if (rc != RDKV_OK) return rc;
+  RDKV_REQUIRE(n_new >= 0 && new_stride_tok >= 128 && new_stride_unit >= 0, "%s: bad zone-C shape", fn);
+  RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "%s: unknown q dtype %d", fn, q_dtype);
+  RDKV_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), "%s: rope_cos and rope_sin go together", fn);
+  RDKV_REQUIRE(!rope_cos || (rope_dtype >= 0 && rope_dtype <= 2), "%s: unknown rope dtype %d", fn, rope_dtype);
+  if (n_units == 0) return RDKV_OK;
+  RDKV_REQUIRE(out && q, "%s: null out / q", fn);
+  RDKV_REQUIRE(n_new == 0 || (k_new && v_new), "%s: null zone-C tensors", fn);
+  hipLaunchKernelGGL(merge_zone_c_kernel, dim3(n_units), dim3(256), 0, (hipStream_t)stream, units,
+                     (const float *)workspace, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new,
+                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
 }

@@ -105,6 +105,8 @@ def merge_zone_c(out_ab: torch.Tensor, lse_ab: torch.Tensor, q_2d: torch.Tensor,
     contributes nothing (never forms -inf - -inf)."""
     H_q, D = q_2d.shape
     H_kv = H_q // num_kv_groups
+    if K_new.shape[-2] == 0:      # nothing appended yet: zones A+B are the whole context
+        return out_ab.clone()
     q_gqa = q_2d.float().view(H_kv, num_kv_groups, D) * INV_SQRT_D
     s_new = torch.bmm(q_gqa, K_new.transpose(-1, -2)).reshape(H_q, -1)
     m = torch.maximum(lse_ab, s_new.max(dim=-1).values)
@@ -116,16 +118,40 @@ def merge_zone_c(out_ab: torch.Tensor, lse_ab: torch.Tensor, q_2d: torch.Tensor,
 
 
 def trizone_attention_fused(cache: StreamCache, q_all: torch.Tensor, K_new: List[torch.Tensor],
-                            V_new: List[torch.Tensor], num_kv_groups: int) -> torch.Tensor:
-    """Zones A+B of every layer / sequence of ``cache`` in one fused launch, then the zone C
-    merge per group.  q_all [groups*H_q,128]; K_new[g], V_new[g] [H_kv,n_new,128] fp32."""
-    out, lse = decode_attn_fused(cache, q_all)
-    H_q = cache.rows // len(K_new)
-    res = torch.empty_like(out)
-    for g, (kn, vn) in enumerate(zip(K_new, V_new)):
-        r = slice(g * H_q, (g + 1) * H_q)
-        res[r] = merge_zone_c(out[r], lse[r], q_all[r], kn, vn, num_kv_groups)
-    return res
+                            V_new: List[torch.Tensor], num_kv_groups: int, *, rope=None,
+                            merge_on_host: bool = False) -> torch.Tensor:
+    """All three zones of every layer / sequence of ``cache`` in two launches: the fused kernel
+    over zones A+B, then a merge launch that also attends over the decode-appended tokens
+    (zone C) and returns the softmax over the union.  q_all [groups*H_q,128]; K_new[g],
+    V_new[g] [H_kv,n_new_g,128] fp32.  ``merge_on_host`` keeps the zone C merge as PyTorch
+    operations per group (``merge_zone_c``), the cross-check of the fused merge."""
+    if merge_on_host:
+        assert rope is None
+        out, lse = decode_attn_fused(cache, q_all)
+        H_q = cache.rows // len(K_new)
+        res = torch.empty_like(out)
+        for g, (kn, vn) in enumerate(zip(K_new, V_new)):
+            r = slice(g * H_q, (g + 1) * H_q)
+            res[r] = merge_zone_c(out[r], lse[r], q_all[r], kn, vn, num_kv_groups)
+        return res
+    n_max = max(int(k.shape[1]) for k in K_new)
+    H_kv = int(K_new[0].shape[0])
+    dev = q_all.device
+    if all(int(k.shape[1]) == n_max for k in K_new):
+        kn = torch.stack([k.float() for k in K_new]).reshape(-1, n_max, 128)
+        vn = torch.stack([v.float() for v in V_new]).reshape(-1, n_max, 128)
+        counts = None
+    else:
+        kn = torch.zeros(len(K_new) * H_kv, n_max, 128, dtype=torch.float32, device=dev)
+        vn = torch.zeros_like(kn)
+        for g, (k, v) in enumerate(zip(K_new, V_new)):
+            kn[g * H_kv:(g + 1) * H_kv, :k.shape[1]] = k
+            vn[g * H_kv:(g + 1) * H_kv, :v.shape[1]] = v
+        counts = torch.tensor([int(k.shape[1]) for k in K_new for _ in range(H_kv)], dtype=torch.int32,
+                              device=dev)
+    zone_c = (kn.contiguous(), vn.contiguous()) if counts is None else (kn, vn, counts)
+    out, _ = decode_attn_fused(cache, q_all, rope=rope, zone_c=zone_c)
+    return out
 
 
 def pre_extract_weights(model):

@@ -308,12 +308,16 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
                       lse: Optional[torch.Tensor] = None, *,
-                      rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+                      rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+                      zone_c: Optional[Tuple[torch.Tensor, ...]] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
-    query); returns (out fp32 [rows,128], lse fp32 [rows]).  Graph-capturable once the
-    workspace exists (first call): one streaming launch plus one small merge launch."""
+    query); returns (out fp32 [rows,128], lse fp32 [rows]).  ``zone_c`` = (K_new, V_new[,
+    n_new_per_unit]): fp32 [n_units, n_new, 128] rows of the decode-appended tokens of every unit
+    (unit = entry * H_kv + kv head; optional int32 [n_units] counts when units differ): the merge
+    launch then returns the exact softmax over packed cache + new tokens.  Graph-capturable once
+    the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
     assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
@@ -334,9 +338,32 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         rope_dt = _lib.DTYPE_CODE[rc.dtype]
     need = lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G)
     ws = _lib.workspace(dev, need)
-    _lib.check(lib.rdkv_decode_fused(
+    stream = _lib.stream_of(dev)
+    if zone_c is None:
+        _lib.check(lib.rdkv_decode_fused(
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+            q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
+            out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        return out, lse
+    K_new, V_new = zone_c[0], zone_c[1]
+    counts = zone_c[2] if len(zone_c) > 2 else None
+    _lib.require_device(K_new, V_new)
+    assert K_new.dtype == torch.float32 and V_new.dtype == torch.float32 and K_new.shape == V_new.shape
+    assert K_new.dim() == 3 and K_new.shape[0] == cache.n_units and K_new.shape[2] == 128, (
+        f"zone C tensors must be [n_units={cache.n_units}, n_new, 128], got {tuple(K_new.shape)}")
+    assert K_new.stride() == V_new.stride() and K_new.stride(2) == 1
+    if counts is not None:
+        assert counts.dtype == torch.int32 and counts.numel() == cache.n_units and counts.is_contiguous()
+    _lib.check(lib.rdkv_decode_fused_partials(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
         _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
-        out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
+        ws.data_ptr(), ws.numel(), stream))
+    n_new = int(K_new.shape[1])
+    _lib.check(lib.rdkv_decode_fused_merge_zone_c(
+        cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
+        q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
+        _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
+        _lib.ptr(counts), out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out, lse

@@ -42,7 +42,10 @@ def test_trizone_attention_three_zones(cfg_idx, ctx, n_new):
     assert torch.equal(out, o2)
     cache = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
     fused = fast_decode.trizone_attention_fused(cache, qd, [Kn], [Vn], cfg.G)
-    attn_close(t2n(fused), exp, "fused + zone C merge")
+    attn_close(t2n(fused), exp, "fused + zone C in the merge launch")
+    fused_host = fast_decode.trizone_attention_fused(cache, qd, [Kn], [Vn], cfg.G, merge_on_host=True)
+    attn_close(t2n(fused_host), exp, "fused + zone C merged by PyTorch operations")
+    assert float((fused - fused_host).abs().max()) < 2e-5
 
 
 def test_zone_c_only_layer():
@@ -188,3 +191,32 @@ def test_rope_inside_the_fused_kernel(dtype):
     assert not torch.equal(q_rot, q_all)
     exp, exp_lse = stream_cache.decode_attn_fused(cache, q_rot)
     assert torch.equal(got, exp) and torch.equal(got_lse, exp_lse)
+
+
+def test_zone_c_merge_ragged_groups_and_rope():
+    """Several layers in one call with different numbers of appended tokens (one with none),
+    the query rotated on the fly: merge launch against the per-group PyTorch merge."""
+    from rdkv_amd import triton_rope
+    cfg = synth.scaled(synth.CONFIGS[1], context=800, layers=3)
+    packed, qs = [], []
+    for layer in range(3):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, q = synth.layer_data(cfg, layer, DEV, outliers=oc)
+        packed.append(packing.pack_layer_per_head(K, V, vb, kb, cfg.G))
+        qs.append(q)
+    q_all = torch.cat(qs).contiguous()
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    g = torch.Generator().manual_seed(11)
+    n_new = [70, 0, 3]
+    K_new = [torch.randn(cfg.H_kv, n, 128, generator=g).to(DEV) for n in n_new]
+    V_new = [torch.randn(cfg.H_kv, n, 128, generator=g).to(DEV) for n in n_new]
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, 128, 2).float() / 128))
+    cos, sin = (900 * inv_freq).cos().half().to(DEV), (900 * inv_freq).sin().half().to(DEV)
+    got = fast_decode.trizone_attention_fused(cache, q_all, K_new, V_new, cfg.G, rope=(cos, sin))
+    q_rot = q_all.clone()
+    triton_rope.fused_rope(q_rot, torch.zeros(1, 128, dtype=q_rot.dtype, device=DEV), cos, sin)
+    exp = fast_decode.trizone_attention_fused(cache, q_rot, K_new, V_new, cfg.G, merge_on_host=True)
+    assert float((got - exp).abs().max()) < 2e-5
+    # the group without new tokens is the plain fused result
+    plain, _ = stream_cache.decode_attn_fused(cache, q_rot)
+    assert torch.equal(got[cfg.H_q:2 * cfg.H_q], plain[cfg.H_q:2 * cfg.H_q])
