@@ -367,3 +367,104 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
         _lib.ptr(counts), out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out, lse
+
+
+# ---------------------------------------------------------------------------
+# On-disk form of a streaming cache (the reference only pickles its Python dataclass,
+# run_latency.py:1987-1991): one file, a JSON header, then the tables and the blobs, all
+# 256-byte aligned, offsets inside the blobs relative so the file can be memory-mapped and
+# uploaded to any address.
+# ---------------------------------------------------------------------------
+_MAGIC = b"RDKVSTR1"
+_ADDR_FIELDS = ("k_off", "sz_off", "qtab_off")
+
+
+def save_stream_cache(cache: StreamCache, path: str) -> None:
+    """Write ``cache`` to ``path`` (device -> host copy of the blobs)."""
+    import json
+    units = cache.units_host.copy()
+    bases = [int(b.data_ptr()) for b in cache.blobs]
+    sizes = [int(b.numel()) for b in cache.blobs]
+    blob_of = np.zeros(len(units), dtype=np.int32)
+    for i in range(len(units)):
+        a = int(units["k_off"][i])
+        j = next(j for j, (b0, n) in enumerate(zip(bases, sizes)) if b0 <= a < b0 + n)
+        blob_of[i] = j
+        for f in _ADDR_FIELDS:
+            units[f][i] -= bases[j]
+        units["v_off"][i] -= bases[j]
+    parts = [("units", units.view(np.uint8).reshape(-1)), ("blob_of", blob_of.view(np.uint8)),
+             ("work", cache.work_host.view(np.uint8).reshape(-1))]
+    if cache.groups_host is not None:
+        parts.append(("groups", cache.groups_host.astype(np.int32).view(np.uint8)))
+    header = {"version": 1, "G": cache.G, "rows": cache.rows, "stream_bytes": cache.stream_bytes,
+              "algorithmic_bytes": cache.algorithmic_bytes, "max_row_dwords": cache.max_row_dwords,
+              "n_units": cache.n_units, "n_work": cache.n_work, "n_groups": cache.n_groups,
+              "sections": {}, "blobs": []}
+    off = 0
+    for name, arr in parts:
+        header["sections"][name] = [off, int(arr.nbytes)]
+        off = _align(off + int(arr.nbytes))
+    for n in sizes:
+        header["blobs"].append([off, n])
+        off = _align(off + n)
+    hj = json.dumps(header).encode()
+    data0 = _align(len(_MAGIC) + 8 + len(hj))
+    with open(path, "wb") as f:
+        f.write(_MAGIC)
+        f.write(np.asarray([len(hj)], dtype="<u8").tobytes())
+        f.write(hj)
+        f.write(b"\0" * (data0 - f.tell()))
+        for (name, arr), (o, n) in zip(parts, header["sections"].values()):
+            f.seek(data0 + o)
+            f.write(arr.tobytes())
+        for blob, (o, n) in zip(cache.blobs, header["blobs"]):
+            f.seek(data0 + o)
+            f.write(blob.cpu().numpy().tobytes())
+        f.truncate(data0 + off)
+
+
+def load_stream_cache(path: str, device) -> StreamCache:
+    """Memory-map ``path`` and upload it to ``device``; the result is usable like a freshly
+    built cache (same outputs, bit for bit)."""
+    import json
+    dev = torch.device(device)
+    if dev.type != "cuda":
+        raise RuntimeError("rdkv HIP backend needs a HIP device; there is no CPU fallback")
+    mm = np.memmap(path, dtype=np.uint8, mode="r")
+    if bytes(mm[:8]) != _MAGIC:
+        raise ValueError(f"{path}: not a streaming-cache file")
+    hlen = int(np.frombuffer(mm[8:16], dtype="<u8")[0])
+    header = json.loads(bytes(mm[16:16 + hlen]))
+    if header["version"] != 1:
+        raise ValueError(f"{path}: unsupported version {header['version']}")
+    data0 = _align(16 + hlen)
+
+    def section(name, dtype):
+        o, n = header["sections"][name]
+        return np.frombuffer(mm[data0 + o:data0 + o + n], dtype=dtype).copy()
+
+    units = section("units", UNIT_DTYPE)
+    blob_of = section("blob_of", np.int32)
+    work = section("work", WORK_DTYPE)
+    groups = section("groups", np.int32) if "groups" in header["sections"] else None
+    blobs = []
+    for o, n in header["blobs"]:
+        t = torch.empty(n, dtype=torch.uint8, device=dev)
+        t.copy_(torch.frombuffer(memoryview(mm)[data0 + o:data0 + o + n], dtype=torch.uint8))
+        assert t.data_ptr() % 256 == 0
+        blobs.append(t)
+    bases = np.asarray([int(b.data_ptr()) for b in blobs], dtype=np.uint64)
+    for f in _ADDR_FIELDS:
+        units[f] += bases[blob_of]
+    units["v_off"] += bases[blob_of][:, None]
+    lib = _lib.load()
+    return StreamCache(
+        blobs=blobs, units=torch.from_numpy(units.view(np.uint8).copy()).to(dev),
+        work=(torch.from_numpy(work.view(np.uint8).copy()).to(dev) if len(work)
+              else torch.zeros(16, dtype=torch.uint8, device=dev)),
+        units_host=units, work_host=work, n_units=header["n_units"], n_work=header["n_work"], G=header["G"],
+        rows=header["rows"], stream_bytes=header["stream_bytes"], algorithmic_bytes=header["algorithmic_bytes"],
+        max_row_dwords=header["max_row_dwords"],
+        groups=torch.from_numpy(groups).to(dev) if groups is not None else None, groups_host=groups,
+        n_groups=header["n_groups"])

@@ -290,3 +290,26 @@ def test_fused_attention_k_row_shapes(counts):
     out, lse = stream_cache.decode_attn_fused(cache, q.to(DEV))
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
+
+
+def test_stream_cache_file_round_trip(tmp_path):
+    """A cache written to disk and loaded again (at other addresses) gives the same bits."""
+    cfg = synth.scaled(synth.CONFIGS[1], context=1200, layers=3)
+    packed, q, _ = _config_case(cfg, 3)
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    out, lse = stream_cache.decode_attn_fused(cache, q)
+    path = str(tmp_path / "cache.rdkv")
+    stream_cache.save_stream_cache(cache, path)
+    keep = [torch.empty(3_000_000, dtype=torch.uint8, device=DEV)]     # shift the allocator
+    loaded = stream_cache.load_stream_cache(path, DEV)
+    assert loaded.n_units == cache.n_units and loaded.n_work == cache.n_work and loaded.n_groups == cache.n_groups
+    assert loaded.algorithmic_bytes == cache.algorithmic_bytes
+    out2, lse2 = stream_cache.decode_attn_fused(loaded, q)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+    with pytest.raises(RuntimeError):
+        stream_cache.load_stream_cache(path, "cpu")
+    bad = tmp_path / "bad.rdkv"
+    bad.write_bytes(b"not a cache file, just sixteen+ bytes")
+    with pytest.raises(ValueError):
+        stream_cache.load_stream_cache(str(bad), DEV)
+    del keep
