@@ -450,8 +450,7 @@ def load_stream_cache(path: str, device) -> StreamCache:
     groups = section("groups", np.int32) if "groups" in header["sections"] else None
     blobs = []
     for o, n in header["blobs"]:
-        t = torch.empty(n, dtype=torch.uint8, device=dev)
-        t.copy_(torch.frombuffer(memoryview(mm)[data0 + o:data0 + o + n], dtype=torch.uint8))
+        t = torch.from_numpy(np.array(mm[data0 + o:data0 + o + n])).to(dev)   # np.array: writable copy
         assert t.data_ptr() % 256 == 0
         blobs.append(t)
     bases = np.asarray([int(b.data_ptr()) for b in blobs], dtype=np.uint64)
