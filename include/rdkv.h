@@ -172,7 +172,9 @@ typedef struct RdkvUnit {
   int32_t  d8, d4, d2;   /* K row dwords holding 8-, 4- and 2-bit channel fields              */
   int32_t  q_row;        /* first query/output row of this unit (G consecutive rows)          */
   int32_t  work_begin;   /* first work item / partial slot of this unit                       */
-  int32_t  work_count;   /* number of work items of this unit                                  */
+  int32_t  work_count;   /* number of work items to merge into the unit's rows.  Several units may
+                            share q_row (sources of one output row, adjacent in the table, their
+                            items contiguous): the first carries the total, the others 0        */
 } RdkvUnit;
 
 typedef struct RdkvSlot {   /* one K channel slot in MFMA consumption order */
@@ -239,9 +241,9 @@ int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int 
 /* rdkv_decode_fused_merge plus the attention over the decode-appended tokens of every unit
  * (zone C; fast_decode.py:1719-1735 scores of the new tokens, :1743-1755 softmax over
  * [old | new], :1777-1784 their V sum): the exact softmax over zones A+B+C, out and lse of the
- * union.  k_new / v_new: fp32 [n_units, >= n_new, 128] (unit u at + u*new_stride_unit, token t
- * at + t*new_stride_tok, elements); n_new tokens per unit, or n_new_per_unit[u] (device int32)
- * when not NULL (n_new is then ignored).  q / rope_*: as passed to rdkv_decode_fused_partials. */
+ * union.  k_new / v_new: fp32 [rows / G, >= n_new, 128], indexed by r = q_row / G of the unit
+ * (row r at + r*new_stride_unit, token t at + t*new_stride_tok, elements); n_new tokens per
+ * row, or n_new_per_unit[r] (device int32) when not NULL (n_new is then ignored).  q / rope_*: as passed to rdkv_decode_fused_partials. */
 int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G,
                                    const void *q, int q_dtype, int64_t q_stride_row,
                                    const void *rope_cos, const void *rope_sin, int rope_dtype,

@@ -750,6 +750,7 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
   const RdkvUnit *u = units + blockIdx.x;
+  if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   merge_unit(partials, u->work_begin, u->work_count, G, u->q_row, out, out_stride, lse, threadIdx.x, 256,
                     scratch);
 }
@@ -775,10 +776,12 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   __shared__ float m_run[8], l_run[8], f_old[8], lse_ab[8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const RdkvUnit *u = units + blockIdx.x;
+  if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   const int q_row = u->q_row;
+  const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
   merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, 256, scratch, acc_ab,
              lse_ab);
-  const int n_new = n_new_per_unit ? n_new_per_unit[blockIdx.x] : n_new_all;
+  const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
   for (int i = tid; i < G * kD; i += 256) {
     const int c = i & 127;
     const int64_t row = (int64_t)(q_row + (i >> 7)) * q_stride;
@@ -803,8 +806,8 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   float acc[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) acc[k] = tid + 256 * k < G * kD ? acc_ab[tid + 256 * k] : 0.0f;
-  const float *kn = k_new + (int64_t)blockIdx.x * new_stride_unit;
-  const float *vn = v_new + (int64_t)blockIdx.x * new_stride_unit;
+  const float *kn = k_new + (int64_t)kv_row * new_stride_unit;
+  const float *vn = v_new + (int64_t)kv_row * new_stride_unit;
   for (int t0 = 0; t0 < n_new; t0 += kZcChunk) {
     const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
     __syncthreads();

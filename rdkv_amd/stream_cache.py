@@ -171,10 +171,17 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
 
 def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
                        work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
-                       groups_per_cu: int = 1, cost: Optional[dict] = None) -> StreamCache:
+                       groups_per_cu: int = 1, cost: Optional[dict] = None,
+                       row_of_entry: Optional[Sequence[int]] = None) -> StreamCache:
     """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
     layer)) into the streaming format.  Query/output row of entry g, query head hq is
     ``g * H_q + hq``.
+
+    ``row_of_entry[i]`` = r makes entry i a *source* of output group r instead (rows
+    ``r * H_q + hq``): several entries with the same r are attended over together, the exact
+    softmax over the union of their tokens, each source keeping its own packing (channel
+    layout, scales) - the multi-source attention of blockwise decode
+    (blockwise_decode.py:812-1121) as one fused call.
 
     Work decomposition: by default the tile stream is cut into one run of equal cost per
     compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
@@ -223,7 +230,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             u = units[h]
             u["n_tok"] = n_tok
             u["d8"], u["d4"], u["d2"] = d8, d4, d2
-            u["q_row"] = gi * H_q + h * G
+            u["q_row"] = (gi if row_of_entry is None else int(row_of_entry[gi])) * H_q + h * G
             u["k_off"] = off
             off = _align(off + sum(tiles) * TILE * 4 * R)
             for c in range(4):
@@ -284,12 +291,24 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         torch.cuda.current_stream(dev).synchronize()
     units_np = np.array(units_all, dtype=UNIT_DTYPE)
     tiles_np = np.asarray(unit_tiles, dtype=np.int64).reshape(-1, 4)
+    R_np = np.asarray(unit_R, dtype=np.int64)
+    if row_of_entry is not None:
+        # sources of one output row next to each other, so that their work items are contiguous
+        order = np.argsort(units_np["q_row"], kind="stable")
+        units_np, tiles_np, R_np = units_np[order], tiles_np[order], R_np[order]
     if work_bytes is None and n_groups is None:
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
-    work_np, groups_np, wb, wc = partition_work(tiles_np, np.asarray(unit_R, dtype=np.int64),
+    work_np, groups_np, wb, wc = partition_work(tiles_np, R_np,
                                                 n_groups=n_groups, work_bytes=work_bytes,
                                                 cost=cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS))
+    if row_of_entry is not None:
+        # the first unit of every output row merges the partials of all its sources
+        qr = units_np["q_row"]
+        first = np.concatenate([[True], qr[1:] != qr[:-1]])
+        run_id = np.cumsum(first) - 1
+        wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
+        n_entries = int(max(row_of_entry)) + 1
     units_np["work_begin"], units_np["work_count"] = wb, wc
     rows = n_entries * H_q
     algo_bytes += rows * 128 * 2 + rows * 128 * 4
@@ -314,8 +333,8 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
     query); returns (out fp32 [rows,128], lse fp32 [rows]).  ``zone_c`` = (K_new, V_new[,
-    n_new_per_unit]): fp32 [n_units, n_new, 128] rows of the decode-appended tokens of every unit
-    (unit = entry * H_kv + kv head; optional int32 [n_units] counts when units differ): the merge
+    n_new_per_row]): fp32 [rows / G, n_new, 128] rows of the decode-appended tokens of every
+    (output group, KV head) (optional int32 [rows / G] counts when they differ): the merge
     launch then returns the exact softmax over packed cache + new tokens.  Graph-capturable once
     the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
@@ -350,11 +369,12 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     counts = zone_c[2] if len(zone_c) > 2 else None
     _lib.require_device(K_new, V_new)
     assert K_new.dtype == torch.float32 and V_new.dtype == torch.float32 and K_new.shape == V_new.shape
-    assert K_new.dim() == 3 and K_new.shape[0] == cache.n_units and K_new.shape[2] == 128, (
-        f"zone C tensors must be [n_units={cache.n_units}, n_new, 128], got {tuple(K_new.shape)}")
+    n_kv_rows = cache.rows // cache.G
+    assert K_new.dim() == 3 and K_new.shape[0] == n_kv_rows and K_new.shape[2] == 128, (
+        f"zone C tensors must be [rows / G = {n_kv_rows}, n_new, 128], got {tuple(K_new.shape)}")
     assert K_new.stride() == V_new.stride() and K_new.stride(2) == 1
     if counts is not None:
-        assert counts.dtype == torch.int32 and counts.numel() == cache.n_units and counts.is_contiguous()
+        assert counts.dtype == torch.int32 and counts.numel() == n_kv_rows and counts.is_contiguous()
     _lib.check(lib.rdkv_decode_fused_partials(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
         _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,

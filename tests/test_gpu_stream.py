@@ -313,3 +313,39 @@ def test_stream_cache_file_round_trip(tmp_path):
     with pytest.raises(ValueError):
         stream_cache.load_stream_cache(str(bad), DEV)
     del keep
+
+
+def test_multi_source_rows():
+    """Two packed sources per output row (each with its own K channel layout and scales) in
+    one cache: the result is the LSE merge of the two single-source results, and with zone C
+    on top the softmax over all three."""
+    from rdkv_amd import fast_decode
+    cfg = synth.scaled(synth.CONFIGS[1], context=900, layers=4)
+    packed, q4, _ = _config_case(cfg, 4)
+    q = q4[:2 * cfg.H_q].contiguous()                  # two output groups
+    # entries 0,2 -> group 0; entries 1,3 -> group 1
+    cache = stream_cache.build_stream_cache(packed, cfg.G, row_of_entry=[0, 1, 0, 1])
+    assert cache.rows == 2 * cfg.H_q and cache.n_units == 4 * cfg.H_kv
+    assert int((cache.units_host["work_count"] == 0).sum()) == 2 * cfg.H_kv
+    out, lse = stream_cache.decode_attn_fused(cache, q)
+    singles = [stream_cache.decode_attn_fused(stream_cache.build_stream_cache([packed[i]], cfg.G),
+                                              q[(i % 2) * cfg.H_q:(i % 2 + 1) * cfg.H_q].contiguous())
+               for i in range(4)]
+    for grp in range(2):
+        (oa, la), (ob, lb) = singles[grp], singles[grp + 2]
+        m = torch.maximum(la, lb)
+        wa, wb = torch.exp(la - m), torch.exp(lb - m)
+        exp_out = (oa * wa[:, None] + ob * wb[:, None]) / (wa + wb)[:, None]
+        exp_lse = m + torch.log(wa + wb)
+        r = slice(grp * cfg.H_q, (grp + 1) * cfg.H_q)
+        assert float((out[r] - exp_out).abs().max()) < 2e-5
+        assert float((lse[r] - exp_lse).abs().max()) < 2e-5
+    # zone C on top, against the PyTorch merge of the two-source result
+    g = torch.Generator().manual_seed(2)
+    K_new = [torch.randn(cfg.H_kv, 9, 128, generator=g).to(DEV) for _ in range(2)]
+    V_new = [torch.randn(cfg.H_kv, 9, 128, generator=g).to(DEV) for _ in range(2)]
+    got = fast_decode.trizone_attention_fused(cache, q, K_new, V_new, cfg.G)
+    for grp in range(2):
+        r = slice(grp * cfg.H_q, (grp + 1) * cfg.H_q)
+        exp = fast_decode.merge_zone_c(out[r], lse[r], q[r], K_new[grp], V_new[grp], cfg.G)
+        assert float((got[r] - exp).abs().max()) < 2e-5
