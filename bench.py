@@ -25,7 +25,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the fused kernel on the default workload, from two rocprofv3 --pmc
 # runs of this command (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors a plain copy
 # kernel of known size gives): (556 752 x 2 + 3 100) KiB.  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: 1143402496}
+MEASURED_TRAFFIC_BYTES = {1: 1143576576}
 
 
 def parse():
