@@ -252,6 +252,42 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
                                    float *out, int64_t out_stride_row, float *lse,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- prefill-time selection feeding the packer ---------------------------------------------
+ * obkv_fast.py:208-249  apply_score_pooling, as used on the per-head token scores at
+ * obkv_fast.py:961-967.  Stride-1 pooling of B rows of T fp32 scores (row stride in elements).
+ * reflect != 0: kernel min(kernel_size, 2T-1), mirrored borders without the edge sample;
+ * else implicit borders of kernel_size/2 (zeros that count in the average's divisor, minus
+ * infinity for the max).  is_avg == 0 is the max.  The window is summed left to right in fp32
+ * starting from zero and divided once.  Writes T + 2*(k/2) - k + 1 values per row. */
+int rdkv_pool_scores(const float *scores, int64_t stride_b, int B, int64_t T, int kernel_size,
+                     int is_avg, int reflect, float *out, int64_t out_stride_b, void *stream);
+
+/* knapsack_solver.py:121-248  knapsack_bit_allocation_batched (called at obkv_fast.py:986-991
+ * for the tokens of every KV head and, through _allocate_k_bits_per_head obkv_fast.py:579-618,
+ * for the channels).  Row b of `scores` [B, T] gets, per token, the option n minimising
+ * score*eps[n] + lambda_b*bits[n] at the lambda_b the reference's fp32 bisection stops at
+ * (same bound, same doubling rounds including their whole-batch exit, same tolerance test,
+ * same fallbacks), bit for bit.  budget: B fp32 values on the device (average bits per token).
+ * bits_host / eps_host: n_options (<= 8) HOST floats; widths must be integers in 0..255.
+ * out: [B, T] of out_elem_size 1 (u8) or 8 (i64) bytes, row stride in elements.  counts: NULL
+ * or device [B, n_options] int32, tokens per option.  T <= 2^20 (the width sums stay exact).
+ * workspace: rdkv_knapsack_workspace_bytes(B) bytes.  Two launches, no host synchronization. */
+int64_t rdkv_knapsack_workspace_bytes(int B);
+int rdkv_knapsack_batched(const float *scores, int64_t stride_b, int B, int64_t T,
+                          const float *budget, const float *bits_host, const float *eps_host,
+                          int n_options, int max_iters, float tol, void *out, int out_elem_size,
+                          int64_t out_stride_b, int32_t *counts, void *workspace,
+                          int64_t workspace_bytes, void *stream);
+
+/* knapsack_solver.py:39-118  knapsack_bit_allocation applied to each of B independent rows:
+ * lambda is bisected in double and rounded to fp32 where it meets the scores, the bound starts
+ * at 0.375*max without a floor and doubles while it is below 1e12, averages are fp32 values
+ * compared in double.  budget: B doubles on the device.  Other arguments as above. */
+int rdkv_knapsack_rows(const float *scores, int64_t stride_b, int B, int64_t T, const double *budget,
+                       const float *bits_host, const float *eps_host, int n_options, int max_iters,
+                       double tol, void *out, int out_elem_size, int64_t out_stride_b,
+                       int32_t *counts, void *stream);
+
 /* ---- measurement helpers (no counterpart in the reference) --------------------------------
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)

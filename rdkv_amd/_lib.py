@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_void_p
 from typing import Optional
 
 import torch
@@ -28,6 +28,8 @@ DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 P = c_void_p
 I = c_int
 L = c_int64
+F = c_float
+Dbl = c_double
 
 # name -> (restype, argtypes); must list every symbol include/rdkv.h declares.
 SIGNATURES = {
@@ -55,6 +57,10 @@ SIGNATURES = {
     "rdkv_decode_fused_merge_zone_c": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, I, P, P, L, P, P, L, P]),
     "rdkv_rope": (I, [P, L, I, P, L, I, I, I, P, P, I, P]),
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
+    "rdkv_pool_scores": (I, [P, L, I, L, I, I, I, P, L, P]),
+    "rdkv_knapsack_workspace_bytes": (L, [I]),
+    "rdkv_knapsack_batched": (I, [P, L, I, L, P, P, P, I, I, F, P, I, L, P, P, L, P]),
+    "rdkv_knapsack_rows": (I, [P, L, I, L, P, P, P, I, I, Dbl, P, I, L, P, P]),
     "rdkv_probe_copy": (I, [P, P, L, P]),
     "rdkv_probe_read": (I, [P, L, L, P, P]),
     "rdkv_probe_read_stream": (I, [P, L, L, P, P]),

@@ -22,7 +22,7 @@ COMMON = [
     "-Wno-unused-command-line-argument",
 ]
 # bit-exact quantizer code must not contract a*b+c into fma
-PER_FILE = {"quantize.hip": ["-ffp-contract=off"]}
+PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "select.hip": ["-ffp-contract=off"]}
 
 
 def _hipcc() -> str:

@@ -1,0 +1,160 @@
+"""Prefill-time selection feeding the packer, with the names of the reference's ``obkv_fast``.
+
+Only the per-layer selection + packing step is here (score pooling, the per-head V knapsack,
+the per-head K allocation and the hand-over to the whole-layer packer); model loading, scoring
+and the decode loops of the reference's module are not part of this package.  Everything runs
+on the GPU: the only device-to-host reads are the packer's (per-head segment sizes and the
+[H_kv, D] K widths, which fix the shapes of the packed tensors).
+"""
+from __future__ import annotations
+
+import time
+from typing import Dict, Optional, Union
+
+import torch
+from torch import Tensor
+
+from . import _lib
+from .knapsack_solver import knapsack_allocate, knapsack_bit_allocation_batched
+from .packing import pack_layer_per_head
+
+
+def apply_score_pooling(scores: Tensor, pool_type: str, kernel_size: int, padding_mode: str = "zero") -> Tensor:
+    """obkv_fast.py:208-249.  Stride-1 pooling of ``[T]`` or ``[B, T]`` scores: "avg" or (anything
+    else) max; "reflect" mirrors the borders (kernel clipped to ``2T-1``), other modes use the
+    library's implicit border (zeros counted in the divisor / minus infinity).  fp32 result."""
+    if scores.dim() not in (1, 2):
+        raise ValueError(f"Expected score tensor rank 1 or 2, got shape={tuple(scores.shape)}.")
+    dev = _lib.require_device(scores)
+    x = scores.detach().float()
+    one_d = x.dim() == 1
+    if one_d:
+        x = x.unsqueeze(0)
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    B, T = int(x.shape[0]), int(x.shape[1])
+    reflect = padding_mode == "reflect"
+    k = int(kernel_size)
+    if reflect:
+        if T <= 0:
+            raise ValueError("Cannot reflect-pool an empty score sequence.")
+        k = min(k, 2 * T - 1)
+    L = T + 2 * (k // 2) - k + 1
+    out = torch.empty(B, max(L, 0), dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().rdkv_pool_scores(
+        _lib.ptr(x), x.stride(0), B, T, int(kernel_size), 1 if pool_type == "avg" else 0, 1 if reflect else 0,
+        _lib.ptr(out), out.stride(0), _lib.stream_of(dev)))
+    return out[0] if one_d else out
+
+
+def _allocate_k_bits_per_head(channel_scores: Tensor, k_avg: Union[float, Tensor], *, epsilon,
+                              bit_options) -> Tensor:
+    """obkv_fast.py:579-618: ``[H_kv, D]`` channel scores, a shared float budget or one per head;
+    one batched solve.  Returns ``[H_kv, D]`` long."""
+    assert channel_scores.dim() == 2, (
+        f"_allocate_k_bits_per_head expects [H_kv, D]; got {tuple(channel_scores.shape)}")
+    H_kv = int(channel_scores.shape[0])
+    if torch.is_tensor(k_avg):
+        assert k_avg.dim() == 1 and int(k_avg.shape[0]) == H_kv, (
+            f"k_avg tensor must be [H_kv={H_kv}]; got {tuple(k_avg.shape)}")
+        k_avg_arg: Union[float, Tensor] = k_avg.detach().float()
+    else:
+        k_avg_arg = float(k_avg)
+    return knapsack_bit_allocation_batched(channel_scores, k_avg_arg, epsilon=epsilon, bit_options=bit_options)
+
+
+def _perhead_select_and_pack_joint(
+    K: Tensor, V: Tensor, layer_scores: Tensor, channel_scores: Tensor, *,
+    gqa_factor: int, token_budget: int, k_budget_ratio: float, obs_window: int,
+    pool_kernel_size: int, pool_padding: str, pool_type: str,
+    v_bit_options: Optional[Tensor], k_bit_options: Optional[Tensor],
+    eps_V: Dict[int, float], eps_K: Dict[int, float],
+    timing: Optional[Dict[str, float]] = None, retain_allocation_metadata: bool = False,
+):
+    """obkv_fast.py:899-1186.  K, V ``[1, H_kv, T, D]`` fp16 on the device; ``layer_scores
+    [H_kv, T]`` and ``channel_scores [H_kv, D]`` (moved to the device if they are not there).
+
+    Per head one knapsack over all T tokens with widths {0,2,4,8,16} at an average of
+    ``(1-r) * 2 * token_budget * 16 / T`` bits per element (0 evicts, 16 keeps fp16), then one
+    knapsack over the head's channels at ``r * 2 * token_budget * D * 16 / (D * kept_h)`` bits,
+    then the whole-layer packer.  Channels with 0 bits are left out of the packed K by the
+    packer, which is all the reference's zeroing of those channels (:1105-1107) amounts to.
+    Returns ``(packed_layer, new_v_only, packed_layer.T_eff)``.  ``timing``, when given, collects
+    the reference's stage times in ms (each stage then ends with a device synchronization)."""
+    assert K.dim() == 4 and V.dim() == 4, f"K/V must be [1,H_kv,T,D], got {tuple(K.shape)}/{tuple(V.shape)}"
+    assert layer_scores.dim() == 2, f"layer_scores must be [H_kv,T], got {tuple(layer_scores.shape)}"
+    assert channel_scores.dim() == 2, (
+        f"_perhead_select_and_pack_joint: channel_scores must be [H_kv, D], got {tuple(channel_scores.shape)}")
+    dev = _lib.require_device(K, V)
+    H_kv, T = int(layer_scores.shape[0]), int(layer_scores.shape[1])
+    head_dim = int(K.shape[3])
+
+    def stamp() -> float:
+        if timing is None:
+            return 0.0
+        torch.cuda.synchronize(dev)
+        return time.perf_counter()
+
+    t0 = stamp()
+    scores_dev = layer_scores.to(dev)
+    if pool_kernel_size > 1:
+        pooled = apply_score_pooling(scores_dev, pool_type=pool_type, kernel_size=pool_kernel_size,
+                                     padding_mode=pool_padding)
+    else:
+        pooled = scores_dev.float()
+    t_pool = stamp()
+
+    total_budget_bits = 2 * token_budget * head_dim * 16
+    v_budget_bits = (1.0 - k_budget_ratio) * total_budget_bits
+    v_avg = v_budget_bits / (T * head_dim)
+    k_budget_bits = k_budget_ratio * total_budget_bits
+    v_bits_all, v_counts = knapsack_allocate(pooled, v_avg, epsilon=eps_V, bit_options=v_bit_options,
+                                             with_counts=True)
+    t_v = stamp()
+
+    # tokens kept by a head = everything that did not take the 0-bit option
+    v_opts = [0.0, 2.0, 4.0, 8.0, 16.0] if v_bit_options is None else [float(b) for b in v_bit_options.tolist()]
+    kept_cols = [i for i, b in enumerate(v_opts) if b > 0]
+    t_eff = v_counts[:, kept_cols].sum(dim=1)
+    # the reference's fp32 expression k_budget_bits / (head_dim * kept.float()) is evaluated by torch as
+    # reciprocal(denominator) * k_budget_bits; each step goes through double here and is rounded to fp32
+    # once, which gives the correctly rounded fp32 value of that step whatever the device's fp32 division does
+    denom = (float(head_dim) * t_eff.clamp(min=1).double()).float()
+    recip = (1.0 / denom.double()).float()
+    k_avg_per_head = (recip.double() * torch.tensor(k_budget_bits, dtype=torch.float32).double().item()).float()
+    k_bits_perhead = _allocate_k_bits_per_head(channel_scores.float().to(dev), k_avg_per_head,
+                                               epsilon=eps_K, bit_options=k_bit_options)
+    t_k = stamp()
+
+    packed_layer, new_v_only = pack_layer_per_head(K, V, v_bits_all, k_bits_perhead, gqa_factor)
+    if retain_allocation_metadata:
+        packed_layer.allocation_v_bits = v_bits_all.to(torch.int16)
+        packed_layer.allocation_k_bits = k_bits_perhead.to(torch.int16)
+    t_pack = stamp()
+
+    if timing is not None:
+        for key, a, b in (("pooling_ms", t0, t_pool), ("v_allocation_ms", t_pool, t_v),
+                          ("k_allocation_ms", t_v, t_k), ("quantization_ms", t_k, t_pack)):
+            timing[key] = timing.get(key, 0.0) + (b - a) * 1000.0
+        timing["packing_ms"] = timing.get("packing_ms", 0.0)    # quantization and packing are one step here
+    return packed_layer, new_v_only, packed_layer.T_eff
+
+
+def _perhead_select_and_pack(
+    K: Tensor, V: Tensor, layer_scores: Tensor, channel_scores: Tensor, *,
+    gqa_factor: int, eviction_mode: str = "joint", token_budget: int, k_budget_ratio: float,
+    obs_window: int, pool_kernel_size: int, pool_padding: str, pool_type: str = "avg",
+    v_bit_options: Optional[Tensor], k_bit_options: Optional[Tensor],
+    eps_V: Dict[int, float], eps_K: Dict[int, float], n_kept_multiplier: float = 5.0,
+    timing: Optional[Dict[str, float]] = None, retain_allocation_metadata: bool = False,
+):
+    """obkv_fast.py:1189-1235: the only eviction mode is "joint"."""
+    if eviction_mode != "joint":
+        raise ValueError(f"Unsupported eviction_mode={eviction_mode!r}; expected 'joint'.")
+    del n_kept_multiplier
+    return _perhead_select_and_pack_joint(
+        K, V, layer_scores, channel_scores, gqa_factor=gqa_factor, token_budget=token_budget,
+        k_budget_ratio=k_budget_ratio, obs_window=obs_window, pool_kernel_size=pool_kernel_size,
+        pool_padding=pool_padding, pool_type=pool_type, v_bit_options=v_bit_options,
+        k_bit_options=k_bit_options, eps_V=eps_V, eps_K=eps_K, timing=timing,
+        retain_allocation_metadata=retain_allocation_metadata)

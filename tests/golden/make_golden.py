@@ -280,6 +280,90 @@ def case_rope():
     save("rope", d)
 
 
+# ---------------------------------------------------------------- knapsack
+def case_knapsack():
+    """Outputs of the reference's Lagrangian solvers (knapsack_solver.py at the reference root;
+    it imports only torch) on seeded score rows: default and per-row budgets, both option sets
+    of the K side, ties, constant and all-zero rows, budgets no allocation can meet (the
+    doubling rounds and their whole-batch exit), single-token rows, and the single-row variants."""
+    import knapsack_solver as ks
+
+    g = torch.Generator().manual_seed(909)
+    lognormal = lambda *shape, mu=2.0, sd=1.5: torch.exp(torch.randn(*shape, generator=g) * sd + mu)
+    d = {}
+    batched = []
+
+    def add_batched(name, scores, budget, eps, options, **kw):
+        out = ks.knapsack_bit_allocation_batched(
+            scores, budget, epsilon=eps,
+            bit_options=None if options is None else torch.tensor(options, dtype=torch.float32), **kw)
+        opts = list(ks.BITS.tolist()) if options is None else options
+        d[f"{name}.scores"] = npy(scores)
+        d[f"{name}.budget"] = npy(budget.float() if torch.is_tensor(budget) else torch.tensor(float(budget)))
+        d[f"{name}.options"] = np.asarray(opts, dtype=np.float32)
+        d[f"{name}.eps"] = np.asarray([eps[int(b)] for b in opts], dtype=np.float64)
+        d[f"{name}.max_iters"] = np.asarray(kw.get("max_iters", 64))
+        d[f"{name}.tol"] = np.asarray(kw.get("tol", 0.01))
+        d[f"{name}.bits"] = npy(out).astype(np.uint8)
+        batched.append(name)
+
+    add_batched("v_default", lognormal(4, 1000), 2.0, ks.DEFAULT_EPSILON_V, None)
+    add_batched("v_rows", lognormal(6, 777), torch.tensor([0.5, 1.0, 3.0, 6.0, 20.0, 0.01]),
+                ks.DEFAULT_EPSILON_V, None)
+    add_batched("v_long", lognormal(2, 5000, sd=2.5), 1.2, ks.DEFAULT_EPSILON, None)
+    add_batched("v_tight_tol", lognormal(3, 600), 2.5, ks.DEFAULT_EPSILON_V, None, tol=1e-5)
+    add_batched("v_few_iters", lognormal(3, 600), 2.5, ks.DEFAULT_EPSILON_V, None, max_iters=3, tol=1e-4)
+    chan = lognormal(8, 128, mu=1.0, sd=1.0)
+    add_batched("k_0248", chan, torch.tensor([0.7, 1.5, 2.0, 3.3, 4.0, 6.5, 8.0, 4096.0]),
+                ks.DEFAULT_EPSILON_K, [0.0, 2.0, 4.0, 8.0])
+    add_batched("k_24816", chan, torch.tensor([2.5, 3.0, 4.0, 5.0, 7.0, 9.0, 12.0, 16.0]),
+                ks.DEFAULT_EPSILON_K, [2.0, 4.0, 8.0, 16.0])
+    # budgets below the smallest option: rows that double for all 40 rounds next to ordinary rows
+    add_batched("k_unreachable_mixed", chan, torch.tensor([1.0, 3.0, 1.5, 5.0, 0.5, 2.0, 2.01, 8.0]),
+                ks.DEFAULT_EPSILON_K, [2.0, 4.0, 8.0, 16.0])
+    # every row unreachable: the doubling stops once every bound has passed 1e12
+    add_batched("k_unreachable_all", lognormal(3, 64, mu=6.0), 1.0, ks.DEFAULT_EPSILON_K, [2.0, 4.0, 8.0, 16.0])
+    ties = torch.randint(0, 4, (5, 300), generator=g).float() * 2.5
+    ties[3] = 1.75
+    ties[4] = 0.0
+    add_batched("ties", ties, torch.tensor([1.0, 2.0, 4.0, 2.0, 2.0]), ks.DEFAULT_EPSILON_V, None)
+    add_batched("tiny", lognormal(4, 1), torch.tensor([0.5, 2.0, 7.9, 16.0]), ks.DEFAULT_EPSILON_V, None)
+    add_batched("pair", lognormal(3, 2), 5.0, ks.DEFAULT_EPSILON_V, None)
+    small = lognormal(2, 400) * 1e-9
+    add_batched("small_scores", small, 2.0, ks.DEFAULT_EPSILON_V, None)
+    d["batched_cases"] = np.array(",".join(batched))
+
+    # single-row variants (lambda in double)
+    rows = lognormal(5, 900)
+    budgets = [1.0, 2.0, 3.0, 4.0, 6.0]
+    d["scalar.scores"] = npy(rows)
+    d["scalar.budgets"] = np.asarray(budgets)
+    d["scalar.bits"] = np.stack([
+        npy(ks.knapsack_bit_allocation(rows[i], budgets[i], epsilon=ks.DEFAULT_EPSILON)).astype(np.uint8)
+        for i in range(5)])
+    d["scalar.bits_k24816"] = np.stack([
+        npy(ks.knapsack_bit_allocation(rows[i, :128], budgets[i] + 1.5, epsilon=ks.DEFAULT_EPSILON_K,
+                                       bit_options=torch.tensor([2.0, 4.0, 8.0, 16.0]))).astype(np.uint8)
+        for i in range(5)])
+    topk = [0, 10, 900, 400, 37]
+    tb = [2.0, 6.0, 3.0, 0.1, 2.0]
+    d["topk.k"] = np.asarray(topk)
+    d["topk.budgets"] = np.asarray(tb)
+    import warnings
+    with warnings.catch_warnings():
+        warnings.simplefilter("ignore")
+        d["topk.bits"] = np.stack([
+            npy(ks.allocate_v_bits_with_fp16_topk(rows[i], tb[i], fp16_topk=topk[i],
+                                                  epsilon=ks.DEFAULT_EPSILON_V)[0]).astype(np.uint8)
+            for i in range(5)])
+    kb, vb = ks.knapsack_solve_kv_split(rows[0], chan[0], budget_per_token=3.0, k_budget_ratio=0.4)
+    d["split.token_scores"] = npy(rows[0])
+    d["split.channel_scores"] = npy(chan[0])
+    d["split.k_bits"] = npy(kb).astype(np.uint8)
+    d["split.v_bits"] = npy(vb).astype(np.uint8)
+    save("knapsack", d)
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
     if len(sys.argv) > 2:                      # python make_golden.py <ref> <case> : one case only
@@ -296,3 +380,5 @@ if __name__ == "__main__":
                       fr=[(0.0, 0.0, 0.0, 0.6), (0.5, 0.0, 0.3, 0.0), (0.0, 0.9, 0.0, 0.1)],
                       k_keep=[(0, 64, 0), (7, 0, 30), (3, 5, 2)], outliers=False)
     case_shared_layout()
+    case_rope()
+    case_knapsack()

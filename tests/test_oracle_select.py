@@ -1,0 +1,158 @@
+"""The selection oracle (score pooling, Lagrangian knapsack, per-head budgets) against the golden
+vectors written by the reference's own solvers, against the library routines the pooling reduces
+to, and against closed forms that a plausible restatement mistake would break."""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import select_oracle as S
+from tests.helpers import load_golden
+
+F32 = np.float32
+
+
+def golden_batched_cases():
+    g = load_golden("knapsack")
+    for name in str(g["batched_cases"]).split(","):
+        opts = g[name + ".options"]
+        eps = {int(b): float(e) for b, e in zip(opts, g[name + ".eps"])}
+        bud = g[name + ".budget"]
+        yield name, dict(scores=g[name + ".scores"], budget=float(bud) if bud.ndim == 0 else bud, eps=eps,
+                         options=opts, max_iters=int(g[name + ".max_iters"]), tol=float(g[name + ".tol"]),
+                         bits=g[name + ".bits"])
+
+
+@pytest.mark.parametrize("name,case", list(golden_batched_cases()), ids=lambda v: v if isinstance(v, str) else "")
+def test_batched_knapsack_matches_reference_outputs(name, case):
+    out = S.knapsack_bit_allocation_batched(case["scores"], case["budget"], epsilon=case["eps"],
+                                            max_iters=case["max_iters"], tol=case["tol"],
+                                            bit_options=case["options"])
+    assert out.dtype == np.int64
+    np.testing.assert_array_equal(out, case["bits"].astype(np.int64))
+
+
+def test_single_row_variants_match_reference_outputs():
+    g = load_golden("knapsack")
+    rows = g["scalar.scores"]
+    for i in range(rows.shape[0]):
+        b = float(g["scalar.budgets"][i])
+        np.testing.assert_array_equal(S.knapsack_bit_allocation(rows[i], b, S.DEFAULT_EPSILON), g["scalar.bits"][i])
+        np.testing.assert_array_equal(
+            S.knapsack_bit_allocation(rows[i, :128], b + 1.5, S.DEFAULT_EPSILON_K, bit_options=(2, 4, 8, 16)),
+            g["scalar.bits_k24816"][i])
+        np.testing.assert_array_equal(
+            S.allocate_v_bits_with_fp16_topk(rows[i], float(g["topk.budgets"][i]), int(g["topk.k"][i]),
+                                             S.DEFAULT_EPSILON_V), g["topk.bits"][i])
+    kb, vb = S.knapsack_solve_kv_split(g["split.token_scores"], g["split.channel_scores"], 3.0, k_budget_ratio=0.4)
+    np.testing.assert_array_equal(kb, g["split.k_bits"])
+    np.testing.assert_array_equal(vb, g["split.v_bits"])
+
+
+def test_knapsack_closed_forms():
+    rng = np.random.default_rng(5)
+    s = np.exp(rng.standard_normal((3, 257)) * 1.5 + 2).astype(F32)
+    # a budget no smaller than the widest option: lambda = 0, every scored token takes 16 bits
+    assert (S.knapsack_bit_allocation_batched(s, 16.0) == 16).all()
+    assert (S.knapsack_bit_allocation_batched(s, np.array([16, 17, 1e9], F32)) == 16).all()
+    # a constant row can only be all-equal; at budget 2 with the default table the bisection stops on 2 bits
+    const = np.full((1, 100), 3.5, F32)
+    out = S.knapsack_bit_allocation_batched(const, 2.0)
+    assert (out == out[0, 0]).all() and out[0, 0] == 2
+    # all-zero scores cost nothing at 0 bits
+    assert (S.knapsack_bit_allocation_batched(np.zeros((2, 9), F32), 3.0) == 0).all()
+    # rows are independent except through the doubling rounds: reachable budgets give the same row alone or batched
+    both = S.knapsack_bit_allocation_batched(s, np.array([1.0, 2.5, 6.0], F32))
+    for r in range(3):
+        alone = S.knapsack_bit_allocation_batched(s[r:r + 1], np.array([[1.0, 2.5, 6.0][r]], F32))
+        np.testing.assert_array_equal(both[r], alone[0])
+    # the result is monotone in the score and meets the budget within the tolerance when it converged
+    out = S.knapsack_bit_allocation_batched(s, 3.0)
+    for r in range(3):
+        order = np.argsort(s[r], kind="stable")
+        assert (np.diff(out[r][order]) >= 0).all()
+        assert abs(out[r].mean() - 3.0) / 3.0 < 0.0101
+
+
+def test_knapsack_is_a_lagrangian_optimum_on_tiny_rows():
+    """Brute force: for the allocation returned there is no other allocation with at most the same
+    number of bits and a strictly smaller distortion (the property a Lagrangian solution has)."""
+    rng = np.random.default_rng(11)
+    opts = (0, 2, 4, 8, 16)
+    eps = S.DEFAULT_EPSILON_V
+    for trial in range(6):
+        s = np.exp(rng.standard_normal((1, 5)) * 1.2 + 1).astype(F32)
+        out = S.knapsack_bit_allocation_batched(s, float(rng.uniform(1.0, 9.0)), epsilon=eps, tol=0.05)[0]
+        used = int(out.sum())
+        dist = sum(float(s[0, t]) * eps[int(out[t])] for t in range(5))
+        for alloc in itertools.product(opts, repeat=5):
+            if sum(alloc) <= used:
+                d = sum(float(s[0, t]) * eps[alloc[t]] for t in range(5))
+                assert d >= dist * (1 - 1e-6), (alloc, out)
+
+
+POOL_CASES = [(1, 1), (1, 7), (2, 7), (3, 7), (4, 7), (5, 3), (64, 7), (257, 7), (100, 5), (100, 4), (33, 1),
+              (9, 13), (31, 2)]
+
+
+@pytest.mark.parametrize("T,k", POOL_CASES)
+@pytest.mark.parametrize("pool_type", ["avg", "max"])
+@pytest.mark.parametrize("padding", ["reflect", "zero"])
+def test_pooling_matches_the_library_routines(T, k, pool_type, padding):
+    rng = np.random.default_rng(T * 31 + k)
+    x = (rng.standard_normal((3, T)) * 4).astype(F32)
+    fn = F.avg_pool1d if pool_type == "avg" else F.max_pool1d
+    xt = torch.from_numpy(x).unsqueeze(1)
+    if padding == "reflect":
+        ke = min(k, 2 * T - 1)
+        ref = fn(F.pad(xt, (ke // 2, ke // 2), mode="reflect") if ke // 2 else xt, kernel_size=ke, stride=1)
+    else:
+        ref = fn(xt, kernel_size=k, stride=1, padding=k // 2)
+    got = S.apply_score_pooling(x, pool_type, k, padding)
+    assert got.dtype == F32
+    np.testing.assert_array_equal(got.view(np.uint32), ref.squeeze(1).numpy().view(np.uint32))
+    one = S.apply_score_pooling(x[0], pool_type, k, padding)
+    np.testing.assert_array_equal(one, got[0])
+
+
+def test_pooling_closed_forms():
+    x = np.arange(1, 8, dtype=F32)[None]                  # 1..7
+    np.testing.assert_array_equal(S.apply_score_pooling(x, "avg", 3, "reflect")[0],
+                                  np.array([(2 + 1 + 2) / 3, 2, 3, 4, 5, 6, (6 + 7 + 6) / 3], F32))
+    np.testing.assert_array_equal(S.apply_score_pooling(x, "avg", 3, "zero")[0],
+                                  np.array([1, 2, 3, 4, 5, 6, 13 / 3], F32).astype(F32))
+    np.testing.assert_array_equal(S.apply_score_pooling(x, "max", 3, "zero")[0], np.array([2, 3, 4, 5, 6, 7, 7], F32))
+    # a kernel wider than the mirrored row is clipped to 2T-1
+    np.testing.assert_array_equal(S.apply_score_pooling(x[:, :2], "avg", 7, "reflect"),
+                                  S.apply_score_pooling(x[:, :2], "avg", 3, "reflect"))
+    with pytest.raises(ValueError):
+        S.apply_score_pooling(np.zeros((1, 0), F32), "avg", 7, "reflect")
+    with pytest.raises(ValueError):
+        S.apply_score_pooling(np.zeros((1, 1, 1), F32), "avg", 7, "reflect")
+
+
+def test_select_joint_budgets():
+    """Budget arithmetic of the per-layer selection: with ratio r, budget B tokens and T tokens the V
+    side averages (1-r)*32*B/T bits; the K side gets r*32*B*D bits per head over D*kept_h elements."""
+    rng = np.random.default_rng(3)
+    H, T, D, B = 3, 600, 128, 150
+    ls = np.exp(rng.standard_normal((H, T)) * 1.5).astype(F32)
+    cs = np.exp(rng.standard_normal((H, D))).astype(F32)
+    pooled, vb, kb, k_avg = S.select_joint(ls, cs, head_dim=D, token_budget=B, k_budget_ratio=0.5,
+                                           pool_kernel_size=7, pool_padding="reflect",
+                                           k_bit_options=(0, 2, 4, 8))
+    np.testing.assert_array_equal(pooled, S.apply_score_pooling(ls, "avg", 7, "reflect"))
+    v_avg = 0.5 * 32 * B / T
+    assert np.all(np.abs(vb.mean(axis=1) - v_avg) / v_avg < 0.0101)
+    kept = (vb > 0).sum(axis=1)
+    np.testing.assert_allclose(k_avg, 0.5 * 32 * B * D / (D * kept), rtol=3e-7)
+    np.testing.assert_array_equal(kb, S.knapsack_bit_allocation_batched(cs, k_avg, epsilon=S.DEFAULT_EPSILON_K,
+                                                                        bit_options=(0, 2, 4, 8)))
+    # a head that keeps nothing divides by one token: its K budget saturates every channel
+    ls0 = ls.copy()
+    ls0[1] = 0.0
+    _, vb0, kb0, k_avg0 = S.select_joint(ls0, cs, head_dim=D, token_budget=B, k_budget_ratio=0.5,
+                                         pool_kernel_size=1, pool_padding="reflect", k_bit_options=(0, 2, 4, 8))
+    assert (vb0[1] == 0).all() and k_avg0[1] == F32(0.5 * 32 * B * D) * (F32(1) / F32(D)) and (kb0[1] == 8).all()
