@@ -117,6 +117,44 @@ def main():
                              "note": "wall time of packing.pack_layer_per_head (+ stream_cache.build_stream_cache) "
                                      "on layer 0, median of 5 after 1 warm-up; K is read twice (min/max pass, "
                                      "then emit)"}
+                # prefill selection feeding the packer on the same layer: score pooling, per-head V
+                # knapsack, per-head K allocation, then the pack (seeded log-normal scores; the
+                # budget is a quarter of the context, half of it for K)
+                from rdkv_amd import knapsack_solver, obkv_fast
+                gsel = torch.Generator().manual_seed(4242)
+                H_kv, T_ctx = int(K.shape[1]), int(K.shape[2])
+                tok_scores = torch.exp(torch.randn(H_kv, T_ctx, generator=gsel) * 1.5 + 2.0).to(dev)
+                ch_scores = torch.exp(torch.randn(H_kv, 128, generator=gsel)).to(dev)
+                sel_kw = dict(gqa_factor=cfg.G, token_budget=max(T_ctx // 4, 1), k_budget_ratio=0.5, obs_window=32,
+                              pool_kernel_size=7, pool_padding="reflect", pool_type="avg", v_bit_options=None,
+                              k_bit_options=torch.tensor([0.0, 2.0, 4.0, 8.0]),
+                              eps_V=knapsack_solver.DEFAULT_EPSILON_V, eps_K=knapsack_solver.DEFAULT_EPSILON_K)
+                sel_ms, stages = [], {}
+                for it in range(6):
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, **sel_kw)
+                    torch.cuda.synchronize()
+                    sel_ms.append((time.perf_counter() - t0) * 1e3)
+                obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, timing=stages, **sel_kw)
+                select_info = {"select_and_pack_ms_per_layer": float(np.median(sel_ms[1:])),
+                               "stages_ms": {k: round(v, 4) for k, v in stages.items()},
+                               "rows": H_kv, "tokens_per_row": T_ctx,
+                               "note": "wall time of obkv_fast._perhead_select_and_pack_joint on layer 0 (median of "
+                                       "5 after 1 warm-up); stages from one extra call that synchronizes after "
+                                       "each stage (quantization_ms = the whole-layer packer)"}
+                if not args.no_cpu_baseline:
+                    from oracle import select_oracle
+                    t0 = time.perf_counter()
+                    select_oracle.select_joint(
+                        tok_scores.cpu().numpy(), ch_scores.cpu().numpy(), head_dim=128,
+                        token_budget=sel_kw["token_budget"], k_budget_ratio=0.5, pool_kernel_size=7,
+                        pool_padding="reflect", k_bit_options=(0, 2, 4, 8))
+                    select_info["cpu_oracle_allocation_ms"] = (time.perf_counter() - t0) * 1e3
+                    select_info["gpu_allocation_ms"] = float(sum(v for k, v in stages.items()
+                                                                 if k in ("pooling_ms", "v_allocation_ms",
+                                                                          "k_allocation_ms")))
+                del tok_scores, ch_scores
             del K, V
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
@@ -307,6 +345,7 @@ def main():
                            speedup_vs_ideal_dense=dense["ideal_ms_at_read_ceiling"] / ms_step,
                            speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None),
         "pack": pack_info,
+        "select": select_info,
         "check": check,
     }
     print(json.dumps(result))

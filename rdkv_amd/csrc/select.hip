@@ -63,7 +63,21 @@ __device__ float solve_avg(const float* __restrict__ row, int T, float lam, cons
 #pragma unroll
   for (int n = 0; n < kMaxOptions; ++n) lb[n] = n < o.n ? __fmul_rn(lam, o.bits[n]) : 0.f;
   int acc = 0;
-  for (int t = threadIdx.x; t < T; t += blockDim.x) {
+  // eight independent loads in flight per thread, then the remainder
+  const int step = blockDim.x;
+  int t = threadIdx.x;
+  for (; t + 7 * step < T; t += 8 * step) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = row[t + u * step];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      int width;
+      choose(v[u], o, lb, width);
+      acc += width;
+    }
+  }
+  for (; t < T; t += step) {
     int width;
     choose(row[t], o, lb, width);
     acc += width;
