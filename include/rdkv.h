@@ -252,6 +252,35 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
                                    float *out, int64_t out_stride_row, float *lse,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Planning for rdkv_pack_layer_per_head on the device (what the reference derives on the host:
+ * packing.py:1417-1431 stable token sort by width, :241-294 channel classes).  v_bits [H_kv, T]
+ * and k_bits [H_kv, D]: integers of 1, 2, 4 or 8 bytes, head strides in elements.  Writes
+ * order [H_kv, T] (token indices, stable by class 2 / 4 / 8 / 16 bit / evicted), rank3 [H_kv, T]
+ * (number of earlier tokens of the head that are quantized) and plan: int32 [H_kv * 12] =
+ * [H_kv][4] (n2, n4, n8, n16) followed by [H_kv][8] (evicted tokens, invalid token widths,
+ * channels at 2 / 4 / 8 bit (16 counts as 8), invalid channel widths, 0, 0).  The caller reads
+ * `plan` once to size the packed tensors. */
+int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t vb_stride_h, const void *k_bits,
+                         int kb_elem_size, int64_t kb_stride_h, int H_kv, int64_t T, int D,
+                         int32_t *order, int64_t order_stride_h, int32_t *rank3, int64_t rank3_stride_h,
+                         int32_t *plan, void *stream);
+
+/* Per-head tables and metadata of the stacked layer (packing.py:399-578 pack_k_mixed_per_head's
+ * index tensors, :1245-1316 of _pad_and_stack_per_head_layers), from `plan` and the layer-wide
+ * sizes the caller derived from it: slot_channel int32 [H_kv, Dp] (source channel per padded
+ * slot, -1 = padding; Dp = n2p + n4p + n8), perm int64 [H_kv, Dp] (padding -> 0), perm_for_q
+ * int64 [H_kv*G, Dp], sort_ch int64 [H_kv, kept_max] (kept channels by width, zero padded),
+ * seg_ch / seg_tok int32 [H_kv, 3], t_eff / t_eff_k / n_v16 int32 [H_kv], sort_idx int64
+ * [tv_ref] (rank among head ref_head's quantized tokens, in sorted order) and softmax_mask fp32
+ * [H_kv*G, max_tv + max_n16] (0 on token columns, -inf on padding).  D <= 1024. */
+int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int H_kv, int D,
+                           int G, const int32_t *plan, int n2p, int n4p, int n8, int kept_max,
+                           int64_t max_tv, int max_n16, const int32_t *order, int64_t order_stride_h,
+                           const int32_t *rank3, int64_t rank3_stride_h, int ref_head, int64_t tv_ref,
+                           int32_t *slot_channel, int64_t *perm, int64_t *perm_for_q, int64_t *sort_ch,
+                           int32_t *seg_ch, int32_t *seg_tok, int32_t *t_eff, int32_t *t_eff_k,
+                           int32_t *n_v16, int64_t *sort_idx, float *softmax_mask, void *stream);
+
 /* ---- prefill-time selection feeding the packer ---------------------------------------------
  * obkv_fast.py:208-249  apply_score_pooling, as used on the per-head token scores at
  * obkv_fast.py:961-967.  Stride-1 pooling of B rows of T fp32 scores (row stride in elements).

@@ -1,0 +1,271 @@
+// Device-side planning for the whole-layer packer: everything the reference derives on the host
+// from the per-head bit allocations (obkv_accel/packing.py:241-294 channel sort / prune / padding,
+// :1417-1431 stable token sort by width, :1245-1260 padding mask, :1262-1316 per-head metadata) is
+// computed here so that the host needs one small read (the per-head class sizes, which fix the
+// shapes of the packed tensors) and no per-head loop.
+#include "rdkv_common.h"
+
+namespace {
+
+constexpr int kPlanThreads = 1024;
+constexpr int kTokClasses = 6;      // 2, 4, 8, 16 bit, evicted (0), anything else
+
+__device__ __forceinline__ int load_int(const void *p, int elem_size, int64_t i) {
+  switch (elem_size) {
+    case 1: return reinterpret_cast<const uint8_t *>(p)[i];
+    case 2: return reinterpret_cast<const int16_t *>(p)[i];
+    case 4: return reinterpret_cast<const int32_t *>(p)[i];
+    default: {
+      const int64_t v = reinterpret_cast<const int64_t *>(p)[i];
+      return (v < -1 || v > 1 << 20) ? -1 : (int)v;
+    }
+  }
+}
+
+__device__ __forceinline__ int token_class(int bits) {
+  return bits == 2 ? 0 : bits == 4 ? 1 : bits == 8 ? 2 : bits == 16 ? 3 : bits == 0 ? 4 : 5;
+}
+
+// widths above 8 are stored as 8 bit; 0 = pruned (-1); anything else is invalid (-2)
+__device__ __forceinline__ int channel_class(int bits) {
+  return bits == 2 ? 0 : bits == 4 ? 1 : (bits == 8 || bits == 16) ? 2 : bits == 0 ? -1 : -2;
+}
+
+__device__ __forceinline__ int lanes_below(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+}
+
+// One workgroup per KV head.  order[h, :] = token indices sorted by class, stable (the classes
+// in the order 2, 4, 8, 16 bit, evicted); rank3[h, t] = number of tokens before t that are
+// quantized (2/4/8 bit); counts4[h] = (n2, n4, n8, n16); info[h] = (n_evicted, n_invalid,
+// channels at 2, 4, 8 bit, invalid channels, 0, 0).
+__global__ void __launch_bounds__(kPlanThreads)
+pack_plan_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_stride_h, int T,
+                 const void *__restrict__ k_bits, int kb_es, int64_t kb_stride_h, int D,
+                 int32_t *__restrict__ order, int64_t order_stride_h, int32_t *__restrict__ rank3,
+                 int64_t rank3_stride_h, int32_t *__restrict__ counts4, int32_t *__restrict__ info) {
+  __shared__ int wcnt[kPlanThreads / 64][kTokClasses];
+  __shared__ int wpre[kPlanThreads / 64][kTokClasses];
+  __shared__ int tot[kTokClasses];
+  __shared__ int kcnt[4];
+  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nwaves = blockDim.x >> 6;
+  const int64_t vrow = (int64_t)h * vb_stride_h;
+  int32_t *ord = order + (int64_t)h * order_stride_h;
+  int32_t *rk = rank3 + (int64_t)h * rank3_stride_h;
+
+  // pass 1: class sizes
+  int c[kTokClasses];
+#pragma unroll
+  for (int k = 0; k < kTokClasses; ++k) c[k] = 0;
+  for (int t = tid; t < T; t += blockDim.x) {
+    const int cls = token_class(load_int(v_bits, vb_es, vrow + t));
+#pragma unroll
+    for (int k = 0; k < kTokClasses; ++k) c[k] += (cls == k) ? 1 : 0;
+  }
+#pragma unroll
+  for (int k = 0; k < kTokClasses; ++k) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) c[k] += __shfl_xor(c[k], off, 64);
+    if (lane == 0) wcnt[wave][k] = c[k];
+  }
+  if (tid < 4) kcnt[tid] = 0;
+  __syncthreads();
+  if (tid < kTokClasses) {
+    int s = 0;
+    for (int w = 0; w < nwaves; ++w) s += wcnt[w][tid];
+    tot[tid] = s;
+  }
+  __syncthreads();
+  int seg_base[kTokClasses], running[kTokClasses];
+  {
+    int acc = 0;
+#pragma unroll
+    for (int k = 0; k < kTokClasses; ++k) { seg_base[k] = acc; acc += tot[k]; running[k] = 0; }
+  }
+  if (tid < 4) counts4[4 * h + tid] = tot[tid];
+  if (tid == 4) info[8 * h + 0] = tot[4];
+  if (tid == 5) info[8 * h + 1] = tot[5];
+  __syncthreads();                                   // tot is rewritten per chunk below
+
+  // pass 2: stable scatter, one chunk of blockDim tokens at a time
+  for (int base = 0; base < T; base += blockDim.x) {
+    const int t = base + tid;
+    const int cls = t < T ? token_class(load_int(v_bits, vb_es, vrow + t)) : -1;
+    int my_rank = 0, my_q = 0;                         // rank inside my class / among quantized, in this wave
+    uint64_t qmask = 0;
+#pragma unroll
+    for (int k = 0; k < kTokClasses; ++k) {
+      const uint64_t m = __ballot(cls == k);
+      if (k < 3) qmask |= m;
+      if (cls == k) my_rank = lanes_below(m);
+      if (lane == 0) wcnt[wave][k] = __popcll(m);
+    }
+    my_q = lanes_below(qmask);
+    __syncthreads();
+    if (tid < kTokClasses) {
+      int s = 0;
+      for (int w = 0; w < nwaves; ++w) { wpre[w][tid] = s; s += wcnt[w][tid]; }
+      tot[tid] = s;
+    }
+    __syncthreads();
+    int pos = 0, before_q = 0;
+#pragma unroll
+    for (int k = 0; k < kTokClasses; ++k) {
+      const int ahead = running[k] + wpre[wave][k];
+      if (cls == k) pos = seg_base[k] + ahead + my_rank;
+      if (k < 3) before_q += ahead;
+      running[k] += tot[k];
+    }
+    if (t < T) {
+      ord[pos] = t;
+      rk[t] = before_q + my_q;
+    }
+  }
+
+  // channel classes of this head
+  int bad = 0;
+  for (int ch = tid; ch < D; ch += blockDim.x) {
+    const int cls = channel_class(load_int(k_bits, kb_es, (int64_t)h * kb_stride_h + ch));
+    if (cls >= 0) atomicAdd(&kcnt[cls], 1);
+    if (cls == -2) bad = 1;
+  }
+  if (bad) atomicAdd(&kcnt[3], 1);
+  __syncthreads();
+  if (tid < 4) info[8 * h + 2 + tid] = kcnt[tid];
+  if (tid >= 4 && tid < 6) info[8 * h + 2 + tid] = 0;
+}
+
+// One workgroup per KV head: channel tables with the layer-wide padded segment sizes, per-head
+// scalars, and (in the block of head `ref`) the sort index of that head's quantized tokens.
+__global__ void __launch_bounds__(kPlanThreads)
+layer_tables_kernel(const void *__restrict__ k_bits, int kb_es, int64_t kb_stride_h, int D, int G,
+                    const int32_t *__restrict__ counts4, const int32_t *__restrict__ info,
+                    int n2p, int n4p, int n8o, int kept_max, int64_t max_tv,
+                    const int32_t *__restrict__ order, int64_t order_stride_h,
+                    const int32_t *__restrict__ rank3, int64_t rank3_stride_h, int ref, int64_t tv_ref,
+                    int32_t *__restrict__ slot_channel, int64_t *__restrict__ perm, int64_t *__restrict__ perm_q,
+                    int64_t *__restrict__ sort_ph, int32_t *__restrict__ seg_ph, int32_t *__restrict__ seg_tok,
+                    int32_t *__restrict__ t_eff, int32_t *__restrict__ t_eff_k, int32_t *__restrict__ n_v16,
+                    int64_t *__restrict__ sort_idx) {
+  __shared__ int wcnt[kPlanThreads / 64][3];
+  __shared__ int wpre[kPlanThreads / 64][3];
+  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+  const int Dp = n2p + n4p + n8o;
+  const int n2 = info[8 * h + 2], n4 = info[8 * h + 3];
+  for (int j = tid; j < Dp; j += blockDim.x) {
+    slot_channel[(int64_t)h * Dp + j] = -1;
+    perm[(int64_t)h * Dp + j] = 0;
+  }
+  for (int j = tid; j < kept_max; j += blockDim.x) sort_ph[(int64_t)h * kept_max + j] = 0;
+  if (tid < 3) {
+    seg_ph[3 * h + tid] = info[8 * h + 2 + tid];
+    seg_tok[3 * h + tid] = counts4[4 * h + tid];
+  }
+  if (tid == 0) {
+    const int tv = counts4[4 * h] + counts4[4 * h + 1] + counts4[4 * h + 2], n16 = counts4[4 * h + 3];
+    t_eff[h] = tv;
+    t_eff_k[h] = tv + n16;
+    n_v16[h] = n16;
+  }
+  const int ch = tid;                                   // D <= blockDim (checked by the host)
+  const int cls = ch < D ? channel_class(load_int(k_bits, kb_es, (int64_t)h * kb_stride_h + ch)) : -1;
+  int my_rank = 0;
+#pragma unroll
+  for (int k = 0; k < 3; ++k) {
+    const uint64_t m = __ballot(cls == k);
+    if (cls == k) my_rank = lanes_below(m);
+    if (lane == 0) wcnt[wave][k] = __popcll(m);
+  }
+  __syncthreads();
+  if (tid < 3) {
+    int s = 0;
+    for (int w = 0; w < nwaves; ++w) { wpre[w][tid] = s; s += wcnt[w][tid]; }
+  }
+  __syncthreads();                                      // also orders the fills above before the scatter
+  if (cls >= 0) {
+    const int r = wpre[wave][cls] + my_rank;
+    const int slot = (cls == 0 ? 0 : cls == 1 ? n2p : n2p + n4p) + r;
+    const int sorted = (cls == 0 ? 0 : cls == 1 ? n2 : n2 + n4) + r;
+    slot_channel[(int64_t)h * Dp + slot] = ch;
+    perm[(int64_t)h * Dp + slot] = ch;
+    sort_ph[(int64_t)h * kept_max + sorted] = ch;
+  }
+  __syncthreads();
+  for (int j = tid; j < G * Dp; j += blockDim.x)
+    perm_q[((int64_t)h * G + j / Dp) * Dp + j % Dp] = perm[(int64_t)h * Dp + j % Dp];
+  if (h == ref) {
+    const int32_t *ord = order + (int64_t)ref * order_stride_h;
+    const int32_t *rk = rank3 + (int64_t)ref * rank3_stride_h;
+    for (int64_t i = tid; i < tv_ref; i += blockDim.x) sort_idx[i] = rk[ord[i]];
+  }
+}
+
+// mask[hq, col] = 0 where the canvas column holds a token of head hq / G, -inf where it is padding
+__global__ void __launch_bounds__(256)
+softmax_mask_kernel(const int32_t *__restrict__ counts4, int G, int64_t max_tv, int64_t max_tk,
+                    float *__restrict__ mask) {
+  const int hq = blockIdx.y, h = hq / G;
+  const int64_t tv = (int64_t)counts4[4 * h] + counts4[4 * h + 1] + counts4[4 * h + 2], n16 = counts4[4 * h + 3];
+  for (int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; col < max_tk;
+       col += (int64_t)gridDim.x * blockDim.x) {
+    const bool valid = col < tv || (col >= max_tv && col < max_tv + n16);
+    mask[(int64_t)hq * max_tk + col] = valid ? 0.0f : -__builtin_inff();
+  }
+}
+
+bool elem_size_ok(int es) { return es == 1 || es == 2 || es == 4 || es == 8; }
+
+}  // namespace
+
+RDKV_API int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t vb_stride_h, const void *k_bits,
+                                  int kb_elem_size, int64_t kb_stride_h, int H_kv, int64_t T, int D,
+                                  int32_t *order, int64_t order_stride_h, int32_t *rank3,
+                                  int64_t rank3_stride_h, int32_t *plan, void *stream) {
+  const char *fn = "rdkv_pack_layer_plan";
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D >= 1 && T >= 0 && T <= 0x7fffffffLL, "%s: bad shape", fn);
+  RDKV_REQUIRE(elem_size_ok(vb_elem_size) && elem_size_ok(kb_elem_size), "%s: element sizes must be 1, 2, 4 or 8", fn);
+  RDKV_REQUIRE(k_bits && plan && (T == 0 || (v_bits && order && rank3)), "%s: null pointer", fn);
+  hipLaunchKernelGGL(pack_plan_kernel, dim3(H_kv), dim3(kPlanThreads), 0, (hipStream_t)stream, v_bits,
+                     vb_elem_size, vb_stride_h, (int)T, k_bits, kb_elem_size, kb_stride_h, D, order, order_stride_h,
+                     rank3, rank3_stride_h, plan, plan + 4 * (int64_t)H_kv);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int H_kv, int D,
+                                    int G, const int32_t *plan, int n2p, int n4p, int n8, int kept_max,
+                                    int64_t max_tv, int max_n16, const int32_t *order, int64_t order_stride_h,
+                                    const int32_t *rank3, int64_t rank3_stride_h, int ref_head, int64_t tv_ref,
+                                    int32_t *slot_channel, int64_t *perm, int64_t *perm_for_q, int64_t *sort_ch,
+                                    int32_t *seg_ch, int32_t *seg_tok, int32_t *t_eff, int32_t *t_eff_k,
+                                    int32_t *n_v16, int64_t *sort_idx, float *softmax_mask, void *stream) {
+  const char *fn = "rdkv_pack_layer_tables";
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D >= 1 && D <= kPlanThreads && G >= 1, "%s: bad shape", fn);
+  RDKV_REQUIRE(elem_size_ok(kb_elem_size), "%s: element size must be 1, 2, 4 or 8", fn);
+  RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0 && kept_max >= 0 &&
+                   kept_max <= n2p + n4p + n8, "%s: bad segment sizes", fn);
+  RDKV_REQUIRE(max_tv >= 0 && max_n16 >= 0 && ref_head >= 0 && ref_head < H_kv && tv_ref >= 0 && tv_ref <= max_tv,
+               "%s: bad token counts", fn);
+  const int Dp = n2p + n4p + n8;
+  RDKV_REQUIRE(k_bits && plan && seg_ch && seg_tok && t_eff && t_eff_k && n_v16, "%s: null pointer", fn);
+  RDKV_REQUIRE(Dp == 0 || (slot_channel && perm && perm_for_q), "%s: null channel table", fn);
+  RDKV_REQUIRE(kept_max == 0 || sort_ch, "%s: null channel sort table", fn);
+  RDKV_REQUIRE(tv_ref == 0 || (sort_idx && order && rank3), "%s: null token tables", fn);
+  hipStream_t s = (hipStream_t)stream;
+  const int threads = ((D + 63) / 64) * 64;
+  hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, k_bits, kb_elem_size, kb_stride_h, D, G,
+                     plan, plan + 4 * (int64_t)H_kv, n2p, n4p, n8, kept_max, max_tv, order, order_stride_h, rank3,
+                     rank3_stride_h, ref_head, tv_ref, slot_channel, perm, perm_for_q, sort_ch, seg_ch, seg_tok,
+                     t_eff, t_eff_k, n_v16, sort_idx);
+  const int64_t max_tk = max_tv + max_n16;
+  if (max_tk > 0) {
+    RDKV_REQUIRE(softmax_mask, "%s: null mask", fn);
+    int64_t bx = rdkv_cdiv(max_tk, 256 * 4);
+    if (bx > 1024) bx = 1024;
+    hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, plan, G,
+                       max_tv, max_tk, softmax_mask);
+  }
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}

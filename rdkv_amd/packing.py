@@ -614,27 +614,17 @@ def _pad_and_stack_per_head_layers(
     return packed, new_v_only
 
 
-_CLASS_TABLES = {}
-
-
-def _class_tables(dev):
-    """(v_bits -> class rank lookup, class rank list) on ``dev``, built once per device."""
-    t = _CLASS_TABLES.get(dev)
-    if t is None:
-        lut = torch.full((17,), 255, dtype=torch.uint8)
-        lut[torch.tensor([2, 4, 8, 16, 0])] = torch.arange(5, dtype=torch.uint8)
-        t = (lut.to(dev), torch.tensor([0, 1, 2, 3, 4, 255], dtype=torch.uint8).to(dev))
-        _CLASS_TABLES[dev] = t
-    return t
-
+_PLAN_INT_DTYPES = (torch.uint8, torch.int16, torch.int32, torch.int64)
 
 def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,
                         gqa_factor: int) -> Tuple[PackedKVLayer, Optional[Tensor]]:
     """Prefill packing of one layer with per-head allocations: the result of the reference's
     composition (obkv_fast.py:1141-1155: per head ``build_packed_layer`` with deferred K,
     packing.py:801-1013, then ``_pad_and_stack_per_head_layers``, packing.py:1019-1317),
-    bit for bit, without the per-head loop: one stable sort of the token classes, then
-    ``rdkv_pack_layer_per_head`` (V rows, K min/max, K emit).  K, V [1,H_kv,T,D] fp16;
+    bit for bit, without the per-head loop: ``rdkv_pack_layer_plan`` (stable token order by class
+    and all class sizes, read once by the host to size the tensors), ``rdkv_pack_layer_tables``
+    (channel tables, per-head metadata, padding mask) and ``rdkv_pack_layer_per_head`` (V rows, K
+    min/max, K emit).  K, V [1,H_kv,T,D] fp16;
     v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
     dev = _lib.require_device(K, V)
     assert K.dim() == 4 and K.shape[0] == 1 and K.shape == V.shape, (
@@ -646,42 +636,69 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     Kf, Vf = _as_f16_heads(K)[0], _as_f16_heads(V)[0]
     if Vf.stride() != Kf.stride():
         Kf, Vf = Kf.contiguous(), Vf.contiguous()
-    # class rank of every token: 2-bit 0, 4-bit 1, 8-bit 2, fp16 3, evicted 4 (255 = invalid)
-    lut, classes = _class_tables(dev)
-    vb = v_bits_per_head.to(dev)
-    key = lut[torch.where((vb >= 0) & (vb <= 16), vb, 1).long()]
-    order = torch.sort(key, dim=1, stable=True).indices.to(torch.int32)
-    counts = (key.unsqueeze(-1) == classes).sum(1)              # [H_kv, 6] on the device
-    counts_h = counts.cpu().tolist()                            # the one synchronization
-    assert all(row[5] == 0 for row in counts_h), "v_bits must be in {0,2,4,8,16}"
-    seg = [tuple(int(v) for v in row[:3]) for row in counts_h]
-    n16 = [int(row[3]) for row in counts_h]
+    lib = _lib.load()
+    stream = _lib.stream_of(dev)
+    vb = v_bits_per_head if v_bits_per_head.device == dev else v_bits_per_head.to(dev)
+    kb = k_bits_per_head if k_bits_per_head.device == dev else k_bits_per_head.to(dev)
+    if vb.dtype not in _PLAN_INT_DTYPES:
+        vb = vb.long()
+    if kb.dtype not in _PLAN_INT_DTYPES:
+        kb = kb.long()
+    if vb.stride(1) != 1:
+        vb = vb.contiguous()
+    if kb.stride(1) != 1:
+        kb = kb.contiguous()
+    # token order (stable by class), quantized-token ranks and all class sizes in one launch
+    order = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
+    rank3 = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
+    plan = torch.empty(H_kv * 12, dtype=torch.int32, device=dev)
+    _lib.check(lib.rdkv_pack_layer_plan(vb.data_ptr(), vb.element_size(), vb.stride(0), kb.data_ptr(),
+                                        kb.element_size(), kb.stride(0), H_kv, T, D, order.data_ptr(),
+                                        order.stride(0), rank3.data_ptr(), rank3.stride(0), plan.data_ptr(), stream))
+    plan_h = plan.cpu().tolist()                                # the one synchronization
+    counts_h = [plan_h[4 * h:4 * h + 4] for h in range(H_kv)]
+    info_h = [plan_h[4 * H_kv + 8 * h:4 * H_kv + 8 * h + 8] for h in range(H_kv)]
+    assert all(row[1] == 0 for row in info_h), "v_bits must be in {0,2,4,8,16}"
+    assert all(row[5] == 0 for row in info_h), "k_bits must be in {0,2,4,8,16}"
+    seg = [tuple(row[:3]) for row in counts_h]
+    n16 = [row[3] for row in counts_h]
     tv = [sum(s3) for s3 in seg]
     tk = [a + b for a, b in zip(tv, n16)]
     max_tv, max_n16 = max(tv), max(n16)
     max_tk = max_tv + max_n16
     mN = [max(s3[i] for s3 in seg) for i in range(3)]
-    rows = k_bits_per_head.detach().cpu().tolist()
-    n_h, (m2, m4, m8) = _per_head_counts(rows)
+    m2, m4, m8 = (max(row[2 + i] for row in info_h) for i in range(3))
+    kept_max = max(sum(row[2:5]) for row in info_h)
     sub2 = _seg_padded_len(m2, 4) // 4
     sub4 = _seg_padded_len(m4, 2) // 2
     Dp = 4 * sub2 + 2 * sub4 + m8
-    if max_tk == 0 or Dp == 0:
+    if max_tk == 0 or Dp == 0 or D > 1024:
         return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
-    plans = [_plan_k_channels(rows[h], sub2 or None, sub4 or None, m8 or None, tuple(n_h[h]))
-             for h in range(H_kv)]
-    # all host-built index tables travel in one copy: [slot_channel | perm | sort | seg] per head
-    kept_max = max((len(p.ch_sort_idx) for p in plans), default=0)
-    table = torch.tensor([p.slot_channel + p.perm_padded + p.ch_sort_idx + [0] * (kept_max - len(p.ch_sort_idx))
-                          + list(n_h[h]) for h, p in enumerate(plans)], dtype=torch.long).to(dev)
-    slot_ch = table[:, :Dp].to(torch.int32).contiguous()
-    perm_ph = table[:, Dp:2 * Dp].contiguous()
-    sort_ph = table[:, 2 * Dp:2 * Dp + kept_max].contiguous()
-    seg_ph = table[:, 2 * Dp + kept_max:].to(torch.int32).contiguous()
-    counts_dev = counts[:, :4].to(torch.int32).contiguous()
+    ref = next((h for h in range(H_kv) if tk[h] > 0), 0)
+    H_q = H_kv * gqa_factor
 
     def u8(n, w):
         return torch.empty(1, H_kv, n, w, dtype=torch.uint8, device=dev) if n > 0 and w > 0 else None
+
+    i32 = dict(dtype=torch.int32, device=dev)
+    i64 = dict(dtype=torch.int64, device=dev)
+    slot_ch = torch.empty(H_kv, Dp, **i32)
+    perm_ph = torch.empty(H_kv, Dp, **i64)
+    perm_q = torch.empty(H_q, Dp, **i64)
+    sort_ph = torch.empty(H_kv, kept_max, **i64)
+    seg_ph = torch.empty(H_kv, 3, **i32)
+    seg_tok = torch.empty(H_kv, 3, **i32)
+    t_eff_ph = torch.empty(H_kv, **i32)
+    t_eff_k_ph = torch.empty(H_kv, **i32)
+    n_v16_ph = torch.empty(H_kv, **i32)
+    sort_idx = torch.empty(tv[ref], **i64)
+    softmax_mask = torch.empty(H_q, max_tk, dtype=torch.float32, device=dev)
+    _lib.check(lib.rdkv_pack_layer_tables(
+        kb.data_ptr(), kb.element_size(), kb.stride(0), H_kv, D, gqa_factor, plan.data_ptr(), 4 * sub2, 2 * sub4,
+        m8, kept_max, max_tv, max_n16, order.data_ptr(), order.stride(0), rank3.data_ptr(), rank3.stride(0), ref,
+        tv[ref], slot_ch.data_ptr(), perm_ph.data_ptr(), perm_q.data_ptr(), _lib.ptr(sort_ph), seg_ph.data_ptr(),
+        seg_tok.data_ptr(), t_eff_ph.data_ptr(), t_eff_k_ph.data_ptr(), n_v16_ph.data_ptr(), _lib.ptr(sort_idx),
+        softmax_mask.data_ptr(), stream))
 
     V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
     V_scale = torch.zeros(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)
@@ -691,41 +708,25 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     ks = torch.empty(1, H_kv, 1, Dp, dtype=torch.float16, device=dev)
     kz = torch.empty_like(ks)
     mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
-    _lib.check(_lib.load().rdkv_pack_layer_per_head(
+    _lib.check(lib.rdkv_pack_layer_per_head(
         Kf.data_ptr(), Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D,
-        order.data_ptr(), order.stride(0), counts_dev.data_ptr(), mN[0], mN[1], mN[2], max_tv, max_n16,
+        order.data_ptr(), order.stride(0), plan.data_ptr(), mN[0], mN[1], mN[2], max_tv, max_n16,
         slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8,
         _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only),
-        _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(),
-        _lib.stream_of(dev)))
+        _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), stream))
 
     # metadata exactly as _pad_and_stack_per_head_layers / pack_k_mixed_per_head produce it
-    ref = next((h for h in range(H_kv) if tk[h] > 0), 0)
-    if tv[ref] > 0:      # pack_v_segments' argsort indexes the head's compressed tokens
-        rank = torch.cumsum((key[ref] < 3).to(torch.long), 0) - 1
-        sort_idx = rank[order[ref, :tv[ref]].long()]
-    else:
-        sort_idx = torch.empty(0, dtype=torch.long, device=dev)
-    tv_t = counts_dev[:, :3].sum(1, keepdim=True)
-    n16_t = counts_dev[:, 3:4]
-    col = torch.arange(max_tk, device=dev).unsqueeze(0)
-    valid = (col < tv_t) | ((col >= max_tv) & (col < max_tv + n16_t))
-    mask_kv = torch.zeros(H_kv, max_tk, dtype=torch.float32, device=dev)
-    mask_kv.masked_fill_(~valid, float("-inf"))
     packed = PackedKVLayer(
         K_2bit=K2, K_4bit=K4, K_8bit=K8, K_ch_scale=ks, K_ch_zp=kz, K_ch_sort_idx=sort_ph[0],
         K_ch_seg_bounds=(m2, m4, m8), K_ch_perm_padded_idx=perm_ph[0],
         V_2bit=V2, V_4bit=V4, V_8bit=V8, V_scale=V_scale, V_zp=V_zp,
         sort_idx=sort_idx, seg_bounds=(mN[0], mN[1], mN[2]), T_eff=max_tv,
-        seg_bounds_per_head=counts_dev[:, :3].contiguous(),
-        T_eff_per_head=tv_t.reshape(H_kv).to(torch.int32),
-        softmax_mask=mask_kv.repeat_interleave(gqa_factor, dim=0).contiguous(),
+        seg_bounds_per_head=seg_tok, T_eff_per_head=t_eff_ph, softmax_mask=softmax_mask,
         n_fp16_per_head=None, fp16_gap_mask=None,
         K_ch_sort_idx_per_head=sort_ph, K_ch_perm_padded_idx_per_head=perm_ph,
-        K_ch_seg_bounds_per_head=seg_ph,
-        K_ch_perm_padded_idx_for_Q=perm_ph.repeat_interleave(gqa_factor, dim=0),
-        T_eff_k=max_tk, n_v16=max_n16, T_eff_k_per_head=counts_dev.sum(1).to(torch.int32),
-        n_v16_per_head=counts_dev[:, 3].contiguous(), allocation_v_bits=None, allocation_k_bits=None)
+        K_ch_seg_bounds_per_head=seg_ph, K_ch_perm_padded_idx_for_Q=perm_q,
+        T_eff_k=max_tk, n_v16=max_n16, T_eff_k_per_head=t_eff_k_ph,
+        n_v16_per_head=n_v16_ph, allocation_v_bits=None, allocation_k_bits=None)
     return packed, new_v_only
 
 
