@@ -256,10 +256,12 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
  * packing.py:1417-1431 stable token sort by width, :241-294 channel classes).  v_bits [H_kv, T]
  * and k_bits [H_kv, D]: integers of 1, 2, 4 or 8 bytes, head strides in elements.  Writes
  * order [H_kv, T] (token indices, stable by class 2 / 4 / 8 / 16 bit / evicted), rank3 [H_kv, T]
- * (number of earlier tokens of the head that are quantized) and plan: int32 [H_kv * 12] =
- * [H_kv][4] (n2, n4, n8, n16) followed by [H_kv][8] (evicted tokens, invalid token widths,
- * channels at 2 / 4 / 8 bit (16 counts as 8), invalid channel widths, 0, 0).  The caller reads
- * `plan` once to size the packed tensors. */
+ * (number of earlier tokens of the head that are quantized) and plan: int32
+ * [rdkv_pack_layer_plan_ints(H_kv, T)], whose first H_kv * 12 values are [H_kv][4] (n2, n4, n8,
+ * n16) followed by [H_kv][8] (evicted tokens, invalid token widths, channels at 2 / 4 / 8 bit
+ * (16 counts as 8), invalid channel widths, 0, 0); the rest is scratch.  The caller reads those
+ * H_kv * 12 values once to size the packed tensors.  T >= 1. */
+int64_t rdkv_pack_layer_plan_ints(int H_kv, int64_t T);
 int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t vb_stride_h, const void *k_bits,
                          int kb_elem_size, int64_t kb_stride_h, int H_kv, int64_t T, int D,
                          int32_t *order, int64_t order_stride_h, int32_t *rank3, int64_t rank3_stride_h,

@@ -57,6 +57,7 @@ SIGNATURES = {
     "rdkv_decode_fused_merge_zone_c": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, I, P, P, L, P, P, L, P]),
     "rdkv_rope": (I, [P, L, I, P, L, I, I, I, P, P, I, P]),
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
+    "rdkv_pack_layer_plan_ints": (L, [I, L]),
     "rdkv_pack_layer_plan": (I, [P, I, L, P, I, L, I, L, I, P, L, P, L, P, P]),
     "rdkv_pack_layer_tables": (I, [P, I, L, I, I, I, P, I, I, I, I, L, I, P, L, P, L, I, L,
                                    P, P, P, P, P, P, P, P, P, P, P, P]),

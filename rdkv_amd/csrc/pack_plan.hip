@@ -35,119 +35,128 @@ __device__ __forceinline__ int lanes_below(uint64_t mask) {
   return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
 }
 
-// One workgroup per KV head.  order[h, :] = token indices sorted by class, stable (the classes
-// in the order 2, 4, 8, 16 bit, evicted); rank3[h, t] = number of tokens before t that are
-// quantized (2/4/8 bit); counts4[h] = (n2, n4, n8, n16); info[h] = (n_evicted, n_invalid,
-// channels at 2, 4, 8 bit, invalid channels, 0, 0).
+// Token planning in two launches over a (chunk, head) grid, kPlanThreads tokens per chunk.
+// First launch: per-chunk class histogram hist[h][chunk][6]; the chunk-0 block of each head also
+// counts the head's channel classes.
 __global__ void __launch_bounds__(kPlanThreads)
-pack_plan_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_stride_h, int T,
+plan_hist_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_stride_h, int T,
                  const void *__restrict__ k_bits, int kb_es, int64_t kb_stride_h, int D,
-                 int32_t *__restrict__ order, int64_t order_stride_h, int32_t *__restrict__ rank3,
-                 int64_t rank3_stride_h, int32_t *__restrict__ counts4, int32_t *__restrict__ info) {
-  __shared__ int wcnt[kPlanThreads / 64][kTokClasses];
-  __shared__ int wpre[kPlanThreads / 64][kTokClasses];
-  __shared__ int tot[kTokClasses];
+                 int32_t *__restrict__ hist, int32_t *__restrict__ info) {
+  __shared__ int cnt[kTokClasses];
   __shared__ int kcnt[4];
-  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int nwaves = blockDim.x >> 6;
-  const int64_t vrow = (int64_t)h * vb_stride_h;
-  int32_t *ord = order + (int64_t)h * order_stride_h;
-  int32_t *rk = rank3 + (int64_t)h * rank3_stride_h;
-
-  // pass 1: class sizes
-  int c[kTokClasses];
-#pragma unroll
-  for (int k = 0; k < kTokClasses; ++k) c[k] = 0;
-  for (int t = tid; t < T; t += blockDim.x) {
-    const int cls = token_class(load_int(v_bits, vb_es, vrow + t));
-#pragma unroll
-    for (int k = 0; k < kTokClasses; ++k) c[k] += (cls == k) ? 1 : 0;
-  }
-#pragma unroll
-  for (int k = 0; k < kTokClasses; ++k) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) c[k] += __shfl_xor(c[k], off, 64);
-    if (lane == 0) wcnt[wave][k] = c[k];
-  }
+  const int h = blockIdx.y, chunk = blockIdx.x, nchunks = gridDim.x, tid = threadIdx.x, lane = tid & 63;
+  if (tid < kTokClasses) cnt[tid] = 0;
   if (tid < 4) kcnt[tid] = 0;
   __syncthreads();
-  if (tid < kTokClasses) {
-    int s = 0;
-    for (int w = 0; w < nwaves; ++w) s += wcnt[w][tid];
-    tot[tid] = s;
+  const int t = chunk * kPlanThreads + tid;
+  const int cls = t < T ? token_class(load_int(v_bits, vb_es, (int64_t)h * vb_stride_h + t)) : -1;
+#pragma unroll
+  for (int k = 0; k < kTokClasses; ++k) {
+    const uint64_t m = __ballot(cls == k);
+    if (lane == 0 && m) atomicAdd(&cnt[k], __popcll(m));
+  }
+  if (chunk == 0) {
+    int bad = 0;
+    for (int ch = tid; ch < D; ch += blockDim.x) {
+      const int kc = channel_class(load_int(k_bits, kb_es, (int64_t)h * kb_stride_h + ch));
+      if (kc >= 0) atomicAdd(&kcnt[kc], 1);
+      if (kc == -2) bad = 1;
+    }
+    if (bad) atomicAdd(&kcnt[3], 1);
   }
   __syncthreads();
-  int seg_base[kTokClasses], running[kTokClasses];
-  {
-    int acc = 0;
-#pragma unroll
-    for (int k = 0; k < kTokClasses; ++k) { seg_base[k] = acc; acc += tot[k]; running[k] = 0; }
+  if (tid < kTokClasses) hist[((int64_t)h * nchunks + chunk) * kTokClasses + tid] = cnt[tid];
+  if (chunk == 0) {
+    if (tid < 4) info[8 * h + 2 + tid] = kcnt[tid];
+    if (tid >= 4 && tid < 6) info[8 * h + 2 + tid] = 0;
   }
-  if (tid < 4) counts4[4 * h + tid] = tot[tid];
-  if (tid == 4) info[8 * h + 0] = tot[4];
-  if (tid == 5) info[8 * h + 1] = tot[5];
-  __syncthreads();                                   // tot is rewritten per chunk below
-
-  // pass 2: stable scatter, one chunk of blockDim tokens at a time
-  for (int base = 0; base < T; base += blockDim.x) {
-    const int t = base + tid;
-    const int cls = t < T ? token_class(load_int(v_bits, vb_es, vrow + t)) : -1;
-    int my_rank = 0, my_q = 0;                         // rank inside my class / among quantized, in this wave
-    uint64_t qmask = 0;
-#pragma unroll
-    for (int k = 0; k < kTokClasses; ++k) {
-      const uint64_t m = __ballot(cls == k);
-      if (k < 3) qmask |= m;
-      if (cls == k) my_rank = lanes_below(m);
-      if (lane == 0) wcnt[wave][k] = __popcll(m);
-    }
-    my_q = lanes_below(qmask);
-    __syncthreads();
-    if (tid < kTokClasses) {
-      int s = 0;
-      for (int w = 0; w < nwaves; ++w) { wpre[w][tid] = s; s += wcnt[w][tid]; }
-      tot[tid] = s;
-    }
-    __syncthreads();
-    int pos = 0, before_q = 0;
-#pragma unroll
-    for (int k = 0; k < kTokClasses; ++k) {
-      const int ahead = running[k] + wpre[wave][k];
-      if (cls == k) pos = seg_base[k] + ahead + my_rank;
-      if (k < 3) before_q += ahead;
-      running[k] += tot[k];
-    }
-    if (t < T) {
-      ord[pos] = t;
-      rk[t] = before_q + my_q;
-    }
-  }
-
-  // channel classes of this head
-  int bad = 0;
-  for (int ch = tid; ch < D; ch += blockDim.x) {
-    const int cls = channel_class(load_int(k_bits, kb_es, (int64_t)h * kb_stride_h + ch));
-    if (cls >= 0) atomicAdd(&kcnt[cls], 1);
-    if (cls == -2) bad = 1;
-  }
-  if (bad) atomicAdd(&kcnt[3], 1);
-  __syncthreads();
-  if (tid < 4) info[8 * h + 2 + tid] = kcnt[tid];
-  if (tid >= 4 && tid < 6) info[8 * h + 2 + tid] = 0;
 }
 
-// One workgroup per KV head: channel tables with the layer-wide padded segment sizes, per-head
-// scalars, and (in the block of head `ref`) the sort index of that head's quantized tokens.
+// Second launch: every block sums the histograms of its head (class totals and what lies before
+// its chunk) and scatters its tokens.  order[h, :] = token indices sorted by class, stable (the
+// classes in the order 2, 4, 8, 16 bit, evicted, invalid); rank3[h, t] = number of tokens before
+// t that are quantized (2/4/8 bit); counts4[h] = (n2, n4, n8, n16); info[h][0..1] = (evicted,
+// invalid widths).
+__global__ void __launch_bounds__(kPlanThreads)
+plan_scatter_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_stride_h, int T,
+                    const int32_t *__restrict__ hist, int32_t *__restrict__ order, int64_t order_stride_h,
+                    int32_t *__restrict__ rank3, int64_t rank3_stride_h, int32_t *__restrict__ counts4,
+                    int32_t *__restrict__ info) {
+  __shared__ int wsum[kPlanThreads / 64][2 * kTokClasses];
+  __shared__ int red[2 * kTokClasses];
+  __shared__ int wcnt[kPlanThreads / 64][kTokClasses];
+  __shared__ int wpre[kPlanThreads / 64][kTokClasses];
+  const int h = blockIdx.y, chunk = blockIdx.x, nchunks = gridDim.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+  // totals over all chunks and over the chunks before this one
+  int acc[2 * kTokClasses];
+#pragma unroll
+  for (int k = 0; k < 2 * kTokClasses; ++k) acc[k] = 0;
+  for (int c = tid; c < nchunks; c += blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < kTokClasses; ++k) {
+      const int v = hist[((int64_t)h * nchunks + c) * kTokClasses + k];
+      acc[k] += v;
+      acc[kTokClasses + k] += c < chunk ? v : 0;
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < 2 * kTokClasses; ++k) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) acc[k] += __shfl_xor(acc[k], off, 64);
+    if (lane == 0) wsum[wave][k] = acc[k];
+  }
+  const int t = chunk * kPlanThreads + tid;
+  const int cls = t < T ? token_class(load_int(v_bits, vb_es, (int64_t)h * vb_stride_h + t)) : -1;
+  int my_rank = 0;
+  uint64_t qmask = 0;
+#pragma unroll
+  for (int k = 0; k < kTokClasses; ++k) {
+    const uint64_t m = __ballot(cls == k);
+    if (k < 3) qmask |= m;
+    if (cls == k) my_rank = lanes_below(m);
+    if (lane == 0) wcnt[wave][k] = __popcll(m);
+  }
+  const int my_q = lanes_below(qmask);
+  __syncthreads();
+  if (tid < 2 * kTokClasses) {
+    int s = 0;
+    for (int w = 0; w < nwaves; ++w) s += wsum[w][tid];
+    red[tid] = s;
+  } else if (tid >= 64 && tid < 64 + kTokClasses) {
+    const int k = tid - 64;
+    int s = 0;
+    for (int w = 0; w < nwaves; ++w) { wpre[w][k] = s; s += wcnt[w][k]; }
+  }
+  __syncthreads();
+  int pos = 0, before_q = 0, seg_base = 0;
+#pragma unroll
+  for (int k = 0; k < kTokClasses; ++k) {
+    const int ahead = red[kTokClasses + k] + wpre[wave][k];
+    if (cls == k) pos = seg_base + ahead + my_rank;
+    if (k < 3) before_q += ahead;
+    seg_base += red[k];
+  }
+  if (t < T) {
+    order[(int64_t)h * order_stride_h + pos] = t;
+    rank3[(int64_t)h * rank3_stride_h + t] = before_q + my_q;
+  }
+  if (chunk == 0) {
+    if (tid < 4) counts4[4 * h + tid] = red[tid];
+    if (tid == 4) info[8 * h + 0] = red[4];
+    if (tid == 5) info[8 * h + 1] = red[5];
+  }
+}
+
+// One workgroup per KV head: channel tables with the layer-wide padded segment sizes and the
+// per-head scalars.
 __global__ void __launch_bounds__(kPlanThreads)
 layer_tables_kernel(const void *__restrict__ k_bits, int kb_es, int64_t kb_stride_h, int D, int G,
                     const int32_t *__restrict__ counts4, const int32_t *__restrict__ info,
                     int n2p, int n4p, int n8o, int kept_max, int64_t max_tv,
-                    const int32_t *__restrict__ order, int64_t order_stride_h,
-                    const int32_t *__restrict__ rank3, int64_t rank3_stride_h, int ref, int64_t tv_ref,
                     int32_t *__restrict__ slot_channel, int64_t *__restrict__ perm, int64_t *__restrict__ perm_q,
                     int64_t *__restrict__ sort_ph, int32_t *__restrict__ seg_ph, int32_t *__restrict__ seg_tok,
-                    int32_t *__restrict__ t_eff, int32_t *__restrict__ t_eff_k, int32_t *__restrict__ n_v16,
-                    int64_t *__restrict__ sort_idx) {
+                    int32_t *__restrict__ t_eff, int32_t *__restrict__ t_eff_k, int32_t *__restrict__ n_v16) {
   __shared__ int wcnt[kPlanThreads / 64][3];
   __shared__ int wpre[kPlanThreads / 64][3];
   const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
@@ -194,18 +203,20 @@ layer_tables_kernel(const void *__restrict__ k_bits, int kb_es, int64_t kb_strid
   __syncthreads();
   for (int j = tid; j < G * Dp; j += blockDim.x)
     perm_q[((int64_t)h * G + j / Dp) * Dp + j % Dp] = perm[(int64_t)h * Dp + j % Dp];
-  if (h == ref) {
-    const int32_t *ord = order + (int64_t)ref * order_stride_h;
-    const int32_t *rk = rank3 + (int64_t)ref * rank3_stride_h;
-    for (int64_t i = tid; i < tv_ref; i += blockDim.x) sort_idx[i] = rk[ord[i]];
-  }
 }
 
-// mask[hq, col] = 0 where the canvas column holds a token of head hq / G, -inf where it is padding
+// mask[hq, col] = 0 where the canvas column holds a token of head hq / G, -inf where it is padding;
+// the first row of blocks also writes the sort index of head `ref`'s quantized tokens
+// (sort_idx[i] = rank among them of the i-th token in sorted order).
 __global__ void __launch_bounds__(256)
 softmax_mask_kernel(const int32_t *__restrict__ counts4, int G, int64_t max_tv, int64_t max_tk,
-                    float *__restrict__ mask) {
+                    float *__restrict__ mask, const int32_t *__restrict__ ord_ref,
+                    const int32_t *__restrict__ rank_ref, int64_t tv_ref, int64_t *__restrict__ sort_idx) {
   const int hq = blockIdx.y, h = hq / G;
+  if (hq == 0) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < tv_ref; i += (int64_t)gridDim.x * blockDim.x)
+      sort_idx[i] = rank_ref[ord_ref[i]];
+  }
   const int64_t tv = (int64_t)counts4[4 * h] + counts4[4 * h + 1] + counts4[4 * h + 2], n16 = counts4[4 * h + 3];
   for (int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; col < max_tk;
        col += (int64_t)gridDim.x * blockDim.x) {
@@ -218,17 +229,27 @@ bool elem_size_ok(int es) { return es == 1 || es == 2 || es == 4 || es == 8; }
 
 }  // namespace
 
+RDKV_API int64_t rdkv_pack_layer_plan_ints(int H_kv, int64_t T) {
+  if (H_kv < 0 || T < 0) return 0;
+  return (int64_t)H_kv * (12 + kTokClasses * rdkv_cdiv(T, kPlanThreads));
+}
+
 RDKV_API int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t vb_stride_h, const void *k_bits,
                                   int kb_elem_size, int64_t kb_stride_h, int H_kv, int64_t T, int D,
                                   int32_t *order, int64_t order_stride_h, int32_t *rank3,
                                   int64_t rank3_stride_h, int32_t *plan, void *stream) {
   const char *fn = "rdkv_pack_layer_plan";
-  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D >= 1 && T >= 0 && T <= 0x7fffffffLL, "%s: bad shape", fn);
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D >= 1 && T >= 1 && T <= (1LL << 30), "%s: bad shape", fn);
   RDKV_REQUIRE(elem_size_ok(vb_elem_size) && elem_size_ok(kb_elem_size), "%s: element sizes must be 1, 2, 4 or 8", fn);
-  RDKV_REQUIRE(k_bits && plan && (T == 0 || (v_bits && order && rank3)), "%s: null pointer", fn);
-  hipLaunchKernelGGL(pack_plan_kernel, dim3(H_kv), dim3(kPlanThreads), 0, (hipStream_t)stream, v_bits,
-                     vb_elem_size, vb_stride_h, (int)T, k_bits, kb_elem_size, kb_stride_h, D, order, order_stride_h,
-                     rank3, rank3_stride_h, plan, plan + 4 * (int64_t)H_kv);
+  RDKV_REQUIRE(k_bits && plan && v_bits && order && rank3, "%s: null pointer", fn);
+  const int64_t nchunks = rdkv_cdiv(T, kPlanThreads);
+  int32_t *counts4 = plan, *info = plan + 4 * (int64_t)H_kv, *hist = plan + 12 * (int64_t)H_kv;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(plan_hist_kernel, dim3((unsigned)nchunks, H_kv), dim3(kPlanThreads), 0, s, v_bits, vb_elem_size,
+                     vb_stride_h, (int)T, k_bits, kb_elem_size, kb_stride_h, D, hist, info);
+  hipLaunchKernelGGL(plan_scatter_kernel, dim3((unsigned)nchunks, H_kv), dim3(kPlanThreads), 0, s, v_bits,
+                     vb_elem_size, vb_stride_h, (int)T, hist, order, order_stride_h, rank3, rank3_stride_h, counts4,
+                     info);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }
@@ -255,16 +276,16 @@ RDKV_API int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_
   hipStream_t s = (hipStream_t)stream;
   const int threads = ((D + 63) / 64) * 64;
   hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, k_bits, kb_elem_size, kb_stride_h, D, G,
-                     plan, plan + 4 * (int64_t)H_kv, n2p, n4p, n8, kept_max, max_tv, order, order_stride_h, rank3,
-                     rank3_stride_h, ref_head, tv_ref, slot_channel, perm, perm_for_q, sort_ch, seg_ch, seg_tok,
-                     t_eff, t_eff_k, n_v16, sort_idx);
+                     plan, plan + 4 * (int64_t)H_kv, n2p, n4p, n8, kept_max, max_tv, slot_channel, perm, perm_for_q,
+                     sort_ch, seg_ch, seg_tok, t_eff, t_eff_k, n_v16);
   const int64_t max_tk = max_tv + max_n16;
   if (max_tk > 0) {
     RDKV_REQUIRE(softmax_mask, "%s: null mask", fn);
     int64_t bx = rdkv_cdiv(max_tk, 256 * 4);
     if (bx > 1024) bx = 1024;
     hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, plan, G,
-                       max_tv, max_tk, softmax_mask);
+                       max_tv, max_tk, softmax_mask, order ? order + (int64_t)ref_head * order_stride_h : nullptr,
+                       rank3 ? rank3 + (int64_t)ref_head * rank3_stride_h : nullptr, tv_ref, sort_idx);
   }
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;

@@ -651,11 +651,11 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     # token order (stable by class), quantized-token ranks and all class sizes in one launch
     order = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
     rank3 = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
-    plan = torch.empty(H_kv * 12, dtype=torch.int32, device=dev)
+    plan = torch.empty(lib.rdkv_pack_layer_plan_ints(H_kv, T), dtype=torch.int32, device=dev)
     _lib.check(lib.rdkv_pack_layer_plan(vb.data_ptr(), vb.element_size(), vb.stride(0), kb.data_ptr(),
                                         kb.element_size(), kb.stride(0), H_kv, T, D, order.data_ptr(),
                                         order.stride(0), rank3.data_ptr(), rank3.stride(0), plan.data_ptr(), stream))
-    plan_h = plan.cpu().tolist()                                # the one synchronization
+    plan_h = plan[:12 * H_kv].cpu().tolist()                    # the one synchronization
     counts_h = [plan_h[4 * h:4 * h + 4] for h in range(H_kv)]
     info_h = [plan_h[4 * H_kv + 8 * h:4 * H_kv + 8 * h + 8] for h in range(H_kv)]
     assert all(row[1] == 0 for row in info_h), "v_bits must be in {0,2,4,8,16}"
