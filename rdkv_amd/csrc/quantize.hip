@@ -95,7 +95,7 @@ __device__ __forceinline__ void quantize_values_d128(float x0, float x1, int lan
   }
 }
 
-#define RDKV_PACK_V_ROWS_PER_WAVE 8
+#define RDKV_PACK_V_ROWS_PER_WAVE 16
 __global__ void __launch_bounds__(256)
 pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stride_t, int D,
                     const int32_t *__restrict__ order, int64_t order_stride_h,
@@ -123,40 +123,84 @@ pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stri
     else { cls = 3; j = i - mN2 - mN4 - mN8; r = n2 + n4 + n8 + j; valid = j < n16; }
   };
   if (d128) {
-    // all row loads of the wavefront go out before the first is used
-    __half xa[RDKV_PACK_V_ROWS_PER_WAVE], xb[RDKV_PACK_V_ROWS_PER_WAVE];
+    // Sixteen lanes per row, four rows per wavefront step.  Lane l of a row holds channels
+    // 32p+2l and 32p+2l+1 of the four quarters p, so every packed byte of every width is
+    // lane-local: a 2-bit byte takes one code of each quarter, a 4-bit byte quarters (0,2) or
+    // (1,3).  All loads of the wavefront go out before the first is used.
+    constexpr int kSteps = RDKV_PACK_V_ROWS_PER_WAVE / 4;
+    const int sub = lane >> 4, l = lane & 15;
+    uint32_t raw[kSteps][4];
+    int cls[kSteps];
+    int64_t j[kSteps], r[kSteps];
+    bool valid[kSteps], inside[kSteps];
 #pragma unroll
-    for (int k = 0; k < RDKV_PACK_V_ROWS_PER_WAVE; ++k) {
-      int cls; int64_t j, r; bool valid;
-      xa[k] = xb[k] = __float2half_rn(0.0f);
-      if (i0 + k < total) {
-        locate(i0 + k, cls, j, r, valid);
-        if (valid) {
-          const __half *xr = Vh + (int64_t)ord[r] * stride_t;
-          xa[k] = xr[lane];
-          xb[k] = xr[lane + 64];
+    for (int s = 0; s < kSteps; ++s) {
+      const int64_t i = i0 + 4 * s + sub;
+      inside[s] = i < total;
+      cls[s] = 0; j[s] = 0; r[s] = 0; valid[s] = false;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) raw[s][p] = 0u;
+      if (inside[s]) {
+        locate(i, cls[s], j[s], r[s], valid[s]);
+        if (valid[s]) {
+          const uint32_t *xr = reinterpret_cast<const uint32_t *>(Vh + (int64_t)ord[r[s]] * stride_t);
+#pragma unroll
+          for (int p = 0; p < 4; ++p) raw[s][p] = xr[16 * p + l];
         }
       }
     }
 #pragma unroll
-    for (int k = 0; k < RDKV_PACK_V_ROWS_PER_WAVE; ++k) {
-      if (i0 + k >= total) break;
-      int cls; int64_t j, r; bool valid;
-      locate(i0 + k, cls, j, r, valid);
-      const float x0 = __half2float(xa[k]), x1 = __half2float(xb[k]);
-      if (cls == 0) {
-        uint8_t *o = V2 + ((int64_t)h * mN2 + j) * 32;
-        if (valid) quantize_values_d128<2>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 32);
-      } else if (cls == 1) {
-        uint8_t *o = V4 + ((int64_t)h * mN4 + j) * 64;
-        if (valid) quantize_values_d128<4>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 64);
-      } else if (cls == 2) {
-        uint8_t *o = V8 + ((int64_t)h * mN8 + j) * 128;
-        if (valid) quantize_values_d128<8>(x0, x1, lane, o, vsh + r, vzh + r); else zero_bytes(o, 128);
+    for (int s = 0; s < kSteps; ++s) {
+      if (!inside[s]) continue;
+      if (cls[s] == 3) {
+        uint32_t *o = reinterpret_cast<uint32_t *>(V16 + ((int64_t)h * max_n16 + j[s]) * 128);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) o[16 * p + l] = raw[s][p];          // zero when the row is padding
+        continue;
+      }
+      uint32_t q[4][2];
+#pragma unroll
+      for (int p = 0; p < 4; ++p) q[p][0] = q[p][1] = 0u;
+      if (valid[s]) {
+        float x[4][2];
+        float mn = INFINITY, mx = -INFINITY;
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          x[p][0] = __half2float(__ushort_as_half((uint16_t)(raw[s][p] & 0xffffu)));
+          x[p][1] = __half2float(__ushort_as_half((uint16_t)(raw[s][p] >> 16)));
+          mn = fminf(mn, fminf(x[p][0], x[p][1]));
+          mx = fmaxf(mx, fmaxf(x[p][0], x[p][1]));
+        }
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+          mn = fminf(mn, __shfl_xor(mn, off, 64));
+          mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        }
+        const float qmax = cls[s] == 0 ? 3.0f : (cls[s] == 1 ? 15.0f : 255.0f);
+        const RdkvQParams qp = rdkv_qparams(mn, mx, qmax);
+        if (l == 0) {
+          vsh[r[s]] = __float2half_rn(qp.scale);
+          vzh[r[s]] = __float2half_rn(qp.zp);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          q[p][0] = rdkv_qcode(x[p][0], qp, qmax);
+          q[p][1] = rdkv_qcode(x[p][1], qp, qmax);
+        }
+      }
+      if (cls[s] == 0) {
+        uint16_t *o = reinterpret_cast<uint16_t *>(V2 + ((int64_t)h * mN2 + j[s]) * 32);
+        const uint32_t b0 = q[0][0] | (q[1][0] << 2) | (q[2][0] << 4) | (q[3][0] << 6);
+        const uint32_t b1 = q[0][1] | (q[1][1] << 2) | (q[2][1] << 4) | (q[3][1] << 6);
+        o[l] = (uint16_t)(b0 | (b1 << 8));
+      } else if (cls[s] == 1) {
+        uint16_t *o = reinterpret_cast<uint16_t *>(V4 + ((int64_t)h * mN4 + j[s]) * 64);
+        o[l] = (uint16_t)((q[0][0] | (q[2][0] << 4)) | ((q[0][1] | (q[2][1] << 4)) << 8));
+        o[16 + l] = (uint16_t)((q[1][0] | (q[3][0] << 4)) | ((q[1][1] | (q[3][1] << 4)) << 8));
       } else {
-        __half *o = V16 + ((int64_t)h * max_n16 + j) * 128;
-        o[lane] = xa[k];          // zero when the row is padding
-        o[lane + 64] = xb[k];
+        uint16_t *o = reinterpret_cast<uint16_t *>(V8 + ((int64_t)h * mN8 + j[s]) * 128);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) o[16 * p + l] = (uint16_t)(q[p][0] | (q[p][1] << 8));
       }
     }
     return;
@@ -376,6 +420,76 @@ k_minmax_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t st
   }
 }
 
+// D == 128, rows 16-byte aligned: sixteen lanes read one row as 16-byte pieces (eight channels
+// each), four rows per wavefront step, four steps in flight; min/max stay packed fp16 (exact)
+// until the end.
+#define RDKV_LAYER_MINMAX_ROWS_D128 512
+__global__ void __launch_bounds__(256)
+k_minmax_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
+                           const int32_t *__restrict__ order, int64_t order_stride_h,
+                           const int32_t *__restrict__ counts, uint32_t *__restrict__ mm) {
+  const int h = blockIdx.y;
+  const int tk = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2] + counts[4 * h + 3];
+  const int t0 = blockIdx.x * RDKV_LAYER_MINMAX_ROWS_D128;
+  if (t0 >= tk) return;
+  const int t1 = min(t0 + RDKV_LAYER_MINMAX_ROWS_D128, tk);
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Kh = K + (int64_t)h * stride_h;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, sub = lane >> 4, l = lane & 15;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  const half2_t pinf = {(_Float16)INFINITY, (_Float16)INFINITY}, ninf = {(_Float16)-INFINITY, (_Float16)-INFINITY};
+  half2_t mn[4] = {pinf, pinf, pinf, pinf}, mx[4] = {ninf, ninf, ninf, ninf};
+  union Piece { uint4 u; half2_t h[4]; };
+  // a block step covers 16 rows (4 waves x 4 rows); 4 steps are loaded before any is reduced
+  for (int base = t0 + wave * 4 + sub; base < t1; base += 64) {
+    Piece v[4];
+    bool in[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = base + 16 * u;
+      in[u] = t < t1;
+      if (in[u]) v[u].u = *reinterpret_cast<const uint4 *>(Kh + (int64_t)ord[t] * stride_t + 8 * l);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (in[u]) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          mn[k] = __builtin_elementwise_min(mn[k], v[u].h[k]);
+          mx[k] = __builtin_elementwise_max(mx[k], v[u].h[k]);
+        }
+      }
+    }
+  }
+  __shared__ float s_mn[4][128];
+  __shared__ float s_mx[4][128];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    float a0 = (float)mn[k].x, a1 = (float)mn[k].y, b0 = (float)mx[k].x, b1 = (float)mx[k].y;
+#pragma unroll
+    for (int off = 16; off < 64; off <<= 1) {
+      a0 = fminf(a0, __shfl_xor(a0, off, 64));
+      a1 = fminf(a1, __shfl_xor(a1, off, 64));
+      b0 = fmaxf(b0, __shfl_xor(b0, off, 64));
+      b1 = fmaxf(b1, __shfl_xor(b1, off, 64));
+    }
+    if (sub == 0) {
+      s_mn[wave][8 * l + 2 * k] = a0; s_mn[wave][8 * l + 2 * k + 1] = a1;
+      s_mx[wave][8 * l + 2 * k] = b0; s_mx[wave][8 * l + 2 * k + 1] = b1;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int c = threadIdx.x;
+    float a = s_mn[0][c], b = s_mx[0][c];
+#pragma unroll
+    for (int w = 1; w < 4; ++w) { a = fminf(a, s_mn[w][c]); b = fmaxf(b, s_mx[w][c]); }
+    uint32_t *mmh = mm + (int64_t)h * 256;
+    atomicMin(&mmh[c], rdkv_float_to_ordered(a));
+    atomicMax(&mmh[128 + c], rdkv_float_to_ordered(b));
+  }
+}
+
 // One wavefront per canvas row: lanes read the row coalesced (channels l, l+64, ...), quantize
 // with their channel's parameters, scatter the codes to their sorted slots in an LDS row
 // buffer, then lanes assemble and store the packed bytes.
@@ -465,6 +579,123 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
       }
     }
     __builtin_amdgcn_wave_barrier();
+  }
+}
+
+// D == 128, rows 16-byte aligned: sixteen lanes per canvas row (eight channels each, one 16-byte
+// load), four rows per wavefront step, the next step's rows in flight while the current ones are
+// quantized.  A lane's channels never change, so their parameters and slots live in registers;
+// codes go to their sorted slots in a per-row LDS buffer and the row's sixteen lanes assemble the
+// packed bytes from it.
+__global__ void __launch_bounds__(256)
+k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
+                         const int32_t *__restrict__ order, int64_t order_stride_h,
+                         const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
+                         const uint32_t *__restrict__ mm, const int32_t *__restrict__ slot_channel,
+                         int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
+                         uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
+                         __half *__restrict__ zp_out, int rows_per_block) {
+  constexpr int D = 128;
+  extern __shared__ float smem[];
+  const int h = blockIdx.y;
+  const int Dp = n2p + n4p + n8;
+  const int Dp4 = (Dp + 3) & ~3;
+  const int tv = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2], n16 = counts[4 * h + 3];
+  const bool has_pad = tv < max_tv || n16 < max_n16;   // zero rows of the canvas join the min/max
+  const int64_t max_tk = max_tv + max_n16;
+  float *c_scale = smem, *c_zp = smem + D, *c_qmax = smem + 2 * D;
+  int *c_slot = reinterpret_cast<int *>(smem + 3 * D);
+  uint8_t *rowbufs = reinterpret_cast<uint8_t *>(smem + 4 * D);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+  const int sub = lane >> 4, l = lane & 15;
+  const uint32_t *mmh = mm + (int64_t)h * 2 * D;
+  for (int c = threadIdx.x; c < D; c += blockDim.x) c_slot[c] = -1;
+  for (int i = threadIdx.x; i < nwaves * 4 * Dp4; i += blockDim.x) rowbufs[i] = 0;  // pad slots stay 0
+  __syncthreads();
+  for (int s = threadIdx.x; s < Dp; s += blockDim.x) {
+    const int ch = slot_channel[(int64_t)h * Dp + s];
+    const float qmax = s < n2p ? 3.0f : (s < n2p + n4p ? 15.0f : 255.0f);
+    float mn = 0.0f, mx = 0.0f;
+    if (ch >= 0) {
+      mn = rdkv_ordered_to_float(mmh[ch]);
+      mx = rdkv_ordered_to_float(mmh[D + ch]);
+      if (has_pad) {
+        mn = fminf(mn, 0.0f);
+        mx = fmaxf(mx, 0.0f);
+      }
+    }
+    const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
+    if (ch >= 0) {
+      c_scale[ch] = p.scale;
+      c_zp[ch] = p.zp;
+      c_qmax[ch] = qmax;
+      c_slot[ch] = s;
+    }
+    if (blockIdx.x == 0) {
+      scale_out[(int64_t)h * Dp + s] = __float2half_rn(p.scale);
+      zp_out[(int64_t)h * Dp + s] = __float2half_rn(p.zp);
+    }
+  }
+  __syncthreads();
+  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
+  const int rowbytes = sub2 + sub4 + n8;
+  if (rowbytes == 0) return;
+  RdkvQParams qp[8];
+  float qm[8];
+  int sl[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int ch = 8 * l + e;
+    sl[e] = c_slot[ch];
+    qp[e].scale = sl[e] >= 0 ? c_scale[ch] : 1.0f;
+    qp[e].zp = sl[e] >= 0 ? c_zp[ch] : 0.0f;
+    qm[e] = sl[e] >= 0 ? c_qmax[ch] : 0.0f;
+  }
+  const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;
+  const int64_t t1 = (t0 + rows_per_block < max_tk) ? t0 + rows_per_block : max_tk;
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Kh = K + (int64_t)h * stride_h;
+  uint8_t *rb = rowbufs + (wave * 4 + sub) * Dp4;
+  union Piece { uint4 u; uint16_t hw[8]; };
+  auto fetch = [&](int64_t t, Piece &v) {
+    v.u = make_uint4(0u, 0u, 0u, 0u);
+    if (t < t1) {
+      // canvas row -> source token (or a zero row)
+      const __half *kr = nullptr;
+      if (t < tv) kr = Kh + (int64_t)ord[t] * stride_t;
+      else if (t >= max_tv && t - max_tv < n16) kr = Kh + (int64_t)ord[tv + (t - max_tv)] * stride_t;
+      if (kr) v.u = *reinterpret_cast<const uint4 *>(kr + 8 * l);
+    }
+  };
+  const int step = nwaves * 4;
+  Piece cur, nxt;
+  fetch(t0 + wave * 4 + sub, cur);
+  for (int64_t tb = t0 + wave * 4; tb < t1; tb += step) {   // wave-uniform loop bound
+    const int64_t t = tb + sub;
+    fetch(t + step, nxt);
+    if (t < t1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (sl[e] >= 0) rb[sl[e]] = (uint8_t)rdkv_qcode(__half2float(__ushort_as_half(cur.hw[e])), qp[e], qm[e]);
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (t < t1) {
+      const int64_t row = (int64_t)h * max_tk + t;
+      for (int j = l; j < rowbytes; j += 16) {
+        if (j < sub2) {
+          K2[row * sub2 + j] = (uint8_t)(rb[j] | (rb[j + sub2] << 2) | (rb[j + 2 * sub2] << 4) | (rb[j + 3 * sub2] << 6));
+        } else if (j < sub2 + sub4) {
+          const int i = j - sub2;
+          K4[row * sub4 + i] = (uint8_t)(rb[n2p + i] | (rb[n2p + i + sub4] << 4));
+        } else {
+          const int i = j - sub2 - sub4;
+          K8[row * (int64_t)n8 + i] = rb[n2p + n4p + i];
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+    cur = nxt;
   }
 }
 
@@ -610,7 +841,7 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
                "%s: bad segment sizes (%d,%d,%d)", fn, n2p, n4p, n8);
   const int Dp = n2p + n4p + n8;
   RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "%s: %d padded channels > %d", fn, Dp, RDKV_MAX_SLOTS);
-  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0,
+  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0 && ((uintptr_t)V_f16 % 4) == 0,
                "%s: rows must be 4-byte aligned", fn);
   const int64_t v_rows = (int64_t)mN2 + mN4 + mN8 + max_n16;
   const int64_t max_tk = max_tv + max_n16;
@@ -639,17 +870,33 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
                        0, s, mm, D, H_kv);
     const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
     RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
-    hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
-                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+    const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
+    if (rows16) {
+      hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
+                         dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv), dim3(256), 0, s,
+                         (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
+    } else {
+      hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
+                         (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+    }
     const int rows_per_block = 64;
     const int64_t eblocks = rdkv_cdiv(max_tk, rows_per_block);
     RDKV_REQUIRE(eblocks <= 0x7fffffffLL, "%s: too many rows", fn);
     const size_t emit_lds = (size_t)D * 16 + 4 * (size_t)((Dp + 3) & ~3);
     RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
-    hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
-                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv,
-                       max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
-                       (__half *)K_zp_f16, rows_per_block);
+    if (rows16) {
+      const int rows_d128 = 256;
+      const size_t lds_d128 = (size_t)128 * 16 + 16 * (size_t)((Dp + 3) & ~3);
+      hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, rows_d128), H_kv), dim3(256),
+                         lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts,
+                         max_tv, max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
+                         (__half *)K_zp_f16, rows_d128);
+    } else {
+      hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
+                         (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv,
+                         max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
+                         (__half *)K_zp_f16, rows_per_block);
+    }
   }
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
