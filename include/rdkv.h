@@ -191,7 +191,10 @@ typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgro
 /* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.
  * src_slot: int16 [H_kv][n_slots_max] = for each stream slot the index of the source channel
  * in the padded sorted order of K_ch_scale (-1 = pad slot).  units: the layer's H_kv
- * descriptors (device).  n2p/n4p: padded 2-/4-bit channel counts of the source layout. */
+ * descriptors (device).  n2p/n4p: padded 2-/4-bit channel counts of the source layout.
+ * perm (int64, head stride in elements, 0 = one table for all heads), kscale / kzp (fp16, head
+ * stride ks_stride_h): the layer's K_ch_perm_padded_idx, K_ch_scale and K_ch_zp, from which the
+ * unit's slot table (RdkvSlot per stream slot, at qtab_off) is written. */
 int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
                                const uint8_t *K4, int64_t k4_stride_h, int64_t k4_stride_t,
                                const uint8_t *K8, int64_t k8_stride_h, int64_t k8_stride_t,
@@ -201,7 +204,8 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
                                const uint8_t *V8, int64_t v8_stride_h,
                                const void *vscale_f16, const void *vzp_f16, int64_t vs_stride_h,
                                const void *V16_f16, int64_t v16_stride_h, int64_t max_T_v,
-                               const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
+                               const int64_t *perm, int64_t perm_stride_h, const void *kscale_f16,
+                               const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
                                int H_kv, uint8_t *blob, void *stream);
 
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32

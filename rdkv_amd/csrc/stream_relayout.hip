@@ -17,6 +17,10 @@ struct SrcLayer {
   const uint16_t *V16;
   int64_t v16_sh;
   int64_t max_T_v;
+  const int64_t *perm;            // padded sorted slot -> source channel, [H_kv, Dp] (stride 0: shared)
+  int64_t perm_sh;
+  const uint16_t *kscale, *kzp;   // fp16 bits per padded sorted slot, [H_kv, Dp]
+  int64_t ks_sh;
 };
 
 __device__ __forceinline__ uint32_t k_code(const SrcLayer &S, int h, int64_t row, int src) {
@@ -62,7 +66,8 @@ relayout_kernel(SrcLayer S, const RdkvUnit *__restrict__ units, const int16_t *_
   int64_t v_dw[4];
   for (int c = 0; c < 4; ++c) v_dw[c] = (int64_t)tiles[c] * (rdkv_v_tile_bytes(c) / 4);
   const int64_t sz_dw = (int64_t)(tstart[3]) * RDKV_TILE;
-  const int64_t total = k_dw + v_dw[0] + v_dw[1] + v_dw[2] + v_dw[3] + sz_dw;
+  const int64_t qt_dw = 2 * 4 * (int64_t)(u.d8 + 2 * u.d4 + 4 * u.d2);   // RdkvSlot = 2 dwords
+  const int64_t total = k_dw + v_dw[0] + v_dw[1] + v_dw[2] + v_dw[3] + sz_dw + qt_dw;
 
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
        idx += (int64_t)gridDim.x * blockDim.x) {
@@ -128,6 +133,19 @@ relayout_kernel(SrcLayer S, const RdkvUnit *__restrict__ units, const int16_t *_
       *reinterpret_cast<uint32_t *>(blob + u.v_off[cls] + 4 * i) = w;
       continue;
     }
+    if (i >= sz_dw) {  // ---- slot table: {channel, scale, zp, 0} per stream slot
+      i -= sz_dw;
+      const int r = slots[i >> 1];
+      uint32_t w = 0;
+      if (r >= 0) {
+        if ((i & 1) == 0)
+          w = (uint32_t)(uint16_t)S.perm[h * S.perm_sh + r] | ((uint32_t)S.kscale[h * S.ks_sh + r] << 16);
+        else
+          w = (uint32_t)S.kzp[h * S.ks_sh + r];
+      }
+      *reinterpret_cast<uint32_t *>(blob + u.qtab_off + 4 * i) = w;
+      continue;
+    }
     // ---- per-token {scale, zp}
     {
       const int ti = (int)(i / RDKV_TILE), t = (int)(i % RDKV_TILE);
@@ -153,9 +171,11 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
                                         int64_t v4_stride_h, const uint8_t *V8, int64_t v8_stride_h,
                                         const void *vscale_f16, const void *vzp_f16, int64_t vs_stride_h,
                                         const void *V16_f16, int64_t v16_stride_h, int64_t max_T_v,
-                                        const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
+                                        const int64_t *perm, int64_t perm_stride_h, const void *kscale_f16,
+                                        const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
                                         int H_kv, uint8_t *blob, void *stream) {
   RDKV_REQUIRE(H_kv > 0 && units && src_slot && n_slots_max > 0, "rdkv_stream_relayout_layer: bad arguments");
+  RDKV_REQUIRE(perm && kscale_f16 && kzp_f16, "rdkv_stream_relayout_layer: null channel tables");
   RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
                "rdkv_stream_relayout_layer: bad padded channel counts (%d,%d)", n2p, n4p);
   SrcLayer S;
@@ -169,6 +189,8 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
   S.vscale = (const uint16_t *)vscale_f16; S.vzp = (const uint16_t *)vzp_f16; S.vs_sh = vs_stride_h;
   S.V16 = (const uint16_t *)V16_f16; S.v16_sh = v16_stride_h;
   S.max_T_v = max_T_v;
+  S.perm = perm; S.perm_sh = perm_stride_h;
+  S.kscale = (const uint16_t *)kscale_f16; S.kzp = (const uint16_t *)kzp_f16; S.ks_sh = ks_stride_h;
   hipLaunchKernelGGL(relayout_kernel, dim3(1024, H_kv), dim3(256), 0, (hipStream_t)stream, S, units, src_slot,
                      n_slots_max, blob);
   RDKV_CHECK_LAUNCH("rdkv_stream_relayout_layer");

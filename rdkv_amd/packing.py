@@ -727,6 +727,10 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
         K_ch_seg_bounds_per_head=seg_ph, K_ch_perm_padded_idx_for_Q=perm_q,
         T_eff_k=max_tk, n_v16=max_n16, T_eff_k_per_head=t_eff_k_ph,
         n_v16_per_head=n_v16_ph, allocation_v_bits=None, allocation_k_bits=None)
+    # the class sizes were read once above; consumers that need them on the host (the streaming
+    # re-layout) find them here instead of reading the device tensors again
+    packed._host_counts = ([tuple(seg[h]) + (n16[h],) for h in range(H_kv)],
+                           [tuple(info_h[h][2:5]) for h in range(H_kv)])
     return packed, new_v_only
 
 

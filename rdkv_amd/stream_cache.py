@@ -79,7 +79,12 @@ class StreamCache:
 
 
 def _layer_counts(pl: PackedKVLayer, H_kv: int):
-    """Per-head (n2,n4,n8,n16) tokens and (c2,c4,c8) channels of a packed layer."""
+    """Per-head (n2,n4,n8,n16) tokens and (c2,c4,c8) channels of a packed layer.  The whole-layer
+    packer leaves them on the layer as ``_host_counts`` (it has read them already); otherwise
+    they are read from the layer's device tensors."""
+    cached = getattr(pl, "_host_counts", None)
+    if cached is not None:
+        return cached
     if pl.seg_bounds_per_head is not None:
         vb = pl.seg_bounds_per_head.detach().cpu().tolist()
         n16 = pl.n_v16_per_head.detach().cpu().tolist() if pl.n_v16_per_head is not None else [0] * H_kv
@@ -191,7 +196,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
     lib = _lib.load()
     dev = _lib.require_device(layers[0][0].K_ch_scale)
     stream = _lib.stream_of(dev)
-    units_all, blobs = [], []
+    units_all, blobs, keep_alive = [], [], []
     unit_tiles, unit_R = [], []
     stream_bytes = algo_bytes = 0
     n_entries = len(layers)
@@ -203,15 +208,8 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         m2, m4, m8 = (int(v) for v in pl.K_ch_seg_bounds)
         n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
         Dp = n2p + n4p + m8
-        scale_h = pl.K_ch_scale.reshape(H_kv, Dp).detach().cpu().numpy().view(np.uint16)
-        zp_h = pl.K_ch_zp.reshape(H_kv, Dp).detach().cpu().numpy().view(np.uint16)
-        if pl.K_ch_perm_padded_idx_per_head is not None:
-            perm_h = pl.K_ch_perm_padded_idx_per_head.detach().cpu().numpy()
-        else:
-            perm_h = np.broadcast_to(pl.K_ch_perm_padded_idx.detach().cpu().numpy(), (H_kv, Dp))
         units = np.zeros(H_kv, dtype=UNIT_DTYPE)
         src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
-        qtabs = []
         off = 0
         for h in range(H_kv):
             n_tok = tok[h]
@@ -220,11 +218,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             steps = d8 + 2 * d4 + 4 * d2
             assert steps <= MAX_STEPS, f"{steps} channel steps exceed {MAX_STEPS}"
             src_tab[h, :len(src)] = src
-            qt = np.zeros(len(src), dtype=SLOT_DTYPE)
-            for s, r in enumerate(src):
-                if r >= 0:
-                    qt[s] = (int(perm_h[h, r]), int(scale_h[h, r]), int(zp_h[h, r]), 0)
-            qtabs.append(qt)
+            qt_nbytes = len(src) * SLOT_DTYPE.itemsize
             tiles = [-(-n // TILE) for n in n_tok]
             R = d8 + d4 + d2
             u = units[h]
@@ -239,10 +233,10 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             u["sz_off"] = off
             off = _align(off + sum(tiles[:3]) * TILE * 4)
             u["qtab_off"] = off
-            off = _align(off + qt.nbytes)
+            off = _align(off + qt_nbytes)
             # accounting
             stream_bytes += (sum(tiles) * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
-                             + sum(tiles[:3]) * TILE * 4 + qt.nbytes)
+                             + sum(tiles[:3]) * TILE * 4 + qt_nbytes)
             row = -(-c2 // 4) + -(-c4 // 2) + c8
             algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
                            + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
@@ -252,10 +246,6 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
         assert base % 256 == 0
-        for h in range(H_kv):
-            qoff = int(units[h]["qtab_off"])
-            if qtabs[h].nbytes:
-                blob[qoff:qoff + qtabs[h].nbytes] = torch.from_numpy(qtabs[h].view(np.uint8).copy()).to(dev)
         rel_units = torch.from_numpy(units.view(np.uint8).copy()).to(dev)
         src_dev = torch.from_numpy(src_tab).to(dev)
 
@@ -275,11 +265,22 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         vs = pl.V_scale.reshape(H_kv, -1).contiguous()
         vz = pl.V_zp.reshape(H_kv, -1).contiguous()
         V16, v16h, _ = seg3(nvo)
+        ks = pl.K_ch_scale.reshape(H_kv, Dp)
+        kz = pl.K_ch_zp.reshape(H_kv, Dp)
+        if ks.stride(1) != 1 or kz.stride() != ks.stride():
+            ks, kz = ks.contiguous(), kz.contiguous()
+        if pl.K_ch_perm_padded_idx_per_head is not None:
+            perm = pl.K_ch_perm_padded_idx_per_head.to(torch.int64).contiguous()
+            perm_sh = perm.stride(0)
+        else:
+            perm = pl.K_ch_perm_padded_idx.to(torch.int64).contiguous()
+            perm_sh = 0
         _lib.check(lib.rdkv_stream_relayout_layer(
             _lib.ptr(K2), k2h, k2t, _lib.ptr(K4), k4h, k4t, _lib.ptr(K8), k8h, k8t, n2p, n4p,
             _lib.ptr(V2), v2h, _lib.ptr(V4), v4h, _lib.ptr(V8), v8h,
             _lib.ptr(vs), _lib.ptr(vz), vs.stride(0) if vs.numel() else 0,
             _lib.ptr(V16), v16h, int(pl.T_eff),
+            perm.data_ptr(), perm_sh, ks.data_ptr(), kz.data_ptr(), ks.stride(0),
             rel_units.data_ptr(), src_dev.data_ptr(), src_tab.shape[1], H_kv, blob.data_ptr(), stream))
         # kernel-side descriptors carry absolute addresses
         for name in ("k_off", "sz_off", "qtab_off"):
@@ -287,8 +288,10 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         units["v_off"] += base
         units_all.extend(units)
         blobs.append(blob)
-        # keep the temporaries alive until the relayout kernel has run
-        torch.cuda.current_stream(dev).synchronize()
+        # the temporaries stay alive until the relayout kernels have run
+        keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
+    torch.cuda.current_stream(dev).synchronize()
+    del keep_alive
     units_np = np.array(units_all, dtype=UNIT_DTYPE)
     tiles_np = np.asarray(unit_tiles, dtype=np.int64).reshape(-1, 4)
     R_np = np.asarray(unit_R, dtype=np.int64)
