@@ -323,6 +323,20 @@ int rdkv_knapsack_rows(const float *scores, int64_t stride_b, int B, int64_t T, 
                        double tol, void *out, int out_elem_size, int64_t out_stride_b,
                        int32_t *counts, void *stream);
 
+/* ---- blockwise decode re-compression ------------------------------------------------------
+ * obkv_accel/blockwise_decode.py:756-791 _score_block and :794-809 _channel_score.  queries
+ * [H_kv*G, Q, D] and keys [H_kv, T, D] of dtype codes q_dtype / k_dtype (strides in elements,
+ * unit channel stride).  token_scores fp32 [H_kv, T]: sum over the group's query heads and the Q
+ * queries of softmax_t(q . k / sqrt(D)) (causal != 0: key t is visible to query q only if t <= q,
+ * which needs Q == T); NULL skips it.  channel_scores fp32 [H_kv, D]: mean_{g,q}(q^2) *
+ * mean_t(k^2).  fp32 arithmetic, fixed summation order.  workspace:
+ * rdkv_block_score_workspace_bytes(H_kv*G, Q, T, D) bytes (-1: T too large for the kernel). */
+int64_t rdkv_block_score_workspace_bytes(int H_q, int Q, int64_t T, int D);
+int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride_h, int64_t q_stride_q,
+                     const void *keys, int k_dtype, int64_t k_stride_h, int64_t k_stride_t, int H_kv,
+                     int G, int Q, int64_t T, int D, int causal, float *token_scores,
+                     float *channel_scores, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* ---- measurement helpers (no counterpart in the reference) --------------------------------
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)

@@ -21,6 +21,9 @@ Parity status:
     constant rows, optimality of the Lagrangian choice, brute force on tiny rows).
   * ``apply_score_pooling``: pinned against the library routines it reduces to
     (``torch.nn.functional.avg_pool1d`` / ``max_pool1d`` / ``pad``) and by closed forms.
+  * ``score_block``, ``logical_layer_bits``: textbook formulas, pinned by the reference's own
+    known-answer tests (tests/test_blockwise_rdkv.py:70-101 of the reference) and by the library
+    routines they reduce to (einsum + softmax).
   * ``select_joint``: the budget arithmetic between the pinned pieces follows
     obkv_fast.py:979-1041 by reading; the reference module that holds it cannot be imported
     without the model stack, so that glue is **parity unpinned** (the pieces either side of it
@@ -297,3 +300,40 @@ def select_joint(layer_scores: np.ndarray, channel_scores: np.ndarray, *, head_d
     k_bits = allocate_k_bits_per_head(np.asarray(channel_scores, dtype=F32), k_avg,
                                       epsilon=eps_K or DEFAULT_EPSILON_K, bit_options=k_bit_options)
     return pooled, v_bits, k_bits, k_avg
+
+
+# ---------------------------------------------------------------------------
+# obkv_accel/blockwise_decode.py:756-809  block scoring
+# ---------------------------------------------------------------------------
+
+def score_block(queries: np.ndarray, keys: np.ndarray, *, num_kv_groups: int, causal: bool):
+    """blockwise_decode.py:756-791.  queries ``[H_q, Q, D]``, keys ``[1, H_kv, T, D]`` ->
+    (token scores ``[H_kv, T]`` = sum over the group's heads and the queries of the softmax over
+    keys of ``q.k / sqrt(D)``, with key t hidden from query q when ``causal`` and t > q; channel
+    scores ``[H_kv, D]`` = mean over (head, query) of q^2 times mean over tokens of k^2).
+    Textbook formulas in fp32; compared within a tolerance (summation order is the library's)."""
+    q = np.asarray(queries, dtype=F32)
+    k = np.asarray(keys, dtype=F32)[0]
+    h_kv, t_len, d = k.shape
+    q_len = q.shape[1]
+    qg = q.reshape(h_kv, num_kv_groups, q_len, d)
+    logits = (np.einsum("hgqd,htd->hgqt", qg, k).astype(F32) * F32(1.0 / np.sqrt(d))).astype(F32)
+    if causal:
+        if q_len != t_len:
+            raise ValueError(f"self-scored final flush requires equal query/key lengths, got Q={q_len}, T={t_len}")
+        hidden = np.arange(t_len)[None, :] > np.arange(q_len)[:, None]
+        logits = np.where(hidden[None, None], F32(-np.inf), logits)
+    e = np.exp(logits - logits.max(axis=-1, keepdims=True)).astype(F32)
+    attn = (e / e.sum(axis=-1, keepdims=True)).astype(F32)
+    token = attn.sum(axis=(1, 2)).astype(F32)
+    channel = (np.square(qg).mean(axis=(1, 2)) * np.square(k).mean(axis=1)).astype(F32)
+    return token, channel
+
+
+def logical_layer_bits(v_bits: np.ndarray, k_bits: np.ndarray, head_dim: int) -> int:
+    """blockwise_decode.py:665-678: V widths times head_dim plus, per head, the K widths times the
+    number of kept (non-zero-width) V positions of that head."""
+    v = np.asarray(v_bits, dtype=np.int64)
+    k = np.asarray(k_bits, dtype=np.int64)
+    kept = (v > 0).sum(axis=1)
+    return int(v.sum() * head_dim + (k.sum(axis=1) * kept).sum())

@@ -35,7 +35,7 @@
 #include <stdint.h>
 
 #define RDKV_TILE 64
-#define RDKV_MAX_STEPS 36  // (128 channel slots + per-type padding) / 4
+#define RDKV_MAX_STEPS 40  // (128 channel slots + up to 3 + 7 + 15 pad slots of the three widths) / 4
 
 static __host__ __device__ inline int rdkv_field_of(int s, int k, int nf) {
   return 2 * s + (k >> 1) + (k & 1) * (nf >> 1);

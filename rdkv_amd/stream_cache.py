@@ -26,7 +26,8 @@ from .packing import PackedKVLayer, _seg_padded_len
 
 TILE = 64
 V_TILE_BYTES = (2048, 4096, 8192, 16384)       # 2-bit, 4-bit, 8-bit, fp16 tiles of 64 tokens
-MAX_STEPS = 36
+MAX_STEPS = 40                                 # 4-slot steps of a K row: (128 channels + class padding) / 4
+MAX_ROW_DWORDS = 32                            # K row length the fused kernel keeps in registers
 
 UNIT_DTYPE = np.dtype([
     ("k_off", "<u8"), ("v_off", "<u8", (4,)), ("sz_off", "<u8"), ("qtab_off", "<u8"),
@@ -46,12 +47,29 @@ def slot_plan(c2: int, c4: int, c8: int, n2p: int, n4p: int):
     """Stream slot order of one head: 8-bit channels first, then 4-bit, then 2-bit, each padded
     to whole dwords (4 / 8 / 16 channels).  Returns (d8, d4, d2, src) where src[slot] is the
     channel's index in the source layer's padded sorted order ([2-bit | 4-bit | 8-bit],
-    obkv_accel/packing.py:364-388) or -1 for a pad slot."""
-    d8, d4, d2 = -(-c8 // 4), -(-c4 // 8), -(-c2 // 16)
-    src = []
-    src += [n2p + n4p + i for i in range(c8)] + [-1] * (4 * d8 - c8)
-    src += [n2p + i for i in range(c4)] + [-1] * (8 * d4 - c4)
-    src += list(range(c2)) + [-1] * (16 * d2 - c2)
+    obkv_accel/packing.py:364-388) or -1 for a pad slot.
+
+    A narrow code is the same number in a wider field (its scale and zero-point travel with the
+    slot), so the stragglers of a narrow class are moved into the pad slots of the wider classes
+    whenever that saves a whole dword of the K row; and a row that would still be longer than
+    the kernel's 32 dwords (many 8-bit channels plus stragglers) is stored entirely as 8 bit.
+    Values are unchanged either way."""
+    l8 = [n2p + n4p + i for i in range(c8)]
+    l4 = [n2p + i for i in range(c4)]
+    l2 = list(range(c2))
+    pad = lambda n, a: (-n) % a
+    r4 = len(l4) % 8
+    if 0 < r4 <= pad(len(l8), 4):
+        l8, l4 = l8 + l4[-r4:], l4[:-r4]
+    r2 = len(l2) % 16
+    p8, p4 = pad(len(l8), 4), pad(len(l4), 8)
+    if 0 < r2 <= p8 + p4:
+        moved, l2 = l2[-r2:], l2[:-r2]
+        l8, l4 = l8 + moved[:min(r2, p8)], l4 + moved[min(r2, p8):]
+    if -(-len(l8) // 4) + -(-len(l4) // 8) + -(-len(l2) // 16) > MAX_ROW_DWORDS:
+        l8, l4, l2 = l8 + l4 + l2, [], []
+    d8, d4, d2 = -(-len(l8) // 4), -(-len(l4) // 8), -(-len(l2) // 16)
+    src = l8 + [-1] * (4 * d8 - len(l8)) + l4 + [-1] * (8 * d4 - len(l4)) + l2 + [-1] * (16 * d2 - len(l2))
     return d8, d4, d2, src
 
 

@@ -263,10 +263,11 @@ def test_fused_attention_full_size_layer(cfg_idx):
 
 
 @pytest.mark.parametrize("counts", [(1, 1, 120), (128, 0, 0), (0, 128, 0), (0, 0, 128), (60, 60, 8), (17, 9, 5),
-                                    (0, 0, 1), (3, 0, 0)])
+                                    (0, 0, 1), (3, 0, 0), (2, 1, 125), (5, 4, 119), (1, 1, 125), (17, 9, 1)])
 def test_fused_attention_k_row_shapes(counts):
-    """K rows of every shape the kernel variants cover: the widest (36 channel steps, 32
-    dwords), a single field width only, a single channel; against the oracle."""
+    """K rows of every shape the kernel variants cover: the widest (32 dwords), a single field
+    width only, a single channel, stragglers that ride in the pad slots of a wider class, and a
+    row that only fits as all-8-bit; against the oracle."""
     c2, c4, c8 = counts
     H_kv, G, T, D = 2, 4, 333, 128
     rng = np.random.default_rng(c2 * 10007 + c4 * 101 + c8)
@@ -286,7 +287,7 @@ def test_fused_attention_k_row_shapes(counts):
     exp_out, exp_lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
     pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
     cache = stream_cache.build_stream_cache([(pl, nvo)], G)
-    assert cache.max_row_dwords == -(-c8 // 4) + -(-c4 // 8) + -(-c2 // 16)
+    assert cache.max_row_dwords == sum(stream_cache.slot_plan(c2, c4, c8, -(-c2 // 4) * 4, -(-c4 // 2) * 2)[:3]) <= 32
     out, lse = stream_cache.decode_attn_fused(cache, q.to(DEV))
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")

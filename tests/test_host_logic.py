@@ -162,3 +162,38 @@ def test_partition_work_all_empty():
     tiles = np.zeros((3, 4), dtype=np.int64)
     work, groups, wb, wc = partition_work(tiles, np.asarray([4, 0, 7]), n_groups=1)
     assert len(work) == 3 and list(groups) == [0, 3] and list(wc) == [1, 1, 1]
+
+
+def test_slot_plan_covers_every_channel_and_fits_the_kernel():
+    """Every (2-bit, 4-bit, 8-bit) channel split of a 128-channel head: each source channel appears
+    once, pads are -1, a code only ever moves to a wider field, the K row fits 32 dwords and the
+    slot count 40 steps; splits that need no repair keep the plain class order."""
+    from rdkv_amd import stream_cache as sc
+    for c8 in range(0, 129):
+        for c4 in range(0, 129 - c8, 3 if c8 % 5 else 1):
+            for c2 in (0, 1, 2, 15, 16, 17, 128 - c8 - c4):
+                if c2 < 0 or c8 + c4 + c2 > 128:
+                    continue
+                n2p, n4p = -(-c2 // 4) * 4, -(-c4 // 2) * 2
+                d8, d4, d2, src = sc.slot_plan(c2, c4, c8, n2p, n4p)
+                assert len(src) == 4 * d8 + 8 * d4 + 16 * d2
+                real = [r for r in src if r >= 0]
+                assert sorted(real) == sorted(list(range(c2)) + [n2p + i for i in range(c4)]
+                                              + [n2p + n4p + i for i in range(c8)])
+                assert d8 + d4 + d2 <= sc.MAX_ROW_DWORDS and d8 + 2 * d4 + 4 * d2 <= sc.MAX_STEPS
+                plain = -(-c8 // 4) + -(-c4 // 8) + -(-c2 // 16)
+                assert d8 + d4 + d2 <= plain
+                for pos, r in enumerate(src):
+                    if r < 0:
+                        continue
+                    width_src = 2 if r < n2p else (4 if r < n2p + n4p else 8)
+                    width_dst = 8 if pos < 4 * d8 else (4 if pos < 4 * d8 + 8 * d4 else 2)
+                    assert width_dst >= width_src
+    assert sc.slot_plan(16, 32, 16, 16, 32) == (4, 4, 1, [48 + i for i in range(16)] + [16 + i for i in range(32)]
+                                                + list(range(16)))
+    # three 4-bit stragglers ride in the 8-bit class's pad slots
+    d8, d4, d2, src = sc.slot_plan(0, 11, 5, 0, 12)
+    assert (d8, d4, d2) == (2, 1, 0) and src[:8] == [12, 13, 14, 15, 16, 8, 9, 10]
+    # 125 8-bit channels + one 4-bit + two 2-bit channels would need 34 dwords: everything is stored as 8 bit
+    d8, d4, d2, src = sc.slot_plan(2, 1, 125, 4, 2)
+    assert (d8, d4, d2) == (32, 0, 0) and sorted(src) == [0, 1, 4] + [6 + i for i in range(125)]
