@@ -90,6 +90,9 @@ class StreamCache:
     groups: Optional[torch.Tensor] = None  # device int32 [n_groups + 1] offsets into ``work`` (or None)
     groups_host: Optional[np.ndarray] = None
     n_groups: int = 0
+    kv_algorithmic_bytes: int = 0        # algorithmic bytes without the query / output rows
+    multi_source: bool = False           # several units may feed one output row
+    h_q: int = 0                         # query heads per output group
 
     @property
     def device(self):
@@ -192,32 +195,15 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     return work, groups, work_begin, work_count
 
 
-def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
-                       work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
-                       groups_per_cu: int = 1, cost: Optional[dict] = None,
-                       row_of_entry: Optional[Sequence[int]] = None) -> StreamCache:
-    """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
-    layer)) into the streaming format.  Query/output row of entry g, query head hq is
-    ``g * H_q + hq``.
-
-    ``row_of_entry[i]`` = r makes entry i a *source* of output group r instead (rows
-    ``r * H_q + hq``): several entries with the same r are attended over together, the exact
-    softmax over the union of their tokens, each source keeping its own packing (channel
-    layout, scales) - the multi-source attention of blockwise decode
-    (blockwise_decode.py:812-1121) as one fused call.
-
-    Work decomposition: by default the tile stream is cut into one run of equal cost per
-    compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
-    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; small caches get
-    fewer runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
-    many streamed bytes with one workgroup per item."""
+def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
+    """Re-lay every (packed layer, new_v_only) entry into its own blob.  Returns the unit
+    descriptors (absolute addresses, work fields unset), the blobs, and the streamed / algorithmic
+    byte counts of the entries."""
     lib = _lib.load()
     dev = _lib.require_device(layers[0][0].K_ch_scale)
     stream = _lib.stream_of(dev)
     units_all, blobs, keep_alive = [], [], []
-    unit_tiles, unit_R = [], []
     stream_bytes = algo_bytes = 0
-    n_entries = len(layers)
     H_q = None
     for gi, (pl, nvo) in enumerate(layers):
         H_kv = pl.K_ch_scale.shape[1]
@@ -242,7 +228,7 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             u = units[h]
             u["n_tok"] = n_tok
             u["d8"], u["d4"], u["d2"] = d8, d4, d2
-            u["q_row"] = (gi if row_of_entry is None else int(row_of_entry[gi])) * H_q + h * G
+            u["q_row"] = int(rows_of_entries[gi]) * H_q + h * G
             u["k_off"] = off
             off = _align(off + sum(tiles) * TILE * 4 * R)
             for c in range(4):
@@ -259,8 +245,6 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
             algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
                            + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
                            + 256 * n_tok[3])
-            unit_tiles.append(tiles)
-            unit_R.append(R)
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
         assert base % 256 == 0
@@ -310,40 +294,89 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
         keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
     torch.cuda.current_stream(dev).synchronize()
     del keep_alive
-    units_np = np.array(units_all, dtype=UNIT_DTYPE)
-    tiles_np = np.asarray(unit_tiles, dtype=np.int64).reshape(-1, 4)
-    R_np = np.asarray(unit_R, dtype=np.int64)
-    if row_of_entry is not None:
+    return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q
+
+
+def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: int, kv_algo_bytes: int, *,
+                  multi_source: bool, work_bytes, n_groups, groups_per_cu: int, cost) -> StreamCache:
+    """Order the units, cut the tile stream into work items and groups, upload the tables."""
+    dev = blobs[0].device
+    if multi_source:
         # sources of one output row next to each other, so that their work items are contiguous
-        order = np.argsort(units_np["q_row"], kind="stable")
-        units_np, tiles_np, R_np = units_np[order], tiles_np[order], R_np[order]
+        units_np = units_np[np.argsort(units_np["q_row"], kind="stable")]
+    tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
+    R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
     if work_bytes is None and n_groups is None:
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
         n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
     work_np, groups_np, wb, wc = partition_work(tiles_np, R_np,
                                                 n_groups=n_groups, work_bytes=work_bytes,
                                                 cost=cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS))
-    if row_of_entry is not None:
+    if multi_source:
         # the first unit of every output row merges the partials of all its sources
         qr = units_np["q_row"]
         first = np.concatenate([[True], qr[1:] != qr[:-1]])
         run_id = np.cumsum(first) - 1
         wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
-        n_entries = int(max(row_of_entry)) + 1
+    units_np = units_np.copy()
     units_np["work_begin"], units_np["work_count"] = wb, wc
-    rows = n_entries * H_q
-    algo_bytes += rows * 128 * 2 + rows * 128 * 4
+    rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
     units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
     work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
         16, dtype=torch.uint8, device=dev)
     groups_dev = torch.from_numpy(groups_np).to(dev) if groups_np is not None else None
-    return StreamCache(blobs=blobs, units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
+    return StreamCache(blobs=list(blobs), units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
                        n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
-                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(algo_bytes),
-                       max_row_dwords=int(max((int(u["d8"]) + int(u["d4"]) + int(u["d2"]) for u in units_np),
-                                              default=0)),
+                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
+                       max_row_dwords=int(R_np.max()) if len(R_np) else 0,
                        groups=groups_dev, groups_host=groups_np,
-                       n_groups=0 if groups_np is None else len(groups_np) - 1)
+                       n_groups=0 if groups_np is None else len(groups_np) - 1,
+                       kv_algorithmic_bytes=int(kv_algo_bytes), multi_source=multi_source, h_q=int(H_q))
+
+
+def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
+                       work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
+                       groups_per_cu: int = 1, cost: Optional[dict] = None,
+                       row_of_entry: Optional[Sequence[int]] = None) -> StreamCache:
+    """Re-lay ``layers`` = [(packed_layer, new_v_only or None), ...] (one entry per (sequence,
+    layer)) into the streaming format.  Query/output row of entry g, query head hq is
+    ``g * H_q + hq``.
+
+    ``row_of_entry[i]`` = r makes entry i a *source* of output group r instead (rows
+    ``r * H_q + hq``): several entries with the same r are attended over together, the exact
+    softmax over the union of their tokens, each source keeping its own packing (channel
+    layout, scales) - the multi-source attention of blockwise decode
+    (blockwise_decode.py:812-1121) as one fused call.
+
+    Work decomposition: by default the tile stream is cut into one run of equal cost per
+    compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
+    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; small caches get
+    fewer runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
+    many streamed bytes with one workgroup per item."""
+    rows_of_entries = list(range(len(layers))) if row_of_entry is None else [int(r) for r in row_of_entry]
+    assert len(rows_of_entries) == len(layers)
+    units_np, blobs, stream_bytes, kv_algo, H_q = _relayout_entries(layers, G, rows_of_entries)
+    return _finish_cache(units_np, blobs, G, H_q, stream_bytes, kv_algo, multi_source=row_of_entry is not None,
+                         work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
+
+
+def extend_stream_cache(cache: StreamCache, layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]],
+                        row_of_entry: Sequence[int], *, work_bytes: Optional[int] = None,
+                        n_groups: Optional[int] = None, groups_per_cu: int = 1,
+                        cost: Optional[dict] = None) -> StreamCache:
+    """A cache with ``layers`` added as further sources of the output groups ``row_of_entry``
+    (existing groups or new ones).  Only the new entries are re-laid; the blobs of ``cache`` are
+    shared with the result, and the work items are cut again over old and new units.  This is
+    how a block compressed at decode time joins the prompt cache (the reference overwrites a
+    pre-allocated slot of its bank instead, blockwise_decode.py:336-355)."""
+    rows_of_entries = [int(r) for r in row_of_entry]
+    assert len(rows_of_entries) == len(layers) and len(layers) > 0
+    new_units, new_blobs, sb, ab, H_q = _relayout_entries(layers, cache.G, rows_of_entries)
+    assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
+    old = cache.units_host.copy()
+    return _finish_cache(np.concatenate([old, new_units]), list(cache.blobs) + new_blobs, cache.G, H_q,
+                         cache.stream_bytes + sb, cache.kv_algorithmic_bytes + ab, multi_source=True,
+                         work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
@@ -441,7 +474,8 @@ def save_stream_cache(cache: StreamCache, path: str) -> None:
     header = {"version": 1, "G": cache.G, "rows": cache.rows, "stream_bytes": cache.stream_bytes,
               "algorithmic_bytes": cache.algorithmic_bytes, "max_row_dwords": cache.max_row_dwords,
               "n_units": cache.n_units, "n_work": cache.n_work, "n_groups": cache.n_groups,
-              "sections": {}, "blobs": []}
+              "kv_algorithmic_bytes": cache.kv_algorithmic_bytes, "multi_source": bool(cache.multi_source),
+              "h_q": cache.h_q, "sections": {}, "blobs": []}
     off = 0
     for name, arr in parts:
         header["sections"][name] = [off, int(arr.nbytes)]
@@ -507,4 +541,5 @@ def load_stream_cache(path: str, device) -> StreamCache:
         rows=header["rows"], stream_bytes=header["stream_bytes"], algorithmic_bytes=header["algorithmic_bytes"],
         max_row_dwords=header["max_row_dwords"],
         groups=torch.from_numpy(groups).to(dev) if groups is not None else None, groups_host=groups,
-        n_groups=header["n_groups"])
+        n_groups=header["n_groups"], kv_algorithmic_bytes=header.get("kv_algorithmic_bytes", 0),
+        multi_source=header.get("multi_source", False), h_q=header.get("h_q", 0))

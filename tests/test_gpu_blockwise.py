@@ -211,6 +211,22 @@ def test_decode_over_prompt_cache_compressed_blocks_and_raw_tail():
     assert cache.rows == H * G
     got = fast_decode.trizone_attention_fused(cache, to_dev(q), [to_dev(K_tail)], [to_dev(V_tail)], G)
 
+    # the same cache grown block by block, as it happens at decode time: same bits
+    grown = stream_cache.build_stream_cache(sources_dev[:1], G)
+    assert not grown.multi_source and grown.h_q == H * G
+    for src in sources_dev[1:]:
+        grown = stream_cache.extend_stream_cache(grown, [src], [0])
+    assert grown.multi_source and grown.n_units == cache.n_units and grown.rows == cache.rows
+    assert grown.stream_bytes == cache.stream_bytes and grown.algorithmic_bytes == cache.algorithmic_bytes
+    got2 = fast_decode.trizone_attention_fused(grown, to_dev(q), [to_dev(K_tail)], [to_dev(V_tail)], G)
+    assert torch.equal(got2, got)
+    # a second output group added later (another sequence joining the batch)
+    two = stream_cache.extend_stream_cache(grown, sources_dev[:1], [1])
+    assert two.rows == 2 * H * G
+    o2, _ = stream_cache.decode_attn_fused(two, to_dev(np.concatenate([q, q])))
+    o_single, _ = stream_cache.decode_attn_fused(stream_cache.build_stream_cache(sources_dev[:1], G), to_dev(q))
+    assert float((o2[H * G:] - o_single).abs().max()) < 2e-5
+
     # dense reference over the union of dequantized tokens
     exp = np.zeros((H * G, D), F32)
     for h in range(H):
