@@ -272,15 +272,17 @@ int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t vb_stride
                          int32_t *plan, void *stream);
 
 /* Per-head tables and metadata of the stacked layer (packing.py:399-578 pack_k_mixed_per_head's
- * index tensors, :1245-1316 of _pad_and_stack_per_head_layers), from `plan` and the layer-wide
- * sizes the caller derived from it: slot_channel int32 [H_kv, Dp] (source channel per padded
+ * index tensors, :1245-1316 of _pad_and_stack_per_head_layers), from the layer's rows of the two
+ * parts of `plan` (counts4: [H_kv][4], info: [H_kv][8]; for a plan made over the heads of several
+ * layers at once these are that layer's slices) and the layer-wide sizes the caller derived: slot_channel int32 [H_kv, Dp] (source channel per padded
  * slot, -1 = padding; Dp = n2p + n4p + n8), perm int64 [H_kv, Dp] (padding -> 0), perm_for_q
  * int64 [H_kv*G, Dp], sort_ch int64 [H_kv, kept_max] (kept channels by width, zero padded),
  * seg_ch / seg_tok int32 [H_kv, 3], t_eff / t_eff_k / n_v16 int32 [H_kv], sort_idx int64
  * [tv_ref] (rank among head ref_head's quantized tokens, in sorted order) and softmax_mask fp32
  * [H_kv*G, max_tv + max_n16] (0 on token columns, -inf on padding).  D <= 1024. */
 int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int H_kv, int D,
-                           int G, const int32_t *plan, int n2p, int n4p, int n8, int kept_max,
+                           int G, const int32_t *counts4, const int32_t *info, int n2p, int n4p, int n8,
+                           int kept_max,
                            int64_t max_tv, int max_n16, const int32_t *order, int64_t order_stride_h,
                            const int32_t *rank3, int64_t rank3_stride_h, int ref_head, int64_t tv_ref,
                            int32_t *slot_channel, int64_t *perm, int64_t *perm_for_q, int64_t *sort_ch,
@@ -306,13 +308,22 @@ int rdkv_pool_scores(const float *scores, int64_t stride_b, int B, int64_t T, in
  * bits_host / eps_host: n_options (<= 8) HOST floats; widths must be integers in 0..255.
  * out: [B, T] of out_elem_size 1 (u8) or 8 (i64) bytes, row stride in elements.  counts: NULL
  * or device [B, n_options] int32, tokens per option.  T <= 2^20 (the width sums stay exact).
+ * group_rows: the doubling rounds end together for every group_rows consecutive rows (what
+ * was one call of the reference; 0 = the whole batch), so many calls can share one launch.
  * workspace: rdkv_knapsack_workspace_bytes(B) bytes.  Two launches, no host synchronization. */
 int64_t rdkv_knapsack_workspace_bytes(int B);
 int rdkv_knapsack_batched(const float *scores, int64_t stride_b, int B, int64_t T,
                           const float *budget, const float *bits_host, const float *eps_host,
-                          int n_options, int max_iters, float tol, void *out, int out_elem_size,
-                          int64_t out_stride_b, int32_t *counts, void *workspace,
+                          int n_options, int max_iters, float tol, int group_rows, void *out,
+                          int out_elem_size, int64_t out_stride_b, int32_t *counts, void *workspace,
                           int64_t workspace_bytes, void *stream);
+
+/* obkv_fast.py:1033-1035: the per-head K budget k_budget_bits / (head_dim * max(kept_h, 1)) as
+ * the reference's fp32 tensor expression evaluates it (product, reciprocal, product), from the
+ * per-option token counts of rdkv_knapsack_batched: kept_h = T - counts[h][zero_option]
+ * (zero_option < 0: every token is kept).  out: fp32 [rows] on the device. */
+int rdkv_k_budget_per_head(const int32_t *counts, int n_options, int zero_option, int rows, int64_t T,
+                           int head_dim, float k_budget_bits, float *out, void *stream);
 
 /* knapsack_solver.py:39-118  knapsack_bit_allocation applied to each of B independent rows:
  * lambda is bisected in double and rounded to fp32 where it meets the scores, the bound starts

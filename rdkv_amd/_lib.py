@@ -59,11 +59,12 @@ SIGNATURES = {
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
     "rdkv_pack_layer_plan_ints": (L, [I, L]),
     "rdkv_pack_layer_plan": (I, [P, I, L, P, I, L, I, L, I, P, L, P, L, P, P]),
-    "rdkv_pack_layer_tables": (I, [P, I, L, I, I, I, P, I, I, I, I, L, I, P, L, P, L, I, L,
+    "rdkv_pack_layer_tables": (I, [P, I, L, I, I, I, P, P, I, I, I, I, L, I, P, L, P, L, I, L,
                                    P, P, P, P, P, P, P, P, P, P, P, P]),
     "rdkv_pool_scores": (I, [P, L, I, L, I, I, I, P, L, P]),
     "rdkv_knapsack_workspace_bytes": (L, [I]),
-    "rdkv_knapsack_batched": (I, [P, L, I, L, P, P, P, I, I, F, P, I, L, P, P, L, P]),
+    "rdkv_knapsack_batched": (I, [P, L, I, L, P, P, P, I, I, F, I, P, I, L, P, P, L, P]),
+    "rdkv_k_budget_per_head": (I, [P, I, I, I, L, I, F, P, P]),
     "rdkv_knapsack_rows": (I, [P, L, I, L, P, P, P, I, I, Dbl, P, I, L, P, P]),
     "rdkv_block_score_workspace_bytes": (L, [I, I, L, I]),
     "rdkv_block_score": (I, [P, I, L, L, P, I, L, L, I, I, I, L, I, I, P, P, P, L, P]),

@@ -388,7 +388,7 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     ``token_scores_by_layer[l]`` ``[H_kv, T]`` the V scores already accumulated for the block.
     Channel scores -> per-head selection + packing with the block budget -> (optionally) fixed-slot
     shapes -> accounting.  Returns the block and the event record the reference logs."""
-    from .obkv_fast import _perhead_select_and_pack
+    from .obkv_fast import _perhead_select_and_pack, _perhead_select_and_pack_layers
 
     timing_on = os.environ.get("OBKV_BLOCKWISE_PHASE_TIMING", "0") == "1"
     t_start = _sync_stamp(target_kv[0].device)
@@ -398,23 +398,32 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     head_dim = int(target_kv[0].shape[-1] // 2)
     h_kv = int(target_kv[0].shape[1])
     fp16_denominator = 2 * h_kv * head_dim * 16
-    for layer_idx, (kv, queries, token_scores) in enumerate(zip(target_kv, query_block, token_scores_by_layer)):
-        keys = kv[..., :head_dim].to(dtype=model_dtype)
-        values = kv[..., head_dim:].to(dtype=model_dtype)
-        t0 = _sync_stamp(kv.device) if timing_on else 0.0
-        channel_scores = _channel_score(queries, keys, num_kv_groups=num_kv_groups)
-        if timing_on:
-            phase["score_ms"] = phase.get("score_ms", 0.0) + (_sync_stamp(kv.device) - t0) * 1000.0
-        layer_timing: Optional[Dict[str, float]] = {} if timing_on else None
-        packed, new_v_only, _ = _perhead_select_and_pack(
-            keys, values, token_scores, channel_scores, gqa_factor=num_kv_groups, eviction_mode="joint",
-            token_budget=config.block_budget_tokens, k_budget_ratio=config.k_budget_ratio,
-            obs_window=config.obs_window, pool_kernel_size=config.pool_kernel_size,
-            pool_padding=config.pool_padding, pool_type="avg", v_bit_options=config.v_bit_options,
-            k_bit_options=config.k_bit_options, eps_V=config.epsilon_v, eps_K=config.epsilon_k,
-            timing=layer_timing, retain_allocation_metadata=True)
-        for key, value in (layer_timing or {}).items():
-            phase[key] = phase.get(key, 0.0) + float(value)
+    keys = [kv[..., :head_dim].to(dtype=model_dtype) for kv in target_kv]
+    values = [kv[..., head_dim:].to(dtype=model_dtype) for kv in target_kv]
+    select_kw = dict(gqa_factor=num_kv_groups, token_budget=config.block_budget_tokens,
+                     k_budget_ratio=config.k_budget_ratio, obs_window=config.obs_window,
+                     pool_kernel_size=config.pool_kernel_size, pool_padding=config.pool_padding, pool_type="avg",
+                     v_bit_options=config.v_bit_options, k_bit_options=config.k_bit_options,
+                     eps_V=config.epsilon_v, eps_K=config.epsilon_k, retain_allocation_metadata=True)
+    same_shape = all(k.shape == keys[0].shape and k.device == keys[0].device for k in keys)
+    if timing_on or not same_shape:
+        # layer by layer, as the reference does (and with its per-stage timing)
+        results = []
+        for kv, k_l, v_l, queries, token_scores in zip(target_kv, keys, values, query_block, token_scores_by_layer):
+            t0 = _sync_stamp(kv.device) if timing_on else 0.0
+            channel_scores = _channel_score(queries, k_l, num_kv_groups=num_kv_groups)
+            if timing_on:
+                phase["score_ms"] = phase.get("score_ms", 0.0) + (_sync_stamp(kv.device) - t0) * 1000.0
+            layer_timing: Optional[Dict[str, float]] = {} if timing_on else None
+            results.append(_perhead_select_and_pack(k_l, v_l, token_scores, channel_scores, eviction_mode="joint",
+                                                    timing=layer_timing, **select_kw))
+            for key, value in (layer_timing or {}).items():
+                phase[key] = phase.get(key, 0.0) + float(value)
+    else:
+        # all layers of the block share their launches and the one host read
+        channel = [_channel_score(q_l, k_l, num_kv_groups=num_kv_groups) for q_l, k_l in zip(query_block, keys)]
+        results = _perhead_select_and_pack_layers(keys, values, token_scores_by_layer, channel, **select_kw)
+    for layer_idx, (packed, new_v_only, _) in enumerate(results):
         if packed.allocation_v_bits is None or packed.allocation_k_bits is None:
             raise RuntimeError("packed block is missing allocator decisions")
         packed_layers.append(packed)

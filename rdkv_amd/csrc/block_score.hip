@@ -17,7 +17,7 @@ constexpr int kMaxQTile = 16;
 __global__ void __launch_bounds__(kScoreThreads)
 block_score_partial_kernel(const void *__restrict__ queries, int q_dtype, int64_t q_stride_h, int64_t q_stride_q,
                            const void *__restrict__ keys, int k_dtype, int64_t k_stride_h, int64_t k_stride_t,
-                           int G, int Q, int T, int D, int QB, int causal, float scale,
+                           int G, int Q, int T, int D, int QB, int causal, float scale, int wide_rows,
                            float *__restrict__ partial) {
   extern __shared__ float smem[];
   float *qs = smem;                       // [QB][D]
@@ -33,11 +33,43 @@ block_score_partial_kernel(const void *__restrict__ queries, int q_dtype, int64_
 #pragma unroll
     for (int j = 0; j < kMaxQTile; ++j) acc[j] = 0.0f;
     const int64_t kbase = (int64_t)h * k_stride_h + (int64_t)t * k_stride_t;
-    for (int d = 0; d < D; ++d) {
-      const float kv = rdkv_load_as_float(keys, k_dtype, kbase + d);
+    if (wide_rows) {
+      // 2-byte keys in 16-byte aligned rows: eight channels per load, the queries read from LDS
+      // four channels at a time (the same address for every lane: a broadcast)
+      const uint4 *krow = reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(keys) + kbase);
+      for (int d8 = 0; d8 < D / 8; ++d8) {
+        const uint4 raw = krow[d8];
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+        float kv[8];
 #pragma unroll
-      for (int j = 0; j < kMaxQTile; ++j)
-        if (j < nq) acc[j] = fmaf(qs[j * D + d], kv, acc[j]);
+        for (int i = 0; i < 4; ++i) {
+          if (k_dtype == RDKV_DTYPE_F16) {
+            kv[2 * i] = __half2float(__ushort_as_half((uint16_t)(w[i] & 0xffffu)));
+            kv[2 * i + 1] = __half2float(__ushort_as_half((uint16_t)(w[i] >> 16)));
+          } else {
+            kv[2 * i] = __uint_as_float(w[i] << 16);
+            kv[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < kMaxQTile; ++j) {
+          if (j < nq) {
+            const float4 qa = *reinterpret_cast<const float4 *>(qs + j * D + 8 * d8);
+            const float4 qb = *reinterpret_cast<const float4 *>(qs + j * D + 8 * d8 + 4);
+            float a = acc[j];
+            a = fmaf(qa.x, kv[0], a); a = fmaf(qa.y, kv[1], a); a = fmaf(qa.z, kv[2], a); a = fmaf(qa.w, kv[3], a);
+            a = fmaf(qb.x, kv[4], a); a = fmaf(qb.y, kv[5], a); a = fmaf(qb.z, kv[6], a); a = fmaf(qb.w, kv[7], a);
+            acc[j] = a;
+          }
+        }
+      }
+    } else {
+      for (int d = 0; d < D; ++d) {
+        const float kv = rdkv_load_as_float(keys, k_dtype, kbase + d);
+#pragma unroll
+        for (int j = 0; j < kMaxQTile; ++j)
+          if (j < nq) acc[j] = fmaf(qs[j * D + d], kv, acc[j]);
+      }
     }
 #pragma unroll
     for (int j = 0; j < kMaxQTile; ++j) {
@@ -150,11 +182,13 @@ RDKV_API int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride
       return RDKV_EWORKSPACE;
     }
     const size_t lds = ((size_t)qb * D + (size_t)qb * T) * 4;
+    const int wide_rows = (k_dtype == RDKV_DTYPE_F16 || k_dtype == RDKV_DTYPE_BF16) && D % 8 == 0 &&
+                          k_stride_h % 8 == 0 && k_stride_t % 8 == 0 && ((uintptr_t)keys % 16) == 0;
     hipFuncSetAttribute(reinterpret_cast<const void *>(block_score_partial_kernel),
                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     hipLaunchKernelGGL(block_score_partial_kernel, dim3(n_qtiles, H_kv * G), dim3(kScoreThreads), lds, s, queries,
                        q_dtype, q_stride_h, q_stride_q, keys, k_dtype, k_stride_h, k_stride_t, G, Q, (int)T, D, qb,
-                       causal, (float)(1.0 / sqrt((double)D)), reinterpret_cast<float *>(workspace));
+                       causal, (float)(1.0 / sqrt((double)D)), wide_rows, reinterpret_cast<float *>(workspace));
     hipLaunchKernelGGL(block_score_reduce_kernel, dim3((unsigned)rdkv_cdiv(T, 256), H_kv), dim3(256), 0, s,
                        reinterpret_cast<const float *>(workspace), G, n_qtiles, (int)T, token_scores);
   }

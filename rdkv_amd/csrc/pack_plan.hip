@@ -255,7 +255,7 @@ RDKV_API int rdkv_pack_layer_plan(const void *v_bits, int vb_elem_size, int64_t 
 }
 
 RDKV_API int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int H_kv, int D,
-                                    int G, const int32_t *plan, int n2p, int n4p, int n8, int kept_max,
+                                    int G, const int32_t *counts4, const int32_t *info, int n2p, int n4p, int n8, int kept_max,
                                     int64_t max_tv, int max_n16, const int32_t *order, int64_t order_stride_h,
                                     const int32_t *rank3, int64_t rank3_stride_h, int ref_head, int64_t tv_ref,
                                     int32_t *slot_channel, int64_t *perm, int64_t *perm_for_q, int64_t *sort_ch,
@@ -269,21 +269,21 @@ RDKV_API int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_
   RDKV_REQUIRE(max_tv >= 0 && max_n16 >= 0 && ref_head >= 0 && ref_head < H_kv && tv_ref >= 0 && tv_ref <= max_tv,
                "%s: bad token counts", fn);
   const int Dp = n2p + n4p + n8;
-  RDKV_REQUIRE(k_bits && plan && seg_ch && seg_tok && t_eff && t_eff_k && n_v16, "%s: null pointer", fn);
+  RDKV_REQUIRE(k_bits && counts4 && info && seg_ch && seg_tok && t_eff && t_eff_k && n_v16, "%s: null pointer", fn);
   RDKV_REQUIRE(Dp == 0 || (slot_channel && perm && perm_for_q), "%s: null channel table", fn);
   RDKV_REQUIRE(kept_max == 0 || sort_ch, "%s: null channel sort table", fn);
   RDKV_REQUIRE(tv_ref == 0 || (sort_idx && order && rank3), "%s: null token tables", fn);
   hipStream_t s = (hipStream_t)stream;
   const int threads = ((D + 63) / 64) * 64;
   hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, k_bits, kb_elem_size, kb_stride_h, D, G,
-                     plan, plan + 4 * (int64_t)H_kv, n2p, n4p, n8, kept_max, max_tv, slot_channel, perm, perm_for_q,
+                     counts4, info, n2p, n4p, n8, kept_max, max_tv, slot_channel, perm, perm_for_q,
                      sort_ch, seg_ch, seg_tok, t_eff, t_eff_k, n_v16);
   const int64_t max_tk = max_tv + max_n16;
   if (max_tk > 0) {
     RDKV_REQUIRE(softmax_mask, "%s: null mask", fn);
     int64_t bx = rdkv_cdiv(max_tk, 256 * 4);
     if (bx > 1024) bx = 1024;
-    hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, plan, G,
+    hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, counts4, G,
                        max_tv, max_tk, softmax_mask, order ? order + (int64_t)ref_head * order_stride_h : nullptr,
                        rank3 ? rank3 + (int64_t)ref_head * rank3_stride_h : nullptr, tv_ref, sort_idx);
   }

@@ -143,7 +143,7 @@ knapsack_expand_kernel(const float* __restrict__ scores, int64_t stride_b, int T
 // Phase 2: replay the doubling rounds of the whole batch (they stop for every row at once when no
 // row asks for more or when every bound has reached 1e12), then bisect this row.
 __global__ void __launch_bounds__(kMaxThreads)
-knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int B, int T,
+knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int group_rows, int T,
                        const float* __restrict__ budget, Options o, int max_iters, float tol,
                        const float* __restrict__ lam0_all, const int* __restrict__ doublings_all,
                        void* __restrict__ out, int out_elem_size, int64_t out_stride_b,
@@ -151,9 +151,11 @@ knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int B
   __shared__ int lds[32];
   const int b = blockIdx.x;
   const float* row = scores + (int64_t)b * stride_b;
-  // rounds the batch executes: min(max_r d_r, 1 + max_r first round after which row r >= 1e12)
+  // rounds the row's batch executes: min(max_r d_r, 1 + max_r first round after which row r >= 1e12),
+  // r over the group_rows consecutive rows that were one call of the reference
+  const int r0 = (b / group_rows) * group_rows;
   int dmax = 0, gmax = 0;
-  for (int r = threadIdx.x; r < B; r += blockDim.x) {
+  for (int r = r0 + threadIdx.x; r < r0 + group_rows; r += blockDim.x) {
     const int d = doublings_all[r];
     float lam = lam0_all[r];
     int g = kMaxDoublings + 1;                     // never reaches 1e12
@@ -249,6 +251,18 @@ int fail(const char* msg) {
   return RDKV_EINVAL;
 }
 
+// Per-head K budget of the joint selection: k_budget_bits / (head_dim * max(kept, 1)) evaluated
+// the way the reference's tensor expression is: fp32 product, fp32 reciprocal, fp32 product.
+__global__ void k_budget_kernel(const int32_t* __restrict__ counts, int n_options, int zero_col, int rows,
+                                int tokens, float head_dim, float k_budget_bits, float* __restrict__ out) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r >= rows) return;
+  int kept = tokens - (zero_col >= 0 ? counts[(int64_t)r * n_options + zero_col] : 0);
+  if (kept < 1) kept = 1;
+  const float denom = __fmul_rn(head_dim, (float)kept);
+  out[r] = __fmul_rn(__fdiv_rn(1.0f, denom), k_budget_bits);
+}
+
 int make_options(const float* bits_host, const float* eps_host, int n, Options* o) {
   if (bits_host == nullptr || eps_host == nullptr || n < 1 || n > kMaxOptions)
     return fail("knapsack: need 1..8 bit options");
@@ -284,8 +298,8 @@ RDKV_API int64_t rdkv_knapsack_workspace_bytes(int B) { return (int64_t)(B > 0 ?
 
 RDKV_API int rdkv_knapsack_batched(const float* scores, int64_t stride_b, int B, int64_t T,
                                    const float* budget, const float* bits_host, const float* eps_host,
-                                   int n_options, int max_iters, float tol, void* out, int out_elem_size,
-                                   int64_t out_stride_b, int32_t* counts, void* workspace,
+                                   int n_options, int max_iters, float tol, int group_rows, void* out,
+                                   int out_elem_size, int64_t out_stride_b, int32_t* counts, void* workspace,
                                    int64_t workspace_bytes, void* stream) {
   Options o;
   if (int rc = make_options(bits_host, eps_host, n_options, &o)) return rc;
@@ -297,13 +311,15 @@ RDKV_API int rdkv_knapsack_batched(const float* scores, int64_t stride_b, int B,
     return RDKV_EWORKSPACE;
   }
   if (max_iters < 0) return fail("knapsack: negative max_iters");
+  if (group_rows <= 0) group_rows = B;
+  if (B % group_rows != 0) return fail("knapsack: the batch is not a whole number of row groups");
   float* lam0 = reinterpret_cast<float*>(workspace);
   int* doublings = reinterpret_cast<int*>(lam0 + B);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int threads = threads_for(T);
   hipLaunchKernelGGL(knapsack_expand_kernel, dim3(B), dim3(threads), 0, s, scores, stride_b, (int)T, budget, o,
                      lam0, doublings);
-  hipLaunchKernelGGL(knapsack_bisect_kernel, dim3(B), dim3(threads), 0, s, scores, stride_b, B, (int)T, budget,
+  hipLaunchKernelGGL(knapsack_bisect_kernel, dim3(B), dim3(threads), 0, s, scores, stride_b, group_rows, (int)T, budget,
                      o, max_iters, tol, lam0, doublings, out, out_elem_size, out_stride_b, counts);
   RDKV_CHECK_LAUNCH("rdkv_knapsack_batched");
   return RDKV_OK;
@@ -347,5 +363,17 @@ RDKV_API int rdkv_pool_scores(const float* scores, int64_t stride_b, int B, int6
   else        { if (reflect) RDKV_POOL(false, true); else RDKV_POOL(false, false); }
 #undef RDKV_POOL
   RDKV_CHECK_LAUNCH("rdkv_pool_scores");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_k_budget_per_head(const int32_t* counts, int n_options, int zero_option, int rows, int64_t T,
+                                    int head_dim, float k_budget_bits, float* out, void* stream) {
+  if (rows < 0 || n_options < 1 || n_options > kMaxOptions || zero_option >= n_options || T < 0 || head_dim < 1)
+    return fail("k_budget_per_head: bad arguments");
+  if (rows == 0) return RDKV_OK;
+  if (counts == nullptr || out == nullptr) return fail("k_budget_per_head: null pointer");
+  hipLaunchKernelGGL(k_budget_kernel, dim3((rows + 255) / 256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                     counts, n_options, zero_option, rows, (int)T, (float)head_dim, k_budget_bits, out);
+  RDKV_CHECK_LAUNCH("rdkv_k_budget_per_head");
   return RDKV_OK;
 }

@@ -39,10 +39,12 @@ def _rows_f32(scores: Tensor) -> Tensor:
 
 def knapsack_allocate(scores: Tensor, budget_per_token: Union[float, Tensor], epsilon=None, max_iters: int = 64,
                       tol: float = 0.01, bit_options: Optional[Tensor] = None, *, out_dtype=torch.uint8,
-                      with_counts: bool = False):
+                      with_counts: bool = False, group_rows: int = 0):
     """``knapsack_bit_allocation_batched`` with the output type of the caller's choice (uint8 for
     the packer, int64 for the reference's return type) and, on request, the per-row number of
-    tokens that took each option (int32 ``[B, n_options]``), both left on the device."""
+    tokens that took each option (int32 ``[B, n_options]``), both left on the device.
+    ``group_rows``: every ``group_rows`` consecutive rows behave as one call of the reference (its
+    doubling rounds end for a whole call at once), so many calls can share one launch."""
     if epsilon is None:
         epsilon = DEFAULT_EPSILON
     assert scores.dim() == 2, f"knapsack_bit_allocation_batched expects [B, T]; got {tuple(scores.shape)}"
@@ -64,7 +66,7 @@ def knapsack_allocate(scores: Tensor, budget_per_token: Union[float, Tensor], ep
     ws = _lib.workspace(dev, ws_bytes)
     _lib.check(lib.rdkv_knapsack_batched(
         _lib.ptr(s), s.stride(0), B, T, _lib.ptr(budget), bits_c, eps_c, n, int(max_iters), float(tol),
-        _lib.ptr(out), out.element_size(), out.stride(0) if B else T, _lib.ptr(counts), ws.data_ptr(), ws_bytes,
+        int(group_rows), _lib.ptr(out), out.element_size(), out.stride(0) if B else T, _lib.ptr(counts), ws.data_ptr(), ws_bytes,
         _lib.stream_of(dev)))
     return (out, counts) if with_counts else out
 

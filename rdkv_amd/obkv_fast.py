@@ -9,14 +9,14 @@ on the GPU: the only device-to-host reads are the packer's (per-head segment siz
 from __future__ import annotations
 
 import time
-from typing import Dict, Optional, Union
+from typing import Dict, List, Optional, Sequence, Union
 
 import torch
 from torch import Tensor
 
 from . import _lib
 from .knapsack_solver import knapsack_allocate, knapsack_bit_allocation_batched
-from .packing import pack_layer_per_head
+from .packing import pack_layer_per_head, pack_layers_per_head
 
 
 def apply_score_pooling(scores: Tensor, pool_type: str, kernel_size: int, padding_mode: str = "zero") -> Tensor:
@@ -61,6 +61,21 @@ def _allocate_k_bits_per_head(channel_scores: Tensor, k_avg: Union[float, Tensor
     else:
         k_avg_arg = float(k_avg)
     return knapsack_bit_allocation_batched(channel_scores, k_avg_arg, epsilon=epsilon, bit_options=bit_options)
+
+
+def _k_budget_per_head(v_counts: Tensor, v_bit_options: Optional[Tensor], T: int, head_dim: int,
+                       k_budget_bits: float) -> Tensor:
+    """obkv_fast.py:1033-1035 from the per-option token counts of the V allocation: the tokens a
+    head keeps are those that did not take the 0-bit option, and its K budget is the reference's
+    fp32 expression ``k_budget_bits / (head_dim * kept.clamp(min=1).float())`` (which torch
+    evaluates as reciprocal times number), one value per row of ``v_counts``, on the device."""
+    opts = [0.0, 2.0, 4.0, 8.0, 16.0] if v_bit_options is None else [float(b) for b in v_bit_options.tolist()]
+    zero_col = opts.index(0.0) if 0.0 in opts else -1
+    rows, n = int(v_counts.shape[0]), int(v_counts.shape[1])
+    out = torch.empty(rows, dtype=torch.float32, device=v_counts.device)
+    _lib.check(_lib.load().rdkv_k_budget_per_head(v_counts.data_ptr(), n, zero_col, rows, T, head_dim,
+                                                  float(k_budget_bits), _lib.ptr(out), _lib.stream_of(v_counts.device)))
+    return out
 
 
 def _perhead_select_and_pack_joint(
@@ -112,16 +127,7 @@ def _perhead_select_and_pack_joint(
                                              with_counts=True)
     t_v = stamp()
 
-    # tokens kept by a head = everything that did not take the 0-bit option
-    v_opts = [0.0, 2.0, 4.0, 8.0, 16.0] if v_bit_options is None else [float(b) for b in v_bit_options.tolist()]
-    kept_cols = [i for i, b in enumerate(v_opts) if b > 0]
-    t_eff = v_counts[:, kept_cols].sum(dim=1)
-    # the reference's fp32 expression k_budget_bits / (head_dim * kept.float()) is evaluated by torch as
-    # reciprocal(denominator) * k_budget_bits; each step goes through double here and is rounded to fp32
-    # once, which gives the correctly rounded fp32 value of that step whatever the device's fp32 division does
-    denom = (float(head_dim) * t_eff.clamp(min=1).double()).float()
-    recip = (1.0 / denom.double()).float()
-    k_avg_per_head = (recip.double() * torch.tensor(k_budget_bits, dtype=torch.float32).double().item()).float()
+    k_avg_per_head = _k_budget_per_head(v_counts, v_bit_options, T, head_dim, k_budget_bits)
     k_bits_perhead = _allocate_k_bits_per_head(channel_scores.float().to(dev), k_avg_per_head,
                                                epsilon=eps_K, bit_options=k_bit_options)
     t_k = stamp()
@@ -158,3 +164,43 @@ def _perhead_select_and_pack(
         pool_padding=pool_padding, pool_type=pool_type, v_bit_options=v_bit_options,
         k_bit_options=k_bit_options, eps_V=eps_V, eps_K=eps_K, timing=timing,
         retain_allocation_metadata=retain_allocation_metadata)
+
+
+
+def _perhead_select_and_pack_layers(
+    Ks: Sequence[Tensor], Vs: Sequence[Tensor], layer_scores: Sequence[Tensor], channel_scores: Sequence[Tensor], *,
+    gqa_factor: int, token_budget: int, k_budget_ratio: float, obs_window: int,
+    pool_kernel_size: int, pool_padding: str, pool_type: str = "avg",
+    v_bit_options: Optional[Tensor], k_bit_options: Optional[Tensor],
+    eps_V: Dict[int, float], eps_K: Dict[int, float], retain_allocation_metadata: bool = False,
+) -> List[tuple]:
+    """``_perhead_select_and_pack`` for several layers of equal shape (the layers of one decode
+    block) with the launches shared: one pooling launch, one V and one K knapsack over all
+    ``L * H_kv`` rows (every layer's rows form a group of their own, so each row gets exactly the
+    allocation the per-layer call gives it), one planning launch and one host read, then the
+    table and data kernels per layer.  Returns ``[(packed_layer, new_v_only, T_eff), ...]``."""
+    L = len(Ks)
+    assert L > 0 and L == len(Vs) == len(layer_scores) == len(channel_scores)
+    dev = _lib.require_device(*Ks, *Vs)
+    H_kv, T = int(layer_scores[0].shape[0]), int(layer_scores[0].shape[1])
+    head_dim = int(Ks[0].shape[3])
+    scores = torch.stack([s.to(dev).float() for s in layer_scores]).reshape(L * H_kv, T)
+    chans = torch.stack([c.to(dev).float() for c in channel_scores]).reshape(L * H_kv, head_dim)
+    pooled = (apply_score_pooling(scores, pool_type=pool_type, kernel_size=pool_kernel_size,
+                                  padding_mode=pool_padding) if pool_kernel_size > 1 else scores)
+    total_budget_bits = 2 * token_budget * head_dim * 16
+    v_avg = (1.0 - k_budget_ratio) * total_budget_bits / (T * head_dim)
+    k_budget_bits = k_budget_ratio * total_budget_bits
+    v_bits, v_counts = knapsack_allocate(pooled, v_avg, epsilon=eps_V, bit_options=v_bit_options, with_counts=True,
+                                         group_rows=H_kv)
+    k_avg = _k_budget_per_head(v_counts, v_bit_options, T, head_dim, k_budget_bits)
+    k_bits = knapsack_allocate(chans, k_avg, epsilon=eps_K, bit_options=k_bit_options, group_rows=H_kv)
+    v_bits, k_bits = v_bits.reshape(L, H_kv, T), k_bits.reshape(L, H_kv, head_dim)
+    packed = pack_layers_per_head(Ks, Vs, v_bits, k_bits, gqa_factor)
+    out = []
+    for l, (layer, new_v_only) in enumerate(packed):
+        if retain_allocation_metadata:
+            layer.allocation_v_bits = v_bits[l].to(torch.int16)
+            layer.allocation_k_bits = k_bits[l].to(torch.int16)
+        out.append((layer, new_v_only, layer.T_eff))
+    return out

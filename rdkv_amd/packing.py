@@ -616,30 +616,13 @@ def _pad_and_stack_per_head_layers(
 
 _PLAN_INT_DTYPES = (torch.uint8, torch.int16, torch.int32, torch.int64)
 
-def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,
-                        gqa_factor: int) -> Tuple[PackedKVLayer, Optional[Tensor]]:
-    """Prefill packing of one layer with per-head allocations: the result of the reference's
-    composition (obkv_fast.py:1141-1155: per head ``build_packed_layer`` with deferred K,
-    packing.py:801-1013, then ``_pad_and_stack_per_head_layers``, packing.py:1019-1317),
-    bit for bit, without the per-head loop: ``rdkv_pack_layer_plan`` (stable token order by class
-    and all class sizes, read once by the host to size the tensors), ``rdkv_pack_layer_tables``
-    (channel tables, per-head metadata, padding mask) and ``rdkv_pack_layer_per_head`` (V rows, K
-    min/max, K emit).  K, V [1,H_kv,T,D] fp16;
-    v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
-    dev = _lib.require_device(K, V)
-    assert K.dim() == 4 and K.shape[0] == 1 and K.shape == V.shape, (
-        f"Expected K, V [1,H_kv,T,D], got {tuple(K.shape)} / {tuple(V.shape)}")
-    H_kv, T, D = int(K.shape[1]), int(K.shape[2]), int(K.shape[3])
-    assert tuple(v_bits_per_head.shape) == (H_kv, T) and tuple(k_bits_per_head.shape) == (H_kv, D)
-    if T == 0:
-        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
-    Kf, Vf = _as_f16_heads(K)[0], _as_f16_heads(V)[0]
-    if Vf.stride() != Kf.stride():
-        Kf, Vf = Kf.contiguous(), Vf.contiguous()
+def _plan_layers(v_bits: Tensor, k_bits: Tensor, dev):
+    """Token order, quantized-token ranks and class sizes of ``[N, T]`` / ``[N, D]`` allocations
+    (N = heads of one layer, or of several layers stacked) in one launch pair and one host read.
+    Returns (order, rank3, plan, counts rows [N][4], info rows [N][8], k_bits as passed on)."""
     lib = _lib.load()
-    stream = _lib.stream_of(dev)
-    vb = v_bits_per_head if v_bits_per_head.device == dev else v_bits_per_head.to(dev)
-    kb = k_bits_per_head if k_bits_per_head.device == dev else k_bits_per_head.to(dev)
+    vb = v_bits if v_bits.device == dev else v_bits.to(dev)
+    kb = k_bits if k_bits.device == dev else k_bits.to(dev)
     if vb.dtype not in _PLAN_INT_DTYPES:
         vb = vb.long()
     if kb.dtype not in _PLAN_INT_DTYPES:
@@ -648,18 +631,32 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
         vb = vb.contiguous()
     if kb.stride(1) != 1:
         kb = kb.contiguous()
-    # token order (stable by class), quantized-token ranks and all class sizes in one launch
-    order = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
-    rank3 = torch.empty(H_kv, T, dtype=torch.int32, device=dev)
-    plan = torch.empty(lib.rdkv_pack_layer_plan_ints(H_kv, T), dtype=torch.int32, device=dev)
+    N, T = int(vb.shape[0]), int(vb.shape[1])
+    order = torch.empty(N, T, dtype=torch.int32, device=dev)
+    rank3 = torch.empty(N, T, dtype=torch.int32, device=dev)
+    plan = torch.empty(lib.rdkv_pack_layer_plan_ints(N, T), dtype=torch.int32, device=dev)
     _lib.check(lib.rdkv_pack_layer_plan(vb.data_ptr(), vb.element_size(), vb.stride(0), kb.data_ptr(),
-                                        kb.element_size(), kb.stride(0), H_kv, T, D, order.data_ptr(),
-                                        order.stride(0), rank3.data_ptr(), rank3.stride(0), plan.data_ptr(), stream))
-    plan_h = plan[:12 * H_kv].cpu().tolist()                    # the one synchronization
-    counts_h = [plan_h[4 * h:4 * h + 4] for h in range(H_kv)]
-    info_h = [plan_h[4 * H_kv + 8 * h:4 * H_kv + 8 * h + 8] for h in range(H_kv)]
+                                        kb.element_size(), kb.stride(0), N, T, int(kb.shape[1]), order.data_ptr(),
+                                        order.stride(0), rank3.data_ptr(), rank3.stride(0), plan.data_ptr(),
+                                        _lib.stream_of(dev)))
+    plan_h = plan[:12 * N].cpu().tolist()                       # the one synchronization
+    counts_h = [plan_h[4 * h:4 * h + 4] for h in range(N)]
+    info_h = [plan_h[4 * N + 8 * h:4 * N + 8 * h + 8] for h in range(N)]
     assert all(row[1] == 0 for row in info_h), "v_bits must be in {0,2,4,8,16}"
     assert all(row[5] == 0 for row in info_h), "k_bits must be in {0,2,4,8,16}"
+    return order, rank3, plan, counts_h, info_h, kb
+
+
+def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: int, n_total: int):
+    """Pack the layer whose heads are rows ``first .. first + H_kv`` of a plan over ``n_total``
+    heads.  Returns None when the layer is degenerate (nothing kept / no channels kept / more
+    than 1024 channels) and must take the composed path."""
+    order, rank3, plan, counts_all, info_all, kb_all = planned
+    dev = K.device
+    lib = _lib.load()
+    stream = _lib.stream_of(dev)
+    H_kv, T, D = int(K.shape[1]), int(K.shape[2]), int(K.shape[3])
+    counts_h, info_h = counts_all[first:first + H_kv], info_all[first:first + H_kv]
     seg = [tuple(row[:3]) for row in counts_h]
     n16 = [row[3] for row in counts_h]
     tv = [sum(s3) for s3 in seg]
@@ -673,9 +670,15 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     sub4 = _seg_padded_len(m4, 2) // 2
     Dp = 4 * sub2 + 2 * sub4 + m8
     if max_tk == 0 or Dp == 0 or D > 1024:
-        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
+        return None
+    Kf, Vf = _as_f16_heads(K)[0], _as_f16_heads(V)[0]
+    if Vf.stride() != Kf.stride():
+        Kf, Vf = Kf.contiguous(), Vf.contiguous()
     ref = next((h for h in range(H_kv) if tk[h] > 0), 0)
     H_q = H_kv * gqa_factor
+    order_l, rank3_l, kb = order[first:first + H_kv], rank3[first:first + H_kv], kb_all[first:first + H_kv]
+    counts4_ptr = plan.data_ptr() + 4 * 4 * first
+    info_ptr = plan.data_ptr() + 4 * (4 * n_total + 8 * first)
 
     def u8(n, w):
         return torch.empty(1, H_kv, n, w, dtype=torch.uint8, device=dev) if n > 0 and w > 0 else None
@@ -694,11 +697,11 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     sort_idx = torch.empty(tv[ref], **i64)
     softmax_mask = torch.empty(H_q, max_tk, dtype=torch.float32, device=dev)
     _lib.check(lib.rdkv_pack_layer_tables(
-        kb.data_ptr(), kb.element_size(), kb.stride(0), H_kv, D, gqa_factor, plan.data_ptr(), 4 * sub2, 2 * sub4,
-        m8, kept_max, max_tv, max_n16, order.data_ptr(), order.stride(0), rank3.data_ptr(), rank3.stride(0), ref,
-        tv[ref], slot_ch.data_ptr(), perm_ph.data_ptr(), perm_q.data_ptr(), _lib.ptr(sort_ph), seg_ph.data_ptr(),
-        seg_tok.data_ptr(), t_eff_ph.data_ptr(), t_eff_k_ph.data_ptr(), n_v16_ph.data_ptr(), _lib.ptr(sort_idx),
-        softmax_mask.data_ptr(), stream))
+        kb.data_ptr(), kb.element_size(), kb.stride(0), H_kv, D, gqa_factor, counts4_ptr, info_ptr, 4 * sub2,
+        2 * sub4, m8, kept_max, max_tv, max_n16, order_l.data_ptr(), order_l.stride(0), rank3_l.data_ptr(),
+        rank3_l.stride(0), ref, tv[ref], slot_ch.data_ptr(), perm_ph.data_ptr(), perm_q.data_ptr(),
+        _lib.ptr(sort_ph), seg_ph.data_ptr(), seg_tok.data_ptr(), t_eff_ph.data_ptr(), t_eff_k_ph.data_ptr(),
+        n_v16_ph.data_ptr(), _lib.ptr(sort_idx), softmax_mask.data_ptr(), stream))
 
     V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
     V_scale = torch.zeros(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)
@@ -710,7 +713,7 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
     _lib.check(lib.rdkv_pack_layer_per_head(
         Kf.data_ptr(), Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D,
-        order.data_ptr(), order.stride(0), plan.data_ptr(), mN[0], mN[1], mN[2], max_tv, max_n16,
+        order_l.data_ptr(), order_l.stride(0), counts4_ptr, mN[0], mN[1], mN[2], max_tv, max_n16,
         slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8,
         _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only),
         _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), stream))
@@ -732,6 +735,52 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     packed._host_counts = ([tuple(seg[h]) + (n16[h],) for h in range(H_kv)],
                            [tuple(info_h[h][2:5]) for h in range(H_kv)])
     return packed, new_v_only
+
+
+def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,
+                        gqa_factor: int) -> Tuple[PackedKVLayer, Optional[Tensor]]:
+    """Prefill packing of one layer with per-head allocations: the result of the reference's
+    composition (obkv_fast.py:1141-1155: per head ``build_packed_layer`` with deferred K,
+    packing.py:801-1013, then ``_pad_and_stack_per_head_layers``, packing.py:1019-1317),
+    bit for bit, without the per-head loop: ``rdkv_pack_layer_plan`` (stable token order by class
+    and all class sizes, read once by the host to size the tensors), ``rdkv_pack_layer_tables``
+    (channel tables, per-head metadata, padding mask) and ``rdkv_pack_layer_per_head`` (V rows, K
+    min/max, K emit).  K, V [1,H_kv,T,D] fp16;
+    v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
+    dev = _lib.require_device(K, V)
+    assert K.dim() == 4 and K.shape[0] == 1 and K.shape == V.shape, (
+        f"Expected K, V [1,H_kv,T,D], got {tuple(K.shape)} / {tuple(V.shape)}")
+    H_kv, T, D = int(K.shape[1]), int(K.shape[2]), int(K.shape[3])
+    assert tuple(v_bits_per_head.shape) == (H_kv, T) and tuple(k_bits_per_head.shape) == (H_kv, D)
+    if T == 0:
+        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
+    planned = _plan_layers(v_bits_per_head, k_bits_per_head, dev)
+    done = _pack_planned_layer(K, V, gqa_factor, planned, 0, H_kv)
+    if done is None:
+        return _pack_layer_per_head_composed(K, V, v_bits_per_head, k_bits_per_head, gqa_factor)
+    return done
+
+
+def pack_layers_per_head(Ks: Sequence[Tensor], Vs: Sequence[Tensor], v_bits: Tensor, k_bits: Tensor,
+                         gqa_factor: int) -> List[Tuple[PackedKVLayer, Optional[Tensor]]]:
+    """``pack_layer_per_head`` for several layers of equal shape with one planning launch and one
+    host read for all of them: ``v_bits [L, H_kv, T]``, ``k_bits [L, H_kv, D]``; layer l is
+    packed from ``Ks[l]``, ``Vs[l]`` exactly as the single-layer call would."""
+    L = len(Ks)
+    dev = _lib.require_device(*Ks, *Vs)
+    assert L == len(Vs) == int(v_bits.shape[0]) == int(k_bits.shape[0]) and L > 0
+    H_kv, T, D = int(Ks[0].shape[1]), int(Ks[0].shape[2]), int(Ks[0].shape[3])
+    assert tuple(v_bits.shape) == (L, H_kv, T) and tuple(k_bits.shape) == (L, H_kv, D)
+    if T == 0:
+        return [_pack_layer_per_head_composed(Ks[l], Vs[l], v_bits[l], k_bits[l], gqa_factor) for l in range(L)]
+    planned = _plan_layers(v_bits.reshape(L * H_kv, T), k_bits.reshape(L * H_kv, D), dev)
+    out = []
+    for l in range(L):
+        assert Ks[l].shape == Ks[0].shape == Vs[l].shape
+        done = _pack_planned_layer(Ks[l], Vs[l], gqa_factor, planned, l * H_kv, L * H_kv)
+        out.append(done if done is not None else
+                   _pack_layer_per_head_composed(Ks[l], Vs[l], v_bits[l], k_bits[l], gqa_factor))
+    return out
 
 
 def _pack_layer_per_head_composed(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_per_head: Tensor,

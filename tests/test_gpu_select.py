@@ -202,3 +202,46 @@ def test_select_and_pack_layer_matches_oracle(case):
             to_dev(K), to_dev(V), to_dev(ls), to_dev(cs), gqa_factor=G, eviction_mode="topk", token_budget=budget,
             k_budget_ratio=ratio, obs_window=32, pool_kernel_size=7, pool_padding="reflect",
             v_bit_options=None, k_bit_options=None, eps_V=ks.DEFAULT_EPSILON_V, eps_K=ks.DEFAULT_EPSILON_K)
+
+
+def test_row_groups_reproduce_separate_calls():
+    """Two golden cases (one with budgets no allocation can meet, whose rows double together for
+    all 40 rounds) stacked into one launch with group_rows = rows per case: every group gets what
+    its own call gave."""
+    g = load_golden("knapsack")
+    names = ("k_24816", "k_unreachable_mixed")
+    scores = np.concatenate([g[n + ".scores"] for n in names])
+    budget = np.concatenate([g[n + ".budget"] for n in names])
+    opts = g[names[0] + ".options"]
+    eps = {int(b): float(e) for b, e in zip(opts, g[names[0] + ".eps"])}
+    out = ks.knapsack_allocate(to_dev(scores), to_dev(budget), eps, bit_options=_opts(opts), group_rows=8)
+    np.testing.assert_array_equal(t2n(out), np.concatenate([g[n + ".bits"] for n in names]))
+    with pytest.raises(AssertionError):
+        ks.knapsack_allocate(to_dev(scores), to_dev(budget), eps, bit_options=_opts(opts), group_rows=5)
+
+
+def test_multi_layer_selection_equals_per_layer():
+    import dataclasses
+    L, H, G, T, D = 3, 2, 2, 200, 128
+    g = torch.Generator().manual_seed(31)
+    Ks = [torch.randn(1, H, T, D, generator=g).half().to(DEV) for _ in range(L)]
+    Vs = [torch.randn(1, H, T, D, generator=g).half().to(DEV) for _ in range(L)]
+    scores = [torch.exp(torch.randn(H, T, generator=g) * 2).to(DEV) for _ in range(L)]
+    scores[1][0] = 0.0                                                      # a head that keeps nothing
+    chans = [torch.exp(torch.randn(H, D, generator=g)).to(DEV) for _ in range(L)]
+    kw = dict(gqa_factor=G, token_budget=40, k_budget_ratio=0.5, obs_window=32, pool_kernel_size=7,
+              pool_padding="reflect", pool_type="avg", v_bit_options=None, k_bit_options=_opts([2, 4, 8, 16]),
+              eps_V=ks.DEFAULT_EPSILON_V, eps_K=ks.DEFAULT_EPSILON_K, retain_allocation_metadata=True)
+    together = obkv_fast._perhead_select_and_pack_layers(Ks, Vs, scores, chans, **kw)
+    for l in range(L):
+        alone = obkv_fast._perhead_select_and_pack(Ks[l], Vs[l], scores[l], chans[l], **kw)
+        assert together[l][2] == alone[2]
+        assert (together[l][1] is None) == (alone[1] is None)
+        if alone[1] is not None:
+            assert torch.equal(together[l][1], alone[1])
+        for f in dataclasses.fields(alone[0]):
+            a, b = getattr(together[l][0], f.name), getattr(alone[0], f.name)
+            if torch.is_tensor(b):
+                assert a.dtype == b.dtype and torch.equal(a, b), f.name
+            else:
+                assert a == b, f.name
