@@ -307,8 +307,13 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
     tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
     R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
     if work_bytes is None and n_groups is None:
+        # Every group costs a fixed amount (set-up, its partials, their merge), every tile a fixed
+        # amount per group that shares the stream: the step time a*tiles/n + b*n is least at
+        # n ~ sqrt(tiles); the factor is fitted to single-layer calls of 4k..128k tokens.  Large
+        # caches get one group per compute unit, tiny ones at least 4 tiles per group.
         cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        n_groups = max(1, min(groups_per_cu * cus, int(tiles_np.sum()) // 4))
+        total_tiles = int(tiles_np.sum())
+        n_groups = max(1, min(groups_per_cu * cus, int(round((6.0 * total_tiles) ** 0.5)), total_tiles // 4))
     work_np, groups_np, wb, wc = partition_work(tiles_np, R_np,
                                                 n_groups=n_groups, work_bytes=work_bytes,
                                                 cost=cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS))
@@ -350,8 +355,8 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
 
     Work decomposition: by default the tile stream is cut into one run of equal cost per
     compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
-    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; small caches get
-    fewer runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
+    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; caches too small to
+    keep every compute unit busy for long get about sqrt(6 * tiles) runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
     many streamed bytes with one workgroup per item."""
     rows_of_entries = list(range(len(layers))) if row_of_entry is None else [int(r) for r in row_of_entry]
     assert len(rows_of_entries) == len(layers)
