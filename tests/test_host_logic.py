@@ -197,3 +197,45 @@ def test_slot_plan_covers_every_channel_and_fits_the_kernel():
     # 125 8-bit channels + one 4-bit + two 2-bit channels would need 34 dwords: everything is stored as 8 bit
     d8, d4, d2, src = sc.slot_plan(2, 1, 125, 4, 2)
     assert (d8, d4, d2) == (32, 0, 0) and sorted(src) == [0, 1, 4] + [6 + i for i in range(125)]
+
+
+def test_selection_and_planning_entry_points_reject_bad_arguments():
+    """Argument checks of the newer entry points run before any device work, so they can be
+    exercised without a GPU: status code and message."""
+    import ctypes
+    lib = _lib.load()
+    f4 = (ctypes.c_float * 4)(0.0, 2.0, 4.0, 8.0)
+    e4 = (ctypes.c_float * 4)(1.0, 0.25, 0.01, 0.0)
+    bad = (ctypes.c_float * 2)(0.0, 2.5)
+
+    def err(rc, text):
+        assert rc == _lib.RDKV_EINVAL, rc
+        assert text.encode() in lib.rdkv_last_error(), lib.rdkv_last_error()
+
+    err(lib.rdkv_knapsack_batched(None, 8, 2, 8, None, f4, e4, 0, 64, 0.01, 0, None, 1, 8, None, None, 0, None),
+        "bit options")
+    err(lib.rdkv_knapsack_batched(None, 8, 2, 8, None, bad, e4, 2, 64, 0.01, 0, None, 1, 8, None, None, 0, None),
+        "integers")
+    err(lib.rdkv_knapsack_batched(None, 8, 2, 0, None, f4, e4, 4, 64, 0.01, 0, None, 1, 8, None, None, 0, None),
+        "empty")
+    err(lib.rdkv_knapsack_batched(None, 8, 2, (1 << 20) + 1, None, f4, e4, 4, 64, 0.01, 0, None, 1, 8, None, None, 0,
+                                  None), "2^20")
+    err(lib.rdkv_knapsack_batched(None, 8, 2, 8, None, f4, e4, 4, 64, 0.01, 0, None, 3, 8, None, None, 0, None),
+        "null pointer")
+    assert lib.rdkv_knapsack_batched(None, 8, 0, 8, None, f4, e4, 4, 64, 0.01, 0, None, 1, 8, None, None, 0, None) == 0
+    assert lib.rdkv_knapsack_workspace_bytes(8) >= 64
+    err(lib.rdkv_knapsack_rows(None, 8, 1, 8, None, f4, e4, 9, 64, 0.01, None, 1, 8, None, None), "bit options")
+    err(lib.rdkv_pool_scores(None, 8, 1, 8, 0, 1, 1, None, 8, None), "bad size")
+    err(lib.rdkv_pool_scores(None, 8, 1, 0, 7, 1, 1, None, 8, None), "empty score sequence")
+    err(lib.rdkv_pool_scores(None, 8, 1, 8, 7, 1, 1, None, 8, None), "null pointer")
+    err(lib.rdkv_k_budget_per_head(None, 5, 5, 1, 8, 128, 1.0, None, None), "bad arguments")
+    err(lib.rdkv_block_score(None, 1, 8, 8, None, 1, 8, 8, 1, 1, 4, 5, 8, 1, None, None, None, 0, None), "null pointer")
+    err(lib.rdkv_block_score(None, 7, 8, 8, None, 1, 8, 8, 1, 1, 4, 4, 8, 0, None, None, None, 0, None), "dtype")
+    assert lib.rdkv_block_score_workspace_bytes(32, 128, 128, 128) == 32 * 8 * 128 * 4
+    assert lib.rdkv_block_score_workspace_bytes(32, 128, 1 << 20, 128) == -1
+    err(lib.rdkv_pack_layer_plan(None, 3, 8, None, 1, 8, 2, 8, 8, None, 8, None, 8, None, None), "element sizes")
+    err(lib.rdkv_pack_layer_plan(None, 1, 8, None, 1, 8, 2, 0, 8, None, 8, None, 8, None, None), "bad shape")
+    assert lib.rdkv_pack_layer_plan_ints(8, 4096) == 8 * (12 + 6 * 4)
+    err(lib.rdkv_pack_layer_tables(None, 1, 8, 2, 2048, 1, None, None, 0, 0, 8, 8, 4, 0, None, 0, None, 0, 0, 0,
+                                   None, None, None, None, None, None, None, None, None, None, None, None),
+        "bad shape")
