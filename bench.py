@@ -26,6 +26,7 @@ HBM_PEAK_GBPS = 8000.0
 # runs of this command (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors a plain copy
 # kernel of known size gives): (556 752 x 2 + 3 100) KiB.  Other workloads: not measured.
 MEASURED_TRAFFIC_BYTES = {1: 1143576576}
+PACK_SAMPLE_LAYERS = 8                      # layers of one sequence packed back to back for the pack throughput
 
 
 def parse():
@@ -86,6 +87,7 @@ def main():
     t_build = time.time()
     groups = []          # (packed layer, new_v_only) per (sequence, layer)
     keep_first = None    # layer 0 of sequence 0: inputs kept for the CPU baseline / checks / dense run
+    pack_sample = []     # fp16 K/V + allocations of the first layers of sequence 0
     for seq in range(cfg.batch):
         for layer in range(cfg.layers):
             vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
@@ -155,7 +157,28 @@ def main():
                                                                  if k in ("pooling_ms", "v_allocation_ms",
                                                                           "k_allocation_ms")))
                 del tok_scores, ch_scores
+            if seq == 0 and layer < PACK_SAMPLE_LAYERS and cfg.layers > 1:
+                pack_sample.append((K, V, vb, kb))
             del K, V
+    if len(pack_sample) > 1:
+        # one sequence's prefill cache packed layer after layer from resident fp16 K/V (a bounded sample
+        # of its first layers): one planning launch and one host read for all of them, the host side of a
+        # layer overlapping the kernels of the one before
+        vb_all = torch.stack([p[2] for p in pack_sample]).to(dev)
+        kb_all = torch.stack([p[3] for p in pack_sample]).to(dev)
+        times = []
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            packing.pack_layers_per_head([p[0] for p in pack_sample], [p[1] for p in pack_sample], vb_all, kb_all, cfg.G)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        sample_bytes = sum(2 * p[0].numel() * p[0].element_size() for p in pack_sample)
+        pack_info["pack_layers_sample"] = len(pack_sample)
+        pack_info["pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
+        pack_info["pack_GBps_of_fp16_input_batched"] = sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
+        del vb_all, kb_all
+    pack_sample.clear()
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
                                             work_bytes=args.work_kib * 1024 if args.work_kib else None,

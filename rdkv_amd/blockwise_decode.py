@@ -205,6 +205,8 @@ def _copy_tensor_field(dst: Optional[Tensor], src: Optional[Tensor]) -> None:
 def _copy_fixed_slot_block_into_bank(*, dst_layers, dst_v16, src_layers, src_v16) -> None:
     """blockwise_decode.py:336-355: overwrite an allocated slot with a fixed-slot block, in place."""
     for dst, src, dst_v, src_v in zip(dst_layers, src_layers, dst_v16, src_v16):
+        if hasattr(dst, "_host_counts"):
+            del dst._host_counts          # host copy of the class sizes the packer left: stale after the overwrite
         for name in _BANK_FIELDS:
             _copy_tensor_field(getattr(dst, name), getattr(src, name))
         _copy_tensor_field(dst_v, src_v)
