@@ -123,8 +123,14 @@ def _layer_counts(pl: PackedKVLayer, H_kv: int):
 # per tile of each V class, per dword of K row per tile, per work item (its set-up is a chain
 # of dependent loads).  Fitted to per-item timestamps of the kernel on MI355X, for G <= 4 (one
 # head group, 16 wavefronts) and for G = 5..8 (two head groups, 12 wavefronts).
-DEFAULT_COST = {"tile": (173.0, 172.0, 264.0, 492.0), "k_dword": 6.5, "item": 9900.0}
-DEFAULT_COST_TWO_HEAD_GROUPS = {"tile": (304.0, 310.0, 325.0, 413.0), "k_dword": 7.0, "item": 8800.0}
+# "group_speed": relative speed by workgroup index, cycled: workgroups are dealt round-robin to the
+# eight compute dies, and with identical work per group the odd dies finish ~2 % later than the even
+# ones on every MI355X measured (500-520 us spread by die on a 128k-context cache), so even groups
+# get 1 % more of the stream and odd ones 1 % less.
+GROUP_SPEED = (1.01, 0.99)
+DEFAULT_COST = {"tile": (173.0, 172.0, 264.0, 492.0), "k_dword": 6.5, "item": 9900.0, "group_speed": GROUP_SPEED}
+DEFAULT_COST_TWO_HEAD_GROUPS = {"tile": (304.0, 310.0, 325.0, 413.0), "k_dword": 7.0, "item": 8800.0,
+                                "group_speed": GROUP_SPEED}
 BYTES_COST = {"tile": (2048.0 + 256, 4096.0 + 256, 8192.0 + 256, 16384.0), "k_dword": 256.0, "item": 0.0}
 
 
@@ -152,7 +158,8 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     per_unit = unit_tiles.sum(axis=1)
     unit_start = np.concatenate([[0], np.cumsum(per_unit)]).astype(np.int64)
     total = int(unit_start[-1])
-    cost = _tile_costs(unit_tiles, unit_R, BYTES_COST if work_bytes is not None else (cost or DEFAULT_COST))
+    model_used = BYTES_COST if work_bytes is not None else (cost or DEFAULT_COST)
+    cost = _tile_costs(unit_tiles, unit_R, model_used)
     cum = np.cumsum(cost)
     if work_bytes is not None:
         # greedy runs inside each unit, closed when the running cost reaches work_bytes
@@ -169,8 +176,12 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
         cut_pts = np.unique(np.asarray(cuts, dtype=np.int64))
     else:
         n_groups = max(1, int(n_groups))
-        target = (float(cum[-1]) if total else 0.0) / n_groups
-        group_cuts = np.searchsorted(cum, target * np.arange(1, n_groups), side="left") + 1 if total else \
+        # equal cost per group, or shares proportional to a relative speed by group index
+        # (cost["group_speed"], cycled over the groups: workgroup i runs on compute die i mod 8)
+        speed = np.asarray((model_used or {}).get("group_speed", (1.0,)), dtype=np.float64)
+        share = speed[np.arange(n_groups) % len(speed)]
+        thresholds = (float(cum[-1]) if total else 0.0) * np.cumsum(share / share.sum())[:-1]
+        group_cuts = np.searchsorted(cum, thresholds, side="left") + 1 if total else \
             np.zeros(n_groups - 1, dtype=np.int64)
         group_cuts = np.minimum(np.concatenate([[0], group_cuts, [total]]).astype(np.int64), total)
         group_cuts = np.maximum.accumulate(group_cuts)
