@@ -348,6 +348,12 @@ int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride_h, int64
                      int G, int Q, int64_t T, int D, int causal, float *token_scores,
                      float *channel_scores, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* obkv_fast.py:889  the V-side token score of a prefill layer: out[h, t] = sum_i x[h, i, t] over the
+ * n_inner = q_per_kv * obs_window attention rows of KV head h (x of dtype code `dtype`, strides in
+ * elements, unit stride along t), accumulated in fp32 and rounded once to x's storage type, as fp32. */
+int rdkv_token_mass(const void *x, int dtype, int64_t stride_h, int64_t stride_i, int H, int n_inner,
+                    int64_t T, float *out, void *stream);
+
 /* ---- measurement helpers (no counterpart in the reference) --------------------------------
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)

@@ -337,3 +337,14 @@ def logical_layer_bits(v_bits: np.ndarray, k_bits: np.ndarray, head_dim: int) ->
     k = np.asarray(k_bits, dtype=np.int64)
     kept = (v > 0).sum(axis=1)
     return int(v.sum() * head_dim + (k.sum(axis=1) * kept).sum())
+
+
+def score_one_layer(aw: np.ndarray, q: np.ndarray, k: np.ndarray):
+    """obkv_fast.py:854-896.  ``aw [B, H_kv, G, W, T]``, ``q [B, H_kv, G, W, D]``, ``k [B, H_kv, T, D]``
+    -> (token ``[B, H_kv, T]`` = sum of the attention weights over (G, W), a value of aw's dtype
+    (:889 sums before ``.float()``), channel ``[B, H_kv, D]`` = mean_{G,W}(q^2) * mean_T(k^2) in fp32).
+    Textbook reductions; compared within a tolerance of one unit in the last place of aw's dtype."""
+    token = aw.astype(F32).sum(axis=(2, 3), dtype=F32).astype(aw.dtype).astype(F32)
+    qf, kf = q.astype(F32), k.astype(F32)
+    channel = (np.square(qf).mean(axis=(2, 3)) * np.square(kf).mean(axis=2)).astype(F32)
+    return token, channel

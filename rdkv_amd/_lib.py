@@ -68,6 +68,7 @@ SIGNATURES = {
     "rdkv_knapsack_rows": (I, [P, L, I, L, P, P, P, I, I, Dbl, P, I, L, P, P]),
     "rdkv_block_score_workspace_bytes": (L, [I, I, L, I]),
     "rdkv_block_score": (I, [P, I, L, L, P, I, L, L, I, I, I, L, I, I, P, P, P, L, P]),
+    "rdkv_token_mass": (I, [P, I, L, L, I, I, L, P, P]),
     "rdkv_probe_copy": (I, [P, P, L, P]),
     "rdkv_probe_read": (I, [P, L, L, P, P]),
     "rdkv_probe_read_stream": (I, [P, L, L, P, P]),

@@ -147,6 +147,19 @@ channel_score_kernel(const void *__restrict__ queries, int q_dtype, int64_t q_st
   }
 }
 
+// out[h, t] = sum over i of x[h, i, t], accumulated in fp32 in index order and rounded once to the
+// input's storage type (a library sum of a half-precision tensor is a half-precision value)
+__global__ void __launch_bounds__(256)
+token_mass_kernel(const void *__restrict__ x, int dtype, int64_t stride_h, int64_t stride_i, int n_inner, int T,
+                  float *__restrict__ out) {
+  const int h = blockIdx.y;
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  float s = 0.0f;
+  for (int i = 0; i < n_inner; ++i) s += rdkv_load_as_float(x, dtype, (int64_t)h * stride_h + (int64_t)i * stride_i + t);
+  out[(int64_t)h * T + t] = rdkv_round_to_dtype(s, dtype);
+}
+
 int q_tile_for(int64_t T, int D) {
   // logits [QB][T] + queries [QB][D] in at most 128 KiB of LDS
   int64_t qb = (128 * 1024 / 4) / (T + D);
@@ -194,6 +207,19 @@ RDKV_API int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride
   }
   hipLaunchKernelGGL(channel_score_kernel, dim3((unsigned)rdkv_cdiv(D, 64), H_kv), dim3(256), 0, s, queries, q_dtype,
                      q_stride_h, q_stride_q, keys, k_dtype, k_stride_h, k_stride_t, G, Q, (int)T, D, channel_scores);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_token_mass(const void *x, int dtype, int64_t stride_h, int64_t stride_i, int H, int n_inner,
+                             int64_t T, float *out, void *stream) {
+  const char *fn = "rdkv_token_mass";
+  RDKV_REQUIRE(H >= 0 && H <= 65535 && n_inner >= 0 && T >= 0 && T <= 0x7fffffffLL, "%s: bad shape", fn);
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2, "%s: unknown dtype", fn);
+  if (H == 0 || T == 0) return RDKV_OK;
+  RDKV_REQUIRE(out && (n_inner == 0 || x), "%s: null pointer", fn);
+  hipLaunchKernelGGL(token_mass_kernel, dim3((unsigned)rdkv_cdiv(T, 256), H), dim3(256), 0, (hipStream_t)stream, x,
+                     dtype, stride_h, stride_i, n_inner, (int)T, out);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

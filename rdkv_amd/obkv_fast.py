@@ -47,6 +47,39 @@ def apply_score_pooling(scores: Tensor, pool_type: str, kernel_size: int, paddin
     return out[0] if one_d else out
 
 
+def _score_one_layer(aw: Tensor, q: Tensor, o, v: Tensor, head_dim: int, v_score_type: str = "attn_linear",
+                     k: Optional[Tensor] = None, k_score_type: str = "think"):
+    """obkv_fast.py:854-896.  Scores of one prefill layer from the captured observation window:
+    ``aw [B, H_kv, q_per_kv, obs, T]`` attention weights, ``q [B, H_kv, q_per_kv, obs, D]``,
+    ``k [B, H_kv, T, D]`` (``o`` and ``v`` are part of the signature and unused).  Returns
+    ``(layer_token [B, H_kv, T], layer_channel [B, H_kv, D])`` fp32: the attention mass every key
+    received (summed in the weights' dtype, or in fp32 under ``OBKV_SCORE_FP32=1``) and the
+    ThinK channel score ``mean(q^2) * mean(k^2)``."""
+    import os
+    from .blockwise_decode import _channel_score
+    if v_score_type != "attn_linear":
+        raise ValueError(f"Unsupported v_score_type={v_score_type!r}; expected 'attn_linear'.")
+    if k_score_type != "think":
+        raise ValueError(f"Unsupported k_score_type={k_score_type!r}; expected 'think'.")
+    if k is None:
+        raise ValueError("k_score_type='think' requires the keys tensor (k=...).")
+    del o, v
+    dev = _lib.require_device(aw, q, k)
+    if os.environ.get("OBKV_SCORE_FP32", "0") == "1" or aw.dtype not in _lib.DTYPE_CODE:
+        aw = aw.float()
+    B, H_kv, G, W, T = (int(x) for x in aw.shape)
+    D = int(q.shape[-1])
+    rows = aw.reshape(B * H_kv, G * W, T)
+    if rows.stride(2) != 1:
+        rows = rows.contiguous()
+    token = torch.empty(B, H_kv, T, dtype=torch.float32, device=dev)
+    _lib.check(_lib.load().rdkv_token_mass(_lib.ptr(rows), _lib.DTYPE_CODE[rows.dtype], rows.stride(0), rows.stride(1),
+                                           B * H_kv, G * W, T, _lib.ptr(token), _lib.stream_of(dev)))
+    channel = torch.stack([_channel_score(q[b].reshape(H_kv * G, W, D), k[b:b + 1], num_kv_groups=G)
+                           for b in range(B)]) if B else torch.empty(0, H_kv, D, dtype=torch.float32, device=dev)
+    return token, channel
+
+
 def _allocate_k_bits_per_head(channel_scores: Tensor, k_avg: Union[float, Tensor], *, epsilon,
                               bit_options) -> Tensor:
     """obkv_fast.py:579-618: ``[H_kv, D]`` channel scores, a shared float budget or one per head;

@@ -245,3 +245,36 @@ def test_multi_layer_selection_equals_per_layer():
                 assert a.dtype == b.dtype and torch.equal(a, b), f.name
             else:
                 assert a == b, f.name
+
+
+@pytest.mark.parametrize("dtype,B", [(torch.float16, 1), (torch.bfloat16, 2), (torch.float32, 1)])
+def test_score_one_layer_matches_library_and_oracle(dtype, B, monkeypatch):
+    """The prefill scores (attention mass per key, ThinK channel score) against the tensor
+    expressions they stand for (obkv_fast.py:889-894 of the reference) and the oracle."""
+    H, G, W, T, D = 2, 4, 8, 300, 128
+    g = torch.Generator().manual_seed(77)
+    aw = torch.softmax(torch.randn(B, H, G, W, T, generator=g) * 2, dim=-1).to(dtype)
+    q = torch.randn(B, H, G, W, D, generator=g).to(dtype)
+    k = torch.randn(B, H, T, D, generator=g).to(dtype)
+    v = torch.randn(B, H, T, D, generator=g).to(dtype)
+    token, channel = obkv_fast._score_one_layer(aw.to(DEV), q.to(DEV), None, v.to(DEV), D, k=k.to(DEV))
+    assert token.dtype == torch.float32 and tuple(token.shape) == (B, H, T) and tuple(channel.shape) == (B, H, D)
+    exp_t = aw.sum(dim=(2, 3)).float()
+    exp_c = (q.float().square().mean(dim=(2, 3)) * k.float().square().mean(dim=2)).float()
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7, torch.float32: 2.0e-6}[dtype]
+    torch.testing.assert_close(token.cpu(), exp_t, rtol=ulp, atol=0)
+    torch.testing.assert_close(channel.cpu(), exp_c, rtol=2e-5, atol=1e-9)
+    np_of = lambda t: t.float().numpy().astype(np.float16 if dtype == torch.float16 else np.float32)
+    if dtype != torch.bfloat16:
+        o_t, o_c = S.score_one_layer(np_of(aw), np_of(q), np_of(k))
+        np.testing.assert_allclose(t2n(token), o_t, rtol=ulp, atol=0)
+        np.testing.assert_allclose(t2n(channel), o_c, rtol=2e-5, atol=1e-9)
+    # every window row spreads one unit of mass: the token scores of a head sum to G * W
+    np.testing.assert_allclose(t2n(token).sum(axis=2), np.full((B, H), G * W, F32), rtol=2e-3)
+    monkeypatch.setenv("OBKV_SCORE_FP32", "1")
+    token32, _ = obkv_fast._score_one_layer(aw.to(DEV), q.to(DEV), None, v.to(DEV), D, k=k.to(DEV))
+    torch.testing.assert_close(token32.cpu(), aw.float().sum(dim=(2, 3)), rtol=1e-5, atol=0)
+    with pytest.raises(ValueError):
+        obkv_fast._score_one_layer(aw.to(DEV), q.to(DEV), None, v.to(DEV), D, k=None)
+    with pytest.raises(ValueError):
+        obkv_fast._score_one_layer(aw.to(DEV), q.to(DEV), None, v.to(DEV), D, v_score_type="other", k=k.to(DEV))
