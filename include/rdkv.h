@@ -107,7 +107,8 @@ int rdkv_dequant_f16(const uint8_t *packed, int64_t rows, int n_cols_unpacked, i
 /* out[hq, t] = (sum_c code[hkv,t,c] * q[hq, perm[c]] * s[hkv,c] - sum_c z*q*s) / sqrt(128),
  * t < T_eff, reading the reference's padded layout.  q: [H_q,128] of q_dtype.
  * perm: int64 [H_q or 1, D_padded] (perm_stride_h == 0 for the shared permutation).
- * K2/K4/K8 may be NULL when their segment is empty. */
+ * K2/K4/K8 may be NULL when their segment is empty.  Rows stored back to back (token stride
+ * = row bytes) are staged through LDS with wide loads; other strides are read in place. */
 int rdkv_k_qk_dot(const void *q, int q_dtype, int64_t q_stride_h, int H_q, int H_kv,
                   const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
                   const uint8_t *K4, int64_t k4_stride_h, int64_t k4_stride_t,
@@ -131,6 +132,8 @@ int rdkv_softmax_rows(const float *scores_old, int64_t so_stride_h, const float 
  * (kernel math triton_v_kernel.py:638-750).  seg_bounds_dev: int32 [H_kv,3] per-head
  * counts read on the device, or NULL to use the host counts N2,N4,N8 for every head.
  * V16/n_v16_dev may be NULL (no zone B).  Zone-B weights are read at column max_T_v + t.
+ * The V segments are read with 16-byte loads: their base addresses and head strides must be
+ * multiples of 16 bytes (any view that starts on a token row is), else RDKV_EINVAL.
  * workspace: rdkv_v_weighted_sum_workspace_bytes(H_q) bytes. */
 int64_t rdkv_v_weighted_sum_workspace_bytes(int H_q);
 int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, int H_kv,

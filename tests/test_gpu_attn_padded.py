@@ -120,3 +120,30 @@ def test_config_shaped_attention_vs_oracle(cfg_idx, ctx):
     raw, w, out = _attend_padded(pl, nvo, q.to(DEV))
     attn_close(t2n(w), exp_w, "weights")
     attn_close(t2n(out), exp_out, "out")
+
+
+def test_k_scores_strided_rows_match_dense_rows():
+    """K rows that are views into wider buffers (token stride > row bytes) take the kernel that
+    reads rows in place; densely stored rows the one that stages them through LDS.  Same scores
+    up to the order in which the zero-point bias is summed."""
+    import dataclasses
+    cfg = synth.scaled(synth.CONFIGS[1], context=1100, layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, q = synth.layer_data(cfg, 0, DEV, outliers=oc)
+    pl, _ = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+    T = pl.T_eff_k
+    dense = kk.k_mixed_qk_dot(q, pl, T)
+
+    def widened(t, extra):
+        if t is None or t.numel() == 0:
+            return t
+        buf = torch.full(t.shape[:-1] + (t.shape[-1] + extra,), 0xA5, dtype=t.dtype, device=t.device)
+        buf[..., :t.shape[-1]] = t
+        return buf[..., :t.shape[-1]]
+
+    sv = dataclasses.replace(pl, K_2bit=widened(pl.K_2bit, 3), K_4bit=widened(pl.K_4bit, 5),
+                             K_8bit=widened(pl.K_8bit, 1))
+    assert any(getattr(sv, n) is not None and getattr(sv, n).numel() and not getattr(sv, n).is_contiguous()
+               for n in ("K_2bit", "K_4bit", "K_8bit"))
+    strided = kk.k_mixed_qk_dot(q, sv, T)
+    torch.testing.assert_close(strided, dense, rtol=0, atol=2e-5)
