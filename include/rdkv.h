@@ -147,6 +147,28 @@ int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, int H_kv,
                         float *out, int64_t out_stride_h,
                         void *workspace, int64_t workspace_bytes, void *stream);
 
+/* ---- fast_decode.py : the per-token operations around the attention ------- */
+/* fast_decode.py:628-633 (_rms_norm) with the residual add in front of it (:1786, :1808):
+ * r = x + delta rounded to `dtype` (delta NULL: r = x); residual_out (NULL, or x itself) <- r;
+ * norm_out <- weight * (r * rsqrt(mean(r^2) + eps)) in fp32, rounded to `dtype`.  rows x dim
+ * elements, row strides in elements; weight: dim values of w_dtype. */
+int rdkv_add_rms_norm(const void *x, int64_t x_stride_row, const void *delta, int64_t delta_stride_row,
+                      const void *weight, int w_dtype, float eps, int rows, int dim, int dtype,
+                      void *residual_out, int64_t residual_stride_row, void *norm_out,
+                      int64_t norm_stride_row, void *stream);
+/* fast_decode.py:1690 + :1722-1724: rotate the new token's k [H_kv, D] as rdkv_rope would
+ * (rounded to `dtype`) and write [k | v] widened to fp32 as row row_dev[0] of the zone C buffer
+ * new_kv (head h, token t at new_kv + h*new_stride_head + t*new_stride_tok, 2*D floats).  The
+ * row index is read on the device, so a captured graph can advance it; a row outside
+ * [0, capacity) writes nothing. */
+int rdkv_rope_append_kv(const void *k, int64_t k_stride_h, const void *v, int64_t v_stride_h, int H_kv,
+                        int D, int dtype, const void *cos_half, const void *sin_half, int cs_dtype,
+                        float *new_kv, int64_t new_stride_head, int64_t new_stride_tok,
+                        const int64_t *row_dev, int64_t capacity, void *stream);
+/* fast_decode.py:1803: out[i] = silu(gate[i]) * up[i], the activation rounded to `dtype` before
+ * the product as the two tensor operations do. */
+int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtype, void *out, void *stream);
+
 /* ---- triton_rope.py : fused_rope (:86-108) -------------------------------- */
 /* Half-split rotary embedding of one decode step, in place: for every head of q [H_q, D] and
  * k [H_kv, D] (dtype code `dtype`, head strides in elements) and i < D/2:

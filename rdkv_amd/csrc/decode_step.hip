@@ -1,0 +1,125 @@
+// Small per-token operations of the decode loop around the attention (reference:
+// obkv_accel/fast_decode.py:628-633 inline RMSNorm, :1640-1690 residual adds, rotary embedding
+// and the zone C append, :1795-1806 the MLP activation), each as one launch instead of the
+// five to eight elementwise launches the tensor expressions take.  Arithmetic follows those
+// expressions: fp32 inside, one rounding to the storage type where the expression stores one.
+#include "rdkv_common.h"
+#include "rope_device.h"
+
+namespace {
+
+// One workgroup per row.  r = x (+ delta, rounded to the storage type like the tensor add);
+// norm = weight * (r * rsqrt(mean(r^2) + eps)) rounded to the storage type.
+__global__ void __launch_bounds__(256)
+add_rms_norm_kernel(const void *x, int64_t x_stride, const void *__restrict__ delta,
+                    int64_t delta_stride, const void *__restrict__ weight, int w_dtype, float eps, int dim,
+                    int dtype, void *residual_out, int64_t res_stride, void *__restrict__ norm_out,
+                    int64_t norm_stride) {
+  __shared__ float s_part[4];
+  const int row = blockIdx.x;
+  const int64_t xo = row * x_stride, dlo = row * delta_stride, ro = row * res_stride, no = row * norm_stride;
+  float ss = 0.0f;
+  for (int i = threadIdx.x; i < dim; i += 256) {
+    float r = rdkv_load_as_float(x, dtype, xo + i);
+    if (delta) r = rdkv_round_to_dtype(r + rdkv_load_as_float(delta, dtype, dlo + i), dtype);
+    if (residual_out) rdkv_store_from_float(residual_out, dtype, ro + i, r);
+    ss += r * r;
+  }
+  ss = rdkv_wave_sum(ss);
+  if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
+  __syncthreads();
+  const float mean = (s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)dim;
+  const float rs = rsqrtf(mean + eps);
+  for (int i = threadIdx.x; i < dim; i += 256) {
+    float r;
+    if (residual_out) r = rdkv_load_as_float(residual_out, dtype, ro + i);   // this thread wrote it
+    else {
+      r = rdkv_load_as_float(x, dtype, xo + i);
+      if (delta) r = rdkv_round_to_dtype(r + rdkv_load_as_float(delta, dtype, dlo + i), dtype);
+    }
+    rdkv_store_from_float(norm_out, dtype, no + i, rdkv_load_as_float(weight, w_dtype, i) * (r * rs));
+  }
+}
+
+// One wavefront per KV head: k rotated (rounded to the storage type, as the in-place rotation
+// stores it) and v, both widened to fp32, written as the row [K | V] of the zone C buffer that the
+// device-held index names.  A row index outside the buffer writes nothing.
+__global__ void __launch_bounds__(64)
+rope_append_kv_kernel(const void *__restrict__ k, int64_t k_stride_h, const void *__restrict__ v,
+                      int64_t v_stride_h, int half_d, int dtype, const void *__restrict__ cos_half,
+                      const void *__restrict__ sin_half, int cs_dtype, float *__restrict__ new_kv,
+                      int64_t new_stride_head, int64_t new_stride_tok, const int64_t *__restrict__ row_dev,
+                      int64_t capacity) {
+  const int64_t row = row_dev[0];
+  if (row < 0 || row >= capacity) return;
+  const int head = blockIdx.x;
+  float *dst = new_kv + head * new_stride_head + row * new_stride_tok;
+  const int64_t ko = head * k_stride_h, vo = head * v_stride_h;
+  for (int i = threadIdx.x; i < half_d; i += 64) {
+    const float lo = rdkv_load_as_float(k, dtype, ko + i), hi = rdkv_load_as_float(k, dtype, ko + i + half_d);
+    const float c = rdkv_load_as_float(cos_half, cs_dtype, i), s = rdkv_load_as_float(sin_half, cs_dtype, i);
+    float out_lo, out_hi;
+    rdkv_rope_pair(lo, hi, c, s, out_lo, out_hi);
+    dst[i] = rdkv_round_to_dtype(out_lo, dtype);
+    dst[i + half_d] = rdkv_round_to_dtype(out_hi, dtype);
+    dst[2 * half_d + i] = rdkv_load_as_float(v, dtype, vo + i);
+    dst[3 * half_d + i] = rdkv_load_as_float(v, dtype, vo + i + half_d);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+silu_mul_kernel(const void *__restrict__ gate, const void *__restrict__ up, int64_t n, int dtype,
+                void *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float g = rdkv_load_as_float(gate, dtype, i);
+  const float act = rdkv_round_to_dtype(g / (1.0f + expf(-g)), dtype);
+  rdkv_store_from_float(out, dtype, i, act * rdkv_load_as_float(up, dtype, i));
+}
+
+}  // namespace
+
+RDKV_API int rdkv_add_rms_norm(const void *x, int64_t x_stride_row, const void *delta, int64_t delta_stride_row,
+                               const void *weight, int w_dtype, float eps, int rows, int dim, int dtype,
+                               void *residual_out, int64_t residual_stride_row, void *norm_out,
+                               int64_t norm_stride_row, void *stream) {
+  RDKV_REQUIRE(rows >= 0 && dim > 0, "rdkv_add_rms_norm: bad shape rows=%d dim=%d", rows, dim);
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && w_dtype >= 0 && w_dtype <= 2, "rdkv_add_rms_norm: unknown dtype");
+  if (rows == 0) return RDKV_OK;
+  RDKV_REQUIRE(x && weight && norm_out, "rdkv_add_rms_norm: null pointer");
+  RDKV_REQUIRE(norm_out != x && norm_out != residual_out, "rdkv_add_rms_norm: norm_out must not alias the input");
+  hipLaunchKernelGGL(add_rms_norm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, x_stride_row, delta,
+                     delta_stride_row, weight, w_dtype, eps, dim, dtype, residual_out, residual_stride_row,
+                     norm_out, norm_stride_row);
+  RDKV_CHECK_LAUNCH("rdkv_add_rms_norm");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_rope_append_kv(const void *k, int64_t k_stride_h, const void *v, int64_t v_stride_h, int H_kv,
+                                 int D, int dtype, const void *cos_half, const void *sin_half, int cs_dtype,
+                                 float *new_kv, int64_t new_stride_head, int64_t new_stride_tok,
+                                 const int64_t *row_dev, int64_t capacity, void *stream) {
+  RDKV_REQUIRE(H_kv >= 0 && D > 0 && D % 2 == 0, "rdkv_rope_append_kv: bad shape H_kv=%d D=%d", H_kv, D);
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && cs_dtype >= 0 && cs_dtype <= 2, "rdkv_rope_append_kv: unknown dtype");
+  if (H_kv == 0) return RDKV_OK;
+  RDKV_REQUIRE(k && v && cos_half && sin_half && new_kv && row_dev, "rdkv_rope_append_kv: null pointer");
+  RDKV_REQUIRE(capacity >= 0 && new_stride_tok >= 2 * D && new_stride_head >= 0,
+               "rdkv_rope_append_kv: bad zone C buffer shape");
+  hipLaunchKernelGGL(rope_append_kv_kernel, dim3(H_kv), dim3(64), 0, (hipStream_t)stream, k, k_stride_h, v,
+                     v_stride_h, D / 2, dtype, cos_half, sin_half, cs_dtype, new_kv, new_stride_head,
+                     new_stride_tok, row_dev, capacity);
+  RDKV_CHECK_LAUNCH("rdkv_rope_append_kv");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtype, void *out, void *stream) {
+  RDKV_REQUIRE(n >= 0 && dtype >= 0 && dtype <= 2, "rdkv_silu_mul: bad arguments");
+  if (n == 0) return RDKV_OK;
+  RDKV_REQUIRE(gate && up && out, "rdkv_silu_mul: null pointer");
+  const int64_t blocks = rdkv_cdiv(n, 256);
+  RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_silu_mul: too many elements");
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, gate, up, n, dtype,
+                     out);
+  RDKV_CHECK_LAUNCH("rdkv_silu_mul");
+  return RDKV_OK;
+}

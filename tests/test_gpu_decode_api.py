@@ -130,10 +130,6 @@ def test_retired_hook_names_raise():
         decode_hook.make_packed_decode_forward(0, None)
     with pytest.raises(NotImplementedError):
         decode_hook.greedy_decode_packed(None, None, None, 1, [], None, 0)
-    with pytest.raises(NotImplementedError):
-        fast_decode.greedy_decode_fast(None, None, None, 1, [], None, 0)
-    with pytest.raises(NotImplementedError):
-        fast_decode.pre_extract_weights(None)
     from rdkv_amd import triton_k_kernel as tk
     ph = tk._ensure_tensor(None, 3, 0, DEV)
     assert ph.shape == (3, 1, 1) and ph.dtype == torch.uint8 and int(ph.sum()) == 0

@@ -1,0 +1,250 @@
+"""The decode loop (``fast_decode.greedy_decode_fast``) on a small random-weight Llama: per-step
+logits against (1) a plain fp32 restatement of the model step whose attention is the oracle's
+three-zone attention over the same packed bytes, and (2) the model's own ``forward`` over its
+dense prompt cache (loose: K is quantized to 8 bits there); eager and HIP-graph runs must give
+the same tokens; observers, EOS and error paths follow fast_decode.py:731-1137."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import rdkv_oracle as O
+from rdkv_amd import fast_decode, packing
+from tests.gpu_util import DEV, require_gpu, t2n
+
+pytestmark = pytest.mark.gpu
+
+T_PROMPT, H_Q, H_KV, D, HID, LAYERS, VOCAB = 300, 4, 2, 128, 512, 2, 1000
+
+
+def _build_setup():
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg = LlamaConfig(hidden_size=HID, intermediate_size=1024, num_hidden_layers=LAYERS, num_attention_heads=H_Q,
+                      num_key_value_heads=H_KV, head_dim=D, vocab_size=VOCAB, max_position_embeddings=4096,
+                      rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False)
+    torch.manual_seed(1234)
+    model = LlamaForCausalLM(cfg)
+    with torch.no_grad():           # wider weights than the default init so that logits are not flat
+        for p in model.parameters():
+            if p.dim() == 2:
+                p.mul_(3.0)
+    model = model.half().to(DEV).eval()
+    g = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, VOCAB, (1, T_PROMPT), generator=g).to(DEV)
+    with torch.no_grad():
+        pre = model(prompt, use_cache=True)
+    kv = []
+    for i in range(LAYERS):
+        layer = pre.past_key_values.layers[i]
+        kv.append((layer.keys.contiguous(), layer.values.contiguous()))
+    return model, prompt, pre, kv
+
+
+@pytest.fixture(scope="module")
+def setup():
+    require_gpu()
+    return _build_setup()
+
+
+def _pack(kv, v_bits, k_bits):
+    layers, v16 = [], []
+    for K, V in kv:
+        pl, nvo = packing.pack_layer_per_head(K, V, v_bits, k_bits, H_Q // H_KV)
+        layers.append(pl)
+        v16.append(nvo)
+    return packing.TriZoneCache(tuple(layers), v16, [None] * len(kv), [None] * len(kv), T_PROMPT)
+
+
+def _mixed_bits(seed):
+    g = torch.Generator().manual_seed(seed)
+    v_bits = torch.tensor([0, 2, 4, 8, 16])[torch.randint(0, 5, (H_KV, T_PROMPT), generator=g)]
+    k_bits = torch.tensor([0, 2, 4, 8])[torch.randint(0, 4, (H_KV, D), generator=g)]
+    return v_bits, k_bits
+
+
+def _rms(x, w, eps):
+    return w * (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps))
+
+
+def _reference_logits(model, kv, v_bits, k_bits, tokens, position0):
+    """fp32 CPU step of the same model, attention = oracle over oracle-packed layers.  For an
+    fp16 model every intermediate is rounded to fp16 where the GPU loop stores one."""
+    cfg = model.config
+    if next(model.parameters()).dtype == torch.float16:
+        r = lambda t: t.half().float()
+    else:
+        r = lambda t: t
+    sd = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    ora = [O.pack_layer_per_head(t2n(K), t2n(V), v_bits.numpy(), k_bits.numpy(), H_Q // H_KV) for K, V in kv]
+    # the module's own table: casting the model to fp16 rounded it, and prefill used it that way
+    inv_freq = model.model.rotary_emb.inv_freq.detach().float().cpu()
+    K_new = [np.zeros((H_KV, 0, D), np.float32) for _ in range(LAYERS)]
+    V_new = [np.zeros((H_KV, 0, D), np.float32) for _ in range(LAYERS)]
+    out = []
+    for step, tok in enumerate(tokens):
+        ang = (position0 + step) * inv_freq
+        cos, sin = r(torch.cos(ang)), r(torch.sin(ang))      # the model hands out tables in its dtype
+
+        def rope(x):       # half-split rotation, rounded to the model dtype like the in-place kernel
+            lo, hi = x[:, :D // 2], x[:, D // 2:]
+            return r(torch.cat([lo * cos - hi * sin, hi * cos + lo * sin], -1))
+
+        h = sd["model.embed_tokens.weight"][tok][None]
+        for i in range(LAYERS):
+            p = f"model.layers.{i}."
+            x = r(_rms(h, sd[p + "input_layernorm.weight"], cfg.rms_norm_eps))
+            q = r(x @ sd[p + "self_attn.q_proj.weight"].T).view(H_Q, D)
+            k = r(x @ sd[p + "self_attn.k_proj.weight"].T).view(H_KV, D)
+            v = r(x @ sd[p + "self_attn.v_proj.weight"].T).view(H_KV, D)
+            q, k = rope(q), rope(k)
+            K_new[i] = np.concatenate([K_new[i], k.numpy()[:, None]], 1)
+            V_new[i] = np.concatenate([V_new[i], v.numpy()[:, None]], 1)
+            a = O.trizone_attention_ref(q.numpy(), ora[i][0], ora[i][1], K_new[i], V_new[i])
+            a = r(torch.from_numpy(np.asarray(a, np.float32))).view(1, H_Q * D)
+            h = r(h + r(a @ sd[p + "self_attn.o_proj.weight"].T))
+            x = r(_rms(h, sd[p + "post_attention_layernorm.weight"], cfg.rms_norm_eps))
+            gate = r(x @ sd[p + "mlp.gate_proj.weight"].T)
+            up = r(x @ sd[p + "mlp.up_proj.weight"].T)
+            act = r(r(torch.nn.functional.silu(gate)) * up)
+            h = r(h + r(act @ sd[p + "mlp.down_proj.weight"].T))
+        h = r(_rms(h, sd["model.norm.weight"], cfg.rms_norm_eps))
+        out.append((h @ sd["lm_head.weight"].T)[0])
+    return out
+
+
+@pytest.mark.parametrize("fp32_model", [True, False])
+def test_decode_loop_matches_restated_model_over_oracle_attention(setup, fp32_model):
+    """With fp32 weights and activations the only differences left are summation orders and the
+    oracle's fp16 rounding of dequantized K / V: 2e-3 of the largest logit.  The fp16 model adds
+    its per-operation roundings, which the restatement follows only approximately: 5e-2."""
+    model, prompt, pre, kv = setup
+    if fp32_model:
+        import copy
+        model = copy.deepcopy(model).float()
+    v_bits, k_bits = _mixed_bits(11)
+    cache = _pack(kv, v_bits, k_bits)
+    first = pre.logits[0, -1]
+    tol = 2e-3 if fp32_model else 5e-2
+    ids, logits = fast_decode.greedy_decode_fast(model, cache, first, 6, [], torch.device(DEV), T_PROMPT,
+                                                 return_logits=True)
+    assert len(ids) == 6 and len(logits) == 6 and ids[0] == int(first.argmax())
+    ref = _reference_logits(model, kv, v_bits, k_bits, ids, T_PROMPT)
+    for step, (got, exp) in enumerate(zip(logits, ref)):
+        got = got[0]
+        scale = float(exp.abs().max())
+        err = float((got - exp).abs().max())
+        assert err <= tol * scale, f"step {step}: logits off by {err} (largest logit {scale})"
+        if step + 1 < len(ids):
+            assert ids[step + 1] == int(got.argmax())
+
+
+def test_decode_loop_tracks_model_forward(setup):
+    """All V kept as fp16, all K channels at 8 bits: the packed cache is the dense one up to the
+    K quantization, so the loop must follow ``model.forward`` over the dense cache closely."""
+    model, prompt, pre, kv = setup
+    v_bits = torch.full((H_KV, T_PROMPT), 16)
+    k_bits = torch.full((H_KV, D), 8)
+    cache = _pack(kv, v_bits, k_bits)
+    first = pre.logits[0, -1]
+    ids, logits = fast_decode.greedy_decode_fast(model, cache, first, 4, [], torch.device(DEV), T_PROMPT,
+                                                 return_logits=True)
+    with torch.no_grad():
+        again = model(prompt, use_cache=True)
+        pkv = again.past_key_values
+        for step, tok in enumerate(ids):
+            o = model(torch.tensor([[tok]], device=DEV), past_key_values=pkv, use_cache=True)
+            pkv = o.past_key_values
+            exp = o.logits[0, -1].float().cpu()
+            got = logits[step][0]
+            cos = float(torch.nn.functional.cosine_similarity(got, exp, dim=0))
+            assert cos > 0.999, f"step {step}: cosine {cos}"
+            assert float((got - exp).abs().max()) <= 0.05 * float(exp.abs().max())
+
+
+def test_graph_replay_gives_the_eager_tokens(setup):
+    model, prompt, pre, kv = setup
+    v_bits, k_bits = _mixed_bits(12)
+    first = pre.logits[0, -1]
+    eager = fast_decode.greedy_decode_fast(model, _pack(kv, v_bits, k_bits), first, 24, [], torch.device(DEV),
+                                           T_PROMPT)
+    cache = _pack(kv, v_bits, k_bits)
+    graphed = fast_decode.greedy_decode_fast(model, cache, first, 24, [], torch.device(DEV), T_PROMPT,
+                                             use_cuda_graph=True)
+    assert graphed == eager and len(eager) == 24
+    # a second run over the same cache object reuses its streaming caches and zone C buffers
+    torch.cuda.synchronize()
+    assert fast_decode.greedy_decode_fast(model, cache, first, 24, [], torch.device(DEV), T_PROMPT,
+                                          use_cuda_graph=True) == eager
+
+
+def test_observers_eos_and_errors(setup):
+    model, prompt, pre, kv = setup
+    v_bits, k_bits = _mixed_bits(13)
+    cache = _pack(kv, v_bits, k_bits)
+    first = pre.logits[0, -1]
+    dev = torch.device(DEV)
+    ids = fast_decode.greedy_decode_fast(model, cache, first, 5, [], dev, T_PROMPT)
+    seen, hid = [], []
+    hidden0 = torch.zeros(1, HID, device=DEV, dtype=torch.float16)
+    out = fast_decode.greedy_decode_fast(
+        model, cache, first, 5, [ids[2]], dev, T_PROMPT, next_token_hidden=hidden0,
+        logits_observer=lambda s, lg, t, e: seen.append((s, tuple(lg.shape), t, e)),
+        hidden_observer=lambda s, hh, t, e: hid.append((s, tuple(hh.shape), t, e)))
+    stop = ids.index(ids[2])           # the loop ends at the first EOS token, which is not returned
+    assert out == ids[:stop]
+    assert [s[0] for s in seen] == list(range(stop + 1)) and seen[-1][3] and not any(s[3] for s in seen[:-1])
+    assert [s[2] for s in seen] == ids[:stop + 1]
+    assert all(s[1] == (1, VOCAB) for s in seen) and all(h_[1] == (1, HID) for h_ in hid)
+    with pytest.raises(NotImplementedError):
+        fast_decode.greedy_decode_fast(model, cache, first, 2, [], dev, T_PROMPT, use_cuda_graph=True,
+                                       return_logits=True)
+    with pytest.raises(ValueError):
+        fast_decode.greedy_decode_fast(model, cache, first, 2, [], dev, T_PROMPT, hidden_observer=lambda *a: None)
+    W = fast_decode.pre_extract_weights(model)
+    assert W is fast_decode.pre_extract_weights(model) and W.num_layers == LAYERS and W.num_kv_groups == H_Q // H_KV
+    assert W.layers[0].qkv_split_sizes == (H_Q * D, H_KV * D, H_KV * D) and W.layers[0].qkv_bias is None
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_step_kernels_match_tensor_expressions(dtype):
+    """The one-launch forms against the tensor expressions of fast_decode.py:628-633, 1690,
+    1722-1724, 1786, 1803 (one unit in the last place where a sum is taken in another order)."""
+    require_gpu()
+    from rdkv_amd.triton_rope import fused_rope
+    g = torch.Generator(device=DEV).manual_seed(5)
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7, torch.float32: 2.0 ** -22}[dtype]
+    for rows, dim in ((1, 4096), (4, 128), (3, 1000)):
+        x = torch.randn(rows, dim, generator=g, device=DEV).to(dtype)
+        d = torch.randn(rows, dim, generator=g, device=DEV).to(dtype)
+        w = (1.0 + 0.1 * torch.randn(dim, generator=g, device=DEV)).to(dtype)
+
+        def expr(t):
+            tf = t.float()
+            return (w * (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + 1e-5))).to(dtype)
+
+        got = fast_decode._rms_norm(x, w, 1e-5)
+        torch.testing.assert_close(got.float(), expr(x).float(), rtol=2 * ulp, atol=1e-6)
+        res = x.clone()
+        got = fast_decode._rms_norm(res, w, 1e-5, delta=d, residual_out=res)      # in place on the residual
+        assert torch.equal(res, x + d)
+        torch.testing.assert_close(got.float(), expr(x + d).float(), rtol=2 * ulp, atol=1e-6)
+    gate = 3 * torch.randn(1, 1, 14336, generator=g, device=DEV).to(dtype)
+    up = torch.randn(1, 1, 14336, generator=g, device=DEV).to(dtype)
+    both = torch.cat([gate, up], -1)
+    got = fast_decode._silu_mul(both[..., :14336], both[..., 14336:])
+    exp = torch.nn.functional.silu(gate) * up
+    torch.testing.assert_close(got.float(), exp.float(), rtol=2 * ulp, atol=1e-6)
+    # rotate + append against the in-place rotation followed by the tensor copy
+    k = torch.randn(8, 128, generator=g, device=DEV).to(dtype)
+    v = torch.randn(8, 128, generator=g, device=DEV).to(dtype)
+    cs = torch.rand(64, generator=g, device=DEV).to(dtype)
+    sn = torch.rand(64, generator=g, device=DEV).to(dtype)
+    buf = torch.full((8, 5, 256), 7.0, device=DEV)
+    row = torch.tensor([3], device=DEV)
+    fast_decode._rope_append_kv(k, v, cs, sn, buf, row)
+    q_dummy = torch.zeros(8, 128, device=DEV, dtype=dtype)
+    k_rot = k.clone()
+    fused_rope(q_dummy, k_rot, cs, sn)
+    assert torch.equal(buf[:, 3], torch.cat([k_rot, v], -1).float())
+    assert float((buf[:, [0, 1, 2, 4]] - 7.0).abs().max()) == 0.0
+    fast_decode._rope_append_kv(k, v, cs, sn, buf, torch.tensor([5], device=DEV))     # outside: nothing written
+    assert float((buf[:, [0, 1, 2, 4]] - 7.0).abs().max()) == 0.0
