@@ -758,11 +758,16 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
 // Merge of a unit's partials followed by the attention over its decode-appended tokens
 // (zone C: fp32 K/V rows that are not part of the packed cache), the exact softmax over the
 // union (fast_decode.py:1719-1735, 1777-1784): the zones A+B result enters as one pseudo-token
-// of weight exp(lse_ab) and value out_ab; the new tokens are folded in 64 at a time with a
-// running maximum.  Natural-log domain, fp32 throughout, q scaled by 1/sqrt(D) first as the
-// reference does.
+// of weight exp(lse_ab) and value out_ab.  The new tokens are taken 64 at a time, one chunk per
+// wavefront (chunk c by wavefront c mod 8): a lane scores its own token (its K row in 16-byte
+// loads against the query group in LDS), the wavefront keeps a running maximum, sum and 128
+// accumulators per head (lane = two channels, weights passed lane to lane), and the eight
+// wavefront states and the A+B state are combined once at the end, in a fixed order.  No
+// workgroup barrier inside the token loop.  Natural-log domain, fp32 throughout, q scaled by
+// 1/sqrt(D) first as the reference does.
 constexpr int kZcChunk = 64;
-__global__ void __launch_bounds__(256)
+constexpr int kZcWaves = 8;
+__global__ void __launch_bounds__(64 * kZcWaves)
 merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride,
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
@@ -770,19 +775,21 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
                     int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
                     float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
-  __shared__ float acc_ab[8 * kD];      // normalized zones A+B output, later unused
-  __shared__ float qz[8][kD];           // q / sqrt(D)
-  __shared__ float sc[8][kZcChunk];     // scores, then weights, of the current chunk
-  __shared__ float m_run[8], l_run[8], f_old[8], lse_ab[8];
+  __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
+  __shared__ __align__(16) float qz[8][kD];        // q / sqrt(D)
+  __shared__ float w_m[kZcWaves][8], w_l[kZcWaves][8];
+  __shared__ float w_acc[kZcWaves][8][kD];
+  __shared__ float lse_ab[8];
+  constexpr int kThreads = 64 * kZcWaves;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const RdkvUnit *u = units + blockIdx.x;
   if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   const int q_row = u->q_row;
   const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
-  merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, 256, scratch, acc_ab,
-             lse_ab);
+  merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, kThreads, scratch,
+             acc_ab, lse_ab);
   const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
-  for (int i = tid; i < G * kD; i += 256) {
+  for (int i = tid; i < G * kD; i += kThreads) {
     const int c = i & 127;
     const int64_t row = (int64_t)(q_row + (i >> 7)) * q_stride;
     float v = load_qv(q, q_dtype, row + c);
@@ -798,65 +805,114 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
     qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
   }
   __syncthreads();
-  if (tid < G) {
-    m_run[tid] = lse_ab[tid];
-    l_run[tid] = lse_ab[tid] == -INFINITY ? 0.0f : 1.0f;
-  }
-  // each thread owns the outputs i = tid + 256*k (head i>>7, channel i&127)
-  float acc[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) acc[k] = tid + 256 * k < G * kD ? acc_ab[tid + 256 * k] : 0.0f;
+
   const float *kn = k_new + (int64_t)kv_row * new_stride_unit;
   const float *vn = v_new + (int64_t)kv_row * new_stride_unit;
-  for (int t0 = 0; t0 < n_new; t0 += kZcChunk) {
-    const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
-    __syncthreads();
-    // scores: one wavefront per token, lanes over the channels
-    for (int t = wave; t < nt; t += 4) {
-      const float *kr = kn + (int64_t)(t0 + t) * new_stride_tok;
-      const float k0 = kr[lane], k1 = kr[lane + 64];
-      for (int h = 0; h < G; ++h) {
-        const float s = rdkv_wave_sum(qz[h][lane] * k0 + qz[h][lane + 64] * k1);
-        if (lane == 0) sc[h][t] = s;
-      }
-    }
-    __syncthreads();
-    if (tid < G) {
-      float cm = -INFINITY;
-      for (int t = 0; t < nt; ++t) cm = fmaxf(cm, sc[tid][t]);
-      const float m_new = fmaxf(m_run[tid], cm);
-      f_old[tid] = m_run[tid] == -INFINITY ? 0.0f : expf(m_run[tid] - m_new);
-      float ls = 0.0f;
-      for (int t = 0; t < nt; ++t) {
-        const float w = expf(sc[tid][t] - m_new);
-        sc[tid][t] = w;
-        ls += w;
-      }
-      l_run[tid] = l_run[tid] * f_old[tid] + ls;
-      m_run[tid] = m_new;
-    }
-    __syncthreads();
+  float m_run[8], l_run[8], acc[8][2];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int i = tid + 256 * k;
-      if (i < G * kD) {
-        const int h = i >> 7, d = i & 127;
-        float a = acc[k] * f_old[h];
-        for (int t = 0; t < nt; ++t) a += sc[h][t] * vn[(int64_t)(t0 + t) * new_stride_tok + d];
-        acc[k] = a;
+  for (int h = 0; h < 8; ++h) {
+    m_run[h] = -INFINITY;
+    l_run[h] = 0.0f;
+    acc[h][0] = acc[h][1] = 0.0f;
+  }
+  for (int t0 = wave * kZcChunk; t0 < n_new; t0 += kZcWaves * kZcChunk) {
+    const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
+    const bool valid = lane < nt;
+    // scores of this lane's token against the G query heads
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) s[h] = 0.0f;
+    const float4 *kr = reinterpret_cast<const float4 *>(kn + (int64_t)(t0 + (valid ? lane : 0)) * new_stride_tok);
+#pragma unroll 1
+    for (int c0 = 0; c0 < kD / 4; c0 += 8) {
+      float4 kv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) kv[e] = kr[c0 + e];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+#pragma unroll
+        for (int h = 0; h < 8; ++h) {
+          if (h < G) {
+            const float4 qv = reinterpret_cast<const float4 *>(qz[h])[c0 + e];
+            s[h] += kv[e].x * qv.x + kv[e].y * qv.y + kv[e].z * qv.z + kv[e].w * qv.w;
+          }
+        }
       }
+    }
+    float wt[8];
+#pragma unroll
+    for (int h = 0; h < 8; ++h) {
+      wt[h] = 0.0f;
+      if (h < G) {
+        const float sh = valid ? s[h] : -INFINITY;
+        const float m_new = fmaxf(m_run[h], rdkv_wave_max(sh));     // finite: the chunk has a token
+        const float f = m_run[h] == -INFINITY ? 0.0f : expf(m_run[h] - m_new);
+        wt[h] = valid ? expf(sh - m_new) : 0.0f;
+        l_run[h] = l_run[h] * f + rdkv_wave_sum(wt[h]);
+        acc[h][0] *= f;
+        acc[h][1] *= f;
+        m_run[h] = m_new;
+      }
+    }
+    // values: lane = channels lane and lane + 64, the weight of token tt comes from lane tt
+    const float *vr = vn + (int64_t)t0 * new_stride_tok;
+    for (int tt0 = 0; tt0 < nt; tt0 += 8) {
+      float v0[8], v1[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int tt = tt0 + e < nt ? tt0 + e : nt - 1;
+        v0[e] = vr[(int64_t)tt * new_stride_tok + lane];
+        v1[e] = vr[(int64_t)tt * new_stride_tok + lane + 64];
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (tt0 + e < nt) {
+#pragma unroll
+          for (int h = 0; h < 8; ++h) {
+            if (h < G) {
+              const float w = __shfl(wt[h], tt0 + e, 64);
+              acc[h][0] += w * v0[e];
+              acc[h][1] += w * v1[e];
+            }
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int h = 0; h < 8; ++h) {
+    if (h < G) {
+      if (lane == 0) {
+        w_m[wave][h] = m_run[h];
+        w_l[wave][h] = l_run[h];
+      }
+      w_acc[wave][h][lane] = acc[h][0];
+      w_acc[wave][h][lane + 64] = acc[h][1];
     }
   }
   __syncthreads();
+  for (int i = tid; i < G * kD; i += kThreads) {
+    const int h = i >> 7, d = i & 127;
+    float M = lse_ab[h];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const int i = tid + 256 * k;
-    if (i < G * kD) {
-      const int h = i >> 7, d = i & 127;
-      const float l = l_run[h];
-      out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? acc[k] / l : 0.0f;
-      if (lse && d == 0) lse[q_row + h] = l > 0.0f ? m_run[h] + logf(l) : -INFINITY;
+    for (int w = 0; w < kZcWaves; ++w) M = fmaxf(M, w_m[w][h]);
+    float o = 0.0f, l = 0.0f;
+    if (lse_ab[h] != -INFINITY) {
+      const float f = expf(lse_ab[h] - M);
+      o = f * acc_ab[i];
+      l = f;
     }
+#pragma unroll
+    for (int w = 0; w < kZcWaves; ++w) {
+      const float mw = w_m[w][h];
+      if (mw != -INFINITY) {
+        const float f = expf(mw - M);
+        o += f * w_acc[w][h][d];
+        l += f * w_l[w][h];
+      }
+    }
+    out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? o / l : 0.0f;
+    if (lse && d == 0) lse[q_row + h] = l > 0.0f ? M + logf(l) : -INFINITY;
   }
 }
 
@@ -997,7 +1053,9 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
   if (n_units == 0) return RDKV_OK;
   RDKV_REQUIRE(out && q, "%s: null out / q", fn);
   RDKV_REQUIRE(n_new == 0 || (k_new && v_new), "%s: null zone-C tensors", fn);
-  hipLaunchKernelGGL(merge_zone_c_kernel, dim3(n_units), dim3(256), 0, (hipStream_t)stream, units,
+  RDKV_REQUIRE(((uintptr_t)k_new % 16) == 0 && new_stride_unit % 4 == 0 && new_stride_tok % 4 == 0,
+               "%s: zone-C key rows must be 16-byte aligned", fn);
+  hipLaunchKernelGGL(merge_zone_c_kernel, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units,
                      (const float *)workspace, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new,
                      v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse);
   RDKV_CHECK_LAUNCH(fn);

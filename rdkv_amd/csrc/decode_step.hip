@@ -9,45 +9,64 @@
 namespace {
 
 // One workgroup per row.  r = x (+ delta, rounded to the storage type like the tensor add);
-// norm = weight * (r * rsqrt(mean(r^2) + eps)) rounded to the storage type.
+// norm = weight * (r * rsqrt(mean(r^2) + eps)) rounded to the storage type.  A thread keeps its
+// EPT elements (i = tid + 256*j) in registers: every load of the row is issued before the first
+// store, so the row costs one memory round trip, not one per element (x may alias residual_out).
+// The storage types are template parameters: with a run-time type every load sits in its own
+// branch and is waited for before the next one is issued.
+template <int EPT, int dtype, int w_dtype>
 __global__ void __launch_bounds__(256)
-add_rms_norm_kernel(const void *x, int64_t x_stride, const void *__restrict__ delta,
-                    int64_t delta_stride, const void *__restrict__ weight, int w_dtype, float eps, int dim,
-                    int dtype, void *residual_out, int64_t res_stride, void *__restrict__ norm_out,
-                    int64_t norm_stride) {
+add_rms_norm_kernel(const void *x, int64_t x_stride, const void *delta, int64_t delta_stride,
+                    const void *__restrict__ weight, float eps, int dim, void *residual_out, int64_t res_stride,
+                    void *__restrict__ norm_out, int64_t norm_stride) {
   __shared__ float s_part[4];
   const int row = blockIdx.x;
   const int64_t xo = row * x_stride, dlo = row * delta_stride, ro = row * res_stride, no = row * norm_stride;
+  float r[EPT], d[EPT], w[EPT];
+  const void *dsrc = delta ? delta : x;      // every load unconditional (index clamped, value selected
+  const int64_t dso = delta ? dlo : xo;      // afterwards), so that none is waited for on its own
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    const int ic = i < dim ? i : 0;
+    r[j] = rdkv_load_as_float(x, dtype, xo + ic);
+    d[j] = rdkv_load_as_float(dsrc, dtype, dso + ic);
+    w[j] = rdkv_load_as_float(weight, w_dtype, ic);
+  }
   float ss = 0.0f;
-  for (int i = threadIdx.x; i < dim; i += 256) {
-    float r = rdkv_load_as_float(x, dtype, xo + i);
-    if (delta) r = rdkv_round_to_dtype(r + rdkv_load_as_float(delta, dtype, dlo + i), dtype);
-    if (residual_out) rdkv_store_from_float(residual_out, dtype, ro + i, r);
-    ss += r * r;
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    if (delta) r[j] = rdkv_round_to_dtype(r[j] + d[j], dtype);
+    if (threadIdx.x + 256 * j >= dim) r[j] = 0.0f;
+    ss += r[j] * r[j];
+  }
+  if (residual_out) {
+#pragma unroll
+    for (int j = 0; j < EPT; ++j) {
+      const int i = threadIdx.x + 256 * j;
+      if (i < dim) rdkv_store_from_float(residual_out, dtype, ro + i, r[j]);
+    }
   }
   ss = rdkv_wave_sum(ss);
   if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
   __syncthreads();
   const float mean = (s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)dim;
   const float rs = rsqrtf(mean + eps);
-  for (int i = threadIdx.x; i < dim; i += 256) {
-    float r;
-    if (residual_out) r = rdkv_load_as_float(residual_out, dtype, ro + i);   // this thread wrote it
-    else {
-      r = rdkv_load_as_float(x, dtype, xo + i);
-      if (delta) r = rdkv_round_to_dtype(r + rdkv_load_as_float(delta, dtype, dlo + i), dtype);
-    }
-    rdkv_store_from_float(norm_out, dtype, no + i, rdkv_load_as_float(weight, w_dtype, i) * (r * rs));
+#pragma unroll
+  for (int j = 0; j < EPT; ++j) {
+    const int i = threadIdx.x + 256 * j;
+    if (i < dim) rdkv_store_from_float(norm_out, dtype, no + i, w[j] * (r[j] * rs));
   }
 }
 
 // One wavefront per KV head: k rotated (rounded to the storage type, as the in-place rotation
 // stores it) and v, both widened to fp32, written as the row [K | V] of the zone C buffer that the
 // device-held index names.  A row index outside the buffer writes nothing.
+template <int dtype, int cs_dtype>
 __global__ void __launch_bounds__(64)
 rope_append_kv_kernel(const void *__restrict__ k, int64_t k_stride_h, const void *__restrict__ v,
-                      int64_t v_stride_h, int half_d, int dtype, const void *__restrict__ cos_half,
-                      const void *__restrict__ sin_half, int cs_dtype, float *__restrict__ new_kv,
+                      int64_t v_stride_h, int half_d, const void *__restrict__ cos_half,
+                      const void *__restrict__ sin_half, float *__restrict__ new_kv,
                       int64_t new_stride_head, int64_t new_stride_tok, const int64_t *__restrict__ row_dev,
                       int64_t capacity) {
   const int64_t row = row_dev[0];
@@ -67,9 +86,9 @@ rope_append_kv_kernel(const void *__restrict__ k, int64_t k_stride_h, const void
   }
 }
 
+template <int dtype>
 __global__ void __launch_bounds__(256)
-silu_mul_kernel(const void *__restrict__ gate, const void *__restrict__ up, int64_t n, int dtype,
-                void *__restrict__ out) {
+silu_mul_kernel(const void *__restrict__ gate, const void *__restrict__ up, int64_t n, void *__restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   const float g = rdkv_load_as_float(gate, dtype, i);
@@ -84,13 +103,35 @@ RDKV_API int rdkv_add_rms_norm(const void *x, int64_t x_stride_row, const void *
                                void *residual_out, int64_t residual_stride_row, void *norm_out,
                                int64_t norm_stride_row, void *stream) {
   RDKV_REQUIRE(rows >= 0 && dim > 0, "rdkv_add_rms_norm: bad shape rows=%d dim=%d", rows, dim);
-  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && w_dtype >= 0 && w_dtype <= 2, "rdkv_add_rms_norm: unknown dtype");
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && (w_dtype == dtype || w_dtype == RDKV_DTYPE_F32),
+               "rdkv_add_rms_norm: weight type %d must be the data type %d or fp32", w_dtype, dtype);
   if (rows == 0) return RDKV_OK;
   RDKV_REQUIRE(x && weight && norm_out, "rdkv_add_rms_norm: null pointer");
   RDKV_REQUIRE(norm_out != x && norm_out != residual_out, "rdkv_add_rms_norm: norm_out must not alias the input");
-  hipLaunchKernelGGL(add_rms_norm_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, x, x_stride_row, delta,
-                     delta_stride_row, weight, w_dtype, eps, dim, dtype, residual_out, residual_stride_row,
-                     norm_out, norm_stride_row);
+  RDKV_REQUIRE(dim <= 256 * 64, "rdkv_add_rms_norm: rows of %d elements exceed %d", dim, 256 * 64);
+#define RDKV_LAUNCH_NORM3(EPT, DT, WDT)                                                                      \
+  hipLaunchKernelGGL((add_rms_norm_kernel<EPT, DT, WDT>), dim3(rows), dim3(256), 0, (hipStream_t)stream, x,    \
+                     x_stride_row, delta, delta_stride_row, weight, eps, dim, residual_out, residual_stride_row, \
+                     norm_out, norm_stride_row)
+#define RDKV_LAUNCH_NORM2(EPT, DT)                    \
+  do {                                                \
+    if (w_dtype == DT) RDKV_LAUNCH_NORM3(EPT, DT, DT); \
+    else RDKV_LAUNCH_NORM3(EPT, DT, RDKV_DTYPE_F32);  \
+  } while (0)
+#define RDKV_LAUNCH_NORM(EPT)                                            \
+  do {                                                                   \
+    if (dtype == RDKV_DTYPE_F32) RDKV_LAUNCH_NORM2(EPT, RDKV_DTYPE_F32); \
+    else if (dtype == RDKV_DTYPE_F16) RDKV_LAUNCH_NORM2(EPT, RDKV_DTYPE_F16); \
+    else RDKV_LAUNCH_NORM2(EPT, RDKV_DTYPE_BF16);                        \
+  } while (0)
+  if (dim <= 256) RDKV_LAUNCH_NORM(1);
+  else if (dim <= 256 * 4) RDKV_LAUNCH_NORM(4);
+  else if (dim <= 256 * 16) RDKV_LAUNCH_NORM(16);
+  else if (dim <= 256 * 32) RDKV_LAUNCH_NORM(32);
+  else RDKV_LAUNCH_NORM(64);
+#undef RDKV_LAUNCH_NORM2
+#undef RDKV_LAUNCH_NORM3
+#undef RDKV_LAUNCH_NORM
   RDKV_CHECK_LAUNCH("rdkv_add_rms_norm");
   return RDKV_OK;
 }
@@ -100,14 +141,22 @@ RDKV_API int rdkv_rope_append_kv(const void *k, int64_t k_stride_h, const void *
                                  float *new_kv, int64_t new_stride_head, int64_t new_stride_tok,
                                  const int64_t *row_dev, int64_t capacity, void *stream) {
   RDKV_REQUIRE(H_kv >= 0 && D > 0 && D % 2 == 0, "rdkv_rope_append_kv: bad shape H_kv=%d D=%d", H_kv, D);
-  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && cs_dtype >= 0 && cs_dtype <= 2, "rdkv_rope_append_kv: unknown dtype");
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2 && (cs_dtype == dtype || cs_dtype == RDKV_DTYPE_F32),
+               "rdkv_rope_append_kv: cos / sin type %d must be the data type %d or fp32", cs_dtype, dtype);
   if (H_kv == 0) return RDKV_OK;
   RDKV_REQUIRE(k && v && cos_half && sin_half && new_kv && row_dev, "rdkv_rope_append_kv: null pointer");
   RDKV_REQUIRE(capacity >= 0 && new_stride_tok >= 2 * D && new_stride_head >= 0,
                "rdkv_rope_append_kv: bad zone C buffer shape");
-  hipLaunchKernelGGL(rope_append_kv_kernel, dim3(H_kv), dim3(64), 0, (hipStream_t)stream, k, k_stride_h, v,
-                     v_stride_h, D / 2, dtype, cos_half, sin_half, cs_dtype, new_kv, new_stride_head,
-                     new_stride_tok, row_dev, capacity);
+#define RDKV_LAUNCH_APPEND(DT, CDT)                                                                          \
+  hipLaunchKernelGGL((rope_append_kv_kernel<DT, CDT>), dim3(H_kv), dim3(64), 0, (hipStream_t)stream, k, k_stride_h, \
+                     v, v_stride_h, D / 2, cos_half, sin_half, new_kv, new_stride_head, new_stride_tok, row_dev, \
+                     capacity)
+  if (dtype == RDKV_DTYPE_F32) RDKV_LAUNCH_APPEND(RDKV_DTYPE_F32, RDKV_DTYPE_F32);
+  else if (dtype == RDKV_DTYPE_F16 && cs_dtype == RDKV_DTYPE_F16) RDKV_LAUNCH_APPEND(RDKV_DTYPE_F16, RDKV_DTYPE_F16);
+  else if (dtype == RDKV_DTYPE_F16) RDKV_LAUNCH_APPEND(RDKV_DTYPE_F16, RDKV_DTYPE_F32);
+  else if (cs_dtype == RDKV_DTYPE_BF16) RDKV_LAUNCH_APPEND(RDKV_DTYPE_BF16, RDKV_DTYPE_BF16);
+  else RDKV_LAUNCH_APPEND(RDKV_DTYPE_BF16, RDKV_DTYPE_F32);
+#undef RDKV_LAUNCH_APPEND
   RDKV_CHECK_LAUNCH("rdkv_rope_append_kv");
   return RDKV_OK;
 }
@@ -118,8 +167,15 @@ RDKV_API int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtyp
   RDKV_REQUIRE(gate && up && out, "rdkv_silu_mul: null pointer");
   const int64_t blocks = rdkv_cdiv(n, 256);
   RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_silu_mul: too many elements");
-  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, gate, up, n, dtype,
-                     out);
+  if (dtype == RDKV_DTYPE_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<RDKV_DTYPE_F32>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       gate, up, n, out);
+  else if (dtype == RDKV_DTYPE_F16)
+    hipLaunchKernelGGL(silu_mul_kernel<RDKV_DTYPE_F16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       gate, up, n, out);
+  else
+    hipLaunchKernelGGL(silu_mul_kernel<RDKV_DTYPE_BF16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       gate, up, n, out);
   RDKV_CHECK_LAUNCH("rdkv_silu_mul");
   return RDKV_OK;
 }

@@ -212,7 +212,7 @@ def test_step_kernels_match_tensor_expressions(dtype):
     from rdkv_amd.triton_rope import fused_rope
     g = torch.Generator(device=DEV).manual_seed(5)
     ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7, torch.float32: 2.0 ** -22}[dtype]
-    for rows, dim in ((1, 4096), (4, 128), (3, 1000)):
+    for rows, dim in ((1, 4096), (4, 128), (3, 1000), (2, 8192), (1, 16384)):
         x = torch.randn(rows, dim, generator=g, device=DEV).to(dtype)
         d = torch.randn(rows, dim, generator=g, device=DEV).to(dtype)
         w = (1.0 + 0.1 * torch.randn(dim, generator=g, device=DEV)).to(dtype)
