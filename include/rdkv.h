@@ -366,8 +366,11 @@ int rdkv_knapsack_rows(const float *scores, int64_t stride_b, int B, int64_t T, 
  * queries of softmax_t(q . k / sqrt(D)) (causal != 0: key t is visible to query q only if t <= q,
  * which needs Q == T); NULL skips it.  channel_scores fp32 [H_kv, D]: mean_{g,q}(q^2) *
  * mean_t(k^2).  fp32 arithmetic, fixed summation order.  workspace:
- * rdkv_block_score_workspace_bytes(H_kv*G, Q, T, D) bytes (-1: T too large for the kernel). */
+ * rdkv_block_score_workspace_bytes(H_kv*G, Q, T, D) bytes (-1: T too large for the token
+ * scores); with token_scores NULL rdkv_channel_score_workspace_bytes(H_kv*G, H_kv, Q, T, D)
+ * suffices (partial sums of squares per 512 rows; any T). */
 int64_t rdkv_block_score_workspace_bytes(int H_q, int Q, int64_t T, int D);
+int64_t rdkv_channel_score_workspace_bytes(int H_q, int H_kv, int Q, int64_t T, int D);
 int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride_h, int64_t q_stride_q,
                      const void *keys, int k_dtype, int64_t k_stride_h, int64_t k_stride_t, int H_kv,
                      int G, int Q, int64_t T, int D, int causal, float *token_scores,

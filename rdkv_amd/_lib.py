@@ -70,6 +70,7 @@ SIGNATURES = {
     "rdkv_k_budget_per_head": (I, [P, I, I, I, L, I, F, P, P]),
     "rdkv_knapsack_rows": (I, [P, L, I, L, P, P, P, I, I, Dbl, P, I, L, P, P]),
     "rdkv_block_score_workspace_bytes": (L, [I, I, L, I]),
+    "rdkv_channel_score_workspace_bytes": (L, [I, I, I, L, I]),
     "rdkv_block_score": (I, [P, I, L, L, P, I, L, L, I, I, I, L, I, I, P, P, P, L, P]),
     "rdkv_token_mass": (I, [P, I, L, L, I, I, L, P, P]),
     "rdkv_probe_copy": (I, [P, P, L, P]),

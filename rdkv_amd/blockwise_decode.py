@@ -358,7 +358,10 @@ def _block_score(queries: Tensor, keys: Tensor, num_kv_groups: int, causal: bool
     lib = _lib.load()
     token = torch.empty(h_kv, t_len, dtype=torch.float32, device=dev) if want_tokens else None
     channel = torch.empty(h_kv, d, dtype=torch.float32, device=dev)
-    ws_bytes = lib.rdkv_block_score_workspace_bytes(h_kv * num_kv_groups, q_len, t_len, d) if want_tokens else 0
+    if want_tokens:
+        ws_bytes = lib.rdkv_block_score_workspace_bytes(h_kv * num_kv_groups, q_len, t_len, d)
+    else:
+        ws_bytes = lib.rdkv_channel_score_workspace_bytes(h_kv * num_kv_groups, h_kv, q_len, t_len, d)
     if ws_bytes < 0:
         raise NotImplementedError(f"blocks of {t_len} keys are beyond the scoring kernel")
     ws = _lib.workspace(dev, max(ws_bytes, 256))

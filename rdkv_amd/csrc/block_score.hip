@@ -111,52 +111,149 @@ block_score_reduce_kernel(const float *__restrict__ partial, int G, int n_qtiles
   const int h = blockIdx.y;
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
+  const int n = G * n_qtiles;
+  const float *base = partial + (int64_t)h * n * T + t;
   float s = 0.0f;
-  for (int i = 0; i < G * n_qtiles; ++i) s += partial[((int64_t)h * G * n_qtiles + i) * T + t];
+  for (int i0 = 0; i0 < n; i0 += 8) {       // eight loads in flight, added in index order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = base[(int64_t)(i0 + u < n ? i0 + u : i0) * T];
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (i0 + u < n) s += v[u];
+  }
   token[(int64_t)h * T + t] = s;
 }
 
-// channel[h, d] = mean over (group head, query) of q^2 * mean over tokens of k^2
+// ThinK channel score: channel[h, d] = mean over (group head, query) of q^2 * mean over tokens of
+// k^2, in two steps.  sumsq_partial_kernel: grid (chunks of kSumsqRows rows, heads); a workgroup
+// sums the squares of its rows per channel and writes partial[(head * n_chunks + chunk) * D + d].
+// WIDE (2-byte elements, D a power of two in 8..2048, 16-byte aligned rows): D/8 lanes share a row,
+// one 16-byte load each, 2048/D rows per step, four steps in flight; the lanes that share a
+// channel are added through LDS in row order.  Otherwise a thread owns channels tid, tid+256, ..
+// and walks the rows.  channel_finish_kernel adds the partials of a head in index order.
+constexpr int kSumsqRows = 512;
+
+template <bool WIDE, int dtype>
 __global__ void __launch_bounds__(256)
-channel_score_kernel(const void *__restrict__ queries, int q_dtype, int64_t q_stride_h, int64_t q_stride_q,
-                     const void *__restrict__ keys, int k_dtype, int64_t k_stride_h, int64_t k_stride_t,
-                     int G, int Q, int T, int D, float *__restrict__ channel) {
-  __shared__ float red[2][4][64];
-  const int h = blockIdx.y;
-  const int dl = threadIdx.x & 63, part = threadIdx.x >> 6;       // 64 channels per block, 4 row partitions
-  const int d = blockIdx.x * 64 + dl;
-  float qs = 0.0f, ks = 0.0f;
-  if (d < D) {
-    for (int i = part; i < G * Q; i += 4) {
-      const float v = rdkv_load_as_float(queries, q_dtype,
-                                         (int64_t)(h * G + i / Q) * q_stride_h + (int64_t)(i % Q) * q_stride_q + d);
-      qs = fmaf(v, v, qs);
+sumsq_partial_kernel(const void *__restrict__ x, int64_t stride_h, int64_t stride_t, int T, int D,
+                     float *__restrict__ partial) {
+  __shared__ float red[2048];
+  const int chunk = blockIdx.x, h = blockIdx.y, n_chunks = gridDim.x;
+  const int t_begin = chunk * kSumsqRows, t_end = min(T, t_begin + kSumsqRows);
+  float *out = partial + ((int64_t)h * n_chunks + chunk) * D;
+  if (WIDE) {
+    const int d8 = D >> 3, rows_per_step = 256 / d8;
+    const int r = threadIdx.x / d8, c8 = threadIdx.x - r * d8;
+    const uint16_t *base = reinterpret_cast<const uint16_t *>(x) + (int64_t)h * stride_h + 8 * c8;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int t0 = t_begin + r; t0 < t_end; t0 += 4 * rows_per_step) {
+      uint4 raw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * rows_per_step;
+        raw[u] = *reinterpret_cast<const uint4 *>(base + (int64_t)(t < t_end ? t : t0) * stride_t);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (t0 + u * rows_per_step < t_end) {
+          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            float lo, hi;
+            if (dtype == RDKV_DTYPE_F16) {
+              lo = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xffffu));
+              hi = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+            } else {
+              lo = __uint_as_float(w[i] << 16);
+              hi = __uint_as_float(w[i] & 0xffff0000u);
+            }
+            acc[2 * i] = fmaf(lo, lo, acc[2 * i]);
+            acc[2 * i + 1] = fmaf(hi, hi, acc[2 * i + 1]);
+          }
+        }
+      }
     }
-    for (int t = part; t < T; t += 4) {
-      const float v = rdkv_load_as_float(keys, k_dtype, (int64_t)h * k_stride_h + (int64_t)t * k_stride_t + d);
-      ks = fmaf(v, v, ks);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) red[r * D + 8 * c8 + i] = acc[i];      // rows_per_step * D = 2048 floats
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += 256) {
+      float s = 0.0f;
+      for (int rr = 0; rr < rows_per_step; ++rr) s += red[rr * D + d];
+      out[d] = s;
+    }
+  } else {
+    for (int d = threadIdx.x; d < D; d += 256) {
+      const int64_t base = (int64_t)h * stride_h + d;
+      float s = 0.0f;
+      for (int t0 = t_begin; t0 < t_end; t0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = rdkv_load_as_float(x, dtype, base + (int64_t)(t0 + u < t_end ? t0 + u : t0) * stride_t);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (t0 + u < t_end) s = fmaf(v[u], v[u], s);
+      }
+      out[d] = s;
     }
   }
-  red[0][part][dl] = qs;
-  red[1][part][dl] = ks;
-  __syncthreads();
-  if (part == 0 && d < D) {
-    const float q2 = (red[0][0][dl] + red[0][1][dl]) + (red[0][2][dl] + red[0][3][dl]);
-    const float k2 = (red[1][0][dl] + red[1][1][dl]) + (red[1][2][dl] + red[1][3][dl]);
-    channel[(int64_t)h * D + d] = (q2 / (float)(G * Q)) * (k2 / (float)T);
-  }
+}
+
+// grid (ceil(D / 256), H_kv): sums of q^2 over the head's G query heads and their chunks, of k^2
+// over the head's chunks, both in index order.
+__global__ void __launch_bounds__(256)
+channel_finish_kernel(const float *__restrict__ q_part, int nq_chunks, const float *__restrict__ k_part,
+                      int nk_chunks, int G, int Q, int T, int D, float *__restrict__ channel) {
+  const int h = blockIdx.y, d = blockIdx.x * 256 + threadIdx.x;
+  if (d >= D) return;
+  float q2 = 0.0f, k2 = 0.0f;
+  for (int i = 0; i < G * nq_chunks; ++i) q2 += q_part[((int64_t)h * G * nq_chunks + i) * D + d];
+  for (int i = 0; i < nk_chunks; ++i) k2 += k_part[((int64_t)h * nk_chunks + i) * D + d];
+  channel[(int64_t)h * D + d] = (q2 / (float)(G * Q)) * (k2 / (float)T);
+}
+
+template <int dtype>
+void launch_sumsq(const void *x, int64_t stride_h, int64_t stride_t, int heads, int T, int D, float *partial,
+                  hipStream_t s) {
+  const bool pow2 = (D & (D - 1)) == 0;
+  const bool wide = dtype != RDKV_DTYPE_F32 && pow2 && D >= 8 && D <= 2048 && stride_h % 8 == 0 &&
+                    stride_t % 8 == 0 && ((uintptr_t)x % 16) == 0;
+  const dim3 grid((unsigned)rdkv_cdiv(T, kSumsqRows), heads);
+  if (wide)
+    hipLaunchKernelGGL((sumsq_partial_kernel<true, dtype>), grid, dim3(256), 0, s, x, stride_h, stride_t, T, D, partial);
+  else
+    hipLaunchKernelGGL((sumsq_partial_kernel<false, dtype>), grid, dim3(256), 0, s, x, stride_h, stride_t, T, D,
+                       partial);
+}
+
+void launch_sumsq_any(const void *x, int dtype, int64_t stride_h, int64_t stride_t, int heads, int T, int D,
+                      float *partial, hipStream_t s) {
+  if (dtype == RDKV_DTYPE_F32) launch_sumsq<RDKV_DTYPE_F32>(x, stride_h, stride_t, heads, T, D, partial, s);
+  else if (dtype == RDKV_DTYPE_F16) launch_sumsq<RDKV_DTYPE_F16>(x, stride_h, stride_t, heads, T, D, partial, s);
+  else launch_sumsq<RDKV_DTYPE_BF16>(x, stride_h, stride_t, heads, T, D, partial, s);
 }
 
 // out[h, t] = sum over i of x[h, i, t], accumulated in fp32 in index order and rounded once to the
 // input's storage type (a library sum of a half-precision tensor is a half-precision value)
+template <int dtype>
 __global__ void __launch_bounds__(256)
-token_mass_kernel(const void *__restrict__ x, int dtype, int64_t stride_h, int64_t stride_i, int n_inner, int T,
+token_mass_kernel(const void *__restrict__ x, int64_t stride_h, int64_t stride_i, int n_inner, int T,
                   float *__restrict__ out) {
   const int h = blockIdx.y;
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
+  const int64_t base = (int64_t)h * stride_h + t;
   float s = 0.0f;
-  for (int i = 0; i < n_inner; ++i) s += rdkv_load_as_float(x, dtype, (int64_t)h * stride_h + (int64_t)i * stride_i + t);
+  for (int i0 = 0; i0 < n_inner; i0 += 8) {        // eight loads in flight, added in index order
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = rdkv_load_as_float(x, dtype, base + (int64_t)(i0 + u < n_inner ? i0 + u : i0) * stride_i);
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (i0 + u < n_inner) s += v[u];
+  }
   out[(int64_t)h * T + t] = rdkv_round_to_dtype(s, dtype);
 }
 
@@ -168,11 +265,26 @@ int q_tile_for(int64_t T, int D) {
 
 }  // namespace
 
-RDKV_API int64_t rdkv_block_score_workspace_bytes(int H_q, int Q, int64_t T, int D) {
-  if (H_q <= 0 || Q <= 0 || T <= 0 || D <= 0) return 0;
+static int64_t token_partial_bytes(int H_q, int Q, int64_t T, int D) {
   const int qb = q_tile_for(T, D);
   if (qb < 1) return -1;
   return (int64_t)H_q * rdkv_cdiv(Q, qb) * T * 4;
+}
+
+static int64_t channel_partial_floats(int heads, int64_t rows, int D) {
+  return (int64_t)heads * rdkv_cdiv(rows, kSumsqRows) * D;
+}
+
+RDKV_API int64_t rdkv_channel_score_workspace_bytes(int H_q, int H_kv, int Q, int64_t T, int D) {
+  if (H_q <= 0 || H_kv <= 0 || Q <= 0 || T <= 0 || D <= 0) return 0;
+  return (channel_partial_floats(H_q, Q, D) + channel_partial_floats(H_kv, T, D)) * 4;
+}
+
+RDKV_API int64_t rdkv_block_score_workspace_bytes(int H_q, int Q, int64_t T, int D) {
+  if (H_q <= 0 || Q <= 0 || T <= 0 || D <= 0) return 0;
+  const int64_t tok = token_partial_bytes(H_q, Q, T, D);
+  if (tok < 0) return -1;
+  return tok + rdkv_channel_score_workspace_bytes(H_q, H_q, Q, T, D);   // H_kv <= H_q
 }
 
 RDKV_API int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride_h, int64_t q_stride_q,
@@ -186,27 +298,39 @@ RDKV_API int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride
   RDKV_REQUIRE(!causal || Q == T, "%s: self-scored final flush requires equal query/key lengths, got Q=%d, T=%lld",
                fn, Q, (long long)T);
   hipStream_t s = (hipStream_t)stream;
+  const int H_q = H_kv * G;
+  int64_t tok_bytes = 0;
+  if (token_scores) {
+    tok_bytes = token_partial_bytes(H_q, Q, T, D);
+    RDKV_REQUIRE(tok_bytes >= 0, "%s: %lld keys do not fit the scoring kernel", fn, (long long)T);
+  }
+  const int64_t need = tok_bytes + rdkv_channel_score_workspace_bytes(H_q, H_kv, Q, T, D);
+  if (workspace == nullptr || workspace_bytes < need) {
+    rdkv_set_error("%s: workspace of %lld bytes required", fn, (long long)need);
+    return RDKV_EWORKSPACE;
+  }
+  RDKV_REQUIRE(T <= 0x7fffffffLL, "%s: too many keys", fn);
   if (token_scores) {
     const int qb = q_tile_for(T, D);
-    RDKV_REQUIRE(qb >= 1, "%s: %lld keys do not fit the scoring kernel", fn, (long long)T);
     const int n_qtiles = (int)rdkv_cdiv(Q, qb);
-    if (workspace == nullptr || workspace_bytes < rdkv_block_score_workspace_bytes(H_kv * G, Q, T, D)) {
-      rdkv_set_error("%s: workspace too small", fn);
-      return RDKV_EWORKSPACE;
-    }
     const size_t lds = ((size_t)qb * D + (size_t)qb * T) * 4;
     const int wide_rows = (k_dtype == RDKV_DTYPE_F16 || k_dtype == RDKV_DTYPE_BF16) && D % 8 == 0 &&
                           k_stride_h % 8 == 0 && k_stride_t % 8 == 0 && ((uintptr_t)keys % 16) == 0;
     hipFuncSetAttribute(reinterpret_cast<const void *>(block_score_partial_kernel),
                         hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    hipLaunchKernelGGL(block_score_partial_kernel, dim3(n_qtiles, H_kv * G), dim3(kScoreThreads), lds, s, queries,
+    hipLaunchKernelGGL(block_score_partial_kernel, dim3(n_qtiles, H_q), dim3(kScoreThreads), lds, s, queries,
                        q_dtype, q_stride_h, q_stride_q, keys, k_dtype, k_stride_h, k_stride_t, G, Q, (int)T, D, qb,
                        causal, (float)(1.0 / sqrt((double)D)), wide_rows, reinterpret_cast<float *>(workspace));
     hipLaunchKernelGGL(block_score_reduce_kernel, dim3((unsigned)rdkv_cdiv(T, 256), H_kv), dim3(256), 0, s,
                        reinterpret_cast<const float *>(workspace), G, n_qtiles, (int)T, token_scores);
   }
-  hipLaunchKernelGGL(channel_score_kernel, dim3((unsigned)rdkv_cdiv(D, 64), H_kv), dim3(256), 0, s, queries, q_dtype,
-                     q_stride_h, q_stride_q, keys, k_dtype, k_stride_h, k_stride_t, G, Q, (int)T, D, channel_scores);
+  float *q_part = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + tok_bytes);
+  float *k_part = q_part + channel_partial_floats(H_q, Q, D);
+  launch_sumsq_any(queries, q_dtype, q_stride_h, q_stride_q, H_q, Q, D, q_part, s);
+  launch_sumsq_any(keys, k_dtype, k_stride_h, k_stride_t, H_kv, (int)T, D, k_part, s);
+  hipLaunchKernelGGL(channel_finish_kernel, dim3((unsigned)rdkv_cdiv(D, 256), H_kv), dim3(256), 0, s, q_part,
+                     (int)rdkv_cdiv(Q, kSumsqRows), k_part, (int)rdkv_cdiv(T, kSumsqRows), G, Q, (int)T, D,
+                     channel_scores);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }
@@ -218,8 +342,16 @@ RDKV_API int rdkv_token_mass(const void *x, int dtype, int64_t stride_h, int64_t
   RDKV_REQUIRE(dtype >= 0 && dtype <= 2, "%s: unknown dtype", fn);
   if (H == 0 || T == 0) return RDKV_OK;
   RDKV_REQUIRE(out && (n_inner == 0 || x), "%s: null pointer", fn);
-  hipLaunchKernelGGL(token_mass_kernel, dim3((unsigned)rdkv_cdiv(T, 256), H), dim3(256), 0, (hipStream_t)stream, x,
-                     dtype, stride_h, stride_i, n_inner, (int)T, out);
+  const dim3 grid((unsigned)rdkv_cdiv(T, 256), H);
+  if (dtype == RDKV_DTYPE_F32)
+    hipLaunchKernelGGL(token_mass_kernel<RDKV_DTYPE_F32>, grid, dim3(256), 0, (hipStream_t)stream, x, stride_h,
+                       stride_i, n_inner, (int)T, out);
+  else if (dtype == RDKV_DTYPE_F16)
+    hipLaunchKernelGGL(token_mass_kernel<RDKV_DTYPE_F16>, grid, dim3(256), 0, (hipStream_t)stream, x, stride_h,
+                       stride_i, n_inner, (int)T, out);
+  else
+    hipLaunchKernelGGL(token_mass_kernel<RDKV_DTYPE_BF16>, grid, dim3(256), 0, (hipStream_t)stream, x, stride_h,
+                       stride_i, n_inner, (int)T, out);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

@@ -231,7 +231,9 @@ def test_selection_and_planning_entry_points_reject_bad_arguments():
     err(lib.rdkv_k_budget_per_head(None, 5, 5, 1, 8, 128, 1.0, None, None), "bad arguments")
     err(lib.rdkv_block_score(None, 1, 8, 8, None, 1, 8, 8, 1, 1, 4, 5, 8, 1, None, None, None, 0, None), "null pointer")
     err(lib.rdkv_block_score(None, 7, 8, 8, None, 1, 8, 8, 1, 1, 4, 4, 8, 0, None, None, None, 0, None), "dtype")
-    assert lib.rdkv_block_score_workspace_bytes(32, 128, 128, 128) == 32 * 8 * 128 * 4
+    # token partials [H_q, 8 query tiles, T] + sums of squares per 512 rows of queries and keys
+    assert lib.rdkv_block_score_workspace_bytes(32, 128, 128, 128) == 32 * 8 * 128 * 4 + 2 * 32 * 128 * 4
+    assert lib.rdkv_channel_score_workspace_bytes(32, 8, 32, 32768, 128) == (32 * 1 + 8 * 64) * 128 * 4
     assert lib.rdkv_block_score_workspace_bytes(32, 128, 1 << 20, 128) == -1
     err(lib.rdkv_pack_layer_plan(None, 3, 8, None, 1, 8, 2, 8, 8, None, 8, None, 8, None, None), "element sizes")
     err(lib.rdkv_pack_layer_plan(None, 1, 8, None, 1, 8, 2, 0, 8, None, 8, None, 8, None, None), "bad shape")
