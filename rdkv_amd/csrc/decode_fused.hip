@@ -126,12 +126,12 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
       for (int k = 0; k < n; ++k) M = fmaxf(M, s_m[k * 8 + h]);
       float o = 0.0f, l = 0.0f;
       const float *base = base0 + h * kPartialStride + d;
-      for (int k0 = 0; k0 < n; k0 += 8) {
-        float v[8];
+      for (int k0 = 0; k0 < n; k0 += 16) {
+        float v[16];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = k0 + e < n ? *(base + (k0 + e) * pstride) : 0.0f;
+        for (int e = 0; e < 16; ++e) v[e] = *(base + (k0 + e < n ? k0 + e : k0) * pstride);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
+        for (int e = 0; e < 16; ++e) {
           if (k0 + e < n) {
             const float mk = s_m[(k0 + e) * 8 + h];
             const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
@@ -767,8 +767,11 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
 // 1/sqrt(D) first as the reference does.
 constexpr int kZcChunk = 64;
 constexpr int kZcWaves = 8;
+// G is a template parameter: the per-head loops unroll into straight-line code (with a run-time
+// G every head of every token is a scalar branch).
+template <int G>
 __global__ void __launch_bounds__(64 * kZcWaves)
-merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
+merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride,
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
                     const float *__restrict__ k_new, const float *__restrict__ v_new, int64_t new_stride_unit,
@@ -786,31 +789,44 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   const int q_row = u->q_row;
   const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
+  // the query (and its rotation table) is fetched before the merge so that the two overlap
+  const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
+  float qv[2], qo[2], qc[2], qs_[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = tid + j * kThreads;
+    const int ic = i < G * kD ? i : 0;
+    const int c = ic & 127;
+    const int64_t row = (int64_t)(q_row + (ic >> 7)) * q_stride;
+    qv[j] = rdkv_load_as_float_nobranch(q, q_dtype, row + c);
+    qo[j] = rdkv_load_as_float_nobranch(q, q_dtype, row + (c ^ 64));
+    qc[j] = rdkv_load_as_float_nobranch(rope_cos ? rope_cos : q, rope_cos ? rope_dtype : q_dtype, rope_cos ? (c & 63) : row);
+    qs_[j] = rdkv_load_as_float_nobranch(rope_sin ? rope_sin : q, rope_sin ? rope_dtype : q_dtype, rope_sin ? (c & 63) : row);
+  }
   merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, kThreads, scratch,
              acc_ab, lse_ab);
-  const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
-  for (int i = tid; i < G * kD; i += kThreads) {
-    const int c = i & 127;
-    const int64_t row = (int64_t)(q_row + (i >> 7)) * q_stride;
-    float v = load_qv(q, q_dtype, row + c);
-    if (rope_cos) {
-      const float other = load_qv(q, q_dtype, row + (c ^ 64));
-      const float cs = rdkv_load_as_float(rope_cos, rope_dtype, c & 63);
-      const float sn = rdkv_load_as_float(rope_sin, rope_dtype, c & 63);
-      float out_lo, out_hi;
-      if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
-      else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
-      v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int i = tid + j * kThreads;
+    if (i < G * kD) {
+      const int c = i & 127;
+      float v = qv[j];
+      if (rope_cos) {
+        float out_lo, out_hi;
+        if (c < 64) rdkv_rope_pair(v, qo[j], qc[j], qs_[j], out_lo, out_hi);
+        else rdkv_rope_pair(qo[j], v, qc[j], qs_[j], out_lo, out_hi);
+        v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+      }
+      qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
     }
-    qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
   }
   __syncthreads();
 
   const float *kn = k_new + (int64_t)kv_row * new_stride_unit;
   const float *vn = v_new + (int64_t)kv_row * new_stride_unit;
-  float m_run[8], l_run[8], acc[8][2];
+  float m_run[G], l_run[G], acc[G][2];
 #pragma unroll
-  for (int h = 0; h < 8; ++h) {
+  for (int h = 0; h < G; ++h) {
     m_run[h] = -INFINITY;
     l_run[h] = 0.0f;
     acc[h][0] = acc[h][1] = 0.0f;
@@ -819,76 +835,67 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
     const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
     const bool valid = lane < nt;
     // scores of this lane's token against the G query heads
-    float s[8];
+    float s[G];
 #pragma unroll
-    for (int h = 0; h < 8; ++h) s[h] = 0.0f;
+    for (int h = 0; h < G; ++h) s[h] = 0.0f;
     const float4 *kr = reinterpret_cast<const float4 *>(kn + (int64_t)(t0 + (valid ? lane : 0)) * new_stride_tok);
 #pragma unroll 1
-    for (int c0 = 0; c0 < kD / 4; c0 += 8) {
-      float4 kv[8];
+    for (int c0 = 0; c0 < kD / 4; c0 += 16) {
+      float4 kv[16];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) kv[e] = kr[c0 + e];
+      for (int e = 0; e < 16; ++e) kv[e] = kr[c0 + e];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 16; ++e) {
 #pragma unroll
-        for (int h = 0; h < 8; ++h) {
-          if (h < G) {
-            const float4 qv = reinterpret_cast<const float4 *>(qz[h])[c0 + e];
-            s[h] += kv[e].x * qv.x + kv[e].y * qv.y + kv[e].z * qv.z + kv[e].w * qv.w;
-          }
+        for (int h = 0; h < G; ++h) {
+          const float4 qv = reinterpret_cast<const float4 *>(qz[h])[c0 + e];
+          s[h] += kv[e].x * qv.x + kv[e].y * qv.y + kv[e].z * qv.z + kv[e].w * qv.w;
         }
       }
     }
-    float wt[8];
+    float wt[G];
 #pragma unroll
-    for (int h = 0; h < 8; ++h) {
-      wt[h] = 0.0f;
-      if (h < G) {
-        const float sh = valid ? s[h] : -INFINITY;
-        const float m_new = fmaxf(m_run[h], rdkv_wave_max(sh));     // finite: the chunk has a token
-        const float f = m_run[h] == -INFINITY ? 0.0f : expf(m_run[h] - m_new);
-        wt[h] = valid ? expf(sh - m_new) : 0.0f;
-        l_run[h] = l_run[h] * f + rdkv_wave_sum(wt[h]);
-        acc[h][0] *= f;
-        acc[h][1] *= f;
-        m_run[h] = m_new;
-      }
+    for (int h = 0; h < G; ++h) {
+      const float sh = valid ? s[h] : -INFINITY;
+      const float m_new = fmaxf(m_run[h], rdkv_wave_max(sh));     // finite: the chunk has a token
+      const float f = m_run[h] == -INFINITY ? 0.0f : expf(m_run[h] - m_new);
+      wt[h] = valid ? expf(sh - m_new) : 0.0f;
+      l_run[h] = l_run[h] * f + rdkv_wave_sum(wt[h]);
+      acc[h][0] *= f;
+      acc[h][1] *= f;
+      m_run[h] = m_new;
     }
     // values: lane = channels lane and lane + 64, the weight of token tt comes from lane tt
     const float *vr = vn + (int64_t)t0 * new_stride_tok;
-    for (int tt0 = 0; tt0 < nt; tt0 += 8) {
-      float v0[8], v1[8];
+    for (int tt0 = 0; tt0 < nt; tt0 += 16) {
+      float v0[16], v1[16];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 16; ++e) {
         const int tt = tt0 + e < nt ? tt0 + e : nt - 1;
         v0[e] = vr[(int64_t)tt * new_stride_tok + lane];
         v1[e] = vr[(int64_t)tt * new_stride_tok + lane + 64];
       }
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
+      for (int e = 0; e < 16; ++e) {
         if (tt0 + e < nt) {
 #pragma unroll
-          for (int h = 0; h < 8; ++h) {
-            if (h < G) {
-              const float w = __shfl(wt[h], tt0 + e, 64);
-              acc[h][0] += w * v0[e];
-              acc[h][1] += w * v1[e];
-            }
+          for (int h = 0; h < G; ++h) {
+            const float w = __shfl(wt[h], tt0 + e, 64);
+            acc[h][0] += w * v0[e];
+            acc[h][1] += w * v1[e];
           }
         }
       }
     }
   }
 #pragma unroll
-  for (int h = 0; h < 8; ++h) {
-    if (h < G) {
-      if (lane == 0) {
-        w_m[wave][h] = m_run[h];
-        w_l[wave][h] = l_run[h];
-      }
-      w_acc[wave][h][lane] = acc[h][0];
-      w_acc[wave][h][lane + 64] = acc[h][1];
+  for (int h = 0; h < G; ++h) {
+    if (lane == 0) {
+      w_m[wave][h] = m_run[h];
+      w_l[wave][h] = l_run[h];
     }
+    w_acc[wave][h][lane] = acc[h][0];
+    w_acc[wave][h][lane + 64] = acc[h][1];
   }
   __syncthreads();
   for (int i = tid; i < G * kD; i += kThreads) {
@@ -1055,9 +1062,21 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
   RDKV_REQUIRE(n_new == 0 || (k_new && v_new), "%s: null zone-C tensors", fn);
   RDKV_REQUIRE(((uintptr_t)k_new % 16) == 0 && new_stride_unit % 4 == 0 && new_stride_tok % 4 == 0,
                "%s: zone-C key rows must be 16-byte aligned", fn);
-  hipLaunchKernelGGL(merge_zone_c_kernel, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units,
-                     (const float *)workspace, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new,
-                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse);
+#define RDKV_LAUNCH_ZC(GT)                                                                                    \
+  hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
+                     (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new, \
+                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse)
+  switch (G) {
+    case 1: RDKV_LAUNCH_ZC(1); break;
+    case 2: RDKV_LAUNCH_ZC(2); break;
+    case 3: RDKV_LAUNCH_ZC(3); break;
+    case 4: RDKV_LAUNCH_ZC(4); break;
+    case 5: RDKV_LAUNCH_ZC(5); break;
+    case 6: RDKV_LAUNCH_ZC(6); break;
+    case 7: RDKV_LAUNCH_ZC(7); break;
+    default: RDKV_LAUNCH_ZC(8); break;
+  }
+#undef RDKV_LAUNCH_ZC
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

@@ -9,6 +9,20 @@ __device__ __forceinline__ float rdkv_load_as_float(const void *p, int dtype, in
   return __uint_as_float((uint32_t)reinterpret_cast<const uint16_t *>(p)[idx] << 16);
 }
 
+// The same value without a branch per storage type: two 16-bit loads that are always issued (the
+// halves of an fp32 element, or the 16-bit element twice) and a selection afterwards.  A run of
+// these loads is in flight together, where the branching form waits for each load in turn.
+__device__ __forceinline__ float rdkv_load_as_float_nobranch(const void *p, int dtype, int64_t idx) {
+  const uint16_t *h = reinterpret_cast<const uint16_t *>(p);
+  const bool f32 = dtype == RDKV_DTYPE_F32;
+  const int64_t e = f32 ? 2 * idx : idx;
+  const uint32_t lo = h[e], hi = h[e + (f32 ? 1 : 0)];
+  const float as32 = __uint_as_float((hi << 16) | lo);
+  const float as16 = (float)__builtin_bit_cast(_Float16, (uint16_t)lo);
+  const float asbf = __uint_as_float(lo << 16);
+  return f32 ? as32 : (dtype == RDKV_DTYPE_F16 ? as16 : asbf);
+}
+
 // fp32 -> bf16 bits, round to nearest even (NaN stays NaN)
 __device__ __forceinline__ uint16_t rdkv_float_to_bf16_bits(float v) {
   uint32_t u = __float_as_uint(v);
