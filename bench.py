@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-decode-loop", action="store_true",
+                    help="skip the whole-model greedy decode loop (random-weight Llama-3.1-8B-shaped model)")
     return ap.parse_args()
 
 
@@ -59,6 +61,48 @@ def time_region(fn, steps, torch):
     end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / steps
+
+
+def decode_loop_section(cfg, torch, dev, tokens=48):
+    """ms per generated token of ``fast_decode.greedy_decode_fast`` on a random-weight model of the
+    Llama-3.1-8B shape (32 layers, hidden 4096, 32 / 8 heads) over a packed cache of the
+    workload's shape: the whole-model figure the reference quotes for its loop (its only
+    published latency, triton_v_kernel.py:53-54).  Reported beside the headline, never as it."""
+    import time
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from rdkv_amd import fast_decode, packing, synth
+    L = 32
+    mcfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=L, num_attention_heads=cfg.H_q,
+                       num_key_value_heads=cfg.H_kv, head_dim=cfg.D, vocab_size=128256,
+                       max_position_embeddings=262144, rms_norm_eps=1e-5, rope_theta=500000.0,
+                       tie_word_embeddings=False)
+    torch.manual_seed(0)
+    with torch.device(dev):
+        model = LlamaForCausalLM(mcfg).half().eval()
+    sc = synth.scaled(cfg, layers=L)
+    layers, v16 = [], []
+    for i in range(L):
+        vb, kb, oc = synth.layer_allocation(sc, i)
+        K, V, _ = synth.layer_data(sc, i, dev, outliers=oc)
+        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, sc.G)
+        layers.append(pl)
+        v16.append(nvo)
+        del K, V
+    cache = packing.TriZoneCache(tuple(layers), v16, [None] * L, [None] * L, sc.context)
+    first = torch.randn(mcfg.vocab_size, device=dev)
+    res = {"model": "Llama-3.1-8B shape, random fp16 weights", "context": sc.context, "tokens": tokens}
+    for name, graph in (("eager", False), ("graph", True)):
+        best = None
+        for _ in range(2):          # the first run builds the streaming caches and warms the libraries
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ids = fast_decode.greedy_decode_fast(model, cache, first, tokens, [], dev, sc.context,
+                                                 use_cuda_graph=graph)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / max(len(ids), 1) * 1e3
+            best = dt if best is None else min(best, dt)
+        res[f"ms_per_token_{name}"] = best
+    return res
 
 
 def main():
@@ -332,6 +376,13 @@ def main():
                                   f"({layer_bytes} algorithmic bytes), 1 warm-up + 3 repeats, median",
                         "ms_per_layer": t_cpu * 1e3, "host_cpus": os.cpu_count()}
 
+    loop_info = None
+    if default_workload and args.config == 1 and not args.no_decode_loop:
+        try:
+            loop_info = decode_loop_section(cfg, torch, dev)
+        except Exception as e:  # informative section; never fail the benchmark on it
+            loop_info = {"error": repr(e)[:300]}
+
     result = {
         "metric": "packed decode-attn achieved HBM GB/s (algorithmic bytes / step time)",
         "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -369,6 +420,7 @@ def main():
                            speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None),
         "pack": pack_info,
         "select": select_info,
+        "decode_loop": loop_info,
         "check": check,
     }
     print(json.dumps(result))

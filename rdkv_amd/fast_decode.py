@@ -78,6 +78,25 @@ def _rope_append_kv(k_2d: torch.Tensor, v_2d: torch.Tensor, cos_half: torch.Tens
         new_kv_rows.stride(0), new_kv_rows.stride(1), row.data_ptr(), new_kv_rows.shape[1], _lib.stream_of(dev)))
 
 
+def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``F.linear(x, weight, bias)`` for the single activation row of a decode step
+    (fast_decode.py:1650-1656, 1786, 1797-1804, 1826): one pass over the weights with
+    ``rdkv_gemv`` when the shape allows it (fp16 / bf16, K a multiple of 512 up to 32768, 16-byte
+    aligned rows), the library GEMM otherwise."""
+    N, K = weight.shape
+    ok = (x.numel() == K and x.dtype == weight.dtype and x.dtype in (torch.float16, torch.bfloat16)
+          and K % 512 == 0 and K <= 32768 and weight.stride(1) == 1 and weight.stride(0) % 8 == 0
+          and weight.data_ptr() % 16 == 0 and x.is_contiguous() and x.data_ptr() % 16 == 0
+          and (bias is None or (bias.dtype == x.dtype and bias.is_contiguous())))
+    if not ok:
+        return F.linear(x, weight, bias)
+    dev = _lib.require_device(x, weight)
+    y = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=dev)
+    _lib.check(_lib.load().rdkv_gemv(weight.data_ptr(), weight.stride(0), x.data_ptr(), _lib.ptr(bias), N, K,
+                                     _lib.DTYPE_CODE[x.dtype], y.data_ptr(), _lib.stream_of(dev)))
+    return y
+
+
 def _silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """``F.silu(gate) * up`` (fast_decode.py:1803) in one launch; both [..., n] with unit stride."""
     dev = _lib.require_device(gate, up)
@@ -346,7 +365,7 @@ class _DecodeStep:
         delta = None                                                     # branch output not yet added to h
         for lw, cache, buf in zip(W.layers, self.caches, self.new_kv_buf):
             x = _rms_norm(h, lw.input_ln_weight, lw.input_ln_eps, delta=delta, residual_out=h)
-            q, k, v = F.linear(x, lw.qkv_weight, lw.qkv_bias).split(lw.qkv_split_sizes, dim=-1)
+            q, k, v = _linear_row(x, lw.qkv_weight, lw.qkv_bias).split(lw.qkv_split_sizes, dim=-1)
             q_2d, k_2d, v_2d = q.view(W.num_heads, D), k.view(W.num_kv_heads, D), v.view(W.num_kv_heads, D)
             if lw.q_norm_weight is not None:
                 q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
@@ -356,12 +375,12 @@ class _DecodeStep:
             _rope_append_kv(k_2d, v_2d, rope[0], rope[1], rows, self.write_row)
             decode_attn_fused(cache, q_2d, out=self.attn_out, lse=self.lse, rope=rope,   # q rotated while staged
                               zone_c=(rows[:, :, :D], rows[:, :, D:], self.n_new))
-            o = F.linear(self.attn_out.to(self.dtype).view(1, 1, W.attn_output_dim), lw.o_proj_weight)
+            o = _linear_row(self.attn_out.to(self.dtype).view(1, 1, W.attn_output_dim), lw.o_proj_weight)
             x = _rms_norm(h, lw.post_ln_weight, lw.post_ln_eps, delta=o, residual_out=h)
-            gate, up = F.linear(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
-            delta = F.linear(_silu_mul(gate, up), lw.down_proj_weight)
+            gate, up = _linear_row(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
+            delta = _linear_row(_silu_mul(gate, up), lw.down_proj_weight)
         self.hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
-        self.logits = F.linear(self.hidden, W.lm_head_weight)
+        self.logits = _linear_row(self.hidden, W.lm_head_weight)
         self.token.copy_(self.logits[:, -1, :].argmax(dim=-1, keepdim=True))
         self.position.add_(1)
         self.write_row.add_(1)

@@ -248,3 +248,27 @@ def test_step_kernels_match_tensor_expressions(dtype):
     assert float((buf[:, [0, 1, 2, 4]] - 7.0).abs().max()) == 0.0
     fast_decode._rope_append_kv(k, v, cs, sn, buf, torch.tensor([5], device=DEV))     # outside: nothing written
     assert float((buf[:, [0, 1, 2, 4]] - 7.0).abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_projection_row_kernel_matches_library(dtype):
+    """``_linear_row`` (one pass over the weights) against an fp64 product of the same values;
+    shapes of the decode step and the edges of the row partition (N below, at and off the
+    multiples of rows per wavefront; strided weight rows; bias)."""
+    require_gpu()
+    g = torch.Generator(device=DEV).manual_seed(9)
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    for N, K, with_bias in ((6144, 4096, False), (4096, 14336, False), (28672, 4096, True), (1, 512, True),
+                            (7, 512, False), (4099, 1024, True), (20000, 512, False)):
+        Wfull = (torch.randn(N, K + 8, generator=g, device=DEV) / K ** 0.5).to(dtype)
+        W = Wfull[:, :K]                                   # row stride K + 8
+        x = torch.randn(1, 1, K, generator=g, device=DEV).to(dtype)
+        b = torch.randn(N, generator=g, device=DEV).to(dtype) if with_bias else None
+        got = fast_decode._linear_row(x, W, b)
+        assert got.shape == (1, 1, N) and got.dtype == dtype
+        exp = x.double().view(1, K) @ W.double().T + (b.double() if b is not None else 0.0)
+        torch.testing.assert_close(got.double().view(1, N), exp, rtol=2 * ulp, atol=2 * ulp)
+    # shapes the kernel does not take go to the library
+    W = torch.randn(16, 100, generator=g, device=DEV).to(dtype)
+    x = torch.randn(1, 100, generator=g, device=DEV).to(dtype)
+    torch.testing.assert_close(fast_decode._linear_row(x, W), torch.nn.functional.linear(x, W))
