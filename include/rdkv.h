@@ -171,11 +171,12 @@ int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtype, void *
 
 /* fast_decode.py:1650-1656, 1786, 1797-1804, 1826: the projections of a decode step, each
  * F.linear on one activation row there.  y[n] = sum_k W[n,k] * x[k] (+ bias[n]); W [N, K] with
- * row stride w_stride_row (elements), x [K], bias [N] or NULL, y [N], all fp16 or all bf16
- * (`dtype`), fp32 accumulation in a fixed order.  K: a multiple of 512, at most 32768; W rows and
- * x 16-byte aligned. */
-int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, const void *bias, int N, int K,
-              int dtype, void *y, void *stream);
+ * row stride w_stride_row (elements), bias [N] or NULL, y [N], all fp16 or all bf16 (`dtype`);
+ * x [K] of x_dtype = `dtype`, or fp32 (then rounded to `dtype` first, as the cast the reference
+ * puts in front of the output projection stores it, fast_decode.py:1785); fp32 accumulation in
+ * a fixed order.  K: a multiple of 512, at most 32768; W rows and x 16-byte aligned. */
+int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x_dtype, const void *bias, int N,
+              int K, int dtype, void *y, void *stream);
 
 /* ---- triton_rope.py : fused_rope (:86-108) -------------------------------- */
 /* Half-split rotary embedding of one decode step, in place: for every head of q [H_q, D] and

@@ -36,13 +36,37 @@ __device__ __forceinline__ float dot8(const uint4 w, const uint4 x, float acc) {
 }
 
 // K % 512 == 0 (every lane takes whole 16-byte pieces: K / 512 per row), rows 16-byte aligned.
+// x32: x is fp32 and is rounded to the weights' type while it is staged (what a cast in front of
+// the product would store).
 template <int dtype, int R>
 __global__ void __launch_bounds__(256)
-gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, const uint16_t *__restrict__ x,
+gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, const void *__restrict__ x, int x32,
             const uint16_t *__restrict__ bias, int N, int K, int rows_per_wave, uint16_t *__restrict__ y) {
   extern __shared__ uint4 xs[];      // K / 8 pieces of x
   const int k8 = K >> 3;
-  for (int i = threadIdx.x; i < k8; i += 256) xs[i] = reinterpret_cast<const uint4 *>(x)[i];
+  if (x32) {
+    const float4 *xf = reinterpret_cast<const float4 *>(x);
+    for (int i = threadIdx.x; i < k8; i += 256) {
+      const float4 a = xf[2 * i], b = xf[2 * i + 1];
+      const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+      uint32_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        uint32_t lo, hi;
+        if (dtype == RDKV_DTYPE_F16) {
+          lo = __builtin_bit_cast(uint16_t, (_Float16)v[2 * j]);
+          hi = __builtin_bit_cast(uint16_t, (_Float16)v[2 * j + 1]);
+        } else {
+          lo = rdkv_float_to_bf16_bits(v[2 * j]);
+          hi = rdkv_float_to_bf16_bits(v[2 * j + 1]);
+        }
+        w[j] = lo | (hi << 16);
+      }
+      xs[i] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  } else {
+    for (int i = threadIdx.x; i < k8; i += 256) xs[i] = reinterpret_cast<const uint4 *>(x)[i];
+  }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int row_begin = wave * rows_per_wave;
@@ -84,8 +108,8 @@ gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, const uint16_t
 }
 
 template <int dtype>
-void launch_gemv(const void *W, int64_t w_stride_row, const void *x, const void *bias, int N, int K, void *y,
-                 int n_cu, hipStream_t s) {
+void launch_gemv(const void *W, int64_t w_stride_row, const void *x, int x32, const void *bias, int N, int K,
+                 void *y, int n_cu, hipStream_t s) {
   // eight wavefronts per compute unit when there are rows enough; a wavefront takes at least R rows
   const int max_waves = n_cu * 8;
   const int R = N >= 4 * max_waves ? 4 : 2;
@@ -97,19 +121,20 @@ void launch_gemv(const void *W, int64_t w_stride_row, const void *x, const void 
   const size_t lds = (size_t)K * 2;
   if (R == 4)
     hipLaunchKernelGGL((gemv_kernel<dtype, 4>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W, w_stride_row,
-                       (const uint16_t *)x, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
+                       x, x32, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
   else
     hipLaunchKernelGGL((gemv_kernel<dtype, 2>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W, w_stride_row,
-                       (const uint16_t *)x, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
+                       x, x32, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
 }
 
 }  // namespace
 
-RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, const void *bias, int N, int K,
-                       int dtype, void *y, void *stream) {
+RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x_dtype, const void *bias, int N,
+                       int K, int dtype, void *y, void *stream) {
   const char *fn = "rdkv_gemv";
   RDKV_REQUIRE(N >= 0 && K > 0, "%s: bad shape N=%d K=%d", fn, N, K);
   RDKV_REQUIRE(dtype == RDKV_DTYPE_F16 || dtype == RDKV_DTYPE_BF16, "%s: fp16 or bf16 weights only", fn);
+  RDKV_REQUIRE(x_dtype == dtype || x_dtype == RDKV_DTYPE_F32, "%s: x must have the weights' type or be fp32", fn);
   RDKV_REQUIRE(K % 512 == 0 && K <= 32768, "%s: K=%d must be a multiple of 512, at most 32768", fn, K);
   if (N == 0) return RDKV_OK;
   RDKV_REQUIRE(W && x && y, "%s: null pointer", fn);
@@ -120,8 +145,8 @@ RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, const
     int v = 0;
     if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n_cu = v;
   }
-  if (dtype == RDKV_DTYPE_F16) launch_gemv<RDKV_DTYPE_F16>(W, w_stride_row, x, bias, N, K, y, n_cu, (hipStream_t)stream);
-  else launch_gemv<RDKV_DTYPE_BF16>(W, w_stride_row, x, bias, N, K, y, n_cu, (hipStream_t)stream);
+  if (dtype == RDKV_DTYPE_F16) launch_gemv<RDKV_DTYPE_F16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
+  else launch_gemv<RDKV_DTYPE_BF16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

@@ -79,21 +79,24 @@ def _rope_append_kv(k_2d: torch.Tensor, v_2d: torch.Tensor, cos_half: torch.Tens
 
 
 def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """``F.linear(x, weight, bias)`` for the single activation row of a decode step
-    (fast_decode.py:1650-1656, 1786, 1797-1804, 1826): one pass over the weights with
-    ``rdkv_gemv`` when the shape allows it (fp16 / bf16, K a multiple of 512 up to 32768, 16-byte
-    aligned rows), the library GEMM otherwise."""
+    """``F.linear(x.to(weight.dtype), weight, bias)`` for the single activation row of a decode
+    step (fast_decode.py:1650-1656, 1785-1786, 1797-1804, 1826): one pass over the weights with
+    ``rdkv_gemv`` when the shape allows it (fp16 / bf16 weights, K a multiple of 512 up to 32768,
+    16-byte aligned rows; x of the weights' type or fp32, which the kernel rounds while staging
+    it), the library GEMM otherwise."""
     N, K = weight.shape
-    ok = (x.numel() == K and x.dtype == weight.dtype and x.dtype in (torch.float16, torch.bfloat16)
+    ok = (x.numel() == K and x.dtype in (weight.dtype, torch.float32)
+          and weight.dtype in (torch.float16, torch.bfloat16)
           and K % 512 == 0 and K <= 32768 and weight.stride(1) == 1 and weight.stride(0) % 8 == 0
           and weight.data_ptr() % 16 == 0 and x.is_contiguous() and x.data_ptr() % 16 == 0
-          and (bias is None or (bias.dtype == x.dtype and bias.is_contiguous())))
+          and (bias is None or (bias.dtype == weight.dtype and bias.is_contiguous())))
     if not ok:
-        return F.linear(x, weight, bias)
+        return F.linear(x.to(weight.dtype), weight, bias)
     dev = _lib.require_device(x, weight)
-    y = torch.empty(x.shape[:-1] + (N,), dtype=x.dtype, device=dev)
-    _lib.check(_lib.load().rdkv_gemv(weight.data_ptr(), weight.stride(0), x.data_ptr(), _lib.ptr(bias), N, K,
-                                     _lib.DTYPE_CODE[x.dtype], y.data_ptr(), _lib.stream_of(dev)))
+    y = torch.empty(x.shape[:-1] + (N,), dtype=weight.dtype, device=dev)
+    _lib.check(_lib.load().rdkv_gemv(weight.data_ptr(), weight.stride(0), x.data_ptr(), _lib.DTYPE_CODE[x.dtype],
+                                     _lib.ptr(bias), N, K, _lib.DTYPE_CODE[weight.dtype], y.data_ptr(),
+                                     _lib.stream_of(dev)))
     return y
 
 
@@ -332,10 +335,11 @@ class _DecodeStep:
     """One greedy decode step over device-resident state, written so that the same calls run
     eagerly or are captured once into a HIP graph: the token, its position, the zone C write row
     and the zone C token counts live in device tensors that the step itself advances, so a replay
-    needs no argument from the host.  Per layer, eleven launches: residual add + RMSNorm, one q/k/v
+    needs no argument from the host.  Per layer, ten launches: residual add + RMSNorm, one q/k/v
     GEMV, rotary embedding of k + append of the fp32 K|V row to zone C, zones A+B+C attention
-    (two launches, q rotated while the kernel stages it), a cast, output projection, residual add +
-    RMSNorm, gate/up GEMV, SiLU * up, down projection."""
+    (two launches, q rotated while the kernel stages it), output projection (its fp32 input rounded
+    to the model type while it is staged), residual add + RMSNorm, gate/up GEMV, SiLU * up, down
+    projection."""
 
     def __init__(self, W: PreExtractedWeights, caches: List[StreamCache], new_kv_buf: List[torch.Tensor],
                  dtype: torch.dtype):
@@ -375,7 +379,7 @@ class _DecodeStep:
             _rope_append_kv(k_2d, v_2d, rope[0], rope[1], rows, self.write_row)
             decode_attn_fused(cache, q_2d, out=self.attn_out, lse=self.lse, rope=rope,   # q rotated while staged
                               zone_c=(rows[:, :, :D], rows[:, :, D:], self.n_new))
-            o = _linear_row(self.attn_out.to(self.dtype).view(1, 1, W.attn_output_dim), lw.o_proj_weight)
+            o = _linear_row(self.attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)     # fp32 in, rounded inside
             x = _rms_norm(h, lw.post_ln_weight, lw.post_ln_eps, delta=o, residual_out=h)
             gate, up = _linear_row(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
             delta = _linear_row(_silu_mul(gate, up), lw.down_proj_weight)

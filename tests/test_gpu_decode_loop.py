@@ -268,6 +268,9 @@ def test_projection_row_kernel_matches_library(dtype):
         assert got.shape == (1, 1, N) and got.dtype == dtype
         exp = x.double().view(1, K) @ W.double().T + (b.double() if b is not None else 0.0)
         torch.testing.assert_close(got.double().view(1, N), exp, rtol=2 * ulp, atol=2 * ulp)
+        # an fp32 row is rounded to the weights' type inside: the same bits as casting it first
+        x32 = torch.randn(1, 1, K, generator=g, device=DEV)
+        assert torch.equal(fast_decode._linear_row(x32, W, b), fast_decode._linear_row(x32.to(dtype), W, b))
     # shapes the kernel does not take go to the library
     W = torch.randn(16, 100, generator=g, device=DEV).to(dtype)
     x = torch.randn(1, 100, generator=g, device=DEV).to(dtype)
