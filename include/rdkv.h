@@ -228,7 +228,9 @@ typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgro
  * descriptors (device).  n2p/n4p: padded 2-/4-bit channel counts of the source layout.
  * perm (int64, head stride in elements, 0 = one table for all heads), kscale / kzp (fp16, head
  * stride ks_stride_h): the layer's K_ch_perm_padded_idx, K_ch_scale and K_ch_zp, from which the
- * unit's slot table (RdkvSlot per stream slot, at qtab_off) is written. */
+ * unit's slot table (RdkvSlot per stream slot, at qtab_off) is written.  n8: bytes per K8 row;
+ * max_tiles: the largest number of 64-token tiles (all classes) of any of the layer's units (one
+ * workgroup per tile and head, the tile's source rows staged through LDS). */
 int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
                                const uint8_t *K4, int64_t k4_stride_h, int64_t k4_stride_t,
                                const uint8_t *K8, int64_t k8_stride_h, int64_t k8_stride_t,
@@ -240,7 +242,7 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
                                const void *V16_f16, int64_t v16_stride_h, int64_t max_T_v,
                                const int64_t *perm, int64_t perm_stride_h, const void *kscale_f16,
                                const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
-                               int H_kv, uint8_t *blob, void *stream);
+                               int H_kv, int n8, int max_tiles, uint8_t *blob, void *stream);
 
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit

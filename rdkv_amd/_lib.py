@@ -50,7 +50,7 @@ SIGNATURES = {
     "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
     "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,
-                                       P, L, P, P, L, P, P, I, I, P, P]),
+                                       P, L, P, P, L, P, P, I, I, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),
     "rdkv_decode_fused": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P, P, L, P]),
     "rdkv_decode_fused_partials": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P]),

@@ -1,6 +1,6 @@
 // Re-lays one packed layer (the reference's padded tensors, obkv_accel/packing.py:43-111) into
-// the streaming format defined in stream_format.h.  One thread per output dword; pure
-// byte/bit shuffling.  Runs once per prompt cache, so it is written for clarity.
+// the streaming format defined in stream_format.h: pure byte / bit shuffling, one workgroup per
+// 64-token tile with the tile's source rows staged through LDS.
 #include "rdkv_common.h"
 #include "stream_format.h"
 
@@ -23,118 +23,60 @@ struct SrcLayer {
   int64_t ks_sh;
 };
 
-__device__ __forceinline__ uint32_t k_code(const SrcLayer &S, int h, int64_t row, int src) {
-  if (src < 0) return 0u;
-  if (src < S.n2p) {
-    const int sub = S.n2p >> 2;
-    const uint32_t b = S.K2[h * S.k2_sh + row * S.k2_st + (src % sub)];
-    return (b >> (2 * (src / sub))) & 3u;
-  }
-  src -= S.n2p;
-  if (src < S.n4p) {
-    const int sub = S.n4p >> 1;
-    const uint32_t b = S.K4[h * S.k4_sh + row * S.k4_st + (src % sub)];
-    return (b >> (4 * (src / sub))) & 15u;
-  }
-  return S.K8[h * S.k8_sh + row * S.k8_st + (src - S.n4p)];
+// Copies n bytes from global memory to LDS with 16-byte loads.  dst must be congruent to src
+// modulo 16; the unaligned head and tail (at most 15 bytes each) go byte by byte.
+__device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *__restrict__ src, int n) {
+  const int head = (int)((16 - ((uintptr_t)src & 15)) & 15);
+  const int h = head < n ? head : n;
+  const int body = (n - h) >> 4, tail = (n - h) & 15;
+  const uint4 *s16 = reinterpret_cast<const uint4 *>(src + h);
+  uint4 *d16 = reinterpret_cast<uint4 *>(dst + h);
+  for (int i = threadIdx.x; i < body; i += 256) d16[i] = s16[i];
+  if ((int)threadIdx.x < h) dst[threadIdx.x] = src[threadIdx.x];
+  if ((int)threadIdx.x < tail) dst[h + 16 * body + threadIdx.x] = src[h + 16 * body + threadIdx.x];
 }
 
-__device__ __forceinline__ uint32_t v_code(const SrcLayer &S, int h, int cls, int64_t tok, int ch) {
-  if (cls == 0) return (S.V2[h * S.v2_sh + tok * 32 + (ch & 31)] >> (2 * (ch >> 5))) & 3u;
-  if (cls == 1) return (S.V4[h * S.v4_sh + tok * 64 + (ch & 63)] >> (4 * (ch >> 6))) & 15u;
-  return S.V8[h * S.v8_sh + tok * 128 + ch];
+// Stages rows [0, nrows) of row_bytes bytes each into the 16-byte aligned LDS region `area` and
+// returns where row 0 landed; rows follow each other row_bytes apart there.  Rows stored back to
+// back in memory go as one run of 16-byte loads, strided rows byte by byte.
+__device__ __forceinline__ const uint8_t *stage_rows(uint8_t *area, const uint8_t *__restrict__ src,
+                                                     int row_bytes, int64_t stride, int nrows) {
+  if (row_bytes == 0 || nrows == 0) return area;
+  if (stride == row_bytes) {
+    uint8_t *dst = area + ((uintptr_t)src & 15);
+    stage_bytes(dst, src, nrows * row_bytes);
+    return dst;
+  }
+  for (int i = threadIdx.x; i < nrows * row_bytes; i += 256) {
+    const int t = i / row_bytes, j = i - t * row_bytes;
+    area[i] = src[t * stride + j];
+  }
+  return area;
 }
 
+// where the code of one stream slot sits in the staged K rows of a tile
+struct SlotSrc {
+  uint16_t base;    // byte offset of (row 0, the slot's byte) from the start of the staged K rows
+  uint16_t pitch;   // bytes between rows of the slot's segment
+  uint8_t shift, mask;
+};
+
+// One workgroup per (64-token tile, KV head); block x == max_tiles writes the head's slot table.
+// The tile's source rows (the packed K rows of its 64 tokens, the V rows of its width class) are
+// staged in LDS with wide loads; every thread then assembles output dwords field by field from
+// LDS and the workgroup writes the tile's K part, V part and scale / zero-point pairs coalesced.
 __global__ void __launch_bounds__(256)
-relayout_kernel(SrcLayer S, const RdkvUnit *__restrict__ units, const int16_t *__restrict__ src_slot,
-                int n_slots_max, uint8_t *__restrict__ blob) {
+relayout_kernel(SrcLayer S, int n8, const RdkvUnit *__restrict__ units, const int16_t *__restrict__ src_slot,
+                int n_slots_max, int max_tiles, uint8_t *__restrict__ blob) {
+  extern __shared__ __align__(16) uint8_t lds[];
   const int h = blockIdx.y;
   const RdkvUnit u = units[h];
   const int R = u.d8 + u.d4 + u.d2;
-  int tiles[4], tstart[4];
-  int nt = 0;
-  for (int c = 0; c < 4; ++c) {
-    tstart[c] = nt;
-    tiles[c] = (u.n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
-    nt += tiles[c];
-  }
-  // source row of token 0 of each class: quantized classes are contiguous from row 0,
-  // zone B starts at max_T_v (packing.py:1035-1046)
-  const int64_t srow0[4] = {0, u.n_tok[0], (int64_t)u.n_tok[0] + u.n_tok[1], S.max_T_v};
+  const int n_slots = 4 * (u.d8 + 2 * u.d4 + 4 * u.d2);
   const int16_t *slots = src_slot + (int64_t)h * n_slots_max;
-  const int64_t k_dw = (int64_t)nt * RDKV_TILE * R;
-  int64_t v_dw[4];
-  for (int c = 0; c < 4; ++c) v_dw[c] = (int64_t)tiles[c] * (rdkv_v_tile_bytes(c) / 4);
-  const int64_t sz_dw = (int64_t)(tstart[3]) * RDKV_TILE;
-  const int64_t qt_dw = 2 * 4 * (int64_t)(u.d8 + 2 * u.d4 + 4 * u.d2);   // RdkvSlot = 2 dwords
-  const int64_t total = k_dw + v_dw[0] + v_dw[1] + v_dw[2] + v_dw[3] + sz_dw + qt_dw;
 
-  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (int64_t)gridDim.x * blockDim.x) {
-    int64_t i = idx;
-    if (i < k_dw) {  // ---- K tile dword
-      const int ti = (int)(i / (RDKV_TILE * R));
-      int rem = (int)(i % (RDKV_TILE * R));
-      int c = rem / 256, wc = 4;
-      if (c >= R / 4) { c = R / 4; wc = R % 4; }
-      rem -= c * 256;
-      const int t = rem / wc, j = 4 * c + rem % wc;
-      int cls = 0;
-      while (cls < 3 && ti >= tstart[cls + 1]) ++cls;
-      const int tk = (ti - tstart[cls]) * RDKV_TILE + t;
-      uint32_t w = 0;
-      if (tk < u.n_tok[cls]) {
-        const int64_t row = srow0[cls] + tk;
-        int nf, step0;
-        if (j < u.d8) { nf = 4; step0 = j; }
-        else if (j < u.d8 + u.d4) { nf = 8; step0 = u.d8 + 2 * (j - u.d8); }
-        else { nf = 16; step0 = u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4); }
-        const int fw = 32 / nf;
-        for (int f = 0; f < nf; ++f) {
-          int s, k;
-          rdkv_operand_of(f, nf, &s, &k);
-          w |= k_code(S, h, row, slots[4 * (step0 + s) + k]) << (fw * f);
-        }
-      }
-      *reinterpret_cast<uint32_t *>(blob + u.k_off + 4 * i) = w;
-      continue;
-    }
-    i -= k_dw;
-    int cls = 0;
-    while (cls < 4 && i >= v_dw[cls]) { i -= v_dw[cls]; ++cls; }
-    if (cls < 4) {  // ---- V tile dword
-      const int per_tile = rdkv_v_tile_bytes(cls) / 4;
-      const int tl = (int)(i / per_tile);
-      const int rem = (int)(i % per_tile);
-      const int l = (rem >> 2) & 63;
-      const int di = ((rem >> 8) << 2) | (rem & 3);  // lane dword index
-      const int64_t tok0 = (int64_t)tl * RDKV_TILE;
-      const int n = u.n_tok[cls];
-      uint32_t w = 0;
-      if (cls == 3) {
-        const int quad = di >> 2, j = (di >> 1) & 1, kk = (di & 1) * 2;
-        for (int e = 0; e < 2; ++e) {
-          const int64_t tok = tok0 + 4 * quad + kk + e;
-          if (tok < n) w |= (uint32_t)S.V16[h * S.v16_sh + tok * 128 + l + 64 * j] << (16 * e);
-        }
-      } else {
-        const int nf = cls == 2 ? 4 : (cls == 1 ? 8 : 16);
-        const int fw = 32 / nf;
-        for (int f = 0; f < nf; ++f) {
-          int s, k, quad, j;
-          rdkv_operand_of(f, nf, &s, &k);
-          if (cls == 2) { quad = di >> 1; j = di & 1; }
-          else if (cls == 1) { quad = di; j = s; }
-          else { quad = 2 * di + (s >> 1); j = s & 1; }
-          const int64_t tok = tok0 + 4 * quad + k;
-          if (tok < n) w |= v_code(S, h, cls, tok, l + 64 * j) << (fw * f);
-        }
-      }
-      *reinterpret_cast<uint32_t *>(blob + u.v_off[cls] + 4 * i) = w;
-      continue;
-    }
-    if (i >= sz_dw) {  // ---- slot table: {channel, scale, zp, 0} per stream slot
-      i -= sz_dw;
+  if ((int)blockIdx.x == max_tiles) {   // ---- slot table: {channel, scale, zp, 0} per stream slot
+    for (int i = threadIdx.x; i < 2 * n_slots; i += 256) {
       const int r = slots[i >> 1];
       uint32_t w = 0;
       if (r >= 0) {
@@ -143,22 +85,133 @@ relayout_kernel(SrcLayer S, const RdkvUnit *__restrict__ units, const int16_t *_
         else
           w = (uint32_t)S.kzp[h * S.ks_sh + r];
       }
-      *reinterpret_cast<uint32_t *>(blob + u.qtab_off + 4 * i) = w;
-      continue;
+      *reinterpret_cast<uint32_t *>(blob + u.qtab_off + 4 * (int64_t)i) = w;
     }
-    // ---- per-token {scale, zp}
-    {
-      const int ti = (int)(i / RDKV_TILE), t = (int)(i % RDKV_TILE);
-      int c = 0;
-      while (c < 2 && ti >= tstart[c + 1]) ++c;
-      const int tk = (ti - tstart[c]) * RDKV_TILE + t;
-      uint32_t w = 0;
-      if (tk < u.n_tok[c]) {
-        const int64_t row = srow0[c] + tk;
-        w = (uint32_t)S.vscale[h * S.vs_sh + row] | ((uint32_t)S.vzp[h * S.vs_sh + row] << 16);
+    return;
+  }
+
+  int tstart[5];
+  tstart[0] = 0;
+  for (int c = 0; c < 4; ++c) tstart[c + 1] = tstart[c] + (u.n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
+  const int ti = blockIdx.x;
+  if (ti >= tstart[4]) return;
+  int cls = 0;
+  while (cls < 3 && ti >= tstart[cls + 1]) ++cls;
+  const int tl = ti - tstart[cls];                              // tile of its class
+  const int tk0 = tl * RDKV_TILE;
+  const int nv = min(RDKV_TILE, u.n_tok[cls] - tk0);            // valid tokens of the tile (>= 1)
+  // source row of token 0 of each class: quantized classes are contiguous from row 0,
+  // zone B starts at max_T_v (packing.py:1035-1046)
+  const int64_t srow0[4] = {0, u.n_tok[0], (int64_t)u.n_tok[0] + u.n_tok[1], S.max_T_v};
+  const int64_t row0 = srow0[cls] + tk0;
+
+  // LDS: [slot sources | K2 rows | K4 rows | K8 rows | V rows], every region 16-byte aligned + slack
+  const int sub2 = S.n2p >> 2, sub4 = S.n4p >> 1;
+  auto region = [](int bytes) { return ((bytes + 15) & ~15) + 16; };
+  SlotSrc *ssrc = reinterpret_cast<SlotSrc *>(lds);
+  uint8_t *a_k2 = lds + region(n_slots_max * (int)sizeof(SlotSrc));
+  uint8_t *a_k4 = a_k2 + region(RDKV_TILE * sub2);
+  uint8_t *a_k8 = a_k4 + region(RDKV_TILE * sub4);
+  uint8_t *a_v = a_k8 + region(RDKV_TILE * n8);
+  const uint8_t *l_k2 = stage_rows(a_k2, S.K2 ? S.K2 + h * S.k2_sh + row0 * S.k2_st : nullptr, S.K2 ? sub2 : 0, S.k2_st, nv);
+  const uint8_t *l_k4 = stage_rows(a_k4, S.K4 ? S.K4 + h * S.k4_sh + row0 * S.k4_st : nullptr, S.K4 ? sub4 : 0, S.k4_st, nv);
+  const uint8_t *l_k8 = stage_rows(a_k8, S.K8 ? S.K8 + h * S.k8_sh + row0 * S.k8_st : nullptr, S.K8 ? n8 : 0, S.k8_st, nv);
+  const int v_row = 32 << cls;                                   // bytes per token: 32 / 64 / 128 / 256
+  const uint8_t *v_src = cls == 0 ? S.V2 + h * S.v2_sh : (cls == 1 ? S.V4 + h * S.v4_sh : (cls == 2 ? S.V8 + h * S.v8_sh
+                         : reinterpret_cast<const uint8_t *>(S.V16 + h * S.v16_sh)));
+  const uint8_t *l_v = stage_rows(a_v, v_src + (int64_t)tk0 * v_row, v_row, v_row, nv);
+  for (int i = threadIdx.x; i < n_slots; i += 256) {
+    int src = slots[i];
+    SlotSrc e = {0, 0, 0, 0};
+    if (src >= 0) {
+      if (src < S.n2p) {
+        e.base = (uint16_t)((l_k2 - lds) + src % sub2);
+        e.pitch = (uint16_t)sub2;
+        e.shift = (uint8_t)(2 * (src / sub2));
+        e.mask = 3;
+      } else if (src < S.n2p + S.n4p) {
+        src -= S.n2p;
+        e.base = (uint16_t)((l_k4 - lds) + src % sub4);
+        e.pitch = (uint16_t)sub4;
+        e.shift = (uint8_t)(4 * (src / sub4));
+        e.mask = 15;
+      } else {
+        e.base = (uint16_t)((l_k8 - lds) + (src - S.n2p - S.n4p));
+        e.pitch = (uint16_t)n8;
+        e.mask = 255;
       }
-      *reinterpret_cast<uint32_t *>(blob + u.sz_off + 4 * i) = w;
     }
+    ssrc[i] = e;
+  }
+  __syncthreads();
+
+  // ---- K tile: 64 rows of R dwords, chunks of up to four dwords per token
+  uint32_t *k_out = reinterpret_cast<uint32_t *>(blob + u.k_off) + (int64_t)ti * RDKV_TILE * R;
+  for (int rem0 = threadIdx.x; rem0 < RDKV_TILE * R; rem0 += 256) {
+    int rem = rem0;
+    int c = rem / 256, wc = 4;
+    if (c >= R / 4) { c = R / 4; wc = R % 4; }
+    rem -= c * 256;
+    const int t = rem / wc, j = 4 * c + rem % wc;
+    uint32_t w = 0;
+    if (t < nv) {
+      int nf, step0;
+      if (j < u.d8) { nf = 4; step0 = j; }
+      else if (j < u.d8 + u.d4) { nf = 8; step0 = u.d8 + 2 * (j - u.d8); }
+      else { nf = 16; step0 = u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4); }
+      const int fw = 32 / nf;
+      for (int f = 0; f < nf; ++f) {
+        int s, k;
+        rdkv_operand_of(f, nf, &s, &k);
+        const SlotSrc e = ssrc[4 * (step0 + s) + k];
+        w |= (uint32_t)((lds[e.base + t * e.pitch] >> e.shift) & e.mask) << (fw * f);
+      }
+    }
+    k_out[rem0] = w;
+  }
+
+  // ---- V tile of the class
+  const int per_tile = rdkv_v_tile_bytes(cls) / 4;
+  uint32_t *v_out = reinterpret_cast<uint32_t *>(blob + u.v_off[cls]) + (int64_t)tl * per_tile;
+  for (int rem = threadIdx.x; rem < per_tile; rem += 256) {
+    const int l = (rem >> 2) & 63;
+    const int di = ((rem >> 8) << 2) | (rem & 3);  // lane dword index
+    uint32_t w = 0;
+    if (cls == 3) {
+      const int quad = di >> 2, j = (di >> 1) & 1, kk = (di & 1) * 2;
+      const uint16_t *rows = reinterpret_cast<const uint16_t *>(l_v);
+      for (int e = 0; e < 2; ++e) {
+        const int t = 4 * quad + kk + e;
+        if (t < nv) w |= (uint32_t)rows[t * 128 + l + 64 * j] << (16 * e);
+      }
+    } else {
+      const int nf = cls == 2 ? 4 : (cls == 1 ? 8 : 16);
+      const int fw = 32 / nf;
+      for (int f = 0; f < nf; ++f) {
+        int s, k, quad, j;
+        rdkv_operand_of(f, nf, &s, &k);
+        if (cls == 2) { quad = di >> 1; j = di & 1; }
+        else if (cls == 1) { quad = di; j = s; }
+        else { quad = 2 * di + (s >> 1); j = s & 1; }
+        const int t = 4 * quad + k, ch = l + 64 * j;
+        if (t < nv) {
+          uint32_t code;
+          if (cls == 0) code = (l_v[t * 32 + (ch & 31)] >> (2 * (ch >> 5))) & 3u;
+          else if (cls == 1) code = (l_v[t * 64 + (ch & 63)] >> (4 * (ch >> 6))) & 15u;
+          else code = l_v[t * 128 + ch];
+          w |= code << (fw * f);
+        }
+      }
+    }
+    v_out[rem] = w;
+  }
+
+  // ---- per-token {scale, zp} of a quantized tile
+  if (cls < 3 && threadIdx.x < RDKV_TILE) {
+    const int t = threadIdx.x;
+    uint32_t w = 0;
+    if (t < nv) w = (uint32_t)S.vscale[h * S.vs_sh + row0 + t] | ((uint32_t)S.vzp[h * S.vs_sh + row0 + t] << 16);
+    *reinterpret_cast<uint32_t *>(blob + u.sz_off + 4 * ((int64_t)ti * RDKV_TILE + t)) = w;
   }
 }
 
@@ -173,7 +226,7 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
                                         const void *V16_f16, int64_t v16_stride_h, int64_t max_T_v,
                                         const int64_t *perm, int64_t perm_stride_h, const void *kscale_f16,
                                         const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
-                                        int H_kv, uint8_t *blob, void *stream) {
+                                        int H_kv, int n8, int max_tiles, uint8_t *blob, void *stream) {
   RDKV_REQUIRE(H_kv > 0 && units && src_slot && n_slots_max > 0, "rdkv_stream_relayout_layer: bad arguments");
   RDKV_REQUIRE(perm && kscale_f16 && kzp_f16, "rdkv_stream_relayout_layer: null channel tables");
   RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
@@ -191,8 +244,15 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
   S.max_T_v = max_T_v;
   S.perm = perm; S.perm_sh = perm_stride_h;
   S.kscale = (const uint16_t *)kscale_f16; S.kzp = (const uint16_t *)kzp_f16; S.ks_sh = ks_stride_h;
-  hipLaunchKernelGGL(relayout_kernel, dim3(1024, H_kv), dim3(256), 0, (hipStream_t)stream, S, units, src_slot,
-                     n_slots_max, blob);
+  RDKV_REQUIRE(n8 >= 0 && max_tiles >= 0 && n_slots_max <= 4 * RDKV_MAX_STEPS,
+               "rdkv_stream_relayout_layer: bad n8 / max_tiles / slot count");
+  auto region = [](int64_t bytes) { return ((bytes + 15) & ~(int64_t)15) + 16; };
+  const int64_t lds = region((int64_t)n_slots_max * (int64_t)sizeof(SlotSrc)) + region(RDKV_TILE * (n2p / 4)) +
+                      region(RDKV_TILE * (n4p / 2)) + region((int64_t)RDKV_TILE * n8) + region(RDKV_TILE * 256);
+  RDKV_REQUIRE(lds <= 64 * 1024, "rdkv_stream_relayout_layer: K rows of %d bytes do not fit the staging area",
+               n2p / 4 + n4p / 2 + n8);
+  hipLaunchKernelGGL(relayout_kernel, dim3(max_tiles + 1, H_kv), dim3(256), (size_t)lds, (hipStream_t)stream, S, n8,
+                     units, src_slot, n_slots_max, max_tiles, blob);
   RDKV_CHECK_LAUNCH("rdkv_stream_relayout_layer");
   return RDKV_OK;
 }

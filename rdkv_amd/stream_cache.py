@@ -226,6 +226,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
         units = np.zeros(H_kv, dtype=UNIT_DTYPE)
         src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
         off = 0
+        max_tiles = 0
         for h in range(H_kv):
             n_tok = tok[h]
             c2, c4, c8 = ch[h]
@@ -235,6 +236,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
             src_tab[h, :len(src)] = src
             qt_nbytes = len(src) * SLOT_DTYPE.itemsize
             tiles = [-(-n // TILE) for n in n_tok]
+            max_tiles = max(max_tiles, sum(tiles))
             R = d8 + d4 + d2
             u = units[h]
             u["n_tok"] = n_tok
@@ -294,7 +296,8 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
             _lib.ptr(vs), _lib.ptr(vz), vs.stride(0) if vs.numel() else 0,
             _lib.ptr(V16), v16h, int(pl.T_eff),
             perm.data_ptr(), perm_sh, ks.data_ptr(), kz.data_ptr(), ks.stride(0),
-            rel_units.data_ptr(), src_dev.data_ptr(), src_tab.shape[1], H_kv, blob.data_ptr(), stream))
+            rel_units.data_ptr(), src_dev.data_ptr(), src_tab.shape[1], H_kv, m8, max_tiles, blob.data_ptr(),
+            stream))
         # kernel-side descriptors carry absolute addresses
         for name in ("k_off", "sz_off", "qtab_off"):
             units[name] += base
