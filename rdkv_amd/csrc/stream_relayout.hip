@@ -54,12 +54,72 @@ __device__ __forceinline__ const uint8_t *stage_rows(uint8_t *area, const uint8_
   return area;
 }
 
-// where the code of one stream slot sits in the staged K rows of a tile
-struct SlotSrc {
-  uint16_t base;    // byte offset of (row 0, the slot's byte) from the start of the staged K rows
-  uint16_t pitch;   // bytes between rows of the slot's segment
-  uint8_t shift, mask;
-};
+// Where the code of one stream slot sits in the staged K rows of a tile, in one dword:
+// bits 0-15 byte offset of (row 0, the slot's byte) in LDS, 16-23 bytes between rows of the slot's
+// segment, 24-27 shift, 28-31 field width in bits (0 for a pad slot: the code is then 0).
+__device__ __forceinline__ uint32_t slot_src(uint32_t base, uint32_t pitch, uint32_t shift, uint32_t width) {
+  return base | (pitch << 16) | (shift << 24) | (width << 28);
+}
+__device__ __forceinline__ uint32_t slot_code(const uint8_t *lds, uint32_t e, int t) {
+  const uint32_t byte = lds[(e & 0xffffu) + t * ((e >> 16) & 0xffu)];
+  return (byte >> ((e >> 24) & 15u)) & ((1u << (e >> 28)) - 1u);
+}
+
+// one K dword of NF fields: field f is element k of operand s (stream_format.h), whose slot is
+// 4 * (step0 + s) + k
+template <int NF>
+__device__ __forceinline__ uint32_t k_dword(const uint8_t *lds, const uint32_t *ssrc, int step0, int t) {
+  uint32_t w = 0;
+#pragma unroll
+  for (int f = 0; f < NF; ++f) {
+    constexpr int half = NF / 2;
+    const int hi = f >= half, r = f - hi * half;
+    const int s = r >> 1, k = ((r & 1) << 1) | hi;
+    w |= slot_code(lds, ssrc[4 * (step0 + s) + k], t) << ((32 / NF) * f);
+  }
+  return w;
+}
+
+// the V tile of class CLS (stream_format.h): lane l owns channels l and l + 64
+template <int CLS>
+__device__ __forceinline__ void v_tile(const uint8_t *l_v, int nv, uint32_t *v_out) {
+  constexpr int per_tile = 512 << CLS;
+  for (int rem = threadIdx.x; rem < per_tile; rem += 256) {
+    const int l = (rem >> 2) & 63;
+    const int di = ((rem >> 8) << 2) | (rem & 3);  // lane dword index
+    uint32_t w = 0;
+    if (CLS == 3) {
+      const int quad = di >> 2, j = (di >> 1) & 1, kk = (di & 1) * 2;
+      const uint16_t *rows = reinterpret_cast<const uint16_t *>(l_v);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const int t = 4 * quad + kk + e;
+        if (t < nv) w |= (uint32_t)rows[t * 128 + l + 64 * j] << (16 * e);
+      }
+    } else {
+      constexpr int NF = CLS == 2 ? 4 : (CLS == 1 ? 8 : 16);
+      constexpr int half = NF / 2;
+#pragma unroll
+      for (int f = 0; f < NF; ++f) {
+        const int hi = f >= half, r = f - hi * half;
+        const int s = r >> 1, k = ((r & 1) << 1) | hi;
+        int quad, j;
+        if (CLS == 2) { quad = di >> 1; j = di & 1; }
+        else if (CLS == 1) { quad = di; j = s; }
+        else { quad = 2 * di + (s >> 1); j = s & 1; }
+        const int t = 4 * quad + k, ch = l + 64 * j;
+        if (t < nv) {
+          uint32_t code;
+          if (CLS == 0) code = (l_v[t * 32 + (ch & 31)] >> (2 * (ch >> 5))) & 3u;
+          else if (CLS == 1) code = (l_v[t * 64 + (ch & 63)] >> (4 * (ch >> 6))) & 15u;
+          else code = l_v[t * 128 + ch];
+          w |= code << ((32 / NF) * f);
+        }
+      }
+    }
+    v_out[rem] = w;
+  }
+}
 
 // One workgroup per (64-token tile, KV head); block x == max_tiles writes the head's slot table.
 // The tile's source rows (the packed K rows of its 64 tokens, the V rows of its width class) are
@@ -108,8 +168,8 @@ relayout_kernel(SrcLayer S, int n8, const RdkvUnit *__restrict__ units, const in
   // LDS: [slot sources | K2 rows | K4 rows | K8 rows | V rows], every region 16-byte aligned + slack
   const int sub2 = S.n2p >> 2, sub4 = S.n4p >> 1;
   auto region = [](int bytes) { return ((bytes + 15) & ~15) + 16; };
-  SlotSrc *ssrc = reinterpret_cast<SlotSrc *>(lds);
-  uint8_t *a_k2 = lds + region(n_slots_max * (int)sizeof(SlotSrc));
+  uint32_t *ssrc = reinterpret_cast<uint32_t *>(lds);
+  uint8_t *a_k2 = lds + region(n_slots_max * 4);
   uint8_t *a_k4 = a_k2 + region(RDKV_TILE * sub2);
   uint8_t *a_k8 = a_k4 + region(RDKV_TILE * sub4);
   uint8_t *a_v = a_k8 + region(RDKV_TILE * n8);
@@ -122,23 +182,15 @@ relayout_kernel(SrcLayer S, int n8, const RdkvUnit *__restrict__ units, const in
   const uint8_t *l_v = stage_rows(a_v, v_src + (int64_t)tk0 * v_row, v_row, v_row, nv);
   for (int i = threadIdx.x; i < n_slots; i += 256) {
     int src = slots[i];
-    SlotSrc e = {0, 0, 0, 0};
+    uint32_t e = 0;
     if (src >= 0) {
       if (src < S.n2p) {
-        e.base = (uint16_t)((l_k2 - lds) + src % sub2);
-        e.pitch = (uint16_t)sub2;
-        e.shift = (uint8_t)(2 * (src / sub2));
-        e.mask = 3;
+        e = slot_src((uint32_t)(l_k2 - lds) + src % sub2, sub2, 2 * (src / sub2), 2);
       } else if (src < S.n2p + S.n4p) {
         src -= S.n2p;
-        e.base = (uint16_t)((l_k4 - lds) + src % sub4);
-        e.pitch = (uint16_t)sub4;
-        e.shift = (uint8_t)(4 * (src / sub4));
-        e.mask = 15;
+        e = slot_src((uint32_t)(l_k4 - lds) + src % sub4, sub4, 4 * (src / sub4), 4);
       } else {
-        e.base = (uint16_t)((l_k8 - lds) + (src - S.n2p - S.n4p));
-        e.pitch = (uint16_t)n8;
-        e.mask = 255;
+        e = slot_src((uint32_t)(l_k8 - lds) + (src - S.n2p - S.n4p), n8, 0, 8);
       }
     }
     ssrc[i] = e;
@@ -147,64 +199,32 @@ relayout_kernel(SrcLayer S, int n8, const RdkvUnit *__restrict__ units, const in
 
   // ---- K tile: 64 rows of R dwords, chunks of up to four dwords per token
   uint32_t *k_out = reinterpret_cast<uint32_t *>(blob + u.k_off) + (int64_t)ti * RDKV_TILE * R;
+  const int full = 256 * (R / 4);                   // dwords of the four-dword chunks
   for (int rem0 = threadIdx.x; rem0 < RDKV_TILE * R; rem0 += 256) {
-    int rem = rem0;
-    int c = rem / 256, wc = 4;
-    if (c >= R / 4) { c = R / 4; wc = R % 4; }
-    rem -= c * 256;
-    const int t = rem / wc, j = 4 * c + rem % wc;
+    int t, j;
+    if (rem0 < full) {
+      t = (rem0 & 255) >> 2;
+      j = 4 * (rem0 >> 8) + (rem0 & 3);
+    } else {
+      const int wc = R & 3, rem = rem0 - full;
+      t = rem / wc;
+      j = 4 * (R / 4) + rem - t * wc;
+    }
     uint32_t w = 0;
     if (t < nv) {
-      int nf, step0;
-      if (j < u.d8) { nf = 4; step0 = j; }
-      else if (j < u.d8 + u.d4) { nf = 8; step0 = u.d8 + 2 * (j - u.d8); }
-      else { nf = 16; step0 = u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4); }
-      const int fw = 32 / nf;
-      for (int f = 0; f < nf; ++f) {
-        int s, k;
-        rdkv_operand_of(f, nf, &s, &k);
-        const SlotSrc e = ssrc[4 * (step0 + s) + k];
-        w |= (uint32_t)((lds[e.base + t * e.pitch] >> e.shift) & e.mask) << (fw * f);
-      }
+      if (j < u.d8) w = k_dword<4>(lds, ssrc, j, t);
+      else if (j < u.d8 + u.d4) w = k_dword<8>(lds, ssrc, u.d8 + 2 * (j - u.d8), t);
+      else w = k_dword<16>(lds, ssrc, u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4), t);
     }
     k_out[rem0] = w;
   }
 
   // ---- V tile of the class
-  const int per_tile = rdkv_v_tile_bytes(cls) / 4;
-  uint32_t *v_out = reinterpret_cast<uint32_t *>(blob + u.v_off[cls]) + (int64_t)tl * per_tile;
-  for (int rem = threadIdx.x; rem < per_tile; rem += 256) {
-    const int l = (rem >> 2) & 63;
-    const int di = ((rem >> 8) << 2) | (rem & 3);  // lane dword index
-    uint32_t w = 0;
-    if (cls == 3) {
-      const int quad = di >> 2, j = (di >> 1) & 1, kk = (di & 1) * 2;
-      const uint16_t *rows = reinterpret_cast<const uint16_t *>(l_v);
-      for (int e = 0; e < 2; ++e) {
-        const int t = 4 * quad + kk + e;
-        if (t < nv) w |= (uint32_t)rows[t * 128 + l + 64 * j] << (16 * e);
-      }
-    } else {
-      const int nf = cls == 2 ? 4 : (cls == 1 ? 8 : 16);
-      const int fw = 32 / nf;
-      for (int f = 0; f < nf; ++f) {
-        int s, k, quad, j;
-        rdkv_operand_of(f, nf, &s, &k);
-        if (cls == 2) { quad = di >> 1; j = di & 1; }
-        else if (cls == 1) { quad = di; j = s; }
-        else { quad = 2 * di + (s >> 1); j = s & 1; }
-        const int t = 4 * quad + k, ch = l + 64 * j;
-        if (t < nv) {
-          uint32_t code;
-          if (cls == 0) code = (l_v[t * 32 + (ch & 31)] >> (2 * (ch >> 5))) & 3u;
-          else if (cls == 1) code = (l_v[t * 64 + (ch & 63)] >> (4 * (ch >> 6))) & 15u;
-          else code = l_v[t * 128 + ch];
-          w |= code << (fw * f);
-        }
-      }
-    }
-    v_out[rem] = w;
-  }
+  uint32_t *v_out = reinterpret_cast<uint32_t *>(blob + u.v_off[cls]) + (int64_t)tl * (rdkv_v_tile_bytes(cls) / 4);
+  if (cls == 0) v_tile<0>(l_v, nv, v_out);
+  else if (cls == 1) v_tile<1>(l_v, nv, v_out);
+  else if (cls == 2) v_tile<2>(l_v, nv, v_out);
+  else v_tile<3>(l_v, nv, v_out);
 
   // ---- per-token {scale, zp} of a quantized tile
   if (cls < 3 && threadIdx.x < RDKV_TILE) {
@@ -244,10 +264,10 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
   S.max_T_v = max_T_v;
   S.perm = perm; S.perm_sh = perm_stride_h;
   S.kscale = (const uint16_t *)kscale_f16; S.kzp = (const uint16_t *)kzp_f16; S.ks_sh = ks_stride_h;
-  RDKV_REQUIRE(n8 >= 0 && max_tiles >= 0 && n_slots_max <= 4 * RDKV_MAX_STEPS,
+  RDKV_REQUIRE(n8 >= 0 && n8 <= 255 && n2p <= 1020 && n4p <= 510 && max_tiles >= 0 && n_slots_max <= 4 * RDKV_MAX_STEPS,
                "rdkv_stream_relayout_layer: bad n8 / max_tiles / slot count");
   auto region = [](int64_t bytes) { return ((bytes + 15) & ~(int64_t)15) + 16; };
-  const int64_t lds = region((int64_t)n_slots_max * (int64_t)sizeof(SlotSrc)) + region(RDKV_TILE * (n2p / 4)) +
+  const int64_t lds = region((int64_t)n_slots_max * 4) + region(RDKV_TILE * (n2p / 4)) +
                       region(RDKV_TILE * (n4p / 2)) + region((int64_t)RDKV_TILE * n8) + region(RDKV_TILE * 256);
   RDKV_REQUIRE(lds <= 64 * 1024, "rdkv_stream_relayout_layer: K rows of %d bytes do not fit the staging area",
                n2p / 4 + n4p / 2 + n8);
