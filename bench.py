@@ -24,8 +24,8 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch of the fused kernel on the default workload, from two rocprofv3 --pmc
 # runs of this command (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors a plain copy
-# kernel of known size gives): (556 752 x 2 + 3 100) KiB.  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: 1143576576}
+# kernel of known size gives): (547 614 x 2 + 1 052) KiB.  Other workloads: not measured.
+MEASURED_TRAFFIC_BYTES = {1: 1122590720}
 PACK_SAMPLE_LAYERS = 8                      # layers of one sequence packed back to back for the pack throughput
 
 
