@@ -330,6 +330,7 @@ k_quantize_pack_kernel(const __half *__restrict__ k, int64_t k_row_stride, int64
     RdkvQParams p;
     p.scale = s_scale[s];
     p.zp = s_zp[s];
+    p.inv = __fdiv_rn(1.0f, p.scale);
     return rdkv_qcode(x, p, qmax);
   };
   for (int64_t idx = threadIdx.x; idx < total; idx += blockDim.x) {
@@ -562,6 +563,7 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
         RdkvQParams p;
         p.scale = c_scale[c];
         p.zp = c_zp[c];
+        p.inv = __fdiv_rn(1.0f, p.scale);
         rb[slot] = (uint8_t)rdkv_qcode(kr ? __half2float(kr[c]) : 0.0f, p, c_qmax[c]);
       }
     }
@@ -649,6 +651,7 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
     sl[e] = c_slot[ch];
     qp[e].scale = sl[e] >= 0 ? c_scale[ch] : 1.0f;
     qp[e].zp = sl[e] >= 0 ? c_zp[ch] : 0.0f;
+    qp[e].inv = __fdiv_rn(1.0f, qp[e].scale);
     qm[e] = sl[e] >= 0 ? c_qmax[ch] : 0.0f;
   }
   const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;

@@ -73,15 +73,32 @@ __device__ __forceinline__ float rdkv_wave_sum(float v) {
 struct RdkvQParams {
   float scale;
   float zp;
+  float inv;   // 1 / scale, correctly rounded: only used to decide when the exact quotient is needed
 };
 __device__ __forceinline__ RdkvQParams rdkv_qparams(float mn, float mx, float qmax) {
   RdkvQParams p;
   p.scale = fmaxf(__fdiv_rn(__fsub_rn(mx, mn), qmax), 1e-8f);
   float z = __fsub_rn(0.0f, __fdiv_rn(mn, p.scale));
   p.zp = rintf(fminf(fmaxf(z, 0.0f), qmax));
+  p.inv = __fdiv_rn(1.0f, p.scale);
   return p;
 }
-__device__ __forceinline__ uint32_t rdkv_qcode(float x, RdkvQParams p, float qmax) {
+// The code of the reference's expression, rint(clamp(x / scale + zp)) with the correctly rounded
+// division.  Only the rounded integer matters, so the quotient is first estimated as x * (1 / scale)
+// (within 1e-4 of the exact expression wherever the clamp does not decide anyway: codes are at most
+// 255 and both forms carry relative errors of a few 2^-24); unless that estimate lies within 2e-4
+// of a rounding boundary k + 1/2 it rounds to the same integer and the division is skipped.  About
+// one element in 2500 takes the exact path.
+__device__ __forceinline__ uint32_t rdkv_qcode_exact(float x, RdkvQParams p, float qmax) {
   float v = __fadd_rn(__fdiv_rn(x, p.scale), p.zp);
   return (uint32_t)rintf(fminf(fmaxf(v, 0.0f), qmax));
+}
+__device__ __forceinline__ uint32_t rdkv_qcode(float x, RdkvQParams p, float qmax) {
+  const float t = fmaf(x, p.inv, p.zp);
+  const float r = rintf(fminf(fmaxf(t, 0.0f), qmax));
+  // |t - r| is the distance to the chosen integer: near 1/2 means near a boundary.  Values the
+  // clamp decides are far from r unless they sit at the clamp's own boundary (-1/2 or qmax + 1/2),
+  // which the same test catches; NaN compares false and gives 0 on both paths.
+  if (fabsf(fabsf(t - r) - 0.5f) < 2e-4f) return rdkv_qcode_exact(x, p, qmax);
+  return (uint32_t)r;
 }
