@@ -73,6 +73,41 @@ def test_quantizer_random_vs_oracle(bits):
         assert_bits_equal(t2n(z), ez)
 
 
+@pytest.mark.parametrize("bits", [2, 4, 8])
+def test_quantizer_at_rounding_boundaries(bits):
+    """Rows whose values sit on the rounding boundaries (k + 1/2 - zp) * scale of their own scale
+    and one fp16 step to either side, for scales that are and are not powers of two and rows on
+    either side of zero: the codes must be those of the correctly rounded division, which the
+    kernel evaluates only near a boundary.  5 % and more of the values are within 2e-4 code units
+    of a boundary (random data: 0.04 %)."""
+    rng = np.random.default_rng(100 + bits)
+    qmax = 2 ** bits - 1
+    rows = []
+    for scale in (2.0 ** -7, 0.01, 0.0371, 1.0 / 3.0, 1.7, 24.0):
+        for offset in (0.0, -0.3 * scale * qmax, -scale * qmax, 5.0 * scale * qmax, -6.0 * scale * qmax):
+            lo, hi = np.float16(offset), np.float16(offset + scale * qmax)
+            mn, mx = np.float32(lo), np.float32(hi)
+            sc = max((mx - mn) / np.float32(qmax), np.float32(1e-8))
+            zp = np.round(np.clip(np.float32(0) - mn / sc, 0, qmax))
+            ks = rng.integers(0, qmax, 126)
+            x = np.float16((ks + 0.5 - zp) * sc)
+            x = (x.view(np.int16) + rng.integers(-1, 2, 126).astype(np.int16)).view(np.float16)
+            rows.append(np.concatenate([np.clip(x, lo, hi), [lo, hi]]).astype(np.float16))
+    x = np.stack(rows)[None, None]                              # [1, 1, 30, 128]
+    assert np.isfinite(x).all()
+    x32 = x.astype(np.float32)
+    mn, mx = x32.min(-1, keepdims=True), x32.max(-1, keepdims=True)
+    sc = np.maximum((mx - mn) / np.float32(qmax), np.float32(1e-8))
+    v = x32 / sc + np.round(np.clip(-mn / sc, 0, qmax))
+    assert (np.abs(np.abs(v - np.round(v)) - 0.5) < 2e-4).mean() > 0.05
+    for dim in (2, 3):
+        q, s, z = packing.quantize_and_pack(to_dev(x), bits, dim)
+        eq, es, ez = O.quantize_and_pack(x, bits, dim)
+        assert_bits_equal(t2n(q), eq)
+        assert_bits_equal(t2n(s), es)
+        assert_bits_equal(t2n(z), ez)
+
+
 def test_reference_test_inputs_segment_counts():
     """tests/test_blockwise_rdkv.py:120-140 with the stored reference outputs as expectation."""
     g = load_golden("ref_test_segment_counts")
