@@ -171,11 +171,8 @@ pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stri
           mn = fminf(mn, fminf(x[p][0], x[p][1]));
           mx = fmaxf(mx, fmaxf(x[p][0], x[p][1]));
         }
-#pragma unroll
-        for (int off = 8; off > 0; off >>= 1) {
-          mn = fminf(mn, __shfl_xor(mn, off, 64));
-          mx = fmaxf(mx, __shfl_xor(mx, off, 64));
-        }
+        mn = rdkv_row16_min(mn);
+        mx = rdkv_row16_max(mx);
         const float qmax = cls[s] == 0 ? 3.0f : (cls[s] == 1 ? 15.0f : 255.0f);
         const RdkvQParams qp = rdkv_qparams(mn, mx, qmax);
         if (l == 0) {

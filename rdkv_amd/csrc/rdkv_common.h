@@ -67,6 +67,26 @@ __device__ __forceinline__ float rdkv_wave_sum(float v) {
   return v;
 }
 
+// Minimum / maximum over the 16 lanes of a row (lanes 16k .. 16k+15), the result in every lane:
+// rotations by 8, 4, 2 and 1 inside the row as data-parallel-primitive moves, which run at vector
+// ALU speed (a shuffle through the LDS crossbar is a ~100-cycle round trip each).
+template <int CTRL>
+__device__ __forceinline__ float rdkv_dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float rdkv_row16_min(float v) {
+  v = fminf(v, rdkv_dpp_mov<0x128>(v));
+  v = fminf(v, rdkv_dpp_mov<0x124>(v));
+  v = fminf(v, rdkv_dpp_mov<0x122>(v));
+  return fminf(v, rdkv_dpp_mov<0x121>(v));
+}
+__device__ __forceinline__ float rdkv_row16_max(float v) {
+  v = fmaxf(v, rdkv_dpp_mov<0x128>(v));
+  v = fmaxf(v, rdkv_dpp_mov<0x124>(v));
+  v = fmaxf(v, rdkv_dpp_mov<0x122>(v));
+  return fmaxf(v, rdkv_dpp_mov<0x121>(v));
+}
+
 // The reference's quantizer (packing.py:153-163) for one value, IEEE fp32 with its
 // operation order: scale = max((mx-mn)/qmax, 1e-8); zp = rint(clamp(0 - mn/scale));
 // q = rint(clamp(x/scale + zp)).  Division must be the correctly rounded one.
