@@ -275,3 +275,54 @@ def test_projection_row_kernel_matches_library(dtype):
     W = torch.randn(16, 100, generator=g, device=DEV).to(dtype)
     x = torch.randn(1, 100, generator=g, device=DEV).to(dtype)
     torch.testing.assert_close(fast_decode._linear_row(x, W), torch.nn.functional.linear(x, W))
+
+
+@pytest.mark.parametrize("family", ["qwen2", "qwen3"])
+def test_decode_loop_follows_other_model_families(family):
+    """q/k/v projection biases (Qwen2) and per-head q/k RMSNorm before the rotary embedding (Qwen3)
+    (fast_decode.py:352-355, 381-384, 1664-1667): the loop tracks ``model.forward`` over the dense
+    prompt cache when V stays fp16 and K gets 8 bits."""
+    require_gpu()
+    import transformers
+    kw = dict(hidden_size=HID, intermediate_size=1024, num_hidden_layers=LAYERS, num_attention_heads=H_Q,
+              num_key_value_heads=H_KV, vocab_size=VOCAB, max_position_embeddings=4096, tie_word_embeddings=False)
+    if family == "qwen2":
+        model = transformers.Qwen2ForCausalLM(transformers.Qwen2Config(**kw))
+    else:
+        model = transformers.Qwen3ForCausalLM(transformers.Qwen3Config(head_dim=D, **kw))
+    torch.manual_seed(4321)
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if p.dim() == 2:
+                p.copy_(torch.randn_like(p) * 0.06)
+            elif name.endswith("bias"):
+                p.copy_(torch.randn_like(p) * 0.5)
+            else:
+                p.copy_(1.0 + 0.2 * torch.randn_like(p))       # norm weights, q_norm / k_norm included
+    model = model.half().to(DEV).eval()
+    W = fast_decode.pre_extract_weights(model)
+    assert (W.layers[0].qkv_bias is not None) == (family == "qwen2")
+    assert (W.layers[0].q_norm_weight is not None) == (family == "qwen3")
+    g = torch.Generator().manual_seed(3)
+    prompt = torch.randint(0, VOCAB, (1, 200), generator=g).to(DEV)
+    with torch.no_grad():
+        pre = model(prompt, use_cache=True)
+        kv = [(l.keys.contiguous(), l.values.contiguous()) for l in pre.past_key_values.layers[:LAYERS]]
+    layers, v16 = [], []
+    for K, V in kv:
+        pl, nvo = packing.pack_layer_per_head(K, V, torch.full((H_KV, 200), 16), torch.full((H_KV, D), 8), H_Q // H_KV)
+        layers.append(pl)
+        v16.append(nvo)
+    cache = packing.TriZoneCache(tuple(layers), v16, [None] * LAYERS, [None] * LAYERS, 200)
+    ids, logits = fast_decode.greedy_decode_fast(model, cache, pre.logits[0, -1], 4, [], torch.device(DEV), 200,
+                                                 return_logits=True)
+    with torch.no_grad():
+        pkv = model(prompt, use_cache=True).past_key_values
+        for step, tok in enumerate(ids):
+            o = model(torch.tensor([[tok]], device=DEV), past_key_values=pkv, use_cache=True)
+            pkv = o.past_key_values
+            exp, got = o.logits[0, -1].float().cpu(), logits[step][0]
+            cos = float(torch.nn.functional.cosine_similarity(got, exp, dim=0))
+            assert cos > 0.999, f"{family} step {step}: cosine {cos}"
+    assert fast_decode.greedy_decode_fast(model, cache, pre.logits[0, -1], 4, [], torch.device(DEV), 200,
+                                          use_cuda_graph=True) == ids
