@@ -140,10 +140,17 @@ RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x
   RDKV_REQUIRE(W && x && y, "%s: null pointer", fn);
   RDKV_REQUIRE(((uintptr_t)W % 16) == 0 && ((uintptr_t)x % 16) == 0 && w_stride_row % 8 == 0 && w_stride_row >= K,
                "%s: W rows and x must be 16-byte aligned", fn);
+  // compute units of the current device, asked once per device (0 = not asked yet; a race between
+  // two first calls stores the same number twice)
+  static int cu_of_device[64];
   int dev = 0, n_cu = 256;
-  if (hipGetDevice(&dev) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n_cu = v;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    if (cu_of_device[dev] == 0) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        cu_of_device[dev] = v;
+    }
+    if (cu_of_device[dev] > 0) n_cu = cu_of_device[dev];
   }
   if (dtype == RDKV_DTYPE_F16) launch_gemv<RDKV_DTYPE_F16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
   else launch_gemv<RDKV_DTYPE_BF16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
