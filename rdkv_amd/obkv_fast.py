@@ -1,8 +1,9 @@
 """Prefill-time selection feeding the packer, with the names of the reference's ``obkv_fast``.
 
 Only the per-layer selection + packing step is here (score pooling, the per-head V knapsack,
-the per-head K allocation and the hand-over to the whole-layer packer); model loading, scoring
-and the decode loops of the reference's module are not part of this package.  Everything runs
+the per-head K allocation and the hand-over to the whole-layer packer) and the prefill scores of
+a layer; model loading and the drivers of the reference's module are not part of this package
+(the decode loop over a packed cache is ``fast_decode.greedy_decode_fast``).  Everything runs
 on the GPU: the only device-to-host reads are the packer's (per-head segment sizes and the
 [H_kv, D] K widths, which fix the shapes of the packed tensors).
 """

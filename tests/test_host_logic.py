@@ -241,3 +241,40 @@ def test_selection_and_planning_entry_points_reject_bad_arguments():
     err(lib.rdkv_pack_layer_tables(None, 1, 8, 2, 2048, 1, None, None, 0, 0, 8, 8, 4, 0, None, 0, None, 0, 0, 0,
                                    None, None, None, None, None, None, None, None, None, None, None, None),
         "bad shape")
+
+
+def test_pre_extract_weights_on_a_cpu_model():
+    """fast_decode.py:418-621: one matrix for q/k/v and one for gate/up, biases concatenated when
+    the model has them, per-head q/k norm weights picked up, the result cached on the model."""
+    import torch
+    import transformers
+    from rdkv_amd import fast_decode
+    kw = dict(hidden_size=256, intermediate_size=512, num_hidden_layers=2, num_attention_heads=2,
+              num_key_value_heads=1, vocab_size=64, max_position_embeddings=128, tie_word_embeddings=False)
+    llama = transformers.LlamaForCausalLM(transformers.LlamaConfig(head_dim=128, **kw))
+    W = fast_decode.pre_extract_weights(llama)
+    assert fast_decode.pre_extract_weights(llama) is W
+    assert (W.num_layers, W.num_heads, W.num_kv_heads, W.head_dim, W.num_kv_groups) == (2, 2, 1, 128, 2)
+    assert (W.hidden_size, W.attn_output_dim) == (256, 256)
+    lw, attn, mlp = W.layers[1], llama.model.layers[1].self_attn, llama.model.layers[1].mlp
+    assert lw.qkv_split_sizes == (256, 128, 128) and lw.gate_up_split_sizes == (512, 512)
+    assert torch.equal(lw.qkv_weight, torch.cat([attn.q_proj.weight, attn.k_proj.weight, attn.v_proj.weight]))
+    assert torch.equal(lw.gate_up_weight, torch.cat([mlp.gate_proj.weight, mlp.up_proj.weight]))
+    assert lw.qkv_bias is None and lw.q_norm_weight is None and lw.k_norm_weight is None
+    assert lw.o_proj_weight is attn.o_proj.weight and lw.down_proj_weight is mlp.down_proj.weight
+    assert W.lm_head_weight is llama.lm_head.weight and W.rotary_emb is llama.model.rotary_emb
+    qwen2 = transformers.Qwen2ForCausalLM(transformers.Qwen2Config(**kw))
+    b = fast_decode.pre_extract_weights(qwen2).layers[0]
+    a2 = qwen2.model.layers[0].self_attn
+    assert torch.equal(b.qkv_bias, torch.cat([a2.q_proj.bias, a2.k_proj.bias, a2.v_proj.bias]))
+    qwen3 = transformers.Qwen3ForCausalLM(transformers.Qwen3Config(head_dim=128, **kw))
+    c = fast_decode.pre_extract_weights(qwen3).layers[0]
+    a3 = qwen3.model.layers[0].self_attn
+    assert c.q_norm_weight is a3.q_norm.weight and c.k_norm_weight is a3.k_norm.weight
+    assert c.qk_norm_eps == a3.q_norm.variance_epsilon and c.qkv_bias is None
+    # the loop itself has no CPU path
+    import pytest
+    from rdkv_amd import packing
+    with pytest.raises((RuntimeError, AssertionError)):
+        fast_decode.greedy_decode_fast(llama, packing.TriZoneCache((), [], [], [], 0), torch.zeros(64), 1, [],
+                                       torch.device("cpu"), 0)
