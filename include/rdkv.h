@@ -283,13 +283,18 @@ int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int 
  * [old | new], :1777-1784 their V sum): the exact softmax over zones A+B+C, out and lse of the
  * union.  k_new / v_new: fp32 [rows / G, >= n_new, 128], indexed by r = q_row / G of the unit
  * (row r at + r*new_stride_unit, token t at + t*new_stride_tok, elements); n_new tokens per
- * row, or n_new_per_unit[r] (device int32) when not NULL (n_new is then ignored).  q / rope_*: as passed to rdkv_decode_fused_partials. */
+ * row, or n_new_per_unit[r] (device int32) when not NULL (n_new is then ignored).  q / rope_*: as passed to rdkv_decode_fused_partials.
+ * zone_c_weights (NULL, or fp32 [rows, >= n_new], row stride in elements): receives the softmax
+ * weight of every zone-C token over the union, per query row - the w_new of fast_decode.py:1755
+ * and the pending weights blockwise decode sums into its block scores
+ * (blockwise_decode.py:2085-2109). */
 int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G,
                                    const void *q, int q_dtype, int64_t q_stride_row,
                                    const void *rope_cos, const void *rope_sin, int rope_dtype,
                                    const float *k_new, const float *v_new, int64_t new_stride_unit,
                                    int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit,
                                    float *out, int64_t out_stride_row, float *lse,
+                                   float *zone_c_weights, int64_t zone_c_weights_stride_row,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Planning for rdkv_pack_layer_per_head on the device (what the reference derives on the host:

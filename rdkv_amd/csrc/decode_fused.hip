@@ -776,8 +776,10 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
                     const float *__restrict__ k_new, const float *__restrict__ v_new, int64_t new_stride_unit,
                     int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
-                    float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
+                    float *__restrict__ out, int64_t out_stride, float *__restrict__ lse,
+                    float *zc_w, int64_t zc_w_stride) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
+  __shared__ float fin_m[8], fin_l[8];             // softmax maximum and sum over the union, per head
   __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
   __shared__ __align__(16) float qz[8][kD];        // q / sqrt(D)
   __shared__ float w_m[kZcWaves][8], w_l[kZcWaves][8];
@@ -853,6 +855,10 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
         }
       }
     }
+    if (zc_w && valid) {      // raw scores now, turned into weights once the union's maximum and sum are known
+#pragma unroll
+      for (int h = 0; h < G; ++h) zc_w[(int64_t)(q_row + h) * zc_w_stride + t0 + lane] = s[h];
+    }
     float wt[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
@@ -920,6 +926,19 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
     }
     out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? o / l : 0.0f;
     if (lse && d == 0) lse[q_row + h] = l > 0.0f ? M + logf(l) : -INFINITY;
+    if (d == 0) {
+      fin_m[h] = M;
+      fin_l[h] = l;
+    }
+  }
+  if (zc_w) {   // softmax weights of the zone C tokens over the union (fast_decode.py:1753-1755 w_new)
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
+      const float M = fin_m[h], inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
+      for (int t = tid; t < n_new; t += kThreads) row[t] = expf(row[t] - M) * inv;
+    }
   }
 }
 
@@ -1048,9 +1067,12 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
                                             const void *rope_sin, int rope_dtype, const float *k_new,
                                             const float *v_new, int64_t new_stride_unit, int64_t new_stride_tok,
                                             int n_new, const int32_t *n_new_per_unit, float *out,
-                                            int64_t out_stride_row, float *lse, void *workspace,
+                                            int64_t out_stride_row, float *lse, float *zone_c_weights,
+                                            int64_t zone_c_weights_stride_row, void *workspace,
                                             int64_t workspace_bytes, void *stream) {
   const char *fn = "rdkv_decode_fused_merge_zone_c";
+  RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= n_new || n_new_per_unit,
+               "%s: rows of the zone-C weights are shorter than n_new", fn);
   int rc = check_fused_args(fn, units, n_units, (const RdkvWork *)units, n_work, G, workspace, workspace_bytes);
   if (rc != RDKV_OK) return rc;
   RDKV_REQUIRE(n_new >= 0 && new_stride_tok >= 128 && new_stride_unit >= 0, "%s: bad zone-C shape", fn);
@@ -1065,7 +1087,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
 #define RDKV_LAUNCH_ZC(GT)                                                                                    \
   hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
                      (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new, \
-                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse)
+                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
+                     zone_c_weights, zone_c_weights_stride_row)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;
     case 2: RDKV_LAUNCH_ZC(2); break;

@@ -401,15 +401,18 @@ def extend_stream_cache(cache: StreamCache, layers: Sequence[Tuple[PackedKVLayer
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,
                       lse: Optional[torch.Tensor] = None, *,
                       rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
-                      zone_c: Optional[Tuple[torch.Tensor, ...]] = None):
+                      zone_c: Optional[Tuple[torch.Tensor, ...]] = None,
+                      zone_c_weights: Optional[torch.Tensor] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
     query); returns (out fp32 [rows,128], lse fp32 [rows]).  ``zone_c`` = (K_new, V_new[,
     n_new_per_row]): fp32 [rows / G, n_new, 128] rows of the decode-appended tokens of every
     (output group, KV head) (optional int32 [rows / G] counts when they differ): the merge
-    launch then returns the exact softmax over packed cache + new tokens.  Graph-capturable once
-    the workspace exists (first call): one streaming launch plus one small merge launch."""
+    launch then returns the exact softmax over packed cache + new tokens.  ``zone_c_weights``
+    (fp32 [rows, >= n_new], with ``zone_c``): receives the softmax weight of every new token over
+    the union, per query row (what blockwise decode sums into its block scores).  Graph-capturable
+    once the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
     assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
@@ -431,6 +434,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     need = lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G)
     ws = _lib.workspace(dev, need)
     stream = _lib.stream_of(dev)
+    assert zone_c_weights is None or zone_c is not None, "zone_c_weights needs zone_c"
     if zone_c is None:
         _lib.check(lib.rdkv_decode_fused(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
@@ -454,11 +458,17 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         ws.data_ptr(), ws.numel(), stream))
     n_new = int(K_new.shape[1])
+    if zone_c_weights is not None:
+        _lib.require_device(zone_c_weights)
+        assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2 and zone_c_weights.stride(1) == 1
+        assert zone_c_weights.shape[0] == cache.rows and zone_c_weights.shape[1] >= n_new, (
+            f"zone_c_weights must be [rows = {cache.rows}, >= {n_new}], got {tuple(zone_c_weights.shape)}")
     _lib.check(lib.rdkv_decode_fused_merge_zone_c(
         cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
-        _lib.ptr(counts), out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+        _lib.ptr(counts), out.data_ptr(), out.stride(0), lse.data_ptr(), _lib.ptr(zone_c_weights),
+        zone_c_weights.stride(0) if zone_c_weights is not None else 0, ws.data_ptr(), ws.numel(), stream))
     return out, lse
 
 

@@ -350,3 +350,39 @@ def test_multi_source_rows():
         r = slice(grp * cfg.H_q, (grp + 1) * cfg.H_q)
         exp = fast_decode.merge_zone_c(out[r], lse[r], q[r], K_new[grp], V_new[grp], cfg.G)
         assert float((got[r] - exp).abs().max()) < 2e-5
+
+
+@pytest.mark.parametrize("n_new", [1, 40, 64, 150, 700])
+def test_zone_c_weights_are_the_softmax_over_the_union(n_new):
+    """``zone_c_weights``: per query row the softmax weight of every decode-appended token over
+    [packed sources | appended tokens] (fast_decode.py:1753-1755, blockwise_decode.py:2085-2109):
+    exp(score - lse_union).  Checked from the lse of the packed part and plain fp32 scores; the
+    mass of the packed part and of the appended tokens adds up to one."""
+    cfg = synth.scaled(synth.CONFIGS[1], context=700, layers=2)
+    packed, q2, _ = _config_case(cfg, 2)
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    q = q2[:cache.rows].contiguous()
+    out_ab, lse_ab = stream_cache.decode_attn_fused(cache, q)
+    g = torch.Generator().manual_seed(n_new)
+    rows_kv = cache.rows // cfg.G
+    cap = n_new + 5
+    buf = torch.randn(rows_kv, cap, 256, generator=g).to(DEV)
+    counts = torch.full((rows_kv,), n_new, dtype=torch.int32, device=DEV)
+    counts[1] = max(1, n_new // 2)                                  # ragged: one row has fewer tokens
+    w = torch.full((cache.rows, cap + 3), -7.0, device=DEV)
+    out, lse = stream_cache.decode_attn_fused(cache, q, zone_c=(buf[:, :, :128], buf[:, :, 128:], counts),
+                                              zone_c_weights=w[:, :cap])
+    for r_kv in range(rows_kv):
+        n = int(counts[r_kv])
+        rows = slice(r_kv * cfg.G, (r_kv + 1) * cfg.G)
+        s = (q[rows].float() @ buf[r_kv, :n, :128].T) * (128 ** -0.5)            # [G, n]
+        lse_union = torch.logsumexp(torch.cat([lse_ab[rows, None], s], dim=1), dim=1)
+        exp_w = torch.exp(s - lse_union[:, None])
+        torch.testing.assert_close(w[rows, :n], exp_w, rtol=2e-4, atol=1e-6)
+        torch.testing.assert_close(lse[rows], lse_union, rtol=0, atol=2e-5)
+        mass_ab = torch.exp(lse_ab[rows] - lse_union)
+        torch.testing.assert_close(mass_ab + w[rows, :n].sum(1), torch.ones(cfg.G, device=DEV), rtol=0, atol=1e-5)
+        assert float((w[rows, n:] + 7.0).abs().max()) == 0.0                      # nothing written past n_new
+    # the weights output changes nothing else
+    out2, lse2 = stream_cache.decode_attn_fused(cache, q, zone_c=(buf[:, :, :128], buf[:, :, 128:], counts))
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
