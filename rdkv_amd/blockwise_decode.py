@@ -5,9 +5,10 @@ What is here is everything between "a decode block of raw K/V is complete" and "
 source the attention reads": the compression schedule, block scoring (``rdkv_block_score``),
 the per-layer selection + packing (``obkv_fast._perhead_select_and_pack``), the logical-bit
 accounting, and the fixed-slot re-shaping the reference uses to keep tensor shapes stable.  The
-model loop around it (``greedy_decode_blockwise``) needs the model stack and is not part of this
-package; the attention over [prompt cache | compressed blocks | raw tail] is
-``stream_cache.build_stream_cache(..., row_of_entry=...)`` + ``decode_attn_fused(..., zone_c=...)``.
+model loop around it is ``greedy_decode_blockwise`` at the end of this module: the attention over
+[prompt cache | compressed blocks | raw tail] is ``stream_cache.extend_stream_cache`` (a block
+becomes a further source of its layer's cache) + ``decode_attn_fused(..., zone_c=...,
+zone_c_weights=...)`` (the tail's softmax weights feed the online block scores).
 """
 from __future__ import annotations
 
@@ -491,3 +492,231 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     }
     print(f"[BLOCKWISE_EVENT] {json.dumps(event, sort_keys=True)}", flush=True)
     return block, event
+
+
+def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logits: Tensor, max_new_tokens: int,
+                            eos_token_ids, primary_device: torch.device, decode_position_start: int,
+                            config: BlockwiseRDKVConfig, use_cuda_graph: bool = False
+                            ) -> Tuple[List[int], Dict[str, Any]]:
+    """Greedy decode that keeps the generated tokens as immutable packed blocks
+    (blockwise_decode.py:1124-2260): same keyword arguments, return value (token ids and the report
+    with the reference's keys) and compression schedule.
+
+    The raw tail holds at most two blocks.  Every step attends over [prompt cache | compressed
+    blocks | raw tail] in two launches per layer (the compressed blocks are further sources of the
+    layer's streaming cache, the tail is zone C) and gets back the tail tokens' softmax weights,
+    which are summed into the block scores exactly as the reference does (:2085-2109): weights of
+    queries on tokens of their own block, and weights of the second block's queries on the first
+    block.  When the tail is full its first block is compressed with the scores of its successor
+    (``_compress_block``) and joins every layer's cache (``extend_stream_cache``); at the end the
+    remaining blocks are flushed, the last one with its own causal scores.
+
+    The reference needs its fixed-slot bank to replay this loop from graphs; that variant is not
+    built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
+    from .fast_decode import (_layer_stream_caches, _linear_row, _rms_norm, _rope_append_kv, _silu_mul,
+                              pre_extract_weights)
+    from .stream_cache import decode_attn_fused, extend_stream_cache
+    from .triton_rope import fused_rope
+
+    config.validate()
+    dev = torch.device(primary_device)
+    if dev.type != "cuda":
+        raise RuntimeError("blockwise packed decode requires CUDA")
+    if use_cuda_graph:
+        raise NotImplementedError("graph replay of the blockwise loop is not built; run it eagerly")
+    eos_set = {int(t) for t in eos_token_ids if t is not None}
+    W = pre_extract_weights(model)
+    model_dtype = next(model.parameters()).dtype
+    h_q, h_kv, groups, D, L = W.num_heads, W.num_kv_heads, W.num_kv_groups, W.head_dim, W.num_layers
+    block = int(config.block_size)
+    capacity = 2 * block
+    prompt_bytes = cache_physical_bytes(dual_cache)
+    caches = list(_layer_stream_caches(dual_cache, groups))      # grown below; the prompt's own list stays as it is
+
+    pending_kv = [torch.zeros(1, h_kv, capacity, 2 * D, dtype=torch.float32, device=dev) for _ in range(L)]
+    pending_q = [torch.empty(h_q, capacity, D, dtype=model_dtype, device=dev) for _ in range(L)]
+    self_scores = [torch.zeros(h_kv, capacity, dtype=torch.float32, device=dev) for _ in range(L)]
+    next_scores = [torch.zeros(h_kv, block, dtype=torch.float32, device=dev) for _ in range(L)]
+    tail_weights = torch.zeros(h_q, capacity, dtype=torch.float32, device=dev)
+    attn_out = torch.empty(h_q, D, dtype=torch.float32, device=dev)
+    lse = torch.empty(h_q, dtype=torch.float32, device=dev)
+    write_row = torch.zeros(1, dtype=torch.long, device=dev)
+    n_tail = torch.zeros(h_kv, dtype=torch.int32, device=dev)
+    one, zero = torch.ones(D // 2, dtype=model_dtype, device=dev), torch.zeros(D // 2, dtype=model_dtype, device=dev)
+
+    generated: List[int] = []
+    compressed: List[CompressedDecodeBlock] = []
+    block_events: List[Dict[str, Any]] = []
+    memory_trace: List[Dict[str, Any]] = []
+    token_events: List[torch.cuda.Event] = []
+    pending_len = pending_start = 0
+    peak_equiv, peak_physical = 0.0, 0
+
+    def compressed_equivalents() -> float:
+        return sum(sum(b.fp16_equivalent_tokens_per_layer) / max(1, len(b.fp16_equivalent_tokens_per_layer))
+                   for b in compressed)
+
+    def record_memory(stage: str) -> None:
+        nonlocal peak_equiv, peak_physical
+        comp_eq = compressed_equivalents()
+        pending_bytes = pending_len * L * h_kv * 2 * D * pending_kv[0].element_size()
+        physical = sum(b.physical_bytes for b in compressed) + pending_bytes
+        peak_equiv = max(peak_equiv, comp_eq + pending_len)
+        peak_physical = max(peak_physical, physical)
+        memory_trace.append({"stage": stage, "generated_tokens": len(generated), "compressed_blocks": len(compressed),
+                             "pending_fp16_tokens": pending_len,
+                             "compressed_history_fp16_equivalent_tokens": comp_eq,
+                             "decode_cache_fp16_equivalent_tokens": comp_eq + pending_len,
+                             "decode_cache_physical_bytes": physical})
+
+    def validate_order() -> None:
+        cursor = 0
+        for b in compressed:
+            if b.token_start != cursor or b.token_end < b.token_start:
+                raise AssertionError(f"decode block order corruption: expected start {cursor}, got "
+                                     f"[{b.token_start},{b.token_end}]")
+            cursor = b.token_end + 1
+        if cursor != pending_start:
+            raise AssertionError(f"pending suffix starts at {pending_start}, expected {cursor}")
+        if pending_start + pending_len != len(generated):
+            raise AssertionError(f"decode token coverage mismatch: compressed+pending does not cover "
+                                 f"[0,{len(generated)})")
+
+    def compress_prefix(target_len: int, *, query_offset: int, query_len: int, is_final_flush: bool,
+                        causal: bool) -> None:
+        """blockwise_decode.py:1787-1866: pack the first ``target_len`` tail tokens, add the block to
+        every layer's cache, move the rest of the tail to the front."""
+        nonlocal pending_len, pending_start
+        if target_len <= 0 or query_len <= 0:
+            return
+        target = [buf[:, :, :target_len, :].clone() for buf in pending_kv]
+        queries = [buf[:, query_offset:query_offset + query_len, :].clone() for buf in pending_q]
+        scores = [(s_self[:, :target_len] if causal else s_next[:, :target_len]).clone()
+                  for s_self, s_next in zip(self_scores, next_scores)]
+        block_id = len(compressed)
+        new_block, event = _compress_block(
+            target_kv=target, query_block=queries, token_scores_by_layer=scores, block_id=block_id,
+            token_start=pending_start, token_end=pending_start + target_len - 1,
+            query_source_block=block_id if causal else block_id + 1, is_final_flush=is_final_flush, causal=causal,
+            config=config, num_kv_groups=groups, model_dtype=model_dtype)
+        compressed.append(new_block)
+        block_events.append(event)
+        for layer in range(L):
+            caches[layer] = extend_stream_cache(caches[layer], [(new_block.packed[layer], new_block.new_v_only[layer])],
+                                                row_of_entry=[0])
+        remain = pending_len - target_len
+        for kv_buf, q_buf, s_self, s_next in zip(pending_kv, pending_q, self_scores, next_scores):
+            if remain:
+                kv_buf[:, :, :remain, :].copy_(kv_buf[:, :, target_len:pending_len, :].clone())
+                q_buf[:, :remain, :].copy_(q_buf[:, target_len:pending_len, :].clone())
+                s_self[:, :remain].copy_(s_self[:, target_len:pending_len].clone())
+            s_self[:, remain:].zero_()
+            s_next.zero_()
+        pending_start += target_len
+        pending_len = remain
+        validate_order()
+        record_memory("final_flush" if is_final_flush else f"compressed_block_{block_id}")
+
+    if next_token_logits.dim() == 1:
+        next_token_logits = next_token_logits.unsqueeze(0)
+    next_token = next_token_logits.argmax(dim=-1, keepdim=True).to(dev)
+    position_ids = torch.zeros((1, 1), dtype=torch.long, device=dev)
+    record_memory("decode_start")
+    t_decode0 = _sync_stamp(dev)
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev0.record()
+
+    with torch.inference_mode():
+        for step in range(max_new_tokens):
+            token_id = int(next_token.item())
+            if token_id in eos_set:
+                break
+            generated.append(token_id)
+            position_ids.fill_(decode_position_start + step)
+            h = W.embed_tokens(next_token)
+            cos, sin = W.rotary_emb(h, position_ids)
+            cos_half, sin_half = cos.view(D)[:D // 2], sin.view(D)[:D // 2]
+            write_pos = pending_len
+            if write_pos >= capacity:
+                raise RuntimeError(f"pending decode cache overflow ({write_pos} >= {capacity})")
+            current_len = write_pos + 1
+            q_block_start = (write_pos // block) * block
+            write_row.fill_(write_pos)
+            n_tail.fill_(current_len)
+            delta = None
+            for layer, lw in enumerate(W.layers):
+                x = _rms_norm(h, lw.input_ln_weight, lw.input_ln_eps, delta=delta, residual_out=h)
+                q, k, v = _linear_row(x, lw.qkv_weight, lw.qkv_bias).split(lw.qkv_split_sizes, dim=-1)
+                q_2d, k_2d, v_2d = q.view(h_q, D), k.view(h_kv, D), v.view(h_kv, D)
+                if lw.q_norm_weight is not None:
+                    q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
+                if lw.k_norm_weight is not None:
+                    k_2d = _rms_norm(k_2d, lw.k_norm_weight, lw.qk_norm_eps)
+                q_2d, k_2d = q_2d.contiguous(), k_2d.contiguous()
+                fused_rope(q_2d, k_2d, cos_half, sin_half)          # the rotated query is kept for the channel scores
+                pending_q[layer][:, write_pos, :].copy_(q_2d)
+                rows = pending_kv[layer][0]
+                _rope_append_kv(k_2d, v_2d, one, zero, rows, write_row)     # k is rotated already: identity table
+                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse,
+                                  zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights)
+                # block scores from the tail's weights (blockwise_decode.py:2085-2109)
+                width = current_len - q_block_start
+                self_scores[layer][:, q_block_start:current_len].add_(
+                    tail_weights[:, q_block_start:current_len].view(h_kv, groups, width).sum(dim=1))
+                if q_block_start >= block:
+                    next_scores[layer].add_(tail_weights[:, :block].view(h_kv, groups, block).sum(dim=1))
+                if config.correctness_check and not torch.isfinite(attn_out).all():
+                    raise FloatingPointError(f"non-finite attention output at layer {layer}")
+                o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)
+                x = _rms_norm(h, lw.post_ln_weight, lw.post_ln_eps, delta=o, residual_out=h)
+                gate, up = _linear_row(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
+                delta = _linear_row(_silu_mul(gate, up), lw.down_proj_weight)
+            hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
+            logits = _linear_row(hidden, W.lm_head_weight)
+            next_token = logits[:, -1, :].argmax(dim=-1, keepdim=True)
+            pending_len += 1
+            ev = torch.cuda.Event(enable_timing=True)
+            ev.record()
+            token_events.append(ev)
+            record_memory(f"token_{len(generated)}")
+            if pending_len == capacity:
+                compress_prefix(block, query_offset=block, query_len=block, is_final_flush=False, causal=False)
+
+    t_pre_flush = _sync_stamp(dev)
+    # a complete block followed by an incomplete successor: the successor's queries drain it
+    while pending_len > block:
+        compress_prefix(block, query_offset=block, query_len=min(block, pending_len - block), is_final_flush=True,
+                        causal=False)
+    t_flush0 = _sync_stamp(dev)
+    if pending_len:
+        compress_prefix(pending_len, query_offset=0, query_len=pending_len, is_final_flush=True, causal=True)
+    t_flush1 = _sync_stamp(dev)
+    record_memory("decode_complete")
+    validate_order()
+    torch.cuda.synchronize(dev)
+    n_gen = len(generated)
+    decode_ms = (t_pre_flush - t_decode0) * 1000.0
+    flush_ms = (t_flush1 - t_flush0) * 1000.0
+    report: Dict[str, Any] = {
+        "decode_blockwise_rdkv": True, "decode_cuda_graph": False, "decode_cuda_graph_active_slot_variants": [],
+        "decode_block_size": block, "decode_block_budget_tokens": config.block_budget_tokens,
+        "generated_tokens": n_gen, "block_events": block_events, "memory_trace": memory_trace,
+        "per_token_timestamps_ms": [ev0.elapsed_time(e) for e in token_events],
+        "decode_wall_time_ms_excluding_final_flush": decode_ms, "avg_tpot_ms": decode_ms / max(1, n_gen),
+        "final_flush_time_ms": flush_ms, "completion_latency_ms": decode_ms + flush_ms,
+        "prompt_compressed_kv_physical_bytes": prompt_bytes,
+        "decode_slot_bank_enabled": False, "decode_slot_bank_slots": 0, "decode_slot_bank_physical_bytes": 0,
+        "decode_cache_peak_fp16_equivalent_tokens": peak_equiv,
+        "decode_cache_final_fp16_equivalent_tokens": compressed_equivalents(),
+        "decode_cache_peak_physical_bytes": peak_physical,
+        "decode_cache_final_physical_bytes": sum(b.physical_bytes for b in compressed),
+        "num_compressed_decode_blocks": len(compressed),
+        "coverage": [[b.token_start, b.token_end] for b in compressed],
+    }
+    expected = plan_block_compressions(n_gen, block)
+    actual = [{key: e[key] for key in ("block_id", "token_start", "token_end", "query_source_block", "is_final_flush",
+                                       "query_mode")} for e in block_events]
+    if actual != expected:
+        raise AssertionError(f"blockwise compression schedule diverged from reference: actual={actual}, "
+                             f"expected={expected}")
+    return generated, report

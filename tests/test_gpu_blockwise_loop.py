@@ -1,0 +1,161 @@
+"""The blockwise decode loop (``blockwise_decode.greedy_decode_blockwise``) on a small
+random-weight Llama: schedule, report and coverage as the reference defines them
+(blockwise_decode.py:1124-2260), tokens / logits against ``model.forward`` when the blocks keep
+full precision, and the bounds the online block scores obey as sums of softmax weights."""
+import pytest
+import torch
+
+from rdkv_amd import blockwise_decode as bw
+from rdkv_amd import fast_decode, knapsack_solver as ks, packing
+from tests.gpu_util import DEV, require_gpu
+
+pytestmark = pytest.mark.gpu
+
+T_PROMPT, H_Q, H_KV, D, HID, LAYERS, VOCAB = 160, 4, 2, 128, 512, 2, 1000
+
+
+@pytest.fixture(scope="module")
+def setup():
+    require_gpu()
+    from transformers import LlamaConfig, LlamaForCausalLM
+    cfg = LlamaConfig(hidden_size=HID, intermediate_size=1024, num_hidden_layers=LAYERS, num_attention_heads=H_Q,
+                      num_key_value_heads=H_KV, head_dim=D, vocab_size=VOCAB, max_position_embeddings=4096,
+                      rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=False)
+    torch.manual_seed(99)
+    model = LlamaForCausalLM(cfg)
+    with torch.no_grad():
+        for p in model.parameters():
+            if p.dim() == 2:
+                p.mul_(3.0)
+    model = model.half().to(DEV).eval()
+    g = torch.Generator().manual_seed(8)
+    prompt = torch.randint(0, VOCAB, (1, T_PROMPT), generator=g).to(DEV)
+    with torch.no_grad():
+        pre = model(prompt, use_cache=True)
+    layers, v16 = [], []
+    for i in range(LAYERS):
+        l = pre.past_key_values.layers[i]
+        pl, nvo = packing.pack_layer_per_head(l.keys.contiguous(), l.values.contiguous(),
+                                              torch.full((H_KV, T_PROMPT), 16), torch.full((H_KV, D), 8), H_Q // H_KV)
+        layers.append(pl)
+        v16.append(nvo)
+    cache = packing.TriZoneCache(tuple(layers), v16, [None] * LAYERS, [None] * LAYERS, T_PROMPT)
+    return model, prompt, pre, cache
+
+
+def _config(block, budget):
+    return bw.BlockwiseRDKVConfig(block_size=block, block_budget_tokens=budget, k_budget_ratio=0.5, obs_window=4,
+                                  pool_kernel_size=3, pool_padding="reflect",
+                                  v_bit_options=torch.tensor([0., 2, 4, 8, 16]),
+                                  k_bit_options=torch.tensor([0., 2, 4, 8]),
+                                  epsilon_v=ks.DEFAULT_EPSILON_V, epsilon_k=ks.DEFAULT_EPSILON_K,
+                                  correctness_check=True)
+
+
+@pytest.mark.parametrize("n_tokens", [37, 48, 5])
+def test_schedule_report_and_coverage(setup, n_tokens):
+    model, prompt, pre, cache = setup
+    block = 16
+    ids, report = bw.greedy_decode_blockwise(
+        model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1], max_new_tokens=n_tokens,
+        eos_token_ids=[], primary_device=torch.device(DEV), decode_position_start=T_PROMPT, config=_config(block, 4))
+    assert len(ids) == n_tokens and report["generated_tokens"] == n_tokens
+    plan = bw.plan_block_compressions(n_tokens, block)
+    assert report["num_compressed_decode_blocks"] == len(plan) == len(report["block_events"])
+    cov = report["coverage"]
+    assert cov[0][0] == 0 and cov[-1][1] == n_tokens - 1
+    assert all(a[1] + 1 == b[0] for a, b in zip(cov, cov[1:]))
+    for ev, exp in zip(report["block_events"], plan):
+        assert all(ev[k] == exp[k] for k in exp)
+    assert len(report["per_token_timestamps_ms"]) == n_tokens
+    assert report["decode_cache_peak_fp16_equivalent_tokens"] <= 2 * block + 4 * len(plan) + 1e-6
+    assert report["memory_trace"][0]["stage"] == "decode_start" and report["memory_trace"][-1]["stage"] == "decode_complete"
+    assert report["avg_tpot_ms"] > 0 and report["decode_cuda_graph"] is False
+    # the prompt's own per-layer caches are untouched: the plain loop still runs on them
+    again = fast_decode.greedy_decode_fast(model, cache, pre.logits[0, -1], 3, [], torch.device(DEV), T_PROMPT)
+    assert again == ids[:3]
+
+
+def test_full_precision_blocks_track_model_forward(setup):
+    """Budget = block size: every block keeps 16-bit V and 8-bit K, so the loop over
+    [prompt | blocks | tail] must follow ``model.forward`` over the dense cache."""
+    model, prompt, pre, cache = setup
+    n_tokens, block = 30, 8
+    seen = []
+    orig = fast_decode._linear_row
+
+    def spy(x, weight, bias=None):
+        y = orig(x, weight, bias)
+        if weight is model.lm_head.weight:
+            seen.append(y[0, -1].float().cpu())
+        return y
+
+    fast_decode._linear_row = spy
+    try:
+        ids, report = bw.greedy_decode_blockwise(
+            model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1], max_new_tokens=n_tokens,
+            eos_token_ids=[], primary_device=torch.device(DEV), decode_position_start=T_PROMPT,
+            config=_config(block, block))
+    finally:
+        fast_decode._linear_row = orig
+    assert report["num_compressed_decode_blocks"] == 4 and len(seen) == n_tokens
+    with torch.no_grad():
+        pkv = model(prompt, use_cache=True).past_key_values
+        for step, tok in enumerate(ids):
+            o = model(torch.tensor([[tok]], device=DEV), past_key_values=pkv, use_cache=True)
+            pkv = o.past_key_values
+            exp = o.logits[0, -1].float().cpu()
+            cos = float(torch.nn.functional.cosine_similarity(seen[step], exp, dim=0))
+            assert cos > 0.998, f"step {step}: cosine {cos}"
+
+
+def test_block_scores_are_sums_of_softmax_weights(setup, monkeypatch):
+    """What ``_compress_block`` receives: per layer [H_kv, block tokens] scores that are sums, over
+    the scoring queries and the group's heads, of softmax weights (blockwise_decode.py:2085-2109):
+    non-negative, and a token cannot collect more than one unit per (query, head)."""
+    model, prompt, pre, cache = setup
+    block, n_tokens, G = 8, 29, H_Q // H_KV
+    calls = []
+    orig = bw._compress_block
+
+    def spy(**kw):
+        calls.append({k: kw[k] for k in ("token_scores_by_layer", "query_block", "causal", "token_start", "token_end")})
+        return orig(**kw)
+
+    monkeypatch.setattr(bw, "_compress_block", spy)
+    bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
+                               max_new_tokens=n_tokens, eos_token_ids=[], primary_device=torch.device(DEV),
+                               decode_position_start=T_PROMPT, config=_config(block, 3))
+    assert len(calls) == 4
+    for c in calls:
+        n_target = c["token_end"] - c["token_start"] + 1
+        n_query = c["query_block"][0].shape[1]
+        for scores, queries in zip(c["token_scores_by_layer"], c["query_block"]):
+            assert tuple(scores.shape) == (H_KV, n_target) and tuple(queries.shape) == (H_Q, n_query, D)
+            assert torch.isfinite(scores).all() and float(scores.min()) >= 0.0
+            assert float(scores.max()) <= G * n_query + 1e-4
+            assert float(scores.sum(dim=1).max()) <= G * n_query + 1e-4
+            if c["causal"]:       # every query attends at least to itself: the diagonal mass is positive
+                assert float(scores.sum()) > 0.0
+
+
+def test_eos_stops_and_flushes(setup):
+    model, prompt, pre, cache = setup
+    ids, _ = bw.greedy_decode_blockwise(
+        model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1], max_new_tokens=20, eos_token_ids=[],
+        primary_device=torch.device(DEV), decode_position_start=T_PROMPT, config=_config(8, 2))
+    out, report = bw.greedy_decode_blockwise(
+        model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1], max_new_tokens=20,
+        eos_token_ids=[ids[11]], primary_device=torch.device(DEV), decode_position_start=T_PROMPT,
+        config=_config(8, 2))
+    stop = ids.index(ids[11])
+    assert out == ids[:stop] and report["generated_tokens"] == stop
+    assert report["coverage"][-1][1] == stop - 1 if stop else report["coverage"] == []
+    with pytest.raises(NotImplementedError):
+        bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
+                                   max_new_tokens=4, eos_token_ids=[], primary_device=torch.device(DEV),
+                                   decode_position_start=T_PROMPT, config=_config(8, 2), use_cuda_graph=True)
+    with pytest.raises(RuntimeError):
+        bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
+                                   max_new_tokens=4, eos_token_ids=[], primary_device=torch.device("cpu"),
+                                   decode_position_start=T_PROMPT, config=_config(8, 2))
