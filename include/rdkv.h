@@ -169,6 +169,14 @@ int rdkv_rope_append_kv(const void *k, int64_t k_stride_h, const void *v, int64_
  * the product as the two tensor operations do. */
 int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtype, void *out, void *stream);
 
+/* blockwise_decode.py:2085-2109: the online block scores of blockwise decode from one step's
+ * zone-C weights w [H_kv*G, >= current_len] (rdkv_decode_fused_merge_zone_c's zone_c_weights):
+ * self_scores[h, t] += sum_g w[h*G+g, t] for t in [q_block_start, current_len), and, when
+ * q_block_start >= block, next_scores[h, t] += sum_g w[h*G+g, t] for t < block. */
+int rdkv_tail_scores(const float *w, int64_t w_stride_row, int H_kv, int G, int q_block_start,
+                     int current_len, int block, float *self_scores, int64_t self_stride_h,
+                     float *next_scores, int64_t next_stride_h, void *stream);
+
 /* fast_decode.py:1650-1656, 1786, 1797-1804, 1826: the projections of a decode step, each
  * F.linear on one activation row there.  y[n] = sum_k W[n,k] * x[k] (+ bias[n]); W [N, K] with
  * row stride w_stride_row (elements), bias [N] or NULL, y [N], all fp16 or all bf16 (`dtype`);

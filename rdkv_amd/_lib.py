@@ -59,6 +59,7 @@ SIGNATURES = {
     "rdkv_add_rms_norm": (I, [P, L, P, L, P, I, F, I, I, I, P, L, P, L, P]),
     "rdkv_rope_append_kv": (I, [P, L, P, L, I, I, I, P, P, I, P, L, L, P, L, P]),
     "rdkv_silu_mul": (I, [P, P, L, I, P, P]),
+    "rdkv_tail_scores": (I, [P, L, I, I, I, I, I, P, L, P, L, P]),
     "rdkv_gemv": (I, [P, L, P, I, P, I, I, I, P, P]),
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
     "rdkv_pack_layer_plan_ints": (L, [I, L]),

@@ -519,6 +519,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     from .triton_rope import fused_rope
 
     config.validate()
+    lib = _lib.load()
     dev = torch.device(primary_device)
     if dev.type != "cuda":
         raise RuntimeError("blockwise packed decode requires CUDA")
@@ -659,12 +660,11 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                 _rope_append_kv(k_2d, v_2d, one, zero, rows, write_row)     # k is rotated already: identity table
                 decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse,
                                   zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights)
-                # block scores from the tail's weights (blockwise_decode.py:2085-2109)
-                width = current_len - q_block_start
-                self_scores[layer][:, q_block_start:current_len].add_(
-                    tail_weights[:, q_block_start:current_len].view(h_kv, groups, width).sum(dim=1))
-                if q_block_start >= block:
-                    next_scores[layer].add_(tail_weights[:, :block].view(h_kv, groups, block).sum(dim=1))
+                # block scores from the tail's weights (blockwise_decode.py:2085-2109), one launch
+                _lib.check(lib.rdkv_tail_scores(
+                    tail_weights.data_ptr(), tail_weights.stride(0), h_kv, groups, q_block_start, current_len, block,
+                    self_scores[layer].data_ptr(), self_scores[layer].stride(0), next_scores[layer].data_ptr(),
+                    next_scores[layer].stride(0), _lib.stream_of(dev)))
                 if config.correctness_check and not torch.isfinite(attn_out).all():
                     raise FloatingPointError(f"non-finite attention output at layer {layer}")
                 o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)

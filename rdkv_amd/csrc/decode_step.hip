@@ -96,7 +96,46 @@ silu_mul_kernel(const void *__restrict__ gate, const void *__restrict__ up, int6
   rdkv_store_from_float(out, dtype, i, act * rdkv_load_as_float(up, dtype, i));
 }
 
+// Online block scores of blockwise decode (blockwise_decode.py:2085-2109) from the raw tail's
+// softmax weights w [H_kv * G, >= current_len] of one step: the weights of this step's query on the
+// tokens of its own block go to self_scores, those on the first block (when the query belongs to
+// the second) to next_scores, each summed over the G query heads of a KV head in head order.
+__global__ void __launch_bounds__(256)
+tail_scores_kernel(const float *__restrict__ w, int64_t w_stride, int G, int q_block_start, int current_len,
+                   int block, float *__restrict__ self_scores, int64_t self_stride,
+                   float *__restrict__ next_scores, int64_t next_stride) {
+  const int h = blockIdx.x;
+  const float *rows = w + (int64_t)h * G * w_stride;
+  for (int t = q_block_start + threadIdx.x; t < current_len; t += 256) {
+    float s = 0.0f;
+    for (int g = 0; g < G; ++g) s += rows[g * w_stride + t];
+    self_scores[h * self_stride + t] += s;
+  }
+  if (q_block_start >= block) {
+    for (int t = threadIdx.x; t < block; t += 256) {
+      float s = 0.0f;
+      for (int g = 0; g < G; ++g) s += rows[g * w_stride + t];
+      next_scores[h * next_stride + t] += s;
+    }
+  }
+}
+
 }  // namespace
+
+RDKV_API int rdkv_tail_scores(const float *w, int64_t w_stride_row, int H_kv, int G, int q_block_start,
+                              int current_len, int block, float *self_scores, int64_t self_stride_h,
+                              float *next_scores, int64_t next_stride_h, void *stream) {
+  RDKV_REQUIRE(H_kv >= 0 && G >= 1 && block >= 1 && q_block_start >= 0 && current_len >= q_block_start,
+               "rdkv_tail_scores: bad arguments");
+  if (H_kv == 0) return RDKV_OK;
+  RDKV_REQUIRE(w && self_scores && next_scores, "rdkv_tail_scores: null pointer");
+  RDKV_REQUIRE(w_stride_row >= current_len && self_stride_h >= current_len && next_stride_h >= block,
+               "rdkv_tail_scores: rows shorter than the tail");
+  hipLaunchKernelGGL(tail_scores_kernel, dim3(H_kv), dim3(256), 0, (hipStream_t)stream, w, w_stride_row, G,
+                     q_block_start, current_len, block, self_scores, self_stride_h, next_scores, next_stride_h);
+  RDKV_CHECK_LAUNCH("rdkv_tail_scores");
+  return RDKV_OK;
+}
 
 RDKV_API int rdkv_add_rms_norm(const void *x, int64_t x_stride_row, const void *delta, int64_t delta_stride_row,
                                const void *weight, int w_dtype, float eps, int rows, int dim, int dtype,

@@ -159,3 +159,28 @@ def test_eos_stops_and_flushes(setup):
         bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
                                    max_new_tokens=4, eos_token_ids=[], primary_device=torch.device("cpu"),
                                    decode_position_start=T_PROMPT, config=_config(8, 2))
+
+
+def test_tail_scores_kernel_matches_tensor_expressions():
+    """``rdkv_tail_scores`` against blockwise_decode.py:2085-2109 of the reference as tensor
+    operations, for a query in the first and in the second block of the tail."""
+    require_gpu()
+    from rdkv_amd import _lib
+    lib = _lib.load()
+    h_kv, G, block = 3, 4, 16
+    g = torch.Generator(device=DEV).manual_seed(6)
+    for write_pos in (0, 5, 15, 16, 23, 31):
+        current_len = write_pos + 1
+        qbs = (write_pos // block) * block
+        w = torch.rand(h_kv * G, 2 * block + 3, generator=g, device=DEV)
+        self_s = torch.rand(h_kv, 2 * block, generator=g, device=DEV)
+        next_s = torch.rand(h_kv, block, generator=g, device=DEV)
+        exp_self, exp_next = self_s.clone(), next_s.clone()
+        exp_self[:, qbs:current_len] += w[:, qbs:current_len].view(h_kv, G, current_len - qbs).sum(dim=1)
+        if qbs >= block:
+            exp_next += w[:, :block].view(h_kv, G, block).sum(dim=1)
+        _lib.check(lib.rdkv_tail_scores(w.data_ptr(), w.stride(0), h_kv, G, qbs, current_len, block,
+                                        self_s.data_ptr(), self_s.stride(0), next_s.data_ptr(), next_s.stride(0),
+                                        _lib.stream_of(torch.device(DEV))))
+        torch.testing.assert_close(self_s, exp_self, rtol=1e-6, atol=1e-6)
+        torch.testing.assert_close(next_s, exp_next, rtol=1e-6, atol=1e-6)
