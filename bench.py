@@ -102,6 +102,26 @@ def decode_loop_section(cfg, torch, dev, tokens=48):
             dt = (time.perf_counter() - t0) / max(len(ids), 1) * 1e3
             best = dt if best is None else min(best, dt)
         res[f"ms_per_token_{name}"] = best
+    # the blockwise variant: the generated tokens are re-compressed in blocks of 128 (budget 16)
+    import contextlib
+    import io
+    from rdkv_amd import blockwise_decode as bw, knapsack_solver as ks
+    conf = bw.BlockwiseRDKVConfig(
+        block_size=128, block_budget_tokens=16, k_budget_ratio=0.5, obs_window=32, pool_kernel_size=5,
+        pool_padding="reflect", v_bit_options=torch.tensor([0., 2, 4, 8, 16]),
+        k_bit_options=torch.tensor([0., 2, 4, 8]), epsilon_v=ks.DEFAULT_EPSILON_V, epsilon_k=ks.DEFAULT_EPSILON_K)
+    n_bw = 272
+    for _ in range(2):
+        with contextlib.redirect_stdout(io.StringIO()):       # the loop logs one event line per block
+            ids, report = bw.greedy_decode_blockwise(
+                model=model, dual_cache=cache, next_token_logits=first, max_new_tokens=n_bw, eos_token_ids=[],
+                primary_device=dev, decode_position_start=sc.context, config=conf)
+    ts = report["per_token_timestamps_ms"]
+    steps = sorted(b - a for a, b in zip(ts, ts[1:]))
+    res["blockwise"] = {"tokens": len(ids), "block_size": 128, "block_budget_tokens": 16,
+                        "ms_per_token_avg": report["avg_tpot_ms"], "ms_per_token_median": steps[len(steps) // 2],
+                        "ms_slowest_step": steps[-1], "compressed_blocks": report["num_compressed_decode_blocks"],
+                        "final_flush_ms": report["final_flush_time_ms"]}
     return res
 
 
