@@ -161,18 +161,18 @@ def test_decode_loop_tracks_model_forward(setup):
 
 
 def test_graph_replay_gives_the_eager_tokens(setup):
-    model, prompt, pre, kv = setup
+    model, prompt, pre, kv = setup          # 80 tokens: the raw tail crosses the 64-token chunk of the merge kernel
     v_bits, k_bits = _mixed_bits(12)
     first = pre.logits[0, -1]
-    eager = fast_decode.greedy_decode_fast(model, _pack(kv, v_bits, k_bits), first, 24, [], torch.device(DEV),
+    eager = fast_decode.greedy_decode_fast(model, _pack(kv, v_bits, k_bits), first, 80, [], torch.device(DEV),
                                            T_PROMPT)
     cache = _pack(kv, v_bits, k_bits)
-    graphed = fast_decode.greedy_decode_fast(model, cache, first, 24, [], torch.device(DEV), T_PROMPT,
+    graphed = fast_decode.greedy_decode_fast(model, cache, first, 80, [], torch.device(DEV), T_PROMPT,
                                              use_cuda_graph=True)
-    assert graphed == eager and len(eager) == 24
+    assert graphed == eager and len(eager) == 80
     # a second run over the same cache object reuses its streaming caches and zone C buffers
     torch.cuda.synchronize()
-    assert fast_decode.greedy_decode_fast(model, cache, first, 24, [], torch.device(DEV), T_PROMPT,
+    assert fast_decode.greedy_decode_fast(model, cache, first, 80, [], torch.device(DEV), T_PROMPT,
                                           use_cuda_graph=True) == eager
 
 
