@@ -326,3 +326,35 @@ def test_decode_loop_follows_other_model_families(family):
             assert cos > 0.999, f"{family} step {step}: cosine {cos}"
     assert fast_decode.greedy_decode_fast(model, cache, pre.logits[0, -1], 4, [], torch.device(DEV), 200,
                                           use_cuda_graph=True) == ids
+
+
+def test_graph_replay_with_model_sized_projections():
+    """Llama-3.1-8B-sized projections and vocabulary (two layers): every token of 70 graph replays
+    equals the eager run's - the argmax over 128 256 logits, the large GEMVs and the merge with a
+    raw tail past one chunk all sit inside the captured step."""
+    require_gpu()
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from rdkv_amd import synth
+    L = 2
+    cfg = LlamaConfig(hidden_size=4096, intermediate_size=14336, num_hidden_layers=L, num_attention_heads=32,
+                      num_key_value_heads=8, head_dim=128, vocab_size=128256, max_position_embeddings=8192,
+                      rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False)
+    torch.manual_seed(0)
+    with torch.device(DEV):
+        model = LlamaForCausalLM(cfg).half().eval()
+    sc = synth.scaled(synth.CONFIGS[1], layers=L, context=1024)
+    layers, v16 = [], []
+    for i in range(L):
+        vb, kb, oc = synth.layer_allocation(sc, i)
+        K, V, _ = synth.layer_data(sc, i, DEV, outliers=oc)
+        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, sc.G)
+        layers.append(pl)
+        v16.append(nvo)
+    cache = packing.TriZoneCache(tuple(layers), v16, [None] * L, [None] * L, sc.context)
+    first = torch.randn(cfg.vocab_size, generator=torch.Generator().manual_seed(1)).to(DEV)
+    dev = torch.device(DEV)
+    eager = fast_decode.greedy_decode_fast(model, cache, first, 70, [], dev, sc.context)
+    graphed = fast_decode.greedy_decode_fast(model, cache, first, 70, [], dev, sc.context, use_cuda_graph=True)
+    assert graphed == eager and len(set(eager)) > 35
+    del model
+    torch.cuda.empty_cache()
