@@ -84,6 +84,7 @@ def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     ``rdkv_gemv`` when the shape allows it (fp16 / bf16 weights, K a multiple of 512 up to 32768,
     16-byte aligned rows; x of the weights' type or fp32, which the kernel rounds while staging
     it), the library GEMM otherwise."""
+    dev = _lib.require_device(x, weight)          # no CPU path: the library product below is the GPU's too
     N, K = weight.shape
     ok = (x.numel() == K and x.dtype in (weight.dtype, torch.float32)
           and weight.dtype in (torch.float16, torch.bfloat16)
@@ -92,7 +93,6 @@ def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
           and (bias is None or (bias.dtype == weight.dtype and bias.is_contiguous())))
     if not ok:
         return F.linear(x.to(weight.dtype), weight, bias)
-    dev = _lib.require_device(x, weight)
     y = torch.empty(x.shape[:-1] + (N,), dtype=weight.dtype, device=dev)
     _lib.check(_lib.load().rdkv_gemv(weight.data_ptr(), weight.stride(0), x.data_ptr(), _lib.DTYPE_CODE[x.dtype],
                                      _lib.ptr(bias), N, K, _lib.DTYPE_CODE[weight.dtype], y.data_ptr(),
