@@ -515,7 +515,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
     from .fast_decode import (_layer_stream_caches, _linear_row, _rms_norm, _rope_append_kv, _silu_mul,
                               pre_extract_weights)
-    from .stream_cache import decode_attn_fused, extend_stream_cache
+    from .stream_cache import decode_attn_fused, extend_stream_caches
     from .triton_rope import fused_rope
 
     config.validate()
@@ -602,9 +602,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
             config=config, num_kv_groups=groups, model_dtype=model_dtype)
         compressed.append(new_block)
         block_events.append(event)
-        for layer in range(L):
-            caches[layer] = extend_stream_cache(caches[layer], [(new_block.packed[layer], new_block.new_v_only[layer])],
-                                                row_of_entry=[0])
+        caches[:] = extend_stream_caches(caches, list(zip(new_block.packed, new_block.new_v_only)))
         remain = pending_len - target_len
         for kv_buf, q_buf, s_self, s_next in zip(pending_kv, pending_q, self_scores, next_scores):
             if remain:

@@ -206,10 +206,10 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     return work, groups, work_begin, work_count
 
 
-def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
+def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_bytes: Optional[list] = None):
     """Re-lay every (packed layer, new_v_only) entry into its own blob.  Returns the unit
     descriptors (absolute addresses, work fields unset), the blobs, and the streamed / algorithmic
-    byte counts of the entries."""
+    byte counts of the entries (``entry_bytes``, when given, also receives them per entry)."""
     lib = _lib.load()
     dev = _lib.require_device(layers[0][0].K_ch_scale)
     stream = _lib.stream_of(dev)
@@ -217,6 +217,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
     stream_bytes = algo_bytes = 0
     H_q = None
     for gi, (pl, nvo) in enumerate(layers):
+        sb0, ab0 = stream_bytes, algo_bytes
         H_kv = pl.K_ch_scale.shape[1]
         H_q = H_kv * G
         tok, ch = _layer_counts(pl, H_kv)
@@ -304,6 +305,8 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int]):
         units["v_off"] += base
         units_all.extend(units)
         blobs.append(blob)
+        if entry_bytes is not None:
+            entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
         # the temporaries stay alive until the relayout kernels have run
         keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
     torch.cuda.current_stream(dev).synchronize()
@@ -396,6 +399,27 @@ def extend_stream_cache(cache: StreamCache, layers: Sequence[Tuple[PackedKVLayer
     return _finish_cache(np.concatenate([old, new_units]), list(cache.blobs) + new_blobs, cache.G, H_q,
                          cache.stream_bytes + sb, cache.kv_algorithmic_bytes + ab, multi_source=True,
                          work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
+
+
+def extend_stream_caches(caches: Sequence[StreamCache],
+                         layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]]) -> List[StreamCache]:
+    """``extend_stream_cache(caches[i], [layers[i]], row_of_entry=[0])`` for every i with one pass
+    over the new entries (one launch sequence, one synchronisation): how a compressed decode block,
+    one packed layer per decoder layer, joins the per-layer caches of a sequential model loop."""
+    assert len(caches) == len(layers) and len(caches) > 0
+    G = caches[0].G
+    assert all(c.G == G for c in caches)
+    per_entry: list = []
+    new_units, new_blobs, _, _, H_q = _relayout_entries(layers, G, [0] * len(layers), per_entry)
+    n_per = len(new_units) // len(layers)
+    out = []
+    for i, cache in enumerate(caches):
+        assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
+        units = np.concatenate([cache.units_host.copy(), new_units[i * n_per:(i + 1) * n_per]])
+        out.append(_finish_cache(units, list(cache.blobs) + [new_blobs[i]], G, H_q, cache.stream_bytes + per_entry[i][0],
+                                 cache.kv_algorithmic_bytes + per_entry[i][1], multi_source=True, work_bytes=None,
+                                 n_groups=None, groups_per_cu=1, cost=None))
+    return out
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,

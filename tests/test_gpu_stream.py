@@ -386,3 +386,21 @@ def test_zone_c_weights_are_the_softmax_over_the_union(n_new):
     # the weights output changes nothing else
     out2, lse2 = stream_cache.decode_attn_fused(cache, q, zone_c=(buf[:, :, :128], buf[:, :, 128:], counts))
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
+def test_extend_many_caches_at_once_equals_one_by_one():
+    """``extend_stream_caches``: every cache gets its own new source exactly as the single-cache
+    call gives it (same units, same result bits)."""
+    cfg = synth.scaled(synth.CONFIGS[1], context=500, layers=6)
+    packed, q6, _ = _config_case(cfg, 6)
+    q = q6[:cfg.H_q].contiguous()
+    base = [stream_cache.build_stream_cache([packed[i]], cfg.G) for i in range(3)]
+    new = [packed[3 + i] for i in range(3)]
+    many = stream_cache.extend_stream_caches(base, new)
+    for i in range(3):
+        one = stream_cache.extend_stream_cache(base[i], [new[i]], row_of_entry=[0])
+        assert many[i].n_units == one.n_units and many[i].n_work == one.n_work
+        assert many[i].stream_bytes == one.stream_bytes and many[i].algorithmic_bytes == one.algorithmic_bytes
+        a, la = stream_cache.decode_attn_fused(many[i], q)
+        b, lb = stream_cache.decode_attn_fused(one, q)
+        assert torch.equal(a, b) and torch.equal(la, lb)
