@@ -169,6 +169,19 @@ int rdkv_rope_append_kv(const void *k, int64_t k_stride_h, const void *v, int64_
  * the product as the two tensor operations do. */
 int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtype, void *out, void *stream);
 
+/* rdkv_gemv with the operation in front of it folded into the staging of the activation row
+ * (every workgroup stages the whole row the same way, a few KB from L2):
+ * rdkv_gemv_norm: x_n = norm_weight * (r * rsqrt(mean(r^2) + eps)), r = x + delta rounded to `dtype`
+ *   (delta NULL: r = x), the RMSNorm of rdkv_add_rms_norm; r is also written to residual_out (NULL,
+ *   or K values that alias neither input); y = W x_n (+ bias).  K at most 8192; norm_weight of `dtype`.
+ * rdkv_gemv_silu: y = W (silu(gate) * up) (+ bias), the activation rounded to `dtype` before the
+ *   product as in rdkv_silu_mul (fast_decode.py:1803-1804). */
+int rdkv_gemv_norm(const void *W, int64_t w_stride_row, const void *x, const void *delta,
+                   const void *norm_weight, float eps, void *residual_out, const void *bias, int N, int K,
+                   int dtype, void *y, void *stream);
+int rdkv_gemv_silu(const void *W, int64_t w_stride_row, const void *gate, const void *up, const void *bias,
+                   int N, int K, int dtype, void *y, void *stream);
+
 /* blockwise_decode.py:2085-2109: the online block scores of blockwise decode from one step's
  * zone-C weights w [H_kv*G, >= current_len] (rdkv_decode_fused_merge_zone_c's zone_c_weights):
  * self_scores[h, t] += sum_g w[h*G+g, t] for t in [q_block_start, current_len), and, when

@@ -61,6 +61,8 @@ SIGNATURES = {
     "rdkv_silu_mul": (I, [P, P, L, I, P, P]),
     "rdkv_tail_scores": (I, [P, L, I, I, I, I, I, P, L, P, L, P]),
     "rdkv_gemv": (I, [P, L, P, I, P, I, I, I, P, P]),
+    "rdkv_gemv_norm": (I, [P, L, P, P, P, F, P, P, I, I, I, P, P]),
+    "rdkv_gemv_silu": (I, [P, L, P, P, P, I, I, I, P, P]),
     "rdkv_decode_fused_merge": (I, [P, I, I, I, P, L, P, P, L, P]),
     "rdkv_pack_layer_plan_ints": (L, [I, L]),
     "rdkv_pack_layer_plan": (I, [P, I, L, P, I, L, I, L, I, P, L, P, L, P, P]),

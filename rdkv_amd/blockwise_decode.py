@@ -513,8 +513,8 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
 
     The reference needs its fixed-slot bank to replay this loop from graphs; that variant is not
     built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
-    from .fast_decode import (_layer_stream_caches, _linear_row, _rms_norm, _rope_append_kv, _silu_mul,
-                              pre_extract_weights)
+    from .fast_decode import (_layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm, _rope_append_kv,
+                              _silu_linear_row, pre_extract_weights)
     from .stream_cache import decode_attn_fused, extend_stream_caches
     from .triton_rope import fused_rope
 
@@ -644,8 +644,8 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
             n_tail.fill_(current_len)
             delta = None
             for layer, lw in enumerate(W.layers):
-                x = _rms_norm(h, lw.input_ln_weight, lw.input_ln_eps, delta=delta, residual_out=h)
-                q, k, v = _linear_row(x, lw.qkv_weight, lw.qkv_bias).split(lw.qkv_split_sizes, dim=-1)
+                qkv, h = _norm_linear_row(h, delta, lw.input_ln_weight, lw.input_ln_eps, lw.qkv_weight, lw.qkv_bias)
+                q, k, v = qkv.split(lw.qkv_split_sizes, dim=-1)
                 q_2d, k_2d, v_2d = q.view(h_q, D), k.view(h_kv, D), v.view(h_kv, D)
                 if lw.q_norm_weight is not None:
                     q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
@@ -666,9 +666,9 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                 if config.correctness_check and not torch.isfinite(attn_out).all():
                     raise FloatingPointError(f"non-finite attention output at layer {layer}")
                 o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)
-                x = _rms_norm(h, lw.post_ln_weight, lw.post_ln_eps, delta=o, residual_out=h)
-                gate, up = _linear_row(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
-                delta = _linear_row(_silu_mul(gate, up), lw.down_proj_weight)
+                gate_up, h = _norm_linear_row(h, o, lw.post_ln_weight, lw.post_ln_eps, lw.gate_up_weight)
+                gate, up = gate_up.split(lw.gate_up_split_sizes, dim=-1)
+                delta = _silu_linear_row(gate, up, lw.down_proj_weight)
             hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
             logits = _linear_row(hidden, W.lm_head_weight)
             next_token = logits[:, -1, :].argmax(dim=-1, keepdim=True)

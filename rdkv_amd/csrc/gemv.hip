@@ -35,37 +35,118 @@ __device__ __forceinline__ float dot8(const uint4 w, const uint4 x, float acc) {
   return acc;
 }
 
+template <int dtype>
+__device__ __forceinline__ void unpack8(const uint4 v, float (&f)[8]) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (dtype == RDKV_DTYPE_F16) {
+      f[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] & 0xffffu));
+      f[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[j] >> 16));
+    } else {
+      f[2 * j] = __uint_as_float(w[j] << 16);
+      f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+template <int dtype>
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {   // rounds to the storage type
+  uint32_t w[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint32_t lo, hi;
+    if (dtype == RDKV_DTYPE_F16) {
+      lo = __builtin_bit_cast(uint16_t, (_Float16)f[2 * j]);
+      hi = __builtin_bit_cast(uint16_t, (_Float16)f[2 * j + 1]);
+    } else {
+      lo = rdkv_float_to_bf16_bits(f[2 * j]);
+      hi = rdkv_float_to_bf16_bits(f[2 * j + 1]);
+    }
+    w[j] = lo | (hi << 16);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// How the activation row reaches LDS.  kPlain: x as stored.  kFromF32: x is fp32 and is rounded to
+// the weights' type (what a cast in front of the product would store).  kNorm: x = weight_n *
+// (r * rsqrt(mean(r^2) + eps)) with r = a + b rounded to the type (b may be NULL), the RMSNorm
+// with its residual add in front; workgroup 0 also writes r to residual_out.  kSilu: x =
+// silu(a) * b with the activation rounded to the type first.  Every workgroup stages the whole
+// row (a few KB from L2), in the same order, so all of them see the same bits.
+enum { kPlain = 0, kFromF32 = 1, kNorm = 2, kSilu = 3 };
+struct RowSource {
+  const void *a, *b, *c;
+  float eps;
+  void *residual_out;
+};
+
 // K % 512 == 0 (every lane takes whole 16-byte pieces: K / 512 per row), rows 16-byte aligned.
-// x32: x is fp32 and is rounded to the weights' type while it is staged (what a cast in front of
-// the product would store).
-template <int dtype, int R>
+template <int dtype, int R, int MODE>
 __global__ void __launch_bounds__(256)
-gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, const void *__restrict__ x, int x32,
+gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, RowSource src,
             const uint16_t *__restrict__ bias, int N, int K, int rows_per_wave, uint16_t *__restrict__ y) {
-  extern __shared__ uint4 xs[];      // K / 8 pieces of x
+  extern __shared__ uint4 xs[];      // K / 8 pieces of x (kNorm: then K / 8 pieces of the norm weight + 4 floats)
   const int k8 = K >> 3;
-  if (x32) {
-    const float4 *xf = reinterpret_cast<const float4 *>(x);
+  if (MODE == kFromF32) {
+    const float4 *xf = reinterpret_cast<const float4 *>(src.a);
     for (int i = threadIdx.x; i < k8; i += 256) {
       const float4 a = xf[2 * i], b = xf[2 * i + 1];
       const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-      uint32_t w[4];
+      xs[i] = pack8<dtype>(v);
+    }
+  } else if (MODE == kNorm) {
+    uint4 *ws = xs + k8;
+    float *s_part = reinterpret_cast<float *>(xs + 2 * k8);
+    const uint4 *pa = reinterpret_cast<const uint4 *>(src.a);
+    const uint4 *pb = reinterpret_cast<const uint4 *>(src.b ? src.b : src.a);   // loads stay unconditional
+    const uint4 *pc = reinterpret_cast<const uint4 *>(src.c);
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < k8; i += 256) {
+      const uint4 va = pa[i], vb = pb[i];
+      ws[i] = pc[i];
+      float fa[8], fb[8];
+      unpack8<dtype>(va, fa);
+      unpack8<dtype>(vb, fb);
+      uint4 r = va;
+      if (src.b) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        uint32_t lo, hi;
-        if (dtype == RDKV_DTYPE_F16) {
-          lo = __builtin_bit_cast(uint16_t, (_Float16)v[2 * j]);
-          hi = __builtin_bit_cast(uint16_t, (_Float16)v[2 * j + 1]);
-        } else {
-          lo = rdkv_float_to_bf16_bits(v[2 * j]);
-          hi = rdkv_float_to_bf16_bits(v[2 * j + 1]);
-        }
-        w[j] = lo | (hi << 16);
+        for (int e = 0; e < 8; ++e) fa[e] += fb[e];
+        r = pack8<dtype>(fa);
+        unpack8<dtype>(r, fa);
       }
-      xs[i] = make_uint4(w[0], w[1], w[2], w[3]);
+      xs[i] = r;
+      if (blockIdx.x == 0 && src.residual_out) reinterpret_cast<uint4 *>(src.residual_out)[i] = r;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += fa[e] * fa[e];
+    }
+    ss = rdkv_wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float rs = rsqrtf((s_part[0] + s_part[1] + s_part[2] + s_part[3]) / (float)K + src.eps);
+    for (int i = threadIdx.x; i < k8; i += 256) {   // the pieces this thread wrote itself
+      float fr[8], fw[8];
+      unpack8<dtype>(xs[i], fr);
+      unpack8<dtype>(ws[i], fw);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) fr[e] = fw[e] * (fr[e] * rs);
+      xs[i] = pack8<dtype>(fr);
+    }
+  } else if (MODE == kSilu) {
+    const uint4 *pa = reinterpret_cast<const uint4 *>(src.a), *pb = reinterpret_cast<const uint4 *>(src.b);
+    for (int i = threadIdx.x; i < k8; i += 256) {
+      float g[8], u[8];
+      unpack8<dtype>(pa[i], g);
+      unpack8<dtype>(pb[i], u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = g[e] / (1.0f + expf(-g[e]));
+      const uint4 act = pack8<dtype>(g);       // the activation is rounded before the product
+      unpack8<dtype>(act, g);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] *= u[e];
+      xs[i] = pack8<dtype>(g);
     }
   } else {
-    for (int i = threadIdx.x; i < k8; i += 256) xs[i] = reinterpret_cast<const uint4 *>(x)[i];
+    for (int i = threadIdx.x; i < k8; i += 256) xs[i] = reinterpret_cast<const uint4 *>(src.a)[i];
   }
   __syncthreads();
   const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -107,9 +188,9 @@ gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, const void *__
   }
 }
 
-template <int dtype>
-void launch_gemv(const void *W, int64_t w_stride_row, const void *x, int x32, const void *bias, int N, int K,
-                 void *y, int n_cu, hipStream_t s) {
+template <int dtype, int MODE>
+void launch_gemv(const void *W, int64_t w_stride_row, const RowSource &src, const void *bias, int N, int K, void *y,
+                 int n_cu, hipStream_t s) {
   // eight wavefronts per compute unit when there are rows enough; a wavefront takes at least R rows
   const int max_waves = n_cu * 8;
   const int R = N >= 4 * max_waves ? 4 : 2;
@@ -118,30 +199,18 @@ void launch_gemv(const void *W, int64_t w_stride_row, const void *x, int x32, co
   int rows_per_wave = (int)rdkv_cdiv(N, waves);
   rows_per_wave = (int)rdkv_cdiv(rows_per_wave, R) * R;
   const int blocks = (int)rdkv_cdiv(rdkv_cdiv(N, rows_per_wave), 4);
-  const size_t lds = (size_t)K * 2;
+  const size_t lds = MODE == kNorm ? (size_t)K * 4 + 16 : (size_t)K * 2;
   if (R == 4)
-    hipLaunchKernelGGL((gemv_kernel<dtype, 4>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W, w_stride_row,
-                       x, x32, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
+    hipLaunchKernelGGL((gemv_kernel<dtype, 4, MODE>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W,
+                       w_stride_row, src, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
   else
-    hipLaunchKernelGGL((gemv_kernel<dtype, 2>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W, w_stride_row,
-                       x, x32, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
+    hipLaunchKernelGGL((gemv_kernel<dtype, 2, MODE>), dim3(blocks), dim3(256), lds, s, (const uint16_t *)W,
+                       w_stride_row, src, (const uint16_t *)bias, N, K, rows_per_wave, (uint16_t *)y);
 }
 
-}  // namespace
-
-RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x_dtype, const void *bias, int N,
-                       int K, int dtype, void *y, void *stream) {
-  const char *fn = "rdkv_gemv";
-  RDKV_REQUIRE(N >= 0 && K > 0, "%s: bad shape N=%d K=%d", fn, N, K);
-  RDKV_REQUIRE(dtype == RDKV_DTYPE_F16 || dtype == RDKV_DTYPE_BF16, "%s: fp16 or bf16 weights only", fn);
-  RDKV_REQUIRE(x_dtype == dtype || x_dtype == RDKV_DTYPE_F32, "%s: x must have the weights' type or be fp32", fn);
-  RDKV_REQUIRE(K % 512 == 0 && K <= 32768, "%s: K=%d must be a multiple of 512, at most 32768", fn, K);
-  if (N == 0) return RDKV_OK;
-  RDKV_REQUIRE(W && x && y, "%s: null pointer", fn);
-  RDKV_REQUIRE(((uintptr_t)W % 16) == 0 && ((uintptr_t)x % 16) == 0 && w_stride_row % 8 == 0 && w_stride_row >= K,
-               "%s: W rows and x must be 16-byte aligned", fn);
-  // compute units of the current device, asked once per device (0 = not asked yet; a race between
-  // two first calls stores the same number twice)
+int compute_units() {
+  // of the current device, asked once per device (0 = not asked yet; a race between two first calls
+  // stores the same number twice)
   static int cu_of_device[64];
   int dev = 0, n_cu = 256;
   if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
@@ -152,8 +221,71 @@ RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x
     }
     if (cu_of_device[dev] > 0) n_cu = cu_of_device[dev];
   }
-  if (dtype == RDKV_DTYPE_F16) launch_gemv<RDKV_DTYPE_F16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
-  else launch_gemv<RDKV_DTYPE_BF16>(W, w_stride_row, x, x_dtype == RDKV_DTYPE_F32, bias, N, K, y, n_cu, (hipStream_t)stream);
+  return n_cu;
+}
+
+int check_gemv(const char *fn, const void *W, int64_t w_stride_row, int N, int K, int dtype, const void *y) {
+  RDKV_REQUIRE(N >= 0 && K > 0, "%s: bad shape N=%d K=%d", fn, N, K);
+  RDKV_REQUIRE(dtype == RDKV_DTYPE_F16 || dtype == RDKV_DTYPE_BF16, "%s: fp16 or bf16 weights only", fn);
+  RDKV_REQUIRE(K % 512 == 0 && K <= 32768, "%s: K=%d must be a multiple of 512, at most 32768", fn, K);
+  if (N == 0) return RDKV_OK;
+  RDKV_REQUIRE(W && y, "%s: null pointer", fn);
+  RDKV_REQUIRE(((uintptr_t)W % 16) == 0 && w_stride_row % 8 == 0 && w_stride_row >= K,
+               "%s: W rows must be 16-byte aligned", fn);
+  return RDKV_OK;
+}
+
+template <int MODE>
+void launch_any(int dtype, const void *W, int64_t w_stride_row, const RowSource &src, const void *bias, int N, int K,
+                void *y, hipStream_t s) {
+  const int n_cu = compute_units();
+  if (dtype == RDKV_DTYPE_F16) launch_gemv<RDKV_DTYPE_F16, MODE>(W, w_stride_row, src, bias, N, K, y, n_cu, s);
+  else launch_gemv<RDKV_DTYPE_BF16, MODE>(W, w_stride_row, src, bias, N, K, y, n_cu, s);
+}
+
+}  // namespace
+
+RDKV_API int rdkv_gemv(const void *W, int64_t w_stride_row, const void *x, int x_dtype, const void *bias, int N,
+                       int K, int dtype, void *y, void *stream) {
+  const char *fn = "rdkv_gemv";
+  int rc = check_gemv(fn, W, w_stride_row, N, K, dtype, y);
+  if (rc != RDKV_OK || N == 0) return rc;
+  RDKV_REQUIRE(x_dtype == dtype || x_dtype == RDKV_DTYPE_F32, "%s: x must have the weights' type or be fp32", fn);
+  RDKV_REQUIRE(x && ((uintptr_t)x % 16) == 0, "%s: x must be 16-byte aligned", fn);
+  const RowSource src = {x, nullptr, nullptr, 0.0f, nullptr};
+  if (x_dtype == RDKV_DTYPE_F32) launch_any<kFromF32>(dtype, W, w_stride_row, src, bias, N, K, y, (hipStream_t)stream);
+  else launch_any<kPlain>(dtype, W, w_stride_row, src, bias, N, K, y, (hipStream_t)stream);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_gemv_norm(const void *W, int64_t w_stride_row, const void *x, const void *delta,
+                            const void *norm_weight, float eps, void *residual_out, const void *bias, int N, int K,
+                            int dtype, void *y, void *stream) {
+  const char *fn = "rdkv_gemv_norm";
+  int rc = check_gemv(fn, W, w_stride_row, N, K, dtype, y);
+  if (rc != RDKV_OK || N == 0) return rc;
+  RDKV_REQUIRE(x && norm_weight, "%s: null pointer", fn);
+  RDKV_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)delta % 16) == 0 && ((uintptr_t)norm_weight % 16) == 0 &&
+                   ((uintptr_t)residual_out % 16) == 0, "%s: rows must be 16-byte aligned", fn);
+  RDKV_REQUIRE(!residual_out || (residual_out != x && residual_out != delta),
+               "%s: residual_out must not alias the inputs (every workgroup reads them)", fn);
+  RDKV_REQUIRE(K <= 8192, "%s: K=%d exceeds 8192", fn, K);
+  const RowSource src = {x, delta, norm_weight, eps, residual_out};
+  launch_any<kNorm>(dtype, W, w_stride_row, src, bias, N, K, y, (hipStream_t)stream);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_gemv_silu(const void *W, int64_t w_stride_row, const void *gate, const void *up, const void *bias,
+                            int N, int K, int dtype, void *y, void *stream) {
+  const char *fn = "rdkv_gemv_silu";
+  int rc = check_gemv(fn, W, w_stride_row, N, K, dtype, y);
+  if (rc != RDKV_OK || N == 0) return rc;
+  RDKV_REQUIRE(gate && up && ((uintptr_t)gate % 16) == 0 && ((uintptr_t)up % 16) == 0,
+               "%s: gate / up must be 16-byte aligned rows", fn);
+  const RowSource src = {gate, up, nullptr, 0.0f, nullptr};
+  launch_any<kSilu>(dtype, W, w_stride_row, src, bias, N, K, y, (hipStream_t)stream);
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

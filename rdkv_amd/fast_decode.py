@@ -100,6 +100,56 @@ def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     return y
 
 
+def _row_ok(*tensors: torch.Tensor) -> bool:
+    return all(t.is_contiguous() and t.data_ptr() % 16 == 0 for t in tensors)
+
+
+def _gemv_weight_ok(weight: torch.Tensor, bias: Optional[torch.Tensor], k_max: int) -> bool:
+    K = weight.shape[1]
+    return (weight.dtype in (torch.float16, torch.bfloat16) and K % 512 == 0 and K <= k_max
+            and weight.stride(1) == 1 and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0
+            and (bias is None or (bias.dtype == weight.dtype and bias.is_contiguous())))
+
+
+def _norm_linear_row(h: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
+                     weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Residual add, RMSNorm and projection of one activation row (fast_decode.py:1640-1656 and
+    1786-1798): returns ``(F.linear(rms_norm(h + delta), weight, bias), h + delta)``.  One launch
+    (``rdkv_gemv_norm``: the norm is folded into the staging of the row) when the shapes allow it,
+    ``_rms_norm`` + ``_linear_row`` otherwise."""
+    dev = _lib.require_device(h, weight)
+    N, K = weight.shape
+    fused = (_gemv_weight_ok(weight, bias, 8192) and h.numel() == K and h.dtype == weight.dtype
+             and norm_weight.dtype == weight.dtype and _row_ok(h, norm_weight)
+             and (delta is None or (delta.dtype == h.dtype and delta.numel() == K and _row_ok(delta))))
+    if not fused:
+        x = _rms_norm(h, norm_weight, eps, delta=delta, residual_out=h)
+        return _linear_row(x, weight, bias), h
+    h_new = torch.empty_like(h) if delta is not None else h
+    y = torch.empty(h.shape[:-1] + (N,), dtype=weight.dtype, device=dev)
+    _lib.check(_lib.load().rdkv_gemv_norm(
+        weight.data_ptr(), weight.stride(0), h.data_ptr(), _lib.ptr(delta), norm_weight.data_ptr(), float(eps),
+        h_new.data_ptr() if delta is not None else None, _lib.ptr(bias), N, K, _lib.DTYPE_CODE[weight.dtype],
+        y.data_ptr(), _lib.stream_of(dev)))
+    return y, h_new
+
+
+def _silu_linear_row(gate: torch.Tensor, up: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """``F.linear(F.silu(gate) * up, weight)`` for one row (fast_decode.py:1803-1804): one launch
+    (``rdkv_gemv_silu``) when the shapes allow it, ``_silu_mul`` + ``_linear_row`` otherwise."""
+    dev = _lib.require_device(gate, up, weight)
+    N, K = weight.shape
+    fused = (_gemv_weight_ok(weight, None, 32768) and gate.numel() == K and up.numel() == K
+             and gate.dtype == weight.dtype and up.dtype == weight.dtype and gate.stride(-1) == 1
+             and up.stride(-1) == 1 and gate.data_ptr() % 16 == 0 and up.data_ptr() % 16 == 0)
+    if not fused:
+        return _linear_row(_silu_mul(gate, up), weight)
+    y = torch.empty(gate.shape[:-1] + (N,), dtype=weight.dtype, device=dev)
+    _lib.check(_lib.load().rdkv_gemv_silu(weight.data_ptr(), weight.stride(0), gate.data_ptr(), up.data_ptr(), None,
+                                          N, K, _lib.DTYPE_CODE[weight.dtype], y.data_ptr(), _lib.stream_of(dev)))
+    return y
+
+
 def _silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """``F.silu(gate) * up`` (fast_decode.py:1803) in one launch; both [..., n] with unit stride."""
     dev = _lib.require_device(gate, up)
@@ -335,11 +385,11 @@ class _DecodeStep:
     """One greedy decode step over device-resident state, written so that the same calls run
     eagerly or are captured once into a HIP graph: the token, its position, the zone C write row
     and the zone C token counts live in device tensors that the step itself advances, so a replay
-    needs no argument from the host.  Per layer, ten launches: residual add + RMSNorm, one q/k/v
-    GEMV, rotary embedding of k + append of the fp32 K|V row to zone C, zones A+B+C attention
-    (two launches, q rotated while the kernel stages it), output projection (its fp32 input rounded
-    to the model type while it is staged), residual add + RMSNorm, gate/up GEMV, SiLU * up, down
-    projection."""
+    needs no argument from the host.  Per layer, seven launches: q/k/v GEMV with the residual add
+    and RMSNorm folded into the staging of its input row, rotary embedding of k + append of the
+    fp32 K|V row to zone C, zones A+B+C attention (two launches, q rotated while the kernel stages
+    it), output projection (its fp32 input rounded to the model type while it is staged), gate/up
+    GEMV (residual add + RMSNorm folded in), down projection (SiLU * up folded in)."""
 
     def __init__(self, W: PreExtractedWeights, caches: List[StreamCache], new_kv_buf: List[torch.Tensor],
                  dtype: torch.dtype):
@@ -368,8 +418,8 @@ class _DecodeStep:
         rope = (cos.view(D)[:D // 2], sin.view(D)[:D // 2])
         delta = None                                                     # branch output not yet added to h
         for lw, cache, buf in zip(W.layers, self.caches, self.new_kv_buf):
-            x = _rms_norm(h, lw.input_ln_weight, lw.input_ln_eps, delta=delta, residual_out=h)
-            q, k, v = _linear_row(x, lw.qkv_weight, lw.qkv_bias).split(lw.qkv_split_sizes, dim=-1)
+            qkv, h = _norm_linear_row(h, delta, lw.input_ln_weight, lw.input_ln_eps, lw.qkv_weight, lw.qkv_bias)
+            q, k, v = qkv.split(lw.qkv_split_sizes, dim=-1)
             q_2d, k_2d, v_2d = q.view(W.num_heads, D), k.view(W.num_kv_heads, D), v.view(W.num_kv_heads, D)
             if lw.q_norm_weight is not None:
                 q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
@@ -380,9 +430,9 @@ class _DecodeStep:
             decode_attn_fused(cache, q_2d, out=self.attn_out, lse=self.lse, rope=rope,   # q rotated while staged
                               zone_c=(rows[:, :, :D], rows[:, :, D:], self.n_new))
             o = _linear_row(self.attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)     # fp32 in, rounded inside
-            x = _rms_norm(h, lw.post_ln_weight, lw.post_ln_eps, delta=o, residual_out=h)
-            gate, up = _linear_row(x, lw.gate_up_weight).split(lw.gate_up_split_sizes, dim=-1)
-            delta = _linear_row(_silu_mul(gate, up), lw.down_proj_weight)
+            gate_up, h = _norm_linear_row(h, o, lw.post_ln_weight, lw.post_ln_eps, lw.gate_up_weight)
+            gate, up = gate_up.split(lw.gate_up_split_sizes, dim=-1)
+            delta = _silu_linear_row(gate, up, lw.down_proj_weight)
         self.hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
         self.logits = _linear_row(self.hidden, W.lm_head_weight)
         self.token.copy_(self.logits[:, -1, :].argmax(dim=-1, keepdim=True))

@@ -358,3 +358,40 @@ def test_graph_replay_with_model_sized_projections():
     assert graphed == eager and len(set(eager)) > 35
     del model
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_fused_row_projections_match_their_compositions(dtype):
+    """``_norm_linear_row`` (residual add + RMSNorm folded into the GEMV's staging) and
+    ``_silu_linear_row`` against the separate launches they replace; shapes the fused kernels do
+    not take fall back to those launches."""
+    require_gpu()
+    g = torch.Generator(device=DEV).manual_seed(21)
+    ulp = {torch.float16: 2.0 ** -10, torch.bfloat16: 2.0 ** -7}[dtype]
+    for N, K in ((6144, 4096), (1000, 512), (28672, 4096), (300, 8192)):
+        W = (torch.randn(N, K, generator=g, device=DEV) / K ** 0.5).to(dtype)
+        h = torch.randn(1, 1, K, generator=g, device=DEV).to(dtype)
+        d = torch.randn(1, 1, K, generator=g, device=DEV).to(dtype)
+        nw = (1.0 + 0.1 * torch.randn(K, generator=g, device=DEV)).to(dtype)
+        b = torch.randn(N, generator=g, device=DEV).to(dtype)
+        for delta, bias in ((d, None), (None, b), (d, b)):
+            h_in = h.clone()
+            y, h_new = fast_decode._norm_linear_row(h_in, delta, nw, 1e-5, W, bias)
+            assert torch.equal(h_in, h), "the fused form leaves its inputs alone"
+            exp_h = h + delta if delta is not None else h
+            assert torch.equal(h_new, exp_h)
+            x = fast_decode._rms_norm(exp_h, nw, 1e-5)
+            exp = x.double().view(1, K) @ W.double().T + (bias.double() if bias is not None else 0.0)
+            torch.testing.assert_close(y.double().view(1, N), exp, rtol=4 * ulp, atol=4 * ulp)
+    for N, K in ((4096, 14336), (512, 1024)):
+        W = (torch.randn(N, K, generator=g, device=DEV) / K ** 0.5).to(dtype)
+        gu = (2 * torch.randn(1, 1, 2 * K, generator=g, device=DEV)).to(dtype)
+        gate, up = gu.split((K, K), dim=-1)
+        assert torch.equal(fast_decode._silu_linear_row(gate, up, W),
+                           fast_decode._linear_row(fast_decode._silu_mul(gate, up), W))
+    # K outside the fused kernels: the separate launches
+    W = torch.randn(32, 16384, generator=g, device=DEV).to(dtype) * 0.01
+    h = torch.randn(1, 1, 16384, generator=g, device=DEV).to(dtype)
+    nw = torch.ones(16384, device=DEV, dtype=dtype)
+    y, h2 = fast_decode._norm_linear_row(h, None, nw, 1e-5, W)
+    torch.testing.assert_close(y, fast_decode._linear_row(fast_decode._rms_norm(h, nw, 1e-5), W))
