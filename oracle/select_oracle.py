@@ -24,10 +24,11 @@ Parity status:
   * ``score_block``, ``logical_layer_bits``: textbook formulas, pinned by the reference's own
     known-answer tests (tests/test_blockwise_rdkv.py:70-101 of the reference) and by the library
     routines they reduce to (einsum + softmax).
-  * ``select_joint``: the budget arithmetic between the pinned pieces follows
-    obkv_fast.py:979-1041 by reading; the reference module that holds it cannot be imported
-    without the model stack, so that glue is **parity unpinned** (the pieces either side of it
-    are pinned as above, and its closed forms are tested: budgets in bits, K rows of empty heads).
+  * ``select_joint`` (obkv_fast.py:979-1041, the budget arithmetic between the pieces above):
+    pinned by ``tests/golden/select_joint_{a,b,c,d}.npz`` (allocations and packed layers returned
+    by the reference's own ``_perhead_select_and_pack_joint`` on seeded inputs: ragged heads, a
+    head that keeps nothing, fp16-kept tokens, each pooling mode) and by its closed forms
+    (budgets in bits, K rows of empty heads).
 """
 from __future__ import annotations
 

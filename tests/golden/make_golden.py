@@ -364,6 +364,48 @@ def case_knapsack():
     save("knapsack", d)
 
 
+def case_select_joint():
+    """Allocations and the packed layer of the reference's joint per-head selection
+    (obkv_fast.py:899-1190) on small seeded CPU inputs: pooled scores -> V knapsack over the
+    whole row, K budget spread over the tokens each head kept, per-head K knapsack, pack.
+    One case has a head whose scores are all zero (it keeps nothing)."""
+    import obkv_fast as of
+
+    def one(name, seed, h_kv, groups, t_len, head_dim, budget, ratio, kernel, pool_type, padding,
+            zero_head=None):
+        g = torch.Generator().manual_seed(seed)
+        K = (torch.randn(1, h_kv, t_len, head_dim, generator=g) * 1.5).half()
+        V = torch.randn(1, h_kv, t_len, head_dim, generator=g).half()
+        ls = torch.exp(torch.randn(h_kv, t_len, generator=g) * 1.5 + 1.0)
+        if zero_head is not None:
+            ls[zero_head] = 0.0
+        cs = torch.exp(torch.randn(h_kv, head_dim, generator=g) * 1.2)
+        packed, new_v, t_eff = of._perhead_select_and_pack_joint(
+            K, V, ls, cs, gqa_factor=groups, token_budget=budget, k_budget_ratio=ratio,
+            obs_window=0, pool_kernel_size=kernel, pool_padding=padding, pool_type=pool_type,
+            v_bit_options=None, k_bit_options=None,
+            eps_V=dict(of.DEFAULT_EPSILON_V), eps_K=dict(of.DEFAULT_EPSILON_K),
+            retain_allocation_metadata=True)
+        d = {"K": npy(K), "V": npy(V), "layer_scores": npy(ls), "channel_scores": npy(cs),
+             "params": np.array([h_kv, groups, t_len, head_dim, budget, kernel], dtype=np.int64),
+             "k_budget_ratio": np.array(ratio, dtype=np.float64),
+             "pool_type": np.array(pool_type), "pool_padding": np.array(padding),
+             "t_eff": np.array(int(t_eff), dtype=np.int64)}
+        put_layer(d, "packed", packed)
+        if isinstance(new_v, (tuple, list)):
+            for i, x in enumerate(new_v):
+                if x is not None:
+                    d[f"new_v.{i}"] = npy(x)
+        elif new_v is not None:
+            d["new_v"] = npy(new_v)
+        save(name, d)
+
+    one("select_joint_a", 1201, 3, 2, 96, 32, 8, 0.5, 7, "avg", "reflect")
+    one("select_joint_b", 1202, 2, 4, 80, 64, 6, 0.375, 5, "max", "zero", zero_head=1)
+    one("select_joint_c", 1203, 2, 1, 64, 32, 40, 0.5, 1, "avg", "zero")
+    one("select_joint_d", 1204, 2, 2, 72, 32, 12, 0.5, 3, "max", "reflect")
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
     if len(sys.argv) > 2:                      # python make_golden.py <ref> <case> : one case only
@@ -382,3 +424,4 @@ if __name__ == "__main__":
     case_shared_layout()
     case_rope()
     case_knapsack()
+    case_select_joint()

@@ -14,8 +14,8 @@ from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
 from rdkv_amd import obkv_fast
 from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev
-from tests.helpers import load_golden
-from tests.test_oracle_select import POOL_CASES, golden_batched_cases
+from tests.helpers import assert_layer_equal, load_golden
+from tests.test_oracle_select import POOL_CASES, SELECT_JOINT_GOLDEN, golden_batched_cases, select_joint_golden
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -161,6 +161,24 @@ SELECT_CASES = {
     "k16": (2, 1, 256, 120, 0.6, (2, 4, 8, 16), False),
     "tight": (4, 4, 1500, 64, 0.5, (0, 2, 4, 8), False),
 }
+
+
+@pytest.mark.parametrize("name", SELECT_JOINT_GOLDEN)
+def test_select_and_pack_joint_matches_reference_outputs(name):
+    """Every field of the packed layer, the retained allocation and the fp16-kept values against what
+    the reference's own `_perhead_select_and_pack_joint` returned for the same inputs."""
+    g, groups, knobs = select_joint_golden(name)
+    knobs.pop("head_dim")
+    layer, new_v, t_eff = obkv_fast._perhead_select_and_pack_joint(
+        to_dev(g["K"]), to_dev(g["V"]), to_dev(g["layer_scores"]), torch.from_numpy(g["channel_scores"]),
+        gqa_factor=groups, obs_window=0, v_bit_options=None, k_bit_options=None,
+        eps_V=ks.DEFAULT_EPSILON_V, eps_K=ks.DEFAULT_EPSILON_K, retain_allocation_metadata=True, **knobs)
+    assert_layer_equal(layer, g, "packed")
+    assert int(t_eff) == int(g["t_eff"])
+    if "new_v" in g:
+        assert_bits_equal(t2n(new_v), g["new_v"])
+    else:
+        assert new_v is None
 
 
 @pytest.mark.parametrize("case", sorted(SELECT_CASES))

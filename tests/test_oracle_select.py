@@ -8,8 +8,9 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
-from tests.helpers import load_golden
+from tests.helpers import assert_layer_equal, load_golden
 
 F32 = np.float32
 
@@ -156,3 +157,33 @@ def test_select_joint_budgets():
     _, vb0, kb0, k_avg0 = S.select_joint(ls0, cs, head_dim=D, token_budget=B, k_budget_ratio=0.5,
                                          pool_kernel_size=1, pool_padding="reflect", k_bit_options=(0, 2, 4, 8))
     assert (vb0[1] == 0).all() and k_avg0[1] == F32(0.5 * 32 * B * D) * (F32(1) / F32(D)) and (kb0[1] == 8).all()
+
+
+SELECT_JOINT_GOLDEN = ("select_joint_a", "select_joint_b", "select_joint_c", "select_joint_d")
+
+
+def select_joint_golden(name):
+    """Inputs and knobs of one stored run of the reference's joint per-head selection."""
+    g = load_golden(name)
+    h_kv, groups, t_len, head_dim, budget, kernel = (int(x) for x in g["params"])
+    knobs = dict(head_dim=head_dim, token_budget=budget, k_budget_ratio=float(g["k_budget_ratio"]),
+                 pool_kernel_size=kernel, pool_padding=str(g["pool_padding"]), pool_type=str(g["pool_type"]))
+    return g, groups, knobs
+
+
+@pytest.mark.parametrize("name", SELECT_JOINT_GOLDEN)
+def test_select_joint_matches_reference_outputs(name):
+    """The allocation the reference's own `_perhead_select_and_pack_joint` made on seeded inputs
+    (heads that keep different token counts, a head that keeps nothing, fp16-kept tokens, max and
+    average pooling, no pooling), and the packed layer it built from it."""
+    g, groups, knobs = select_joint_golden(name)
+    _, vb, kb, _ = S.select_joint(g["layer_scores"], g["channel_scores"], **knobs)
+    np.testing.assert_array_equal(vb, g["packed.allocation_v_bits"].astype(np.int64))
+    np.testing.assert_array_equal(kb, g["packed.allocation_k_bits"].astype(np.int64))
+    layer, v16 = O.pack_layer_per_head(g["K"], g["V"], vb, kb, groups)
+    assert_layer_equal(layer, g, "packed", skip=("allocation_v_bits", "allocation_k_bits"))
+    assert int(g["t_eff"]) == layer.T_eff
+    if "new_v" in g:
+        assert np.array_equal(np.asarray(v16).view(np.uint8), g["new_v"].view(np.uint8))
+    else:
+        assert v16 is None
