@@ -87,6 +87,35 @@ gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, RowSource src,
             const uint16_t *__restrict__ bias, int N, int K, int rows_per_wave, uint16_t *__restrict__ y) {
   extern __shared__ uint4 xs[];      // K / 8 pieces of x (kNorm: then K / 8 pieces of the norm weight + 4 floats)
   const int k8 = K >> 3;
+  // A wavefront walks its rows R at a time and each group of rows in pieces of 256 x 16 bytes
+  // ("tiles": 4 loads per row and lane).  The loads of the next tile are issued before the
+  // current one is consumed, and those of the first tile before the row is staged, so the
+  // staging and every reduction overlap a weight fetch that is already in flight.
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(blockIdx.x * 4 + (threadIdx.x >> 6));
+  const int row_begin = wave * rows_per_wave;
+  const int row_end = min(N, row_begin + rows_per_wave);
+  const int n_j = (k8 + 255) >> 8;
+  struct Cur { int r0, jj; };
+  auto next = [&](Cur c) __attribute__((always_inline)) -> Cur {
+    if (c.jj + 1 < n_j) return Cur{c.r0, c.jj + 1};
+    return Cur{c.r0 + R, 0};
+  };
+  auto load_tile = [&](Cur c, uint4 (&wv)[R][4]) __attribute__((always_inline)) {
+    const int j0 = lane + 256 * c.jj;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = j0 + 64 * u < k8 ? j0 + 64 * u : j0;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int row = c.r0 + r < row_end ? c.r0 + r : c.r0;
+        wv[r][u] = load_stream(reinterpret_cast<const uint4 *>(W + (int64_t)row * w_stride_row) + j);
+      }
+    }
+  };
+  uint4 wa[R][4], wb[R][4];
+  Cur ca{row_begin, 0};
+  if (ca.r0 < row_end) load_tile(ca, wa);
   if (MODE == kFromF32) {
     const float4 *xf = reinterpret_cast<const float4 *>(src.a);
     for (int i = threadIdx.x; i < k8; i += 256) {
@@ -149,42 +178,39 @@ gemv_kernel(const uint16_t *__restrict__ W, int64_t w_stride_row, RowSource src,
     for (int i = threadIdx.x; i < k8; i += 256) xs[i] = reinterpret_cast<const uint4 *>(src.a)[i];
   }
   __syncthreads();
-  const int lane = threadIdx.x & 63, wave = blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int row_begin = wave * rows_per_wave;
-  const int row_end = min(N, row_begin + rows_per_wave);
-  for (int r0 = row_begin; r0 < row_end; r0 += R) {
-    float acc[R];
-    const uint4 *wr[R];
+  float acc[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      acc[r] = 0.0f;
-      wr[r] = reinterpret_cast<const uint4 *>(W + (int64_t)(r0 + r < row_end ? r0 + r : r0) * w_stride_row);
-    }
-    for (int j0 = lane; j0 < k8; j0 += 64 * 4) {
-      uint4 wv[R][4];
+  for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+  auto compute_tile = [&](Cur c, const uint4 (&wv)[R][4]) __attribute__((always_inline)) {
+    const int j0 = lane + 256 * c.jj;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int j = j0 + 64 * u < k8 ? j0 + 64 * u : j0;
+    for (int u = 0; u < 4; ++u) {
+      if (j0 + 64 * u < k8) {
+        const uint4 xv = xs[j0 + 64 * u];
 #pragma unroll
-        for (int r = 0; r < R; ++r) wv[r][u] = load_stream(wr[r] + j);
+        for (int r = 0; r < R; ++r) acc[r] = dot8<dtype>(wv[r][u], xv, acc[r]);
       }
+    }
+    if (c.jj + 1 == n_j) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (j0 + 64 * u < k8) {
-          const uint4 xv = xs[j0 + 64 * u];
-#pragma unroll
-          for (int r = 0; r < R; ++r) acc[r] = dot8<dtype>(wv[r][u], xv, acc[r]);
+      for (int r = 0; r < R; ++r) {
+        const float s = rdkv_wave_sum(acc[r]);
+        if (lane == 0 && c.r0 + r < row_end) {
+          const float b = bias ? rdkv_load_as_float(bias, dtype, c.r0 + r) : 0.0f;
+          rdkv_store_from_float(y, dtype, c.r0 + r, s + b);
         }
+        acc[r] = 0.0f;
       }
     }
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const float s = rdkv_wave_sum(acc[r]);
-      if (lane == 0 && r0 + r < row_end) {
-        const float b = bias ? rdkv_load_as_float(bias, dtype, r0 + r) : 0.0f;
-        rdkv_store_from_float(y, dtype, r0 + r, s + b);
-      }
-    }
+  };
+  while (ca.r0 < row_end) {
+    const Cur cb = next(ca);
+    if (cb.r0 < row_end) load_tile(cb, wb);
+    compute_tile(ca, wa);
+    if (cb.r0 >= row_end) break;
+    ca = next(cb);
+    if (ca.r0 < row_end) load_tile(ca, wa);
+    compute_tile(cb, wb);
   }
 }
 
