@@ -318,6 +318,28 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
                                    float *zone_c_weights, int64_t zone_c_weights_stride_row,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 
+/* rdkv_decode_fused_merge_zone_c with the append of the step's own token folded into the same
+ * launch (fast_decode.py:1690 rotary embedding of the new key, :1722-1724 its append to the new
+ * zone, then the attention above): k_step / v_step are the un-rotated key and value rows
+ * [rows / G, 128] of kv_dtype (head r at + r*stride, elements).  The workgroup of output row r
+ * rotates the key with rope_cos / rope_sin (NULL: taken as it is), rounds it to kv_dtype as the
+ * in-place rotation would store it, and writes fp32 key and value to token row_dev[0] (device
+ * int64; outside 0..capacity-1: nothing is written) of k_new / v_new before it attends over
+ * n_new_per_unit[r] tokens (required; they include the new row).  capacity: tokens per row of the
+ * zone-C buffers.  Saves the separate rdkv_rope_append_kv launch of a decode step. */
+int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, int n_work, int G,
+                                          const void *q, int q_dtype, int64_t q_stride_row,
+                                          const void *rope_cos, const void *rope_sin, int rope_dtype,
+                                          float *k_new, float *v_new, int64_t new_stride_unit,
+                                          int64_t new_stride_tok, int64_t capacity,
+                                          const int32_t *n_new_per_unit,
+                                          const void *k_step, int64_t k_stride_h,
+                                          const void *v_step, int64_t v_stride_h, int kv_dtype,
+                                          const int64_t *row_dev,
+                                          float *out, int64_t out_stride_row, float *lse,
+                                          float *zone_c_weights, int64_t zone_c_weights_stride_row,
+                                          void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Planning for rdkv_pack_layer_per_head on the device (what the reference derives on the host:
  * packing.py:1417-1431 stable token sort by width, :241-294 channel classes).  v_bits [H_kv, T]
  * and k_bits [H_kv, D]: integers of 1, 2, 4 or 8 bytes, head strides in elements.  Writes

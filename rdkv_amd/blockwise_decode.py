@@ -513,7 +513,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
 
     The reference needs its fixed-slot bank to replay this loop from graphs; that variant is not
     built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
-    from .fast_decode import (_layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm, _rope_append_kv,
+    from .fast_decode import (_layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
                               _silu_linear_row, pre_extract_weights)
     from .stream_cache import decode_attn_fused, extend_stream_caches
     from .triton_rope import fused_rope
@@ -543,7 +543,6 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     lse = torch.empty(h_q, dtype=torch.float32, device=dev)
     write_row = torch.zeros(1, dtype=torch.long, device=dev)
     n_tail = torch.zeros(h_kv, dtype=torch.int32, device=dev)
-    one, zero = torch.ones(D // 2, dtype=model_dtype, device=dev), torch.zeros(D // 2, dtype=model_dtype, device=dev)
 
     generated: List[int] = []
     compressed: List[CompressedDecodeBlock] = []
@@ -655,9 +654,9 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                 fused_rope(q_2d, k_2d, cos_half, sin_half)          # the rotated query is kept for the channel scores
                 pending_q[layer][:, write_pos, :].copy_(q_2d)
                 rows = pending_kv[layer][0]
-                _rope_append_kv(k_2d, v_2d, one, zero, rows, write_row)     # k is rotated already: identity table
-                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse,
-                                  zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights)
+                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse,       # k is rotated already: appended as it is
+                                  zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights,
+                                  append=(k_2d, v_2d, write_row))
                 # block scores from the tail's weights (blockwise_decode.py:2085-2109), one launch
                 _lib.check(lib.rdkv_tail_scores(
                     tail_weights.data_ptr(), tail_weights.stride(0), h_kv, groups, q_block_start, current_len, block,

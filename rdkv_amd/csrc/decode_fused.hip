@@ -767,6 +767,14 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
 // 1/sqrt(D) first as the reference does.
 constexpr int kZcChunk = 64;
 constexpr int kZcWaves = 8;
+// The new token's un-rotated key and value rows (k == nullptr: nothing to append).
+struct ZcAppend {
+  const void *k, *v;
+  int64_t k_stride_h, v_stride_h;
+  const int64_t *row_dev;
+  int64_t capacity;
+  int dtype;
+};
 // G is a template parameter: the per-head loops unroll into straight-line code (with a run-time
 // G every head of every token is a scalar branch).
 template <int G>
@@ -774,10 +782,10 @@ __global__ void __launch_bounds__(64 * kZcWaves)
 merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride,
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
-                    const float *__restrict__ k_new, const float *__restrict__ v_new, int64_t new_stride_unit,
+                    float *k_new, float *v_new, int64_t new_stride_unit,   // written when a row is appended
                     int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
                     float *__restrict__ out, int64_t out_stride, float *__restrict__ lse,
-                    float *zc_w, int64_t zc_w_stride) {
+                    float *zc_w, int64_t zc_w_stride, ZcAppend ap) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
   __shared__ float fin_m[8], fin_l[8];             // softmax maximum and sum over the union, per head
   __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
@@ -793,6 +801,33 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
   // the query (and its rotation table) is fetched before the merge so that the two overlap
   const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
+  if (ap.k) {
+    // The step's own token joins zone C here (first wavefront; the others go on): k rotated and
+    // rounded to its storage type as the in-place rotation stores it, k and v widened to fp32.
+    // The barriers between here and the token loop make the row visible to every wavefront.
+    const int64_t row = ap.row_dev[0];
+    if (row >= 0 && row < ap.capacity && tid < 64) {
+      const int64_t ko = (int64_t)kv_row * ap.k_stride_h, vo = (int64_t)kv_row * ap.v_stride_h;
+      const float lo = rdkv_load_as_float_nobranch(ap.k, ap.dtype, ko + tid);
+      const float hi = rdkv_load_as_float_nobranch(ap.k, ap.dtype, ko + tid + 64);
+      const float v_lo = rdkv_load_as_float_nobranch(ap.v, ap.dtype, vo + tid);
+      const float v_hi = rdkv_load_as_float_nobranch(ap.v, ap.dtype, vo + tid + 64);
+      float out_lo = lo, out_hi = hi;
+      if (rope_cos) {
+        const float c = rdkv_load_as_float_nobranch(rope_cos, rope_dtype, tid);
+        const float sn = rdkv_load_as_float_nobranch(rope_sin, rope_dtype, tid);
+        rdkv_rope_pair(lo, hi, c, sn, out_lo, out_hi);
+        out_lo = rdkv_round_to_dtype(out_lo, ap.dtype);
+        out_hi = rdkv_round_to_dtype(out_hi, ap.dtype);
+      }
+      const int64_t off = (int64_t)kv_row * new_stride_unit + row * new_stride_tok;
+      float *kd = k_new + off, *vd = v_new + off;
+      kd[tid] = out_lo;
+      kd[tid + 64] = out_hi;
+      vd[tid] = v_lo;
+      vd[tid + 64] = v_hi;
+    }
+  }
   float qv[2], qo[2], qc[2], qs_[2];
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -1062,15 +1097,13 @@ RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n
                                  workspace_bytes, stream);
 }
 
-RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
-                                            int q_dtype, int64_t q_stride_row, const void *rope_cos,
-                                            const void *rope_sin, int rope_dtype, const float *k_new,
-                                            const float *v_new, int64_t new_stride_unit, int64_t new_stride_tok,
-                                            int n_new, const int32_t *n_new_per_unit, float *out,
-                                            int64_t out_stride_row, float *lse, float *zone_c_weights,
-                                            int64_t zone_c_weights_stride_row, void *workspace,
-                                            int64_t workspace_bytes, void *stream) {
-  const char *fn = "rdkv_decode_fused_merge_zone_c";
+static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
+                               int q_dtype, int64_t q_stride_row, const void *rope_cos, const void *rope_sin,
+                               int rope_dtype, const float *k_new, const float *v_new, int64_t new_stride_unit,
+                               int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit, float *out,
+                               int64_t out_stride_row, float *lse, float *zone_c_weights,
+                               int64_t zone_c_weights_stride_row, void *workspace, int64_t workspace_bytes,
+                               const ZcAppend &append, void *stream) {
   RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= n_new || n_new_per_unit,
                "%s: rows of the zone-C weights are shorter than n_new", fn);
   int rc = check_fused_args(fn, units, n_units, (const RdkvWork *)units, n_work, G, workspace, workspace_bytes);
@@ -1086,9 +1119,9 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
                "%s: zone-C key rows must be 16-byte aligned", fn);
 #define RDKV_LAUNCH_ZC(GT)                                                                                    \
   hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
-                     (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype, k_new, \
-                     v_new, new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
-                     zone_c_weights, zone_c_weights_stride_row)
+                     (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,        \
+                     const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
+                     zone_c_weights, zone_c_weights_stride_row, append)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;
     case 2: RDKV_LAUNCH_ZC(2); break;
@@ -1102,4 +1135,39 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
 #undef RDKV_LAUNCH_ZC
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
+}
+
+RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
+                                            int q_dtype, int64_t q_stride_row, const void *rope_cos,
+                                            const void *rope_sin, int rope_dtype, const float *k_new,
+                                            const float *v_new, int64_t new_stride_unit, int64_t new_stride_tok,
+                                            int n_new, const int32_t *n_new_per_unit, float *out,
+                                            int64_t out_stride_row, float *lse, float *zone_c_weights,
+                                            int64_t zone_c_weights_stride_row, void *workspace,
+                                            int64_t workspace_bytes, void *stream) {
+  const ZcAppend none = {nullptr, nullptr, 0, 0, nullptr, 0, 0};
+  return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, n_units, n_work, G, q, q_dtype, q_stride_row,
+                             rope_cos, rope_sin, rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, n_new,
+                             n_new_per_unit, out, out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row,
+                             workspace, workspace_bytes, none, stream);
+}
+
+RDKV_API int rdkv_decode_fused_merge_zone_c_append(
+    const RdkvUnit *units, int n_units, int n_work, int G, const void *q, int q_dtype, int64_t q_stride_row,
+    const void *rope_cos, const void *rope_sin, int rope_dtype, float *k_new, float *v_new, int64_t new_stride_unit,
+    int64_t new_stride_tok, int64_t capacity, const int32_t *n_new_per_unit, const void *k_step, int64_t k_stride_h,
+    const void *v_step, int64_t v_stride_h, int kv_dtype, const int64_t *row_dev, float *out, int64_t out_stride_row,
+    float *lse, float *zone_c_weights, int64_t zone_c_weights_stride_row, void *workspace, int64_t workspace_bytes,
+    void *stream) {
+  const char *fn = "rdkv_decode_fused_merge_zone_c_append";
+  RDKV_REQUIRE(k_step && v_step && row_dev && n_new_per_unit && k_new && v_new, "%s: null pointer", fn);
+  RDKV_REQUIRE(kv_dtype >= 0 && kv_dtype <= 2, "%s: unknown k/v dtype %d", fn, kv_dtype);
+  RDKV_REQUIRE(capacity >= 0 && capacity <= 0x7fffffffLL, "%s: bad zone-C capacity", fn);
+  RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= capacity,
+               "%s: rows of the zone-C weights are shorter than the buffer", fn);
+  const ZcAppend ap = {k_step, v_step, k_stride_h, v_stride_h, row_dev, capacity, kv_dtype};
+  return launch_merge_zone_c(fn, units, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,
+                             k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
+                             out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row, workspace,
+                             workspace_bytes, ap, stream);
 }

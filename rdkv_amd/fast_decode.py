@@ -385,10 +385,10 @@ class _DecodeStep:
     """One greedy decode step over device-resident state, written so that the same calls run
     eagerly or are captured once into a HIP graph: the token, its position, the zone C write row
     and the zone C token counts live in device tensors that the step itself advances, so a replay
-    needs no argument from the host.  Per layer, seven launches: q/k/v GEMV with the residual add
-    and RMSNorm folded into the staging of its input row, rotary embedding of k + append of the
-    fp32 K|V row to zone C, zones A+B+C attention (two launches, q rotated while the kernel stages
-    it), output projection (its fp32 input rounded to the model type while it is staged), gate/up
+    needs no argument from the host.  Per layer, six launches: q/k/v GEMV with the residual add
+    and RMSNorm folded into the staging of its input row, zones A+B+C attention (two launches: q
+    rotated while the streaming kernel stages it; the merge launch rotates k and appends the fp32
+    K|V row to zone C first), output projection (its fp32 input rounded to the model type while it is staged), gate/up
     GEMV (residual add + RMSNorm folded in), down projection (SiLU * up folded in)."""
 
     def __init__(self, W: PreExtractedWeights, caches: List[StreamCache], new_kv_buf: List[torch.Tensor],
@@ -426,9 +426,9 @@ class _DecodeStep:
             if lw.k_norm_weight is not None:
                 k_2d = _rms_norm(k_2d, lw.k_norm_weight, lw.qk_norm_eps)
             rows = buf[0]                                                # [H_kv, capacity, 2D] fp32, K | V
-            _rope_append_kv(k_2d, v_2d, rope[0], rope[1], rows, self.write_row)
             decode_attn_fused(cache, q_2d, out=self.attn_out, lse=self.lse, rope=rope,   # q rotated while staged
-                              zone_c=(rows[:, :, :D], rows[:, :, D:], self.n_new))
+                              zone_c=(rows[:, :, :D], rows[:, :, D:], self.n_new),
+                              append=(k_2d, v_2d, self.write_row))        # k rotated + appended by the merge launch
             o = _linear_row(self.attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)     # fp32 in, rounded inside
             gate_up, h = _norm_linear_row(h, o, lw.post_ln_weight, lw.post_ln_eps, lw.gate_up_weight)
             gate, up = gate_up.split(lw.gate_up_split_sizes, dim=-1)

@@ -426,7 +426,8 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                       lse: Optional[torch.Tensor] = None, *,
                       rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                       zone_c: Optional[Tuple[torch.Tensor, ...]] = None,
-                      zone_c_weights: Optional[torch.Tensor] = None):
+                      zone_c_weights: Optional[torch.Tensor] = None,
+                      append: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
@@ -435,7 +436,11 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     (output group, KV head) (optional int32 [rows / G] counts when they differ): the merge
     launch then returns the exact softmax over packed cache + new tokens.  ``zone_c_weights``
     (fp32 [rows, >= n_new], with ``zone_c``): receives the softmax weight of every new token over
-    the union, per query row (what blockwise decode sums into its block scores).  Graph-capturable
+    the union, per query row (what blockwise decode sums into its block scores).  ``append`` =
+    (k, v, row) with ``zone_c`` = (K_buf, V_buf, counts): the step's own un-rotated key and value
+    rows [rows / G, 128] (q's type) are rotated with ``rope`` (taken as they are without it),
+    widened to fp32 and stored as row ``row[0]`` (device int64) of the zone C buffers by the merge
+    launch itself, before it attends over ``counts`` tokens (which include that row).  Graph-capturable
     once the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
@@ -482,6 +487,27 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         ws.data_ptr(), ws.numel(), stream))
     n_new = int(K_new.shape[1])
+    if append is not None:
+        k_step, v_step, row = append
+        _lib.require_device(k_step, v_step, row)
+        assert counts is not None, "append needs the per-row token counts"
+        assert k_step.shape == (n_kv_rows, 128) and v_step.shape == (n_kv_rows, 128)
+        assert k_step.dtype == v_step.dtype and k_step.dtype in _lib.DTYPE_CODE
+        assert k_step.stride(1) == 1 and v_step.stride(1) == 1 and row.dtype == torch.int64 and row.numel() == 1
+        if zone_c_weights is not None:
+            _lib.require_device(zone_c_weights)
+            assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2
+            assert zone_c_weights.stride(1) == 1 and zone_c_weights.shape[0] == cache.rows
+            assert zone_c_weights.shape[1] >= n_new, f"zone_c_weights rows must hold {n_new} tokens"
+        _lib.check(lib.rdkv_decode_fused_merge_zone_c_append(
+            cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
+            q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
+            _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
+            counts.data_ptr(), k_step.data_ptr(), k_step.stride(0), v_step.data_ptr(), v_step.stride(0),
+            _lib.DTYPE_CODE[k_step.dtype], row.data_ptr(), out.data_ptr(), out.stride(0), lse.data_ptr(),
+            _lib.ptr(zone_c_weights), zone_c_weights.stride(0) if zone_c_weights is not None else 0,
+            ws.data_ptr(), ws.numel(), stream))
+        return out, lse
     if zone_c_weights is not None:
         _lib.require_device(zone_c_weights)
         assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2 and zone_c_weights.stride(1) == 1

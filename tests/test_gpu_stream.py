@@ -388,6 +388,52 @@ def test_zone_c_weights_are_the_softmax_over_the_union(n_new):
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
+@pytest.mark.parametrize("dtype,with_rope", [(torch.float16, True), (torch.bfloat16, True), (torch.float16, False)])
+def test_append_inside_the_merge_launch_equals_the_separate_append(dtype, with_rope):
+    """``append``: the merge launch rotates the step's key, stores the fp32 K|V row in zone C and
+    attends over it - the same buffer bits and the same result bits as ``rdkv_rope_append_kv``
+    followed by the plain zone C call, over several steps, with the appended row the only token,
+    in the middle and last in the buffer, and a row index outside the buffer writing nothing."""
+    from rdkv_amd import fast_decode
+    cfg = synth.scaled(synth.CONFIGS[1], context=600, layers=1)
+    packed, q1, _ = _config_case(cfg, 1)
+    cache = stream_cache.build_stream_cache(packed, cfg.G)
+    rows_kv = cache.rows // cfg.G
+    g = torch.Generator().manual_seed(77)
+    cap = 70
+    buf_a = torch.zeros(rows_kv, cap, 256, device=DEV)
+    buf_b = torch.zeros(rows_kv, cap, 256, device=DEV)
+    row = torch.zeros(1, dtype=torch.int64, device=DEV)
+    counts = torch.zeros(rows_kv, dtype=torch.int32, device=DEV)
+    ang = torch.rand(64, generator=g) * 6.28
+    rope = (torch.cos(ang).to(dtype).to(DEV), torch.sin(ang).to(dtype).to(DEV)) if with_rope else None
+    ident = (torch.ones(64, dtype=dtype, device=DEV), torch.zeros(64, dtype=dtype, device=DEV))
+    for step in (0, 1, 2, 40, 69):
+        row.fill_(step)
+        counts.fill_(step + 1)
+        q = torch.randn(cache.rows, 128, generator=g).to(dtype).to(DEV)
+        kv = torch.randn(rows_kv, 2, 128, generator=g).to(dtype).to(DEV)       # strided k / v rows
+        k, v = kv[:, 0], kv[:, 1]
+        if step > 2:                                                             # rows the loop did not visit
+            fill = torch.randn(rows_kv, cap, 256, generator=g).to(DEV)
+            buf_a.copy_(fill)
+            buf_b.copy_(fill)
+        fast_decode._rope_append_kv(k, v, *(rope or ident), buf_a, row)
+        exp = stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_a[:, :, :128], buf_a[:, :, 128:], counts))
+        w = torch.zeros(cache.rows, cap, device=DEV)
+        got = stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_b[:, :, :128], buf_b[:, :, 128:], counts),
+                                             append=(k, v, row), zone_c_weights=w)
+        assert torch.equal(buf_a, buf_b), f"step {step}: zone C rows differ"
+        assert torch.equal(exp[0], got[0]) and torch.equal(exp[1], got[1]), f"step {step}: attention differs"
+        assert float(w[:, :step + 1].sum(1).min()) > 0.0
+    before = buf_b.clone()
+    for bad in (-1, cap):
+        row.fill_(bad)
+        stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_b[:, :, :128], buf_b[:, :, 128:], counts),
+                                       append=(k, v, row))
+        assert torch.equal(before, buf_b)
+
+
 def test_extend_many_caches_at_once_equals_one_by_one():
     """``extend_stream_caches``: every cache gets its own new source exactly as the single-cache
     call gives it (same units, same result bits)."""
