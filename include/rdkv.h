@@ -190,6 +190,15 @@ int rdkv_tail_scores(const float *w, int64_t w_stride_row, int H_kv, int G, int 
                      int current_len, int block, float *self_scores, int64_t self_stride_h,
                      float *next_scores, int64_t next_stride_h, void *stream);
 
+/* Greedy choice of the next token and advance of a decode step's device-held state in one launch
+ * (fast_decode.py:1827 `logits.argmax(dim=-1)`, and the position / cache-length bookkeeping the
+ * reference keeps on the host, fast_decode.py:1606-1616): token[0] = index of the largest of the n
+ * logits (dtype fp32 / fp16 / bf16, 16-byte aligned; ties: the lowest index; a NaN counts as the
+ * largest value, as in the library routine), then counter_a[0] += 1 and counter_b[0] += 1 (device
+ * int64, each may be NULL) and counts[0..n_counts-1] += 1 (device int32, n_counts <= 1024). */
+int rdkv_argmax_advance(const void *logits, int n, int dtype, int64_t *token, int64_t *counter_a,
+                        int64_t *counter_b, int32_t *counts, int n_counts, void *stream);
+
 /* fast_decode.py:1650-1656, 1786, 1797-1804, 1826: the projections of a decode step, each
  * F.linear on one activation row there.  y[n] = sum_k W[n,k] * x[k] (+ bias[n]); W [N, K] with
  * row stride w_stride_row (elements), bias [N] or NULL, y [N], all fp16 or all bf16 (`dtype`);

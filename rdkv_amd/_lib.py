@@ -62,6 +62,7 @@ SIGNATURES = {
     "rdkv_rope_append_kv": (I, [P, L, P, L, I, I, I, P, P, I, P, L, L, P, L, P]),
     "rdkv_silu_mul": (I, [P, P, L, I, P, P]),
     "rdkv_tail_scores": (I, [P, L, I, I, I, I, I, P, L, P, L, P]),
+    "rdkv_argmax_advance": (I, [P, I, I, P, P, P, P, I, P]),
     "rdkv_gemv": (I, [P, L, P, I, P, I, I, I, P, P]),
     "rdkv_gemv_norm": (I, [P, L, P, P, P, F, P, P, I, I, I, P, P]),
     "rdkv_gemv_silu": (I, [P, L, P, P, P, I, I, I, P, P]),

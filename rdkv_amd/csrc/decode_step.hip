@@ -120,6 +120,79 @@ tail_scores_kernel(const float *__restrict__ w, int64_t w_stride, int G, int q_b
   }
 }
 
+// Greedy choice of the next token (fast_decode.py:1827 argmax of the step's logits) and the advance
+// of the step's device-held state, one workgroup: a thread scans pieces of 16 bytes, 1024 pieces
+// apart, sixteen loads in flight (a 128k vocabulary in fp16 is one batch); ties go to the lowest index and a NaN counts as the largest value
+// (the library's argmax).  counters: int64 values incremented by one (position, zone C write
+// row), counts: n_counts int32 values incremented by one (zone C lengths).
+struct Best { float v; int i; };
+__device__ __forceinline__ bool best_before(float a, int ia, float b, int ib) {
+  const bool na = a != a, nb = b != b;
+  if (na != nb) return na;
+  if (!na && a != b) return a > b;
+  return ia < ib;
+}
+template <int dtype>
+__global__ void __launch_bounds__(1024)
+argmax_advance_kernel(const void *__restrict__ logits, int n, int64_t *__restrict__ token,
+                      int64_t *__restrict__ counter_a, int64_t *__restrict__ counter_b,
+                      int32_t *__restrict__ counts, int n_counts) {
+  constexpr int EPP = dtype == RDKV_DTYPE_F32 ? 4 : 8;     // elements per 16-byte piece
+  __shared__ float s_v[16];
+  __shared__ int s_i[16];
+  const int tid = threadIdx.x, pieces = n / EPP;
+  const uint4 *src = reinterpret_cast<const uint4 *>(logits);
+  // A thread meets its indices in ascending order, so "strictly better" keeps the first of equal
+  // values and needs no index comparison; selects instead of branches (the branchy form took
+  // 22 us, nearly all of it in the compare chain).
+  float bv = -INFINITY;
+  int bi = tid < pieces ? tid * EPP : (pieces * EPP + tid < n ? pieces * EPP + tid : 0x7fffffff);
+  auto take = [&](float v, int idx) __attribute__((always_inline)) {
+    const bool better = (v > bv) | ((v != v) & (bv == bv));
+    bv = better ? v : bv;
+    bi = better ? idx : bi;
+  };
+  constexpr int U = 16;   // one compute unit hides the memory latency only with many loads in flight
+  for (int p0 = tid; p0 < pieces; p0 += U * 1024) {
+    uint4 pc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) pc[u] = src[p0 + 1024 * u < pieces ? p0 + 1024 * u : p0];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      // a piece past the end is a second copy of the thread's first piece: never strictly better
+      const uint32_t w[4] = {pc[u].x, pc[u].y, pc[u].z, pc[u].w};
+#pragma unroll
+      for (int e = 0; e < EPP; ++e) {
+        float v;
+        if (dtype == RDKV_DTYPE_F32) v = __uint_as_float(w[e]);
+        else {
+          const uint16_t h = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+          v = dtype == RDKV_DTYPE_F16 ? (float)__builtin_bit_cast(_Float16, h) : __uint_as_float((uint32_t)h << 16);
+        }
+        take(v, (p0 + 1024 * u) * EPP + e);
+      }
+    }
+  }
+  for (int i = pieces * EPP + tid; i < n; i += 1024)       // a tail shorter than one piece
+    take(rdkv_load_as_float(logits, dtype, i), i);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, 64);
+    const int oi = __shfl_xor(bi, o, 64);
+    if (best_before(ov, oi, bv, bi)) { bv = ov; bi = oi; }
+  }
+  if ((tid & 63) == 0) { s_v[tid >> 6] = bv; s_i[tid >> 6] = bi; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int w = 1; w < 16; ++w)
+      if (best_before(s_v[w], s_i[w], bv, bi)) { bv = s_v[w]; bi = s_i[w]; }
+    token[0] = bi;
+    if (counter_a) counter_a[0] += 1;
+    if (counter_b) counter_b[0] += 1;
+  }
+  if (tid < n_counts) counts[tid] += 1;
+}
+
 }  // namespace
 
 RDKV_API int rdkv_tail_scores(const float *w, int64_t w_stride_row, int H_kv, int G, int q_block_start,
@@ -216,5 +289,26 @@ RDKV_API int rdkv_silu_mul(const void *gate, const void *up, int64_t n, int dtyp
     hipLaunchKernelGGL(silu_mul_kernel<RDKV_DTYPE_BF16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                        gate, up, n, out);
   RDKV_CHECK_LAUNCH("rdkv_silu_mul");
+  return RDKV_OK;
+}
+
+RDKV_API int rdkv_argmax_advance(const void *logits, int n, int dtype, int64_t *token, int64_t *counter_a,
+                                 int64_t *counter_b, int32_t *counts, int n_counts, void *stream) {
+  const char *fn = "rdkv_argmax_advance";
+  RDKV_REQUIRE(logits && token && n >= 1, "%s: needs logits, a token slot and n >= 1", fn);
+  RDKV_REQUIRE(dtype >= 0 && dtype <= 2, "%s: unknown dtype %d", fn, dtype);
+  RDKV_REQUIRE(((uintptr_t)logits % 16) == 0, "%s: logits must be 16-byte aligned", fn);
+  RDKV_REQUIRE(n_counts >= 0 && n_counts <= 1024 && (n_counts == 0 || counts), "%s: bad counts", fn);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RDKV_DTYPE_F32)
+    hipLaunchKernelGGL(argmax_advance_kernel<RDKV_DTYPE_F32>, dim3(1), dim3(1024), 0, s, logits, n, token,
+                       counter_a, counter_b, counts, n_counts);
+  else if (dtype == RDKV_DTYPE_F16)
+    hipLaunchKernelGGL(argmax_advance_kernel<RDKV_DTYPE_F16>, dim3(1), dim3(1024), 0, s, logits, n, token,
+                       counter_a, counter_b, counts, n_counts);
+  else
+    hipLaunchKernelGGL(argmax_advance_kernel<RDKV_DTYPE_BF16>, dim3(1), dim3(1024), 0, s, logits, n, token,
+                       counter_a, counter_b, counts, n_counts);
+  RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }

@@ -78,6 +78,22 @@ def _rope_append_kv(k_2d: torch.Tensor, v_2d: torch.Tensor, cos_half: torch.Tens
         new_kv_rows.stride(0), new_kv_rows.stride(1), row.data_ptr(), new_kv_rows.shape[1], _lib.stream_of(dev)))
 
 
+def _argmax_advance(logits: torch.Tensor, token: torch.Tensor, position: torch.Tensor, write_row: torch.Tensor,
+                    n_new: torch.Tensor) -> None:
+    """``token <- argmax(logits)`` (fast_decode.py:1827) and ``position``, ``write_row`` (int64, one
+    element each) and every ``n_new`` (int32) advanced by one, in one launch instead of the
+    reduction's two and four elementwise ones."""
+    dev = _lib.require_device(logits, token, position, write_row, n_new)
+    row = logits.reshape(-1)
+    assert row.is_contiguous() and row.dtype in _lib.DTYPE_CODE and row.data_ptr() % 16 == 0
+    assert token.dtype == torch.int64 and position.dtype == torch.int64 and write_row.dtype == torch.int64
+    assert token.numel() == 1 and position.numel() == 1 and write_row.numel() == 1
+    assert n_new.dtype == torch.int32 and n_new.is_contiguous() and n_new.numel() <= 1024
+    _lib.check(_lib.load().rdkv_argmax_advance(row.data_ptr(), row.numel(), _lib.DTYPE_CODE[row.dtype],
+                                               token.data_ptr(), position.data_ptr(), write_row.data_ptr(),
+                                               n_new.data_ptr(), n_new.numel(), _lib.stream_of(dev)))
+
+
 def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``F.linear(x.to(weight.dtype), weight, bias)`` for the single activation row of a decode
     step (fast_decode.py:1650-1656, 1785-1786, 1797-1804, 1826): one pass over the weights with
@@ -435,10 +451,7 @@ class _DecodeStep:
             delta = _silu_linear_row(gate, up, lw.down_proj_weight)
         self.hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
         self.logits = _linear_row(self.hidden, W.lm_head_weight)
-        self.token.copy_(self.logits[:, -1, :].argmax(dim=-1, keepdim=True))
-        self.position.add_(1)
-        self.write_row.add_(1)
-        self.n_new.add_(1)
+        _argmax_advance(self.logits, self.token, self.position, self.write_row, self.n_new)
 
 
 def _layer_stream_caches(dual_cache, num_kv_groups: int) -> List[StreamCache]:

@@ -395,3 +395,31 @@ def test_fused_row_projections_match_their_compositions(dtype):
     nw = torch.ones(16384, device=DEV, dtype=dtype)
     y, h2 = fast_decode._norm_linear_row(h, None, nw, 1e-5, W)
     torch.testing.assert_close(y, fast_decode._linear_row(fast_decode._rms_norm(h, nw, 1e-5), W))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_argmax_and_advance_matches_the_library_argmax(dtype):
+    """`rdkv_argmax_advance`: the index `argmax` returns (first of equal maxima, a NaN before any
+    number) for vocabulary sizes with and without a ragged end, and the step's counters moved on."""
+    g = torch.Generator().manual_seed(11)
+    for n in (128256, 151936, 8193, 1000, 9, 7, 1):
+        x = torch.randn(n, generator=g) * 3
+        cases = [x.clone()]
+        if n > 8:
+            tie = x.clone()
+            tie[[n - 1, n // 2, 5]] = 50.0                      # equal maxima: the lowest index wins
+            nan = x.clone()
+            nan[[n - 2, 3]] = float("nan")                       # a NaN counts as the maximum
+            low = torch.full((n,), -float("inf"))
+            last = x.clone()
+            last[n - 1] = 60.0                                    # the maximum in the ragged end
+            cases += [tie, nan, low, last]
+        for c in cases:
+            logits = c.to(dtype).to(DEV).view(1, 1, n)
+            token = torch.full((1, 1), -1, dtype=torch.long, device=DEV)
+            pos = torch.tensor([[41]], dtype=torch.long, device=DEV)
+            row = torch.tensor([6], dtype=torch.long, device=DEV)
+            counts = torch.tensor([3, 9, 1], dtype=torch.int32, device=DEV)
+            fast_decode._argmax_advance(logits, token, pos, row, counts)
+            assert int(token) == int(torch.argmax(c.to(dtype).float())), (n, dtype)
+            assert int(pos) == 42 and int(row) == 7 and counts.tolist() == [4, 10, 2]
