@@ -114,6 +114,17 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
   const float *base0 = partials + (int64_t)work_begin * pstride;
   if (n <= kMergeMaxK) {
     float *s_m = scratch, *s_l = scratch + kMergeMaxK * 8;
+    // The first kMergeAhead accumulator values of the thread's first column are requested together
+    // with the max / sum columns, before the barrier that publishes those: the usual unit (up to
+    // kMergeAhead partials, one column per thread) then costs one memory round trip, not three.
+    constexpr int kMergeAhead = 32;
+    float ahead[kMergeAhead];
+    {
+      const int i0 = tid < G * kD ? tid : 0;
+      const float *b0 = base0 + (i0 >> 7) * kPartialStride + (i0 & 127);
+#pragma unroll
+      for (int e = 0; e < kMergeAhead; ++e) ahead[e] = *(b0 + (e < n ? e : 0) * pstride);
+    }
     for (int i = tid; i < n * G; i += nthreads) {
       const int k = i / G, h = i - k * G;
       s_m[k * 8 + h] = *(base0 + k * pstride + h * kPartialStride + 128);
@@ -126,7 +137,20 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
       for (int k = 0; k < n; ++k) M = fmaxf(M, s_m[k * 8 + h]);
       float o = 0.0f, l = 0.0f;
       const float *base = base0 + h * kPartialStride + d;
-      for (int k0 = 0; k0 < n; k0 += 16) {
+      int k_from = 0;
+      if (i == tid) {       // the column fetched ahead
+#pragma unroll
+        for (int e = 0; e < kMergeAhead; ++e) {
+          if (e < n) {
+            const float mk = s_m[e * 8 + h];
+            const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
+            o += f * ahead[e];
+            l += f * s_l[e * 8 + h];
+          }
+        }
+        k_from = kMergeAhead;
+      }
+      for (int k0 = k_from; k0 < n; k0 += 16) {
         float v[16];
 #pragma unroll
         for (int e = 0; e < 16; ++e) v[e] = *(base + (k0 + e < n ? k0 + e : k0) * pstride);
