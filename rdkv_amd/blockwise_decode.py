@@ -513,7 +513,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
 
     The reference needs its fixed-slot bank to replay this loop from graphs; that variant is not
     built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
-    from .fast_decode import (_layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
+    from .fast_decode import (_argmax_advance, _layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
                               _silu_linear_row, pre_extract_weights)
     from .stream_cache import decode_attn_fused, extend_stream_caches
     from .triton_rope import fused_rope
@@ -617,7 +617,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
 
     if next_token_logits.dim() == 1:
         next_token_logits = next_token_logits.unsqueeze(0)
-    next_token = next_token_logits.argmax(dim=-1, keepdim=True).to(dev)
+    next_token = next_token_logits.argmax(dim=-1, keepdim=True).to(dev).reshape(1, 1).clone()   # rewritten in place
     position_ids = torch.zeros((1, 1), dtype=torch.long, device=dev)
     record_memory("decode_start")
     t_decode0 = _sync_stamp(dev)
@@ -670,7 +670,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                 delta = _silu_linear_row(gate, up, lw.down_proj_weight)
             hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
             logits = _linear_row(hidden, W.lm_head_weight)
-            next_token = logits[:, -1, :].argmax(dim=-1, keepdim=True)
+            _argmax_advance(logits, next_token)
             pending_len += 1
             ev = torch.cuda.Event(enable_timing=True)
             ev.record()

@@ -78,20 +78,22 @@ def _rope_append_kv(k_2d: torch.Tensor, v_2d: torch.Tensor, cos_half: torch.Tens
         new_kv_rows.stride(0), new_kv_rows.stride(1), row.data_ptr(), new_kv_rows.shape[1], _lib.stream_of(dev)))
 
 
-def _argmax_advance(logits: torch.Tensor, token: torch.Tensor, position: torch.Tensor, write_row: torch.Tensor,
-                    n_new: torch.Tensor) -> None:
-    """``token <- argmax(logits)`` (fast_decode.py:1827) and ``position``, ``write_row`` (int64, one
-    element each) and every ``n_new`` (int32) advanced by one, in one launch instead of the
-    reduction's two and four elementwise ones."""
-    dev = _lib.require_device(logits, token, position, write_row, n_new)
+def _argmax_advance(logits: torch.Tensor, token: torch.Tensor, position: Optional[torch.Tensor] = None,
+                    write_row: Optional[torch.Tensor] = None, n_new: Optional[torch.Tensor] = None) -> None:
+    """``token <- argmax(logits)`` (fast_decode.py:1827) and, where given, ``position``, ``write_row``
+    (int64, one element each) and every ``n_new`` (int32) advanced by one, in one launch instead of
+    the reduction's two and four elementwise ones."""
+    dev = _lib.require_device(logits, token, *(t for t in (position, write_row, n_new) if t is not None))
     row = logits.reshape(-1)
     assert row.is_contiguous() and row.dtype in _lib.DTYPE_CODE and row.data_ptr() % 16 == 0
-    assert token.dtype == torch.int64 and position.dtype == torch.int64 and write_row.dtype == torch.int64
-    assert token.numel() == 1 and position.numel() == 1 and write_row.numel() == 1
-    assert n_new.dtype == torch.int32 and n_new.is_contiguous() and n_new.numel() <= 1024
+    assert token.dtype == torch.int64 and token.numel() == 1
+    for t in (position, write_row):
+        assert t is None or (t.dtype == torch.int64 and t.numel() == 1)
+    assert n_new is None or (n_new.dtype == torch.int32 and n_new.is_contiguous() and n_new.numel() <= 1024)
     _lib.check(_lib.load().rdkv_argmax_advance(row.data_ptr(), row.numel(), _lib.DTYPE_CODE[row.dtype],
-                                               token.data_ptr(), position.data_ptr(), write_row.data_ptr(),
-                                               n_new.data_ptr(), n_new.numel(), _lib.stream_of(dev)))
+                                               token.data_ptr(), _lib.ptr(position), _lib.ptr(write_row),
+                                               _lib.ptr(n_new), 0 if n_new is None else n_new.numel(),
+                                               _lib.stream_of(dev)))
 
 
 def _linear_row(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
