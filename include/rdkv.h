@@ -335,7 +335,11 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
  * in-place rotation would store it, and writes fp32 key and value to token row_dev[0] (device
  * int64; outside 0..capacity-1: nothing is written) of k_new / v_new before it attends over
  * n_new_per_unit[r] tokens (required; they include the new row).  capacity: tokens per row of the
- * zone-C buffers.  Saves the separate rdkv_rope_append_kv launch of a decode step. */
+ * zone-C buffers.  q_rotated_out (NULL, or [rows, 128] of q_dtype, row stride in elements):
+ * receives the query rows as rotated with rope_cos / rope_sin (what the in-place rotation of
+ * triton_rope.py:36-77 leaves in q), for callers that keep the rotated queries
+ * (blockwise_decode.py:2060-2075 pending queries of the channel scores).  Saves the separate
+ * rdkv_rope_append_kv (and rdkv_rope) launches of a decode step. */
 int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, int n_work, int G,
                                           const void *q, int q_dtype, int64_t q_stride_row,
                                           const void *rope_cos, const void *rope_sin, int rope_dtype,
@@ -347,6 +351,7 @@ int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, in
                                           const int64_t *row_dev,
                                           float *out, int64_t out_stride_row, float *lse,
                                           float *zone_c_weights, int64_t zone_c_weights_stride_row,
+                                          void *q_rotated_out, int64_t q_rotated_stride_row,
                                           void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Planning for rdkv_pack_layer_per_head on the device (what the reference derives on the host:

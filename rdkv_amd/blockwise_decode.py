@@ -516,7 +516,6 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     from .fast_decode import (_argmax_advance, _layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
                               _silu_linear_row, pre_extract_weights)
     from .stream_cache import decode_attn_fused, extend_stream_caches
-    from .triton_rope import fused_rope
 
     config.validate()
     lib = _lib.load()
@@ -650,13 +649,12 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                     q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
                 if lw.k_norm_weight is not None:
                     k_2d = _rms_norm(k_2d, lw.k_norm_weight, lw.qk_norm_eps)
-                q_2d, k_2d = q_2d.contiguous(), k_2d.contiguous()
-                fused_rope(q_2d, k_2d, cos_half, sin_half)          # the rotated query is kept for the channel scores
-                pending_q[layer][:, write_pos, :].copy_(q_2d)
                 rows = pending_kv[layer][0]
-                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse,       # k is rotated already: appended as it is
+                # q and k are rotated inside the attention launches; the merge launch appends k | v to
+                # the raw tail and leaves the rotated query (kept for the channel scores) in pending_q
+                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse, rope=(cos_half, sin_half),
                                   zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights,
-                                  append=(k_2d, v_2d, write_row))
+                                  append=(k_2d, v_2d, write_row), q_rotated_out=pending_q[layer][:, write_pos, :])
                 # block scores from the tail's weights (blockwise_decode.py:2085-2109), one launch
                 _lib.check(lib.rdkv_tail_scores(
                     tail_weights.data_ptr(), tail_weights.stride(0), h_kv, groups, q_block_start, current_len, block,

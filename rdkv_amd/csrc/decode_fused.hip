@@ -809,7 +809,8 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
                     float *k_new, float *v_new, int64_t new_stride_unit,   // written when a row is appended
                     int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
                     float *__restrict__ out, int64_t out_stride, float *__restrict__ lse,
-                    float *zc_w, int64_t zc_w_stride, ZcAppend ap) {
+                    float *zc_w, int64_t zc_w_stride, ZcAppend ap, void *__restrict__ q_rot_out,
+                    int64_t q_rot_stride) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
   __shared__ float fin_m[8], fin_l[8];             // softmax maximum and sum over the union, per head
   __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
@@ -879,6 +880,8 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
         v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
       }
       qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
+      // the rotated query as the in-place rotation would have left it, for callers that keep it
+      if (q_rot_out) rdkv_store_from_float(q_rot_out, q_dtype, (int64_t)(q_row + (i >> 7)) * q_rot_stride + c, v);
     }
   }
   __syncthreads();
@@ -1127,7 +1130,7 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
                                int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit, float *out,
                                int64_t out_stride_row, float *lse, float *zone_c_weights,
                                int64_t zone_c_weights_stride_row, void *workspace, int64_t workspace_bytes,
-                               const ZcAppend &append, void *stream) {
+                               const ZcAppend &append, void *q_rot_out, int64_t q_rot_stride, void *stream) {
   RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= n_new || n_new_per_unit,
                "%s: rows of the zone-C weights are shorter than n_new", fn);
   int rc = check_fused_args(fn, units, n_units, (const RdkvWork *)units, n_work, G, workspace, workspace_bytes);
@@ -1145,7 +1148,7 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
   hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
                      (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,        \
                      const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
-                     zone_c_weights, zone_c_weights_stride_row, append)
+                     zone_c_weights, zone_c_weights_stride_row, append, q_rot_out, q_rot_stride)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;
     case 2: RDKV_LAUNCH_ZC(2); break;
@@ -1173,7 +1176,7 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
   return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, n_units, n_work, G, q, q_dtype, q_stride_row,
                              rope_cos, rope_sin, rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, n_new,
                              n_new_per_unit, out, out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row,
-                             workspace, workspace_bytes, none, stream);
+                             workspace, workspace_bytes, none, nullptr, 0, stream);
 }
 
 RDKV_API int rdkv_decode_fused_merge_zone_c_append(
@@ -1181,9 +1184,10 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
     const void *rope_cos, const void *rope_sin, int rope_dtype, float *k_new, float *v_new, int64_t new_stride_unit,
     int64_t new_stride_tok, int64_t capacity, const int32_t *n_new_per_unit, const void *k_step, int64_t k_stride_h,
     const void *v_step, int64_t v_stride_h, int kv_dtype, const int64_t *row_dev, float *out, int64_t out_stride_row,
-    float *lse, float *zone_c_weights, int64_t zone_c_weights_stride_row, void *workspace, int64_t workspace_bytes,
-    void *stream) {
+    float *lse, float *zone_c_weights, int64_t zone_c_weights_stride_row, void *q_rotated_out,
+    int64_t q_rotated_stride_row, void *workspace, int64_t workspace_bytes, void *stream) {
   const char *fn = "rdkv_decode_fused_merge_zone_c_append";
+  RDKV_REQUIRE(!q_rotated_out || q_rotated_stride_row >= 128, "%s: rows of the rotated query are shorter than 128", fn);
   RDKV_REQUIRE(k_step && v_step && row_dev && n_new_per_unit && k_new && v_new, "%s: null pointer", fn);
   RDKV_REQUIRE(kv_dtype >= 0 && kv_dtype <= 2, "%s: unknown k/v dtype %d", fn, kv_dtype);
   RDKV_REQUIRE(capacity >= 0 && capacity <= 0x7fffffffLL, "%s: bad zone-C capacity", fn);
@@ -1193,5 +1197,5 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
   return launch_merge_zone_c(fn, units, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,
                              k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
                              out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row, workspace,
-                             workspace_bytes, ap, stream);
+                             workspace_bytes, ap, q_rotated_out, q_rotated_stride_row, stream);
 }

@@ -427,7 +427,8 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                       rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
                       zone_c: Optional[Tuple[torch.Tensor, ...]] = None,
                       zone_c_weights: Optional[torch.Tensor] = None,
-                      append: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None):
+                      append: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
+                      q_rotated_out: Optional[torch.Tensor] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
@@ -440,7 +441,9 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     (k, v, row) with ``zone_c`` = (K_buf, V_buf, counts): the step's own un-rotated key and value
     rows [rows / G, 128] (q's type) are rotated with ``rope`` (taken as they are without it),
     widened to fp32 and stored as row ``row[0]`` (device int64) of the zone C buffers by the merge
-    launch itself, before it attends over ``counts`` tokens (which include that row).  Graph-capturable
+    launch itself, before it attends over ``counts`` tokens (which include that row);
+    ``q_rotated_out`` ([rows, 128] of q's type, unit stride in the last dimension, with ``append``)
+    then receives the rotated query rows.  Graph-capturable
     once the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
@@ -499,6 +502,9 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
             assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2
             assert zone_c_weights.stride(1) == 1 and zone_c_weights.shape[0] == cache.rows
             assert zone_c_weights.shape[1] >= n_new, f"zone_c_weights rows must hold {n_new} tokens"
+        if q_rotated_out is not None:
+            _lib.require_device(q_rotated_out)
+            assert q_rotated_out.shape == q.shape and q_rotated_out.dtype == q.dtype and q_rotated_out.stride(1) == 1
         _lib.check(lib.rdkv_decode_fused_merge_zone_c_append(
             cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
@@ -506,8 +512,10 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
             counts.data_ptr(), k_step.data_ptr(), k_step.stride(0), v_step.data_ptr(), v_step.stride(0),
             _lib.DTYPE_CODE[k_step.dtype], row.data_ptr(), out.data_ptr(), out.stride(0), lse.data_ptr(),
             _lib.ptr(zone_c_weights), zone_c_weights.stride(0) if zone_c_weights is not None else 0,
+            _lib.ptr(q_rotated_out), q_rotated_out.stride(0) if q_rotated_out is not None else 0,
             ws.data_ptr(), ws.numel(), stream))
         return out, lse
+    assert q_rotated_out is None, "q_rotated_out needs append"
     if zone_c_weights is not None:
         _lib.require_device(zone_c_weights)
         assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2 and zone_c_weights.stride(1) == 1

@@ -393,8 +393,9 @@ def test_append_inside_the_merge_launch_equals_the_separate_append(dtype, with_r
     """``append``: the merge launch rotates the step's key, stores the fp32 K|V row in zone C and
     attends over it - the same buffer bits and the same result bits as ``rdkv_rope_append_kv``
     followed by the plain zone C call, over several steps, with the appended row the only token,
-    in the middle and last in the buffer, and a row index outside the buffer writing nothing."""
-    from rdkv_amd import fast_decode
+    in the middle and last in the buffer, and a row index outside the buffer writing nothing.
+    ``q_rotated_out`` receives the query exactly as ``fused_rope`` rotates it in place."""
+    from rdkv_amd import fast_decode, triton_rope
     cfg = synth.scaled(synth.CONFIGS[1], context=600, layers=1)
     packed, q1, _ = _config_case(cfg, 1)
     cache = stream_cache.build_stream_cache(packed, cfg.G)
@@ -421,8 +422,13 @@ def test_append_inside_the_merge_launch_equals_the_separate_append(dtype, with_r
         fast_decode._rope_append_kv(k, v, *(rope or ident), buf_a, row)
         exp = stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_a[:, :, :128], buf_a[:, :, 128:], counts))
         w = torch.zeros(cache.rows, cap, device=DEV)
+        q_keep = torch.zeros(cache.rows, 3, 128, dtype=dtype, device=DEV)       # rows of a larger tensor
         got = stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_b[:, :, :128], buf_b[:, :, 128:], counts),
-                                             append=(k, v, row), zone_c_weights=w)
+                                             append=(k, v, row), zone_c_weights=w, q_rotated_out=q_keep[:, 1, :])
+        q_exp, k_unused = q.clone(), k.contiguous().clone()
+        if with_rope:
+            triton_rope.fused_rope(q_exp, k_unused, *rope)
+        assert torch.equal(q_keep[:, 1, :], q_exp) and float(q_keep[:, 0].abs().max() + q_keep[:, 2].abs().max()) == 0.0
         assert torch.equal(buf_a, buf_b), f"step {step}: zone C rows differ"
         assert torch.equal(exp[0], got[0]) and torch.equal(exp[1], got[1]), f"step {step}: attention differs"
         assert float(w[:, :step + 1].sum(1).min()) > 0.0
