@@ -338,8 +338,20 @@ int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_wor
  * zone-C buffers.  q_rotated_out (NULL, or [rows, 128] of q_dtype, row stride in elements):
  * receives the query rows as rotated with rope_cos / rope_sin (what the in-place rotation of
  * triton_rope.py:36-77 leaves in q), for callers that keep the rotated queries
- * (blockwise_decode.py:2060-2075 pending queries of the channel scores).  Saves the separate
+ * (blockwise_decode.py:2060-2075 pending queries of the channel scores).  tail_scores (host
+ * pointer, NULL = none; needs zone_c_weights): what rdkv_tail_scores does with those weights, in
+ * the same launch (the same sums, head by head) - per KV head r and zone-C token t the weights
+ * summed over the G query heads are added to self_scores[r][t] for t >= q_block_start and, when
+ * q_block_start >= block, to next_scores[r][t] for t < block.  Saves the separate
  * rdkv_rope_append_kv (and rdkv_rope) launches of a decode step. */
+typedef struct RdkvTailScores {   /* online block scores of blockwise decode, see below */
+  float  *self_scores;            /* fp32 [rows / G, >= tokens], row stride self_stride_h (elements) */
+  int64_t self_stride_h;
+  float  *next_scores;            /* likewise; may be NULL while q_block_start < block */
+  int64_t next_stride_h;
+  int32_t q_block_start;          /* first zone-C token of the block the step's query belongs to */
+  int32_t block;                  /* block size in tokens */
+} RdkvTailScores;
 int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, int n_work, int G,
                                           const void *q, int q_dtype, int64_t q_stride_row,
                                           const void *rope_cos, const void *rope_sin, int rope_dtype,
@@ -352,6 +364,7 @@ int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, in
                                           float *out, int64_t out_stride_row, float *lse,
                                           float *zone_c_weights, int64_t zone_c_weights_stride_row,
                                           void *q_rotated_out, int64_t q_rotated_stride_row,
+                                          const RdkvTailScores *tail_scores,
                                           void *workspace, int64_t workspace_bytes, void *stream);
 
 /* Planning for rdkv_pack_layer_per_head on the device (what the reference derives on the host:

@@ -14,6 +14,12 @@ from typing import Optional
 
 import torch
 
+
+class RdkvTailScores(ctypes.Structure):
+    """``RdkvTailScores`` of include/rdkv.h (read by the library during the call)."""
+    _fields_ = [("self_scores", c_void_p), ("self_stride_h", c_int64), ("next_scores", c_void_p),
+                ("next_stride_h", c_int64), ("q_block_start", ctypes.c_int32), ("block", ctypes.c_int32)]
+
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "librdkv_hip.so")
 
@@ -56,7 +62,7 @@ SIGNATURES = {
     "rdkv_decode_fused_partials": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P]),
     "rdkv_decode_fused_merge_zone_c": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, I, P, P, L, P, P, L, P, L, P]),
     "rdkv_decode_fused_merge_zone_c_append": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, L, P, P, L, P, L, I, P,
-                                                  P, L, P, P, L, P, L, P, L, P]),
+                                                  P, L, P, P, L, P, L, P, P, L, P]),
     "rdkv_rope": (I, [P, L, I, P, L, I, I, I, P, P, I, P]),
     "rdkv_add_rms_norm": (I, [P, L, P, L, P, I, F, I, I, I, P, L, P, L, P]),
     "rdkv_rope_append_kv": (I, [P, L, P, L, I, I, I, P, P, I, P, L, L, P, L, P]),

@@ -8,7 +8,8 @@ accounting, and the fixed-slot re-shaping the reference uses to keep tensor shap
 model loop around it is ``greedy_decode_blockwise`` at the end of this module: the attention over
 [prompt cache | compressed blocks | raw tail] is ``stream_cache.extend_stream_cache`` (a block
 becomes a further source of its layer's cache) + ``decode_attn_fused(..., zone_c=...,
-zone_c_weights=...)`` (the tail's softmax weights feed the online block scores).
+zone_c_weights=..., append=..., q_rotated_out=..., tail_scores=...)`` (the merge launch appends the
+step's K/V row, keeps the rotated query and adds the tail's softmax weights to the online block scores).
 """
 from __future__ import annotations
 
@@ -654,12 +655,9 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
                 # the raw tail and leaves the rotated query (kept for the channel scores) in pending_q
                 decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse, rope=(cos_half, sin_half),
                                   zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights,
-                                  append=(k_2d, v_2d, write_row), q_rotated_out=pending_q[layer][:, write_pos, :])
-                # block scores from the tail's weights (blockwise_decode.py:2085-2109), one launch
-                _lib.check(lib.rdkv_tail_scores(
-                    tail_weights.data_ptr(), tail_weights.stride(0), h_kv, groups, q_block_start, current_len, block,
-                    self_scores[layer].data_ptr(), self_scores[layer].stride(0), next_scores[layer].data_ptr(),
-                    next_scores[layer].stride(0), _lib.stream_of(dev)))
+                                  append=(k_2d, v_2d, write_row), q_rotated_out=pending_q[layer][:, write_pos, :],
+                                  # block scores from the tail's weights (blockwise_decode.py:2085-2109)
+                                  tail_scores=(self_scores[layer], next_scores[layer], q_block_start, block))
                 if config.correctness_check and not torch.isfinite(attn_out).all():
                     raise FloatingPointError(f"non-finite attention output at layer {layer}")
                 o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)

@@ -810,7 +810,7 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
                     int64_t new_stride_tok, int n_new_all, const int32_t *__restrict__ n_new_per_unit,
                     float *__restrict__ out, int64_t out_stride, float *__restrict__ lse,
                     float *zc_w, int64_t zc_w_stride, ZcAppend ap, void *__restrict__ q_rot_out,
-                    int64_t q_rot_stride) {
+                    int64_t q_rot_stride, RdkvTailScores ts) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
   __shared__ float fin_m[8], fin_l[8];             // softmax maximum and sum over the union, per head
   __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
@@ -995,11 +995,21 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   }
   if (zc_w) {   // softmax weights of the zone C tokens over the union (fast_decode.py:1753-1755 w_new)
     __syncthreads();
+    for (int t = tid; t < n_new; t += kThreads) {
+      float s = 0.0f;     // over the group's heads in head order, as rdkv_tail_scores sums them
 #pragma unroll
-    for (int h = 0; h < G; ++h) {
-      float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
-      const float M = fin_m[h], inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
-      for (int t = tid; t < n_new; t += kThreads) row[t] = expf(row[t] - M) * inv;
+      for (int h = 0; h < G; ++h) {
+        float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
+        const float inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
+        const float w = expf(row[t] - fin_m[h]) * inv;
+        row[t] = w;
+        s = __fadd_rn(s, w);   // the stored weight is what is summed: no fusing with the product above
+      }
+      // online block scores of blockwise decode (blockwise_decode.py:2085-2109): the query's weights
+      // on its own block, and on the first block when the query belongs to the second
+      if (ts.self_scores && t >= ts.q_block_start) ts.self_scores[(int64_t)kv_row * ts.self_stride_h + t] += s;
+      if (ts.next_scores && ts.q_block_start >= ts.block && t < ts.block)
+        ts.next_scores[(int64_t)kv_row * ts.next_stride_h + t] += s;
     }
   }
 }
@@ -1130,7 +1140,8 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
                                int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit, float *out,
                                int64_t out_stride_row, float *lse, float *zone_c_weights,
                                int64_t zone_c_weights_stride_row, void *workspace, int64_t workspace_bytes,
-                               const ZcAppend &append, void *q_rot_out, int64_t q_rot_stride, void *stream) {
+                               const ZcAppend &append, void *q_rot_out, int64_t q_rot_stride,
+                               const RdkvTailScores &tail, void *stream) {
   RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= n_new || n_new_per_unit,
                "%s: rows of the zone-C weights are shorter than n_new", fn);
   int rc = check_fused_args(fn, units, n_units, (const RdkvWork *)units, n_work, G, workspace, workspace_bytes);
@@ -1148,7 +1159,7 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
   hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
                      (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,        \
                      const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
-                     zone_c_weights, zone_c_weights_stride_row, append, q_rot_out, q_rot_stride)
+                     zone_c_weights, zone_c_weights_stride_row, append, q_rot_out, q_rot_stride, tail)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;
     case 2: RDKV_LAUNCH_ZC(2); break;
@@ -1176,7 +1187,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
   return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, n_units, n_work, G, q, q_dtype, q_stride_row,
                              rope_cos, rope_sin, rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, n_new,
                              n_new_per_unit, out, out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row,
-                             workspace, workspace_bytes, none, nullptr, 0, stream);
+                             workspace, workspace_bytes, none, nullptr, 0, RdkvTailScores{nullptr, 0, nullptr, 0, 0, 0},
+                             stream);
 }
 
 RDKV_API int rdkv_decode_fused_merge_zone_c_append(
@@ -1185,7 +1197,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
     int64_t new_stride_tok, int64_t capacity, const int32_t *n_new_per_unit, const void *k_step, int64_t k_stride_h,
     const void *v_step, int64_t v_stride_h, int kv_dtype, const int64_t *row_dev, float *out, int64_t out_stride_row,
     float *lse, float *zone_c_weights, int64_t zone_c_weights_stride_row, void *q_rotated_out,
-    int64_t q_rotated_stride_row, void *workspace, int64_t workspace_bytes, void *stream) {
+    int64_t q_rotated_stride_row, const RdkvTailScores *tail_scores, void *workspace, int64_t workspace_bytes,
+    void *stream) {
   const char *fn = "rdkv_decode_fused_merge_zone_c_append";
   RDKV_REQUIRE(!q_rotated_out || q_rotated_stride_row >= 128, "%s: rows of the rotated query are shorter than 128", fn);
   RDKV_REQUIRE(k_step && v_step && row_dev && n_new_per_unit && k_new && v_new, "%s: null pointer", fn);
@@ -1193,9 +1206,17 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
   RDKV_REQUIRE(capacity >= 0 && capacity <= 0x7fffffffLL, "%s: bad zone-C capacity", fn);
   RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= capacity,
                "%s: rows of the zone-C weights are shorter than the buffer", fn);
+  RdkvTailScores tail = {nullptr, 0, nullptr, 0, 0, 0};
+  if (tail_scores) {
+    tail = *tail_scores;
+    RDKV_REQUIRE(zone_c_weights, "%s: the block scores are summed from zone_c_weights", fn);
+    RDKV_REQUIRE(tail.self_scores && tail.q_block_start >= 0 && tail.block >= 1 &&
+                     (tail.next_scores || tail.q_block_start < tail.block),
+                 "%s: bad tail score arguments", fn);
+  }
   const ZcAppend ap = {k_step, v_step, k_stride_h, v_stride_h, row_dev, capacity, kv_dtype};
   return launch_merge_zone_c(fn, units, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,
                              k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
                              out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row, workspace,
-                             workspace_bytes, ap, q_rotated_out, q_rotated_stride_row, stream);
+                             workspace_bytes, ap, q_rotated_out, q_rotated_stride_row, tail, stream);
 }

@@ -15,6 +15,7 @@ packed tensors in place keep using the padded-layout entry points.
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
@@ -428,7 +429,8 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                       zone_c: Optional[Tuple[torch.Tensor, ...]] = None,
                       zone_c_weights: Optional[torch.Tensor] = None,
                       append: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
-                      q_rotated_out: Optional[torch.Tensor] = None):
+                      q_rotated_out: Optional[torch.Tensor] = None,
+                      tail_scores: Optional[Tuple[torch.Tensor, Optional[torch.Tensor], int, int]] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
@@ -443,7 +445,11 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     widened to fp32 and stored as row ``row[0]`` (device int64) of the zone C buffers by the merge
     launch itself, before it attends over ``counts`` tokens (which include that row);
     ``q_rotated_out`` ([rows, 128] of q's type, unit stride in the last dimension, with ``append``)
-    then receives the rotated query rows.  Graph-capturable
+    then receives the rotated query rows.  ``tail_scores`` = (self_scores, next_scores,
+    q_block_start, block) (with ``append`` and ``zone_c_weights``; fp32 [rows / G, >= tokens]):
+    the merge launch also adds the new tokens' weights, summed over a KV head's query heads, to
+    ``self_scores[:, q_block_start:]`` and, when ``q_block_start >= block``, to
+    ``next_scores[:, :block]`` - what ``rdkv_tail_scores`` does as a launch of its own.  Graph-capturable
     once the workspace exists (first call): one streaming launch plus one small merge launch."""
     lib = _lib.load()
     dev = _lib.require_device(q)
@@ -505,6 +511,18 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         if q_rotated_out is not None:
             _lib.require_device(q_rotated_out)
             assert q_rotated_out.shape == q.shape and q_rotated_out.dtype == q.dtype and q_rotated_out.stride(1) == 1
+        tail = None
+        if tail_scores is not None:
+            self_s, next_s, q_block_start, block = tail_scores
+            assert zone_c_weights is not None, "tail_scores are summed from zone_c_weights"
+            for t, width in ((self_s, n_new), (next_s, block)):
+                if t is not None:
+                    _lib.require_device(t)
+                    assert t.dtype == torch.float32 and t.dim() == 2 and t.shape[0] == n_kv_rows and t.stride(1) == 1
+                    assert t.shape[1] >= width, f"score rows must hold {width} tokens"
+            assert next_s is not None or q_block_start < block
+            tail = _lib.RdkvTailScores(self_s.data_ptr(), self_s.stride(0), _lib.ptr(next_s),
+                                       next_s.stride(0) if next_s is not None else 0, int(q_block_start), int(block))
         _lib.check(lib.rdkv_decode_fused_merge_zone_c_append(
             cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
@@ -513,9 +531,10 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
             _lib.DTYPE_CODE[k_step.dtype], row.data_ptr(), out.data_ptr(), out.stride(0), lse.data_ptr(),
             _lib.ptr(zone_c_weights), zone_c_weights.stride(0) if zone_c_weights is not None else 0,
             _lib.ptr(q_rotated_out), q_rotated_out.stride(0) if q_rotated_out is not None else 0,
+            ctypes.addressof(tail) if tail is not None else None,
             ws.data_ptr(), ws.numel(), stream))
         return out, lse
-    assert q_rotated_out is None, "q_rotated_out needs append"
+    assert q_rotated_out is None and tail_scores is None, "q_rotated_out / tail_scores need append"
     if zone_c_weights is not None:
         _lib.require_device(zone_c_weights)
         assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2 and zone_c_weights.stride(1) == 1

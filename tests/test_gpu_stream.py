@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import rdkv_oracle as O
-from rdkv_amd import packing, stream_cache, synth
+from rdkv_amd import _lib, packing, stream_cache, synth
 from tests.gpu_util import (DEV, attn_close, layer_to_device, require_gpu, t2n, to_dev)
 from tests.helpers import golden_to_oracle_layer, load_golden
 from tests.stream_decode import decode_unit
@@ -429,6 +429,23 @@ def test_append_inside_the_merge_launch_equals_the_separate_append(dtype, with_r
         if with_rope:
             triton_rope.fused_rope(q_exp, k_unused, *rope)
         assert torch.equal(q_keep[:, 1, :], q_exp) and float(q_keep[:, 0].abs().max() + q_keep[:, 2].abs().max()) == 0.0
+        # the block scores summed inside the merge launch == rdkv_tail_scores on the same weights
+        block = 32
+        qbs = (step // block) * block
+        self_a, next_a = torch.rand(rows_kv, cap, generator=g).to(DEV), torch.rand(rows_kv, block, generator=g).to(DEV)
+        self_b, next_b = self_a.clone(), next_a.clone()
+        w2 = torch.zeros(cache.rows, cap, device=DEV)
+        stream_cache.decode_attn_fused(cache, q, rope=rope, zone_c=(buf_b[:, :, :128], buf_b[:, :, 128:], counts),
+                                       append=(k, v, row), zone_c_weights=w2, tail_scores=(self_b, next_b, qbs, block))
+        lib = _lib.load()
+        _lib.check(lib.rdkv_tail_scores(w.data_ptr(), w.stride(0), rows_kv, cfg.G, qbs, step + 1, block,
+                                        self_a.data_ptr(), self_a.stride(0), next_a.data_ptr(), next_a.stride(0),
+                                        _lib.stream_of(DEV)))
+        assert torch.equal(w, w2), f"step {step}"
+        torch.testing.assert_close(self_b, self_a, rtol=1e-6, atol=1e-8)       # the same sums, to the last rounding
+        torch.testing.assert_close(next_b, next_a, rtol=1e-6, atol=1e-8)
+        if qbs >= block:
+            assert float((next_b - next_a).abs().max()) < 1e-6 and not torch.equal(next_b, torch.zeros_like(next_b))
         assert torch.equal(buf_a, buf_b), f"step {step}: zone C rows differ"
         assert torch.equal(exp[0], got[0]) and torch.equal(exp[1], got[1]), f"step {step}: attention differs"
         assert float(w[:, :step + 1].sum(1).min()) > 0.0
