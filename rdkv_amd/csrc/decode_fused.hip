@@ -1158,7 +1158,8 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
 #define RDKV_LAUNCH_ZC(GT)                                                                                    \
   hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
                      (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,        \
-                     const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse,        \
+                     const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok,   \
+                     n_new, n_new_per_unit, out, out_stride_row, lse,                                           \
                      zone_c_weights, zone_c_weights_stride_row, append, q_rot_out, q_rot_stride, tail)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;

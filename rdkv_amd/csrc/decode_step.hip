@@ -122,9 +122,10 @@ tail_scores_kernel(const float *__restrict__ w, int64_t w_stride, int G, int q_b
 
 // Greedy choice of the next token (fast_decode.py:1827 argmax of the step's logits) and the advance
 // of the step's device-held state, one workgroup: a thread scans pieces of 16 bytes, 1024 pieces
-// apart, sixteen loads in flight (a 128k vocabulary in fp16 is one batch); ties go to the lowest index and a NaN counts as the largest value
-// (the library's argmax).  counters: int64 values incremented by one (position, zone C write
-// row), counts: n_counts int32 values incremented by one (zone C lengths).
+// apart, sixteen loads in flight (a 128k vocabulary in fp16 is one batch); ties go to the lowest
+// index and a NaN counts as the largest value (the library's argmax).  counters: int64 values
+// incremented by one (position, zone C write row), counts: n_counts int32 values incremented by
+// one (zone C lengths).
 struct Best { float v; int i; };
 __device__ __forceinline__ bool best_before(float a, int ia, float b, int ib) {
   const bool na = a != a, nb = b != b;
