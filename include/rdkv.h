@@ -308,6 +308,22 @@ int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int 
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);
 
+/* rdkv_decode_fused for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and same results, bit for bit, as rdkv_decode_fused without the
+ * workspace: the partials live in a fixed array of rdkv_decode_fused_static_max_bytes() = 8 MiB
+ * that every GPU the library runs on holds until the process ends; the call allocates and frees
+ * nothing.  n_work * G * 528 bytes must fit (15887 work-item heads: a whole 32-layer step of a
+ * 32k-token cache needs 1.1 MB), else RDKV_EWORKSPACE.  All calls on one GPU share that array:
+ * calls that overlap on one GPU (two streams, two threads) race.  The array's address is looked
+ * up on the first call on each device; make that call outside graph capture. */
+int64_t rdkv_decode_fused_static_max_bytes(void);
+int rdkv_decode_fused_static(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                             const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                             int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
+                             const void *rope_cos, const void *rope_sin, int rope_dtype,
+                             float *out, int64_t out_stride_row, float *lse, void *stream);
+
 /* rdkv_decode_fused_merge plus the attention over the decode-appended tokens of every unit
  * (zone C; fast_decode.py:1719-1735 scores of the new tokens, :1743-1755 softmax over
  * [old | new], :1777-1784 their V sum): the exact softmax over zones A+B+C, out and lse of the

@@ -26,6 +26,8 @@
 
 #include <stdlib.h>
 
+#include <mutex>
+
 namespace {
 
 typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
@@ -1220,4 +1222,67 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
                              k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
                              out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row, workspace,
                              workspace_bytes, ap, q_rotated_out, q_rotated_stride_row, tail, stream);
+}
+
+// ---- rdkv_decode_fused for callers that cannot allocate ---------------------------------------
+// The partials of rdkv_decode_fused live in a fixed array in device memory instead of a workspace
+// the caller brings.  Each GPU the library runs on holds its own copy of the array (at its own
+// address) until the process ends.  In host code the array's name only identifies the symbol: the
+// device address is looked up once per device and that pointer is what the kernels receive.
+#define RDKV_STATIC_SCRATCH_BYTES (8 << 20)
+static __device__ __align__(256) unsigned char scratch[RDKV_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_scratch_ptr[kMaxDevices];            // device address of `scratch`, per device ordinal
+std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of `scratch` (looked up on the first call on that device).
+int static_scratch(const char *fn, void **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    rdkv_set_error("%s: hipGetDevice: %s", fn, hipGetErrorString(e));
+    return RDKV_ELAUNCH;
+  }
+  RDKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device ordinal %d outside 0..%d", fn, dev, kMaxDevices - 1);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      rdkv_set_error("%s: hipGetSymbolAddress(scratch) on device %d: %s", fn, dev, hipGetErrorString(e));
+      return RDKV_ELAUNCH;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return RDKV_OK;
+}
+}  // namespace
+
+RDKV_API int64_t rdkv_decode_fused_static_max_bytes(void) { return RDKV_STATIC_SCRATCH_BYTES; }
+
+RDKV_API int rdkv_decode_fused_static(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                                      const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                                      int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row,
+                                      int G, const void *rope_cos, const void *rope_sin, int rope_dtype,
+                                      float *out, int64_t out_stride_row, float *lse, void *stream) {
+  const char *fn = "rdkv_decode_fused_static";
+  RDKV_REQUIRE(n_work >= 0 && G >= 1 && G <= 8, "%s: bad n_work=%d or G=%d", fn, n_work, G);
+  const int64_t need = rdkv_decode_fused_workspace_bytes(n_work, G);
+  if (need > RDKV_STATIC_SCRATCH_BYTES) {
+    rdkv_set_error("%s: %d work items x %d heads need %lld bytes of partials, the fixed buffer holds %d "
+                   "(use rdkv_decode_fused with a workspace)", fn, n_work, G, (long long)need,
+                   RDKV_STATIC_SCRATCH_BYTES);
+    return RDKV_EWORKSPACE;
+  }
+  void *ptr = nullptr;
+  const int rc = static_scratch(fn, &ptr);
+  if (rc != RDKV_OK) return rc;
+  // every partial a merge reads is written in full by the streaming launch of the same call, so
+  // nothing in the buffer has to start at zero
+  return rdkv_decode_fused(blob, units, n_units, work, n_work, groups, n_groups, max_row_dwords, q, q_dtype,
+                           q_stride_row, G, rope_cos, rope_sin, rope_dtype, out, out_stride_row, lse, ptr,
+                           RDKV_STATIC_SCRATCH_BYTES, stream);
 }
