@@ -69,3 +69,28 @@ def attn_close(got, exp, what=""):
     assert err <= 2e-3, f"{what}: max-abs error {err:.3e} > 2e-3"
     assert err <= 1e-2 * max(ref, 1e-30), f"{what}: relative error {err / ref:.3e} > 1e-2"
     return err
+
+
+def layer_to_oracle(pl):
+    """rdkv_amd PackedKVLayer (device tensors) -> oracle PackedKVLayer over the same bytes."""
+    import dataclasses
+    kw = {}
+    for f in dataclasses.fields(O.PackedKVLayer):
+        v = getattr(pl, f.name)
+        kw[f.name] = t2n(v) if torch.is_tensor(v) else v
+    return O.PackedKVLayer(**kw)
+
+
+def lse_merge(parts):
+    """Exact softmax over the union of several token sets from their (out [R,D], lse [R]) pairs,
+    in float64: out = sum_i exp(lse_i - L) * out_i with L = log sum_i exp(lse_i).  A source
+    without tokens has lse = -inf and weight 0."""
+    outs = [np.asarray(o, np.float64) for o, _ in parts]
+    lses = [np.asarray(l, np.float64) for _, l in parts]
+    m = np.max(np.stack(lses), axis=0)
+    ws = [np.where(np.isneginf(l), 0.0, np.exp(l - np.where(np.isneginf(m), 0.0, m))) for l in lses]
+    tot = np.sum(ws, axis=0)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        out = np.where(tot[:, None] > 0, sum(w[:, None] * o for w, o in zip(ws, outs)) / tot[:, None], 0.0)
+        lse = np.where(tot > 0, m + np.log(tot), -np.inf)
+    return out, lse

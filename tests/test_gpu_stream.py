@@ -6,7 +6,8 @@ import torch
 
 from oracle import rdkv_oracle as O
 from rdkv_amd import _lib, packing, stream_cache, synth
-from tests.gpu_util import (DEV, attn_close, layer_to_device, require_gpu, t2n, to_dev)
+from tests.gpu_util import (DEV, attn_close, layer_to_device, layer_to_oracle, lse_merge, require_gpu, t2n,
+                            to_dev)
 from tests.helpers import golden_to_oracle_layer, load_golden
 from tests.stream_decode import decode_unit
 
@@ -207,9 +208,19 @@ def test_fused_empty_unit_and_lse_merge():
     m = torch.maximum(la, lb)[:2]
     wa, wb = torch.exp(la[:2] - m), torch.exp(lb[:2] - m)
     merged = (oa[:2] * wa[:, None] + ob[:2] * wb[:, None]) / (wa + wb)[:, None]
-    # K is re-quantized per source (per-channel ranges differ), so compare loosely to the
-    # single-source result and tightly to the two-source oracle
+    # K is re-quantized per source (per-channel ranges differ), so the single-source result is
+    # only loosely the same; the two-source oracle (dequantize-then-attend per source, exact
+    # merge of the two softmaxes) is the reference
     assert float((merged - out[:2]).abs().max()) < 5e-2
+    ora_parts = []
+    for v in (vb_a, vb_b):
+        ora, ora_nvo = O.pack_layer_per_head(t2n(K), t2n(V), v.numpy(), kb.numpy(), 2)
+        eo, el, _ = O.decode_attn_ref(t2n(q), ora, ora_nvo)
+        ora_parts.append((eo, el))
+    exp_out, exp_lse = lse_merge(ora_parts)
+    attn_close(t2n(merged), exp_out[:2], "two-source merge")
+    lm = m + torch.log(wa + wb)
+    attn_close(t2n(lm), exp_lse[:2], "two-source lse")
 
 
 def test_fused_attention_under_graph_replay():
@@ -242,11 +253,11 @@ def test_fused_attention_under_graph_replay():
         assert torch.equal(out_g, exp_out) and torch.equal(lse_g, exp_lse), f"replay {rep}"
 
 
-@pytest.mark.parametrize("cfg_idx", [1, 3])
+@pytest.mark.parametrize("cfg_idx", [1, 2, 3])
 def test_fused_attention_full_size_layer(cfg_idx):
-    """One layer at the configuration's full context (32k for C1, 128k with 8 query heads per
-    KV head for C3), packed on the GPU, against the CPU oracle of the same packed layer."""
-    import dataclasses
+    """One layer at the configuration's full context (32k for C1; 128k, mostly 2-bit V and K
+    without 8-bit channels for C2; 128k with 8 query heads per KV head for C3), packed on the GPU,
+    against the CPU oracle of the same packed layer."""
     cfg = synth.scaled(synth.CONFIGS[cfg_idx], layers=1)
     vb, kb, oc = synth.layer_allocation(cfg, 0)
     K, V, q = synth.layer_data(cfg, 0, DEV, outliers=oc)
@@ -254,12 +265,44 @@ def test_fused_attention_full_size_layer(cfg_idx):
     del K, V
     cache = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
     out, lse = stream_cache.decode_attn_fused(cache, q)
-    kw = {f.name: (t2n(getattr(pl, f.name)) if torch.is_tensor(getattr(pl, f.name)) else getattr(pl, f.name))
-          for f in dataclasses.fields(O.PackedKVLayer)}
-    exp_out, exp_lse, _ = O.decode_attn_ref(t2n(q), O.PackedKVLayer(**kw), t2n(nvo) if nvo is not None else None)
+    exp_out, exp_lse, _ = O.decode_attn_ref(t2n(q), layer_to_oracle(pl), t2n(nvo) if nvo is not None else None)
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
     assert cache.n_groups >= 128      # the layer alone already spreads over the compute units
+    if cfg_idx == 2:
+        assert cfg.context == 131072 and all(int(u["d8"]) == 0 for u in cache.units_host)
+
+
+def test_fused_attention_ragged_batch():
+    """Configuration 4's shape: several independent sequences of different context lengths (drawn
+    from the configuration's range 16k..64k), each with its own per-head allocations, all (sequence,
+    layer) units in ONE launch.  The reference is strictly batch 1 (packing.py:234,432), so every
+    sequence's rows are held against the oracle of that sequence's own packed layer."""
+    cfg = synth.scaled(synth.CONFIGS[4], batch=4, layers=2)
+    contexts = [synth.seq_context(cfg, s) for s in range(cfg.batch)]
+    assert len(set(contexts)) == cfg.batch and min(contexts) >= 16384 and max(contexts) <= 65536
+    entries, qs = [], []
+    for seq in range(cfg.batch):
+        for layer in range(cfg.layers):
+            vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
+            K, V, q = synth.layer_data(cfg, layer, DEV, seq, outliers=oc)
+            assert K.shape[2] == contexts[seq]
+            entries.append(packing.pack_layer_per_head(K, V, vb, kb, cfg.G))
+            qs.append(q)
+            del K, V
+    cache = stream_cache.build_stream_cache(entries, cfg.G)
+    assert cache.n_units == cfg.batch * cfg.layers * cfg.H_kv and cache.rows == len(entries) * cfg.H_q
+    out, lse = stream_cache.decode_attn_fused(cache, torch.cat(qs).contiguous())
+    out, lse = t2n(out), t2n(lse)
+    algo = 0
+    for i, (pl, nvo) in enumerate(entries):
+        ora = layer_to_oracle(pl)
+        exp_out, exp_lse, _ = O.decode_attn_ref(t2n(qs[i]), ora, t2n(nvo) if nvo is not None else None)
+        rows = slice(i * cfg.H_q, (i + 1) * cfg.H_q)
+        attn_close(out[rows], exp_out, f"out sequence {i // cfg.layers} layer {i % cfg.layers}")
+        attn_close(lse[rows], exp_lse, f"lse sequence {i // cfg.layers} layer {i % cfg.layers}")
+        algo += O.algorithmic_bytes(ora, cfg.H_q)
+    assert cache.algorithmic_bytes == algo
 
 
 @pytest.mark.parametrize("counts", [(1, 1, 120), (128, 0, 0), (0, 128, 0), (0, 0, 128), (60, 60, 8), (17, 9, 5),
@@ -324,6 +367,7 @@ def test_multi_source_rows():
     cfg = synth.scaled(synth.CONFIGS[1], context=900, layers=4)
     packed, q4, _ = _config_case(cfg, 4)
     q = q4[:2 * cfg.H_q].contiguous()                  # two output groups
+    q_np = t2n(q)
     # entries 0,2 -> group 0; entries 1,3 -> group 1
     cache = stream_cache.build_stream_cache(packed, cfg.G, row_of_entry=[0, 1, 0, 1])
     assert cache.rows == 2 * cfg.H_q and cache.n_units == 4 * cfg.H_kv
@@ -341,6 +385,15 @@ def test_multi_source_rows():
         r = slice(grp * cfg.H_q, (grp + 1) * cfg.H_q)
         assert float((out[r] - exp_out).abs().max()) < 2e-5
         assert float((lse[r] - exp_lse).abs().max()) < 2e-5
+        # ... and against the oracle: dequantize-then-attend per source with this group's query,
+        # then the exact softmax over the union of the two sources' tokens
+        parts = []
+        for i in (grp, grp + 2):
+            pl_i, nvo_i = packed[i]
+            parts.append(O.decode_attn_ref(q_np[r], layer_to_oracle(pl_i), t2n(nvo_i) if nvo_i is not None else None)[:2])
+        ora_out, ora_lse = lse_merge(parts)
+        attn_close(t2n(out[r]), ora_out, f"union of two sources, group {grp}")
+        attn_close(t2n(lse[r]), ora_lse, f"union lse, group {grp}")
     # zone C on top, against the PyTorch merge of the two-source result
     g = torch.Generator().manual_seed(2)
     K_new = [torch.randn(cfg.H_kv, 9, 128, generator=g).to(DEV) for _ in range(2)]
