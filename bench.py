@@ -45,6 +45,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--sequential-only", action="store_true",
+                    help="only the one-layer-per-call leg (for profiling): prints its JSON and exits")
     ap.add_argument("--no-decode-loop", action="store_true",
                     help="skip the whole-model greedy decode loop (random-weight Llama-3.1-8B-shaped model)")
     return ap.parse_args()
@@ -125,6 +127,51 @@ def decode_loop_section(cfg, torch, dev, tokens=48):
     return res
 
 
+def sequential_section(cfg, torch, dev, layers=8, replays=50):
+    """One layer per call, the form a sequential model loop issues: ``layers`` single-layer streaming
+    caches (distinct buffers), their fused calls (streaming launch + merge launch each) recorded one
+    after the other into one HIP graph, the graph replayed back to back.  Returns us per layer."""
+    import numpy as np
+    from rdkv_amd import packing, stream_cache, synth
+    caches, qs, outs = [], [], []
+    for layer in range(layers):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, q = synth.layer_data(cfg, layer, dev, outliers=oc)
+        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+        del K, V
+        c = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
+        caches.append(c)
+        qs.append(q)
+        outs.append((torch.empty(c.rows, 128, device=dev), torch.empty(c.rows, device=dev)))
+
+    def all_layers():
+        for c, q, (o, l) in zip(caches, qs, outs):
+            stream_cache.decode_attn_fused(c, q, o, l)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        all_layers()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            all_layers()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        ms_graph = time_region(graph.replay, replays, torch) / layers
+        ms_eager = time_region(all_layers, replays, torch) / layers
+    torch.cuda.current_stream().wait_stream(side)
+    algo = float(np.mean([c.algorithmic_bytes for c in caches]))
+    return {"layers_rotated": layers, "context": cfg.context,
+            "us_per_layer_graph_replay": ms_graph * 1e3, "us_per_layer_eager": ms_eager * 1e3,
+            "algorithmic_bytes_per_layer": algo,
+            "GBps_graph_replay": algo / (ms_graph * 1e-3) / 1e9,
+            "frac_hbm_peak_graph_replay": algo / (ms_graph * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+            "workgroups_per_layer": caches[0].n_groups or caches[0].n_work, "work_items_per_layer": caches[0].n_work,
+            "note": "one layer per call (streaming launch + merge launch), calls of distinct layers back to back"}
+
+
 def main():
     args = parse()
     default_workload = (args.layers is None and args.context is None and args.batch is None
@@ -148,6 +195,9 @@ def main():
 
     cfg = synth.CONFIGS[args.config]
     cfg = synth.scaled(cfg, context=args.context, layers=args.layers, batch=args.batch)
+    if args.sequential_only:
+        print(json.dumps(sequential_section(cfg, torch, dev, replays=args.steps)))
+        return
     t_build = time.time()
     groups = []          # (packed layer, new_v_only) per (sequence, layer)
     keep_first = None    # layer 0 of sequence 0: inputs kept for the CPU baseline / checks / dense run
