@@ -325,15 +325,20 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   uint32_t krow[kRowA];
   uint32_t ktail[kRowB > 0 ? kRowB : 1];
   uint4 ksz;
-  auto issue_k = [&](int ti) __attribute__((always_inline)) {
-    const uint8_t *ktile = it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R;
+  // ok == false (a wavefront without a tile in this item): every load reads the first 16 bytes
+  // of the unit table instead, so the same number of loads is in flight on every path and no
+  // address outside the unit's regions is formed.
+  auto issue_k = [&](int ti, bool ok = true) __attribute__((always_inline)) {
+    const uint8_t *ktile = ok ? it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R
+                              : reinterpret_cast<const uint8_t *>(units);
+    const int lane_k = ok ? lane : 0;
 #pragma unroll
     for (int ch = 0; ch < RMAX / 4; ++ch) {
-      const int che = ch < it.nchunks ? ch : 0;
+      const int che = (ok && ch < it.nchunks) ? ch : 0;
       const int wce = che == it.nchunk_full ? it.wc_last : 4;
       // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
       // the next token (or the region that follows) and are never used
-      const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane * 4 * wce);
+      const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane_k * 4 * wce);
       if (4 * ch < kRowA) {
         krow[4 * ch] = v.x; krow[4 * ch + 1] = v.y; krow[4 * ch + 2] = v.z; krow[4 * ch + 3] = v.w;
       } else {
@@ -342,15 +347,18 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
       }
     }
     ksz = *reinterpret_cast<const uint4 *>(
-        it.sz_base + (ti < it.ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0));
+        ok ? it.sz_base + (ti < it.ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0)
+           : reinterpret_cast<const uint8_t *>(units));
   };
-  auto issue_v = [&](const Cursor &c, VRegs &r) __attribute__((always_inline)) {
-    const uint4 *vt = reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc;
-    const int hi = c.cls != 0 ? 128 : 0;
+  auto issue_v = [&](const Cursor &c, VRegs &r, bool ok = true) __attribute__((always_inline)) {
+    const uint4 *vt = ok ? reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc
+                         : reinterpret_cast<const uint4 *>(units);
+    const int hi = (ok && c.cls != 0) ? 128 : 0;
+    const int second = ok ? 64 : 0;
     r.v[0] = ld16_stream(vt);
-    r.v[1] = ld16_stream(vt + 64);
+    r.v[1] = ld16_stream(vt + second);
     r.v[2] = ld16_stream(vt + hi);
-    r.v[3] = ld16_stream(vt + hi + 64);
+    r.v[3] = ld16_stream(vt + hi + second);
   };
 
   VRegs va, vb;
@@ -375,38 +383,67 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_o));
   const int tid_o = wave * 64 + lane_o;
 
-  // The first item's first loads go out before anything else so that they overlap the staging.
-  start_item(batch);
-
   // ---------------- staging: qs = fp16(q * scale * log2e/sqrt(D) * 2^8), bias, per item ---
-  // The slot tables and the query rows of all items are fetched side by side (one memory
-  // latency, not a table -> gather chain) and combined from LDS.
-  for (int b = 0; b < nb; ++b) {
-    const Item sb = load_item(batch + b);
-    const RdkvSlot *tab = reinterpret_cast<const RdkvSlot *>(sb.qtab_base);
-    const int nslot = 4 * sb.NS;
-    for (int i = tid_o; i < nslot; i += kThreads) {
-      const RdkvSlot sl = tab[i];
-      sm.slot_channel[b][i] = sl.channel;
-      sm.slot_scale[b][i] = (float)__builtin_bit_cast(_Float16, sl.scale_f16);
-      sm.slot_zp[b][i] = (float)__builtin_bit_cast(_Float16, sl.zp_f16);
-    }
-    for (int i = tid_o; i < G * kD; i += kThreads) {
-      const int c = i & 127;
-      const int64_t row = (int64_t)(sb.q_row + (i >> 7)) * q_stride;
-      float v = load_qv(q, q_dtype, row + c);
-      if (rope_cos) {
-        // rotary embedding of the query on the fly (triton_rope.py:36-77): what the reference
-        // writes back to q in its storage type before the K kernel reads it
-        const float other = load_qv(q, q_dtype, row + (c ^ 64));
-        const float cs = rdkv_load_as_float(rope_cos, rope_dtype, c & 63);
-        const float sn = rdkv_load_as_float(rope_sin, rope_dtype, c & 63);
-        float out_lo, out_hi;
-        if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
-        else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
-        v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+  // Order of the global loads: the slot tables and query rows of the batch's items first (a few
+  // KB, fetched side by side into registers), then the first tile of the first item.  Loads
+  // complete in the order they were issued, so the other way round the staging would wait for
+  // the whole first round of tiles of the compute unit (160 KB) to arrive.  No branch around
+  // any of these loads: an item index past the batch repeats item 0, an element index past the
+  // table re-reads element 0.
+  it = load_item(batch);
+  set_tile(c0, it.tile_begin + wave);
+  constexpr int kQPer = (NH * 4 * kD + kThreads - 1) / kThreads;   // query elements per thread
+  uint2 st_slot[kBatch];
+  uint32_t st_q[kBatch][kQPer], st_qo[kBatch][kQPer], st_cs[kBatch][kQPer], st_sn[kBatch][kQPer];
+#pragma unroll
+  for (int b = 0; b < kBatch; ++b) {
+    const Item sb = load_item(batch + (b < nb ? b : 0));
+    const uint2 *tab = reinterpret_cast<const uint2 *>(sb.qtab_base);
+    st_slot[b] = tab[tid_o < 4 * sb.NS ? tid_o : 0];
+#pragma unroll
+    for (int e = 0; e < kQPer; ++e) {
+      const int i = tid_o + e * kThreads;
+      const int ic = i < G * kD ? i : 0;
+      const int64_t at = (int64_t)(sb.q_row + (ic >> 7)) * q_stride + (ic & 127);
+      st_q[b][e] = rdkv_load_dword_of(q, q_dtype, at);
+      st_qo[b][e] = st_cs[b][e] = st_sn[b][e] = 0;
+      if (rope_cos) {   // rotary embedding on the fly: the partner channel, the angle's cosine and sine
+        st_qo[b][e] = rdkv_load_dword_of(q, q_dtype, at ^ 64);
+        st_cs[b][e] = rdkv_load_dword_of(rope_cos, rope_dtype, ic & 63);
+        st_sn[b][e] = rdkv_load_dword_of(rope_sin, rope_dtype, ic & 63);
       }
-      sm.qraw[b][i >> 7][c] = v;
+    }
+  }
+  // the first tile of the first item
+  issue_k(c0.ti, c0.valid);
+  issue_v(c0, va, c0.valid);
+#pragma unroll
+  for (int b = 0; b < kBatch; ++b) {
+    if (tid_o < 4 * RDKV_MAX_STEPS) {
+      sm.slot_channel[b][tid_o] = (uint16_t)(st_slot[b].x & 0xffffu);
+      sm.slot_scale[b][tid_o] = (float)__builtin_bit_cast(_Float16, (uint16_t)(st_slot[b].x >> 16));
+      sm.slot_zp[b][tid_o] = (float)__builtin_bit_cast(_Float16, (uint16_t)(st_slot[b].y & 0xffffu));
+    }
+#pragma unroll
+    for (int e = 0; e < kQPer; ++e) {
+      const int i = tid_o + e * kThreads;
+      if (i < G * kD) {
+        const int c = i & 127;
+        const int64_t at = (int64_t)(load_item(batch + (b < nb ? b : 0)).q_row + (i >> 7)) * q_stride + c;
+        float v = rdkv_decode_dword(st_q[b][e], q, q_dtype, at);
+        if (rope_cos) {
+          // what the reference writes back to q in its storage type before the K kernel reads
+          // it (triton_rope.py:36-77)
+          const float other = rdkv_decode_dword(st_qo[b][e], q, q_dtype, at ^ 64);
+          const float cs = rdkv_decode_dword(st_cs[b][e], rope_cos, rope_dtype, c & 63);
+          const float sn = rdkv_decode_dword(st_sn[b][e], rope_sin, rope_dtype, c & 63);
+          float out_lo, out_hi;
+          if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
+          else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
+          v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
+        }
+        sm.qraw[b][i >> 7][c] = v;
+      }
     }
   }
   __syncthreads();

@@ -23,6 +23,22 @@ __device__ __forceinline__ float rdkv_load_as_float_nobranch(const void *p, int 
   return f32 ? as32 : (dtype == RDKV_DTYPE_F16 ? as16 : asbf);
 }
 
+// The same value from ONE load: the aligned dword that holds the element (the fp32 element
+// itself, or the pair of 16-bit elements one of which is wanted), decoded by rdkv_decode_dword.
+// The dword never leaves the allocation the element lives in (allocations are at least 4-byte
+// aligned).  Splitting load and decode lets a caller put many loads in flight first.
+__device__ __forceinline__ uint32_t rdkv_load_dword_of(const void *p, int dtype, int64_t idx) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p) + (dtype == RDKV_DTYPE_F32 ? 4 : 2) * (uintptr_t)idx;
+  return *reinterpret_cast<const uint32_t *>(a & ~(uintptr_t)3);
+}
+__device__ __forceinline__ float rdkv_decode_dword(uint32_t w, const void *p, int dtype, int64_t idx) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p) + 2 * (uintptr_t)idx;
+  const uint32_t h = (a & 2) ? (w >> 16) : (w & 0xffffu);
+  const float as16 = (float)__builtin_bit_cast(_Float16, (uint16_t)h);
+  const float asbf = __uint_as_float(h << 16);
+  return dtype == RDKV_DTYPE_F32 ? __uint_as_float(w) : (dtype == RDKV_DTYPE_F16 ? as16 : asbf);
+}
+
 // fp32 -> bf16 bits, round to nearest even (NaN stays NaN)
 __device__ __forceinline__ uint16_t rdkv_float_to_bf16_bits(float v) {
   uint32_t u = __float_as_uint(v);
