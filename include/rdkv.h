@@ -248,8 +248,15 @@ typedef struct RdkvSlot {   /* one K channel slot in MFMA consumption order */
   uint16_t reserved;
 } RdkvSlot;
 
-typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgroup */
-  int32_t unit, tile_begin, tile_end, reserved;
+typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgroup; 128 bytes */
+  int32_t  unit, tile_begin, tile_end;
+  int32_t  merge_unit;      /* the unit whose work_begin / work_count cover this item's partial: `unit`
+                               itself, or the first source of its output row                        */
+  RdkvUnit u;               /* copy of units[unit]: the streaming kernel reads the descriptor here
+                               (one fetch, where work -> unit would be two dependent ones)          */
+  int32_t  merge_begin;     /* work_begin and work_count of units[merge_unit]                       */
+  int32_t  merge_count;
+  int32_t  reserved[2];
 } RdkvWork;
 
 /* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.
@@ -307,6 +314,20 @@ int rdkv_decode_fused_partials(const uint8_t *blob, const RdkvUnit *units, int n
 int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_work, int G,
                             float *out, int64_t out_stride_row, float *lse,
                             void *workspace, int64_t workspace_bytes, void *stream);
+
+/* rdkv_decode_fused as ONE launch (same arguments, same results bit for bit): the workgroup that
+ * delivers the last partial of an output row combines that row's partials itself, in index
+ * order, instead of a second launch doing it - what a sequential model loop wants, where one
+ * layer's call is short and the second launch is a third of its time.  tickets: device int32
+ * [n_units], all zero before the first call; every call returns it to zero.  Calls that share
+ * tickets or a workspace must not overlap.  No counterpart in the reference as an interface (it
+ * replaces fast_decode.py:1707-1768 like rdkv_decode_fused). */
+int rdkv_decode_fused_one_launch(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                                 const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                                 int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
+                                 const void *rope_cos, const void *rope_sin, int rope_dtype,
+                                 float *out, int64_t out_stride_row, float *lse,
+                                 void *workspace, int64_t workspace_bytes, int32_t *tickets, void *stream);
 
 /* rdkv_decode_fused for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the

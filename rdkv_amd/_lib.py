@@ -59,6 +59,7 @@ SIGNATURES = {
                                        P, L, P, P, L, P, P, I, I, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),
     "rdkv_decode_fused": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P, P, L, P]),
+    "rdkv_decode_fused_one_launch": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P, P, L, P, P]),
     "rdkv_decode_fused_static_max_bytes": (L, []),
     "rdkv_decode_fused_static": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P, P]),
     "rdkv_decode_fused_partials": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P]),

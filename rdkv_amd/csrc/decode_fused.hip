@@ -24,8 +24,6 @@
 #include "rope_device.h"
 #include "stream_format.h"
 
-#include <stdlib.h>
-
 #include <mutex>
 
 namespace {
@@ -107,8 +105,23 @@ __device__ __forceinline__ float quadcol_max(float v) {
 // costs about one memory latency instead of one per partial.
 constexpr int kMergeMaxK = 128;
 
+// A partial value as another workgroup of the SAME launch left it: partials are written with
+// device-scope stores (pstore) and read here with device-scope loads, which are served from the
+// level of the memory hierarchy all compute dies share instead of a die's own caches.
+__device__ __forceinline__ void pstore(float *p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool COHERENT>
+__device__ __forceinline__ float pload(const float *p) {
+  if (COHERENT) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return *p;
+}
+
 // keep_o / keep_lse (LDS, [8][128] and [8], or null): when given, the normalized result and the
 // natural-log sum-exp stay there for a following zone-C pass instead of being written out.
+// COHERENT: the partials were written earlier in the same launch (merge inside the streaming
+// kernel); otherwise by a launch that has completed.
+template <bool COHERENT = false>
 __device__ __forceinline__ void merge_unit(const float *partials, int work_begin, int n, int G, int q_row,
                                            float *out, int64_t out_stride, float *lse, int tid, int nthreads,
                                            float *scratch, float *keep_o = nullptr, float *keep_lse = nullptr) {
@@ -125,12 +138,12 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
       const int i0 = tid < G * kD ? tid : 0;
       const float *b0 = base0 + (i0 >> 7) * kPartialStride + (i0 & 127);
 #pragma unroll
-      for (int e = 0; e < kMergeAhead; ++e) ahead[e] = *(b0 + (e < n ? e : 0) * pstride);
+      for (int e = 0; e < kMergeAhead; ++e) ahead[e] = pload<COHERENT>(b0 + (e < n ? e : 0) * pstride);
     }
     for (int i = tid; i < n * G; i += nthreads) {
       const int k = i / G, h = i - k * G;
-      s_m[k * 8 + h] = *(base0 + k * pstride + h * kPartialStride + 128);
-      s_l[k * 8 + h] = *(base0 + k * pstride + h * kPartialStride + 129);
+      s_m[k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 128);
+      s_l[k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 129);
     }
     __syncthreads();
     for (int i = tid; i < G * kD; i += nthreads) {
@@ -155,7 +168,7 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
       for (int k0 = k_from; k0 < n; k0 += 16) {
         float v[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) v[e] = *(base + (k0 + e < n ? k0 + e : k0) * pstride);
+        for (int e = 0; e < 16; ++e) v[e] = pload<COHERENT>(base + (k0 + e < n ? k0 + e : k0) * pstride);
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           if (k0 + e < n) {
@@ -183,14 +196,14 @@ __device__ __forceinline__ void merge_unit(const float *partials, int work_begin
     const int h = i >> 7, d = i & 127;
     const float *base = base0 + h * kPartialStride;
     float M = -INFINITY;
-    for (int k = 0; k < n; ++k) M = fmaxf(M, *(base + k * pstride + 128));
+    for (int k = 0; k < n; ++k) M = fmaxf(M, pload<COHERENT>(base + k * pstride + 128));
     float o = 0.0f, l = 0.0f;
     for (int k = 0; k < n; ++k) {
       const float *p = base + k * pstride;
-      const float mk = *(p + 128);
+      const float mk = pload<COHERENT>(p + 128);
       const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
-      o += f * *(p + d);
-      l += f * *(p + 129);
+      o += f * pload<COHERENT>(p + d);
+      l += f * pload<COHERENT>(p + 129);
     }
     const int64_t row = q_row + h;
     const float o_n = l > 0.0f ? o / l : 0.0f;
@@ -216,6 +229,7 @@ struct Smem {
   float slot_scale[kBatch][4 * RDKV_MAX_STEPS], slot_zp[kBatch][4 * RDKV_MAX_STEPS];
   uint16_t slot_channel[kBatch][4 * RDKV_MAX_STEPS];
   int progress[16];                                              // tiles done per wavefront
+  int ticket[kBatch];                                            // arrival order of the batch's partials at their units
   float wm[kBatch][NW][NH * 4];                                  // per-wavefront results of an item
   float wl[kBatch][NW][NH * 4];
   float wo[kBatch][NW][NH * 4][kD];
@@ -240,6 +254,7 @@ struct Cursor {  // wave-uniform position in the tile/piece sequence of this wav
 struct Item {
   int tile_begin, tile_end, d8, d4, d2, R, NS, n0, n1, n2, n3, ts1, ts2, ts3, q_row;
   int nchunk_full, wc_last, nchunks;
+  int merge_unit, merge_begin, merge_count;
   const uint8_t *k_base, *sz_base, *v_base0, *v_base1, *v_base2, *v_base3, *qtab_base;
 };
 
@@ -256,13 +271,14 @@ __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
 // waiting for the others (wavefronts drift apart by several tiles over an item; a barrier per
 // item cost 12-15 us of idle time each), parks its result per item in LDS, and one barrier
 // later the workgroup combines and writes the partials of the batch.
-template <int NH, int RMAX, int WPE>
+template <int NH, int RMAX, int WPE, bool MERGE>
 __global__ void __launch_bounds__(256 * WPE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
-decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict__ units,
+decode_fused_kernel(const uint8_t *__restrict__ blob,
                     const RdkvWork *__restrict__ work, const int32_t *__restrict__ groups,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride, int G,
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
-                    float *__restrict__ partials) {
+                    float *partials, int32_t *tickets, float *__restrict__ out, int64_t out_stride,
+                    float *__restrict__ lse) {
   constexpr int kWaves = 4 * WPE, kThreads = 64 * kWaves;
   __shared__ Smem<NH, kWaves> sm;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -274,8 +290,9 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
 
   auto load_item = [&](int item) __attribute__((always_inline)) -> Item {
     const RdkvWork *wkp = work + item;
-    const RdkvUnit *up = units + wkp->unit;
+    const RdkvUnit *up = &wkp->u;    // the unit's descriptor travels with the work item
     Item it;
+    it.merge_unit = wkp->merge_unit; it.merge_begin = wkp->merge_begin; it.merge_count = wkp->merge_count;
     it.tile_begin = wkp->tile_begin;
     it.tile_end = wkp->tile_end;
     it.d8 = up->d8; it.d4 = up->d4; it.d2 = up->d2;
@@ -326,11 +343,11 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   uint32_t ktail[kRowB > 0 ? kRowB : 1];
   uint4 ksz;
   // ok == false (a wavefront without a tile in this item): every load reads the first 16 bytes
-  // of the unit table instead, so the same number of loads is in flight on every path and no
+  // of the work table instead, so the same number of loads is in flight on every path and no
   // address outside the unit's regions is formed.
   auto issue_k = [&](int ti, bool ok = true) __attribute__((always_inline)) {
     const uint8_t *ktile = ok ? it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R
-                              : reinterpret_cast<const uint8_t *>(units);
+                              : reinterpret_cast<const uint8_t *>(work);
     const int lane_k = ok ? lane : 0;
 #pragma unroll
     for (int ch = 0; ch < RMAX / 4; ++ch) {
@@ -348,11 +365,11 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
     }
     ksz = *reinterpret_cast<const uint4 *>(
         ok ? it.sz_base + (ti < it.ts3 ? (uint64_t)ti * (RDKV_TILE * 4) + lb * 16 : 0)
-           : reinterpret_cast<const uint8_t *>(units));
+           : reinterpret_cast<const uint8_t *>(work));
   };
   auto issue_v = [&](const Cursor &c, VRegs &r, bool ok = true) __attribute__((always_inline)) {
     const uint4 *vt = ok ? reinterpret_cast<const uint4 *>(c.vtile) + lane + 256 * c.pc
-                         : reinterpret_cast<const uint4 *>(units);
+                         : reinterpret_cast<const uint4 *>(work);
     const int hi = (ok && c.cls != 0) ? 128 : 0;
     const int second = ok ? 64 : 0;
     r.v[0] = ld16_stream(vt);
@@ -795,10 +812,38 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
         o += f * sm.wo[b][w][h][d];
         l += f * sm.wl[b][w][h];
       }
-      part[h * kPartialStride + d] = o;
+      pstore(part + h * kPartialStride + d, o);
       if (d == 0) {
-        part[h * kPartialStride + 128] = M;
-        part[h * kPartialStride + 129] = l;
+        pstore(part + h * kPartialStride + 128, M);
+        pstore(part + h * kPartialStride + 129, l);
+      }
+    }
+  }
+  if (MERGE) {
+    // ---------------- merge inside this launch: the last partial to arrive at a unit merges it ----
+    // Every thread waits until its partial stores have completed at device scope, the workgroup
+    // meets, one thread takes a ticket per item at the item's merging unit (device-scope atomic);
+    // whoever draws the last ticket of a unit finds all of that unit's partials complete, puts the
+    // counter back to zero for the next launch and combines them in index order - the same
+    // arithmetic in the same order as the separate merge launch, whoever happens to be last.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid_o < nb) {
+      const RdkvWork *wkp = work + batch + tid_o;
+      sm.ticket[tid_o] = __hip_atomic_fetch_add(tickets + wkp->merge_unit, 1, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    for (int b = 0; b < nb; ++b) {
+      const Item mi = load_item(batch + b);
+      if (sm.ticket[b] == mi.merge_count - 1) {      // uniform over the workgroup
+        if (tid_o == 0) __hip_atomic_store(tickets + mi.merge_unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the wavefront results of the batch have been consumed: their LDS serves as scratch
+        float *scratch = &sm.wo[0][0][0][0];
+        static_assert(sizeof(sm.wo) >= 2 * kMergeMaxK * 8 * sizeof(float), "merge scratch does not fit");
+        merge_unit<true>(partials, mi.merge_begin, mi.merge_count, G, mi.q_row, out, out_stride, lse, tid_o,
+                         kThreads, scratch);
+        __syncthreads();
       }
     }
   }
@@ -806,8 +851,11 @@ decode_fused_kernel(const uint8_t *__restrict__ blob, const RdkvUnit *__restrict
   }  // batches of this group
 }
 
-// One workgroup per unit combines its partials (second launch of a step).  Merging inside the
-// streaming kernel (last-arriver ticket with device-scope stores) was measured 7% slower.
+// One workgroup per unit combines its partials (second launch of a step).  The MERGE variant of
+// the streaming kernel does the same inside its launch (last-arriver ticket per output row, partials
+// stored and loaded at device scope): 0.8-1.5 us faster on a single 32k-token layer (24.7 against
+// 25.5 us per call), slower from about 200 work items on (the step of a whole model: 0.183 against
+// 0.182 ms), because every workgroup then waits for its stores and a ticket before it may leave.
 __global__ void __launch_bounds__(256)
 merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
@@ -1079,7 +1127,8 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
                         const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
                         int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
                         const void *rope_cos, const void *rope_sin, int rope_dtype, void *workspace,
-                        int64_t workspace_bytes, void *stream) {
+                        int64_t workspace_bytes, void *stream, int32_t *tickets = nullptr, float *out = nullptr,
+                        int64_t out_stride_row = 0, float *lse = nullptr) {
   int rc = check_fused_args(fn, units, n_units, work, n_work, G, workspace, workspace_bytes);
   RDKV_REQUIRE((rope_cos == nullptr) == (rope_sin == nullptr), "%s: rope_cos and rope_sin go together", fn);
   RDKV_REQUIRE(!rope_cos || (rope_dtype >= 0 && rope_dtype <= 2), "%s: unknown rope dtype %d", fn, rope_dtype);
@@ -1096,40 +1145,30 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   float *partials = (float *)workspace;
   // Occupancy target (wavefronts per SIMD) of each variant: the highest at which the variant
   // keeps everything in registers; spilling costs far more than the lost occupancy.
-  // RDKV_FUSED_WPE overrides it (2, 3 or 4) for experiments.
-  static const int wpe_env = getenv("RDKV_FUSED_WPE") ? atoi(getenv("RDKV_FUSED_WPE")) : 0;
+  // (the variant that merges in the launch is a kernel of its own: the merge's registers would
+  // otherwise push the two-launch form into scratch memory)
+#define RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, MERGE)                                                             \
+  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE, MERGE>), dim3(n_wg), dim3(256 * WPE), 0, s, blob, work, \
+                     groups, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, partials, tickets,  \
+                     out, out_stride_row, lse)
 #define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE)                                                               \
-  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE>), dim3(n_wg), dim3(256 * WPE), 0, s, blob, units, \
-                     work, groups, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, partials)
-  // one head group: 2..4 wavefronts per SIMD
-#define RDKV_LAUNCH_FUSED(NH, RMAX, WPE_DEFAULT)                                                           \
   do {                                                                                                     \
-    const int wpe = wpe_env ? wpe_env : WPE_DEFAULT;                                                       \
-    if (wpe >= 4) RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 4);                                                      \
-    else if (wpe == 3) RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 3);                                                 \
-    else RDKV_LAUNCH_FUSED_WPE(NH, RMAX, 2);                                                               \
+    if (tickets) RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, true);                                                 \
+    else RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, false);                                                        \
   } while (0)
-  // two head groups: the per-wavefront result buffers of 16 wavefronts would not fit in LDS
-#define RDKV_LAUNCH_FUSED2(RMAX, WPE_DEFAULT)                                                              \
-  do {                                                                                                     \
-    const int wpe = wpe_env ? wpe_env : WPE_DEFAULT;                                                       \
-    if (wpe >= 3) RDKV_LAUNCH_FUSED_WPE(2, RMAX, 3);                                                       \
-    else RDKV_LAUNCH_FUSED_WPE(2, RMAX, 2);                                                                \
-  } while (0)
-  if (G <= 4) {
-    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED(1, 12, 4);
-    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED(1, 16, 4);
-    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED(1, 20, 4);
-    else RDKV_LAUNCH_FUSED(1, 32, 3);
-  } else {
-    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED2(12, 3);
-    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED2(16, 3);
-    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED2(20, 3);
-    else RDKV_LAUNCH_FUSED2(32, 2);
+  if (G <= 4) {   // one head group
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED_WPE(1, 12, 4);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED_WPE(1, 16, 4);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED_WPE(1, 20, 4);
+    else RDKV_LAUNCH_FUSED_WPE(1, 32, 3);
+  } else {        // two head groups: the per-wavefront result buffers of 16 wavefronts would not fit in LDS
+    if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED_WPE(2, 12, 3);
+    else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED_WPE(2, 16, 3);
+    else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED_WPE(2, 20, 3);
+    else RDKV_LAUNCH_FUSED_WPE(2, 32, 2);
   }
-#undef RDKV_LAUNCH_FUSED2
 #undef RDKV_LAUNCH_FUSED_WPE
-#undef RDKV_LAUNCH_FUSED
+#undef RDKV_LAUNCH_FUSED_M
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }
@@ -1171,6 +1210,22 @@ RDKV_API int rdkv_decode_fused(const uint8_t *blob, const RdkvUnit *units, int n
   if (rc != RDKV_OK) return rc;
   return rdkv_decode_fused_merge(units, n_units, n_work, G, out, out_stride_row, lse, workspace,
                                  workspace_bytes, stream);
+}
+
+// rdkv_decode_fused as one launch: the workgroup that delivers the last partial of an output row
+// merges that row's partials itself (in index order, so the result does not depend on who is
+// last).  tickets: int32 [n_units], zero before the first call; every call leaves it zero.
+RDKV_API int rdkv_decode_fused_one_launch(const uint8_t *blob, const RdkvUnit *units, int n_units,
+                                          const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
+                                          int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row,
+                                          int G, const void *rope_cos, const void *rope_sin, int rope_dtype,
+                                          float *out, int64_t out_stride_row, float *lse, void *workspace,
+                                          int64_t workspace_bytes, int32_t *tickets, void *stream) {
+  const char *fn = "rdkv_decode_fused_one_launch";
+  RDKV_REQUIRE(n_units == 0 || (out && tickets), "%s: null out / tickets", fn);
+  return launch_fused(fn, blob, units, n_units, work, n_work, groups, n_groups, max_row_dwords, q, q_dtype,
+                      q_stride_row, G, rope_cos, rope_sin, rope_dtype, workspace, workspace_bytes, stream, tickets,
+                      out, out_stride_row, lse);
 }
 
 static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_units, int n_work, int G, const void *q,

@@ -35,9 +35,16 @@ UNIT_DTYPE = np.dtype([
     ("n_tok", "<i4", (4,)), ("d8", "<i4"), ("d4", "<i4"), ("d2", "<i4"),
     ("q_row", "<i4"), ("work_begin", "<i4"), ("work_count", "<i4")], align=True)
 SLOT_DTYPE = np.dtype([("channel", "<u2"), ("scale", "<u2"), ("zp", "<u2"), ("reserved", "<u2")])
-WORK_DTYPE = np.dtype([("unit", "<i4"), ("tile_begin", "<i4"), ("tile_end", "<i4"), ("reserved", "<i4")])
-assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.itemsize == 16
+# A work item carries a copy of its unit's descriptor (the kernel reads it with the item, one fetch
+# instead of two dependent ones) and the partial range of the output row it belongs to.
+WORK_DTYPE = np.dtype([("unit", "<i4"), ("tile_begin", "<i4"), ("tile_end", "<i4"), ("merge_unit", "<i4"),
+                       ("u", UNIT_DTYPE), ("merge_begin", "<i4"), ("merge_count", "<i4"), ("reserved", "<i4", (2,))])
+assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.itemsize == 128
 
+
+
+# Caches with at most this many work items run rdkv_decode_fused as one launch by default.
+ONE_LAUNCH_MAX_WORK = 160
 
 
 def _align(x: int, a: int = 256) -> int:
@@ -94,6 +101,8 @@ class StreamCache:
     kv_algorithmic_bytes: int = 0        # algorithmic bytes without the query / output rows
     multi_source: bool = False           # several units may feed one output row
     h_q: int = 0                         # query heads per output group
+    tickets: Optional[torch.Tensor] = None  # device int32 [n_units], zero between calls (one-launch form)
+    partition: Optional[dict] = None     # the work-partition arguments the cache was built with
 
     @property
     def device(self):
@@ -319,6 +328,7 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
                   multi_source: bool, work_bytes, n_groups, groups_per_cu: int, cost) -> StreamCache:
     """Order the units, cut the tile stream into work items and groups, upload the tables."""
     dev = blobs[0].device
+    n_groups_arg, cost_arg = n_groups, cost
     if multi_source:
         # sources of one output row next to each other, so that their work items are contiguous
         units_np = units_np[np.argsort(units_np["q_row"], kind="stable")]
@@ -343,12 +353,24 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
         wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
     units_np = units_np.copy()
     units_np["work_begin"], units_np["work_count"] = wb, wc
+    # every item knows the unit that merges its output row (the unit itself, or the row's first source)
+    if len(units_np):
+        merger = np.maximum.accumulate(np.where(wc > 0, np.arange(len(units_np)), 0)) if multi_source \
+            else np.arange(len(units_np))
+        iu = work_np["unit"]
+        work_np["u"] = units_np[iu]
+        work_np["merge_unit"] = merger[iu]
+        work_np["merge_begin"] = wb[merger[iu]]
+        work_np["merge_count"] = wc[merger[iu]]
     rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
     units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
     work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
-        16, dtype=torch.uint8, device=dev)
+        WORK_DTYPE.itemsize, dtype=torch.uint8, device=dev)
     groups_dev = torch.from_numpy(groups_np).to(dev) if groups_np is not None else None
-    return StreamCache(blobs=list(blobs), units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
+    return StreamCache(tickets=torch.zeros(max(1, len(units_np)), dtype=torch.int32, device=dev),
+                       partition={"work_bytes": work_bytes, "n_groups": n_groups_arg, "groups_per_cu": groups_per_cu,
+                                  "cost": cost_arg},
+                       blobs=list(blobs), units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
                        n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
                        stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
                        max_row_dwords=int(R_np.max()) if len(R_np) else 0,
@@ -373,9 +395,10 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
 
     Work decomposition: by default the tile stream is cut into one run of equal cost per
     compute unit (the fused kernel's workgroups fill a compute unit each); ``cost`` replaces
-    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count; caches too small to
-    keep every compute unit busy for long get about sqrt(6 * tiles) runs, at least 4 tiles each.  ``work_bytes`` instead asks for items of about that
-    many streamed bytes with one workgroup per item."""
+    the built-in cost model (DEFAULT_COST).  ``n_groups`` overrides the count.  ``work_bytes``
+    instead asks for items of about that many streamed bytes with one workgroup per item.  Caches
+    too small to keep every compute unit busy for long get about sqrt(6 * tiles) runs, at least 4
+    tiles each."""
     rows_of_entries = list(range(len(layers))) if row_of_entry is None else [int(r) for r in row_of_entry]
     assert len(rows_of_entries) == len(layers)
     units_np, blobs, stream_bytes, kv_algo, H_q = _relayout_entries(layers, G, rows_of_entries)
@@ -430,7 +453,8 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                       zone_c_weights: Optional[torch.Tensor] = None,
                       append: Optional[Tuple[torch.Tensor, torch.Tensor, torch.Tensor]] = None,
                       q_rotated_out: Optional[torch.Tensor] = None,
-                      tail_scores: Optional[Tuple[torch.Tensor, Optional[torch.Tensor], int, int]] = None):
+                      tail_scores: Optional[Tuple[torch.Tensor, Optional[torch.Tensor], int, int]] = None,
+                      one_launch: Optional[bool] = None):
     """One decode step over every unit of ``cache``.  q: [rows,128] fp16/bf16/fp32 (already
     rotated, or un-rotated together with ``rope`` = (cos_half, sin_half) of 64 values each: the
     kernel then applies the rotary embedding of ``triton_rope.fused_rope`` while it stages the
@@ -450,7 +474,10 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     the merge launch also adds the new tokens' weights, summed over a KV head's query heads, to
     ``self_scores[:, q_block_start:]`` and, when ``q_block_start >= block``, to
     ``next_scores[:, :block]`` - what ``rdkv_tail_scores`` does as a launch of its own.  Graph-capturable
-    once the workspace exists (first call): one streaming launch plus one small merge launch."""
+    once the workspace exists (first call): one streaming launch plus one small merge launch.
+    ``one_launch`` (without ``zone_c``): the streaming launch merges the partials itself (the last
+    workgroup to deliver a partial of an output row combines that row; same bits); default: for
+    caches of at most ONE_LAUNCH_MAX_WORK work items, where the second launch weighs most."""
     lib = _lib.load()
     dev = _lib.require_device(q)
     assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
@@ -473,6 +500,17 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     ws = _lib.workspace(dev, need)
     stream = _lib.stream_of(dev)
     assert zone_c_weights is None or zone_c is not None, "zone_c_weights needs zone_c"
+    if one_launch is None:
+        one_launch = zone_c is None and cache.n_work <= ONE_LAUNCH_MAX_WORK
+    assert not (one_launch and zone_c is not None), "one_launch does not take zone_c"
+    if one_launch:
+        _lib.check(lib.rdkv_decode_fused_one_launch(
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+            q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
+            out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), cache.tickets.data_ptr(),
+            stream))
+        return out, lse
     if zone_c is None:
         _lib.check(lib.rdkv_decode_fused(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
@@ -551,18 +589,63 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
 
 # ---------------------------------------------------------------------------
 # On-disk form of a streaming cache (the reference only pickles its Python dataclass,
-# run_latency.py:1987-1991): one file, a JSON header, then the tables and the blobs, all
-# 256-byte aligned, offsets inside the blobs relative so the file can be memory-mapped and
-# uploaded to any address.
+# run_latency.py:1987-1991, 2036-2041): one little-endian file - magic, header length, CRC-32 of
+# the header, a JSON header, then the unit table and the blobs, all 256-byte aligned, offsets
+# inside the blobs relative so the file can be memory-mapped and uploaded to any address.  The
+# file holds the layout only: the work items and groups (which depend on the number of compute
+# units of the device) are cut again on load for the device at hand.  Every section carries a
+# CRC-32, and every extent a kernel would follow is checked against the file before upload.
 # ---------------------------------------------------------------------------
 _MAGIC = b"RDKVSTR1"
+_FORMAT_VERSION = 2
 _ADDR_FIELDS = ("k_off", "sz_off", "qtab_off")
+
+
+def _unit_regions(u) -> list:
+    """(field, offset, bytes) of every region of the blob a unit's descriptor points to."""
+    tiles = [-(-int(n) // TILE) for n in u["n_tok"]]
+    R = int(u["d8"]) + int(u["d4"]) + int(u["d2"])
+    slots = 4 * int(u["d8"]) + 8 * int(u["d4"]) + 16 * int(u["d2"])
+    out = [("k_off", int(u["k_off"]), sum(tiles) * TILE * 4 * R)]
+    out += [(f"v_off[{c}]", int(u["v_off"][c]), tiles[c] * V_TILE_BYTES[c]) for c in range(4)]
+    out.append(("sz_off", int(u["sz_off"]), sum(tiles[:3]) * TILE * 4))
+    out.append(("qtab_off", int(u["qtab_off"]), slots * SLOT_DTYPE.itemsize))
+    return out
+
+
+def validate_units(units: np.ndarray, blob_of: np.ndarray, blob_sizes: Sequence[int], G: int, rows: int,
+                   what: str = "stream cache") -> None:
+    """Raise ValueError unless every descriptor stays inside its blob and inside what the fused
+    kernel assumes (row length, slot steps, output rows).  Offsets are blob-relative here."""
+    if len(blob_of) != len(units):
+        raise ValueError(f"{what}: {len(blob_of)} blob indices for {len(units)} units")
+    if not 1 <= int(G) <= 8:
+        raise ValueError(f"{what}: G={G} outside 1..8")
+    for i, u in enumerate(units):
+        d8, d4, d2 = int(u["d8"]), int(u["d4"]), int(u["d2"])
+        if min(d8, d4, d2) < 0 or d8 + d4 + d2 > MAX_ROW_DWORDS or d8 + 2 * d4 + 4 * d2 > MAX_STEPS:
+            raise ValueError(f"{what}: unit {i}: K row of {d8}+{d4}+{d2} dwords is outside the kernel's limits")
+        if (np.asarray(u["n_tok"]) < 0).any() or int(np.asarray(u["n_tok"], dtype=np.int64).sum()) >= 2 ** 31 - 64:
+            raise ValueError(f"{what}: unit {i}: bad token counts {list(u['n_tok'])}")
+        if int(u["q_row"]) < 0 or int(u["q_row"]) + int(G) > int(rows):
+            raise ValueError(f"{what}: unit {i}: output rows {int(u['q_row'])}..+{G} outside 0..{rows}")
+        b = int(blob_of[i])
+        if not 0 <= b < len(blob_sizes):
+            raise ValueError(f"{what}: unit {i}: blob index {b} outside 0..{len(blob_sizes) - 1}")
+        for name, off, nbytes in _unit_regions(u):
+            # the kernel reads whole 16-byte pieces: a region (an empty one too) may be over-read by 16 bytes
+            if off % 16 or off < 0 or off + nbytes + 16 > int(blob_sizes[b]):
+                raise ValueError(f"{what}: unit {i}: region {name} = [{off}, +{nbytes}) leaves blob {b} "
+                                 f"of {int(blob_sizes[b])} bytes")
 
 
 def save_stream_cache(cache: StreamCache, path: str) -> None:
     """Write ``cache`` to ``path`` (device -> host copy of the blobs)."""
     import json
+    import zlib
     units = cache.units_host.copy()
+    units["work_begin"] = 0
+    units["work_count"] = 0
     bases = [int(b.data_ptr()) for b in cache.blobs]
     sizes = [int(b.numel()) for b in cache.blobs]
     blob_of = np.zeros(len(units), dtype=np.int32)
@@ -573,79 +656,117 @@ def save_stream_cache(cache: StreamCache, path: str) -> None:
         for f in _ADDR_FIELDS:
             units[f][i] -= bases[j]
         units["v_off"][i] -= bases[j]
-    parts = [("units", units.view(np.uint8).reshape(-1)), ("blob_of", blob_of.view(np.uint8)),
-             ("work", cache.work_host.view(np.uint8).reshape(-1))]
-    if cache.groups_host is not None:
-        parts.append(("groups", cache.groups_host.astype(np.int32).view(np.uint8)))
-    header = {"version": 1, "G": cache.G, "rows": cache.rows, "stream_bytes": cache.stream_bytes,
-              "algorithmic_bytes": cache.algorithmic_bytes, "max_row_dwords": cache.max_row_dwords,
-              "n_units": cache.n_units, "n_work": cache.n_work, "n_groups": cache.n_groups,
+    parts = [("units", units.view(np.uint8).reshape(-1)), ("blob_of", blob_of.view(np.uint8))]
+    part = dict(cache.partition or {})
+    if part.get("cost") is not None:
+        part["cost"] = {k: list(v) if isinstance(v, (tuple, list)) else v for k, v in part["cost"].items()}
+    header = {"version": _FORMAT_VERSION, "byteorder": "little", "G": cache.G, "rows": cache.rows,
+              "stream_bytes": cache.stream_bytes, "algorithmic_bytes": cache.algorithmic_bytes,
+              "max_row_dwords": cache.max_row_dwords, "n_units": cache.n_units,
               "kv_algorithmic_bytes": cache.kv_algorithmic_bytes, "multi_source": bool(cache.multi_source),
-              "h_q": cache.h_q, "sections": {}, "blobs": []}
+              "h_q": cache.h_q, "partition": part, "sections": {}, "blobs": []}
     off = 0
     for name, arr in parts:
-        header["sections"][name] = [off, int(arr.nbytes)]
+        header["sections"][name] = [off, int(arr.nbytes), zlib.crc32(arr.tobytes())]
         off = _align(off + int(arr.nbytes))
-    for n in sizes:
-        header["blobs"].append([off, n])
+    blob_bytes = [blob.cpu().numpy() for blob in cache.blobs]
+    for n, data in zip(sizes, blob_bytes):
+        header["blobs"].append([off, n, zlib.crc32(data)])
         off = _align(off + n)
     hj = json.dumps(header).encode()
-    data0 = _align(len(_MAGIC) + 8 + len(hj))
+    data0 = _align(len(_MAGIC) + 16 + len(hj))
     with open(path, "wb") as f:
         f.write(_MAGIC)
         f.write(np.asarray([len(hj)], dtype="<u8").tobytes())
+        f.write(np.asarray([zlib.crc32(hj), 0], dtype="<u4").tobytes())
         f.write(hj)
         f.write(b"\0" * (data0 - f.tell()))
-        for (name, arr), (o, n) in zip(parts, header["sections"].values()):
+        for (name, arr), (o, n, _) in zip(parts, header["sections"].values()):
             f.seek(data0 + o)
             f.write(arr.tobytes())
-        for blob, (o, n) in zip(cache.blobs, header["blobs"]):
+        for data, (o, n, _) in zip(blob_bytes, header["blobs"]):
             f.seek(data0 + o)
-            f.write(blob.cpu().numpy().tobytes())
+            f.write(data.tobytes())
         f.truncate(data0 + off)
 
 
-def load_stream_cache(path: str, device) -> StreamCache:
-    """Memory-map ``path`` and upload it to ``device``; the result is usable like a freshly
-    built cache (same outputs, bit for bit)."""
+def read_stream_cache_file(path: str, verify: bool = True):
+    """Host side of ``load_stream_cache``: parse and check ``path`` without touching a device.
+    Returns (header, units with blob-relative offsets, blob_of, [memory-mapped blob bytes]).
+    Raises ValueError for a file that is not a streaming cache, has another format version, is
+    truncated, fails a checksum (``verify``) or describes regions outside its blobs."""
     import json
+    import zlib
+    mm = np.memmap(path, dtype=np.uint8, mode="r")
+    if len(mm) < 24 or bytes(mm[:8]) != _MAGIC:
+        raise ValueError(f"{path}: not a streaming-cache file")
+    hlen = int(np.frombuffer(mm[8:16], dtype="<u8")[0])
+    hcrc = int(np.frombuffer(mm[16:20], dtype="<u4")[0])
+    if hlen > len(mm) - 24:
+        raise ValueError(f"{path}: truncated header")
+    hj = bytes(mm[24:24 + hlen])
+    try:
+        header = json.loads(hj)
+        version = header["version"]
+    except Exception as e:    # an older layout keeps its JSON elsewhere: it does not parse here
+        raise ValueError(f"{path}: unreadable header (another format version?): {e}") from None
+    if version != _FORMAT_VERSION:
+        raise ValueError(f"{path}: unsupported version {version} (this build reads version {_FORMAT_VERSION})")
+    if zlib.crc32(hj) != hcrc:
+        raise ValueError(f"{path}: header checksum mismatch")
+    if header.get("byteorder") != "little":
+        raise ValueError(f"{path}: byte order {header.get('byteorder')!r} not supported")
+    data0 = _align(24 + hlen)
+
+    def extent(name, o, n, crc):
+        if o < 0 or n < 0 or data0 + o + n > len(mm):
+            raise ValueError(f"{path}: {name} = [{o}, +{n}) lies outside the file ({len(mm)} bytes): truncated?")
+        view = mm[data0 + o:data0 + o + n]
+        if verify and zlib.crc32(view) != crc:
+            raise ValueError(f"{path}: checksum mismatch in {name}")
+        return view
+
+    units = np.frombuffer(extent("units", *header["sections"]["units"]), dtype=UNIT_DTYPE).copy()
+    blob_of = np.frombuffer(extent("blob_of", *header["sections"]["blob_of"]), dtype=np.int32).copy()
+    if len(units) != header["n_units"]:
+        raise ValueError(f"{path}: {len(units)} units in the table, header says {header['n_units']}")
+    blobs = [extent(f"blob {j}", o, n, crc) for j, (o, n, crc) in enumerate(header["blobs"])]
+    validate_units(units, blob_of, [len(b) for b in blobs], header["G"], header["rows"], what=path)
+    R = units["d8"] + units["d4"] + units["d2"]
+    if len(units) and int(R.max()) > header["max_row_dwords"]:
+        raise ValueError(f"{path}: max_row_dwords={header['max_row_dwords']} below the longest K row {int(R.max())}")
+    return header, units, blob_of, blobs
+
+
+def load_stream_cache(path: str, device, verify: bool = True, **partition) -> StreamCache:
+    """Read ``path`` (see ``read_stream_cache_file`` for the checks), upload it to ``device`` and cut
+    the work items for that device with the arguments the cache was built with (``partition``:
+    ``n_groups`` / ``work_bytes`` / ``groups_per_cu`` / ``cost`` replace the stored ones); the
+    result is usable like a freshly built cache (with the same partition on a device with the same
+    number of compute units: the same outputs, bit for bit)."""
     dev = torch.device(device)
     if dev.type != "cuda":
         raise RuntimeError("rdkv HIP backend needs a HIP device; there is no CPU fallback")
-    mm = np.memmap(path, dtype=np.uint8, mode="r")
-    if bytes(mm[:8]) != _MAGIC:
-        raise ValueError(f"{path}: not a streaming-cache file")
-    hlen = int(np.frombuffer(mm[8:16], dtype="<u8")[0])
-    header = json.loads(bytes(mm[16:16 + hlen]))
-    if header["version"] != 1:
-        raise ValueError(f"{path}: unsupported version {header['version']}")
-    data0 = _align(16 + hlen)
-
-    def section(name, dtype):
-        o, n = header["sections"][name]
-        return np.frombuffer(mm[data0 + o:data0 + o + n], dtype=dtype).copy()
-
-    units = section("units", UNIT_DTYPE)
-    blob_of = section("blob_of", np.int32)
-    work = section("work", WORK_DTYPE)
-    groups = section("groups", np.int32) if "groups" in header["sections"] else None
+    header, units, blob_of, blob_views = read_stream_cache_file(path, verify=verify)
+    _lib.load()
     blobs = []
-    for o, n in header["blobs"]:
-        t = torch.from_numpy(np.array(mm[data0 + o:data0 + o + n])).to(dev)   # np.array: writable copy
+    for view in blob_views:
+        t = torch.from_numpy(np.array(view)).to(dev)   # np.array: writable copy
         assert t.data_ptr() % 256 == 0
         blobs.append(t)
     bases = np.asarray([int(b.data_ptr()) for b in blobs], dtype=np.uint64)
     for f in _ADDR_FIELDS:
         units[f] += bases[blob_of]
     units["v_off"] += bases[blob_of][:, None]
-    lib = _lib.load()
-    return StreamCache(
-        blobs=blobs, units=torch.from_numpy(units.view(np.uint8).copy()).to(dev),
-        work=(torch.from_numpy(work.view(np.uint8).copy()).to(dev) if len(work)
-              else torch.zeros(16, dtype=torch.uint8, device=dev)),
-        units_host=units, work_host=work, n_units=header["n_units"], n_work=header["n_work"], G=header["G"],
-        rows=header["rows"], stream_bytes=header["stream_bytes"], algorithmic_bytes=header["algorithmic_bytes"],
-        max_row_dwords=header["max_row_dwords"],
-        groups=torch.from_numpy(groups).to(dev) if groups is not None else None, groups_host=groups,
-        n_groups=header["n_groups"], kv_algorithmic_bytes=header.get("kv_algorithmic_bytes", 0),
-        multi_source=header.get("multi_source", False), h_q=header.get("h_q", 0))
+    unknown = set(partition) - {"n_groups", "work_bytes", "groups_per_cu", "cost"}
+    if unknown:
+        raise TypeError(f"load_stream_cache: unknown arguments {sorted(unknown)}")
+    part = dict(header.get("partition") or {})
+    part.update(partition)
+    cost = part.get("cost")
+    if cost is not None:
+        cost = {k: tuple(v) if isinstance(v, list) else v for k, v in cost.items()}
+    return _finish_cache(units, blobs, header["G"], header["h_q"], header["stream_bytes"],
+                         header["kv_algorithmic_bytes"], multi_source=header["multi_source"],
+                         work_bytes=part.get("work_bytes"), n_groups=part.get("n_groups"),
+                         groups_per_cu=part.get("groups_per_cu", 1), cost=cost)

@@ -94,3 +94,17 @@ def lse_merge(parts):
         out = np.where(tot[:, None] > 0, sum(w[:, None] * o for w, o in zip(ws, outs)) / tot[:, None], 0.0)
         lse = np.where(tot > 0, m + np.log(tot), -np.inf)
     return out, lse
+
+
+def fused_both(cache, q, **kw):
+    """``decode_attn_fused`` as two launches and, twice in a row, as one launch (the last workgroup
+    to deliver a partial of an output row merges that row): the same bits every time, and the
+    ticket counters are back at zero after every call.  Returns the two-launch result."""
+    from rdkv_amd import stream_cache
+    out, lse = stream_cache.decode_attn_fused(cache, q, one_launch=False, **kw)
+    for rep in range(2):
+        o1, l1 = stream_cache.decode_attn_fused(cache, q, one_launch=True, **kw)
+        assert torch.equal(o1, out), f"one-launch out differs from the two-launch result (call {rep})"
+        assert torch.equal(l1.view(torch.int32), lse.view(torch.int32)), f"one-launch lse differs (call {rep})"
+        assert int(cache.tickets.abs().max()) == 0, f"ticket counters not back at zero (call {rep})"
+    return out, lse

@@ -6,7 +6,7 @@ import torch
 
 from oracle import rdkv_oracle as O
 from rdkv_amd import _lib, packing, stream_cache, synth
-from tests.gpu_util import (DEV, attn_close, layer_to_device, layer_to_oracle, lse_merge, require_gpu, t2n,
+from tests.gpu_util import (DEV, attn_close, fused_both, layer_to_device, layer_to_oracle, lse_merge, require_gpu, t2n,
                             to_dev)
 from tests.helpers import golden_to_oracle_layer, load_golden
 from tests.stream_decode import decode_unit
@@ -96,20 +96,20 @@ def test_fused_attention_golden(name):
     nvo = g.get("new_v_only")
     cache = stream_cache.build_stream_cache(
         [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G)
-    out, lse = stream_cache.decode_attn_fused(cache, to_dev(g["q"]))
+    out, lse = fused_both(cache, to_dev(g["q"]))
     attn_close(t2n(out), g["out"], "out")
     _, exp_lse, _ = O.decode_attn_ref(g["q"], ora, nvo)
     attn_close(t2n(lse), exp_lse, "lse")
     # same result through a different work partition (every tile its own work item)
     cache1 = stream_cache.build_stream_cache(
         [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G, work_bytes=1)
-    out1, lse1 = stream_cache.decode_attn_fused(cache1, to_dev(g["q"]))
+    out1, lse1 = fused_both(cache1, to_dev(g["q"]))
     attn_close(t2n(out1), g["out"], "out(work_bytes=1)")
     # ... and with three workgroups that each walk several items across unit boundaries
     cache3 = stream_cache.build_stream_cache(
         [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G, n_groups=3)
     assert cache3.n_groups == 3 and cache3.n_work >= cache3.n_units
-    out3, lse3 = stream_cache.decode_attn_fused(cache3, to_dev(g["q"]))
+    out3, lse3 = fused_both(cache3, to_dev(g["q"]))
     attn_close(t2n(out3), g["out"], "out(n_groups=3)")
     attn_close(t2n(lse3), exp_lse, "lse(n_groups=3)")
     # run-to-run determinism
@@ -135,7 +135,7 @@ def _config_case(cfg, layers):
 @pytest.mark.parametrize("cfg_idx,ctx,layers", [(0, 4096, 1), (1, 3000, 2), (2, 2500, 1), (3, 1500, 2)])
 def test_fused_attention_config_shaped(cfg_idx, ctx, layers, partition):
     """C0 at its full size; C1/C2/C3 shapes (incl. GQA 8) at reduced context, several layers in
-    one launch; with the default balanced workgroups and with one workgroup per 64 KiB item, and with
+    one launch; with the default balanced workgroups, with one workgroup per 64 KiB item, and with
     three workgroups that each walk many items across unit boundaries."""
     cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=layers)
     packed, q, exp = _config_case(cfg, layers)
@@ -144,7 +144,7 @@ def test_fused_attention_config_shaped(cfg_idx, ctx, layers, partition):
     assert (cache.groups is not None) == (partition != "items")
     if partition == "few_groups":      # workgroups walk several units each
         assert cache.n_groups == 3 and np.diff(cache.groups_host).min() >= 3
-    out, lse = stream_cache.decode_attn_fused(cache, q)
+    out, lse = fused_both(cache, q)
     out, lse = t2n(out), t2n(lse)
     for layer, (eo, el, _) in enumerate(exp):
         rows = slice(layer * cfg.H_q, (layer + 1) * cfg.H_q)
@@ -161,7 +161,7 @@ def test_fused_zero_query_gives_token_mean():
     K, V, q = synth.layer_data(cfg, 0, DEV, outliers=oc)
     pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
     cache = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
-    out, lse = stream_cache.decode_attn_fused(cache, torch.zeros_like(q))
+    out, lse = fused_both(cache, torch.zeros_like(q))
     sb = pl.seg_bounds_per_head.cpu().tolist()
     n16 = pl.n_v16_per_head.cpu().tolist()
     for h in range(cfg.H_kv):
@@ -194,7 +194,7 @@ def test_fused_empty_unit_and_lse_merge():
     kb = torch.full((2, D), 8)
     pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, 2)
     cache = stream_cache.build_stream_cache([(pl, nvo)], 2)
-    out, lse = stream_cache.decode_attn_fused(cache, q)
+    out, lse = fused_both(cache, q)
     assert float(out[2:].abs().max()) == 0.0 and bool(torch.isinf(lse[2:]).all()) and bool((lse[2:] < 0).all())
     assert bool(torch.isfinite(out[:2]).all())
     # split head 0's tokens into two sources and merge
@@ -264,7 +264,7 @@ def test_fused_attention_full_size_layer(cfg_idx):
     pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
     del K, V
     cache = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
-    out, lse = stream_cache.decode_attn_fused(cache, q)
+    out, lse = fused_both(cache, q)
     exp_out, exp_lse, _ = O.decode_attn_ref(t2n(q), layer_to_oracle(pl), t2n(nvo) if nvo is not None else None)
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
@@ -292,7 +292,7 @@ def test_fused_attention_ragged_batch():
             del K, V
     cache = stream_cache.build_stream_cache(entries, cfg.G)
     assert cache.n_units == cfg.batch * cfg.layers * cfg.H_kv and cache.rows == len(entries) * cfg.H_q
-    out, lse = stream_cache.decode_attn_fused(cache, torch.cat(qs).contiguous())
+    out, lse = fused_both(cache, torch.cat(qs).contiguous())
     out, lse = t2n(out), t2n(lse)
     algo = 0
     for i, (pl, nvo) in enumerate(entries):
@@ -331,23 +331,33 @@ def test_fused_attention_k_row_shapes(counts):
     pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
     cache = stream_cache.build_stream_cache([(pl, nvo)], G)
     assert cache.max_row_dwords == sum(stream_cache.slot_plan(c2, c4, c8, -(-c2 // 4) * 4, -(-c4 // 2) * 2)[:3]) <= 32
-    out, lse = stream_cache.decode_attn_fused(cache, q.to(DEV))
+    out, lse = fused_both(cache, q.to(DEV))
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
 
 
 def test_stream_cache_file_round_trip(tmp_path):
-    """A cache written to disk and loaded again (at other addresses) gives the same bits."""
+    """A cache written to disk and loaded again (at other addresses): the oracle's results within
+    the attention tolerance and the live cache's bits; loaded with another work partition (what a
+    device with another number of compute units gets) still the oracle's results."""
     cfg = synth.scaled(synth.CONFIGS[1], context=1200, layers=3)
-    packed, q, _ = _config_case(cfg, 3)
+    packed, q, exp = _config_case(cfg, 3)
     cache = stream_cache.build_stream_cache(packed, cfg.G)
     out, lse = stream_cache.decode_attn_fused(cache, q)
     path = str(tmp_path / "cache.rdkv")
     stream_cache.save_stream_cache(cache, path)
     keep = [torch.empty(3_000_000, dtype=torch.uint8, device=DEV)]     # shift the allocator
+    del cache, packed
     loaded = stream_cache.load_stream_cache(path, DEV)
-    assert loaded.n_units == cache.n_units and loaded.n_work == cache.n_work and loaded.n_groups == cache.n_groups
-    assert loaded.algorithmic_bytes == cache.algorithmic_bytes
+    other = stream_cache.load_stream_cache(path, DEV, n_groups=5)
+    assert other.n_groups == 5 and loaded.n_groups != 5
+    for name, c in (("same partition", loaded), ("five workgroups", other)):
+        o, l = fused_both(c, q)
+        for layer, (eo, el, _) in enumerate(exp):
+            rows = slice(layer * cfg.H_q, (layer + 1) * cfg.H_q)
+            attn_close(t2n(o)[rows], eo, f"{name}: out layer {layer}")
+            attn_close(t2n(l)[rows], el, f"{name}: lse layer {layer}")
+        assert c.algorithmic_bytes == sum(e[2] for e in exp)
     out2, lse2 = stream_cache.decode_attn_fused(loaded, q)
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
     with pytest.raises(RuntimeError):
@@ -355,6 +365,12 @@ def test_stream_cache_file_round_trip(tmp_path):
     bad = tmp_path / "bad.rdkv"
     bad.write_bytes(b"not a cache file, just sixteen+ bytes")
     with pytest.raises(ValueError):
+        stream_cache.load_stream_cache(str(bad), DEV)
+    # one flipped bit in a blob: refused before anything reaches the device
+    raw = bytearray(open(path, "rb").read())
+    raw[len(raw) // 2] ^= 0x10
+    bad.write_bytes(bytes(raw))
+    with pytest.raises(ValueError, match="checksum"):
         stream_cache.load_stream_cache(str(bad), DEV)
     del keep
 
@@ -372,7 +388,7 @@ def test_multi_source_rows():
     cache = stream_cache.build_stream_cache(packed, cfg.G, row_of_entry=[0, 1, 0, 1])
     assert cache.rows == 2 * cfg.H_q and cache.n_units == 4 * cfg.H_kv
     assert int((cache.units_host["work_count"] == 0).sum()) == 2 * cfg.H_kv
-    out, lse = stream_cache.decode_attn_fused(cache, q)
+    out, lse = fused_both(cache, q)
     singles = [stream_cache.decode_attn_fused(stream_cache.build_stream_cache([packed[i]], cfg.G),
                                               q[(i % 2) * cfg.H_q:(i % 2 + 1) * cfg.H_q].contiguous())
                for i in range(4)]
