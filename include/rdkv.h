@@ -256,7 +256,12 @@ typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgro
                                (one fetch, where work -> unit would be two dependent ones)          */
   int32_t  merge_begin;     /* work_begin and work_count of units[merge_unit]                       */
   int32_t  merge_count;
-  int32_t  reserved[2];
+  float    k_scale_max;     /* largest K channel scale of the unit (the kernel bounds its q*scale
+                               operands with it and scales them by a power of two when they would
+                               leave the fp16 range)                                               */
+  int32_t  v_shift;         /* e >= 0: the quantized V classes' weights carry a further 2^-e, chosen
+                               so that (largest V scale of the unit) * 2^(6-e) < 2^15; 0 for V scales
+                               below 512                                                            */
 } RdkvWork;
 
 /* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.

@@ -33,11 +33,17 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kD = 128;
 constexpr int kPartialStride = 132;  // 128 acc + max + sum + 2 pad (floats, per head)
-// fixed-point style power-of-two scalings (all exact)
+// Fixed-point style power-of-two scalings (all exact).  The two operands that are rounded to fp16
+// after such a scaling keep below 2^15 for any input: an item whose largest |q * scale| (bounded by
+// max |q| over its heads times the unit's largest K scale) would pass it is scaled down by a further
+// power of two, found while the query is staged, and a unit whose largest V scale would pass it by
+// one the host stores with the work item; both are undone in fp32.  For ordinary magnitudes
+// (|q * scale| < 1000, V scales < 512) the extra powers are 2^0 and nothing changes.
 constexpr float kQScale = 256.0f;                  // q*scale is multiplied by 2^8 before fp16 rounding
 constexpr float kSBack = 65536.0f;                 // 2^(24-8): K-side accumulator -> score
-constexpr float kPScaleQ = 64.0f;                  // p*scale*2^6 for quantized classes
-constexpr float kOBackQ = 262144.0f;               // 2^(24-6)
+constexpr int kPScaleQLog2 = 6;                    // p*scale*2^6 for quantized classes
+constexpr int kOBackQLog2 = 24 - kPScaleQLog2;     // V-side accumulator -> output
+constexpr float kOperandLimit = 32768.0f;          // fp16 operands stay below this
 constexpr float kPScaleH = 16384.0f;               // p*2^14 for the fp16 class
 constexpr float kOBackH = 1.0f / 16384.0f;
 constexpr float kLog2eOverSqrtD = 0.12751743074602468f;  // log2(e)/sqrt(128)
@@ -225,6 +231,8 @@ struct Smem {
   alignas(16) _Float16 qs[kBatch][RDKV_MAX_STEPS][NH][2][4][4];  // [item][step][head group][hi|lo][head][k]
   alignas(16) _Float16 p[NW][16][NH][4][4];                      // [wave][quad][head group][head][k]
   float bias[kBatch][NH * 4];
+  float qmaxw[kBatch][NH * 4 * 2];                               // max |q| per 64 query elements (half a head)
+  float kup[kBatch];                                             // 2^e: the item's q*scale operands carry 2^-e
   float qraw[kBatch][NH * 4][kD];                                // the unit's query rows as loaded
   float slot_scale[kBatch][4 * RDKV_MAX_STEPS], slot_zp[kBatch][4 * RDKV_MAX_STEPS];
   uint16_t slot_channel[kBatch][4 * RDKV_MAX_STEPS];
@@ -255,6 +263,8 @@ struct Item {
   int tile_begin, tile_end, d8, d4, d2, R, NS, n0, n1, n2, n3, ts1, ts2, ts3, q_row;
   int nchunk_full, wc_last, nchunks;
   int merge_unit, merge_begin, merge_count;
+  int v_shift;          // the quantized classes' p*scale operand carries a further 2^-v_shift
+  float k_scale_max;    // largest K channel scale of the unit
   const uint8_t *k_base, *sz_base, *v_base0, *v_base1, *v_base2, *v_base3, *qtab_base;
 };
 
@@ -293,6 +303,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
     const RdkvUnit *up = &wkp->u;    // the unit's descriptor travels with the work item
     Item it;
     it.merge_unit = wkp->merge_unit; it.merge_begin = wkp->merge_begin; it.merge_count = wkp->merge_count;
+    it.v_shift = wkp->v_shift; it.k_scale_max = wkp->k_scale_max;
     it.tile_begin = wkp->tile_begin;
     it.tile_end = wkp->tile_end;
     it.d8 = up->d8; it.d4 = up->d4; it.d2 = up->d2;
@@ -460,12 +471,24 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
           v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
         }
         sm.qraw[b][i >> 7][c] = v;
+        // (a wavefront holds 64 consecutive elements of one head: uniform branch, whole-wave maximum)
+        const float am = rdkv_wave_max(fabsf(v));
+        if (lane_o == 0) sm.qmaxw[b][i >> 6] = am;
       }
     }
   }
   __syncthreads();
   for (int b = 0; b < nb; ++b) {
-    const int nslot = 4 * load_item(batch + b).NS;
+    const Item ib = load_item(batch + b);
+    const int nslot = 4 * ib.NS;
+    // the item's power of two: 2^-e brings the largest possible |q * scale * 2^8| below 2^15
+    float qm = 0.0f;
+    for (int w2 = 0; w2 < 2 * G; ++w2) qm = fmaxf(qm, sm.qmaxw[b][w2]);
+    const float bound = qm * ib.k_scale_max * (kLog2eOverSqrtD * kQScale);
+    int e = (int)((__float_as_uint(bound) >> 23) & 0xffu) - 127 - 14;
+    e = bound < kOperandLimit ? 0 : (e > 100 ? 100 : e);
+    const float down = __uint_as_float((uint32_t)(127 - e) << 23);
+    if (tid_o == 0) sm.kup[b] = __uint_as_float((uint32_t)(127 + e) << 23);
     for (int i = tid_o; i < nslot * NH * 4; i += kThreads) {
       const int slot = i % nslot, head = i / nslot;
       _Float16 hi = (_Float16)0.0f, lo = (_Float16)0.0f;
@@ -473,7 +496,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         // two fp16 terms carry ~22 bits of q*scale: one fp16 alone loses the outlier channels'
         // low bits and costs ~1e-3 in the scores
         const float x = sm.qraw[b][head][sm.slot_channel[b][slot]] * sm.slot_scale[b][slot] *
-                        (kLog2eOverSqrtD * kQScale);
+                        (kLog2eOverSqrtD * kQScale) * down;
         hi = (_Float16)x;
         lo = (_Float16)(x - (float)hi);
       }
@@ -491,7 +514,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
       bsum += ((float)sm.qs[b][slot >> 2][head >> 2][0][head & 3][slot & 3] +
                (float)sm.qs[b][slot >> 2][head >> 2][1][head & 3][slot & 3]) * sm.slot_zp[b][slot];
     bsum = rdkv_wave_sum(bsum);
-    if (lane_o == 0) sm.bias[b][head] = bsum * (1.0f / kQScale);
+    if (lane_o == 0) sm.bias[b][head] = bsum * (1.0f / kQScale) * sm.kup[b];
   }
   __syncthreads();
 
@@ -519,6 +542,12 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
       accq[hg][j] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
   }
+  // the item's powers of two (wave-uniform)
+  const float sback = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(
+      __builtin_bit_cast(int, kSBack * sm.kup[b])));
+  // (the V-side powers of two are formed from the item's v_shift where they are used: two scalar
+  // instructions each, instead of three more scalars that stay live across the tile loop)
+  auto pow2 = [&](int e) __attribute__((always_inline)) { return __uint_as_float((uint32_t)(127 + e) << 23); };
   const _Float16 *qs_item = &sm.qs[b][0][0][0][0][0];
   auto qs_op = [&](int step, int hg, int part) -> const _Float16 * {
     return qs_item + (((step * NH + hg) * 2 + part) * 4 + ln) * 4;
@@ -626,7 +655,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
       for (int hg = 0; hg < NH; ++hg) sacc[hg] += sacc_lo[hg];
       // ---- online softmax (base-2 domain) --------------------------------------------------
       const int n_valid = c.n_valid;
-      const float pscale = c.cls < 3 ? kPScaleQ : kPScaleH;
+      const float pscale = c.cls < 3 ? pow2(kPScaleQLog2 - it.v_shift) : kPScaleH;
       float sc4[4], zp4[4];
       {
         const uint32_t szw[4] = {ksz.x, ksz.y, ksz.z, ksz.w};
@@ -646,7 +675,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          float sv = sacc[hg][j] * kSBack - bias_own[hg];
+          float sv = sacc[hg][j] * sback - bias_own[hg];
           sv = (4 * lb + j < n_valid) ? sv : -INFINITY;
           s2[hg][j] = sv;
           mx = fmaxf(mx, sv);
@@ -745,7 +774,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
 #pragma unroll
         for (int hg = 0; hg < NH; ++hg)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) accq[hg][j] *= kOBackQ / kOBackH;
+          for (int j = 0; j < 2; ++j) accq[hg][j] *= pow2(kOBackQLog2 + it.v_shift + 14);   // / kOBackH = * 2^14
       }
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
@@ -778,7 +807,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
 #pragma unroll
   for (int hg = 0; hg < NH; ++hg) {
     const float l_tot = quadcol_sum(l_run[hg]);
-    const float zb_tot = quadcol_sum(zb_run[hg]) * (1.0f / kPScaleQ);
+    const float zb_tot = quadcol_sum(zb_run[hg]) * pow2(it.v_shift - kPScaleQLog2);
     if (lane_o < 4) {
       sm.wm[b][wave][hg * 4 + lane_o] = m_run[hg];
       sm.wl[b][wave][hg * 4 + lane_o] = l_tot;
@@ -788,7 +817,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
       const float zb = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, zb_tot), r));
 #pragma unroll
       for (int j = 0; j < 2; ++j)
-        sm.wo[b][wave][hg * 4 + r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : kOBackQ) - zb;
+        sm.wo[b][wave][hg * 4 + r][lane_o + 64 * j] = accq[hg][j][r] * (acc_fp16 ? kOBackH : pow2(kOBackQLog2 + it.v_shift)) - zb;
     }
   }
   // straight on to the next item of the batch: its first loads go out now

@@ -38,7 +38,7 @@ SLOT_DTYPE = np.dtype([("channel", "<u2"), ("scale", "<u2"), ("zp", "<u2"), ("re
 # A work item carries a copy of its unit's descriptor (the kernel reads it with the item, one fetch
 # instead of two dependent ones) and the partial range of the output row it belongs to.
 WORK_DTYPE = np.dtype([("unit", "<i4"), ("tile_begin", "<i4"), ("tile_end", "<i4"), ("merge_unit", "<i4"),
-                       ("u", UNIT_DTYPE), ("merge_begin", "<i4"), ("merge_count", "<i4"), ("reserved", "<i4", (2,))])
+                       ("u", UNIT_DTYPE), ("merge_begin", "<i4"), ("merge_count", "<i4"), ("k_scale_max", "<f4"), ("v_shift", "<i4")])
 assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.itemsize == 128
 
 
@@ -103,6 +103,7 @@ class StreamCache:
     h_q: int = 0                         # query heads per output group
     tickets: Optional[torch.Tensor] = None  # device int32 [n_units], zero between calls (one-launch form)
     partition: Optional[dict] = None     # the work-partition arguments the cache was built with
+    unit_scale_max: Optional[np.ndarray] = None   # fp32 [n_units, 2]: largest K channel scale, largest V token scale
 
     @property
     def device(self):
@@ -223,7 +224,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
     lib = _lib.load()
     dev = _lib.require_device(layers[0][0].K_ch_scale)
     stream = _lib.stream_of(dev)
-    units_all, blobs, keep_alive = [], [], []
+    units_all, blobs, keep_alive, scale_max = [], [], [], []
     stream_bytes = algo_bytes = 0
     H_q = None
     for gi, (pl, nvo) in enumerate(layers):
@@ -295,6 +296,11 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         kz = pl.K_ch_zp.reshape(H_kv, Dp)
         if ks.stride(1) != 1 or kz.stride() != ks.stride():
             ks, kz = ks.contiguous(), kz.contiguous()
+        # per head: the largest K channel scale and the largest V token scale (the kernel keeps its
+        # fp16 operands in range with them)
+        zero = torch.zeros(H_kv, dtype=torch.float32, device=dev)
+        scale_max.append(torch.stack([ks.float().abs().amax(dim=1) if Dp else zero,
+                                      vs.float().abs().amax(dim=1) if vs.numel() else zero], dim=1))
         if pl.K_ch_perm_padded_idx_per_head is not None:
             perm = pl.K_ch_perm_padded_idx_per_head.to(torch.int64).contiguous()
             perm_sh = perm.stride(0)
@@ -319,19 +325,30 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
         # the temporaries stay alive until the relayout kernels have run
         keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
+    scale_max_np = torch.cat(scale_max).cpu().numpy().astype(np.float32)   # (synchronizes)
     torch.cuda.current_stream(dev).synchronize()
     del keep_alive
-    return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q
+    return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
 
 
-def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: int, kv_algo_bytes: int, *,
-                  multi_source: bool, work_bytes, n_groups, groups_per_cu: int, cost) -> StreamCache:
+def v_shift_of(v_scale_max: np.ndarray) -> np.ndarray:
+    """Power of two the fused kernel takes out of the quantized V classes' weights: the smallest
+    e >= 0 with v_scale_max * 2^(6 - e) < 2^15 (0 for scales below 512)."""
+    v = np.nan_to_num(np.asarray(v_scale_max, dtype=np.float64), nan=0.0, posinf=2.0 ** 40)
+    _, ex = np.frexp(np.maximum(v, 0.0))          # v = m * 2^ex, 0.5 <= m < 1
+    return np.clip(ex - 9, 0, 40).astype(np.int32)
+
+
+def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: int, kv_algo_bytes: int,
+                  scale_max: np.ndarray, *, multi_source: bool, work_bytes, n_groups, groups_per_cu: int,
+                  cost) -> StreamCache:
     """Order the units, cut the tile stream into work items and groups, upload the tables."""
     dev = blobs[0].device
     n_groups_arg, cost_arg = n_groups, cost
     if multi_source:
         # sources of one output row next to each other, so that their work items are contiguous
-        units_np = units_np[np.argsort(units_np["q_row"], kind="stable")]
+        order = np.argsort(units_np["q_row"], kind="stable")
+        units_np, scale_max = units_np[order], scale_max[order]
     tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
     R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
     if work_bytes is None and n_groups is None:
@@ -362,6 +379,8 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
         work_np["merge_unit"] = merger[iu]
         work_np["merge_begin"] = wb[merger[iu]]
         work_np["merge_count"] = wc[merger[iu]]
+        work_np["k_scale_max"] = scale_max[iu, 0]
+        work_np["v_shift"] = v_shift_of(scale_max[:, 1])[iu]
     rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
     units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
     work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
@@ -369,7 +388,7 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
     groups_dev = torch.from_numpy(groups_np).to(dev) if groups_np is not None else None
     return StreamCache(tickets=torch.zeros(max(1, len(units_np)), dtype=torch.int32, device=dev),
                        partition={"work_bytes": work_bytes, "n_groups": n_groups_arg, "groups_per_cu": groups_per_cu,
-                                  "cost": cost_arg},
+                                  "cost": cost_arg}, unit_scale_max=scale_max,
                        blobs=list(blobs), units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
                        n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
                        stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
@@ -401,8 +420,8 @@ def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tens
     tiles each."""
     rows_of_entries = list(range(len(layers))) if row_of_entry is None else [int(r) for r in row_of_entry]
     assert len(rows_of_entries) == len(layers)
-    units_np, blobs, stream_bytes, kv_algo, H_q = _relayout_entries(layers, G, rows_of_entries)
-    return _finish_cache(units_np, blobs, G, H_q, stream_bytes, kv_algo, multi_source=row_of_entry is not None,
+    units_np, blobs, stream_bytes, kv_algo, H_q, scale_max = _relayout_entries(layers, G, rows_of_entries)
+    return _finish_cache(units_np, blobs, G, H_q, stream_bytes, kv_algo, scale_max, multi_source=row_of_entry is not None,
                          work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
 
 
@@ -417,11 +436,12 @@ def extend_stream_cache(cache: StreamCache, layers: Sequence[Tuple[PackedKVLayer
     pre-allocated slot of its bank instead, blockwise_decode.py:336-355)."""
     rows_of_entries = [int(r) for r in row_of_entry]
     assert len(rows_of_entries) == len(layers) and len(layers) > 0
-    new_units, new_blobs, sb, ab, H_q = _relayout_entries(layers, cache.G, rows_of_entries)
+    new_units, new_blobs, sb, ab, H_q, new_scale_max = _relayout_entries(layers, cache.G, rows_of_entries)
     assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
     old = cache.units_host.copy()
     return _finish_cache(np.concatenate([old, new_units]), list(cache.blobs) + new_blobs, cache.G, H_q,
-                         cache.stream_bytes + sb, cache.kv_algorithmic_bytes + ab, multi_source=True,
+                         cache.stream_bytes + sb, cache.kv_algorithmic_bytes + ab,
+                         np.concatenate([cache.unit_scale_max, new_scale_max]), multi_source=True,
                          work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
 
 
@@ -434,14 +454,16 @@ def extend_stream_caches(caches: Sequence[StreamCache],
     G = caches[0].G
     assert all(c.G == G for c in caches)
     per_entry: list = []
-    new_units, new_blobs, _, _, H_q = _relayout_entries(layers, G, [0] * len(layers), per_entry)
+    new_units, new_blobs, _, _, H_q, new_scale_max = _relayout_entries(layers, G, [0] * len(layers), per_entry)
     n_per = len(new_units) // len(layers)
     out = []
     for i, cache in enumerate(caches):
         assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
         units = np.concatenate([cache.units_host.copy(), new_units[i * n_per:(i + 1) * n_per]])
         out.append(_finish_cache(units, list(cache.blobs) + [new_blobs[i]], G, H_q, cache.stream_bytes + per_entry[i][0],
-                                 cache.kv_algorithmic_bytes + per_entry[i][1], multi_source=True, work_bytes=None,
+                                 cache.kv_algorithmic_bytes + per_entry[i][1],
+                                 np.concatenate([cache.unit_scale_max, new_scale_max[i * n_per:(i + 1) * n_per]]),
+                                 multi_source=True, work_bytes=None,
                                  n_groups=None, groups_per_cu=1, cost=None))
     return out
 
@@ -656,7 +678,8 @@ def save_stream_cache(cache: StreamCache, path: str) -> None:
         for f in _ADDR_FIELDS:
             units[f][i] -= bases[j]
         units["v_off"][i] -= bases[j]
-    parts = [("units", units.view(np.uint8).reshape(-1)), ("blob_of", blob_of.view(np.uint8))]
+    parts = [("units", units.view(np.uint8).reshape(-1)), ("blob_of", blob_of.view(np.uint8)),
+             ("scale_max", np.ascontiguousarray(cache.unit_scale_max, dtype="<f4").view(np.uint8).reshape(-1))]
     part = dict(cache.partition or {})
     if part.get("cost") is not None:
         part["cost"] = {k: list(v) if isinstance(v, (tuple, list)) else v for k, v in part["cost"].items()}
@@ -692,7 +715,8 @@ def save_stream_cache(cache: StreamCache, path: str) -> None:
 
 def read_stream_cache_file(path: str, verify: bool = True):
     """Host side of ``load_stream_cache``: parse and check ``path`` without touching a device.
-    Returns (header, units with blob-relative offsets, blob_of, [memory-mapped blob bytes]).
+    Returns (header, units with blob-relative offsets, blob_of, [memory-mapped blob bytes], largest
+    K / V scale per unit).
     Raises ValueError for a file that is not a streaming cache, has another format version, is
     truncated, fails a checksum (``verify``) or describes regions outside its blobs."""
     import json
@@ -728,14 +752,17 @@ def read_stream_cache_file(path: str, verify: bool = True):
 
     units = np.frombuffer(extent("units", *header["sections"]["units"]), dtype=UNIT_DTYPE).copy()
     blob_of = np.frombuffer(extent("blob_of", *header["sections"]["blob_of"]), dtype=np.int32).copy()
+    scale_max = np.frombuffer(extent("scale_max", *header["sections"]["scale_max"]), dtype="<f4").copy()
     if len(units) != header["n_units"]:
         raise ValueError(f"{path}: {len(units)} units in the table, header says {header['n_units']}")
+    if scale_max.size != 2 * len(units) or not (scale_max >= 0).all():       # (a NaN fails the comparison)
+        raise ValueError(f"{path}: the table of largest scales does not fit the {len(units)} units")
     blobs = [extent(f"blob {j}", o, n, crc) for j, (o, n, crc) in enumerate(header["blobs"])]
     validate_units(units, blob_of, [len(b) for b in blobs], header["G"], header["rows"], what=path)
     R = units["d8"] + units["d4"] + units["d2"]
     if len(units) and int(R.max()) > header["max_row_dwords"]:
         raise ValueError(f"{path}: max_row_dwords={header['max_row_dwords']} below the longest K row {int(R.max())}")
-    return header, units, blob_of, blobs
+    return header, units, blob_of, blobs, scale_max.reshape(-1, 2)
 
 
 def load_stream_cache(path: str, device, verify: bool = True, **partition) -> StreamCache:
@@ -747,7 +774,7 @@ def load_stream_cache(path: str, device, verify: bool = True, **partition) -> St
     dev = torch.device(device)
     if dev.type != "cuda":
         raise RuntimeError("rdkv HIP backend needs a HIP device; there is no CPU fallback")
-    header, units, blob_of, blob_views = read_stream_cache_file(path, verify=verify)
+    header, units, blob_of, blob_views, scale_max = read_stream_cache_file(path, verify=verify)
     _lib.load()
     blobs = []
     for view in blob_views:
@@ -767,6 +794,6 @@ def load_stream_cache(path: str, device, verify: bool = True, **partition) -> St
     if cost is not None:
         cost = {k: tuple(v) if isinstance(v, list) else v for k, v in cost.items()}
     return _finish_cache(units, blobs, header["G"], header["h_q"], header["stream_bytes"],
-                         header["kv_algorithmic_bytes"], multi_source=header["multi_source"],
+                         header["kv_algorithmic_bytes"], scale_max, multi_source=header["multi_source"],
                          work_bytes=part.get("work_bytes"), n_groups=part.get("n_groups"),
                          groups_per_cu=part.get("groups_per_cu", 1), cost=cost)

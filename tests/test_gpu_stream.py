@@ -336,6 +336,61 @@ def test_fused_attention_k_row_shapes(counts):
     attn_close(t2n(lse), exp_lse, "lse")
 
 
+@pytest.mark.parametrize("k_mul,v_mul,q_mul,widths,G", [
+    (16.0, 1.0, 1.0, "mixed", 4), (64.0, 1.0, 1.0, "mixed", 4), (1.0, 16.0, 1.0, "mixed", 4),
+    (1.0, 64.0, 1.0, "mixed", 4), (1.0, 1.0, 64.0, "mixed", 4), (64.0, 64.0, 1.0, "two_bit", 4),
+    (16.0, 64.0, 8.0, "two_bit", 8), (1.0, 1.0, 1e-3, "mixed", 4), (1e-3, 1e-3, 1.0, "two_bit", 4)])
+def test_fused_attention_magnitude_sweep(k_mul, v_mul, q_mul, widths, G):
+    """Keys, values and queries far outside N(0,1) - K and V scaled by 16 and 64 on top of outlier
+    channels / tokens (|K| up to ~2000, V scales of the 2-bit class above 1000), queries by 64, and
+    the same scaled down by 1000; mixed widths and everything 2 bit (the largest scales): the
+    kernel's fp16 operands stay in range (no inf / NaN) and the results follow the oracle.  The
+    dequantize-then-attend oracle rounds the dequantized K and V to fp16, an error that grows with
+    the scores (0.05 in lse at |score| ~ 500), so the comparison here is first with its un-rounded
+    form (K and V dequantized in fp32: the arithmetic of the reference's packed kernels) at 2e-3 of
+    the largest reference value for out and 2e-3 + 1e-4 relative for lse (the kernel forms a score
+    as sum(code * q') - sum(zp * q'), two sums about twenty times the score: 2^-15 relative, where
+    the fp32 dot product of dequantized values has 2^-20), then with the rounded form at the looser
+    2e-2 for out / 2e-3 times the magnitudes for lse."""
+    H_kv, T, D = 2, 700, 128
+    seed = int(k_mul * 7 + v_mul * 13 + q_mul * 1000) + G
+    g = torch.Generator().manual_seed(seed)
+    rng = np.random.default_rng(seed)
+    K = torch.randn(1, H_kv, T, D, generator=g)
+    K[..., rng.choice(D, 4, replace=False)] *= 8.0                    # outlier channels
+    V = torch.randn(1, H_kv, T, D, generator=g)
+    V[:, :, rng.choice(T, 20, replace=False)] *= 8.0                  # outlier tokens
+    K, V = (K * k_mul).half(), (V * v_mul).half()
+    q = (torch.randn(H_kv * G, D, generator=g) * q_mul).half()
+    assert torch.isfinite(K).all() and torch.isfinite(V).all() and torch.isfinite(q).all()
+    if widths == "two_bit":
+        vb = torch.full((H_kv, T), 2, dtype=torch.int64)
+        kb = torch.full((H_kv, D), 2, dtype=torch.int64)
+    else:
+        vb = torch.from_numpy(rng.choice(np.array([2, 4, 8, 16]), size=(H_kv, T)))
+        kb = torch.from_numpy(rng.choice(np.array([2, 4, 8]), size=(H_kv, D)))
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+    exp_out, exp_lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+    assert np.isfinite(exp_out).all() and np.isfinite(exp_lse).all()
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
+    cache = stream_cache.build_stream_cache([(pl, nvo)], G)
+    if v_mul >= 64.0 and widths == "two_bit":
+        assert cache.work_host["v_shift"].max() >= 1, "this case is meant to exceed the fixed V-side scaling"
+    out, lse = fused_both(cache, q.to(DEV))
+    out, lse = t2n(out), t2n(lse)
+    assert np.isfinite(out).all() and np.isfinite(lse).all()
+    x_out, x_lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo, round_fp16=False)
+    ref = float(np.abs(x_out).max())
+    err = float(np.abs(out - x_out).max())
+    assert err <= 2e-3 * ref, f"out: max-abs error {err:.3e} against a largest reference value of {ref:.3e}"
+    lerr = np.abs(lse - x_lse)
+    assert (lerr <= 2e-3 + 1e-4 * np.abs(x_lse)).all(), f"lse: error {lerr.max():.3e}"
+    err = float(np.abs(out - exp_out).max())
+    assert err <= 2e-2 * ref, f"out against the fp16-rounded oracle: max-abs error {err:.3e}, reference {ref:.3e}"
+    lerr = np.abs(lse - exp_lse)
+    assert (lerr <= 2e-3 * max(1.0, k_mul * q_mul) + 1e-4 * np.abs(exp_lse)).all(), f"lse: error {lerr.max():.3e}"
+
+
 def test_stream_cache_file_round_trip(tmp_path):
     """A cache written to disk and loaded again (at other addresses): the oracle's results within
     the attention tolerance and the live cache's bits; loaded with another work partition (what a

@@ -157,6 +157,18 @@ def test_partition_work_groups_and_items(seed):
             assert len(work) == U
 
 
+def test_v_shift_keeps_the_weight_operand_in_range():
+    """v_shift is the smallest e >= 0 with v_scale_max * 2^(6 - e) < 2^15: zero up to scales of
+    512, and finite for inf / NaN scales."""
+    from rdkv_amd.stream_cache import v_shift_of
+    v = np.asarray([0.0, 1e-8, 1.0, 511.9, 512.0, 1023.0, 1024.0, 1333.0, 65504.0, np.inf, np.nan], dtype=np.float32)
+    e = v_shift_of(v)
+    assert e.tolist() == [0, 0, 0, 0, 1, 1, 2, 2, 7, 32, 0]
+    fin = np.isfinite(v)
+    assert (v[fin].astype(np.float64) * 2.0 ** (6 - e[fin]) < 2 ** 15).all()
+    assert ((e[fin] == 0) | (v[fin].astype(np.float64) * 2.0 ** (7 - e[fin]) >= 2 ** 15)).all()
+
+
 def test_partition_work_all_empty():
     from rdkv_amd.stream_cache import partition_work
     tiles = np.zeros((3, 4), dtype=np.int64)

@@ -60,8 +60,13 @@ def _check_attention(g, pl, nvo, D):
     Tk = pl.T_eff_k if pl.T_eff_k > 0 else pl.T_eff
     K_hat = O.unpack_k_mixed(pl, D=D)
     assert np.array_equal(K_hat.view(np.uint16), g["K_hat"].view(np.uint16))
+    # the un-rounded form differs from the reference's K_hat by that one rounding to fp16 only
+    K32 = O.unpack_k_mixed(pl, D=D, round_fp16=False)
+    assert K32.dtype == np.float32 and np.array_equal(K32.astype(np.float16).view(np.uint16), g["K_hat"].view(np.uint16))
     s = O.k_mixed_qk_dot_ref(q, pl, Tk, D)
     np.testing.assert_allclose(s, g["scores"], rtol=0, atol=2e-6)
+    out32, lse32, _ = O.decode_attn_ref(q, pl, nvo, D, round_fp16=False)
+    np.testing.assert_allclose(out32, g["out"], rtol=0, atol=2e-3)
     out, lse, w = O.decode_attn_ref(q, pl, nvo, D)
     np.testing.assert_allclose(w, g["weights"], rtol=0, atol=1e-6)
     np.testing.assert_allclose(out, g["out"], rtol=0, atol=2e-6)

@@ -40,6 +40,7 @@ def _fake_cache(n_units=3, G=4, seed=0):
                           work_host=np.zeros(0, dtype=sc.WORK_DTYPE), n_units=n_units, n_work=0, G=G,
                           rows=n_units * G, stream_bytes=off, algorithmic_bytes=off, max_row_dwords=9,
                           kv_algorithmic_bytes=off, h_q=n_units * G,
+                          unit_scale_max=rng.random((n_units, 2)).astype(np.float32),
                           partition={"work_bytes": None, "n_groups": 7, "groups_per_cu": 1,
                                      "cost": dict(sc.DEFAULT_COST)})
 
@@ -61,7 +62,8 @@ def test_file_reads_back_what_was_written(tmp_path):
     cache = _fake_cache()
     path = str(tmp_path / "c.rdkv")
     sc.save_stream_cache(cache, path)
-    header, units, blob_of, blobs = sc.read_stream_cache_file(path)
+    header, units, blob_of, blobs, scale_max = sc.read_stream_cache_file(path)
+    assert np.array_equal(scale_max, cache.unit_scale_max)
     assert header["version"] == 2 and header["byteorder"] == "little" and header["n_units"] == 3
     assert header["partition"]["n_groups"] == 7 and header["partition"]["cost"]["item"] == sc.DEFAULT_COST["item"]
     assert list(blob_of) == [0, 0, 0] and len(blobs) == 1
@@ -72,7 +74,7 @@ def test_file_reads_back_what_was_written(tmp_path):
     assert (units["n_tok"] == cache.units_host["n_tok"]).all()
     assert np.array_equal(np.asarray(blobs[0]), cache.blobs[0].numpy())
     # nothing device-specific is stored: no work items, no groups
-    assert set(header["sections"]) == {"units", "blob_of"}
+    assert set(header["sections"]) == {"units", "blob_of", "scale_max"}
 
 
 def test_truncated_and_corrupt_files_are_refused(tmp_path):
