@@ -16,7 +16,8 @@ import torch
 from torch import Tensor
 
 from . import _lib
-from .knapsack_solver import knapsack_allocate, knapsack_bit_allocation_batched
+from .knapsack_solver import (DEFAULT_EPSILON_K, DEFAULT_EPSILON_V, knapsack_allocate,   # noqa: F401 (re-exported
+                              knapsack_bit_allocation_batched, load_epsilon_kv_from_calibration)  # as obkv_fast.py:38-46 does)
 from .packing import pack_layer_per_head, pack_layers_per_head
 
 

@@ -36,3 +36,15 @@ def fused_rope(q: torch.Tensor, k: torch.Tensor, cos_half: torch.Tensor, sin_hal
         _lib.ptr(q), q.stride(0), H_q, _lib.ptr(k), k.stride(0), H_kv, D, _lib.DTYPE_CODE[q.dtype],
         cos_half.data_ptr(), sin_half.data_ptr(), _lib.DTYPE_CODE[cos_half.dtype], _lib.stream_of(dev)))
     return q, k
+
+
+def fused_rope_ref(q: torch.Tensor, k: torch.Tensor, cos_half: torch.Tensor, sin_half: torch.Tensor):
+    """The rotation of ``fused_rope`` as tensor expressions, not in place (triton_rope.py:113-136):
+    fp32 products and sums, one rounding back to the input type; returns new (q, k).  Runs where its
+    inputs live (it is the check for ``fused_rope``, not a kernel path)."""
+    def rotate(x):
+        lo, hi = x[:, :HALF_D].float(), x[:, HALF_D:].float()
+        c, s = cos_half.float(), sin_half.float()
+        return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1).to(x.dtype)
+
+    return rotate(q), rotate(k)
