@@ -161,14 +161,21 @@ def stream_of(dev: torch.device) -> int:
 
 
 _workspaces = {}
+_retired_workspaces = []
 
 
 def workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     """Per (device, stream) scratch buffer, grown on demand and then reused so that
-    steady-state calls (and HIP-graph capture after a warm-up call) never allocate."""
+    steady-state calls (and HIP-graph capture after a warm-up call) never allocate.  A buffer
+    that is outgrown is kept alive, not freed: a HIP graph captured earlier on that stream has its
+    address baked in, and its replays must not write into memory another tensor has since been
+    given.  (Growth is by doubling, so the retired buffers add up to less than the live one.)"""
     key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=dev)
+        if buf is not None:
+            _retired_workspaces.append(buf)
+        grown = 2 * buf.numel() if buf is not None else 0
+        buf = torch.empty(max(int(nbytes), grown, 1 << 20), dtype=torch.uint8, device=dev)
         _workspaces[key] = buf
     return buf

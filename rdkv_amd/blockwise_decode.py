@@ -24,7 +24,10 @@ from torch import Tensor
 
 from . import _lib
 from .fast_decode import _pre_squeeze_packed
-from .packing import PackedKVLayer, TriZoneCache, _seg_padded_len
+from .k_kernel import k_mixed_qk_dot
+from .packing import PackedKVLayer, TriZoneCache, _seg_padded_len, unpack_k_mixed
+from .trizone_decompress import _unpack_v_perhead
+from .v_kernel import _get_v16_dummy, v_dequant_weighted_sum_dispatch
 
 
 @dataclass(frozen=True)
@@ -341,6 +344,38 @@ def _logical_layer_bits(packed, head_dim: int) -> int:
     return int(_logical_layer_bits_tensor(packed, head_dim).item())
 
 
+def _validate_packed_layer_reference(packed: PackedKVLayer, squeezed: PackedKVLayer, new_v_only: Optional[Tensor],
+                                     query: Tensor, *, num_kv_groups: int, head_dim: int) -> None:
+    """blockwise_decode.py:681-753.  The packed K and V kernels against explicit dequantization of
+    the same block, at the reference's tolerances: scores of ``query`` [H_q, D] over the block's
+    keys (2e-2 / 2e-2) and the uniformly weighted value sum over its kept tokens (3e-2 / 3e-2).
+    The dequantizers are the HIP ones (``unpack_k_mixed``, ``_unpack_v_perhead``); the comparison
+    itself is tensor expressions on the device, as in the reference."""
+    t_eff_k = squeezed.T_eff_k if squeezed.T_eff_k > 0 else squeezed.T_eff
+    if t_eff_k == 0:
+        return
+    q = query.float()
+    actual_k = k_mixed_qk_dot(q, squeezed, t_eff_k)
+    unpacked_k = unpack_k_mixed(packed, D=head_dim)[0].float()
+    expected_k = torch.einsum("hd,htd->ht", q, unpacked_k.repeat_interleave(num_kv_groups, dim=0)) / (head_dim ** 0.5)
+    torch.testing.assert_close(actual_k, expected_k, rtol=2e-2, atol=2e-2,
+                               msg="packed K block diverges from explicit dequantization")
+    v_zone_a = _unpack_v_perhead(packed, head_dim=head_dim)[0].float()
+    unpacked_v = torch.cat([v_zone_a, new_v_only[0].float()], dim=1) if new_v_only is not None else v_zone_a
+    logits = torch.zeros(q.shape[0], t_eff_k, dtype=torch.float32, device=q.device)
+    if squeezed.softmax_mask is not None:
+        logits.add_(squeezed.softmax_mask)
+    weights = torch.softmax(logits, dim=-1)
+    dummy_v, zero_counts = _get_v16_dummy(q.device, unpacked_v.shape[0])
+    actual_v = v_dequant_weighted_sum_dispatch(
+        weights, squeezed, V16=new_v_only[0].contiguous() if new_v_only is not None else dummy_v,
+        n_v16_per_head=squeezed.n_v16_per_head if squeezed.n_v16_per_head is not None else zero_counts,
+        max_T_v=squeezed.T_eff)
+    expected_v = (weights.view(unpacked_v.shape[0], num_kv_groups, t_eff_k) @ unpacked_v).reshape(q.shape[0], head_dim)
+    torch.testing.assert_close(actual_v, expected_v, rtol=3e-2, atol=3e-2,
+                               msg="packed V block diverges from explicit dequantization")
+
+
 def _rows(x: Tensor) -> Tensor:
     if x.dtype not in _lib.DTYPE_CODE:
         x = x.float()
@@ -452,6 +487,14 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     t_meta = _sync_stamp(target_kv[0].device) if timing_on else 0.0
     packed_tuple = tuple(packed_layers)
     squeezed = _pre_squeeze_packed(packed_tuple)
+    if config.correctness_check:
+        for layer_idx, (packed, packed_squeezed, v16, queries) in enumerate(
+                zip(packed_layers, squeezed, v16_layers, query_block)):
+            try:
+                _validate_packed_layer_reference(packed, packed_squeezed, v16, queries[:, -1, :],
+                                                 num_kv_groups=num_kv_groups, head_dim=head_dim)
+            except Exception as error:
+                raise AssertionError(f"packed reference check failed at layer {layer_idx}") from error
     physical_bytes = _tensor_storage_bytes((packed_tuple, v16_layers))
     t_end = _sync_stamp(target_kv[0].device)
     if timing_on:

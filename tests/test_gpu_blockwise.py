@@ -246,3 +246,28 @@ def test_decode_over_prompt_cache_compressed_blocks_and_raw_tail():
             exp[h * G + g] = (w / w.sum()) @ Vall
     err = float(np.abs(t2n(got) - exp).max())
     assert err <= 2e-3 and err <= 1e-2 * float(np.abs(exp).max()), err
+
+
+def test_run_time_check_of_a_packed_block_against_explicit_dequantization():
+    """``correctness_check`` of the blockwise loop (blockwise_decode.py:681-753, 964-980): the packed
+    K and V kernels on a freshly compressed block agree with explicit dequantization at the
+    reference's tolerances; a block whose squeezed view does not describe the packed tensors (K
+    scales off by half, V zero-points moved) is caught, and ``_compress_block`` reports the layer."""
+    import dataclasses
+    L, H, G, T, D = 2, 2, 4, 64, 128
+    kv, queries, scores = _block_inputs(11, L, H, G, T, D)
+    config = _config(T, 16)
+    assert config.correctness_check
+    block, _ = bw._compress_block(
+        target_kv=kv, query_block=queries, token_scores_by_layer=scores, block_id=0, token_start=0, token_end=T - 1,
+        query_source_block=1, is_final_flush=False, causal=False, config=config, num_kv_groups=G,
+        model_dtype=torch.float16)
+    q_last = queries[0][:, -1, :]
+    packed, squeezed, v16 = block.packed[0], block.squeezed[0], block.new_v_only[0]
+    bw._validate_packed_layer_reference(packed, squeezed, v16, q_last, num_kv_groups=G, head_dim=D)
+    bad_k = dataclasses.replace(squeezed, K_ch_scale=squeezed.K_ch_scale * 1.5)
+    with pytest.raises(AssertionError, match="packed K block diverges"):
+        bw._validate_packed_layer_reference(packed, bad_k, v16, q_last, num_kv_groups=G, head_dim=D)
+    bad_v = dataclasses.replace(squeezed, V_zp=squeezed.V_zp + 3)
+    with pytest.raises(AssertionError, match="packed V block diverges"):
+        bw._validate_packed_layer_reference(packed, bad_v, v16, q_last, num_kv_groups=G, head_dim=D)

@@ -187,3 +187,88 @@ def test_select_joint_matches_reference_outputs(name):
         assert np.array_equal(np.asarray(v16).view(np.uint8), g["new_v"].view(np.uint8))
     else:
         assert v16 is None
+
+
+def test_score_block_known_answers():
+    """Pins of ``select_oracle.score_block`` (blockwise_decode.py:756-791) that do not retype it:
+    the cases of the reference's own tests (tests/test_blockwise_rdkv.py:70-93: the explicit
+    einsum + softmax + sum of the library, and the causal final flush), and closed forms - a zero
+    query weights every visible key equally, every softmax row sums to one, one dominant key takes
+    all the mass, constant inputs give the product of the squares."""
+    import math
+    torch.manual_seed(7)
+    h_kv, groups, q_len, t_len, dim = 2, 2, 5, 4, 8
+    q = torch.randn(h_kv * groups, q_len, dim)
+    k = torch.randn(1, h_kv, t_len, dim)
+    token, channel = S.score_block(q.numpy(), k.numpy(), num_kv_groups=groups, causal=False)
+    qg = q.view(h_kv, groups, q_len, dim)
+    logits = torch.einsum("hgqd,htd->hgqt", qg, k[0]) / math.sqrt(dim)
+    np.testing.assert_allclose(token, logits.softmax(-1).sum((1, 2)).numpy(), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(channel, (qg.square().mean((1, 2)) * k[0].square().mean(1)).numpy(), rtol=1e-5, atol=1e-7)
+    np.testing.assert_allclose(token.sum(axis=1), groups * q_len, rtol=1e-6)        # rows of a softmax sum to one
+    # the causal final flush of the reference's test: the last key is seen by the last query only
+    qc = np.ones((1, 4, 2), np.float32)
+    kc = np.asarray([[[[1.0, 0.0], [0.0, 1.0], [1.0, 1.0], [2.0, 0.0]]]], np.float32)
+    tok, _ = S.score_block(qc, kc, num_kv_groups=1, causal=True)
+    assert tok[0, 0] > tok[0, 3] and np.isfinite(tok).all()
+    # the same numbers by hand: query i sees keys 0..i with logits (1, 1, 2, 2) / sqrt(2)
+    e = np.exp(np.asarray([1.0, 1.0, 2.0, 2.0]) / math.sqrt(2.0))
+    by_hand = np.zeros(4)
+    for i in range(4):
+        by_hand[:i + 1] += e[:i + 1] / e[:i + 1].sum()
+    np.testing.assert_allclose(tok[0], by_hand, rtol=1e-6)
+    with pytest.raises(ValueError):
+        S.score_block(np.ones((1, 3, 2), np.float32), kc, num_kv_groups=1, causal=True)
+    # zero queries: uniform weights - G*Q/T per key, and G * sum_{i>=t} 1/(i+1) under the causal mask
+    H, G, Q, T, D = 3, 2, 6, 6, 4
+    rng = np.random.default_rng(1)
+    keys = rng.standard_normal((1, H, T, D)).astype(np.float32)
+    tok, ch = S.score_block(np.zeros((H * G, Q, D), np.float32), keys, num_kv_groups=G, causal=False)
+    np.testing.assert_allclose(tok, np.full((H, T), G * Q / T), rtol=1e-6)
+    assert (ch == 0).all()
+    tok, _ = S.score_block(np.zeros((H * G, Q, D), np.float32), keys, num_kv_groups=G, causal=True)
+    harmonic = np.asarray([sum(1.0 / (i + 1) for i in range(t, T)) for t in range(T)])
+    np.testing.assert_allclose(tok, np.broadcast_to(G * harmonic, (H, T)), rtol=1e-6)
+    # one key far ahead of the others takes the whole mass of every query
+    keys = np.zeros((1, 1, 5, 4), np.float32)
+    keys[0, 0, 2] = 50.0
+    tok, _ = S.score_block(np.ones((2, 3, 4), np.float32), keys, num_kv_groups=2, causal=False)
+    np.testing.assert_allclose(tok[0], [0, 0, 6, 0, 0], atol=1e-6)
+    # constants: mean(q^2) * mean(k^2); and the GQA grouping is head-major (heads 0..G-1 -> KV head 0)
+    qs = np.stack([np.full((3, 4), 1.0), np.full((3, 4), 3.0), np.full((3, 4), 2.0), np.full((3, 4), 2.0)]).astype(np.float32)
+    ks2 = np.stack([np.full((5, 4), 2.0), np.full((5, 4), 0.5)])[None].astype(np.float32)
+    _, ch = S.score_block(qs, ks2, num_kv_groups=2, causal=False)
+    np.testing.assert_allclose(ch, [[5.0 * 4.0] * 4, [4.0 * 0.25] * 4], rtol=1e-6)
+
+
+def test_score_one_layer_known_answers():
+    """Pins of ``select_oracle.score_one_layer`` (obkv_fast.py:854-896): the tensor expressions of
+    the reference evaluated by the library (sum over (G, W) in the weights' type, then float; mean
+    of squares times mean of squares), and closed forms - attention rows that sum to one give
+    G*W per layer summed over the keys, constants give the product of the squares, the fp16 sum is
+    rounded to fp16 (2049 ones sum to 2048)."""
+    rng = np.random.default_rng(3)
+    B, H, G, W, T, D = 1, 2, 3, 4, 7, 8
+    aw = torch.softmax(torch.from_numpy(rng.standard_normal((B, H, G, W, T)).astype(np.float32)), dim=-1)
+    q = torch.from_numpy(rng.standard_normal((B, H, G, W, D)).astype(np.float32))
+    k = torch.from_numpy(rng.standard_normal((B, H, T, D)).astype(np.float32))
+    for dt, tol in ((torch.float32, 1e-6), (torch.float16, 1e-3), (torch.bfloat16, 8e-3)):
+        a, qq, kk = aw.to(dt), q.to(dt), k.to(dt)
+        token, channel = S.score_one_layer(t2np(a), t2np(qq), t2np(kk))
+        exp_token = a.sum(dim=(2, 3)).float().numpy()                       # obkv_fast.py:889
+        exp_channel = (qq.float().square().mean(dim=(2, 3)) * kk.float().square().mean(dim=2)).numpy()
+        np.testing.assert_allclose(token, exp_token, rtol=tol, atol=tol)
+        np.testing.assert_allclose(channel, exp_channel, rtol=1e-5, atol=1e-7)
+    token, _ = S.score_one_layer(aw.numpy(), q.numpy(), k.numpy())
+    np.testing.assert_allclose(token.sum(axis=-1), G * W, rtol=1e-6)
+    ones = np.ones((1, 1, 1, 2049, 1), np.float16)
+    tok16, _ = S.score_one_layer(ones, np.ones((1, 1, 1, 2049, 2), np.float16), np.ones((1, 1, 1, 2), np.float16))
+    assert tok16.dtype == np.float32 and tok16[0, 0, 0] == 2048.0           # the sum is a value of the weights' type
+    _, ch = S.score_one_layer(np.zeros((1, 2, 1, 1, 3), np.float32), np.full((1, 2, 1, 1, 4), 3.0, np.float32),
+                              np.stack([np.full((3, 4), 2.0), np.full((3, 4), 0.5)])[None].astype(np.float32))
+    np.testing.assert_allclose(ch, [[[36.0] * 4, [2.25] * 4]], rtol=1e-6)
+
+
+def t2np(t):
+    """torch tensor -> NumPy array of the same type (bfloat16 through its fp32 value: NumPy has no bf16)."""
+    return t.float().numpy() if t.dtype == torch.bfloat16 else t.numpy()
