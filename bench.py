@@ -7,7 +7,10 @@ for one query per layer and writes out [L*H_q,128] + lse.  Inputs are synthetic,
 resident in HBM before the timed region.  Default workload: configuration 1 (Llama-3.1-8B
 shapes, 32 layers, 32k context, per-head Dirichlet bit allocation).
 
-Prints ONE JSON line (see README / DESIGN for the fields).
+Prints ONE JSON line (see README / DESIGN for the fields): the headline on configuration 1 with
+`roofline` and `cpu_baseline`, and beside it compact figures of the other configurations
+(`configs`), the one-layer-per-call form (`sequential`), the reference-layout entry points
+(`padded`), the prefill packer (`pack`, `select`) and the whole-model decode loops (`decode_loop`).
 """
 from __future__ import annotations
 
@@ -22,10 +25,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per launch of the fused kernel on the default workload, from two rocprofv3 --pmc
-# runs of this command (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the factors a plain copy
-# kernel of known size gives): (547 614 x 2 + 1 052) KiB.  Other workloads: not measured.
-MEASURED_TRAFFIC_BYTES = {1: 1122590720}
+# HBM bytes per launch of the fused kernel by workload configuration, from two rocprofv3 --pmc runs
+# of `python3 bench.py --config N --fused-only` (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000, the
+# factors a plain copy kernel of known size gives in the same runs).  A constant read off the named
+# profile summary, not something a run of this script observes: it goes stale when the layout
+# changes, which is why the JSON names its source.
+MEASURED_TRAFFIC = {
+    1: (1122590720, "profiles/decode_fused_kernel_c1_llama31_8b_32k.txt"),
+}
 PACK_SAMPLE_LAYERS = 8                      # layers of one sequence packed back to back for the pack throughput
 
 
@@ -45,8 +52,16 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-check", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="skip the compact figures of the other configurations")
+    ap.add_argument("--configs", type=str, default="0,2,3,4", help="configurations of the compact block")
+    ap.add_argument("--fused-only", action="store_true",
+                    help="only build the workload and run the fused step (for profiling): prints a short JSON")
     ap.add_argument("--sequential-only", action="store_true",
                     help="only the one-layer-per-call leg (for profiling): prints its JSON and exits")
+    ap.add_argument("--padded-only", action="store_true",
+                    help="only the reference-layout entry points on one layer (for profiling): prints its JSON")
+    ap.add_argument("--pack-only", action="store_true",
+                    help="only the prefill pack of one sequence of the workload (for profiling): prints its JSON")
     ap.add_argument("--no-decode-loop", action="store_true",
                     help="skip the whole-model greedy decode loop (random-weight Llama-3.1-8B-shaped model)")
     return ap.parse_args()
@@ -65,12 +80,392 @@ def time_region(fn, steps, torch):
     return start.elapsed_time(end) / steps
 
 
+def graph_of(fn, torch):
+    """`fn` (which neither allocates nor synchronizes once warm) captured on a side stream; returns
+    (graph, stream).  Time `graph.replay` inside `with torch.cuda.stream(stream)`."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()                                  # workspaces of this stream exist before capture
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            fn()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+    return graph, side
+
+
+# ---------------------------------------------------------------------------------------------
+# workload construction and the fused step
+# ---------------------------------------------------------------------------------------------
+def build_workload(cfg, dev, torch, on_first=None, pack_sample=None):
+    """Pack every (sequence, layer) of `cfg` with the HIP packer.  Returns the list of
+    (packed layer, new_v_only, q).  `on_first(K, V, q, vb, kb)` sees the fp16 inputs of layer 0 of
+    sequence 0; `pack_sample` (a list) receives (K, V, vb, kb) of the first layers of sequence 0."""
+    from rdkv_amd import packing, synth
+    groups = []
+    for seq in range(cfg.batch):
+        for layer in range(cfg.layers):
+            vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
+            K, V, q = synth.layer_data(cfg, layer, dev, seq, outliers=oc)
+            pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+            groups.append((pl, nvo, q))
+            if seq == 0 and layer == 0 and on_first is not None:
+                on_first(K, V, q, vb, kb)
+            if pack_sample is not None and seq == 0 and layer < PACK_SAMPLE_LAYERS and cfg.layers > 1:
+                pack_sample.append((K, V, vb, kb))
+            del K, V
+    return groups
+
+
+def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True):
+    """ms per step of the fused call (streaming launch + merge launch) issued eagerly and replayed
+    from a HIP graph, and ms per launch of the streaming kernel alone."""
+    from rdkv_amd import _lib, stream_cache
+    lib = _lib.load()
+    dev = qs.device
+
+    def step():
+        stream_cache.decode_attn_fused(cache, qs, out, lse)
+
+    # untimed: the W warm-up steps, then keep stepping for ~0.3 s so that the device clocks have
+    # ramped before the timed region (a 0.3 ms step is far shorter than the governor's window)
+    for _ in range(max(warmup, 1)):
+        step()
+    torch.cuda.synchronize()
+    t_ramp = time.time()
+    while time.time() - t_ramp < 0.3:
+        for _ in range(20):
+            step()
+        torch.cuda.synchronize()
+    ms_eager = time_region(step, steps, torch)
+    ms_graph = None
+    if graph:
+        g, side = graph_of(step, torch)
+        with torch.cuda.stream(side):
+            ms_graph = time_region(g.replay, steps, torch)
+        torch.cuda.current_stream().wait_stream(side)
+    ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
+    stream = _lib.stream_of(dev)
+
+    def partials_only():
+        _lib.check(lib.rdkv_decode_fused_partials(
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, None, None, 0,
+            ws.data_ptr(), ws.numel(), stream))
+
+    partials_only()
+    ms_kernel = time_region(partials_only, steps, torch)
+    return step, ms_eager, ms_graph, ms_kernel
+
+
+def oracle_layer(pl, nvo, torch):
+    """The packed layer as the NumPy oracle's dataclass over the same bytes."""
+    import dataclasses
+    from oracle import rdkv_oracle as O
+    kw = {}
+    for f in dataclasses.fields(O.PackedKVLayer):
+        v = getattr(pl, f.name)
+        kw[f.name] = v.detach().cpu().numpy() if torch.is_tensor(v) else v
+    return O.PackedKVLayer(**kw), (nvo.cpu().numpy() if nvo is not None else None)
+
+
+def check_layer0(first_pl, first_nvo, q0, got, torch):
+    """Layer 0 of what was timed against the CPU oracle (tolerance of the parity tests)."""
+    import numpy as np
+    from oracle import rdkv_oracle as O
+    ora, ora_nvo = oracle_layer(first_pl, first_nvo, torch)
+    exp_out, _, _ = O.decode_attn_ref(q0, ora, ora_nvo)
+    err = float(np.abs(got - exp_out).max())
+    return {"layer0_max_abs_err": err, "layer0_ref_max_abs": float(np.abs(exp_out).max()),
+            "within_tolerance": bool(err <= 2e-3 and err <= 1e-2 * np.abs(exp_out).max())}
+
+
+def compact_config(index, args, torch, dev):
+    """One configuration measured the same way as the headline, in short: build, eager step,
+    streaming kernel alone, layer-0 check.  Configuration 4 also packs one whole sequence (all
+    its layers) from resident fp16 K/V: its second metric."""
+    import numpy as np
+    from rdkv_amd import packing, stream_cache, synth
+    cfg = synth.CONFIGS[index]
+    t0 = time.time()
+    sample = [] if index == 4 else None
+    groups = build_workload(cfg, dev, torch)
+    qs = torch.cat([g[2] for g in groups]).contiguous()
+    cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G)
+    first_pl, first_nvo = groups[0][0], groups[0][1]
+    del groups
+    torch.cuda.empty_cache()
+    torch.cuda.synchronize()
+    build_s = time.time() - t0
+    out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
+    lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
+    steps = max(5, min(args.steps, int(2000 / max(cache.algorithmic_bytes / 6e9, 0.01))))   # ~2 s at most
+    _, ms_eager, _, ms_kernel = fused_step_times(cache, qs, out, lse, steps, args.warmup, torch, graph=False)
+    algo = cache.algorithmic_bytes
+    n_groups = cfg.batch * cfg.layers
+    res = {"workload": cfg.name, "layers": cfg.layers, "batch": cfg.batch, "context": cfg.context, "G": cfg.G,
+           "steps": steps, "ms_per_step": ms_eager, "ms_per_launch_fused_kernel": ms_kernel,
+           "algorithmic_bytes_per_step": algo, "GBps": algo / (ms_eager * 1e-3) / 1e9,
+           "frac_step": algo / (ms_eager * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+           "frac_kernel": algo / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+           "us_per_sequence_layer": ms_eager * 1e3 / n_groups, "work_items": cache.n_work,
+           "kernel_variant_max_row_dwords": cache.max_row_dwords,
+           "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo, "build_seconds": build_s}
+    if not args.no_check:
+        res["check"] = check_layer0(first_pl, first_nvo, qs[:cfg.H_q].cpu().numpy(), out[:cfg.H_q].cpu().numpy(), torch)
+    del cache, out, lse, qs, first_pl, first_nvo
+    torch.cuda.empty_cache()
+    if index == 4:
+        res["pack_one_sequence"] = pack_sequence_section(cfg, torch, dev)
+    return res
+
+
+# ---------------------------------------------------------------------------------------------
+# the prefill packer
+# ---------------------------------------------------------------------------------------------
+def pack_sequence_section(cfg, torch, dev, seq=0):
+    """One sequence's full prefill cache (every layer of sequence `seq`) packed from resident fp16
+    K and V: wall time of `packing.pack_layers_per_head`, as GB/s of the fp16 input read once."""
+    import numpy as np
+    from rdkv_amd import packing, synth
+    Ks, Vs, vbs, kbs = [], [], [], []
+    for layer in range(cfg.layers):
+        vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
+        K, V, _ = synth.layer_data(cfg, layer, dev, seq, outliers=oc)
+        Ks.append(K), Vs.append(V), vbs.append(vb), kbs.append(kb)
+    vb_all, kb_all = torch.stack(vbs).to(dev), torch.stack(kbs).to(dev)
+    times = []
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        packing.pack_layers_per_head(Ks, Vs, vb_all, kb_all, cfg.G)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    in_bytes = sum(2 * k.numel() * k.element_size() for k in Ks)
+    ms = float(np.median(times[1:]))
+    return {"layers": cfg.layers, "tokens": int(Ks[0].shape[2]), "fp16_input_bytes": in_bytes, "pack_ms": ms,
+            "pack_ms_per_layer": ms / cfg.layers, "pack_GBps_of_fp16_input": in_bytes / (ms * 1e-3) / 1e9,
+            "note": "packing.pack_layers_per_head over all layers of one sequence, wall time, median of 3 after 1 warm-up"}
+
+
+def pack_layer_sections(cfg, K, V, vb, kb, args, torch, dev):
+    """Layer 0: wall time of the whole-layer packer and of the re-layout, and of the prefill
+    selection feeding the packer (pooling, per-head V knapsack, per-head K allocation, pack)."""
+    import numpy as np
+    from rdkv_amd import knapsack_solver, obkv_fast, packing, stream_cache
+    pack_ms, relayout_ms = [], []
+    for _ in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        pl_t, nvo_t = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        stream_cache.build_stream_cache([(pl_t, nvo_t)], cfg.G)
+        torch.cuda.synchronize()
+        pack_ms.append((t1 - t0) * 1e3)
+        relayout_ms.append((time.perf_counter() - t1) * 1e3)
+    del pl_t, nvo_t
+    in_bytes = 2 * K.numel() * K.element_size()
+    pack_info = {"fp16_input_bytes_per_layer": in_bytes,
+                 "pack_ms_per_layer": float(np.median(pack_ms[1:])),
+                 "pack_GBps_of_fp16_input": in_bytes / (float(np.median(pack_ms[1:])) * 1e-3) / 1e9,
+                 "relayout_ms_per_layer": float(np.median(relayout_ms[1:])),
+                 "note": "wall time of packing.pack_layer_per_head (+ stream_cache.build_stream_cache) "
+                         "on layer 0, median of 5 after 1 warm-up; K is read twice (min/max pass, then emit)"}
+    # seeded log-normal scores; the budget is a quarter of the context, half of it for K
+    gsel = torch.Generator().manual_seed(4242)
+    H_kv, T_ctx = int(K.shape[1]), int(K.shape[2])
+    tok_scores = torch.exp(torch.randn(H_kv, T_ctx, generator=gsel) * 1.5 + 2.0).to(dev)
+    ch_scores = torch.exp(torch.randn(H_kv, 128, generator=gsel)).to(dev)
+    sel_kw = dict(gqa_factor=cfg.G, token_budget=max(T_ctx // 4, 1), k_budget_ratio=0.5, obs_window=32,
+                  pool_kernel_size=7, pool_padding="reflect", pool_type="avg", v_bit_options=None,
+                  k_bit_options=torch.tensor([0.0, 2.0, 4.0, 8.0]),
+                  eps_V=knapsack_solver.DEFAULT_EPSILON_V, eps_K=knapsack_solver.DEFAULT_EPSILON_K)
+    sel_ms, stages = [], {}
+    for _ in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, **sel_kw)
+        torch.cuda.synchronize()
+        sel_ms.append((time.perf_counter() - t0) * 1e3)
+    obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, timing=stages, **sel_kw)
+    select_info = {"select_and_pack_ms_per_layer": float(np.median(sel_ms[1:])),
+                   "stages_ms": {k: round(v, 4) for k, v in stages.items()},
+                   "rows": H_kv, "tokens_per_row": T_ctx,
+                   "note": "wall time of obkv_fast._perhead_select_and_pack_joint on layer 0 (median of "
+                           "5 after 1 warm-up); stages from one extra call that synchronizes after "
+                           "each stage (quantization_ms = the whole-layer packer)"}
+    if not args.no_cpu_baseline:
+        from oracle import select_oracle
+        t0 = time.perf_counter()
+        select_oracle.select_joint(
+            tok_scores.cpu().numpy(), ch_scores.cpu().numpy(), head_dim=128,
+            token_budget=sel_kw["token_budget"], k_budget_ratio=0.5, pool_kernel_size=7,
+            pool_padding="reflect", k_bit_options=(0, 2, 4, 8))
+        select_info["cpu_oracle_allocation_ms"] = (time.perf_counter() - t0) * 1e3
+        select_info["gpu_allocation_ms"] = float(sum(v for k, v in stages.items()
+                                                     if k in ("pooling_ms", "v_allocation_ms", "k_allocation_ms")))
+    return pack_info, select_info
+
+
+def pack_sample_section(pack_sample, pack_info, cfg, torch, dev):
+    """The first layers of a sequence packed back to back (one planning launch and one host read
+    for all of them, the host side of a layer overlapping the kernels of the one before)."""
+    import numpy as np
+    from rdkv_amd import packing
+    vb_all = torch.stack([p[2] for p in pack_sample]).to(dev)
+    kb_all = torch.stack([p[3] for p in pack_sample]).to(dev)
+    times = []
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        packing.pack_layers_per_head([p[0] for p in pack_sample], [p[1] for p in pack_sample], vb_all, kb_all, cfg.G)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    sample_bytes = sum(2 * p[0].numel() * p[0].element_size() for p in pack_sample)
+    pack_info["pack_layers_sample"] = len(pack_sample)
+    pack_info["pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
+    pack_info["pack_GBps_of_fp16_input_batched"] = sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
+
+
+# ---------------------------------------------------------------------------------------------
+# one layer per call, and the reference-layout entry points
+# ---------------------------------------------------------------------------------------------
+def sequential_section(cfg, torch, dev, layers=8, replays=50):
+    """One layer per call, the form a sequential model loop issues: `layers` single-layer streaming
+    caches (distinct buffers, 280 MB together: more than the last-level cache), their fused calls
+    recorded one after the other into one HIP graph, the graph replayed back to back - as two
+    launches per call and as one (the merge inside the streaming launch).  Beside it the same number
+    of bytes per launch read by a plain streaming kernel, the floor of any single launch of this size."""
+    import numpy as np
+    from rdkv_amd import _lib, packing, stream_cache, synth
+    lib = _lib.load()
+    caches, qs, outs = [], [], []
+    for layer in range(layers):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, q = synth.layer_data(cfg, layer, dev, outliers=oc)
+        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+        del K, V
+        c = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
+        caches.append(c)
+        qs.append(q)
+        outs.append((torch.empty(c.rows, 128, device=dev), torch.empty(c.rows, device=dev)))
+    res = {"layers_rotated": layers, "context": cfg.context}
+    algo = float(np.mean([c.algorithmic_bytes for c in caches]))
+    for name, one in (("two_launches", False), ("one_launch", True)):
+        def all_layers():
+            for c, q, (o, l) in zip(caches, qs, outs):
+                stream_cache.decode_attn_fused(c, q, o, l, one_launch=one)
+        g, side = graph_of(all_layers, torch)
+        with torch.cuda.stream(side):
+            us_graph = time_region(g.replay, replays, torch) / layers * 1e3
+            us_eager = time_region(all_layers, replays, torch) / layers * 1e3
+        torch.cuda.current_stream().wait_stream(side)
+        res[name] = {"us_per_layer_graph_replay": us_graph, "us_per_layer_eager": us_eager,
+                     "GBps_graph_replay": algo / us_graph / 1e3,
+                     "frac_hbm_peak_graph_replay": algo / us_graph / 1e3 / HBM_PEAK_GBPS}
+    default_one = caches[0].n_work <= stream_cache.ONE_LAUNCH_MAX_WORK
+    res["default_form"] = "one_launch" if default_one else "two_launches"
+    res["us_per_layer_sequential"] = res[res["default_form"]]["us_per_layer_graph_replay"]
+    res["frac_hbm_peak"] = res[res["default_form"]]["frac_hbm_peak_graph_replay"]
+    # a plain read of the same number of bytes per launch, rotated over as many distinct buffers
+    nbytes = int(np.mean([c.stream_bytes for c in caches])) // 4096 * 4096
+    bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255) for _ in range(layers)]
+    sink = torch.zeros(1024, dtype=torch.uint8, device=dev)
+
+    def plain_reads():
+        st = _lib.stream_of(dev)
+        for b in bufs:
+            _lib.check(lib.rdkv_probe_read_stream(b.data_ptr(), nbytes, 16 * 1024, sink.data_ptr(), st))
+    g, side = graph_of(plain_reads, torch)
+    with torch.cuda.stream(side):
+        us_read = time_region(g.replay, replays, torch) / layers * 1e3
+    torch.cuda.current_stream().wait_stream(side)
+    res.update({"algorithmic_bytes_per_layer": algo, "streamed_bytes_per_layer": nbytes,
+                "plain_read_us_per_launch": us_read, "plain_read_GBps": nbytes / us_read / 1e3,
+                "workgroups_per_layer": caches[0].n_groups or caches[0].n_work,
+                "work_items_per_layer": caches[0].n_work,
+                "note": "one layer per call, calls of distinct layers back to back in one replayed HIP graph; "
+                        "plain_read = a streaming read kernel over the same number of bytes per launch"})
+    return res
+
+
+def padded_section(cfg, torch, dev, steps=50, layers=4):
+    """The three reference entry points on the reference layout (k_mixed_qk_dot_into, the masked
+    softmax, v_dequant_weighted_sum_dispatch_into), each timed alone over `layers` distinct layers of
+    the workload in rotation, against its algorithmic bytes (per-head counts, no padding)."""
+    import numpy as np
+    from rdkv_amd import _lib, packing, stream_cache, synth
+    from rdkv_amd.fast_decode import _pre_squeeze_packed
+    from rdkv_amd.k_kernel import k_mixed_qk_dot_into
+    from rdkv_amd.v_kernel import v_dequant_weighted_sum_dispatch_into
+    lib = _lib.load()
+    items = []
+    k_bytes = v_bytes = s_bytes = 0
+    for layer in range(layers):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, q = synth.layer_data(cfg, layer, dev, outliers=oc)
+        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
+        del K, V
+        sp = _pre_squeeze_packed((pl,))[0]
+        T_v = int(sp.T_eff)
+        T_old = int(sp.T_eff_k) if sp.T_eff_k > 0 else T_v
+        scores = torch.empty(cfg.H_q, T_old, dtype=torch.float32, device=dev)
+        out = torch.empty(cfg.H_q, 128, dtype=torch.float32, device=dev)
+        items.append((q.float(), sp, nvo[0].contiguous() if nvo is not None else None, T_v, T_old, scores, out))
+        tok, ch = stream_cache._layer_counts(pl, cfg.H_kv)
+        for (n2, n4, n8, n16), (c2, c4, c8) in zip(tok, ch):
+            kept = n2 + n4 + n8 + n16
+            k_bytes += kept * (-(-c2 // 4) + -(-c4 // 2) + c8) + 4 * (c2 + c4 + c8) + cfg.G * kept * 4
+            v_bytes += 32 * n2 + 64 * n4 + 128 * n8 + 4 * (n2 + n4 + n8) + 256 * n16 + cfg.G * kept * 4
+            s_bytes += cfg.G * kept * 4 * 2 + kept * 4
+        k_bytes += cfg.H_q * 128 * 4
+        v_bytes += cfg.H_q * 128 * 4
+    k_bytes, v_bytes, s_bytes = k_bytes / layers, v_bytes / layers, s_bytes / layers
+
+    def run_k():
+        for q32, sp, _, _, T_old, scores, _ in items:
+            k_mixed_qk_dot_into(q32, sp, T_old, scores)
+
+    def run_softmax():
+        st = _lib.stream_of(dev)
+        for _, sp, _, _, T_old, scores, _ in items:
+            mask = sp.softmax_mask
+            _lib.check(lib.rdkv_softmax_rows(
+                scores.data_ptr(), scores.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0,
+                T_old, None, 0, 0, scores.data_ptr(), scores.stride(0), None, 0, cfg.H_q, st))
+
+    def run_v():
+        for _, sp, v16, T_v, _, scores, out in items:
+            v_dequant_weighted_sum_dispatch_into(scores, sp, out, V16=v16, n_v16_per_head=sp.n_v16_per_head, max_T_v=T_v)
+
+    res = {"layers_rotated": layers, "context": cfg.context}
+    for name, fn, nbytes in (("k_mixed_qk_dot_into", run_k, k_bytes), ("softmax_rows", run_softmax, s_bytes),
+                             ("v_dequant_weighted_sum_dispatch_into", run_v, v_bytes)):
+        fn()
+        us = time_region(fn, steps, torch) / layers * 1e3
+        res[name] = {"us_per_layer": us, "algorithmic_bytes_per_layer": nbytes, "GBps": nbytes / us / 1e3,
+                     "frac_hbm_peak": nbytes / us / 1e3 / HBM_PEAK_GBPS}
+    res["us_per_layer_total"] = sum(res[k]["us_per_layer"] for k in
+                                    ("k_mixed_qk_dot_into", "softmax_rows", "v_dequant_weighted_sum_dispatch_into"))
+    res["note"] = ("the reference's K / softmax / V call sequence on PackedKVLayer tensors, eager launches; bytes: "
+                   "codes + scale/zp + query + fp32 scores written (K), fp32 weights read + codes + scale/zp + "
+                   "fp16 zone B + out (V), scores read and written + mask (softmax)")
+    return res
+
+
+# ---------------------------------------------------------------------------------------------
+# whole-model decode loops (beside the headline, never as it)
+# ---------------------------------------------------------------------------------------------
 def decode_loop_section(cfg, torch, dev, tokens=48):
     """ms per generated token of ``fast_decode.greedy_decode_fast`` on a random-weight model of the
     Llama-3.1-8B shape (32 layers, hidden 4096, 32 / 8 heads) over a packed cache of the
     workload's shape: the whole-model figure the reference quotes for its loop (its only
     published latency, triton_v_kernel.py:53-54).  Reported beside the headline, never as it."""
-    import time
     from transformers import LlamaConfig, LlamaForCausalLM
     from rdkv_amd import fast_decode, packing, synth
     L = 32
@@ -127,49 +522,64 @@ def decode_loop_section(cfg, torch, dev, tokens=48):
     return res
 
 
-def sequential_section(cfg, torch, dev, layers=8, replays=50):
-    """One layer per call, the form a sequential model loop issues: ``layers`` single-layer streaming
-    caches (distinct buffers), their fused calls (streaming launch + merge launch each) recorded one
-    after the other into one HIP graph, the graph replayed back to back.  Returns us per layer."""
+# ---------------------------------------------------------------------------------------------
+# CPU baseline
+# ---------------------------------------------------------------------------------------------
+def cpu_baseline_section(ora, ora_nvo, q0, H_q, torch):
+    """The NumPy oracle (dequantize-then-attend, the reference's own CPU-checkable form) on layer 0
+    of the workload: 2 warm-ups + 3 repeats, median (the protocol of run_latency.py:107-108), on
+    one core (the calling thread pinned to one CPU, library thread pools limited to 1) and on all
+    cores of this process (one oracle call per core at a time, as concurrent threads: NumPy's
+    array operations release the interpreter lock)."""
     import numpy as np
-    from rdkv_amd import packing, stream_cache, synth
-    caches, qs, outs = [], [], []
-    for layer in range(layers):
-        vb, kb, oc = synth.layer_allocation(cfg, layer)
-        K, V, q = synth.layer_data(cfg, layer, dev, outliers=oc)
-        pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
-        del K, V
-        c = stream_cache.build_stream_cache([(pl, nvo)], cfg.G)
-        caches.append(c)
-        qs.append(q)
-        outs.append((torch.empty(c.rows, 128, device=dev), torch.empty(c.rows, device=dev)))
+    from concurrent.futures import ThreadPoolExecutor
+    from threadpoolctl import threadpool_limits
+    from oracle import rdkv_oracle as O
+    layer_bytes = O.algorithmic_bytes(ora, H_q)
+    cpus = sorted(os.sched_getaffinity(0))
+    env_threads = os.environ.get("OMP_NUM_THREADS")
+    n_all = min(len(cpus), int(env_threads)) if env_threads and env_threads.isdigit() else len(cpus)
 
-    def all_layers():
-        for c, q, (o, l) in zip(caches, qs, outs):
-            stream_cache.decode_attn_fused(c, q, o, l)
+    def one():
+        return O.decode_attn_ref(q0, ora, ora_nvo)
 
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        all_layers()
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            all_layers()
-        for _ in range(5):
-            graph.replay()
-        torch.cuda.synchronize()
-        ms_graph = time_region(graph.replay, replays, torch) / layers
-        ms_eager = time_region(all_layers, replays, torch) / layers
-    torch.cuda.current_stream().wait_stream(side)
-    algo = float(np.mean([c.algorithmic_bytes for c in caches]))
-    return {"layers_rotated": layers, "context": cfg.context,
-            "us_per_layer_graph_replay": ms_graph * 1e3, "us_per_layer_eager": ms_eager * 1e3,
-            "algorithmic_bytes_per_layer": algo,
-            "GBps_graph_replay": algo / (ms_graph * 1e-3) / 1e9,
-            "frac_hbm_peak_graph_replay": algo / (ms_graph * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-            "workgroups_per_layer": caches[0].n_groups or caches[0].n_work, "work_items_per_layer": caches[0].n_work,
-            "note": "one layer per call (streaming launch + merge launch), calls of distinct layers back to back"}
+    def timed(fn, warm=2, reps=3):
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    torch_threads_before = torch.get_num_threads()
+    with threadpool_limits(limits=1):
+        torch.set_num_threads(1)
+        os.sched_setaffinity(0, {cpus[0]})
+        try:
+            t1 = timed(one)
+        finally:
+            os.sched_setaffinity(0, set(cpus))
+            torch.set_num_threads(torch_threads_before)
+        # all cores: n_all oracle calls in flight, each on a thread of its own, library pools still 1 per call
+        with ThreadPoolExecutor(max_workers=n_all) as ex:
+            def wave():
+                list(ex.map(lambda _: one(), range(n_all)))
+            t_all = timed(wave, warm=1, reps=3)
+    print(f"bench.py: cpu baseline threads: 1-core leg 1 thread on cpu {cpus[0]}; all-cores leg {n_all} threads; "
+          f"torch.get_num_threads()={torch.get_num_threads()}", file=sys.stderr)
+    return {"value": layer_bytes / t1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"NumPy dequantize-then-attend oracle on layer 0 of the workload ({layer_bytes} algorithmic "
+                      f"bytes), 2 warm-ups + 3 repeats, median; calling thread pinned to one CPU, library thread "
+                      f"pools limited to 1",
+            "ms_per_layer": t1 * 1e3,
+            "all_cores": {"value": n_all * layer_bytes / t_all / 1e9, "unit": "GB/s", "cores": n_all,
+                          "ms_per_layer": t_all * 1e3 / n_all,
+                          "sample": f"{n_all} concurrent oracle calls on layer 0 (one thread each), 1 warm-up + 3 "
+                                    f"repeats, median"},
+            "host_cpus": os.cpu_count(), "cpus_of_this_process": len(cpus),
+            "torch_num_threads": torch.get_num_threads()}
 
 
 def main():
@@ -183,7 +593,7 @@ def main():
     import numpy as np
     import torch
 
-    from rdkv_amd import _lib, packing, stream_cache, synth
+    from rdkv_amd import _lib, stream_cache, synth
 
     if not _lib.available():
         import __graft_entry__
@@ -198,106 +608,29 @@ def main():
     if args.sequential_only:
         print(json.dumps(sequential_section(cfg, torch, dev, replays=args.steps)))
         return
+    if args.padded_only:
+        print(json.dumps(padded_section(cfg, torch, dev, steps=args.steps)))
+        return
+    if args.pack_only:
+        print(json.dumps(pack_sequence_section(cfg, torch, dev)))
+        return
     t_build = time.time()
-    groups = []          # (packed layer, new_v_only) per (sequence, layer)
-    keep_first = None    # layer 0 of sequence 0: inputs kept for the CPU baseline / checks / dense run
-    pack_sample = []     # fp16 K/V + allocations of the first layers of sequence 0
-    for seq in range(cfg.batch):
-        for layer in range(cfg.layers):
-            vb, kb, oc = synth.layer_allocation(cfg, layer, seq)
-            K, V, q = synth.layer_data(cfg, layer, dev, seq, outliers=oc)
-            pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
-            groups.append((pl, nvo, q))
-            if keep_first is None:
-                keep_first = (K, V, q, pl, nvo)
-                # prefill pack throughput: quantize + bit-pack of this layer's fp16 K and V
-                # (reference layout) and the re-layout into the streaming format, as wall
-                # time including the host side, GB/s of fp16 input read once
-                pack_ms, relayout_ms = [], []
-                for _ in range(6):
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
-                    pl_t, nvo_t = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
-                    torch.cuda.synchronize()
-                    t1 = time.perf_counter()
-                    stream_cache.build_stream_cache([(pl_t, nvo_t)], cfg.G)
-                    torch.cuda.synchronize()
-                    pack_ms.append((t1 - t0) * 1e3)
-                    relayout_ms.append((time.perf_counter() - t1) * 1e3)
-                del pl_t, nvo_t
-                in_bytes = 2 * K.numel() * K.element_size()
-                pack_info = {"fp16_input_bytes_per_layer": in_bytes,
-                             "pack_ms_per_layer": float(np.median(pack_ms[1:])),
-                             "pack_GBps_of_fp16_input": in_bytes / (float(np.median(pack_ms[1:])) * 1e-3) / 1e9,
-                             "relayout_ms_per_layer": float(np.median(relayout_ms[1:])),
-                             "note": "wall time of packing.pack_layer_per_head (+ stream_cache.build_stream_cache) "
-                                     "on layer 0, median of 5 after 1 warm-up; K is read twice (min/max pass, "
-                                     "then emit)"}
-                # prefill selection feeding the packer on the same layer: score pooling, per-head V
-                # knapsack, per-head K allocation, then the pack (seeded log-normal scores; the
-                # budget is a quarter of the context, half of it for K)
-                from rdkv_amd import knapsack_solver, obkv_fast
-                gsel = torch.Generator().manual_seed(4242)
-                H_kv, T_ctx = int(K.shape[1]), int(K.shape[2])
-                tok_scores = torch.exp(torch.randn(H_kv, T_ctx, generator=gsel) * 1.5 + 2.0).to(dev)
-                ch_scores = torch.exp(torch.randn(H_kv, 128, generator=gsel)).to(dev)
-                sel_kw = dict(gqa_factor=cfg.G, token_budget=max(T_ctx // 4, 1), k_budget_ratio=0.5, obs_window=32,
-                              pool_kernel_size=7, pool_padding="reflect", pool_type="avg", v_bit_options=None,
-                              k_bit_options=torch.tensor([0.0, 2.0, 4.0, 8.0]),
-                              eps_V=knapsack_solver.DEFAULT_EPSILON_V, eps_K=knapsack_solver.DEFAULT_EPSILON_K)
-                sel_ms, stages = [], {}
-                for it in range(6):
-                    torch.cuda.synchronize()
-                    t0 = time.perf_counter()
-                    obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, **sel_kw)
-                    torch.cuda.synchronize()
-                    sel_ms.append((time.perf_counter() - t0) * 1e3)
-                obkv_fast._perhead_select_and_pack_joint(K, V, tok_scores, ch_scores, timing=stages, **sel_kw)
-                select_info = {"select_and_pack_ms_per_layer": float(np.median(sel_ms[1:])),
-                               "stages_ms": {k: round(v, 4) for k, v in stages.items()},
-                               "rows": H_kv, "tokens_per_row": T_ctx,
-                               "note": "wall time of obkv_fast._perhead_select_and_pack_joint on layer 0 (median of "
-                                       "5 after 1 warm-up); stages from one extra call that synchronizes after "
-                                       "each stage (quantization_ms = the whole-layer packer)"}
-                if not args.no_cpu_baseline:
-                    from oracle import select_oracle
-                    t0 = time.perf_counter()
-                    select_oracle.select_joint(
-                        tok_scores.cpu().numpy(), ch_scores.cpu().numpy(), head_dim=128,
-                        token_budget=sel_kw["token_budget"], k_budget_ratio=0.5, pool_kernel_size=7,
-                        pool_padding="reflect", k_bit_options=(0, 2, 4, 8))
-                    select_info["cpu_oracle_allocation_ms"] = (time.perf_counter() - t0) * 1e3
-                    select_info["gpu_allocation_ms"] = float(sum(v for k, v in stages.items()
-                                                                 if k in ("pooling_ms", "v_allocation_ms",
-                                                                          "k_allocation_ms")))
-                del tok_scores, ch_scores
-            if seq == 0 and layer < PACK_SAMPLE_LAYERS and cfg.layers > 1:
-                pack_sample.append((K, V, vb, kb))
-            del K, V
+    first = {}
+    pack_sample = []
+
+    def on_first(K, V, q, vb, kb):
+        if not args.fused_only:
+            first["pack"], first["select"] = pack_layer_sections(cfg, K, V, vb, kb, args, torch, dev)
+
+    groups = build_workload(cfg, dev, torch, on_first=on_first, pack_sample=None if args.fused_only else pack_sample)
+    pack_info, select_info = first.get("pack"), first.get("select")
     if len(pack_sample) > 1:
-        # one sequence's prefill cache packed layer after layer from resident fp16 K/V (a bounded sample
-        # of its first layers): one planning launch and one host read for all of them, the host side of a
-        # layer overlapping the kernels of the one before
-        vb_all = torch.stack([p[2] for p in pack_sample]).to(dev)
-        kb_all = torch.stack([p[3] for p in pack_sample]).to(dev)
-        times = []
-        for _ in range(4):
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            packing.pack_layers_per_head([p[0] for p in pack_sample], [p[1] for p in pack_sample], vb_all, kb_all, cfg.G)
-            torch.cuda.synchronize()
-            times.append((time.perf_counter() - t0) * 1e3)
-        sample_bytes = sum(2 * p[0].numel() * p[0].element_size() for p in pack_sample)
-        pack_info["pack_layers_sample"] = len(pack_sample)
-        pack_info["pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
-        pack_info["pack_GBps_of_fp16_input_batched"] = sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
-        del vb_all, kb_all
+        pack_sample_section(pack_sample, pack_info, cfg, torch, dev)
     pack_sample.clear()
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
                                             work_bytes=args.work_kib * 1024 if args.work_kib else None,
                                             groups_per_cu=args.groups_per_cu)
-    padded_bytes = 0
     first_pl, first_nvo = groups[0][0], groups[0][1]
     del groups
     torch.cuda.empty_cache()
@@ -307,53 +640,23 @@ def main():
 
     out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
     lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
-
-    def step():
-        stream_cache.decode_attn_fused(cache, qs, out, lse)
-
-    # untimed: the W warm-up steps, then keep stepping for ~0.3 s so that the device clocks have
-    # ramped before the timed region (a 0.3 ms step is far shorter than the governor's window)
-    for _ in range(max(args.warmup, 1)):
-        step()
-    torch.cuda.synchronize()
-    t_ramp = time.time()
-    while time.time() - t_ramp < 0.3:
-        for _ in range(20):
-            step()
+    step, ms_step_eager, ms_step_graph, ms_kernel = fused_step_times(
+        cache, qs, out, lse, args.steps, args.warmup, torch, graph=not args.no_graph)
+    # the headline is the eagerly issued step (two launches per step), the mode every run reports;
+    # the graph-replayed step stands beside it
+    ms_step = ms_step_eager
+    algo = cache.algorithmic_bytes
+    if args.fused_only:
+        # one plain copy of known size in the same process: the launch against which a profiler run
+        # of this command scales its traffic counters
+        probe = torch.empty(2, 1 << 30, dtype=torch.uint8, device=dev)
+        _lib.check(lib.rdkv_probe_copy(probe[0].data_ptr(), probe[1].data_ptr(), 1 << 30, _lib.stream_of(dev)))
         torch.cuda.synchronize()
-    ms_step_eager = time_region(step, args.steps, torch)
-    # The same step captured once into a HIP graph and replayed: how a decode loop issues it
-    # (the entry points neither allocate nor synchronize, so they capture as they are).
-    ms_step_graph = None
-    if not args.no_graph:
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()                               # workspace of this stream exists before capture
-            torch.cuda.synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=side):
-                step()
-            for _ in range(3):
-                graph.replay()
-            torch.cuda.synchronize()
-            ms_step_graph = time_region(graph.replay, args.steps, torch)
-        torch.cuda.current_stream().wait_stream(side)
-    ms_step = ms_step_eager if ms_step_graph is None else min(ms_step_eager, ms_step_graph)
-
-    # dominant kernel alone (streaming kernel without the merge launch)
-    ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
+        print(json.dumps({"workload": cfg.name, "ms_per_step_eager": ms_step_eager, "ms_per_launch_fused_kernel": ms_kernel,
+                          "algorithmic_bytes_per_step": algo, "streamed_bytes_per_step": cache.stream_bytes,
+                          "frac_kernel": algo / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBPS}))
+        return
     stream = _lib.stream_of(dev)
-
-    def partials_only():
-        _lib.check(lib.rdkv_decode_fused_partials(
-            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
-            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, None, None, 0,
-            ws.data_ptr(), ws.numel(), stream))
-
-    partials_only()
-    ms_kernel = time_region(partials_only, args.steps, torch)
 
     # plain copy kernel of known size (1 GiB in, 1 GiB out): reference launch for scaling the
     # hardware traffic counters of a profiler run of this same command
@@ -412,54 +715,54 @@ def main():
         except Exception as e:  # the comparison is informative; never fail the benchmark on it
             dense["sdpa_error"] = repr(e)[:200]
 
-    algo = cache.algorithmic_bytes
     gbps = algo / (ms_step * 1e-3) / 1e9
     kernel_gbps = algo / (ms_kernel * 1e-3) / 1e9
 
-    # ---- correctness of what was timed (layer 0 against the CPU oracle) -------------------
+    # ---- correctness of what was timed (layer 0 against the CPU oracle), CPU baseline -----
     check = None
     cpu_base = None
-    if not (args.no_check and args.no_cpu_baseline):
-        from oracle import rdkv_oracle as O
-        import dataclasses
-        kw = {}
-        for f in dataclasses.fields(O.PackedKVLayer):
-            v = getattr(first_pl, f.name)
-            kw[f.name] = v.detach().cpu().numpy() if torch.is_tensor(v) else v
-        ora = O.PackedKVLayer(**kw)
-        ora_nvo = first_nvo.cpu().numpy() if first_nvo is not None else None
-        q0 = qs[:cfg.H_q].cpu().numpy()
-        reps = []
-        for i in range(1 if args.no_cpu_baseline else 4):
-            t0 = time.perf_counter()
-            exp_out, exp_lse, _ = O.decode_attn_ref(q0, ora, ora_nvo)
-            reps.append(time.perf_counter() - t0)
-        got = out[:cfg.H_q].cpu().numpy()
-        err = float(np.abs(got - exp_out).max())
-        check = {"layer0_max_abs_err": err, "layer0_ref_max_abs": float(np.abs(exp_out).max()),
-                 "within_tolerance": bool(err <= 2e-3 and err <= 1e-2 * np.abs(exp_out).max())}
-        if not args.no_cpu_baseline:
-            t_cpu = float(np.median(reps[1:]))
-            layer_bytes = O.algorithmic_bytes(ora, cfg.H_q)
-            cpu_base = {"value": layer_bytes / t_cpu / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-                        "sample": f"NumPy dequantize-then-attend oracle on layer 0 of the workload "
-                                  f"({layer_bytes} algorithmic bytes), 1 warm-up + 3 repeats, median",
-                        "ms_per_layer": t_cpu * 1e3, "host_cpus": os.cpu_count()}
+    if not args.no_check:
+        check = check_layer0(first_pl, first_nvo, qs[:cfg.H_q].cpu().numpy(), out[:cfg.H_q].cpu().numpy(), torch)
+    if not args.no_cpu_baseline:
+        ora, ora_nvo = oracle_layer(first_pl, first_nvo, torch)
+        cpu_base = cpu_baseline_section(ora, ora_nvo, qs[:cfg.H_q].cpu().numpy(), cfg.H_q, torch)
+        del ora, ora_nvo
 
+    main_run = default_workload and args.config == 1
+    sequential = padded = None
+    stream_bytes, n_work, n_wg = cache.stream_bytes, cache.n_work, cache.n_groups or cache.n_work
+    if main_run:
+        del cache, step
+        torch.cuda.empty_cache()
+        sequential = sequential_section(cfg, torch, dev, replays=args.steps)
+        padded = padded_section(cfg, torch, dev, steps=args.steps)
+        torch.cuda.empty_cache()
+    configs = None
+    if main_run and not args.no_configs:
+        configs = {}
+        for idx in (int(x) for x in args.configs.split(",") if x.strip()):
+            try:
+                configs[f"C{idx}"] = compact_config(idx, args, torch, dev)
+            except Exception as e:  # the block is informative; a configuration that fails says so
+                configs[f"C{idx}"] = {"error": repr(e)[:300]}
+            torch.cuda.empty_cache()
     loop_info = None
-    if default_workload and args.config == 1 and not args.no_decode_loop:
+    if main_run and not args.no_decode_loop:
         try:
             loop_info = decode_loop_section(cfg, torch, dev)
         except Exception as e:  # informative section; never fail the benchmark on it
             loop_info = {"error": repr(e)[:300]}
 
+    traffic = MEASURED_TRAFFIC.get(args.config) if default_workload else None
     result = {
         "metric": "packed decode-attn achieved HBM GB/s (algorithmic bytes / step time)",
         "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8/fp16 codes, fp32 accumulate", "data": "synthetic",
+        "timing_mode": "eager launches (streaming launch + merge launch per step)",
         "ms_per_step_eager": ms_step_eager, "ms_per_step_graph_replay": ms_step_graph,
         "us_per_step_per_layer": ms_step * 1e3 / n_groups,
+        "us_per_layer_sequential": sequential["us_per_layer_sequential"] if sequential else None,
         "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
         "config": {"workload": cfg.name, "config_index": cfg.index, "layers": cfg.layers, "batch": cfg.batch,
                    "H_q": cfg.H_q, "H_kv": cfg.H_kv, "head_dim": cfg.D, "context": cfg.context,
@@ -467,16 +770,17 @@ def main():
                    "launch": "one fused launch + one merge launch per step over all layers",
                    "class_fractions_apply_to": "context tokens",
                    "algorithmic_bytes_per_step": algo, "algorithmic_bytes_per_layer": algo / n_groups,
-                   "streamed_bytes_per_step": cache.stream_bytes, "work_items": cache.n_work, "workgroups": cache.n_groups or cache.n_work,
+                   "streamed_bytes_per_step": stream_bytes, "work_items": n_work, "workgroups": n_wg,
                    "dense_fp16_bytes_per_layer": synth.dense_fp16_bytes(cfg),
                    "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo,
                    "build_seconds": t_build},
         "roofline": {"bound": "hbm", "achieved": kernel_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": kernel_gbps / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if default_workload else None,
+                     "traffic": traffic[0] if traffic else None,
+                     "traffic_source": (f"{traffic[1]}, a constant from that profiler run (not observed by this run)"
+                                        if traffic else None),
                      "kernel": "decode_fused_kernel", "ms_per_launch": ms_kernel,
-                     "algorithmic_bytes_per_launch": algo,
-                     "streamed_bytes_per_launch": cache.stream_bytes,
+                     "algorithmic_bytes_per_launch": algo, "streamed_bytes_per_launch": stream_bytes,
                      "ms_per_step_flushed_caches": ms_step_cold,
                      "step_GBps_flushed_caches": algo / (ms_step_cold * 1e-3) / 1e9,
                      "device_read_ceiling_GBps": probe_bytes / (ms_read * 1e-3) / 1e9,
@@ -488,6 +792,9 @@ def main():
                            required_speedup=0.7 * dense_bytes / algo,
                            speedup_vs_ideal_dense=dense["ideal_ms_at_read_ceiling"] / ms_step,
                            speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None),
+        "sequential": sequential,
+        "padded": padded,
+        "configs": configs,
         "pack": pack_info,
         "select": select_info,
         "decode_loop": loop_info,

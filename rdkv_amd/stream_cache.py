@@ -43,8 +43,11 @@ assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.ite
 
 
 
-# Caches with at most this many work items run rdkv_decode_fused as one launch by default.
-ONE_LAUNCH_MAX_WORK = 160
+# Caches with at most this many work items run rdkv_decode_fused as one launch by default.  Zero:
+# never.  Measured on single 32k-token layers (147 work items) the one-launch form is within +-1 us
+# of the two launches (24.7 / 25.5 us in one run, 26.8 / 26.5 us in another): the wait for the
+# partial stores and the ticket costs what the second launch does, so it stays an option.
+ONE_LAUNCH_MAX_WORK = 0
 
 
 def _align(x: int, a: int = 256) -> int:
@@ -499,7 +502,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     once the workspace exists (first call): one streaming launch plus one small merge launch.
     ``one_launch`` (without ``zone_c``): the streaming launch merges the partials itself (the last
     workgroup to deliver a partial of an output row combines that row; same bits); default: for
-    caches of at most ONE_LAUNCH_MAX_WORK work items, where the second launch weighs most."""
+    caches of at most ONE_LAUNCH_MAX_WORK work items (none, as shipped)."""
     lib = _lib.load()
     dev = _lib.require_device(q)
     assert q.dim() == 2 and q.shape == (cache.rows, 128) and q.stride(1) == 1, f"q must be [{cache.rows},128]"
