@@ -32,6 +32,8 @@ HBM_PEAK_GBPS = 8000.0
 # changes, which is why the JSON names its source.
 MEASURED_TRAFFIC = {
     1: (1122590720, "profiles/decode_fused_kernel_c1_llama31_8b_32k.txt"),
+    2: (2856499001, "profiles/decode_fused_kernel_c2_mistral_7b_128k.txt"),
+    3: (11113864300, "profiles/decode_fused_kernel_c3_qwen25_72b_128k.txt"),
 }
 PACK_SAMPLE_LAYERS = 8                      # layers of one sequence packed back to back for the pack throughput
 
@@ -414,7 +416,9 @@ def padded_section(cfg, torch, dev, steps=50, layers=4):
         sp = _pre_squeeze_packed((pl,))[0]
         T_v = int(sp.T_eff)
         T_old = int(sp.T_eff_k) if sp.T_eff_k > 0 else T_v
-        scores = torch.empty(cfg.H_q, T_old, dtype=torch.float32, device=dev)
+        # a scores buffer with 256-byte aligned rows, as a decode loop keeps it (the reference slices
+        # one buffer of its longest bucket, fast_decode.py:1397-1403)
+        scores = torch.empty(cfg.H_q, -(-T_old // 64) * 64, dtype=torch.float32, device=dev)[:, :T_old]
         out = torch.empty(cfg.H_q, 128, dtype=torch.float32, device=dev)
         items.append((q.float(), sp, nvo[0].contiguous() if nvo is not None else None, T_v, T_old, scores, out))
         tok, ch = stream_cache._layer_counts(pl, cfg.H_kv)

@@ -252,6 +252,109 @@ softmax_rows_kernel(const float *__restrict__ so, int64_t so_sh, const float *__
   for (int64_t t = threadIdx.x; t < n_new; t += blockDim.x) wn[h * wn_sh + t] = __expf(b[t] - mx) * inv;
 }
 
+// The same softmax for rows whose zone A+B part can be read and written 16 bytes at a time (bases
+// and row strides 16-byte aligned): a thread keeps its share of the row in registers (NV float4:
+// rows of up to 4096 * NV scores are read once and written once; mask added on the way in), or
+// (NV = 0, longer rows) streams the row three times with 16-byte accesses.  In place is fine: a
+// thread only ever rewrites elements it has read itself.  MASK_VEC: the mask rows are 16-byte
+// aligned too; otherwise (the packer's mask rows are as long as the layer has keys, any number) the
+// four mask values of a float4 of scores are loaded one by one.
+template <int NV, bool MASK_VEC>
+__global__ void __launch_bounds__(1024)
+softmax_rows_vec_kernel(const float *__restrict__ so, int64_t so_sh, const float *__restrict__ mask,
+                        int64_t mask_sh, int64_t T_old, const float *__restrict__ sn, int64_t sn_sh,
+                        int64_t n_new, float *wo, int64_t wo_sh, float *wn, int64_t wn_sh) {
+  __shared__ float scratch[16];
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const float *a = so + h * so_sh;
+  const float *m = mask ? mask + h * mask_sh : nullptr;
+  const float *b = sn ? sn + h * sn_sh : nullptr;
+  const float4 *a4 = reinterpret_cast<const float4 *>(a);
+  const float4 *m4 = reinterpret_cast<const float4 *>(m);
+  float4 *w4 = reinterpret_cast<float4 *>(wo + h * wo_sh);
+  const int64_t n4 = T_old >> 2;
+  constexpr int kKeep = NV > 0 ? NV : 1;
+  float4 x[kKeep];
+  auto mask4 = [&](int64_t i) {
+    if (MASK_VEC) return m4[i];
+    return make_float4(m[4 * i], m[4 * i + 1], m[4 * i + 2], m[4 * i + 3]);
+  };
+  auto load4 = [&](int64_t i) {
+    float4 v = a4[i];
+    if (m) {
+      const float4 k = mask4(i);
+      v.x += k.x; v.y += k.y; v.z += k.z; v.w += k.w;
+    }
+    return v;
+  };
+  float mx = -INFINITY;
+  if (NV > 0) {
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) {
+      const int64_t i = tid + (int64_t)k * 1024;
+      x[k] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+      if (i < n4) x[k] = a4[i];
+    }
+    if (m) {
+#pragma unroll
+      for (int k = 0; k < kKeep; ++k) {
+        const int64_t i = tid + (int64_t)k * 1024;
+        if (i < n4) {
+          const float4 kk = mask4(i);
+          x[k].x += kk.x; x[k].y += kk.y; x[k].z += kk.z; x[k].w += kk.w;
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) mx = fmaxf(fmaxf(mx, fmaxf(x[k].x, x[k].y)), fmaxf(x[k].z, x[k].w));
+  } else {
+    for (int64_t i = tid; i < n4; i += 1024) {
+      const float4 v = load4(i);
+      mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+    }
+  }
+  // the last T_old % 4 scores and the new zone, element by element
+  for (int64_t t = 4 * n4 + tid; t < T_old; t += 1024) mx = fmaxf(mx, a[t] + (m ? m[t] : 0.0f));
+  for (int64_t t = tid; t < n_new; t += 1024) mx = fmaxf(mx, b[t]);
+  mx = block_reduce(mx, true, scratch);
+  float sum = 0.0f;
+  if (NV > 0) {
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) {   // (slots past the row hold -inf: their weight is 0)
+      x[k].x = __expf(x[k].x - mx); x[k].y = __expf(x[k].y - mx);
+      x[k].z = __expf(x[k].z - mx); x[k].w = __expf(x[k].w - mx);
+      sum += (x[k].x + x[k].y) + (x[k].z + x[k].w);
+    }
+  } else {
+    for (int64_t i = tid; i < n4; i += 1024) {
+      const float4 v = load4(i);
+      sum += (__expf(v.x - mx) + __expf(v.y - mx)) + (__expf(v.z - mx) + __expf(v.w - mx));
+    }
+  }
+  for (int64_t t = 4 * n4 + tid; t < T_old; t += 1024) sum += __expf(a[t] + (m ? m[t] : 0.0f) - mx);
+  for (int64_t t = tid; t < n_new; t += 1024) sum += __expf(b[t] - mx);
+  sum = block_reduce(sum, false, scratch);
+  const float inv = 1.0f / sum;
+  // tail first: in place, its inputs must be read before anything of the row is rewritten by
+  // this thread (other threads never touch these elements)
+  for (int64_t t = 4 * n4 + tid; t < T_old; t += 1024)
+    wo[h * wo_sh + t] = __expf(a[t] + (m ? m[t] : 0.0f) - mx) * inv;
+  if (NV > 0) {
+#pragma unroll
+    for (int k = 0; k < kKeep; ++k) {
+      const int64_t i = tid + (int64_t)k * 1024;
+      if (i < n4) w4[i] = make_float4(x[k].x * inv, x[k].y * inv, x[k].z * inv, x[k].w * inv);
+    }
+  } else {
+    for (int64_t i = tid; i < n4; i += 1024) {
+      const float4 v = load4(i);
+      w4[i] = make_float4(__expf(v.x - mx) * inv, __expf(v.y - mx) * inv, __expf(v.z - mx) * inv,
+                          __expf(v.w - mx) * inv);
+    }
+  }
+  for (int64_t t = tid; t < n_new; t += 1024) wn[h * wn_sh + t] = __expf(b[t] - mx) * inv;
+}
+
 // ---------------------------------------------------------------------------
 // V weighted sum.  grid = (kVChunks, H_kv), block = 4 wavefronts.
 // Each class of the head's tokens (2-bit | 4-bit | 8-bit | fp16 zone B) is cut into kVChunks equal
@@ -477,9 +580,25 @@ RDKV_API int rdkv_softmax_rows(const float *scores_old, int64_t so_stride_h, con
   RDKV_REQUIRE(T_old + n_new > 0, "rdkv_softmax_rows: empty rows");
   RDKV_REQUIRE(T_old == 0 || (scores_old && w_old), "rdkv_softmax_rows: null old-zone pointer");
   RDKV_REQUIRE(n_new == 0 || (scores_new && w_new), "rdkv_softmax_rows: null new-zone pointer");
-  hipLaunchKernelGGL(softmax_rows_kernel, dim3(H_q), dim3(1024), 0, (hipStream_t)stream, scores_old, so_stride_h,
-                     mask, mask_stride_h, T_old, scores_new, sn_stride_h, n_new, w_old, wo_stride_h, w_new,
-                     wn_stride_h);
+  // 16-byte accesses need aligned rows; views that are not go element by element
+  const bool vec = T_old >= 4 && ((uintptr_t)scores_old % 16) == 0 && so_stride_h % 4 == 0 &&
+                   ((uintptr_t)w_old % 16) == 0 && wo_stride_h % 4 == 0;
+  const bool mask_vec = !mask || (((uintptr_t)mask % 16) == 0 && mask_stride_h % 4 == 0);
+#define RDKV_LAUNCH_SOFTMAX(KERNEL)                                                                             \
+  hipLaunchKernelGGL(KERNEL, dim3(H_q), dim3(1024), 0, (hipStream_t)stream, scores_old, so_stride_h, mask,      \
+                     mask_stride_h, T_old, scores_new, sn_stride_h, n_new, w_old, wo_stride_h, w_new, wn_stride_h)
+#define RDKV_LAUNCH_SOFTMAX_NV(NV)                                             \
+  do {                                                                         \
+    if (mask_vec) RDKV_LAUNCH_SOFTMAX((softmax_rows_vec_kernel<NV, true>));    \
+    else RDKV_LAUNCH_SOFTMAX((softmax_rows_vec_kernel<NV, false>));            \
+  } while (0)
+  if (!vec) RDKV_LAUNCH_SOFTMAX(softmax_rows_kernel);
+  else if (T_old <= 4096 * 2) RDKV_LAUNCH_SOFTMAX_NV(2);
+  else if (T_old <= 4096 * 8) RDKV_LAUNCH_SOFTMAX_NV(8);
+  else if (T_old <= 4096 * 16) RDKV_LAUNCH_SOFTMAX_NV(16);
+  else RDKV_LAUNCH_SOFTMAX_NV(0);
+#undef RDKV_LAUNCH_SOFTMAX_NV
+#undef RDKV_LAUNCH_SOFTMAX
   RDKV_CHECK_LAUNCH("rdkv_softmax_rows");
   return RDKV_OK;
 }

@@ -147,3 +147,48 @@ def test_k_scores_strided_rows_match_dense_rows():
                for n in ("K_2bit", "K_4bit", "K_8bit"))
     strided = kk.k_mixed_qk_dot(q, sv, T)
     torch.testing.assert_close(strided, dense, rtol=0, atol=2e-5)
+
+
+@pytest.mark.parametrize("T_old,n_new,masked,aligned", [
+    (4096, 1, True, True), (5, 0, False, True), (3, 2, True, True), (8191, 7, True, True), (8192, 0, True, True),
+    (32768, 3, True, True), (32771, 64, False, True), (65536, 1, True, True), (70001, 5, True, True),
+    (200000, 0, False, True), (4097, 9, True, False), (40000, 1, False, False), (0, 17, False, True),
+    (29563, 1, "unaligned", True), (70003, 0, "unaligned", True)])
+def test_softmax_rows_matches_the_library_softmax(T_old, n_new, masked, aligned):
+    """``rdkv_softmax_rows`` (fast_decode.py:1743-1755: mask added, softmax over [old | new], the
+    weights written back in place) against the library's fp32 softmax over the concatenated row, for
+    every row length the kernel variants split on (rows kept in registers up to 8k / 32k / 64k scores,
+    streamed beyond; lengths that are not a multiple of 4; no old zone at all), masked columns at
+    -inf, and row views that are not 16-byte aligned (the element-wise kernel).  Tolerance 2e-7
+    absolute + 2e-5 relative (fp32, another summation order)."""
+    from rdkv_amd import _lib
+    lib = _lib.load()
+    H = 5
+    g = torch.Generator().manual_seed(T_old * 31 + n_new)
+    width = T_old + n_new + 8
+    off = 0 if aligned else 1                       # rows that start one float past a 16-byte boundary
+    buf = (torch.randn(H, width + off, generator=g) * 3.0).to(DEV)
+    rows = buf[:, off:]
+    s_old, s_new = rows[:, :T_old], rows[:, T_old:T_old + n_new]
+    mask = None
+    if masked and T_old:
+        mask = torch.zeros(H, T_old + off)
+        mask[:, off:][torch.rand(H, T_old, generator=g) < 0.3] = float("-inf")
+        mask[:, off] = 0.0                           # at least one visible key per row
+        mask = mask.to(DEV)[:, off:]
+        if masked == "unaligned":                    # mask rows exactly as long as the old zone (the packer's)
+            mask = mask[:, :T_old].contiguous()
+    ref_in = torch.cat([s_old + (mask if mask is not None else 0.0), s_new], dim=1)
+    ref = torch.softmax(ref_in, dim=-1)
+    _lib.check(lib.rdkv_softmax_rows(
+        _lib.ptr(s_old), rows.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0, T_old,
+        _lib.ptr(s_new), rows.stride(0), n_new, _lib.ptr(s_old), rows.stride(0), _lib.ptr(s_new), rows.stride(0),
+        H, _lib.stream_of(torch.device(DEV))))
+    got = rows[:, :T_old + n_new]
+    assert torch.isfinite(got).all()
+    err = (got - ref).abs()
+    assert bool((err <= 2e-7 + 2e-5 * ref).all()), f"max error {float(err.max()):.3e}"
+    torch.testing.assert_close(got.sum(dim=1), torch.ones(H, device=DEV), rtol=0, atol=2e-5)
+    # nothing beyond the row was written
+    assert torch.equal(buf[:, off + T_old + n_new:].cpu(), (torch.randn(H, width + off, generator=torch.Generator().manual_seed(
+        T_old * 31 + n_new)) * 3.0)[:, off + T_old + n_new:])
