@@ -435,6 +435,20 @@ __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, i
   }
 }
 
+// v + the values of the lanes that differ from this one in bits 3, 4 and 5 of the lane index (the
+// eight token lanes that own the same channels): a rotation by 8 inside each row of 16 lanes, then
+// an exchange of neighbouring rows and of the two halves of the wavefront, all in the vector ALU
+// (three shuffles through the LDS crossbar, for each of 64 accumulators, were a third of the kernel).
+__device__ __forceinline__ float fold_token_lanes(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, true));
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
+  u = __builtin_bit_cast(unsigned, v);
+  auto t = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return __builtin_bit_cast(float, (unsigned)t[0]) + __builtin_bit_cast(float, (unsigned)t[1]);
+}
+
 template <int GB>
 __global__ void __launch_bounds__(64 * kVWaves)
 v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
@@ -485,10 +499,7 @@ v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
     for (int g = 0; g < GB; ++g) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        float v = acc[g][i];
-        v += __shfl_xor(v, 8, 64);
-        v += __shfl_xor(v, 16, 64);
-        v += __shfl_xor(v, 32, 64);
+        const float v = fold_token_lanes(acc[g][i]);
         if (sub == 0) s_acc[wave][g][16 * li + i] = v;
       }
     }
