@@ -719,6 +719,24 @@ def main():
 
             dense_step()
             dense["sdpa_ms"] = time_region(dense_step, max(3, args.steps // 5), torch)
+            # the same dense cache through this library's own dense fp16 flash-decoding kernel (two
+            # launches per layer): a dense kernel that does run near the read ceiling
+            if cfg.G in (4, 8):
+                chunks = 32
+                ws_d = torch.empty(lib.rdkv_probe_dense_decode_workspace_bytes(cfg.H_q, chunks), dtype=torch.uint8,
+                                   device=dev)
+                out_d = torch.empty(cfg.layers, cfg.H_q, cfg.D, dtype=torch.float32, device=dev)
+                q16 = qs.half().view(cfg.layers, cfg.H_q, cfg.D)
+
+                def dense_hip_step():
+                    for i in range(cfg.layers):
+                        _lib.check(lib.rdkv_probe_dense_decode(
+                            q16[i].data_ptr(), Kd[i].data_ptr(), Vd[i].data_ptr(), T, cfg.H_kv, cfg.G, chunks,
+                            out_d[i].data_ptr(), ws_d.data_ptr(), ws_d.numel(), stream))
+
+                dense_hip_step()
+                dense["dense_hip_kernel_ms"] = time_region(dense_hip_step, max(3, args.steps // 5), torch)
+                dense["dense_hip_kernel_GBps"] = dense_bytes / (dense["dense_hip_kernel_ms"] * 1e-3) / 1e9
             del Kd, Vd
         except Exception as e:  # the comparison is informative; never fail the benchmark on it
             dense["sdpa_error"] = repr(e)[:200]
@@ -799,7 +817,9 @@ def main():
         "dense_fp16": dict(dense, compression_ratio=dense_bytes / algo,
                            required_speedup=0.7 * dense_bytes / algo,
                            speedup_vs_ideal_dense=dense["ideal_ms_at_read_ceiling"] / ms_step,
-                           speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None),
+                           speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None,
+                           speedup_vs_dense_hip_kernel=(dense["dense_hip_kernel_ms"] / ms_step)
+                           if dense.get("dense_hip_kernel_ms") else None),
         "sequential": sequential,
         "padded": padded,
         "configs": configs,

@@ -519,6 +519,16 @@ int rdkv_probe_copy(const void *src, void *dst, int64_t bytes, void *stream);
 int rdkv_probe_read(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream);
 int rdkv_probe_read_stream(const void *src, int64_t bytes, int64_t span_bytes, void *sink, void *stream);
 
+/* Measurement helper, no counterpart in the reference: decode attention over an UNCOMPRESSED fp16
+ * cache, the comparator the packed path is priced against.  out[hq, :] = softmax(q[hq] . K[hq / G]^T /
+ * sqrt(128)) . V[hq / G]; q [H_kv * G, 128], K and V [H_kv, T, 128], all fp16, contiguous, 16-byte
+ * aligned; out fp32 [H_kv * G, 128]; G is 4 or 8.  The tokens of a head are cut into n_chunks pieces
+ * (one workgroup each; 32 per head is fastest for 8 heads of 32k tokens), the partials combined by a second launch.
+ * workspace: rdkv_probe_dense_decode_workspace_bytes(H_kv * G, n_chunks) bytes. */
+int64_t rdkv_probe_dense_decode_workspace_bytes(int H_q, int n_chunks);
+int rdkv_probe_dense_decode(const void *q_f16, const void *K_f16, const void *V_f16, int64_t T, int H_kv, int G,
+                            int n_chunks, float *out, void *workspace, int64_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -92,6 +92,8 @@ SIGNATURES = {
     "rdkv_probe_copy": (I, [P, P, L, P]),
     "rdkv_probe_read": (I, [P, L, L, P, P]),
     "rdkv_probe_read_stream": (I, [P, L, L, P, P]),
+    "rdkv_probe_dense_decode_workspace_bytes": (L, [I, I]),
+    "rdkv_probe_dense_decode": (I, [P, P, P, L, I, I, I, P, P, L, P]),
 }
 
 _lib: Optional[ctypes.CDLL] = None
