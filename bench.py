@@ -516,17 +516,18 @@ def decode_loop_section(cfg, torch, dev, tokens=48):
         pool_padding="reflect", v_bit_options=torch.tensor([0., 2, 4, 8, 16]),
         k_bit_options=torch.tensor([0., 2, 4, 8]), epsilon_v=ks.DEFAULT_EPSILON_V, epsilon_k=ks.DEFAULT_EPSILON_K)
     n_bw = 272
-    for _ in range(2):
-        with contextlib.redirect_stdout(io.StringIO()):       # the loop logs one event line per block
-            ids, report = bw.greedy_decode_blockwise(
-                model=model, dual_cache=cache, next_token_logits=first, max_new_tokens=n_bw, eos_token_ids=[],
-                primary_device=dev, decode_position_start=sc.context, config=conf)
-    ts = report["per_token_timestamps_ms"]
-    steps = sorted(b - a for a, b in zip(ts, ts[1:]))
-    res["blockwise"] = {"tokens": len(ids), "block_size": 128, "block_budget_tokens": 16,
-                        "ms_per_token_avg": report["avg_tpot_ms"], "ms_per_token_median": steps[len(steps) // 2],
-                        "ms_slowest_step": steps[-1], "compressed_blocks": report["num_compressed_decode_blocks"],
-                        "final_flush_ms": report["final_flush_time_ms"]}
+    for name, graph in (("blockwise", False), ("blockwise_graph", True)):
+        for _ in range(2):
+            with contextlib.redirect_stdout(io.StringIO()):       # the loop logs one event line per block
+                ids, report = bw.greedy_decode_blockwise(
+                    model=model, dual_cache=cache, next_token_logits=first, max_new_tokens=n_bw, eos_token_ids=[],
+                    primary_device=dev, decode_position_start=sc.context, config=conf, use_cuda_graph=graph)
+        ts = report["per_token_timestamps_ms"]
+        steps = sorted(b - a for a, b in zip(ts, ts[1:]))
+        res[name] = {"tokens": len(ids), "block_size": 128, "block_budget_tokens": 16,
+                     "ms_per_token_avg": report["avg_tpot_ms"], "ms_per_token_median": steps[len(steps) // 2],
+                     "ms_slowest_step": steps[-1], "compressed_blocks": report["num_compressed_decode_blocks"],
+                     "final_flush_ms": report["final_flush_time_ms"]}
     return res
 
 

@@ -391,8 +391,13 @@ typedef struct RdkvTailScores {   /* online block scores of blockwise decode, se
   int64_t self_stride_h;
   float  *next_scores;            /* likewise; may be NULL while q_block_start < block */
   int64_t next_stride_h;
-  int32_t q_block_start;          /* first zone-C token of the block the step's query belongs to */
+  int32_t q_block_start;          /* first zone-C token of the block the step's query belongs to; negative:
+                                     taken on the device as (row_dev[0] / block) * block, so that a replayed
+                                     graph needs no host value per step (next_scores is then required) */
   int32_t block;                  /* block size in tokens */
+  int64_t q_rotated_stride_tok;   /* 0: q_rotated_out holds this step's rows [rows, 128].  Otherwise (elements)
+                                     q_rotated_out is a buffer [rows, tokens, 128] and the step's rows go to
+                                     token row_dev[0] of it: again no host value per step */
 } RdkvTailScores;
 int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, int n_work, int G,
                                           const void *q, int q_dtype, int64_t q_stride_row,

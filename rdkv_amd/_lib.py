@@ -18,7 +18,8 @@ import torch
 class RdkvTailScores(ctypes.Structure):
     """``RdkvTailScores`` of include/rdkv.h (read by the library during the call)."""
     _fields_ = [("self_scores", c_void_p), ("self_stride_h", c_int64), ("next_scores", c_void_p),
-                ("next_stride_h", c_int64), ("q_block_start", ctypes.c_int32), ("block", ctypes.c_int32)]
+                ("next_stride_h", c_int64), ("q_block_start", ctypes.c_int32), ("block", ctypes.c_int32),
+                ("q_rotated_stride_tok", c_int64)]
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG, "librdkv_hip.so")

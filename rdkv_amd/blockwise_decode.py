@@ -555,8 +555,14 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     (``_compress_block``) and joins every layer's cache (``extend_stream_cache``); at the end the
     remaining blocks are flushed, the last one with its own causal scores.
 
-    The reference needs its fixed-slot bank to replay this loop from graphs; that variant is not
-    built: ``use_cuda_graph=True`` raises ``NotImplementedError``."""
+    ``use_cuda_graph`` (blockwise_decode.py:1991-2117): the step is replayed from a HIP graph.  The
+    reference needs a bank of fixed-shape slots for that, because the shapes of its tensors are the
+    lengths of its segments; here the lengths are data in the unit / work tables and the step's own
+    scalars (token, position, tail row, tail length, the block the query belongs to) live on the
+    device and are advanced by the step itself, so ONE graph of the whole step (every layer, LM head,
+    argmax) serves every step between two compressions.  A compression adds units to every layer's
+    tables, so the first step after it runs eagerly and the graph is recorded again (once per block
+    of tokens)."""
     from .fast_decode import (_argmax_advance, _layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
                               _silu_linear_row, pre_extract_weights)
     from .stream_cache import decode_attn_fused, extend_stream_caches
@@ -566,8 +572,6 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     dev = torch.device(primary_device)
     if dev.type != "cuda":
         raise RuntimeError("blockwise packed decode requires CUDA")
-    if use_cuda_graph:
-        raise NotImplementedError("graph replay of the blockwise loop is not built; run it eagerly")
     eos_set = {int(t) for t in eos_token_ids if t is not None}
     W = pre_extract_weights(model)
     model_dtype = next(model.parameters()).dtype
@@ -655,6 +659,8 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
             s_next.zero_()
         pending_start += target_len
         pending_len = remain
+        write_row.fill_(pending_len)          # the step's device-held scalars follow the shortened tail
+        n_tail.fill_(pending_len + 1)
         validate_order()
         record_memory("final_flush" if is_final_flush else f"compressed_block_{block_id}")
 
@@ -667,49 +673,66 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     ev0 = torch.cuda.Event(enable_timing=True)
     ev0.record()
 
+    def run_step(check: bool) -> None:
+        """One decode step; everything that changes from step to step is read from device tensors
+        (next_token, position_ids, write_row, n_tail) and advanced at the end, so the same calls
+        run eagerly or are recorded once and replayed."""
+        h = W.embed_tokens(next_token)
+        cos, sin = W.rotary_emb(h, position_ids)
+        cos_half, sin_half = cos.view(D)[:D // 2], sin.view(D)[:D // 2]
+        delta = None
+        for layer, lw in enumerate(W.layers):
+            qkv, h = _norm_linear_row(h, delta, lw.input_ln_weight, lw.input_ln_eps, lw.qkv_weight, lw.qkv_bias)
+            q, k, v = qkv.split(lw.qkv_split_sizes, dim=-1)
+            q_2d, k_2d, v_2d = q.view(h_q, D), k.view(h_kv, D), v.view(h_kv, D)
+            if lw.q_norm_weight is not None:
+                q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
+            if lw.k_norm_weight is not None:
+                k_2d = _rms_norm(k_2d, lw.k_norm_weight, lw.qk_norm_eps)
+            rows = pending_kv[layer][0]
+            # q and k are rotated inside the attention launches; the merge launch appends k | v to
+            # the raw tail at row write_row and leaves the rotated query (kept for the channel
+            # scores) in that row of pending_q
+            decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse, rope=(cos_half, sin_half),
+                              zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights,
+                              append=(k_2d, v_2d, write_row), q_rotated_out=pending_q[layer],
+                              # block scores from the tail's weights (blockwise_decode.py:2085-2109); the
+                              # block of the query follows from write_row on the device
+                              tail_scores=(self_scores[layer], next_scores[layer], None, block))
+            if check and not torch.isfinite(attn_out).all():
+                raise FloatingPointError(f"non-finite attention output at layer {layer}")
+            o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)
+            gate_up, h = _norm_linear_row(h, o, lw.post_ln_weight, lw.post_ln_eps, lw.gate_up_weight)
+            gate, up = gate_up.split(lw.gate_up_split_sizes, dim=-1)
+            delta = _silu_linear_row(gate, up, lw.down_proj_weight)
+        hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
+        logits = _linear_row(hidden, W.lm_head_weight)
+        _argmax_advance(logits, next_token, position_ids, write_row, n_tail)
+
+    position_ids.fill_(int(decode_position_start))
+    write_row.zero_()
+    n_tail.fill_(1)
+    graph = None                  # the step recorded for the current set of unit tables
+    eager_steps = 0               # steps run eagerly since the tables last changed
     with torch.inference_mode():
         for step in range(max_new_tokens):
             token_id = int(next_token.item())
             if token_id in eos_set:
                 break
             generated.append(token_id)
-            position_ids.fill_(decode_position_start + step)
-            h = W.embed_tokens(next_token)
-            cos, sin = W.rotary_emb(h, position_ids)
-            cos_half, sin_half = cos.view(D)[:D // 2], sin.view(D)[:D // 2]
-            write_pos = pending_len
-            if write_pos >= capacity:
-                raise RuntimeError(f"pending decode cache overflow ({write_pos} >= {capacity})")
-            current_len = write_pos + 1
-            q_block_start = (write_pos // block) * block
-            write_row.fill_(write_pos)
-            n_tail.fill_(current_len)
-            delta = None
-            for layer, lw in enumerate(W.layers):
-                qkv, h = _norm_linear_row(h, delta, lw.input_ln_weight, lw.input_ln_eps, lw.qkv_weight, lw.qkv_bias)
-                q, k, v = qkv.split(lw.qkv_split_sizes, dim=-1)
-                q_2d, k_2d, v_2d = q.view(h_q, D), k.view(h_kv, D), v.view(h_kv, D)
-                if lw.q_norm_weight is not None:
-                    q_2d = _rms_norm(q_2d, lw.q_norm_weight, lw.qk_norm_eps)
-                if lw.k_norm_weight is not None:
-                    k_2d = _rms_norm(k_2d, lw.k_norm_weight, lw.qk_norm_eps)
-                rows = pending_kv[layer][0]
-                # q and k are rotated inside the attention launches; the merge launch appends k | v to
-                # the raw tail and leaves the rotated query (kept for the channel scores) in pending_q
-                decode_attn_fused(caches[layer], q_2d, out=attn_out, lse=lse, rope=(cos_half, sin_half),
-                                  zone_c=(rows[:, :, :D], rows[:, :, D:], n_tail), zone_c_weights=tail_weights,
-                                  append=(k_2d, v_2d, write_row), q_rotated_out=pending_q[layer][:, write_pos, :],
-                                  # block scores from the tail's weights (blockwise_decode.py:2085-2109)
-                                  tail_scores=(self_scores[layer], next_scores[layer], q_block_start, block))
+            if pending_len >= capacity:
+                raise RuntimeError(f"pending decode cache overflow ({pending_len} >= {capacity})")
+            if use_cuda_graph and eager_steps >= 1:
+                if graph is None:     # the eager step before this one warmed every workspace
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        run_step(False)
+                graph.replay()
                 if config.correctness_check and not torch.isfinite(attn_out).all():
-                    raise FloatingPointError(f"non-finite attention output at layer {layer}")
-                o = _linear_row(attn_out.view(1, 1, W.attn_output_dim), lw.o_proj_weight)
-                gate_up, h = _norm_linear_row(h, o, lw.post_ln_weight, lw.post_ln_eps, lw.gate_up_weight)
-                gate, up = gate_up.split(lw.gate_up_split_sizes, dim=-1)
-                delta = _silu_linear_row(gate, up, lw.down_proj_weight)
-            hidden = _rms_norm(h, W.final_norm_weight, W.final_norm_eps, delta=delta, residual_out=h)
-            logits = _linear_row(hidden, W.lm_head_weight)
-            _argmax_advance(logits, next_token)
+                    raise FloatingPointError("non-finite attention output in the last layer")
+            else:
+                run_step(config.correctness_check)
+                eager_steps += 1
             pending_len += 1
             ev = torch.cuda.Event(enable_timing=True)
             ev.record()
@@ -717,6 +740,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
             record_memory(f"token_{len(generated)}")
             if pending_len == capacity:
                 compress_prefix(block, query_offset=block, query_len=block, is_final_flush=False, causal=False)
+                graph, eager_steps = None, 0      # the unit tables moved: record the step again
 
     t_pre_flush = _sync_stamp(dev)
     # a complete block followed by an incomplete successor: the successor's queries drain it
@@ -734,7 +758,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     decode_ms = (t_pre_flush - t_decode0) * 1000.0
     flush_ms = (t_flush1 - t_flush0) * 1000.0
     report: Dict[str, Any] = {
-        "decode_blockwise_rdkv": True, "decode_cuda_graph": False, "decode_cuda_graph_active_slot_variants": [],
+        "decode_blockwise_rdkv": True, "decode_cuda_graph": bool(use_cuda_graph), "decode_cuda_graph_active_slot_variants": [],
         "decode_block_size": block, "decode_block_budget_tokens": config.block_budget_tokens,
         "generated_tokens": n_gen, "block_events": block_events, "memory_trace": memory_trace,
         "per_token_timestamps_ms": [ev0.elapsed_time(e) for e in token_events],

@@ -942,11 +942,15 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
   const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
   // the query (and its rotation table) is fetched before the merge so that the two overlap
   const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
+  // the zone-C row of this step (device-held, so that a replayed graph needs nothing from the host)
+  const int64_t step_row = ap.k ? ap.row_dev[0] : 0;
+  const int q_block_start = ts.q_block_start >= 0 || ts.block <= 0 ? ts.q_block_start
+                                                                    : (int)(step_row / ts.block) * ts.block;
   if (ap.k) {
     // The step's own token joins zone C here (first wavefront; the others go on): k rotated and
     // rounded to its storage type as the in-place rotation stores it, k and v widened to fp32.
     // The barriers between here and the token loop make the row visible to every wavefront.
-    const int64_t row = ap.row_dev[0];
+    const int64_t row = step_row;
     if (row >= 0 && row < ap.capacity && tid < 64) {
       const int64_t ko = (int64_t)kv_row * ap.k_stride_h, vo = (int64_t)kv_row * ap.v_stride_h;
       const float lo = rdkv_load_as_float_nobranch(ap.k, ap.dtype, ko + tid);
@@ -997,7 +1001,9 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
       }
       qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
       // the rotated query as the in-place rotation would have left it, for callers that keep it
-      if (q_rot_out) rdkv_store_from_float(q_rot_out, q_dtype, (int64_t)(q_row + (i >> 7)) * q_rot_stride + c, v);
+      if (q_rot_out)
+        rdkv_store_from_float(q_rot_out, q_dtype,
+                              (int64_t)(q_row + (i >> 7)) * q_rot_stride + step_row * ts.q_rotated_stride_tok + c, v);
     }
   }
   __syncthreads();
@@ -1123,8 +1129,8 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
       }
       // online block scores of blockwise decode (blockwise_decode.py:2085-2109): the query's weights
       // on its own block, and on the first block when the query belongs to the second
-      if (ts.self_scores && t >= ts.q_block_start) ts.self_scores[(int64_t)kv_row * ts.self_stride_h + t] += s;
-      if (ts.next_scores && ts.q_block_start >= ts.block && t < ts.block)
+      if (ts.self_scores && t >= q_block_start) ts.self_scores[(int64_t)kv_row * ts.self_stride_h + t] += s;
+      if (ts.next_scores && q_block_start >= ts.block && t < ts.block)
         ts.next_scores[(int64_t)kv_row * ts.next_stride_h + t] += s;
     }
   }
@@ -1311,7 +1317,7 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
   return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, n_units, n_work, G, q, q_dtype, q_stride_row,
                              rope_cos, rope_sin, rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, n_new,
                              n_new_per_unit, out, out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row,
-                             workspace, workspace_bytes, none, nullptr, 0, RdkvTailScores{nullptr, 0, nullptr, 0, 0, 0},
+                             workspace, workspace_bytes, none, nullptr, 0, RdkvTailScores{nullptr, 0, nullptr, 0, 0, 0, 0},
                              stream);
 }
 
@@ -1330,13 +1336,15 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
   RDKV_REQUIRE(capacity >= 0 && capacity <= 0x7fffffffLL, "%s: bad zone-C capacity", fn);
   RDKV_REQUIRE(!zone_c_weights || zone_c_weights_stride_row >= capacity,
                "%s: rows of the zone-C weights are shorter than the buffer", fn);
-  RdkvTailScores tail = {nullptr, 0, nullptr, 0, 0, 0};
+  RdkvTailScores tail = {nullptr, 0, nullptr, 0, 0, 0, 0};
   if (tail_scores) {
     tail = *tail_scores;
     RDKV_REQUIRE(zone_c_weights, "%s: the block scores are summed from zone_c_weights", fn);
-    RDKV_REQUIRE(tail.self_scores && tail.q_block_start >= 0 && tail.block >= 1 &&
-                     (tail.next_scores || tail.q_block_start < tail.block),
+    RDKV_REQUIRE(tail.self_scores && tail.block >= 1 &&
+                     (tail.next_scores || (tail.q_block_start >= 0 && tail.q_block_start < tail.block)),
                  "%s: bad tail score arguments", fn);
+    RDKV_REQUIRE(tail.q_rotated_stride_tok >= 0 && (tail.q_rotated_stride_tok == 0 || q_rotated_out),
+                 "%s: bad stride of the rotated-query buffer", fn);
   }
   const ZcAppend ap = {k_step, v_step, k_stride_h, v_stride_h, row_dev, capacity, kv_dtype};
   return launch_merge_zone_c(fn, units, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,

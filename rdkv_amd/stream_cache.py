@@ -498,7 +498,10 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     q_block_start, block) (with ``append`` and ``zone_c_weights``; fp32 [rows / G, >= tokens]):
     the merge launch also adds the new tokens' weights, summed over a KV head's query heads, to
     ``self_scores[:, q_block_start:]`` and, when ``q_block_start >= block``, to
-    ``next_scores[:, :block]`` - what ``rdkv_tail_scores`` does as a launch of its own.  Graph-capturable
+    ``next_scores[:, :block]`` - what ``rdkv_tail_scores`` does as a launch of its own;
+    ``q_block_start=None`` lets the launch derive it from ``row`` (``row // block * block``) and a
+    3-D ``q_rotated_out`` [rows, tokens, 128] receives the rotated query at token ``row``: the forms
+    a replayed graph uses, with nothing per step coming from the host.  Graph-capturable
     once the workspace exists (first call): one streaming launch plus one small merge launch.
     ``one_launch`` (without ``zone_c``): the streaming launch merges the partials itself (the last
     workgroup to deliver a partial of an output row combines that row; same bits); default: for
@@ -571,9 +574,17 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
             assert zone_c_weights.dtype == torch.float32 and zone_c_weights.dim() == 2
             assert zone_c_weights.stride(1) == 1 and zone_c_weights.shape[0] == cache.rows
             assert zone_c_weights.shape[1] >= n_new, f"zone_c_weights rows must hold {n_new} tokens"
+        q_rot_tok = 0
         if q_rotated_out is not None:
             _lib.require_device(q_rotated_out)
-            assert q_rotated_out.shape == q.shape and q_rotated_out.dtype == q.dtype and q_rotated_out.stride(1) == 1
+            assert q_rotated_out.dtype == q.dtype and q_rotated_out.stride(-1) == 1
+            if q_rotated_out.dim() == 3:      # [rows, tokens, 128]: the step's rows go to token row[0]
+                assert tail_scores is not None, "a per-token buffer of rotated queries comes with tail_scores"
+                assert q_rotated_out.shape[0] == q.shape[0] and q_rotated_out.shape[2] == 128
+                assert q_rotated_out.shape[1] >= n_new, f"rotated-query buffer must hold {n_new} tokens"
+                q_rot_tok = q_rotated_out.stride(1)
+            else:
+                assert q_rotated_out.shape == q.shape
         tail = None
         if tail_scores is not None:
             self_s, next_s, q_block_start, block = tail_scores
@@ -583,9 +594,10 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                     _lib.require_device(t)
                     assert t.dtype == torch.float32 and t.dim() == 2 and t.shape[0] == n_kv_rows and t.stride(1) == 1
                     assert t.shape[1] >= width, f"score rows must hold {width} tokens"
-            assert next_s is not None or q_block_start < block
+            assert next_s is not None or (q_block_start is not None and q_block_start < block)
             tail = _lib.RdkvTailScores(self_s.data_ptr(), self_s.stride(0), _lib.ptr(next_s),
-                                       next_s.stride(0) if next_s is not None else 0, int(q_block_start), int(block))
+                                       next_s.stride(0) if next_s is not None else 0,
+                                       -1 if q_block_start is None else int(q_block_start), int(block), int(q_rot_tok))
         _lib.check(lib.rdkv_decode_fused_merge_zone_c_append(
             cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,

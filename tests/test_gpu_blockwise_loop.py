@@ -151,10 +151,6 @@ def test_eos_stops_and_flushes(setup):
     stop = ids.index(ids[11])
     assert out == ids[:stop] and report["generated_tokens"] == stop
     assert report["coverage"][-1][1] == stop - 1 if stop else report["coverage"] == []
-    with pytest.raises(NotImplementedError):
-        bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
-                                   max_new_tokens=4, eos_token_ids=[], primary_device=torch.device(DEV),
-                                   decode_position_start=T_PROMPT, config=_config(8, 2), use_cuda_graph=True)
     with pytest.raises(RuntimeError):
         bw.greedy_decode_blockwise(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1],
                                    max_new_tokens=4, eos_token_ids=[], primary_device=torch.device("cpu"),
@@ -184,3 +180,31 @@ def test_tail_scores_kernel_matches_tensor_expressions():
                                         _lib.stream_of(torch.device(DEV))))
         torch.testing.assert_close(self_s, exp_self, rtol=1e-6, atol=1e-6)
         torch.testing.assert_close(next_s, exp_next, rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("n_tokens,block", [(45, 8), (16, 8), (3, 8), (70, 16)])
+def test_graph_replayed_loop_equals_the_eager_loop(setup, n_tokens, block):
+    """``use_cuda_graph=True`` (blockwise_decode.py:1991-2117): the step replayed from a HIP graph,
+    recorded again after every compression, gives the eager loop's tokens, compression events and
+    report - through several compressions, for a run that ends on a block boundary, one shorter
+    than the first graph, and with an EOS in the middle; and again on a second run over the same
+    prompt cache."""
+    model, prompt, pre, cache = setup
+    common = dict(model=model, dual_cache=cache, next_token_logits=pre.logits[0, -1], max_new_tokens=n_tokens,
+                  primary_device=torch.device(DEV), decode_position_start=T_PROMPT, config=_config(block, 4))
+    ids_e, rep_e = bw.greedy_decode_blockwise(eos_token_ids=[], **common)
+    for run in range(2):
+        ids_g, rep_g = bw.greedy_decode_blockwise(eos_token_ids=[], use_cuda_graph=True, **common)
+        assert ids_g == ids_e, f"run {run}: tokens differ"
+        assert rep_g["decode_cuda_graph"] is True and rep_e["decode_cuda_graph"] is False
+        assert rep_g["coverage"] == rep_e["coverage"]
+        for eg, ee in zip(rep_g["block_events"], rep_e["block_events"]):
+            for key in ("block_id", "token_start", "token_end", "query_source_block", "is_final_flush", "query_mode",
+                        "logical_allocated_bits_per_layer", "v_bit_histogram", "k_bit_histogram", "physical_bytes"):
+                assert eg[key] == ee[key], (key, eg[key], ee[key])
+        assert len(rep_g["per_token_timestamps_ms"]) == len(ids_g)
+    if len(ids_e) > 6:
+        eos = ids_e[len(ids_e) // 2]
+        stop = ids_e.index(eos)
+        ids_s, rep_s = bw.greedy_decode_blockwise(eos_token_ids=[eos], use_cuda_graph=True, **common)
+        assert ids_s == ids_e[:stop] and rep_s["generated_tokens"] == stop
