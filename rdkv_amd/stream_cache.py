@@ -301,9 +301,13 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             ks, kz = ks.contiguous(), kz.contiguous()
         # per head: the largest K channel scale and the largest V token scale (the kernel keeps its
         # fp16 operands in range with them)
-        zero = torch.zeros(H_kv, dtype=torch.float32, device=dev)
-        scale_max.append(torch.stack([ks.float().abs().amax(dim=1) if Dp else zero,
-                                      vs.float().abs().amax(dim=1) if vs.numel() else zero], dim=1))
+        # (one reduction launch each, written straight into the entry's rows of one buffer)
+        sm = torch.zeros(2, H_kv, dtype=torch.float32, device=dev)
+        if Dp:
+            torch.linalg.vector_norm(ks, ord=float("inf"), dim=1, dtype=torch.float32, out=sm[0])
+        if vs.numel():
+            torch.linalg.vector_norm(vs, ord=float("inf"), dim=1, dtype=torch.float32, out=sm[1])
+        scale_max.append(sm)
         if pl.K_ch_perm_padded_idx_per_head is not None:
             perm = pl.K_ch_perm_padded_idx_per_head.to(torch.int64).contiguous()
             perm_sh = perm.stride(0)
@@ -328,7 +332,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
         # the temporaries stay alive until the relayout kernels have run
         keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
-    scale_max_np = torch.cat(scale_max).cpu().numpy().astype(np.float32)   # (synchronizes)
+    scale_max_np = torch.stack(scale_max).transpose(1, 2).reshape(-1, 2).cpu().numpy().astype(np.float32)  # (synchronizes)
     torch.cuda.current_stream(dev).synchronize()
     del keep_alive
     return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
