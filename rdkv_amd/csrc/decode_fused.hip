@@ -885,14 +885,18 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
 // stored and loaded at device scope): 0.8-1.5 us faster on a single 32k-token layer (24.7 against
 // 25.5 us per call), slower from about 200 work items on (the step of a whole model: 0.183 against
 // 0.182 ms), because every workgroup then waits for its stores and a ticket before it may leave.
-__global__ void __launch_bounds__(256)
+// One thread per output column (G * 128 threads): every thread's accumulator loads are the ones
+// requested ahead of the barrier, so the whole merge is two dependent memory round trips (the
+// unit's descriptor, then all partial values at once); with a fixed 256 threads a G = 4 unit
+// paid two more for its second column.
+__global__ void __launch_bounds__(1024)
 merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
   __shared__ float scratch[2 * kMergeMaxK * 8];
   const RdkvUnit *u = units + blockIdx.x;
   if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
-  merge_unit(partials, u->work_begin, u->work_count, G, u->q_row, out, out_stride, lse, threadIdx.x, 256,
-                    scratch);
+  merge_unit(partials, u->work_begin, u->work_count, G, u->q_row, out, out_stride, lse, threadIdx.x,
+             (int)blockDim.x, scratch);
 }
 
 // Merge of a unit's partials followed by the attention over its decode-appended tokens
@@ -1227,7 +1231,7 @@ RDKV_API int rdkv_decode_fused_merge(const RdkvUnit *units, int n_units, int n_w
   if (rc != RDKV_OK) return rc;
   if (n_units == 0) return RDKV_OK;
   RDKV_REQUIRE(out, "rdkv_decode_fused_merge: null out");
-  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(256), 0, (hipStream_t)stream, units,
+  hipLaunchKernelGGL(merge_kernel, dim3(n_units), dim3(128 * G), 0, (hipStream_t)stream, units,
                      (const float *)workspace, G, out, out_stride_row, lse);
   RDKV_CHECK_LAUNCH("rdkv_decode_fused_merge");
   return RDKV_OK;
