@@ -584,8 +584,9 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
 // D == 128, rows 16-byte aligned: sixteen lanes per canvas row (eight channels each, one 16-byte
 // load), four rows per wavefront step, the next step's rows in flight while the current ones are
 // quantized.  A lane's channels never change, so their parameters and slots live in registers;
-// codes go to their sorted slots in a per-row LDS buffer and the row's sixteen lanes assemble the
-// packed bytes from it.
+// codes go to their sorted slots in a per-row LDS buffer (one byte per slot; a pruned channel's
+// zero goes to a spare byte, so nothing branches) and each of the row's sixteen lanes assembles
+// four consecutive packed bytes of every class from aligned dwords of that buffer.
 __global__ void __launch_bounds__(256)
 k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
                          const int32_t *__restrict__ order, int64_t order_stride_h,
@@ -598,7 +599,13 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
   extern __shared__ float smem[];
   const int h = blockIdx.y;
   const int Dp = n2p + n4p + n8;
-  const int Dp4 = (Dp + 3) & ~3;
+  // Slot buffer of a row: the four quarter ranges of the 2-bit class, the two halves of the 4-bit
+  // class and the 8-bit class each start on a 4-byte boundary, so that four consecutive output
+  // bytes are assembled from aligned dwords; then a spare byte for pruned channels.
+  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
+  const int sub2p = (sub2 + 3) & ~3, sub4p = (sub4 + 3) & ~3;
+  const int o4 = 4 * sub2p, o8 = o4 + 2 * sub4p;
+  const int Dp4 = o8 + ((n8 + 3) & ~3) + 4;
   const int tv = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2], n16 = counts[4 * h + 3];
   const bool has_pad = tv < max_tv || n16 < max_n16;   // zero rows of the canvas join the min/max
   const int64_t max_tk = max_tv + max_n16;
@@ -628,7 +635,11 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
       c_scale[ch] = p.scale;
       c_zp[ch] = p.zp;
       c_qmax[ch] = qmax;
-      c_slot[ch] = s;
+      int at;      // where sorted slot s lives in the row's slot buffer
+      if (s < n2p) at = (s / sub2) * sub2p + s % sub2;
+      else if (s < n2p + n4p) at = o4 + ((s - n2p) / sub4) * sub4p + (s - n2p) % sub4;
+      else at = o8 + (s - n2p - n4p);
+      c_slot[ch] = at;
     }
     if (blockIdx.x == 0) {
       scale_out[(int64_t)h * Dp + s] = __float2half_rn(p.scale);
@@ -636,9 +647,7 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
     }
   }
   __syncthreads();
-  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
-  const int rowbytes = sub2 + sub4 + n8;
-  if (rowbytes == 0) return;
+  if (sub2 + sub4 + n8 == 0) return;
   RdkvQParams qp[8];
   float qm[8];
   int sl[8];
@@ -650,6 +659,7 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
     qp[e].zp = sl[e] >= 0 ? c_zp[ch] : 0.0f;
     qp[e].inv = __fdiv_rn(1.0f, qp[e].scale);
     qm[e] = sl[e] >= 0 ? c_qmax[ch] : 0.0f;
+    if (sl[e] < 0) sl[e] = Dp4 - 4;          // a pruned channel's code is 0 (qmax 0): the spare byte takes it
   }
   const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;
   const int64_t t1 = (t0 + rows_per_block < max_tk) ? t0 + rows_per_block : max_tk;
@@ -674,25 +684,48 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
     const int64_t t = tb + sub;
     fetch(t + step, nxt);
     if (t < t1) {
+      float x[8];
+      uint32_t code[8];
+      bool near[8], any = false;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        if (sl[e] >= 0) rb[sl[e]] = (uint8_t)rdkv_qcode(__half2float(__ushort_as_half(cur.hw[e])), qp[e], qm[e]);
+        x[e] = __half2float(__ushort_as_half(cur.hw[e]));
+        code[e] = rdkv_qcode_estimate(x[e], qp[e], qm[e], near[e]);
+        any = any || near[e];
       }
+      if (any) {                     // about one value in 2500 needs the exact quotient
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (near[e]) code[e] = rdkv_qcode_exact(x[e], qp[e], qm[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rb[sl[e]] = (uint8_t)code[e];
     }
     __builtin_amdgcn_wave_barrier();
     if (t < t1) {
       const int64_t row = (int64_t)h * max_tk + t;
-      for (int j = l; j < rowbytes; j += 16) {
-        if (j < sub2) {
-          K2[row * sub2 + j] = (uint8_t)(rb[j] | (rb[j + sub2] << 2) | (rb[j + 2 * sub2] << 4) | (rb[j + 3 * sub2] << 6));
-        } else if (j < sub2 + sub4) {
-          const int i = j - sub2;
-          K4[row * sub4 + i] = (uint8_t)(rb[n2p + i] | (rb[n2p + i + sub4] << 4));
+      const uint32_t *rb32 = reinterpret_cast<const uint32_t *>(rb);
+      // four bytes j0 .. j0+3 of an n-byte output row: one dword store where the address allows it
+      auto put = [&](uint8_t *dst, int n, int j0, uint32_t v) {
+        if (j0 + 4 <= n && (reinterpret_cast<uintptr_t>(dst + j0) & 3) == 0) {
+          *reinterpret_cast<uint32_t *>(dst + j0) = v;
         } else {
-          const int i = j - sub2 - sub4;
-          K8[row * (int64_t)n8 + i] = rb[n2p + n4p + i];
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+            if (j0 + k < n) dst[j0 + k] = (uint8_t)(v >> (8 * k));
         }
+      };
+      const int j0 = 4 * l;
+      // (codes of the 2- and 4-bit classes are below 4 and 16: the shifts never carry into the next byte)
+      if (j0 < sub2) {
+        const int w = j0 >> 2, q = sub2p >> 2;
+        put(K2 + row * sub2, sub2, j0, rb32[w] | (rb32[w + q] << 2) | (rb32[w + 2 * q] << 4) | (rb32[w + 3 * q] << 6));
       }
+      if (j0 < sub4) {
+        const int w = (o4 + j0) >> 2;
+        put(K4 + row * sub4, sub4, j0, rb32[w] | (rb32[w + (sub4p >> 2)] << 4));
+      }
+      for (int j = j0; j < n8; j += 64) put(K8 + row * (int64_t)n8, n8, j, rb32[(o8 + j) >> 2]);
     }
     __builtin_amdgcn_wave_barrier();
     cur = nxt;
@@ -886,7 +919,8 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
     RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
     if (rows16) {
       const int rows_d128 = 256;
-      const size_t lds_d128 = (size_t)128 * 16 + 16 * (size_t)((Dp + 3) & ~3);
+      const size_t lds_d128 = (size_t)128 * 16 +
+                              16 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
       hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, rows_d128), H_kv), dim3(256),
                          lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts,
                          max_tv, max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,

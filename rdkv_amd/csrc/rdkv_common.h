@@ -113,6 +113,15 @@ __device__ __forceinline__ uint32_t rdkv_qcode_exact(float x, RdkvQParams p, flo
   float v = __fadd_rn(__fdiv_rn(x, p.scale), p.zp);
   return (uint32_t)rintf(fminf(fmaxf(v, 0.0f), qmax));
 }
+// The estimate of rdkv_qcode alone: the code from x * (1 / scale) + zp, and whether it lies so close
+// to a rounding boundary that the exact quotient has to decide (callers that quantize several
+// values collect the flags and branch once).
+__device__ __forceinline__ uint32_t rdkv_qcode_estimate(float x, const RdkvQParams &p, float qmax, bool &near) {
+  const float t = fmaf(x, p.inv, p.zp);
+  const float r = rintf(fminf(fmaxf(t, 0.0f), qmax));
+  near = fabsf(fabsf(t - r) - 0.5f) < 2e-4f;
+  return (uint32_t)r;
+}
 __device__ __forceinline__ uint32_t rdkv_qcode(float x, RdkvQParams p, float qmax) {
   const float t = fmaf(x, p.inv, p.zp);
   const float r = rintf(fminf(fmaxf(t, 0.0f), qmax));
