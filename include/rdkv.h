@@ -84,7 +84,7 @@ int rdkv_k_quantize_pack(const void *k_f16, int64_t k_row_stride, int64_t T, int
  * [H_kv, n2p+n4p+n8] padded sorted slot -> source channel, -1 = pad (shared-max widths).
  * Outputs, all head-stacked and zero-padded as the reference lays them out:
  * V2 [H_kv,mN2,D/4], V4 [H_kv,mN4,D/2], V8 [H_kv,mN8,D], V_scale/V_zp fp16 [H_kv,max_tv]
- * (rows beyond a head's count are NOT written: pass zeroed buffers), V16 fp16
+ * (entries past a head's own quantized rows are written as zero), V16 fp16
  * [H_kv,max_n16,D], K2/K4/K8 [H_kv,max_tv+max_n16,sub], K_scale/K_zp fp16 [H_kv,Dp].
  * A head with fewer rows than the maxima has zero rows in the K canvas, so 0 joins its
  * per-channel min/max.  minmax_ws: H_kv*2*D floats of scratch. */

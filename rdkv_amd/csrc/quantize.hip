@@ -102,13 +102,24 @@ pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stri
                     const int32_t *__restrict__ counts, int mN2, int mN4, int mN8, int max_n16,
                     int64_t max_tv, uint8_t *__restrict__ V2, uint8_t *__restrict__ V4,
                     uint8_t *__restrict__ V8, __half *__restrict__ vs, __half *__restrict__ vz,
-                    __half *__restrict__ V16) {
+                    __half *__restrict__ V16, uint32_t *__restrict__ mm_init) {
   const int lane = threadIdx.x & 63;
   const int h = blockIdx.y;
   const int n2 = counts[4 * h], n4 = counts[4 * h + 1], n8 = counts[4 * h + 2], n16 = counts[4 * h + 3];
   const int32_t *ord = order + (int64_t)h * order_stride_h;
   const __half *Vh = V + (int64_t)h * stride_h;
   __half *vsh = vs + (int64_t)h * max_tv, *vzh = vz + (int64_t)h * max_tv;
+  // Two small jobs ride along instead of being launches of their own: scale / zero-point of the
+  // rows past the head's own quantized tokens are zero (the caller passes uninitialised tensors),
+  // and the per-channel (min, max) accumulators of the K pass that follows start at (+inf, -inf).
+  for (int64_t i = (int64_t)n2 + n4 + n8 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < max_tv;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    vsh[i] = __float2half_rn(0.0f);
+    vzh[i] = __float2half_rn(0.0f);
+  }
+  if (mm_init && blockIdx.x == 0)
+    for (int i = threadIdx.x; i < 2 * D; i += blockDim.x)
+      mm_init[(int64_t)h * 2 * D + i] = rdkv_float_to_ordered(i >= D ? -INFINITY : INFINITY);
   const bool d128 = D == 128;
   auto zero_bytes = [&](uint8_t *o, int n) {
     for (int c = lane; c < n; c += 64) o[c] = 0;
@@ -891,7 +902,7 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
     hipLaunchKernelGGL(pack_v_layer_kernel, dim3((unsigned)blocks, H_kv), dim3(64 * waves), 0, s,
                        (const __half *)V_f16, stride_h, stride_t, D, order, order_stride_h, counts, mN2, mN4,
                        mN8, max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16,
-                       (__half *)V16_f16);
+                       (__half *)V16_f16, (Dp > 0 && max_tk > 0) ? reinterpret_cast<uint32_t *>(minmax_ws) : nullptr);
   }
   if (Dp > 0 && max_tk > 0) {
     RDKV_REQUIRE(slot_channel && minmax_ws && K_scale_f16 && K_zp_f16 && (n2p == 0 || K2) &&
@@ -899,8 +910,9 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
                  "%s: null K output", fn);
     uint32_t *mm = reinterpret_cast<uint32_t *>(minmax_ws);
     // (+inf, -inf) in the ordered-int encoding, per head D mins then D maxes
-    hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256),
-                       0, s, mm, D, H_kv);
+    if (v_rows == 0)      // (otherwise the V launch above has set them)
+      hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256),
+                         0, s, mm, D, H_kv);
     const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
     RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
     const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;

@@ -704,8 +704,8 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
         n_v16_ph.data_ptr(), _lib.ptr(sort_idx), softmax_mask.data_ptr(), stream))
 
     V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
-    V_scale = torch.zeros(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)
-    V_zp = torch.zeros_like(V_scale)
+    V_scale = torch.empty(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)    # rows past a head's own
+    V_zp = torch.empty_like(V_scale)                                               # tokens are zeroed by the call
     new_v_only = (torch.empty(1, H_kv, max_n16, D, dtype=torch.float16, device=dev) if max_n16 > 0 else None)
     K2, K4, K8 = u8(max_tk, sub2), u8(max_tk, sub4), u8(max_tk, m8)
     ks = torch.empty(1, H_kv, 1, Dp, dtype=torch.float16, device=dev)
