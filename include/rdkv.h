@@ -96,6 +96,25 @@ int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int64_t strid
                              void *V16_f16, uint8_t *K2, uint8_t *K4, uint8_t *K8,
                              void *K_scale_f16, void *K_zp_f16, float *minmax_ws, void *stream);
 
+/* The two halves of rdkv_pack_layer_per_head as calls of their own (same arguments, same
+ * outputs), for a host that sizes and allocates the K outputs while the V rows are already
+ * being packed: the V rows need neither the channel tables nor the K outputs
+ * (V rows: pack_v_segments, packing.py:885; K rows: the deferred pack_k_mixed_per_head of the
+ * stacking step, packing.py:1185-1213).  minmax_start: NULL, or the K half's
+ * minmax_ws, whose start values this launch then writes; pass minmax_started != 0 to the K
+ * half in that case (both calls on one stream, V half first). */
+int rdkv_pack_layer_v_rows(const void *V_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                           const int32_t *order, int64_t order_stride_h, const int32_t *counts,
+                           int mN2, int mN4, int mN8, int64_t max_tv, int max_n16,
+                           uint8_t *V2, uint8_t *V4, uint8_t *V8, void *V_scale_f16, void *V_zp_f16,
+                           void *V16_f16, float *minmax_start, void *stream);
+int rdkv_pack_layer_k_rows(const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                           const int32_t *order, int64_t order_stride_h, const int32_t *counts,
+                           int64_t max_tv, int max_n16, const int32_t *slot_channel,
+                           int n2p, int n4p, int n8, uint8_t *K2, uint8_t *K4, uint8_t *K8,
+                           void *K_scale_f16, void *K_zp_f16, float *minmax_ws, int minmax_started,
+                           void *stream);
+
 /* Dequantize (codes - zp) * scale -> fp16 (unpack_v_segment packing.py:1427-1444 and the
  * per-segment step of unpack_k_mixed packing.py:629-651).  per_row != 0: scale/zp indexed by
  * row (V); per_row == 0: indexed by unpacked column (K).  out row stride in elements. */

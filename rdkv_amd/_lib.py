@@ -51,6 +51,8 @@ SIGNATURES = {
     "rdkv_k_quantize_pack": (I, [P, L, L, I, P, P, I, I, I, P, P, P, P, P, P]),
     "rdkv_pack_layer_per_head": (I, [P, P, L, L, I, I, P, L, P, I, I, I, L, I, P, I, I, I,
                                      P, P, P, P, P, P, P, P, P, P, P, P, P]),
+    "rdkv_pack_layer_v_rows": (I, [P, L, L, I, I, P, L, P, I, I, I, L, I, P, P, P, P, P, P, P, P]),
+    "rdkv_pack_layer_k_rows": (I, [P, L, L, I, I, P, L, P, L, I, P, I, I, I, P, P, P, P, P, P, I, P]),
     "rdkv_dequant_f16": (I, [P, L, I, I, P, P, I, P, L, P]),
     "rdkv_k_qk_dot": (I, [P, I, L, I, I, P, L, L, P, L, L, P, L, L, P, P, L, P, L, I, I, I, L, P, L, P]),
     "rdkv_softmax_rows": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P]),

@@ -870,6 +870,96 @@ RDKV_API int rdkv_dequant_f16(const uint8_t *packed, int64_t rows, int n_cols_un
   return RDKV_OK;
 }
 
+// The V half of the layer packer: quantized V rows by class, fp16 V rows, the zeroed tails of the
+// per-token scale / zero-point canvases and (when `mm_init` is given) the start values of the K
+// min/max accumulators.
+static int pack_layer_v_rows(const char *fn, const void *V_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                             const int32_t *order, int64_t order_stride_h, const int32_t *counts, int mN2, int mN4,
+                             int mN8, int64_t max_tv, int max_n16, uint8_t *V2, uint8_t *V4, uint8_t *V8,
+                             void *V_scale_f16, void *V_zp_f16, void *V16_f16, float *mm_init, hipStream_t s) {
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D > 0 && D % 4 == 0, "%s: bad H_kv=%d / D=%d", fn, H_kv, D);
+  RDKV_REQUIRE(mN2 >= 0 && mN4 >= 0 && mN8 >= 0 && max_n16 >= 0 && max_tv >= 0, "%s: negative counts", fn);
+  RDKV_REQUIRE(max_tv <= (int64_t)mN2 + mN4 + mN8, "%s: max_tv exceeds the class maxima", fn);
+  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)V_f16 % 4) == 0,
+               "%s: rows must be 4-byte aligned", fn);
+  const int64_t v_rows = (int64_t)mN2 + mN4 + mN8 + max_n16;
+  if (v_rows == 0) return RDKV_OK;
+  RDKV_REQUIRE(V_f16 && order && counts, "%s: null input", fn);
+  RDKV_REQUIRE((mN2 == 0 || V2) && (mN4 == 0 || V4) && (mN8 == 0 || V8) && (max_n16 == 0 || V16_f16) &&
+                   (max_tv == 0 || (V_scale_f16 && V_zp_f16)),
+               "%s: null V output", fn);
+  const int waves = 4;
+  const int64_t blocks = rdkv_cdiv(v_rows, waves * RDKV_PACK_V_ROWS_PER_WAVE);
+  RDKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many rows", fn);
+  hipLaunchKernelGGL(pack_v_layer_kernel, dim3((unsigned)blocks, H_kv), dim3(64 * waves), 0, s,
+                     (const __half *)V_f16, stride_h, stride_t, D, order, order_stride_h, counts, mN2, mN4, mN8,
+                     max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16, (__half *)V16_f16,
+                     reinterpret_cast<uint32_t *>(mm_init));
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+// The K half: per-channel min/max over each head's kept rows, then scales, zero points and the
+// packed K segments.  `mm_ready` says the accumulators in `minmax_ws` already hold their start
+// values (the V half wrote them on the same stream).
+static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                             const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tv,
+                             int max_n16, const int32_t *slot_channel, int n2p, int n4p, int n8, uint8_t *K2,
+                             uint8_t *K4, uint8_t *K8, void *K_scale_f16, void *K_zp_f16, float *minmax_ws,
+                             bool mm_ready, hipStream_t s) {
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D > 0 && D % 4 == 0, "%s: bad H_kv=%d / D=%d", fn, H_kv, D);
+  RDKV_REQUIRE(max_n16 >= 0 && max_tv >= 0, "%s: negative counts", fn);
+  RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
+               "%s: bad segment sizes (%d,%d,%d)", fn, n2p, n4p, n8);
+  const int Dp = n2p + n4p + n8;
+  RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "%s: %d padded channels > %d", fn, Dp, RDKV_MAX_SLOTS);
+  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0,
+               "%s: rows must be 4-byte aligned", fn);
+  const int64_t max_tk = max_tv + max_n16;
+  if (Dp == 0 || max_tk == 0) return RDKV_OK;
+  RDKV_REQUIRE(K_f16 && order && counts, "%s: null input", fn);
+  RDKV_REQUIRE(slot_channel && minmax_ws && K_scale_f16 && K_zp_f16 && (n2p == 0 || K2) && (n4p == 0 || K4) &&
+                   (n8 == 0 || K8),
+               "%s: null K output", fn);
+  uint32_t *mm = reinterpret_cast<uint32_t *>(minmax_ws);
+  // (+inf, -inf) in the ordered-int encoding, per head D mins then D maxes
+  if (!mm_ready)
+    hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256), 0,
+                       s, mm, D, H_kv);
+  const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
+  RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
+  const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
+  if (rows16) {
+    hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
+                       dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv), dim3(256), 0, s,
+                       (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
+  } else {
+    hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
+                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+  }
+  const int rows_per_block = 64;
+  const int64_t eblocks = rdkv_cdiv(max_tk, rows_per_block);
+  RDKV_REQUIRE(eblocks <= 0x7fffffffLL, "%s: too many rows", fn);
+  const size_t emit_lds = (size_t)D * 16 + 4 * (size_t)((Dp + 3) & ~3);
+  RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
+  if (rows16) {
+    const int rows_d128 = 256;
+    const size_t lds_d128 = (size_t)128 * 16 +
+                            16 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
+    hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, rows_d128), H_kv), dim3(256),
+                       lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, max_tv,
+                       max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
+                       (__half *)K_zp_f16, rows_d128);
+  } else {
+    hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
+                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv, max_n16,
+                       mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16, (__half *)K_zp_f16,
+                       rows_per_block);
+  }
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
 RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
                                       int H_kv, int D, const int32_t *order, int64_t order_stride_h,
                                       const int32_t *counts, int mN2, int mN4, int mN8, int64_t max_tv,
@@ -878,72 +968,35 @@ RDKV_API int rdkv_pack_layer_per_head(const void *K_f16, const void *V_f16, int6
                                       void *V_zp_f16, void *V16_f16, uint8_t *K2, uint8_t *K4, uint8_t *K8,
                                       void *K_scale_f16, void *K_zp_f16, float *minmax_ws, void *stream) {
   const char *fn = "rdkv_pack_layer_per_head";
-  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && D > 0 && D % 4 == 0, "%s: bad H_kv=%d / D=%d", fn, H_kv, D);
   RDKV_REQUIRE(mN2 >= 0 && mN4 >= 0 && mN8 >= 0 && max_n16 >= 0 && max_tv >= 0, "%s: negative counts", fn);
-  RDKV_REQUIRE(max_tv <= (int64_t)mN2 + mN4 + mN8, "%s: max_tv exceeds the class maxima", fn);
-  RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
-               "%s: bad segment sizes (%d,%d,%d)", fn, n2p, n4p, n8);
-  const int Dp = n2p + n4p + n8;
-  RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "%s: %d padded channels > %d", fn, Dp, RDKV_MAX_SLOTS);
-  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0 && ((uintptr_t)V_f16 % 4) == 0,
-               "%s: rows must be 4-byte aligned", fn);
   const int64_t v_rows = (int64_t)mN2 + mN4 + mN8 + max_n16;
-  const int64_t max_tk = max_tv + max_n16;
-  if (v_rows == 0 && max_tk == 0) return RDKV_OK;
-  RDKV_REQUIRE(K_f16 && V_f16 && order && counts, "%s: null input", fn);
-  RDKV_REQUIRE((mN2 == 0 || V2) && (mN4 == 0 || V4) && (mN8 == 0 || V8) && (max_n16 == 0 || V16_f16) &&
-                   (max_tv == 0 || (V_scale_f16 && V_zp_f16)),
-               "%s: null V output", fn);
-  hipStream_t s = (hipStream_t)stream;
-  if (v_rows > 0) {
-    const int waves = 4;
-    const int64_t blocks = rdkv_cdiv(v_rows, waves * RDKV_PACK_V_ROWS_PER_WAVE);
-    RDKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many rows", fn);
-    hipLaunchKernelGGL(pack_v_layer_kernel, dim3((unsigned)blocks, H_kv), dim3(64 * waves), 0, s,
-                       (const __half *)V_f16, stride_h, stride_t, D, order, order_stride_h, counts, mN2, mN4,
-                       mN8, max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16,
-                       (__half *)V16_f16, (Dp > 0 && max_tk > 0) ? reinterpret_cast<uint32_t *>(minmax_ws) : nullptr);
-  }
-  if (Dp > 0 && max_tk > 0) {
-    RDKV_REQUIRE(slot_channel && minmax_ws && K_scale_f16 && K_zp_f16 && (n2p == 0 || K2) &&
-                     (n4p == 0 || K4) && (n8 == 0 || K8),
-                 "%s: null K output", fn);
-    uint32_t *mm = reinterpret_cast<uint32_t *>(minmax_ws);
-    // (+inf, -inf) in the ordered-int encoding, per head D mins then D maxes
-    if (v_rows == 0)      // (otherwise the V launch above has set them)
-      hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256),
-                         0, s, mm, D, H_kv);
-    const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
-    RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
-    const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
-    if (rows16) {
-      hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
-                         dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv), dim3(256), 0, s,
-                         (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
-    } else {
-      hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
-                         (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
-    }
-    const int rows_per_block = 64;
-    const int64_t eblocks = rdkv_cdiv(max_tk, rows_per_block);
-    RDKV_REQUIRE(eblocks <= 0x7fffffffLL, "%s: too many rows", fn);
-    const size_t emit_lds = (size_t)D * 16 + 4 * (size_t)((Dp + 3) & ~3);
-    RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
-    if (rows16) {
-      const int rows_d128 = 256;
-      const size_t lds_d128 = (size_t)128 * 16 +
-                              16 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
-      hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, rows_d128), H_kv), dim3(256),
-                         lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts,
-                         max_tv, max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
-                         (__half *)K_zp_f16, rows_d128);
-    } else {
-      hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
-                         (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv,
-                         max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
-                         (__half *)K_zp_f16, rows_per_block);
-    }
-  }
-  RDKV_CHECK_LAUNCH(fn);
-  return RDKV_OK;
+  const bool k_half = (int64_t)n2p + n4p + n8 > 0 && max_tv + max_n16 > 0;
+  RDKV_REQUIRE(!k_half || minmax_ws, "%s: null K output", fn);
+  int rc = pack_layer_v_rows(fn, V_f16, stride_h, stride_t, H_kv, D, order, order_stride_h, counts, mN2, mN4, mN8,
+                             max_tv, max_n16, V2, V4, V8, V_scale_f16, V_zp_f16, V16_f16,
+                             k_half ? minmax_ws : nullptr, (hipStream_t)stream);
+  if (rc != RDKV_OK) return rc;
+  return pack_layer_k_rows(fn, K_f16, stride_h, stride_t, H_kv, D, order, order_stride_h, counts, max_tv, max_n16,
+                           slot_channel, n2p, n4p, n8, K2, K4, K8, K_scale_f16, K_zp_f16, minmax_ws, v_rows > 0,
+                           (hipStream_t)stream);
+}
+
+RDKV_API int rdkv_pack_layer_v_rows(const void *V_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                                    const int32_t *order, int64_t order_stride_h, const int32_t *counts, int mN2,
+                                    int mN4, int mN8, int64_t max_tv, int max_n16, uint8_t *V2, uint8_t *V4,
+                                    uint8_t *V8, void *V_scale_f16, void *V_zp_f16, void *V16_f16,
+                                    float *minmax_start, void *stream) {
+  return pack_layer_v_rows("rdkv_pack_layer_v_rows", V_f16, stride_h, stride_t, H_kv, D, order, order_stride_h,
+                           counts, mN2, mN4, mN8, max_tv, max_n16, V2, V4, V8, V_scale_f16, V_zp_f16, V16_f16,
+                           minmax_start, (hipStream_t)stream);
+}
+
+RDKV_API int rdkv_pack_layer_k_rows(const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                                    const int32_t *order, int64_t order_stride_h, const int32_t *counts,
+                                    int64_t max_tv, int max_n16, const int32_t *slot_channel, int n2p, int n4p,
+                                    int n8, uint8_t *K2, uint8_t *K4, uint8_t *K8, void *K_scale_f16,
+                                    void *K_zp_f16, float *minmax_ws, int minmax_started, void *stream) {
+  return pack_layer_k_rows("rdkv_pack_layer_k_rows", K_f16, stride_h, stride_t, H_kv, D, order, order_stride_h,
+                           counts, max_tv, max_n16, slot_channel, n2p, n4p, n8, K2, K4, K8, K_scale_f16, K_zp_f16,
+                           minmax_ws, minmax_started != 0, (hipStream_t)stream);
 }

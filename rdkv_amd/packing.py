@@ -683,6 +683,19 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
     def u8(n, w):
         return torch.empty(1, H_kv, n, w, dtype=torch.uint8, device=dev) if n > 0 and w > 0 else None
 
+    # V rows first: they need neither the channel tables nor the K outputs, so the device packs
+    # them while the host sizes and allocates the rest
+    V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
+    V_scale = torch.empty(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)    # rows past a head's own
+    V_zp = torch.empty_like(V_scale)                                               # tokens are zeroed by the call
+    new_v_only = (torch.empty(1, H_kv, max_n16, D, dtype=torch.float16, device=dev) if max_n16 > 0 else None)
+    mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
+    v_rows = mN[0] + mN[1] + mN[2] + max_n16
+    _lib.check(lib.rdkv_pack_layer_v_rows(
+        Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0), counts4_ptr,
+        mN[0], mN[1], mN[2], max_tv, max_n16, _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale),
+        _lib.ptr(V_zp), _lib.ptr(new_v_only), mm.data_ptr(), stream))
+
     i32 = dict(dtype=torch.int32, device=dev)
     i64 = dict(dtype=torch.int64, device=dev)
     slot_ch = torch.empty(H_kv, Dp, **i32)
@@ -703,20 +716,13 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
         _lib.ptr(sort_ph), seg_ph.data_ptr(), seg_tok.data_ptr(), t_eff_ph.data_ptr(), t_eff_k_ph.data_ptr(),
         n_v16_ph.data_ptr(), _lib.ptr(sort_idx), softmax_mask.data_ptr(), stream))
 
-    V2, V4, V8 = u8(mN[0], D // 4), u8(mN[1], D // 2), u8(mN[2], D)
-    V_scale = torch.empty(1, H_kv, max_tv, 1, dtype=torch.float16, device=dev)    # rows past a head's own
-    V_zp = torch.empty_like(V_scale)                                               # tokens are zeroed by the call
-    new_v_only = (torch.empty(1, H_kv, max_n16, D, dtype=torch.float16, device=dev) if max_n16 > 0 else None)
     K2, K4, K8 = u8(max_tk, sub2), u8(max_tk, sub4), u8(max_tk, m8)
     ks = torch.empty(1, H_kv, 1, Dp, dtype=torch.float16, device=dev)
     kz = torch.empty_like(ks)
-    mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
-    _lib.check(lib.rdkv_pack_layer_per_head(
-        Kf.data_ptr(), Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D,
-        order_l.data_ptr(), order_l.stride(0), counts4_ptr, mN[0], mN[1], mN[2], max_tv, max_n16,
-        slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8,
-        _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only),
-        _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), stream))
+    _lib.check(lib.rdkv_pack_layer_k_rows(
+        Kf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0), counts4_ptr,
+        max_tv, max_n16, slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8, _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8),
+        ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), 1 if v_rows > 0 else 0, stream))
 
     # metadata exactly as _pad_and_stack_per_head_layers / pack_k_mixed_per_head produce it
     packed = PackedKVLayer(
