@@ -647,10 +647,12 @@ def _plan_layers(v_bits: Tensor, k_bits: Tensor, dev):
     return order, rank3, plan, counts_h, info_h, kb
 
 
-def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: int, n_total: int):
+def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: int, n_total: int,
+                        one_call: bool = False):
     """Pack the layer whose heads are rows ``first .. first + H_kv`` of a plan over ``n_total``
     heads.  Returns None when the layer is degenerate (nothing kept / no channels kept / more
-    than 1024 channels) and must take the composed path."""
+    than 1024 channels) and must take the composed path.  ``one_call`` packs V and K rows with
+    the single ``rdkv_pack_layer_per_head`` call instead of its two halves (same result)."""
     order, rank3, plan, counts_all, info_all, kb_all = planned
     dev = K.device
     lib = _lib.load()
@@ -691,10 +693,11 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
     new_v_only = (torch.empty(1, H_kv, max_n16, D, dtype=torch.float16, device=dev) if max_n16 > 0 else None)
     mm = torch.empty(H_kv * 2 * D, dtype=torch.float32, device=dev)
     v_rows = mN[0] + mN[1] + mN[2] + max_n16
-    _lib.check(lib.rdkv_pack_layer_v_rows(
-        Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0), counts4_ptr,
-        mN[0], mN[1], mN[2], max_tv, max_n16, _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale),
-        _lib.ptr(V_zp), _lib.ptr(new_v_only), mm.data_ptr(), stream))
+    if not one_call:
+        _lib.check(lib.rdkv_pack_layer_v_rows(
+            Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0),
+            counts4_ptr, mN[0], mN[1], mN[2], max_tv, max_n16, _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8),
+            _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only), mm.data_ptr(), stream))
 
     i32 = dict(dtype=torch.int32, device=dev)
     i64 = dict(dtype=torch.int64, device=dev)
@@ -719,10 +722,18 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
     K2, K4, K8 = u8(max_tk, sub2), u8(max_tk, sub4), u8(max_tk, m8)
     ks = torch.empty(1, H_kv, 1, Dp, dtype=torch.float16, device=dev)
     kz = torch.empty_like(ks)
-    _lib.check(lib.rdkv_pack_layer_k_rows(
-        Kf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0), counts4_ptr,
-        max_tv, max_n16, slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8, _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8),
-        ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), 1 if v_rows > 0 else 0, stream))
+    if one_call:
+        _lib.check(lib.rdkv_pack_layer_per_head(
+            Kf.data_ptr(), Vf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D,
+            order_l.data_ptr(), order_l.stride(0), counts4_ptr, mN[0], mN[1], mN[2], max_tv, max_n16,
+            slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8,
+            _lib.ptr(V2), _lib.ptr(V4), _lib.ptr(V8), _lib.ptr(V_scale), _lib.ptr(V_zp), _lib.ptr(new_v_only),
+            _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), stream))
+    else:
+        _lib.check(lib.rdkv_pack_layer_k_rows(
+            Kf.data_ptr(), Kf.stride(0), Kf.stride(1), H_kv, D, order_l.data_ptr(), order_l.stride(0),
+            counts4_ptr, max_tv, max_n16, slot_ch.data_ptr(), 4 * sub2, 2 * sub4, m8, _lib.ptr(K2), _lib.ptr(K4),
+            _lib.ptr(K8), ks.data_ptr(), kz.data_ptr(), mm.data_ptr(), 1 if v_rows > 0 else 0, stream))
 
     # metadata exactly as _pad_and_stack_per_head_layers / pack_k_mixed_per_head produce it
     packed = PackedKVLayer(

@@ -249,3 +249,10 @@ def test_whole_layer_packer_matches_composition(case):
     assert (got_nvo is None) == (exp_nvo is None)
     if exp_nvo is not None:
         assert torch.equal(got_nvo.view(torch.uint8), exp_nvo.view(torch.uint8))
+    # the single call that packs V and K rows together gives the same layer as its two halves
+    planned = packing._plan_layers(vb.to(DEV), kb.to(DEV), DEV)
+    one = packing._pack_planned_layer(K, V, G, planned, 0, H, one_call=True)
+    assert one is not None
+    _layers_identical(one[0], exp)
+    if exp_nvo is not None:
+        assert torch.equal(one[1].view(torch.uint8), exp_nvo.view(torch.uint8))
