@@ -6,6 +6,9 @@
 // fp32 math throughout, fixed summation order (deterministic).
 #include "rdkv_common.h"
 
+#include <algorithm>
+#include <type_traits>
+
 namespace {
 
 constexpr float kInvSqrtD = 0.08838834764831845f;  // 1/sqrt(128), triton_k_kernel.py:280
@@ -24,7 +27,7 @@ __device__ __forceinline__ float load_q(const void *q, int dtype, int64_t idx) {
 // qs[g][c] = q[hq, perm[c]] * scale[c]; bias[g] = sum_c zp[c]*qs[g][c];
 // out = (sum_c code*qs - bias) / sqrt(128)      (triton_k_kernel.py:14-17)
 // This kernel reads the rows where they lie, a byte at a time, whatever their strides;
-// k_qk_dot_staged_kernel below is the one for densely stored rows.
+// k_qk_dot_mfma_kernel below is the one for densely stored rows.
 // ---------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
 k_qk_dot_strided_kernel(const void *__restrict__ q, int q_dtype, int64_t q_stride_h, int G,
@@ -101,112 +104,439 @@ k_qk_dot_strided_kernel(const void *__restrict__ q, int q_dtype, int64_t q_strid
   }
 }
 
-// Copies n bytes from global memory to LDS with 16-byte loads.  dst must be congruent to src
-// modulo 16; the unaligned head and tail (at most 15 bytes each) go byte by byte.
-__device__ __forceinline__ void stage_bytes(uint8_t *dst, const uint8_t *__restrict__ src, int n) {
-  const int head = (int)((16 - ((uintptr_t)src & 15)) & 15);
-  const int h = head < n ? head : n;
-  const int body = (n - h) >> 4, tail = (n - h) & 15;
-  const uint4 *s16 = reinterpret_cast<const uint4 *>(src + h);
-  uint4 *d16 = reinterpret_cast<uint4 *>(dst + h);
-  int i = threadIdx.x;
-  for (; i + 3 * 256 < body; i += 4 * 256) {
-    const uint4 a = s16[i], b = s16[i + 256], c = s16[i + 512], d = s16[i + 768];
-    d16[i] = a;
-    d16[i + 256] = b;
-    d16[i + 512] = c;
-    d16[i + 768] = d;
-  }
-  for (; i < body; i += 256) d16[i] = s16[i];
-  if ((int)threadIdx.x < h) dst[threadIdx.x] = src[threadIdx.x];
-  if ((int)threadIdx.x < tail) dst[h + 16 * body + threadIdx.x] = src[h + 16 * body + threadIdx.x];
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ half4_t mk_op(uint32_t a, uint32_t b) {
+  union { uint32_t u[2]; half4_t h; } x;
+  x.u[0] = a;
+  x.u[1] = b;
+  return x.h;
 }
 
-// The arithmetic of k_qk_dot_strided_kernel (the bias summed by a wavefront instead of a thread) for
-// rows stored back to back (token stride = row bytes): the 256 rows of a workgroup are one
-// contiguous run per segment, copied to LDS with coalesced 16-byte loads and read from there.
-// Dynamic LDS: kGB*Dp + 2*kGB floats, then 256 rows of each segment, each run with 16 bytes of slack.
-__global__ void __launch_bounds__(256)
-k_qk_dot_staged_kernel(const void *__restrict__ q, int q_dtype, int64_t q_stride_h, int G,
-                       const uint8_t *__restrict__ K2, int64_t k2_sh, const uint8_t *__restrict__ K4,
-                       int64_t k4_sh, const uint8_t *__restrict__ K8, int64_t k8_sh,
-                       const __half *__restrict__ scale, const __half *__restrict__ zp, int64_t ks_sh,
-                       const int64_t *__restrict__ perm, int64_t perm_sh, int n2p, int n4p, int n8,
-                       int64_t T, float *__restrict__ out, int64_t out_sh) {
-  extern __shared__ __align__(16) float smem[];
-  const int Dp = n2p + n4p + n8;
-  const int hkv = blockIdx.y;
-  float *s_qs = smem;               // [Dp][kGB]
-  float *s_bias = smem + kGB * Dp;  // [kGB]
-  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
-  const int64_t t0 = (int64_t)blockIdx.x * 256;
-  const int ntok = T - t0 < 256 ? (int)(T - t0) : 256;
-  uint8_t *rows = reinterpret_cast<uint8_t *>(smem + kGB * Dp + 2 * kGB);
-  const uint8_t *g2 = K2 ? K2 + hkv * k2_sh + t0 * sub2 : nullptr;
-  const uint8_t *g4 = K4 ? K4 + hkv * k4_sh + t0 * sub4 : nullptr;
-  const uint8_t *g8 = K8 ? K8 + hkv * k8_sh + t0 * n8 : nullptr;
-  uint8_t *l2 = rows + ((uintptr_t)g2 & 15);
-  uint8_t *l4 = rows + ((256 * sub2 + 15) & ~15) + 16 + ((uintptr_t)g4 & 15);
-  uint8_t *l8 = rows + ((256 * sub2 + 15) & ~15) + ((256 * sub4 + 15) & ~15) + 32 + ((uintptr_t)g8 & 15);
-  if (sub2) stage_bytes(l2, g2, ntok * sub2);
-  if (sub4) stage_bytes(l4, g4, ntok * sub4);
-  if (n8) stage_bytes(l8, g8, ntok * n8);
-  const int tl = threadIdx.x;
-  const uint8_t *r2 = l2 + tl * sub2, *r4 = l4 + tl * sub4, *r8 = l8 + tl * n8;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 
-  for (int g0 = 0; g0 < G; g0 += kGB) {
-    __syncthreads();
-    for (int i = threadIdx.x; i < kGB * Dp; i += blockDim.x) {
-      const int g = i / Dp, c = i - g * Dp;
-      float v = 0.0f;
-      if (g0 + g < G) {
-        const int hq = hkv * G + g0 + g;
-        const int64_t ch = perm[(perm_sh ? hq : 0) * perm_sh + c];
-        v = load_q(q, q_dtype, hq * q_stride_h + ch) * __half2float(scale[hkv * ks_sh + c]);
+// The part of a zero point that the fp16 operand code - zp carries exactly: its nearest integer,
+// kept within +-1024.  The quantizer only produces integers in 0..255, for which nothing is left
+// over; whatever is left of another value enters as a bias term.
+__device__ __forceinline__ float zp_whole(float z) { return fminf(fmaxf(rintf(z), -1024.0f), 1024.0f); }
+
+// Bytes `lo_byte` and `lo_byte + 2` of `codes` (each a code below 256), as the fp16 pair
+// (1024 + code) - z with z = 1024 + zp: the exact integers code - zp.  0x64 over a code byte is the
+// bit pattern of 1024 + code; one byte permute builds both halves.
+template <int LO_BYTE>
+__device__ __forceinline__ uint32_t centered(uint32_t codes, uint32_t z) {
+  union { uint32_t u; half2_t h; } a, b;
+  a.u = __builtin_amdgcn_perm(codes, 0x64646464u, LO_BYTE == 0 ? 0x00060004u : 0x00070005u);
+  b.u = z;
+  a.h = a.h - b.h;
+  return a.u;
+}
+
+// q*scale halves and zero points of one step: what k_segment_steps multiplies a plane of codes by.
+template <int NG>
+struct KStepOps {
+  half4_t q[NG][2];   // [head group][value | rounding remainder], this lane's head
+  uint2 z;            // 1024 + zero point of the four codes
+};
+template <int NG>
+__device__ __forceinline__ KStepOps<NG> k_load_ops(const _Float16 *op, const uint2 *zop, int e) {
+  KStepOps<NG> o;
+#pragma unroll
+  for (int hg = 0; hg < NG; ++hg) {
+    o.q[hg][0] = *reinterpret_cast<const half4_t *>(op + (size_t)(e * NG + hg) * 32);
+    o.q[hg][1] = *reinterpret_cast<const half4_t *>(op + (size_t)(e * NG + hg) * 32 + 16);
+  }
+  o.z = zop[e];
+  return o;
+}
+
+// Step number -> (dword of the row, plane) when a segment runs p_eff (1..4) planes per dword.
+__device__ __forceinline__ void k_split_step(int r, int p_eff, int &jd, int &p) {
+  if (p_eff == 1) { jd = r; p = 0; }
+  else if (p_eff == 2) { jd = r >> 1; p = r & 1; }
+  else if (p_eff == 4) { jd = r >> 2; p = r & 3; }
+  else { jd = (r * 21846) >> 16; p = r - 3 * jd; }   // r / 3 for r < 32768
+}
+
+// One segment of a token's row on the matrix cores.  The row lies in LDS at byte offset `off`
+// from `lds32` (any alignment): dword jd of the row is cut from two aligned LDS dwords.  A dword
+// holds 8/BITS planes of four codes (plane p = bit field p of each byte), of which the first PE
+// are in use; a step multiplies the four values code - zp of one plane (exact in fp16) by the
+// 4 x 4 table of q*scale halves of that step: codes of bytes (0, 2, 1, 3), which is the order the
+// tables are built in.  The tables hold the executed steps in execution order (entry `e` counts
+// across the segments).  Steps alternate between two operand sets: the set a step has used is
+// reloaded for the step after the next, a whole step ahead of its use, with no register copies
+// (a reload that is waited for in the same step costs an LDS round trip per step).  For that
+// every segment runs an even number of steps: with an odd PE the dwords go two per iteration,
+// and a last single dword is followed by a padding step whose table entry is never multiplied.
+template <int BITS, int PE, int NG>
+__device__ __forceinline__ void k_segment_steps(const uint32_t *lds32, int off, int nd, const _Float16 *op,
+                                                const uint2 *zop, int &e, KStepOps<NG> (&cur)[2],
+                                                floatx4 (&acc)[NG][2]) {
+  constexpr uint32_t kMask = ((1u << BITS) - 1u) * 0x01010101u;
+  constexpr int U = (PE & 1) ? 2 : 1;
+  if (nd == 0) return;
+  const uint32_t *W = lds32 + (off >> 2);
+  const uint32_t sh = (uint32_t)off & 3u;
+  // aligned dwords jd .. jd + U of the row are in w[] when an iteration starts; the next U are
+  // requested at its start and not looked at before the next one
+  uint32_t w[U + 1];
+#pragma unroll
+  for (int i = 0; i <= U; ++i) w[i] = W[i];
+  auto dword = [&](uint32_t lo_w, uint32_t hi_w, auto first_slot) __attribute__((always_inline)) {
+    constexpr int S0 = decltype(first_slot)::value;
+    const uint32_t wd = __builtin_amdgcn_alignbyte(hi_w, lo_w, sh);
+#pragma unroll
+    for (int p = 0; p < PE; ++p) {
+      KStepOps<NG> &c = cur[(S0 + p) & 1];
+      const uint32_t ws = BITS == 8 ? wd : (wd >> (BITS * p)) & kMask;   // plane p: one code per byte
+      const half4_t a = mk_op(centered<0>(ws, c.z.x), centered<1>(ws, c.z.y));
+#pragma unroll
+      for (int hg = 0; hg < NG; ++hg) {
+        acc[hg][0] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, c.q[hg][0], acc[hg][0], 0, 0, 0);
+        acc[hg][1] = __builtin_amdgcn_mfma_f32_4x4x4f16(a, c.q[hg][1], acc[hg][1], 0, 0, 0);
       }
-      s_qs[c * kGB + g] = v;
+      c = k_load_ops<NG>(op, zop, e + 2);
+      ++e;
     }
-    __syncthreads();
-    {  // bias of head g by wavefront g: lanes stride the channels, then a fixed shuffle tree
-      const int g = threadIdx.x >> 6;
-      float b = 0.0f;
-      for (int c = threadIdx.x & 63; c < Dp; c += 64) b += __half2float(zp[hkv * ks_sh + c]) * s_qs[c * kGB + g];
-      b = rdkv_wave_sum(b);
-      if ((threadIdx.x & 63) == 0) s_bias[g] = b;
-    }
-    __syncthreads();
-    if (tl < ntok) {
-      float acc[kGB];
+  };
+  int jd = 0;
+  for (; jd + U <= nd; jd += U) {
+    uint32_t nx[U];
 #pragma unroll
-      for (int g = 0; g < kGB; ++g) acc[g] = 0.0f;
-      const float4 *qs4 = reinterpret_cast<const float4 *>(s_qs);
-      auto fma4 = [&](float cv, int c) {
-        const float4 w = qs4[c];
-        acc[0] += cv * w.x;
-        acc[1] += cv * w.y;
-        acc[2] += cv * w.z;
-        acc[3] += cv * w.w;
-      };
-      for (int j = 0; j < sub2; ++j) {
-        const uint32_t b = r2[j];
+    for (int i = 0; i < U; ++i) nx[i] = W[jd + U + 1 + i];
+    dword(w[0], w[1], std::integral_constant<int, 0>{});
+    if constexpr (U == 2) dword(w[1], w[2], std::integral_constant<int, PE & 1>{});
+    w[0] = w[U];
 #pragma unroll
-        for (int f = 0; f < 4; ++f) fma4((float)((b >> (2 * f)) & 3u), j + f * sub2);
-      }
-      for (int j = 0; j < sub4; ++j) {
-        const uint32_t b = r4[j];
-        const float4 wl = qs4[n2p + j], wh = qs4[n2p + j + sub4];
-        const float lo = (float)(b & 15u), hi = (float)(b >> 4);
-        acc[0] += lo * wl.x + hi * wh.x;
-        acc[1] += lo * wl.y + hi * wh.y;
-        acc[2] += lo * wl.z + hi * wh.z;
-        acc[3] += lo * wl.w + hi * wh.w;
-      }
-      for (int j = 0; j < n8; ++j) fma4((float)r8[j], n2p + n4p + j);
-#pragma unroll
-      for (int g = 0; g < kGB; ++g)
-        if (g0 + g < G) out[(int64_t)(hkv * G + g0 + g) * out_sh + t0 + tl] = (acc[g] - s_bias[g]) * kInvSqrtD;
+    for (int i = 0; i < U; ++i) w[1 + i] = nx[i];
+  }
+  if constexpr (U == 2) {
+    if (jd < nd) {
+      dword(w[0], w[1], std::integral_constant<int, 0>{});
+      cur[1] = k_load_ops<NG>(op, zop, e + 2);   // the padding step
+      ++e;
     }
   }
+}
+
+// K scores for rows stored back to back (token stride = row bytes), query heads g0 .. g0 + 4 NG of
+// every KV head.  A workgroup walks 256-token tiles of one KV head (tile = blockIdx.x, + gridDim.x,
+// ...).  The rows of a tile are one contiguous run per segment, copied to LDS with coalesced
+// 16-byte loads (the next tile's are in flight while the current one is computed); a lane owns a
+// token and feeds its codes to v_mfma_f32_4x4x4_16b_f16 (16 blocks of 4 tokens x 4 channels x
+// 4 heads per instruction) as code - zp, an exact fp16 integer, with q*scale as an fp16 pair
+// (value and rounding remainder, two accumulators) after a power of two that brings the largest
+// |q*scale| of the head group just under 2^14: the sum runs over the signed products themselves
+// (no large code*q*scale and zp*q*scale sums that cancel), in fp32.  The reference layout pads
+// every head's segments to the widest head's: channels whose stored scale is zero contribute
+// exactly nothing, so the steps past a head's last such channel are skipped.
+// Every global load of the set-up is issued before any of them is consumed, oldest chain first
+// (channel tables, the rows, then the query elements the permutation points to).  The row pieces
+// are loaded by hand-placed instructions: left to the compiler, each load moves down to its LDS
+// store, behind the query loads; they are waited for by the explicit wait before the stores.
+// CPT = channels per thread (Dp <= 256 CPT), KMAX = 16-byte row pieces per thread.
+// Dynamic LDS: [Dp][4 NG] floats of q*scale, 4 NG biases, 20 words, Dp zero points, the step tables
+// (64 NG bytes of q*scale and 8 of zero points per step, six spare steps), then 256 rows of each
+// segment, each run with 16 bytes of slack.
+// Wavefronts per SIMD (= resident workgroups per compute unit) the variants are compiled for.
+constexpr int k_mfma_residency(int ng, int kmax) { return kmax > 8 ? (ng == 2 ? 2 : 3) : (ng == 2 ? 3 : 4); }
+
+template <int NG, int KMAX, int CPT>
+__global__ void __launch_bounds__(256, k_mfma_residency(NG, KMAX))
+k_qk_dot_mfma_kernel(const void *__restrict__ q, int q_dtype, int64_t q_stride_h, int G, int g0,
+                     const uint8_t *__restrict__ K2, int64_t k2_sh, const uint8_t *__restrict__ K4,
+                     int64_t k4_sh, const uint8_t *__restrict__ K8, int64_t k8_sh,
+                     const __half *__restrict__ scale, const __half *__restrict__ zp, int64_t ks_sh,
+                     const int64_t *__restrict__ perm, int64_t perm_sh, int n2p, int n4p, int n8,
+                     int64_t T, float *__restrict__ out, int64_t out_sh) {
+  extern __shared__ __align__(16) float smem[];
+  constexpr int NHD = 4 * NG;
+  const int Dp = n2p + n4p + n8;
+  const int hkv = blockIdx.y;
+  const int sub2 = n2p >> 2, sub4 = n4p >> 1;
+  const int nd2 = (sub2 + 3) >> 2, nd4 = (sub4 + 3) >> 2, nd8 = (n8 + 3) >> 2;
+  const int nsteps = 4 * nd2 + 2 * nd4 + nd8;
+  float *s_qs = smem;                                    // [Dp][NHD]
+  float *s_bias = s_qs + Dp * NHD;                       // [NHD]
+  float *s_red = s_bias + NHD;                           // [4]
+  int *s_ext = reinterpret_cast<int *>(s_red + 4);       // [4 wavefronts][4]
+  float *s_zpf = reinterpret_cast<float *>(s_ext + 16);  // [Dp] zero points
+  _Float16 *s_op = reinterpret_cast<_Float16 *>(s_zpf + ((Dp + 3) & ~3));   // [nsteps + 6][NG][2][4 heads][4 codes]
+  _Float16 *s_zp = s_op + (size_t)(nsteps + 6) * NG * 32;                   // [nsteps + 6][4 codes]: 1024 + zp
+  uint8_t *rows = reinterpret_cast<uint8_t *>(s_zp + (size_t)(((nsteps + 6) * 4 + 7) & ~7));
+  const int tl = threadIdx.x, lane = tl & 63, wave = tl >> 6, ln = lane & 3;
+  const __half *sc_h = scale + hkv * ks_sh, *zp_h = zp + hkv * ks_sh;
+  const int ntiles = (int)((T + 255) >> 8);
+  const int rowb[3] = {sub2, sub4, n8};
+  const int seg_lds[3] = {0, ((256 * sub2 + 15) & ~15) + 16, ((256 * sub2 + 15) & ~15) + ((256 * sub4 + 15) & ~15) + 32};
+  const int spare_lds = 256 * (sub2 + sub4 + n8) + 80;   // 16 bytes nobody reads: pieces without an owner go here
+  // a mapped, aligned address for the loads of threads that have no piece
+  const uint64_t dummy = (uint64_t)(uintptr_t)(reinterpret_cast<const uint8_t *>(sc_h) - ((uintptr_t)sc_h & 15));
+  const uint32_t *lds32 = reinterpret_cast<const uint32_t *>(smem);
+  const int rows_off = (int)(rows - reinterpret_cast<uint8_t *>(smem));
+
+  // The three row runs of a tile: global start, bytes, unaligned head, 16-byte pieces, LDS position
+  // (congruent to the global address modulo 16).
+  struct Run { uint64_t g; int n, h, body, lds; };
+  auto run_of = [&](int tile, int sgm) -> Run {
+    const int64_t t0 = (int64_t)tile * 256;
+    const int ntok = T - t0 < 256 ? (int)(T - t0) : 256;
+    const uint8_t *base = sgm == 0 ? K2 + hkv * k2_sh : sgm == 1 ? K4 + hkv * k4_sh : K8 + hkv * k8_sh;
+    Run r;
+    r.g = rowb[sgm] ? (uint64_t)(uintptr_t)(base + t0 * rowb[sgm]) : dummy;
+    r.n = ntok * rowb[sgm];
+    const int h = (int)((16 - (r.g & 15)) & 15);
+    r.h = h < r.n ? h : r.n;
+    r.body = (r.n - r.h) >> 4;
+    r.lds = seg_lds[sgm] + (int)(r.g & 15);
+    return r;
+  };
+  u32x4 buf[KMAX];
+  uint32_t eb[6];
+  // Piece blocks are uniform: blocks 0 .. ceil(body/256) of run 0, then of run 1, then of run 2, so the
+  // base address of a load is a scalar and a thread only adds its own offset.
+  auto issue_rows = [&](int tile) __attribute__((always_inline)) {
+    const Run r0 = run_of(tile, 0), r1 = run_of(tile, 1), r2 = run_of(tile, 2);
+    const int k0 = (r0.body + 255) >> 8, k1 = k0 + ((r1.body + 255) >> 8), k2 = k1 + ((r2.body + 255) >> 8);
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const uint64_t base = k < k0 ? r0.g + r0.h : k < k1 ? r1.g + r1.h : k < k2 ? r2.g + r2.h : dummy;
+      const int body = k < k0 ? r0.body : k < k1 ? r1.body : k < k2 ? r2.body : 0;
+      const int piece = tl + 256 * (k < k0 ? k : k < k1 ? k - k0 : k - k1);
+      const uint32_t voff = piece < body ? 16u * (uint32_t)piece : 0u;
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=&v"(buf[k]) : "v"(voff), "s"(base) : "memory");
+    }
+    // the unaligned ends of the three runs (at most 15 bytes each): byte tl of each, if it exists
+#pragma unroll
+    for (int sgm = 0; sgm < 3; ++sgm) {
+      const Run r = sgm == 0 ? r0 : sgm == 1 ? r1 : r2;
+      const uint32_t vh = tl < r.h ? (uint32_t)tl : 0u;
+      const uint32_t vt = tl < ((r.n - r.h) & 15) ? (uint32_t)(r.h + 16 * r.body + tl) : 0u;
+      const uint64_t base = r.n > 0 ? r.g : dummy;
+      asm volatile("global_load_ubyte %0, %1, %2" : "=&v"(eb[2 * sgm]) : "v"(vh), "s"(base) : "memory");
+      asm volatile("global_load_ubyte %0, %1, %2" : "=&v"(eb[2 * sgm + 1]) : "v"(vt), "s"(base) : "memory");
+    }
+  };
+  auto store_rows = [&](int tile) __attribute__((always_inline)) {
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(buf[k]) : : "memory");
+#pragma unroll
+    for (int k = 0; k < 6; ++k) asm volatile("s_waitcnt vmcnt(0)" : "+v"(eb[k]) : : "memory");
+    const Run r0 = run_of(tile, 0), r1 = run_of(tile, 1), r2 = run_of(tile, 2);
+    const int k0 = (r0.body + 255) >> 8, k1 = k0 + ((r1.body + 255) >> 8), k2 = k1 + ((r2.body + 255) >> 8);
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int start = k < k0 ? r0.lds + r0.h : k < k1 ? r1.lds + r1.h : k < k2 ? r2.lds + r2.h : spare_lds;
+      const int body = k < k0 ? r0.body : k < k1 ? r1.body : k < k2 ? r2.body : 0;
+      const int piece = tl + 256 * (k < k0 ? k : k < k1 ? k - k0 : k - k1);
+      *reinterpret_cast<u32x4 *>(rows + (piece < body ? start + 16 * piece : spare_lds)) = buf[k];
+    }
+#pragma unroll
+    for (int sgm = 0; sgm < 3; ++sgm) {
+      const Run r = sgm == 0 ? r0 : sgm == 1 ? r1 : r2;
+      if (tl < r.h) rows[r.lds + tl] = (uint8_t)eb[2 * sgm];
+      if (tl < ((r.n - r.h) & 15)) rows[r.lds + r.h + 16 * r.body + tl] = (uint8_t)eb[2 * sgm + 1];
+    }
+  };
+
+  // ---- set-up: channel tables, the first tile's rows, the query --------------------------------
+  int tile = blockIdx.x;
+  int64_t ch[CPT][NHD];
+  float scv[CPT], zpv[CPT];
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    const int c = min(tl + 256 * u, Dp - 1);
+    scv[u] = __half2float(sc_h[c]);
+    zpv[u] = __half2float(zp_h[c]);
+#pragma unroll
+    for (int g = 0; g < NHD; ++g) {
+      const int hq = hkv * G + min(g0 + g, G - 1);
+      ch[u][g] = perm[(perm_sh ? hq : 0) * perm_sh + c];
+    }
+  }
+  issue_rows(tile);
+  float qv[CPT][NHD];
+  auto q_loads = [&](auto elem) __attribute__((always_inline)) {   // one straight run of loads per query type
+#pragma unroll
+    for (int u = 0; u < CPT; ++u)
+#pragma unroll
+      for (int g = 0; g < NHD; ++g) {
+        const int hq = hkv * G + min(g0 + g, G - 1);
+        qv[u][g] = elem(hq * q_stride_h + ch[u][g]);
+      }
+  };
+  if (q_dtype == RDKV_DTYPE_F32)
+    q_loads([&](int64_t i) { return reinterpret_cast<const float *>(q)[i]; });
+  else if (q_dtype == RDKV_DTYPE_F16)
+    q_loads([&](int64_t i) { return __half2float(reinterpret_cast<const __half *>(q)[i]); });
+  else
+    q_loads([&](int64_t i) { return __uint_as_float((uint32_t)reinterpret_cast<const uint16_t *>(q)[i] << 16); });
+  store_rows(tile);
+  float mloc = 0.0f;
+  int last2 = 0, last4 = 0, last8 = 0;   // channels of a segment up to the last one with a nonzero scale
+#pragma unroll
+  for (int u = 0; u < CPT; ++u) {
+    const int c = tl + 256 * u;
+    if (c < Dp) {
+      float vv[NHD];
+#pragma unroll
+      for (int g = 0; g < NHD; ++g) {
+        vv[g] = g0 + g < G ? qv[u][g] * scv[u] : 0.0f;
+        mloc = fmaxf(mloc, fabsf(vv[g]));
+      }
+#pragma unroll
+      for (int hg = 0; hg < NG; ++hg)
+        reinterpret_cast<float4 *>(s_qs + c * NHD)[hg] =
+            make_float4(vv[4 * hg], vv[4 * hg + 1], vv[4 * hg + 2], vv[4 * hg + 3]);
+      s_zpf[c] = zpv[u];
+      if (scv[u] != 0.0f) {
+        if (c < n2p) last2 = max(last2, c + 1);
+        else if (c < n2p + n4p) last4 = max(last4, c - n2p + 1);
+        else last8 = max(last8, c - n2p - n4p + 1);
+      }
+    }
+  }
+  mloc = rdkv_wave_max(mloc);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    last2 = max(last2, __shfl_xor(last2, o, 64));
+    last4 = max(last4, __shfl_xor(last4, o, 64));
+    last8 = max(last8, __shfl_xor(last8, o, 64));
+  }
+  if (lane == 0) {
+    s_red[wave] = mloc;
+    s_ext[4 * wave] = last2;
+    s_ext[4 * wave + 1] = last4;
+    s_ext[4 * wave + 2] = last8;
+  }
+  __syncthreads();
+  // executed steps: p planes of d dwords per segment
+  const int e2 = max(max(s_ext[0], s_ext[4]), max(s_ext[8], s_ext[12])), e4 = max(max(s_ext[1], s_ext[5]), max(s_ext[9], s_ext[13])),
+            e8 = max(max(s_ext[2], s_ext[6]), max(s_ext[10], s_ext[14]));
+  const int p2 = sub2 ? (e2 + sub2 - 1) / sub2 : 0, p4 = sub4 ? (e4 + sub4 - 1) / sub4 : 0, p8 = e8 ? 1 : 0;
+  const int d2 = p2 > 1 ? nd2 : (e2 + 3) >> 2, d4 = p4 > 1 ? nd4 : (e4 + 3) >> 2, d8 = (e8 + 3) >> 2;
+  // (table entries per segment: its steps, made even by a padding entry)
+  const int E2 = (d2 * p2 + 1) & ~1, E4 = (d4 * p4 + 1) & ~1, E8 = (d8 * p8 + 1) & ~1, E = E2 + E4 + E8;
+  // entry -> dword, plane, first channel and row bytes of its segment; sub = 0 for an entry that
+  // is padding or lies past the end (the operand reloads run two entries ahead)
+  auto entry_of = [&](int en, int &jd, int &p, int &sub, int &c0) {
+    jd = p = sub = c0 = 0;
+    if (en < E2) { if (en < d2 * p2) { k_split_step(en, p2, jd, p); sub = sub2; } }
+    else if (en < E2 + E4) { if (en - E2 < d4 * p4) { k_split_step(en - E2, p4, jd, p); sub = sub4; c0 = n2p; } }
+    else if (en - E2 - E4 < d8 * p8) { jd = en - E2 - E4; sub = n8; c0 = n2p + n4p; }
+  };
+  for (int i = tl; i < (E + 2) * 4; i += 256) {   // 1024 + zero point of every code of every step
+    const int k = i & 3;
+    int jd, p, sub, c0;
+    entry_of(i >> 2, jd, p, sub, c0);
+    const int j = 4 * jd + (k & 1) * 2 + (k >> 1);
+    s_zp[i] = (_Float16)(1024.0f + (j < sub ? zp_whole(s_zpf[c0 + p * sub + j]) : 0.0f));
+  }
+#pragma unroll
+  for (int hh = 0; hh < NG; ++hh) {  // what the operands do not carry of the zero points (normally 0)
+    const int g = wave + 4 * hh;
+    float b = 0.0f;
+    for (int c = lane; c < Dp; c += 64) {
+      const float z = s_zpf[c];
+      b += (z - zp_whole(z)) * s_qs[c * NHD + g];
+    }
+    b = rdkv_wave_sum(b);
+    if (lane == 0) s_bias[g] = b;
+  }
+  const float big = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  int ex = 0;   // big = m * 2^x with 0.5 <= m < 1  ->  2^(14 - x)
+  if (big > 0.0f && big <= 3.0e38f) ex = min(max(14 - ((int)((__float_as_uint(big) >> 23) & 0xffu) - 126), -100), 100);
+  const float up = __uint_as_float((uint32_t)(127 + ex) << 23), back = __uint_as_float((uint32_t)(127 - ex) << 23);
+  for (int i = tl; i < (E + 2) * NG * 4; i += 256) {
+    const int hl = i & 3, hg = (i >> 2) % NG, en = (i >> 2) / NG;
+    int jd, p, sub, c0;
+    entry_of(en, jd, p, sub, c0);
+    _Float16 hi[4], lo[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int j = 4 * jd + (k & 1) * 2 + (k >> 1);
+      const float x = j < sub ? s_qs[(c0 + p * sub + j) * NHD + 4 * hg + hl] * up : 0.0f;
+      hi[k] = (_Float16)x;
+      lo[k] = (_Float16)(x - (float)hi[k]);
+    }
+    _Float16 *o = s_op + (size_t)(en * NG + hg) * 32 + hl * 4;
+    *reinterpret_cast<half4_t *>(o) = half4_t{hi[0], hi[1], hi[2], hi[3]};
+    *reinterpret_cast<half4_t *>(o + 16) = half4_t{lo[0], lo[1], lo[2], lo[3]};
+  }
+  __syncthreads();
+
+  // ---- tiles ------------------------------------------------------------------------------------
+  // (Giving each wavefront a quarter of the steps for all 256 tokens, so that one LDS read of a
+  // step's tables serves four tokens, was measured slower: the four accumulator sets cost a
+  // third of the resident workgroups.)
+  const _Float16 *op = s_op + ln * 4;
+  const uint2 *zop = reinterpret_cast<const uint2 *>(s_zp);
+  for (;;) {
+    const int next = tile + gridDim.x;
+    const bool more = next < ntiles;
+    if (more) issue_rows(next);
+    const int64_t t0 = (int64_t)tile * 256;
+    const int ntok = T - t0 < 256 ? (int)(T - t0) : 256;
+    floatx4 acc[NG][2];
+#pragma unroll
+    for (int hg = 0; hg < NG; ++hg) acc[hg][0] = acc[hg][1] = floatx4{0.f, 0.f, 0.f, 0.f};
+    {
+      const Run r0 = run_of(tile, 0), r1 = run_of(tile, 1), r2 = run_of(tile, 2);
+      int e = 0;
+      KStepOps<NG> cur[2] = {k_load_ops<NG>(op, zop, 0), k_load_ops<NG>(op, zop, 1)};
+      const int f2 = rows_off + r0.lds + tl * sub2, f4 = rows_off + r1.lds + tl * sub4, f8 = rows_off + r2.lds + tl * n8;
+      if (p2 == 1) k_segment_steps<2, 1, NG>(lds32, f2, d2, op, zop, e, cur, acc);
+      else if (p2 == 2) k_segment_steps<2, 2, NG>(lds32, f2, d2, op, zop, e, cur, acc);
+      else if (p2 == 3) k_segment_steps<2, 3, NG>(lds32, f2, d2, op, zop, e, cur, acc);
+      else if (p2 == 4) k_segment_steps<2, 4, NG>(lds32, f2, d2, op, zop, e, cur, acc);
+      if (p4 == 1) k_segment_steps<4, 1, NG>(lds32, f4, d4, op, zop, e, cur, acc);
+      else if (p4 == 2) k_segment_steps<4, 2, NG>(lds32, f4, d4, op, zop, e, cur, acc);
+      if (p8 == 1) k_segment_steps<8, 1, NG>(lds32, f8, d8, op, zop, e, cur, acc);
+    }
+    const int tok = wave * 64 + (lane & ~3);   // this lane holds tokens tok..tok+3 of head ln
+#pragma unroll
+    for (int hg = 0; hg < NG; ++hg) {
+      const int g = g0 + 4 * hg + ln;
+      if (g < G && tok < ntok) {
+        const float bias = s_bias[4 * hg + ln];
+        float v[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = ((acc[hg][0][i] + acc[hg][1][i]) * back - bias) * kInvSqrtD;
+        float *dst = out + (int64_t)(hkv * G + g) * out_sh + t0 + tok;
+        if (tok + 3 < ntok && ((uintptr_t)dst & 15) == 0) {
+          *reinterpret_cast<float4 *>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (tok + i < ntok) dst[i] = v[i];
+        }
+      }
+    }
+    if (!more) break;
+    __syncthreads();   // every wavefront has read its rows
+    store_rows(next);
+    __syncthreads();
+    tile = next;
+  }
+}
+
+// Compute units of the current device, asked once per device (0 = not asked yet; a race between
+// two first calls stores the same number twice).
+int compute_units() {
+  static int cu_of_device[64];
+  int dev = 0, n_cu = 256;
+  if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+    if (cu_of_device[dev] == 0) {
+      int v = 0;
+      if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+        cu_of_device[dev] = v;
+    }
+    if (cu_of_device[dev] > 0) n_cu = cu_of_device[dev];
+  }
+  return n_cu;
 }
 
 __global__ void zero_rows_kernel(float *out, int64_t out_sh, int64_t T) {
@@ -566,16 +896,41 @@ RDKV_API int rdkv_k_qk_dot(const void *q, int q_dtype, int64_t q_stride_h, int H
   const int sub2 = n2p / 4, sub4 = n4p / 2;
   const bool dense = (n2p == 0 || k2_stride_t == sub2) && (n4p == 0 || k4_stride_t == sub4) &&
                      (n8 == 0 || k8_stride_t == n8);
-  const size_t staged = shmem + (size_t)256 * (sub2 + sub4 + n8) + 3 * 32;
-  static_assert(kGB == 4, "k_qk_dot_staged_kernel reads four heads as one float4");
-  if (dense && staged <= 64 * 1024) {
-    hipLaunchKernelGGL(k_qk_dot_staged_kernel, dim3((unsigned)tblocks, H_kv), dim3(256), staged, s, q, q_dtype,
-                       q_stride_h, H_q / H_kv, K2, k2_stride_h, K4, k4_stride_h, K8, k8_stride_h,
-                       (const __half *)scale_f16, (const __half *)zp_f16, ks_stride_h, perm, perm_stride_h, n2p,
-                       n4p, n8, T_eff, out, out_stride_h);
+  const int G = H_q / H_kv;
+  const int ng = G > 4 ? 2 : 1;
+  const int nsteps = 4 * ((sub2 + 3) / 4) + 2 * ((sub4 + 3) / 4) + (n8 + 3) / 4;
+  const size_t staged = (size_t)(4 * ng * Dp + 4 * ng + 4 + 16 + ((Dp + 3) & ~3)) * sizeof(float) +
+                        (size_t)(nsteps + 6) * ng * 64 + (size_t)(((nsteps + 6) * 4 + 7) & ~7) * 2 +
+                        (size_t)256 * (sub2 + sub4 + n8) + 3 * 32;
+  const int pieces = (sub2 + 15) / 16 + (sub4 + 15) / 16 + (n8 + 15) / 16;   // 16-byte row pieces per thread
+  if (dense && staged <= 64 * 1024 && Dp <= 512 && pieces <= 16) {
+    // workgroups per KV head: all tiles when they are resident at once, else an even share of the tiles
+    const int cus = compute_units();
+    const bool wide = pieces > 8, two = Dp > 256;
+    // resident workgroups per compute unit: by registers (what the variant is compiled for), by LDS
+    const int64_t by_regs = k_mfma_residency(ng, wide ? 16 : 8);
+    const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>(by_regs, (int64_t)(160 * 1024) / (int64_t)(staged + 1024)));
+    const int64_t slots = std::max<int64_t>(1, per_cu * cus / H_kv);
+    const int64_t rounds = rdkv_cdiv(tblocks, slots);
+    const unsigned wph = (unsigned)rdkv_cdiv(tblocks, rounds);
+#define RDKV_LAUNCH_K_MFMA(NG_, KMAX_, CPT_)                                                                      \
+  for (int g0 = 0; g0 < G; g0 += 4 * NG_)                                                                          \
+  hipLaunchKernelGGL((k_qk_dot_mfma_kernel<NG_, KMAX_, CPT_>), dim3(wph, H_kv), dim3(256), staged, s, q, q_dtype,  \
+                     q_stride_h, G, g0, K2, k2_stride_h, K4, k4_stride_h, K8, k8_stride_h,                         \
+                     (const __half *)scale_f16, (const __half *)zp_f16, ks_stride_h, perm, perm_stride_h, n2p,    \
+                     n4p, n8, T_eff, out, out_stride_h)
+    if (ng == 1 && !wide && !two) RDKV_LAUNCH_K_MFMA(1, 8, 1);
+    else if (ng == 1 && !wide) RDKV_LAUNCH_K_MFMA(1, 8, 2);
+    else if (ng == 1 && !two) RDKV_LAUNCH_K_MFMA(1, 16, 1);
+    else if (ng == 1) RDKV_LAUNCH_K_MFMA(1, 16, 2);
+    else if (!wide && !two) RDKV_LAUNCH_K_MFMA(2, 8, 1);
+    else if (!wide) RDKV_LAUNCH_K_MFMA(2, 8, 2);
+    else if (!two) RDKV_LAUNCH_K_MFMA(2, 16, 1);
+    else RDKV_LAUNCH_K_MFMA(2, 16, 2);
+#undef RDKV_LAUNCH_K_MFMA
   } else {
     hipLaunchKernelGGL(k_qk_dot_strided_kernel, dim3((unsigned)tblocks, H_kv), dim3(256), shmem, s, q, q_dtype,
-                       q_stride_h, H_q / H_kv, K2, k2_stride_h, k2_stride_t, K4, k4_stride_h, k4_stride_t, K8,
+                       q_stride_h, G, K2, k2_stride_h, k2_stride_t, K4, k4_stride_h, k4_stride_t, K8,
                        k8_stride_h, k8_stride_t, (const __half *)scale_f16, (const __half *)zp_f16, ks_stride_h,
                        perm, perm_stride_h, n2p, n4p, n8, T_eff, out, out_stride_h);
   }
