@@ -318,7 +318,7 @@ def pack_layer_sections(cfg, K, V, vb, kb, args, torch, dev):
     return pack_info, select_info
 
 
-def pack_sample_section(pack_sample, pack_info, cfg, torch, dev):
+def pack_sample_section(pack_sample, pack_info, cfg, torch, dev, select_info=None):
     """The first layers of a sequence packed back to back (one planning launch and one host read
     for all of them, the host side of a layer overlapping the kernels of the one before)."""
     import numpy as np
@@ -336,6 +336,28 @@ def pack_sample_section(pack_sample, pack_info, cfg, torch, dev):
     pack_info["pack_layers_sample"] = len(pack_sample)
     pack_info["pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
     pack_info["pack_GBps_of_fp16_input_batched"] = sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
+    if select_info is not None:
+        # selection + packing of the same layers in one call: the knapsack launches see
+        # layers x heads rows at once instead of one layer's heads
+        from rdkv_amd import knapsack_solver, obkv_fast
+        gsel = torch.Generator().manual_seed(4243)
+        Ks, Vs = [p[0] for p in pack_sample], [p[1] for p in pack_sample]
+        H_kv, T_ctx = int(Ks[0].shape[1]), int(Ks[0].shape[2])
+        tok = [torch.exp(torch.randn(H_kv, T_ctx, generator=gsel) * 1.5 + 2.0).to(dev) for _ in Ks]
+        chn = [torch.exp(torch.randn(H_kv, 128, generator=gsel)).to(dev) for _ in Ks]
+        sel_kw = dict(gqa_factor=cfg.G, token_budget=max(T_ctx // 4, 1), k_budget_ratio=0.5, obs_window=32,
+                      pool_kernel_size=7, pool_padding="reflect", pool_type="avg", v_bit_options=None,
+                      k_bit_options=torch.tensor([0.0, 2.0, 4.0, 8.0]),
+                      eps_V=knapsack_solver.DEFAULT_EPSILON_V, eps_K=knapsack_solver.DEFAULT_EPSILON_K)
+        times = []
+        for _ in range(4):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            obkv_fast._perhead_select_and_pack_layers(Ks, Vs, tok, chn, **sel_kw)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t0) * 1e3)
+        select_info["select_and_pack_layers_sample"] = len(pack_sample)
+        select_info["select_and_pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
 
 
 # ---------------------------------------------------------------------------------------------
@@ -634,7 +656,7 @@ def main():
     groups = build_workload(cfg, dev, torch, on_first=on_first, pack_sample=None if args.fused_only else pack_sample)
     pack_info, select_info = first.get("pack"), first.get("select")
     if len(pack_sample) > 1:
-        pack_sample_section(pack_sample, pack_info, cfg, torch, dev)
+        pack_sample_section(pack_sample, pack_info, cfg, torch, dev, select_info)
     pack_sample.clear()
     qs = torch.cat([g[2] for g in groups]).contiguous()
     cache = stream_cache.build_stream_cache([(g[0], g[1]) for g in groups], cfg.G,
