@@ -192,3 +192,103 @@ def test_softmax_rows_matches_the_library_softmax(T_old, n_new, masked, aligned)
     # nothing beyond the row was written
     assert torch.equal(buf[:, off + T_old + n_new:].cpu(), (torch.randn(H, width + off, generator=torch.Generator().manual_seed(
         T_old * 31 + n_new)) * 3.0)[:, off + T_old + n_new:])
+
+
+def _random_k_layer(rng, H_kv, G, T, widths, *, pad_tail=True, byte_offset=0, fractional_zp=False):
+    """A K layer in the reference layout built by hand: random codes, per-channel scale / zero
+    point, a random per-query-head channel permutation; trailing channels of every segment get a
+    zero scale for some heads (the padding of a head narrower than the widest one), one channel in
+    the middle of a segment too.  Returns (layer, float64 scores function)."""
+    import types
+    sub2, sub4, n8 = widths
+    n2p, n4p = 4 * sub2, 2 * sub4
+    Dp = n2p + n4p + n8
+    H_q = H_kv * G
+
+    def seg(width):
+        if width == 0:
+            return None
+        flat = torch.from_numpy(rng.integers(0, 256, size=H_kv * T * width + byte_offset, dtype=np.uint8)).to(DEV)
+        return flat[byte_offset:].view(1, H_kv, T, width)       # dense rows, base address off by byte_offset
+
+    K2, K4, K8 = seg(sub2), seg(sub4), seg(n8)
+    scale = rng.uniform(0.002, 0.02, size=(H_kv, Dp)).astype(np.float16)
+    if pad_tail:
+        for h in range(H_kv):
+            for lo, n in ((0, n2p), (n2p, n4p), (n2p + n4p, n8)):
+                if n > 1 and h % 2 == 1:
+                    scale[h, lo + n - max(1, n // (2 + h % 3)):lo + n] = 0      # a narrower head
+            if Dp > 8:
+                scale[h, (3 * h + 5) % Dp] = 0                                   # a dead channel in the middle
+    zp = rng.integers(0, 200, size=(H_kv, Dp)).astype(np.float16)
+    if fractional_zp:
+        zp = (zp.astype(np.float32) + rng.uniform(-0.5, 0.5, size=zp.shape)).astype(np.float16)
+    perm = np.stack([rng.permutation(128)[np.arange(Dp) % 128] for _ in range(H_q)]).astype(np.int64)
+    layer = types.SimpleNamespace(
+        K_2bit=K2, K_4bit=K4, K_8bit=K8, K_ch_seg_bounds=(n2p, n4p, n8),
+        K_ch_scale=torch.from_numpy(scale).to(DEV).view(1, H_kv, 1, Dp),
+        K_ch_zp=torch.from_numpy(zp).to(DEV).view(1, H_kv, 1, Dp),
+        K_ch_perm_padded_idx_for_Q=torch.from_numpy(perm).to(DEV), K_ch_perm_padded_idx=None)
+
+    def scores64(q):
+        out = np.empty((H_q, T), np.float64)
+        q64 = q.astype(np.float64)
+        for h in range(H_kv):
+            cols = []
+            if sub2:
+                b = t2n(K2[0, h]).astype(np.int64)
+                cols += [(b >> (2 * f)) & 3 for f in range(4)]          # byte j, field f -> channel j + f*sub2
+            if sub4:
+                b = t2n(K4[0, h]).astype(np.int64)
+                cols += [b & 15, b >> 4]                                 # byte j -> channels j, j + sub4
+            if n8:
+                cols.append(t2n(K8[0, h]).astype(np.int64))
+            codes = np.concatenate(cols, axis=1).astype(np.float64)      # [T, Dp] in padded channel order
+            deq = (codes - zp[h].astype(np.float64)) * scale[h].astype(np.float64)
+            for g in range(G):
+                hq = h * G + g
+                out[hq] = deq @ q64[hq, perm[hq]] / np.sqrt(128.0)
+        return out
+
+    return layer, scores64
+
+
+@pytest.mark.parametrize("H_kv,G,T,widths,kw", [
+    (8, 4, 40000, (12, 21, 59), {}),                          # more tiles than resident workgroups: the tile loop
+    (2, 8, 257, (0, 0, 128), {}),                             # 8-bit only, two head groups at once
+    (1, 1, 1, (32, 0, 0), {"pad_tail": False}),               # one token, 2-bit only, all four planes in use
+    (3, 5, 700, (5, 7, 3), {"byte_offset": 3}),               # odd widths, unaligned rows, G not a multiple of 4
+    (3, 12, 300, (0, 64, 0), {}),                             # 4-bit only, G = 12: two launches of eight heads
+    (2, 4, 600, (8, 32, 128), {"fractional_zp": True}),       # 288 padded channels, 168-byte rows, odd zero points
+    (4, 4, 5000, (3, 2, 9), {"byte_offset": 5}),              # short rows
+])
+@pytest.mark.parametrize("q_dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_k_scores_random_layouts(H_kv, G, T, widths, kw, q_dtype):
+    """The matrix-core K kernel on hand-built layers against float64 arithmetic on the same bytes
+    (every token), and against the kernel that reads rows in place on widened views."""
+    import dataclasses
+    if q_dtype != torch.float32 and T > 1000:
+        pytest.skip("the long case runs once")
+    rng = np.random.default_rng(H_kv * 1000 + G * 100 + T + sum(widths))
+    layer, scores64 = _random_k_layer(rng, H_kv, G, T, widths, **kw)
+    q = (torch.from_numpy(rng.standard_normal((H_kv * G, 128)).astype(np.float32)) * 3.0).to(q_dtype)
+    exp = scores64(q.float().numpy())
+    buf = torch.full((H_kv * G, T + 5), 7.0, device=DEV)
+    kk.k_mixed_qk_dot_into(q.to(DEV), layer, T, buf[:, 1:T + 1])          # rows off 16-byte alignment
+    got = t2n(buf[:, 1:T + 1]).astype(np.float64)
+    scale = max(1.0, float(np.abs(exp).max()))
+    assert np.abs(got - exp).max() <= 4e-6 * scale, f"max error {np.abs(got - exp).max():.3e} at |scores| <= {scale:.1f}"
+    assert float((buf[:, 0] - 7.0).abs().max()) == 0.0 and float((buf[:, T + 1:] - 7.0).abs().max()) == 0.0
+
+    def widened(t):
+        if t is None:
+            return None
+        wide = torch.zeros(t.shape[:-1] + (t.shape[-1] + 2,), dtype=t.dtype, device=t.device)
+        wide[..., :t.shape[-1]] = t
+        return wide[..., :t.shape[-1]]
+
+    import copy
+    in_place = copy.copy(layer)
+    in_place.K_2bit, in_place.K_4bit, in_place.K_8bit = widened(layer.K_2bit), widened(layer.K_4bit), widened(layer.K_8bit)
+    other = t2n(kk.k_mixed_qk_dot(q.to(DEV), in_place, T)).astype(np.float64)
+    assert np.abs(other - exp).max() <= 4e-5 * scale
