@@ -874,6 +874,7 @@ RDKV_API int rdkv_k_qk_dot(const void *q, int q_dtype, int64_t q_stride_h, int H
                            int n8, int64_t T_eff, float *out, int64_t out_stride_h, void *stream) {
   RDKV_REQUIRE(H_q > 0 && H_kv > 0 && H_q % H_kv == 0, "rdkv_k_qk_dot: H_q=%d not a multiple of H_kv=%d", H_q,
                H_kv);
+  RDKV_REQUIRE(H_kv <= 65535, "rdkv_k_qk_dot: H_kv=%d exceeds the launch grid", H_kv);
   RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "rdkv_k_qk_dot: unknown q dtype %d", q_dtype);
   RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
                "rdkv_k_qk_dot: bad segment sizes (%d,%d,%d)", n2p, n4p, n8);
