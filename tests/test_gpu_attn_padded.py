@@ -253,7 +253,7 @@ def _random_k_layer(rng, H_kv, G, T, widths, *, pad_tail=True, byte_offset=0, fr
     return layer, scores64
 
 
-@pytest.mark.parametrize("H_kv,G,T,widths,kw", [
+_K_LAYOUT_CASES = [
     (8, 4, 40000, (12, 21, 59), {}),                          # more tiles than resident workgroups: the tile loop
     (2, 8, 257, (0, 0, 128), {}),                             # 8-bit only, two head groups at once
     (1, 1, 1, (32, 0, 0), {"pad_tail": False}),               # one token, 2-bit only, all four planes in use
@@ -261,14 +261,15 @@ def _random_k_layer(rng, H_kv, G, T, widths, *, pad_tail=True, byte_offset=0, fr
     (3, 12, 300, (0, 64, 0), {}),                             # 4-bit only, G = 12: two launches of eight heads
     (2, 4, 600, (8, 32, 128), {"fractional_zp": True}),       # 288 padded channels, 168-byte rows, odd zero points
     (4, 4, 5000, (3, 2, 9), {"byte_offset": 5}),              # short rows
-])
-@pytest.mark.parametrize("q_dtype", [torch.float32, torch.float16, torch.bfloat16])
+]
+
+
+@pytest.mark.parametrize("H_kv,G,T,widths,kw,q_dtype", [
+    case + (dt,) for case in _K_LAYOUT_CASES for dt in (torch.float32, torch.float16, torch.bfloat16)
+    if dt == torch.float32 or case[2] <= 1000])               # the long cases run once
 def test_k_scores_random_layouts(H_kv, G, T, widths, kw, q_dtype):
     """The matrix-core K kernel on hand-built layers against float64 arithmetic on the same bytes
     (every token), and against the kernel that reads rows in place on widened views."""
-    import dataclasses
-    if q_dtype != torch.float32 and T > 1000:
-        pytest.skip("the long case runs once")
     rng = np.random.default_rng(H_kv * 1000 + G * 100 + T + sum(widths))
     layer, scores64 = _random_k_layer(rng, H_kv, G, T, widths, **kw)
     q = (torch.from_numpy(rng.standard_normal((H_kv * G, 128)).astype(np.float32)) * 3.0).to(q_dtype)
