@@ -102,8 +102,19 @@ SIGNATURES = {
 _lib: Optional[ctypes.CDLL] = None
 
 
+_seen_library: Optional[str] = None
+
+
 def available() -> bool:
-    return os.path.exists(LIB_PATH)
+    """Whether the built library is there.  Asked on every call of every entry point, so a path
+    that has been seen once is not looked up again (a library that is missing is)."""
+    global _seen_library
+    if _seen_library == LIB_PATH:
+        return True
+    if os.path.exists(LIB_PATH):
+        _seen_library = LIB_PATH
+        return True
+    return False
 
 
 def load() -> ctypes.CDLL:
@@ -161,7 +172,14 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(dev: torch.device) -> int:
+    """The current HIP stream of ``dev`` as the handle the C ABI takes (the raw query costs a
+    tenth of building a ``torch.cuda.Stream`` object, which the per-layer entry points feel)."""
+    if _raw_stream is not None:
+        return _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(dev).cuda_stream
 
 
@@ -175,7 +193,7 @@ def workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     that is outgrown is kept alive, not freed: a HIP graph captured earlier on that stream has its
     address baked in, and its replays must not write into memory another tensor has since been
     given.  (Growth is by doubling, so the retired buffers add up to less than the live one.)"""
-    key = (dev.index, torch.cuda.current_stream(dev).cuda_stream)
+    key = (dev.index, stream_of(dev))
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
         if buf is not None:

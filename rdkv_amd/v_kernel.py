@@ -53,23 +53,30 @@ def _sq(t):
 
 
 def _seg(t, width):
-    t = _sq(t)
-    if t is None or t.numel() == 0:
+    """-> (address or None, head stride) of a [H_kv, N, width] code tensor with dense rows."""
+    if t is None:
+        return None, 0
+    if t.dim() == 4:
+        t = t.squeeze(0)
+    if t.numel() == 0:
         return None, 0
     assert t.shape[-1] == width
-    t = t if t.is_contiguous() or (t.stride(2) == 1 and t.stride(1) == width) else t.contiguous()
-    return t, t.stride(0)
+    if not (t.stride(2) == 1 and t.stride(1) == width):
+        t = t.contiguous()
+    return t.data_ptr(), t.stride(0)
 
 
 def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_head, seg_bounds,
             out, V16, n_v16_per_head, max_T_v):
-    if not _lib.available():
-        raise RuntimeError("rdkv HIP backend is not available.")
-    dev = _lib.require_device(attn_weights, out)
-    H_q = attn_weights.shape[0]
+    # (this runs once per layer and decode step: views and helper calls are kept to what the launch needs)
+    lib = _lib.load()
+    w = attn_weights
+    if not (w.is_cuda and out.is_cuda):
+        _lib.require_device(w, out)
+    dev = w.device
+    H_q = w.shape[0]
     sc, zp = _sq(V_scale), _sq(V_zp)
     H_kv = sc.shape[0]
-    w = attn_weights
     if w.dtype != torch.float32:
         w = w.float()
     if w.stride(1) != 1:
@@ -78,24 +85,25 @@ def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_
     V2, v2h = _seg(V_2bit, D // 4)
     V4, v4h = _seg(V_4bit, D // 2)
     V8, v8h = _seg(V_8bit, D)
-    sc = sc.reshape(H_kv, -1)
-    zp = zp.reshape(H_kv, -1)
-    if sc.numel() and sc.stride(1) != 1:
-        sc, zp = sc.contiguous(), zp.contiguous()
-    N2, N4, N8 = (int(v) for v in seg_bounds)
-    v16, v16h = None, 0
+    # scale / zero point rows: [H_kv, T] or [H_kv, T, 1] with unit token stride
+    n_meta = sc.numel()
+    if n_meta and not (sc.stride(1) == 1 and zp.stride(1) == 1 and zp.stride(0) == sc.stride(0)):
+        sc, zp = sc.reshape(H_kv, -1).contiguous(), zp.reshape(H_kv, -1).contiguous()
+    N2, N4, N8 = seg_bounds
+    v16 = v16h = n16 = None
     if V16 is not None and n_v16_per_head is not None:
         v16 = V16 if V16.is_contiguous() else V16.contiguous()
         v16h = v16.stride(0)
-    lib = _lib.load()
-    need = lib.rdkv_v_weighted_sum_workspace_bytes(H_q)
-    ws = _lib.workspace(dev, need)
+        n16 = n_v16_per_head.data_ptr()
+        v16 = v16.data_ptr() if v16.numel() else None
+    stream = _lib.stream_of(dev)
+    ws = _lib.workspace(dev, lib.rdkv_v_weighted_sum_workspace_bytes(H_q))
     _lib.check(lib.rdkv_v_weighted_sum(
-        w.data_ptr(), w.stride(0), H_q, H_kv, _lib.ptr(V2), v2h, _lib.ptr(V4), v4h, _lib.ptr(V8), v8h,
-        _lib.ptr(sc), _lib.ptr(zp), sc.stride(0) if sc.numel() else 0,
-        _lib.ptr(seg_bounds_per_head), N2, N4, N8,
-        _lib.ptr(v16), v16h, _lib.ptr(n_v16_per_head) if v16 is not None else None, int(max_T_v),
-        out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
+        w.data_ptr(), w.stride(0), H_q, H_kv, V2, v2h, V4, v4h, V8, v8h,
+        sc.data_ptr() if n_meta else None, zp.data_ptr() if n_meta else None, sc.stride(0) if n_meta else 0,
+        None if seg_bounds_per_head is None else seg_bounds_per_head.data_ptr(), int(N2), int(N4), int(N8),
+        v16, v16h or 0, n16 if v16 is not None else None, int(max_T_v),
+        out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), stream))
 
 
 # ---- single bit-width entry points (triton_v_kernel.py:1108-1220) -----------------------
