@@ -336,6 +336,18 @@ def pack_sample_section(pack_sample, pack_info, cfg, torch, dev, select_info=Non
     pack_info["pack_layers_sample"] = len(pack_sample)
     pack_info["pack_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
     pack_info["pack_GBps_of_fp16_input_batched"] = sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
+    # the streaming re-layout of the same layers in one call (one unit table, one partition)
+    from rdkv_amd import stream_cache
+    packed = packing.pack_layers_per_head([p[0] for p in pack_sample], [p[1] for p in pack_sample], vb_all, kb_all, cfg.G)
+    times = []
+    for _ in range(4):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        stream_cache.build_stream_cache(packed, cfg.G)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+    pack_info["relayout_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
+    del packed
     if select_info is not None:
         # selection + packing of the same layers in one call: the knapsack launches see
         # layers x heads rows at once instead of one layer's heads

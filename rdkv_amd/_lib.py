@@ -179,6 +179,8 @@ def stream_of(dev: torch.device) -> int:
     """The current HIP stream of ``dev`` as the handle the C ABI takes (the raw query costs a
     tenth of building a ``torch.cuda.Stream`` object, which the per-layer entry points feel)."""
     if _raw_stream is not None:
+        if not isinstance(dev, torch.device):
+            dev = torch.device(dev)
         return _raw_stream(dev.index if dev.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(dev).cuda_stream
 

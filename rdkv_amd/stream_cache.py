@@ -230,6 +230,9 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
     units_all, blobs, keep_alive, scale_max = [], [], [], []
     stream_bytes = algo_bytes = 0
     H_q = None
+    # First the host side of every entry (unit descriptors with offsets relative to the entry's
+    # blob, slot tables, sizes), then ONE upload of all descriptors and tables, then the launches.
+    plans = []
     for gi, (pl, nvo) in enumerate(layers):
         sb0, ab0 = stream_bytes, algo_bytes
         H_kv = pl.K_ch_scale.shape[1]
@@ -237,7 +240,6 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         tok, ch = _layer_counts(pl, H_kv)
         m2, m4, m8 = (int(v) for v in pl.K_ch_seg_bounds)
         n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
-        Dp = n2p + n4p + m8
         units = np.zeros(H_kv, dtype=UNIT_DTYPE)
         src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
         off = 0
@@ -273,11 +275,21 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
                            + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
                            + 256 * n_tok[3])
+        plans.append((units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p))
+        if entry_bytes is not None:
+            entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
+    units_dev = torch.from_numpy(np.concatenate([pn[0] for pn in plans]).view(np.uint8).copy()).to(dev)
+    src_dev_all = torch.from_numpy(np.concatenate([pn[1] for pn in plans])).to(dev)
+    unit_row = src_row = 0
+    for (pl, nvo), (units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p) in zip(layers, plans):
+        Dp = n2p + n4p + m8
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
         assert base % 256 == 0
-        rel_units = torch.from_numpy(units.view(np.uint8).copy()).to(dev)
-        src_dev = torch.from_numpy(src_tab).to(dev)
+        rel_units_ptr = units_dev.data_ptr() + unit_row * UNIT_DTYPE.itemsize
+        src_ptr = src_dev_all.data_ptr() + src_row * src_tab.shape[1] * 2
+        unit_row += H_kv
+        src_row += H_kv
 
         def seg3(t):
             if t is None or t.numel() == 0:
@@ -320,7 +332,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             _lib.ptr(vs), _lib.ptr(vz), vs.stride(0) if vs.numel() else 0,
             _lib.ptr(V16), v16h, int(pl.T_eff),
             perm.data_ptr(), perm_sh, ks.data_ptr(), kz.data_ptr(), ks.stride(0),
-            rel_units.data_ptr(), src_dev.data_ptr(), src_tab.shape[1], H_kv, m8, max_tiles, blob.data_ptr(),
+            rel_units_ptr, src_ptr, src_tab.shape[1], H_kv, m8, max_tiles, blob.data_ptr(),
             stream))
         # kernel-side descriptors carry absolute addresses
         for name in ("k_off", "sz_off", "qtab_off"):
@@ -328,13 +340,11 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         units["v_off"] += base
         units_all.extend(units)
         blobs.append(blob)
-        if entry_bytes is not None:
-            entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
         # the temporaries stay alive until the relayout kernels have run
-        keep_alive.append((rel_units, src_dev, K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
+        keep_alive.append((K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
     scale_max_np = torch.stack(scale_max).transpose(1, 2).reshape(-1, 2).cpu().numpy().astype(np.float32)  # (synchronizes)
     torch.cuda.current_stream(dev).synchronize()
-    del keep_alive
+    del keep_alive, units_dev, src_dev_all
     return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
 
 
