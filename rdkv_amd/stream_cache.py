@@ -244,6 +244,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
         off = 0
         max_tiles = 0
+        rows = []            # per head: the descriptor's fields, written to the record array in one go
         for h in range(H_kv):
             n_tok = tok[h]
             c2, c4, c8 = ch[h]
@@ -253,28 +254,30 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             src_tab[h, :len(src)] = src
             qt_nbytes = len(src) * SLOT_DTYPE.itemsize
             tiles = [-(-n // TILE) for n in n_tok]
-            max_tiles = max(max_tiles, sum(tiles))
+            n_tiles, n_q_tiles = sum(tiles), sum(tiles[:3])
+            max_tiles = max(max_tiles, n_tiles)
             R = d8 + d4 + d2
-            u = units[h]
-            u["n_tok"] = n_tok
-            u["d8"], u["d4"], u["d2"] = d8, d4, d2
-            u["q_row"] = int(rows_of_entries[gi]) * H_q + h * G
-            u["k_off"] = off
-            off = _align(off + sum(tiles) * TILE * 4 * R)
+            k_off = off
+            off = _align(off + n_tiles * TILE * 4 * R)
+            v_off = []
             for c in range(4):
-                u["v_off"][c] = off
+                v_off.append(off)
                 off = _align(off + tiles[c] * V_TILE_BYTES[c])
-            u["sz_off"] = off
-            off = _align(off + sum(tiles[:3]) * TILE * 4)
-            u["qtab_off"] = off
+            sz_off = off
+            off = _align(off + n_q_tiles * TILE * 4)
+            qtab_off = off
             off = _align(off + qt_nbytes)
+            rows.append((tuple(n_tok), d8, d4, d2, int(rows_of_entries[gi]) * H_q + h * G, k_off, tuple(v_off),
+                         sz_off, qtab_off))
             # accounting
-            stream_bytes += (sum(tiles) * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
-                             + sum(tiles[:3]) * TILE * 4 + qt_nbytes)
+            stream_bytes += (n_tiles * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
+                             + n_q_tiles * TILE * 4 + qt_nbytes)
             row = -(-c2 // 4) + -(-c4 // 2) + c8
             algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
                            + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
                            + 256 * n_tok[3])
+        for i, name in enumerate(("n_tok", "d8", "d4", "d2", "q_row", "k_off", "v_off", "sz_off", "qtab_off")):
+            units[name] = [r[i] for r in rows]
         plans.append((units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p))
         if entry_bytes is not None:
             entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
