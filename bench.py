@@ -475,11 +475,12 @@ def padded_section(cfg, torch, dev, steps=50, layers=4):
 
     def run_softmax():
         st = _lib.stream_of(dev)
+        ws = _lib.workspace(dev, lib.rdkv_softmax_rows_workspace_bytes(cfg.H_q))
         for _, sp, _, _, T_old, scores, _ in items:
             mask = sp.softmax_mask
-            _lib.check(lib.rdkv_softmax_rows(
+            _lib.check(lib.rdkv_softmax_rows_ws(
                 scores.data_ptr(), scores.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0,
-                T_old, None, 0, 0, scores.data_ptr(), scores.stride(0), None, 0, cfg.H_q, st))
+                T_old, None, 0, 0, scores.data_ptr(), scores.stride(0), None, 0, cfg.H_q, ws.data_ptr(), ws.numel(), st))
 
     def run_v():
         for _, sp, v16, T_v, _, scores, out in items:

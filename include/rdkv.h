@@ -146,6 +146,17 @@ int rdkv_softmax_rows(const float *scores_old, int64_t so_stride_h, const float 
                       float *w_old, int64_t wo_stride_h, float *w_new, int64_t wn_stride_h,
                       int H_q, void *stream);
 
+/* rdkv_softmax_rows with a workspace of rdkv_softmax_rows_workspace_bytes(H_q) bytes: long rows
+ * (more than 64k scores) of few heads (one workgroup per head leaves most of the device idle) are then cut into up to
+ * 32 pieces, two launches (piece maxima and sums, then the weights); the same values up to the
+ * rounding of the sum.  Without a workspace, or for short rows, the call is rdkv_softmax_rows. */
+int64_t rdkv_softmax_rows_workspace_bytes(int H_q);
+int rdkv_softmax_rows_ws(const float *scores_old, int64_t so_stride_h, const float *mask,
+                         int64_t mask_stride_h, int64_t T_old, const float *scores_new,
+                         int64_t sn_stride_h, int64_t n_new, float *w_old, int64_t wo_stride_h,
+                         float *w_new, int64_t wn_stride_h, int H_q, void *workspace,
+                         int64_t workspace_bytes, void *stream);
+
 /* ---- triton_v_kernel.py : v_dequant_weighted_sum_dispatch_into (:1729-1760) */
 /* out[hq,d] = sum over 2/4/8-bit segments of w*(code-zp)*scale + fp16 zone B
  * (kernel math triton_v_kernel.py:638-750).  seg_bounds_dev: int32 [H_kv,3] per-head

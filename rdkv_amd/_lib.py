@@ -56,6 +56,8 @@ SIGNATURES = {
     "rdkv_dequant_f16": (I, [P, L, I, I, P, P, I, P, L, P]),
     "rdkv_k_qk_dot": (I, [P, I, L, I, I, P, L, L, P, L, L, P, L, L, P, P, L, P, L, I, I, I, L, P, L, P]),
     "rdkv_softmax_rows": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P]),
+    "rdkv_softmax_rows_workspace_bytes": (L, [I]),
+    "rdkv_softmax_rows_ws": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P, L, P]),
     "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
     "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,

@@ -231,11 +231,12 @@ def trizone_attention(q_2d: torch.Tensor, sp: PackedKVLayer, V16: Optional[torch
     s_new.copy_(torch.bmm(q_gqa, K_new.transpose(-1, -2)).reshape(H_q, n_new))
     # mask + global softmax over [A | B | C], written back in place as weights (:1743-1755)
     mask = sp.softmax_mask if (T_old > 0 and sp.softmax_mask is not None) else None
-    _lib.check(lib.rdkv_softmax_rows(
+    ws = _lib.workspace(dev, lib.rdkv_softmax_rows_workspace_bytes(H_q))
+    _lib.check(lib.rdkv_softmax_rows_ws(
         _lib.ptr(s_old), scores_buf.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0,
         T_old, s_new.data_ptr(), scores_buf.stride(0), n_new,
         _lib.ptr(s_old), scores_buf.stride(0), s_new.data_ptr(), scores_buf.stride(0), H_q,
-        _lib.stream_of(dev)))
+        ws.data_ptr(), ws.numel(), _lib.stream_of(dev)))
     if T_old > 0:
         v_dequant_weighted_sum_dispatch_into(s_old, sp, out, V16=V16, n_v16_per_head=n_v16_per_head,
                                              max_T_v=T_v)

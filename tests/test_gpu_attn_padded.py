@@ -154,13 +154,16 @@ def test_k_scores_strided_rows_match_dense_rows():
     (32768, 3, True, True), (32771, 64, False, True), (65536, 1, True, True), (70001, 5, True, True),
     (200000, 0, False, True), (4097, 9, True, False), (40000, 1, False, False), (0, 17, False, True),
     (29563, 1, "unaligned", True), (70003, 0, "unaligned", True)])
-def test_softmax_rows_matches_the_library_softmax(T_old, n_new, masked, aligned):
+@pytest.mark.parametrize("workspace", [False, True])
+def test_softmax_rows_matches_the_library_softmax(T_old, n_new, masked, aligned, workspace):
     """``rdkv_softmax_rows`` (fast_decode.py:1743-1755: mask added, softmax over [old | new], the
     weights written back in place) against the library's fp32 softmax over the concatenated row, for
     every row length the kernel variants split on (rows kept in registers up to 8k / 32k / 64k scores,
     streamed beyond; lengths that are not a multiple of 4; no old zone at all), masked columns at
-    -inf, and row views that are not 16-byte aligned (the element-wise kernel).  Tolerance 2e-7
-    absolute + 2e-5 relative (fp32, another summation order)."""
+    -inf, and row views that are not 16-byte aligned (the element-wise kernel).  With a workspace,
+    rows of more than 64k scores are cut into pieces, one workgroup each (two launches); a run of
+    columns as long as a piece is masked out entirely.  Tolerance 2e-7 absolute + 2e-5 relative
+    (fp32, another summation order)."""
     from rdkv_amd import _lib
     lib = _lib.load()
     H = 5
@@ -175,15 +178,24 @@ def test_softmax_rows_matches_the_library_softmax(T_old, n_new, masked, aligned)
         mask = torch.zeros(H, T_old + off)
         mask[:, off:][torch.rand(H, T_old, generator=g) < 0.3] = float("-inf")
         mask[:, off] = 0.0                           # at least one visible key per row
+        if T_old >= 32768:
+            mask[1::2, off + T_old // 4: off + T_old // 4 + T_old // 8] = float("-inf")   # whole pieces masked out
         mask = mask.to(DEV)[:, off:]
         if masked == "unaligned":                    # mask rows exactly as long as the old zone (the packer's)
             mask = mask[:, :T_old].contiguous()
     ref_in = torch.cat([s_old + (mask if mask is not None else 0.0), s_new], dim=1)
     ref = torch.softmax(ref_in, dim=-1)
-    _lib.check(lib.rdkv_softmax_rows(
-        _lib.ptr(s_old), rows.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0, T_old,
-        _lib.ptr(s_new), rows.stride(0), n_new, _lib.ptr(s_old), rows.stride(0), _lib.ptr(s_new), rows.stride(0),
-        H, _lib.stream_of(torch.device(DEV))))
+    if workspace:
+        ws = torch.empty(lib.rdkv_softmax_rows_workspace_bytes(H), dtype=torch.uint8, device=DEV)
+        _lib.check(lib.rdkv_softmax_rows_ws(
+            _lib.ptr(s_old), rows.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0, T_old,
+            _lib.ptr(s_new), rows.stride(0), n_new, _lib.ptr(s_old), rows.stride(0), _lib.ptr(s_new), rows.stride(0),
+            H, ws.data_ptr(), ws.numel(), _lib.stream_of(torch.device(DEV))))
+    else:
+        _lib.check(lib.rdkv_softmax_rows(
+            _lib.ptr(s_old), rows.stride(0), _lib.ptr(mask), mask.stride(0) if mask is not None else 0, T_old,
+            _lib.ptr(s_new), rows.stride(0), n_new, _lib.ptr(s_old), rows.stride(0), _lib.ptr(s_new), rows.stride(0),
+            H, _lib.stream_of(torch.device(DEV))))
     got = rows[:, :T_old + n_new]
     assert torch.isfinite(got).all()
     err = (got - ref).abs()
