@@ -802,7 +802,7 @@ template <int CLS, int GB>
 __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, int64_t a, int64_t b,
                                             const __half *__restrict__ sc, const __half *__restrict__ zz,
                                             int64_t meta0, const float *const *wr, int64_t wbase, int ng,
-                                            float (&acc)[GB][16], int lane, int wave) {
+                                            float (&acc)[GB][16], float (&zacc)[GB], int lane, int wave) {
   if (a >= b) return;
   constexpr int ROW = CLS == 0 ? 32 : (CLS == 1 ? 64 : (CLS == 2 ? 128 : 256));   // bytes per token
   constexpr int NL = CLS == 3 ? 2 : 1;                                            // 16-byte loads per lane
@@ -838,22 +838,42 @@ __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, i
 #pragma unroll
     for (int u = 0; u < kUnroll; ++u) {
       if (!in[u]) continue;
+      if (CLS == 3) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        float v;
-        if (CLS == 3) {
+        for (int i = 0; i < 16; ++i) {
           const uint4 r = raw[u][i >> 3];
           const uint32_t wd = ((i >> 1) & 3) == 0 ? r.x : (((i >> 1) & 3) == 1 ? r.y : (((i >> 1) & 3) == 2 ? r.z : r.w));
-          v = __half2float(__ushort_as_half((uint16_t)(wd >> (16 * (i & 1)))));
-        } else {
-          const uint4 r = raw[u][0];
-          const uint32_t wd = (i >> 2) == 0 ? r.x : ((i >> 2) == 1 ? r.y : ((i >> 2) == 2 ? r.z : r.w));
-          const uint32_t byte = wd >> (8 * (i & 3));
-          const uint32_t code = CLS == 0 ? ((byte >> shift) & 3u) : (CLS == 1 ? ((byte >> shift) & 15u) : (byte & 255u));
-          v = ((float)code - z[u]) * s[u];
-        }
+          const float v = __half2float(__ushort_as_half((uint16_t)(wd >> (16 * (i & 1)))));
 #pragma unroll
-        for (int g = 0; g < GB; ++g) acc[g][i] += wv[u][g] * v;
+          for (int g = 0; g < GB; ++g) acc[g][i] += wv[u][g] * v;
+        }
+      } else {
+        // sum_t w s (code - z) = sum_t (w s) code - sum_t (w s) z: the token's factor is folded into its
+        // weights once, a code costs its conversion (one byte of a dword whose field has been shifted
+        // down and masked for all four bytes at once) and one multiply-add per query head; the second
+        // sum is the same for all channels of a head and is carried in zacc.
+        float ws[GB];
+#pragma unroll
+        for (int g = 0; g < GB; ++g) {
+          ws[g] = wv[u][g] * s[u];
+          zacc[g] += ws[g] * z[u];
+        }
+        const uint4 r = raw[u][0];
+        const uint32_t dw[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t f = CLS == 0 ? ((dw[q] >> shift) & 0x03030303u)
+                                      : (CLS == 1 ? ((dw[q] >> shift) & 0x0F0F0F0Fu) : dw[q]);
+          const float c0 = (float)(f & 255u), c1 = (float)((f >> 8) & 255u), c2 = (float)((f >> 16) & 255u),
+                      c3 = (float)(f >> 24);
+#pragma unroll
+          for (int g = 0; g < GB; ++g) {
+            acc[g][4 * q + 0] += ws[g] * c0;
+            acc[g][4 * q + 1] += ws[g] * c1;
+            acc[g][4 * q + 2] += ws[g] * c2;
+            acc[g][4 * q + 3] += ws[g] * c3;
+          }
+        }
       }
     }
   }
@@ -907,23 +927,25 @@ v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
     const float *wr[GB];
 #pragma unroll
     for (int g = 0; g < GB; ++g) wr[g] = w + (int64_t)(hkv * G + (g < ng ? g0 + g : g0)) * w_sh;
-    float acc[GB][16];
+    float acc[GB][16], zacc[GB];   // zacc: this lane's sum of weight * scale * zero point per head
 #pragma unroll
-    for (int g = 0; g < GB; ++g)
+    for (int g = 0; g < GB; ++g) {
+      zacc[g] = 0.0f;
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[g][i] = 0.0f;
-    if (V2) v_class_sum<0, GB>(V2 + hkv * v2_sh, lo(N2), hi(N2), sc, zz, 0, wr, 0, ng, acc, lane, wave);
-    if (V4) v_class_sum<1, GB>(V4 + hkv * v4_sh, lo(N4), hi(N4), sc, zz, c1, wr, c1, ng, acc, lane, wave);
-    if (V8) v_class_sum<2, GB>(V8 + hkv * v8_sh, lo(N8), hi(N8), sc, zz, c2, wr, c2, ng, acc, lane, wave);
+    }
+    if (V2) v_class_sum<0, GB>(V2 + hkv * v2_sh, lo(N2), hi(N2), sc, zz, 0, wr, 0, ng, acc, zacc, lane, wave);
+    if (V4) v_class_sum<1, GB>(V4 + hkv * v4_sh, lo(N4), hi(N4), sc, zz, c1, wr, c1, ng, acc, zacc, lane, wave);
+    if (V8) v_class_sum<2, GB>(V8 + hkv * v8_sh, lo(N8), hi(N8), sc, zz, c2, wr, c2, ng, acc, zacc, lane, wave);
     if (N16 > 0)
       v_class_sum<3, GB>(reinterpret_cast<const uint8_t *>(V16 + hkv * v16_sh), lo(N16), hi(N16), sc, zz, 0, wr,
-                         max_T_v, ng, acc, lane, wave);
+                         max_T_v, ng, acc, zacc, lane, wave);
     // fold the eight token lanes of the wavefront (same li), then the wavefronts, in a fixed order
 #pragma unroll
     for (int g = 0; g < GB; ++g) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const float v = fold_token_lanes(acc[g][i]);
+        const float v = fold_token_lanes(acc[g][i] - zacc[g]);
         if (sub == 0) s_acc[wave][g][16 * li + i] = v;
       }
     }
