@@ -798,18 +798,51 @@ constexpr int kVWaves = 4;
 // j+64) those channels are one nibble of bytes 16*(li&3)..; in a 2-bit row (byte j = channels j,
 // j+32, j+64, j+96) one field of bytes 16*(li&1)..; an fp16 token is two 16-byte loads per lane.
 // wbase: column of class-local token 0 in the weight rows.
+// One quantized token of a lane (its 16 bytes of codes) for GB query heads.
+// sum_t w s (code - z) = sum_t (w s) code - sum_t (w s) z: the token's factor is folded into its
+// weights once, a code costs its conversion (one byte of a dword whose field has been shifted
+// down and masked for all four bytes at once) and one multiply-add per query head; the second
+// sum is the same for all channels of a head and is carried in zacc.
 template <int CLS, int GB>
-__device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, int64_t a, int64_t b,
-                                            const __half *__restrict__ sc, const __half *__restrict__ zz,
-                                            int64_t meta0, const float *const *wr, int64_t wbase, int ng,
-                                            float (&acc)[GB][16], float (&zacc)[GB], int lane, int wave) {
+__device__ __forceinline__ void v_token_quant(const uint4 r, float s, float z, const float (&wv)[GB], int shift,
+                                              float (&acc)[GB][16], float (&zacc)[GB]) {
+  float ws[GB];
+#pragma unroll
+  for (int g = 0; g < GB; ++g) {
+    ws[g] = wv[g] * s;
+    zacc[g] += ws[g] * z;
+  }
+  const uint32_t dw[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t f = CLS == 0 ? ((dw[q] >> shift) & 0x03030303u)
+                                : (CLS == 1 ? ((dw[q] >> shift) & 0x0F0F0F0Fu) : dw[q]);
+    const float c0 = (float)(f & 255u), c1 = (float)((f >> 8) & 255u), c2 = (float)((f >> 16) & 255u),
+                c3 = (float)(f >> 24);
+#pragma unroll
+    for (int g = 0; g < GB; ++g) {
+      acc[g][4 * q + 0] += ws[g] * c0;
+      acc[g][4 * q + 1] += ws[g] * c1;
+      acc[g][4 * q + 2] += ws[g] * c2;
+      acc[g][4 * q + 3] += ws[g] * c3;
+    }
+  }
+}
+
+// Tokens [a, b) one at a time per lane group (any alignment of the weight and scale rows): the
+// eight lane groups of the block's wavefronts take tokens 32 apart, four of them in flight.
+template <int CLS, int GB>
+__device__ __forceinline__ void v_class_range(const uint8_t *__restrict__ codes, int64_t a, int64_t b,
+                                              const __half *__restrict__ sc, const __half *__restrict__ zz,
+                                              int64_t meta0, const float *const *wr, int64_t wbase, int ng,
+                                              float (&acc)[GB][16], float (&zacc)[GB], int lane, int wave) {
   if (a >= b) return;
   constexpr int ROW = CLS == 0 ? 32 : (CLS == 1 ? 64 : (CLS == 2 ? 128 : 256));   // bytes per token
   constexpr int NL = CLS == 3 ? 2 : 1;                                            // 16-byte loads per lane
   const int sub = lane >> 3, li = lane & 7;
   const int off = CLS == 0 ? 16 * (li & 1) : (CLS == 1 ? 16 * (li & 3) : (CLS == 2 ? 16 * li : 32 * li));
   const int shift = CLS == 0 ? 2 * (li >> 1) : (CLS == 1 ? 4 * (li >> 2) : 0);    // field inside each byte
-  constexpr int kUnroll = CLS == 3 ? 2 : 4;
+  constexpr int kUnroll = (CLS == 3 || GB > 4) ? 2 : 4;   // tokens in flight per lane group
   constexpr int kStep = kVWaves * 8;               // tokens per block step
   for (int64_t t0 = a + wave * 8 + sub; t0 < b; t0 += (int64_t)kUnroll * kStep) {
     uint4 raw[kUnroll][NL];
@@ -848,34 +881,87 @@ __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, i
           for (int g = 0; g < GB; ++g) acc[g][i] += wv[u][g] * v;
         }
       } else {
-        // sum_t w s (code - z) = sum_t (w s) code - sum_t (w s) z: the token's factor is folded into its
-        // weights once, a code costs its conversion (one byte of a dword whose field has been shifted
-        // down and masked for all four bytes at once) and one multiply-add per query head; the second
-        // sum is the same for all channels of a head and is carried in zacc.
-        float ws[GB];
-#pragma unroll
-        for (int g = 0; g < GB; ++g) {
-          ws[g] = wv[u][g] * s[u];
-          zacc[g] += ws[g] * z[u];
-        }
-        const uint4 r = raw[u][0];
-        const uint32_t dw[4] = {r.x, r.y, r.z, r.w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const uint32_t f = CLS == 0 ? ((dw[q] >> shift) & 0x03030303u)
-                                      : (CLS == 1 ? ((dw[q] >> shift) & 0x0F0F0F0Fu) : dw[q]);
-          const float c0 = (float)(f & 255u), c1 = (float)((f >> 8) & 255u), c2 = (float)((f >> 16) & 255u),
-                      c3 = (float)(f >> 24);
-#pragma unroll
-          for (int g = 0; g < GB; ++g) {
-            acc[g][4 * q + 0] += ws[g] * c0;
-            acc[g][4 * q + 1] += ws[g] * c1;
-            acc[g][4 * q + 2] += ws[g] * c2;
-            acc[g][4 * q + 3] += ws[g] * c3;
-          }
-        }
+        v_token_quant<CLS, GB>(raw[u][0], s[u], z[u], wv[u], shift, acc, zacc);
       }
     }
+  }
+}
+
+// Adds tokens [a, b) (class-local) of class CLS, weighted for query heads g0 .. g0+GB-1, to
+// acc[g][i]: lane li (0..7) of a token always owns channels 16*li .. 16*li+15, whatever the class,
+// so one set of accumulators serves all four classes.  In a 4-bit row (byte j = channels j and
+// j+64) those channels are one nibble of bytes 16*(li&3)..; in a 2-bit row (byte j = channels j,
+// j+32, j+64, j+96) one field of bytes 16*(li&1)..; an fp16 token is two 16-byte loads per lane.
+// wbase: column of class-local token 0 in the weight rows.
+// A quantized class whose weight rows allow 16-byte loads (w16: row bases and strides 16-byte
+// aligned) is walked four consecutive tokens per lane group from the first token whose weight
+// column is a multiple of four: one 16-byte load per query head brings the four weights, one
+// 8-byte load the four scales and one the zero points (when those addresses are 8-byte aligned),
+// instead of 4 (GB + 2) scalar loads - the per-token scalars were most of the kernel's load
+// instructions.  What precedes and follows the aligned run goes token by token.  (GROUPED is the
+// launch's choice: it pays on long rows, 55 -> 43 us on a 128k layer with four query heads per KV
+// head, costs a microsecond at 32k, and with eight query heads the registers of the wider loads halve
+// the resident wavefronts.)
+template <int CLS, int GB, bool GROUPED>
+__device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, int64_t a, int64_t b,
+                                            const __half *__restrict__ sc, const __half *__restrict__ zz,
+                                            int64_t meta0, const float *const *wr, int64_t wbase, int ng,
+                                            float (&acc)[GB][16], float (&zacc)[GB], int lane, int wave, bool w16) {
+  if (a >= b) return;
+  if (CLS == 3 || !GROUPED) {
+    v_class_range<CLS, GB>(codes, a, b, sc, zz, meta0, wr, wbase, ng, acc, zacc, lane, wave);
+    return;
+  }
+  constexpr int ROW = CLS == 0 ? 32 : (CLS == 1 ? 64 : 128);
+  const int sub = lane >> 3, li = lane & 7;
+  const int off = CLS == 0 ? 16 * (li & 1) : (CLS == 1 ? 16 * (li & 3) : 16 * li);
+  const int shift = CLS == 0 ? 2 * (li >> 1) : (CLS == 1 ? 4 * (li >> 2) : 0);
+  // groups of four tokens whose weight column is a multiple of four; the first and the last group
+  // may stick out of [a, b): their tokens outside get weight 0 and are loaded one by one
+  const int64_t t_first = a - ((wbase + a) & 3);
+  const int64_t groups = (b - t_first + 3) >> 2;
+  const bool meta8 = (((uintptr_t)(sc + meta0 + t_first)) & 7) == 0 && (((uintptr_t)(zz + meta0 + t_first)) & 7) == 0;
+  for (int64_t gi = wave * 8 + sub; gi < groups; gi += kVWaves * 8) {
+    const int64_t t = t_first + 4 * gi;
+    const bool full = w16 && t >= a && t + 3 < b;   // (rows that do not allow 16-byte loads: every group one by one)
+    uint4 raw[4];
+    float s4[4], z4[4], wv[4][GB];
+    if (full) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4 *>(codes + (t + u) * ROW + off);
+#pragma unroll
+      for (int g = 0; g < GB; ++g) {
+        const float4 w4 = g < ng ? *reinterpret_cast<const float4 *>(wr[g] + wbase + t) : make_float4(0.f, 0.f, 0.f, 0.f);
+        wv[0][g] = w4.x; wv[1][g] = w4.y; wv[2][g] = w4.z; wv[3][g] = w4.w;
+      }
+      if (meta8) {
+        const uint2 sr = *reinterpret_cast<const uint2 *>(sc + meta0 + t), zr = *reinterpret_cast<const uint2 *>(zz + meta0 + t);
+        s4[0] = rdkv_h2f((uint16_t)sr.x); s4[1] = rdkv_h2f((uint16_t)(sr.x >> 16));
+        s4[2] = rdkv_h2f((uint16_t)sr.y); s4[3] = rdkv_h2f((uint16_t)(sr.y >> 16));
+        z4[0] = rdkv_h2f((uint16_t)zr.x); z4[1] = rdkv_h2f((uint16_t)(zr.x >> 16));
+        z4[2] = rdkv_h2f((uint16_t)zr.y); z4[3] = rdkv_h2f((uint16_t)(zr.y >> 16));
+      } else {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          s4[u] = __half2float(sc[meta0 + t + u]);
+          z4[u] = __half2float(zz[meta0 + t + u]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t tu = t + u;
+        const bool in = tu >= a && tu < b;
+        const int64_t tc = in ? tu : a;                  // a token that exists, weighted 0
+        raw[u] = *reinterpret_cast<const uint4 *>(codes + tc * ROW + off);
+        s4[u] = __half2float(sc[meta0 + tc]);
+        z4[u] = __half2float(zz[meta0 + tc]);
+#pragma unroll
+        for (int g = 0; g < GB; ++g) wv[u][g] = (in && g < ng) ? wr[g][wbase + tc] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v_token_quant<CLS, GB>(raw[u], s4[u], z4[u], wv[u], shift, acc, zacc);
   }
 }
 
@@ -893,7 +979,7 @@ __device__ __forceinline__ float fold_token_lanes(float v) {
   return __builtin_bit_cast(float, (unsigned)t[0]) + __builtin_bit_cast(float, (unsigned)t[1]);
 }
 
-template <int GB>
+template <int GB, bool GROUPED>
 __global__ void __launch_bounds__(64 * kVWaves)
 v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
                       const uint8_t *__restrict__ V2, int64_t v2_sh, const uint8_t *__restrict__ V4,
@@ -922,6 +1008,7 @@ v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
   auto hi = [&](int64_t n) { const int64_t per = (n + kVChunks - 1) / kVChunks, b = (chunk + 1) * per; return b < n ? b : n; };
 
   const int sub = lane >> 3, li = lane & 7;
+  const bool w16 = (((uintptr_t)w) & 15) == 0 && (w_sh & 3) == 0;   // weight rows allow 16-byte loads
   for (int g0 = 0; g0 < G; g0 += GB) {
     const int ng = G - g0 < GB ? G - g0 : GB;
     const float *wr[GB];
@@ -934,12 +1021,12 @@ v_weighted_sum_kernel(const float *__restrict__ w, int64_t w_sh, int G,
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[g][i] = 0.0f;
     }
-    if (V2) v_class_sum<0, GB>(V2 + hkv * v2_sh, lo(N2), hi(N2), sc, zz, 0, wr, 0, ng, acc, zacc, lane, wave);
-    if (V4) v_class_sum<1, GB>(V4 + hkv * v4_sh, lo(N4), hi(N4), sc, zz, c1, wr, c1, ng, acc, zacc, lane, wave);
-    if (V8) v_class_sum<2, GB>(V8 + hkv * v8_sh, lo(N8), hi(N8), sc, zz, c2, wr, c2, ng, acc, zacc, lane, wave);
+    if (V2) v_class_sum<0, GB, GROUPED>(V2 + hkv * v2_sh, lo(N2), hi(N2), sc, zz, 0, wr, 0, ng, acc, zacc, lane, wave, w16);
+    if (V4) v_class_sum<1, GB, GROUPED>(V4 + hkv * v4_sh, lo(N4), hi(N4), sc, zz, c1, wr, c1, ng, acc, zacc, lane, wave, w16);
+    if (V8) v_class_sum<2, GB, GROUPED>(V8 + hkv * v8_sh, lo(N8), hi(N8), sc, zz, c2, wr, c2, ng, acc, zacc, lane, wave, w16);
     if (N16 > 0)
-      v_class_sum<3, GB>(reinterpret_cast<const uint8_t *>(V16 + hkv * v16_sh), lo(N16), hi(N16), sc, zz, 0, wr,
-                         max_T_v, ng, acc, zacc, lane, wave);
+      v_class_sum<3, GB, GROUPED>(reinterpret_cast<const uint8_t *>(V16 + hkv * v16_sh), lo(N16), hi(N16), sc, zz, 0, wr,
+                         max_T_v, ng, acc, zacc, lane, wave, w16);
     // fold the eight token lanes of the wavefront (same li), then the wavefronts, in a fixed order
 #pragma unroll
     for (int g = 0; g < GB; ++g) {
@@ -1149,14 +1236,15 @@ RDKV_API int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, in
                    v8_stride_h % 16 == 0 && v16_stride_h % 8 == 0,
                "rdkv_v_weighted_sum: V segments must be 16-byte aligned");
   const int G = H_q / H_kv;
-#define RDKV_LAUNCH_V(GB)                                                                                      \
-  hipLaunchKernelGGL((v_weighted_sum_kernel<GB>), dim3(kVChunks, H_kv), dim3(64 * kVWaves), 0, s, w, w_stride_h, G, \
+#define RDKV_LAUNCH_V(GB, GROUPED)                                                                             \
+  hipLaunchKernelGGL((v_weighted_sum_kernel<GB, GROUPED>), dim3(kVChunks, H_kv), dim3(64 * kVWaves), 0, s, w, w_stride_h, G, \
                      V2, v2_stride_h, V4, v4_stride_h, V8, v8_stride_h, (const __half *)scale_f16,             \
                      (const __half *)zp_f16, vs_stride_h, seg_bounds_dev, N2, N4, N8, (const __half *)V16_f16, \
                      v16_stride_h, n_v16_dev, max_T_v, (float *)workspace, H_q)
-  if (G <= 2) RDKV_LAUNCH_V(2);
-  else if (G <= 4 || G > 8) RDKV_LAUNCH_V(4);
-  else RDKV_LAUNCH_V(8);
+  const bool long_rows = (int64_t)N2 + N4 + N8 >= 65536;   // four consecutive tokens per lane group pay from here on
+  if (G <= 2) { if (long_rows) RDKV_LAUNCH_V(2, true); else RDKV_LAUNCH_V(2, false); }
+  else if (G <= 4 || G > 8) { if (long_rows) RDKV_LAUNCH_V(4, true); else RDKV_LAUNCH_V(4, false); }
+  else RDKV_LAUNCH_V(8, false);
 #undef RDKV_LAUNCH_V
   hipLaunchKernelGGL(v_reduce_kernel, dim3(H_q), dim3(8 * kD), 0, s, (const float *)workspace, H_q, out, out_stride_h);
   RDKV_CHECK_LAUNCH("rdkv_v_weighted_sum");

@@ -305,3 +305,47 @@ def test_k_scores_random_layouts(H_kv, G, T, widths, kw, q_dtype):
     in_place.K_2bit, in_place.K_4bit, in_place.K_8bit = widened(layer.K_2bit), widened(layer.K_4bit), widened(layer.K_8bit)
     other = t2n(kk.k_mixed_qk_dot(q.to(DEV), in_place, T)).astype(np.float64)
     assert np.abs(other - exp).max() <= 4e-5 * scale
+
+
+@pytest.mark.parametrize("H_kv,G,counts,w_offset", [
+    (2, 4, (30001, 25003, 20000), 0),      # long rows: four consecutive tokens per lane group, classes off alignment
+    (2, 2, (70000, 0, 3), 0),              # two query heads per KV head, 2-bit only + a 3-token class
+    (1, 4, (1, 66000, 1), 1),              # weight rows one float off a 16-byte boundary: every group one by one
+    (2, 8, (40000, 30000, 10000), 0),      # eight query heads: the one-token-at-a-time form
+    (3, 4, (500, 700, 300), 0),            # short rows
+])
+def test_v_weighted_sum_random_layers(H_kv, G, counts, w_offset):
+    """The V weighted sum on hand-built shared-layout layers (random codes, per-token scale and zero
+    point, random weights) against float64 arithmetic on the same bytes, on both sides of the row
+    length from which the launch reads four consecutive tokens per lane group."""
+    N2, N4, N8 = counts
+    T = N2 + N4 + N8
+    H_q = H_kv * G
+    rng = np.random.default_rng(T + H_q)
+    V2 = torch.from_numpy(rng.integers(0, 256, size=(H_kv, N2, 32), dtype=np.uint8)).to(DEV)
+    V4 = torch.from_numpy(rng.integers(0, 256, size=(H_kv, N4, 64), dtype=np.uint8)).to(DEV)
+    V8 = torch.from_numpy(rng.integers(0, 256, size=(H_kv, N8, 128), dtype=np.uint8)).to(DEV)
+    scale = rng.uniform(0.01, 0.1, size=(H_kv, T, 1)).astype(np.float16)
+    zp = np.concatenate([rng.integers(0, 4, size=(H_kv, N2, 1)), rng.integers(0, 16, size=(H_kv, N4, 1)),
+                         rng.integers(0, 256, size=(H_kv, N8, 1))], axis=1).astype(np.float16)
+    w = rng.random((H_q, T)).astype(np.float32)
+    w /= w.sum(axis=1, keepdims=True)
+    wbuf = torch.zeros(H_q, T + 8 + w_offset, device=DEV)
+    wd = wbuf[:, w_offset:w_offset + T]
+    wd.copy_(torch.from_numpy(w))
+    out = torch.full((H_q, 128 + 3), 9.0, device=DEV)
+    vk.v_dequant_weighted_sum_unified_into(wd, V2, V4, V8, torch.from_numpy(scale).to(DEV), torch.from_numpy(zp).to(DEV),
+                                           counts, out[:, :128])
+    # float64 reference: 2-bit byte j holds channels j, j+32, j+64, j+96; 4-bit byte j channels j and j+64
+    exp = np.zeros((H_q, 128))
+    for h in range(H_kv):
+        b2, b4, b8 = t2n(V2[h]).astype(np.int64), t2n(V4[h]).astype(np.int64), t2n(V8[h]).astype(np.float64)
+        codes = np.concatenate([
+            np.concatenate([(b2 >> (2 * f)) & 3 for f in range(4)], axis=1).astype(np.float64),
+            np.concatenate([b4 & 15, b4 >> 4], axis=1).astype(np.float64), b8], axis=0)      # [T, 128]
+        deq = (codes - zp[h].astype(np.float64)) * scale[h].astype(np.float64)
+        for g in range(G):
+            exp[h * G + g] = w[h * G + g].astype(np.float64) @ deq
+    got = t2n(out[:, :128]).astype(np.float64)
+    assert np.abs(got - exp).max() <= 2e-5 * max(1.0, np.abs(exp).max()), f"max error {np.abs(got - exp).max():.3e}"
+    assert float((out[:, 128:] - 9.0).abs().max()) == 0.0
