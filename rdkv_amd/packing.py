@@ -13,6 +13,8 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
+import threading
+
 import torch
 from torch import Tensor
 
@@ -616,6 +618,21 @@ def _pad_and_stack_per_head_layers(
 
 _PLAN_INT_DTYPES = (torch.uint8, torch.int16, torch.int32, torch.int64)
 
+_pinned_ints: dict = {}
+
+
+def _read_ints(t: Tensor, n: int) -> list:
+    """The first ``n`` int32 of a device tensor as a Python list, through a pinned host buffer
+    that is kept (a pageable copy allocates and stages on every call)."""
+    key = (t.device.index, max(1024, 1 << (n - 1).bit_length()), threading.get_ident())   # one buffer per host thread
+    buf = _pinned_ints.get(key)
+    if buf is None:
+        buf = _pinned_ints[key] = torch.empty(key[1], dtype=torch.int32, pin_memory=True)
+    buf[:n].copy_(t[:n], non_blocking=True)
+    torch.cuda.current_stream(t.device).synchronize()
+    return buf[:n].tolist()
+
+
 def _plan_layers(v_bits: Tensor, k_bits: Tensor, dev):
     """Token order, quantized-token ranks and class sizes of ``[N, T]`` / ``[N, D]`` allocations
     (N = heads of one layer, or of several layers stacked) in one launch pair and one host read.
@@ -639,7 +656,7 @@ def _plan_layers(v_bits: Tensor, k_bits: Tensor, dev):
                                         kb.element_size(), kb.stride(0), N, T, int(kb.shape[1]), order.data_ptr(),
                                         order.stride(0), rank3.data_ptr(), rank3.stride(0), plan.data_ptr(),
                                         _lib.stream_of(dev)))
-    plan_h = plan[:12 * N].cpu().tolist()                       # the one synchronization
+    plan_h = _read_ints(plan, 12 * N)                           # the one synchronization
     counts_h = [plan_h[4 * h:4 * h + 4] for h in range(N)]
     info_h = [plan_h[4 * N + 8 * h:4 * N + 8 * h + 8] for h in range(N)]
     assert all(row[1] == 0 for row in info_h), "v_bits must be in {0,2,4,8,16}"
