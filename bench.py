@@ -7,7 +7,7 @@ for one query per layer and writes out [L*H_q,128] + lse.  Inputs are synthetic,
 resident in HBM before the timed region.  Default workload: configuration 1 (Llama-3.1-8B
 shapes, 32 layers, 32k context, per-head Dirichlet bit allocation).
 
-Prints ONE JSON line (see README / DESIGN for the fields): the headline on configuration 1 with
+Prints ONE JSON line: the headline on configuration 1 with
 `roofline` and `cpu_baseline`, and beside it compact figures of the other configurations
 (`configs`), the one-layer-per-call form (`sequential`), the reference-layout entry points
 (`padded`), the prefill packer (`pack`, `select`) and the whole-model decode loops (`decode_loop`).
