@@ -223,6 +223,10 @@ def compact_config(index, args, torch, dev):
     torch.cuda.empty_cache()
     if index == 4:
         res["pack_one_sequence"] = pack_sequence_section(cfg, torch, dev)
+    if index in (2, 3):
+        # the long-context configurations through the reference-layout entry points as well
+        pad = padded_section(cfg, torch, dev, layers=2, steps=10)
+        res["padded_us_per_layer"] = {k: v["us_per_layer"] for k, v in pad.items() if isinstance(v, dict)}
     return res
 
 
