@@ -916,40 +916,57 @@ __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, i
   const int sub = lane >> 3, li = lane & 7;
   const int off = CLS == 0 ? 16 * (li & 1) : (CLS == 1 ? 16 * (li & 3) : 16 * li);
   const int shift = CLS == 0 ? 2 * (li >> 1) : (CLS == 1 ? 4 * (li >> 2) : 0);
-  // groups of four tokens whose weight column is a multiple of four; the first and the last group
-  // may stick out of [a, b): their tokens outside get weight 0 and are loaded one by one
-  const int64_t t_first = a - ((wbase + a) & 3);
-  const int64_t groups = (b - t_first + 3) >> 2;
-  const bool meta8 = (((uintptr_t)(sc + meta0 + t_first)) & 7) == 0 && (((uintptr_t)(zz + meta0 + t_first)) & 7) == 0;
+  // groups of TOK tokens whose weight column is a multiple of TOK (four, or two with eight query
+  // heads: the wider loads must not cost a resident wavefront); the first and the last group may
+  // stick out of [a, b): their tokens outside get weight 0 and are loaded one by one
+  constexpr int TOK = GB > 4 ? 2 : 4;
+  const int64_t t_first = a - ((wbase + a) & (TOK - 1));
+  const int64_t groups = (b - t_first + TOK - 1) / TOK;
+  const bool meta_vec = (((uintptr_t)(sc + meta0 + t_first)) & (2 * TOK - 1)) == 0 &&
+                        (((uintptr_t)(zz + meta0 + t_first)) & (2 * TOK - 1)) == 0;
   for (int64_t gi = wave * 8 + sub; gi < groups; gi += kVWaves * 8) {
-    const int64_t t = t_first + 4 * gi;
-    const bool full = w16 && t >= a && t + 3 < b;   // (rows that do not allow 16-byte loads: every group one by one)
-    uint4 raw[4];
-    float s4[4], z4[4], wv[4][GB];
+    const int64_t t = t_first + TOK * gi;
+    const bool full = w16 && t >= a && t + TOK - 1 < b;   // (rows that do not allow vector loads: every group one by one)
+    uint4 raw[TOK];
+    float s4[TOK], z4[TOK], wv[TOK][GB];
     if (full) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) raw[u] = *reinterpret_cast<const uint4 *>(codes + (t + u) * ROW + off);
+      for (int u = 0; u < TOK; ++u) raw[u] = *reinterpret_cast<const uint4 *>(codes + (t + u) * ROW + off);
 #pragma unroll
       for (int g = 0; g < GB; ++g) {
-        const float4 w4 = g < ng ? *reinterpret_cast<const float4 *>(wr[g] + wbase + t) : make_float4(0.f, 0.f, 0.f, 0.f);
-        wv[0][g] = w4.x; wv[1][g] = w4.y; wv[2][g] = w4.z; wv[3][g] = w4.w;
+        if (TOK == 4) {
+          const float4 w4 = g < ng ? *reinterpret_cast<const float4 *>(wr[g] + wbase + t) : make_float4(0.f, 0.f, 0.f, 0.f);
+          wv[0][g] = w4.x; wv[1][g] = w4.y; wv[TOK - 2][g] = w4.z; wv[TOK - 1][g] = w4.w;
+        } else {
+          const float2 w2 = g < ng ? *reinterpret_cast<const float2 *>(wr[g] + wbase + t) : make_float2(0.f, 0.f);
+          wv[0][g] = w2.x; wv[1][g] = w2.y;
+        }
       }
-      if (meta8) {
-        const uint2 sr = *reinterpret_cast<const uint2 *>(sc + meta0 + t), zr = *reinterpret_cast<const uint2 *>(zz + meta0 + t);
-        s4[0] = rdkv_h2f((uint16_t)sr.x); s4[1] = rdkv_h2f((uint16_t)(sr.x >> 16));
-        s4[2] = rdkv_h2f((uint16_t)sr.y); s4[3] = rdkv_h2f((uint16_t)(sr.y >> 16));
-        z4[0] = rdkv_h2f((uint16_t)zr.x); z4[1] = rdkv_h2f((uint16_t)(zr.x >> 16));
-        z4[2] = rdkv_h2f((uint16_t)zr.y); z4[3] = rdkv_h2f((uint16_t)(zr.y >> 16));
+      if (meta_vec) {
+        uint32_t sr[2], zr[2];
+        if (TOK == 4) {
+          const uint2 a2 = *reinterpret_cast<const uint2 *>(sc + meta0 + t), b2 = *reinterpret_cast<const uint2 *>(zz + meta0 + t);
+          sr[0] = a2.x; sr[1] = a2.y; zr[0] = b2.x; zr[1] = b2.y;
+        } else {
+          sr[0] = *reinterpret_cast<const uint32_t *>(sc + meta0 + t);
+          zr[0] = *reinterpret_cast<const uint32_t *>(zz + meta0 + t);
+          sr[1] = zr[1] = 0;
+        }
+#pragma unroll
+        for (int u = 0; u < TOK; ++u) {
+          s4[u] = rdkv_h2f((uint16_t)(sr[u >> 1] >> (16 * (u & 1))));
+          z4[u] = rdkv_h2f((uint16_t)(zr[u >> 1] >> (16 * (u & 1))));
+        }
       } else {
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < TOK; ++u) {
           s4[u] = __half2float(sc[meta0 + t + u]);
           z4[u] = __half2float(zz[meta0 + t + u]);
         }
       }
     } else {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < TOK; ++u) {
         const int64_t tu = t + u;
         const bool in = tu >= a && tu < b;
         const int64_t tc = in ? tu : a;                  // a token that exists, weighted 0
@@ -961,7 +978,7 @@ __device__ __forceinline__ void v_class_sum(const uint8_t *__restrict__ codes, i
       }
     }
 #pragma unroll
-    for (int u = 0; u < 4; ++u) v_token_quant<CLS, GB>(raw[u], s4[u], z4[u], wv[u], shift, acc, zacc);
+    for (int u = 0; u < TOK; ++u) v_token_quant<CLS, GB>(raw[u], s4[u], z4[u], wv[u], shift, acc, zacc);
   }
 }
 
@@ -1244,7 +1261,7 @@ RDKV_API int rdkv_v_weighted_sum(const float *w, int64_t w_stride_h, int H_q, in
   const bool long_rows = (int64_t)N2 + N4 + N8 >= 65536;   // four consecutive tokens per lane group pay from here on
   if (G <= 2) { if (long_rows) RDKV_LAUNCH_V(2, true); else RDKV_LAUNCH_V(2, false); }
   else if (G <= 4 || G > 8) { if (long_rows) RDKV_LAUNCH_V(4, true); else RDKV_LAUNCH_V(4, false); }
-  else RDKV_LAUNCH_V(8, false);
+  else RDKV_LAUNCH_V(8, false);   // (two-token groups with eight heads: 68 against 62 us on a 128k layer)
 #undef RDKV_LAUNCH_V
   hipLaunchKernelGGL(v_reduce_kernel, dim3(H_q), dim3(8 * kD), 0, s, (const float *)workspace, H_q, out, out_stride_h);
   RDKV_CHECK_LAUNCH("rdkv_v_weighted_sum");
