@@ -349,3 +349,35 @@ def test_v_weighted_sum_random_layers(H_kv, G, counts, w_offset):
     got = t2n(out[:, :128]).astype(np.float64)
     assert np.abs(got - exp).max() <= 2e-5 * max(1.0, np.abs(exp).max()), f"max error {np.abs(got - exp).max():.3e}"
     assert float((out[:, 128:] - 9.0).abs().max()) == 0.0
+
+
+def test_entry_points_reject_bad_arguments():
+    """Argument checks of the C entry points behind this file's kernels: every call returns the
+    invalid-argument status (an AssertionError through ``_lib.check``) before anything is launched."""
+    from rdkv_amd import _lib
+    lib = _lib.load()
+    st = _lib.stream_of(torch.device(DEV))
+    buf = torch.zeros(4096, device=DEV)
+    p = buf.data_ptr()
+    with pytest.raises(AssertionError):          # query heads not a multiple of KV heads
+        _lib.check(lib.rdkv_k_qk_dot(p, 0, 128, 5, 2, p, 0, 4, None, 0, 0, None, 0, 0, p, p, 16, p, 0, 16, 0, 0, 8,
+                                     p, 64, st))
+    with pytest.raises(AssertionError):          # more KV heads than the launch grid has rows
+        _lib.check(lib.rdkv_k_qk_dot(p, 0, 128, 70000, 70000, p, 0, 4, None, 0, 0, None, 0, 0, p, p, 16, p, 0, 16, 0,
+                                     0, 8, p, 64, st))
+    with pytest.raises(AssertionError):          # a 2-bit segment that is not whole bytes
+        _lib.check(lib.rdkv_k_qk_dot(p, 0, 128, 4, 1, p, 0, 4, None, 0, 0, None, 0, 0, p, p, 16, p, 0, 6, 0, 0, 8,
+                                     p, 64, st))
+    with pytest.raises(AssertionError):          # empty softmax rows
+        _lib.check(lib.rdkv_softmax_rows_ws(p, 64, None, 0, 0, None, 0, 0, p, 64, None, 0, 4, None, 0, st))
+    with pytest.raises(AssertionError):          # an old zone without its output
+        _lib.check(lib.rdkv_softmax_rows_ws(p, 64, None, 0, 8, None, 0, 0, None, 64, None, 0, 4, None, 0, st))
+    assert lib.rdkv_softmax_rows_workspace_bytes(32) == 32 * 32 * 2 * 4 and lib.rdkv_softmax_rows_workspace_bytes(-1) == 0
+    # a workspace that is too small is not an error: the call keeps to one workgroup per row
+    rows = torch.randn(2, 70000, device=DEV)
+    ref = torch.softmax(rows, dim=-1)
+    small = torch.empty(8, dtype=torch.uint8, device=DEV)
+    _lib.check(lib.rdkv_softmax_rows_ws(rows.data_ptr(), rows.stride(0), None, 0, 70000, None, 0, 0, rows.data_ptr(),
+                                        rows.stride(0), None, 0, 2, small.data_ptr(), small.numel(), st))
+    assert float((rows - ref).abs().max()) < 1e-6
+    assert float(buf.abs().max()) == 0.0
