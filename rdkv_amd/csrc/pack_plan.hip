@@ -100,10 +100,14 @@ plan_scatter_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_strid
       acc[kTokClasses + k] += c < chunk ? v : 0;
     }
   }
+  // (a wavefront none of whose threads had a chunk has nothing to add up)
+  const bool wave_has_chunks = wave * 64 < nchunks;
 #pragma unroll
   for (int k = 0; k < 2 * kTokClasses; ++k) {
+    if (wave_has_chunks) {
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) acc[k] += __shfl_xor(acc[k], off, 64);
+      for (int off = 32; off > 0; off >>= 1) acc[k] += __shfl_xor(acc[k], off, 64);
+    }
     if (lane == 0) wsum[wave][k] = acc[k];
   }
   const int t = chunk * kPlanThreads + tid;

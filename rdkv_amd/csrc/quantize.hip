@@ -233,6 +233,182 @@ pack_v_layer_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stri
   }
 }
 
+// D == 128 with 16-byte aligned rows and 8-byte aligned outputs.  A workgroup takes 64 rows of
+// ONE class (the grid is the sum of the classes' block counts), so everything that depends on
+// the class is a compile-time constant of the instantiation it branches to.  Sixteen lanes per
+// row, lane l holding channels 8l .. 8l+7 (one 16-byte load); a wavefront takes sixteen rows,
+// four per instruction.  Nothing between the loads is conditional: every lane first fetches the
+// source indices of its four rows, then requests the four rows, and only then looks at the first
+// - two dependent round trips per wavefront (padding rows read row 0 and discard it).
+// The quantizer's parameters (three correctly rounded divisions) are computed once for the four
+// rows: lane l of a row takes row l & 3's extremes and the results go back by a broadcast inside
+// each group of four lanes.  Codes leave the converter as bytes (v_cvt_pk_u8_f32), so a lane's
+// eight codes are two dwords; the lanes that share an output byte (channels i, i+32, i+64, i+96
+// of a 2-bit byte, i and i+64 of a 4-bit byte) shift their dwords to the field's position and
+// OR them together with lane rotations of 4 and 8 inside the row's sixteen lanes, and the first
+// 4 / 8 / 16 lanes store eight bytes each.
+template <int CTRL>
+__device__ __forceinline__ uint32_t rdkv_dpp_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+// lane q of every group of four lanes, broadcast to the group
+template <int Q>
+__device__ __forceinline__ float rdkv_quad_bcast(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), Q * 0x55, 0xf, 0xf, true));
+}
+
+// CLS 0 / 1 / 2: 2- / 4- / 8-bit rows; 3: fp16 rows.  `first` = the workgroup's first row within
+// the class, `n_own` the head's own rows of the class, `n_max` the widest head's (rows between
+// the two are zero), `r0` = what precedes the class in the head's sorted order.
+template <int CLS>
+__device__ __forceinline__ void
+pack_v_rows_d128(const __half *__restrict__ Vh, int64_t stride_t, const int32_t *__restrict__ ord, int first,
+                 int n_own, int n_max, int r0, uint8_t *__restrict__ out_rows, __half *__restrict__ vsh,
+                 __half *__restrict__ vzh) {
+  constexpr int kSteps = RDKV_PACK_V_ROWS_PER_WAVE / 4;
+  constexpr int kRowBytes = CLS == 0 ? 32 : CLS == 1 ? 64 : CLS == 2 ? 128 : 256;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane >> 4, l = lane & 15;
+  const int j0 = first + wave * RDKV_PACK_V_ROWS_PER_WAVE + sub;      // this lane's row of step 0
+  int src[kSteps];
+  uint32_t valid[kSteps];      // all ones for a row the head owns
+  // (masked with AND, not selected: a select invites the compiler to branch around the load,
+  // which puts a full wait between that load and its neighbours)
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) {
+    valid[s] = j0 + 4 * s < n_own ? 0xffffffffu : 0u;
+    src[s] = ord[(r0 + j0 + 4 * s) & (int)valid[s]];
+  }
+  uint4 raw[kSteps];
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s)
+    raw[s] = *reinterpret_cast<const uint4 *>(Vh + (int64_t)(src[s] & (int)valid[s]) * stride_t + 8 * l);
+  __builtin_amdgcn_sched_barrier(0);   // every request is out before the first row is touched
+  if (CLS == 3) {
+#pragma unroll
+    for (int s = 0; s < kSteps; ++s) {
+      const int j = j0 + 4 * s;
+      if (j < n_max)
+        reinterpret_cast<uint4 *>(out_rows + (int64_t)j * kRowBytes)[l] =
+            make_uint4(raw[s].x & valid[s], raw[s].y & valid[s], raw[s].z & valid[s], raw[s].w & valid[s]);
+    }
+    return;
+  }
+  constexpr float qmax = CLS == 0 ? 3.0f : CLS == 1 ? 15.0f : 255.0f;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  // fp16 min / max are exact, so a row's extremes can be taken before widening
+  float mn[kSteps], mx[kSteps];
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) {
+    const half2_t a = __builtin_bit_cast(half2_t, raw[s].x), b = __builtin_bit_cast(half2_t, raw[s].y),
+                  c = __builtin_bit_cast(half2_t, raw[s].z), d = __builtin_bit_cast(half2_t, raw[s].w);
+    const half2_t mn2 = __builtin_elementwise_min(__builtin_elementwise_min(a, b), __builtin_elementwise_min(c, d));
+    const half2_t mx2 = __builtin_elementwise_max(__builtin_elementwise_max(a, b), __builtin_elementwise_max(c, d));
+    mn[s] = rdkv_row16_min(fminf((float)mn2.x, (float)mn2.y));
+    mx[s] = rdkv_row16_max(fmaxf((float)mx2.x, (float)mx2.y));
+  }
+  static_assert(kSteps == 4, "one row of the wavefront's four per lane of a group of four");
+  const int mine = l & 3;
+  const float mn_sel = mine == 0 ? mn[0] : mine == 1 ? mn[1] : mine == 2 ? mn[2] : mn[3];
+  const float mx_sel = mine == 0 ? mx[0] : mine == 1 ? mx[1] : mine == 2 ? mx[2] : mx[3];
+  const RdkvQParams mine_qp = rdkv_qparams(mn_sel, mx_sel, qmax);
+  RdkvQParams qps[kSteps];
+  qps[0] = {rdkv_quad_bcast<0>(mine_qp.scale), rdkv_quad_bcast<0>(mine_qp.zp), rdkv_quad_bcast<0>(mine_qp.inv)};
+  qps[1] = {rdkv_quad_bcast<1>(mine_qp.scale), rdkv_quad_bcast<1>(mine_qp.zp), rdkv_quad_bcast<1>(mine_qp.inv)};
+  qps[2] = {rdkv_quad_bcast<2>(mine_qp.scale), rdkv_quad_bcast<2>(mine_qp.zp), rdkv_quad_bcast<2>(mine_qp.inv)};
+  qps[3] = {rdkv_quad_bcast<3>(mine_qp.scale), rdkv_quad_bcast<3>(mine_qp.zp), rdkv_quad_bcast<3>(mine_qp.inv)};
+#pragma unroll
+  for (int s = 0; s < kSteps; ++s) {
+    const int j = j0 + 4 * s;
+    if (j >= n_max) continue;
+    uint32_t w0 = 0u, w1 = 0u;
+    if (valid[s]) {
+      const RdkvQParams qp = qps[s];
+      if (l == 0) {
+        vsh[r0 + j] = __float2half_rn(qp.scale);
+        vzh[r0 + j] = __float2half_rn(qp.zp);
+      }
+      const uint32_t rw[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
+      float x[8], t[8], q[8];
+      float dmin = 1.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const half2_t hv = __builtin_bit_cast(half2_t, rw[e >> 1]);
+        x[e] = (float)((e & 1) ? hv.y : hv.x);
+        t[e] = fmaf(x[e], qp.inv, qp.zp);
+        q[e] = rintf(__builtin_amdgcn_fmed3f(t[e], 0.0f, qmax));
+        dmin = fminf(dmin, fabsf(fabsf(t[e] - q[e]) - 0.5f));
+      }
+      if (dmin < 2e-4f) {              // some value sits at a rounding boundary: the exact quotient decides
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (fabsf(fabsf(t[e] - q[e]) - 0.5f) < 2e-4f) q[e] = (float)rdkv_qcode_exact(x[e], qp, qmax);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        w0 = __builtin_amdgcn_cvt_pk_u8_f32(q[e], e, w0);
+        w1 = __builtin_amdgcn_cvt_pk_u8_f32(q[4 + e], e, w1);
+      }
+    }
+    // field position of this lane's codes inside the output bytes, then the lanes that share bytes
+    // (a row's sixteen lanes are all in or all out of every branch above)
+    if (CLS == 0) {
+      w0 <<= 2 * (l >> 2);
+      w1 <<= 2 * (l >> 2);
+      w0 |= rdkv_dpp_u32<0x124>(w0);
+      w1 |= rdkv_dpp_u32<0x124>(w1);
+    }
+    if (CLS == 1) {
+      w0 <<= 4 * (l >> 3);
+      w1 <<= 4 * (l >> 3);
+    }
+    if (CLS <= 1) {
+      w0 |= rdkv_dpp_u32<0x128>(w0);
+      w1 |= rdkv_dpp_u32<0x128>(w1);
+    }
+    if (l < kRowBytes / 8) reinterpret_cast<uint2 *>(out_rows + (int64_t)j * kRowBytes)[l] = make_uint2(w0, w1);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+pack_v_layer_d128_kernel(const __half *__restrict__ V, int64_t stride_h, int64_t stride_t,
+                         const int32_t *__restrict__ order, int64_t order_stride_h,
+                         const int32_t *__restrict__ counts, int mN2, int mN4, int mN8, int max_n16,
+                         int64_t max_tv, uint8_t *__restrict__ V2, uint8_t *__restrict__ V4,
+                         uint8_t *__restrict__ V8, __half *__restrict__ vs, __half *__restrict__ vz,
+                         __half *__restrict__ V16, uint32_t *__restrict__ mm_init) {
+  constexpr int D = 128;
+  constexpr int kRows = 4 * RDKV_PACK_V_ROWS_PER_WAVE;          // rows of a workgroup
+  const int h = blockIdx.y;
+  const int n2 = counts[4 * h], n4 = counts[4 * h + 1], n8 = counts[4 * h + 2], n16 = counts[4 * h + 3];
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Vh = V + (int64_t)h * stride_h;
+  __half *vsh = vs + (int64_t)h * max_tv, *vzh = vz + (int64_t)h * max_tv;
+  // Two small jobs ride along instead of being launches of their own (see pack_v_layer_kernel).
+  for (int64_t i = (int64_t)n2 + n4 + n8 + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < max_tv;
+       i += (int64_t)gridDim.x * blockDim.x) {
+    vsh[i] = __float2half_rn(0.0f);
+    vzh[i] = __float2half_rn(0.0f);
+  }
+  if (mm_init && blockIdx.x == 0)
+    for (int i = threadIdx.x; i < 2 * D; i += blockDim.x)
+      mm_init[(int64_t)h * 2 * D + i] = rdkv_float_to_ordered(i >= D ? -INFINITY : INFINITY);
+  // block -> (class, first row): the classes' blocks follow each other
+  const int b2 = (mN2 + kRows - 1) / kRows, b4 = (mN4 + kRows - 1) / kRows, b8 = (mN8 + kRows - 1) / kRows;
+  int b = blockIdx.x;
+  if (b < b2) {
+    pack_v_rows_d128<0>(Vh, stride_t, ord, b * kRows, n2, mN2, 0, V2 + (int64_t)h * mN2 * 32, vsh, vzh);
+  } else if ((b -= b2) < b4) {
+    pack_v_rows_d128<1>(Vh, stride_t, ord, b * kRows, n4, mN4, n2, V4 + (int64_t)h * mN4 * 64, vsh, vzh);
+  } else if ((b -= b4) < b8) {
+    pack_v_rows_d128<2>(Vh, stride_t, ord, b * kRows, n8, mN8, n2 + n4, V8 + (int64_t)h * mN8 * 128, vsh, vzh);
+  } else {
+    b -= b8;
+    pack_v_rows_d128<3>(Vh, stride_t, ord, b * kRows, n16, max_n16, n2 + n4 + n8,
+                        reinterpret_cast<uint8_t *>(V16 + (int64_t)h * max_n16 * D), vsh, vzh);
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Per-column (per-channel over T) min/max.
 // ---------------------------------------------------------------------------
@@ -430,10 +606,14 @@ k_minmax_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t st
 }
 
 // D == 128, rows 16-byte aligned: sixteen lanes read one row as 16-byte pieces (eight channels
-// each), four rows per wavefront step, four steps in flight; min/max stay packed fp16 (exact)
-// until the end.
-#define RDKV_LAYER_MINMAX_ROWS_D128 512
-__global__ void __launch_bounds__(256)
+// each), four rows per wavefront instruction.  A workgroup owns 256 rows: every lane first fetches
+// the source indices of its sixteen rows, then requests all sixteen pieces before it reduces the
+// first - two dependent round trips per workgroup, whatever the row count (a loop that fetched
+// index and piece step by step left the launch waiting on memory 87 % of its time).  min/max stay
+// packed fp16 (exact) until the end.
+#define RDKV_LAYER_MINMAX_WAVES_D128 8
+#define RDKV_LAYER_MINMAX_ROWS_D128 (64 * RDKV_LAYER_MINMAX_WAVES_D128)
+__global__ void __launch_bounds__(64 * RDKV_LAYER_MINMAX_WAVES_D128)
 k_minmax_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
                            const int32_t *__restrict__ order, int64_t order_stride_h,
                            const int32_t *__restrict__ counts, uint32_t *__restrict__ mm) {
@@ -449,29 +629,29 @@ k_minmax_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64
   const half2_t pinf = {(_Float16)INFINITY, (_Float16)INFINITY}, ninf = {(_Float16)-INFINITY, (_Float16)-INFINITY};
   half2_t mn[4] = {pinf, pinf, pinf, pinf}, mx[4] = {ninf, ninf, ninf, ninf};
   union Piece { uint4 u; half2_t h[4]; };
-  // a block step covers 16 rows (4 waves x 4 rows); 4 steps are loaded before any is reduced
-  for (int base = t0 + wave * 4 + sub; base < t1; base += 64) {
-    Piece v[4];
-    bool in[4];
+  constexpr int kWaves = RDKV_LAYER_MINMAX_WAVES_D128;
+  constexpr int kRowsPerLane = 16;              // a workgroup instruction covers 4 * kWaves rows
+  // row u of this lane; rows past the end repeat the workgroup's first row (min/max are idempotent)
+  int src[kRowsPerLane];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = base + 16 * u;
-      in[u] = t < t1;
-      if (in[u]) v[u].u = *reinterpret_cast<const uint4 *>(Kh + (int64_t)ord[t] * stride_t + 8 * l);
-    }
+  for (int u = 0; u < kRowsPerLane; ++u) {
+    const int t = t0 + wave * 4 + sub + 4 * kWaves * u;
+    src[u] = ord[t < t1 ? t : t0];
+  }
+  Piece v[kRowsPerLane];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      if (in[u]) {
+  for (int u = 0; u < kRowsPerLane; ++u)
+    v[u].u = *reinterpret_cast<const uint4 *>(Kh + (int64_t)src[u] * stride_t + 8 * l);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          mn[k] = __builtin_elementwise_min(mn[k], v[u].h[k]);
-          mx[k] = __builtin_elementwise_max(mx[k], v[u].h[k]);
-        }
-      }
+  for (int u = 0; u < kRowsPerLane; ++u) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      mn[k] = __builtin_elementwise_min(mn[k], v[u].h[k]);
+      mx[k] = __builtin_elementwise_max(mx[k], v[u].h[k]);
     }
   }
-  __shared__ float s_mn[4][128];
-  __shared__ float s_mx[4][128];
+  __shared__ float s_mn[kWaves][128];
+  __shared__ float s_mx[kWaves][128];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     float a0 = (float)mn[k].x, a1 = (float)mn[k].y, b0 = (float)mx[k].x, b1 = (float)mx[k].y;
@@ -492,7 +672,7 @@ k_minmax_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64
     const int c = threadIdx.x;
     float a = s_mn[0][c], b = s_mx[0][c];
 #pragma unroll
-    for (int w = 1; w < 4; ++w) { a = fminf(a, s_mn[w][c]); b = fmaxf(b, s_mx[w][c]); }
+    for (int w = 1; w < kWaves; ++w) { a = fminf(a, s_mn[w][c]); b = fmaxf(b, s_mx[w][c]); }
     uint32_t *mmh = mm + (int64_t)h * 256;
     atomicMin(&mmh[c], rdkv_float_to_ordered(a));
     atomicMax(&mmh[128 + c], rdkv_float_to_ordered(b));
@@ -592,65 +772,132 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
   }
 }
 
-// D == 128, rows 16-byte aligned: sixteen lanes per canvas row (eight channels each, one 16-byte
-// load), four rows per wavefront step, the next step's rows in flight while the current ones are
-// quantized.  A lane's channels never change, so their parameters and slots live in registers;
-// codes go to their sorted slots in a per-row LDS buffer (one byte per slot; a pruned channel's
-// zero goes to a spare byte, so nothing branches) and each of the row's sixteen lanes assembles
-// four consecutive packed bytes of every class from aligned dwords of that buffer.
-__global__ void __launch_bounds__(256)
-k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
-                         const int32_t *__restrict__ order, int64_t order_stride_h,
-                         const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
-                         const uint32_t *__restrict__ mm, const int32_t *__restrict__ slot_channel,
-                         int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
-                         uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
-                         __half *__restrict__ zp_out, int rows_per_block) {
+// D == 128, rows 16-byte aligned.  A workgroup owns 128 consecutive canvas rows of one head;
+// sixteen lanes take a row (eight channels each, one 16-byte load), four rows per wavefront
+// step, eight steps.  Nothing between the loads is conditional: every lane fetches the source
+// indices of all its rows, then requests all the rows, and while those are on their way the
+// workgroup derives the channels' parameters - two dependent round trips per workgroup.  A zero
+// row of the canvas reads row 0 and discards it; a workgroup whose rows are all zero rows (the
+// gap between a head's own tokens and the widest head's) loads nothing.
+// A lane's channels never change, so their parameters and slots live in registers; codes go to
+// their sorted slots in a per-row LDS buffer (one byte per slot; a pruned channel's zero goes to
+// a spare byte, so nothing branches) and each of the row's sixteen lanes assembles four
+// consecutive packed bytes of every class from aligned dwords of that buffer and stores them
+// as one dword, aligned or not (the rows of K_2bit / K_4bit / K_8bit are 1 to 128 bytes long);
+// the up to three bytes at the end of a row are stored one by one.
+#define RDKV_EMIT_ROWS_D128 128
+// ANY_ROW: some row of the workgroup exists (otherwise all are zero rows and nothing is loaded;
+// the two cases are separate instantiations so that the waits of one do not constrain the other).
+template <bool ANY_ROW>
+__device__ __forceinline__ void
+k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
+                       const int32_t *__restrict__ order, int64_t order_stride_h,
+                       const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
+                       const uint32_t *__restrict__ mm, const int32_t *__restrict__ slot_channel,
+                       int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
+                       uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
+                       __half *__restrict__ zp_out) {
   constexpr int D = 128;
-  extern __shared__ float smem[];
+  constexpr int kSteps = RDKV_EMIT_ROWS_D128 / 16;
   const int h = blockIdx.y;
   const int Dp = n2p + n4p + n8;
-  // Slot buffer of a row: the four quarter ranges of the 2-bit class, the two halves of the 4-bit
-  // class and the 8-bit class each start on a 4-byte boundary, so that four consecutive output
-  // bytes are assembled from aligned dwords; then a spare byte for pruned channels.
   const int sub2 = n2p >> 2, sub4 = n4p >> 1;
-  const int sub2p = (sub2 + 3) & ~3, sub4p = (sub4 + 3) & ~3;
-  const int o4 = 4 * sub2p, o8 = o4 + 2 * sub4p;
-  const int Dp4 = o8 + ((n8 + 3) & ~3) + 4;
   const int tv = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2], n16 = counts[4 * h + 3];
   const bool has_pad = tv < max_tv || n16 < max_n16;   // zero rows of the canvas join the min/max
   const int64_t max_tk = max_tv + max_n16;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int sub = lane >> 4, l = lane & 15;
+  const int t0 = blockIdx.x * RDKV_EMIT_ROWS_D128;
+  const int t1 = (int)((int64_t)t0 + RDKV_EMIT_ROWS_D128 < max_tk ? (int64_t)t0 + RDKV_EMIT_ROWS_D128 : max_tk);
+  const int mtv = (int)max_tv;
+  const int rl = wave * 4 + sub;               // this lane's row of step 0, within the workgroup
+  // ---- first round trip: this thread's slot of the channel plan, the source indices of its rows --
+  // (requests are grouped by hand and pinned with scheduling barriers: the load counter returns
+  // in order, so a wait for the channel parameters must not stand behind the rows)
+  const int32_t *ord = order + (int64_t)h * order_stride_h;
+  const __half *Kh = K + (int64_t)h * stride_h;
+  // this thread's slots of the channel plan: threadIdx.x and threadIdx.x + 256 (the host checks Dp <= 512)
+  int ch[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int slot = (int)threadIdx.x + 256 * k;
+    ch[k] = slot_channel[(int64_t)h * Dp + (slot < Dp ? slot : 0)];
+  }
+  // (zero rows are masked with AND, not selected: a select invites the compiler to branch around
+  // the load, which puts a full wait between that load and its neighbours)
+  uint32_t real[kSteps];       // all ones for a row that exists, zero for a zero row of the canvas
+  int src[kSteps];
+#pragma unroll
+  for (int u = 0; u < kSteps; ++u) {
+    const int t = t0 + rl + 16 * u;
+    const bool head = t < tv, tail = t >= mtv && t - mtv < n16;
+    real[u] = (t < t1 && (head || tail)) ? 0xffffffffu : 0u;
+    src[u] = 0;
+  }
+  if (ANY_ROW) {
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u) {
+      const int t = t0 + rl + 16 * u;
+      src[u] = ord[(t < tv ? t : tv + (t - mtv)) & (int)real[u]];
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- second round trip: the channel's extremes, then the rows ---------------------------------
+  const uint32_t *mmh = mm + (int64_t)h * 2 * D;
+  uint32_t mn_bits[2], mx_bits[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const bool has_ch = (int)threadIdx.x + 256 * k < Dp && ch[k] >= 0;
+    mn_bits[k] = mmh[has_ch ? ch[k] : 0];
+    mx_bits[k] = mmh[D + (has_ch ? ch[k] : 0)];
+  }
+  uint4 piece[kSteps];
+#pragma unroll
+  for (int u = 0; u < kSteps; ++u) piece[u] = make_uint4(0u, 0u, 0u, 0u);
+  if (ANY_ROW) {
+#pragma unroll
+    for (int u = 0; u < kSteps; ++u)
+      piece[u] = *reinterpret_cast<const uint4 *>(Kh + (int64_t)(src[u] & (int)real[u]) * stride_t + 8 * l);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- LDS: channel parameters, then a slot buffer per row in flight --------------------------
+  // Slot buffer of a row: the four quarter ranges of the 2-bit class, the two halves of the 4-bit
+  // class and the 8-bit class each start on a 4-byte boundary, so that four consecutive output
+  // bytes are assembled from aligned dwords; then a spare byte for pruned channels.
+  const int sub2p = (sub2 + 3) & ~3, sub4p = (sub4 + 3) & ~3;
+  const int o4 = 4 * sub2p, o8 = o4 + 2 * sub4p;
+  const int Dp4 = o8 + ((n8 + 3) & ~3) + 4;
   float *c_scale = smem, *c_zp = smem + D, *c_qmax = smem + 2 * D;
   int *c_slot = reinterpret_cast<int *>(smem + 3 * D);
   uint8_t *rowbufs = reinterpret_cast<uint8_t *>(smem + 4 * D);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
-  const int sub = lane >> 4, l = lane & 15;
-  const uint32_t *mmh = mm + (int64_t)h * 2 * D;
   for (int c = threadIdx.x; c < D; c += blockDim.x) c_slot[c] = -1;
-  for (int i = threadIdx.x; i < nwaves * 4 * Dp4; i += blockDim.x) rowbufs[i] = 0;  // pad slots stay 0
+  for (int i = threadIdx.x; i < 16 * Dp4 / 4; i += blockDim.x)
+    reinterpret_cast<uint32_t *>(rowbufs)[i] = 0u;               // slots without a channel stay 0
   __syncthreads();
-  for (int s = threadIdx.x; s < Dp; s += blockDim.x) {
-    const int ch = slot_channel[(int64_t)h * Dp + s];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int s = (int)threadIdx.x + 256 * k;
+    if (s >= Dp) continue;
     const float qmax = s < n2p ? 3.0f : (s < n2p + n4p ? 15.0f : 255.0f);
     float mn = 0.0f, mx = 0.0f;
-    if (ch >= 0) {
-      mn = rdkv_ordered_to_float(mmh[ch]);
-      mx = rdkv_ordered_to_float(mmh[D + ch]);
+    if (ch[k] >= 0) {
+      mn = rdkv_ordered_to_float(mn_bits[k]);
+      mx = rdkv_ordered_to_float(mx_bits[k]);
       if (has_pad) {
         mn = fminf(mn, 0.0f);
         mx = fmaxf(mx, 0.0f);
       }
     }
     const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
-    if (ch >= 0) {
-      c_scale[ch] = p.scale;
-      c_zp[ch] = p.zp;
-      c_qmax[ch] = qmax;
+    if (ch[k] >= 0) {
+      c_scale[ch[k]] = p.scale;
+      c_zp[ch[k]] = p.zp;
+      c_qmax[ch[k]] = qmax;
       int at;      // where sorted slot s lives in the row's slot buffer
       if (s < n2p) at = (s / sub2) * sub2p + s % sub2;
       else if (s < n2p + n4p) at = o4 + ((s - n2p) / sub4) * sub4p + (s - n2p) % sub4;
       else at = o8 + (s - n2p - n4p);
-      c_slot[ch] = at;
+      c_slot[ch[k]] = at;
     }
     if (blockIdx.x == 0) {
       scale_out[(int64_t)h * Dp + s] = __float2half_rn(p.scale);
@@ -664,83 +911,99 @@ k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t
   int sl[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const int ch = 8 * l + e;
-    sl[e] = c_slot[ch];
-    qp[e].scale = sl[e] >= 0 ? c_scale[ch] : 1.0f;
-    qp[e].zp = sl[e] >= 0 ? c_zp[ch] : 0.0f;
+    const int c = 8 * l + e;
+    sl[e] = c_slot[c];
+    qp[e].scale = sl[e] >= 0 ? c_scale[c] : 1.0f;
+    qp[e].zp = sl[e] >= 0 ? c_zp[c] : 0.0f;
     qp[e].inv = __fdiv_rn(1.0f, qp[e].scale);
-    qm[e] = sl[e] >= 0 ? c_qmax[ch] : 0.0f;
+    qm[e] = sl[e] >= 0 ? c_qmax[c] : 0.0f;
     if (sl[e] < 0) sl[e] = Dp4 - 4;          // a pruned channel's code is 0 (qmax 0): the spare byte takes it
   }
-  const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;
-  const int64_t t1 = (t0 + rows_per_block < max_tk) ? t0 + rows_per_block : max_tk;
-  const int32_t *ord = order + (int64_t)h * order_stride_h;
-  const __half *Kh = K + (int64_t)h * stride_h;
-  uint8_t *rb = rowbufs + (wave * 4 + sub) * Dp4;
-  union Piece { uint4 u; uint16_t hw[8]; };
-  auto fetch = [&](int64_t t, Piece &v) {
-    v.u = make_uint4(0u, 0u, 0u, 0u);
-    if (t < t1) {
-      // canvas row -> source token (or a zero row)
-      const __half *kr = nullptr;
-      if (t < tv) kr = Kh + (int64_t)ord[t] * stride_t;
-      else if (t >= max_tv && t - max_tv < n16) kr = Kh + (int64_t)ord[tv + (t - max_tv)] * stride_t;
-      if (kr) v.u = *reinterpret_cast<const uint4 *>(kr + 8 * l);
+  uint8_t *rb = rowbufs + rl * Dp4;
+  const uint32_t *rb32 = reinterpret_cast<const uint32_t *>(rb);
+  // this lane's four bytes of a row (and of the row's second 64 bytes of the 8-bit class)
+  const int j0 = 4 * l;
+  const int q2 = sub2p >> 2, q4 = sub4p >> 2;
+  const int full2 = sub2 >> 2, full4 = sub4 >> 2, full8 = n8 >> 2;     // whole dwords of a row
+  const int64_t row0 = (int64_t)h * max_tk + t0 + rl;                  // this lane's row of step 0
+  uint8_t *p2 = K2 + row0 * sub2 + j0, *p4 = K4 + row0 * sub4 + j0, *p8 = K8 + row0 * n8 + j0;
+  typedef uint32_t __attribute__((aligned(1))) unaligned_u32;
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+  // a row's dword l, or the row's last one to three bytes
+  auto put = [&](uint8_t *dst, int full, int rem, uint32_t v) {
+    if (l < full) *reinterpret_cast<unaligned_u32 *>(dst) = v;
+    if (rem != 0 && l == full) {
+      dst[0] = (uint8_t)v;
+      if (rem > 1) dst[1] = (uint8_t)(v >> 8);
+      if (rem > 2) dst[2] = (uint8_t)(v >> 16);
     }
   };
-  const int step = nwaves * 4;
-  Piece cur, nxt;
-  fetch(t0 + wave * 4 + sub, cur);
-  for (int64_t tb = t0 + wave * 4; tb < t1; tb += step) {   // wave-uniform loop bound
-    const int64_t t = tb + sub;
-    fetch(t + step, nxt);
-    if (t < t1) {
-      float x[8];
-      uint32_t code[8];
-      bool near[8], any = false;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        x[e] = __half2float(__ushort_as_half(cur.hw[e]));
-        code[e] = rdkv_qcode_estimate(x[e], qp[e], qm[e], near[e]);
-        any = any || near[e];
-      }
-      if (any) {                     // about one value in 2500 needs the exact quotient
+  for (int u = 0; u < kSteps; ++u) {
+    const uint32_t rw[4] = {piece[u].x & real[u], piece[u].y & real[u], piece[u].z & real[u],
+                            piece[u].w & real[u]};
+    float x[8], tq[8], q[8];
+    float dmin = 1.0f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (near[e]) code[e] = rdkv_qcode_exact(x[e], qp[e], qm[e]);
-      }
+    for (int e = 0; e < 8; ++e) {
+      const half2_t hv = __builtin_bit_cast(half2_t, rw[e >> 1]);
+      x[e] = (float)((e & 1) ? hv.y : hv.x);
+      tq[e] = fmaf(x[e], qp[e].inv, qp[e].zp);
+      q[e] = rintf(__builtin_amdgcn_fmed3f(tq[e], 0.0f, qm[e]));
+      dmin = fminf(dmin, fabsf(fabsf(tq[e] - q[e]) - 0.5f));
+    }
+    if (dmin < 2e-4f) {                // about one value in 2500 needs the exact quotient
 #pragma unroll
-      for (int e = 0; e < 8; ++e) rb[sl[e]] = (uint8_t)code[e];
+      for (int e = 0; e < 8; ++e)
+        if (fabsf(fabsf(tq[e] - q[e]) - 0.5f) < 2e-4f) q[e] = (float)rdkv_qcode_exact(x[e], qp[e], qm[e]);
+    }
+    uint32_t w0 = 0u, w1 = 0u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      w0 = __builtin_amdgcn_cvt_pk_u8_f32(q[e], e, w0);
+      w1 = __builtin_amdgcn_cvt_pk_u8_f32(q[4 + e], e, w1);
+    }
+    // (rows past the workgroup's last one only touch their own slot buffer)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      rb[sl[e]] = (uint8_t)(w0 >> (8 * e));
+      rb[sl[4 + e]] = (uint8_t)(w1 >> (8 * e));
     }
     __builtin_amdgcn_wave_barrier();
-    if (t < t1) {
-      const int64_t row = (int64_t)h * max_tk + t;
-      const uint32_t *rb32 = reinterpret_cast<const uint32_t *>(rb);
-      // four bytes j0 .. j0+3 of an n-byte output row: one dword store where the address allows it
-      auto put = [&](uint8_t *dst, int n, int j0, uint32_t v) {
-        if (j0 + 4 <= n && (reinterpret_cast<uintptr_t>(dst + j0) & 3) == 0) {
-          *reinterpret_cast<uint32_t *>(dst + j0) = v;
-        } else {
-#pragma unroll
-          for (int k = 0; k < 4; ++k)
-            if (j0 + k < n) dst[j0 + k] = (uint8_t)(v >> (8 * k));
-        }
-      };
-      const int j0 = 4 * l;
+    if (t0 + rl + 16 * u < t1) {
       // (codes of the 2- and 4-bit classes are below 4 and 16: the shifts never carry into the next byte)
-      if (j0 < sub2) {
-        const int w = j0 >> 2, q = sub2p >> 2;
-        put(K2 + row * sub2, sub2, j0, rb32[w] | (rb32[w + q] << 2) | (rb32[w + 2 * q] << 4) | (rb32[w + 3 * q] << 6));
-      }
-      if (j0 < sub4) {
-        const int w = (o4 + j0) >> 2;
-        put(K4 + row * sub4, sub4, j0, rb32[w] | (rb32[w + (sub4p >> 2)] << 4));
-      }
-      for (int j = j0; j < n8; j += 64) put(K8 + row * (int64_t)n8, n8, j, rb32[(o8 + j) >> 2]);
+      if (j0 < sub2)
+        put(p2 + (int64_t)(16 * u) * sub2, full2, sub2 & 3,
+            rb32[l] | (rb32[l + q2] << 2) | (rb32[l + 2 * q2] << 4) | (rb32[l + 3 * q2] << 6));
+      if (j0 < sub4)
+        put(p4 + (int64_t)(16 * u) * sub4, full4, sub4 & 3, rb32[(o4 >> 2) + l] | (rb32[(o4 >> 2) + l + q4] << 4));
+      if (j0 < n8) put(p8 + (int64_t)(16 * u) * n8, full8, n8 & 3, rb32[(o8 >> 2) + l]);
+      if (j0 + 64 < n8)                            // bytes 64 .. 127 of a long 8-bit row
+        put(p8 + (int64_t)(16 * u) * n8 + 64, full8 - 16, n8 & 3, rb32[(o8 >> 2) + l + 16]);
     }
     __builtin_amdgcn_wave_barrier();
-    cur = nxt;
   }
+}
+
+__global__ void __launch_bounds__(256)
+k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
+                         const int32_t *__restrict__ order, int64_t order_stride_h,
+                         const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
+                         const uint32_t *__restrict__ mm, const int32_t *__restrict__ slot_channel,
+                         int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
+                         uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
+                         __half *__restrict__ zp_out) {
+  extern __shared__ float smem[];
+  const int h = blockIdx.y;
+  const int tv = counts[4 * h] + counts[4 * h + 1] + counts[4 * h + 2], n16 = counts[4 * h + 3];
+  const int64_t t0 = (int64_t)blockIdx.x * RDKV_EMIT_ROWS_D128;
+  const int64_t t1 = t0 + RDKV_EMIT_ROWS_D128 < max_tv + max_n16 ? t0 + RDKV_EMIT_ROWS_D128 : max_tv + max_n16;
+  if (t0 < tv || (t1 > max_tv && t0 < max_tv + n16))               // uniform over the workgroup
+    k_emit_layer_d128_body<true>(smem, K, stride_h, stride_t, order, order_stride_h, counts, max_tv, max_n16, mm,
+                                 slot_channel, n2p, n4p, n8, K2, K4, K8, scale_out, zp_out);
+  else
+    k_emit_layer_d128_body<false>(smem, K, stride_h, stride_t, order, order_stride_h, counts, max_tv, max_n16, mm,
+                                  slot_channel, n2p, n4p, n8, K2, K4, K8, scale_out, zp_out);
 }
 
 // ---------------------------------------------------------------------------
@@ -891,6 +1154,21 @@ static int pack_layer_v_rows(const char *fn, const void *V_f16, int64_t stride_h
   const int waves = 4;
   const int64_t blocks = rdkv_cdiv(v_rows, waves * RDKV_PACK_V_ROWS_PER_WAVE);
   RDKV_REQUIRE(blocks <= 0x7fffffffLL, "%s: too many rows", fn);
+  const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)V_f16 % 16) == 0 &&
+                      ((uintptr_t)V2 % 8) == 0 && ((uintptr_t)V4 % 8) == 0 && ((uintptr_t)V8 % 8) == 0 &&
+                      ((uintptr_t)V16_f16 % 16) == 0 && v_rows < 0x7fff0000LL;
+  if (rows16) {
+    // a workgroup takes rows of one class: the grid is the sum of the classes' block counts
+    const int rows_wg = waves * RDKV_PACK_V_ROWS_PER_WAVE;
+    const int64_t class_blocks = rdkv_cdiv(mN2, rows_wg) + rdkv_cdiv(mN4, rows_wg) + rdkv_cdiv(mN8, rows_wg) +
+                                 rdkv_cdiv(max_n16, rows_wg);
+    hipLaunchKernelGGL(pack_v_layer_d128_kernel, dim3((unsigned)class_blocks, H_kv), dim3(64 * waves), 0, s,
+                       (const __half *)V_f16, stride_h, stride_t, order, order_stride_h, counts, mN2, mN4, mN8,
+                       max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16, (__half *)V16_f16,
+                       reinterpret_cast<uint32_t *>(mm_init));
+    RDKV_CHECK_LAUNCH(fn);
+    return RDKV_OK;
+  }
   hipLaunchKernelGGL(pack_v_layer_kernel, dim3((unsigned)blocks, H_kv), dim3(64 * waves), 0, s,
                      (const __half *)V_f16, stride_h, stride_t, D, order, order_stride_h, counts, mN2, mN4, mN8,
                      max_n16, max_tv, V2, V4, V8, (__half *)V_scale_f16, (__half *)V_zp_f16, (__half *)V16_f16,
@@ -913,6 +1191,7 @@ static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h
                "%s: bad segment sizes (%d,%d,%d)", fn, n2p, n4p, n8);
   const int Dp = n2p + n4p + n8;
   RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "%s: %d padded channels > %d", fn, Dp, RDKV_MAX_SLOTS);
+  RDKV_REQUIRE(D != 128 || Dp <= 512, "%s: %d padded channels for D = 128", fn, Dp);
   RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0,
                "%s: rows must be 4-byte aligned", fn);
   const int64_t max_tk = max_tv + max_n16;
@@ -931,7 +1210,8 @@ static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h
   const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
   if (rows16) {
     hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
-                       dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv), dim3(256), 0, s,
+                       dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv),
+                       dim3(64 * RDKV_LAYER_MINMAX_WAVES_D128), 0, s,
                        (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
   } else {
     hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
@@ -943,13 +1223,13 @@ static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h
   const size_t emit_lds = (size_t)D * 16 + 4 * (size_t)((Dp + 3) & ~3);
   RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
   if (rows16) {
-    const int rows_d128 = 256;
     const size_t lds_d128 = (size_t)128 * 16 +
                             16 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
-    hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, rows_d128), H_kv), dim3(256),
-                       lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, max_tv,
-                       max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
-                       (__half *)K_zp_f16, rows_d128);
+    RDKV_REQUIRE(max_tk < 0x7fff0000LL, "%s: too many rows", fn);
+    hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, RDKV_EMIT_ROWS_D128), H_kv),
+                       dim3(256), lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h,
+                       counts, max_tv, max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
+                       (__half *)K_zp_f16);
   } else {
     hipLaunchKernelGGL(k_emit_layer_kernel, dim3((unsigned)eblocks, H_kv), dim3(256), emit_lds, s,
                        (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, max_tv, max_n16,

@@ -217,12 +217,15 @@ def _layers_identical(a, b):
 
 
 @pytest.mark.parametrize("case", ["ragged", "equal_counts", "empty_head", "fp16_only_head", "no_fp16",
-                                  "one_class", "strided_input"])
+                                  "one_class", "strided_input", "rows_not_16_byte_aligned", "many_blocks",
+                                  "many_blocks_gap"])
 def test_whole_layer_packer_matches_composition(case):
     """The few-launch layer packer against the call-for-call composition it replaces (which is
     itself pinned to the oracle and the golden vectors), on layouts that stress the padding."""
     rng = np.random.default_rng(sum(map(ord, case)))
     H, T, D, G = 3, 157, 128, 2
+    if case.startswith("many_blocks"):       # several workgroups per head in every kernel of the packer
+        T = 2900
     K = torch.randn(1, H, T, D, device=DEV).half()
     V = torch.randn(1, H, T, D, device=DEV).half()
     choices = np.array([0, 2, 4, 8, 16])
@@ -242,6 +245,14 @@ def test_whole_layer_packer_matches_composition(case):
     elif case == "strided_input":
         big = torch.randn(1, H, T, 2 * D, device=DEV).half()
         K, V = big[..., :D], big[..., D:]
+    elif case == "rows_not_16_byte_aligned":   # 4-byte aligned rows: the kernels that read 16-byte pieces step aside
+        big = torch.randn(1, H, T, 2 * D + 4, device=DEV).half()
+        K, V = big[..., 2:D + 2], big[..., D + 2:2 * D + 2]
+    elif case == "many_blocks_gap":
+        # one head keeps few tokens: its canvas has a long run of zero rows (whole workgroups of them),
+        # and its fp16 rows start far behind its own compressed rows
+        vb[2] = torch.from_numpy(rng.choice(choices, size=T, p=[0.9, 0.02, 0.03, 0.03, 0.02]))
+        K = K + 0.75                         # a zero row is not in the middle of the value range
     kb = torch.from_numpy(rng.choice(np.array([0, 0, 2, 4, 8, 16]), size=(H, D)))
     got, got_nvo = packing.pack_layer_per_head(K, V, vb, kb, G)
     exp, exp_nvo = packing._pack_layer_per_head_composed(K, V, vb, kb, G)
