@@ -772,10 +772,10 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
   }
 }
 
-// D == 128, rows 16-byte aligned.  A workgroup owns 128 consecutive canvas rows of one head;
-// sixteen lanes take a row (eight channels each, one 16-byte load), four rows per wavefront
-// step, eight steps.  Nothing between the loads is conditional: every lane fetches the source
-// indices of all its rows, then requests all the rows, and while those are on their way the
+// D == 128, rows 16-byte aligned.  A workgroup of four wavefronts owns 128 consecutive canvas
+// rows of one head; sixteen lanes take a row (eight channels each, one 16-byte load), four rows
+// per wavefront step, eight steps.  Nothing between the loads is conditional: every lane fetches
+// the source indices of all its rows, then requests all the rows, and while those are on their way the
 // workgroup derives the channels' parameters - two dependent round trips per workgroup.  A zero
 // row of the canvas reads row 0 and discards it; a workgroup whose rows are all zero rows (the
 // gap between a head's own tokens and the widest head's) loads nothing.
@@ -785,7 +785,9 @@ k_emit_layer_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stri
 // consecutive packed bytes of every class from aligned dwords of that buffer and stores them
 // as one dword, aligned or not (the rows of K_2bit / K_4bit / K_8bit are 1 to 128 bytes long);
 // the up to three bytes at the end of a row are stored one by one.
-#define RDKV_EMIT_ROWS_D128 128
+#define RDKV_EMIT_WAVES_D128 4     // eight were measured slower (32 against 30 us on a 32k-token layer)
+#define RDKV_EMIT_STEP_ROWS_D128 (4 * RDKV_EMIT_WAVES_D128)      // rows of a workgroup step
+#define RDKV_EMIT_ROWS_D128 (8 * RDKV_EMIT_STEP_ROWS_D128)
 // ANY_ROW: some row of the workgroup exists (otherwise all are zero rows and nothing is loaded;
 // the two cases are separate instantiations so that the waits of one do not constrain the other).
 template <bool ANY_ROW>
@@ -798,7 +800,9 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
                        uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
                        __half *__restrict__ zp_out) {
   constexpr int D = 128;
-  constexpr int kSteps = RDKV_EMIT_ROWS_D128 / 16;
+  constexpr int kStepRows = RDKV_EMIT_STEP_ROWS_D128, kThreads = 64 * RDKV_EMIT_WAVES_D128;
+  constexpr int kSteps = RDKV_EMIT_ROWS_D128 / kStepRows;
+  constexpr int kSlotPasses = (512 + kThreads - 1) / kThreads;     // the host checks Dp <= 512
   const int h = blockIdx.y;
   const int Dp = n2p + n4p + n8;
   const int sub2 = n2p >> 2, sub4 = n4p >> 1;
@@ -816,11 +820,11 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
   // in order, so a wait for the channel parameters must not stand behind the rows)
   const int32_t *ord = order + (int64_t)h * order_stride_h;
   const __half *Kh = K + (int64_t)h * stride_h;
-  // this thread's slots of the channel plan: threadIdx.x and threadIdx.x + 256 (the host checks Dp <= 512)
-  int ch[2];
+  // this thread's slot(s) of the channel plan
+  int ch[kSlotPasses];
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const int slot = (int)threadIdx.x + 256 * k;
+  for (int k = 0; k < kSlotPasses; ++k) {
+    const int slot = (int)threadIdx.x + kThreads * k;
     ch[k] = slot_channel[(int64_t)h * Dp + (slot < Dp ? slot : 0)];
   }
   // (zero rows are masked with AND, not selected: a select invites the compiler to branch around
@@ -829,7 +833,7 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
   int src[kSteps];
 #pragma unroll
   for (int u = 0; u < kSteps; ++u) {
-    const int t = t0 + rl + 16 * u;
+    const int t = t0 + rl + kStepRows * u;
     const bool head = t < tv, tail = t >= mtv && t - mtv < n16;
     real[u] = (t < t1 && (head || tail)) ? 0xffffffffu : 0u;
     src[u] = 0;
@@ -837,17 +841,17 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
   if (ANY_ROW) {
 #pragma unroll
     for (int u = 0; u < kSteps; ++u) {
-      const int t = t0 + rl + 16 * u;
+      const int t = t0 + rl + kStepRows * u;
       src[u] = ord[(t < tv ? t : tv + (t - mtv)) & (int)real[u]];
     }
   }
   __builtin_amdgcn_sched_barrier(0);
   // ---- second round trip: the channel's extremes, then the rows ---------------------------------
   const uint32_t *mmh = mm + (int64_t)h * 2 * D;
-  uint32_t mn_bits[2], mx_bits[2];
+  uint32_t mn_bits[kSlotPasses], mx_bits[kSlotPasses];
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const bool has_ch = (int)threadIdx.x + 256 * k < Dp && ch[k] >= 0;
+  for (int k = 0; k < kSlotPasses; ++k) {
+    const bool has_ch = (int)threadIdx.x + kThreads * k < Dp && ch[k] >= 0;
     mn_bits[k] = mmh[has_ch ? ch[k] : 0];
     mx_bits[k] = mmh[D + (has_ch ? ch[k] : 0)];
   }
@@ -871,12 +875,12 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
   int *c_slot = reinterpret_cast<int *>(smem + 3 * D);
   uint8_t *rowbufs = reinterpret_cast<uint8_t *>(smem + 4 * D);
   for (int c = threadIdx.x; c < D; c += blockDim.x) c_slot[c] = -1;
-  for (int i = threadIdx.x; i < 16 * Dp4 / 4; i += blockDim.x)
+  for (int i = threadIdx.x; i < kStepRows * Dp4 / 4; i += blockDim.x)
     reinterpret_cast<uint32_t *>(rowbufs)[i] = 0u;               // slots without a channel stay 0
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < 2; ++k) {
-    const int s = (int)threadIdx.x + 256 * k;
+  for (int k = 0; k < kSlotPasses; ++k) {
+    const int s = (int)threadIdx.x + kThreads * k;
     if (s >= Dp) continue;
     const float qmax = s < n2p ? 3.0f : (s < n2p + n4p ? 15.0f : 255.0f);
     float mn = 0.0f, mx = 0.0f;
@@ -970,22 +974,22 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
       rb[sl[4 + e]] = (uint8_t)(w1 >> (8 * e));
     }
     __builtin_amdgcn_wave_barrier();
-    if (t0 + rl + 16 * u < t1) {
+    if (t0 + rl + kStepRows * u < t1) {
       // (codes of the 2- and 4-bit classes are below 4 and 16: the shifts never carry into the next byte)
       if (j0 < sub2)
-        put(p2 + (int64_t)(16 * u) * sub2, full2, sub2 & 3,
+        put(p2 + (int64_t)(kStepRows * u) * sub2, full2, sub2 & 3,
             rb32[l] | (rb32[l + q2] << 2) | (rb32[l + 2 * q2] << 4) | (rb32[l + 3 * q2] << 6));
       if (j0 < sub4)
-        put(p4 + (int64_t)(16 * u) * sub4, full4, sub4 & 3, rb32[(o4 >> 2) + l] | (rb32[(o4 >> 2) + l + q4] << 4));
-      if (j0 < n8) put(p8 + (int64_t)(16 * u) * n8, full8, n8 & 3, rb32[(o8 >> 2) + l]);
+        put(p4 + (int64_t)(kStepRows * u) * sub4, full4, sub4 & 3, rb32[(o4 >> 2) + l] | (rb32[(o4 >> 2) + l + q4] << 4));
+      if (j0 < n8) put(p8 + (int64_t)(kStepRows * u) * n8, full8, n8 & 3, rb32[(o8 >> 2) + l]);
       if (j0 + 64 < n8)                            // bytes 64 .. 127 of a long 8-bit row
-        put(p8 + (int64_t)(16 * u) * n8 + 64, full8 - 16, n8 & 3, rb32[(o8 >> 2) + l + 16]);
+        put(p8 + (int64_t)(kStepRows * u) * n8 + 64, full8 - 16, n8 & 3, rb32[(o8 >> 2) + l + 16]);
     }
     __builtin_amdgcn_wave_barrier();
   }
 }
 
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * RDKV_EMIT_WAVES_D128)
 k_emit_layer_d128_kernel(const __half *__restrict__ K, int64_t stride_h, int64_t stride_t,
                          const int32_t *__restrict__ order, int64_t order_stride_h,
                          const int32_t *__restrict__ counts, int64_t max_tv, int max_n16,
@@ -1224,10 +1228,10 @@ static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h
   RDKV_REQUIRE(emit_lds <= 60 * 1024, "%s: D=%d too large for the emit kernel", fn, D);
   if (rows16) {
     const size_t lds_d128 = (size_t)128 * 16 +
-                            16 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
+                            RDKV_EMIT_STEP_ROWS_D128 * (size_t)(4 * ((n2p / 4 + 3) & ~3) + 2 * ((n4p / 2 + 3) & ~3) + ((n8 + 3) & ~3) + 4);
     RDKV_REQUIRE(max_tk < 0x7fff0000LL, "%s: too many rows", fn);
     hipLaunchKernelGGL(k_emit_layer_d128_kernel, dim3((unsigned)rdkv_cdiv(max_tk, RDKV_EMIT_ROWS_D128), H_kv),
-                       dim3(256), lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h,
+                       dim3(64 * RDKV_EMIT_WAVES_D128), lds_d128, s, (const __half *)K_f16, stride_h, stride_t, order, order_stride_h,
                        counts, max_tv, max_n16, mm, slot_channel, n2p, n4p, n8, K2, K4, K8, (__half *)K_scale_f16,
                        (__half *)K_zp_f16);
   } else {
