@@ -625,13 +625,27 @@ softmax_rows_vec_kernel(const float *__restrict__ so, int64_t so_sh, const float
       x[k] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
       if (i < n4) x[k] = a4[i];
     }
-    if (m) {
+    if (m && n4 > 0) {
+      // The mask values of eight float4s are requested together and none of the loads is conditional
+      // (a slot past the row reads the row's first float4 and drops it): with the load inside the
+      // range check the compiler waits for each one before it issues the next, sixteen round trips
+      // one after the other, which was most of this kernel's time.
+      constexpr int kB = kKeep < 8 ? kKeep : 8;
 #pragma unroll
-      for (int k = 0; k < kKeep; ++k) {
-        const int64_t i = tid + (int64_t)k * 1024;
-        if (i < n4) {
-          const float4 kk = mask4(i);
-          x[k].x += kk.x; x[k].y += kk.y; x[k].z += kk.z; x[k].w += kk.w;
+      for (int k0 = 0; k0 < kKeep; k0 += kB) {
+        float4 mk[kB];
+#pragma unroll
+        for (int j = 0; j < kB; ++j) {
+          const int64_t i = tid + (int64_t)(k0 + j) * 1024;
+          mk[j] = mask4(i < n4 ? i : 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kB; ++j) {
+          const int64_t i = tid + (int64_t)(k0 + j) * 1024;
+          if (i < n4) {
+            x[k0 + j].x += mk[j].x; x[k0 + j].y += mk[j].y; x[k0 + j].z += mk[j].z; x[k0 + j].w += mk[j].w;
+          }
         }
       }
     }
@@ -718,13 +732,21 @@ softmax_rows_split_kernel(const float *__restrict__ so, int64_t so_sh, const flo
     x[k] = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
     if (i < hi) x[k] = a4[i];
   }
-  if (m) {
+  if (m && lo < hi) {
+    // (all mask loads of the piece requested together, none conditional: see softmax_rows_vec_kernel)
+    float4 mk[kSoftmaxPieceVec];
+#pragma unroll
+    for (int k = 0; k < kSoftmaxPieceVec; ++k) {
+      const int64_t i = lo + tid + (int64_t)k * 1024;
+      const int64_t ic = i < hi ? i : lo;
+      mk[k] = MASK_VEC ? m4[ic] : make_float4(m[4 * ic], m[4 * ic + 1], m[4 * ic + 2], m[4 * ic + 3]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int k = 0; k < kSoftmaxPieceVec; ++k) {
       const int64_t i = lo + tid + (int64_t)k * 1024;
       if (i < hi) {
-        const float4 kk = MASK_VEC ? m4[i] : make_float4(m[4 * i], m[4 * i + 1], m[4 * i + 2], m[4 * i + 3]);
-        x[k].x += kk.x; x[k].y += kk.y; x[k].z += kk.z; x[k].w += kk.w;
+        x[k].x += mk[k].x; x[k].y += mk[k].y; x[k].z += mk[k].z; x[k].w += mk[k].w;
       }
     }
   }
