@@ -154,16 +154,39 @@ plan_scatter_kernel(const void *__restrict__ v_bits, int vb_es, int64_t vb_strid
 
 // One workgroup per KV head: channel tables with the layer-wide padded segment sizes and the
 // per-head scalars.
-__global__ void __launch_bounds__(kPlanThreads)
-layer_tables_kernel(const void *__restrict__ k_bits, int kb_es, int64_t kb_stride_h, int D, int G,
-                    const int32_t *__restrict__ counts4, const int32_t *__restrict__ info,
-                    int n2p, int n4p, int n8o, int kept_max, int64_t max_tv,
-                    int32_t *__restrict__ slot_channel, int64_t *__restrict__ perm, int64_t *__restrict__ perm_q,
-                    int64_t *__restrict__ sort_ph, int32_t *__restrict__ seg_ph, int32_t *__restrict__ seg_tok,
-                    int32_t *__restrict__ t_eff, int32_t *__restrict__ t_eff_k, int32_t *__restrict__ n_v16) {
+struct LayerTables {
+  const void *k_bits;
+  int kb_es;
+  int64_t kb_stride_h;
+  int D, G;
+  const int32_t *counts4, *info;
+  int n2p, n4p, n8o, kept_max;
+  int64_t max_tv;
+  int32_t *slot_channel;
+  int64_t *perm, *perm_q, *sort_ph;
+  int32_t *seg_ph, *seg_tok, *t_eff, *t_eff_k, *n_v16;
+};
+struct LayerMask {
+  const int32_t *counts4;
+  int G;
+  int64_t max_tv, max_tk;
+  float *mask;
+  const int32_t *ord_ref, *rank_ref;
+  int64_t tv_ref;
+  int64_t *sort_idx;
+};
+
+__device__ __forceinline__ void layer_tables_block(const LayerTables &a, int h) {
+  const void *k_bits = a.k_bits;
+  const int kb_es = a.kb_es, D = a.D, G = a.G, n2p = a.n2p, n4p = a.n4p, n8o = a.n8o, kept_max = a.kept_max;
+  const int64_t kb_stride_h = a.kb_stride_h;
+  const int32_t *counts4 = a.counts4, *info = a.info;
+  int32_t *slot_channel = a.slot_channel, *seg_ph = a.seg_ph, *seg_tok = a.seg_tok, *t_eff = a.t_eff,
+          *t_eff_k = a.t_eff_k, *n_v16 = a.n_v16;
+  int64_t *perm = a.perm, *perm_q = a.perm_q, *sort_ph = a.sort_ph;
   __shared__ int wcnt[kPlanThreads / 64][3];
   __shared__ int wpre[kPlanThreads / 64][3];
-  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
   const int Dp = n2p + n4p + n8o;
   const int n2 = info[8 * h + 2], n4 = info[8 * h + 3];
   for (int j = tid; j < Dp; j += blockDim.x) {
@@ -209,23 +232,38 @@ layer_tables_kernel(const void *__restrict__ k_bits, int kb_es, int64_t kb_strid
     perm_q[((int64_t)h * G + j / Dp) * Dp + j % Dp] = perm[(int64_t)h * Dp + j % Dp];
 }
 
+__global__ void __launch_bounds__(kPlanThreads) layer_tables_kernel(LayerTables a) { layer_tables_block(a, blockIdx.x); }
+
 // mask[hq, col] = 0 where the canvas column holds a token of head hq / G, -inf where it is padding;
 // the first row of blocks also writes the sort index of head `ref`'s quantized tokens
 // (sort_idx[i] = rank among them of the i-th token in sorted order).
-__global__ void __launch_bounds__(256)
-softmax_mask_kernel(const int32_t *__restrict__ counts4, int G, int64_t max_tv, int64_t max_tk,
-                    float *__restrict__ mask, const int32_t *__restrict__ ord_ref,
-                    const int32_t *__restrict__ rank_ref, int64_t tv_ref, int64_t *__restrict__ sort_idx) {
-  const int hq = blockIdx.y, h = hq / G;
+__device__ __forceinline__ void softmax_mask_block(const LayerMask &a, int bx, int nbx, int hq) {
+  const int h = hq / a.G;
   if (hq == 0) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < tv_ref; i += (int64_t)gridDim.x * blockDim.x)
-      sort_idx[i] = rank_ref[ord_ref[i]];
+    for (int64_t i = (int64_t)bx * blockDim.x + threadIdx.x; i < a.tv_ref; i += (int64_t)nbx * blockDim.x)
+      a.sort_idx[i] = a.rank_ref[a.ord_ref[i]];
   }
-  const int64_t tv = (int64_t)counts4[4 * h] + counts4[4 * h + 1] + counts4[4 * h + 2], n16 = counts4[4 * h + 3];
-  for (int64_t col = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; col < max_tk;
-       col += (int64_t)gridDim.x * blockDim.x) {
-    const bool valid = col < tv || (col >= max_tv && col < max_tv + n16);
-    mask[(int64_t)hq * max_tk + col] = valid ? 0.0f : -__builtin_inff();
+  const int64_t tv = (int64_t)a.counts4[4 * h] + a.counts4[4 * h + 1] + a.counts4[4 * h + 2], n16 = a.counts4[4 * h + 3];
+  for (int64_t col = (int64_t)bx * blockDim.x + threadIdx.x; col < a.max_tk; col += (int64_t)nbx * blockDim.x) {
+    const bool valid = col < tv || (col >= a.max_tv && col < a.max_tv + n16);
+    a.mask[(int64_t)hq * a.max_tk + col] = valid ? 0.0f : -__builtin_inff();
+  }
+}
+
+__global__ void __launch_bounds__(256) softmax_mask_kernel(LayerMask a) {
+  softmax_mask_block(a, blockIdx.x, gridDim.x, blockIdx.y);
+}
+
+// Both in one launch (heads of up to 256 channels): blocks [0, H_kv) build the channel tables, the
+// nbx * H_q blocks after them write the mask - two launches of a few microseconds each were a
+// tenth of a 32k-token layer's packing time.
+__global__ void __launch_bounds__(256) layer_tables_mask_kernel(LayerTables t, LayerMask m, int H_kv, int nbx) {
+  const int b = blockIdx.x;
+  if (b < H_kv) {
+    layer_tables_block(t, b);
+  } else {
+    const int r = b - H_kv;
+    softmax_mask_block(m, r % nbx, nbx, r / nbx);
   }
 }
 
@@ -279,17 +317,30 @@ RDKV_API int rdkv_pack_layer_tables(const void *k_bits, int kb_elem_size, int64_
   RDKV_REQUIRE(tv_ref == 0 || (sort_idx && order && rank3), "%s: null token tables", fn);
   hipStream_t s = (hipStream_t)stream;
   const int threads = ((D + 63) / 64) * 64;
-  hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, k_bits, kb_elem_size, kb_stride_h, D, G,
-                     counts4, info, n2p, n4p, n8, kept_max, max_tv, slot_channel, perm, perm_for_q,
-                     sort_ch, seg_ch, seg_tok, t_eff, t_eff_k, n_v16);
+  LayerTables t;
+  t.k_bits = k_bits; t.kb_es = kb_elem_size; t.kb_stride_h = kb_stride_h; t.D = D; t.G = G;
+  t.counts4 = counts4; t.info = info; t.n2p = n2p; t.n4p = n4p; t.n8o = n8; t.kept_max = kept_max; t.max_tv = max_tv;
+  t.slot_channel = slot_channel; t.perm = perm; t.perm_q = perm_for_q; t.sort_ph = sort_ch;
+  t.seg_ph = seg_ch; t.seg_tok = seg_tok; t.t_eff = t_eff; t.t_eff_k = t_eff_k; t.n_v16 = n_v16;
   const int64_t max_tk = max_tv + max_n16;
   if (max_tk > 0) {
     RDKV_REQUIRE(softmax_mask, "%s: null mask", fn);
     int64_t bx = rdkv_cdiv(max_tk, 256 * 4);
     if (bx > 1024) bx = 1024;
-    hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, counts4, G,
-                       max_tv, max_tk, softmax_mask, order ? order + (int64_t)ref_head * order_stride_h : nullptr,
-                       rank3 ? rank3 + (int64_t)ref_head * rank3_stride_h : nullptr, tv_ref, sort_idx);
+    LayerMask m;
+    m.counts4 = counts4; m.G = G; m.max_tv = max_tv; m.max_tk = max_tk; m.mask = softmax_mask;
+    m.ord_ref = order ? order + (int64_t)ref_head * order_stride_h : nullptr;
+    m.rank_ref = rank3 ? rank3 + (int64_t)ref_head * rank3_stride_h : nullptr;
+    m.tv_ref = tv_ref; m.sort_idx = sort_idx;
+    const int64_t blocks = (int64_t)H_kv + bx * H_kv * G;
+    if (threads <= 256 && blocks <= 0x7fffffffLL) {
+      hipLaunchKernelGGL(layer_tables_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, t, m, H_kv, (int)bx);
+    } else {
+      hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, t);
+      hipLaunchKernelGGL(softmax_mask_kernel, dim3((unsigned)bx, (unsigned)(H_kv * G)), dim3(256), 0, s, m);
+    }
+  } else {
+    hipLaunchKernelGGL(layer_tables_kernel, dim3(H_kv), dim3(threads), 0, s, t);
   }
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
