@@ -92,7 +92,11 @@ def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_
     N2, N4, N8 = seg_bounds
     v16 = v16h = n16 = None
     if V16 is not None and n_v16_per_head is not None:
-        v16 = V16 if V16.is_contiguous() else V16.contiguous()
+        v16 = _sq(V16)                    # [H_kv, n16_max, 128]; the packer's new_v_only carries a leading 1
+        assert v16.dim() == 3 and v16.shape[0] == H_kv and v16.shape[2] == D and v16.dtype == torch.float16, \
+            f"V16 must be fp16 [H_kv={H_kv}, n, {D}], got {tuple(V16.shape)} {V16.dtype}"
+        assert n_v16_per_head.numel() == H_kv and n_v16_per_head.dtype == torch.int32
+        v16 = v16 if v16.is_contiguous() else v16.contiguous()
         v16h = v16.stride(0)
         n16 = n_v16_per_head.data_ptr()
         v16 = v16.data_ptr() if v16.numel() else None

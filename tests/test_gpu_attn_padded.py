@@ -52,6 +52,15 @@ def test_padded_attention_golden(name):
         n_v16_per_head=pl.n_v16_per_head, max_T_v=pl.T_eff)
     attn_close(t2n(obuf[:, :128]), g["out"], "out(strided)")
     assert float(obuf[:, 128:].abs().max()) == 0.0
+    if nvo is not None:
+        # the packer's fp16 rows as it returns them ([1, H_kv, n, 128]) are taken as they are; a tensor
+        # whose first dimension is not the KV heads is refused on the host, before any launch
+        o4 = vk.v_dequant_weighted_sum_dispatch(to_dev(g["weights"]), pl, V16=nvo, n_v16_per_head=pl.n_v16_per_head,
+                                                max_T_v=pl.T_eff)
+        assert torch.equal(o4, obuf[:, :128])
+        with pytest.raises(AssertionError):
+            vk.v_dequant_weighted_sum_dispatch(to_dev(g["weights"]), pl, V16=nvo[0].reshape(1, -1, 128),
+                                               n_v16_per_head=pl.n_v16_per_head, max_T_v=pl.T_eff)
     # K kernel into a strided buffer; fp16 query accepted as is
     sbuf = torch.full((q.shape[0], raw.shape[1] + 7), 123.0, device=DEV)
     kk.k_mixed_qk_dot_into(q, pl, raw.shape[1], sbuf)
