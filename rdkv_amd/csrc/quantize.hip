@@ -330,19 +330,22 @@ pack_v_rows_d128(const __half *__restrict__ Vh, int64_t stride_t, const int32_t 
       }
       const uint32_t rw[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
       float x[8], t[8], q[8];
-      float dmin = 1.0f;
+      // The estimate decides unless it lies within 2e-4 of a rounding boundary, i.e. unless it is
+      // more than 0.4998 away from the integer it rounds to (an estimate beyond the clamp's ends is
+      // caught by the same test and simply takes the exact path): one comparison per eight values.
+      float dmax = 0.0f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const half2_t hv = __builtin_bit_cast(half2_t, rw[e >> 1]);
         x[e] = (float)((e & 1) ? hv.y : hv.x);
         t[e] = fmaf(x[e], qp.inv, qp.zp);
         q[e] = rintf(__builtin_amdgcn_fmed3f(t[e], 0.0f, qmax));
-        dmin = fminf(dmin, fabsf(fabsf(t[e] - q[e]) - 0.5f));
+        dmax = fmaxf(dmax, fabsf(t[e] - q[e]));
       }
-      if (dmin < 2e-4f) {              // some value sits at a rounding boundary: the exact quotient decides
+      if (dmax > 0.4998f) {
 #pragma unroll
         for (int e = 0; e < 8; ++e)
-          if (fabsf(fabsf(t[e] - q[e]) - 0.5f) < 2e-4f) q[e] = (float)rdkv_qcode_exact(x[e], qp, qmax);
+          if (fabsf(t[e] - q[e]) > 0.4998f) q[e] = (float)rdkv_qcode_exact(x[e], qp, qmax);
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -919,7 +922,8 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
     sl[e] = c_slot[c];
     qp[e].scale = sl[e] >= 0 ? c_scale[c] : 1.0f;
     qp[e].zp = sl[e] >= 0 ? c_zp[c] : 0.0f;
-    qp[e].inv = __fdiv_rn(1.0f, qp[e].scale);
+    // (a pruned channel: estimate 0 whatever the value, so that it never asks for the exact quotient)
+    qp[e].inv = sl[e] >= 0 ? __fdiv_rn(1.0f, qp[e].scale) : 0.0f;
     qm[e] = sl[e] >= 0 ? c_qmax[c] : 0.0f;
     if (sl[e] < 0) sl[e] = Dp4 - 4;          // a pruned channel's code is 0 (qmax 0): the spare byte takes it
   }
@@ -947,32 +951,25 @@ k_emit_layer_d128_body(float *smem, const __half *__restrict__ K, int64_t stride
     const uint32_t rw[4] = {piece[u].x & real[u], piece[u].y & real[u], piece[u].z & real[u],
                             piece[u].w & real[u]};
     float x[8], tq[8], q[8];
-    float dmin = 1.0f;
+    // (the estimate decides unless it is more than 0.4998 away from the integer it rounds to: about
+    // one value in 2500 needs the exact quotient; one comparison per eight values finds them)
+    float dmax = 0.0f;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const half2_t hv = __builtin_bit_cast(half2_t, rw[e >> 1]);
       x[e] = (float)((e & 1) ? hv.y : hv.x);
       tq[e] = fmaf(x[e], qp[e].inv, qp[e].zp);
       q[e] = rintf(__builtin_amdgcn_fmed3f(tq[e], 0.0f, qm[e]));
-      dmin = fminf(dmin, fabsf(fabsf(tq[e] - q[e]) - 0.5f));
+      dmax = fmaxf(dmax, fabsf(tq[e] - q[e]));
     }
-    if (dmin < 2e-4f) {                // about one value in 2500 needs the exact quotient
+    if (dmax > 0.4998f) {
 #pragma unroll
       for (int e = 0; e < 8; ++e)
-        if (fabsf(fabsf(tq[e] - q[e]) - 0.5f) < 2e-4f) q[e] = (float)rdkv_qcode_exact(x[e], qp[e], qm[e]);
-    }
-    uint32_t w0 = 0u, w1 = 0u;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      w0 = __builtin_amdgcn_cvt_pk_u8_f32(q[e], e, w0);
-      w1 = __builtin_amdgcn_cvt_pk_u8_f32(q[4 + e], e, w1);
+        if (fabsf(tq[e] - q[e]) > 0.4998f) q[e] = (float)rdkv_qcode_exact(x[e], qp[e], qm[e]);
     }
     // (rows past the workgroup's last one only touch their own slot buffer)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      rb[sl[e]] = (uint8_t)(w0 >> (8 * e));
-      rb[sl[4 + e]] = (uint8_t)(w1 >> (8 * e));
-    }
+    for (int e = 0; e < 8; ++e) rb[sl[e]] = (uint8_t)(uint32_t)q[e];
     __builtin_amdgcn_wave_barrier();
     if (t0 + rl + kStepRows * u < t1) {
       // (codes of the 2- and 4-bit classes are below 4 and 16: the shifts never carry into the next byte)
