@@ -1,0 +1,142 @@
+"""GPU parity on seeded random workloads: allocations, head counts and lengths that no hand-written
+case has - every class present or absent, one to 128 kept K channels, 1 to 1700 tokens, 1 to 8 query
+heads per KV head.  The whole-layer packer is compared with the call-for-call composition (bit for
+bit; the composition is pinned to the oracle and the golden vectors elsewhere), the fused decode
+path (GPU packer -> streaming cache -> fused kernel) with the oracle's attention over the oracle's
+own packing of the same inputs."""
+import dataclasses
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import rdkv_oracle as O
+from rdkv_amd import packing, stream_cache
+from tests.gpu_util import DEV, require_gpu
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    require_gpu()
+
+
+def _first_difference(a, b):
+    for f in dataclasses.fields(a):
+        x, y = getattr(a, f.name), getattr(b, f.name)
+        if torch.is_tensor(x) or torch.is_tensor(y):
+            if not (torch.is_tensor(x) and torch.is_tensor(y)):
+                return f"{f.name}: tensor against {type(y).__name__}"
+            if x.dtype != y.dtype or x.shape != y.shape:
+                return f"{f.name}: {x.dtype} {tuple(x.shape)} against {y.dtype} {tuple(y.shape)}"
+            xv = x.view(torch.uint8) if x.dtype == torch.float16 else x
+            yv = y.view(torch.uint8) if y.dtype == torch.float16 else y
+            if not torch.equal(xv, yv):
+                return f"{f.name}: values"
+        elif x != y:
+            return f"{f.name}: {x} against {y}"
+    return None
+
+
+def _class_probabilities(rng, n):
+    p = rng.random(n) * (rng.random(n) < 0.7)
+    if p.sum() == 0:
+        p[int(rng.integers(0, n))] = 1.0
+    return p / p.sum()
+
+
+@pytest.mark.parametrize("block", range(4))
+def test_whole_layer_packer_random_layouts(block):
+    """60 layers per block: random class mixes for tokens and channels (a class may be missing, a head
+    may keep nothing or only fp16 rows), data at three magnitudes and with an offset, constant rows,
+    inputs that are views into wider tensors."""
+    widths = np.array([0, 2, 4, 8, 16])
+    for case in range(60):
+        rng = np.random.default_rng(7000 + 100 * block + case)
+        H, G = int(rng.integers(1, 6)), int(rng.choice([1, 2, 4]))
+        T = int(rng.choice([1, 2, 3, 17, 63, 64, 65, 127, 129, 300, 700, 1500, 2500]))
+        D = 128
+        vb = torch.from_numpy(rng.choice(widths, size=(H, T), p=_class_probabilities(rng, 5)))
+        if rng.random() < 0.3:
+            vb[int(rng.integers(0, H))] = int(rng.choice(widths))
+        kb = torch.from_numpy(rng.choice(widths, size=(H, D), p=_class_probabilities(rng, 5)))
+        scale = float(rng.choice([1.0, 0.01, 30.0]))
+        K = (torch.randn(1, H, T, D, device=DEV) * scale + float(rng.choice([0.0, 0.75, -2.0]))).half()
+        V = (torch.randn(1, H, T, D, device=DEV) * scale).half()
+        if rng.random() < 0.2:
+            V[0, 0, : max(1, T // 3)] = 0.5
+        if rng.random() < 0.2:
+            big = torch.randn(1, H, T, 2 * D, device=DEV).half()
+            K, V = big[..., :D], big[..., D:]
+        what = f"block {block} case {case}: H={H} G={G} T={T}"
+        try:
+            exp, exp_n = packing._pack_layer_per_head_composed(K, V, vb, kb, G)
+        except (AssertionError, ValueError):            # a layout the composition refuses: so must the packer
+            with pytest.raises((AssertionError, ValueError)):
+                packing.pack_layer_per_head(K, V, vb, kb, G)
+            continue
+        got, got_n = packing.pack_layer_per_head(K, V, vb, kb, G)
+        assert _first_difference(got, exp) is None, f"{what}: {_first_difference(got, exp)}"
+        assert (got_n is None) == (exp_n is None), what
+        if exp_n is not None:
+            assert torch.equal(got_n.view(torch.uint8), exp_n.view(torch.uint8)), what
+
+
+@pytest.mark.parametrize("block", range(3))
+def test_fused_attention_random_workloads(block):
+    """40 workloads per block, one to three layers in one launch: max-abs error of the output within
+    2e-3 of the oracle's (2e-3 of its largest value where that exceeds 1: data is drawn at three
+    magnitudes), log-sum-exp within 2e-3 (times the square of the magnitude, which the scores scale
+    with), rows that attend to nothing infinite in both."""
+    for case in range(40):
+        rng = np.random.default_rng(9000 + 100 * block + case)
+        H_kv, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8]))
+        H_q = H_kv * G
+        T = int(rng.choice([1, 5, 63, 64, 65, 130, 400, 900, 1700]))
+        layers = int(rng.integers(1, 4))
+        p = rng.random(5) * (rng.random(5) < 0.75)
+        if p[1:].sum() == 0:
+            p[int(rng.integers(1, 5))] = 1.0
+        p = p / p.sum()
+        keep = int(rng.choice([8, 33, 64, 100, 128]))
+        kk = rng.multinomial(keep, rng.dirichlet([1, 1, 1]))
+        what = f"block {block} case {case}: H_kv={H_kv} G={G} T={T} layers={layers} channels={tuple(int(x) for x in kk)}"
+        packed, qs, exp = [], [], []
+        for _ in range(layers):
+            vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T), p=p))
+            kb = np.zeros((H_kv, 128), dtype=np.int64)
+            for h in range(H_kv):
+                ch = rng.permutation(128)
+                kb[h, ch[:kk[0]]] = 2
+                kb[h, ch[kk[0]:kk[0] + kk[1]]] = 4
+                kb[h, ch[kk[0] + kk[1]:keep]] = 8
+            kb = torch.from_numpy(kb)
+            scale = float(rng.choice([1.0, 0.05, 8.0]))
+            K = (torch.from_numpy(rng.standard_normal((1, H_kv, T, 128)).astype(np.float32)) * scale).half()
+            V = (torch.from_numpy(rng.standard_normal((1, H_kv, T, 128)).astype(np.float32)) * scale).half()
+            q = torch.from_numpy(rng.standard_normal((H_q, 128)).astype(np.float32)).half()
+            try:
+                ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+            except (AssertionError, ValueError):        # a layer the reference's packer refuses (nothing kept)
+                packed = None
+                break
+            out, lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+            exp.append((out, lse, scale))
+            packed.append(packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G))
+            qs.append(q)
+        if packed is None:
+            continue
+        cache = stream_cache.build_stream_cache(packed, G)
+        out, lse = stream_cache.decode_attn_fused(cache, torch.cat(qs).to(DEV))
+        out, lse = out.float().cpu().numpy(), lse.float().cpu().numpy()
+        for layer, (eo, el, scale) in enumerate(exp):
+            rows = slice(layer * H_q, (layer + 1) * H_q)
+            fin = np.isfinite(el)
+            assert np.array_equal(np.isfinite(lse[rows]), fin), f"{what}, layer {layer}: rows without tokens"
+            eo = np.where(np.isfinite(eo), eo, 0.0)
+            err = float(np.abs(out[rows] - eo).max()) / max(1.0, float(np.abs(eo).max()))
+            assert err < 2e-3, f"{what}, layer {layer} (magnitude {scale}): output error {err:.3e}"
+            if fin.any():
+                err_l = float(np.abs(lse[rows][fin] - el[fin]).max())
+                assert err_l < 2e-3 * max(1.0, 16 * scale * scale), f"{what}, layer {layer}: lse error {err_l:.3e}"
