@@ -3,7 +3,8 @@ case has - every class present or absent, one to 128 kept K channels, 1 to 1700 
 heads per KV head.  The whole-layer packer is compared with the call-for-call composition (bit for
 bit; the composition is pinned to the oracle and the golden vectors elsewhere), the fused decode
 path (GPU packer -> streaming cache -> fused kernel) with the oracle's attention over the oracle's
-own packing of the same inputs."""
+own packing of the same inputs, and so are the reference-layout entry points (K scores, the
+caller's masked softmax, V sum) with per-head K allocations that differ in their class sizes."""
 import dataclasses
 
 import numpy as np
@@ -12,6 +13,8 @@ import torch
 
 from oracle import rdkv_oracle as O
 from rdkv_amd import packing, stream_cache
+from rdkv_amd import triton_k_kernel as kk
+from rdkv_amd import triton_v_kernel as vk
 from tests.gpu_util import DEV, require_gpu
 
 pytestmark = pytest.mark.gpu
@@ -140,3 +143,54 @@ def test_fused_attention_random_workloads(block):
             if fin.any():
                 err_l = float(np.abs(lse[rows][fin] - el[fin]).max())
                 assert err_l < 2e-3 * max(1.0, 16 * scale * scale), f"{what}, layer {layer}: lse error {err_l:.3e}"
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_reference_layout_entry_points_random_layers(block):
+    """40 layers per block through k_mixed_qk_dot -> + mask -> softmax -> v_dequant_weighted_sum_dispatch,
+    as fast_decode.py:1707-1768 chains them: output within 2e-3 of the oracle's (relative to its
+    largest value where that exceeds 1; 4e-3 at magnitude 8, where the oracle's fp16 rounding of
+    the dequantized values shows)."""
+    for case in range(40):
+        rng = np.random.default_rng(11000 + 100 * block + case)
+        H_kv, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 3, 4, 8]))
+        H_q = H_kv * G
+        T = int(rng.choice([1, 5, 63, 64, 65, 130, 255, 256, 257, 400, 900, 1700]))
+        p = rng.random(5) * (rng.random(5) < 0.75)
+        if p[1:].sum() == 0:
+            p[int(rng.integers(1, 5))] = 1.0
+        p = p / p.sum()
+        keep = int(rng.choice([4, 8, 33, 64, 100, 128]))
+        shared = rng.multinomial(keep, rng.dirichlet([1, 1, 1]))
+        per_head = rng.random() < 0.5
+        vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T), p=p))
+        kb = np.zeros((H_kv, 128), dtype=np.int64)
+        for h in range(H_kv):
+            kc = rng.multinomial(keep, rng.dirichlet([1, 1, 1])) if per_head else shared
+            ch = rng.permutation(128)
+            kb[h, ch[:kc[0]]] = 2
+            kb[h, ch[kc[0]:kc[0] + kc[1]]] = 4
+            kb[h, ch[kc[0] + kc[1]:keep]] = 8
+        kb = torch.from_numpy(kb)
+        scale = float(rng.choice([1.0, 0.05, 8.0]))
+        K = (torch.from_numpy(rng.standard_normal((1, H_kv, T, 128)).astype(np.float32)) * scale).half()
+        V = (torch.from_numpy(rng.standard_normal((1, H_kv, T, 128)).astype(np.float32)) * scale).half()
+        q = torch.from_numpy(rng.standard_normal((H_q, 128)).astype(np.float32)).half()
+        what = f"block {block} case {case}: H_kv={H_kv} G={G} T={T} kept channels {keep} magnitude {scale}"
+        try:
+            ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+        except (AssertionError, ValueError):
+            continue
+        exp, lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+        pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
+        T_old = pl.T_eff_k if pl.T_eff_k > 0 else pl.T_eff
+        scores = kk.k_mixed_qk_dot(q.to(DEV).float(), pl, T_old)
+        if pl.softmax_mask is not None:
+            scores.add_(pl.softmax_mask)
+        w = torch.nan_to_num(torch.softmax(scores, dim=-1), nan=0.0)      # a head without tokens: no weights
+        out = vk.v_dequant_weighted_sum_dispatch(w, pl, V16=nvo, n_v16_per_head=pl.n_v16_per_head,
+                                                 max_T_v=pl.T_eff).float().cpu().numpy()
+        rows = np.isfinite(lse)
+        if rows.any():
+            err = float(np.abs(out[rows] - exp[rows]).max()) / max(1.0, float(np.abs(exp[rows]).max()))
+            assert err < (4e-3 if scale > 1 else 2e-3), f"{what}: output error {err:.3e}"
