@@ -118,15 +118,25 @@ def _quantize_rows(x2d: Tensor, n_bits: int, pack: bool, row_idx: Optional[Tenso
     return out, scale, zp
 
 
+def _require_rows_to_reduce(n: int, dim: int) -> None:
+    """The quantizer's minimum over an empty dimension does not exist: torch's ``amin`` raises
+    IndexError for it (packing.py:153), which is what a caller of the reference sees when it packs
+    K channels over zero rows (packing.py:304-351)."""
+    if n == 0:
+        raise IndexError(f"amin(): Expected reduction dim {dim} to have non-zero size.")
+
+
 def quantize_and_pack(x: Tensor, n_bits: int, dim: int) -> Tuple[Tensor, Tensor, Tensor]:
     """Uniform asymmetric quantization along ``dim`` (packing.py:141-165).
 
     scale = max((max-min)/(2^b-1), 1e-8); zp = round(clamp(-min/scale)); codes =
     round(clamp(x/scale + zp)); returns (uint8 codes shaped like x, fp16 scale, fp16 zp
     with keepdim).  Codes use the fp32 scale, the returned scale is its fp16 rounding.
+    A reduction over no element raises IndexError, as the reference's ``amin`` does (packing.py:153).
     """
     _lib.require_device(x)
     dim = dim % x.dim()
+    _require_rows_to_reduce(int(x.shape[dim]), dim)
     xt = x.to(torch.float16).movedim(dim, -1).contiguous()
     lead = xt.shape[:-1]
     codes, scale, zp = _quantize_rows(xt.reshape(-1, xt.shape[-1]), n_bits, pack=False)
@@ -224,6 +234,8 @@ def pack_k_mixed(K: Tensor, k_bits: Tensor, *, sub_2_target: Optional[int] = Non
     H, T, D = K.shape[1], K.shape[2], K.shape[3]
     plan = _plan_k_channels(k_bits.detach().cpu().tolist(), sub_2_target, sub_4_target,
                             n_ch_8_target, segment_counts)
+    if sum(plan.padded) > 0:
+        _require_rows_to_reduce(T, 2)
     Kf = _as_f16_heads(K)
     heads = [_k_emit(Kf[0, h], plan) for h in range(H)]
     n2p, n4p, n8o = plan.padded
@@ -274,9 +286,11 @@ def pack_k_mixed_per_head(K: Tensor, k_bits_ph: Tensor):
     sub4 = _seg_padded_len(m4, 2) // 2
     plans = [_plan_k_channels(rows[h], sub2 or None, sub4 or None, m8 or None, tuple(n_h[h]))
              for h in range(H)]
+    Dp = 4 * sub2 + 2 * sub4 + m8
+    if Dp > 0:
+        _require_rows_to_reduce(T, 2)
     Kf = _as_f16_heads(K)
     heads = [_k_emit(Kf[0, h], plans[h]) for h in range(H)]
-    Dp = 4 * sub2 + 2 * sub4 + m8
 
     def stack(i, width):
         if width == 0:

@@ -189,6 +189,26 @@ def test_contract_violations_and_degenerate_inputs():
     # zero kept channels
     out = packing.pack_k_mixed(K, torch.zeros(8, dtype=torch.long))
     assert out[0] is None and out[1] is None and out[2] is None and out[3].shape == (1, 2, 1, 0)
+    # K channels over zero rows: the quantizer's minimum does not exist (amin at packing.py:153 raises)
+    none = K[:, :, :0]
+    with pytest.raises(IndexError):
+        packing.quantize_and_pack(none, 4, dim=2)
+    with pytest.raises(IndexError):
+        packing.pack_k_mixed(none, torch.full((8,), 4))
+    with pytest.raises(IndexError):
+        packing.pack_k_mixed_per_head(none, torch.full((2, 8), 4))
+    assert packing.pack_k_mixed(none, torch.zeros(8, dtype=torch.long))[3].shape == (1, 2, 1, 0)
+    assert packing.quantize_and_pack(none, 4, dim=3)[0].shape == (1, 2, 0, 8)
+    # a layer in which no head keeps a token ends in that call (packing.py:1186-1221), so it is refused
+    # like the oracle refuses it; without kept channels there is nothing to quantize and it passes
+    K128, V128 = torch.randn(1, 2, 6, 128, device=DEV).half(), torch.randn(1, 2, 6, 128, device=DEV).half()
+    nothing = torch.zeros(2, 6, dtype=torch.long)
+    with pytest.raises(IndexError):
+        packing.pack_layer_per_head(K128, V128, nothing, torch.full((2, 128), 4), 2)
+    with pytest.raises(IndexError):
+        O.pack_layer_per_head(t2n(K128), t2n(V128), nothing.numpy(), np.full((2, 128), 4), 2)
+    pl, nvo = packing.pack_layer_per_head(K128, V128, nothing, torch.zeros(2, 128, dtype=torch.long), 2)
+    assert pl.T_eff == 0 and pl.T_eff_k == 0 and nvo is None
 
 
 @pytest.mark.parametrize("cfg_idx,ctx", [(0, 512), (1, 700), (2, 384)])

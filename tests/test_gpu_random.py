@@ -4,7 +4,10 @@ heads per KV head.  The whole-layer packer is compared with the call-for-call co
 bit; the composition is pinned to the oracle and the golden vectors elsewhere), the fused decode
 path (GPU packer -> streaming cache -> fused kernel) with the oracle's attention over the oracle's
 own packing of the same inputs, and so are the reference-layout entry points (K scores, the
-caller's masked softmax, V sum) with per-head K allocations that differ in their class sizes."""
+caller's masked softmax, V sum) with per-head K allocations that differ in their class sizes.  The
+prefill-time selection (knapsack rows; pooling, both allocations and the packer as one call) is
+compared bit for bit with the oracle over random budgets, option sets, pooling windows and score
+rows with ties, zeros and constant values."""
 import dataclasses
 
 import numpy as np
@@ -12,10 +15,12 @@ import pytest
 import torch
 
 from oracle import rdkv_oracle as O
-from rdkv_amd import packing, stream_cache
+from oracle import select_oracle as S
+from rdkv_amd import knapsack_solver as ks
+from rdkv_amd import obkv_fast, packing, stream_cache
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
-from tests.gpu_util import DEV, require_gpu
+from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -75,8 +80,8 @@ def test_whole_layer_packer_random_layouts(block):
         what = f"block {block} case {case}: H={H} G={G} T={T}"
         try:
             exp, exp_n = packing._pack_layer_per_head_composed(K, V, vb, kb, G)
-        except (AssertionError, ValueError):            # a layout the composition refuses: so must the packer
-            with pytest.raises((AssertionError, ValueError)):
+        except (AssertionError, ValueError, IndexError):            # a layout the composition refuses: so must the packer
+            with pytest.raises((AssertionError, ValueError, IndexError)):
                 packing.pack_layer_per_head(K, V, vb, kb, G)
             continue
         got, got_n = packing.pack_layer_per_head(K, V, vb, kb, G)
@@ -121,7 +126,7 @@ def test_fused_attention_random_workloads(block):
             q = torch.from_numpy(rng.standard_normal((H_q, 128)).astype(np.float32)).half()
             try:
                 ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
-            except (AssertionError, ValueError):        # a layer the reference's packer refuses (nothing kept)
+            except (AssertionError, ValueError, IndexError):        # a layer the reference's packer refuses (nothing kept)
                 packed = None
                 break
             out, lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
@@ -179,7 +184,7 @@ def test_reference_layout_entry_points_random_layers(block):
         what = f"block {block} case {case}: H_kv={H_kv} G={G} T={T} kept channels {keep} magnitude {scale}"
         try:
             ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
-        except (AssertionError, ValueError):
+        except (AssertionError, ValueError, IndexError):
             continue
         exp, lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
         pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
@@ -194,3 +199,87 @@ def test_reference_layout_entry_points_random_layers(block):
         if rows.any():
             err = float(np.abs(out[rows] - exp[rows]).max()) / max(1.0, float(np.abs(exp[rows]).max()))
             assert err < (4e-3 if scale > 1 else 2e-3), f"{what}: output error {err:.3e}"
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_knapsack_random_rows(block):
+    """100 batches per block through knapsack_bit_allocation_batched (knapsack_solver.py:121-248):
+    1 to 11 rows of 1 to 20 000 scores, budgets from 0.05 to 17 bits, six option sets, 1 to 60
+    bisection rounds, three tolerances."""
+    option_sets = [None, (0, 2, 4, 8), (2, 4, 8, 16), (0, 2, 4, 8, 16), (0, 4), (2, 8)]
+    for case in range(100):
+        rng = np.random.default_rng(50000 + 1000 * block + case)
+        B = int(rng.integers(1, 12))
+        T = int(rng.choice([1, 2, 7, 63, 64, 65, 128, 1000, 1024, 1025, 4097, 20000]))
+        kind = int(rng.integers(0, 5))
+        s = np.exp(rng.standard_normal((B, T)) * rng.uniform(0.2, 3.0) + rng.uniform(-4, 4)).astype(np.float32)
+        if kind == 1:
+            s = np.round(s, 1).astype(np.float32)                           # many equal scores
+        elif kind == 2:
+            s[rng.random((B, T)) < 0.5] = 0.0
+        elif kind == 3:
+            s[:] = s[:, :1]                                                 # constant rows
+        elif kind == 4:
+            s[int(rng.integers(0, B))] = 0.0
+        budget = rng.uniform(0.05, 17.0, size=B).astype(np.float32)
+        opts = option_sets[int(rng.integers(0, 6))]
+        eps = S.DEFAULT_EPSILON_V if rng.random() < 0.5 else S.DEFAULT_EPSILON_K
+        rounds, tol = int(rng.choice([40, 5, 1, 60])), float(rng.choice([0.01, 0.001, 0.1]))
+        exp = S.knapsack_bit_allocation_batched(s, budget, epsilon=eps, bit_options=opts, max_iters=rounds, tol=tol)
+        got = ks.knapsack_bit_allocation_batched(
+            to_dev(s), to_dev(budget), epsilon=eps, max_iters=rounds, tol=tol,
+            bit_options=None if opts is None else torch.tensor(opts, dtype=torch.float32))
+        assert np.array_equal(t2n(got), exp), (
+            f"block {block} case {case}: B={B} T={T} kind={kind} options={opts} rounds={rounds} tol={tol}")
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_selection_random_layers(block):
+    """60 layers per block through _perhead_select_and_pack (obkv_fast.py:899-1186): every field of
+    the packed layer, the fp16-kept rows and the retained allocation against the oracle's selection
+    followed by the oracle's packer; a layer that the oracle refuses (no head keeps a token, so the
+    K quantizer has no row to reduce over) must be refused."""
+    for case in range(60):
+        rng = np.random.default_rng(60000 + 1000 * block + case)
+        H, G, D = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4])), 128
+        T = int(rng.choice([40, 64, 100, 257, 777, 1500, 3000]))
+        budget, ratio = int(rng.choice([8, 33, 64, 100, 400])), float(rng.choice([0.2, 0.35, 0.5, 0.6, 0.8]))
+        k_opts = [(0, 2, 4, 8), (2, 4, 8, 16), (0, 2, 4, 8, 16)][int(rng.integers(0, 3))]
+        window = int(rng.choice([1, 3, 7, 13]))
+        padding, pool = str(rng.choice(["reflect", "zero"])), str(rng.choice(["avg", "max"]))
+        K = (rng.standard_normal((1, H, T, D)) * (1 + 3 * rng.random((1, H, 1, D)))).astype(np.float16)
+        V = rng.standard_normal((1, H, T, D)).astype(np.float16)
+        ls = np.exp(rng.standard_normal((H, T)) * rng.uniform(0.5, 2.5)).astype(np.float32)
+        if rng.random() < 0.2:
+            ls[int(rng.integers(0, H))] = 0.0                               # a head that keeps nothing
+        cs = np.exp(rng.standard_normal((H, D))).astype(np.float32)
+        what = (f"block {block} case {case}: H={H} G={G} T={T} budget={budget} ratio={ratio} "
+                f"K options {k_opts} pooling {window}/{padding}/{pool}")
+
+        def run():
+            return obkv_fast._perhead_select_and_pack(
+                to_dev(K), to_dev(V), to_dev(ls), torch.from_numpy(cs), gqa_factor=G, token_budget=budget,
+                k_budget_ratio=ratio, obs_window=32, pool_kernel_size=window, pool_padding=padding,
+                pool_type=pool, v_bit_options=None, k_bit_options=torch.tensor(k_opts, dtype=torch.float32),
+                eps_V=ks.DEFAULT_EPSILON_V, eps_K=ks.DEFAULT_EPSILON_K, retain_allocation_metadata=True)
+
+        _, vb, kb, _ = S.select_joint(ls, cs, head_dim=D, token_budget=budget, k_budget_ratio=ratio,
+                                      pool_kernel_size=window, pool_padding=padding, pool_type=pool,
+                                      k_bit_options=k_opts)
+        try:
+            exp_layer, exp_v16 = O.pack_layer_per_head(K, V, vb, kb, G)
+        except IndexError:
+            with pytest.raises(IndexError):
+                run()
+            continue
+        layer, new_v, t_eff = run()
+        try:
+            assert_layers_equal(layer, exp_layer, skip=("allocation_v_bits", "allocation_k_bits"))
+        except AssertionError as e:
+            raise AssertionError(f"{what}: {e}") from None
+        assert t_eff == exp_layer.T_eff, what
+        assert (new_v is None) == (exp_v16 is None), what
+        if exp_v16 is not None:
+            assert_bits_equal(t2n(new_v), exp_v16)
+        assert np.array_equal(t2n(layer.allocation_v_bits), vb.astype(np.int16)), what
+        assert np.array_equal(t2n(layer.allocation_k_bits), kb.astype(np.int16)), what

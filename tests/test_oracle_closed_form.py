@@ -71,6 +71,12 @@ def test_quantizer_special_cases():
     x = np.array([0.0, 3.0, 0.5, 1.5, 2.5], np.float16).reshape(1, 1, 1, 5)
     q, _, _ = O.quantize_and_pack(x, 2, 3)
     assert q.reshape(-1).tolist() == [0, 3, 0, 2, 2]
+    # no element to reduce over: torch's amin (packing.py:153) raises IndexError; other empty dims pass
+    with pytest.raises(IndexError):
+        O.quantize_and_pack(np.empty((1, 1, 0, 4), np.float16), 4, 2)
+    assert O.quantize_and_pack(np.empty((1, 1, 0, 4), np.float16), 4, 3)[0].shape == (1, 1, 0, 4)
+    with pytest.raises(IndexError):
+        O.pack_k_mixed(np.empty((1, 1, 0, 8), np.float16), np.full(8, 4))
     # 8-bit NMSE sanity of the reference's own smoke check (knapsack_solver.py:537-548)
     rng = np.random.default_rng(0)
     v = rng.standard_normal((1, 8, 512, 128)).astype(np.float16)
