@@ -248,9 +248,11 @@ RDKV_API int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, 
                                         const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
                                         int H_kv, int n8, int max_tiles, uint8_t *blob, void *stream) {
   RDKV_REQUIRE(H_kv > 0 && units && src_slot && n_slots_max > 0, "rdkv_stream_relayout_layer: bad arguments");
-  RDKV_REQUIRE(perm && kscale_f16 && kzp_f16, "rdkv_stream_relayout_layer: null channel tables");
   RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
                "rdkv_stream_relayout_layer: bad padded channel counts (%d,%d)", n2p, n4p);
+  // a layer without kept K channels has no channel tables, and no slot that would read them
+  RDKV_REQUIRE((perm && kscale_f16 && kzp_f16) || (n2p == 0 && n4p == 0 && n8 == 0),
+               "rdkv_stream_relayout_layer: null channel tables");
   SrcLayer S;
   S.K2 = K2; S.K4 = K4; S.K8 = K8;
   S.k2_sh = k2_stride_h; S.k2_st = k2_stride_t;

@@ -120,7 +120,7 @@ def _quantize_rows(x2d: Tensor, n_bits: int, pack: bool, row_idx: Optional[Tenso
 
 def _require_rows_to_reduce(n: int, dim: int) -> None:
     """The quantizer's minimum over an empty dimension does not exist: torch's ``amin`` raises
-    IndexError for it (packing.py:153), which is what a caller of the reference sees when it packs
+    IndexError for it (packing.py:156), which is what a caller of the reference sees when it packs
     K channels over zero rows (packing.py:304-351)."""
     if n == 0:
         raise IndexError(f"amin(): Expected reduction dim {dim} to have non-zero size.")
@@ -132,7 +132,7 @@ def quantize_and_pack(x: Tensor, n_bits: int, dim: int) -> Tuple[Tensor, Tensor,
     scale = max((max-min)/(2^b-1), 1e-8); zp = round(clamp(-min/scale)); codes =
     round(clamp(x/scale + zp)); returns (uint8 codes shaped like x, fp16 scale, fp16 zp
     with keepdim).  Codes use the fp32 scale, the returned scale is its fp16 rounding.
-    A reduction over no element raises IndexError, as the reference's ``amin`` does (packing.py:153).
+    A reduction over no element raises IndexError, as the reference's ``amin`` does (packing.py:156).
     """
     _lib.require_device(x)
     dim = dim % x.dim()

@@ -49,11 +49,15 @@ def test_trizone_attention_three_zones(cfg_idx, ctx, n_new):
 
 
 def test_zone_c_only_layer():
-    """A layer whose prompt tokens were all evicted: attention runs over zone C alone."""
+    """A layer whose prompt tokens were all evicted: attention runs over zone C alone.  The packer
+    accepts such a layer only without kept K channels (with them the reference's quantizer reduces
+    over zero rows and raises, packing.py:156)."""
     cfg = synth.scaled(synth.CONFIGS[1], context=64, layers=1)
     K, V, q = synth.layer_data(cfg, 0, DEV)
     vb = torch.zeros(cfg.H_kv, 64, dtype=torch.long)
-    kb = torch.full((cfg.H_kv, 128), 4)
+    with pytest.raises(IndexError):
+        packing.pack_layer_per_head(K, V, vb, torch.full((cfg.H_kv, 128), 4), cfg.G)
+    kb = torch.zeros(cfg.H_kv, 128, dtype=torch.long)
     pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, cfg.G)
     assert pl.T_eff_k == 0 and nvo is None
     Kn = torch.randn(cfg.H_kv, 3, 128, device=DEV)
@@ -64,6 +68,36 @@ def test_zone_c_only_layer():
     exp = torch.bmm(torch.softmax(s, -1), Vn).reshape(cfg.H_q, 128)
     assert float((fused - exp).abs().max()) < 1e-5
     assert bool(torch.isfinite(fused).all())
+
+
+def test_layer_without_kept_k_channels():
+    """Every K channel pruned, tokens kept: all scores are zero (the reference's K entry point
+    zero-fills, triton_k_kernel.py:1265-1268), so every kept token weighs the same and the
+    log-sum-exp is the logarithm of the head's token count - through the reference-layout entry
+    points and through the streaming cache, against the oracle."""
+    rng = np.random.default_rng(5)
+    H, T, G = 2, 150, 2
+    K = torch.from_numpy(rng.standard_normal((1, H, T, 128)).astype(np.float16))
+    V = torch.from_numpy(rng.standard_normal((1, H, T, 128)).astype(np.float16))
+    vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8, 16]), size=(H, T)))
+    kb = torch.zeros(H, 128, dtype=torch.long)
+    q = torch.from_numpy(rng.standard_normal((H * G, 128)).astype(np.float16))
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+    exp, exp_lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+    np.testing.assert_allclose(exp_lse, np.log(np.repeat((vb > 0).sum(1).numpy(), G)), rtol=1e-6)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G)
+    assert pl.K_2bit is None and pl.K_4bit is None and pl.K_8bit is None and pl.K_ch_scale.shape[-1] == 0
+    from rdkv_amd import triton_k_kernel as kk, triton_v_kernel as vk
+    scores = kk.k_mixed_qk_dot(q.to(DEV).float(), pl, pl.T_eff_k)
+    assert float(scores.abs().max()) == 0.0
+    w = torch.softmax(scores + pl.softmax_mask, dim=-1)
+    out = vk.v_dequant_weighted_sum_dispatch(w, pl, V16=nvo, n_v16_per_head=pl.n_v16_per_head, max_T_v=pl.T_eff)
+    attn_close(t2n(out), exp, "reference-layout entry points")
+    cache = stream_cache.build_stream_cache([(pl, nvo)], G)
+    assert cache.max_row_dwords == 0
+    fused, lse = stream_cache.decode_attn_fused(cache, q.to(DEV))
+    attn_close(t2n(fused.float()), exp, "fused")
+    np.testing.assert_allclose(t2n(lse.float()), exp_lse, atol=1e-5)
 
 
 @pytest.mark.parametrize("name", ["perhead_d128_a", "shared_layout"])

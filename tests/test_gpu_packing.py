@@ -189,7 +189,7 @@ def test_contract_violations_and_degenerate_inputs():
     # zero kept channels
     out = packing.pack_k_mixed(K, torch.zeros(8, dtype=torch.long))
     assert out[0] is None and out[1] is None and out[2] is None and out[3].shape == (1, 2, 1, 0)
-    # K channels over zero rows: the quantizer's minimum does not exist (amin at packing.py:153 raises)
+    # K channels over zero rows: the quantizer's minimum does not exist (amin at packing.py:156 raises)
     none = K[:, :, :0]
     with pytest.raises(IndexError):
         packing.quantize_and_pack(none, 4, dim=2)

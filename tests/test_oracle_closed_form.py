@@ -71,7 +71,7 @@ def test_quantizer_special_cases():
     x = np.array([0.0, 3.0, 0.5, 1.5, 2.5], np.float16).reshape(1, 1, 1, 5)
     q, _, _ = O.quantize_and_pack(x, 2, 3)
     assert q.reshape(-1).tolist() == [0, 3, 0, 2, 2]
-    # no element to reduce over: torch's amin (packing.py:153) raises IndexError; other empty dims pass
+    # no element to reduce over: torch's amin (packing.py:156) raises IndexError; other empty dims pass
     with pytest.raises(IndexError):
         O.quantize_and_pack(np.empty((1, 1, 0, 4), np.float16), 4, 2)
     assert O.quantize_and_pack(np.empty((1, 1, 0, 4), np.float16), 4, 3)[0].shape == (1, 1, 0, 4)
