@@ -1032,7 +1032,11 @@ dequant_f16_kernel(const uint8_t *__restrict__ packed, int64_t rows, int ncols,
     q = (b >> (2 * (c / n))) & 3u;
   }
   const int64_t pi = per_row ? r : c;
-  const float v = __fmul_rn(__fsub_rn((float)q, __half2float(zp[pi])), __half2float(scale[pi]));
+  float v = __fmul_rn(__fsub_rn((float)q, __half2float(zp[pi])), __half2float(scale[pi]));
+  // The product must exist as an fp32 value before it is rounded: left alone, the compiler merges
+  // the multiplication and the conversion into one fused multiply-add with +0 as the addend, which
+  // turns (code - zp) * 0 = -0 (a constant negative row or column: code 0, zp = qmax, scale 0) into +0.
+  asm volatile("" : "+v"(v));
   out[r * out_row_stride + c] = __float2half_rn(v);
 }
 

@@ -211,6 +211,32 @@ def test_contract_violations_and_degenerate_inputs():
     assert pl.T_eff == 0 and pl.T_eff_k == 0 and nvo is None
 
 
+def test_dequantizing_constant_negative_values_keeps_the_sign_of_zero():
+    """A constant negative column (K) or row (V) quantizes to code 0, zero point qmax and an fp16
+    scale of 0, so (code - zp) * scale is -0.0 in the reference's fp32 arithmetic
+    (packing.py:629-651, :1427-1444) and stays -0.0 through .half(): the same bits here."""
+    K = torch.full((1, 1, 5, 8), -0.75, device=DEV).half()
+    K[0, 0, :, 4:] = 0.75
+    Vs = torch.randn(1, 1, 5, 8, device=DEV).half()
+    for bits in (2, 4, 8):
+        pl, _, _ = packing.build_packed_layer(K, Vs, torch.full((5,), 4), torch.full((8,), bits))
+        opl, _, _ = O.build_packed_layer(t2n(K), t2n(Vs), np.full(5, 4), np.full(8, bits))
+        exp = O.unpack_k_mixed(opl, 8)
+        assert np.signbit(exp[0, 0, :, :4]).all() and not np.signbit(exp[0, 0, :, 4:]).any() and not exp.any()
+        assert_bits_equal(t2n(packing.unpack_k_mixed(pl, D=8)), exp)
+        V = torch.full((1, 1, 3, 128), -0.5, device=DEV).half()
+        V[0, 0, 1] = 0.5
+        q, sc, zp = packing.quantize_and_pack(V, bits, dim=3)
+        pack = {2: bitpack.transfer_8bit_to_2bit_batchwise, 4: bitpack.transfer_8bit_to_4bit_batchwise,
+                8: lambda x: x}[bits]
+        got = packing.unpack_v_segment(pack(q.clone()), sc, zp, bits)
+        oq, osc, ozp = O.quantize_and_pack(t2n(V), bits, 3)
+        opack = {2: O.transfer_8bit_to_2bit_batchwise, 4: O.transfer_8bit_to_4bit_batchwise, 8: lambda x: x}[bits]
+        exp_v = O.unpack_v_segment(opack(oq.copy()), osc, ozp, bits)
+        assert np.signbit(exp_v[0, 0, 0]).all() and not np.signbit(exp_v[0, 0, 1]).any()
+        assert_bits_equal(t2n(got), exp_v)
+
+
 @pytest.mark.parametrize("cfg_idx,ctx", [(0, 512), (1, 700), (2, 384)])
 def test_config_shaped_layer_vs_oracle(cfg_idx, ctx):
     """Per-head packing of a configuration-shaped layer (reduced context) is bit-identical to the oracle."""

@@ -18,6 +18,7 @@ from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
 from rdkv_amd import obkv_fast, packing, stream_cache
+from rdkv_amd import trizone_decompress as tz
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
 from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev
@@ -283,3 +284,42 @@ def test_selection_random_layers(block):
             assert_bits_equal(t2n(new_v), exp_v16)
         assert np.array_equal(t2n(layer.allocation_v_bits), vb.astype(np.int16)), what
         assert np.array_equal(t2n(layer.allocation_k_bits), kb.astype(np.int16)), what
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_dequantize_back_random_layers(block):
+    """80 layers per block through the dequantize-then-attend route's unpackers (unpack_k_mixed,
+    packing.py:581-709; _unpack_v_perhead, trizone_decompress.py:91-144; unpack_trizone_to_past_kv,
+    :185-195): the fp16 bits of the oracle's, signed zeros of constant negative channels (layers of
+    one token) included."""
+    for case in range(80):
+        rng = np.random.default_rng(70000 + 1000 * block + case)
+        H, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4]))
+        T = int(rng.choice([1, 1, 5, 63, 64, 65, 130, 400, 900, 1700]))
+        vb = rng.choice(np.array([0, 2, 4, 8, 16]), size=(H, T), p=_class_probabilities(rng, 5))
+        kb = rng.choice(np.array([0, 2, 4, 8, 16]), size=(H, 128), p=_class_probabilities(rng, 5))
+        scale = float(rng.choice([1.0, 0.01, 30.0]))
+        K = (rng.standard_normal((1, H, T, 128)) * scale + rng.choice([0.0, 0.75])).astype(np.float16)
+        V = (rng.standard_normal((1, H, T, 128)) * scale).astype(np.float16)
+        if rng.random() < 0.3:
+            V[0, :, : max(1, T // 4)] = -0.5                                # constant negative rows
+        what = f"block {block} case {case}: H={H} G={G} T={T} magnitude {scale}"
+        try:
+            ora, ora_nvo = O.pack_layer_per_head(K, V, vb, kb, G)
+        except (IndexError, AssertionError, ValueError):
+            continue
+        pl, nvo = packing.pack_layer_per_head(torch.from_numpy(K).to(DEV), torch.from_numpy(V).to(DEV),
+                                              torch.from_numpy(vb), torch.from_numpy(kb), G)
+        exp_v = O._unpack_v_perhead(ora, head_dim=128)
+        assert_bits_equal(t2n(tz._unpack_v_perhead(pl, head_dim=128)), exp_v)
+        cache = packing.TriZoneCache(packed=(pl,), new_v_only=[nvo], new_both_k=[None], new_both_v=[None],
+                                     original_seq_len=T)
+        (K_full, V_full), = tz.unpack_trizone_to_past_kv(cache, head_dim=128)
+        if ora.T_eff_k > 0:
+            exp_k = O.unpack_k_mixed(ora, 128)
+            assert_bits_equal(t2n(packing.unpack_k_mixed(pl, D=128)), exp_k)
+            assert_bits_equal(t2n(K_full), exp_k)
+        tv = int(pl.T_eff)
+        assert_bits_equal(t2n(V_full[:, :, :tv]), exp_v.reshape(1, H, tv, 128))
+        if nvo is not None:
+            assert_bits_equal(t2n(V_full[:, :, tv:]), ora_nvo)
