@@ -105,7 +105,8 @@ def _quantize_rows(x2d: Tensor, n_bits: int, pack: bool, row_idx: Optional[Tenso
                    rows: Optional[int] = None):
     """x2d: fp16 [R, D] with unit channel stride.  Returns (codes|packed [rows, *], scale, zp [rows])."""
     dev = _lib.require_device(x2d)
-    assert x2d.dtype == torch.float16 and x2d.stride(-1) == 1
+    # (the stride of a dimension of size one carries no information and may be anything)
+    assert x2d.dtype == torch.float16 and (x2d.shape[-1] == 1 or x2d.stride(-1) == 1)
     D = x2d.shape[1]
     rows = x2d.shape[0] if rows is None else rows
     width = D * n_bits // 8 if pack else D

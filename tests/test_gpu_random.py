@@ -17,7 +17,7 @@ import torch
 from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
-from rdkv_amd import obkv_fast, packing, stream_cache
+from rdkv_amd import bitpack, obkv_fast, packing, stream_cache
 from rdkv_amd import trizone_decompress as tz
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
@@ -323,3 +323,83 @@ def test_dequantize_back_random_layers(block):
         assert_bits_equal(t2n(V_full[:, :, :tv]), exp_v.reshape(1, H, tv, 128))
         if nvo is not None:
             assert_bits_equal(t2n(V_full[:, :, tv:]), ora_nvo)
+
+
+def _same_tuple(got, exp, what):
+    assert len(got) == len(exp), what
+    for i, (g, e) in enumerate(zip(got, exp)):
+        if e is None:
+            assert g is None, f"{what}[{i}]"
+        elif isinstance(e, tuple):
+            assert tuple(int(v) for v in g) == tuple(int(v) for v in e), f"{what}[{i}]"
+        else:
+            assert_bits_equal(t2n(g), e, f"{what}[{i}]")
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_packer_building_blocks_random(block):
+    """100 draws per block for each building block of the packer, bit for bit against the oracle:
+    the four bitpack transfers on tensors of rank 1-4 (empty leading dimensions and non-contiguous
+    views included; the packing transfers overwrite the head of their input as bitpack.py:17 does),
+    quantize_and_pack over any dimension of a rank 1-4 tensor (a dimension of one element included),
+    pack_k_mixed, pack_k_mixed_per_head, pack_v_segments and build_packed_layer (shared and
+    per-head K allocation) at head dimensions 8-256."""
+    bits5 = np.array([0, 2, 4, 8, 16])
+    for case in range(100):
+        rng = np.random.default_rng(80000 + 1000 * block + case)
+        what = f"block {block} case {case}"
+        lead = tuple(int(v) for v in rng.integers(0, 5, size=int(rng.integers(0, 4))))
+        n_last = int(rng.choice([4, 8, 12, 32, 128, 260]))
+        for limit, fn, inv in ((4, "transfer_8bit_to_2bit_batchwise", "transfer_2bit_to_8bit_batchwise"),
+                               (16, "transfer_8bit_to_4bit_batchwise", "transfer_4bit_to_8bit_batchwise")):
+            x = rng.integers(0, limit, size=lead + (n_last,), dtype=np.uint8)
+            x_exp = x.copy()
+            exp = getattr(O, fn)(x_exp)
+            x_dev = to_dev(x)
+            if rng.random() < 0.4 and x_dev.dim() >= 2:
+                wide = torch.zeros(*x_dev.shape[:-1], 2 * n_last, dtype=torch.uint8, device=DEV)
+                wide[..., :n_last] = x_dev
+                x_dev = wide[..., :n_last]
+            got = getattr(bitpack, fn)(x_dev)
+            assert_bits_equal(t2n(got), exp, f"{what}: {fn} {lead}")
+            assert_bits_equal(t2n(x_dev), x_exp, f"{what}: input after {fn}")
+            back = getattr(bitpack, inv)(got)
+            assert back.dtype == (torch.float32 if limit == 16 else torch.uint8)
+            assert_bits_equal(t2n(back), getattr(O, inv)(exp), f"{what}: {inv}")
+        rank = int(rng.integers(1, 5))
+        shape = tuple(int(v) for v in rng.integers(1, 9, size=rank))
+        dim, bits = int(rng.integers(-rank, rank)), int(rng.choice([2, 4, 8]))
+        x = (rng.standard_normal(shape) * float(rng.choice([1.0, 1e-3, 100.0])) + float(rng.choice([0, 3.0]))).astype(np.float16)
+        if rng.random() < 0.3:
+            x = np.round(x)
+        _same_tuple(packing.quantize_and_pack(to_dev(x), bits, dim), O.quantize_and_pack(x, bits, dim),
+                    f"{what}: quantize_and_pack {shape} dim {dim} {bits} bit")
+        D, H = int(rng.choice([8, 16, 32, 64, 96, 128, 256])), int(rng.integers(1, 4))
+        T = int(rng.choice([1, 2, 7, 64, 65, 200]))
+        what += f": D={D} H={H} T={T}"
+        K = (rng.standard_normal((1, H, T, D)) * 2).astype(np.float16)
+        V = rng.standard_normal((1, H, T, D)).astype(np.float16)
+        p_k = _class_probabilities(rng, 5)
+        kb, kb_heads = rng.choice(bits5, size=D, p=p_k), rng.choice(bits5, size=(H, D), p=p_k)
+        _same_tuple(packing.pack_k_mixed(to_dev(K), torch.from_numpy(kb)), O.pack_k_mixed(K, kb), f"{what} pack_k_mixed")
+        _same_tuple(packing.pack_k_mixed_per_head(to_dev(K), torch.from_numpy(kb_heads)),
+                    O.pack_k_mixed_per_head(K, kb_heads), f"{what} pack_k_mixed_per_head")
+        p_v = rng.random(3) + 0.01
+        vb3 = rng.choice(np.array([2, 4, 8]), size=T, p=p_v / p_v.sum())
+        _same_tuple(packing.pack_v_segments(to_dev(V), torch.from_numpy(vb3)), O.pack_v_segments(V, vb3),
+                    f"{what} pack_v_segments")
+        vb = rng.choice(bits5, size=T, p=_class_probabilities(rng, 5))
+        for k_bits in (kb, kb_heads):
+            kw = dict(gqa_factor=2) if k_bits.ndim == 2 else {}
+            args = (to_dev(K), to_dev(V), torch.from_numpy(vb), torch.from_numpy(k_bits))
+            exp_layer, exp_tk, exp_v16 = O.build_packed_layer(K, V, vb, k_bits, **kw)
+            layer, tk, v16 = packing.build_packed_layer(*args, **kw)
+            try:
+                assert_layers_equal(layer, exp_layer)
+            except AssertionError as e:
+                raise AssertionError(f"{what} build_packed_layer: {e}") from None
+            assert tk == exp_tk and (v16 is None) == (exp_v16 is None), what
+            if exp_v16 is not None:
+                assert_bits_equal(t2n(v16), exp_v16)
+            if exp_tk > 0:
+                assert_bits_equal(t2n(packing.unpack_k_mixed(layer, D=D)), O.unpack_k_mixed(exp_layer, D))
