@@ -1125,11 +1125,12 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
       float s = 0.0f;     // over the group's heads in head order, as rdkv_tail_scores sums them
 #pragma unroll
       for (int h = 0; h < G; ++h) {
+#pragma clang fp contract(off)   // the stored weight is what is summed: no fusing with the product
         float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
         const float inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
         const float w = expf(row[t] - fin_m[h]) * inv;
         row[t] = w;
-        s = __fadd_rn(s, w);   // the stored weight is what is summed: no fusing with the product above
+        s = s + w;
       }
       // online block scores of blockwise decode (blockwise_decode.py:2085-2109): the query's weights
       // on its own block, and on the first block when the query belongs to the second

@@ -61,9 +61,13 @@ __device__ __forceinline__ void rdkv_store_from_float(void *p, int dtype, int64_
 }
 
 // out_lo = lo*c - hi*s, out_hi = hi*c + lo*s with every operation rounded on its own
-// (triton_rope.py:68-70; its PyTorch statement :127-131)
+// (triton_rope.py:68-70; its PyTorch statement :127-131).  The pragma is what keeps the products
+// and the sum apart wherever this is inlined: HIP's __fmul_rn / __fadd_rn are plain operators, which
+// the compiler may contract into a fused multiply-add (one rounding less, another last bit).
 __device__ __forceinline__ void rdkv_rope_pair(float lo, float hi, float c, float s, float &out_lo,
                                                float &out_hi) {
-  out_lo = __fsub_rn(__fmul_rn(lo, c), __fmul_rn(hi, s));
-  out_hi = __fadd_rn(__fmul_rn(hi, c), __fmul_rn(lo, s));
+#pragma clang fp contract(off)
+  const float lc = lo * c, hs = hi * s, hc = hi * c, ls = lo * s;
+  out_lo = lc - hs;
+  out_hi = hc + ls;
 }

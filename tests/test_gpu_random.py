@@ -17,7 +17,8 @@ import torch
 from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
-from rdkv_amd import bitpack, obkv_fast, packing, stream_cache
+from rdkv_amd import bitpack, fast_decode, obkv_fast, packing, stream_cache, triton_rope
+from rdkv_amd import blockwise_decode as bw
 from rdkv_amd import trizone_decompress as tz
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
@@ -403,3 +404,85 @@ def test_packer_building_blocks_random(block):
                 assert_bits_equal(t2n(v16), exp_v16)
             if exp_tk > 0:
                 assert_bits_equal(t2n(packing.unpack_k_mixed(layer, D=D)), O.unpack_k_mixed(exp_layer, D))
+
+
+def test_rotary_embedding_random_heads():
+    """150 draws of fused_rope (triton_rope.py:36-108) in fp16, bf16 and fp32, 1-39 query and 1-9 KV
+    heads, positions up to 200 000 at two bases: the oracle's bits (two products and one sum or
+    difference, each rounded on its own - a fused multiply-add shows in the last bit of fp32)."""
+    kinds = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+    for case in range(150):
+        rng = np.random.default_rng(90000 + case)
+        kind = str(rng.choice(list(kinds)))
+        dt = kinds[kind]
+        H_q, H_kv = int(rng.integers(1, 40)), int(rng.integers(1, 10))
+        q = torch.from_numpy(rng.standard_normal((H_q, 128)).astype(np.float32) * 3).to(dt)
+        k = torch.from_numpy(rng.standard_normal((H_kv, 128)).astype(np.float32) * 3).to(dt)
+        ang = float(rng.integers(0, 200000)) / (float(rng.choice([10000.0, 500000.0])) ** (np.arange(0, 128, 2) / 128))
+        cos = torch.from_numpy(np.cos(ang).astype(np.float32)).to(dt)
+        sin = torch.from_numpy(np.sin(ang).astype(np.float32)).to(dt)
+        exp_q, exp_k = O.fused_rope_ref(q.float().numpy(), k.float().numpy(), cos.float().numpy(),
+                                        sin.float().numpy(), kind)
+        q_dev, k_dev = q.to(DEV), k.to(DEV)
+        triton_rope.fused_rope(q_dev, k_dev, cos.to(DEV), sin.to(DEV))
+        what = f"case {case}: {kind} H_q={H_q} H_kv={H_kv}"
+        assert np.array_equal(q_dev.float().cpu().numpy(), exp_q.astype(np.float32)), what
+        assert np.array_equal(k_dev.float().cpu().numpy(), exp_k.astype(np.float32)), what
+
+
+def test_block_scores_random_blocks():
+    """120 draws of the blockwise scorer (blockwise_decode.py:197-253): 1-4 KV heads, 1-8 query heads
+    each, 1-1000 keys, head dimensions 64 and 128, causal or not, three dtypes, against the oracle."""
+    for case in range(120):
+        rng = np.random.default_rng(91000 + case)
+        H, G, D = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8])), int(rng.choice([64, 128]))
+        causal = bool(rng.random() < 0.5)
+        T = int(rng.choice([1, 3, 32, 37, 64, 100, 128, 300, 1000]))
+        Q = T if causal else int(rng.choice([1, 5, 32, 64, 128]))
+        dt = [torch.float16, torch.bfloat16, torch.float32][int(rng.integers(0, 3))]
+        q = (torch.from_numpy(rng.standard_normal((H * G, Q, D)).astype(np.float32)) * 1.5).to(dt)
+        k = (torch.from_numpy(rng.standard_normal((1, H, T, D)).astype(np.float32)) * 1.5).to(dt)
+        token, channel = bw._score_block(q.to(DEV), k.to(DEV), num_kv_groups=G, causal=causal)
+        exp_t, exp_c = S.score_block(q.float().numpy(), k.float().numpy(), num_kv_groups=G, causal=causal)
+        what = f"case {case}: H={H} G={G} Q={Q} T={T} D={D} causal={causal} {dt}"
+        np.testing.assert_allclose(t2n(token), exp_t, rtol=5e-5, atol=2e-6, err_msg=what)
+        np.testing.assert_allclose(t2n(channel), exp_c, rtol=2e-5, atol=1e-9, err_msg=what)
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_three_zone_attention_random_layers(block):
+    """60 layers per block with 1-200 appended fp32 tokens (fast_decode.py:1701-1784): the
+    reference-layout route and the streaming cache with zone C merged in its second launch, max-abs
+    error of the output within 2e-3 of the oracle's three-zone attention."""
+    for case in range(60):
+        rng = np.random.default_rng(92000 + 1000 * block + case)
+        H_kv, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8]))
+        T, n_new = int(rng.choice([1, 5, 64, 65, 130, 400, 900])), int(rng.choice([1, 2, 17, 64, 65, 200]))
+        vb = rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T), p=_class_probabilities(rng, 5))
+        keep = int(rng.choice([8, 33, 64, 128]))
+        kb = np.zeros((H_kv, 128), dtype=np.int64)
+        for h in range(H_kv):
+            kc, ch = rng.multinomial(keep, rng.dirichlet([1, 1, 1])), rng.permutation(128)
+            kb[h, ch[:kc[0]]] = 2
+            kb[h, ch[kc[0]:kc[0] + kc[1]]] = 4
+            kb[h, ch[kc[0] + kc[1]:keep]] = 8
+        K = rng.standard_normal((1, H_kv, T, 128)).astype(np.float16)
+        V = rng.standard_normal((1, H_kv, T, 128)).astype(np.float16)
+        q = rng.standard_normal((H_kv * G, 128)).astype(np.float16)
+        K_new = rng.standard_normal((H_kv, n_new, 128)).astype(np.float32)
+        V_new = rng.standard_normal((H_kv, n_new, 128)).astype(np.float32)
+        what = f"block {block} case {case}: H_kv={H_kv} G={G} T={T} appended {n_new}"
+        try:
+            ora, ora_nvo = O.pack_layer_per_head(K, V, vb, kb, G)
+        except IndexError:                                  # no head keeps a token: the packer refuses
+            continue
+        exp = O.trizone_attention_ref(q, ora, ora_nvo, K_new, V_new)
+        pl, nvo = packing.pack_layer_per_head(to_dev(K), to_dev(V), torch.from_numpy(vb), torch.from_numpy(kb), G)
+        sp = fast_decode._pre_squeeze_packed((pl,))[0]
+        q_dev, Kn, Vn = to_dev(q), to_dev(K_new), to_dev(V_new)
+        out = fast_decode.trizone_attention(q_dev, sp, nvo[0].contiguous() if nvo is not None else None,
+                                            sp.n_v16_per_head, Kn, Vn, G)
+        assert float(np.abs(t2n(out) - exp).max()) < 2e-3, what + " (reference layout)"
+        cache = stream_cache.build_stream_cache([(pl, nvo)], G)
+        fused = fast_decode.trizone_attention_fused(cache, q_dev, [Kn], [Vn], G)
+        assert float(np.abs(t2n(fused) - exp).max()) < 2e-3, what + " (streaming cache)"
