@@ -17,12 +17,13 @@ import torch
 from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
-from rdkv_amd import bitpack, fast_decode, obkv_fast, packing, stream_cache, triton_rope
+from rdkv_amd import _lib, bitpack, fast_decode, obkv_fast, packing, stream_cache, triton_rope
 from rdkv_amd import blockwise_decode as bw
 from rdkv_amd import trizone_decompress as tz
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
-from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev
+from tests.gpu_util import (DEV, assert_bits_equal, assert_layers_equal, fused_both, lse_merge, require_gpu, t2n,
+                            to_dev)
 
 pytestmark = pytest.mark.gpu
 
@@ -486,3 +487,92 @@ def test_three_zone_attention_random_layers(block):
         cache = stream_cache.build_stream_cache([(pl, nvo)], G)
         fused = fast_decode.trizone_attention_fused(cache, q_dev, [Kn], [Vn], G)
         assert float(np.abs(t2n(fused) - exp).max()) < 2e-3, what + " (streaming cache)"
+
+
+def _random_entry(rng, H_kv, G, T):
+    """One packed layer by the oracle and by the GPU packer from the same random inputs."""
+    p = rng.random(5) * (rng.random(5) < 0.75)
+    if p[1:].sum() == 0:
+        p[int(rng.integers(1, 5))] = 1.0
+    vb = rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T), p=p / p.sum())
+    keep = int(rng.choice([8, 33, 64, 100, 128]))
+    kb = np.zeros((H_kv, 128), dtype=np.int64)
+    for h in range(H_kv):
+        kc, ch = rng.multinomial(keep, rng.dirichlet([1, 1, 1])), rng.permutation(128)
+        kb[h, ch[:kc[0]]] = 2
+        kb[h, ch[kc[0]:kc[0] + kc[1]]] = 4
+        kb[h, ch[kc[0] + kc[1]:keep]] = 8
+    K = rng.standard_normal((1, H_kv, T, 128)).astype(np.float16)
+    V = rng.standard_normal((1, H_kv, T, 128)).astype(np.float16)
+    return (O.pack_layer_per_head(K, V, vb, kb, G),
+            packing.pack_layer_per_head(to_dev(K), to_dev(V), torch.from_numpy(vb), torch.from_numpy(kb), G))
+
+
+def _check_against_merged_oracle(cache, q, q_np, oracle_entries, rows_of, H_q, what):
+    """Fused attention over ``cache`` (two launches and one launch: same bits) against the oracle's
+    attention per source, merged into the exact softmax over each output group's sources."""
+    out, lse = fused_both(cache, q)
+    o, l = t2n(out), t2n(lse)
+    for r in range(max(rows_of) + 1):
+        rows = slice(r * H_q, (r + 1) * H_q)
+        parts = []
+        for entry, row in zip(oracle_entries, rows_of):
+            if row == r:
+                po, pl = O.decode_attn_ref(q_np[rows], *entry)[:2]
+                empty = ~np.isfinite(pl)                                     # a head without tokens
+                parts.append((np.where(empty[:, None], 0.0, po), np.where(empty, -np.inf, pl)))
+        exp_o, exp_l = lse_merge(parts)
+        fin = np.isfinite(exp_l)
+        assert np.array_equal(np.isfinite(l[rows]), fin), f"{what}: rows without tokens, group {r}"
+        assert float(np.abs(o[rows] - np.where(np.isfinite(exp_o), exp_o, 0.0)).max()) < 2e-3, f"{what}: out, group {r}"
+        if fin.any():
+            assert float(np.abs(l[rows][fin] - exp_l[fin]).max()) < 2e-3, f"{what}: lse, group {r}"
+    return out, lse
+
+
+@pytest.mark.parametrize("block", range(2))
+def test_stream_caches_random_sources_partitions_files(block, tmp_path):
+    """40 caches per block: 1-3 output groups with 1-3 packed sources each (multi-source attention,
+    blockwise_decode.py:812-1121), a random work partition, then the same cache through the entry
+    point that allocates nothing (same bits), through a file (same bits; loaded with another
+    partition: the oracle's results) and extended by one more source."""
+    lib = _lib.load()
+    for case in range(40):
+        rng = np.random.default_rng(100000 + 1000 * block + case)
+        H_kv, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8]))
+        H_q = H_kv * G
+        n_rows = int(rng.integers(1, 4))
+        rows_of = list(range(n_rows)) + [int(rng.integers(0, n_rows)) for _ in range(int(rng.integers(0, 3)))]
+        rng.shuffle(rows_of)
+        what = f"block {block} case {case}: H_kv={H_kv} G={G} groups of the sources {rows_of}"
+        try:
+            entries = [_random_entry(rng, H_kv, G, int(rng.choice([1, 5, 63, 64, 65, 130, 400, 900, 1700])))
+                       for _ in rows_of]
+            extra = _random_entry(rng, H_kv, G, int(rng.choice([1, 16, 64, 200])))
+        except IndexError:                                  # a source in which no head keeps a token
+            continue
+        oracle_entries, packed = [e[0] for e in entries], [e[1] for e in entries]
+        q_np = rng.standard_normal((n_rows * H_q, 128)).astype(np.float16)
+        q = to_dev(q_np)
+        partition = [{}, dict(n_groups=int(rng.integers(1, 40))), dict(work_bytes=int(rng.choice([4096, 65536, 1 << 20]))),
+                     dict(groups_per_cu=2)][int(rng.integers(0, 4))]
+        cache = stream_cache.build_stream_cache(packed, G, row_of_entry=rows_of, **partition)
+        out, lse = _check_against_merged_oracle(cache, q, q_np, oracle_entries, rows_of, H_q, f"{what}, {partition}")
+        if lib.rdkv_decode_fused_workspace_bytes(cache.n_work, G) <= lib.rdkv_decode_fused_static_max_bytes():
+            out_s, lse_s = torch.full_like(out, float("nan")), torch.full_like(lse, float("nan"))
+            _lib.check(lib.rdkv_decode_fused_static(
+                None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+                _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords, q.data_ptr(), _lib.DTYPE_CODE[q.dtype],
+                q.stride(0), G, None, None, 0, out_s.data_ptr(), out_s.stride(0), lse_s.data_ptr(),
+                _lib.stream_of(q.device)))
+            assert torch.equal(out_s, out) and torch.equal(lse_s, lse), f"{what}: entry point without allocations"
+        path = str(tmp_path / f"cache_{case}.rdkv")
+        stream_cache.save_stream_cache(cache, path)
+        out_f, lse_f = stream_cache.decode_attn_fused(stream_cache.load_stream_cache(path, DEV), q)
+        assert torch.equal(out_f, out) and torch.equal(lse_f, lse), f"{what}: loaded from its file"
+        other = stream_cache.load_stream_cache(path, DEV, n_groups=int(rng.integers(1, 30)))
+        _check_against_merged_oracle(other, q, q_np, oracle_entries, rows_of, H_q, f"{what}, loaded with another partition")
+        row = int(rng.integers(0, n_rows))
+        longer = stream_cache.extend_stream_cache(cache, [extra[1]], row_of_entry=[row])
+        _check_against_merged_oracle(longer, q, q_np, oracle_entries + [extra[0]], rows_of + [row], H_q,
+                                     f"{what}, one more source in group {row}")
