@@ -2,6 +2,7 @@
 known-answer tests and the oracle, compression of a block against the oracle's selection +
 packing, and the decode-time attention over [prompt cache | compressed blocks | raw tail] against
 dense attention over the dequantized union."""
+import dataclasses
 import math
 
 import numpy as np
@@ -145,6 +146,40 @@ def test_compress_block_matches_oracle(capsys):
         assert key in event, key
     assert event["query_mode"] == "next_block" and event["logical_allocated_bits"] == sum(block.logical_bits_per_layer)
     assert len(event["slot_shape_signature"]) == L and event["slot_shape_signature"][0]["T_eff"] == block.packed[0].T_eff
+
+
+def test_compress_block_random_blocks(capsys):
+    """60 seeded blocks (1-3 layers, 1-4 KV heads, 1-8 query heads each, 16-256 tokens, budgets 2-16,
+    three K option sets, pooling windows 1-7 with both paddings, next-block and causal queries): every
+    layer's packed tensors, allocation and logical bit count against the oracle's selection + packer."""
+    for case in range(60):
+        rng = np.random.default_rng(110000 + case)
+        L, H, G, D = int(rng.integers(1, 4)), int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8])), 128
+        T, budget = int(rng.choice([16, 32, 64, 100, 128, 256])), int(rng.choice([2, 8, 16]))
+        k_opts = [(0, 2, 4, 8), (2, 4, 8, 16), (0, 2, 4, 8, 16)][int(rng.integers(0, 3))]
+        causal = bool(rng.random() < 0.4)
+        kv, queries, scores = _block_inputs(110000 + case, L, H, G, T, D)
+        config = dataclasses.replace(
+            _config(T, budget, k_opts), pool_kernel_size=int(rng.choice([1, 3, 5, 7])),
+            pool_padding=str(rng.choice(["reflect", "zero"])), k_budget_ratio=float(rng.choice([0.3, 0.5, 0.7])))
+        config.validate()
+        block, _ = bw._compress_block(
+            target_kv=kv, query_block=queries, token_scores_by_layer=scores, block_id=1, token_start=T,
+            token_end=2 * T - 1, query_source_block=2, is_final_flush=causal, causal=causal, config=config,
+            num_kv_groups=G, model_dtype=torch.float16)
+        capsys.readouterr()
+        what = f"case {case}: L={L} H={H} G={G} T={T} budget={budget} K options {k_opts} causal={causal}"
+        for l, (pl, v16, vb, kb) in enumerate(_expected_block(kv, queries, scores, config, G, D)):
+            try:
+                assert_layers_equal(block.packed[l], pl, skip=("allocation_v_bits", "allocation_k_bits"))
+            except AssertionError as e:
+                raise AssertionError(f"{what}, layer {l}: {e}") from None
+            np.testing.assert_array_equal(t2n(block.packed[l].allocation_v_bits), vb.astype(np.int16), err_msg=what)
+            np.testing.assert_array_equal(t2n(block.packed[l].allocation_k_bits), kb.astype(np.int16), err_msg=what)
+            assert (block.new_v_only[l] is None) == (v16 is None), what
+            if v16 is not None:
+                assert_bits_equal(t2n(block.new_v_only[l]), v16)
+            assert block.logical_bits_per_layer[l] == S.logical_layer_bits(vb, kb, D), what
 
 
 def test_compress_block_fixed_slot_and_phase_timing(monkeypatch):
