@@ -300,7 +300,8 @@ typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgro
  * descriptors (device).  n2p/n4p: padded 2-/4-bit channel counts of the source layout.
  * perm (int64, head stride in elements, 0 = one table for all heads), kscale / kzp (fp16, head
  * stride ks_stride_h): the layer's K_ch_perm_padded_idx, K_ch_scale and K_ch_zp, from which the
- * unit's slot table (RdkvSlot per stream slot, at qtab_off) is written.  n8: bytes per K8 row;
+ * unit's slot table (RdkvSlot per stream slot, at qtab_off) is written; a layer without kept K
+ * channels (n2p = n4p = n8 = 0: no slot reads them) may pass null for the three.  n8: bytes per K8 row;
  * max_tiles: the largest number of 64-token tiles (all classes) of any of the layer's units (one
  * workgroup per tile and head, the tile's source rows staged through LDS). */
 int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k2_stride_t,
