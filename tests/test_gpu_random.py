@@ -576,3 +576,55 @@ def test_stream_caches_random_sources_partitions_files(block, tmp_path):
         longer = stream_cache.extend_stream_cache(cache, [extra[1]], row_of_entry=[row])
         _check_against_merged_oracle(longer, q, q_np, oracle_entries + [extra[0]], rows_of + [row], H_q,
                                      f"{what}, one more source in group {row}")
+
+
+def test_reference_layout_entry_points_shared_layout_and_views():
+    """120 layers of the shared layout (build_packed_layer: one V allocation for all heads, K
+    allocation shared or per head; 3-D or 4-D tensors) through k_mixed_qk_dot[_into] and
+    v_dequant_weighted_sum_dispatch[_into] with scores, weights and outputs that are column slices
+    of wider buffers: the oracle's kernel-level references within 2e-3 (times the magnitude), nothing
+    written outside the views, allocating and in-place forms bit-identical.  On this layout the V
+    dispatch leaves the fp16-kept rows to the caller (triton_v_kernel.py:1751-1760)."""
+    for case in range(120):
+        rng = np.random.default_rng(130000 + case)
+        H, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8]))
+        H_q = H * G
+        T = int(rng.choice([1, 5, 63, 64, 65, 130, 255, 256, 257, 400, 900, 1700]))
+        p = rng.random(5) * (rng.random(5) < 0.75)
+        if p[1:].sum() == 0:
+            p[int(rng.integers(1, 5))] = 1.0
+        vb = rng.choice(np.array([0, 2, 4, 8, 16]), size=T, p=p / p.sum())
+        p_k = rng.random(5) * (rng.random(5) < 0.75)
+        if p_k[1:].sum() == 0:
+            p_k[int(rng.integers(1, 5))] = 1.0
+        per_head_k = bool(rng.random() < 0.5)
+        kb = rng.choice(np.array([0, 2, 4, 8, 16]), size=(H, 128) if per_head_k else 128, p=p_k / p_k.sum())
+        scale = float(rng.choice([1.0, 0.05, 8.0]))
+        K = (rng.standard_normal((1, H, T, 128)) * scale).astype(np.float16)
+        V = (rng.standard_normal((1, H, T, 128)) * scale).astype(np.float16)
+        q = rng.standard_normal((H_q, 128)).astype(np.float32)
+        what = f"case {case}: H={H} G={G} T={T} K allocation per head={per_head_k} magnitude {scale}"
+        kw = dict(gqa_factor=G) if per_head_k else {}
+        ora, tk, _ = O.build_packed_layer(K, V, vb, kb, **kw)
+        if tk == 0:
+            continue
+        pl, _, _ = packing.build_packed_layer(to_dev(K), to_dev(V), torch.from_numpy(vb), torch.from_numpy(kb), **kw)
+        if rng.random() < 0.5:
+            pl = fast_decode._pre_squeeze_packed((pl,))[0]
+        q_dev = to_dev(q)
+        exp_s = O.k_mixed_qk_dot_ref(q, ora, tk, round_fp16=False)
+        got = kk.k_mixed_qk_dot(q_dev, pl, tk)
+        assert float(np.abs(t2n(got) - exp_s).max()) < 2e-3 * max(1.0, 4 * scale), what + ": scores"
+        pad = int(rng.choice([0, 7, 64]))
+        buf = torch.full((H_q, tk + pad + 3), float("nan"), device=DEV)
+        kk.k_mixed_qk_dot_into(q_dev, pl, tk, buf[:, 3:3 + tk + pad], T_alloc=tk + pad)
+        assert torch.equal(buf[:, 3:3 + tk], got) and bool(torch.isnan(buf[:, :3]).all()), what + ": score view"
+        w_np = O.softmax_rows(exp_s)
+        w_wide = torch.zeros(H_q, tk + 5, device=DEV)
+        w_wide[:, :tk] = to_dev(w_np)
+        exp_o = O.v_dequant_weighted_sum_ref(w_np, ora, V16=None, round_fp16=False)
+        out_wide = torch.full((H_q, 130), float("nan"), device=DEV)
+        vk.v_dequant_weighted_sum_dispatch_into(w_wide[:, :tk], pl, out_wide[:, 1:129])
+        assert float(np.abs(t2n(out_wide[:, 1:129]) - exp_o).max()) < 2e-3 * max(1.0, scale), what + ": V sum"
+        assert bool(torch.isnan(out_wide[:, 0]).all() and torch.isnan(out_wide[:, 129]).all()), what + ": out view"
+        assert torch.equal(vk.v_dequant_weighted_sum_dispatch(w_wide[:, :tk], pl), out_wide[:, 1:129]), what
