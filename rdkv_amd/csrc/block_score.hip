@@ -316,8 +316,9 @@ RDKV_API int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride
     const size_t lds = ((size_t)qb * D + (size_t)qb * T) * 4;
     const int wide_rows = (k_dtype == RDKV_DTYPE_F16 || k_dtype == RDKV_DTYPE_BF16) && D % 8 == 0 &&
                           k_stride_h % 8 == 0 && k_stride_t % 8 == 0 && ((uintptr_t)keys % 16) == 0;
-    hipFuncSetAttribute(reinterpret_cast<const void *>(block_score_partial_kernel),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    RDKV_REQUIRE(hipFuncSetAttribute(reinterpret_cast<const void *>(block_score_partial_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) == hipSuccess,
+                 "%s: the device refuses 160 KB of LDS per workgroup", fn);
     hipLaunchKernelGGL(block_score_partial_kernel, dim3(n_qtiles, H_q), dim3(kScoreThreads), lds, s, queries,
                        q_dtype, q_stride_h, q_stride_q, keys, k_dtype, k_stride_h, k_stride_t, G, Q, (int)T, D, qb,
                        causal, (float)(1.0 / sqrt((double)D)), wide_rows, reinterpret_cast<float *>(workspace));

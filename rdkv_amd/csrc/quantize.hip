@@ -4,6 +4,11 @@
 // scales and zero-points are bit-identical to the reference's CPU results.
 #include "rdkv_common.h"
 
+// No fused multiply-adds in this file, whatever the command line says: the reference rounds every
+// product and every sum on its own, and HIP's __fmul_rn / __fadd_rn do not stop the compiler from
+// contracting them.  (The explicit fmaf calls below stay what they are.)
+#pragma clang fp contract(off)
+
 namespace {
 
 // ---------------------------------------------------------------------------

@@ -11,6 +11,11 @@
 // expressions imply; this file is compiled without floating-point contraction.
 #include "rdkv_common.h"
 
+// No fused multiply-adds in this file, whatever the command line says: the reference rounds every
+// product and every sum on its own, and HIP's __fmul_rn / __fadd_rn do not stop the compiler from
+// contracting them.  (The explicit fmaf calls below stay what they are.)
+#pragma clang fp contract(off)
+
 namespace {
 
 constexpr int kMaxOptions = 8;
