@@ -77,6 +77,15 @@ def test_quantizer_special_cases():
     assert O.quantize_and_pack(np.empty((1, 1, 0, 4), np.float16), 4, 3)[0].shape == (1, 1, 0, 4)
     with pytest.raises(IndexError):
         O.pack_k_mixed(np.empty((1, 1, 0, 8), np.float16), np.full(8, 4))
+    # a constant negative vector: code 0, zp = qmax, fp16 scale 0 -> (0 - qmax) * 0 = -0.0 in fp32 and in
+    # fp16 (packing.py:1427-1444 multiplies the difference by the scale and only then rounds)
+    for bits in (2, 4, 8):
+        x = np.full((1, 1, 2, 128), -0.5, np.float16)
+        q, s, z = O.quantize_and_pack(x, bits, 3)
+        assert not q.any() and float(z.max()) == float(z.min()) == 2 ** bits - 1 and not s.any()
+        pack = {2: O.transfer_8bit_to_2bit_batchwise, 4: O.transfer_8bit_to_4bit_batchwise, 8: lambda v: v}[bits]
+        back = O.unpack_v_segment(pack(q.copy()), s, z, bits)
+        assert back.dtype == np.float16 and np.signbit(back).all() and not back.any()
     # 8-bit NMSE sanity of the reference's own smoke check (knapsack_solver.py:537-548)
     rng = np.random.default_rng(0)
     v = rng.standard_normal((1, 8, 512, 128)).astype(np.float16)
