@@ -64,6 +64,9 @@ def parse():
                     help="only the reference-layout entry points on one layer (for profiling): prints its JSON")
     ap.add_argument("--pack-only", action="store_true",
                     help="only the prefill pack of one sequence of the workload (for profiling): prints its JSON")
+    ap.add_argument("--knapsack-only", action="store_true",
+                    help="only the V knapsack of the selection over 1, 8 and all layers' score rows per launch "
+                         "(for profiling): prints its JSON")
     ap.add_argument("--no-decode-loop", action="store_true",
                     help="skip the whole-model greedy decode loop (random-weight Llama-3.1-8B-shaped model)")
     return ap.parse_args()
@@ -391,6 +394,32 @@ def pack_sample_section(pack_sample, pack_info, cfg, torch, dev, select_info=Non
 # ---------------------------------------------------------------------------------------------
 # one layer per call, and the reference-layout entry points
 # ---------------------------------------------------------------------------------------------
+def knapsack_rows_section(cfg, torch, dev, steps=20):
+    """The V allocation of the prefill-time selection (knapsack_solver.knapsack_allocate: one workgroup per
+    score row) with the rows of 1, 8 and all layers of the workload in one launch pair: a single layer's
+    H_kv rows leave most compute units idle, the rows of a prompt's layers together fill them."""
+    from rdkv_amd import knapsack_solver as ks
+    g = torch.Generator(device="cpu").manual_seed(4242)
+    T, H = cfg.context, cfg.H_kv
+    budget = 4.0                                            # bits per element: a quarter of fp16
+    out = {"workload": cfg.name, "tokens_per_row": T, "rows_per_layer": H,
+           "budget_bits_per_element": budget, "launches": []}
+    for layers in (1, 8, cfg.layers):
+        rows = layers * H
+        scores = torch.exp(torch.randn(rows, T, generator=g) * 1.5 + 2.0).to(dev)
+        bud = torch.full((rows,), budget, device=dev)
+
+        def call():
+            ks.knapsack_allocate(scores, bud, ks.DEFAULT_EPSILON_V, group_rows=H, with_counts=True)
+        for _ in range(3):
+            call()
+        ms = time_region(call, steps, torch)
+        out["launches"].append({"layers": layers, "rows": rows, "us_per_call": ms * 1e3,
+                                "us_per_layer": ms * 1e3 / layers})
+        del scores
+    return out
+
+
 def sequential_section(cfg, torch, dev, layers=8, replays=50):
     """One layer per call, the form a sequential model loop issues: `layers` single-layer streaming
     caches (distinct buffers, 280 MB together: more than the last-level cache), their fused calls
@@ -673,6 +702,9 @@ def main():
         return
     if args.pack_only:
         print(json.dumps(pack_sequence_section(cfg, torch, dev)))
+        return
+    if args.knapsack_only:
+        print(json.dumps(knapsack_rows_section(cfg, torch, dev, steps=args.steps)))
         return
     t_build = time.time()
     first = {}
