@@ -182,7 +182,8 @@ def test_tail_scores_kernel_matches_tensor_expressions():
         torch.testing.assert_close(next_s, exp_next, rtol=1e-6, atol=1e-6)
 
 
-@pytest.mark.parametrize("n_tokens,block", [(45, 8), (16, 8), (3, 8), (70, 16)])
+@pytest.mark.parametrize("n_tokens,block", [(45, 8), (16, 8), (3, 8), (70, 16), (1, 8), (8, 8), (9, 8), (33, 4), (64, 32),
+                                            (17, 16)])
 def test_graph_replayed_loop_equals_the_eager_loop(setup, n_tokens, block):
     """``use_cuda_graph=True`` (blockwise_decode.py:1991-2117): the step replayed from a HIP graph,
     recorded again after every compression, gives the eager loop's tokens, compression events and
