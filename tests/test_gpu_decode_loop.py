@@ -160,19 +160,20 @@ def test_decode_loop_tracks_model_forward(setup):
             assert float((got - exp).abs().max()) <= 0.05 * float(exp.abs().max())
 
 
-def test_graph_replay_gives_the_eager_tokens(setup):
+@pytest.mark.parametrize("n_tokens,seed", [(80, 12), (1, 3), (2, 4), (63, 5), (65, 6), (130, 7)])
+def test_graph_replay_gives_the_eager_tokens(setup, n_tokens, seed):
     model, prompt, pre, kv = setup          # 80 tokens: the raw tail crosses the 64-token chunk of the merge kernel
-    v_bits, k_bits = _mixed_bits(12)
+    v_bits, k_bits = _mixed_bits(seed)
     first = pre.logits[0, -1]
-    eager = fast_decode.greedy_decode_fast(model, _pack(kv, v_bits, k_bits), first, 80, [], torch.device(DEV),
+    eager = fast_decode.greedy_decode_fast(model, _pack(kv, v_bits, k_bits), first, n_tokens, [], torch.device(DEV),
                                            T_PROMPT)
     cache = _pack(kv, v_bits, k_bits)
-    graphed = fast_decode.greedy_decode_fast(model, cache, first, 80, [], torch.device(DEV), T_PROMPT,
+    graphed = fast_decode.greedy_decode_fast(model, cache, first, n_tokens, [], torch.device(DEV), T_PROMPT,
                                              use_cuda_graph=True)
-    assert graphed == eager and len(eager) == 80
+    assert graphed == eager and len(eager) == n_tokens
     # a second run over the same cache object reuses its streaming caches and zone C buffers
     torch.cuda.synchronize()
-    assert fast_decode.greedy_decode_fast(model, cache, first, 80, [], torch.device(DEV), T_PROMPT,
+    assert fast_decode.greedy_decode_fast(model, cache, first, n_tokens, [], torch.device(DEV), T_PROMPT,
                                           use_cuda_graph=True) == eager
 
 
