@@ -373,7 +373,8 @@ int rdkv_decode_fused_one_launch(const uint8_t *blob, const RdkvUnit *units, int
  * nothing.  n_work * G * 528 bytes must fit (15887 work-item heads: a whole 32-layer step of a
  * 32k-token cache needs 1.1 MB), else RDKV_EWORKSPACE.  All calls on one GPU share that array:
  * calls that overlap on one GPU (two streams, two threads) race.  The array's address is looked
- * up on the first call on each device; make that call outside graph capture. */
+ * up on the first call on each device; make that call outside graph capture.  The stream must
+ * belong to the current device (checked: the array of another device sits at another address). */
 int64_t rdkv_decode_fused_static_max_bytes(void);
 int rdkv_decode_fused_static(const uint8_t *blob, const RdkvUnit *units, int n_units,
                              const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,

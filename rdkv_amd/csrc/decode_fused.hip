@@ -855,17 +855,22 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
     // whoever draws the last ticket of a unit finds all of that unit's partials complete, puts the
     // counter back to zero for the next launch and combines them in index order - the same
     // arithmetic in the same order as the separate merge launch, whoever happens to be last.
+    // Ordering: the partial stores of every thread happen before the workgroup barrier, the ticket is
+    // drawn after it with release semantics at device scope (the barrier carries the other threads'
+    // stores into what the release publishes), and the workgroup that draws the last ticket of a unit
+    // passes an acquire fence at device scope before it reads that unit's partials.
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (tid_o < nb) {
       const RdkvWork *wkp = work + batch + tid_o;
-      sm.ticket[tid_o] = __hip_atomic_fetch_add(tickets + wkp->merge_unit, 1, __ATOMIC_RELAXED,
+      sm.ticket[tid_o] = __hip_atomic_fetch_add(tickets + wkp->merge_unit, 1, __ATOMIC_RELEASE,
                                                 __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     for (int b = 0; b < nb; ++b) {
       const Item mi = load_item(batch + b);
       if (sm.ticket[b] == mi.merge_count - 1) {      // uniform over the workgroup
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         if (tid_o == 0) __hip_atomic_store(tickets + mi.merge_unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // the wavefront results of the batch have been consumed: their LDS serves as scratch
         float *scratch = &sm.wo[0][0][0][0];
@@ -1004,8 +1009,10 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
         v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
       }
       qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
-      // the rotated query as the in-place rotation would have left it, for callers that keep it
-      if (q_rot_out)
+      // the rotated query as the in-place rotation would have left it, for callers that keep it (a
+      // buffer with one row per token takes it at the step's row, under the same range check as the
+      // appended key: a device-held row that has run past the buffer writes nothing)
+      if (q_rot_out && (ts.q_rotated_stride_tok == 0 || (step_row >= 0 && step_row < ap.capacity)))
         rdkv_store_from_float(q_rot_out, q_dtype,
                               (int64_t)(q_row + (i >> 7)) * q_rot_stride + step_row * ts.q_rotated_stride_tok + c, v);
     }
@@ -1372,12 +1379,24 @@ void *g_scratch_ptr[kMaxDevices];            // device address of `scratch`, per
 std::mutex g_scratch_mutex;
 
 // Address of the current device's copy of `scratch` (looked up on the first call on that device).
-int static_scratch(const char *fn, void **ptr) {
+// The stream has to belong to the current device: the kernels run where the stream lives, and
+// another device's copy of the array sits at another address.
+int static_scratch(const char *fn, hipStream_t stream, void **ptr) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) {
     rdkv_set_error("%s: hipGetDevice: %s", fn, hipGetErrorString(e));
     return RDKV_ELAUNCH;
+  }
+  if (stream) {
+    hipDevice_t sdev = -1;
+    e = hipStreamGetDevice(stream, &sdev);
+    if (e != hipSuccess) {
+      rdkv_set_error("%s: hipStreamGetDevice: %s", fn, hipGetErrorString(e));
+      return RDKV_ELAUNCH;
+    }
+    RDKV_REQUIRE((int)sdev == dev, "%s: the stream belongs to device %d, the current device is %d", fn, (int)sdev,
+                 dev);
   }
   RDKV_REQUIRE(dev >= 0 && dev < kMaxDevices, "%s: device ordinal %d outside 0..%d", fn, dev, kMaxDevices - 1);
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
@@ -1412,7 +1431,7 @@ RDKV_API int rdkv_decode_fused_static(const uint8_t *blob, const RdkvUnit *units
     return RDKV_EWORKSPACE;
   }
   void *ptr = nullptr;
-  const int rc = static_scratch(fn, &ptr);
+  const int rc = static_scratch(fn, (hipStream_t)stream, &ptr);
   if (rc != RDKV_OK) return rc;
   // every partial a merge reads is written in full by the streaming launch of the same call, so
   // nothing in the buffer has to start at zero

@@ -745,6 +745,64 @@ def save_stream_cache(cache: StreamCache, path: str) -> None:
         f.truncate(data0 + off)
 
 
+def _check_header(path: str, header) -> None:
+    """Raise ValueError unless the JSON header has every key the loader follows, of the type and in
+    the range it assumes: nothing from the file reaches ``_finish_cache`` or a kernel unchecked."""
+    def bad(msg):
+        raise ValueError(f"{path}: header: {msg}")
+
+    def is_int(v):
+        return isinstance(v, int) and not isinstance(v, bool)
+
+    if not isinstance(header, dict):
+        bad("not a JSON object")
+    for key in ("G", "rows", "h_q", "n_units", "stream_bytes", "kv_algorithmic_bytes", "max_row_dwords"):
+        if not is_int(header.get(key)) or header[key] < 0:
+            bad(f"{key!r} missing or not a non-negative integer")
+    if not isinstance(header.get("multi_source"), bool):
+        bad("'multi_source' missing or not a boolean")
+    G, h_q, rows = header["G"], header["h_q"], header["rows"]
+    if not 1 <= G <= 8:
+        bad(f"G={G} outside 1..8")
+    if h_q <= 0 or h_q % G:
+        bad(f"h_q={h_q} is not a positive multiple of G={G}")
+    if rows % h_q:
+        bad(f"rows={rows} is not a multiple of h_q={h_q}")
+    sections = header.get("sections")
+    if not isinstance(sections, dict):
+        bad("'sections' missing")
+    for name in ("units", "blob_of", "scale_max"):
+        ext = sections.get(name)
+        if not (isinstance(ext, list) and len(ext) == 3 and all(is_int(v) for v in ext)):
+            bad(f"section {name!r} missing or not [offset, bytes, crc]")
+    blobs = header.get("blobs")
+    if not isinstance(blobs, list) or not all(isinstance(b, list) and len(b) == 3 and all(is_int(v) for v in b)
+                                              for b in blobs):
+        bad("'blobs' missing or not a list of [offset, bytes, crc]")
+    part = header.get("partition")
+    if part is None:
+        return
+    if not isinstance(part, dict):
+        bad("'partition' is not an object")
+    for key in ("n_groups", "work_bytes"):
+        v = part.get(key)
+        if v is not None and not (is_int(v) and 1 <= v < 2 ** 31):
+            bad(f"partition[{key!r}]={v!r} is not a positive integer")
+    v = part.get("groups_per_cu", 1)
+    if not (is_int(v) and 1 <= v <= 64):
+        bad(f"partition['groups_per_cu']={v!r} outside 1..64")
+    cost = part.get("cost")
+    if cost is not None:
+        def num(x):
+            return isinstance(x, (int, float)) and not isinstance(x, bool) and np.isfinite(x) and x >= 0
+        ok = (isinstance(cost, dict) and isinstance(cost.get("tile"), list) and len(cost["tile"]) == 4
+              and all(num(x) for x in cost["tile"]) and num(cost.get("k_dword")) and num(cost.get("item")))
+        speed = cost.get("group_speed", [1.0]) if isinstance(cost, dict) else None
+        ok = ok and isinstance(speed, list) and 1 <= len(speed) <= 64 and all(num(x) and x > 0 for x in speed)
+        if not ok or set(cost) - {"tile", "k_dword", "item", "group_speed"}:
+            bad("partition['cost'] is not a cost model (tile[4], k_dword, item, group_speed)")
+
+
 def read_stream_cache_file(path: str, verify: bool = True):
     """Host side of ``load_stream_cache``: parse and check ``path`` without touching a device.
     Returns (header, units with blob-relative offsets, blob_of, [memory-mapped blob bytes], largest
@@ -773,6 +831,7 @@ def read_stream_cache_file(path: str, verify: bool = True):
     if header.get("byteorder") != "little":
         raise ValueError(f"{path}: byte order {header.get('byteorder')!r} not supported")
     data0 = _align(24 + hlen)
+    _check_header(path, header)
 
     def extent(name, o, n, crc):
         if o < 0 or n < 0 or data0 + o + n > len(mm):

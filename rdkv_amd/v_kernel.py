@@ -53,17 +53,20 @@ def _sq(t):
 
 
 def _seg(t, width):
-    """-> (address or None, head stride) of a [H_kv, N, width] code tensor with dense rows."""
+    """-> (tensor, address or None, head stride) of a [H_kv, N, width] code tensor with dense rows.
+    The tensor is what the address points into (a dense copy when the rows were strided): the caller
+    holds it until the launch is enqueued, or the allocator may hand the copy's block to the next
+    copy, which the stream runs before the kernel."""
     if t is None:
-        return None, 0
+        return None, None, 0
     if t.dim() == 4:
         t = t.squeeze(0)
     if t.numel() == 0:
-        return None, 0
+        return None, None, 0
     assert t.shape[-1] == width
     if not (t.stride(2) == 1 and t.stride(1) == width):
         t = t.contiguous()
-    return t.data_ptr(), t.stride(0)
+    return t, t.data_ptr(), t.stride(0)
 
 
 def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_head, seg_bounds,
@@ -82,24 +85,24 @@ def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_
     if w.stride(1) != 1:
         w = w.contiguous()
     assert out.dtype == torch.float32 and out.stride(1) == 1 and out.shape[1] == D
-    V2, v2h = _seg(V_2bit, D // 4)
-    V4, v4h = _seg(V_4bit, D // 2)
-    V8, v8h = _seg(V_8bit, D)
+    keep2, V2, v2h = _seg(V_2bit, D // 4)
+    keep4, V4, v4h = _seg(V_4bit, D // 2)
+    keep8, V8, v8h = _seg(V_8bit, D)
     # scale / zero point rows: [H_kv, T] or [H_kv, T, 1] with unit token stride
     n_meta = sc.numel()
     if n_meta and not (sc.stride(1) == 1 and zp.stride(1) == 1 and zp.stride(0) == sc.stride(0)):
         sc, zp = sc.reshape(H_kv, -1).contiguous(), zp.reshape(H_kv, -1).contiguous()
     N2, N4, N8 = seg_bounds
-    v16 = v16h = n16 = None
+    v16 = v16h = n16 = keep16 = None
     if V16 is not None and n_v16_per_head is not None:
         v16 = _sq(V16)                    # [H_kv, n16_max, 128]; the packer's new_v_only carries a leading 1
         assert v16.dim() == 3 and v16.shape[0] == H_kv and v16.shape[2] == D and v16.dtype == torch.float16, \
             f"V16 must be fp16 [H_kv={H_kv}, n, {D}], got {tuple(V16.shape)} {V16.dtype}"
         assert n_v16_per_head.numel() == H_kv and n_v16_per_head.dtype == torch.int32
-        v16 = v16 if v16.is_contiguous() else v16.contiguous()
-        v16h = v16.stride(0)
+        keep16 = v16 if v16.is_contiguous() else v16.contiguous()
+        v16h = keep16.stride(0)
         n16 = n_v16_per_head.data_ptr()
-        v16 = v16.data_ptr() if v16.numel() else None
+        v16 = keep16.data_ptr() if keep16.numel() else None
     stream = _lib.stream_of(dev)
     ws = _lib.workspace(dev, lib.rdkv_v_weighted_sum_workspace_bytes(H_q))
     _lib.check(lib.rdkv_v_weighted_sum(
@@ -108,6 +111,7 @@ def _launch(attn_weights, V_2bit, V_4bit, V_8bit, V_scale, V_zp, seg_bounds_per_
         None if seg_bounds_per_head is None else seg_bounds_per_head.data_ptr(), int(N2), int(N4), int(N8),
         v16, v16h or 0, n16 if v16 is not None else None, int(max_T_v),
         out.data_ptr(), out.stride(0), ws.data_ptr(), ws.numel(), stream))
+    del keep2, keep4, keep8, keep16     # dense copies live until the launch above is enqueued
 
 
 # ---- single bit-width entry points (triton_v_kernel.py:1108-1220) -----------------------

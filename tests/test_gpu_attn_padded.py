@@ -158,6 +158,44 @@ def test_k_scores_strided_rows_match_dense_rows():
     torch.testing.assert_close(strided, dense, rtol=0, atol=2e-5)
 
 
+def test_v_sum_strided_code_rows_and_v16_match_dense():
+    """V segments whose rows are column slices of wider buffers (stride(1) != width) and a V16 whose
+    heads are not stored back to back: the entry point makes dense copies of them, and every copy has
+    to stay allocated until the launch is enqueued.  The result is compared with the oracle and with
+    the call on the dense tensors (same kernel, same bytes: same bits)."""
+    import dataclasses
+    cfg = synth.scaled(synth.CONFIGS[1], context=2300, layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, q = synth.layer_data(cfg, 0, "cpu", outliers=oc)
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), cfg.G)
+    exp_out, _, exp_w = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, cfg.G)
+    w = to_dev(exp_w.astype(np.float32))
+    V16 = nvo[0].contiguous()
+    dense = vk.v_dequant_weighted_sum_dispatch(w, pl, V16=V16, n_v16_per_head=pl.n_v16_per_head, max_T_v=pl.T_eff)
+
+    def widened(t, extra):
+        buf = torch.full(t.shape[:-1] + (t.shape[-1] + extra,), 0xA5, dtype=t.dtype, device=t.device)
+        buf[..., :t.shape[-1]] = t
+        return buf[..., :t.shape[-1]]
+
+    assert all(getattr(pl, n) is not None and getattr(pl, n).numel() for n in ("V_2bit", "V_4bit", "V_8bit"))
+    sv = dataclasses.replace(pl, V_2bit=widened(pl.V_2bit, 32), V_4bit=widened(pl.V_4bit, 64),
+                             V_8bit=widened(pl.V_8bit, 128))
+    assert not any(getattr(sv, n).is_contiguous() for n in ("V_2bit", "V_4bit", "V_8bit"))
+    # V16 [H_kv, n, 128] as a view whose head dimension is the middle one of its buffer
+    v16_buf = torch.full((V16.shape[1], V16.shape[0], 128), 7.0, dtype=torch.float16, device=DEV)
+    v16_buf.copy_(V16.transpose(0, 1))
+    v16_view = v16_buf.transpose(0, 1)
+    assert not v16_view.is_contiguous() and torch.equal(v16_view, V16)
+    torch.cuda.empty_cache()            # the copies below draw fresh blocks, one after the other
+    for rep in range(3):
+        got = vk.v_dequant_weighted_sum_dispatch(w, sv, V16=v16_view, n_v16_per_head=pl.n_v16_per_head,
+                                                 max_T_v=pl.T_eff)
+        assert torch.equal(got, dense), f"strided segments give other bits than dense ones (call {rep})"
+    attn_close(t2n(got), exp_out, "out (strided V segments)")
+
+
 @pytest.mark.parametrize("T_old,n_new,masked,aligned", [
     (4096, 1, True, True), (5, 0, False, True), (3, 2, True, True), (8191, 7, True, True), (8192, 0, True, True),
     (32768, 3, True, True), (32771, 64, False, True), (65536, 1, True, True), (70001, 5, True, True),

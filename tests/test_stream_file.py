@@ -166,7 +166,7 @@ def test_blob_index_and_table_length_are_checked(tmp_path):
     open(bad, "wb").write(_rewrite_header(raw, lambda h: h.update(n_units=4)))
     with pytest.raises(ValueError, match="header says 4"):
         sc.read_stream_cache_file(bad)
-    open(bad, "wb").write(_rewrite_header(raw, lambda h: h.update(rows=4)))
+    open(bad, "wb").write(_rewrite_header(raw, lambda h: h.update(rows=0)))
     with pytest.raises(ValueError, match="output rows"):
         sc.read_stream_cache_file(bad)
     open(bad, "wb").write(_rewrite_header(raw, lambda h: h.update(max_row_dwords=5)))
@@ -175,3 +175,61 @@ def test_blob_index_and_table_length_are_checked(tmp_path):
     open(bad, "wb").write(_rewrite_header(raw, lambda h: h.update(G=9)))
     with pytest.raises(ValueError, match="G=9"):
         sc.read_stream_cache_file(bad)
+
+
+def _drop(*keys):
+    def edit(h):
+        d = h
+        for k in keys[:-1]:
+            d = d[k]
+        del d[keys[-1]]
+    return edit
+
+
+def _set(value, *keys):
+    def edit(h):
+        d = h
+        for k in keys[:-1]:
+            d = d[k]
+        d[keys[-1]] = value
+    return edit
+
+
+@pytest.mark.parametrize("edit,match", [
+    (_set(0, "h_q"), "h_q=0"), (_set(6, "h_q"), "h_q=6"), (_set(-12, "h_q"), "'h_q'"), (_set("12", "h_q"), "'h_q'"),
+    (_set(16, "rows"), "rows=16"), (_set(1.5, "rows"), "'rows'"), (_set(True, "G"), "'G'"),
+    (_drop("h_q"), "'h_q'"), (_drop("G"), "'G'"), (_drop("rows"), "'rows'"), (_drop("n_units"), "'n_units'"),
+    (_drop("stream_bytes"), "'stream_bytes'"), (_drop("kv_algorithmic_bytes"), "'kv_algorithmic_bytes'"),
+    (_drop("max_row_dwords"), "'max_row_dwords'"), (_drop("multi_source"), "'multi_source'"),
+    (_set("yes", "multi_source"), "'multi_source'"), (_drop("sections"), "'sections'"),
+    (_drop("sections", "units"), "section 'units'"), (_drop("sections", "blob_of"), "section 'blob_of'"),
+    (_drop("sections", "scale_max"), "section 'scale_max'"), (_set([0, 5], "sections", "units"), "section 'units'"),
+    (_drop("blobs"), "'blobs'"), (_set([[0, "x", 0]], "blobs"), "'blobs'"),
+    (_set(0, "partition", "n_groups"), "n_groups"), (_set(-3, "partition", "work_bytes"), "work_bytes"),
+    (_set("7", "partition", "n_groups"), "n_groups"), (_set(0, "partition", "groups_per_cu"), "groups_per_cu"),
+    (_set([1, 2], "partition"), "'partition'"), (_set({"tile": [1, 2, 3]}, "partition", "cost"), "cost model"),
+    (_set({"tile": [1, 2, 3, 4], "k_dword": 1, "item": float("nan")}, "partition", "cost"), "cost model"),
+    (_set({"tile": [1, 2, 3, 4], "k_dword": 1, "item": 1, "group_speed": [0.0]}, "partition", "cost"), "cost model"),
+])
+def test_header_values_are_checked_before_they_are_used(tmp_path, edit, match):
+    """Every header key the loader follows is required, typed and range-checked: a missing key or
+    a value like h_q = 0 is a ValueError of the reader, not a KeyError or ZeroDivisionError later."""
+    cache = _fake_cache(seed=5)
+    path = str(tmp_path / "c.rdkv")
+    sc.save_stream_cache(cache, path)
+    raw = open(path, "rb").read()
+    bad = str(tmp_path / "bad.rdkv")
+    open(bad, "wb").write(_rewrite_header(raw, edit))
+    with pytest.raises(ValueError, match=match):
+        sc.read_stream_cache_file(bad)
+
+
+def test_header_without_partition_reads(tmp_path):
+    cache = _fake_cache(seed=6)
+    path = str(tmp_path / "c.rdkv")
+    sc.save_stream_cache(cache, path)
+    raw = open(path, "rb").read()
+    ok = str(tmp_path / "ok.rdkv")
+    open(ok, "wb").write(_rewrite_header(raw, _drop("partition")))
+    header, units, _, _, _ = sc.read_stream_cache_file(ok)
+    assert "partition" not in header and len(units) == 3

@@ -42,6 +42,7 @@ def test_static_entry_point_matches_workspace_entry_point():
     assert lib.rdkv_decode_fused_static_max_bytes() == 8 << 20
     big = _case(3000, 2, 0)
     small = _case(700, 1, 5)
+    first = True
     for cfg, cache, q, exp in (big, small):            # two calls in a row, the second one smaller
         need = lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G)
         assert 0 < need <= lib.rdkv_decode_fused_static_max_bytes()
@@ -50,10 +51,20 @@ def test_static_entry_point_matches_workspace_entry_point():
         lse_ws = torch.full((cache.rows,), float("nan"), device=DEV)
         out_st, lse_st = out_ws.clone(), lse_ws.clone()
         _lib.check(_call(lib, "rdkv_decode_fused", cache, q, out_ws, lse_ws, ws.data_ptr(), ws.numel()))
+        if first:   # the first call on a device looks up the address of the fixed buffer
+            first = False
+            _lib.check(_call(lib, "rdkv_decode_fused_static", cache, q, out_st, lse_st))
+            out_st.fill_(float("nan"))
+            lse_st.fill_(float("nan"))
+        torch.cuda.synchronize()
+        # two counters: torch's allocator (a tensor made on the way would show here) and the driver's
+        # free memory (a hipMalloc inside the library, which torch's counter never sees)
         before = torch.cuda.memory_stats(DEV)["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info(DEV)[0]
         _lib.check(_call(lib, "rdkv_decode_fused_static", cache, q, out_st, lse_st))
         torch.cuda.synchronize()
         assert torch.cuda.memory_stats(DEV)["allocation.all.allocated"] == before
+        assert torch.cuda.mem_get_info(DEV)[0] == free_before, "device memory was allocated or freed by the call"
         assert torch.equal(out_st, out_ws) and torch.equal(lse_st, lse_ws), f"context {cfg.context}"
         o, l = t2n(out_st), t2n(lse_st)
         for layer, (eo, el) in enumerate(exp):
