@@ -49,25 +49,29 @@ int rdkv_bitunpack4_f32(const uint8_t *packed, float *codes, int64_t rows, int64
 
 /* ---- packing.py : quantizer ---------------------------------------------- */
 /* quantize_and_pack(x, n_bits, dim=last) (packing.py:141-165) fused with the bit-pack of
- * pack_v_segments (packing.py:751-773).  x: fp16 rows of D channels, row r read at
+ * pack_v_segments (packing.py:751-773).  x: rows of D channels stored as x_dtype (RDKV_DTYPE_*:
+ * the reference quantizes the fp32 value of whatever it is given, packing.py:153, so fp16 and
+ * bf16 elements are widened exactly and fp32 ones taken as they are), row r read at
  * x + row_idx[r]*x_row_stride (row_idx NULL = identity; this fuses V[:, :, sort_idx]).
  * pack != 0 writes D*n_bits/8 packed bytes per row, pack == 0 writes D raw codes. */
-int rdkv_quantize_rows(const void *x_f16, int64_t x_row_stride, const int64_t *row_idx,
+int rdkv_quantize_rows(const void *x, int x_dtype, int64_t x_row_stride, const int64_t *row_idx,
                        int64_t rows, int D, int n_bits, int pack,
                        uint8_t *out, void *scale_f16, void *zp_f16, void *stream);
 
-/* Column (per-channel over T) min/max of K[T, D] fp16 (first half of quantize_and_pack(dim=2)
- * inside pack_k_mixed, packing.py:315,331,347).  minmax: float[2*D] = {min[D], max[D]}. */
-int rdkv_col_minmax(const void *x_f16, int64_t x_row_stride, int64_t T, int D,
+/* Column (per-channel over T) min/max of K[T, D] stored as x_dtype (first half of
+ * quantize_and_pack(dim=2) inside pack_k_mixed, packing.py:315,331,347).
+ * minmax: float[2*D] = {min[D], max[D]}. */
+int rdkv_col_minmax(const void *x, int x_dtype, int64_t x_row_stride, int64_t T, int D,
                     float *minmax, void *stream);
 
 /* Second half of pack_k_mixed (packing.py:296-351): gather sorted channels, zero-pad,
  * quantize per channel with the min/max from rdkv_col_minmax, bit-pack per segment.
+ * k: [T, D] stored as k_dtype.
  * slot_channel[D_padded] maps padded sorted slot -> source channel, -1 = zero pad channel.
  * Slots [0,n2p) 2-bit (n2p%4==0), [n2p,n2p+n4p) 4-bit (n4p%2==0), then n8 8-bit slots.
  * Outputs K2[T,n2p/4], K4[T,n4p/2], K8[T,n8] (contiguous; may be NULL when the segment is
  * empty) and scale/zp fp16 [D_padded]. */
-int rdkv_k_quantize_pack(const void *k_f16, int64_t k_row_stride, int64_t T, int D,
+int rdkv_k_quantize_pack(const void *k, int k_dtype, int64_t k_row_stride, int64_t T, int D,
                          const float *minmax, const int32_t *slot_channel,
                          int n2p, int n4p, int n8,
                          uint8_t *K2, uint8_t *K4, uint8_t *K8,

@@ -46,9 +46,9 @@ SIGNATURES = {
     "rdkv_bitunpack2": (I, [P, P, L, L, P]),
     "rdkv_bitpack4": (I, [P, P, L, L, P]),
     "rdkv_bitunpack4_f32": (I, [P, P, L, L, P]),
-    "rdkv_quantize_rows": (I, [P, L, P, L, I, I, I, P, P, P, P]),
-    "rdkv_col_minmax": (I, [P, L, L, I, P, P]),
-    "rdkv_k_quantize_pack": (I, [P, L, L, I, P, P, I, I, I, P, P, P, P, P, P]),
+    "rdkv_quantize_rows": (I, [P, I, L, P, L, I, I, I, P, P, P, P]),
+    "rdkv_col_minmax": (I, [P, I, L, L, I, P, P]),
+    "rdkv_k_quantize_pack": (I, [P, I, L, L, I, P, P, I, I, I, P, P, P, P, P, P]),
     "rdkv_pack_layer_per_head": (I, [P, P, L, L, I, I, P, L, P, I, I, I, L, I, P, I, I, I,
                                      P, P, P, P, P, P, P, P, P, P, P, P, P]),
     "rdkv_pack_layer_v_rows": (I, [P, L, L, I, I, P, L, P, I, I, I, L, I, P, P, P, P, P, P, P, P]),

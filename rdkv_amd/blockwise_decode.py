@@ -344,36 +344,65 @@ def _logical_layer_bits(packed, head_dim: int) -> int:
     return int(_logical_layer_bits_tensor(packed, head_dim).item())
 
 
+def _dense_block(packed: PackedKVLayer, new_v_only: Optional[Tensor], head_dim: int) -> Tuple[Tensor, Tensor]:
+    """The block dequantized by the HIP unpackers: (K_hat, V_hat), fp32 [H_kv, T, head_dim] each, V as
+    its quantized stripe followed by the fp16-kept rows - the column order of the kernels' score and
+    weight rows."""
+    k_hat = unpack_k_mixed(packed, D=head_dim).squeeze(0).float()
+    v_hat = _unpack_v_perhead(packed, head_dim=head_dim).squeeze(0).float()
+    if new_v_only is not None:
+        v_hat = torch.cat([v_hat, new_v_only.squeeze(0).float()], dim=1)
+    return k_hat, v_hat
+
+
+def _require_close(got: Tensor, want: Tensor, tol: float, what: str) -> None:
+    """AssertionError unless |got - want| <= tol + tol * |want| everywhere (the criterion of the
+    reference's check, blockwise_decode.py:704-708, 747-751, with rtol = atol = ``tol``)."""
+    excess = (got - want).abs() - (tol + tol * want.abs())
+    bad = ~(excess <= 0)                                  # a NaN on either side counts as a miss
+    if bool(bad.any()):
+        worst = float((got - want).abs()[bad].max()) if not bool(torch.isnan(got - want).any()) else float("nan")
+        raise AssertionError(f"{what} diverges from explicit dequantization: {int(bad.sum())} of {bad.numel()} "
+                             f"values outside rtol = atol = {tol:g}, largest error {worst:.3e}")
+
+
 def _validate_packed_layer_reference(packed: PackedKVLayer, squeezed: PackedKVLayer, new_v_only: Optional[Tensor],
                                      query: Tensor, *, num_kv_groups: int, head_dim: int) -> None:
-    """blockwise_decode.py:681-753.  The packed K and V kernels against explicit dequantization of
-    the same block, at the reference's tolerances: scores of ``query`` [H_q, D] over the block's
-    keys (2e-2 / 2e-2) and the uniformly weighted value sum over its kept tokens (3e-2 / 3e-2).
-    The dequantizers are the HIP ones (``unpack_k_mixed``, ``_unpack_v_perhead``); the comparison
-    itself is tensor expressions on the device, as in the reference."""
-    t_eff_k = squeezed.T_eff_k if squeezed.T_eff_k > 0 else squeezed.T_eff
-    if t_eff_k == 0:
+    """The run-time self-check of a compressed block (role of blockwise_decode.py:681-753): the two
+    packed kernels must reproduce attention over the dequantized block.  Scores of ``query``
+    [H_q, D] over the block's keys are held to 2e-2, and the value sum under uniform weights over the
+    tokens each head keeps (what softmax makes of a zero row plus the layer's padding mask) to 3e-2
+    - the reference's tolerances.  Raises AssertionError naming the side that differs."""
+    n_cols = int(squeezed.T_eff_k) or int(squeezed.T_eff)
+    if n_cols == 0:
         return
-    q = query.float()
-    actual_k = k_mixed_qk_dot(q, squeezed, t_eff_k)
-    unpacked_k = unpack_k_mixed(packed, D=head_dim)[0].float()
-    expected_k = torch.einsum("hd,htd->ht", q, unpacked_k.repeat_interleave(num_kv_groups, dim=0)) / (head_dim ** 0.5)
-    torch.testing.assert_close(actual_k, expected_k, rtol=2e-2, atol=2e-2,
-                               msg="packed K block diverges from explicit dequantization")
-    v_zone_a = _unpack_v_perhead(packed, head_dim=head_dim)[0].float()
-    unpacked_v = torch.cat([v_zone_a, new_v_only[0].float()], dim=1) if new_v_only is not None else v_zone_a
-    logits = torch.zeros(q.shape[0], t_eff_k, dtype=torch.float32, device=q.device)
+    k_hat, v_hat = _dense_block(packed, new_v_only, head_dim)
+    h_kv = k_hat.shape[0]
+    q_groups = query.float().reshape(h_kv, num_kv_groups, head_dim)
+
+    scores = k_mixed_qk_dot(query.float(), squeezed, n_cols)
+    want_scores = torch.bmm(q_groups, k_hat[:, :n_cols].transpose(1, 2)).mul_(head_dim ** -0.5)
+    _require_close(scores, want_scores.reshape(scores.shape), 2e-2, "packed K block")
+
     if squeezed.softmax_mask is not None:
-        logits.add_(squeezed.softmax_mask)
-    weights = torch.softmax(logits, dim=-1)
-    dummy_v, zero_counts = _get_v16_dummy(q.device, unpacked_v.shape[0])
-    actual_v = v_dequant_weighted_sum_dispatch(
-        weights, squeezed, V16=new_v_only[0].contiguous() if new_v_only is not None else dummy_v,
-        n_v16_per_head=squeezed.n_v16_per_head if squeezed.n_v16_per_head is not None else zero_counts,
-        max_T_v=squeezed.T_eff)
-    expected_v = (weights.view(unpacked_v.shape[0], num_kv_groups, t_eff_k) @ unpacked_v).reshape(q.shape[0], head_dim)
-    torch.testing.assert_close(actual_v, expected_v, rtol=3e-2, atol=3e-2,
-                               msg="packed V block diverges from explicit dequantization")
+        visible = torch.isfinite(squeezed.softmax_mask[:, :n_cols]).float()
+    else:
+        visible = torch.ones_like(scores)
+    n_visible = visible.sum(dim=-1, keepdim=True)
+    if bool((n_visible == 0).any()):
+        # the reference's softmax over a fully masked row is NaN and its comparison fails on it
+        raise AssertionError("packed V block diverges from explicit dequantization: a head of the block keeps "
+                             "no token, so its weight row has no softmax")
+    weights = visible / n_visible
+    v16, counts = _get_v16_dummy(query.device, h_kv)
+    if new_v_only is not None:
+        v16 = new_v_only.squeeze(0).contiguous()
+    if squeezed.n_v16_per_head is not None:
+        counts = squeezed.n_v16_per_head
+    summed = v_dequant_weighted_sum_dispatch(weights, squeezed, V16=v16, n_v16_per_head=counts,
+                                             max_T_v=squeezed.T_eff)
+    want_sum = torch.bmm(weights.reshape(h_kv, num_kv_groups, n_cols), v_hat[:, :n_cols])
+    _require_close(summed, want_sum.reshape(summed.shape), 3e-2, "packed V block")
 
 
 def _rows(x: Tensor) -> Tensor:

@@ -14,15 +14,32 @@ namespace {
 // ---------------------------------------------------------------------------
 // Per-row (per-token) quantizer, one wavefront per row.
 // ---------------------------------------------------------------------------
+// Storage type of the values to quantize.  The reference quantizes the fp32 value of whatever it
+// is given (packing.py:153: x.float()), so an element is widened exactly and never rounded first.
+struct InF16 {
+  typedef __half raw;
+  static __device__ __forceinline__ float get(const raw *p, int64_t i) { return __half2float(p[i]); }
+};
+struct InBF16 {
+  typedef uint16_t raw;
+  static __device__ __forceinline__ float get(const raw *p, int64_t i) {
+    return __uint_as_float((uint32_t)p[i] << 16);
+  }
+};
+struct InF32 {
+  typedef float raw;
+  static __device__ __forceinline__ float get(const raw *p, int64_t i) { return p[i]; }
+};
+
 // One wavefront quantizes one row of D channels: min/max -> scale/zp -> codes -> packed bytes.
-template <int BITS>
-__device__ __forceinline__ void quantize_one_row(const __half *__restrict__ xr, int D, int pack, int lane,
+template <int BITS, typename In = InF16>
+__device__ __forceinline__ void quantize_one_row(const typename In::raw *__restrict__ xr, int D, int pack, int lane,
                                                  uint8_t *__restrict__ o, __half *__restrict__ scale_out,
                                                  __half *__restrict__ zp_out) {
   const float qmax = (float)((1 << BITS) - 1);
   float mn = INFINITY, mx = -INFINITY;
   for (int c = lane; c < D; c += 64) {
-    float v = __half2float(xr[c]);
+    float v = In::get(xr, c);
     mn = fminf(mn, v);
     mx = fmaxf(mx, v);
   }
@@ -34,29 +51,29 @@ __device__ __forceinline__ void quantize_one_row(const __half *__restrict__ xr, 
     *zp_out = __float2half_rn(p.zp);
   }
   if (!pack || BITS == 8) {
-    for (int c = lane; c < D; c += 64) o[c] = (uint8_t)rdkv_qcode(__half2float(xr[c]), p, qmax);
+    for (int c = lane; c < D; c += 64) o[c] = (uint8_t)rdkv_qcode(In::get(xr, c), p, qmax);
   } else if (BITS == 4) {
     const int n = D >> 1;
     for (int i = lane; i < n; i += 64) {
-      uint32_t lo = rdkv_qcode(__half2float(xr[i]), p, qmax);
-      uint32_t hi = rdkv_qcode(__half2float(xr[i + n]), p, qmax);
+      uint32_t lo = rdkv_qcode(In::get(xr, i), p, qmax);
+      uint32_t hi = rdkv_qcode(In::get(xr, i + n), p, qmax);
       o[i] = (uint8_t)(lo | (hi << 4));
     }
   } else {
     const int n = D >> 2;
     for (int i = lane; i < n; i += 64) {
-      uint32_t b = rdkv_qcode(__half2float(xr[i]), p, qmax);
-      b |= rdkv_qcode(__half2float(xr[i + n]), p, qmax) << 2;
-      b |= rdkv_qcode(__half2float(xr[i + 2 * n]), p, qmax) << 4;
-      b |= rdkv_qcode(__half2float(xr[i + 3 * n]), p, qmax) << 6;
+      uint32_t b = rdkv_qcode(In::get(xr, i), p, qmax);
+      b |= rdkv_qcode(In::get(xr, i + n), p, qmax) << 2;
+      b |= rdkv_qcode(In::get(xr, i + 2 * n), p, qmax) << 4;
+      b |= rdkv_qcode(In::get(xr, i + 3 * n), p, qmax) << 6;
       o[i] = (uint8_t)b;
     }
   }
 }
 
-template <int BITS>
+template <int BITS, typename In>
 __global__ void __launch_bounds__(256)
-quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
+quantize_rows_kernel(const typename In::raw *__restrict__ x, int64_t x_row_stride,
                      const int64_t *__restrict__ row_idx, int64_t rows, int D, int pack,
                      uint8_t *__restrict__ out, __half *__restrict__ scale_out,
                      __half *__restrict__ zp_out) {
@@ -65,8 +82,8 @@ quantize_rows_kernel(const __half *__restrict__ x, int64_t x_row_stride,
   if (r >= rows) return;
   const int64_t src = row_idx ? row_idx[r] : r;
   const int width = (!pack || BITS == 8) ? D : (BITS == 4 ? D >> 1 : D >> 2);
-  quantize_one_row<BITS>(x + src * x_row_stride, D, pack, lane, out + r * (int64_t)width, scale_out + r,
-                         zp_out + r);
+  quantize_one_row<BITS, In>(x + src * x_row_stride, D, pack, lane, out + r * (int64_t)width, scale_out + r,
+                             zp_out + r);
 }
 
 // ---------------------------------------------------------------------------
@@ -474,6 +491,40 @@ col_minmax_kernel(const __half *__restrict__ x, int64_t x_row_stride, int64_t T,
   }
 }
 
+// The same reduction for bf16 / fp32 rows (any alignment): one column per thread.
+template <typename In>
+__global__ void __launch_bounds__(256)
+col_minmax_any_kernel(const typename In::raw *__restrict__ x, int64_t x_row_stride, int64_t T, int D,
+                      uint32_t *__restrict__ mm) {
+  // blockDim = (64, 4): threadIdx.x walks columns, threadIdx.y walks rows.
+  const int64_t t0 = (int64_t)blockIdx.x * RDKV_MINMAX_ROWS;
+  const int64_t t1 = (t0 + RDKV_MINMAX_ROWS < T) ? t0 + RDKV_MINMAX_ROWS : T;
+  __shared__ float s_mn[4][64], s_mx[4][64];
+  for (int c0 = 0; c0 < D; c0 += 64) {
+    const int c = c0 + threadIdx.x;
+    float mn = INFINITY, mx = -INFINITY;
+    if (c < D) {
+      for (int64_t t = t0 + threadIdx.y; t < t1; t += 4) {
+        const float a = In::get(x, t * x_row_stride + c);
+        mn = fminf(mn, a);
+        mx = fmaxf(mx, a);
+      }
+    }
+    s_mn[threadIdx.y][threadIdx.x] = mn;
+    s_mx[threadIdx.y][threadIdx.x] = mx;
+    __syncthreads();
+    if (threadIdx.y == 0 && c < D) {
+      for (int y = 1; y < 4; ++y) {
+        mn = fminf(mn, s_mn[y][threadIdx.x]);
+        mx = fmaxf(mx, s_mx[y][threadIdx.x]);
+      }
+      atomicMin(&mm[c], rdkv_float_to_ordered(mn));
+      atomicMax(&mm[D + c], rdkv_float_to_ordered(mx));
+    }
+    __syncthreads();
+  }
+}
+
 __global__ void minmax_finalize_kernel(uint32_t *mm, int n) {
   int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c < n) reinterpret_cast<float *>(mm)[c] = rdkv_ordered_to_float(mm[c]);
@@ -484,8 +535,9 @@ __global__ void minmax_finalize_kernel(uint32_t *mm, int n) {
 // One thread per output byte.
 // ---------------------------------------------------------------------------
 #define RDKV_MAX_SLOTS 1024
+template <typename In>
 __global__ void __launch_bounds__(256)
-k_quantize_pack_kernel(const __half *__restrict__ k, int64_t k_row_stride, int64_t T, int D,
+k_quantize_pack_kernel(const typename In::raw *__restrict__ k, int64_t k_row_stride, int64_t T, int D,
                        const float *__restrict__ minmax, const int32_t *__restrict__ slot_channel,
                        int n2p, int n4p, int n8, uint8_t *__restrict__ K2, uint8_t *__restrict__ K4,
                        uint8_t *__restrict__ K8, __half *__restrict__ scale_out,
@@ -516,9 +568,9 @@ k_quantize_pack_kernel(const __half *__restrict__ k, int64_t k_row_stride, int64
   const int64_t t0 = (int64_t)blockIdx.x * rows_per_block;
   const int64_t t1 = (t0 + rows_per_block < T) ? t0 + rows_per_block : T;
   const int64_t total = (t1 - t0) * rowbytes;
-  auto code = [&](const __half *kr, int s, float qmax) -> uint32_t {
+  auto code = [&](const typename In::raw *kr, int s, float qmax) -> uint32_t {
     const int ch = s_ch[s];
-    const float x = ch >= 0 ? __half2float(kr[ch]) : 0.0f;
+    const float x = ch >= 0 ? In::get(kr, ch) : 0.0f;
     RdkvQParams p;
     p.scale = s_scale[s];
     p.zp = s_zp[s];
@@ -528,7 +580,7 @@ k_quantize_pack_kernel(const __half *__restrict__ k, int64_t k_row_stride, int64
   for (int64_t idx = threadIdx.x; idx < total; idx += blockDim.x) {
     const int64_t t = t0 + idx / rowbytes;
     const int j = (int)(idx % rowbytes);
-    const __half *kr = k + t * k_row_stride;
+    const typename In::raw *kr = k + t * k_row_stride;
     if (j < sub2) {
       uint32_t b = code(kr, j, 3.0f);
       b |= code(kr, j + sub2, 3.0f) << 2;
@@ -1047,73 +1099,97 @@ dequant_f16_kernel(const uint8_t *__restrict__ packed, int64_t rows, int ncols,
 
 }  // namespace
 
-RDKV_API int rdkv_quantize_rows(const void *x_f16, int64_t x_row_stride, const int64_t *row_idx,
+RDKV_API int rdkv_quantize_rows(const void *x, int x_dtype, int64_t x_row_stride, const int64_t *row_idx,
                                 int64_t rows, int D, int n_bits, int pack, uint8_t *out,
                                 void *scale_f16, void *zp_f16, void *stream) {
   RDKV_REQUIRE(n_bits == 2 || n_bits == 4 || n_bits == 8, "rdkv_quantize_rows: n_bits=%d not in {2,4,8}",
                n_bits);
+  RDKV_REQUIRE(x_dtype >= 0 && x_dtype <= 2, "rdkv_quantize_rows: unknown input dtype %d", x_dtype);
   RDKV_REQUIRE(rows >= 0 && D > 0, "rdkv_quantize_rows: bad shape rows=%lld D=%d", (long long)rows, D);
   RDKV_REQUIRE(!pack || n_bits == 8 || D % (8 / n_bits) == 0,
                "rdkv_quantize_rows: D=%d not divisible by %d for %d-bit packing", D, 8 / n_bits, n_bits);
   if (rows == 0) return RDKV_OK;
-  RDKV_REQUIRE(x_f16 && out && scale_f16 && zp_f16, "rdkv_quantize_rows: null pointer");
+  RDKV_REQUIRE(x && out && scale_f16 && zp_f16, "rdkv_quantize_rows: null pointer");
   const int waves = 4;
   int64_t blocks = rdkv_cdiv(rows, waves);
   RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_quantize_rows: too many rows");
   dim3 g((unsigned)blocks), b(64 * waves);
   hipStream_t s = (hipStream_t)stream;
-  const __half *x = (const __half *)x_f16;
   __half *sc = (__half *)scale_f16, *zp = (__half *)zp_f16;
-  if (n_bits == 2)
-    hipLaunchKernelGGL(quantize_rows_kernel<2>, g, b, 0, s, x, x_row_stride, row_idx, rows, D, pack, out, sc, zp);
-  else if (n_bits == 4)
-    hipLaunchKernelGGL(quantize_rows_kernel<4>, g, b, 0, s, x, x_row_stride, row_idx, rows, D, pack, out, sc, zp);
-  else
-    hipLaunchKernelGGL(quantize_rows_kernel<8>, g, b, 0, s, x, x_row_stride, row_idx, rows, D, pack, out, sc, zp);
+#define RDKV_LAUNCH_QROWS(BITS, IN)                                                                          \
+  hipLaunchKernelGGL((quantize_rows_kernel<BITS, IN>), g, b, 0, s, (const IN::raw *)x, x_row_stride, row_idx, \
+                     rows, D, pack, out, sc, zp)
+#define RDKV_LAUNCH_QROWS_IN(IN)                 \
+  do {                                           \
+    if (n_bits == 2) RDKV_LAUNCH_QROWS(2, IN);   \
+    else if (n_bits == 4) RDKV_LAUNCH_QROWS(4, IN); \
+    else RDKV_LAUNCH_QROWS(8, IN);               \
+  } while (0)
+  if (x_dtype == RDKV_DTYPE_F16) RDKV_LAUNCH_QROWS_IN(InF16);
+  else if (x_dtype == RDKV_DTYPE_BF16) RDKV_LAUNCH_QROWS_IN(InBF16);
+  else RDKV_LAUNCH_QROWS_IN(InF32);
+#undef RDKV_LAUNCH_QROWS_IN
+#undef RDKV_LAUNCH_QROWS
   RDKV_CHECK_LAUNCH("rdkv_quantize_rows");
   return RDKV_OK;
 }
 
-RDKV_API int rdkv_col_minmax(const void *x_f16, int64_t x_row_stride, int64_t T, int D, float *minmax,
+RDKV_API int rdkv_col_minmax(const void *x, int x_dtype, int64_t x_row_stride, int64_t T, int D, float *minmax,
                              void *stream) {
   RDKV_REQUIRE(T >= 0 && D > 0 && minmax, "rdkv_col_minmax: bad arguments");
-  RDKV_REQUIRE(x_row_stride % 2 == 0 && ((uintptr_t)x_f16 % 4) == 0,
-               "rdkv_col_minmax: rows must be 4-byte aligned");
+  RDKV_REQUIRE(x_dtype >= 0 && x_dtype <= 2, "rdkv_col_minmax: unknown input dtype %d", x_dtype);
   hipStream_t s = (hipStream_t)stream;
   uint32_t *mm = reinterpret_cast<uint32_t *>(minmax);
   hipLaunchKernelGGL(minmax_init_kernel, dim3((D + 255) / 256), dim3(256), 0, s, mm, D);
   if (T > 0) {
-    RDKV_REQUIRE(x_f16, "rdkv_col_minmax: null input");
+    RDKV_REQUIRE(x, "rdkv_col_minmax: null input");
     int64_t blocks = rdkv_cdiv(T, RDKV_MINMAX_ROWS);
     RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_col_minmax: too many rows");
-    hipLaunchKernelGGL(col_minmax_kernel, dim3((unsigned)blocks), dim3(64, 4), 0, s,
-                       (const __half *)x_f16, x_row_stride, T, D, mm);
+    // fp16 rows that start on 4-byte boundaries are read two channels at a time
+    if (x_dtype == RDKV_DTYPE_F16 && x_row_stride % 2 == 0 && ((uintptr_t)x % 4) == 0)
+      hipLaunchKernelGGL(col_minmax_kernel, dim3((unsigned)blocks), dim3(64, 4), 0, s, (const __half *)x,
+                         x_row_stride, T, D, mm);
+    else if (x_dtype == RDKV_DTYPE_F16)
+      hipLaunchKernelGGL(col_minmax_any_kernel<InF16>, dim3((unsigned)blocks), dim3(64, 4), 0, s,
+                         (const __half *)x, x_row_stride, T, D, mm);
+    else if (x_dtype == RDKV_DTYPE_BF16)
+      hipLaunchKernelGGL(col_minmax_any_kernel<InBF16>, dim3((unsigned)blocks), dim3(64, 4), 0, s,
+                         (const uint16_t *)x, x_row_stride, T, D, mm);
+    else
+      hipLaunchKernelGGL(col_minmax_any_kernel<InF32>, dim3((unsigned)blocks), dim3(64, 4), 0, s,
+                         (const float *)x, x_row_stride, T, D, mm);
   }
   hipLaunchKernelGGL(minmax_finalize_kernel, dim3((2 * D + 255) / 256), dim3(256), 0, s, mm, 2 * D);
   RDKV_CHECK_LAUNCH("rdkv_col_minmax");
   return RDKV_OK;
 }
 
-RDKV_API int rdkv_k_quantize_pack(const void *k_f16, int64_t k_row_stride, int64_t T, int D,
+RDKV_API int rdkv_k_quantize_pack(const void *k, int k_dtype, int64_t k_row_stride, int64_t T, int D,
                                   const float *minmax, const int32_t *slot_channel, int n2p, int n4p,
                                   int n8, uint8_t *K2, uint8_t *K4, uint8_t *K8, void *scale_f16,
                                   void *zp_f16, void *stream) {
   RDKV_REQUIRE(n2p >= 0 && n4p >= 0 && n8 >= 0 && n2p % 4 == 0 && n4p % 2 == 0,
                "rdkv_k_quantize_pack: bad segment sizes (%d,%d,%d)", n2p, n4p, n8);
+  RDKV_REQUIRE(k_dtype >= 0 && k_dtype <= 2, "rdkv_k_quantize_pack: unknown input dtype %d", k_dtype);
   const int Dp = n2p + n4p + n8;
   RDKV_REQUIRE(Dp <= RDKV_MAX_SLOTS, "rdkv_k_quantize_pack: %d padded channels > %d", Dp, RDKV_MAX_SLOTS);
   RDKV_REQUIRE(T >= 0 && D > 0, "rdkv_k_quantize_pack: bad shape");
   if (Dp == 0) return RDKV_OK;
   RDKV_REQUIRE(minmax && slot_channel && scale_f16 && zp_f16, "rdkv_k_quantize_pack: null pointer");
-  RDKV_REQUIRE(T == 0 || (k_f16 && (n2p == 0 || K2) && (n4p == 0 || K4) && (n8 == 0 || K8)),
+  RDKV_REQUIRE(T == 0 || (k && (n2p == 0 || K2) && (n4p == 0 || K4) && (n8 == 0 || K8)),
                "rdkv_k_quantize_pack: null data pointer");
   const int rows_per_block = 64;
   int64_t blocks = T > 0 ? rdkv_cdiv(T, rows_per_block) : 1;
   RDKV_REQUIRE(blocks <= 0x7fffffffLL, "rdkv_k_quantize_pack: too many rows");
   size_t shmem = (size_t)Dp * 12;
-  hipLaunchKernelGGL(k_quantize_pack_kernel, dim3((unsigned)blocks), dim3(256), shmem, (hipStream_t)stream,
-                     (const __half *)k_f16, k_row_stride, T, D, minmax, slot_channel, n2p, n4p, n8, K2, K4,
-                     K8, (__half *)scale_f16, (__half *)zp_f16, rows_per_block);
+#define RDKV_LAUNCH_KQP(IN)                                                                                     \
+  hipLaunchKernelGGL(k_quantize_pack_kernel<IN>, dim3((unsigned)blocks), dim3(256), shmem, (hipStream_t)stream, \
+                     (const IN::raw *)k, k_row_stride, T, D, minmax, slot_channel, n2p, n4p, n8, K2, K4, K8,    \
+                     (__half *)scale_f16, (__half *)zp_f16, rows_per_block)
+  if (k_dtype == RDKV_DTYPE_F16) RDKV_LAUNCH_KQP(InF16);
+  else if (k_dtype == RDKV_DTYPE_BF16) RDKV_LAUNCH_KQP(InBF16);
+  else RDKV_LAUNCH_KQP(InF32);
+#undef RDKV_LAUNCH_KQP
   RDKV_CHECK_LAUNCH("rdkv_k_quantize_pack");
   return RDKV_OK;
 }

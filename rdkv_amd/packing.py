@@ -103,10 +103,11 @@ def _seg_padded_len(n: int, align: int) -> int:
 
 def _quantize_rows(x2d: Tensor, n_bits: int, pack: bool, row_idx: Optional[Tensor] = None,
                    rows: Optional[int] = None):
-    """x2d: fp16 [R, D] with unit channel stride.  Returns (codes|packed [rows, *], scale, zp [rows])."""
+    """x2d: fp16 / bf16 / fp32 [R, D] with unit channel stride.  Returns (codes|packed [rows, *], scale,
+    zp [rows])."""
     dev = _lib.require_device(x2d)
     # (the stride of a dimension of size one carries no information and may be anything)
-    assert x2d.dtype == torch.float16 and (x2d.shape[-1] == 1 or x2d.stride(-1) == 1)
+    assert x2d.dtype in _lib.DTYPE_CODE and (x2d.shape[-1] == 1 or x2d.stride(-1) == 1)
     D = x2d.shape[1]
     rows = x2d.shape[0] if rows is None else rows
     width = D * n_bits // 8 if pack else D
@@ -114,9 +115,16 @@ def _quantize_rows(x2d: Tensor, n_bits: int, pack: bool, row_idx: Optional[Tenso
     scale = torch.empty(rows, dtype=torch.float16, device=dev)
     zp = torch.empty(rows, dtype=torch.float16, device=dev)
     _lib.check(_lib.load().rdkv_quantize_rows(
-        x2d.data_ptr(), x2d.stride(0), _lib.ptr(row_idx), rows, D, n_bits, int(pack),
+        x2d.data_ptr(), _lib.DTYPE_CODE[x2d.dtype], x2d.stride(0), _lib.ptr(row_idx), rows, D, n_bits, int(pack),
         _lib.ptr(out), _lib.ptr(scale), _lib.ptr(zp), _lib.stream_of(dev)))
     return out, scale, zp
+
+
+def _as_quantizer_input(x: Tensor) -> Tensor:
+    """The tensor the quantizer kernels read: fp16, bf16 and fp32 as they are (the kernels widen each
+    element to fp32, which is the reference's ``x.float()``, packing.py:153); anything else through
+    ``float()`` as the reference does.  No input is rounded to a narrower type."""
+    return x if x.dtype in _lib.DTYPE_CODE else x.float()
 
 
 def _require_rows_to_reduce(n: int, dim: int) -> None:
@@ -138,7 +146,7 @@ def quantize_and_pack(x: Tensor, n_bits: int, dim: int) -> Tuple[Tensor, Tensor,
     _lib.require_device(x)
     dim = dim % x.dim()
     _require_rows_to_reduce(int(x.shape[dim]), dim)
-    xt = x.to(torch.float16).movedim(dim, -1).contiguous()
+    xt = _as_quantizer_input(x).movedim(dim, -1).contiguous()
     lead = xt.shape[:-1]
     codes, scale, zp = _quantize_rows(xt.reshape(-1, xt.shape[-1]), n_bits, pack=False)
     codes = codes.reshape(*lead, xt.shape[-1]).movedim(-1, dim).contiguous()
@@ -193,7 +201,7 @@ def _plan_k_channels(k_bits: Sequence[int], sub_2_target=None, sub_4_target=None
 
 
 def _k_emit(K_h: Tensor, plan: _KPlan):
-    """Quantize + pack one head: K_h fp16 [T, D] (unit channel stride) -> segment tensors."""
+    """Quantize + pack one head: K_h fp16 / bf16 / fp32 [T, D] (unit channel stride) -> segment tensors."""
     dev = K_h.device
     lib = _lib.load()
     stream = _lib.stream_of(dev)
@@ -208,15 +216,24 @@ def _k_emit(K_h: Tensor, plan: _KPlan):
     if Dp:
         minmax = torch.empty(2 * D, dtype=torch.float32, device=dev)
         slot_ch = torch.tensor(plan.slot_channel, dtype=torch.int32, device=dev)
-        _lib.check(lib.rdkv_col_minmax(K_h.data_ptr(), K_h.stride(0), T, D, minmax.data_ptr(), stream))
+        dt = _lib.DTYPE_CODE[K_h.dtype]
+        _lib.check(lib.rdkv_col_minmax(K_h.data_ptr(), dt, K_h.stride(0), T, D, minmax.data_ptr(), stream))
         _lib.check(lib.rdkv_k_quantize_pack(
-            K_h.data_ptr(), K_h.stride(0), T, D, minmax.data_ptr(), slot_ch.data_ptr(),
+            K_h.data_ptr(), dt, K_h.stride(0), T, D, minmax.data_ptr(), slot_ch.data_ptr(),
             n2p, n4p, n8, _lib.ptr(K2), _lib.ptr(K4), _lib.ptr(K8),
             scale.data_ptr(), zp.data_ptr(), stream))
     return K2, K4, K8, scale, zp
 
 
+def _as_heads(K: Tensor) -> Tensor:
+    """[1, H, T, D] input of a per-segment packer in a type the kernels read, unit channel stride."""
+    K = _as_quantizer_input(K)
+    return K if K.stride(-1) == 1 else K.contiguous()
+
+
 def _as_f16_heads(K: Tensor) -> Tensor:
+    """fp16 rows with unit channel stride, for the whole-layer packer's kernels (callers pass fp16, or
+    K on its way into the reference's fp16 canvas, packing.py:1186-1190)."""
     K = K.to(torch.float16)
     return K if K.stride(-1) == 1 else K.contiguous()
 
@@ -226,7 +243,8 @@ def pack_k_mixed(K: Tensor, k_bits: Tensor, *, sub_2_target: Optional[int] = Non
                  segment_counts: Optional[Tuple[int, int, int]] = None):
     """Per-channel mixed-precision K packer (packing.py:177-391).
 
-    K [1,H,T,D] fp16, k_bits [D] in {0,2,4,8,16} -> (K_2bit, K_4bit, K_8bit, K_ch_scale,
+    K [1,H,T,D] (fp16; bf16 / fp32 values are quantized as they are, packing.py:153), k_bits [D] in
+    {0,2,4,8,16} -> (K_2bit, K_4bit, K_8bit, K_ch_scale,
     K_ch_zp, ch_sort_idx, ch_perm_padded_idx, (n2,n4,n8)).  Channels are quantized over all
     T rows (dim=2), pad channels are zero columns (scale fp16 0, zp 0, codes 0).
     """
@@ -237,7 +255,7 @@ def pack_k_mixed(K: Tensor, k_bits: Tensor, *, sub_2_target: Optional[int] = Non
                             n_ch_8_target, segment_counts)
     if sum(plan.padded) > 0:
         _require_rows_to_reduce(T, 2)
-    Kf = _as_f16_heads(K)
+    Kf = _as_heads(K)
     heads = [_k_emit(Kf[0, h], plan) for h in range(H)]
     n2p, n4p, n8o = plan.padded
 
@@ -290,7 +308,7 @@ def pack_k_mixed_per_head(K: Tensor, k_bits_ph: Tensor):
     Dp = 4 * sub2 + 2 * sub4 + m8
     if Dp > 0:
         _require_rows_to_reduce(T, 2)
-    Kf = _as_f16_heads(K)
+    Kf = _as_heads(K)
     heads = [_k_emit(Kf[0, h], plans[h]) for h in range(H)]
 
     def stack(i, width):
@@ -368,7 +386,7 @@ def pack_v_segments(V: Tensor, v_bits: Tensor, *,
                     segment_counts: Optional[Tuple[int, int, int]] = None):
     """Stable-sort tokens by bit-width and pack each V segment per token (packing.py:715-778).
 
-    V [1,H,T,D] fp16, v_bits [T] in {2,4,8} -> (V_2bit, V_4bit, V_8bit, V_scale, V_zp, sort_idx,
+    V [1,H,T,D] (fp16; bf16 / fp32 values are quantized as they are), v_bits [T] in {2,4,8} -> (V_2bit, V_4bit, V_8bit, V_scale, V_zp, sort_idx,
     (N_2,N_4,N_8)).  The token gather is fused into the quantize kernel.
     """
     dev = _lib.require_device(V)
@@ -381,7 +399,7 @@ def pack_v_segments(V: Tensor, v_bits: Tensor, *,
     else:
         N2, N4, N8 = (int(v) for v in segment_counts)
     assert N2 + N4 + N8 == T, f"Segment sizes {N2}+{N4}+{N8} != T_eff={T}"
-    Vf = _as_f16_heads(V)
+    Vf = _as_heads(V)
     segs = {2: [], 4: [], 8: []}
     scales: List[List[Tensor]] = [[] for _ in range(H)]
     zps: List[List[Tensor]] = [[] for _ in range(H)]
@@ -604,6 +622,11 @@ def _pad_and_stack_per_head_layers(
         softmax_mask = torch.empty(H_q, 0, dtype=torch.float32, device=dev)
 
     if max_n16 > 0:
+        for v16 in per_head_v16_V:
+            if v16 is not None and v16.dtype != torch.float16:
+                # (the reference keeps such rows in their own type; the V kernels here read fp16 rows,
+                # and rounding them silently would change the values attended over)
+                raise TypeError(f"fp16-kept V rows must be fp16, got {v16.dtype}: cast V to fp16 before packing")
         new_v_only = torch.cat([_pad_rows(per_head_v16_V[h], n16[h] if per_head_v16_V[h] is not None else 0,
                                           max_n16, head_dim, torch.float16, dev)
                                 for h in range(H_kv)], dim=1).contiguous()
@@ -705,7 +728,12 @@ def _pack_planned_layer(K: Tensor, V: Tensor, gqa_factor: int, planned, first: i
     Dp = 4 * sub2 + 2 * sub4 + m8
     if max_tk == 0 or Dp == 0 or D > 1024:
         return None
-    Kf, Vf = _as_f16_heads(K)[0], _as_f16_heads(V)[0]
+    if V.dtype != torch.float16:
+        # V rows are quantized from the values as given (packing.py:153), which the whole-layer V
+        # kernel only does for fp16 storage: such a layer takes the per-segment composition.  K goes
+        # through the reference's fp16 canvas (packing.py:1186-1190) whatever its type.
+        return None
+    Kf, Vf = _as_f16_heads(K)[0], V[0] if V.stride(-1) == 1 else V.contiguous()[0]
     if Vf.stride() != Kf.stride():
         Kf, Vf = Kf.contiguous(), Vf.contiguous()
     ref = next((h for h in range(H_kv) if tk[h] > 0), 0)
@@ -794,8 +822,10 @@ def pack_layer_per_head(K: Tensor, V: Tensor, v_bits_per_head: Tensor, k_bits_pe
     bit for bit, without the per-head loop: ``rdkv_pack_layer_plan`` (stable token order by class
     and all class sizes, read once by the host to size the tensors), ``rdkv_pack_layer_tables``
     (channel tables, per-head metadata, padding mask) and ``rdkv_pack_layer_per_head`` (V rows, K
-    min/max, K emit).  K, V [1,H_kv,T,D] fp16;
-    v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
+    min/max, K emit).  K, V [1,H_kv,T,D] fp16 (K of another type is rounded to fp16 first, which is
+    what the reference's fp16 canvas does to it, packing.py:1186-1190; V of another type is quantized
+    from its own values by the per-segment composition, and its fp16-kept rows are refused with
+    TypeError); v_bits [H_kv,T] in {0,2,4,8,16}; k_bits [H_kv,D].  Returns (layer, new_v_only)."""
     dev = _lib.require_device(K, V)
     assert K.dim() == 4 and K.shape[0] == 1 and K.shape == V.shape, (
         f"Expected K, V [1,H_kv,T,D], got {tuple(K.shape)} / {tuple(V.shape)}")

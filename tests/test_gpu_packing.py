@@ -313,3 +313,102 @@ def test_whole_layer_packer_matches_composition(case):
     _layers_identical(one[0], exp)
     if exp_nvo is not None:
         assert torch.equal(one[1].view(torch.uint8), exp_nvo.view(torch.uint8))
+
+
+def _bf16_values(a32):
+    """fp32 array -> the nearest bf16 values (round to nearest even), still as fp32."""
+    u = np.ascontiguousarray(a32, np.float32).view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32)
+
+
+def _typed_inputs(seed, shape, kind, big=True):
+    """Values that a rounding to fp16 would change (fp32: 24-bit mantissas and magnitudes outside
+    fp16's range; bf16: exponents fp16 does not have), the NumPy array the oracle sees (fp32 values)
+    and the device tensor in its storage type."""
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal(shape) * rng.uniform(0.01, 30, shape[:-1] + (1,))).astype(np.float32)
+    x[..., 0, :] *= 1e-6                     # below fp16's normal range
+    if big:
+        x[..., 1, :] *= 3e3                  # beyond 65504 here and there
+    if kind == "bf16":
+        x = _bf16_values(x)
+        t = torch.from_numpy(x).to(torch.bfloat16)
+        assert np.array_equal(t.float().numpy(), x)
+    else:
+        t = torch.from_numpy(x)
+    assert not np.array_equal(x.astype(np.float16).astype(np.float32), x)
+    return x, t.to(DEV)
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+def test_packers_quantize_the_values_as_given(kind):
+    """packing.py:153 widens whatever it is given to fp32 and quantizes that: fp32 and bf16 inputs
+    are not rounded to fp16 on the way.  Every per-segment packer against the oracle on the same
+    values, bit for bit."""
+    x, xd = _typed_inputs(31, (1, 3, 130, 128), kind)
+    for bits in (2, 4, 8):
+        for dim in (2, 3):
+            q, s, z = packing.quantize_and_pack(xd, bits, dim)
+            eq, es, ez = O.quantize_and_pack(x, bits, dim)
+            assert_bits_equal(t2n(q), eq, f"codes b{bits} d{dim}")
+            assert_bits_equal(t2n(s), es, f"scale b{bits} d{dim}")
+            assert_bits_equal(t2n(z), ez, f"zp b{bits} d{dim}")
+    rng = np.random.default_rng(32)
+    kb = rng.choice([0, 2, 4, 8, 16], size=128).astype(np.int64)
+    got = packing.pack_k_mixed(xd, torch.from_numpy(kb))
+    exp = O.pack_k_mixed(x, kb)
+    for i, (a, b) in enumerate(zip(got[:7], exp[:7])):
+        if b is None:
+            assert a is None
+        else:
+            assert_bits_equal(t2n(a), b, f"pack_k_mixed[{i}]")
+    kb_ph = rng.choice([0, 2, 4, 8], size=(3, 128)).astype(np.int64)
+    got = packing.pack_k_mixed_per_head(xd, torch.from_numpy(kb_ph))
+    exp = O.pack_k_mixed_per_head(x, kb_ph)
+    for i, (a, b) in enumerate(zip(got[:8], exp[:8])):
+        if b is None:
+            assert a is None
+        else:
+            assert_bits_equal(t2n(a), np.asarray(b), f"pack_k_mixed_per_head[{i}]")
+    vb = rng.choice([2, 4, 8], size=130).astype(np.int64)
+    got = packing.pack_v_segments(xd, torch.from_numpy(vb))
+    exp = O.pack_v_segments(x, vb)
+    for i, (a, b) in enumerate(zip(got[:6], exp[:6])):
+        if b is None:
+            assert a is None
+        else:
+            assert_bits_equal(t2n(a), b, f"pack_v_segments[{i}]")
+
+
+@pytest.mark.parametrize("kind", ["f32", "bf16"])
+def test_layer_packers_on_other_input_types(kind):
+    """``build_packed_layer`` quantizes K and V from their own values; the per-head composition sends
+    K through the reference's fp16 canvas (packing.py:1186-1190) and quantizes V from its own values;
+    fp16-kept V rows of another type are refused instead of being rounded."""
+    k, kd = _typed_inputs(41, (1, 2, 90, 128), kind)
+    v, vd = _typed_inputs(42, (1, 2, 90, 128), kind)
+    rng = np.random.default_rng(43)
+    vb = rng.choice([0, 2, 4, 8], size=90).astype(np.int64)
+    kb = rng.choice([0, 2, 4, 8, 16], size=128).astype(np.int64)
+    pl, tk, v16 = packing.build_packed_layer(kd, vd, torch.from_numpy(vb), torch.from_numpy(kb))
+    epl, etk, ev16 = O.build_packed_layer(k, v, vb, kb)
+    assert tk == etk and v16 is None and ev16 is None
+    assert_layers_equal(pl, epl)
+    # (K inside fp16's range from here on: the canvas would turn larger values into infinities)
+    k, kd = _typed_inputs(44, (1, 2, 90, 128), kind, big=False)
+    vb_ph = rng.choice([0, 2, 4, 8], size=(2, 90)).astype(np.int64)
+    kb_ph = rng.choice([0, 2, 4, 8], size=(2, 128)).astype(np.int64)
+    pl, nvo = packing.pack_layer_per_head(kd, vd, torch.from_numpy(vb_ph), torch.from_numpy(kb_ph), 4)
+    epl, envo = O.pack_layer_per_head(k, v, vb_ph, kb_ph, 4)
+    assert nvo is None and envo is None
+    assert_layers_equal(pl, epl)
+    # K of another type beside fp16 V takes the whole-layer kernels (K through fp16, as the canvas does)
+    v16_in = v.astype(np.float16)
+    vb_ph[:, ::7] = 16
+    pl, nvo = packing.pack_layer_per_head(kd, to_dev(v16_in), torch.from_numpy(vb_ph), torch.from_numpy(kb_ph), 4)
+    epl, envo = O.pack_layer_per_head(k, v16_in, vb_ph, kb_ph, 4)
+    assert_layers_equal(pl, epl)
+    assert_bits_equal(t2n(nvo), envo, "new_v_only")
+    with pytest.raises(TypeError, match="fp16-kept V rows"):
+        packing.pack_layer_per_head(kd, vd, torch.from_numpy(vb_ph), torch.from_numpy(kb_ph), 4)

@@ -74,7 +74,7 @@ def test_argument_errors_without_device_work():
     assert lib.rdkv_bitpack2(None, None, 1, 6, None) == _lib.RDKV_EINVAL
     assert b"multiple of 4" in lib.rdkv_last_error()
     with pytest.raises(AssertionError):
-        _lib.check(lib.rdkv_quantize_rows(None, 0, None, 1, 128, 3, 1, None, None, None, None))
+        _lib.check(lib.rdkv_quantize_rows(None, 1, 0, None, 1, 128, 3, 1, None, None, None, None))
 
 
 def test_product_does_not_import_oracle():

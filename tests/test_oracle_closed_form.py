@@ -159,3 +159,23 @@ def test_attention_special_cases():
     b = O.algorithmic_bytes(pl, H_kv * G)
     per_head = (8 + 4 + 4 + 4) * 128 + 4 * 128 + 32 * 4 + 64 * 4 + 128 * 8 + 4 * 16 + 256 * 4
     assert b == H_kv * per_head + H_kv * G * 128 * 6
+
+
+def test_quantizer_takes_fp32_values_as_given():
+    """packing.py:153 widens its input to fp32 and never rounds it to fp16 first.  A row whose codes
+    differ between the two readings, worked by hand: x = (0, 1 + 2^-12, 3) at 2 bits has scale 1,
+    zero point 0 and x[1] / scale = 1.000244 -> code 1; rounded to fp16 first x[1] would be 1.0
+    (same code), so take x[1] = 1.5 + 2^-12: the fp32 value rounds to code 2, the fp16 rounding
+    1.5 is a tie and rounds to the even code 2 as well; x[1] = 0.5 + 2^-13 separates them: fp32
+    -> code 1, fp16 (0.5, a tie) -> code 0."""
+    x = np.array([[0.0, 0.5 + 2.0 ** -13, 3.0]], np.float32)
+    q, s, z = O.quantize_and_pack(x, 2, 1)
+    assert q.tolist() == [[0, 1, 3]] and float(s[0, 0]) == 1.0 and float(z[0, 0]) == 0.0
+    q16, _, _ = O.quantize_and_pack(x.astype(np.float16), 2, 1)
+    assert q16.tolist() == [[0, 0, 3]]
+    # magnitudes outside fp16's range keep their fp32 range: scale = (1e6 - 0) / 255
+    big = np.array([[0.0, 1.0e6, 5.0e5]], np.float32)
+    q, s, z = O.quantize_and_pack(big, 8, 1)
+    assert q.tolist() == [[0, 255, 128]] or q.tolist() == [[0, 255, 127]]
+    assert q[0, 2] == int(np.round(np.float32(5.0e5) / (np.float32(1.0e6) / np.float32(255.0))))
+    assert np.isclose(float(s[0, 0]), 1.0e6 / 255.0, rtol=1e-3)
