@@ -126,8 +126,13 @@ def build_workload(cfg, dev, torch, on_first=None, pack_sample=None):
 
 
 def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True):
-    """ms per step of the fused call (streaming launch + merge launch) issued eagerly and replayed
-    from a HIP graph, and ms per launch of the streaming kernel alone."""
+    """The timed region of the fused step.  Every step is the library's two launches (streaming
+    kernel, then merge) issued eagerly, with a HIP event on the same stream before and after the
+    streaming launch: ms per step is the whole region divided by its steps, ms per launch of the
+    streaming kernel is the mean of the in-step event intervals - one loop gives both, so the kernel
+    can never come out slower than the step that contains it.  Beside it: the same step through
+    ``decode_attn_fused`` without the inner events (what they cost), and replayed from a HIP graph.
+    Returns (step, ms_step, ms_kernel, extras)."""
     from rdkv_amd import _lib, stream_cache
     lib = _lib.load()
     dev = qs.device
@@ -145,26 +150,36 @@ def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True):
         for _ in range(20):
             step()
         torch.cuda.synchronize()
-    ms_eager = time_region(step, steps, torch)
-    ms_graph = None
+    ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
+    stream = _lib.stream_of(dev)
+    q_dt = _lib.DTYPE_CODE[qs.dtype]
+    before = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    after = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(steps):
+        before[i].record()
+        _lib.check(lib.rdkv_decode_fused_partials(
+            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
+            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords, qs.data_ptr(), q_dt, qs.stride(0),
+            cache.G, None, None, 0, ws.data_ptr(), ws.numel(), stream))
+        after[i].record()
+        _lib.check(lib.rdkv_decode_fused_merge(cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
+                                               out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(),
+                                               ws.numel(), stream))
+    end.record()
+    torch.cuda.synchronize()
+    ms_step = start.elapsed_time(end) / steps
+    ms_kernel = sum(a.elapsed_time(b) for a, b in zip(before, after)) / steps
+    extras = {"ms_per_step_without_inner_events": time_region(step, steps, torch), "ms_per_step_graph_replay": None}
     if graph:
         g, side = graph_of(step, torch)
         with torch.cuda.stream(side):
-            ms_graph = time_region(g.replay, steps, torch)
+            extras["ms_per_step_graph_replay"] = time_region(g.replay, steps, torch)
         torch.cuda.current_stream().wait_stream(side)
-    ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
-    stream = _lib.stream_of(dev)
-
-    def partials_only():
-        _lib.check(lib.rdkv_decode_fused_partials(
-            None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
-            qs.data_ptr(), _lib.DTYPE_CODE[qs.dtype], qs.stride(0), cache.G, None, None, 0,
-            ws.data_ptr(), ws.numel(), stream))
-
-    partials_only()
-    ms_kernel = time_region(partials_only, steps, torch)
-    return step, ms_eager, ms_graph, ms_kernel
+    return step, ms_step, ms_kernel, extras
 
 
 def oracle_layer(pl, nvo, torch):
@@ -209,7 +224,7 @@ def compact_config(index, args, torch, dev):
     out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
     lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
     steps = max(5, min(args.steps, int(2000 / max(cache.algorithmic_bytes / 6e9, 0.01))))   # ~2 s at most
-    _, ms_eager, _, ms_kernel = fused_step_times(cache, qs, out, lse, steps, args.warmup, torch, graph=False)
+    _, ms_eager, ms_kernel, _ = fused_step_times(cache, qs, out, lse, steps, args.warmup, torch, graph=False)
     algo = cache.algorithmic_bytes
     n_groups = cfg.batch * cfg.layers
     res = {"workload": cfg.name, "layers": cfg.layers, "batch": cfg.batch, "context": cfg.context, "G": cfg.G,
@@ -615,22 +630,22 @@ def decode_loop_section(cfg, torch, dev, tokens=48):
 # CPU baseline
 # ---------------------------------------------------------------------------------------------
 def cpu_baseline_section(ora, ora_nvo, q0, H_q, torch):
-    """The NumPy oracle (dequantize-then-attend, the reference's own CPU-checkable form) on layer 0
-    of the workload: 2 warm-ups + 3 repeats, median (the protocol of run_latency.py:107-108), on
-    one core (the calling thread pinned to one CPU, library thread pools limited to 1) and on all
-    cores of this process (one oracle call per core at a time, as concurrent threads: NumPy's
-    array operations release the interpreter lock)."""
+    """The reference's dequantize-then-attend path on layer 0 of the workload, on the box's host
+    cores, in two restatements: ``torch_port`` (oracle/torch_port.py: the same op sequence on torch
+    CPU tensors, the library the reference computes in; one call on one thread, and one call on all
+    of this process's cores through the library's own thread pool) and ``numpy_port`` (the NumPy
+    oracle: one call pinned to one core, and one call per core at a time as concurrent threads).
+    2 warm-ups + 3 repeats, median (the protocol of run_latency.py:107-108).  The top-level value
+    is the torch port on one core."""
     import numpy as np
     from concurrent.futures import ThreadPoolExecutor
     from threadpoolctl import threadpool_limits
     from oracle import rdkv_oracle as O
+    from oracle import torch_port as TP
     layer_bytes = O.algorithmic_bytes(ora, H_q)
     cpus = sorted(os.sched_getaffinity(0))
     env_threads = os.environ.get("OMP_NUM_THREADS")
     n_all = min(len(cpus), int(env_threads)) if env_threads and env_threads.isdigit() else len(cpus)
-
-    def one():
-        return O.decode_attn_ref(q0, ora, ora_nvo)
 
     def timed(fn, warm=2, reps=3):
         for _ in range(warm):
@@ -642,33 +657,57 @@ def cpu_baseline_section(ora, ora_nvo, q0, H_q, torch):
             ts.append(time.perf_counter() - t0)
         return float(np.median(ts))
 
+    def one_numpy():
+        return O.decode_attn_ref(q0, ora, ora_nvo)
+
+    tl = TP.TorchLayer(ora, ora_nvo)
+    q_t = torch.from_numpy(q0)
+
+    def one_torch():
+        return TP.decode_attn(q_t, tl)
+
     torch_threads_before = torch.get_num_threads()
-    with threadpool_limits(limits=1):
-        torch.set_num_threads(1)
-        os.sched_setaffinity(0, {cpus[0]})
-        try:
-            t1 = timed(one)
-        finally:
-            os.sched_setaffinity(0, set(cpus))
-            torch.set_num_threads(torch_threads_before)
-        # all cores: n_all oracle calls in flight, each on a thread of its own, library pools still 1 per call
-        with ThreadPoolExecutor(max_workers=n_all) as ex:
-            def wave():
-                list(ex.map(lambda _: one(), range(n_all)))
-            t_all = timed(wave, warm=1, reps=3)
-    print(f"bench.py: cpu baseline threads: 1-core leg 1 thread on cpu {cpus[0]}; all-cores leg {n_all} threads; "
-          f"torch.get_num_threads()={torch.get_num_threads()}", file=sys.stderr)
-    return {"value": layer_bytes / t1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"NumPy dequantize-then-attend oracle on layer 0 of the workload ({layer_bytes} algorithmic "
-                      f"bytes), 2 warm-ups + 3 repeats, median; calling thread pinned to one CPU, library thread "
-                      f"pools limited to 1",
-            "ms_per_layer": t1 * 1e3,
-            "all_cores": {"value": n_all * layer_bytes / t_all / 1e9, "unit": "GB/s", "cores": n_all,
-                          "ms_per_layer": t_all * 1e3 / n_all,
-                          "sample": f"{n_all} concurrent oracle calls on layer 0 (one thread each), 1 warm-up + 3 "
-                                    f"repeats, median"},
-            "host_cpus": os.cpu_count(), "cpus_of_this_process": len(cpus),
-            "torch_num_threads": torch.get_num_threads()}
+    try:
+        with threadpool_limits(limits=1):
+            torch.set_num_threads(1)
+            os.sched_setaffinity(0, {cpus[0]})
+            try:
+                t1_np = timed(one_numpy)
+                t1_t = timed(one_torch)
+            finally:
+                os.sched_setaffinity(0, set(cpus))
+            # NumPy on all cores: n_all oracle calls in flight, each on a thread of its own, library
+            # pools still 1 per call (NumPy's elementwise loops are single-threaded)
+            with ThreadPoolExecutor(max_workers=n_all) as ex:
+                def wave():
+                    list(ex.map(lambda _: one_numpy(), range(n_all)))
+                t_all_np = timed(wave, warm=1, reps=3)
+        # torch on all cores: ONE call, the library's intra-op pool at n_all threads
+        torch.set_num_threads(n_all)
+        t_all_t = timed(one_torch)
+        torch_threads_all = torch.get_num_threads()
+    finally:
+        torch.set_num_threads(torch_threads_before)
+    print(f"bench.py: cpu baseline threads: 1-core legs 1 thread on cpu {cpus[0]}; NumPy all-cores leg {n_all} "
+          f"concurrent calls; torch all-cores leg one call, torch.get_num_threads()={torch_threads_all}",
+          file=sys.stderr)
+
+    def leg(seconds, cores, calls=1):
+        return {"value": calls * layer_bytes / seconds / 1e9, "unit": "GB/s", "cores": cores,
+                "ms_per_layer": seconds * 1e3 / calls}
+
+    protocol = "2 warm-ups + 3 repeats, median"
+    torch_leg = dict(leg(t1_t, 1), kind="port", library=f"torch {torch.__version__} CPU",
+                     sample=f"oracle/torch_port.decode_attn on layer 0 of the workload ({layer_bytes} algorithmic "
+                            f"bytes), {protocol}; torch.set_num_threads(1), calling thread pinned to one CPU",
+                     all_cores=dict(leg(t_all_t, n_all), sample=f"one call, torch.set_num_threads({n_all}), {protocol}"))
+    numpy_leg = dict(leg(t1_np, 1), kind="port", library=f"numpy {np.__version__}",
+                     sample=f"oracle/rdkv_oracle.decode_attn_ref on the same layer, {protocol}; calling thread pinned "
+                            f"to one CPU, library thread pools limited to 1",
+                     all_cores=dict(leg(t_all_np, n_all, calls=n_all),
+                                    sample=f"{n_all} concurrent calls (one thread each), 1 warm-up + 3 repeats, median"))
+    return dict(torch_leg, torch_port=torch_leg, numpy_port=numpy_leg, host_cpus=os.cpu_count(),
+                cpus_of_this_process=len(cpus), torch_num_threads=torch.get_num_threads())
 
 
 def main():
@@ -732,11 +771,12 @@ def main():
 
     out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
     lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
-    step, ms_step_eager, ms_step_graph, ms_kernel = fused_step_times(
+    step, ms_step_eager, ms_kernel, step_extras = fused_step_times(
         cache, qs, out, lse, args.steps, args.warmup, torch, graph=not args.no_graph)
-    # the headline is the eagerly issued step (two launches per step), the mode every run reports;
-    # the graph-replayed step stands beside it
+    # the headline is the eagerly issued step (two launches per step, an event on either side of the
+    # streaming launch), the mode every run reports; the graph-replayed step stands beside it
     ms_step = ms_step_eager
+    ms_step_graph = step_extras["ms_per_step_graph_replay"]
     algo = cache.algorithmic_bytes
     if args.fused_only:
         # one plain copy of known size in the same process: the launch against which a profiler run
@@ -869,8 +909,11 @@ def main():
         "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8/fp16 codes, fp32 accumulate", "data": "synthetic",
-        "timing_mode": "eager launches (streaming launch + merge launch per step)",
+        "timing_mode": "eager launches (streaming launch + merge launch per step); one region of `steps` steps "
+                       "with a HIP event before and after every streaming launch: ms_per_step is the region / "
+                       "steps, roofline.ms_per_launch the mean in-step event interval of the same region",
         "ms_per_step_eager": ms_step_eager, "ms_per_step_graph_replay": ms_step_graph,
+        "ms_per_step_without_inner_events": step_extras["ms_per_step_without_inner_events"],
         "us_per_step_per_layer": ms_step * 1e3 / n_groups,
         "us_per_layer_sequential": sequential["us_per_layer_sequential"] if sequential else None,
         "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,

@@ -49,6 +49,14 @@ def assert_layers_equal(dev_layer, ora_layer, skip=()):
             assert_bits_equal(t2n(a), b, f.name)
 
 
+def with_allocation(ora_layer, v_bits, k_bits):
+    """The oracle layer with the allocator's decisions attached the way the reference keeps them when
+    asked to (packing.py:1305-1314: int16 copies of v_bits [H_kv, T] and k_bits [H_kv, D])."""
+    import dataclasses
+    return dataclasses.replace(ora_layer, allocation_v_bits=np.asarray(v_bits).astype(np.int16),
+                               allocation_k_bits=np.asarray(k_bits).astype(np.int16))
+
+
 def layer_to_device(pl):
     """Oracle (NumPy) PackedKVLayer -> rdkv_amd PackedKVLayer with device tensors."""
     import dataclasses

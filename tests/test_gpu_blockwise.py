@@ -13,7 +13,8 @@ from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import blockwise_decode as bw
 from rdkv_amd import fast_decode, knapsack_solver as ks, stream_cache
-from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, layer_to_device, require_gpu, t2n, to_dev
+from tests.gpu_util import (DEV, assert_bits_equal, assert_layers_equal, layer_to_device, require_gpu, t2n, to_dev,
+                            with_allocation)
 
 pytestmark = pytest.mark.gpu
 F32 = np.float32
@@ -118,9 +119,7 @@ def test_compress_block_matches_oracle(capsys):
     v_hist = {str(b): 0 for b in (0, 2, 4, 8, 16)}
     k_hist = dict(v_hist)
     for l, (pl, v16, vb, kb) in enumerate(expected):
-        assert_layers_equal(block.packed[l], pl, skip=("allocation_v_bits", "allocation_k_bits"))
-        np.testing.assert_array_equal(t2n(block.packed[l].allocation_v_bits), vb.astype(np.int16))
-        np.testing.assert_array_equal(t2n(block.packed[l].allocation_k_bits), kb.astype(np.int16))
+        assert_layers_equal(block.packed[l], with_allocation(pl, vb, kb))     # every field, the allocation included
         if v16 is None:
             assert block.new_v_only[l] is None
         else:
@@ -171,11 +170,9 @@ def test_compress_block_random_blocks(capsys):
         what = f"case {case}: L={L} H={H} G={G} T={T} budget={budget} K options {k_opts} causal={causal}"
         for l, (pl, v16, vb, kb) in enumerate(_expected_block(kv, queries, scores, config, G, D)):
             try:
-                assert_layers_equal(block.packed[l], pl, skip=("allocation_v_bits", "allocation_k_bits"))
+                assert_layers_equal(block.packed[l], with_allocation(pl, vb, kb))
             except AssertionError as e:
                 raise AssertionError(f"{what}, layer {l}: {e}") from None
-            np.testing.assert_array_equal(t2n(block.packed[l].allocation_v_bits), vb.astype(np.int16), err_msg=what)
-            np.testing.assert_array_equal(t2n(block.packed[l].allocation_k_bits), kb.astype(np.int16), err_msg=what)
             assert (block.new_v_only[l] is None) == (v16 is None), what
             if v16 is not None:
                 assert_bits_equal(t2n(block.new_v_only[l]), v16)

@@ -249,6 +249,26 @@ def test_config_shaped_layer_vs_oracle(cfg_idx, ctx):
     assert_bits_equal(t2n(nvo), ora_nvo)
 
 
+@pytest.mark.parametrize("cfg_idx,ctx", [(1, 32768), (2, 131072), (4, 49058)])
+def test_full_size_layer_vs_oracle(cfg_idx, ctx):
+    """The whole-layer packer at the workloads' real sizes - a C1 layer (32k tokens), a C2 layer (128k
+    tokens, 2-bit heavy) and a layer of the C4 sequence the pack throughput is quoted on (49 058
+    tokens) - against the NumPy oracle on the same CPU data: every field of the layer and the fp16
+    zone, bit for bit.  At these sizes every kernel of the packer runs many workgroups per head
+    (multi-chunk planning histograms and scatter, cross-workgroup min/max, the separate tables and
+    mask launches), which the small cases do not reach."""
+    cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=1)
+    vb, kb, oc = synth.layer_allocation(cfg, 0)
+    K, V, _ = synth.layer_data(cfg, 0, "cpu", outliers=oc)
+    ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), cfg.G)
+    pl, nvo = packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, cfg.G)
+    assert int(pl.T_eff_k) > ctx // 2
+    assert_layers_equal(pl, ora)
+    assert (nvo is None) == (ora_nvo is None)
+    if ora_nvo is not None:
+        assert_bits_equal(t2n(nvo), ora_nvo, "new_v_only")
+
+
 def _layers_identical(a, b):
     import dataclasses
     for f in dataclasses.fields(a):
@@ -404,7 +424,7 @@ def test_layer_packers_on_other_input_types(kind):
     assert nvo is None and envo is None
     assert_layers_equal(pl, epl)
     # K of another type beside fp16 V takes the whole-layer kernels (K through fp16, as the canvas does)
-    v16_in = v.astype(np.float16)
+    v16_in = _typed_inputs(45, (1, 2, 90, 128), kind, big=False)[0].astype(np.float16)
     vb_ph[:, ::7] = 16
     pl, nvo = packing.pack_layer_per_head(kd, to_dev(v16_in), torch.from_numpy(vb_ph), torch.from_numpy(kb_ph), 4)
     epl, envo = O.pack_layer_per_head(k, v16_in, vb_ph, kb_ph, 4)

@@ -23,7 +23,7 @@ from rdkv_amd import trizone_decompress as tz
 from rdkv_amd import triton_k_kernel as kk
 from rdkv_amd import triton_v_kernel as vk
 from tests.gpu_util import (DEV, assert_bits_equal, assert_layers_equal, fused_both, lse_merge, require_gpu, t2n,
-                            to_dev)
+                            to_dev, with_allocation)
 
 pytestmark = pytest.mark.gpu
 
@@ -277,15 +277,13 @@ def test_selection_random_layers(block):
             continue
         layer, new_v, t_eff = run()
         try:
-            assert_layers_equal(layer, exp_layer, skip=("allocation_v_bits", "allocation_k_bits"))
+            assert_layers_equal(layer, with_allocation(exp_layer, vb, kb))
         except AssertionError as e:
             raise AssertionError(f"{what}: {e}") from None
         assert t_eff == exp_layer.T_eff, what
         assert (new_v is None) == (exp_v16 is None), what
         if exp_v16 is not None:
             assert_bits_equal(t2n(new_v), exp_v16)
-        assert np.array_equal(t2n(layer.allocation_v_bits), vb.astype(np.int16)), what
-        assert np.array_equal(t2n(layer.allocation_k_bits), kb.astype(np.int16)), what
 
 
 @pytest.mark.parametrize("block", range(2))

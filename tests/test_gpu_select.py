@@ -13,7 +13,7 @@ from oracle import rdkv_oracle as O
 from oracle import select_oracle as S
 from rdkv_amd import knapsack_solver as ks
 from rdkv_amd import obkv_fast
-from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev
+from tests.gpu_util import DEV, assert_bits_equal, assert_layers_equal, require_gpu, t2n, to_dev, with_allocation
 from tests.helpers import assert_layer_equal, load_golden
 from tests.test_oracle_select import POOL_CASES, SELECT_JOINT_GOLDEN, golden_batched_cases, select_joint_golden
 
@@ -201,18 +201,13 @@ def test_select_and_pack_layer_matches_oracle(case):
         k_budget_ratio=ratio, obs_window=32, pool_kernel_size=7, pool_padding="reflect", pool_type="avg",
         v_bit_options=None, k_bit_options=_opts(k_opts), eps_V=ks.DEFAULT_EPSILON_V, eps_K=ks.DEFAULT_EPSILON_K,
         timing=timing, retain_allocation_metadata=retain)
-    skip = ("allocation_v_bits", "allocation_k_bits")
-    assert_layers_equal(layer, exp_layer, skip=skip)
+    # every field; the allocation is kept on the layer only when asked for (packing.py:1305-1314)
+    assert_layers_equal(layer, with_allocation(exp_layer, vb, kb) if retain else exp_layer)
     assert t_eff == exp_layer.T_eff
     if exp_v16 is None:
         assert new_v is None
     else:
         assert_bits_equal(t2n(new_v), exp_v16)
-    if retain:
-        np.testing.assert_array_equal(t2n(layer.allocation_v_bits), vb.astype(np.int16))
-        np.testing.assert_array_equal(t2n(layer.allocation_k_bits), kb.astype(np.int16))
-    else:
-        assert layer.allocation_v_bits is None and layer.allocation_k_bits is None
     if timing is not None:
         assert set(timing) == {"pooling_ms", "v_allocation_ms", "k_allocation_ms", "quantization_ms", "packing_ms"}
     with pytest.raises(ValueError):
