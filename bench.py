@@ -125,14 +125,18 @@ def build_workload(cfg, dev, torch, on_first=None, pack_sample=None):
     return groups
 
 
-def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True):
-    """The timed region of the fused step.  Every step is the library's two launches (streaming
-    kernel, then merge) issued eagerly, with a HIP event on the same stream before and after the
-    streaming launch: ms per step is the whole region divided by its steps, ms per launch of the
-    streaming kernel is the mean of the in-step event intervals - one loop gives both, so the kernel
-    can never come out slower than the step that contains it.  Beside it: the same step through
-    ``decode_attn_fused`` without the inner events (what they cost), and replayed from a HIP graph.
-    Returns (step, ms_step, ms_kernel, extras)."""
+def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True, rounds=5):
+    """The timed regions of the fused step, `rounds` times in alternation so that clock and
+    temperature drift reach all of them alike, the median of each kind reported:
+      (a) `steps` steps through ``decode_attn_fused`` (streaming launch + merge launch, eagerly
+          issued), bracketed by events and synchronization: ms per step, the headline;
+      (b) the same steps issued as the library's two calls with a HIP event on the same stream
+          before and after every streaming launch: the mean in-step interval is the duration of the
+          streaming kernel inside a step (it cannot exceed the step of its own region; the events
+          themselves cost that region ~3 %, which is why (a) is the headline);
+      (c) `steps` launches of the streaming kernel alone, back to back.
+    Beside them the step replayed from a HIP graph.  Returns (step, ms_step, ms_kernel, extras)."""
+    import numpy as np
     from rdkv_amd import _lib, stream_cache
     lib = _lib.load()
     dev = qs.device
@@ -153,33 +157,52 @@ def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True):
     ws = _lib.workspace(dev, lib.rdkv_decode_fused_workspace_bytes(cache.n_work, cache.G))
     stream = _lib.stream_of(dev)
     q_dt = _lib.DTYPE_CODE[qs.dtype]
-    before = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    after = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    start.record()
-    for i in range(steps):
-        before[i].record()
+
+    def partials_only():
         _lib.check(lib.rdkv_decode_fused_partials(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
             _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords, qs.data_ptr(), q_dt, qs.stride(0),
             cache.G, None, None, 0, ws.data_ptr(), ws.numel(), stream))
-        after[i].record()
+
+    def merge_only():
         _lib.check(lib.rdkv_decode_fused_merge(cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
                                                out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(),
                                                ws.numel(), stream))
-    end.record()
-    torch.cuda.synchronize()
-    ms_step = start.elapsed_time(end) / steps
-    ms_kernel = sum(a.elapsed_time(b) for a, b in zip(before, after)) / steps
-    extras = {"ms_per_step_without_inner_events": time_region(step, steps, torch), "ms_per_step_graph_replay": None}
+
+    before = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    after = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+
+    def evented_region():
+        torch.cuda.synchronize()
+        start.record()
+        for i in range(steps):
+            before[i].record()
+            partials_only()
+            after[i].record()
+            merge_only()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / steps, sum(a.elapsed_time(b) for a, b in zip(before, after)) / steps
+
+    plain, ev_step, ev_kernel, alone = [], [], [], []
+    for _ in range(rounds):
+        plain.append(time_region(step, steps, torch))
+        es, ek = evented_region()
+        ev_step.append(es)
+        ev_kernel.append(ek)
+        alone.append(time_region(partials_only, steps, torch))
+    med = lambda v: float(np.median(v))
+    extras = {"timing_rounds": rounds, "ms_per_step_regions": plain,
+              "ms_per_step_with_inner_events": med(ev_step), "ms_per_launch_kernel_alone": med(alone),
+              "ms_per_step_graph_replay": None}
     if graph:
         g, side = graph_of(step, torch)
         with torch.cuda.stream(side):
             extras["ms_per_step_graph_replay"] = time_region(g.replay, steps, torch)
         torch.cuda.current_stream().wait_stream(side)
-    return step, ms_step, ms_kernel, extras
+    return step, med(plain), med(ev_kernel), extras
 
 
 def oracle_layer(pl, nvo, torch):
@@ -224,7 +247,7 @@ def compact_config(index, args, torch, dev):
     out = torch.empty(cache.rows, 128, dtype=torch.float32, device=dev)
     lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
     steps = max(5, min(args.steps, int(2000 / max(cache.algorithmic_bytes / 6e9, 0.01))))   # ~2 s at most
-    _, ms_eager, ms_kernel, _ = fused_step_times(cache, qs, out, lse, steps, args.warmup, torch, graph=False)
+    _, ms_eager, ms_kernel, _ = fused_step_times(cache, qs, out, lse, steps, args.warmup, torch, graph=False, rounds=3)
     algo = cache.algorithmic_bytes
     n_groups = cfg.batch * cfg.layers
     res = {"workload": cfg.name, "layers": cfg.layers, "batch": cfg.batch, "context": cfg.context, "G": cfg.G,
@@ -773,8 +796,8 @@ def main():
     lse = torch.empty(cache.rows, dtype=torch.float32, device=dev)
     step, ms_step_eager, ms_kernel, step_extras = fused_step_times(
         cache, qs, out, lse, args.steps, args.warmup, torch, graph=not args.no_graph)
-    # the headline is the eagerly issued step (two launches per step, an event on either side of the
-    # streaming launch), the mode every run reports; the graph-replayed step stands beside it
+    # the headline is the eagerly issued step (two launches per step), the mode every run reports;
+    # the graph-replayed step stands beside it
     ms_step = ms_step_eager
     ms_step_graph = step_extras["ms_per_step_graph_replay"]
     algo = cache.algorithmic_bytes
@@ -909,11 +932,12 @@ def main():
         "value": gbps, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u8/fp16 codes, fp32 accumulate", "data": "synthetic",
-        "timing_mode": "eager launches (streaming launch + merge launch per step); one region of `steps` steps "
-                       "with a HIP event before and after every streaming launch: ms_per_step is the region / "
-                       "steps, roofline.ms_per_launch the mean in-step event interval of the same region",
+        "timing_mode": f"eager launches (streaming launch + merge launch per step); median of "
+                       f"{step_extras['timing_rounds']} regions of `steps` steps each, alternating with the regions "
+                       f"roofline.ms_per_launch comes from (the same steps with a HIP event before and after every "
+                       f"streaming launch: mean in-step interval)",
         "ms_per_step_eager": ms_step_eager, "ms_per_step_graph_replay": ms_step_graph,
-        "ms_per_step_without_inner_events": step_extras["ms_per_step_without_inner_events"],
+        "ms_per_step_regions": step_extras["ms_per_step_regions"],
         "us_per_step_per_layer": ms_step * 1e3 / n_groups,
         "us_per_layer_sequential": sequential["us_per_layer_sequential"] if sequential else None,
         "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
@@ -933,6 +957,8 @@ def main():
                      "traffic_source": (f"{traffic[1]}, a constant from that profiler run (not observed by this run)"
                                         if traffic else None),
                      "kernel": "decode_fused_kernel", "ms_per_launch": ms_kernel,
+                     "ms_per_step_of_the_regions_with_inner_events": step_extras["ms_per_step_with_inner_events"],
+                     "ms_per_launch_kernel_alone": step_extras["ms_per_launch_kernel_alone"],
                      "algorithmic_bytes_per_launch": algo, "streamed_bytes_per_launch": stream_bytes,
                      "ms_per_step_flushed_caches": ms_step_cold,
                      "step_GBps_flushed_caches": algo / (ms_step_cold * 1e-3) / 1e9,
