@@ -202,6 +202,18 @@ def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True, roun
         with torch.cuda.stream(side):
             extras["ms_per_step_graph_replay"] = time_region(g.replay, steps, torch)
         torch.cuda.current_stream().wait_stream(side)
+        # the same step eight times per graph: what a replay costs beyond its kernels is paid once per
+        # replay, not once per launch, so it shrinks with the number of steps a graph holds
+        per_graph = 8
+
+        def eight_steps():
+            for _ in range(per_graph):
+                step()
+        g8, side = graph_of(eight_steps, torch)
+        with torch.cuda.stream(side):
+            extras["ms_per_step_graph_replay_8_steps_per_graph"] = (
+                time_region(g8.replay, max(steps // per_graph, 3), torch) / per_graph)
+        torch.cuda.current_stream().wait_stream(side)
     return step, med(plain), med(ev_kernel), extras
 
 
@@ -937,6 +949,7 @@ def main():
                        f"roofline.ms_per_launch comes from (the same steps with a HIP event before and after every "
                        f"streaming launch: mean in-step interval)",
         "ms_per_step_eager": ms_step_eager, "ms_per_step_graph_replay": ms_step_graph,
+        "ms_per_step_graph_replay_8_steps_per_graph": step_extras.get("ms_per_step_graph_replay_8_steps_per_graph"),
         "ms_per_step_regions": step_extras["ms_per_step_regions"],
         "us_per_step_per_layer": ms_step * 1e3 / n_groups,
         "us_per_layer_sequential": sequential["us_per_layer_sequential"] if sequential else None,

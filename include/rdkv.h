@@ -395,8 +395,13 @@ int rdkv_decode_fused_static(const uint8_t *blob, const RdkvUnit *units, int n_u
  * zone_c_weights (NULL, or fp32 [rows, >= n_new], row stride in elements): receives the softmax
  * weight of every zone-C token over the union, per query row - the w_new of fast_decode.py:1755
  * and the pending weights blockwise decode sums into its block scores
- * (blockwise_decode.py:2085-2109). */
-int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G,
+ * (blockwise_decode.py:2085-2109).
+ * units_host_or_null (HOST pointer, NULL = none): the caller's host copy of the same unit table.
+ * When given and the table is short (up to 16 units: a single layer's call), the units' merge
+ * fields travel with the kernel arguments, which saves the launch a dependent memory round trip;
+ * it is read during the call only. */
+int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, const RdkvUnit *units_host_or_null, int n_units,
+                                   int n_work, int G,
                                    const void *q, int q_dtype, int64_t q_stride_row,
                                    const void *rope_cos, const void *rope_sin, int rope_dtype,
                                    const float *k_new, const float *v_new, int64_t new_stride_unit,
@@ -435,7 +440,8 @@ typedef struct RdkvTailScores {   /* online block scores of blockwise decode, se
                                      q_rotated_out is a buffer [rows, tokens, 128] and the step's rows go to
                                      token row_dev[0] of it: again no host value per step */
 } RdkvTailScores;
-int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, int n_units, int n_work, int G,
+int rdkv_decode_fused_merge_zone_c_append(const RdkvUnit *units, const RdkvUnit *units_host_or_null, int n_units,
+                                          int n_work, int G,
                                           const void *q, int q_dtype, int64_t q_stride_row,
                                           const void *rope_cos, const void *rope_sin, int rope_dtype,
                                           float *k_new, float *v_new, int64_t new_stride_unit,

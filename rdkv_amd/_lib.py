@@ -68,8 +68,8 @@ SIGNATURES = {
     "rdkv_decode_fused_static_max_bytes": (L, []),
     "rdkv_decode_fused_static": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P, P]),
     "rdkv_decode_fused_partials": (I, [P, P, I, P, I, P, I, I, P, I, L, I, P, P, I, P, L, P]),
-    "rdkv_decode_fused_merge_zone_c": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, I, P, P, L, P, P, L, P, L, P]),
-    "rdkv_decode_fused_merge_zone_c_append": (I, [P, I, I, I, P, I, L, P, P, I, P, P, L, L, L, P, P, L, P, L, I, P,
+    "rdkv_decode_fused_merge_zone_c": (I, [P, P, I, I, I, P, I, L, P, P, I, P, P, L, L, I, P, P, L, P, P, L, P, L, P]),
+    "rdkv_decode_fused_merge_zone_c_append": (I, [P, P, I, I, I, P, I, L, P, P, I, P, P, L, L, L, P, P, L, P, L, I, P,
                                                   P, L, P, P, L, P, L, P, P, L, P]),
     "rdkv_rope": (I, [P, L, I, P, L, I, I, I, P, P, I, P]),
     "rdkv_add_rms_norm": (I, [P, L, P, L, P, I, F, I, I, I, P, L, P, L, P]),

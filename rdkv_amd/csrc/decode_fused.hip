@@ -105,11 +105,21 @@ __device__ __forceinline__ float quadcol_max(float v) {
   return fmaxf(__builtin_bit_cast(float, (unsigned)t[0]), __builtin_bit_cast(float, (unsigned)t[1]));
 }
 
-// Combine the partials [work_begin, work_begin + n) of one unit in index order with a whole
-// workgroup.  The max / sum columns are staged in LDS first (scratch: 2 * kMergeMaxK * 8
-// floats) so that the accumulator loads of a thread are independent and overlap: the merge
-// costs about one memory latency instead of one per partial.
+// ---- merge of a unit's partials --------------------------------------------------------------
+// The partials [work_begin, work_begin + n) of one unit are combined in index order by a whole
+// workgroup, in three stages that all callers share (so that the separate merge launch, the merge
+// inside the streaming launch and the merge with zone C give the same bits):
+//   1. the max / sum columns of the partials go to LDS;
+//   2. wavefront h takes head h (lane = partial): the head's maximum M, every partial's factor
+//      exp2(m_k - M) into LDS, the sum L of factor x l_k, log2-sum-exp2 and 1 / L;
+//   3. a thread takes an output column: sum over k, ascending, of factor_k x acc_k, times 1 / L.
+// The first kMergeAhead accumulator values of a column are requested before stage 1's barrier, so
+// the usual unit (up to kMergeAhead partials) costs one memory round trip.
 constexpr int kMergeMaxK = 128;
+constexpr int kMergeAhead = 32;
+// LDS scratch of a merge (floats): m[k * 8 + h], l[k * 8 + h], factor[h * kMergeMaxK + k], l2[h], inv[h]
+constexpr int kMergeM = 0, kMergeL = kMergeMaxK * 8, kMergeF = 2 * kMergeMaxK * 8, kMergeL2 = 3 * kMergeMaxK * 8,
+              kMergeInv = kMergeL2 + 8, kMergeScratchFloats = kMergeInv + 8;
 
 // A partial value as another workgroup of the SAME launch left it: partials are written with
 // device-scope stores (pstore) and read here with device-scope loads, which are served from the
@@ -123,104 +133,148 @@ __device__ __forceinline__ float pload(const float *p) {
   return *p;
 }
 
-// keep_o / keep_lse (LDS, [8][128] and [8], or null): when given, the normalized result and the
-// natural-log sum-exp stay there for a following zone-C pass instead of being written out.
+// Maximum / sum over all 64 lanes of a wavefront without LDS traffic, the same bits in every lane:
+// exchanges at distance 1 and 2 inside a quad, a mirror inside 8 and inside 16 lanes (data-parallel
+// moves; at every level all lanes of a group already hold the same value and partners only swap
+// operands), then the two rows of a half and the two halves by lane-permute swaps, whose two
+// results are the same pair of values in every lane.
+template <bool MAX>
+__device__ __forceinline__ float wave_rows_reduce(float v) {      // across the four rows of 16 lanes
+  auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = op(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+  u = __builtin_bit_cast(unsigned, v);
+  auto t = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return op(__builtin_bit_cast(float, (unsigned)t[0]), __builtin_bit_cast(float, (unsigned)t[1]));
+}
+template <bool MAX>
+__device__ __forceinline__ float wave_reduce(float v) {
+  auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+  v = op(v, rdkv_dpp_mov<0xB1>(v));    // quad_perm [1,0,3,2]
+  v = op(v, rdkv_dpp_mov<0x4E>(v));    // quad_perm [2,3,0,1]
+  v = op(v, rdkv_dpp_mov<0x141>(v));   // row_half_mirror
+  v = op(v, rdkv_dpp_mov<0x140>(v));   // row_mirror
+  return wave_rows_reduce<MAX>(v);
+}
+
+// Stage 2 for the heads wave, wave + n_waves, ... (n <= kMergeMaxK).
+__device__ __forceinline__ void merge_factors(int n, int G, int wave, int lane, int n_waves, float *scratch) {
+  for (int h = wave; h < G; h += n_waves) {
+    float M = -INFINITY;
+    for (int k0 = 0; k0 < n; k0 += 64) {
+      const int k = k0 + lane;
+      M = fmaxf(M, k < n ? scratch[kMergeM + k * 8 + h] : -INFINITY);
+    }
+    M = wave_reduce<true>(M);
+    float L = 0.0f;
+    for (int k0 = 0; k0 < n; k0 += 64) {
+      const int k = k0 + lane;
+      const float mk = k < n ? scratch[kMergeM + k * 8 + h] : -INFINITY;
+      const float f = mk == -INFINITY ? 0.0f : fast_exp2(mk - M);
+      if (k < n) {
+        scratch[kMergeF + h * kMergeMaxK + k] = f;
+        L = fmaf(f, scratch[kMergeL + k * 8 + h], L);
+      }
+    }
+    L = wave_reduce<false>(L);
+    if (lane == 0) {
+      scratch[kMergeL2 + h] = L > 0.0f ? M + log2f(L) : -INFINITY;   // a unit without tokens gives 0 / -inf
+      scratch[kMergeInv + h] = L > 0.0f ? 1.0f / L : 0.0f;
+    }
+  }
+}
+
+// Stage 3 for one column: `ahead` holds the column's first kMergeAhead accumulator values (entries
+// past n: anything finite or not - they enter with factor zero by selection), `base` points at the
+// column of partial 0, pstride is the distance between partials.  Returns the normalized value.
+template <bool COHERENT>
+__device__ __forceinline__ float merge_column(int n, int h, const float (&ahead)[kMergeAhead], const float *base,
+                                              int64_t pstride, const float *scratch) {
+  const float *fh = scratch + kMergeF + h * kMergeMaxK;
+  float o = 0.0f;
+#pragma unroll
+  for (int e0 = 0; e0 < kMergeAhead; e0 += 4) {
+    const float4 f4 = *reinterpret_cast<const float4 *>(fh + e0);
+    const float fe[4] = {f4.x, f4.y, f4.z, f4.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o = fmaf(e0 + e < n ? fe[e] : 0.0f, e0 + e < n ? ahead[e0 + e] : 0.0f, o);
+  }
+  for (int k0 = kMergeAhead; k0 < n; k0 += 16) {
+    float v[16];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = pload<COHERENT>(base + (k0 + e < n ? k0 + e : k0) * pstride);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o = fmaf(k0 + e < n ? fh[k0 + e] : 0.0f, v[e], o);
+  }
+  return o * scratch[kMergeInv + h];
+}
+
+// The column of a unit with more than kMergeMaxK partials: plain two-pass loops, nothing staged.
+// Returns the normalized value and the column's log2-sum-exp2.
+template <bool COHERENT>
+__device__ __forceinline__ float merge_column_long(int n, const float *head_base, int d, int64_t pstride, float &l2) {
+  float M = -INFINITY;
+  for (int k = 0; k < n; ++k) M = fmaxf(M, pload<COHERENT>(head_base + k * pstride + 128));
+  float o = 0.0f, l = 0.0f;
+  for (int k = 0; k < n; ++k) {
+    const float *p = head_base + k * pstride;
+    const float mk = pload<COHERENT>(p + 128);
+    const float f = mk == -INFINITY ? 0.0f : fast_exp2(mk - M);
+    o = fmaf(f, pload<COHERENT>(p + d), o);
+    l = fmaf(f, pload<COHERENT>(p + 129), l);
+  }
+  l2 = l > 0.0f ? M + log2f(l) : -INFINITY;
+  return l > 0.0f ? o * (1.0f / l) : 0.0f;
+}
+
+// The whole merge of one unit by a workgroup of `nthreads` threads (a multiple of 64, at least
+// 64 * G): out rows q_row .. q_row + G, lse in natural logarithm.  scratch: kMergeScratchFloats
+// floats of LDS, 16-byte aligned.  Contains two workgroup barriers (none for a unit of more than
+// kMergeMaxK partials).
 // COHERENT: the partials were written earlier in the same launch (merge inside the streaming
 // kernel); otherwise by a launch that has completed.
 template <bool COHERENT = false>
 __device__ __forceinline__ void merge_unit(const float *partials, int work_begin, int n, int G, int q_row,
                                            float *out, int64_t out_stride, float *lse, int tid, int nthreads,
-                                           float *scratch, float *keep_o = nullptr, float *keep_lse = nullptr) {
+                                           float *scratch) {
   const int64_t pstride = (int64_t)G * kPartialStride;
   const float *base0 = partials + (int64_t)work_begin * pstride;
-  if (n <= kMergeMaxK) {
-    float *s_m = scratch, *s_l = scratch + kMergeMaxK * 8;
-    // The first kMergeAhead accumulator values of the thread's first column are requested together
-    // with the max / sum columns, before the barrier that publishes those: the usual unit (up to
-    // kMergeAhead partials, one column per thread) then costs one memory round trip, not three.
-    constexpr int kMergeAhead = 32;
-    float ahead[kMergeAhead];
-    {
-      const int i0 = tid < G * kD ? tid : 0;
-      const float *b0 = base0 + (i0 >> 7) * kPartialStride + (i0 & 127);
-#pragma unroll
-      for (int e = 0; e < kMergeAhead; ++e) ahead[e] = pload<COHERENT>(b0 + (e < n ? e : 0) * pstride);
-    }
-    for (int i = tid; i < n * G; i += nthreads) {
-      const int k = i / G, h = i - k * G;
-      s_m[k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 128);
-      s_l[k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 129);
-    }
-    __syncthreads();
+  if (n > kMergeMaxK) {          // very long units
     for (int i = tid; i < G * kD; i += nthreads) {
       const int h = i >> 7, d = i & 127;
-      float M = -INFINITY;
-      for (int k = 0; k < n; ++k) M = fmaxf(M, s_m[k * 8 + h]);
-      float o = 0.0f, l = 0.0f;
-      const float *base = base0 + h * kPartialStride + d;
-      int k_from = 0;
-      if (i == tid) {       // the column fetched ahead
-#pragma unroll
-        for (int e = 0; e < kMergeAhead; ++e) {
-          if (e < n) {
-            const float mk = s_m[e * 8 + h];
-            const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
-            o += f * ahead[e];
-            l += f * s_l[e * 8 + h];
-          }
-        }
-        k_from = kMergeAhead;
-      }
-      for (int k0 = k_from; k0 < n; k0 += 16) {
-        float v[16];
-#pragma unroll
-        for (int e = 0; e < 16; ++e) v[e] = pload<COHERENT>(base + (k0 + e < n ? k0 + e : k0) * pstride);
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          if (k0 + e < n) {
-            const float mk = s_m[(k0 + e) * 8 + h];
-            const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
-            o += f * v[e];
-            l += f * s_l[(k0 + e) * 8 + h];
-          }
-        }
-      }
-      const int64_t row = q_row + h;
-      const float o_n = l > 0.0f ? o / l : 0.0f;  // a unit without tokens gives 0 / -inf
-      const float lse_n = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
-      if (keep_o) {
-        keep_o[i] = o_n;
-        if (d == 0) keep_lse[h] = lse_n;
-      } else {
-        out[row * out_stride + d] = o_n;
-        if (lse && d == 0) lse[row] = lse_n;
-      }
+      float l2;
+      const float o = merge_column_long<COHERENT>(n, base0 + h * kPartialStride, d, pstride, l2);
+      out[(int64_t)(q_row + h) * out_stride + d] = o;
+      if (lse && d == 0) lse[q_row + h] = l2 * kLn2;
     }
     return;
   }
-  for (int i = tid; i < G * kD; i += nthreads) {  // very long units: plain two-pass loop
+  // the accumulator values of the thread's first column, requested with the max / sum columns
+  float ahead[kMergeAhead];
+  {
+    const int i0 = tid < G * kD ? tid : 0;
+    const float *b0 = base0 + (i0 >> 7) * kPartialStride + (i0 & 127);
+#pragma unroll
+    for (int e = 0; e < kMergeAhead; ++e) ahead[e] = pload<COHERENT>(b0 + (e < n ? e : 0) * pstride);
+  }
+  for (int i = tid; i < n * G; i += nthreads) {
+    const int k = i / G, h = i - k * G;
+    scratch[kMergeM + k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 128);
+    scratch[kMergeL + k * 8 + h] = pload<COHERENT>(base0 + k * pstride + h * kPartialStride + 129);
+  }
+  __syncthreads();
+  merge_factors(n, G, tid >> 6, tid & 63, nthreads >> 6, scratch);
+  __syncthreads();
+  for (int i = tid; i < G * kD; i += nthreads) {
     const int h = i >> 7, d = i & 127;
-    const float *base = base0 + h * kPartialStride;
-    float M = -INFINITY;
-    for (int k = 0; k < n; ++k) M = fmaxf(M, pload<COHERENT>(base + k * pstride + 128));
-    float o = 0.0f, l = 0.0f;
-    for (int k = 0; k < n; ++k) {
-      const float *p = base + k * pstride;
-      const float mk = pload<COHERENT>(p + 128);
-      const float f = mk == -INFINITY ? 0.0f : exp2f(mk - M);
-      o += f * pload<COHERENT>(p + d);
-      l += f * pload<COHERENT>(p + 129);
+    const float *base = base0 + h * kPartialStride + d;
+    if (i != tid) {      // a further column of this thread: its values are fetched now
+#pragma unroll
+      for (int e = 0; e < kMergeAhead; ++e) ahead[e] = pload<COHERENT>(base + (e < n ? e : 0) * pstride);
     }
-    const int64_t row = q_row + h;
-    const float o_n = l > 0.0f ? o / l : 0.0f;
-    const float lse_n = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
-    if (keep_o) {
-      keep_o[i] = o_n;
-      if (d == 0) keep_lse[h] = lse_n;
-    } else {
-      out[row * out_stride + d] = o_n;
-      if (lse && d == 0) lse[row] = lse_n;
-    }
+    out[(int64_t)(q_row + h) * out_stride + d] = merge_column<COHERENT>(n, h, ahead, base, pstride, scratch);
+    if (lse && d == 0) lse[q_row + h] = scratch[kMergeL2 + h] * kLn2;
   }
 }
 
@@ -240,7 +294,7 @@ struct Smem {
   int ticket[kBatch];                                            // arrival order of the batch's partials at their units
   float wm[kBatch][NW][NH * 4];                                  // per-wavefront results of an item
   float wl[kBatch][NW][NH * 4];
-  float wo[kBatch][NW][NH * 4][kD];
+  alignas(16) float wo[kBatch][NW][NH * 4][kD];                  // (also the scratch of a merge inside the launch)
 };
 
 // Register images of the loads in flight.  The K row of the lane's token and the {scale,zp}
@@ -874,7 +928,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         if (tid_o == 0) __hip_atomic_store(tickets + mi.merge_unit, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         // the wavefront results of the batch have been consumed: their LDS serves as scratch
         float *scratch = &sm.wo[0][0][0][0];
-        static_assert(sizeof(sm.wo) >= 2 * kMergeMaxK * 8 * sizeof(float), "merge scratch does not fit");
+        static_assert(sizeof(sm.wo) >= kMergeScratchFloats * sizeof(float), "merge scratch does not fit");
         merge_unit<true>(partials, mi.merge_begin, mi.merge_count, G, mi.q_row, out, out_stride, lse, tid_o,
                          kThreads, scratch);
         __syncthreads();
@@ -897,7 +951,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
 __global__ void __launch_bounds__(1024)
 merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials, int G,
              float *__restrict__ out, int64_t out_stride, float *__restrict__ lse) {
-  __shared__ float scratch[2 * kMergeMaxK * 8];
+  __shared__ __align__(16) float scratch[kMergeScratchFloats];
   const RdkvUnit *u = units + blockIdx.x;
   if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   merge_unit(partials, u->work_begin, u->work_count, G, u->q_row, out, out_stride, lse, threadIdx.x,
@@ -907,15 +961,31 @@ merge_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ parti
 // Merge of a unit's partials followed by the attention over its decode-appended tokens
 // (zone C: fp32 K/V rows that are not part of the packed cache), the exact softmax over the
 // union (fast_decode.py:1719-1735, 1777-1784): the zones A+B result enters as one pseudo-token
-// of weight exp(lse_ab) and value out_ab.  The new tokens are taken 64 at a time, one chunk per
-// wavefront (chunk c by wavefront c mod 8): a lane scores its own token (its K row in 16-byte
-// loads against the query group in LDS), the wavefront keeps a running maximum, sum and 128
-// accumulators per head (lane = two channels, weights passed lane to lane), and the eight
-// wavefront states and the A+B state are combined once at the end, in a fixed order.  No
-// workgroup barrier inside the token loop.  Natural-log domain, fp32 throughout, q scaled by
-// 1/sqrt(D) first as the reference does.
+// of weight exp(lse_ab) and value out_ab.  fp32 throughout; scores in the base-2 domain (q is
+// scaled by log2(e) / sqrt(D) once, as the streaming kernel does), the log-sum-exp returned in
+// natural logarithm.
+//
+// The launch sits on the critical path of every layer of a decode step and moves well under a
+// megabyte, so it is built around its DEPENDENT memory round trips and its instruction count:
+//  * one round trip when the host passes the units' three merge fields with the kernel arguments
+//    (single-layer calls, up to kZcInlineUnits units), two otherwise: the unit's descriptor, then
+//    everything else at once - the token count, the step's write row, the query rows and rotation
+//    table, the step's own key / value row, the partials' max / sum columns and accumulator
+//    columns, and the first 64 zone C tokens' K and V rows (requested before the count is known:
+//    rows up to the buffer's end exist, a row past the count is discarded);
+//  * one workgroup of eight wavefronts per unit; wavefront w owns tokens 8w .. 8w + 7 of every
+//    chunk of 64 and keeps its own online-softmax state, so the token loop has no barrier and no
+//    LDS traffic beyond the query: a token's K row is split over eight lanes (16-byte loads, 128
+//    contiguous bytes per token and instruction), the partial dot products are folded inside the
+//    eight lanes and the maximum / sum across the wavefront's eight tokens by data-parallel moves
+//    and lane-permute swaps, the weights are read lane to lane for weight x V (lane = channel
+//    pair, one whole 512-byte row per load instruction), the next chunk's rows in flight meanwhile;
+//  * the eight wavefront states and the zones A+B state are combined once, in a fixed order.
+// The step's own token never comes back through memory: its rotated key and its value are kept
+// in LDS and stand in for whatever the row's loads returned.
 constexpr int kZcChunk = 64;
 constexpr int kZcWaves = 8;
+constexpr int kZcInlineUnits = 16;
 // The new token's un-rotated key and value rows (k == nullptr: nothing to append).
 struct ZcAppend {
   const void *k, *v;
@@ -924,11 +994,51 @@ struct ZcAppend {
   int64_t capacity;
   int dtype;
 };
+// The merge fields of the first units of the table, passed by value (n == 0: read the table).
+struct ZcInline {
+  int n;
+  int q_row[kZcInlineUnits], work_begin[kZcInlineUnits], work_count[kZcInlineUnits];
+};
+
+// Maximum / sum over the eight tokens of a wavefront (a token's value sits in the eight lanes
+// lane >> 3 == token), the same bits in every lane: the two tokens of a row of 16 lanes by a
+// mirror inside the row (lane i <-> 15 - i lies in the other token's lanes), then the two rows of
+// a half and the two halves of the wavefront by lane-permute swaps, whose two results are the
+// same pair of values in every lane.
+template <bool MAX>
+__device__ __forceinline__ float zc_tokens_reduce(float v) {
+  auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+  v = op(v, rdkv_dpp_mov<0x140>(v));   // row_mirror
+  unsigned u = __builtin_bit_cast(unsigned, v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = op(__builtin_bit_cast(float, (unsigned)r[0]), __builtin_bit_cast(float, (unsigned)r[1]));
+  u = __builtin_bit_cast(unsigned, v);
+  auto t = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return op(__builtin_bit_cast(float, (unsigned)t[0]), __builtin_bit_cast(float, (unsigned)t[1]));
+}
+// Maximum / sum over all 64 lanes, the same bits in every lane.
+template <bool MAX>
+__device__ __forceinline__ float zc_wave_reduce(float v) {
+  auto op = [](float a, float b) { return MAX ? fmaxf(a, b) : a + b; };
+  v = op(v, rdkv_dpp_mov<0xB1>(v));    // quad_perm [1,0,3,2]
+  v = op(v, rdkv_dpp_mov<0x4E>(v));    // quad_perm [2,3,0,1]
+  v = op(v, rdkv_dpp_mov<0x141>(v));   // row_half_mirror
+  return zc_tokens_reduce<MAX>(v);
+}
+// Sum over the eight lanes that share (lane >> 3), the same bits in each of them (exchanges at
+// distance 1 and 2 inside a quad, then a mirror inside the eight lanes).
+__device__ __forceinline__ float zc_oct_sum(float v) {
+  v += rdkv_dpp_mov<0xB1>(v);          // quad_perm [1,0,3,2]
+  v += rdkv_dpp_mov<0x4E>(v);          // quad_perm [2,3,0,1]
+  return v + rdkv_dpp_mov<0x141>(v);   // row_half_mirror
+}
+
 // G is a template parameter: the per-head loops unroll into straight-line code (with a run-time
 // G every head of every token is a scalar branch).
-template <int G>
+// INLINE: the units' merge fields come with the kernel arguments (iu), not from the table.
+template <int G, bool INLINE>
 __global__ void __launch_bounds__(64 * kZcWaves)
-merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict__ partials,
+merge_zone_c_kernel(const RdkvUnit *__restrict__ units, ZcInline iu, const float *__restrict__ partials,
                     const void *__restrict__ q, int q_dtype, int64_t q_stride,
                     const void *__restrict__ rope_cos, const void *__restrict__ rope_sin, int rope_dtype,
                     float *k_new, float *v_new, int64_t new_stride_unit,   // written when a row is appended
@@ -936,91 +1046,222 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
                     float *__restrict__ out, int64_t out_stride, float *__restrict__ lse,
                     float *zc_w, int64_t zc_w_stride, ZcAppend ap, void *__restrict__ q_rot_out,
                     int64_t q_rot_stride, RdkvTailScores ts) {
-  __shared__ float scratch[2 * kMergeMaxK * 8];
-  __shared__ float fin_m[8], fin_l[8];             // softmax maximum and sum over the union, per head
-  __shared__ float acc_ab[8 * kD];                 // normalized zones A+B output
-  __shared__ __align__(16) float qz[8][kD];        // q / sqrt(D)
-  __shared__ float w_m[kZcWaves][8], w_l[kZcWaves][8];
-  __shared__ float w_acc[kZcWaves][8][kD];
-  __shared__ float lse_ab[8];
   constexpr int kThreads = 64 * kZcWaves;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const RdkvUnit *u = units + blockIdx.x;
-  if (u->work_count == 0) return;  // a further source of an output row: merged by the row's first unit
-  const int q_row = u->q_row;
+  constexpr int kCols = (G * kD + kThreads - 1) / kThreads;   // output columns per thread
+  constexpr int kAhead = kMergeAhead;                         // partials whose accumulators are requested at once
+  __shared__ __align__(16) float scratch[kMergeScratchFloats]; // the merge of zones A+B (see merge_unit)
+  __shared__ __align__(16) float qz[8][kD];                   // q * log2(e) / sqrt(D)
+  __shared__ __align__(16) float k_self[kD], v_self[kD];      // the step's own token (rotated key, value)
+  __shared__ float w_m[kZcWaves][8], w_l[kZcWaves][8];        // every wavefront's zone C softmax state ...
+  __shared__ __align__(8) float w_acc[kZcWaves][8][kD];       // ... and its share of sum weight x V
+  __shared__ float fin_m[8], fin_l[8];                        // softmax maximum and sum over the union, per head
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  // ---- the unit: from the kernel arguments, or the first round trip ------------------------------
+  int work_count, q_row, work_begin;
+  if (INLINE) {
+    q_row = iu.q_row[blockIdx.x];
+    work_begin = iu.work_begin[blockIdx.x];
+    work_count = iu.work_count[blockIdx.x];
+  } else {
+    const RdkvUnit *u = units + blockIdx.x;
+    q_row = u->q_row;
+    work_begin = u->work_begin;
+    work_count = u->work_count;
+  }
+  if (work_count == 0) return;  // a further source of an output row: merged by the row's first unit
   const int kv_row = q_row / G;    // zone-C tensors are indexed by output (group, KV head)
-  // the query (and its rotation table) is fetched before the merge so that the two overlap
-  const int n_new = n_new_per_unit ? n_new_per_unit[kv_row] : n_new_all;
-  // the zone-C row of this step (device-held, so that a replayed graph needs nothing from the host)
-  const int64_t step_row = ap.k ? ap.row_dev[0] : 0;
-  const int q_block_start = ts.q_block_start >= 0 || ts.block <= 0 ? ts.q_block_start
-                                                                    : (int)(step_row / ts.block) * ts.block;
-  if (ap.k) {
-    // The step's own token joins zone C here (first wavefront; the others go on): k rotated and
-    // rounded to its storage type as the in-place rotation stores it, k and v widened to fp32.
-    // The barriers between here and the token loop make the row visible to every wavefront.
-    const int64_t row = step_row;
-    if (row >= 0 && row < ap.capacity && tid < 64) {
-      const int64_t ko = (int64_t)kv_row * ap.k_stride_h, vo = (int64_t)kv_row * ap.v_stride_h;
-      const float lo = rdkv_load_as_float_nobranch(ap.k, ap.dtype, ko + tid);
-      const float hi = rdkv_load_as_float_nobranch(ap.k, ap.dtype, ko + tid + 64);
-      const float v_lo = rdkv_load_as_float_nobranch(ap.v, ap.dtype, vo + tid);
-      const float v_hi = rdkv_load_as_float_nobranch(ap.v, ap.dtype, vo + tid + 64);
-      float out_lo = lo, out_hi = hi;
-      if (rope_cos) {
-        const float c = rdkv_load_as_float_nobranch(rope_cos, rope_dtype, tid);
-        const float sn = rdkv_load_as_float_nobranch(rope_sin, rope_dtype, tid);
-        rdkv_rope_pair(lo, hi, c, sn, out_lo, out_hi);
-        out_lo = rdkv_round_to_dtype(out_lo, ap.dtype);
-        out_hi = rdkv_round_to_dtype(out_hi, ap.dtype);
-      }
-      const int64_t off = (int64_t)kv_row * new_stride_unit + row * new_stride_tok;
-      float *kd = k_new + off, *vd = v_new + off;
-      kd[tid] = out_lo;
-      kd[tid + 64] = out_hi;
-      vd[tid] = v_lo;
-      vd[tid + 64] = v_hi;
+
+  // ---- one round trip: everything else, requested before anything is used ------------------------
+  // The zone-C row of this step (device-held, so that a replayed graph needs nothing from the host)
+  // and the unit's token count: requested as vector loads like everything else (an address the
+  // compiler cannot prove uniform), so that nothing waits for them before the other requests are out.
+  int lane_zero;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(lane_zero));
+  const int64_t *row_ptr = (ap.k ? ap.row_dev : reinterpret_cast<const int64_t *>(units)) + lane_zero;
+  const int32_t *cnt_ptr = (n_new_per_unit ? n_new_per_unit + kv_row : reinterpret_cast<const int32_t *>(units)) + lane_zero;
+  const int64_t step_row_v = *row_ptr;
+  const int32_t n_new_v = *cnt_ptr;
+  // (a) the step's own key / value row and its rotation angles (first wavefront): lane l takes
+  // channels l and l + 64
+  uint32_t a_raw[6] = {0u, 0u, 0u, 0u, 0u, 0u};
+  const int64_t a_ko = (int64_t)kv_row * ap.k_stride_h, a_vo = (int64_t)kv_row * ap.v_stride_h;
+  if (ap.k && wave == 0) {
+    a_raw[0] = rdkv_load_dword_of(ap.k, ap.dtype, a_ko + lane);
+    a_raw[1] = rdkv_load_dword_of(ap.k, ap.dtype, a_ko + lane + 64);
+    a_raw[2] = rdkv_load_dword_of(ap.v, ap.dtype, a_vo + lane);
+    a_raw[3] = rdkv_load_dword_of(ap.v, ap.dtype, a_vo + lane + 64);
+    if (rope_cos) {
+      a_raw[4] = rdkv_load_dword_of(rope_cos, rope_dtype, lane);
+      a_raw[5] = rdkv_load_dword_of(rope_sin, rope_dtype, lane);
     }
   }
-  float qv[2], qo[2], qc[2], qs_[2];
+  // (b) the query rows, each element with its rotation partner and angle
+  uint32_t q_raw[kCols][4];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < kCols; ++j) {
     const int i = tid + j * kThreads;
     const int ic = i < G * kD ? i : 0;
     const int c = ic & 127;
     const int64_t row = (int64_t)(q_row + (ic >> 7)) * q_stride;
-    qv[j] = rdkv_load_as_float_nobranch(q, q_dtype, row + c);
-    qo[j] = rdkv_load_as_float_nobranch(q, q_dtype, row + (c ^ 64));
-    qc[j] = rdkv_load_as_float_nobranch(rope_cos ? rope_cos : q, rope_cos ? rope_dtype : q_dtype, rope_cos ? (c & 63) : row);
-    qs_[j] = rdkv_load_as_float_nobranch(rope_sin ? rope_sin : q, rope_sin ? rope_dtype : q_dtype, rope_sin ? (c & 63) : row);
+    q_raw[j][0] = rdkv_load_dword_of(q, q_dtype, row + c);
+    q_raw[j][1] = q_raw[j][2] = q_raw[j][3] = 0u;
+    if (rope_cos) {
+      q_raw[j][1] = rdkv_load_dword_of(q, q_dtype, row + (c ^ 64));
+      q_raw[j][2] = rdkv_load_dword_of(rope_cos, rope_dtype, c & 63);
+      q_raw[j][3] = rdkv_load_dword_of(rope_sin, rope_dtype, c & 63);
+    }
   }
-  merge_unit(partials, u->work_begin, u->work_count, G, q_row, out, out_stride, lse, tid, kThreads, scratch,
-             acc_ab, lse_ab);
+  // (c) the partials: max / sum columns (thread i takes partial i / G, head i % G), then the first
+  // kAhead accumulator values of each of the thread's output columns, eight partials at a time
+  const int n_part = work_count;
+  const int64_t pstride = (int64_t)G * kPartialStride;
+  const float *base0 = partials + (int64_t)work_begin * pstride;
+  const bool staged = n_part <= kMergeMaxK;        // the max / sum columns fit in LDS (else: plain loops)
+  constexpr int kMl = (kMergeMaxK * G + kThreads - 1) / kThreads;
+  float pm[kMl], pl[kMl];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < kMl; ++j) {
+    pm[j] = pl[j] = 0.0f;
+    if (j * kThreads < n_part * G) {      // uniform: later batches only for units with many partials
+      const int i = tid + j * kThreads;
+      const int ic = (staged && i < n_part * G) ? i : 0;
+      const int k = ic / G, h = ic - k * G;
+      pm[j] = base0[k * pstride + h * kPartialStride + 128];
+      pl[j] = base0[k * pstride + h * kPartialStride + 129];
+    }
+  }
+  float ahead[kCols][kAhead];
+#pragma unroll
+  for (int j = 0; j < kCols; ++j) {
+    const int i = tid + j * kThreads;
+    const int ic = i < G * kD ? i : 0;
+    const float *b0 = base0 + (ic >> 7) * kPartialStride + (ic & 127);
+#pragma unroll
+    for (int e0 = 0; e0 < kAhead; e0 += 8) {
+#pragma unroll
+      for (int e = e0; e < e0 + 8; ++e) ahead[j][e] = 0.0f;
+      if (e0 < n_part) {                  // uniform
+#pragma unroll
+        for (int e = e0; e < e0 + 8; ++e) ahead[j][e] = b0[(e < n_part ? e : 0) * pstride];
+      }
+    }
+  }
+  // (d) the first chunk of zone C.  K: token 8 * wave + lane / 8, sixteen of its channels (four
+  // 16-byte pieces, piece j of lane group member c being floats 32j + 4c ..); V: tokens 8 * wave + i,
+  // channels 2 * lane and 2 * lane + 1.  Rows are requested up to the buffer's last row.
+  const int tg = lane >> 3, kc = lane & 7;
+  const float *kn = k_new + (int64_t)kv_row * new_stride_unit;
+  const float *vn = v_new + (int64_t)kv_row * new_stride_unit;
+  const int last_row = n_new_all > 0 ? n_new_all - 1 : 0;
+  const bool have_rows = n_new_all > 0 && k_new != nullptr;
+  float4 kreg[4];
+  float2 vreg[8];
+  auto request_chunk = [&](int t0) __attribute__((always_inline)) {
+    const int tw = t0 + 8 * wave;
+    if (!have_rows || tw > last_row) return;     // uniform
+    const int tr = tw + tg < last_row ? tw + tg : last_row;
+    const float4 *kr = reinterpret_cast<const float4 *>(kn + (int64_t)tr * new_stride_tok);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kreg[j] = kr[8 * j + kc];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int tvr = tw + i < last_row ? tw + i : last_row;
+      vreg[i] = reinterpret_cast<const float2 *>(vn + (int64_t)tvr * new_stride_tok)[lane];
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < 4; ++j) kreg[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) vreg[i] = make_float2(0.f, 0.f);
+  request_chunk(0);
+  const int64_t step_row = ap.k ? (int64_t)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(step_row_v >> 32)) << 32) |
+                                            (uint32_t)__builtin_amdgcn_readfirstlane((int)step_row_v))
+                                : -1;
+  int n_new = n_new_per_unit ? __builtin_amdgcn_readfirstlane(n_new_v) : n_new_all;
+  n_new = n_new < n_new_all ? n_new : n_new_all;   // never past the buffer
+  n_new = n_new > 0 ? n_new : 0;
+  const bool appending = ap.k != nullptr && step_row >= 0 && step_row < ap.capacity;
+
+  // ---- the step's own token joins zone C (first wavefront) --------------------------------------
+  // k rotated and rounded to its storage type as the in-place rotation stores it, k and v widened
+  // to fp32; the row goes to memory for the steps to come and to LDS for this one.
+  if (ap.k && wave == 0) {
+    const float k_lo = rdkv_decode_dword(a_raw[0], ap.k, ap.dtype, a_ko + lane);
+    const float k_hi = rdkv_decode_dword(a_raw[1], ap.k, ap.dtype, a_ko + lane + 64);
+    const float v_lo = rdkv_decode_dword(a_raw[2], ap.v, ap.dtype, a_vo + lane);
+    const float v_hi = rdkv_decode_dword(a_raw[3], ap.v, ap.dtype, a_vo + lane + 64);
+    float out_lo = k_lo, out_hi = k_hi;
+    if (rope_cos) {
+      const float cs = rdkv_decode_dword(a_raw[4], rope_cos, rope_dtype, lane);
+      const float sn = rdkv_decode_dword(a_raw[5], rope_sin, rope_dtype, lane);
+      rdkv_rope_pair(k_lo, k_hi, cs, sn, out_lo, out_hi);
+      out_lo = rdkv_round_to_dtype(out_lo, ap.dtype);
+      out_hi = rdkv_round_to_dtype(out_hi, ap.dtype);
+    }
+    k_self[lane] = out_lo;
+    k_self[lane + 64] = out_hi;
+    v_self[lane] = v_lo;
+    v_self[lane + 64] = v_hi;
+    if (appending) {
+      const int64_t off = (int64_t)kv_row * new_stride_unit + step_row * new_stride_tok;
+      float *kd = k_new + off, *vd = v_new + off;
+      kd[lane] = out_lo;
+      kd[lane + 64] = out_hi;
+      vd[lane] = v_lo;
+      vd[lane + 64] = v_hi;
+    }
+  }
+  // ---- the query: rotated, rounded to its storage type, scaled, staged --------------------------
+  const int q_block_start = ts.q_block_start >= 0 || ts.block <= 0 ? ts.q_block_start
+                                                                    : (int)((step_row < 0 ? 0 : step_row) / ts.block) * ts.block;
+#pragma unroll
+  for (int j = 0; j < kCols; ++j) {
     const int i = tid + j * kThreads;
     if (i < G * kD) {
       const int c = i & 127;
-      float v = qv[j];
+      const int64_t row = (int64_t)(q_row + (i >> 7)) * q_stride;
+      float v = rdkv_decode_dword(q_raw[j][0], q, q_dtype, row + c);
       if (rope_cos) {
+        const float other = rdkv_decode_dword(q_raw[j][1], q, q_dtype, row + (c ^ 64));
+        const float cs = rdkv_decode_dword(q_raw[j][2], rope_cos, rope_dtype, c & 63);
+        const float sn = rdkv_decode_dword(q_raw[j][3], rope_sin, rope_dtype, c & 63);
         float out_lo, out_hi;
-        if (c < 64) rdkv_rope_pair(v, qo[j], qc[j], qs_[j], out_lo, out_hi);
-        else rdkv_rope_pair(qo[j], v, qc[j], qs_[j], out_lo, out_hi);
+        if (c < 64) rdkv_rope_pair(v, other, cs, sn, out_lo, out_hi);
+        else rdkv_rope_pair(other, v, cs, sn, out_lo, out_hi);
         v = rdkv_round_to_dtype(c < 64 ? out_lo : out_hi, q_dtype);
       }
-      qz[i >> 7][c] = v * 0.08838834764831845f;   // 1/sqrt(128)
+      qz[i >> 7][c] = v * kLog2eOverSqrtD;
       // the rotated query as the in-place rotation would have left it, for callers that keep it (a
       // buffer with one row per token takes it at the step's row, under the same range check as the
       // appended key: a device-held row that has run past the buffer writes nothing)
-      if (q_rot_out && (ts.q_rotated_stride_tok == 0 || (step_row >= 0 && step_row < ap.capacity)))
+      if (q_rot_out && (ts.q_rotated_stride_tok == 0 || appending))
         rdkv_store_from_float(q_rot_out, q_dtype,
-                              (int64_t)(q_row + (i >> 7)) * q_rot_stride + step_row * ts.q_rotated_stride_tok + c, v);
+                              (int64_t)(q_row + (i >> 7)) * q_rot_stride +
+                                  (ts.q_rotated_stride_tok ? step_row * ts.q_rotated_stride_tok : 0) + c, v);
     }
   }
-  __syncthreads();
+  // ---- the partials' max / sum columns ----------------------------------------------------------
+  if (staged) {
+#pragma unroll
+    for (int j = 0; j < kMl; ++j) {
+      const int i = tid + j * kThreads;
+      if (i < n_part * G) {
+        const int k = i / G, h = i - k * G;
+        scratch[kMergeM + k * 8 + h] = pm[j];
+        scratch[kMergeL + k * 8 + h] = pl[j];
+      }
+    }
+  }
+  __syncthreads();   // qz, k_self / v_self, s_m / s_l
 
-  const float *kn = k_new + (int64_t)kv_row * new_stride_unit;
-  const float *vn = v_new + (int64_t)kv_row * new_stride_unit;
+  // ---- zones A+B: the softmax factors of the unit's partials, once per (partial, head) ------------
+  // (stage 2 of the merge; the accumulator columns are weighted with these factors after the token
+  // loop, behind the barrier that ends it)
+  if (staged) merge_factors(n_part, G, wave, lane, kZcWaves, scratch);
+
+  // ---- zone C, 64 tokens at a time, eight per wavefront ------------------------------------------
   float m_run[G], l_run[G], acc[G][2];
 #pragma unroll
   for (int h = 0; h < G; ++h) {
@@ -1028,64 +1269,55 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
     l_run[h] = 0.0f;
     acc[h][0] = acc[h][1] = 0.0f;
   }
-  for (int t0 = wave * kZcChunk; t0 < n_new; t0 += kZcWaves * kZcChunk) {
-    const int nt = n_new - t0 < kZcChunk ? n_new - t0 : kZcChunk;
-    const bool valid = lane < nt;
-    // scores of this lane's token against the G query heads
-    float s[G];
+  const int self_tok = appending ? (int)step_row : -1;
+  const float2 v_own = reinterpret_cast<const float2 *>(v_self)[lane];
+  for (int t0 = 0; t0 + 8 * wave < n_new; t0 += kZcChunk) {
+    const int tw = t0 + 8 * wave;                 // this wavefront's first token of the chunk: exists
+    // this chunk's rows, the step's own token from LDS; then the next chunk's rows are requested
+    float4 kcur[4];
+    float2 vcur[8];
+    const bool k_is_self = tw + tg == self_tok;
 #pragma unroll
-    for (int h = 0; h < G; ++h) s[h] = 0.0f;
-    const float4 *kr = reinterpret_cast<const float4 *>(kn + (int64_t)(t0 + (valid ? lane : 0)) * new_stride_tok);
-#pragma unroll 1
-    for (int c0 = 0; c0 < kD / 4; c0 += 16) {
-      float4 kv[16];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) kv[e] = kr[c0 + e];
-#pragma unroll
-      for (int e = 0; e < 16; ++e) {
-#pragma unroll
-        for (int h = 0; h < G; ++h) {
-          const float4 qv = reinterpret_cast<const float4 *>(qz[h])[c0 + e];
-          s[h] += kv[e].x * qv.x + kv[e].y * qv.y + kv[e].z * qv.z + kv[e].w * qv.w;
-        }
-      }
+    for (int j = 0; j < 4; ++j) {
+      const float4 ks = reinterpret_cast<const float4 *>(k_self)[8 * j + kc];
+      kcur[j] = k_is_self ? ks : kreg[j];
     }
-    if (zc_w && valid) {      // raw scores now, turned into weights once the union's maximum and sum are known
 #pragma unroll
-      for (int h = 0; h < G; ++h) zc_w[(int64_t)(q_row + h) * zc_w_stride + t0 + lane] = s[h];
+    for (int i = 0; i < 8; ++i) {
+      vcur[i] = tw + i == self_tok ? v_own : vreg[i];
+      if (tw + i >= n_new) vcur[i] = make_float2(0.f, 0.f);     // a row past the count may hold anything
     }
+    if (tw + kZcChunk < n_new) request_chunk(t0 + kZcChunk);
+    // scores of this lane group's token against the G query heads: sixteen channels per lane
+    const bool tok_valid = tw + tg < n_new;
     float wt[G];
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      const float sh = valid ? s[h] : -INFINITY;
-      const float m_new = fmaxf(m_run[h], rdkv_wave_max(sh));     // finite: the chunk has a token
-      const float f = m_run[h] == -INFINITY ? 0.0f : expf(m_run[h] - m_new);
-      wt[h] = valid ? expf(sh - m_new) : 0.0f;
-      l_run[h] = l_run[h] * f + rdkv_wave_sum(wt[h]);
+      float a = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 qq = reinterpret_cast<const float4 *>(qz[h])[8 * j + kc];
+        a += kcur[j].x * qq.x + kcur[j].y * qq.y + kcur[j].z * qq.z + kcur[j].w * qq.w;
+      }
+      const float sh = tok_valid ? zc_oct_sum(a) : -INFINITY;
+      // raw scores now, turned into weights once the union's maximum and sum are known
+      if (zc_w && kc == 0 && tok_valid) zc_w[(int64_t)(q_row + h) * zc_w_stride + tw + tg] = sh;
+      const float m_new = fmaxf(m_run[h], zc_tokens_reduce<true>(sh));    // finite: token tw exists
+      const float f = fast_exp2(m_run[h] - m_new);                         // 0 on the first chunk
+      wt[h] = fast_exp2(sh - m_new);                                       // 0 for a token past the count
+      l_run[h] = l_run[h] * f + zc_tokens_reduce<false>(wt[h]);
       acc[h][0] *= f;
       acc[h][1] *= f;
       m_run[h] = m_new;
     }
-    // values: lane = channels lane and lane + 64, the weight of token tt comes from lane tt
-    const float *vr = vn + (int64_t)t0 * new_stride_tok;
-    for (int tt0 = 0; tt0 < nt; tt0 += 16) {
-      float v0[16], v1[16];
+    // values: token tw + i, its weight read from the first lane of its group
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int tt = tt0 + e < nt ? tt0 + e : nt - 1;
-        v0[e] = vr[(int64_t)tt * new_stride_tok + lane];
-        v1[e] = vr[(int64_t)tt * new_stride_tok + lane + 64];
-      }
+    for (int i = 0; i < 8; ++i) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        if (tt0 + e < nt) {
-#pragma unroll
-          for (int h = 0; h < G; ++h) {
-            const float w = __shfl(wt[h], tt0 + e, 64);
-            acc[h][0] += w * v0[e];
-            acc[h][1] += w * v1[e];
-          }
-        }
+      for (int h = 0; h < G; ++h) {
+        const float w = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, wt[h]), 8 * i));
+        acc[h][0] += w * vcur[i].x;
+        acc[h][1] += w * vcur[i].y;
       }
     }
   }
@@ -1095,35 +1327,45 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
       w_m[wave][h] = m_run[h];
       w_l[wave][h] = l_run[h];
     }
-    w_acc[wave][h][lane] = acc[h][0];
-    w_acc[wave][h][lane + 64] = acc[h][1];
+    reinterpret_cast<float2 *>(w_acc[wave][h])[lane] = make_float2(acc[h][0], acc[h][1]);
   }
   __syncthreads();
-  for (int i = tid; i < G * kD; i += kThreads) {
-    const int h = i >> 7, d = i & 127;
-    float M = lse_ab[h];
+  // ---- the union: zones A+B as one pseudo-token, the eight wavefront states of zone C ------------
 #pragma unroll
-    for (int w = 0; w < kZcWaves; ++w) M = fmaxf(M, w_m[w][h]);
-    float o = 0.0f, l = 0.0f;
-    if (lse_ab[h] != -INFINITY) {
-      const float f = expf(lse_ab[h] - M);
-      o = f * acc_ab[i];
-      l = f;
-    }
+  for (int j = 0; j < kCols; ++j) {
+    const int i = tid + j * kThreads;
+    if (i < G * kD) {
+      const int h = i >> 7, d = i & 127;
+      // zones A+B: this column of the partials under their factors, normalized (stage 3 of the merge)
+      float o_ab, mab;
+      if (staged) {
+        o_ab = merge_column<false>(n_part, h, ahead[j], base0 + h * kPartialStride + d, pstride, scratch);
+        mab = scratch[kMergeL2 + h];
+      } else {
+        o_ab = merge_column_long<false>(n_part, base0 + h * kPartialStride, d, pstride, mab);
+      }
+      float M = mab;
 #pragma unroll
-    for (int w = 0; w < kZcWaves; ++w) {
-      const float mw = w_m[w][h];
-      if (mw != -INFINITY) {
-        const float f = expf(mw - M);
+      for (int w = 0; w < kZcWaves; ++w) M = fmaxf(M, w_m[w][h]);
+      float o = 0.0f, l = 0.0f;
+      {
+        const float f = mab == -INFINITY ? 0.0f : fast_exp2(mab - M);
+        o = f * o_ab;
+        l = f;
+      }
+#pragma unroll
+      for (int w = 0; w < kZcWaves; ++w) {
+        const float mw = w_m[w][h];
+        const float f = mw == -INFINITY ? 0.0f : fast_exp2(mw - M);
         o += f * w_acc[w][h][d];
         l += f * w_l[w][h];
       }
-    }
-    out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? o / l : 0.0f;
-    if (lse && d == 0) lse[q_row + h] = l > 0.0f ? M + logf(l) : -INFINITY;
-    if (d == 0) {
-      fin_m[h] = M;
-      fin_l[h] = l;
+      out[(int64_t)(q_row + h) * out_stride + d] = l > 0.0f ? o / l : 0.0f;
+      if (lse && d == 0) lse[q_row + h] = l > 0.0f ? (M + log2f(l)) * kLn2 : -INFINITY;
+      if (d == 0) {
+        fin_m[h] = M;
+        fin_l[h] = l;
+      }
     }
   }
   if (zc_w) {   // softmax weights of the zone C tokens over the union (fast_decode.py:1753-1755 w_new)
@@ -1135,7 +1377,7 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, const float *__restrict_
 #pragma clang fp contract(off)   // the stored weight is what is summed: no fusing with the product
         float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
         const float inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
-        const float w = expf(row[t] - fin_m[h]) * inv;
+        const float w = fast_exp2(row[t] - fin_m[h]) * inv;
         row[t] = w;
         s = s + w;
       }
@@ -1275,7 +1517,8 @@ RDKV_API int rdkv_decode_fused_one_launch(const uint8_t *blob, const RdkvUnit *u
                       out, out_stride_row, lse);
 }
 
-static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
+static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, const RdkvUnit *units_host, int n_units,
+                               int n_work, int G, const void *q,
                                int q_dtype, int64_t q_stride_row, const void *rope_cos, const void *rope_sin,
                                int rope_dtype, const float *k_new, const float *v_new, int64_t new_stride_unit,
                                int64_t new_stride_tok, int n_new, const int32_t *n_new_per_unit, float *out,
@@ -1296,12 +1539,29 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
   RDKV_REQUIRE(n_new == 0 || (k_new && v_new), "%s: null zone-C tensors", fn);
   RDKV_REQUIRE(((uintptr_t)k_new % 16) == 0 && new_stride_unit % 4 == 0 && new_stride_tok % 4 == 0,
                "%s: zone-C key rows must be 16-byte aligned", fn);
-#define RDKV_LAUNCH_ZC(GT)                                                                                    \
-  hipLaunchKernelGGL(merge_zone_c_kernel<GT>, dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, units, \
-                     (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,        \
-                     const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit, new_stride_tok,   \
-                     n_new, n_new_per_unit, out, out_stride_row, lse,                                           \
-                     zone_c_weights, zone_c_weights_stride_row, append, q_rot_out, q_rot_stride, tail)
+  // a short unit table whose host copy the caller has: its merge fields travel with the kernel
+  // arguments, and the launch's first memory round trip goes to the data instead of the table
+  ZcInline iu;
+  iu.n = 0;
+  if (units_host && n_units <= kZcInlineUnits) {
+    iu.n = n_units;
+    for (int i = 0; i < n_units; ++i) {
+      iu.q_row[i] = units_host[i].q_row;
+      iu.work_begin[i] = units_host[i].work_begin;
+      iu.work_count[i] = units_host[i].work_count;
+    }
+  }
+#define RDKV_LAUNCH_ZC_I(GT, INL)                                                                             \
+  hipLaunchKernelGGL((merge_zone_c_kernel<GT, INL>), dim3(n_units), dim3(64 * kZcWaves), 0, (hipStream_t)stream, \
+                     units, iu, (const float *)workspace, q, q_dtype, q_stride_row, rope_cos, rope_sin,         \
+                     rope_dtype, const_cast<float *>(k_new), const_cast<float *>(v_new), new_stride_unit,       \
+                     new_stride_tok, n_new, n_new_per_unit, out, out_stride_row, lse, zone_c_weights,           \
+                     zone_c_weights_stride_row, append, q_rot_out, q_rot_stride, tail)
+#define RDKV_LAUNCH_ZC(GT)                  \
+  do {                                      \
+    if (iu.n > 0) RDKV_LAUNCH_ZC_I(GT, true); \
+    else RDKV_LAUNCH_ZC_I(GT, false);       \
+  } while (0)
   switch (G) {
     case 1: RDKV_LAUNCH_ZC(1); break;
     case 2: RDKV_LAUNCH_ZC(2); break;
@@ -1313,11 +1573,13 @@ static int launch_merge_zone_c(const char *fn, const RdkvUnit *units, int n_unit
     default: RDKV_LAUNCH_ZC(8); break;
   }
 #undef RDKV_LAUNCH_ZC
+#undef RDKV_LAUNCH_ZC_I
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;
 }
 
-RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, int n_work, int G, const void *q,
+RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, const RdkvUnit *units_host, int n_units,
+                                            int n_work, int G, const void *q,
                                             int q_dtype, int64_t q_stride_row, const void *rope_cos,
                                             const void *rope_sin, int rope_dtype, const float *k_new,
                                             const float *v_new, int64_t new_stride_unit, int64_t new_stride_tok,
@@ -1326,7 +1588,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
                                             int64_t zone_c_weights_stride_row, void *workspace,
                                             int64_t workspace_bytes, void *stream) {
   const ZcAppend none = {nullptr, nullptr, 0, 0, nullptr, 0, 0};
-  return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, n_units, n_work, G, q, q_dtype, q_stride_row,
+  return launch_merge_zone_c("rdkv_decode_fused_merge_zone_c", units, units_host, n_units, n_work, G, q, q_dtype,
+                             q_stride_row,
                              rope_cos, rope_sin, rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, n_new,
                              n_new_per_unit, out, out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row,
                              workspace, workspace_bytes, none, nullptr, 0, RdkvTailScores{nullptr, 0, nullptr, 0, 0, 0, 0},
@@ -1334,7 +1597,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c(const RdkvUnit *units, int n_units, 
 }
 
 RDKV_API int rdkv_decode_fused_merge_zone_c_append(
-    const RdkvUnit *units, int n_units, int n_work, int G, const void *q, int q_dtype, int64_t q_stride_row,
+    const RdkvUnit *units, const RdkvUnit *units_host, int n_units, int n_work, int G, const void *q, int q_dtype,
+    int64_t q_stride_row,
     const void *rope_cos, const void *rope_sin, int rope_dtype, float *k_new, float *v_new, int64_t new_stride_unit,
     int64_t new_stride_tok, int64_t capacity, const int32_t *n_new_per_unit, const void *k_step, int64_t k_stride_h,
     const void *v_step, int64_t v_stride_h, int kv_dtype, const int64_t *row_dev, float *out, int64_t out_stride_row,
@@ -1359,8 +1623,8 @@ RDKV_API int rdkv_decode_fused_merge_zone_c_append(
                  "%s: bad stride of the rotated-query buffer", fn);
   }
   const ZcAppend ap = {k_step, v_step, k_stride_h, v_stride_h, row_dev, capacity, kv_dtype};
-  return launch_merge_zone_c(fn, units, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin, rope_dtype,
-                             k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
+  return launch_merge_zone_c(fn, units, units_host, n_units, n_work, G, q, q_dtype, q_stride_row, rope_cos, rope_sin,
+                             rope_dtype, k_new, v_new, new_stride_unit, new_stride_tok, (int)capacity, n_new_per_unit, out,
                              out_stride_row, lse, zone_c_weights, zone_c_weights_stride_row, workspace,
                              workspace_bytes, ap, q_rotated_out, q_rotated_stride_row, tail, stream);
 }

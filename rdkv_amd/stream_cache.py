@@ -616,7 +616,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
                                        next_s.stride(0) if next_s is not None else 0,
                                        -1 if q_block_start is None else int(q_block_start), int(block), int(q_rot_tok))
         _lib.check(lib.rdkv_decode_fused_merge_zone_c_append(
-            cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
+            cache.units.data_ptr(), cache.units_host.ctypes.data, cache.n_units, cache.n_work, cache.G,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
             _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
             counts.data_ptr(), k_step.data_ptr(), k_step.stride(0), v_step.data_ptr(), v_step.stride(0),
@@ -633,7 +633,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         assert zone_c_weights.shape[0] == cache.rows and zone_c_weights.shape[1] >= n_new, (
             f"zone_c_weights must be [rows = {cache.rows}, >= {n_new}], got {tuple(zone_c_weights.shape)}")
     _lib.check(lib.rdkv_decode_fused_merge_zone_c(
-        cache.units.data_ptr(), cache.n_units, cache.n_work, cache.G,
+        cache.units.data_ptr(), cache.units_host.ctypes.data, cache.n_units, cache.n_work, cache.G,
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         _lib.ptr(K_new), _lib.ptr(V_new), K_new.stride(0), K_new.stride(1) if n_new else 128, n_new,
         _lib.ptr(counts), out.data_ptr(), out.stride(0), lse.data_ptr(), _lib.ptr(zone_c_weights),
