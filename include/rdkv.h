@@ -321,6 +321,28 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
                                const void *kzp_f16, int64_t ks_stride_h, const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
                                int H_kv, int n8, int max_tiles, uint8_t *blob, void *stream);
 
+/* The prefill packer that writes the streaming format directly: fp16 K and V [H_kv, T, 128] ->
+ * the blob a rdkv_pack_layer_per_head call followed by rdkv_stream_relayout_layer would produce,
+ * bit for bit (the composition of obkv_fast.py:1141-1155, packing.py:801-1013 and
+ * packing.py:1019-1317, then the re-layout), without the padded intermediate: two launches (the
+ * per-channel K min / max, then one workgroup per 64-token tile and head).  order / counts: as
+ * rdkv_pack_layer_plan leaves them (token order by width class, [H_kv, 4] class sizes; device).
+ * k_bits [H_kv, 128]: integers of kb_elem_size bytes, 16 counted as 8, 0 = pruned (device).
+ * n2p / n4p / n8: the layer's padded channel counts (maxima over heads; what src_slot refers to);
+ * max_tv / max_n16: maxima over heads of the quantized / fp16-kept token counts (a head below
+ * either has zero rows in the reference's K canvas, packing.py:1186-1215, so 0 joins its
+ * per-channel min / max).  units (device, offsets relative to blob), src_slot, n_slots_max,
+ * max_tiles: as for rdkv_stream_relayout_layer.  minmax_ws: H_kv * 256 floats of scratch.
+ * scale_max: float [2][H_kv], zero before the call: receives per head the largest K channel scale
+ * and the largest V token scale (as the fp16 values stored), which RdkvWork.k_scale_max / v_shift
+ * are made from.  K and V rows must be 16-byte aligned (RDKV_EUNSUPPORTED otherwise). */
+int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
+                           int H_kv, const int32_t *order, int64_t order_stride_h, const int32_t *counts,
+                           const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int n2p, int n4p, int n8,
+                           int64_t max_tv, int max_n16, const RdkvUnit *units, const int16_t *src_slot,
+                           int n_slots_max, int max_tiles, uint8_t *blob, float *minmax_ws, float *scale_max,
+                           void *stream);
+
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit
  * without tokens), so callers can merge further zones exactly.  G = query heads per KV head

@@ -60,6 +60,7 @@ SIGNATURES = {
     "rdkv_softmax_rows_ws": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P, L, P]),
     "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
     "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
+    "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, P, P, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,
                                        P, L, P, P, L, P, P, I, I, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),

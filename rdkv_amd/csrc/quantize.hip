@@ -1263,6 +1263,40 @@ static int pack_layer_v_rows(const char *fn, const void *V_f16, int64_t stride_h
   return RDKV_OK;
 }
 
+// Per-channel min / max over each head's kept rows into mm (per head D minima then D maxima, in the
+// order-preserving integer encoding); `init` writes the start values (+inf, -inf) first.
+static int layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                          const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tk,
+                          uint32_t *mm, bool init, hipStream_t s) {
+  if (init)
+    hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256), 0,
+                       s, mm, D, H_kv);
+  if (max_tk == 0) return RDKV_OK;
+  const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
+  RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
+  const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
+  if (rows16) {
+    hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
+                       dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv),
+                       dim3(64 * RDKV_LAYER_MINMAX_WAVES_D128), 0, s,
+                       (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
+  } else {
+    hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
+                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+  }
+  return RDKV_OK;
+}
+
+// (for the packer that writes the streaming format, stream_pack.hip)
+int rdkv_layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                        const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tk,
+                        float *minmax_ws, hipStream_t s) {
+  RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0, "%s: rows must be 4-byte aligned",
+               fn);
+  return layer_k_minmax(fn, K_f16, stride_h, stride_t, H_kv, D, order, order_stride_h, counts, max_tk,
+                        reinterpret_cast<uint32_t *>(minmax_ws), true, s);
+}
+
 // The K half: per-channel min/max over each head's kept rows, then scales, zero points and the
 // packed K segments.  `mm_ready` says the accumulators in `minmax_ws` already hold their start
 // values (the V half wrote them on the same stream).
@@ -1287,21 +1321,11 @@ static int pack_layer_k_rows(const char *fn, const void *K_f16, int64_t stride_h
                    (n8 == 0 || K8),
                "%s: null K output", fn);
   uint32_t *mm = reinterpret_cast<uint32_t *>(minmax_ws);
-  // (+inf, -inf) in the ordered-int encoding, per head D mins then D maxes
-  if (!mm_ready)
-    hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256), 0,
-                       s, mm, D, H_kv);
-  const int64_t mblocks = rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS);
-  RDKV_REQUIRE(mblocks <= 0x7fffffffLL, "%s: too many rows", fn);
   const bool rows16 = D == 128 && stride_t % 8 == 0 && stride_h % 8 == 0 && ((uintptr_t)K_f16 % 16) == 0;
-  if (rows16) {
-    hipLaunchKernelGGL(k_minmax_layer_d128_kernel,
-                       dim3((unsigned)rdkv_cdiv(max_tk, RDKV_LAYER_MINMAX_ROWS_D128), H_kv),
-                       dim3(64 * RDKV_LAYER_MINMAX_WAVES_D128), 0, s,
-                       (const __half *)K_f16, stride_h, stride_t, order, order_stride_h, counts, mm);
-  } else {
-    hipLaunchKernelGGL(k_minmax_layer_kernel, dim3((unsigned)mblocks, H_kv), dim3(64, 4), 0, s,
-                       (const __half *)K_f16, stride_h, stride_t, D, order, order_stride_h, counts, mm);
+  {
+    const int rc = layer_k_minmax(fn, K_f16, stride_h, stride_t, H_kv, D, order, order_stride_h, counts, max_tk, mm,
+                                  !mm_ready, s);
+    if (rc != RDKV_OK) return rc;
   }
   const int rows_per_block = 64;
   const int64_t eblocks = rdkv_cdiv(max_tk, rows_per_block);

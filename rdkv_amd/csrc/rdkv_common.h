@@ -32,6 +32,13 @@ void rdkv_set_error(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 
 static inline int64_t rdkv_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// Library-internal (quantize.hip): per-channel min / max of every head's kept K rows, gathered
+// through `order` (counts: device int32 [H_kv, 4]), into minmax_ws (H_kv * 2 * D floats, as
+// order-preserving integers).  Launches only.
+int rdkv_layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
+                        const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tk,
+                        float *minmax_ws, hipStream_t s);
+
 #define RDKV_WAVE 64
 
 __device__ __forceinline__ float rdkv_h2f(uint16_t bits) {

@@ -220,6 +220,54 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     return work, groups, work_begin, work_count
 
 
+def _plan_entry_units(tok, ch, n2p: int, n4p: int, first_row: int, G: int):
+    """Host side of one entry (a packed layer): the unit descriptors of its heads with offsets
+    relative to the entry's blob, the slot tables (stream slot -> position in the source layer's
+    padded sorted channel order), the blob size, the largest tile count of a head, and the streamed /
+    algorithmic byte counts.  tok[h] = (n2, n4, n8, n16) tokens, ch[h] = (c2, c4, c8) channels of
+    head h; head h answers query rows first_row + h * G .. + G."""
+    H_kv = len(tok)
+    units = np.zeros(H_kv, dtype=UNIT_DTYPE)
+    src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
+    off = 0
+    max_tiles = 0
+    stream_bytes = algo_bytes = 0
+    rows = []            # per head: the descriptor's fields, written to the record array in one go
+    for h in range(H_kv):
+        n_tok = tok[h]
+        c2, c4, c8 = ch[h]
+        d8, d4, d2, src = slot_plan(c2, c4, c8, n2p, n4p)
+        steps = d8 + 2 * d4 + 4 * d2
+        assert steps <= MAX_STEPS, f"{steps} channel steps exceed {MAX_STEPS}"
+        src_tab[h, :len(src)] = src
+        qt_nbytes = len(src) * SLOT_DTYPE.itemsize
+        tiles = [-(-n // TILE) for n in n_tok]
+        n_tiles, n_q_tiles = sum(tiles), sum(tiles[:3])
+        max_tiles = max(max_tiles, n_tiles)
+        R = d8 + d4 + d2
+        k_off = off
+        off = _align(off + n_tiles * TILE * 4 * R)
+        v_off = []
+        for c in range(4):
+            v_off.append(off)
+            off = _align(off + tiles[c] * V_TILE_BYTES[c])
+        sz_off = off
+        off = _align(off + n_q_tiles * TILE * 4)
+        qtab_off = off
+        off = _align(off + qt_nbytes)
+        rows.append((tuple(n_tok), d8, d4, d2, first_row + h * G, k_off, tuple(v_off), sz_off, qtab_off))
+        # accounting
+        stream_bytes += (n_tiles * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
+                         + n_q_tiles * TILE * 4 + qt_nbytes)
+        row = -(-c2 // 4) + -(-c4 // 2) + c8
+        algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
+                       + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
+                       + 256 * n_tok[3])
+    for i, name in enumerate(("n_tok", "d8", "d4", "d2", "q_row", "k_off", "v_off", "sz_off", "qtab_off")):
+        units[name] = [r[i] for r in rows]
+    return units, src_tab, off, max_tiles, int(stream_bytes), int(algo_bytes)
+
+
 def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_bytes: Optional[list] = None):
     """Re-lay every (packed layer, new_v_only) entry into its own blob.  Returns the unit
     descriptors (absolute addresses, work fields unset), the blobs, and the streamed / algorithmic
@@ -240,44 +288,9 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         tok, ch = _layer_counts(pl, H_kv)
         m2, m4, m8 = (int(v) for v in pl.K_ch_seg_bounds)
         n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
-        units = np.zeros(H_kv, dtype=UNIT_DTYPE)
-        src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
-        off = 0
-        max_tiles = 0
-        rows = []            # per head: the descriptor's fields, written to the record array in one go
-        for h in range(H_kv):
-            n_tok = tok[h]
-            c2, c4, c8 = ch[h]
-            d8, d4, d2, src = slot_plan(c2, c4, c8, n2p, n4p)
-            steps = d8 + 2 * d4 + 4 * d2
-            assert steps <= MAX_STEPS, f"{steps} channel steps exceed {MAX_STEPS}"
-            src_tab[h, :len(src)] = src
-            qt_nbytes = len(src) * SLOT_DTYPE.itemsize
-            tiles = [-(-n // TILE) for n in n_tok]
-            n_tiles, n_q_tiles = sum(tiles), sum(tiles[:3])
-            max_tiles = max(max_tiles, n_tiles)
-            R = d8 + d4 + d2
-            k_off = off
-            off = _align(off + n_tiles * TILE * 4 * R)
-            v_off = []
-            for c in range(4):
-                v_off.append(off)
-                off = _align(off + tiles[c] * V_TILE_BYTES[c])
-            sz_off = off
-            off = _align(off + n_q_tiles * TILE * 4)
-            qtab_off = off
-            off = _align(off + qt_nbytes)
-            rows.append((tuple(n_tok), d8, d4, d2, int(rows_of_entries[gi]) * H_q + h * G, k_off, tuple(v_off),
-                         sz_off, qtab_off))
-            # accounting
-            stream_bytes += (n_tiles * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
-                             + n_q_tiles * TILE * 4 + qt_nbytes)
-            row = -(-c2 // 4) + -(-c4 // 2) + c8
-            algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
-                           + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
-                           + 256 * n_tok[3])
-        for i, name in enumerate(("n_tok", "d8", "d4", "d2", "q_row", "k_off", "v_off", "sz_off", "qtab_off")):
-            units[name] = [r[i] for r in rows]
+        units, src_tab, off, max_tiles, sb, ab = _plan_entry_units(tok, ch, n2p, n4p, int(rows_of_entries[gi]) * H_q, G)
+        stream_bytes += sb
+        algo_bytes += ab
         plans.append((units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p))
         if entry_bytes is not None:
             entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
@@ -349,6 +362,146 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
     torch.cuda.current_stream(dev).synchronize()
     del keep_alive, units_dev, src_dev_all
     return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
+
+
+def _direct_packable(K: torch.Tensor, V: torch.Tensor) -> bool:
+    """Whether ``rdkv_pack_layer_stream`` takes these tensors: fp16 [1, H_kv, T, 128] on a device,
+    K and V of one stride pattern, rows 16-byte aligned."""
+    return (K.dim() == 4 and K.shape == V.shape and K.shape[0] == 1 and K.shape[3] == 128 and K.shape[2] > 0
+            and K.dtype == torch.float16 and V.dtype == torch.float16 and K.is_cuda and V.is_cuda
+            and K.stride() == V.stride() and K.stride(3) == 1 and K.stride(2) % 8 == 0 and K.stride(1) % 8 == 0
+            and K.data_ptr() % 16 == 0 and V.data_ptr() % 16 == 0)
+
+
+def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_bytes: Optional[list] = None):
+    """What ``_relayout_entries`` returns, from fp16 K / V and bit allocations instead of packed
+    layers: every entry (K, V [1, H_kv, T, 128] fp16, v_bits [H_kv, T], k_bits [H_kv, 128]) is
+    quantized and laid out by ``rdkv_pack_layer_stream`` in two launches, the blob being what the
+    per-layer packer followed by the re-layout writes, bit for bit.  One planning launch pair and one
+    host read serve all entries of one shape.  An entry the direct kernel does not take (other types
+    or strides, nothing kept, no K channel kept) goes through ``packing.pack_layer_per_head`` and the
+    re-layout instead."""
+    from . import packing
+    lib = _lib.load()
+    dev = _lib.require_device(entries[0][0])
+    stream = _lib.stream_of(dev)
+    n = len(entries)
+    out: list = [None] * n                       # per entry: (units, blob, stream bytes, algorithmic bytes, scale max)
+    H_q = None
+    # entries by shape: one plan per group
+    groups: dict = {}
+    for i, (K, V, vb, kb) in enumerate(entries):
+        H_q = int(K.shape[1]) * G
+        if _direct_packable(K, V):
+            groups.setdefault((int(K.shape[1]), int(K.shape[2])), []).append(i)
+        else:
+            groups.setdefault(("two-step", i), []).append(i)
+    pending = []                                 # (entry index, units, blob, scale_max tensor, keep-alive)
+    for key, idx in groups.items():
+        if key[0] == "two-step":
+            i = idx[0]
+            K, V, vb, kb = entries[i]
+            pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, G)
+            per = []
+            u, b, _, _, _, sm = _relayout_entries([(pl, nvo)], G, [rows_of_entries[i]], per)
+            out[i] = (u, b[0], per[0][0], per[0][1], sm)
+            continue
+        H_kv, T = key
+        vb_all = torch.cat([entries[i][2].reshape(H_kv, T) for i in idx]) if len(idx) > 1 else entries[idx[0]][2]
+        kb_all = torch.cat([entries[i][3].reshape(H_kv, 128) for i in idx]) if len(idx) > 1 else entries[idx[0]][3]
+        order, _, plan, counts_h, info_h, kb_dev = packing._plan_layers(vb_all.reshape(-1, T), kb_all.reshape(-1, 128), dev)
+        plans = []
+        for j, i in enumerate(idx):
+            rows = slice(j * H_kv, (j + 1) * H_kv)
+            tok = [tuple(int(x) for x in r[:4]) for r in counts_h[rows]]
+            ch = [tuple(int(x) for x in r[2:5]) for r in info_h[rows]]
+            m2, m4, m8 = (max(c[k] for c in ch) for k in range(3))
+            max_tv, max_n16 = max(sum(t[:3]) for t in tok), max(t[3] for t in tok)
+            if max_tv + max_n16 == 0 or m2 + m4 + m8 == 0:
+                plans.append(None)               # degenerate: the two-step path knows the reference's behaviour
+                continue
+            n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
+            units, src_tab, off, max_tiles, sb, ab = _plan_entry_units(tok, ch, n2p, n4p,
+                                                                       int(rows_of_entries[i]) * H_q, G)
+            plans.append((units, src_tab, off, max_tiles, sb, ab, n2p, n4p, m8, max_tv, max_n16))
+        live = [p for p in plans if p is not None]
+        if live:
+            units_dev = torch.from_numpy(np.concatenate([p[0] for p in live]).view(np.uint8).copy()).to(dev)
+            src_dev = torch.from_numpy(np.concatenate([p[1] for p in live])).to(dev)
+        row = 0
+        for j, (i, p) in enumerate(zip(idx, plans)):
+            K, V, vb, kb = entries[i]
+            if p is None:
+                pl, nvo = packing.pack_layer_per_head(K, V, vb, kb, G)
+                per = []
+                u, b, _, _, _, sm = _relayout_entries([(pl, nvo)], G, [rows_of_entries[i]], per)
+                out[i] = (u, b[0], per[0][0], per[0][1], sm)
+                continue
+            units, src_tab, off, max_tiles, sb, ab, n2p, n4p, m8, max_tv, max_n16 = p
+            blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
+            assert blob.data_ptr() % 256 == 0
+            mm = torch.empty(H_kv * 256, dtype=torch.float32, device=dev)
+            sm = torch.zeros(2, H_kv, dtype=torch.float32, device=dev)
+            kb_rows = kb_dev[j * H_kv:(j + 1) * H_kv]
+            order_rows = order[j * H_kv:(j + 1) * H_kv]
+            _lib.check(lib.rdkv_pack_layer_stream(
+                K.data_ptr(), V.data_ptr(), K.stride(1), K.stride(2), H_kv, order_rows.data_ptr(), order_rows.stride(0),
+                plan.data_ptr() + 16 * j * H_kv, kb_rows.data_ptr(), kb_rows.element_size(), kb_rows.stride(0),
+                n2p, n4p, m8, max_tv, max_n16, units_dev.data_ptr() + row * UNIT_DTYPE.itemsize,
+                src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, blob.data_ptr(),
+                mm.data_ptr(), sm.data_ptr(), stream))
+            row += H_kv
+            base = blob.data_ptr()
+            for name in ("k_off", "sz_off", "qtab_off"):
+                units[name] += base
+            units["v_off"] += base
+            pending.append((i, units, blob, sm, sb, ab, (mm, kb_rows, order_rows, plan)))
+        if live:
+            pending.append((None, None, None, None, 0, 0, (units_dev, src_dev)))
+    if pending:
+        sms = [pn[3] for pn in pending if pn[0] is not None]
+        sm_all = torch.stack(sms).transpose(1, 2).cpu().numpy().astype(np.float32) if sms else None   # (synchronizes)
+        torch.cuda.current_stream(dev).synchronize()
+        k = 0
+        for i, units, blob, _, sb, ab, _ in pending:
+            if i is None:
+                continue
+            out[i] = (units, blob, sb, ab, sm_all[k].reshape(-1, 2))
+            k += 1
+    units_all = np.concatenate([np.asarray(o[0], dtype=UNIT_DTYPE) for o in out])
+    blobs = [o[1] for o in out]
+    if entry_bytes is not None:
+        entry_bytes.extend((int(o[2]), int(o[3])) for o in out)
+    return (units_all, blobs, int(sum(o[2] for o in out)), int(sum(o[3] for o in out)), H_q,
+            np.concatenate([o[4] for o in out]).astype(np.float32))
+
+
+def build_stream_cache_from_kv(entries: Sequence[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]],
+                               G: int, *, work_bytes: Optional[int] = None, n_groups: Optional[int] = None,
+                               groups_per_cu: int = 1, cost: Optional[dict] = None,
+                               row_of_entry: Optional[Sequence[int]] = None) -> StreamCache:
+    """``build_stream_cache`` over the layers ``packing.pack_layer_per_head(K, V, v_bits, k_bits, G)``
+    would give for the ``entries`` (K, V, v_bits, k_bits), without building them: the prefill packer
+    writes the streaming format directly (``rdkv_pack_layer_stream``), the same bits as packing and
+    re-laying."""
+    rows_of_entries = list(range(len(entries))) if row_of_entry is None else [int(r) for r in row_of_entry]
+    assert len(rows_of_entries) == len(entries) and len(entries) > 0
+    units_np, blobs, stream_bytes, kv_algo, H_q, scale_max = _pack_entries_direct(entries, G, rows_of_entries)
+    return _finish_cache(units_np, blobs, G, H_q, stream_bytes, kv_algo, scale_max, multi_source=row_of_entry is not None,
+                         work_bytes=work_bytes, n_groups=n_groups, groups_per_cu=groups_per_cu, cost=cost)
+
+
+def extend_stream_caches_from_kv(caches: Sequence[StreamCache],
+                                 entries: Sequence[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]]
+                                 ) -> List[StreamCache]:
+    """``extend_stream_caches`` from fp16 K / V and allocations: entry i (K, V, v_bits, k_bits) becomes
+    a further source of output group 0 of ``caches[i]``, quantized and laid out directly."""
+    assert len(caches) == len(entries) and len(caches) > 0
+    G = caches[0].G
+    assert all(c.G == G for c in caches)
+    per_entry: list = []
+    new_units, new_blobs, _, _, H_q, new_scale_max = _pack_entries_direct(entries, G, [0] * len(entries), per_entry)
+    return _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max)
 
 
 def v_shift_of(v_scale_max: np.ndarray) -> np.ndarray:
@@ -475,7 +628,13 @@ def extend_stream_caches(caches: Sequence[StreamCache],
     assert all(c.G == G for c in caches)
     per_entry: list = []
     new_units, new_blobs, _, _, H_q, new_scale_max = _relayout_entries(layers, G, [0] * len(layers), per_entry)
-    n_per = len(new_units) // len(layers)
+    return _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max)
+
+
+def _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max) -> List[StreamCache]:
+    """caches[i] with entry i of a freshly laid run of entries (equal unit counts) as a further source."""
+    G = caches[0].G
+    n_per = len(new_units) // len(caches)
     out = []
     for i, cache in enumerate(caches):
         assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"

@@ -31,15 +31,9 @@ def _padded_k_codes(pl, h):
     return np.concatenate(parts, axis=1)
 
 
-@pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b", "shared_layout"])
-def test_stream_format_round_trip(name):
-    """Every packed bit of the reference layout is recoverable from the streaming blobs."""
-    g = load_golden(name)
-    G = int(g["groups"])
-    ora = golden_to_oracle_layer(g, "pl")
-    nvo = g.get("new_v_only")
-    cache = stream_cache.build_stream_cache(
-        [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G)
+def _assert_cache_holds_layer(cache, ora, nvo):
+    """Every packed bit of the reference-layout layer `ora` (an oracle PackedKVLayer, with its fp16
+    zone `nvo`) is found in the one-entry streaming cache, decoded by the test-side NumPy decoder."""
     blob = t2n(cache.blobs[0])
     base = cache.blobs[0].data_ptr()
     H_kv = ora.K_ch_scale.shape[1]
@@ -86,6 +80,108 @@ def test_stream_format_round_trip(name):
                 assert qt[s]["zp"] == ora.K_ch_zp[0, h, 0, r].view(np.uint16)
             else:
                 assert qt[s]["scale"] == 0
+
+
+@pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b", "shared_layout"])
+def test_stream_format_round_trip(name):
+    """Every packed bit of the reference layout is recoverable from the streaming blobs."""
+    g = load_golden(name)
+    G = int(g["groups"])
+    ora = golden_to_oracle_layer(g, "pl")
+    nvo = g.get("new_v_only")
+    cache = stream_cache.build_stream_cache(
+        [(layer_to_device(ora), to_dev(nvo) if nvo is not None else None)], G)
+    _assert_cache_holds_layer(cache, ora, nvo)
+
+
+def _assert_same_cache(a, b):
+    """Two one-blob-per-entry caches hold the same bytes at the same relative places."""
+    assert a.n_units == b.n_units and a.stream_bytes == b.stream_bytes and a.rows == b.rows
+    assert a.kv_algorithmic_bytes == b.kv_algorithmic_bytes and a.max_row_dwords == b.max_row_dwords
+    assert len(a.blobs) == len(b.blobs)
+    ua, ub = a.units_host.copy(), b.units_host.copy()
+    for units, cache in ((ua, a), (ub, b)):
+        bases = np.array([blob.data_ptr() for blob in cache.blobs], dtype=np.uint64)
+        sizes = np.array([blob.numel() for blob in cache.blobs], dtype=np.uint64)
+        which = np.array([int(np.nonzero((bases <= k) & (k < bases + sizes))[0][0]) for k in units["k_off"]])
+        for f in ("k_off", "sz_off", "qtab_off"):
+            units[f] -= bases[which]
+        units["v_off"] -= bases[which][:, None]
+    assert np.array_equal(ua.view(np.uint8), ub.view(np.uint8)), "unit descriptors differ"
+    assert np.array_equal(a.unit_scale_max, b.unit_scale_max), "largest scales differ"
+    for i, (x, y) in enumerate(zip(a.blobs, b.blobs)):
+        assert x.numel() == y.numel() and torch.equal(x, y), f"blob {i} differs"
+
+
+@pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b"])
+def test_direct_stream_packer_golden(name):
+    """fp16 K / V + allocations straight into the streaming format: every bit the reference wrote
+    for the layer (its own packed tensors, stored as golden data) is found in the blob."""
+    g = load_golden(name)
+    G = int(g["groups"])
+    ora = golden_to_oracle_layer(g, "pl")
+    cache = stream_cache.build_stream_cache_from_kv(
+        [(to_dev(g["keys"]), to_dev(g["values"]), torch.from_numpy(g["v_bits"]), torch.from_numpy(g["k_bits"]))], G)
+    _assert_cache_holds_layer(cache, ora, g.get("new_v_only"))
+    out, lse = stream_cache.decode_attn_fused(cache, to_dev(g["q"]))
+    attn_close(t2n(out), g["out"], "out")
+
+
+@pytest.mark.parametrize("cfg_idx,ctx,layers", [(0, 700, 1), (1, 2300, 2), (2, 1500, 1), (3, 900, 2), (1, 64, 1), (0, 130, 1), (1, 32768, 1), (2, 131072, 1)])
+def test_direct_stream_packer_matches_pack_then_relayout(cfg_idx, ctx, layers):
+    """The direct packer's cache against packing + re-layout of the same layers: the same unit
+    descriptors, largest scales and blob bytes; and the layer the oracle packs from the same CPU
+    data is found in the blob."""
+    cfg = synth.scaled(synth.CONFIGS[cfg_idx], context=ctx, layers=layers)
+    entries, packed, oracle_layers = [], [], []
+    for layer in range(layers):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, _ = synth.layer_data(cfg, layer, "cpu", outliers=oc)
+        if ctx <= 700 and layer == 0:
+            oracle_layers.append(O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), cfg.G))
+        K, V = K.to(DEV), V.to(DEV)
+        entries.append((K, V, vb, kb))
+        packed.append(packing.pack_layer_per_head(K, V, vb, kb, cfg.G))
+    direct = stream_cache.build_stream_cache_from_kv(entries, cfg.G)
+    two_step = stream_cache.build_stream_cache(packed, cfg.G)
+    _assert_same_cache(direct, two_step)
+    if ctx <= 700:      # (the NumPy decoder walks the blob field by field)
+        one = stream_cache.build_stream_cache_from_kv(entries[:1], cfg.G)
+        _assert_cache_holds_layer(one, *oracle_layers[0])
+
+
+def test_direct_stream_packer_ragged_and_degenerate_entries():
+    """Heads that keep nothing, a head that keeps only fp16 tokens, a layer where every head keeps
+    the same counts (no zero rows in the K canvas: 0 must not join a min / max), inputs the direct
+    kernel does not take (a strided view, fp32 values): always the bytes of packing + re-layout."""
+    rng = np.random.default_rng(77)
+    H, T, G = 3, 300, 2
+    choices = np.array([0, 2, 4, 8, 16])
+
+    def run(K, V, vb, kb):
+        direct = stream_cache.build_stream_cache_from_kv([(K, V, vb, kb)], G)
+        two_step = stream_cache.build_stream_cache([packing.pack_layer_per_head(K, V, vb, kb, G)], G)
+        _assert_same_cache(direct, two_step)
+
+    kb = torch.from_numpy(rng.choice(np.array([0, 0, 2, 4, 8, 16]), size=(H, 128)))
+    K = (torch.randn(1, H, T, 128, device=DEV).abs() + 1.0).half()     # strictly positive: a spurious 0 shows
+    V = torch.randn(1, H, T, 128, device=DEV).half()
+    vb = torch.from_numpy(rng.choice(choices, size=(H, T)))
+    vb[1] = 0                                                          # a head that keeps nothing
+    run(K, V, vb, kb)
+    vb = torch.from_numpy(rng.choice(choices, size=(H, T)))
+    vb[0] = torch.from_numpy(rng.choice(np.array([0, 16]), size=T))    # only fp16-kept tokens
+    run(K, V, vb, kb)
+    row = rng.choice(choices, size=T)
+    vb = torch.from_numpy(np.stack([rng.permutation(row) for _ in range(H)]))   # equal counts in every head
+    run(K, V, vb, kb)
+    vb = torch.full((H, T), 4)                                         # one class only
+    run(K, V, vb, kb)
+    big = torch.randn(1, H, T, 256 + 4, device=DEV).half()             # rows 8-byte aligned only
+    run(big[..., 2:130], big[..., 130:258], torch.from_numpy(rng.choice(choices, size=(H, T))), kb)
+    kb0 = kb.clone()
+    kb0[2] = 0                                                         # a head without kept channels
+    run(K, V, torch.from_numpy(rng.choice(choices, size=(H, T))), kb0)
 
 
 @pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b", "shared_layout"])
