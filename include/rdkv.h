@@ -298,6 +298,25 @@ typedef struct RdkvWork {   /* a run of tiles of one unit handled by one workgro
                                below 512                                                            */
 } RdkvWork;
 
+/* Host side of the streaming format for one layer (no GPU work; every pointer is host memory): the
+ * H_kv unit descriptors, slot tables and sizes that rdkv_stream_relayout_layer and
+ * rdkv_pack_layer_stream take.  tok_counts[h * tok_stride + c]: tokens of head h with 2-bit, 4-bit,
+ * 8-bit and fp16-kept V rows (c = 0..3; the packed layer's seg_bounds_per_head and n_v16 of
+ * packing.py:801-1013).  ch_counts[h * ch_stride + c]: kept K channels of head h of 2, 4 and 8 bit
+ * (K_ch_seg_bounds_per_head, packing.py:364-388).  n2p / n4p: the layer's padded 2- / 4-bit
+ * channel counts.  Head h answers query rows first_q_row + h * G .. + G - 1.
+ * units[H_kv]: offsets relative to the layer's blob, work_begin / work_count zero.
+ * src_slot: int16 [H_kv][n_slots_max], n_slots_max = 160: stream slot -> position in the source
+ * layer's padded sorted channel order, -1 = pad slot.  8-bit channels come first, then 4-bit, then
+ * 2-bit, each padded to whole dwords; stragglers of a narrow class move into pad slots of a wider
+ * class when that shortens the K row by a dword, and a row that would exceed 32 dwords is stored
+ * entirely as 8 bit (values are unchanged: a narrow code is the same number in a wider field).
+ * sizes[4]: bytes of the blob, largest tile count of a head, bytes the fused kernel streams from the
+ * blob, bytes the reference's layout holds for the same content. */
+int rdkv_stream_plan_layer(const int32_t *tok_counts, int64_t tok_stride, const int32_t *ch_counts,
+                           int64_t ch_stride, int H_kv, int n2p, int n4p, int first_q_row, int G,
+                           RdkvUnit *units, int16_t *src_slot, int n_slots_max, int64_t *sizes);
+
 /* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.
  * src_slot: int16 [H_kv][n_slots_max] = for each stream slot the index of the source channel
  * in the padded sorted order of K_ch_scale (-1 = pad slot).  units: the layer's H_kv
@@ -324,24 +343,28 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
 /* The prefill packer that writes the streaming format directly: fp16 K and V [H_kv, T, 128] ->
  * the blob a rdkv_pack_layer_per_head call followed by rdkv_stream_relayout_layer would produce,
  * bit for bit (the composition of obkv_fast.py:1141-1155, packing.py:801-1013 and
- * packing.py:1019-1317, then the re-layout), without the padded intermediate: two launches (the
- * per-channel K min / max, then one workgroup per 64-token tile and head).  order / counts: as
+ * packing.py:1019-1317, then the re-layout), without the padded intermediate: the per-channel K min / max,
+ * a small launch that makes every stream slot's quantizer and the slot tables, then one workgroup
+ * per 64-token tile and head.  order / counts: as
  * rdkv_pack_layer_plan leaves them (token order by width class, [H_kv, 4] class sizes; device).
  * k_bits [H_kv, 128]: integers of kb_elem_size bytes, 16 counted as 8, 0 = pruned (device).
  * n2p / n4p / n8: the layer's padded channel counts (maxima over heads; what src_slot refers to);
  * max_tv / max_n16: maxima over heads of the quantized / fp16-kept token counts (a head below
  * either has zero rows in the reference's K canvas, packing.py:1186-1215, so 0 joins its
  * per-channel min / max).  units (device, offsets relative to blob), src_slot, n_slots_max,
- * max_tiles: as for rdkv_stream_relayout_layer.  minmax_ws: H_kv * 256 floats of scratch.
- * scale_max: float [2][H_kv], zero before the call: receives per head the largest K channel scale
- * and the largest V token scale (as the fp16 values stored), which RdkvWork.k_scale_max / v_shift
- * are made from.  K and V rows must be 16-byte aligned (RDKV_EUNSUPPORTED otherwise). */
+ * max_tiles: as for rdkv_stream_relayout_layer.  blob_bytes: size of the blob (a multiple of 4, at
+ * least sizes[0] of rdkv_stream_plan_layer): the launches write every byte of it, so it need not be
+ * cleared.  minmax_ws: H_kv * 768 floats of scratch, 16-byte aligned (min / max accumulators, then
+ * the quantizer of every channel).
+ * scale_max: float [2][H_kv]: receives per head the largest K channel scale and the largest V token
+ * scale (as the fp16 values stored), which RdkvWork.k_scale_max / v_shift are made from.  K and V
+ * rows must be 16-byte aligned (RDKV_EUNSUPPORTED otherwise). */
 int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
                            int H_kv, const int32_t *order, int64_t order_stride_h, const int32_t *counts,
                            const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int n2p, int n4p, int n8,
                            int64_t max_tv, int max_n16, const RdkvUnit *units, const int16_t *src_slot,
-                           int n_slots_max, int max_tiles, uint8_t *blob, float *minmax_ws, float *scale_max,
-                           void *stream);
+                           int n_slots_max, int max_tiles, uint8_t *blob, int64_t blob_bytes, float *minmax_ws,
+                           float *scale_max, void *stream);
 
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit

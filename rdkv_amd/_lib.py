@@ -60,7 +60,8 @@ SIGNATURES = {
     "rdkv_softmax_rows_ws": (I, [P, L, P, L, L, P, L, L, P, L, P, L, I, P, L, P]),
     "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
     "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
-    "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, P, P, P]),
+    "rdkv_stream_plan_layer": (I, [P, L, P, L, I, I, I, I, I, P, P, I, P]),
+    "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, L, P, P, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,
                                        P, L, P, P, L, P, P, I, I, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),
@@ -207,3 +208,59 @@ def workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
         buf = torch.empty(max(int(nbytes), grown, 1 << 20), dtype=torch.uint8, device=dev)
         _workspaces[key] = buf
     return buf
+
+
+# ---- small host <-> device transfers that do not stall the host ---------------------------------
+# A copy from pageable host memory waits until it has been carried out, behind everything already
+# queued on the stream; from pinned memory it is queued and the host goes on.  The staging buffers
+# are kept; one that still has a copy in flight is left alone and another is taken.
+_stagers: dict = {}
+
+
+def upload(dev: torch.device, *arrays) -> list:
+    """The NumPy arrays as byte tensors on ``dev`` (views of one device buffer, each 256-byte
+    aligned), sent as one queued copy on the current stream."""
+    import threading
+
+    import numpy as np
+    offs, total = [], 0
+    for a in arrays:
+        offs.append(total)
+        total += -(-max(int(a.nbytes), 1) // 256) * 256
+    key = (dev.index, threading.get_ident())
+    pool = _stagers.setdefault(key, [])
+    slot = None
+    for s in pool:
+        if s[0].numel() >= total and (s[1] is None or s[1].query()):
+            slot = s
+            break
+    if slot is None:
+        slot = [torch.empty(max(1 << 16, 1 << (total - 1).bit_length()), dtype=torch.uint8, pin_memory=True), None]
+        pool.append(slot)
+    host = slot[0].numpy()
+    for a, o in zip(arrays, offs):
+        if a.nbytes:
+            host[o:o + a.nbytes] = np.ascontiguousarray(a).reshape(-1).view(np.uint8)
+    d = torch.empty(total, dtype=torch.uint8, device=dev)
+    d.copy_(slot[0][:total], non_blocking=True)
+    ev = torch.cuda.Event()
+    ev.record(torch.cuda.current_stream(dev))
+    slot[1] = ev
+    return [d[o:o + max(int(a.nbytes), 0)] for a, o in zip(arrays, offs)]
+
+
+_pinned_reads: dict = {}
+
+
+def download(t: torch.Tensor):
+    """A small device tensor as a NumPy array, through a kept pinned buffer; waits for the stream."""
+    import threading
+    n = t.numel() * t.element_size()
+    key = (t.device.index, threading.get_ident(), max(4096, 1 << (max(n, 1) - 1).bit_length()))
+    buf = _pinned_reads.get(key)
+    if buf is None:
+        buf = _pinned_reads[key] = torch.empty(key[2], dtype=torch.uint8, pin_memory=True)
+    flat = t.contiguous().reshape(-1).view(torch.uint8)
+    buf[:n].copy_(flat, non_blocking=True)
+    torch.cuda.current_stream(t.device).synchronize()
+    return buf[:n].numpy().view(torch.empty(0, dtype=t.dtype).numpy().dtype).reshape(tuple(t.shape)).copy()

@@ -7,12 +7,15 @@
 // re-quantizes K from (packing.py:1186-1215: a head with fewer rows than the layer's maxima has
 // zero rows there, so 0 joins its per-channel min / max).
 //
-// One workgroup per (64-token tile, KV head): the tile's K and V rows (gathered through the head's
-// class-sorted token order) are staged in LDS with 16-byte loads, every request out before the
-// first is used; per-token V parameters and per-slot K parameters meet there too; every thread then
-// assembles output dwords field by field and the workgroup writes the tile's K part, V part and
-// {scale, zp} pairs coalesced.  A last workgroup per head writes the slot table.
+// Three launches: the per-channel K min / max of every head (quantize.hip), one small workgroup per
+// head that turns them into the quantizer of every channel and writes the unit's slot table, and one
+// workgroup per (64-token tile, KV head) that reads the tile's K and V rows (gathered through the
+// head's class-sorted token order) with 16-byte loads, every request out before the first is used,
+// quantizes them in registers, parks the codes in LDS as bytes and assembles the tile's dwords from
+// there.  Between them the launches write every byte of the blob.
 #include "rdkv_common.h"
+#include <string.h>
+
 #include "stream_format.h"
 
 #pragma clang fp contract(off)   // the quantizer rounds every product and sum on its own
@@ -49,253 +52,427 @@ struct StreamPackArgs {
   uint8_t *blob;
   uint32_t *scale_max;            // [2][H_kv] float bits: largest K channel scale, largest V token scale
   int H_kv;
+  int64_t blob_bytes;
 };
 
-// Per-slot quantizer of the K side, in LDS.
-struct SlotParams {
-  float scale[kMaxSlots], zp[kMaxSlots], inv[kMaxSlots], qmax[kMaxSlots];
-  int channel[kMaxSlots];         // source channel, -1 for a pad slot
-};
+// The K quantizer of one channel: scale, zero point, 1 / scale (rdkv_qcode's estimate) and, as bits,
+// the channel's stream slot with its width class (slot | class << 8; -1 for a channel that is not
+// kept).  One launch per layer makes them for every head (slot_params_kernel), the tile workgroups
+// read them.
+__device__ __forceinline__ float4 make_chan(float scale, float zp, float inv, int slot_cls) {
+  return make_float4(scale, zp, inv, __int_as_float(slot_cls));
+}
 
-// The K parameters of every stream slot of head h: slot -> position in the reference's padded
-// sorted channel order (src_slot) -> width class and rank in the class -> the rank-th channel of
-// that width in ascending channel order (the stable sort of packing.py:241-294).
-__device__ __forceinline__ void slot_params(const StreamPackArgs &a, int h, const RdkvUnit &u, int n_slots,
-                                            SlotParams &sp, int *ch_of /* [3][128] */, int *cls_count /* [3] */) {
-  const int tid = threadIdx.x, lane = tid & 63;
+// One workgroup per head: stream slot -> position in the reference's padded sorted channel order
+// (src_slot) -> width class and rank in the class -> the rank-th channel of that width in ascending
+// channel order (the stable sort of packing.py:241-294) -> the channel's parameters from its
+// min / max.  Writes the per-channel parameters, the unit's slot table in the blob (with the
+// alignment gap behind it, and behind the last head the rest of the blob: no byte of the blob is
+// left to the caller), and starts the head's two scale maxima.
+__global__ void __launch_bounds__(128)
+slot_params_kernel(StreamPackArgs a, float4 *__restrict__ chan_params) {
+  __shared__ int ch_of[3 * kD], first_wave_count[3], slot_of_ch[kD];
+  __shared__ float4 slot_p[kMaxSlots];
+  __shared__ float wave_max[2];
+  const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63;
+  const RdkvUnit u = a.units[h];
+  const int n_slots = 4 * (u.d8 + 2 * u.d4 + 4 * u.d2);
   // rank of channel c inside its width class = channels below it of the same class: a ballot per
   // class in each of the two wavefronts that hold the 128 channels, plus the first wavefront's count
-  int cls = -1, rank = 0;
-  if (tid < kD) {
-    int b = load_bits(a.k_bits, a.kb_elem_size, (int64_t)h * a.kb_stride_h + tid);
-    b = b > 8 ? 8 : b;                                           // 16 is stored as 8 bit
-    cls = b == 2 ? 0 : (b == 4 ? 1 : (b == 8 ? 2 : -1));
+  int b = load_bits(a.k_bits, a.kb_elem_size, (int64_t)h * a.kb_stride_h + tid);
+  b = b > 8 ? 8 : b;                                             // 16 is stored as 8 bit
+  const int cls = b == 2 ? 0 : (b == 4 ? 1 : (b == 8 ? 2 : -1));
+  int rank = 0;
 #pragma unroll
-    for (int x = 0; x < 3; ++x) {
-      const unsigned long long m = __ballot(cls == x);
-      if (cls == x) rank = __popcll(m & ((1ull << lane) - 1ull));
-      if (tid == 0) cls_count[x] = __popcll(m);                  // the class's channels among 0 .. 63
-    }
+  for (int x = 0; x < 3; ++x) {
+    const unsigned long long m = __ballot(cls == x);
+    if (cls == x) rank = __popcll(m & ((1ull << lane) - 1ull));
+    if (tid == 0) first_wave_count[x] = __popcll(m);
   }
+  slot_of_ch[tid] = -1;
   __syncthreads();
-  if (tid < kD && cls >= 0) ch_of[cls * kD + rank + (tid >= 64 ? cls_count[cls] : 0)] = tid;
+  if (cls >= 0) ch_of[cls * kD + rank + (tid >= 64 ? first_wave_count[cls] : 0)] = tid;
   __syncthreads();
   const int tv = u.n_tok[0] + u.n_tok[1] + u.n_tok[2];
   const bool has_pad = tv < a.max_tv || u.n_tok[3] < a.max_n16;   // zero rows of the canvas join the min / max
   const int16_t *slots = a.src_slot + (int64_t)h * a.n_slots_max;
-  for (int i = tid; i < n_slots; i += blockDim.x) {
+  float smax = 0.0f;
+  for (int i = tid; i < n_slots; i += 128) {
     const int r = slots[i];
-    float scale = 0.f, zp = 0.f, inv = 0.f, qmax = 0.f;
-    int ch = -1;
+    uint32_t w0 = 0, w1 = 0;
     if (r >= 0) {
-      int cls, rank;
-      if (r < a.n2p) { cls = 0; rank = r; }
-      else if (r < a.n2p + a.n4p) { cls = 1; rank = r - a.n2p; }
-      else { cls = 2; rank = r - a.n2p - a.n4p; }
-      ch = ch_of[cls * kD + rank];
-      qmax = cls == 0 ? 3.0f : (cls == 1 ? 15.0f : 255.0f);
+      int c, rk;
+      if (r < a.n2p) { c = 0; rk = r; }
+      else if (r < a.n2p + a.n4p) { c = 1; rk = r - a.n2p; }
+      else { c = 2; rk = r - a.n2p - a.n4p; }
+      const int ch = ch_of[c * kD + rk];
+      const float qmax = c == 0 ? 3.0f : (c == 1 ? 15.0f : 255.0f);
       float mn = rdkv_ordered_to_float(a.mm[(int64_t)h * 2 * kD + ch]);
       float mx = rdkv_ordered_to_float(a.mm[(int64_t)h * 2 * kD + kD + ch]);
       if (has_pad) {
         mn = fminf(mn, 0.0f);
         mx = fmaxf(mx, 0.0f);
       }
-      const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
-      scale = p.scale; zp = p.zp; inv = p.inv;
+      const RdkvQParams q = rdkv_qparams(mn, mx, qmax);
+      slot_p[i] = make_chan(q.scale, q.zp, q.inv, i | (c << 8));
+      slot_of_ch[ch] = i;
+      const uint16_t sc = rdkv_f2h(q.scale);
+      w0 = (uint32_t)ch | ((uint32_t)sc << 16);
+      w1 = (uint32_t)rdkv_f2h(q.zp);
+      smax = fmaxf(smax, rdkv_h2f(sc));
     }
-    sp.scale[i] = scale; sp.zp[i] = zp; sp.inv[i] = inv; sp.qmax[i] = qmax; sp.channel[i] = ch;
+    uint32_t *qt = reinterpret_cast<uint32_t *>(a.blob + u.qtab_off + 8 * (int64_t)i);   // {channel, scale, zp, 0}
+    qt[0] = w0;
+    qt[1] = w1;
   }
+  // the bytes behind the slot table: up to the next 256-byte boundary, or to the end of the blob
+  {
+    const int64_t from = (int64_t)u.qtab_off + 8 * (int64_t)n_slots;
+    const int64_t to = h == a.H_kv - 1 ? a.blob_bytes : (from + 255) / 256 * 256;
+    uint32_t *z = reinterpret_cast<uint32_t *>(a.blob + from);
+    for (int64_t i = tid; i < (to - from) / 4; i += 128) z[i] = 0u;
+  }
+  for (int o = 1; o < 64; o <<= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
+  if (lane == 0) wave_max[tid >> 6] = smax;
   __syncthreads();
+  const int s = slot_of_ch[tid];
+  chan_params[(int64_t)h * kD + tid] = s >= 0 ? slot_p[s] : make_chan(0.f, 0.f, 0.f, -1);
+  if (tid == 0) {
+    // largest K scale (as the fp16 value the decode kernel reads); the tile workgroups raise the V one
+    a.scale_max[h] = __float_as_uint(fmaxf(wave_max[0], wave_max[1]));
+    a.scale_max[a.H_kv + h] = 0u;
+  }
 }
 
-__device__ __forceinline__ uint32_t k_code(const SlotParams &sp, int slot, const __half *row) {
-  const int ch = sp.channel[slot];
-  if (ch < 0) return 0u;
-  RdkvQParams p;
-  p.scale = sp.scale[slot]; p.zp = sp.zp[slot]; p.inv = sp.inv[slot];
-  return rdkv_qcode(__half2float(row[ch]), p, sp.qmax[slot]);
+// min and max over the sixteen lanes of a row (lane ^ 1, lane ^ 2, mirror of eight, mirror of sixteen)
+__device__ __forceinline__ float row16_min(float v) {
+  v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false)));
+  v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false)));
+  v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false)));
+  v = fminf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false)));
+  return v;
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, false)));
+  v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, false)));
+  return v;
 }
 
-// one K dword of NF fields: field f is element k of operand s (stream_format.h), whose slot is
-// 4 * (step0 + s) + k
+__device__ __forceinline__ float half_at(const uint4 &v, int e) {      // element e of eight fp16 values
+  const uint32_t w = e < 2 ? v.x : (e < 4 ? v.y : (e < 6 ? v.z : v.w));
+  return __half2float(__ushort_as_half((uint16_t)((e & 1) ? (w >> 16) : (w & 0xffffu))));
+}
+
+// The code estimate of x (rdkv_qcode's x * (1 / scale) + zp, clamped, rounded to the nearest even
+// integer by the byte conversion) placed in byte B of `old`, and whether the estimate lies so close
+// to a rounding boundary that the exact quotient has to decide.  For estimates inside the clamp's
+// range the distance to the boundary is |fract(t) - 1/2|, the same number rdkv_qcode tests; outside
+// it the test can only raise the flag needlessly.  Callers collect the flags of several codes and
+// branch once (a branch per code cost more than the arithmetic).
+template <int B>
+__device__ __forceinline__ uint32_t code_byte(float x, const RdkvQParams &q, float qmax, uint32_t old, bool &near) {
+  const float t = fmaf(x, q.inv, q.zp);
+  near |= fabsf(__builtin_amdgcn_fractf(t) - 0.5f) < 2e-4f;
+  return __builtin_amdgcn_cvt_pk_u8_f32(fminf(fmaxf(t, 0.0f), qmax), B, old);
+}
+__device__ __forceinline__ bool code_is_near(float x, const RdkvQParams &q) {
+  return fabsf(__builtin_amdgcn_fractf(fmaf(x, q.inv, q.zp)) - 0.5f) < 2e-4f;
+}
+
+// lane N of every row of sixteen lanes to all lanes of the row
+template <int N>
+__device__ __forceinline__ float row16_bcast(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x150 + N, 0xF, 0xF, false));
+}
+
+// The V tile of class CLS from the tile's code bytes (fp16 bits for the fp16-kept class): thread
+// (l, g) assembles the dwords that hold channels l and l + 64 of quads 4g .. 4g + 3
+// (stream_format.h: element k of an operand is token 4 * quad + k; 8-bit dword 2 * quad + j, 4-bit
+// dword quad with operand j, 2-bit dword quad >> 1 with operand 2 * (quad & 1) + j; j = channel half).
+template <int CLS>
+__device__ __forceinline__ void v_tile(const uint8_t (*cv)[kD], const uint16_t (*raw)[kD], int nv,
+                                       uint32_t *v_out) {
+  const int l = threadIdx.x & 63, g = threadIdx.x >> 6;
+  // dword di of lane l sits at v_out[((di >> 2) * 64 + l) * 4 + (di & 3)]: a lane's dwords 4n .. 4n + 3 are 16 contiguous bytes
+  uint4 *out4 = reinterpret_cast<uint4 *>(v_out);
+  if (CLS == 3) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int quad = 4 * g + q;
+      uint32_t w[4] = {0u, 0u, 0u, 0u};             // dwords 4 * quad + 2 * j + {0, 1}
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int t = 4 * quad + k;
+          const uint32_t bits = t < nv ? (uint32_t)raw[t][l + 64 * j] : 0u;
+          w[2 * j + (k >> 1)] |= bits << (16 * (k & 1));
+        }
+      out4[quad * 64 + l] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+    return;
+  }
+  constexpr int NF = CLS == 2 ? 4 : (CLS == 1 ? 8 : 16);
+  constexpr int FW = 32 / NF;
+  uint32_t w8[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};   // class 2: dwords 8g .. 8g + 7; class 1: 4g .. 4g + 3; class 0: 2g, 2g + 1
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int quad = 4 * g + q;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = 4 * quad + k;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint32_t c = t < nv ? (uint32_t)cv[t][l + 64 * j] : 0u;
+        if (CLS == 2) w8[2 * q + j] |= c << (FW * rdkv_field_of(0, k, NF));
+        else if (CLS == 1) w8[q] |= c << (FW * rdkv_field_of(j, k, NF));
+        else w8[q >> 1] |= c << (FW * rdkv_field_of(2 * (q & 1) + j, k, NF));
+      }
+    }
+  }
+  if (CLS == 2) {
+    out4[(2 * g) * 64 + l] = make_uint4(w8[0], w8[1], w8[2], w8[3]);
+    out4[(2 * g + 1) * 64 + l] = make_uint4(w8[4], w8[5], w8[6], w8[7]);
+  } else if (CLS == 1) {
+    out4[g * 64 + l] = make_uint4(w8[0], w8[1], w8[2], w8[3]);
+  } else {
+    *reinterpret_cast<uint2 *>(v_out + ((g >> 1) * 64 + l) * 4 + 2 * (g & 1)) = make_uint2(w8[0], w8[1]);
+  }
+}
+
+// one K dword of NF fields from the tile's code bytes: field f is element k of operand s
+// (stream_format.h), whose slot is 4 * (step0 + s) + k
 template <int NF>
-__device__ __forceinline__ uint32_t k_dword(const SlotParams &sp, int step0, const __half *row) {
+__device__ __forceinline__ uint32_t k_dword(const uint8_t *codes_t, int step0) {
   uint32_t w = 0;
 #pragma unroll
   for (int f = 0; f < NF; ++f) {
     int s, k;
     rdkv_operand_of(f, NF, &s, &k);
-    w |= k_code(sp, 4 * (step0 + s) + k, row) << ((32 / NF) * f);
+    w |= (uint32_t)codes_t[4 * (step0 + s) + k] << ((32 / NF) * f);
   }
   return w;
 }
 
-template <int CLS>
-__device__ __forceinline__ void v_tile(const __half (*lv)[kD], const float *vt_scale, const float *vt_zp,
-                                       const float *vt_inv, int nv, uint32_t *v_out) {
-  constexpr int per_tile = 512 << CLS;
-  constexpr float qmax = CLS == 0 ? 3.0f : (CLS == 1 ? 15.0f : 255.0f);
-  for (int rem = threadIdx.x; rem < per_tile; rem += 256) {
-    const int l = (rem >> 2) & 63;
-    const int di = ((rem >> 8) << 2) | (rem & 3);  // lane dword index
-    uint32_t w = 0;
-    if (CLS == 3) {
-      const int quad = di >> 2, j = (di >> 1) & 1, kk = (di & 1) * 2;
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int t = 4 * quad + kk + e;
-        if (t < nv) w |= (uint32_t)__half_as_ushort(lv[t][l + 64 * j]) << (16 * e);
-      }
-    } else {
-      constexpr int NF = CLS == 2 ? 4 : (CLS == 1 ? 8 : 16);
-#pragma unroll
-      for (int f = 0; f < NF; ++f) {
-        int s, k;
-        rdkv_operand_of(f, NF, &s, &k);
-        int quad, j;
-        if (CLS == 2) { quad = di >> 1; j = di & 1; }
-        else if (CLS == 1) { quad = di; j = s; }
-        else { quad = 2 * di + (s >> 1); j = s & 1; }
-        const int t = 4 * quad + k;
-        if (t < nv) {
-          RdkvQParams p;
-          p.scale = vt_scale[t]; p.zp = vt_zp[t]; p.inv = vt_inv[t];
-          w |= rdkv_qcode(__half2float(lv[t][l + 64 * j]), p, qmax) << ((32 / NF) * f);
-        }
-      }
-    }
-    v_out[rem] = w;
-  }
+// Where tile ti of a unit lies: its class, index inside the class, valid tokens and first row in the
+// head's sorted token order (quantized classes, then the fp16 zone).  Selects, no indexed arrays.
+struct TileInfo {
+  int cls, tl, nv;
+  int64_t row0;
+};
+__device__ __forceinline__ TileInfo tile_info(const RdkvUnit &u, int ti) {
+  const int t0 = (u.n_tok[0] + RDKV_TILE - 1) / RDKV_TILE, t1 = t0 + (u.n_tok[1] + RDKV_TILE - 1) / RDKV_TILE;
+  const int t2 = t1 + (u.n_tok[2] + RDKV_TILE - 1) / RDKV_TILE;
+  TileInfo r;
+  r.cls = ti < t0 ? 0 : (ti < t1 ? 1 : (ti < t2 ? 2 : 3));
+  r.tl = ti - (r.cls == 0 ? 0 : (r.cls == 1 ? t0 : (r.cls == 2 ? t1 : t2)));
+  const int n = r.cls == 0 ? u.n_tok[0] : (r.cls == 1 ? u.n_tok[1] : (r.cls == 2 ? u.n_tok[2] : u.n_tok[3]));
+  const int64_t c0 = r.cls == 0 ? 0
+                                : (r.cls == 1 ? (int64_t)u.n_tok[0]
+                                              : (r.cls == 2 ? (int64_t)u.n_tok[0] + u.n_tok[1]
+                                                            : (int64_t)u.n_tok[0] + u.n_tok[1] + u.n_tok[2]));
+  r.nv = min(RDKV_TILE, n - r.tl * RDKV_TILE);
+  r.row0 = c0 + (int64_t)r.tl * RDKV_TILE;
+  return r;
 }
 
-__global__ void __launch_bounds__(256)
-stream_pack_kernel(StreamPackArgs a) {
-  __shared__ SlotParams sp;
-  __shared__ int ch_of[3 * kD], cls_count[3];
-  __shared__ __align__(16) __half lk[RDKV_TILE][kD], lv[RDKV_TILE][kD];
-  __shared__ float vt_scale[RDKV_TILE], vt_zp[RDKV_TILE], vt_inv[RDKV_TILE];
-  const int h = blockIdx.y, tid = threadIdx.x;
+// Workgroup (x, head) takes the head's 64-token tiles x, x + gridDim.x, ...  Thread (p = tid % 16,
+// r = tid / 16) loads 16 bytes (eight channels, 8p .. 8p + 7) of the K and the V row of tokens r,
+// r + 16, r + 32, r + 48 and turns them into codes in registers: the K parameters of its eight
+// channels stay in registers for every tile, the V parameters of a token come from a min / max over
+// the sixteen lanes that hold it.  Codes are parked in LDS as bytes (K at its stream slot, V at its
+// channel), from where the dwords of the K rows and of the V tile are assembled and stored
+// coalesced.  The token indices of the workgroup's next tile are requested before the current tile
+// is worked on; several workgroups share a compute unit and cover each other's waits.
+__global__ void __launch_bounds__(256, 3)
+stream_pack_kernel(StreamPackArgs a, const float4 *__restrict__ chan_params) {
+  __shared__ __align__(16) uint8_t ck[RDKV_TILE][kMaxSlots];        // K code of (token, stream slot)
+  __shared__ __align__(16) uint8_t cv_bytes[RDKV_TILE * kD * 2];    // V code of (token, channel); fp16 bits for class 3
+  __shared__ float4 chan[kD];                                       // the head's channel quantizers
+  uint8_t (*cv)[kD] = reinterpret_cast<uint8_t (*)[kD]>(cv_bytes);
+  uint16_t (*raw)[kD] = reinterpret_cast<uint16_t (*)[kD]>(cv_bytes);
+  const int h = blockIdx.y, tid = threadIdx.x, stride = gridDim.x;
   const RdkvUnit u = a.units[h];
   const int R = u.d8 + u.d4 + u.d2;
-  const int n_slots = 4 * (u.d8 + 2 * u.d4 + 4 * u.d2);
+  const int n_tiles = (u.n_tok[0] + RDKV_TILE - 1) / RDKV_TILE + (u.n_tok[1] + RDKV_TILE - 1) / RDKV_TILE +
+                      (u.n_tok[2] + RDKV_TILE - 1) / RDKV_TILE + (u.n_tok[3] + RDKV_TILE - 1) / RDKV_TILE;
+  int ti = blockIdx.x;
+  if (ti >= n_tiles) return;
+  const int p = tid & 15, r = tid >> 4;
+  const int32_t *ord = a.order + (int64_t)h * a.order_stride_h;
+  const __half *Kh = a.K + (int64_t)h * a.stride_h, *Vh = a.V + (int64_t)h * a.stride_h;
 
-  int tstart[5];
-  tstart[0] = 0;
-  for (int c = 0; c < 4; ++c) tstart[c + 1] = tstart[c] + (u.n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
-  const int ti = blockIdx.x;
-  const bool table_block = ti == a.max_tiles;
-  if (!table_block && ti >= tstart[4]) return;
-
-  // ---- the tile's rows: requested first (token index, then the two rows), used after the slot set-up
-  int cls = 0, tl = 0, tk0 = 0, nv = 0;
-  int64_t row0 = 0;
-  uint4 kraw[4], vraw[4];
-  const int trow = tid >> 2, tq = tid & 3;                 // row of the tile, quarter of the row (64 bytes)
-  if (!table_block) {
-    while (cls < 3 && ti >= tstart[cls + 1]) ++cls;
-    tl = ti - tstart[cls];
-    tk0 = tl * RDKV_TILE;
-    nv = min(RDKV_TILE, u.n_tok[cls] - tk0);               // valid tokens of the tile (>= 1)
-    // position of the class in the head's sorted token order (quantized classes, then the fp16 zone)
-    const int64_t cstart[4] = {0, u.n_tok[0], (int64_t)u.n_tok[0] + u.n_tok[1],
-                               (int64_t)u.n_tok[0] + u.n_tok[1] + u.n_tok[2]};
-    row0 = cstart[cls] + tk0;
-    const int32_t tok = a.order[(int64_t)h * a.order_stride_h + row0 + (trow < nv ? trow : 0)];
-    const uint4 *kr = reinterpret_cast<const uint4 *>(a.K + (int64_t)h * a.stride_h + (int64_t)tok * a.stride_t) + 4 * tq;
-    const uint4 *vr = reinterpret_cast<const uint4 *>(a.V + (int64_t)h * a.stride_h + (int64_t)tok * a.stride_t) + 4 * tq;
+  // token indices of a tile (tokens past the tile's end repeat its first row; their codes are
+  // dropped at assembly) and the rows behind them
+  auto load_tok = [&](int tile, int32_t (&tok)[4]) {
+    const TileInfo t = tile_info(u, tile);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) kraw[i] = kr[i];
+    for (int i = 0; i < 4; ++i) tok[i] = ord[t.row0 + (r + 16 * i < t.nv ? r + 16 * i : 0)];
+  };
+  auto load_rows = [&](const int32_t (&tok)[4], uint4 (&kr)[4], uint4 (&vr)[4]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) vraw[i] = vr[i];
-  }
-
-  slot_params(a, h, u, n_slots, sp, ch_of, cls_count);
-
-  if (table_block) {   // ---- slot table {channel, scale, zp, 0} per stream slot; the largest K scale
-    float smax = 0.0f;
-    for (int i = tid; i < n_slots; i += 256) {
-      uint32_t w0 = 0, w1 = 0;
-      if (sp.channel[i] >= 0) {
-        const uint16_t sc = rdkv_f2h(sp.scale[i]);
-        w0 = (uint32_t)sp.channel[i] | ((uint32_t)sc << 16);
-        w1 = (uint32_t)rdkv_f2h(sp.zp[i]);
-        smax = fmaxf(smax, rdkv_h2f(sc));
-      }
-      uint32_t *q = reinterpret_cast<uint32_t *>(a.blob + u.qtab_off + 8 * (int64_t)i);
-      q[0] = w0;
-      q[1] = w1;
+    for (int i = 0; i < 4; ++i) {
+      kr[i] = *(reinterpret_cast<const uint4 *>(Kh + (int64_t)tok[i] * a.stride_t) + p);
+      vr[i] = *(reinterpret_cast<const uint4 *>(Vh + (int64_t)tok[i] * a.stride_t) + p);
     }
-    // (non-negative floats order like their bit patterns)
-    if (smax > 0.0f) atomicMax(&a.scale_max[h], __float_as_uint(smax));
-    return;
-  }
+  };
 
+  int32_t tok[4];
+  load_tok(ti, tok);
+  if (tid < kD) chan[tid] = chan_params[(int64_t)h * kD + tid];
+  // pad slots hold code 0: nothing writes them afterwards
+  {
+    uint4 *z = reinterpret_cast<uint4 *>(&ck[0][0]);
+    for (int i = tid; i < RDKV_TILE * kMaxSlots / 16; i += 256) z[i] = make_uint4(0u, 0u, 0u, 0u);
+  }
+  float v_scale_max = 0.0f;          // largest V scale among the tokens whose parameters this lane worked out
+
+  for (; ti < n_tiles; ti += stride) {
+    const TileInfo t = tile_info(u, ti);
+    const int cls = t.cls, nv = t.nv;
+    // the tile's rows, then the token indices of the workgroup's next tile
+    uint4 kraw[4], vraw[4];
+    load_rows(tok, kraw, vraw);
+    if (ti + stride < n_tiles) load_tok(ti + stride, tok);
+    __syncthreads();   // the previous tile's assembly has read the code bytes (first tile: pad zeros and channel table are written)
+
+    // ---- V: per-token parameters and codes (quantized classes), or the rows as they are
+    if (cls < 3) {
+      const float qmax = cls == 0 ? 3.0f : (cls == 1 ? 15.0f : 255.0f);
+      float mn[4], mx[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    reinterpret_cast<uint4 *>(&lk[trow][0])[4 * tq + i] = kraw[i];
-    reinterpret_cast<uint4 *>(&lv[trow][0])[4 * tq + i] = vraw[i];
-  }
-  __syncthreads();
-
-  // ---- per-token V parameters (quantized classes): four threads per row
-  if (cls < 3) {
-    const float qmax = cls == 0 ? 3.0f : (cls == 1 ? 15.0f : 255.0f);
-    float mn = INFINITY, mx = -INFINITY;
-#pragma unroll 8
-    for (int c = 0; c < 32; ++c) {
-      const float x = __half2float(lv[trow][32 * tq + c]);
-      mn = fminf(mn, x);
-      mx = fmaxf(mx, x);
-    }
-    mn = fminf(mn, __shfl_xor(mn, 1, 64)); mx = fmaxf(mx, __shfl_xor(mx, 1, 64));
-    mn = fminf(mn, __shfl_xor(mn, 2, 64)); mx = fmaxf(mx, __shfl_xor(mx, 2, 64));
-    if (tq == 0) {
-      uint32_t w = 0;
-      float sc_h = 0.0f;
-      if (trow < nv) {
-        const RdkvQParams p = rdkv_qparams(mn, mx, qmax);
-        vt_scale[trow] = p.scale; vt_zp[trow] = p.zp; vt_inv[trow] = p.inv;
-        const uint16_t sc = rdkv_f2h(p.scale);
-        w = (uint32_t)sc | ((uint32_t)rdkv_f2h(p.zp) << 16);
-        sc_h = rdkv_h2f(sc);
+      for (int i = 0; i < 4; ++i) {
+        float lo = half_at(vraw[i], 0), hi = lo;
+#pragma unroll
+        for (int e = 1; e < 8; ++e) {
+          lo = fminf(lo, half_at(vraw[i], e));
+          hi = fmaxf(hi, half_at(vraw[i], e));
+        }
+        mn[i] = row16_min(lo);
+        mx[i] = row16_max(hi);
       }
-      *reinterpret_cast<uint32_t *>(a.blob + u.sz_off + 4 * ((int64_t)ti * RDKV_TILE + trow)) = w;
-      // the head's largest V scale (as the fp16 value the kernel will read)
-      float m = sc_h;
-      for (int o = 4; o < 64; o <<= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-      if ((tid & 63) == 0 && m > 0.0f) atomicMax(&a.scale_max[a.H_kv + h], __float_as_uint(m));
+      // lane p works out the parameters of token r + 16 * (p % 4) (three divisions), the row shares them
+      const int mine = p & 3;
+      const RdkvQParams qm = rdkv_qparams(mine == 0 ? mn[0] : (mine == 1 ? mn[1] : (mine == 2 ? mn[2] : mn[3])),
+                                          mine == 0 ? mx[0] : (mine == 1 ? mx[1] : (mine == 2 ? mx[2] : mx[3])), qmax);
+      if (p < 4) {
+        const int tt = r + 16 * p;
+        const uint16_t sc = rdkv_f2h(qm.scale);
+        *reinterpret_cast<uint32_t *>(a.blob + u.sz_off + 4 * ((int64_t)ti * RDKV_TILE + tt)) =
+            tt < nv ? (uint32_t)sc | ((uint32_t)rdkv_f2h(qm.zp) << 16) : 0u;
+        if (tt < nv) v_scale_max = fmaxf(v_scale_max, rdkv_h2f(sc));
+      }
+      RdkvQParams qt[4];
+      qt[0].scale = row16_bcast<0>(qm.scale); qt[0].zp = row16_bcast<0>(qm.zp); qt[0].inv = row16_bcast<0>(qm.inv);
+      qt[1].scale = row16_bcast<1>(qm.scale); qt[1].zp = row16_bcast<1>(qm.zp); qt[1].inv = row16_bcast<1>(qm.inv);
+      qt[2].scale = row16_bcast<2>(qm.scale); qt[2].zp = row16_bcast<2>(qm.zp); qt[2].inv = row16_bcast<2>(qm.inv);
+      qt[3].scale = row16_bcast<3>(qm.scale); qt[3].zp = row16_bcast<3>(qm.zp); qt[3].inv = row16_bcast<3>(qm.inv);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const RdkvQParams q = qt[i];
+        bool near = false;
+        uint32_t w0 = 0, w1 = 0;
+        w0 = code_byte<0>(half_at(vraw[i], 0), q, qmax, w0, near);
+        w0 = code_byte<1>(half_at(vraw[i], 1), q, qmax, w0, near);
+        w0 = code_byte<2>(half_at(vraw[i], 2), q, qmax, w0, near);
+        w0 = code_byte<3>(half_at(vraw[i], 3), q, qmax, w0, near);
+        w1 = code_byte<0>(half_at(vraw[i], 4), q, qmax, w1, near);
+        w1 = code_byte<1>(half_at(vraw[i], 5), q, qmax, w1, near);
+        w1 = code_byte<2>(half_at(vraw[i], 6), q, qmax, w1, near);
+        w1 = code_byte<3>(half_at(vraw[i], 7), q, qmax, w1, near);
+        if (near) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float x = half_at(vraw[i], e);
+            if (code_is_near(x, q)) {
+              const uint32_t c = rdkv_qcode_exact(x, q, qmax);
+              uint32_t &w = e < 4 ? w0 : w1;
+              w = (w & ~(0xffu << (8 * (e & 3)))) | (c << (8 * (e & 3)));
+            }
+          }
+        }
+        *reinterpret_cast<uint2 *>(&cv[r + 16 * i][8 * p]) = make_uint2(w0, w1);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<uint4 *>(&raw[r + 16 * i][8 * p]) = vraw[i];
+    }
+
+    // ---- K codes to their stream slots
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float4 cp = chan[8 * p + e];
+      const int slot_cls = __float_as_int(cp.w);
+      if (slot_cls >= 0) {
+        const int slot = slot_cls & 0xff, c = slot_cls >> 8;
+        const float qmax = c == 0 ? 3.0f : (c == 1 ? 15.0f : 255.0f);
+        RdkvQParams q;
+        q.scale = cp.x; q.zp = cp.y; q.inv = cp.z;
+        bool near = false;
+        uint32_t c4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) c4[i] = code_byte<0>(half_at(kraw[i], e), q, qmax, 0u, near);
+        if (near) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float x = half_at(kraw[i], e);
+            if (code_is_near(x, q)) c4[i] = rdkv_qcode_exact(x, q, qmax);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ck[r + 16 * i][slot] = (uint8_t)c4[i];
+      }
     }
     __syncthreads();
+
+    // ---- K tile: 64 rows of R dwords, chunks of up to four dwords per token
+    uint32_t *k_out = reinterpret_cast<uint32_t *>(a.blob + u.k_off) + (int64_t)ti * RDKV_TILE * R;
+    const int full = 256 * (R / 4);                   // dwords of the four-dword chunks
+    for (int rem0 = tid; rem0 < RDKV_TILE * R; rem0 += 256) {
+      int tt, j;
+      if (rem0 < full) {
+        tt = (rem0 & 255) >> 2;
+        j = 4 * (rem0 >> 8) + (rem0 & 3);
+      } else {
+        const int wc = R & 3, rem = rem0 - full;
+        tt = wc == 1 ? rem : (wc == 2 ? rem >> 1 : rem / 3);
+        j = 4 * (R / 4) + rem - tt * wc;
+      }
+      uint32_t w = 0;
+      if (tt < nv) {
+        if (j < u.d8) w = k_dword<4>(ck[tt], j);
+        else if (j < u.d8 + u.d4) w = k_dword<8>(ck[tt], u.d8 + 2 * (j - u.d8));
+        else w = k_dword<16>(ck[tt], u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4));
+      }
+      k_out[rem0] = w;
+    }
+
+    // ---- V tile of the class
+    const uint64_t v_base = cls == 0 ? u.v_off[0] : (cls == 1 ? u.v_off[1] : (cls == 2 ? u.v_off[2] : u.v_off[3]));
+    uint32_t *v_out = reinterpret_cast<uint32_t *>(a.blob + v_base) + (int64_t)t.tl * (rdkv_v_tile_bytes(cls) / 4);
+    if (cls == 0) v_tile<0>(cv, raw, nv, v_out);
+    else if (cls == 1) v_tile<1>(cv, raw, nv, v_out);
+    else if (cls == 2) v_tile<2>(cv, raw, nv, v_out);
+    else v_tile<3>(cv, raw, nv, v_out);
+
   }
 
-  // ---- K tile: 64 rows of R dwords, chunks of up to four dwords per token
-  uint32_t *k_out = reinterpret_cast<uint32_t *>(a.blob + u.k_off) + (int64_t)ti * RDKV_TILE * R;
-  const int full = 256 * (R / 4);                   // dwords of the four-dword chunks
-  for (int rem0 = tid; rem0 < RDKV_TILE * R; rem0 += 256) {
-    int t, j;
-    if (rem0 < full) {
-      t = (rem0 & 255) >> 2;
-      j = 4 * (rem0 >> 8) + (rem0 & 3);
-    } else {
-      const int wc = R & 3, rem = rem0 - full;
-      t = rem / wc;
-      j = 4 * (R / 4) + rem - t * wc;
-    }
-    uint32_t w = 0;
-    if (t < nv) {
-      if (j < u.d8) w = k_dword<4>(sp, j, lk[t]);
-      else if (j < u.d8 + u.d4) w = k_dword<8>(sp, u.d8 + 2 * (j - u.d8), lk[t]);
-      else w = k_dword<16>(sp, u.d8 + 2 * u.d4 + 4 * (j - u.d8 - u.d4), lk[t]);
-    }
-    k_out[rem0] = w;
+  // the head's largest V scale (as the fp16 value the decode kernel will read): one atomic per
+  // workgroup at most, none once the stored maximum has reached it (thousands of same-address
+  // atomics would otherwise queue up behind each other)
+  for (int o = 1; o < 64; o <<= 1) v_scale_max = fmaxf(v_scale_max, __shfl_xor(v_scale_max, o, 64));
+  __syncthreads();                       // (the last tile's assembly has read cv_bytes)
+  float *wave_max = reinterpret_cast<float *>(cv_bytes);
+  if ((tid & 63) == 0) wave_max[tid >> 6] = v_scale_max;
+  __syncthreads();
+  if (tid == 0) {
+    const float m = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    uint32_t *dst = &a.scale_max[a.H_kv + h];
+    const uint32_t mine = __float_as_uint(m);
+    if (mine > __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) atomicMax(dst, mine);
   }
-
-  // ---- V tile of the class: lane l owns channels l and l + 64 (stream_format.h)
-  uint32_t *v_out = reinterpret_cast<uint32_t *>(a.blob + u.v_off[cls]) + (int64_t)tl * (rdkv_v_tile_bytes(cls) / 4);
-  if (cls == 0) v_tile<0>(lv, vt_scale, vt_zp, vt_inv, nv, v_out);
-  else if (cls == 1) v_tile<1>(lv, vt_scale, vt_zp, vt_inv, nv, v_out);
-  else if (cls == 2) v_tile<2>(lv, vt_scale, vt_zp, vt_inv, nv, v_out);
-  else v_tile<3>(lv, vt_scale, vt_zp, vt_inv, nv, v_out);
 }
 
 }  // namespace
@@ -305,10 +482,14 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
                                     const int32_t *counts, const void *k_bits, int kb_elem_size,
                                     int64_t kb_stride_h, int n2p, int n4p, int n8, int64_t max_tv, int max_n16,
                                     const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
-                                    int max_tiles, uint8_t *blob, float *minmax_ws, float *scale_max,
-                                    void *stream) {
+                                    int max_tiles, uint8_t *blob, int64_t blob_bytes, float *minmax_ws,
+                                    float *scale_max, void *stream) {
+  // (minmax_ws holds the min / max accumulators, H_kv * 256 floats, then the channel parameters,
+  // H_kv * 128 * 4 floats)
   const char *fn = "rdkv_pack_layer_stream";
-  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && max_tiles >= 0 && max_tv >= 0 && max_n16 >= 0, "%s: bad shape", fn);
+  RDKV_REQUIRE(H_kv >= 1 && H_kv <= 65535 && max_tiles >= 0 && max_tv >= 0 && max_n16 >= 0 && blob_bytes >= 0 &&
+                   blob_bytes % 4 == 0,
+               "%s: bad shape", fn);
   RDKV_REQUIRE(K_f16 && V_f16 && order && counts && k_bits && units && src_slot && blob && minmax_ws && scale_max,
                "%s: null pointer", fn);
   RDKV_REQUIRE(kb_elem_size == 1 || kb_elem_size == 2 || kb_elem_size == 4 || kb_elem_size == 8,
@@ -339,7 +520,135 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
   a.blob = blob;
   a.scale_max = reinterpret_cast<uint32_t *>(scale_max);
   a.H_kv = H_kv;
-  hipLaunchKernelGGL(stream_pack_kernel, dim3(max_tiles + 1, H_kv), dim3(256), 0, s, a);
+  a.blob_bytes = blob_bytes;
+  float4 *params = reinterpret_cast<float4 *>(minmax_ws + (int64_t)H_kv * 2 * kD);
+  hipLaunchKernelGGL(slot_params_kernel, dim3(H_kv), dim3(128), 0, s, a, params);
+  if (max_tiles > 0) {
+    // as many workgroups as the device holds at once, each with the same number of tiles of the longest head
+    static int resident_of_device[64];     // (0 = not asked yet; a race between first callers writes the same value)
+    int resident = 512, dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64) {
+      if (resident_of_device[dev] == 0) {
+        int cus = 0, per_cu = 0;
+        const bool ok = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
+                        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, stream_pack_kernel, 256, 0) == hipSuccess &&
+                        per_cu > 0;
+        resident_of_device[dev] = ok ? cus * per_cu : 512;
+      }
+      resident = resident_of_device[dev];
+    }
+    const int target = (resident + H_kv - 1) / H_kv;
+    const int per = (max_tiles + target - 1) / target;
+    const int gx = (max_tiles + per - 1) / per;
+    hipLaunchKernelGGL(stream_pack_kernel, dim3(gx, H_kv), dim3(256), 0, s, a, params);
+  }
   RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
+// Host side of the streaming format (no GPU work): the unit descriptors of one layer's heads.
+namespace {
+struct SlotList {
+  int16_t v[kMaxSlots + 3 * kD];
+  int n = 0;
+  void push(int x) { v[n++] = (int16_t)x; }
+};
+inline int pad_to(int n, int a) { return (a - n % a) % a; }
+inline int64_t align256(int64_t x) { return (x + 255) / 256 * 256; }
+}  // namespace
+
+RDKV_API int rdkv_stream_plan_layer(const int32_t *tok_counts, int64_t tok_stride, const int32_t *ch_counts,
+                                    int64_t ch_stride, int H_kv, int n2p, int n4p, int first_q_row, int G,
+                                    RdkvUnit *units, int16_t *src_slot, int n_slots_max, int64_t *sizes) {
+  const char *fn = "rdkv_stream_plan_layer";
+  RDKV_REQUIRE(tok_counts && ch_counts && units && src_slot && sizes, "%s: null pointer", fn);
+  RDKV_REQUIRE(H_kv >= 1 && G >= 1 && n2p >= 0 && n4p >= 0 && n2p % 4 == 0 && n4p % 2 == 0, "%s: bad shape", fn);
+  RDKV_REQUIRE(n_slots_max == kMaxSlots, "%s: n_slots_max must be %d", fn, kMaxSlots);
+  int64_t off = 0, stream_bytes = 0, algo_bytes = 0;
+  int max_tiles = 0;
+  for (int h = 0; h < H_kv; ++h) {
+    const int32_t *nt = tok_counts + h * tok_stride, *cc = ch_counts + h * ch_stride;
+    const int c2 = cc[0], c4 = cc[1], c8 = cc[2];
+    RDKV_REQUIRE(c2 >= 0 && c4 >= 0 && c8 >= 0 && c2 <= n2p && c4 <= n4p && c2 + c4 + c8 <= kD &&
+                     nt[0] >= 0 && nt[1] >= 0 && nt[2] >= 0 && nt[3] >= 0,
+                 "%s: bad counts of head %d", fn, h);
+    // Slot order: 8-bit channels, 4-bit, 2-bit, each padded to whole dwords (4 / 8 / 16 channels).
+    // A narrow code is the same number in a wider field, so the stragglers of a narrow class move
+    // into the pad slots of the wider ones when that saves a whole dword of the K row; a row still
+    // longer than RDKV_MAX_ROW_DWORDS is stored entirely as 8 bit.
+    SlotList l8, l4, l2;
+    for (int i = 0; i < c8; ++i) l8.push(n2p + n4p + i);
+    for (int i = 0; i < c4; ++i) l4.push(n2p + i);
+    for (int i = 0; i < c2; ++i) l2.push(i);
+    const int r4 = l4.n % 8;
+    if (r4 > 0 && r4 <= pad_to(l8.n, 4)) {
+      for (int i = l4.n - r4; i < l4.n; ++i) l8.push(l4.v[i]);
+      l4.n -= r4;
+    }
+    const int r2 = l2.n % 16, p8 = pad_to(l8.n, 4), p4 = pad_to(l4.n, 8);
+    if (r2 > 0 && r2 <= p8 + p4) {
+      const int first = l2.n - r2, to8 = r2 < p8 ? r2 : p8;
+      for (int i = 0; i < to8; ++i) l8.push(l2.v[first + i]);
+      for (int i = to8; i < r2; ++i) l4.push(l2.v[first + i]);
+      l2.n = first;
+    }
+    if ((l8.n + 3) / 4 + (l4.n + 7) / 8 + (l2.n + 15) / 16 > 32) {
+      for (int i = 0; i < l4.n; ++i) l8.push(l4.v[i]);
+      for (int i = 0; i < l2.n; ++i) l8.push(l2.v[i]);
+      l4.n = l2.n = 0;
+    }
+    const int d8 = (l8.n + 3) / 4, d4 = (l4.n + 7) / 8, d2 = (l2.n + 15) / 16;
+    const int steps = d8 + 2 * d4 + 4 * d2;
+    RDKV_REQUIRE(steps <= RDKV_MAX_STEPS, "%s: %d channel steps exceed %d", fn, steps, RDKV_MAX_STEPS);
+    int16_t *src = src_slot + (int64_t)h * n_slots_max;
+    int n = 0;
+    for (int i = 0; i < l8.n; ++i) src[n++] = l8.v[i];
+    while (n < 4 * d8) src[n++] = -1;
+    for (int i = 0; i < l4.n; ++i) src[n++] = l4.v[i];
+    while (n < 4 * d8 + 8 * d4) src[n++] = -1;
+    for (int i = 0; i < l2.n; ++i) src[n++] = l2.v[i];
+    while (n < n_slots_max) src[n++] = -1;
+    const int n_slots = 4 * steps;
+    const int64_t qt_bytes = (int64_t)n_slots * (int64_t)sizeof(RdkvSlot);
+    int64_t tiles[4], n_tiles = 0, n_q_tiles = 0;
+    for (int c = 0; c < 4; ++c) {
+      tiles[c] = ((int64_t)nt[c] + RDKV_TILE - 1) / RDKV_TILE;
+      n_tiles += tiles[c];
+      if (c < 3) n_q_tiles += tiles[c];
+    }
+    RDKV_REQUIRE(n_tiles <= 0x7fffffff, "%s: too many tiles", fn);
+    if (n_tiles > max_tiles) max_tiles = (int)n_tiles;
+    const int R = d8 + d4 + d2;
+    RdkvUnit u;
+    memset(&u, 0, sizeof(u));
+    u.k_off = (uint64_t)off;
+    off = align256(off + n_tiles * RDKV_TILE * 4 * R);
+    int64_t v_bytes = 0;
+    for (int c = 0; c < 4; ++c) {
+      u.v_off[c] = (uint64_t)off;
+      off = align256(off + tiles[c] * rdkv_v_tile_bytes(c));
+      v_bytes += tiles[c] * rdkv_v_tile_bytes(c);
+    }
+    u.sz_off = (uint64_t)off;
+    off = align256(off + n_q_tiles * RDKV_TILE * 4);
+    u.qtab_off = (uint64_t)off;
+    off = align256(off + qt_bytes);
+    for (int c = 0; c < 4; ++c) u.n_tok[c] = nt[c];
+    u.d8 = d8; u.d4 = d4; u.d2 = d2;
+    u.q_row = first_q_row + h * G;
+    units[h] = u;
+    stream_bytes += n_tiles * RDKV_TILE * 4 * R + v_bytes + n_q_tiles * RDKV_TILE * 4 + qt_bytes;
+    // the reference's own bytes for the same content: packed K rows and channel parameters, packed
+    // V rows, per-token parameters, fp16-kept rows
+    const int64_t row = (c2 + 3) / 4 + (c4 + 1) / 2 + c8;
+    const int64_t n_all = (int64_t)nt[0] + nt[1] + nt[2] + nt[3];
+    algo_bytes += n_all * row + 4 * (4 * ((c2 + 3) / 4) + 2 * ((c4 + 1) / 2) + c8) + 32 * (int64_t)nt[0] +
+                  64 * (int64_t)nt[1] + 128 * (int64_t)nt[2] + 4 * ((int64_t)nt[0] + nt[1] + nt[2]) +
+                  256 * (int64_t)nt[3];
+  }
+  sizes[0] = off;
+  sizes[1] = max_tiles;
+  sizes[2] = stream_bytes;
+  sizes[3] = algo_bytes;
   return RDKV_OK;
 }

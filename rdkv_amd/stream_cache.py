@@ -49,6 +49,10 @@ assert UNIT_DTYPE.itemsize == 96 and SLOT_DTYPE.itemsize == 8 and WORK_DTYPE.ite
 # partial stores and the ticket costs what the second launch does, so it stays an option.
 ONE_LAUNCH_MAX_WORK = 0
 
+# Tests set this: the direct packer's blobs then start out as 0xAB bytes instead of whatever the
+# allocator hands over, so that a byte the launches failed to write shows.
+_POISON_BLOBS = False
+
 
 def _align(x: int, a: int = 256) -> int:
     return -(-x // a) * a
@@ -228,44 +232,14 @@ def _plan_entry_units(tok, ch, n2p: int, n4p: int, first_row: int, G: int):
     head h; head h answers query rows first_row + h * G .. + G."""
     H_kv = len(tok)
     units = np.zeros(H_kv, dtype=UNIT_DTYPE)
-    src_tab = np.full((H_kv, 4 * MAX_STEPS), -1, dtype=np.int16)
-    off = 0
-    max_tiles = 0
-    stream_bytes = algo_bytes = 0
-    rows = []            # per head: the descriptor's fields, written to the record array in one go
-    for h in range(H_kv):
-        n_tok = tok[h]
-        c2, c4, c8 = ch[h]
-        d8, d4, d2, src = slot_plan(c2, c4, c8, n2p, n4p)
-        steps = d8 + 2 * d4 + 4 * d2
-        assert steps <= MAX_STEPS, f"{steps} channel steps exceed {MAX_STEPS}"
-        src_tab[h, :len(src)] = src
-        qt_nbytes = len(src) * SLOT_DTYPE.itemsize
-        tiles = [-(-n // TILE) for n in n_tok]
-        n_tiles, n_q_tiles = sum(tiles), sum(tiles[:3])
-        max_tiles = max(max_tiles, n_tiles)
-        R = d8 + d4 + d2
-        k_off = off
-        off = _align(off + n_tiles * TILE * 4 * R)
-        v_off = []
-        for c in range(4):
-            v_off.append(off)
-            off = _align(off + tiles[c] * V_TILE_BYTES[c])
-        sz_off = off
-        off = _align(off + n_q_tiles * TILE * 4)
-        qtab_off = off
-        off = _align(off + qt_nbytes)
-        rows.append((tuple(n_tok), d8, d4, d2, first_row + h * G, k_off, tuple(v_off), sz_off, qtab_off))
-        # accounting
-        stream_bytes += (n_tiles * TILE * 4 * R + sum(t * b for t, b in zip(tiles, V_TILE_BYTES))
-                         + n_q_tiles * TILE * 4 + qt_nbytes)
-        row = -(-c2 // 4) + -(-c4 // 2) + c8
-        algo_bytes += (sum(n_tok) * row + 4 * (4 * -(-c2 // 4) + 2 * -(-c4 // 2) + c8)
-                       + 32 * n_tok[0] + 64 * n_tok[1] + 128 * n_tok[2] + 4 * sum(n_tok[:3])
-                       + 256 * n_tok[3])
-    for i, name in enumerate(("n_tok", "d8", "d4", "d2", "q_row", "k_off", "v_off", "sz_off", "qtab_off")):
-        units[name] = [r[i] for r in rows]
-    return units, src_tab, off, max_tiles, int(stream_bytes), int(algo_bytes)
+    src_tab = np.empty((H_kv, 4 * MAX_STEPS), dtype=np.int16)
+    tok_a = np.ascontiguousarray(tok, dtype=np.int32).reshape(H_kv, 4)
+    ch_a = np.ascontiguousarray(ch, dtype=np.int32).reshape(H_kv, 3)
+    sizes = np.zeros(4, dtype=np.int64)
+    _lib.check(_lib.load().rdkv_stream_plan_layer(tok_a.ctypes.data, 4, ch_a.ctypes.data, 3, H_kv, int(n2p), int(n4p),
+                                                  int(first_row), int(G), units.ctypes.data, src_tab.ctypes.data,
+                                                  4 * MAX_STEPS, sizes.ctypes.data))
+    return units, src_tab, int(sizes[0]), int(sizes[1]), int(sizes[2]), int(sizes[3])
 
 
 def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_bytes: Optional[list] = None):
@@ -411,12 +385,12 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
         kb_all = torch.cat([entries[i][3].reshape(H_kv, 128) for i in idx]) if len(idx) > 1 else entries[idx[0]][3]
         order, _, plan, counts_h, info_h, kb_dev = packing._plan_layers(vb_all.reshape(-1, T), kb_all.reshape(-1, 128), dev)
         plans = []
+        counts_a = np.asarray(counts_h, dtype=np.int32).reshape(-1, 4)
+        chan_a = np.ascontiguousarray(np.asarray(info_h, dtype=np.int32).reshape(-1, 8)[:, 2:5])
         for j, i in enumerate(idx):
-            rows = slice(j * H_kv, (j + 1) * H_kv)
-            tok = [tuple(int(x) for x in r[:4]) for r in counts_h[rows]]
-            ch = [tuple(int(x) for x in r[2:5]) for r in info_h[rows]]
-            m2, m4, m8 = (max(c[k] for c in ch) for k in range(3))
-            max_tv, max_n16 = max(sum(t[:3]) for t in tok), max(t[3] for t in tok)
+            tok, ch = counts_a[j * H_kv:(j + 1) * H_kv], chan_a[j * H_kv:(j + 1) * H_kv]
+            m2, m4, m8 = (int(x) for x in ch.max(axis=0))
+            max_tv, max_n16 = int(tok[:, :3].sum(axis=1).max()), int(tok[:, 3].max())
             if max_tv + max_n16 == 0 or m2 + m4 + m8 == 0:
                 plans.append(None)               # degenerate: the two-step path knows the reference's behaviour
                 continue
@@ -426,8 +400,9 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
             plans.append((units, src_tab, off, max_tiles, sb, ab, n2p, n4p, m8, max_tv, max_n16))
         live = [p for p in plans if p is not None]
         if live:
-            units_dev = torch.from_numpy(np.concatenate([p[0] for p in live]).view(np.uint8).copy()).to(dev)
-            src_dev = torch.from_numpy(np.concatenate([p[1] for p in live])).to(dev)
+            units_dev, src_dev = _lib.upload(dev, np.concatenate([p[0] for p in live]), np.concatenate([p[1] for p in live]))
+            mm_all = torch.empty(len(live), H_kv * 768, dtype=torch.float32, device=dev)   # min / max, channel quantizers
+            sm_all = torch.empty(len(live), 2, H_kv, dtype=torch.float32, device=dev)
         row = 0
         for j, (i, p) in enumerate(zip(idx, plans)):
             K, V, vb, kb = entries[i]
@@ -438,42 +413,54 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
                 out[i] = (u, b[0], per[0][0], per[0][1], sm)
                 continue
             units, src_tab, off, max_tiles, sb, ab, n2p, n4p, m8, max_tv, max_n16 = p
-            blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
-            assert blob.data_ptr() % 256 == 0
-            mm = torch.empty(H_kv * 256, dtype=torch.float32, device=dev)
-            sm = torch.zeros(2, H_kv, dtype=torch.float32, device=dev)
-            kb_rows = kb_dev[j * H_kv:(j + 1) * H_kv]
-            order_rows = order[j * H_kv:(j + 1) * H_kv]
-            _lib.check(lib.rdkv_pack_layer_stream(
-                K.data_ptr(), V.data_ptr(), K.stride(1), K.stride(2), H_kv, order_rows.data_ptr(), order_rows.stride(0),
-                plan.data_ptr() + 16 * j * H_kv, kb_rows.data_ptr(), kb_rows.element_size(), kb_rows.stride(0),
-                n2p, n4p, m8, max_tv, max_n16, units_dev.data_ptr() + row * UNIT_DTYPE.itemsize,
-                src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, blob.data_ptr(),
-                mm.data_ptr(), sm.data_ptr(), stream))
-            row += H_kv
+            # + slack for 16-byte tail reads; the launches write every byte, so no clearing
+            blob_bytes = max(off, 256) + 256
+            blob = torch.full((blob_bytes,), 0xAB, dtype=torch.uint8, device=dev) if _POISON_BLOBS else \
+                torch.empty(blob_bytes, dtype=torch.uint8, device=dev)
             base = blob.data_ptr()
+            assert base % 256 == 0
+            k = row // H_kv
+            _lib.check(lib.rdkv_pack_layer_stream(
+                K.data_ptr(), V.data_ptr(), K.stride(1), K.stride(2), H_kv,
+                order.data_ptr() + 4 * j * H_kv * order.stride(0), order.stride(0),
+                plan.data_ptr() + 16 * j * H_kv, kb_dev.data_ptr() + j * H_kv * kb_dev.stride(0) * kb_dev.element_size(),
+                kb_dev.element_size(), kb_dev.stride(0),
+                n2p, n4p, m8, max_tv, max_n16, units_dev.data_ptr() + row * UNIT_DTYPE.itemsize,
+                src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, base, blob_bytes,
+                mm_all.data_ptr() + 4 * k * mm_all.stride(0), sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
+            row += H_kv
             for name in ("k_off", "sz_off", "qtab_off"):
                 units[name] += base
             units["v_off"] += base
-            pending.append((i, units, blob, sm, sb, ab, (mm, kb_rows, order_rows, plan)))
+            pending.append((i, units, blob, sm_all[k], sb, ab, None))
         if live:
-            pending.append((None, None, None, None, 0, 0, (units_dev, src_dev)))
+            pending.append((None, None, None, None, 0, 0, (units_dev, src_dev, mm_all, sm_all, kb_dev, order, plan)))
+    sm_dev = None
     if pending:
         sms = [pn[3] for pn in pending if pn[0] is not None]
-        sm_all = torch.stack(sms).transpose(1, 2).cpu().numpy().astype(np.float32) if sms else None   # (synchronizes)
-        torch.cuda.current_stream(dev).synchronize()
+        sm_dev = torch.stack(sms).transpose(1, 2) if sms else None
         k = 0
         for i, units, blob, _, sb, ab, _ in pending:
-            if i is None:
-                continue
-            out[i] = (units, blob, sb, ab, sm_all[k].reshape(-1, 2))
-            k += 1
+            if i is not None:
+                out[i] = (units, blob, sb, ab, k)        # k: the entry's row of sm_dev
+                k += 1
     units_all = np.concatenate([np.asarray(o[0], dtype=UNIT_DTYPE) for o in out])
     blobs = [o[1] for o in out]
     if entry_bytes is not None:
         entry_bytes.extend((int(o[2]), int(o[3])) for o in out)
-    return (units_all, blobs, int(sum(o[2] for o in out)), int(sum(o[3] for o in out)), H_q,
-            np.concatenate([o[4] for o in out]).astype(np.float32))
+    resolved: list = []
+
+    def scale_max():
+        """The units' largest K channel and V token scales, read back from the launches above (the
+        one synchronization of the direct path; callers do their host work first)."""
+        if not resolved:
+            sm_host = _lib.download(sm_dev) if sm_dev is not None else None   # (synchronizes)
+            del pending[:]
+            parts = [sm_host[o[4]].reshape(-1, 2) if isinstance(o[4], int) else o[4] for o in out]
+            resolved.append(np.concatenate(parts).astype(np.float32))
+        return resolved[0]
+
+    return (units_all, blobs, int(sum(o[2] for o in out)), int(sum(o[3] for o in out)), H_q, scale_max)
 
 
 def build_stream_cache_from_kv(entries: Sequence[Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]],
@@ -515,13 +502,16 @@ def v_shift_of(v_scale_max: np.ndarray) -> np.ndarray:
 def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: int, kv_algo_bytes: int,
                   scale_max: np.ndarray, *, multi_source: bool, work_bytes, n_groups, groups_per_cu: int,
                   cost) -> StreamCache:
-    """Order the units, cut the tile stream into work items and groups, upload the tables."""
+    """Order the units, cut the tile stream into work items and groups, upload the tables.
+    ``scale_max``: fp32 [n_units, 2], or a function returning it, called once everything that does
+    not need it is done (the direct packer's launches are still running until then)."""
     dev = blobs[0].device
     n_groups_arg, cost_arg = n_groups, cost
+    order = None
     if multi_source:
         # sources of one output row next to each other, so that their work items are contiguous
         order = np.argsort(units_np["q_row"], kind="stable")
-        units_np, scale_max = units_np[order], scale_max[order]
+        units_np = units_np[order]
     tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
     R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
     if work_bytes is None and n_groups is None:
@@ -548,17 +538,24 @@ def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: i
         merger = np.maximum.accumulate(np.where(wc > 0, np.arange(len(units_np)), 0)) if multi_source \
             else np.arange(len(units_np))
         iu = work_np["unit"]
-        work_np["u"] = units_np[iu]
+        # (the descriptor copies as bytes: assignment between record arrays goes field by field)
+        work_np.view(np.uint8).reshape(-1, WORK_DTYPE.itemsize)[:, 16:16 + UNIT_DTYPE.itemsize] = \
+            units_np.view(np.uint8).reshape(-1, UNIT_DTYPE.itemsize)[iu]
         work_np["merge_unit"] = merger[iu]
         work_np["merge_begin"] = wb[merger[iu]]
         work_np["merge_count"] = wc[merger[iu]]
+    rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
+    if callable(scale_max):
+        scale_max = scale_max()
+    if order is not None:
+        scale_max = scale_max[order]
+    if len(units_np):
         work_np["k_scale_max"] = scale_max[iu, 0]
         work_np["v_shift"] = v_shift_of(scale_max[:, 1])[iu]
-    rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
-    units_dev = torch.from_numpy(units_np.view(np.uint8).copy()).to(dev)
-    work_dev = torch.from_numpy(work_np.view(np.uint8).copy()).to(dev) if len(work_np) else torch.zeros(
-        WORK_DTYPE.itemsize, dtype=torch.uint8, device=dev)
-    groups_dev = torch.from_numpy(groups_np).to(dev) if groups_np is not None else None
+    units_dev, work_dev, groups_dev = _lib.upload(
+        dev, units_np, work_np if len(work_np) else np.zeros(1, dtype=WORK_DTYPE),
+        groups_np if groups_np is not None else np.zeros(1, dtype=np.int32))
+    groups_dev = groups_dev.view(torch.int32) if groups_np is not None else None
     return StreamCache(tickets=torch.zeros(max(1, len(units_np)), dtype=torch.int32, device=dev),
                        partition={"work_bytes": work_bytes, "n_groups": n_groups_arg, "groups_per_cu": groups_per_cu,
                                   "cost": cost_arg}, unit_scale_max=scale_max,
@@ -639,9 +636,12 @@ def _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max) -> Li
     for i, cache in enumerate(caches):
         assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
         units = np.concatenate([cache.units_host.copy(), new_units[i * n_per:(i + 1) * n_per]])
+        def scale_max(i=i, cache=cache):
+            new = new_scale_max() if callable(new_scale_max) else new_scale_max
+            return np.concatenate([cache.unit_scale_max, new[i * n_per:(i + 1) * n_per]])
+
         out.append(_finish_cache(units, list(cache.blobs) + [new_blobs[i]], G, H_q, cache.stream_bytes + per_entry[i][0],
-                                 cache.kv_algorithmic_bytes + per_entry[i][1],
-                                 np.concatenate([cache.unit_scale_max, new_scale_max[i * n_per:(i + 1) * n_per]]),
+                                 cache.kv_algorithmic_bytes + per_entry[i][1], scale_max,
                                  multi_source=True, work_bytes=None,
                                  n_groups=None, groups_per_cu=1, cost=None))
     return out

@@ -113,8 +113,14 @@ def _assert_same_cache(a, b):
         assert x.numel() == y.numel() and torch.equal(x, y), f"blob {i} differs"
 
 
+@pytest.fixture
+def poisoned_blobs(monkeypatch):
+    """The direct packer's blobs start as 0xAB bytes: a byte its launches leave out cannot pass for a zero."""
+    monkeypatch.setattr(stream_cache, "_POISON_BLOBS", True)
+
+
 @pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b"])
-def test_direct_stream_packer_golden(name):
+def test_direct_stream_packer_golden(name, poisoned_blobs):
     """fp16 K / V + allocations straight into the streaming format: every bit the reference wrote
     for the layer (its own packed tensors, stored as golden data) is found in the blob."""
     g = load_golden(name)
@@ -128,7 +134,7 @@ def test_direct_stream_packer_golden(name):
 
 
 @pytest.mark.parametrize("cfg_idx,ctx,layers", [(0, 700, 1), (1, 2300, 2), (2, 1500, 1), (3, 900, 2), (1, 64, 1), (0, 130, 1), (1, 32768, 1), (2, 131072, 1)])
-def test_direct_stream_packer_matches_pack_then_relayout(cfg_idx, ctx, layers):
+def test_direct_stream_packer_matches_pack_then_relayout(cfg_idx, ctx, layers, poisoned_blobs):
     """The direct packer's cache against packing + re-layout of the same layers: the same unit
     descriptors, largest scales and blob bytes; and the layer the oracle packs from the same CPU
     data is found in the blob."""
@@ -150,7 +156,7 @@ def test_direct_stream_packer_matches_pack_then_relayout(cfg_idx, ctx, layers):
         _assert_cache_holds_layer(one, *oracle_layers[0])
 
 
-def test_direct_stream_packer_ragged_and_degenerate_entries():
+def test_direct_stream_packer_ragged_and_degenerate_entries(poisoned_blobs):
     """Heads that keep nothing, a head that keeps only fp16 tokens, a layer where every head keeps
     the same counts (no zero rows in the K canvas: 0 must not join a min / max), inputs the direct
     kernel does not take (a strided view, fp32 values): always the bytes of packing + re-layout."""

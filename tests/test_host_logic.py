@@ -211,6 +211,56 @@ def test_slot_plan_covers_every_channel_and_fits_the_kernel():
     assert (d8, d4, d2) == (32, 0, 0) and sorted(src) == [0, 1, 4] + [6 + i for i in range(125)]
 
 
+def test_stream_plan_layer_matches_the_slot_plan_and_lays_sections_out_in_order():
+    """The library's host-side planner against ``slot_plan`` (the slot order) and against the layout
+    rules restated here: sections K, V2, V4, V8, V16, {scale, zp} pairs, slot table, each 256-byte
+    aligned, in that order, head after head; sizes and byte counts from the tile counts."""
+    from rdkv_amd import stream_cache as sc
+    rng = np.random.default_rng(31)
+    splits = [(16, 32, 16), (0, 11, 5), (2, 1, 125), (0, 0, 0), (128, 0, 0), (0, 128, 0), (0, 0, 128), (17, 9, 3)]
+    while len(splits) < 120:
+        c8 = int(rng.integers(0, 129)); c4 = int(rng.integers(0, 129 - c8)); c2 = int(rng.integers(0, 129 - c8 - c4))
+        splits.append((c2, c4, c8))
+    tiles_of = lambda n: -(-n // 64)
+    for start in range(0, len(splits), 8):
+        ch = splits[start:start + 8]
+        H = len(ch)
+        tok = [tuple(int(x) for x in rng.choice([0, 1, 63, 64, 65, 700, 5000], size=4)) for _ in range(H)]
+        n2p = max(-(-c[0] // 4) * 4 for c in ch)
+        n4p = max(-(-c[1] // 2) * 2 for c in ch)
+        G, first = int(rng.integers(1, 9)), int(rng.integers(0, 50)) * 8
+        units, src_tab, off, max_tiles, sb, ab = sc._plan_entry_units(tok, ch, n2p, n4p, first, G)
+        pos = 0
+        want_sb = 0
+        for h in range(H):
+            d8, d4, d2, src = sc.slot_plan(*ch[h], n2p, n4p)
+            u = units[h]
+            assert (int(u["d8"]), int(u["d4"]), int(u["d2"])) == (d8, d4, d2)
+            assert list(src_tab[h, :len(src)]) == src and (src_tab[h, len(src):] == -1).all()
+            assert tuple(int(x) for x in u["n_tok"]) == tok[h] and int(u["q_row"]) == first + h * G
+            assert int(u["work_begin"]) == 0 and int(u["work_count"]) == 0
+            t = [tiles_of(n) for n in tok[h]]
+            sections = [("k_off", sum(t) * 64 * 4 * (d8 + d4 + d2))]
+            sections += [(("v_off", c), t[c] * (2048 << c)) for c in range(4)]
+            sections += [("sz_off", sum(t[:3]) * 256), ("qtab_off", 8 * len(src))]
+            for name, nbytes in sections:
+                got = int(u[name[0]][name[1]]) if isinstance(name, tuple) else int(u[name])
+                assert got == pos and pos % 256 == 0, (name, got, pos)
+                pos = -(-(pos + nbytes) // 256) * 256
+                want_sb += nbytes
+        assert off == pos and sb == want_sb and max_tiles == max(sum(tiles_of(n) for n in tk) for tk in tok)
+        c2s, c4s, c8s = (np.array([c[k] for c in ch]) for k in range(3))
+        nt = np.array(tok, dtype=np.int64)
+        rows = -(-c2s // 4) + -(-c4s // 2) + c8s
+        want_ab = int((nt.sum(1) * rows + 4 * (4 * -(-c2s // 4) + 2 * -(-c4s // 2) + c8s) + 32 * nt[:, 0] + 64 * nt[:, 1]
+                       + 128 * nt[:, 2] + 4 * nt[:, :3].sum(1) + 256 * nt[:, 3]).sum())
+        assert ab == want_ab
+    # more channel steps than the format holds are refused by name
+    import pytest
+    with pytest.raises(Exception, match="bad counts"):
+        sc._plan_entry_units([(1, 0, 0, 0)], [(100, 100, 0)], 100, 100, 0, 1)
+
+
 def test_selection_and_planning_entry_points_reject_bad_arguments():
     """Argument checks of the newer entry points run before any device work, so they can be
     exercised without a GPU: status code and message."""
