@@ -317,6 +317,27 @@ int rdkv_stream_plan_layer(const int32_t *tok_counts, int64_t tok_stride, const 
                            int64_t ch_stride, int H_kv, int n2p, int n4p, int first_q_row, int G,
                            RdkvUnit *units, int16_t *src_slot, int n_slots_max, int64_t *sizes);
 
+/* Host side of the fused kernel's work decomposition (no GPU work; every pointer is host memory).
+ * The unit-major, class-minor sequence of 64-token tiles of units[n_units] is cut into n_groups
+ * contiguous runs of equal modelled cost, one per workgroup of the streaming launch (shares
+ * proportional to speed[g % n_speed]; n_speed = 0: equal shares).  A tile costs
+ * cost_tile[class] + cost_k_dword * (d8 + d4 + d2), the first tile of a unit cost_item more
+ * (sums in double precision, in order).  A run that crosses a unit boundary becomes several work
+ * items; a unit without tiles gets one empty item.  Written: work_begin / work_count of every unit
+ * (multi_source != 0: units of equal q_row are adjacent sources of one output row, the first
+ * carries the run's item count, the others 0); work[0 .. *n_work) with unit, tile range, a copy of
+ * the unit's descriptor and the merging unit's item range (work_capacity >= n_groups + 2 * n_units);
+ * groups[n_groups + 1], offsets into work.  k_scale_max / v_shift: rdkv_stream_work_scales. */
+int rdkv_stream_partition(RdkvUnit *units, int n_units, int n_groups, const double *cost_tile,
+                          double cost_k_dword, double cost_item, const double *speed, int n_speed,
+                          int multi_source, RdkvWork *work, int work_capacity, int32_t *groups, int *n_work);
+
+/* k_scale_max and v_shift of every work item from its unit's largest scales (host memory):
+ * scale_max[2 * unit] = largest K channel scale, [2 * unit + 1] = largest V token scale, as
+ * rdkv_pack_layer_stream reports them.  v_shift: the smallest e >= 0 with scale * 2^(6 - e) < 2^15,
+ * at most 40. */
+int rdkv_stream_work_scales(RdkvWork *work, int n_work, const float *scale_max, int n_units);
+
 /* Re-lay one layer (H_kv units) from the reference's padded tensors into the blob.
  * src_slot: int16 [H_kv][n_slots_max] = for each stream slot the index of the source channel
  * in the padded sorted order of K_ch_scale (-1 = pad slot).  units: the layer's H_kv
@@ -355,10 +376,12 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
  * max_tiles: as for rdkv_stream_relayout_layer.  blob_bytes: size of the blob (a multiple of 4, at
  * least sizes[0] of rdkv_stream_plan_layer): the launches write every byte of it, so it need not be
  * cleared.  minmax_ws: H_kv * 768 floats of scratch, 16-byte aligned (min / max accumulators, then
- * the quantizer of every channel).
+ * the quantizer of every channel), prepared once by rdkv_pack_layer_stream_ws_init: every call
+ * leaves the accumulators at their start values again, so calls on one stream can share it.
  * scale_max: float [2][H_kv]: receives per head the largest K channel scale and the largest V token
  * scale (as the fp16 values stored), which RdkvWork.k_scale_max / v_shift are made from.  K and V
  * rows must be 16-byte aligned (RDKV_EUNSUPPORTED otherwise). */
+int rdkv_pack_layer_stream_ws_init(float *minmax_ws, int H_kv, void *stream);
 int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
                            int H_kv, const int32_t *order, int64_t order_stride_h, const int32_t *counts,
                            const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int n2p, int n4p, int n8,

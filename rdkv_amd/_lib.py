@@ -61,6 +61,9 @@ SIGNATURES = {
     "rdkv_v_weighted_sum_workspace_bytes": (L, [I]),
     "rdkv_v_weighted_sum": (I, [P, L, I, I, P, L, P, L, P, L, P, P, L, P, I, I, I, P, L, P, L, P, L, P, L, P]),
     "rdkv_stream_plan_layer": (I, [P, L, P, L, I, I, I, I, I, P, P, I, P]),
+    "rdkv_stream_partition": (I, [P, I, I, P, ctypes.c_double, ctypes.c_double, P, I, I, P, I, P, P]),
+    "rdkv_stream_work_scales": (I, [P, I, P, I]),
+    "rdkv_pack_layer_stream_ws_init": (I, [P, I, P]),
     "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, L, P, P, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,
                                        P, L, P, P, L, P, P, I, I, I, I, P, P]),

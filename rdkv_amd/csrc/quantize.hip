@@ -1290,11 +1290,17 @@ static int layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, i
 // (for the packer that writes the streaming format, stream_pack.hip)
 int rdkv_layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
                         const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tk,
-                        float *minmax_ws, hipStream_t s) {
+                        float *minmax_ws, bool init, hipStream_t s) {
   RDKV_REQUIRE(stride_t % 2 == 0 && stride_h % 2 == 0 && ((uintptr_t)K_f16 % 4) == 0, "%s: rows must be 4-byte aligned",
                fn);
   return layer_k_minmax(fn, K_f16, stride_h, stride_t, H_kv, D, order, order_stride_h, counts, max_tk,
-                        reinterpret_cast<uint32_t *>(minmax_ws), true, s);
+                        reinterpret_cast<uint32_t *>(minmax_ws), init, s);
+}
+
+// start values of H_kv heads' accumulators (D minima, D maxima each)
+void rdkv_layer_k_minmax_init(float *minmax_ws, int H_kv, int D, hipStream_t s) {
+  hipLaunchKernelGGL(minmax_init_layer_kernel, dim3((unsigned)rdkv_cdiv((int64_t)H_kv * 2 * D, 256)), dim3(256), 0, s,
+                     reinterpret_cast<uint32_t *>(minmax_ws), D, H_kv);
 }
 
 // The K half: per-channel min/max over each head's kept rows, then scales, zero points and the

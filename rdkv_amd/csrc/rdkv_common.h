@@ -37,7 +37,8 @@ static inline int64_t rdkv_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; 
 // order-preserving integers).  Launches only.
 int rdkv_layer_k_minmax(const char *fn, const void *K_f16, int64_t stride_h, int64_t stride_t, int H_kv, int D,
                         const int32_t *order, int64_t order_stride_h, const int32_t *counts, int64_t max_tk,
-                        float *minmax_ws, hipStream_t s);
+                        float *minmax_ws, bool init, hipStream_t s);
+void rdkv_layer_k_minmax_init(float *minmax_ws, int H_kv, int D, hipStream_t s);
 
 #define RDKV_WAVE 64
 

@@ -14,7 +14,11 @@
 // quantizes them in registers, parks the codes in LDS as bytes and assembles the tile's dwords from
 // there.  Between them the launches write every byte of the blob.
 #include "rdkv_common.h"
+#include <math.h>
 #include <string.h>
+
+#include <algorithm>
+#include <vector>
 
 #include "stream_format.h"
 
@@ -45,7 +49,7 @@ struct StreamPackArgs {
   int n2p, n4p;                   // the layer's padded 2-bit / 4-bit channel counts (maxima over heads)
   int64_t max_tv;
   int max_n16;
-  const uint32_t *mm;             // per head: 128 minima, 128 maxima (order-preserving integers)
+  uint32_t *mm;                   // per head: 128 minima, 128 maxima (order-preserving integers)
   const RdkvUnit *units;          // offsets relative to `blob`
   const int16_t *src_slot;
   int n_slots_max, max_tiles;
@@ -135,6 +139,9 @@ slot_params_kernel(StreamPackArgs a, float4 *__restrict__ chan_params) {
   for (int o = 1; o < 64; o <<= 1) smax = fmaxf(smax, __shfl_xor(smax, o, 64));
   if (lane == 0) wave_max[tid >> 6] = smax;
   __syncthreads();
+  // the accumulators go back to their start values: the next call finds them ready
+  a.mm[(int64_t)h * 2 * kD + tid] = rdkv_float_to_ordered(INFINITY);
+  a.mm[(int64_t)h * 2 * kD + kD + tid] = rdkv_float_to_ordered(-INFINITY);
   const int s = slot_of_ch[tid];
   chan_params[(int64_t)h * kD + tid] = s >= 0 ? slot_p[s] : make_chan(0.f, 0.f, 0.f, -1);
   if (tid == 0) {
@@ -477,6 +484,14 @@ stream_pack_kernel(StreamPackArgs a, const float4 *__restrict__ chan_params) {
 
 }  // namespace
 
+RDKV_API int rdkv_pack_layer_stream_ws_init(float *minmax_ws, int H_kv, void *stream) {
+  const char *fn = "rdkv_pack_layer_stream_ws_init";
+  RDKV_REQUIRE(minmax_ws && H_kv >= 1 && H_kv <= 65535, "%s: bad arguments", fn);
+  rdkv_layer_k_minmax_init(minmax_ws, H_kv, kD, (hipStream_t)stream);
+  RDKV_CHECK_LAUNCH(fn);
+  return RDKV_OK;
+}
+
 RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_h, int64_t stride_t,
                                     int H_kv, const int32_t *order, int64_t order_stride_h,
                                     const int32_t *counts, const void *k_bits, int kb_elem_size,
@@ -506,7 +521,7 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
   const int64_t max_tk = max_tv + max_n16;
   // per-channel min / max of every head's kept rows (the K canvas without its zero rows)
   int rc = rdkv_layer_k_minmax(fn, K_f16, stride_h, stride_t, H_kv, kD, order, order_stride_h, counts, max_tk,
-                               minmax_ws, s);
+                               minmax_ws, /*init=*/false, s);
   if (rc != RDKV_OK) return rc;
   StreamPackArgs a;
   a.K = (const __half *)K_f16; a.V = (const __half *)V_f16;
@@ -515,7 +530,7 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
   a.k_bits = k_bits; a.kb_elem_size = kb_elem_size; a.kb_stride_h = kb_stride_h;
   a.n2p = n2p; a.n4p = n4p;
   a.max_tv = max_tv; a.max_n16 = max_n16;
-  a.mm = reinterpret_cast<const uint32_t *>(minmax_ws);
+  a.mm = reinterpret_cast<uint32_t *>(minmax_ws);
   a.units = units; a.src_slot = src_slot; a.n_slots_max = n_slots_max; a.max_tiles = max_tiles;
   a.blob = blob;
   a.scale_max = reinterpret_cast<uint32_t *>(scale_max);
@@ -650,5 +665,160 @@ RDKV_API int rdkv_stream_plan_layer(const int32_t *tok_counts, int64_t tok_strid
   sizes[1] = max_tiles;
   sizes[2] = stream_bytes;
   sizes[3] = algo_bytes;
+  return RDKV_OK;
+}
+
+// Host side of the fused kernel's work decomposition (no GPU work): cut the unit-major, class-minor
+// sequence of 64-token tiles into n_groups contiguous runs of equal modelled cost (shares
+// proportional to speed[g % n_speed]), one run per workgroup; a run that crosses a unit boundary
+// becomes several work items; a unit without tiles gets one empty item.  Every tile costs
+// cost_tile[class] + cost_k_dword * (d8 + d4 + d2), the first tile of a unit cost_item more.
+// Cumulative costs and shares are summed in order, in double precision.
+// units[n_units] (ordered; with multi_source the sources of one output row adjacent): work_begin /
+// work_count are written; with multi_source the first unit of a run of equal q_row carries the
+// run's item count, the others 0.  work[work_capacity >= n_groups + 2 * n_units]: unit, tile range,
+// the unit's descriptor, the merging unit and its item range (k_scale_max / v_shift: see
+// rdkv_stream_work_scales).  groups[n_groups + 1]: offsets into work.  Returns the item count in
+// *n_work.
+RDKV_API int rdkv_stream_partition(RdkvUnit *units, int n_units, int n_groups, const double *cost_tile,
+                                   double cost_k_dword, double cost_item, const double *speed, int n_speed,
+                                   int multi_source, RdkvWork *work, int work_capacity, int32_t *groups,
+                                   int *n_work) {
+  const char *fn = "rdkv_stream_partition";
+  RDKV_REQUIRE(units && cost_tile && work && groups && n_work && n_units >= 0 && n_groups >= 1, "%s: bad arguments", fn);
+  RDKV_REQUIRE(n_speed >= 0 && (n_speed == 0 || speed), "%s: bad speed table", fn);
+  RDKV_REQUIRE((int64_t)work_capacity >= (int64_t)n_groups + 2 * (int64_t)n_units, "%s: work table too small", fn);
+  const int U = n_units;
+  std::vector<int64_t> unit_start((size_t)U + 1, 0);
+  for (int u = 0; u < U; ++u) {
+    int64_t t = 0;
+    for (int c = 0; c < 4; ++c) {
+      RDKV_REQUIRE(units[u].n_tok[c] >= 0, "%s: negative token count", fn);
+      t += ((int64_t)units[u].n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
+    }
+    unit_start[u + 1] = unit_start[u] + t;
+  }
+  const int64_t total = unit_start[U];
+  RDKV_REQUIRE(total <= 0x7fffffffLL, "%s: too many tiles", fn);
+  // cumulative cost of every tile
+  std::vector<double> cum((size_t)total);
+  {
+    double acc = 0.0;
+    int64_t i = 0;
+    for (int u = 0; u < U; ++u) {
+      const double R = (double)((int64_t)units[u].d8 + units[u].d4 + units[u].d2);
+      bool first = true;
+      for (int c = 0; c < 4; ++c) {
+        const int64_t nt = ((int64_t)units[u].n_tok[c] + RDKV_TILE - 1) / RDKV_TILE;
+        const double seg = cost_k_dword * R + cost_tile[c];
+        for (int64_t t = 0; t < nt; ++t) {
+          acc += first ? seg + cost_item : seg;
+          first = false;
+          cum[(size_t)i++] = acc;
+        }
+      }
+    }
+  }
+  // group boundaries
+  std::vector<int64_t> group_cuts((size_t)n_groups + 1, 0);
+  group_cuts[n_groups] = total;
+  if (total > 0 && n_groups > 1) {
+    std::vector<double> share_cum((size_t)n_groups);
+    double acc = 0.0;
+    for (int g = 0; g < n_groups; ++g) {
+      acc += n_speed ? speed[g % n_speed] : 1.0;
+      share_cum[g] = acc;
+    }
+    const double all = cum[(size_t)total - 1];
+    for (int g = 0; g + 1 < n_groups; ++g) {
+      const double thr = all * (share_cum[g] / share_cum[n_groups - 1]);
+      const int64_t idx = std::lower_bound(cum.begin(), cum.end(), thr) - cum.begin();   // first cum >= thr
+      group_cuts[g + 1] = std::min(idx + 1, total);
+    }
+  }
+  for (int g = 1; g <= n_groups; ++g) group_cuts[g] = std::max(group_cuts[g], group_cuts[g - 1]);
+  // items: walk units and group cuts together
+  int nw = 0, g = 0;
+  std::vector<int32_t> item_group;
+  item_group.reserve((size_t)n_groups + 2 * (size_t)U);
+  for (int u = 0; u < U; ++u) {
+    const int64_t a = unit_start[u], b = unit_start[u + 1];
+    units[u].work_begin = nw;
+    if (a == b) {
+      // an empty unit: one empty item, in the group of the position it sits at
+      while (g + 1 < n_groups && group_cuts[g + 1] <= a) ++g;
+      RdkvWork &w = work[nw++];
+      memset(&w, 0, sizeof(w));
+      w.unit = u;
+      item_group.push_back(std::min(g, n_groups - 1));
+    } else {
+      int64_t s = a;
+      while (s < b) {
+        while (g + 1 < n_groups && group_cuts[g + 1] <= s) ++g;
+        const int64_t next_cut = g + 1 <= n_groups ? group_cuts[g + 1] : total;
+        const int64_t e = std::min(b, next_cut > s ? next_cut : b);
+        RdkvWork &w = work[nw++];
+        memset(&w, 0, sizeof(w));
+        w.unit = u;
+        w.tile_begin = (int32_t)(s - a);
+        w.tile_end = (int32_t)(e - a);
+        item_group.push_back(std::min(g, n_groups - 1));
+        s = e;
+      }
+    }
+    units[u].work_count = nw - units[u].work_begin;
+  }
+  // group offsets: first item of every group
+  {
+    int i = 0;
+    for (int gg = 0; gg <= n_groups; ++gg) {
+      while (i < nw && item_group[(size_t)i] < gg) ++i;
+      groups[gg] = i;
+    }
+  }
+  // the unit that merges an output row: the unit itself, or the first source of its row
+  std::vector<int32_t> merger((size_t)U);
+  if (multi_source) {
+    int first = 0;
+    for (int u = 0; u < U; ++u) {
+      if (u == 0 || units[u].q_row != units[u - 1].q_row) first = u;
+      else {
+        units[first].work_count += units[u].work_count;
+        units[u].work_count = 0;
+      }
+      merger[u] = first;
+    }
+  } else {
+    for (int u = 0; u < U; ++u) merger[u] = u;
+  }
+  for (int i = 0; i < nw; ++i) {
+    RdkvWork &w = work[i];
+    const int m = merger[(size_t)w.unit];
+    w.u = units[w.unit];
+    w.merge_unit = m;
+    w.merge_begin = units[m].work_begin;
+    w.merge_count = units[m].work_count;
+  }
+  *n_work = nw;
+  return RDKV_OK;
+}
+
+// k_scale_max and v_shift of every work item from its unit's largest scales (scale_max[unit][0] = K
+// channel scale, [1] = V token scale): v_shift = the smallest e >= 0 with scale * 2^(6 - e) < 2^15,
+// at most 40 (0 for a NaN).
+RDKV_API int rdkv_stream_work_scales(RdkvWork *work, int n_work, const float *scale_max, int n_units) {
+  const char *fn = "rdkv_stream_work_scales";
+  RDKV_REQUIRE(n_work >= 0 && (n_work == 0 || (work && scale_max)), "%s: bad arguments", fn);
+  for (int i = 0; i < n_work; ++i) {
+    const int u = work[i].unit;
+    RDKV_REQUIRE(u >= 0 && u < n_units, "%s: item %d names unit %d", fn, i, u);
+    work[i].k_scale_max = scale_max[2 * u];
+    double v = (double)scale_max[2 * u + 1];
+    if (!(v == v)) v = 0.0;
+    v = std::min(std::max(v, 0.0), 1099511627776.0);     // 2^40 stands for infinity
+    int ex = 0;
+    frexp(v, &ex);                                         // v = m * 2^ex, 0.5 <= m < 1
+    work[i].v_shift = std::min(std::max(ex - 9, 0), 40);
+  }
   return RDKV_OK;
 }

@@ -197,8 +197,8 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
         # equal cost per group, or shares proportional to a relative speed by group index
         # (cost["group_speed"], cycled over the groups: workgroup i runs on compute die i mod 8)
         speed = np.asarray((model_used or {}).get("group_speed", (1.0,)), dtype=np.float64)
-        share = speed[np.arange(n_groups) % len(speed)]
-        thresholds = (float(cum[-1]) if total else 0.0) * np.cumsum(share / share.sum())[:-1]
+        share_cum = np.cumsum(speed[np.arange(n_groups) % len(speed)])
+        thresholds = (float(cum[-1]) if total else 0.0) * (share_cum[:-1] / share_cum[-1])
         group_cuts = np.searchsorted(cum, thresholds, side="left") + 1 if total else \
             np.zeros(n_groups - 1, dtype=np.int64)
         group_cuts = np.minimum(np.concatenate([[0], group_cuts, [total]]).astype(np.int64), total)
@@ -268,10 +268,10 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         plans.append((units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p))
         if entry_bytes is not None:
             entry_bytes.append((int(stream_bytes - sb0), int(algo_bytes - ab0)))
-    units_dev = torch.from_numpy(np.concatenate([pn[0] for pn in plans]).view(np.uint8).copy()).to(dev)
-    src_dev_all = torch.from_numpy(np.concatenate([pn[1] for pn in plans])).to(dev)
+    units_dev, src_dev_all = _lib.upload(dev, np.concatenate([pn[0] for pn in plans]), np.concatenate([pn[1] for pn in plans]))
+    sm_all = torch.zeros(len(plans), 2, max(pn[4] for pn in plans), dtype=torch.float32, device=dev)
     unit_row = src_row = 0
-    for (pl, nvo), (units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p) in zip(layers, plans):
+    for li, ((pl, nvo), (units, src_tab, off, max_tiles, H_kv, m8, n2p, n4p)) in enumerate(zip(layers, plans)):
         Dp = n2p + n4p + m8
         blob = torch.zeros(max(off, 256) + 256, dtype=torch.uint8, device=dev)   # + slack for 16-byte tail reads
         base = blob.data_ptr()
@@ -304,7 +304,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         # per head: the largest K channel scale and the largest V token scale (the kernel keeps its
         # fp16 operands in range with them)
         # (one reduction launch each, written straight into the entry's rows of one buffer)
-        sm = torch.zeros(2, H_kv, dtype=torch.float32, device=dev)
+        sm = sm_all[li, :, :H_kv]
         if Dp:
             torch.linalg.vector_norm(ks, ord=float("inf"), dim=1, dtype=torch.float32, out=sm[0])
         if vs.numel():
@@ -328,14 +328,14 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
         for name in ("k_off", "sz_off", "qtab_off"):
             units[name] += base
         units["v_off"] += base
-        units_all.extend(units)
+        units_all.append(units)
         blobs.append(blob)
         # the temporaries stay alive until the relayout kernels have run
         keep_alive.append((K2, K4, K8, V2, V4, V8, vs, vz, V16, ks, kz, perm))
-    scale_max_np = torch.stack(scale_max).transpose(1, 2).reshape(-1, 2).cpu().numpy().astype(np.float32)  # (synchronizes)
-    torch.cuda.current_stream(dev).synchronize()
+    sm_host = _lib.download(sm_all)                                     # (synchronizes)
+    scale_max_np = np.concatenate([sm_host[li, :, :pn[4]].T for li, pn in enumerate(plans)]).astype(np.float32)
     del keep_alive, units_dev, src_dev_all
-    return np.array(units_all, dtype=UNIT_DTYPE), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
+    return np.concatenate(units_all), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
 
 
 def _direct_packable(K: torch.Tensor, V: torch.Tensor) -> bool:
@@ -345,6 +345,20 @@ def _direct_packable(K: torch.Tensor, V: torch.Tensor) -> bool:
             and K.dtype == torch.float16 and V.dtype == torch.float16 and K.is_cuda and V.is_cuda
             and K.stride() == V.stride() and K.stride(3) == 1 and K.stride(2) % 8 == 0 and K.stride(1) % 8 == 0
             and K.data_ptr() % 16 == 0 and V.data_ptr() % 16 == 0)
+
+
+_pack_scratch_of: dict = {}
+
+
+def _pack_scratch(dev, stream: int, H_kv: int) -> torch.Tensor:
+    """The direct packer's scratch (min / max accumulators and channel quantizers of one layer's
+    heads), one per device, stream and head count: prepared when made, left ready by every call."""
+    key = (dev.index, stream, H_kv)
+    t = _pack_scratch_of.get(key)
+    if t is None:
+        t = _pack_scratch_of[key] = torch.empty(H_kv * 768, dtype=torch.float32, device=dev)
+        _lib.check(_lib.load().rdkv_pack_layer_stream_ws_init(t.data_ptr(), H_kv, stream))
+    return t
 
 
 def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_bytes: Optional[list] = None):
@@ -387,21 +401,33 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
         plans = []
         counts_a = np.asarray(counts_h, dtype=np.int32).reshape(-1, 4)
         chan_a = np.ascontiguousarray(np.asarray(info_h, dtype=np.int32).reshape(-1, 8)[:, 2:5])
+        tok_l, ch_l = counts_a.reshape(len(idx), H_kv, 4), chan_a.reshape(len(idx), H_kv, 3)
+        ch_max = ch_l.max(axis=1).tolist()
+        tv_max, n16_max = tok_l[:, :, :3].sum(axis=2).max(axis=1).tolist(), tok_l[:, :, 3].max(axis=1).tolist()
+        # the unit descriptors and slot tables of all entries in two arrays (one upload), a library call per entry
+        units_grp = np.zeros(len(idx) * H_kv, dtype=UNIT_DTYPE)
+        src_grp = np.empty((len(idx) * H_kv, 4 * MAX_STEPS), dtype=np.int16)
+        sizes_grp = np.zeros((len(idx), 4), dtype=np.int64)
+        n_live = 0
         for j, i in enumerate(idx):
-            tok, ch = counts_a[j * H_kv:(j + 1) * H_kv], chan_a[j * H_kv:(j + 1) * H_kv]
-            m2, m4, m8 = (int(x) for x in ch.max(axis=0))
-            max_tv, max_n16 = int(tok[:, :3].sum(axis=1).max()), int(tok[:, 3].max())
+            (m2, m4, m8), max_tv, max_n16 = ch_max[j], tv_max[j], n16_max[j]
             if max_tv + max_n16 == 0 or m2 + m4 + m8 == 0:
                 plans.append(None)               # degenerate: the two-step path knows the reference's behaviour
                 continue
             n2p, n4p = _seg_padded_len(m2, 4), _seg_padded_len(m4, 2)
-            units, src_tab, off, max_tiles, sb, ab = _plan_entry_units(tok, ch, n2p, n4p,
-                                                                       int(rows_of_entries[i]) * H_q, G)
-            plans.append((units, src_tab, off, max_tiles, sb, ab, n2p, n4p, m8, max_tv, max_n16))
+            r0 = n_live * H_kv
+            _lib.check(lib.rdkv_stream_plan_layer(
+                counts_a.ctypes.data + 16 * j * H_kv, 4, chan_a.ctypes.data + 12 * j * H_kv, 3, H_kv, n2p, n4p,
+                int(rows_of_entries[i]) * H_q, G, units_grp.ctypes.data + r0 * UNIT_DTYPE.itemsize,
+                src_grp.ctypes.data + r0 * 8 * MAX_STEPS, 4 * MAX_STEPS, sizes_grp.ctypes.data + 32 * n_live))
+            off, max_tiles, sb, ab = (int(x) for x in sizes_grp[n_live])
+            plans.append((units_grp[r0:r0 + H_kv], src_grp[r0:r0 + H_kv], off, max_tiles, sb, ab, n2p, n4p, m8,
+                          max_tv, max_n16))
+            n_live += 1
         live = [p for p in plans if p is not None]
         if live:
-            units_dev, src_dev = _lib.upload(dev, np.concatenate([p[0] for p in live]), np.concatenate([p[1] for p in live]))
-            mm_all = torch.empty(len(live), H_kv * 768, dtype=torch.float32, device=dev)   # min / max, channel quantizers
+            units_dev, src_dev = _lib.upload(dev, units_grp[:n_live * H_kv], src_grp[:n_live * H_kv])
+            mm = _pack_scratch(dev, stream, H_kv)
             sm_all = torch.empty(len(live), 2, H_kv, dtype=torch.float32, device=dev)
         row = 0
         for j, (i, p) in enumerate(zip(idx, plans)):
@@ -427,14 +453,14 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
                 kb_dev.element_size(), kb_dev.stride(0),
                 n2p, n4p, m8, max_tv, max_n16, units_dev.data_ptr() + row * UNIT_DTYPE.itemsize,
                 src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, base, blob_bytes,
-                mm_all.data_ptr() + 4 * k * mm_all.stride(0), sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
+                mm.data_ptr(), sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
             row += H_kv
             for name in ("k_off", "sz_off", "qtab_off"):
                 units[name] += base
             units["v_off"] += base
             pending.append((i, units, blob, sm_all[k], sb, ab, None))
         if live:
-            pending.append((None, None, None, None, 0, 0, (units_dev, src_dev, mm_all, sm_all, kb_dev, order, plan)))
+            pending.append((None, None, None, None, 0, 0, (units_dev, src_dev, sm_all, kb_dev, order, plan)))
     sm_dev = None
     if pending:
         sms = [pn[3] for pn in pending if pn[0] is not None]
@@ -499,73 +525,123 @@ def v_shift_of(v_scale_max: np.ndarray) -> np.ndarray:
     return np.clip(ex - 9, 0, 40).astype(np.int32)
 
 
+def _partition_units(units_np: np.ndarray, n_groups: int, cost: dict, multi_source: bool):
+    """``partition_work`` over the tiles of ``units_np`` with ``n_groups`` runs of equal cost, by the
+    library's host routine: a copy of the units with their item ranges, the work items (descriptor
+    copies and merge ranges filled) and the group offsets."""
+    units_np = np.ascontiguousarray(units_np).copy()
+    n_groups = max(1, n_groups)
+    U = len(units_np)
+    work_np = np.zeros(n_groups + 2 * U, dtype=WORK_DTYPE)
+    groups_np = np.zeros(n_groups + 1, dtype=np.int32)
+    tile = np.asarray(cost["tile"], dtype=np.float64)
+    speed = np.asarray(cost.get("group_speed", (1.0,)), dtype=np.float64)
+    n_work = np.zeros(1, dtype=np.int32)
+    _lib.check(_lib.load().rdkv_stream_partition(
+        units_np.ctypes.data, U, n_groups, tile.ctypes.data, float(cost["k_dword"]), float(cost["item"]),
+        speed.ctypes.data, len(speed), int(bool(multi_source)), work_np.ctypes.data, len(work_np),
+        groups_np.ctypes.data, n_work.ctypes.data))
+    return units_np, work_np[:int(n_work[0])], groups_np
+
+
 def _finish_cache(units_np: np.ndarray, blobs, G: int, H_q: int, stream_bytes: int, kv_algo_bytes: int,
                   scale_max: np.ndarray, *, multi_source: bool, work_bytes, n_groups, groups_per_cu: int,
                   cost) -> StreamCache:
     """Order the units, cut the tile stream into work items and groups, upload the tables.
     ``scale_max``: fp32 [n_units, 2], or a function returning it, called once everything that does
     not need it is done (the direct packer's launches are still running until then)."""
-    dev = blobs[0].device
-    n_groups_arg, cost_arg = n_groups, cost
-    order = None
-    if multi_source:
-        # sources of one output row next to each other, so that their work items are contiguous
-        order = np.argsort(units_np["q_row"], kind="stable")
-        units_np = units_np[order]
-    tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
-    R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
-    if work_bytes is None and n_groups is None:
-        # Every group costs a fixed amount (set-up, its partials, their merge), every tile a fixed
-        # amount per group that shares the stream: the step time a*tiles/n + b*n is least at
-        # n ~ sqrt(tiles); the factor is fitted to single-layer calls of 4k..128k tokens.  Large
-        # caches get one group per compute unit, tiny ones at least 4 tiles per group.
-        cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        total_tiles = int(tiles_np.sum())
-        n_groups = max(1, min(groups_per_cu * cus, int(round((6.0 * total_tiles) ** 0.5)), total_tiles // 4))
-    work_np, groups_np, wb, wc = partition_work(tiles_np, R_np,
-                                                n_groups=n_groups, work_bytes=work_bytes,
-                                                cost=cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS))
-    if multi_source:
-        # the first unit of every output row merges the partials of all its sources
-        qr = units_np["q_row"]
-        first = np.concatenate([[True], qr[1:] != qr[:-1]])
-        run_id = np.cumsum(first) - 1
-        wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
-    units_np = units_np.copy()
-    units_np["work_begin"], units_np["work_count"] = wb, wc
-    # every item knows the unit that merges its output row (the unit itself, or the row's first source)
-    if len(units_np):
-        merger = np.maximum.accumulate(np.where(wc > 0, np.arange(len(units_np)), 0)) if multi_source \
-            else np.arange(len(units_np))
-        iu = work_np["unit"]
-        # (the descriptor copies as bytes: assignment between record arrays goes field by field)
-        work_np.view(np.uint8).reshape(-1, WORK_DTYPE.itemsize)[:, 16:16 + UNIT_DTYPE.itemsize] = \
-            units_np.view(np.uint8).reshape(-1, UNIT_DTYPE.itemsize)[iu]
-        work_np["merge_unit"] = merger[iu]
-        work_np["merge_begin"] = wb[merger[iu]]
-        work_np["merge_count"] = wc[merger[iu]]
-    rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
-    if callable(scale_max):
-        scale_max = scale_max()
-    if order is not None:
-        scale_max = scale_max[order]
-    if len(units_np):
-        work_np["k_scale_max"] = scale_max[iu, 0]
-        work_np["v_shift"] = v_shift_of(scale_max[:, 1])[iu]
-    units_dev, work_dev, groups_dev = _lib.upload(
-        dev, units_np, work_np if len(work_np) else np.zeros(1, dtype=WORK_DTYPE),
-        groups_np if groups_np is not None else np.zeros(1, dtype=np.int32))
-    groups_dev = groups_dev.view(torch.int32) if groups_np is not None else None
-    return StreamCache(tickets=torch.zeros(max(1, len(units_np)), dtype=torch.int32, device=dev),
-                       partition={"work_bytes": work_bytes, "n_groups": n_groups_arg, "groups_per_cu": groups_per_cu,
-                                  "cost": cost_arg}, unit_scale_max=scale_max,
-                       blobs=list(blobs), units=units_dev, work=work_dev, units_host=units_np, work_host=work_np,
-                       n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
-                       stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
-                       max_row_dwords=int(R_np.max()) if len(R_np) else 0,
-                       groups=groups_dev, groups_host=groups_np,
-                       n_groups=0 if groups_np is None else len(groups_np) - 1,
-                       kv_algorithmic_bytes=int(kv_algo_bytes), multi_source=multi_source, h_q=int(H_q))
+    return _finish_caches([(units_np, blobs, G, H_q, stream_bytes, kv_algo_bytes, scale_max,
+                            dict(multi_source=multi_source, work_bytes=work_bytes, n_groups=n_groups,
+                                 groups_per_cu=groups_per_cu, cost=cost))])[0]
+
+
+_cus_of_device: dict = {}
+
+
+def _finish_caches(specs) -> List[StreamCache]:
+    """``_finish_cache`` for several caches on one device at once: the host side of all of them
+    first, then their unit and group tables in one queued copy, the largest scales (the one wait, when
+    they come from launches still running), the work tables in a second copy."""
+    dev = specs[0][1][0].device
+    if dev.index not in _cus_of_device:
+        _cus_of_device[dev.index] = torch.cuda.get_device_properties(dev).multi_processor_count
+    cus = _cus_of_device[dev.index]
+    plans = []
+    for units_np, blobs, G, H_q, stream_bytes, kv_algo_bytes, scale_max, opt in specs:
+        multi_source, work_bytes, n_groups, cost = opt["multi_source"], opt["work_bytes"], opt["n_groups"], opt["cost"]
+        order = None
+        if multi_source:
+            # sources of one output row next to each other, so that their work items are contiguous
+            order = np.argsort(units_np["q_row"], kind="stable")
+            units_np = units_np[order]
+        tiles_np = -(-units_np["n_tok"].astype(np.int64) // TILE)
+        R_np = (units_np["d8"] + units_np["d4"] + units_np["d2"]).astype(np.int64)
+        if work_bytes is None and n_groups is None:
+            # Every group costs a fixed amount (set-up, its partials, their merge), every tile a fixed
+            # amount per group that shares the stream: the step time a*tiles/n + b*n is least at
+            # n ~ sqrt(tiles); the factor is fitted to single-layer calls of 4k..128k tokens.  Large
+            # caches get one group per compute unit, tiny ones at least 4 tiles per group.
+            total_tiles = int(tiles_np.sum())
+            n_groups = max(1, min(opt["groups_per_cu"] * cus, int(round((6.0 * total_tiles) ** 0.5)), total_tiles // 4))
+        model = cost or (DEFAULT_COST if G <= 4 else DEFAULT_COST_TWO_HEAD_GROUPS)
+        if work_bytes is None:
+            units_np, work_np, groups_np = _partition_units(units_np, int(n_groups), model, multi_source)
+        else:
+            work_np, groups_np, wb, wc = partition_work(tiles_np, R_np, n_groups=n_groups, work_bytes=work_bytes,
+                                                        cost=model)
+            if multi_source:
+                # the first unit of every output row merges the partials of all its sources
+                qr = units_np["q_row"]
+                first = np.concatenate([[True], qr[1:] != qr[:-1]])
+                run_id = np.cumsum(first) - 1
+                wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
+            units_np = units_np.copy()
+            units_np["work_begin"], units_np["work_count"] = wb, wc
+            # every item knows the unit that merges its output row (the unit itself, or the row's first source)
+            if len(units_np):
+                merger = np.maximum.accumulate(np.where(wc > 0, np.arange(len(units_np)), 0)) if multi_source \
+                    else np.arange(len(units_np))
+                iu = work_np["unit"]
+                # (the descriptor copies as bytes: assignment between record arrays goes field by field)
+                work_np.view(np.uint8).reshape(-1, WORK_DTYPE.itemsize)[:, 16:16 + UNIT_DTYPE.itemsize] = \
+                    units_np.view(np.uint8).reshape(-1, UNIT_DTYPE.itemsize)[iu]
+                work_np["merge_unit"] = merger[iu]
+                work_np["merge_begin"] = wb[merger[iu]]
+                work_np["merge_count"] = wc[merger[iu]]
+        rows = (int(units_np["q_row"].max()) // H_q + 1) * H_q if len(units_np) else 0
+        plans.append((units_np, work_np, groups_np, order, rows, int(R_np.max()) if len(R_np) else 0))
+    tables = _lib.upload(dev, *[a for pl in plans for a in (pl[0], pl[2] if pl[2] is not None else np.zeros(1, dtype=np.int32))])
+    n_tickets = [max(1, len(pl[0])) for pl in plans]
+    tickets = torch.zeros(sum(n_tickets), dtype=torch.int32, device=dev)
+    ticket_at = np.concatenate([[0], np.cumsum(n_tickets)])
+    scales = []
+    for (units_np, work_np, groups_np, order, rows, r_max), spec in zip(plans, specs):
+        scale_max = spec[6]
+        if callable(scale_max):
+            scale_max = scale_max()
+        if order is not None:
+            scale_max = scale_max[order]
+        scale_max = np.ascontiguousarray(scale_max, dtype=np.float32)
+        if len(units_np):
+            _lib.check(_lib.load().rdkv_stream_work_scales(work_np.ctypes.data, len(work_np), scale_max.ctypes.data,
+                                                           len(units_np)))
+        scales.append(scale_max)
+    work_tables = _lib.upload(dev, *[pl[1] if len(pl[1]) else np.zeros(1, dtype=WORK_DTYPE) for pl in plans])
+    out = []
+    for k, ((units_np, work_np, groups_np, order, rows, r_max), spec) in enumerate(zip(plans, specs)):
+        _, blobs, G, H_q, stream_bytes, kv_algo_bytes, _, opt = spec
+        out.append(StreamCache(
+            tickets=tickets[int(ticket_at[k]):int(ticket_at[k + 1])],
+            partition={"work_bytes": opt["work_bytes"], "n_groups": opt["n_groups"], "groups_per_cu": opt["groups_per_cu"],
+                       "cost": opt["cost"]}, unit_scale_max=scales[k],
+            blobs=list(blobs), units=tables[2 * k], work=work_tables[k], units_host=units_np, work_host=work_np,
+            n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
+            stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
+            max_row_dwords=r_max,
+            groups=tables[2 * k + 1].view(torch.int32) if groups_np is not None else None, groups_host=groups_np,
+            n_groups=0 if groups_np is None else len(groups_np) - 1,
+            kv_algorithmic_bytes=int(kv_algo_bytes), multi_source=opt["multi_source"], h_q=int(H_q)))
+    return out
 
 
 def build_stream_cache(layers: Sequence[Tuple[PackedKVLayer, Optional[torch.Tensor]]], G: int, *,
@@ -632,19 +708,19 @@ def _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max) -> Li
     """caches[i] with entry i of a freshly laid run of entries (equal unit counts) as a further source."""
     G = caches[0].G
     n_per = len(new_units) // len(caches)
-    out = []
+    specs = []
     for i, cache in enumerate(caches):
         assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
-        units = np.concatenate([cache.units_host.copy(), new_units[i * n_per:(i + 1) * n_per]])
+        units = np.concatenate([cache.units_host, new_units[i * n_per:(i + 1) * n_per]])
+
         def scale_max(i=i, cache=cache):
             new = new_scale_max() if callable(new_scale_max) else new_scale_max
             return np.concatenate([cache.unit_scale_max, new[i * n_per:(i + 1) * n_per]])
 
-        out.append(_finish_cache(units, list(cache.blobs) + [new_blobs[i]], G, H_q, cache.stream_bytes + per_entry[i][0],
-                                 cache.kv_algorithmic_bytes + per_entry[i][1], scale_max,
-                                 multi_source=True, work_bytes=None,
-                                 n_groups=None, groups_per_cu=1, cost=None))
-    return out
+        specs.append((units, list(cache.blobs) + [new_blobs[i]], G, H_q, cache.stream_bytes + per_entry[i][0],
+                      cache.kv_algorithmic_bytes + per_entry[i][1], scale_max,
+                      dict(multi_source=True, work_bytes=None, n_groups=None, groups_per_cu=1, cost=None)))
+    return _finish_caches(specs)
 
 
 def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.Tensor] = None,

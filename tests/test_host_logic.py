@@ -261,6 +261,60 @@ def test_stream_plan_layer_matches_the_slot_plan_and_lays_sections_out_in_order(
         sc._plan_entry_units([(1, 0, 0, 0)], [(100, 100, 0)], 100, 100, 0, 1)
 
 
+def test_library_partition_matches_partition_work():
+    """The library's host-side work partition against ``partition_work`` and the merge bookkeeping
+    restated here, on random unit tables: empty units (leading, trailing, in runs), single-tile
+    units, more groups than tiles, multi-source rows; and the scale fields against ``v_shift_of``."""
+    from rdkv_amd import stream_cache as sc
+    rng = np.random.default_rng(5)
+    for case in range(60):
+        U = int(rng.integers(1, 40))
+        units = np.zeros(U, dtype=sc.UNIT_DTYPE)
+        units["n_tok"] = rng.choice([0, 0, 1, 64, 65, 300, 5000], size=(U, 4))
+        if case % 7 == 0:
+            units["n_tok"][rng.integers(0, U)] = 0
+            units["n_tok"][0 if case % 2 else U - 1] = 0
+        if case == 3:
+            units["n_tok"] = 0
+        units["d8"], units["d4"], units["d2"] = rng.integers(0, 12, U), rng.integers(0, 10, U), rng.integers(0, 8, U)
+        multi = case % 3 == 0
+        units["q_row"] = np.sort(rng.integers(0, max(1, U // 3), U)) * 8 if multi else np.arange(U) * 8
+        n_groups = int(rng.choice([1, 2, 7, 64, 256, 1000]))
+        cost = sc.DEFAULT_COST if case % 2 else sc.DEFAULT_COST_TWO_HEAD_GROUPS
+        got_units, got_work, got_groups = sc._partition_units(units, n_groups, cost, multi)
+        tiles = -(-units["n_tok"].astype(np.int64) // 64)
+        R = (units["d8"] + units["d4"] + units["d2"]).astype(np.int64)
+        work, groups, wb, wc = sc.partition_work(tiles, R, n_groups=n_groups, cost=cost)
+        assert len(got_work) == len(work) and np.array_equal(got_groups, groups)
+        for f in ("unit", "tile_begin", "tile_end"):
+            assert np.array_equal(got_work[f], work[f]), f
+        if multi:
+            qr = units["q_row"]
+            first = np.concatenate([[True], qr[1:] != qr[:-1]])
+            run_id = np.cumsum(first) - 1
+            wc = np.where(first, np.bincount(run_id, weights=wc).astype(np.int32)[run_id], 0).astype(np.int32)
+            merger = np.maximum.accumulate(np.where(first, np.arange(U), 0))
+        else:
+            merger = np.arange(U)
+        assert np.array_equal(got_units["work_begin"], wb) and np.array_equal(got_units["work_count"], wc)
+        iu = got_work["unit"]
+        assert np.array_equal(got_work["merge_unit"], merger[iu])
+        assert np.array_equal(got_work["merge_begin"], wb[merger[iu]])
+        assert np.array_equal(got_work["merge_count"], wc[merger[iu]])
+        assert got_work["u"].tobytes() == got_units[iu].tobytes()
+        # every tile of every unit is covered once, in order
+        for u in range(U):
+            mine = got_work[iu == u]
+            assert len(mine) >= 1 and int(mine["tile_begin"][0]) == 0 and int(mine["tile_end"][-1]) == int(tiles[u].sum())
+            assert np.array_equal(mine["tile_begin"][1:], mine["tile_end"][:-1])
+        sm = np.abs(rng.standard_normal((U, 2))).astype(np.float32) * rng.choice([1e-3, 1.0, 600.0, 1e6], size=(U, 2)).astype(np.float32)
+        sm[rng.integers(0, U), 1] = np.inf
+        sm[rng.integers(0, U), 1] = np.nan
+        _lib.check(_lib.load().rdkv_stream_work_scales(got_work.ctypes.data, len(got_work), sm.ctypes.data, U))
+        assert np.array_equal(got_work["k_scale_max"], sm[iu, 0], equal_nan=True)
+        assert np.array_equal(got_work["v_shift"], sc.v_shift_of(sm[:, 1])[iu])
+
+
 def test_selection_and_planning_entry_points_reject_bad_arguments():
     """Argument checks of the newer entry points run before any device work, so they can be
     exercised without a GPU: status code and message."""
