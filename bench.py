@@ -417,6 +417,26 @@ def pack_sample_section(pack_sample, pack_info, cfg, torch, dev, select_info=Non
         times.append((time.perf_counter() - t0) * 1e3)
     pack_info["relayout_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
     del packed
+    # the same layers from fp16 K / V straight into the streaming format (rdkv_pack_layer_stream):
+    # quantization and layout in one pass, the cache ready for the fused kernel
+    entries = [(p[0], p[1], p[2].to(dev), p[3].to(dev)) for p in pack_sample]
+    times = []
+    for _ in range(6):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        c = stream_cache.build_stream_cache_from_kv(entries, cfg.G)
+        torch.cuda.synchronize()
+        times.append((time.perf_counter() - t0) * 1e3)
+        del c
+    pack_info["pack_to_stream_ms_per_layer_batched"] = float(np.median(times[1:])) / len(pack_sample)
+    pack_info["pack_to_stream_GBps_of_fp16_input_batched"] = \
+        sample_bytes / (float(np.median(times[1:])) * 1e-3) / 1e9
+    pack_info["pack_then_relayout_ms_per_layer_batched"] = \
+        pack_info["pack_ms_per_layer_batched"] + pack_info["relayout_ms_per_layer_batched"]
+    pack_info["note_pack_to_stream"] = (
+        "pack_to_stream_*: stream_cache.build_stream_cache_from_kv over the sample layers (fp16 K / V and bit "
+        "allocations -> streaming cache, wall time incl. the work partition and table uploads, median of 5 after 1 "
+        "warm-up); pack_then_relayout_*: the two-step path it replaces (pack_layers_per_head, then build_stream_cache)")
     if select_info is not None:
         # selection + packing of the same layers in one call: the knapsack launches see
         # layers x heads rows at once instead of one layer's heads

@@ -238,7 +238,8 @@ def upload(dev: torch.device, *arrays) -> list:
             slot = s
             break
     if slot is None:
-        slot = [torch.empty(max(1 << 16, 1 << (total - 1).bit_length()), dtype=torch.uint8, pin_memory=True), None]
+        with torch.inference_mode(False):      # a kept buffer must stay writable outside the mode it was made in
+            slot = [torch.empty(max(1 << 16, 1 << (total - 1).bit_length()), dtype=torch.uint8, pin_memory=True), None]
         pool.append(slot)
     host = slot[0].numpy()
     for a, o in zip(arrays, offs):
@@ -262,7 +263,8 @@ def download(t: torch.Tensor):
     key = (t.device.index, threading.get_ident(), max(4096, 1 << (max(n, 1) - 1).bit_length()))
     buf = _pinned_reads.get(key)
     if buf is None:
-        buf = _pinned_reads[key] = torch.empty(key[2], dtype=torch.uint8, pin_memory=True)
+        with torch.inference_mode(False):      # a kept buffer must stay writable outside the mode it was made in
+            buf = _pinned_reads[key] = torch.empty(key[2], dtype=torch.uint8, pin_memory=True)
     flat = t.contiguous().reshape(-1).view(torch.uint8)
     buf[:n].copy_(flat, non_blocking=True)
     torch.cuda.current_stream(t.device).synchronize()

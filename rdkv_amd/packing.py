@@ -665,7 +665,8 @@ def _read_ints(t: Tensor, n: int) -> list:
     key = (t.device.index, max(1024, 1 << (n - 1).bit_length()), threading.get_ident())   # one buffer per host thread
     buf = _pinned_ints.get(key)
     if buf is None:
-        buf = _pinned_ints[key] = torch.empty(key[1], dtype=torch.int32, pin_memory=True)
+        with torch.inference_mode(False):      # a kept buffer must stay writable outside the mode it was made in
+            buf = _pinned_ints[key] = torch.empty(key[1], dtype=torch.int32, pin_memory=True)
     buf[:n].copy_(t[:n], non_blocking=True)
     torch.cuda.current_stream(t.device).synchronize()
     return buf[:n].tolist()

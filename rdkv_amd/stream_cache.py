@@ -335,7 +335,8 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
     sm_host = _lib.download(sm_all)                                     # (synchronizes)
     scale_max_np = np.concatenate([sm_host[li, :, :pn[4]].T for li, pn in enumerate(plans)]).astype(np.float32)
     del keep_alive, units_dev, src_dev_all
-    return np.concatenate(units_all), blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
+    units_np = np.concatenate([u.view(np.uint8) for u in units_all]).view(UNIT_DTYPE)
+    return units_np, blobs, int(stream_bytes), int(algo_bytes), H_q, scale_max_np
 
 
 def _direct_packable(K: torch.Tensor, V: torch.Tensor) -> bool:
@@ -532,8 +533,8 @@ def _partition_units(units_np: np.ndarray, n_groups: int, cost: dict, multi_sour
     units_np = np.ascontiguousarray(units_np).copy()
     n_groups = max(1, n_groups)
     U = len(units_np)
-    work_np = np.zeros(n_groups + 2 * U, dtype=WORK_DTYPE)
-    groups_np = np.zeros(n_groups + 1, dtype=np.int32)
+    work_np = np.empty(n_groups + 2 * U, dtype=WORK_DTYPE)       # (the routine writes every item it reports)
+    groups_np = np.empty(n_groups + 1, dtype=np.int32)
     tile = np.asarray(cost["tile"], dtype=np.float64)
     speed = np.asarray(cost.get("group_speed", (1.0,)), dtype=np.float64)
     n_work = np.zeros(1, dtype=np.int32)
@@ -711,7 +712,9 @@ def _extended(caches, new_units, new_blobs, per_entry, H_q, new_scale_max) -> Li
     specs = []
     for i, cache in enumerate(caches):
         assert H_q == cache.h_q, f"all sources of a cache share the head counts ({H_q} != {cache.h_q} query heads)"
-        units = np.concatenate([cache.units_host, new_units[i * n_per:(i + 1) * n_per]])
+        # (joined as bytes: concatenating record arrays goes field by field)
+        units = np.concatenate([np.ascontiguousarray(cache.units_host).view(np.uint8),
+                                np.ascontiguousarray(new_units[i * n_per:(i + 1) * n_per]).view(np.uint8)]).view(UNIT_DTYPE)
 
         def scale_max(i=i, cache=cache):
             new = new_scale_max() if callable(new_scale_max) else new_scale_max
