@@ -453,7 +453,8 @@ def _channel_score(queries: Tensor, keys: Tensor, *, num_kv_groups: int) -> Tens
 def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token_scores_by_layer: List[Tensor],
                     block_id: int, token_start: int, token_end: int, query_source_block: int,
                     is_final_flush: bool, causal: bool, config: BlockwiseRDKVConfig, num_kv_groups: int,
-                    model_dtype: torch.dtype) -> Tuple[CompressedDecodeBlock, Dict[str, Any]]:
+                    model_dtype: torch.dtype,
+                    kv_out: Optional[list] = None) -> Tuple[CompressedDecodeBlock, Dict[str, Any]]:
     """blockwise_decode.py:812-1121.  Per layer: ``target_kv[l]`` is ``[1, H_kv, T, 2*D]`` (keys then
     values along the last axis), ``query_block[l]`` ``[H_q, Q, D]`` the scoring queries and
     ``token_scores_by_layer[l]`` ``[H_kv, T]`` the V scores already accumulated for the block.
@@ -471,6 +472,8 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     fp16_denominator = 2 * h_kv * head_dim * 16
     keys = [kv[..., :head_dim].to(dtype=model_dtype) for kv in target_kv]
     values = [kv[..., head_dim:].to(dtype=model_dtype) for kv in target_kv]
+    if kv_out is not None:           # (the caller lays the block out for the fused kernel from the same rows)
+        kv_out.extend(zip(keys, values))
     select_kw = dict(gqa_factor=num_kv_groups, token_budget=config.block_budget_tokens,
                      k_budget_ratio=config.k_budget_ratio, obs_window=config.obs_window,
                      pool_kernel_size=config.pool_kernel_size, pool_padding=config.pool_padding, pool_type="avg",
@@ -594,7 +597,7 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
     of tokens)."""
     from .fast_decode import (_argmax_advance, _layer_stream_caches, _linear_row, _norm_linear_row, _rms_norm,
                               _silu_linear_row, pre_extract_weights)
-    from .stream_cache import decode_attn_fused, extend_stream_caches
+    from .stream_cache import decode_attn_fused, extend_stream_caches, extend_stream_caches_from_kv
 
     config.validate()
     lib = _lib.load()
@@ -670,14 +673,22 @@ def greedy_decode_blockwise(*, model, dual_cache: TriZoneCache, next_token_logit
         scores = [(s_self[:, :target_len] if causal else s_next[:, :target_len]).clone()
                   for s_self, s_next in zip(self_scores, next_scores)]
         block_id = len(compressed)
+        block_kv: list = []
         new_block, event = _compress_block(
             target_kv=target, query_block=queries, token_scores_by_layer=scores, block_id=block_id,
             token_start=pending_start, token_end=pending_start + target_len - 1,
             query_source_block=block_id if causal else block_id + 1, is_final_flush=is_final_flush, causal=causal,
-            config=config, num_kv_groups=groups, model_dtype=model_dtype)
+            config=config, num_kv_groups=groups, model_dtype=model_dtype, kv_out=block_kv)
         compressed.append(new_block)
         block_events.append(event)
-        caches[:] = extend_stream_caches(caches, list(zip(new_block.packed, new_block.new_v_only)))
+        if model_dtype == torch.float16 and not _fixed_slot_enabled():
+            # the block's rows and the allocator's decisions straight into the streaming format (the same
+            # bytes as re-laying the packed block, without reading it back)
+            caches[:] = extend_stream_caches_from_kv(
+                caches, [(k_l, v_l, p.allocation_v_bits, p.allocation_k_bits)
+                         for (k_l, v_l), p in zip(block_kv, new_block.packed)])
+        else:
+            caches[:] = extend_stream_caches(caches, list(zip(new_block.packed, new_block.new_v_only)))
         remain = pending_len - target_len
         for kv_buf, q_buf, s_self, s_next in zip(pending_kv, pending_q, self_scores, next_scores):
             if remain:

@@ -195,6 +195,392 @@ knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int g
        out_elem_size, counts ? counts + (int64_t)b * o.n : nullptr, lds);
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same solver with every row shared by several workgroups, for batches too small to fill the
+// device with one workgroup per row (one layer's eight heads of 32k tokens kept eight compute units
+// busy for ~60 dependent passes).  A row's S workgroups each own a contiguous chunk of it, held in
+// registers.  One pass evaluates up to 16 candidate lambdas at once - the next 15 doublings, or
+// lambda = 0 and the 15 midpoints four bisection levels can reach - as integer width sums of the
+// chunk.  The workgroups then exchange their sums: each stores its own as words that carry the
+// pass number in their top byte, and reads every workgroup's words until all of them carry it
+// (double-buffered by pass parity: a workgroup can be at most one pass ahead of another of its row).
+// So a pass costs one store and one load round trip between workgroups, no atomic operation meets
+// another on one address, and no ordinary memory changes hands (nothing to write back or
+// invalidate).  Every workgroup adds the same integers and takes the same decisions with the
+// arithmetic of the one-workgroup kernels.  The launch is sized so that all its workgroups are
+// resident together; a wait that does not end within a bound makes the workgroup give up and write
+// the invalid width 255 instead of hanging.
+// ---------------------------------------------------------------------------------------------
+constexpr int kCoopThreads = 256;
+constexpr int kCoopMaxSplit = 64;          // workgroups per row at most
+constexpr int kCoopWords = 16;             // words a workgroup publishes per pass
+constexpr int kCoopMaxIters = 64;          // passes stay below the 255 the tag byte can tell apart
+constexpr int kCoopSpinLimit = 1 << 20;
+constexpr uint32_t kCoopValueMask = 0xffffffu;
+#define RDKV_COOP_SCOPE __HIP_MEMORY_SCOPE_AGENT
+
+// per row: uint32 [2][kCoopMaxSplit][kCoopWords] exchange words, then 4 words for the row's group
+constexpr int kCoopRowWords = 2 * kCoopMaxSplit * kCoopWords + 4;
+
+struct CoopCtx {
+  int S, sub, t0, t1;
+  uint32_t* words;     // the row's exchange words
+  int pass;
+  int* tot;            // LDS, kCoopWords ints: the totals of the last exchange
+  int* failed;         // LDS flag
+};
+
+template <int SCOPE>
+__device__ __forceinline__ uint32_t coop_poll(const uint32_t* p, uint32_t tag, int* failed) {
+  uint32_t w = __hip_atomic_load(p, __ATOMIC_RELAXED, SCOPE);
+  int spins = 0;
+  while ((w >> 24) != tag) {
+    if (*failed || ++spins > kCoopSpinLimit) {
+      *failed = 1;
+      return 0u;
+    }
+    __builtin_amdgcn_s_sleep(1);
+    w = __hip_atomic_load(p, __ATOMIC_RELAXED, SCOPE);
+  }
+  return w & kCoopValueMask;
+}
+
+// Publishes this workgroup's n values (mine[i] in LDS, each below 2^24) and leaves in c.tot[i] their
+// sum over the row's workgroups (MAX: the maximum of the 32-bit numbers mine[0] << 16 | mine[1]
+// in c.tot[0]).
+template <bool MAX>
+__device__ void coop_exchange(CoopCtx& c, int n, const int* mine) {
+  const uint32_t tag = (uint32_t)(c.pass + 1);
+  uint32_t* buf = c.words + (c.pass & 1) * (kCoopMaxSplit * kCoopWords);
+  if ((int)threadIdx.x < n)
+    __hip_atomic_store(&buf[c.sub * kCoopWords + threadIdx.x], (tag << 24) | ((uint32_t)mine[threadIdx.x] & kCoopValueMask),
+                       __ATOMIC_RELAXED, RDKV_COOP_SCOPE);
+  if ((int)threadIdx.x < kCoopWords) c.tot[threadIdx.x] = 0;
+  __syncthreads();
+  if (MAX) {
+    for (int wg = threadIdx.x; wg < c.S; wg += blockDim.x) {
+      const uint32_t hi = coop_poll<RDKV_COOP_SCOPE>(&buf[wg * kCoopWords], tag, c.failed);
+      const uint32_t lo = coop_poll<RDKV_COOP_SCOPE>(&buf[wg * kCoopWords + 1], tag, c.failed);
+      atomicMax(reinterpret_cast<unsigned int*>(&c.tot[0]), (hi << 16) | lo);
+    }
+  } else {
+    // a thread's words (S * 16 <= 4 * 256) are requested together and asked for again until all carry the tag
+    constexpr int kPer = kCoopMaxSplit * kCoopWords / kCoopThreads;
+    const int i = threadIdx.x & (kCoopWords - 1);
+    uint32_t w[kPer];
+    bool want[kPer];
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) {
+      want[k] = i < n && (int)threadIdx.x + k * kCoopThreads < c.S * kCoopWords;
+      w[k] = tag << 24;
+    }
+    int spins = 0;
+    for (;;) {
+#pragma unroll
+      for (int k = 0; k < kPer; ++k)
+        if (want[k]) w[k] = __hip_atomic_load(&buf[threadIdx.x + k * kCoopThreads], __ATOMIC_RELAXED, RDKV_COOP_SCOPE);
+      bool ok = true;
+#pragma unroll
+      for (int k = 0; k < kPer; ++k) ok = ok && (w[k] >> 24) == tag;
+      if (ok) break;
+      if (*c.failed || ++spins > kCoopSpinLimit) {
+        *c.failed = 1;
+#pragma unroll
+        for (int k = 0; k < kPer; ++k) w[k] = 0u;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    int sum = 0;
+#pragma unroll
+    for (int k = 0; k < kPer; ++k) sum += want[k] ? (int)(w[k] & kCoopValueMask) : 0;
+    // lanes l, l ^ 16, l ^ 32 and l ^ 48 hold the same i
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    if ((threadIdx.x & 63) < kCoopWords && i < n) atomicAdd(&c.tot[i], sum);
+  }
+  __syncthreads();
+  ++c.pass;
+}
+
+// Width sums of this workgroup's chunk at n candidate lambdas (lam[0 .. n) in LDS), summed over the
+// workgroup into red[0 .. n) (LDS, zero on entry).  se[j][k] = held score j times eps[k], +inf for
+// the options past the last (their cost is never the smallest, so all eight are walked without a
+// branch); valid[j]: the thread has a j-th score.
+template <int HELD, int NOPT>
+__device__ void coop_chunk_sums_n(const float* __restrict__ row, const CoopCtx& c, const float (&se)[HELD][kMaxOptions],
+                                  const bool (&valid)[HELD], const float* lam, int n, const Options& o, int* red) {
+#pragma unroll 2
+  for (int i = 0; i < n; ++i) {
+    float lb[kMaxOptions];
+#pragma unroll
+    for (int k = 0; k < kMaxOptions; ++k) lb[k] = __fmul_rn(lam[i], o.bits[k]);
+    int acc = 0;
+#pragma unroll
+    for (int j = 0; j < HELD; ++j) {
+      float best = __fadd_rn(se[j][0], lb[0]);
+      int width = o.ibits[0];
+#pragma unroll
+      for (int k = 1; k < NOPT; ++k) {
+        const float cst = __fadd_rn(se[j][k], lb[k]);
+        const bool lt = cst < best;                                  // strict: the first minimum wins
+        best = lt ? cst : best;
+        width = lt ? o.ibits[k] : width;
+      }
+      acc += valid[j] ? width : 0;
+    }
+    for (int t = c.t0 + (int)threadIdx.x + HELD * (int)blockDim.x; t < c.t1; t += blockDim.x) {
+      int width;
+      choose(row[t], o, lb, width);
+      acc += width;
+    }
+    // the wavefront's sum without a trip through LDS per step: within rows of sixteen lanes by
+    // lane permutations, then the four row totals
+    acc += __builtin_amdgcn_update_dpp(0, acc, 0xB1, 0xF, 0xF, false);     // lane ^ 1
+    acc += __builtin_amdgcn_update_dpp(0, acc, 0x4E, 0xF, 0xF, false);     // lane ^ 2
+    acc += __builtin_amdgcn_update_dpp(0, acc, 0x141, 0xF, 0xF, false);    // mirror within eight
+    acc += __builtin_amdgcn_update_dpp(0, acc, 0x140, 0xF, 0xF, false);    // mirror within sixteen
+    const int total = __builtin_amdgcn_readlane(acc, 0) + __builtin_amdgcn_readlane(acc, 16) +
+                      __builtin_amdgcn_readlane(acc, 32) + __builtin_amdgcn_readlane(acc, 48);
+    if ((threadIdx.x & 63) == 0) atomicAdd(&red[i], total);
+  }
+  __syncthreads();
+}
+
+// (the options are walked to a compile-time count: the usual four or five, or all eight)
+template <int HELD>
+__device__ void coop_chunk_sums(const float* __restrict__ row, const CoopCtx& c, const float (&se)[HELD][kMaxOptions],
+                                const bool (&valid)[HELD], const float* lam, int n, const Options& o, int* red) {
+  if (o.n <= 4) coop_chunk_sums_n<HELD, 4>(row, c, se, valid, lam, n, o, red);
+  else if (o.n == 5) coop_chunk_sums_n<HELD, 5>(row, c, se, valid, lam, n, o, red);
+  else coop_chunk_sums_n<HELD, kMaxOptions>(row, c, se, valid, lam, n, o, red);
+}
+
+__global__ void coop_init_kernel(uint32_t* state, int64_t n_words) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_words) state[i] = 0u;
+}
+
+template <int HELD>
+__global__ void __launch_bounds__(kCoopThreads)
+knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int group_rows, int T, int S,
+                     const float* __restrict__ budget, Options o, int max_iters, float tol,
+                     uint32_t* __restrict__ state, void* __restrict__ out, int out_elem_size,
+                     int64_t out_stride_b, int* __restrict__ counts) {
+  __shared__ int lds[64];
+  __shared__ int red[kCoopWords];
+  __shared__ int tot[kCoopWords];
+  __shared__ float cand[kCoopWords + 1];   // the pass's candidate lambdas (and the next doubling base)
+  __shared__ int failed;
+  const int b = blockIdx.x / S;
+  CoopCtx c;
+  c.S = S; c.sub = blockIdx.x % S;
+  const int chunk = (T + S - 1) / S;
+  c.t0 = min(T, c.sub * chunk);
+  c.t1 = min(T, c.t0 + chunk);
+  c.words = state + (int64_t)b * kCoopRowWords;
+  c.pass = 0;
+  c.tot = tot;
+  c.failed = &failed;
+  if (threadIdx.x < kCoopWords) red[threadIdx.x] = 0;
+  if (threadIdx.x == 0) failed = 0;
+  const float* row = scores + (int64_t)b * stride_b;
+  const float bud = budget[b];
+  float se[HELD][kMaxOptions];
+  bool valid[HELD];
+  float m = -__builtin_inff();
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int t = c.t0 + (int)threadIdx.x + j * kCoopThreads;
+    valid[j] = t < c.t1;
+    const float v = valid[j] ? row[t] : 0.f;
+    if (valid[j]) m = fmaxf(m, v);
+#pragma unroll
+    for (int k = 0; k < kMaxOptions; ++k) se[j][k] = k < o.n ? __fmul_rn(v, o.eps[k]) : __builtin_inff();
+  }
+  for (int t = c.t0 + (int)threadIdx.x + HELD * kCoopThreads; t < c.t1; t += kCoopThreads) m = fmaxf(m, row[t]);
+  __syncthreads();
+
+  // ---- the row maximum
+  m = block_reduce(m, MaxF(), reinterpret_cast<float*>(lds));
+  if (threadIdx.x == 0) {
+    const uint32_t bits = rdkv_float_to_ordered(m);
+    red[0] = (int)(bits >> 16);
+    red[1] = (int)(bits & 0xffffu);
+  }
+  __syncthreads();
+  coop_exchange<true>(c, 2, red);
+  const float lam0 = fmaxf(__fmul_rn(rdkv_ordered_to_float((uint32_t)tot[0]), 0.375f), 1e-8f);
+  __syncthreads();
+  if (threadIdx.x < 2) red[threadIdx.x] = 0;
+
+  // ---- doublings the row asks for on its own: the first k with avg(lam0 * 2^k) <= budget
+  int d = -1;
+  {
+    float lam = lam0;
+    for (int base = 0; base < kMaxDoublings && d < 0; base += 15) {
+      const int n = min(15, kMaxDoublings - base);
+      if (threadIdx.x == 0) {
+        for (int i = 0; i < n; ++i) {
+          cand[i] = lam;
+          lam = __fmul_rn(lam, 2.0f);
+        }
+        cand[kCoopWords] = lam;
+      }
+      __syncthreads();
+      lam = cand[kCoopWords];
+      coop_chunk_sums<HELD>(row, c, se, valid, cand, n, o, red);
+      coop_exchange<false>(c, n, red);
+      if ((int)threadIdx.x < n) red[threadIdx.x] = 0;
+      for (int i = 0; i < n; ++i) {
+        const float avg = __fdiv_rn((float)tot[i], (float)T);
+        if (!(avg > bud)) {
+          d = base + i;
+          break;
+        }
+      }
+      __syncthreads();
+    }
+    if (d < 0) d = kMaxDoublings;
+  }
+  // ---- the rounds the row's group executes (as in knapsack_bisect_kernel): every row publishes
+  // its lam0 and doublings, every workgroup reads those of its group
+  const int r0 = (b / group_rows) * group_rows;
+  {
+    if (c.sub == 0 && threadIdx.x < 3) {
+      const uint32_t bits = __float_as_uint(lam0);
+      const uint32_t v = threadIdx.x == 0 ? bits >> 16 : (threadIdx.x == 1 ? bits & 0xffffu : (uint32_t)d);
+      __hip_atomic_store(&c.words[2 * kCoopMaxSplit * kCoopWords + threadIdx.x], (0xA5u << 24) | v, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);            // (the rows of a group sit on different dies)
+    }
+    int dmax = 0, gmax = 0;
+    for (int r = r0 + threadIdx.x; r < r0 + group_rows; r += blockDim.x) {
+      const uint32_t* gw = state + (int64_t)r * kCoopRowWords + 2 * kCoopMaxSplit * kCoopWords;
+      uint32_t w3[3] = {0u, 0u, 0u};
+      for (int spins = 0;; ++spins) {                      // the three words together, until all carry the tag
+#pragma unroll
+        for (int k = 0; k < 3; ++k) w3[k] = __hip_atomic_load(&gw[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((w3[0] >> 24) == 0xA5u && (w3[1] >> 24) == 0xA5u && (w3[2] >> 24) == 0xA5u) break;
+        if (failed || spins > kCoopSpinLimit) {
+          failed = 1;
+          w3[0] = w3[1] = w3[2] = 0u;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(1);
+      }
+      const uint32_t hi = w3[0] & kCoopValueMask, lo = w3[1] & kCoopValueMask;
+      const int dr = (int)(w3[2] & kCoopValueMask);
+      float lam = __uint_as_float((hi << 16) | lo);
+      int g = kMaxDoublings + 1;                     // never reaches 1e12
+      for (int it = 0; it < kMaxDoublings; ++it) {
+        if (it < dr) lam = __fmul_rn(lam, 2.0f);
+        if (lam >= 1e12f) { g = it; break; }
+      }
+      dmax = max(dmax, dr);
+      gmax = max(gmax, g);
+    }
+    dmax = block_reduce(dmax, MaxI(), lds);
+    gmax = block_reduce(gmax, MaxI(), lds);
+    __syncthreads();
+    const int rounds = min(min(dmax, gmax + 1), kMaxDoublings);
+    d = min(d, rounds);
+  }
+  float lam_hi = lam0;
+  for (int i = 0; i < d; ++i) lam_hi = __fmul_rn(lam_hi, 2.0f);
+
+  // ---- bisection, four levels per pass: node 1 is the midpoint of (lo, hi), node 2n that of the
+  // lower half of node n's interval, node 2n + 1 that of the upper half
+  float lam_lo = 0.f, lam_final = 0.f;
+  {
+    const float denom = fmaxf(bud, 1e-8f);
+    bool first = true, done = max_iters <= 0;
+    int it = 0;
+    // (with max_iters = 0 the reference still evaluates lambda = 0, but nothing depends on it)
+    while (!done) {
+      if (threadIdx.x == 0) {
+        float lo[16], hi[16];
+        lo[1] = lam_lo; hi[1] = lam_hi;
+        cand[0] = 0.f;   // lambda = 0 decides whether to bisect at all (first pass; unused afterwards)
+#pragma unroll
+        for (int n = 1; n < 16; ++n) {
+          const float mid = __fdiv_rn(__fadd_rn(lo[n], hi[n]), 2.0f);
+          cand[n] = mid;
+          if (2 * n < 16) {
+            lo[2 * n] = lo[n]; hi[2 * n] = mid;
+            lo[2 * n + 1] = mid; hi[2 * n + 1] = hi[n];
+          }
+        }
+      }
+      __syncthreads();
+      coop_chunk_sums<HELD>(row, c, se, valid, cand, 16, o, red);
+      coop_exchange<false>(c, 16, red);
+      if (threadIdx.x < kCoopWords) red[threadIdx.x] = 0;
+      if (first) {
+        first = false;
+        if (__fdiv_rn((float)tot[0], (float)T) <= bud) done = true;
+      }
+      int node = 1;
+      for (int lvl = 0; lvl < 4 && !done; ++lvl) {
+        const float mid = cand[node];
+        const float avg = __fdiv_rn((float)tot[node], (float)T);
+        lam_final = mid;
+        ++it;
+        const float rel = __fdiv_rn(fabsf(__fsub_rn(avg, bud)), denom);
+        if (rel < tol) {
+          done = true;
+        } else if (avg > bud) {
+          lam_lo = mid;
+          node = 2 * node + 1;
+        } else {
+          lam_hi = mid;
+          node = 2 * node;
+        }
+        if (it >= max_iters) done = true;
+      }
+      __syncthreads();                                // everyone has read the totals before the next pass rewrites them
+    }
+  }
+
+  // ---- the allocation of this workgroup's chunk and the per-option counts of the row
+  {
+    float lb[kMaxOptions];
+#pragma unroll
+    for (int n = 0; n < kMaxOptions; ++n) lb[n] = n < o.n ? __fmul_rn(lam_final, o.bits[n]) : 0.f;
+    int cnt[kMaxOptions];
+#pragma unroll
+    for (int n = 0; n < kMaxOptions; ++n) cnt[n] = 0;
+    uint8_t* out_row = reinterpret_cast<uint8_t*>(out) + (int64_t)b * out_stride_b * out_elem_size;
+    const bool bad = failed != 0;
+    for (int t = c.t0 + threadIdx.x; t < c.t1; t += blockDim.x) {
+      int w;
+      const int idx = choose(row[t], o, lb, w);
+      if (bad) w = 255;
+#pragma unroll
+      for (int n = 0; n < kMaxOptions; ++n) cnt[n] += (n == idx) ? 1 : 0;
+      if (out_elem_size == 1) out_row[t] = (uint8_t)w;
+      else reinterpret_cast<int64_t*>(out_row)[t] = (int64_t)w;
+    }
+    if (counts != nullptr) {
+#pragma unroll
+      for (int n = 0; n < kMaxOptions; ++n) {
+        if (n < o.n) {
+          int v = cnt[n];
+          v += __builtin_amdgcn_update_dpp(0, v, 0xB1, 0xF, 0xF, false);
+          v += __builtin_amdgcn_update_dpp(0, v, 0x4E, 0xF, 0xF, false);
+          v += __builtin_amdgcn_update_dpp(0, v, 0x141, 0xF, 0xF, false);
+          v += __builtin_amdgcn_update_dpp(0, v, 0x140, 0xF, 0xF, false);
+          const int total = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) +
+                            __builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48);
+          if ((threadIdx.x & 63) == 0) atomicAdd(&red[n], total);
+        }
+      }
+      __syncthreads();
+      coop_exchange<false>(c, o.n, red);
+      if (c.sub == 0 && (int)threadIdx.x < o.n) counts[(int64_t)b * o.n + threadIdx.x] = tot[threadIdx.x];
+    }
+  }
+}
+
 // Independent rows with lambda kept in double (the single-row solver applied to each row).
 __global__ void __launch_bounds__(kMaxThreads)
 knapsack_rows_kernel(const float* __restrict__ scores, int64_t stride_b, int T,
@@ -299,7 +685,35 @@ int check_common(const void* scores, int B, int64_t T, const void* budget, const
 
 }  // namespace
 
-RDKV_API int64_t rdkv_knapsack_workspace_bytes(int B) { return (int64_t)(B > 0 ? B : 0) * 8 + 256; }
+// Workgroups a row is shared by in the cooperative form (0: one workgroup per row, the two-launch
+// form): chunks of at least 512 scores, at most 64 per row, the whole launch on at most half of the
+// workgroup slots the device has for this kernel, and only when that gives a row at least sixteen
+// (with fewer, one workgroup per row was as fast or faster on 64 rows of 32k scores).
+static int coop_split(int B, int64_t T, int max_iters) {
+  if (B <= 0 || T < 4096 || max_iters > kCoopMaxIters) return 0;
+  static int slots_of_device[64];          // (0 = not asked yet; a race between first callers writes the same value)
+  int dev = 0, slots = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (slots_of_device[dev] == 0) {
+    int cus = 0, per_cu = 0;
+    const bool ok = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
+                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, knapsack_coop_kernel<8>, kCoopThreads, 0) == hipSuccess &&
+                    per_cu > 0;
+    slots_of_device[dev] = ok ? cus * per_cu : -1;
+  }
+  slots = slots_of_device[dev];
+  if (slots <= 0) return 0;
+  int64_t S = T / 512;
+  if (S > kCoopMaxSplit) S = kCoopMaxSplit;
+  if (S > slots / 2 / B) S = slots / 2 / B;
+  // (a chunk's width sum must fit the 24 value bits of an exchange word)
+  return S >= 16 && (T + S - 1) / S <= 32768 ? (int)S : 0;
+}
+
+RDKV_API int64_t rdkv_knapsack_workspace_bytes(int B) {
+  const int64_t b = B > 0 ? B : 0;
+  return b * 8 + 256 + b * (int64_t)kCoopRowWords * 4;
+}
 
 RDKV_API int rdkv_knapsack_batched(const float* scores, int64_t stride_b, int B, int64_t T,
                                    const float* budget, const float* bits_host, const float* eps_host,
@@ -321,6 +735,20 @@ RDKV_API int rdkv_knapsack_batched(const float* scores, int64_t stride_b, int B,
   float* lam0 = reinterpret_cast<float*>(workspace);
   int* doublings = reinterpret_cast<int*>(lam0 + B);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (const int S = coop_split(B, T, max_iters)) {
+    // few long rows: every row shared by S workgroups, one launch after clearing its state
+    uint8_t* base = reinterpret_cast<uint8_t*>(workspace) + (((int64_t)B * 8 + 255) / 256) * 256;
+    uint32_t* state = reinterpret_cast<uint32_t*>(base);
+    const int64_t n_words = (int64_t)B * kCoopRowWords;
+    hipLaunchKernelGGL(coop_init_kernel, dim3((unsigned)rdkv_cdiv(n_words, 256)), dim3(256), 0, s, state, n_words);
+    const int64_t chunk = (T + S - 1) / S;
+    auto kernel = chunk <= 2 * kCoopThreads ? knapsack_coop_kernel<2>
+                                            : (chunk <= 4 * kCoopThreads ? knapsack_coop_kernel<4> : knapsack_coop_kernel<8>);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(B * S)), dim3(kCoopThreads), 0, s, scores, stride_b, group_rows, (int)T, S,
+                       budget, o, max_iters, tol, state, out, out_elem_size, out_stride_b, counts);
+    RDKV_CHECK_LAUNCH("rdkv_knapsack_batched");
+    return RDKV_OK;
+  }
   const int threads = threads_for(T);
   hipLaunchKernelGGL(knapsack_expand_kernel, dim3(B), dim3(threads), 0, s, scores, stride_b, (int)T, budget, o,
                      lam0, doublings);

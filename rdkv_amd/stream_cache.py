@@ -224,6 +224,13 @@ def partition_work(unit_tiles: np.ndarray, unit_R: np.ndarray, *, n_groups: Opti
     return work, groups, work_begin, work_count
 
 
+def _add_base(units: np.ndarray, base: int) -> None:
+    """Turn the blob-relative offsets of contiguous unit descriptors into addresses: the seven offset
+    fields (k_off, v_off[4], sz_off, qtab_off) are the first 56 bytes of a record."""
+    assert UNIT_DTYPE.fields["qtab_off"][1] == 48
+    units.view(np.uint8).reshape(-1, UNIT_DTYPE.itemsize)[:, :56].view(np.uint64)[...] += np.uint64(base)
+
+
 def _plan_entry_units(tok, ch, n2p: int, n4p: int, first_row: int, G: int):
     """Host side of one entry (a packed layer): the unit descriptors of its heads with offsets
     relative to the entry's blob, the slot tables (stream slot -> position in the source layer's
@@ -325,9 +332,7 @@ def _relayout_entries(layers, G: int, rows_of_entries: Sequence[int], entry_byte
             rel_units_ptr, src_ptr, src_tab.shape[1], H_kv, m8, max_tiles, blob.data_ptr(),
             stream))
         # kernel-side descriptors carry absolute addresses
-        for name in ("k_off", "sz_off", "qtab_off"):
-            units[name] += base
-        units["v_off"] += base
+        _add_base(units, base)
         units_all.append(units)
         blobs.append(blob)
         # the temporaries stay alive until the relayout kernels have run
@@ -456,9 +461,7 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
                 src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, base, blob_bytes,
                 mm.data_ptr(), sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
             row += H_kv
-            for name in ("k_off", "sz_off", "qtab_off"):
-                units[name] += base
-            units["v_off"] += base
+            _add_base(units, base)
             pending.append((i, units, blob, sm_all[k], sb, ab, None))
         if live:
             pending.append((None, None, None, None, 0, 0, (units_dev, src_dev, sm_all, kb_dev, order, plan)))
@@ -526,6 +529,9 @@ def v_shift_of(v_scale_max: np.ndarray) -> np.ndarray:
     return np.clip(ex - 9, 0, 40).astype(np.int32)
 
 
+_cost_arrays: dict = {}      # id(cost model) -> (the model, its tile costs, its group speeds) as arrays
+
+
 def _partition_units(units_np: np.ndarray, n_groups: int, cost: dict, multi_source: bool):
     """``partition_work`` over the tiles of ``units_np`` with ``n_groups`` runs of equal cost, by the
     library's host routine: a copy of the units with their item ranges, the work items (descriptor
@@ -535,8 +541,11 @@ def _partition_units(units_np: np.ndarray, n_groups: int, cost: dict, multi_sour
     U = len(units_np)
     work_np = np.empty(n_groups + 2 * U, dtype=WORK_DTYPE)       # (the routine writes every item it reports)
     groups_np = np.empty(n_groups + 1, dtype=np.int32)
-    tile = np.asarray(cost["tile"], dtype=np.float64)
-    speed = np.asarray(cost.get("group_speed", (1.0,)), dtype=np.float64)
+    arrays = _cost_arrays.get(id(cost))
+    if arrays is None or arrays[0] is not cost:
+        arrays = _cost_arrays[id(cost)] = (cost, np.asarray(cost["tile"], dtype=np.float64),
+                                           np.asarray(cost.get("group_speed", (1.0,)), dtype=np.float64))
+    _, tile, speed = arrays
     n_work = np.zeros(1, dtype=np.int32)
     _lib.check(_lib.load().rdkv_stream_partition(
         units_np.ctypes.data, U, n_groups, tile.ctypes.data, float(cost["k_dword"]), float(cost["item"]),

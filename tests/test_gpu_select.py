@@ -86,6 +86,35 @@ def test_batched_knapsack_matches_oracle_on_seeded_rows(B, T, seed):
     np.testing.assert_array_equal(t2n(got), S.knapsack_bit_allocation_batched(s, budget, epsilon=S.DEFAULT_EPSILON_V))
 
 
+@pytest.mark.parametrize("max_iters,tol", [(64, 0.01), (64, 1e-9), (3, 0.01), (5, 1e-9), (1, 0.5), (0, 0.01)])
+def test_knapsack_long_rows_shared_by_workgroups(max_iters, tol):
+    """Few long rows (the solver's form with several workgroups per row): rows whose budget no
+    allocation meets double for all 40 rounds beside rows that need none, two groups of four rows
+    each ending their doubling rounds as a group, iteration limits that end inside a pass of four
+    levels and tolerances that never end one early; allocation and per-option counts against the
+    oracle."""
+    rng = np.random.default_rng(17)
+    B, T = 8, 8192
+    s = np.exp(rng.standard_normal((B, T)) * 1.7 + 1.0).astype(F32)
+    s[3] = np.round(s[3], 0)
+    s[6, 100:] = 0.0
+    budget = np.array([4.0, 1e-6, 0.7, 2.5, 15.9, 1e-6, 3.0, 9.0], dtype=F32)
+    exp = np.concatenate([S.knapsack_bit_allocation_batched(s[g:g + 4], budget[g:g + 4], epsilon=S.DEFAULT_EPSILON_V,
+                                                            max_iters=max_iters, tol=tol) for g in (0, 4)])
+    got, counts = ks.knapsack_allocate(to_dev(s), to_dev(budget), ks.DEFAULT_EPSILON_V, max_iters=max_iters, tol=tol,
+                                       with_counts=True, group_rows=4, out_dtype=torch.int64)
+    np.testing.assert_array_equal(t2n(got), exp)
+    options = sorted(ks.DEFAULT_EPSILON_V)
+    want_counts = np.stack([[int((exp[b] == o).sum()) for o in options] for b in range(B)])
+    assert sorted(t2n(counts).sum(axis=1).tolist()) == [T] * B
+    np.testing.assert_array_equal(np.sort(t2n(counts), axis=1), np.sort(want_counts, axis=1))
+    # the whole batch as one group gives every row what its own group of one call gives the oracle
+    one = ks.knapsack_allocate(to_dev(s), to_dev(budget), ks.DEFAULT_EPSILON_V, max_iters=max_iters, tol=tol,
+                               out_dtype=torch.int64)
+    np.testing.assert_array_equal(t2n(one), S.knapsack_bit_allocation_batched(s, budget, epsilon=S.DEFAULT_EPSILON_V,
+                                                                              max_iters=max_iters, tol=tol))
+
+
 def test_knapsack_edges():
     z = torch.zeros(0, 16, device=DEV)
     assert ks.knapsack_bit_allocation_batched(z, 2.0).shape == (0, 16)
