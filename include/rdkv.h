@@ -578,7 +578,12 @@ int rdkv_pool_scores(const float *scores, int64_t stride_b, int B, int64_t T, in
  * or device [B, n_options] int32, tokens per option.  T <= 2^20 (the width sums stay exact).
  * group_rows: the doubling rounds end together for every group_rows consecutive rows (what
  * was one call of the reference; 0 = the whole batch), so many calls can share one launch.
- * workspace: rdkv_knapsack_workspace_bytes(B) bytes.  Two launches, no host synchronization. */
+ * workspace: rdkv_knapsack_workspace_bytes(B) bytes.  Two launches, no host synchronization.
+ * Batches of few long rows (T >= 8192, max_iters <= 64, so few rows that each can have 16 or
+ * more resident workgroups) run with every row shared by up to 64 workgroups that exchange
+ * integer width sums once per pass of 15 doublings or four bisection levels; the same bits.  The
+ * workgroups wait for each other with a bound: should a wait not end (it cannot while the launch
+ * is resident as sized), the row's output is the invalid width 255 instead of a hang. */
 int64_t rdkv_knapsack_workspace_bytes(int B);
 int rdkv_knapsack_batched(const float *scores, int64_t stride_b, int B, int64_t T,
                           const float *budget, const float *bits_host, const float *eps_host,
