@@ -630,7 +630,12 @@ int rdkv_block_score(const void *queries, int q_dtype, int64_t q_stride_h, int64
 int rdkv_token_mass(const void *x, int dtype, int64_t stride_h, int64_t stride_i, int H, int n_inner,
                     int64_t T, float *out, void *stream);
 
-/* ---- measurement helpers (no counterpart in the reference) --------------------------------
+/* ==== MEASUREMENT ONLY: everything from here to the end of the header ========================
+ * The rdkv_probe_* entry points are not part of the drop-in boundary: no reference interface
+ * corresponds to them, no product path calls them, and a binding of the library for RDKV need not
+ * declare them.  bench.py uses them to calibrate counters, to find the device's read ceiling and
+ * to price the packed path against an uncompressed cache.
+ *
  * Plain kernels of known size used by the benchmark: a 16-byte-per-lane copy (bytes read and
  * bytes written = `bytes`; hardware traffic counters are scaled by what they report for it)
  * and a read-only sweep in contiguous spans of span_bytes per workgroup (sink: >= 1 KiB),
