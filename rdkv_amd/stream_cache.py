@@ -401,8 +401,17 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
             out[i] = (u, b[0], per[0][0], per[0][1], sm)
             continue
         H_kv, T = key
-        vb_all = torch.cat([entries[i][2].reshape(H_kv, T) for i in idx]) if len(idx) > 1 else entries[idx[0]][2]
-        kb_all = torch.cat([entries[i][3].reshape(H_kv, 128) for i in idx]) if len(idx) > 1 else entries[idx[0]][3]
+        def joined(which: int, width: int):
+            """The group's allocations as one tensor (on the device, in one integer type when they differ)."""
+            ts = [entries[i][which].reshape(H_kv, width) for i in idx]
+            if len(ts) == 1:
+                return ts[0]
+            ts = [t if t.device == dev else t.to(dev) for t in ts]
+            if any(t.dtype != ts[0].dtype for t in ts) or ts[0].is_floating_point():
+                ts = [t.to(torch.int16) for t in ts]
+            return torch.cat(ts)
+
+        vb_all, kb_all = joined(2, T), joined(3, 128)
         order, _, plan, counts_h, info_h, kb_dev = packing._plan_layers(vb_all.reshape(-1, T), kb_all.reshape(-1, 128), dev)
         plans = []
         counts_a = np.asarray(counts_h, dtype=np.int32).reshape(-1, 4)
@@ -468,7 +477,9 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
     sm_dev = None
     if pending:
         sms = [pn[3] for pn in pending if pn[0] is not None]
-        sm_dev = torch.stack(sms).transpose(1, 2) if sms else None
+        # (entries of different head counts are possible: one flat buffer, cut by entry below)
+        sm_dev = torch.cat([t.reshape(-1) for t in sms]) if sms else None
+        sm_heads = [int(t.shape[1]) for t in sms]
         k = 0
         for i, units, blob, _, sb, ab, _ in pending:
             if i is not None:
@@ -484,7 +495,13 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
         """The units' largest K channel and V token scales, read back from the launches above (the
         one synchronization of the direct path; callers do their host work first)."""
         if not resolved:
-            sm_host = _lib.download(sm_dev) if sm_dev is not None else None   # (synchronizes)
+            sm_host = []
+            if sm_dev is not None:
+                flat = _lib.download(sm_dev)                                  # (synchronizes)
+                at = 0
+                for hk in sm_heads:
+                    sm_host.append(flat[at:at + 2 * hk].reshape(2, hk).T)
+                    at += 2 * hk
             del pending[:]
             parts = [sm_host[o[4]].reshape(-1, 2) if isinstance(o[4], int) else o[4] for o in out]
             resolved.append(np.concatenate(parts).astype(np.float32))

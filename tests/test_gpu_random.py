@@ -576,6 +576,70 @@ def test_stream_caches_random_sources_partitions_files(block, tmp_path):
                                      f"{what}, one more source in group {row}")
 
 
+@pytest.mark.parametrize("block", range(3))
+def test_direct_stream_packer_random_layers(block, monkeypatch):
+    """40 calls per block of the packer that writes the streaming format directly, each over 1-4
+    random layers (lengths may differ inside a call; allocations on the device or on
+    the host, in several integer types; classes missing, heads that keep nothing, constant rows,
+    offsets, three magnitudes): the same unit descriptors, largest scales and blob bytes as packing
+    every layer and re-laying it, on blobs that start as 0xAB bytes; every fourth call also extends
+    per-layer caches by the layers as further sources, both ways."""
+    monkeypatch.setattr(stream_cache, "_POISON_BLOBS", True)
+    from tests.test_gpu_stream import _assert_same_cache
+    widths = np.array([0, 2, 4, 8, 16])
+    for case in range(40):
+        rng = np.random.default_rng(9100 + 100 * block + case)
+        G = int(rng.choice([1, 2, 4, 8]))
+        same_shape = rng.random() < 0.5
+        H0 = int(rng.integers(1, 6))
+        T0 = int(rng.choice([1, 3, 63, 64, 65, 129, 300, 700, 1500, 2500]))
+        entries = []
+        for _ in range(int(rng.integers(1, 5))):
+            H = H0                                   # (the entries of a cache share their head counts)
+            T = T0 if same_shape else int(rng.choice([1, 3, 63, 64, 65, 129, 300, 700, 1500, 2500]))
+            vb = torch.from_numpy(rng.choice(widths, size=(H, T), p=_class_probabilities(rng, 5)))
+            if rng.random() < 0.3:
+                vb[int(rng.integers(0, H))] = int(rng.choice(widths))
+            kb = torch.from_numpy(rng.choice(widths, size=(H, 128), p=_class_probabilities(rng, 5)))
+            scale = float(rng.choice([1.0, 0.01, 30.0]))
+            K = (torch.randn(1, H, T, 128, device=DEV) * scale + float(rng.choice([0.0, 0.75, -2.0]))).half()
+            V = (torch.randn(1, H, T, 128, device=DEV) * scale).half()
+            if rng.random() < 0.2:
+                V[0, 0, : max(1, T // 3)] = 0.5
+            if rng.random() < 0.2:
+                K[0, :, :, int(rng.integers(0, 128))] = -1.25
+            dt = [torch.int64, torch.int32, torch.int16, torch.uint8][int(rng.integers(0, 4))]
+            vb, kb = vb.to(dt), kb.to(dt)
+            if rng.random() < 0.5:
+                vb, kb = vb.to(DEV), kb.to(DEV)
+            entries.append((K, V, vb, kb))
+        what = f"block {block} case {case}: G={G}, shapes {[tuple(e[0].shape[1:3]) for e in entries]}"
+        try:
+            packed = [packing.pack_layer_per_head(K, V, vb, kb, G) for K, V, vb, kb in entries]
+        except (AssertionError, ValueError, IndexError):            # a layout the packer refuses: so must the direct one
+            with pytest.raises((AssertionError, ValueError, IndexError)):
+                stream_cache.build_stream_cache_from_kv(entries, G)
+            continue
+        try:
+            _assert_same_cache(stream_cache.build_stream_cache_from_kv(entries, G),
+                               stream_cache.build_stream_cache(packed, G))
+        except AssertionError as e:
+            raise AssertionError(f"{what}: {e}") from e
+        if case % 4 == 0 and same_shape:
+            base = [stream_cache.build_stream_cache([pl], G) for pl in packed]
+            a = stream_cache.extend_stream_caches_from_kv(base, entries)
+            b = stream_cache.extend_stream_caches(base, packed)
+            for x, y in zip(a, b):
+                try:
+                    _assert_same_cache(x, y)
+                except AssertionError as e:
+                    raise AssertionError(f"{what} (extension): {e}") from e
+                assert np.array_equal(x.groups_host, y.groups_host)
+                for f in ("unit", "tile_begin", "tile_end", "merge_unit", "merge_begin", "merge_count", "k_scale_max",
+                          "v_shift"):
+                    assert np.array_equal(x.work_host[f], y.work_host[f]), f
+
+
 def test_reference_layout_entry_points_shared_layout_and_views():
     """120 layers of the shared layout (build_packed_layer: one V allocation for all heads, K
     allocation shared or per head; 3-D or 4-D tensors) through k_mixed_qk_dot[_into] and
