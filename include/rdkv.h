@@ -376,8 +376,10 @@ int rdkv_stream_relayout_layer(const uint8_t *K2, int64_t k2_stride_h, int64_t k
  * max_tiles: as for rdkv_stream_relayout_layer.  blob_bytes: size of the blob (a multiple of 4, at
  * least sizes[0] of rdkv_stream_plan_layer): the launches write every byte of it, so it need not be
  * cleared.  minmax_ws: H_kv * 768 floats of scratch, 16-byte aligned (min / max accumulators, then
- * the quantizer of every channel), prepared once by rdkv_pack_layer_stream_ws_init: every call
- * leaves the accumulators at their start values again, so calls on one stream can share it.
+ * the quantizer of every channel).  minmax_ws_ready = 0: the call starts the accumulators itself (one
+ * more small launch); != 0: they already hold their start values - after
+ * rdkv_pack_layer_stream_ws_init, and after every earlier call on the same stream, which leaves them
+ * at their start values again - so a scratch that is kept needs preparing once.
  * scale_max: float [2][H_kv]: receives per head the largest K channel scale and the largest V token
  * scale (as the fp16 values stored), which RdkvWork.k_scale_max / v_shift are made from.  K and V
  * rows must be 16-byte aligned (RDKV_EUNSUPPORTED otherwise). */
@@ -387,7 +389,7 @@ int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_
                            const void *k_bits, int kb_elem_size, int64_t kb_stride_h, int n2p, int n4p, int n8,
                            int64_t max_tv, int max_n16, const RdkvUnit *units, const int16_t *src_slot,
                            int n_slots_max, int max_tiles, uint8_t *blob, int64_t blob_bytes, float *minmax_ws,
-                           float *scale_max, void *stream);
+                           int minmax_ws_ready, float *scale_max, void *stream);
 
 /* Fused decode attention over n_work work items.  q: [rows,128] of q_dtype; out: fp32
  * [rows,128]; lse: fp32 [rows] natural-log sum-exp of the scaled scores (-inf for a unit

@@ -64,7 +64,7 @@ SIGNATURES = {
     "rdkv_stream_partition": (I, [P, I, I, P, ctypes.c_double, ctypes.c_double, P, I, I, P, I, P, P]),
     "rdkv_stream_work_scales": (I, [P, I, P, I]),
     "rdkv_pack_layer_stream_ws_init": (I, [P, I, P]),
-    "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, L, P, P, P]),
+    "rdkv_pack_layer_stream": (I, [P, P, L, L, I, P, L, P, P, I, L, I, I, I, L, I, P, P, I, I, P, L, P, I, P, P]),
     "rdkv_stream_relayout_layer": (I, [P, L, L, P, L, L, P, L, L, I, I, P, L, P, L, P, L, P, P, L, P, L, L,
                                        P, L, P, P, L, P, P, I, I, I, I, P, P]),
     "rdkv_decode_fused_workspace_bytes": (L, [I, I]),

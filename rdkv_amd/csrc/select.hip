@@ -699,7 +699,8 @@ static int coop_split(int B, int64_t T, int max_iters) {
     const bool ok = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
                     hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, knapsack_coop_kernel<8>, kCoopThreads, 0) == hipSuccess &&
                     per_cu > 0;
-    slots_of_device[dev] = ok ? cus * per_cu : -1;
+    if (!ok) return 0;                     // (asked again next time: the query can fail while a stream is being captured)
+    slots_of_device[dev] = cus * per_cu;
   }
   slots = slots_of_device[dev];
   if (slots <= 0) return 0;

@@ -498,7 +498,7 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
                                     int64_t kb_stride_h, int n2p, int n4p, int n8, int64_t max_tv, int max_n16,
                                     const RdkvUnit *units, const int16_t *src_slot, int n_slots_max,
                                     int max_tiles, uint8_t *blob, int64_t blob_bytes, float *minmax_ws,
-                                    float *scale_max, void *stream) {
+                                    int minmax_ws_ready, float *scale_max, void *stream) {
   // (minmax_ws holds the min / max accumulators, H_kv * 256 floats, then the channel parameters,
   // H_kv * 128 * 4 floats)
   const char *fn = "rdkv_pack_layer_stream";
@@ -521,7 +521,7 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
   const int64_t max_tk = max_tv + max_n16;
   // per-channel min / max of every head's kept rows (the K canvas without its zero rows)
   int rc = rdkv_layer_k_minmax(fn, K_f16, stride_h, stride_t, H_kv, kD, order, order_stride_h, counts, max_tk,
-                               minmax_ws, /*init=*/false, s);
+                               minmax_ws, /*init=*/minmax_ws_ready == 0, s);
   if (rc != RDKV_OK) return rc;
   StreamPackArgs a;
   a.K = (const __half *)K_f16; a.V = (const __half *)V_f16;
@@ -548,9 +548,9 @@ RDKV_API int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_
         const bool ok = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
                         hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, stream_pack_kernel, 256, 0) == hipSuccess &&
                         per_cu > 0;
-        resident_of_device[dev] = ok ? cus * per_cu : 512;
+        if (ok) resident_of_device[dev] = cus * per_cu;   // (otherwise asked again next time)
       }
-      resident = resident_of_device[dev];
+      if (resident_of_device[dev] > 0) resident = resident_of_device[dev];
     }
     const int target = (resident + H_kv - 1) / H_kv;
     const int per = (max_tiles + target - 1) / target;

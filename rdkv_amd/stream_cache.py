@@ -354,6 +354,7 @@ def _direct_packable(K: torch.Tensor, V: torch.Tensor) -> bool:
 
 
 _pack_scratch_of: dict = {}
+_SCRATCH_PREPARED = 1        # what the packer is told about its scratch (tests hand it an unprepared one)
 
 
 def _pack_scratch(dev, stream: int, H_kv: int) -> torch.Tensor:
@@ -468,7 +469,7 @@ def _pack_entries_direct(entries, G: int, rows_of_entries: Sequence[int], entry_
                 kb_dev.element_size(), kb_dev.stride(0),
                 n2p, n4p, m8, max_tv, max_n16, units_dev.data_ptr() + row * UNIT_DTYPE.itemsize,
                 src_dev.data_ptr() + row * src_tab.shape[1] * 2, src_tab.shape[1], max_tiles, base, blob_bytes,
-                mm.data_ptr(), sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
+                mm.data_ptr(), _SCRATCH_PREPARED, sm_all.data_ptr() + 4 * k * sm_all.stride(0), stream))
             row += H_kv
             _add_base(units, base)
             pending.append((i, units, blob, sm_all[k], sb, ab, None))

@@ -190,6 +190,25 @@ def test_direct_stream_packer_ragged_and_degenerate_entries(poisoned_blobs):
     run(K, V, torch.from_numpy(rng.choice(choices, size=(H, T))), kb0)
 
 
+def test_direct_stream_packer_prepares_an_unprepared_scratch(monkeypatch, poisoned_blobs):
+    """Told that its scratch is not prepared, the packer starts the min / max accumulators itself:
+    the same cache from a scratch full of ones as from the kept, prepared one - and the call leaves
+    the scratch prepared (a second call that is told so gives the same bytes again)."""
+    cfg = synth.scaled(synth.CONFIGS[1], context=900, layers=2)
+    entries = []
+    for layer in range(2):
+        vb, kb, oc = synth.layer_allocation(cfg, layer)
+        K, V, _ = synth.layer_data(cfg, layer, DEV, outliers=oc)
+        entries.append((K, V, vb.to(DEV), kb.to(DEV)))
+    want = stream_cache.build_stream_cache_from_kv(entries, cfg.G)
+    dirty = torch.ones(cfg.H_kv * 768, dtype=torch.float32, device=DEV)
+    monkeypatch.setattr(stream_cache, "_pack_scratch", lambda dev, stream, H_kv: dirty)
+    monkeypatch.setattr(stream_cache, "_SCRATCH_PREPARED", 0)
+    _assert_same_cache(stream_cache.build_stream_cache_from_kv(entries, cfg.G), want)
+    monkeypatch.setattr(stream_cache, "_SCRATCH_PREPARED", 1)
+    _assert_same_cache(stream_cache.build_stream_cache_from_kv(entries, cfg.G), want)
+
+
 @pytest.mark.parametrize("name", ["perhead_d128_a", "perhead_d128_b", "shared_layout"])
 def test_fused_attention_golden(name):
     g = load_golden(name)
