@@ -130,8 +130,12 @@ def cache_physical_bytes(cache: TriZoneCache) -> int:
     return _tensor_storage_bytes((cache.packed, cache.new_v_only))
 
 
+def _bit_histogram_tensor(bits: Tensor) -> Tensor:
+    return torch.stack([(bits.detach() == b).sum() for b in (0, 2, 4, 8, 16)])
+
+
 def _bit_histogram(bits: Tensor) -> Dict[str, int]:
-    counts = torch.stack([(bits.detach() == b).sum() for b in (0, 2, 4, 8, 16)]).cpu().tolist()
+    counts = _bit_histogram_tensor(bits).cpu().tolist()
     return {str(b): int(c) for b, c in zip((0, 2, 4, 8, 16), counts)}
 
 
@@ -340,6 +344,22 @@ def _logical_layer_bits_tensor(packed, head_dim: int) -> Tensor:
     return v_bits.to(torch.int64).sum() * int(head_dim) + (k_bits.to(torch.int64).sum(dim=1) * kept).sum()
 
 
+def _logical_bits_of_layers(packed_layers, head_dim: int) -> Tensor:
+    """``_logical_layer_bits_tensor`` of every layer as one int64 vector; layers whose allocation
+    tables have one shape share their launches."""
+    v_all = [p.allocation_v_bits for p in packed_layers]
+    k_all = [p.allocation_k_bits for p in packed_layers]
+    if any(v is None or k is None for v, k in zip(v_all, k_all)):
+        raise RuntimeError("packed block is missing allocator decisions")
+    if not all(v.shape == v_all[0].shape and v.device == v_all[0].device and v.dim() == 2 for v in v_all) or \
+            not all(k.shape == k_all[0].shape and k.device == k_all[0].device and k.dim() == 2 for k in k_all):
+        return torch.stack([_logical_layer_bits_tensor(p, head_dim) for p in packed_layers])
+    v = torch.stack(v_all).to(torch.int64)                # [L, H_kv, T]
+    k = torch.stack(k_all).to(torch.int64)                # [L, H_kv, D]
+    kept = (v > 0).sum(dim=2)
+    return v.sum(dim=(1, 2)) * int(head_dim) + (k.sum(dim=2) * kept).sum(dim=1)
+
+
 def _logical_layer_bits(packed, head_dim: int) -> int:
     return int(_logical_layer_bits_tensor(packed, head_dim).item())
 
@@ -506,7 +526,7 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
             for value in (packed.K_ch_scale, packed.K_ch_zp, packed.V_scale, packed.V_zp, new_v_only):
                 if value is not None and value.is_floating_point() and not torch.isfinite(value).all():
                     raise FloatingPointError(f"non-finite packed metadata in layer {layer_idx}")
-    logical_dev = torch.stack([_logical_layer_bits_tensor(p, head_dim) for p in packed_layers])
+    logical_dev = _logical_bits_of_layers(packed_layers, head_dim)
     all_v = torch.cat([p.allocation_v_bits.reshape(-1) for p in packed_layers])
     all_k = torch.cat([p.allocation_k_bits.reshape(-1) for p in packed_layers])
     if _fixed_slot_enabled():
@@ -531,9 +551,14 @@ def _compress_block(*, target_kv: List[Tensor], query_block: List[Tensor], token
     t_end = _sync_stamp(target_kv[0].device)
     if timing_on:
         phase["metadata_update_ms"] = (t_end - t_meta) * 1000.0
-    logical_bits = [int(v) for v in logical_dev.cpu().tolist()]
+    # one host read for the accounting: per-layer bits, then the two histograms
+    accounting = torch.cat([logical_dev.to(torch.int64), _bit_histogram_tensor(all_v).to(torch.int64),
+                            _bit_histogram_tensor(all_k).to(torch.int64)]).cpu().tolist()
+    n_l = len(packed_layers)
+    logical_bits = [int(v) for v in accounting[:n_l]]
     equivalents = [v / fp16_denominator for v in logical_bits]
-    v_hist, k_hist = _bit_histogram(all_v), _bit_histogram(all_k)
+    v_hist = {str(b): int(c) for b, c in zip((0, 2, 4, 8, 16), accounting[n_l:n_l + 5])}
+    k_hist = {str(b): int(c) for b, c in zip((0, 2, 4, 8, 16), accounting[n_l + 5:n_l + 10])}
     block = CompressedDecodeBlock(
         block_id=block_id, token_start=token_start, token_end=token_end, packed=packed_tuple, squeezed=squeezed,
         new_v_only=v16_layers, logical_bits_per_layer=logical_bits, fp16_equivalent_tokens_per_layer=equivalents,

@@ -67,6 +67,26 @@ def test_raw_bit_accounting_uses_kept_v_positions_for_k():
 
     with pytest.raises(RuntimeError):
         bw._logical_layer_bits(Missing(), 2)
+    with pytest.raises(RuntimeError):
+        bw._logical_bits_of_layers([Allocation(), Missing()], 2)
+
+
+def test_raw_bit_accounting_of_a_block_matches_the_layers_one_by_one():
+    gen = torch.Generator().manual_seed(5)
+    widths = torch.tensor([0, 2, 4, 8, 16])
+
+    def layer(h, t, d):
+        class Allocation:
+            allocation_v_bits = widths[torch.randint(0, 5, (h, t), generator=gen)]
+            allocation_k_bits = widths[torch.randint(1, 5, (h, d), generator=gen)]
+        return Allocation()
+
+    same = [layer(3, 17, 8) for _ in range(5)]
+    want = [bw._logical_layer_bits(p, 8) for p in same]
+    assert bw._logical_bits_of_layers(same, 8).tolist() == want
+    assert want == [S.logical_layer_bits(p.allocation_v_bits.numpy(), p.allocation_k_bits.numpy(), 8) for p in same]
+    ragged = same[:2] + [layer(3, 9, 8), layer(2, 17, 8)]
+    assert bw._logical_bits_of_layers(ragged, 8).tolist() == [bw._logical_layer_bits(p, 8) for p in ragged]
 
 
 def test_protocol_config_validation():
