@@ -161,7 +161,7 @@ def fused_step_times(cache, qs, out, lse, steps, warmup, torch, graph=True, roun
     def partials_only():
         _lib.check(lib.rdkv_decode_fused_partials(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords, qs.data_ptr(), q_dt, qs.stride(0),
+            _lib.ptr(cache.groups), cache.n_groups, cache.row_dwords_arg, qs.data_ptr(), q_dt, qs.stride(0),
             cache.G, None, None, 0, ws.data_ptr(), ws.numel(), stream))
 
     def merge_only():

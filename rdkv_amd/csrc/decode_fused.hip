@@ -317,6 +317,7 @@ struct Item {
   int tile_begin, tile_end, d8, d4, d2, R, NS, n0, n1, n2, n3, ts1, ts2, ts3, q_row;
   int nchunk_full, wc_last, nchunks;
   int merge_unit, merge_begin, merge_count;
+  bool shape_ok;        // fixed-shape variants: the unit's K row has the variant's shape
   int v_shift;          // the quantized classes' p*scale operand carries a further 2^-v_shift
   float k_scale_max;    // largest K channel scale of the unit
   const uint8_t *k_base, *sz_base, *v_base0, *v_base1, *v_base2, *v_base3, *qtab_base;
@@ -335,7 +336,12 @@ __device__ __forceinline__ T sel4(int c, T a0, T a1, T a2, T a3) {
 // waiting for the others (wavefronts drift apart by several tiles over an item; a barrier per
 // item cost 12-15 us of idle time each), parks its result per item in LDS, and one barrier
 // later the workgroup combines and writes the partials of the batch.
-template <int NH, int RMAX, int WPE, bool MERGE>
+// SHAPE != 0 (d8 << 16 | d4 << 8 | d2) builds the kernel for units whose K rows all have that
+// many dwords of 8-, 4- and 2-bit fields: the K side becomes straight-line code over registers
+// with fixed numbers, its LDS operands requested two steps ahead, and RMAX is the row rounded up
+// to whole 16-byte chunks.  A unit of another shape is skipped (none of its tiles is read) and
+// its partials are written as NaN (merged output rows: NaN, lse -inf).
+template <int NH, int RMAX, int WPE, bool MERGE, int SHAPE = 0>
 __global__ void __launch_bounds__(256 * WPE) __attribute__((amdgpu_waves_per_eu(WPE, WPE)))
 decode_fused_kernel(const uint8_t *__restrict__ blob,
                     const RdkvWork *__restrict__ work, const int32_t *__restrict__ groups,
@@ -351,6 +357,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
   const int ln = lane & 3, lb = lane >> 2;
   const int item_begin = groups ? groups[blockIdx.x] : (int)blockIdx.x;
   const int item_end = groups ? groups[blockIdx.x + 1] : (int)blockIdx.x + 1;
+  constexpr int kD8 = (SHAPE >> 16) & 255, kD4 = (SHAPE >> 8) & 255, kD2 = SHAPE & 255, kR = kD8 + kD4 + kD2;
+  static_assert(SHAPE == 0 || (kR >= 1 && RMAX == (kR + 3) / 4 * 4), "RMAX of a fixed shape is its row in whole chunks");
 
   auto load_item = [&](int item) __attribute__((always_inline)) -> Item {
     const RdkvWork *wkp = work + item;
@@ -375,6 +383,8 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
     it.q_row = up->q_row;
     it.nchunk_full = it.R >> 2; it.wc_last = it.R & 3;
     it.nchunks = it.nchunk_full + (it.wc_last ? 1 : 0);
+    it.shape_ok = SHAPE == 0 || (it.d8 == kD8 && it.d4 == kD4 && it.d2 == kD2);
+    if (!it.shape_ok) it.tile_end = it.tile_begin;
     return it;
   };
 
@@ -411,13 +421,14 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
   // of the work table instead, so the same number of loads is in flight on every path and no
   // address outside the unit's regions is formed.
   auto issue_k = [&](int ti, bool ok = true) __attribute__((always_inline)) {
-    const uint8_t *ktile = ok ? it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * it.R
+    const uint8_t *ktile = ok ? it.k_base + (uint64_t)ti * (RDKV_TILE * 4) * (SHAPE != 0 ? kR : it.R)
                               : reinterpret_cast<const uint8_t *>(work);
     const int lane_k = ok ? lane : 0;
 #pragma unroll
     for (int ch = 0; ch < RMAX / 4; ++ch) {
-      const int che = (ok && ch < it.nchunks) ? ch : 0;
-      const int wce = che == it.nchunk_full ? it.wc_last : 4;
+      const int che = (ok && (SHAPE != 0 || ch < it.nchunks)) ? ch : 0;
+      const int wce = SHAPE != 0 ? ((kR & 3) != 0 && che == (kR >> 2) ? (kR & 3) : 4)
+                                 : (che == it.nchunk_full ? it.wc_last : 4);
       // a partial last chunk is read with a 16-byte load too: the surplus dwords belong to
       // the next token (or the region that follows) and are never used
       const uint4 v = *reinterpret_cast<const uint4 *>(ktile + che * 1024 + lane_k * 4 * wce);
@@ -670,7 +681,39 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
           sacc_lo[hg] = mfma(a, o.v[hg][1], sacc_lo[hg]);
         }
       };
-      {
+      if constexpr (SHAPE != 0) {
+        // Fixed shape: step s takes a field pair of a dword with a fixed register number at a
+        // fixed shift; the operands of step s + 2 are requested from LDS before step s is
+        // multiplied (same steps in the same order as the loops below: same bits).
+        constexpr int kSteps = kD8 + 2 * kD4 + 4 * kD2, kAhead = 2;
+        auto k_fixed = [&](int idx) __attribute__((always_inline)) -> uint32_t {
+          return idx < kRowA ? krow[idx < kRowA ? idx : 0] : ktail[idx >= kRowA ? idx - kRowA : 0];
+        };
+        auto k_op = [&](int s2) __attribute__((always_inline)) -> half4_t {
+          if (s2 < kD8) {
+            const uint32_t w = k_fixed(s2);
+            return mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu);
+          }
+          s2 -= kD8;
+          if (s2 < 2 * kD4) {
+            const uint32_t w = k_fixed(kD8 + (s2 >> 1));
+            const int sh = (s2 & 1) * 8;
+            return mk_op((w >> sh) & 0x000F000Fu, (w >> (sh + 4)) & 0x000F000Fu);
+          }
+          s2 -= 2 * kD4;
+          const uint32_t w = k_fixed(kD8 + kD4 + (s2 >> 2));
+          const int sh = (s2 & 3) * 4;
+          return mk_op((w >> sh) & 0x00030003u, (w >> (sh + 2)) & 0x00030003u);
+        };
+        QOp ops[kAhead + 1];
+#pragma unroll
+        for (int s2 = 0; s2 < kAhead; ++s2) ops[s2] = q_load(s2);
+#pragma unroll
+        for (int s2 = 0; s2 < kSteps; ++s2) {
+          ops[(s2 + kAhead) % (kAhead + 1)] = q_load(s2 + kAhead < kSteps ? s2 + kAhead : kSteps - 1);
+          k_step(k_op(s2), ops[s2 % (kAhead + 1)]);
+        }
+      } else {
         // Software-pipelined: the operands of the next step(s) are read from LDS while the
         // current ones are multiplied (reads one step past the end stay inside the LDS block).
         const int d8 = it.d8, d4 = it.d4, d2 = it.d2;
@@ -895,6 +938,7 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         o += f * sm.wo[b][w][h][d];
         l += f * sm.wl[b][w][h];
       }
+      if (SHAPE != 0 && !load_item(batch + b).shape_ok) o = M = __builtin_nanf("");
       pstore(part + h * kPartialStride + d, o);
       if (d == 0) {
         pstore(part + h * kPartialStride + 128, M);
@@ -1412,6 +1456,8 @@ static int check_fused_args(const char *fn, const RdkvUnit *units, int n_units, 
 }
 
 // Launch of the streaming kernel (writes one partial per work item).
+constexpr int kShape_0_5_2 = (5 << 8) | 2, kShape_0_16_0 = 16 << 8, kShape_0_0_8 = 8;
+
 static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *units, int n_units,
                         const RdkvWork *work, int n_work, const int32_t *groups, int n_groups,
                         int max_row_dwords, const void *q, int q_dtype, int64_t q_stride_row, int G,
@@ -1426,8 +1472,14 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
                n_groups);
   const int n_wg = groups ? n_groups : n_work;
   RDKV_REQUIRE(q_dtype >= 0 && q_dtype <= 2, "%s: unknown q dtype %d", fn, q_dtype);
+  // bits 8..31: the one K row shape of every unit (d8 << 16 | d4 << 8 | d2), or 0
+  const int row_shape = max_row_dwords >> 8;
+  max_row_dwords &= 255;
   RDKV_REQUIRE(max_row_dwords >= 0 && max_row_dwords <= 32, "%s: max_row_dwords=%d outside 0..32", fn,
                max_row_dwords);
+  RDKV_REQUIRE(row_shape >= 0 && (row_shape == 0 || ((row_shape >> 16) & 255) + ((row_shape >> 8) & 255) +
+                                                            (row_shape & 255) == max_row_dwords),
+               "%s: row shape %#x does not add up to max_row_dwords=%d", fn, row_shape, max_row_dwords);
   if (n_work == 0) return RDKV_OK;
   RDKV_REQUIRE(q, "%s: null q", fn);
   hipStream_t s = (hipStream_t)stream;
@@ -1436,16 +1488,22 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
   // keeps everything in registers; spilling costs far more than the lost occupancy.
   // (the variant that merges in the launch is a kernel of its own: the merge's registers would
   // otherwise push the two-launch form into scratch memory)
-#define RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, MERGE)                                                             \
-  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE, MERGE>), dim3(n_wg), dim3(256 * WPE), 0, s, blob, work, \
-                     groups, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype, partials, tickets,  \
-                     out, out_stride_row, lse)
-#define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE)                                                               \
+#define RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, MERGE, SHAPE)                                                      \
+  hipLaunchKernelGGL((decode_fused_kernel<NH, RMAX, WPE, MERGE, SHAPE>), dim3(n_wg), dim3(256 * WPE), 0, s,   \
+                     blob, work, groups, q, q_dtype, q_stride_row, G, rope_cos, rope_sin, rope_dtype,         \
+                     partials, tickets, out, out_stride_row, lse)
+#define RDKV_LAUNCH_FUSED_SHAPE(NH, RMAX, WPE, SHAPE)                                                      \
   do {                                                                                                     \
-    if (tickets) RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, true);                                                 \
-    else RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, false);                                                        \
+    if (tickets) RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, true, SHAPE);                                          \
+    else RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, false, SHAPE);                                                 \
   } while (0)
-  if (G <= 4) {   // one head group
+#define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE) RDKV_LAUNCH_FUSED_SHAPE(NH, RMAX, WPE, 0)
+  // Row shapes with a kernel of their own (one head group): every channel at 4 bits, every
+  // channel at 2 bits, and the 4- / 2-bit mix of the 128k-context benchmark workload.
+  if (G <= 4 && row_shape == kShape_0_5_2) RDKV_LAUNCH_FUSED_SHAPE(1, 8, 4, kShape_0_5_2);
+  else if (G <= 4 && row_shape == kShape_0_16_0) RDKV_LAUNCH_FUSED_SHAPE(1, 16, 4, kShape_0_16_0);
+  else if (G <= 4 && row_shape == kShape_0_0_8) RDKV_LAUNCH_FUSED_SHAPE(1, 8, 4, kShape_0_0_8);
+  else if (G <= 4) {   // one head group
     if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED_WPE(1, 12, 4);
     else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED_WPE(1, 16, 4);
     else if (max_row_dwords <= 20) RDKV_LAUNCH_FUSED_WPE(1, 20, 4);
@@ -1457,6 +1515,7 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
     else RDKV_LAUNCH_FUSED_WPE(2, 32, 2);
   }
 #undef RDKV_LAUNCH_FUSED_WPE
+#undef RDKV_LAUNCH_FUSED_SHAPE
 #undef RDKV_LAUNCH_FUSED_M
   RDKV_CHECK_LAUNCH(fn);
   return RDKV_OK;

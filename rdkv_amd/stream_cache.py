@@ -102,6 +102,7 @@ class StreamCache:
     stream_bytes: int                    # bytes the fused kernel reads from the blobs per step
     algorithmic_bytes: int               # unpadded bytes (reference accounting) incl. q and out
     max_row_dwords: int = 32             # max over units of the K row length in dwords
+    row_shape: int = 0                   # d8 << 16 | d4 << 8 | d2 when every unit's K row has that shape, else 0
     groups: Optional[torch.Tensor] = None  # device int32 [n_groups + 1] offsets into ``work`` (or None)
     groups_host: Optional[np.ndarray] = None
     n_groups: int = 0
@@ -115,6 +116,21 @@ class StreamCache:
     @property
     def device(self):
         return self.units.device
+
+    @property
+    def row_dwords_arg(self) -> int:
+        """The ``max_row_dwords`` argument of the fused entry points: the longest K row, and in
+        bits 8 and up the one row shape of all units (the library has kernels for some shapes)."""
+        return int(self.max_row_dwords) | (int(self.row_shape) << 8)
+
+
+def uniform_row_shape(units: np.ndarray) -> int:
+    """``d8 << 16 | d4 << 8 | d2`` when every unit of the table has that K row shape, else 0."""
+    if len(units) == 0:
+        return 0
+    d8, d4, d2 = int(units["d8"][0]), int(units["d4"][0]), int(units["d2"][0])
+    same = (units["d8"] == d8).all() and (units["d4"] == d4).all() and (units["d2"] == d2).all()
+    return (d8 << 16 | d4 << 8 | d2) if same else 0
 
 
 def _layer_counts(pl: PackedKVLayer, H_kv: int):
@@ -665,7 +681,7 @@ def _finish_caches(specs) -> List[StreamCache]:
             blobs=list(blobs), units=tables[2 * k], work=work_tables[k], units_host=units_np, work_host=work_np,
             n_units=len(units_np), n_work=len(work_np), G=G, rows=rows,
             stream_bytes=int(stream_bytes), algorithmic_bytes=int(kv_algo_bytes + rows * 128 * 6),
-            max_row_dwords=r_max,
+            max_row_dwords=r_max, row_shape=uniform_row_shape(units_np),
             groups=tables[2 * k + 1].view(torch.int32) if groups_np is not None else None, groups_host=groups_np,
             n_groups=0 if groups_np is None else len(groups_np) - 1,
             kv_algorithmic_bytes=int(kv_algo_bytes), multi_source=opt["multi_source"], h_q=int(H_q)))
@@ -816,7 +832,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     if one_launch:
         _lib.check(lib.rdkv_decode_fused_one_launch(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+            _lib.ptr(cache.groups), cache.n_groups, cache.row_dwords_arg,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
             out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), cache.tickets.data_ptr(),
             stream))
@@ -824,7 +840,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
     if zone_c is None:
         _lib.check(lib.rdkv_decode_fused(
             None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-            _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+            _lib.ptr(cache.groups), cache.n_groups, cache.row_dwords_arg,
             q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
             out.data_ptr(), out.stride(0), lse.data_ptr(), ws.data_ptr(), ws.numel(), stream))
         return out, lse
@@ -840,7 +856,7 @@ def decode_attn_fused(cache: StreamCache, q: torch.Tensor, out: Optional[torch.T
         assert counts.dtype == torch.int32 and counts.numel() == n_kv_rows and counts.is_contiguous()
     _lib.check(lib.rdkv_decode_fused_partials(
         None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work,
-        _lib.ptr(cache.groups), cache.n_groups, cache.max_row_dwords,
+        _lib.ptr(cache.groups), cache.n_groups, cache.row_dwords_arg,
         q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, _lib.ptr(rc), _lib.ptr(rs), rope_dt,
         ws.data_ptr(), ws.numel(), stream))
     n_new = int(K_new.shape[1])

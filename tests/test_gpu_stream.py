@@ -1,5 +1,7 @@
 """GPU parity of the streaming format (bit-exact, invertible) and of the fused decode kernel
 (max-abs 2e-3 / relative 1e-2 against the dequantize-then-attend oracle)."""
+import dataclasses
+
 import numpy as np
 import pytest
 import torch
@@ -455,6 +457,85 @@ def test_fused_attention_k_row_shapes(counts):
     out, lse = fused_both(cache, q.to(DEV))
     attn_close(t2n(out), exp_out, "out")
     attn_close(t2n(lse), exp_lse, "lse")
+
+
+def _uniform_shape_case(c2, c4, c8, H_kv, G, T, seed):
+    rng = np.random.default_rng(seed)
+    g = torch.Generator().manual_seed(seed)
+    K = torch.randn(1, H_kv, T, 128, generator=g).half()
+    V = torch.randn(1, H_kv, T, 128, generator=g).half()
+    q = torch.randn(H_kv * G, 128, generator=g).half()
+    vb = torch.from_numpy(rng.choice(np.array([0, 2, 4, 8, 16]), size=(H_kv, T)))
+    kb = np.zeros((H_kv, 128), dtype=np.int64)
+    for h in range(H_kv):
+        ch = rng.permutation(128)
+        kb[h, ch[:c2]] = 2
+        kb[h, ch[c2:c2 + c4]] = 4
+        kb[h, ch[c2 + c4:c2 + c4 + c8]] = 8
+    return K, V, q, vb, torch.from_numpy(kb)
+
+
+@pytest.mark.parametrize("counts,shape", [((32, 40, 0), (0, 5, 2)), ((24, 36, 0), (0, 5, 2)), ((0, 128, 0), (0, 16, 0)),
+                                          ((128, 0, 0), (0, 0, 8)), ((113, 0, 0), (0, 0, 8))])
+@pytest.mark.parametrize("G", [4, 2])
+def test_fused_attention_fixed_shape_kernels_equal_the_general_kernel(counts, shape, G):
+    """Caches whose units all have one K row shape state it in the row argument; for the shapes the
+    library has kernels of their own for, those kernels give the general kernel's bits (two launches,
+    one launch, allocation-free entry point) and the oracle's values; several layers per call, a token
+    count that leaves partial tiles."""
+    H_kv, T = 3, 1333
+    layers, qs, exp = [], [], []
+    for layer in range(2):
+        K, V, q, vb, kb = _uniform_shape_case(*counts, H_kv, G, T, seed=sum(counts) * 31 + G + layer)
+        ora, ora_nvo = O.pack_layer_per_head(K.numpy(), V.numpy(), vb.numpy(), kb.numpy(), G)
+        exp.append(O.decode_attn_ref(q.numpy(), ora, ora_nvo)[:2])
+        layers.append(packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G))
+        qs.append(q)
+    q = torch.cat(qs).to(DEV)
+    cache = stream_cache.build_stream_cache(layers, G, n_groups=5)
+    d8, d4, d2 = shape
+    assert cache.row_shape == (d8 << 16 | d4 << 8 | d2) and cache.max_row_dwords == d8 + d4 + d2
+    assert cache.row_dwords_arg == cache.max_row_dwords | cache.row_shape << 8
+    general = dataclasses.replace(cache, row_shape=0)
+    assert general.row_dwords_arg == cache.max_row_dwords
+    out, lse = fused_both(cache, q)
+    out_g, lse_g = fused_both(general, q)
+    assert torch.equal(out, out_g) and torch.equal(lse.view(torch.int32), lse_g.view(torch.int32))
+    o, l = t2n(out), t2n(lse)
+    for layer, (eo, el) in enumerate(exp):
+        rows = slice(layer * H_kv * G, (layer + 1) * H_kv * G)
+        attn_close(o[rows], eo, f"out layer {layer}")
+        attn_close(l[rows], el, f"lse layer {layer}")
+    lib = _lib.load()
+    out_s = torch.empty_like(out)
+    lse_s = torch.empty_like(lse)
+    _lib.check(lib.rdkv_decode_fused_static(
+        None, cache.units.data_ptr(), cache.n_units, cache.work.data_ptr(), cache.n_work, _lib.ptr(cache.groups),
+        cache.n_groups, cache.row_dwords_arg, q.data_ptr(), _lib.DTYPE_CODE[q.dtype], q.stride(0), cache.G, None, None,
+        0, out_s.data_ptr(), out_s.stride(0), lse_s.data_ptr(), _lib.stream_of(q.device)))
+    assert torch.equal(out_s, out) and torch.equal(lse_s.view(torch.int32), lse.view(torch.int32))
+
+
+def test_fused_attention_row_shape_argument_is_checked():
+    """A shape that does not add up to the row length is refused; units of another shape than the
+    stated one are not read and their rows come back as NaN (lse: -inf), the other units' rows are unchanged."""
+    H_kv, G, T = 2, 4, 500
+    a = _uniform_shape_case(32, 40, 0, H_kv, G, T, seed=5)          # rows of 0/5/2 dwords
+    b = _uniform_shape_case(0, 56, 0, H_kv, G, T, seed=6)           # rows of 0/7/0 dwords: as long, another shape
+    layers = [packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G) for K, V, _, vb, kb in (a, b)]
+    q = torch.cat([a[2], b[2]]).to(DEV)
+    cache = stream_cache.build_stream_cache(layers, G)
+    assert cache.row_shape == 0 and cache.max_row_dwords == 7
+    want, _ = stream_cache.decode_attn_fused(cache, q)
+    assert bool(torch.isfinite(want).all())
+    wrong = dataclasses.replace(cache, row_shape=5 << 8 | 2)
+    got, got_lse = stream_cache.decode_attn_fused(wrong, q, one_launch=False)
+    torch.cuda.synchronize()
+    n = H_kv * G
+    assert torch.equal(got[:n], want[:n])
+    assert bool(torch.isnan(got[n:]).all()) and bool(torch.isinf(got_lse[n:]).all())
+    with pytest.raises(AssertionError, match="row shape"):
+        stream_cache.decode_attn_fused(dataclasses.replace(cache, row_shape=5 << 8 | 3), q)
 
 
 @pytest.mark.parametrize("k_mul,v_mul,q_mul,widths,G", [
