@@ -269,6 +269,8 @@ def compact_config(index, args, torch, dev):
            "frac_kernel": algo / (ms_kernel * 1e-3) / 1e9 / HBM_PEAK_GBPS,
            "us_per_sequence_layer": ms_eager * 1e3 / n_groups, "work_items": cache.n_work,
            "kernel_variant_max_row_dwords": cache.max_row_dwords,
+           "kernel_variant_row_shape": [cache.row_shape >> 16, (cache.row_shape >> 8) & 255, cache.row_shape & 255]
+           if cache.row_shape else None,
            "compression_ratio": synth.dense_fp16_bytes(cfg) * n_groups / algo, "build_seconds": build_s}
     if not args.no_check:
         res["check"] = check_layer0(first_pl, first_nvo, qs[:cfg.H_q].cpu().numpy(), out[:cfg.H_q].cpu().numpy(), torch)
