@@ -908,8 +908,9 @@ def main():
         try:
             import torch.nn.functional as F
             T = cfg.context
-            Kd = [torch.randn(1, cfg.H_kv, T, cfg.D, device=dev, dtype=torch.float16) for _ in range(cfg.layers)]
-            Vd = [torch.randn(1, cfg.H_kv, T, cfg.D, device=dev, dtype=torch.float16) for _ in range(cfg.layers)]
+            K_all = torch.randn(cfg.layers, 1, cfg.H_kv, T, cfg.D, device=dev, dtype=torch.float16)
+            V_all = torch.randn(cfg.layers, 1, cfg.H_kv, T, cfg.D, device=dev, dtype=torch.float16)
+            Kd, Vd = list(K_all), list(V_all)
             qd = qs.view(cfg.layers, 1, cfg.H_q, 1, cfg.D)
 
             def dense_step():
@@ -936,7 +937,25 @@ def main():
                 dense_hip_step()
                 dense["dense_hip_kernel_ms"] = time_region(dense_hip_step, max(3, args.steps // 5), torch)
                 dense["dense_hip_kernel_GBps"] = dense_bytes / (dense["dense_hip_kernel_ms"] * 1e-3) / 1e9
-            del Kd, Vd
+                # ... and with all layers in one launch (+ one merge), the form the packed step is timed in
+                heads_all = cfg.layers * cfg.H_kv
+                chunks_all = max(1, min(32, 2048 // heads_all))
+                ws_all = torch.empty(lib.rdkv_probe_dense_decode_workspace_bytes(heads_all * cfg.G, chunks_all),
+                                     dtype=torch.uint8, device=dev)
+
+                def dense_hip_one_launch():
+                    _lib.check(lib.rdkv_probe_dense_decode(
+                        q16.data_ptr(), K_all.data_ptr(), V_all.data_ptr(), T, heads_all, cfg.G, chunks_all,
+                        out_d.data_ptr(), ws_all.data_ptr(), ws_all.numel(), stream))
+
+                out_layers = out_d.clone()
+                dense_hip_one_launch()
+                torch.cuda.synchronize()
+                dense["dense_hip_one_launch_max_abs_diff_vs_per_layer"] = float((out_d - out_layers).abs().max())
+                dense["dense_hip_kernel_one_launch_ms"] = time_region(dense_hip_one_launch, max(3, args.steps // 5), torch)
+                dense["dense_hip_kernel_one_launch_GBps"] = dense_bytes / (dense["dense_hip_kernel_one_launch_ms"] * 1e-3) / 1e9
+                del ws_all
+            del Kd, Vd, K_all, V_all
         except Exception as e:  # the comparison is informative; never fail the benchmark on it
             dense["sdpa_error"] = repr(e)[:200]
 
@@ -1025,7 +1044,9 @@ def main():
                            speedup_vs_ideal_dense=dense["ideal_ms_at_read_ceiling"] / ms_step,
                            speedup_vs_sdpa=(dense["sdpa_ms"] / ms_step) if dense.get("sdpa_ms") else None,
                            speedup_vs_dense_hip_kernel=(dense["dense_hip_kernel_ms"] / ms_step)
-                           if dense.get("dense_hip_kernel_ms") else None),
+                           if dense.get("dense_hip_kernel_ms") else None,
+                           speedup_vs_dense_hip_kernel_one_launch=(dense["dense_hip_kernel_one_launch_ms"] / ms_step)
+                           if dense.get("dense_hip_kernel_one_launch_ms") else None),
         "sequential": sequential,
         "padded": padded,
         "configs": configs,
