@@ -453,8 +453,20 @@ knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int gro
       __hip_atomic_store(&c.words[2 * kCoopMaxSplit * kCoopWords + threadIdx.x], (0xA5u << 24) | v, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);            // (the rows of a group sit on different dies)
     }
+    // The group can only lower this row's count when another row's rounds end early, and they
+    // end no earlier than this row's own lambda reaches 1e12 (g_own, below): while g_own + 1 >= d
+    // the minimum leaves d as it is whatever the other rows say, and nothing is waited for.
+    int g_own = kMaxDoublings + 1;
+    {
+      float lam = lam0;
+      for (int it = 0; it < kMaxDoublings; ++it) {
+        if (it < d) lam = __fmul_rn(lam, 2.0f);
+        if (lam >= 1e12f) { g_own = it; break; }
+      }
+    }
+    const bool ask_group = g_own + 1 < d;
     int dmax = 0, gmax = 0;
-    for (int r = r0 + threadIdx.x; r < r0 + group_rows; r += blockDim.x) {
+    for (int r = r0 + threadIdx.x; ask_group && r < r0 + group_rows; r += blockDim.x) {
       const uint32_t* gw = state + (int64_t)r * kCoopRowWords + 2 * kCoopMaxSplit * kCoopWords;
       uint32_t w3[3] = {0u, 0u, 0u};
       for (int spins = 0;; ++spins) {                      // the three words together, until all carry the tag
@@ -479,11 +491,13 @@ knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int gro
       dmax = max(dmax, dr);
       gmax = max(gmax, g);
     }
-    dmax = block_reduce(dmax, MaxI(), lds);
-    gmax = block_reduce(gmax, MaxI(), lds);
-    __syncthreads();
-    const int rounds = min(min(dmax, gmax + 1), kMaxDoublings);
-    d = min(d, rounds);
+    if (ask_group) {                                   // (uniform over the workgroup)
+      dmax = block_reduce(dmax, MaxI(), lds);
+      gmax = block_reduce(gmax, MaxI(), lds);
+      __syncthreads();
+      const int rounds = min(min(dmax, gmax + 1), kMaxDoublings);
+      d = min(d, rounds);
+    }
   }
   float lam_hi = lam0;
   for (int i = 0; i < d; ++i) lam_hi = __fmul_rn(lam_hi, 2.0f);

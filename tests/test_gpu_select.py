@@ -113,6 +113,20 @@ def test_knapsack_long_rows_shared_by_workgroups(max_iters, tol):
                                out_dtype=torch.int64)
     np.testing.assert_array_equal(t2n(one), S.knapsack_bit_allocation_batched(s, budget, epsilon=S.DEFAULT_EPSILON_V,
                                                                               max_iters=max_iters, tol=tol))
+    # rows whose multiplier passes the 1e12 limit of the doubling rounds at once, after a few rounds and
+    # never, side by side in one group (the group's rounds end with the row that passes it last)
+    big = s.copy()
+    big[1] *= np.float32(3e12)
+    big[2] *= np.float32(2e9)
+    big[5] *= np.float32(5e10)
+    tight = np.array([4.0, 1e-6, 1e-6, 2.5, 15.9, 1e-6, 3.0, 1e-6], dtype=F32)
+    for rows in (4, 8):
+        exp_big = np.concatenate([S.knapsack_bit_allocation_batched(big[g:g + rows], tight[g:g + rows],
+                                                                    epsilon=S.DEFAULT_EPSILON_V, max_iters=max_iters,
+                                                                    tol=tol) for g in range(0, B, rows)])
+        got_big = ks.knapsack_allocate(to_dev(big), to_dev(tight), ks.DEFAULT_EPSILON_V, max_iters=max_iters, tol=tol,
+                                       group_rows=rows, out_dtype=torch.int64)
+        np.testing.assert_array_equal(t2n(got_big), exp_big)
 
 
 def test_knapsack_edges():
