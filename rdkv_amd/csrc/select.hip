@@ -199,9 +199,9 @@ knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int g
 // The same solver with every row shared by several workgroups, for batches too small to fill the
 // device with one workgroup per row (one layer's eight heads of 32k tokens kept eight compute units
 // busy for ~60 dependent passes).  A row's S workgroups each own a contiguous chunk of it, held in
-// registers.  One pass evaluates up to 16 candidate lambdas at once - the next 15 doublings, or
-// lambda = 0 and the 15 midpoints four bisection levels can reach - as integer width sums of the
-// chunk.  The workgroups then exchange their sums: each stores its own as words that carry the
+// registers.  One pass evaluates up to 17 candidate lambdas at once - the next 15 doublings, or
+// lambda = 0 and the 15 midpoints four bisection levels can reach (in the first pass together with
+// the row's starting lambda, which usually needs no doubling) - as integer width sums of the chunk.  The workgroups then exchange their sums: each stores its own as words that carry the
 // pass number in their top byte, and reads every workgroup's words until all of them carry it
 // (double-buffered by pass parity: a workgroup can be at most one pass ahead of another of its row).
 // So a pass costs one store and one load round trip between workgroups, no atomic operation meets
@@ -213,7 +213,7 @@ knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int g
 // ---------------------------------------------------------------------------------------------
 constexpr int kCoopThreads = 256;
 constexpr int kCoopMaxSplit = 64;          // workgroups per row at most
-constexpr int kCoopWords = 16;             // words a workgroup publishes per pass
+constexpr int kCoopWords = 32;             // words a workgroup can publish per pass (17 are used at most)
 constexpr int kCoopMaxIters = 64;          // passes stay below the 255 the tag byte can tell apart
 constexpr int kCoopSpinLimit = 1 << 20;
 constexpr uint32_t kCoopValueMask = 0xffffffu;
@@ -264,8 +264,10 @@ __device__ void coop_exchange(CoopCtx& c, int n, const int* mine) {
       atomicMax(reinterpret_cast<unsigned int*>(&c.tot[0]), (hi << 16) | lo);
     }
   } else {
-    // a thread's words (S * 16 <= 4 * 256) are requested together and asked for again until all carry the tag
+    // a thread's words (word i of every kCoopThreads / kCoopWords-th workgroup) are requested together and
+    // asked for again until all carry the tag
     constexpr int kPer = kCoopMaxSplit * kCoopWords / kCoopThreads;
+    static_assert(kCoopWords == 32 && kCoopThreads % kCoopWords == 0, "the lane pairing below assumes 32 words");
     const int i = threadIdx.x & (kCoopWords - 1);
     uint32_t w[kPer];
     bool want[kPer];
@@ -294,8 +296,7 @@ __device__ void coop_exchange(CoopCtx& c, int n, const int* mine) {
     int sum = 0;
 #pragma unroll
     for (int k = 0; k < kPer; ++k) sum += want[k] ? (int)(w[k] & kCoopValueMask) : 0;
-    // lanes l, l ^ 16, l ^ 32 and l ^ 48 hold the same i
-    sum += __shfl_xor(sum, 16, 64);
+    // lanes l and l ^ 32 hold the same i
     sum += __shfl_xor(sum, 32, 64);
     if ((threadIdx.x & 63) < kCoopWords && i < n) atomicAdd(&c.tot[i], sum);
   }
@@ -362,7 +363,7 @@ __global__ void coop_init_kernel(uint32_t* state, int64_t n_words) {
 }
 
 template <int HELD>
-__global__ void __launch_bounds__(kCoopThreads)
+__global__ void __launch_bounds__(kCoopThreads) __attribute__((amdgpu_waves_per_eu(4)))
 knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int group_rows, int T, int S,
                      const float* __restrict__ budget, Options o, int max_iters, float tol,
                      uint32_t* __restrict__ state, void* __restrict__ out, int out_elem_size,
@@ -414,11 +415,36 @@ knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int gro
   __syncthreads();
   if (threadIdx.x < 2) red[threadIdx.x] = 0;
 
-  // ---- doublings the row asks for on its own: the first k with avg(lam0 * 2^k) <= budget
+  // ---- first pass: lam0 itself (the first candidate of the doubling rounds) together with what the
+  // bisection starts with when the row needs no doubling, which is the usual case: lambda = 0 and the
+  // 15 midpoints of four bisection levels over (0, lam0).  A row that does need doubling goes through
+  // the rounds 15 candidates at a time and bisects from scratch.
+  // d: the first k with avg(lam0 * 2^k) <= budget
   int d = -1;
   {
-    float lam = lam0;
-    for (int base = 0; base < kMaxDoublings && d < 0; base += 15) {
+    if (threadIdx.x == 0) {
+      float lo[16], hi[16];
+      lo[1] = 0.f; hi[1] = lam0;
+      cand[0] = lam0;
+      cand[1] = 0.f;
+#pragma unroll
+      for (int n = 1; n < 16; ++n) {
+        const float mid = __fdiv_rn(__fadd_rn(lo[n], hi[n]), 2.0f);
+        cand[1 + n] = mid;
+        if (2 * n < 16) {
+          lo[2 * n] = lo[n]; hi[2 * n] = mid;
+          lo[2 * n + 1] = mid; hi[2 * n + 1] = hi[n];
+        }
+      }
+    }
+    __syncthreads();
+    coop_chunk_sums<HELD>(row, c, se, valid, cand, 17, o, red);
+    coop_exchange<false>(c, 17, red);
+    if ((int)threadIdx.x < 17) red[threadIdx.x] = 0;
+    if (!(__fdiv_rn((float)tot[0], (float)T) > bud)) d = 0;
+    __syncthreads();
+    float lam = __fmul_rn(lam0, 2.0f);
+    for (int base = 1; base < kMaxDoublings && d < 0; base += 15) {
       const int n = min(15, kMaxDoublings - base);
       if (threadIdx.x == 0) {
         for (int i = 0; i < n; ++i) {
@@ -443,6 +469,8 @@ knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int gro
     }
     if (d < 0) d = kMaxDoublings;
   }
+  // (d == 0: the first pass's sums of lambda = 0 and the 15 midpoints are what the bisection's first pass needs)
+  bool have_first = d == 0;
   // ---- the rounds the row's group executes (as in knapsack_bisect_kernel): every row publishes
   // its lam0 and doublings, every workgroup reads those of its group
   const int r0 = (b / group_rows) * group_rows;
@@ -511,32 +539,36 @@ knapsack_coop_kernel(const float* __restrict__ scores, int64_t stride_b, int gro
     int it = 0;
     // (with max_iters = 0 the reference still evaluates lambda = 0, but nothing depends on it)
     while (!done) {
-      if (threadIdx.x == 0) {
-        float lo[16], hi[16];
-        lo[1] = lam_lo; hi[1] = lam_hi;
-        cand[0] = 0.f;   // lambda = 0 decides whether to bisect at all (first pass; unused afterwards)
+      const int at = have_first ? 1 : 0;   // where lambda = 0 sits in cand / tot; the nodes follow it
+      if (!have_first) {
+        if (threadIdx.x == 0) {
+          float lo[16], hi[16];
+          lo[1] = lam_lo; hi[1] = lam_hi;
+          cand[0] = 0.f;   // lambda = 0 decides whether to bisect at all (first pass; unused afterwards)
 #pragma unroll
-        for (int n = 1; n < 16; ++n) {
-          const float mid = __fdiv_rn(__fadd_rn(lo[n], hi[n]), 2.0f);
-          cand[n] = mid;
-          if (2 * n < 16) {
-            lo[2 * n] = lo[n]; hi[2 * n] = mid;
-            lo[2 * n + 1] = mid; hi[2 * n + 1] = hi[n];
+          for (int n = 1; n < 16; ++n) {
+            const float mid = __fdiv_rn(__fadd_rn(lo[n], hi[n]), 2.0f);
+            cand[n] = mid;
+            if (2 * n < 16) {
+              lo[2 * n] = lo[n]; hi[2 * n] = mid;
+              lo[2 * n + 1] = mid; hi[2 * n + 1] = hi[n];
+            }
           }
         }
+        __syncthreads();
+        coop_chunk_sums<HELD>(row, c, se, valid, cand, 16, o, red);
+        coop_exchange<false>(c, 16, red);
+        if (threadIdx.x < kCoopWords) red[threadIdx.x] = 0;
       }
-      __syncthreads();
-      coop_chunk_sums<HELD>(row, c, se, valid, cand, 16, o, red);
-      coop_exchange<false>(c, 16, red);
-      if (threadIdx.x < kCoopWords) red[threadIdx.x] = 0;
+      have_first = false;
       if (first) {
         first = false;
-        if (__fdiv_rn((float)tot[0], (float)T) <= bud) done = true;
+        if (__fdiv_rn((float)tot[at], (float)T) <= bud) done = true;
       }
       int node = 1;
       for (int lvl = 0; lvl < 4 && !done; ++lvl) {
-        const float mid = cand[node];
-        const float avg = __fdiv_rn((float)tot[node], (float)T);
+        const float mid = cand[at + node];
+        const float avg = __fdiv_rn((float)tot[at + node], (float)T);
         lam_final = mid;
         ++it;
         const float rel = __fdiv_rn(fabsf(__fsub_rn(avg, bud)), denom);
@@ -703,26 +735,46 @@ int check_common(const void* scores, int B, int64_t T, const void* budget, const
 // form): chunks of at least 512 scores, at most 64 per row, the whole launch on at most half of the
 // workgroup slots the device has for this kernel, and only when that gives a row at least sixteen
 // (with fewer, one workgroup per row was as fast or faster on 64 rows of 32k scores).
+// 0 / 1 / 2: the kernel that holds 2 / 4 / 8 scores of a chunk per thread in registers
+static int coop_held_index(int64_t chunk) { return chunk <= 2 * kCoopThreads ? 0 : (chunk <= 4 * kCoopThreads ? 1 : 2); }
+
 static int coop_split(int B, int64_t T, int max_iters) {
   if (B <= 0 || T < 4096 || max_iters > kCoopMaxIters) return 0;
-  static int slots_of_device[64];          // (0 = not asked yet; a race between first callers writes the same value)
-  int dev = 0, slots = 0;
+  // workgroup slots of the device for the kernel that holds 2 / 4 / 8 scores per thread
+  static int slots_of_device[64][3];       // (0 = not asked yet; a race between first callers writes the same value)
+  int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-  if (slots_of_device[dev] == 0) {
-    int cus = 0, per_cu = 0;
-    const bool ok = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
-                    hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, knapsack_coop_kernel<8>, kCoopThreads, 0) == hipSuccess &&
-                    per_cu > 0;
+  if (slots_of_device[dev][2] == 0) {
+    int cus = 0, per_cu[3] = {0, 0, 0};
+    const bool ok =
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0 &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[0], knapsack_coop_kernel<2>, kCoopThreads, 0) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[1], knapsack_coop_kernel<4>, kCoopThreads, 0) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu[2], knapsack_coop_kernel<8>, kCoopThreads, 0) == hipSuccess &&
+        per_cu[0] > 0 && per_cu[1] > 0 && per_cu[2] > 0;
     if (!ok) return 0;                     // (asked again next time: the query can fail while a stream is being captured)
-    slots_of_device[dev] = cus * per_cu;
+    for (int k = 0; k < 3; ++k) slots_of_device[dev][k] = cus * per_cu[k];
   }
-  slots = slots_of_device[dev];
-  if (slots <= 0) return 0;
   int64_t S = T / 512;
   if (S > kCoopMaxSplit) S = kCoopMaxSplit;
-  if (S > slots / 2 / B) S = slots / 2 / B;
+  // the launch may take half the slots of the kernel its chunk length selects (a shorter split means
+  // longer chunks, which can select the next kernel: settle in at most three steps)
+  // (a power of two: chunks of a whole number of scores per thread measured faster than the larger
+  // split in between - 16 rows of 32k: 68 us with 32 workgroups per row, 74 us with 40)
+  auto pow2_floor = [](int64_t v) { int64_t p = 1; while (2 * p <= v) p *= 2; return v >= 1 ? p : 0; };
+  S = pow2_floor(S);
+  for (int step = 0; step < 3 && S >= 1; ++step) {
+    const int64_t chunk = (T + S - 1) / S;
+    const int k = coop_held_index(chunk);
+    const int64_t cap = slots_of_device[dev][k] / 2 / B;
+    if (S <= cap) break;
+    S = pow2_floor(cap);
+  }
+  if (S < 16) return 0;
+  const int64_t chunk = (T + S - 1) / S;
+  if ((int64_t)B * S > slots_of_device[dev][coop_held_index(chunk)] / 2) return 0;
   // (a chunk's width sum must fit the 24 value bits of an exchange word)
-  return S >= 16 && (T + S - 1) / S <= 32768 ? (int)S : 0;
+  return chunk <= 32768 ? (int)S : 0;
 }
 
 RDKV_API int64_t rdkv_knapsack_workspace_bytes(int B) {
@@ -757,8 +809,8 @@ RDKV_API int rdkv_knapsack_batched(const float* scores, int64_t stride_b, int B,
     const int64_t n_words = (int64_t)B * kCoopRowWords;
     hipLaunchKernelGGL(coop_init_kernel, dim3((unsigned)rdkv_cdiv(n_words, 256)), dim3(256), 0, s, state, n_words);
     const int64_t chunk = (T + S - 1) / S;
-    auto kernel = chunk <= 2 * kCoopThreads ? knapsack_coop_kernel<2>
-                                            : (chunk <= 4 * kCoopThreads ? knapsack_coop_kernel<4> : knapsack_coop_kernel<8>);
+    const int held = coop_held_index(chunk);
+    auto kernel = held == 0 ? knapsack_coop_kernel<2> : (held == 1 ? knapsack_coop_kernel<4> : knapsack_coop_kernel<8>);
     hipLaunchKernelGGL(kernel, dim3((unsigned)(B * S)), dim3(kCoopThreads), 0, s, scores, stride_b, group_rows, (int)T, S,
                        budget, o, max_iters, tol, state, out, out_elem_size, out_stride_b, counts);
     RDKV_CHECK_LAUNCH("rdkv_knapsack_batched");
