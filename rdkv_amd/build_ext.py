@@ -22,7 +22,9 @@ COMMON = [
     "-Wno-unused-command-line-argument",
 ]
 # bit-exact quantizer code must not contract a*b+c into fma
-PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "select.hip": ["-ffp-contract=off"]}
+# (select.hip: an unroll request on the candidate loop of the shared-row knapsack is honoured at some of
+# its inlined call sites only - measured 3 % faster with it - and the optimizer says so for the others)
+PER_FILE = {"quantize.hip": ["-ffp-contract=off"], "select.hip": ["-ffp-contract=off", "-Wno-pass-failed"]}
 
 
 def _hipcc() -> str:
