@@ -719,7 +719,6 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         const int d8 = it.d8, d4 = it.d4, d2 = it.d2;
         int step = 0;
         QOp cur = q_load(0);
-#pragma unroll 2
         for (int i = 0; i < d8; ++i) {
           const QOp nxt = q_load(step + 1);
           const uint32_t w = k_dword(i);
