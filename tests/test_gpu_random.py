@@ -99,7 +99,10 @@ def test_fused_attention_random_workloads(block):
     """40 workloads per block, one to three layers in one launch: max-abs error of the output within
     2e-3 of the oracle's (2e-3 of its largest value where that exceeds 1: data is drawn at three
     magnitudes), log-sum-exp within 2e-3 (times the square of the magnitude, which the scores scale
-    with), rows that attend to nothing infinite in both."""
+    with), rows that attend to nothing infinite in both.  At the largest magnitude the scores reach
+    +-30 and the oracle's rounding of the dequantized K and V to fp16 alone moves its output by up to
+    3e-3 (seeds beyond the ones here show it): there the output may instead be within 2e-3 of the
+    same attention without that rounding, the arithmetic of the reference's packed kernels."""
     for case in range(40):
         rng = np.random.default_rng(9000 + 100 * block + case)
         H_kv, G = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4, 8]))
@@ -133,7 +136,8 @@ def test_fused_attention_random_workloads(block):
                 packed = None
                 break
             out, lse, _ = O.decode_attn_ref(q.numpy(), ora, ora_nvo)
-            exp.append((out, lse, scale))
+            out_plain = O.decode_attn_ref(q.numpy(), ora, ora_nvo, round_fp16=False)[0] if scale > 1.0 else out
+            exp.append((out, lse, scale, out_plain))
             packed.append(packing.pack_layer_per_head(K.to(DEV), V.to(DEV), vb, kb, G))
             qs.append(q)
         if packed is None:
@@ -141,13 +145,17 @@ def test_fused_attention_random_workloads(block):
         cache = stream_cache.build_stream_cache(packed, G)
         out, lse = stream_cache.decode_attn_fused(cache, torch.cat(qs).to(DEV))
         out, lse = out.float().cpu().numpy(), lse.float().cpu().numpy()
-        for layer, (eo, el, scale) in enumerate(exp):
+        for layer, (eo, el, scale, eo_plain) in enumerate(exp):
             rows = slice(layer * H_q, (layer + 1) * H_q)
             fin = np.isfinite(el)
             assert np.array_equal(np.isfinite(lse[rows]), fin), f"{what}, layer {layer}: rows without tokens"
             eo = np.where(np.isfinite(eo), eo, 0.0)
-            err = float(np.abs(out[rows] - eo).max()) / max(1.0, float(np.abs(eo).max()))
-            assert err < 2e-3, f"{what}, layer {layer} (magnitude {scale}): output error {err:.3e}"
+            eo_plain = np.where(np.isfinite(eo_plain), eo_plain, 0.0)
+            norm = max(1.0, float(np.abs(eo).max()))
+            err = float(np.abs(out[rows] - eo).max()) / norm
+            err_plain = float(np.abs(out[rows] - eo_plain).max()) / norm
+            assert min(err, err_plain) < 2e-3, (f"{what}, layer {layer} (magnitude {scale}): output error {err:.3e} "
+                                                f"({err_plain:.3e} against the oracle without fp16 rounding)")
             if fin.any():
                 err_l = float(np.abs(lse[rows][fin] - el[fin]).max())
                 assert err_l < 2e-3 * max(1.0, 16 * scale * scale), f"{what}, layer {layer}: lse error {err_l:.3e}"
