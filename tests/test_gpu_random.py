@@ -94,7 +94,7 @@ def test_whole_layer_packer_random_layouts(block):
             assert torch.equal(got_n.view(torch.uint8), exp_n.view(torch.uint8)), what
 
 
-@pytest.mark.parametrize("block", range(3))
+@pytest.mark.parametrize("block", [0, 1, 2, 21, 22])
 def test_fused_attention_random_workloads(block):
     """40 workloads per block, one to three layers in one launch: max-abs error of the output within
     2e-3 of the oracle's (2e-3 of its largest value where that exceeds 1: data is drawn at three

@@ -359,6 +359,31 @@ def test_selection_and_planning_entry_points_reject_bad_arguments():
         "bad shape")
 
 
+def test_row_shape_statement_of_the_fused_entry_points():
+    """The one-row-shape statement travels in the upper bits of ``max_row_dwords``: derived from the unit
+    table on the host, refused by the entry points when it does not add up to the row length (checked
+    before any device work)."""
+    from rdkv_amd import stream_cache as sc
+    units = np.zeros(3, dtype=sc.UNIT_DTYPE)
+    assert sc.uniform_row_shape(units[:0]) == 0
+    units["d8"], units["d4"], units["d2"] = 0, 5, 2
+    assert sc.uniform_row_shape(units) == (5 << 8 | 2)
+    units["d2"][1] = 1
+    assert sc.uniform_row_shape(units) == 0
+    units["d8"], units["d4"], units["d2"] = 32, 0, 0
+    assert sc.uniform_row_shape(units) == 32 << 16
+    lib = _lib.load()
+
+    def call(row_arg):
+        return lib.rdkv_decode_fused_partials(None, None, 0, None, 0, None, 0, row_arg, None, 1, 128, 4, None, None, 0,
+                                              None, 0, None)
+
+    assert call(7) == 0 and call(7 | (5 << 8 | 2) << 8) == 0 and call(32 | (32 << 16) << 8) == 0
+    for bad in (7 | (5 << 8 | 3) << 8, 8 | (5 << 8 | 2) << 8, 33, -1):
+        assert call(bad) == _lib.RDKV_EINVAL, bad
+    assert b"row shape" in lib.rdkv_last_error() or b"max_row_dwords" in lib.rdkv_last_error()
+
+
 def test_pre_extract_weights_on_a_cpu_model():
     """fast_decode.py:418-621: one matrix for q/k/v and one for gate/up, biases concatenated when
     the model has them, per-head q/k norm weights picked up, the result cached on the model."""
