@@ -588,8 +588,9 @@ int rdkv_pool_scores(const float *scores, int64_t stride_b, int B, int64_t T, in
  * was one call of the reference; 0 = the whole batch), so many calls can share one launch.
  * workspace: rdkv_knapsack_workspace_bytes(B) bytes.  Two launches, no host synchronization.
  * Batches of few long rows (T >= 8192, max_iters <= 64, so few rows that each can have 16 or
- * more resident workgroups) run with every row shared by up to 64 workgroups that exchange
- * integer width sums once per pass of 15 doublings or four bisection levels; the same bits.  The
+ * more resident workgroups) run with every row shared by 16, 32 or 64 workgroups that exchange
+ * integer width sums once per pass of 15 doublings or four bisection levels (the first pass takes
+ * the starting multiplier and the first four levels together); the same bits.  The
  * workgroups wait for each other with a bound: should a wait not end (it cannot while the launch
  * is resident as sized), the row's output is the invalid width 255 instead of a hang. */
 int64_t rdkv_knapsack_workspace_bytes(int B);

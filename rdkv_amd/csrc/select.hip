@@ -201,7 +201,8 @@ knapsack_bisect_kernel(const float* __restrict__ scores, int64_t stride_b, int g
 // busy for ~60 dependent passes).  A row's S workgroups each own a contiguous chunk of it, held in
 // registers.  One pass evaluates up to 17 candidate lambdas at once - the next 15 doublings, or
 // lambda = 0 and the 15 midpoints four bisection levels can reach (in the first pass together with
-// the row's starting lambda, which usually needs no doubling) - as integer width sums of the chunk.  The workgroups then exchange their sums: each stores its own as words that carry the
+// the row's starting lambda, which usually needs no doubling) - as integer width sums of the
+// chunk.  The workgroups then exchange their sums: each stores its own as words that carry the
 // pass number in their top byte, and reads every workgroup's words until all of them carry it
 // (double-buffered by pass parity: a workgroup can be at most one pass ahead of another of its row).
 // So a pass costs one store and one load round trip between workgroups, no atomic operation meets
@@ -731,13 +732,14 @@ int check_common(const void* scores, int B, int64_t T, const void* budget, const
 
 }  // namespace
 
-// Workgroups a row is shared by in the cooperative form (0: one workgroup per row, the two-launch
-// form): chunks of at least 512 scores, at most 64 per row, the whole launch on at most half of the
-// workgroup slots the device has for this kernel, and only when that gives a row at least sixteen
-// (with fewer, one workgroup per row was as fast or faster on 64 rows of 32k scores).
 // 0 / 1 / 2: the kernel that holds 2 / 4 / 8 scores of a chunk per thread in registers
 static int coop_held_index(int64_t chunk) { return chunk <= 2 * kCoopThreads ? 0 : (chunk <= 4 * kCoopThreads ? 1 : 2); }
 
+// Workgroups a row is shared by in the cooperative form (0: one workgroup per row, the two-launch
+// form): a power of two, chunks of at least 512 scores, at most 64 per row, the whole launch on at
+// most half of the workgroup slots the device has for the kernel variant the chunk length selects,
+// and only when that gives a row at least sixteen (with fewer, one workgroup per row was as fast or
+// faster on 64 rows of 32k scores).
 static int coop_split(int B, int64_t T, int max_iters) {
   if (B <= 0 || T < 4096 || max_iters > kCoopMaxIters) return 0;
   // workgroup slots of the device for the kernel that holds 2 / 4 / 8 scores per thread
