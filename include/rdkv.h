@@ -398,7 +398,7 @@ int rdkv_pack_layer_stream(const void *K_f16, const void *V_f16, int64_t stride_
  * the kernel) in bits 0..7.  Bits 8..31 are 0, or - only when EVERY unit of the call has the
  * same K row shape - that shape as d8 << 16 | d4 << 8 | d2 (so the argument is
  * R | d8 << 24 | d4 << 16 | d2 << 8 with R = d8 + d4 + d2): for the shapes the library has a
- * kernel of their own for (G <= 4: 32/0/0, 0/16/0, 0/0/8, 0/5/2) the call runs about 5 % faster, with
+ * kernel of their own for (32/0/0, 0/16/0, 0/0/8, 0/5/2) the call runs about 5 % faster, with
  * the same results bit for bit; any other shape runs the general kernel.  A unit whose shape
  * is not the stated one is not read and its output rows are NaN (lse: -inf).
  * workspace: rdkv_decode_fused_workspace_bytes(n_work, G) bytes.

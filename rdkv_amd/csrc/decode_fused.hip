@@ -1497,12 +1497,16 @@ static int launch_fused(const char *fn, const uint8_t *blob, const RdkvUnit *uni
     else RDKV_LAUNCH_FUSED_M(NH, RMAX, WPE, false, SHAPE);                                                 \
   } while (0)
 #define RDKV_LAUNCH_FUSED_WPE(NH, RMAX, WPE) RDKV_LAUNCH_FUSED_SHAPE(NH, RMAX, WPE, 0)
-  // Row shapes with a kernel of their own (one head group): every channel at 8, at 4 or at 2 bits,
-  // and the 4- / 2-bit mix of the 128k-context benchmark workload.
+  // Row shapes with a kernel of their own: every channel at 8, at 4 or at 2 bits, and the 4- / 2-bit
+  // mix of the 128k-context benchmark workload.
   if (G <= 4 && row_shape == kShape_0_5_2) RDKV_LAUNCH_FUSED_SHAPE(1, 8, 4, kShape_0_5_2);
   else if (G <= 4 && row_shape == kShape_0_16_0) RDKV_LAUNCH_FUSED_SHAPE(1, 16, 4, kShape_0_16_0);
   else if (G <= 4 && row_shape == kShape_0_0_8) RDKV_LAUNCH_FUSED_SHAPE(1, 8, 4, kShape_0_0_8);
   else if (G <= 4 && row_shape == kShape_32_0_0) RDKV_LAUNCH_FUSED_SHAPE(1, 32, 3, kShape_32_0_0);
+  else if (G > 4 && row_shape == kShape_0_5_2) RDKV_LAUNCH_FUSED_SHAPE(2, 8, 3, kShape_0_5_2);
+  else if (G > 4 && row_shape == kShape_0_16_0) RDKV_LAUNCH_FUSED_SHAPE(2, 16, 3, kShape_0_16_0);
+  else if (G > 4 && row_shape == kShape_0_0_8) RDKV_LAUNCH_FUSED_SHAPE(2, 8, 3, kShape_0_0_8);
+  else if (G > 4 && row_shape == kShape_32_0_0) RDKV_LAUNCH_FUSED_SHAPE(2, 32, 2, kShape_32_0_0);
   else if (G <= 4) {   // one head group
     if (max_row_dwords <= 12) RDKV_LAUNCH_FUSED_WPE(1, 12, 4);
     else if (max_row_dwords <= 16) RDKV_LAUNCH_FUSED_WPE(1, 16, 4);

@@ -477,7 +477,7 @@ def _uniform_shape_case(c2, c4, c8, H_kv, G, T, seed):
 
 @pytest.mark.parametrize("counts,shape", [((32, 40, 0), (0, 5, 2)), ((24, 36, 0), (0, 5, 2)), ((0, 128, 0), (0, 16, 0)),
                                           ((128, 0, 0), (0, 0, 8)), ((113, 0, 0), (0, 0, 8)), ((0, 0, 128), (32, 0, 0))])
-@pytest.mark.parametrize("G", [4, 2])
+@pytest.mark.parametrize("G", [4, 2, 8, 5])
 def test_fused_attention_fixed_shape_kernels_equal_the_general_kernel(counts, shape, G):
     """Caches whose units all have one K row shape state it in the row argument; for the shapes the
     library has kernels of their own for, those kernels give the general kernel's bits (two launches,
