@@ -20,6 +20,7 @@
 // Zero-points never touch the codes: K uses bias[h] = sum_c zp_c*qs[h][c], V accumulates
 // sum_t p'_t*zp_t per head next to the MFMA accumulators.
 // HBM-bound by design: the MFMA and VALU work per byte is far below the machine balance.
+#include <type_traits>
 #include "rdkv_common.h"
 #include "rope_device.h"
 #include "stream_format.h"
@@ -641,9 +642,10 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         ++tiles_done;
       }
       // ---- K side: scores for tokens 4*lb..4*lb+3 of head 4*hg+ln -------------------------
-      // Three loops, one per field width, over the dwords of that width; the K row is indexed
-      // dynamically (register-relative addressing), so each loop body is straight-line code for
-      // its width and the accumulators never leave their registers.  The hi and lo terms of
+      // One pass per field width over the dwords of that width: the 8-bit dwords, which start the
+      // row, with fixed register numbers; the 4- and 2-bit dwords as loops over the row indexed
+      // dynamically (register-relative addressing), each loop body straight-line code for its
+      // width.  The accumulators never leave their registers.  The hi and lo terms of
       // q*scale feed separate accumulators: two independent matrix-core chains.
       floatx4 sacc[NH], sacc_lo[NH];
 #pragma unroll
@@ -719,13 +721,23 @@ decode_fused_kernel(const uint8_t *__restrict__ blob,
         const int d8 = it.d8, d4 = it.d4, d2 = it.d2;
         int step = 0;
         QOp cur = q_load(0);
-        for (int i = 0; i < d8; ++i) {
-          const QOp nxt = q_load(step + 1);
-          const uint32_t w = k_dword(i);
-          k_step(mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu), cur);
-          cur = nxt;
-          step += 1;
-        }
+        // The 8-bit dwords start the row, so their register numbers and LDS offsets are fixed: nested
+        // "one more?" tests instead of a loop over an indexed register (written as a recursion: an
+        // unrolled loop with an exit per step is turned back into the indexed loop).
+        auto k8 = [&](auto self, auto at) __attribute__((always_inline)) -> void {
+          constexpr int I = decltype(at)::value;
+          if constexpr (I < RMAX) {
+            if (I < d8) {
+              const QOp nxt = q_load(I + 1);
+              const uint32_t w = I < kRowA ? krow[I < kRowA ? I : 0] : ktail[I >= kRowA ? I - kRowA : 0];
+              k_step(mk_op(w & 0x00FF00FFu, (w >> 8) & 0x00FF00FFu), cur);
+              cur = nxt;
+              self(self, std::integral_constant<int, I + 1>{});
+            }
+          }
+        };
+        k8(k8, std::integral_constant<int, 0>{});
+        step = d8;
         for (int i = 0; i < d4; ++i) {
           const QOp n1 = q_load(step + 1), n2 = q_load(step + 2);
           const uint32_t w = k_dword(d8 + i);
