@@ -1426,21 +1426,31 @@ merge_zone_c_kernel(const RdkvUnit *__restrict__ units, ZcInline iu, const float
   if (zc_w) {   // softmax weights of the zone C tokens over the union (fast_decode.py:1753-1755 w_new)
     __syncthreads();
     for (int t = tid; t < n_new; t += kThreads) {
+      // everything this token needs is requested first (the raw scores of the G heads, the two block
+      // scores it adds to): stores to one row may not be moved past loads of another by the compiler,
+      // which made this a chain of G + 2 round trips
+      float raw[G];
+#pragma unroll
+      for (int h = 0; h < G; ++h) raw[h] = zc_w[(int64_t)(q_row + h) * zc_w_stride + t];
+      // online block scores of blockwise decode (blockwise_decode.py:2085-2109): the query's weights
+      // on its own block, and on the first block when the query belongs to the second
+      const bool to_self = ts.self_scores && t >= q_block_start;
+      const bool to_next = ts.next_scores && q_block_start >= ts.block && t < ts.block;
+      float *self_at = to_self ? ts.self_scores + (int64_t)kv_row * ts.self_stride_h + t : nullptr;
+      float *next_at = to_next ? ts.next_scores + (int64_t)kv_row * ts.next_stride_h + t : nullptr;
+      const float self_old = to_self ? *self_at : 0.0f;
+      const float next_old = to_next ? *next_at : 0.0f;
       float s = 0.0f;     // over the group's heads in head order, as rdkv_tail_scores sums them
 #pragma unroll
       for (int h = 0; h < G; ++h) {
 #pragma clang fp contract(off)   // the stored weight is what is summed: no fusing with the product
-        float *row = zc_w + (int64_t)(q_row + h) * zc_w_stride;
         const float inv = fin_l[h] > 0.0f ? 1.0f / fin_l[h] : 0.0f;
-        const float w = fast_exp2(row[t] - fin_m[h]) * inv;
-        row[t] = w;
+        const float w = fast_exp2(raw[h] - fin_m[h]) * inv;
+        zc_w[(int64_t)(q_row + h) * zc_w_stride + t] = w;
         s = s + w;
       }
-      // online block scores of blockwise decode (blockwise_decode.py:2085-2109): the query's weights
-      // on its own block, and on the first block when the query belongs to the second
-      if (ts.self_scores && t >= q_block_start) ts.self_scores[(int64_t)kv_row * ts.self_stride_h + t] += s;
-      if (ts.next_scores && q_block_start >= ts.block && t < ts.block)
-        ts.next_scores[(int64_t)kv_row * ts.next_stride_h + t] += s;
+      if (to_self) *self_at = self_old + s;
+      if (to_next) *next_at = next_old + s;
     }
   }
 }
